@@ -1,0 +1,286 @@
+"""ctypes front-end of the CPU oracle (``libnbla_quant_oracle.so``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by ``__graft_entry__.smoke()``
+and by the CPU-baseline leg of ``bench.py``.  The product package never imports
+this module.  Every function takes and returns numpy arrays (fp32 / int32,
+C-contiguous) and maps one-to-one onto an ``orc_*`` entry point, which in turn
+cites the nnabla file:line it restates.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libnbla_quant_oracle.so")
+
+_c_float_p = ctypes.POINTER(ctypes.c_float)
+_c_int_p = ctypes.POINTER(ctypes.c_int)
+_c_long_p = ctypes.POINTER(ctypes.c_long)
+
+
+def build(force=False):
+    """Compile the oracle with its Makefile (g++ -O3, no -march, no FMA)."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.check_call(["make", "-s", "-C", _HERE])
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.orc_inq_create.restype = ctypes.c_void_p
+        _lib.orc_inq_counter.restype = ctypes.c_long
+    return _lib
+
+
+class OracleError(ValueError):
+    pass
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise OracleError("%s failed with nbla error code %d" % (what, rc))
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _fp(a):
+    return None if a is None else a.ctypes.data_as(_c_float_p)
+
+
+def _ip(a):
+    return a.ctypes.data_as(_c_int_p)
+
+
+def _longs(seq):
+    arr = (ctypes.c_long * len(seq))(*[int(v) for v in seq])
+    return arr
+
+
+def fixed_point_quantize(x, sign=True, n=8, delta=2.0 ** -4):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _check(lib().orc_fixed_point_quantize(_fp(x), _fp(y), ctypes.c_long(x.size), int(sign), int(n),
+                                          ctypes.c_float(delta)), "fixed_point_quantize")
+    return y
+
+
+def pow2_quantize(x, sign=True, with_zero=True, n=8, m=1):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _check(lib().orc_pow2_quantize(_fp(x), _fp(y), ctypes.c_long(x.size), int(sign), int(with_zero), int(n),
+                                   int(m)), "pow2_quantize")
+    return y
+
+
+def round_log2(a):
+    return lib().orc_round_log2(ctypes.c_float(a))
+
+
+def inq_exponent(a):
+    return lib().orc_inq_exponent(ctypes.c_float(a))
+
+
+def inq_n1(a):
+    return lib().orc_inq_n1(ctypes.c_float(a))
+
+
+def min_max_reduce(x, qshape):
+    x = _f32(x)
+    qshape = tuple(int(s) for s in qshape)
+    mn = np.empty(qshape, np.float32)
+    mx = np.empty(qshape, np.float32)
+    lib().orc_min_max_reduce(_fp(x), _longs(x.shape), x.ndim, _longs(qshape), _fp(mn), _fp(mx))
+    return mn, mx
+
+
+def min_max_quantize(x, qr_min, qr_max, ql_min, ql_max, decay=0.999, x_min_max=False, ema=False, eps=0.01):
+    """Returns (y, qr_min_new, qr_max_new, scale); the inputs are not modified."""
+    x = _f32(x)
+    qr_min = _f32(qr_min).copy()
+    qr_max = _f32(qr_max).copy()
+    ql_min = _f32(ql_min)
+    ql_max = _f32(ql_max)
+    assert qr_min.shape == qr_max.shape == ql_min.shape == ql_max.shape and qr_min.ndim == x.ndim
+    y = np.empty_like(x)
+    scale = np.empty_like(qr_min)
+    _check(lib().orc_min_max_quantize(_fp(x), _fp(y), _longs(x.shape), x.ndim, _longs(qr_min.shape), _fp(qr_min),
+                                      _fp(qr_max), _fp(ql_min), _fp(ql_max), ctypes.c_float(decay), int(x_min_max),
+                                      int(ema), ctypes.c_float(eps), _fp(scale)), "min_max_quantize")
+    return y, qr_min, qr_max, scale
+
+
+def sign(x, alpha0=1.0):
+    x = _f32(x)
+    y = np.empty_like(x)
+    lib().orc_sign(_fp(x), _fp(y), ctypes.c_long(x.size), ctypes.c_float(alpha0))
+    return y
+
+
+def affine(x, w, b=None):
+    x = _f32(x)
+    w = _f32(w)
+    M, K = x.shape
+    N = w.size // K
+    b = None if b is None else _f32(b)
+    y = np.empty((M, N), np.float32)
+    _check(lib().orc_affine(_fp(x), _fp(w), _fp(b), _fp(y), ctypes.c_long(M), ctypes.c_long(K), ctypes.c_long(N)),
+           "affine")
+    return y
+
+
+def binary_weight_prepare(W, quantize_zero_to=1.0, want_scaled=False):
+    """Returns (Wb, alpha[, scaled]) for W viewed as [K, N]."""
+    W = _f32(W)
+    K = W.shape[0]
+    N = W.size // K
+    Wb = np.empty_like(W)
+    alpha = np.empty(N, np.float32)
+    scaled = np.empty_like(W) if want_scaled else None
+    lib().orc_binary_weight_prepare(_fp(W), _fp(Wb), _fp(alpha), _fp(scaled), ctypes.c_long(K), ctypes.c_long(N),
+                                    ctypes.c_float(quantize_zero_to))
+    return (Wb, alpha, scaled) if want_scaled else (Wb, alpha)
+
+
+def binary_weight_affine(x, W, b=None, quantize_zero_to=1.0):
+    """Returns (y, Wb, alpha)."""
+    x = _f32(x)
+    W = _f32(W)
+    M, K = x.shape
+    N = W.size // K
+    b = None if b is None else _f32(b)
+    Wb = np.empty_like(W)
+    alpha = np.empty(N, np.float32)
+    y = np.empty((M, N), np.float32)
+    _check(lib().orc_binary_weight_affine(_fp(x), _fp(W), _fp(Wb), _fp(alpha), _fp(b), _fp(y), ctypes.c_long(M),
+                                          ctypes.c_long(K), ctypes.c_long(N), ctypes.c_float(quantize_zero_to)),
+           "binary_weight_affine")
+    return y, Wb, alpha
+
+
+def binary_connect_affine(x, W, b=None, quantize_zero_to=1.0):
+    """Returns (y, Wb)."""
+    x = _f32(x)
+    W = _f32(W)
+    M, K = x.shape
+    N = W.size // K
+    b = None if b is None else _f32(b)
+    Wb = np.empty_like(W)
+    y = np.empty((M, N), np.float32)
+    _check(lib().orc_binary_connect_affine(_fp(x), _fp(W), _fp(Wb), _fp(b), _fp(y), ctypes.c_long(M),
+                                           ctypes.c_long(K), ctypes.c_long(N), ctypes.c_float(quantize_zero_to)),
+           "binary_connect_affine")
+    return y, Wb
+
+
+def _conv_args(x, W, pad, stride, dilation, group):
+    x = _f32(x)
+    W = _f32(W)
+    nd = W.ndim - 2
+    outer = int(np.prod(x.shape[:x.ndim - nd - 1], dtype=np.int64))
+    C = x.shape[x.ndim - nd - 1]
+    in_sp = x.shape[x.ndim - nd:]
+    O = W.shape[0]
+    kernel = W.shape[2:]
+    pad = tuple(pad) if pad is not None else (0,) * nd
+    stride = tuple(stride) if stride is not None else (1,) * nd
+    dilation = tuple(dilation) if dilation is not None else (1,) * nd
+    out_sp = (ctypes.c_long * nd)()
+    tail = (ctypes.c_long(outer), ctypes.c_long(C), nd, _longs(in_sp), ctypes.c_long(O), _longs(kernel), _longs(pad),
+            _longs(stride), _longs(dilation), ctypes.c_long(group))
+    _check(lib().orc_convolution(None, None, None, None, *tail, out_sp), "convolution geometry")
+    yshape = tuple(x.shape[:x.ndim - nd - 1]) + (O,) + tuple(out_sp)
+    return x, W, tail, yshape
+
+
+def convolution(x, W, b=None, pad=None, stride=None, dilation=None, group=1):
+    x, W, tail, yshape = _conv_args(x, W, pad, stride, dilation, group)
+    b = None if b is None else _f32(b)
+    y = np.empty(yshape, np.float32)
+    _check(lib().orc_convolution(_fp(x), _fp(W), _fp(b), _fp(y), *tail, None), "convolution")
+    return y
+
+
+def binary_weight_convolution(x, W, b=None, pad=None, stride=None, dilation=None, group=1, quantize_zero_to=1.0):
+    """Returns (y, Wb, alpha)."""
+    x, W, tail, yshape = _conv_args(x, W, pad, stride, dilation, group)
+    b = None if b is None else _f32(b)
+    y = np.empty(yshape, np.float32)
+    Wb = np.empty_like(W)
+    alpha = np.empty(W.shape[0], np.float32)
+    _check(lib().orc_binary_weight_convolution(_fp(x), _fp(W), _fp(Wb), _fp(alpha), _fp(b), _fp(y), *tail,
+                                               ctypes.c_float(quantize_zero_to)), "binary_weight_convolution")
+    return y, Wb, alpha
+
+
+def binary_connect_convolution(x, W, b=None, pad=None, stride=None, dilation=None, group=1, quantize_zero_to=1.0):
+    """Returns (y, Wb)."""
+    x, W, tail, yshape = _conv_args(x, W, pad, stride, dilation, group)
+    b = None if b is None else _f32(b)
+    y = np.empty(yshape, np.float32)
+    Wb = np.empty_like(W)
+    _check(lib().orc_binary_connect_convolution(_fp(x), _fp(W), _fp(Wb), _fp(b), _fp(y), *tail,
+                                                ctypes.c_float(quantize_zero_to)), "binary_connect_convolution")
+    return y, Wb
+
+
+class Inq(object):
+    """Stateful INQ weight logic (one object per INQAffine / INQConvolution)."""
+
+    def __init__(self, size, num_bits=4, inq_iterations=(), selection_algorithm="largest_abs", seed=-1):
+        its = (ctypes.c_int * max(1, len(inq_iterations)))(*[int(i) for i in inq_iterations])
+        self._h = lib().orc_inq_create(ctypes.c_long(size), int(num_bits), its, len(inq_iterations),
+                                       selection_algorithm.encode(), int(seed))
+        if not self._h:
+            raise OracleError("invalid selection algorithm %r" % (selection_algorithm,))
+        self._h = ctypes.c_void_p(self._h)
+        self.size = size
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().orc_inq_destroy(self._h)
+            self._h = None
+
+    @property
+    def counter(self):
+        return lib().orc_inq_counter(self._h)
+
+    def quantize_weights(self, W, I):
+        """Steps A-C in place on fp32 W and int32 I; returns (n1, n2)."""
+        assert W.dtype == np.float32 and I.dtype == np.int32 and W.flags.c_contiguous and I.flags.c_contiguous
+        n1 = ctypes.c_int()
+        n2 = ctypes.c_int()
+        lib().orc_inq_quantize_weights(self._h, _fp(W), _ip(I), ctypes.byref(n1), ctypes.byref(n2))
+        return n1.value, n2.value
+
+    def commit(self, W, I):
+        lib().orc_inq_commit(self._h, _fp(W), _ip(I))
+
+    def affine(self, x, W, I, b=None):
+        """Full INQAffine forward; W and I are updated in place; returns y."""
+        x = _f32(x)
+        M, K = x.shape
+        N = W.size // K
+        b = None if b is None else _f32(b)
+        y = np.empty((M, N), np.float32)
+        _check(lib().orc_inq_affine(self._h, _fp(x), _fp(W), _ip(I), _fp(b), _fp(y), ctypes.c_long(M),
+                                    ctypes.c_long(K), ctypes.c_long(N)), "inq_affine")
+        return y
+
+    def convolution(self, x, W, I, b=None, pad=None, stride=None, dilation=None, group=1):
+        x, _, tail, yshape = _conv_args(x, W, pad, stride, dilation, group)
+        b = None if b is None else _f32(b)
+        y = np.empty(yshape, np.float32)
+        _check(lib().orc_inq_convolution(self._h, _fp(x), _fp(W), _ip(I), _fp(b), _fp(y), *tail), "inq_convolution")
+        return y
