@@ -1,0 +1,191 @@
+/*
+ * nbla_hip_kernels.h -- C-ABI of the MI355X (gfx950) kernels behind nnabla's
+ * quantization function family.
+ *
+ * Each entry point is what the `forward_impl` of a "hip:float" Function class
+ * calls in place of the loop (or the chain of helper Functions) that nnabla's
+ * CPU class runs; the reference interface it replaces is cited per function
+ * (paths relative to the nnabla source tree).
+ *
+ * Conventions
+ *   - plain C: raw DEVICE pointers, element counts, scalars; no C++/torch types.
+ *   - every call is asynchronous on `stream` (a hipStream_t passed as void*;
+ *     NULL = the default stream) unless its comment says it synchronises.
+ *   - nothing here allocates device memory: scratch comes in through
+ *     `workspace` arguments sized by the matching *_workspace_bytes() query.
+ *     Workspaces must be 256-byte aligned.
+ *   - return value: NBLA_HIP_OK (0); a negative NBLA_HIP_ERR_* for argument
+ *     errors (mirroring nbla::error_code of the NBLA_CHECK the CPU class would
+ *     raise); or a positive hipError_t.  nbla_hip_last_error() returns the
+ *     message of the last failure on the calling thread.
+ *   - all tensors are dense, C-contiguous fp32 unless stated otherwise.
+ */
+#ifndef NBLA_HIP_KERNELS_H_
+#define NBLA_HIP_KERNELS_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NBLA_HIP_OK 0
+#define NBLA_HIP_ERR_NOT_IMPLEMENTED (-2) /* nbla::error_code::not_implemented */
+#define NBLA_HIP_ERR_VALUE (-3)           /* nbla::error_code::value           */
+#define NBLA_HIP_ERR_MEMORY (-5)          /* workspace too small / misaligned  */
+#define NBLA_HIP_ERR_RUNTIME (-10)        /* library not initialised, bad arch */
+
+/* ---------------------------------------------------------------- library */
+
+/* Initialise the library for `device` (makes it current): checks that the
+ * device is gfx950 and uploads the three per-binade cut tables that make
+ * Pow2Quantize / INQ bit-exact against the host's libm (log2f is evaluated on
+ * the host once per binade boundary, never per element).  Idempotent and
+ * thread-safe; every other entry point calls it lazily for the current device.
+ * Mirrors the role of init_cpu(): src/nbla/init.cpp.tmpl:44-111. */
+int nbla_hip_init(int device);
+
+const char *nbla_hip_last_error(void);
+const char *nbla_hip_version(void);
+
+/* Host-side view of the calibrated tables (277 uint32 entries each, indexed by
+ * binade: subnormal binades 0..22, normal exponent field e at index e+22).
+ * which: 0 = roundf(log2f(a)) (pow2_quantize.cpp:60), 1 = INQ weight exponent
+ * (inq_affine.cpp:176-179), 2 = INQ n1 (inq_affine.cpp:161-164). */
+int nbla_hip_cut_table(int which, uint32_t *out277);
+
+/* ------------------------------------------------------ FixedPointQuantize */
+
+/* y = FixedPointQuantize(x; sign, n, delta).
+ * Replaces FixedPointQuantize<float>::forward_impl,
+ * src/nbla/function/generic/fixed_point_quantize.cpp:46-66 (bounds from
+ * setup_impl :29-43).  NBLA_HIP_ERR_VALUE when n <= 0, delta <= 0 or the
+ * sign-adjusted width is <= 0, as the NBLA_CHECKs at :31-32 and :41-42.
+ * In-place (y == x) is allowed. */
+int nbla_hip_fixed_point_quantize_f32(const float *x, float *y, size_t size,
+                                      int sign, int n, float delta,
+                                      void *stream);
+
+/* ------------------------------------------------------------ Pow2Quantize */
+
+/* y = Pow2Quantize(x; sign, with_zero, n, m).
+ * Replaces Pow2Quantize<float>::forward_impl,
+ * src/nbla/function/generic/pow2_quantize.cpp:48-82 (setup :29-45).
+ * NBLA_HIP_ERR_VALUE as the NBLA_CHECKs at :32 and :41-44;
+ * NBLA_HIP_ERR_NOT_IMPLEMENTED when 2^m or 2^(m-(2^n'-1)) is not a finite
+ * non-zero fp32 number. */
+int nbla_hip_pow2_quantize_f32(const float *x, float *y, size_t size, int sign,
+                               int with_zero, int n, int m, void *stream);
+
+/* ---------------------------------------------------------- MinMaxQuantize */
+
+/* Scratch for the min/max reduction partials and the nudged-range table. */
+size_t nbla_hip_min_max_quantize_workspace_bytes(const int64_t *xshape,
+                                                 int ndim,
+                                                 const int64_t *qshape);
+
+/* y = MinMaxQuantize(x, qr_min, qr_max, ql_min, ql_max; decay, x_min_max, ema,
+ * eps).  Replaces MinMaxQuantize<float>::forward_impl,
+ * src/nbla/function/generic/min_max_quantize.cpp:130-223 with nudge_range
+ * (:353-361) and nudge_qr_min_max (:363-390): the ~20 helper-Function passes
+ * become one min/max reduction (only when x_min_max) and one elementwise pass.
+ * qshape has ndim entries, each 1 (reduced axis) or equal to xshape[i]; the four
+ * q tensors and `scale` (the content of scale_sptr_, written) have that shape.
+ * qr_min / qr_max are UPDATED IN PLACE exactly as the reference updates its
+ * parameters.  NBLA_HIP_ERR_VALUE for a shape mismatch (:69-81). */
+int nbla_hip_min_max_quantize_f32(const float *x, float *y,
+                                  const int64_t *xshape, int ndim,
+                                  const int64_t *qshape, float *qr_min,
+                                  float *qr_max, const float *ql_min,
+                                  const float *ql_max, float *scale,
+                                  float decay, int x_min_max, int ema,
+                                  float eps, void *workspace,
+                                  size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------- binary weights: sign/alpha/pack */
+
+/* Bytes of the 1-bit packed GEMM operand for a [K, N] weight matrix. */
+size_t nbla_hip_packed_bits_bytes(int64_t K, int64_t N);
+/* Bytes of the bf16x3-split, fragment-ordered GEMM operand for x [M, K]. */
+size_t nbla_hip_split_operand_bytes(int64_t M, int64_t K);
+/* Scratch of nbla_hip_binarize_weights_f32 (column-sum partials, zero count). */
+size_t nbla_hip_binarize_workspace_bytes(int64_t K, int64_t N);
+
+/* Sign-binarise W and (optionally) compute alpha, in one pass over W:
+ *   Wb[k,n]  = w>0 ? 1 : w<0 ? -1 : quantize_zero_to   (sign.hpp:48-50)
+ *   alpha[n] = (sum_k |W[k,n]|) * ((float)1 / K)       (alpha may be NULL)
+ *   bits     = 1 bit per weight (set = negative), in MFMA fragment order
+ * The GEMM view is always B[k, n] with k the contraction index.
+ *   transposed == 0: W is stored [K, N] (affine weights); replaces the
+ *     Transpose/Abs/Sum/MulScalar/Sign passes of
+ *     binary_weight_affine.cpp:85-102 and the Sign of
+ *     binary_connect_affine.cpp:63-64.
+ *   transposed == 1: W is stored [N, K] (convolution weights viewed
+ *     [channels_o, col_w]); replaces binary_weight_convolution.cpp:83-98 and
+ *     binary_connect_convolution.cpp:71-72.
+ * Wb has W's own storage layout.  zero_count (device int, may be NULL) receives
+ * the number of exact zeros in W: a non-zero count with quantize_zero_to other
+ * than +-1 means `bits` alone cannot represent Wb. */
+int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha,
+                                  uint32_t *bits, int64_t K, int64_t N,
+                                  int transposed, float quantize_zero_to,
+                                  int *zero_count, void *workspace,
+                                  size_t workspace_bytes, void *stream);
+
+/* Split x [M, K] (row stride ldx elements) into three bf16 planes
+ * (x == hi + mid + lo exactly) stored in MFMA fragment order. */
+int nbla_hip_split_bf16x3_f32(const float *x, int64_t ldx, void *xsplit,
+                              int64_t M, int64_t K, void *stream);
+
+/* y[m, n] = (sum_k x[m,k] * (+-1)[k,n]) * alpha[n] + bias[n]
+ * with x given as the split operand and the weights as packed bits; alpha and
+ * bias may be NULL.  fp32 accumulation of exact bf16 products on the MFMA
+ * units.  Output addressing: element (m, n) is written at
+ *   y[(m / inner) * outer_stride + n * n_stride + (m % inner)]
+ * so a row-major [M, N] result is (inner=1, outer_stride=N, n_stride=1) and a
+ * convolution result [batch, O, Ho*Wo] is (inner=Ho*Wo, outer_stride=O*Ho*Wo,
+ * n_stride=Ho*Wo).  Replaces the Eigen product of affine.cpp:87-95 /
+ * convolution.cpp:185-193 for binarised weights. */
+int nbla_hip_gemm_bits_f32(const void *xsplit, const uint32_t *bits,
+                           const float *alpha, const float *bias, float *y,
+                           int64_t M, int64_t K, int64_t N, int64_t inner,
+                           int64_t outer_stride, int64_t n_stride,
+                           void *stream);
+
+/* ------------------------------------------------------- whole-op forwards */
+
+size_t nbla_hip_binary_affine_workspace_bytes(int64_t M, int64_t K, int64_t N);
+
+/* BinaryWeightAffine forward: x [M,K], W [K,N] -> Wb [K,N], alpha [N], y [M,N]
+ * (bias [N] may be NULL).  Replaces BinaryWeightAffine<float>::forward_impl,
+ * src/nbla/function/generic/binary_weight_affine.cpp:75-122.
+ * When quantize_zero_to is neither +1 nor -1 the call synchronises the stream
+ * once to learn whether W holds exact zeros (then the product runs on the
+ * materialised fp32 weights instead of the packed bits). */
+int nbla_hip_binary_weight_affine_f32(const float *x, const float *W,
+                                      float *Wb, float *alpha,
+                                      const float *bias, float *y, int64_t M,
+                                      int64_t K, int64_t N,
+                                      float quantize_zero_to, void *workspace,
+                                      size_t workspace_bytes, void *stream);
+
+/* BinaryConnectAffine forward (no alpha).  Replaces
+ * BinaryConnectAffine<float>::forward_impl,
+ * src/nbla/function/generic/binary_connect_affine.cpp:60-71. */
+int nbla_hip_binary_connect_affine_f32(const float *x, const float *W,
+                                       float *Wb, const float *bias, float *y,
+                                       int64_t M, int64_t K, int64_t N,
+                                       float quantize_zero_to, void *workspace,
+                                       size_t workspace_bytes, void *stream);
+
+/* Plain fp32 GEMM y[M,N] = x[M,K] * w[K,N] (+ bias[N]) on the fp32 MFMA units.
+ * Replaces Affine<float>::forward_impl, src/nbla/function/generic/affine.cpp:81-96. */
+int nbla_hip_affine_f32(const float *x, const float *w, const float *bias,
+                        float *y, int64_t M, int64_t K, int64_t N,
+                        void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NBLA_HIP_KERNELS_H_ */

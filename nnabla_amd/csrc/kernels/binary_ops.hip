@@ -1,0 +1,96 @@
+// Whole-operation forwards of BinaryWeightAffine / BinaryConnectAffine: weight
+// preparation, activation split and the bit-weight product chained on one stream.
+#include "common.hpp"
+#include "gemm_layout.hpp"
+
+namespace nbla_hip {
+
+int launch_gemm_f32(const float *x, const float *w, const float *colscale, const float *bias, float *y, int64_t M,
+                    int64_t K, int64_t N, hipStream_t stream);
+
+namespace {
+
+struct AffineWorkspace {
+  size_t bits_off, split_off, prep_off, count_off, total;
+};
+
+AffineWorkspace plan_affine(int64_t M, int64_t K, int64_t N) {
+  AffineWorkspace w;
+  size_t off = 0;
+  w.bits_off = off;
+  off += round_up(nbla_hip_packed_bits_bytes(K, N), 256);
+  w.split_off = off;
+  off += round_up(nbla_hip_split_operand_bytes(M, K), 256);
+  w.prep_off = off;
+  off += round_up(nbla_hip_binarize_workspace_bytes(K, N), 256);
+  w.count_off = off;
+  off += 256;
+  w.total = off;
+  return w;
+}
+
+int binary_affine_forward(const float *x, const float *W, float *Wb, float *alpha, const float *bias, float *y,
+                          int64_t M, int64_t K, int64_t N, float zero_to, void *workspace, size_t workspace_bytes,
+                          void *stream_) {
+  if (M <= 0 || K <= 0 || N <= 0)
+    return fail(NBLA_HIP_ERR_VALUE, "invalid affine shape (M=%lld, K=%lld, N=%lld).", (long long)M, (long long)K,
+                (long long)N);
+  const AffineWorkspace ws = plan_affine(M, K, N);
+  if (workspace_bytes < ws.total || !aligned256(workspace))
+    return fail(NBLA_HIP_ERR_MEMORY, "binary affine workspace too small (%zu < %zu) or misaligned.", workspace_bytes,
+                ws.total);
+  char *base = static_cast<char *>(workspace);
+  uint32_t *bits = reinterpret_cast<uint32_t *>(base + ws.bits_off);
+  void *xsplit = base + ws.split_off;
+  void *prep = base + ws.prep_off;
+  int *count = reinterpret_cast<int *>(base + ws.count_off);
+  const bool representable = (zero_to == 1.0f || zero_to == -1.0f);
+
+  int rc = nbla_hip_binarize_weights_f32(W, Wb, alpha, bits, K, N, 0, zero_to, representable ? nullptr : count, prep,
+                                         nbla_hip_binarize_workspace_bytes(K, N), stream_);
+  if (rc)
+    return rc;
+  if (!representable) {
+    // Sign(0) = zero_to is neither +1 nor -1: the packed bits are only valid when
+    // W holds no exact zero.  One scalar comes back to the host to decide.
+    int host_count = 0;
+    hipError_t e = hipMemcpyAsync(&host_count, count, sizeof(int), hipMemcpyDeviceToHost, as_stream(stream_));
+    if (e == hipSuccess)
+      e = hipStreamSynchronize(as_stream(stream_));
+    if (e != hipSuccess)
+      return fail_hip(e, "reading the zero-weight count");
+    if (host_count != 0)
+      return launch_gemm_f32(x, Wb, alpha, bias, y, M, K, N, as_stream(stream_));
+  }
+  rc = nbla_hip_split_bf16x3_f32(x, K, xsplit, M, K, stream_);
+  if (rc)
+    return rc;
+  return nbla_hip_gemm_bits_f32(xsplit, bits, alpha, bias, y, M, K, N, 1, N, 1, stream_);
+}
+
+} // namespace
+} // namespace nbla_hip
+
+using namespace nbla_hip;
+
+extern "C" {
+
+size_t nbla_hip_binary_affine_workspace_bytes(int64_t M, int64_t K, int64_t N) { return plan_affine(M, K, N).total; }
+
+int nbla_hip_binary_weight_affine_f32(const float *x, const float *W, float *Wb, float *alpha, const float *bias,
+                                      float *y, int64_t M, int64_t K, int64_t N, float quantize_zero_to,
+                                      void *workspace, size_t workspace_bytes, void *stream) {
+  if (!alpha)
+    return fail(NBLA_HIP_ERR_VALUE, "BinaryWeightAffine needs an alpha output of size N.");
+  return binary_affine_forward(x, W, Wb, alpha, bias, y, M, K, N, quantize_zero_to, workspace, workspace_bytes,
+                               stream);
+}
+
+int nbla_hip_binary_connect_affine_f32(const float *x, const float *W, float *Wb, const float *bias, float *y,
+                                       int64_t M, int64_t K, int64_t N, float quantize_zero_to, void *workspace,
+                                       size_t workspace_bytes, void *stream) {
+  return binary_affine_forward(x, W, Wb, nullptr, bias, y, M, K, N, quantize_zero_to, workspace, workspace_bytes,
+                               stream);
+}
+
+} // extern "C"

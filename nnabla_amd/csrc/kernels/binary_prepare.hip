@@ -1,0 +1,350 @@
+// Operand preparation for the binary-weight products: one pass over W that
+// writes Sign(W), the 1-bit packed MFMA operand and the |W| column sums, and the
+// bf16x3 split of the activations.
+#include "common.hpp"
+#include "gemm_layout.hpp"
+
+#include <cmath>
+
+namespace nbla_hip {
+namespace {
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kPrepBlock = 256;
+constexpr int kKSlice = 512; // k rows handled by one block of binarize_kn (16 k-tiles)
+
+// sign.hpp:48-50
+__device__ __forceinline__ float sign_of(float w, float zero_to) {
+  return (w > 0.0f) ? 1.0f : ((w < 0.0f) ? -1.0f : zero_to);
+}
+
+// Workspace: colsum partials [slices][Np] floats, then zero-count partials
+// [slices * col_groups] ints.  slices depends on the source layout.
+struct PrepPlan {
+  int64_t k_tiles, col_groups, Np, slices;
+  size_t sums_bytes, zeros_bytes;
+};
+
+PrepPlan make_prep_plan(int64_t K, int64_t N, bool transposed) {
+  PrepPlan P;
+  P.k_tiles = bits_k_tiles(K);
+  P.col_groups = bits_col_groups(N);
+  P.Np = P.col_groups * kColGroup;
+  P.slices = transposed ? ceil_div(P.k_tiles, 4) : ceil_div(K, kKSlice);
+  P.sums_bytes = round_up((size_t)P.slices * P.Np * sizeof(float), 256);
+  P.zeros_bytes = round_up((size_t)P.slices * P.col_groups * sizeof(int), 256);
+  return P;
+}
+
+// W stored [K, N].  Block = 16 teams of 16 threads; team t handles k-tile
+// (slice * 16 + t) of column group blockIdx.x.  Thread (nq, g) of a team owns
+// columns f*32 + 4*nq + {0..3} (f = 0, 1) and k offsets s*16 + g*8 + {0..7}
+// (s = 0, 1): 32 bits for each of four packed words, which are exactly the
+// words of lanes g*32 + 4*nq + {0..3}.
+template <bool kVec>
+__global__ __launch_bounds__(kPrepBlock) void binarize_kn(const float *__restrict__ W, float *__restrict__ Wb,
+                                                          uint32_t *__restrict__ bits, float *__restrict__ sums,
+                                                          int *__restrict__ zeros, int64_t K, int64_t N,
+                                                          int64_t col_groups, int64_t Np, float zero_to) {
+  const int team = threadIdx.x >> 4, tt = threadIdx.x & 15;
+  const int nq = tt & 7, g = tt >> 3;
+  const int64_t cg = blockIdx.x;
+  const int64_t kt = (int64_t)blockIdx.y * 16 + team;
+  uint32_t word[4] = {0u, 0u, 0u, 0u};
+  float asum[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  int nzero = 0;
+  if (kt * kTileK < K) {
+#pragma unroll
+    for (int f = 0; f < 2; ++f) {
+      const int64_t n0 = cg * kColGroup + f * 32 + 4 * nq;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int64_t k = kt * kTileK + s * 16 + g * 8 + e;
+          if (k >= K || n0 >= N)
+            continue;
+          float w[4];
+          if (kVec) {
+            const float4_t v = *reinterpret_cast<const float4_t *>(W + k * N + n0);
+            w[0] = v.x, w[1] = v.y, w[2] = v.z, w[3] = v.w;
+          } else {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+              w[c] = (n0 + c < N) ? W[k * N + n0 + c] : 1.0f;
+          }
+          float b[4];
+          const int pos = packed_bit_position(f, s, e);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            b[c] = sign_of(w[c], zero_to);
+            const bool in = kVec || (n0 + c < N);
+            const bool is_zero = !(w[c] > 0.0f) && !(w[c] < 0.0f); // +-0 (and NaN) take zero_to
+            const bool neg = (w[c] < 0.0f) || (is_zero && zero_to < 0.0f);
+            word[c] |= (in && neg) ? (1u << pos) : 0u;
+            asum[f][c] += in ? fabsf(w[c]) : 0.0f;
+            nzero += (in && is_zero) ? 1 : 0;
+          }
+          if (kVec) {
+            float4_t o;
+            o.x = b[0], o.y = b[1], o.z = b[2], o.w = b[3];
+            *reinterpret_cast<float4_t *>(Wb + k * N + n0) = o;
+          } else {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+              if (n0 + c < N)
+                Wb[k * N + n0 + c] = b[c];
+          }
+        }
+      }
+    }
+    uint4_t wv;
+    wv.x = word[0], wv.y = word[1], wv.z = word[2], wv.w = word[3];
+    *reinterpret_cast<uint4_t *>(bits + (kt * col_groups + cg) * 64 + g * 32 + 4 * nq) = wv;
+  }
+  // |W| column sums of this k slice: fixed-order fold of the 32 (team, g) partials.
+  __shared__ float s_sum[32][kColGroup];
+  __shared__ int s_zero[kPrepBlock / 64];
+#pragma unroll
+  for (int f = 0; f < 2; ++f)
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      s_sum[team * 2 + g][f * 32 + 4 * nq + c] = asum[f][c];
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1)
+    nzero += __shfl_xor(nzero, off);
+  if ((threadIdx.x & 63) == 0)
+    s_zero[threadIdx.x >> 6] = nzero;
+  __syncthreads();
+  if (threadIdx.x < kColGroup) {
+    float acc = 0.0f;
+    for (int r = 0; r < 32; ++r)
+      acc += s_sum[r][threadIdx.x];
+    sums[(int64_t)blockIdx.y * Np + cg * kColGroup + threadIdx.x] = acc;
+  }
+  if (threadIdx.x == 0)
+    zeros[(int64_t)blockIdx.y * col_groups + cg] = s_zero[0] + s_zero[1] + s_zero[2] + s_zero[3];
+}
+
+// W stored [N, K] (convolution weights viewed [channels_o, col_w]).  Wavefront w
+// of the block handles k-tile blockIdx.y*4 + w of column group blockIdx.x; lane
+// l builds its own packed word from 4 runs of 8 consecutive k of rows n(f).
+__global__ __launch_bounds__(kPrepBlock) void binarize_nk(const float *__restrict__ W, float *__restrict__ Wb,
+                                                          uint32_t *__restrict__ bits, float *__restrict__ sums,
+                                                          int *__restrict__ zeros, int64_t K, int64_t N,
+                                                          int64_t col_groups, int64_t Np, int64_t k_tiles,
+                                                          float zero_to) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int g = lane >> 5, r = lane & 31;
+  const int64_t cg = blockIdx.x;
+  const int64_t kt = (int64_t)blockIdx.y * 4 + wave;
+  uint32_t word = 0u;
+  float asum[2] = {0.f, 0.f};
+  int nzero = 0;
+  if (kt < k_tiles) {
+#pragma unroll
+    for (int f = 0; f < 2; ++f) {
+      const int64_t n = cg * kColGroup + f * 32 + r;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int64_t k = kt * kTileK + s * 16 + g * 8 + e;
+          if (n < N && k < K) {
+            const float w = W[n * K + k];
+            Wb[n * K + k] = sign_of(w, zero_to);
+            const bool is_zero = !(w > 0.0f) && !(w < 0.0f);
+            const bool neg = (w < 0.0f) || (is_zero && zero_to < 0.0f);
+            word |= neg ? (1u << packed_bit_position(f, s, e)) : 0u;
+            asum[f] += fabsf(w);
+            nzero += is_zero ? 1 : 0;
+          }
+        }
+      }
+    }
+    bits[(kt * col_groups + cg) * 64 + lane] = word;
+  }
+  __shared__ float s_sum[8][kColGroup];
+  __shared__ int s_zero[kPrepBlock / 64];
+  s_sum[wave * 2 + g][r] = asum[0];
+  s_sum[wave * 2 + g][32 + r] = asum[1];
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1)
+    nzero += __shfl_xor(nzero, off);
+  if (lane == 0)
+    s_zero[wave] = nzero;
+  __syncthreads();
+  if (threadIdx.x < kColGroup) {
+    float acc = 0.0f;
+    for (int q = 0; q < 8; ++q)
+      acc += s_sum[q][threadIdx.x];
+    sums[(int64_t)blockIdx.y * Np + cg * kColGroup + threadIdx.x] = acc;
+  }
+  if (threadIdx.x == 0)
+    zeros[(int64_t)blockIdx.y * col_groups + cg] = s_zero[0] + s_zero[1] + s_zero[2] + s_zero[3];
+}
+
+// alpha[n] = (sum over slices) * ((float)1 / K)   (binary_weight_affine.cpp:68,
+// binary_weight_convolution.cpp:66: a multiply by the rounded reciprocal), and
+// the total zero count.
+__global__ __launch_bounds__(kPrepBlock) void binarize_finalize(const float *__restrict__ sums, const int *__restrict__ zeros,
+                                                                float *__restrict__ alpha, int *__restrict__ zero_count,
+                                                                int64_t N, int64_t Np, int64_t slices,
+                                                                int64_t zero_entries, float inv_k) {
+  const int64_t n = (int64_t)blockIdx.x * kPrepBlock + threadIdx.x;
+  if (alpha && n < N) {
+    float acc = 0.0f;
+    for (int64_t s = 0; s < slices; ++s)
+      acc += sums[s * Np + n];
+    alpha[n] = acc * inv_k;
+  }
+  if (zero_count && blockIdx.x == 0) {
+    int z = 0;
+    for (int64_t i = threadIdx.x; i < zero_entries; i += kPrepBlock)
+      z += zeros[i];
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1)
+      z += __shfl_xor(z, off);
+    __shared__ int s_z[kPrepBlock / 64];
+    if ((threadIdx.x & 63) == 0)
+      s_z[threadIdx.x >> 6] = z;
+    __syncthreads();
+    if (threadIdx.x == 0)
+      *zero_count = s_z[0] + s_z[1] + s_z[2] + s_z[3];
+  }
+}
+
+// ------------------------------------------------------------------ bf16 split
+__device__ __forceinline__ uint32_t bf16_rne(float v) { // finite v
+  const uint32_t u = __float_as_uint(v);
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ float bf16_to_float(uint32_t h) { return __uint_as_float(h << 16); }
+
+// x == hi + mid + lo with each part a bf16: the residuals are exact in fp32.
+// Non-finite x keeps its class in `hi` alone.
+__device__ __forceinline__ void split3(float x, uint32_t &hi, uint32_t &mid, uint32_t &lo) {
+  const uint32_t u = __float_as_uint(x);
+  if ((u & 0x7f800000u) == 0x7f800000u) {
+    hi = (u >> 16) | ((u & 0xffffu) ? 0x40u : 0u);
+    mid = lo = 0u;
+    return;
+  }
+  hi = bf16_rne(x);
+  if ((hi & 0x7f80u) == 0x7f80u)
+    hi = u >> 16; // rounding up would overflow to infinity: truncate instead
+  const float r1 = x - bf16_to_float(hi);
+  mid = bf16_rne(r1);
+  const float r2 = r1 - bf16_to_float(mid);
+  lo = bf16_rne(r2);
+}
+
+// One wavefront per (row block, k block) fragment; lane l converts the eight
+// values x[rb*32 + l%32][kb*16 + (l/32)*8 + 0..7].
+__global__ __launch_bounds__(kPrepBlock) void split_bf16x3(const float *__restrict__ x, int64_t ldx, uint4_t *__restrict__ out,
+                                                           int64_t M, int64_t K, int64_t k_blocks, int64_t frags) {
+  const int64_t frag = (int64_t)blockIdx.x * (kPrepBlock / 64) + (threadIdx.x >> 6);
+  if (frag >= frags)
+    return;
+  const int lane = threadIdx.x & 63;
+  const int64_t rb = frag / k_blocks, kb = frag - rb * k_blocks;
+  const int64_t m = rb * kFragRows + (lane & 31);
+  const int64_t k0 = kb * kFragK + (lane >> 5) * 8;
+  float v[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    v[e] = (m < M && k0 + e < K) ? x[m * ldx + k0 + e] : 0.0f;
+  uint32_t h[8], mi[8], l[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    split3(v[e], h[e], mi[e], l[e]);
+  uint4_t o;
+  uint4_t *dst = out + frag * 3 * 64 + lane;
+  o.x = h[0] | (h[1] << 16), o.y = h[2] | (h[3] << 16), o.z = h[4] | (h[5] << 16), o.w = h[6] | (h[7] << 16);
+  dst[0] = o;
+  o.x = mi[0] | (mi[1] << 16), o.y = mi[2] | (mi[3] << 16), o.z = mi[4] | (mi[5] << 16), o.w = mi[6] | (mi[7] << 16);
+  dst[64] = o;
+  o.x = l[0] | (l[1] << 16), o.y = l[2] | (l[3] << 16), o.z = l[4] | (l[5] << 16), o.w = l[6] | (l[7] << 16);
+  dst[128] = o;
+}
+
+} // namespace
+} // namespace nbla_hip
+
+using namespace nbla_hip;
+
+extern "C" {
+
+size_t nbla_hip_packed_bits_bytes(int64_t K, int64_t N) {
+  return (size_t)bits_k_tiles(K) * bits_col_groups(N) * 64 * sizeof(uint32_t);
+}
+
+size_t nbla_hip_split_operand_bytes(int64_t M, int64_t K) {
+  return (size_t)split_row_blocks(M) * split_k_blocks(K) * 3 * kFragBytes;
+}
+
+size_t nbla_hip_binarize_workspace_bytes(int64_t K, int64_t N) {
+  const PrepPlan a = make_prep_plan(K, N, false), b = make_prep_plan(K, N, true);
+  const size_t wa = a.sums_bytes + a.zeros_bytes, wb = b.sums_bytes + b.zeros_bytes;
+  return wa > wb ? wa : wb;
+}
+
+int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint32_t *bits, int64_t K, int64_t N,
+                                  int transposed, float quantize_zero_to, int *zero_count, void *workspace,
+                                  size_t workspace_bytes, void *stream_) {
+  if (K <= 0 || N <= 0)
+    return fail(NBLA_HIP_ERR_VALUE, "weight matrix must not be empty (K=%lld, N=%lld).", (long long)K, (long long)N);
+  const PrepPlan P = make_prep_plan(K, N, transposed != 0);
+  if (workspace_bytes < P.sums_bytes + P.zeros_bytes || !aligned256(workspace))
+    return fail(NBLA_HIP_ERR_MEMORY, "binarize workspace too small or misaligned.");
+  if (!aligned16(bits))
+    return fail(NBLA_HIP_ERR_MEMORY, "packed-bit buffer must be 16-byte aligned.");
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  hipStream_t stream = as_stream(stream_);
+  float *sums = static_cast<float *>(workspace);
+  int *zeros = reinterpret_cast<int *>(static_cast<char *>(workspace) + P.sums_bytes);
+  if (!transposed) {
+    const dim3 grid((unsigned)P.col_groups, (unsigned)P.slices);
+    if (N % 4 == 0 && aligned16(W) && aligned16(Wb))
+      hipLaunchKernelGGL(binarize_kn<true>, grid, dim3(kPrepBlock), 0, stream, W, Wb, bits, sums, zeros, K, N,
+                         P.col_groups, P.Np, quantize_zero_to);
+    else
+      hipLaunchKernelGGL(binarize_kn<false>, grid, dim3(kPrepBlock), 0, stream, W, Wb, bits, sums, zeros, K, N,
+                         P.col_groups, P.Np, quantize_zero_to);
+  } else {
+    const dim3 grid((unsigned)P.col_groups, (unsigned)P.slices);
+    hipLaunchKernelGGL(binarize_nk, grid, dim3(kPrepBlock), 0, stream, W, Wb, bits, sums, zeros, K, N, P.col_groups,
+                       P.Np, P.k_tiles, quantize_zero_to);
+  }
+  NBLA_HIP_LAUNCH_CHECK("binarize_weights");
+  if (alpha || zero_count) {
+    const float inv_k = (float)1 / K;
+    hipLaunchKernelGGL(binarize_finalize, dim3((unsigned)ceil_div(N, kPrepBlock)), dim3(kPrepBlock), 0, stream, sums,
+                       zeros, alpha, zero_count, N, P.Np, P.slices, P.slices * P.col_groups, inv_k);
+    NBLA_HIP_LAUNCH_CHECK("binarize_finalize");
+  }
+  return NBLA_HIP_OK;
+}
+
+int nbla_hip_split_bf16x3_f32(const float *x, int64_t ldx, void *xsplit, int64_t M, int64_t K, void *stream_) {
+  if (M <= 0 || K <= 0 || ldx < K)
+    return fail(NBLA_HIP_ERR_VALUE, "invalid split operand shape (M=%lld, K=%lld, ldx=%lld).", (long long)M,
+                (long long)K, (long long)ldx);
+  if (!aligned16(xsplit))
+    return fail(NBLA_HIP_ERR_MEMORY, "split operand buffer must be 16-byte aligned.");
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  const int64_t k_blocks = split_k_blocks(K);
+  const int64_t frags = split_row_blocks(M) * k_blocks;
+  hipLaunchKernelGGL(split_bf16x3, dim3((unsigned)ceil_div(frags, kPrepBlock / 64)), dim3(kPrepBlock), 0,
+                     as_stream(stream_), x, ldx, static_cast<uint4_t *>(xsplit), M, K, k_blocks, frags);
+  NBLA_HIP_LAUNCH_CHECK("split_bf16x3");
+  return NBLA_HIP_OK;
+}
+
+} // extern "C"

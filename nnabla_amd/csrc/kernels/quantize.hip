@@ -1,0 +1,653 @@
+// Elementwise quantizers (FixedPointQuantize, Pow2Quantize, MinMaxQuantize) as
+// HBM-bound gfx950 kernels: 128-bit coalesced loads/stores, every fp32
+// operation rounded on its own (the file is compiled with -ffp-contract=off and
+// correctly rounded division), wavefront-shuffle reductions for the min/max.
+#include "common.hpp"
+
+#include <cmath>
+#include <cstring>
+
+namespace nbla_hip {
+namespace {
+
+constexpr int kBlock = 256;  // threads per block: 4 wavefronts
+constexpr int kUnroll = 4;   // float4 per thread per block tile
+constexpr int kTile = kBlock * kUnroll; // float4 per block
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float4_t load4(const float *p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const float4_t *>(p));
+}
+__device__ __forceinline__ void store4(float *p, float4_t v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<float4_t *>(p));
+}
+
+// Generic driver: applies `op` (a functor float -> float) to `size` elements.
+// The vector body covers size/4 float4s; the tail (size % 4) is done by block 0.
+template <typename Op> __global__ __launch_bounds__(kBlock) void map_vec4(const float *__restrict__ x, float *__restrict__ y, size_t n4, size_t size, Op op) {
+  op.prepare();
+  const size_t base = (size_t)blockIdx.x * kTile + threadIdx.x;
+  float4_t v[kUnroll];
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const size_t i = base + (size_t)j * kBlock;
+    if (i < n4)
+      v[j] = load4(x + 4 * i);
+  }
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const size_t i = base + (size_t)j * kBlock;
+    if (i < n4) {
+      float4_t r;
+      r.x = op(v[j].x);
+      r.y = op(v[j].y);
+      r.z = op(v[j].z);
+      r.w = op(v[j].w);
+      store4(y + 4 * i, r);
+    }
+  }
+  if (blockIdx.x == 0) {
+    const size_t i = 4 * n4 + threadIdx.x;
+    if (i < size)
+      y[i] = op(x[i]);
+  }
+}
+
+// Fallback for pointers that are not 16-byte aligned.
+template <typename Op> __global__ __launch_bounds__(kBlock) void map_scalar(const float *__restrict__ x, float *__restrict__ y, size_t size, Op op) {
+  op.prepare();
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < size; i += (size_t)gridDim.x * kBlock)
+    y[i] = op(x[i]);
+}
+
+template <typename Op> int launch_map(const float *x, float *y, size_t size, Op op, hipStream_t stream, const char *what) {
+  if (size == 0)
+    return NBLA_HIP_OK;
+  if (aligned16(x) && aligned16(y)) {
+    const size_t n4 = size / 4;
+    const size_t blocks = n4 ? (n4 + kTile - 1) / kTile : 1;
+    hipLaunchKernelGGL(map_vec4<Op>, dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, y, n4, size, op);
+  } else {
+    size_t blocks = (size + kBlock - 1) / kBlock;
+    if (blocks > 65536)
+      blocks = 65536;
+    hipLaunchKernelGGL(map_scalar<Op>, dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, y, size, op);
+  }
+  NBLA_HIP_LAUNCH_CHECK(what);
+  return NBLA_HIP_OK;
+}
+
+// ------------------------------------------------------------------ FixedPoint
+// fixed_point_quantize.cpp:53-65.  q = |x| / delta is an fp32 divide; adding 0.5
+// in double and truncating equals trunc(q) + (q - trunc(q) >= 0.5), all exact in
+// fp32; the product with delta is one fp32 multiply.  When delta is a power of
+// two the divide is replaced by the (bit-identical) multiply with 1/delta.
+template <bool kPow2Delta> struct FixedPointOp {
+  float max_, min_, delta, inv_delta;
+  __device__ __forceinline__ void prepare() {}
+  __device__ __forceinline__ float operator()(float x) const {
+    if (x > max_)
+      return max_;
+    if (x < min_)
+      return min_;
+    const float a = fabsf(x);
+    const float q = kPow2Delta ? a * inv_delta : a / delta;
+    const float t = truncf(q);
+    const float k = (q - t >= 0.5f) ? t + 1.0f : t;
+    const float y = k * delta;
+    return (x < 0.0f) ? -y : y;
+  }
+};
+
+// ------------------------------------------------------------------------ Pow2
+// pow2_quantize.cpp:55-81.  r = roundf(log2f(|x|)) comes from the calibrated
+// per-binade cut (staged in LDS); 2^r, the clamps and the sign are exact.
+struct Pow2Op {
+  const uint32_t *cuts; // device table, kNumBinades entries
+  float p_max, p_min, thr;
+  int e_max, e_min; // log2 of p_max / p_min
+  int sign, with_zero;
+  __device__ __forceinline__ void prepare() {
+    __shared__ uint32_t s_cut[kNumBinades];
+    for (int i = threadIdx.x; i < kNumBinades; i += blockDim.x)
+      s_cut[i] = cuts[i];
+    __syncthreads();
+    lds = s_cut;
+  }
+  const uint32_t *lds;
+  __device__ __forceinline__ float operator()(float x) const {
+    const uint32_t u = __float_as_uint(x) & 0x7fffffffu;
+    const float a = __uint_as_float(u);
+    float q;
+    if (u > 0x7f800000u) {
+      q = a; // NaN propagates through every comparison of the reference
+    } else {
+      int r;
+      if (u == 0u)
+        r = -100000; // log2f(0) = -inf -> 2^-inf = 0, below every p_min
+      else if (u == 0x7f800000u)
+        r = 100000;
+      else {
+        const int idx = binade_of(u);
+        r = binade_exponent(idx) + (u >= lds[idx] ? 1 : 0);
+      }
+      if (r > e_max)
+        q = p_max;
+      else if (r < e_min)
+        q = with_zero ? ((a < thr) ? 0.0f : p_min) : p_min;
+      else
+        q = pow2_int(r);
+    }
+    const bool neg = x < 0.0f;
+    if (sign)
+      return neg ? -q : q;
+    return neg ? (with_zero ? 0.0f : p_min) : q;
+  }
+};
+
+} // namespace
+} // namespace nbla_hip
+
+using namespace nbla_hip;
+
+extern "C" {
+
+int nbla_hip_fixed_point_quantize_f32(const float *x, float *y, size_t size, int sign, int n, float delta,
+                                      void *stream) {
+  if (!(n > 0 && delta > 0.))
+    return fail(NBLA_HIP_ERR_VALUE, "Both bit width and delta should be positive.");
+  const int nn = sign ? n - 1 : n;
+  if (!(nn > 0))
+    return fail(NBLA_HIP_ERR_VALUE, "bit width should be positive when considering sign (1bit).");
+  if (nn > 30)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "bit widths above 30 overflow the reference's int conversion.");
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  // fixed_point_quantize.cpp:38-40: double arithmetic, stored to float members
+  const float max_ = (float)((std::pow(2, nn) - 1) * delta);
+  const float min_ = sign ? (float)(-max_) : 0.0f;
+  int exp2 = 0;
+  const bool pow2_delta = std::frexp(delta, &exp2) == 0.5f && std::isnormal(1.0f / delta) && std::isnormal(delta);
+  if (pow2_delta) {
+    FixedPointOp<true> op{max_, min_, delta, 1.0f / delta};
+    return launch_map(x, y, size, op, as_stream(stream), "fixed_point_quantize");
+  }
+  FixedPointOp<false> op{max_, min_, delta, 0.0f};
+  return launch_map(x, y, size, op, as_stream(stream), "fixed_point_quantize");
+}
+
+int nbla_hip_pow2_quantize_f32(const float *x, float *y, size_t size, int sign, int with_zero, int n, int m,
+                               void *stream) {
+  if (!(n > 0))
+    return fail(NBLA_HIP_ERR_VALUE, "bit width should be positive.");
+  int nn = sign ? n - 1 : n;
+  nn = with_zero ? nn - 1 : nn;
+  if (!(nn > 0))
+    return fail(NBLA_HIP_ERR_VALUE, "bit width should be positive when considering zero (1bit) and sign (1bit).");
+  if (nn > 9)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than 2^9 power-of-two levels leave the fp32 exponent range.");
+  const int e_max = m, e_min = m - ((1 << nn) - 1);
+  if (e_max > 127 || e_min < -149)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "2^%d .. 2^%d is outside the finite non-zero fp32 range.", e_min, e_max);
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  Pow2Op op;
+  op.cuts = device_cut_table(kCutPow2Round);
+  op.p_max = (float)std::pow(2., e_max);                 // pow2_quantize.cpp:37
+  op.p_min = (float)std::pow(2., e_min);                 // :38
+  op.thr = (float)((float)op.p_min * std::pow(2., -0.5)); // :39 (float member times double)
+  op.e_max = e_max;
+  op.e_min = e_min;
+  op.sign = sign;
+  op.with_zero = with_zero;
+  op.lds = nullptr;
+  return launch_map(x, y, size, op, as_stream(stream), "pow2_quantize");
+}
+
+} // extern "C"
+
+// ---------------------------------------------------------------------- MinMax
+namespace nbla_hip {
+namespace {
+
+// (x shape, q shape) collapsed to element index = (r0 * K + k) * R1 + r1 with k
+// the kept (per-channel) index and r0, r1 the reduced ones.
+struct MinMaxLayout {
+  int64_t R0, K, R1, total;
+  bool ok;
+};
+
+MinMaxLayout collapse(const int64_t *xshape, int ndim, const int64_t *qshape) {
+  // runs of (kept?) axes, ignoring size-1 axes
+  int64_t sizes[3] = {1, 1, 1};
+  int stage = 0; // 0: leading reduced, 1: kept, 2: trailing reduced
+  MinMaxLayout L{1, 1, 1, 1, true};
+  for (int i = 0; i < ndim; ++i) {
+    const int64_t s = xshape[i];
+    L.total *= s;
+    if (s == 1)
+      continue;
+    const bool kept = qshape[i] != 1;
+    if (kept) {
+      if (stage == 0)
+        stage = 1;
+      else if (stage == 2) {
+        L.ok = false; // kept, reduced, kept: not a single (R0, K, R1) pattern
+        continue;
+      }
+      sizes[1] *= s;
+    } else {
+      if (stage == 1)
+        stage = 2;
+      sizes[stage == 0 ? 0 : 2] *= s;
+    }
+  }
+  L.R0 = sizes[0];
+  L.K = sizes[1];
+  L.R1 = sizes[2];
+  if (L.K == 1) { // per-tensor: one flat run
+    L.R1 = L.R0 * L.R1;
+    L.R0 = 1;
+  }
+  return L;
+}
+
+constexpr int kRedBlock = 256;
+constexpr int kRedTile = kRedBlock * 4; // elements per block tile
+constexpr int kMaxChunks = 2048;
+
+struct MinMaxPlan {
+  MinMaxLayout L;
+  int64_t tiles_per_row; // tiles covering one run of R1 elements
+  int64_t tiles_per_k;   // R0 * tiles_per_row
+  int nchunks;           // blocks (and partials) per k
+  size_t params_bytes, partial_bytes;
+};
+
+MinMaxPlan make_plan(const int64_t *xshape, int ndim, const int64_t *qshape) {
+  MinMaxPlan P;
+  P.L = collapse(xshape, ndim, qshape);
+  P.tiles_per_row = (P.L.R1 + kRedTile - 1) / kRedTile;
+  P.tiles_per_k = P.L.R0 * P.tiles_per_row;
+  int64_t want = (4096 + P.L.K - 1) / P.L.K;
+  if (want > kMaxChunks)
+    want = kMaxChunks;
+  if (want > P.tiles_per_k)
+    want = P.tiles_per_k;
+  if (want < 1)
+    want = 1;
+  P.nchunks = (int)want;
+  P.params_bytes = round_up((size_t)P.L.K * 16, 256);
+  P.partial_bytes = round_up((size_t)P.L.K * P.nchunks * 16, 256);
+  return P;
+}
+
+struct MinMaxPartial {
+  float vmin;
+  uint32_t imin;
+  float vmax;
+  uint32_t imax;
+};
+
+// min.cpp:29-41 / max.cpp:48-60 scan the slice in index order with strict
+// comparisons starting from +-1e8; the first of several equal extrema (which can
+// only differ for +0/-0) wins.  Tracking (value, first index) and combining with
+// "smaller value, then smaller index" reproduces that for any traversal order.
+struct Extrema {
+  float vmin, vmax;
+  uint32_t imin, imax;
+  __device__ __forceinline__ void init() {
+    vmin = 1e+8f;
+    vmax = -1e+8f;
+    imin = imax = 0xffffffffu;
+  }
+  __device__ __forceinline__ void take(float v, uint32_t i) { // i increases per thread
+    if (v < vmin) {
+      vmin = v;
+      imin = i;
+    }
+    if (v > vmax) {
+      vmax = v;
+      imax = i;
+    }
+  }
+  __device__ __forceinline__ void merge(float omin, uint32_t oimin, float omax, uint32_t oimax) {
+    if (omin < vmin || (omin == vmin && oimin < imin)) {
+      vmin = omin;
+      imin = oimin;
+    }
+    if (omax > vmax || (omax == vmax && oimax < imax)) {
+      vmax = omax;
+      imax = oimax;
+    }
+  }
+  __device__ __forceinline__ void wave_reduce() {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      const float a = __shfl_xor(vmin, off);
+      const uint32_t ai = __shfl_xor(imin, off);
+      const float b = __shfl_xor(vmax, off);
+      const uint32_t bi = __shfl_xor(imax, off);
+      merge(a, ai, b, bi);
+    }
+  }
+};
+
+// Stage 1: block (chunk c, channel k) scans tiles c, c+nchunks, ... of channel k.
+template <bool kVec>
+__global__ __launch_bounds__(kRedBlock) void minmax_reduce_tiles(const float *__restrict__ x, MinMaxPartial *__restrict__ partial,
+                                                                 int64_t K, int64_t R1, int64_t tiles_per_row,
+                                                                 int64_t tiles_per_k, int nchunks) {
+  const int64_t k = blockIdx.y;
+  Extrema ex;
+  ex.init();
+  for (int64_t t = blockIdx.x; t < tiles_per_k; t += nchunks) {
+    const int64_t r0 = t / tiles_per_row;
+    const int64_t r1 = (t - r0 * tiles_per_row) * kRedTile + 4 * threadIdx.x;
+    if (r1 >= R1)
+      continue;
+    const float *p = x + (r0 * K + k) * R1 + r1;
+    const uint32_t idx = (uint32_t)(r0 * R1 + r1);
+    if (kVec) { // R1 % 4 == 0 and x 16-byte aligned
+      const float4_t v = *reinterpret_cast<const float4_t *>(p);
+      ex.take(v.x, idx);
+      ex.take(v.y, idx + 1);
+      ex.take(v.z, idx + 2);
+      ex.take(v.w, idx + 3);
+    } else {
+      const int n = (R1 - r1) < 4 ? (int)(R1 - r1) : 4;
+      for (int j = 0; j < n; ++j)
+        ex.take(p[j], idx + j);
+    }
+  }
+  ex.wave_reduce();
+  __shared__ MinMaxPartial s_part[kRedBlock / 64];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0)
+    s_part[wave] = MinMaxPartial{ex.vmin, ex.imin, ex.vmax, ex.imax};
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kRedBlock / 64; ++w)
+      ex.merge(s_part[w].vmin, s_part[w].imin, s_part[w].vmax, s_part[w].imax);
+    partial[k * nchunks + blockIdx.x] = MinMaxPartial{ex.vmin, ex.imin, ex.vmax, ex.imax};
+  }
+}
+
+// Per-tensor stage 1 (K == 1, 16-byte aligned): a flat grid-strided scan with
+// four independent 128-bit loads in flight per thread.
+__global__ __launch_bounds__(kRedBlock) void minmax_reduce_flat(const float *__restrict__ x, MinMaxPartial *__restrict__ partial,
+                                                                size_t n4, size_t size) {
+  Extrema ex;
+  ex.init();
+  const size_t stride = (size_t)gridDim.x * kRedBlock;
+  size_t i = (size_t)blockIdx.x * kRedBlock + threadIdx.x;
+  for (; i + 3 * stride < n4; i += 4 * stride) {
+    float4_t v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      v[j] = load4(x + 4 * (i + j * stride));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t idx = (uint32_t)(4 * (i + j * stride));
+      ex.take(v[j].x, idx);
+      ex.take(v[j].y, idx + 1);
+      ex.take(v[j].z, idx + 2);
+      ex.take(v[j].w, idx + 3);
+    }
+  }
+  for (; i < n4; i += stride) {
+    const float4_t v = load4(x + 4 * i);
+    const uint32_t idx = (uint32_t)(4 * i);
+    ex.take(v.x, idx);
+    ex.take(v.y, idx + 1);
+    ex.take(v.z, idx + 2);
+    ex.take(v.w, idx + 3);
+  }
+  if (blockIdx.x == gridDim.x - 1) { // tail elements, highest indices
+    const size_t t = 4 * n4 + threadIdx.x;
+    if (t < size)
+      ex.take(x[t], (uint32_t)t);
+  }
+  ex.wave_reduce();
+  __shared__ MinMaxPartial s_part[kRedBlock / 64];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0)
+    s_part[wave] = MinMaxPartial{ex.vmin, ex.imin, ex.vmax, ex.imax};
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kRedBlock / 64; ++w)
+      ex.merge(s_part[w].vmin, s_part[w].imin, s_part[w].vmax, s_part[w].imax);
+    partial[blockIdx.x] = MinMaxPartial{ex.vmin, ex.imin, ex.vmax, ex.imax};
+  }
+}
+
+// Stage 2: one wavefront per channel folds the partials, then lane 0 applies the
+// EMA (min_max_quantize.cpp:159-178), nudge_range (:353-361), the scale
+// (:188-190) and nudge_qr_min_max (:363-390), one rounded fp32 op at a time.
+struct MinMaxScalars {
+  float decay, one_minus_decay, eps;
+  int x_min_max, ema;
+};
+
+__global__ __launch_bounds__(64) void minmax_finalize(const MinMaxPartial *__restrict__ partial, int nchunks,
+                                                      float *__restrict__ qr_min, float *__restrict__ qr_max,
+                                                      const float *__restrict__ ql_min,
+                                                      const float *__restrict__ ql_max, float *__restrict__ scale_out,
+                                                      float4_t *__restrict__ params, MinMaxScalars s) {
+  const int64_t k = blockIdx.x;
+  Extrema ex;
+  ex.init();
+  if (s.x_min_max) {
+    for (int c = threadIdx.x; c < nchunks; c += 64) {
+      const MinMaxPartial p = partial[k * nchunks + c];
+      ex.merge(p.vmin, p.imin, p.vmax, p.imax);
+    }
+    ex.wave_reduce();
+  }
+  if (threadIdx.x != 0)
+    return;
+  float lo = qr_min[k], hi = qr_max[k];
+  if (s.x_min_max && s.ema) {
+    const float a = ex.vmin * s.one_minus_decay;
+    lo = lo * s.decay;
+    lo = lo + a;
+    const float b = ex.vmax * s.one_minus_decay;
+    hi = hi * s.decay;
+    hi = hi + b;
+  } else if (s.x_min_max) {
+    lo = ex.vmin;
+    hi = ex.vmax;
+  }
+  if (hi - lo < s.eps)
+    hi = lo + s.eps;
+  qr_min[k] = lo;
+  qr_max[k] = hi;
+  const float qlo = ql_min[k], qhi = ql_max[k];
+  float scale = hi - lo;
+  const float levels = qhi - qlo;
+  scale = scale / levels;
+  const float zp_from_min = qlo - lo / scale;
+  float zp;
+  if (zp_from_min <= qlo)
+    zp = qlo;
+  else if (zp_from_min >= qhi)
+    zp = qhi;
+  else
+    zp = round_half_away(zp_from_min);
+  const float m_n = (qlo - zp) * scale;
+  const float M_n = (qhi - zp) * scale;
+  scale_out[k] = scale;
+  float4_t pr;
+  pr.x = m_n;
+  pr.y = M_n;
+  pr.z = scale;
+  pr.w = 0.0f;
+  params[k] = pr;
+}
+
+// min_max_quantize.cpp:213-222: seven separately rounded fp32 operations.
+__device__ __forceinline__ float minmax_apply(float x, float m_n, float M_n, float scale) {
+  float t = (x > m_n) ? x : m_n;
+  t = (t < M_n) ? t : M_n;
+  t = t - m_n;
+  t = t / scale;
+  t = round_half_away(t);
+  t = t * scale;
+  return t + m_n;
+}
+
+// Stage 3a: per-tensor, 16-byte aligned.
+__global__ __launch_bounds__(kBlock) void minmax_apply_flat(const float *__restrict__ x, float *__restrict__ y, size_t n4,
+                                                            size_t size, const float4_t *__restrict__ params) {
+  const float4_t pr = params[0];
+  const size_t base = (size_t)blockIdx.x * kTile + threadIdx.x;
+  float4_t v[kUnroll];
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const size_t i = base + (size_t)j * kBlock;
+    if (i < n4)
+      v[j] = load4(x + 4 * i);
+  }
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const size_t i = base + (size_t)j * kBlock;
+    if (i < n4) {
+      float4_t r;
+      r.x = minmax_apply(v[j].x, pr.x, pr.y, pr.z);
+      r.y = minmax_apply(v[j].y, pr.x, pr.y, pr.z);
+      r.z = minmax_apply(v[j].z, pr.x, pr.y, pr.z);
+      r.w = minmax_apply(v[j].w, pr.x, pr.y, pr.z);
+      store4(y + 4 * i, r);
+    }
+  }
+  if (blockIdx.x == 0) {
+    const size_t i = 4 * n4 + threadIdx.x;
+    if (i < size)
+      y[i] = minmax_apply(x[i], pr.x, pr.y, pr.z);
+  }
+}
+
+// Stage 3b: per-channel rows of R1 contiguous elements (R1 % 4 == 0, aligned):
+// blockIdx.x = row (r0 * K + k), blockIdx.y = tile along the row.
+__global__ __launch_bounds__(kBlock) void minmax_apply_rows(const float *__restrict__ x, float *__restrict__ y, int64_t K,
+                                                            int64_t R1, const float4_t *__restrict__ params) {
+  const int64_t row = blockIdx.x;
+  const float4_t pr = params[row % K];
+  const int64_t n4 = R1 / 4;
+  const float *xr = x + row * R1;
+  float *yr = y + row * R1;
+  for (int64_t i = (int64_t)blockIdx.y * kBlock + threadIdx.x; i < n4; i += (int64_t)gridDim.y * kBlock) {
+    const float4_t v = load4(xr + 4 * i);
+    float4_t r;
+    r.x = minmax_apply(v.x, pr.x, pr.y, pr.z);
+    r.y = minmax_apply(v.y, pr.x, pr.y, pr.z);
+    r.z = minmax_apply(v.z, pr.x, pr.y, pr.z);
+    r.w = minmax_apply(v.w, pr.x, pr.y, pr.z);
+    store4(yr + 4 * i, r);
+  }
+}
+
+// Stage 3c: any layout / alignment, one element per step.
+__global__ __launch_bounds__(kBlock) void minmax_apply_generic(const float *__restrict__ x, float *__restrict__ y, int64_t total,
+                                                               int64_t K, int64_t R1,
+                                                               const float4_t *__restrict__ params) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
+    const float4_t pr = params[(i / R1) % K];
+    y[i] = minmax_apply(x[i], pr.x, pr.y, pr.z);
+  }
+}
+
+} // namespace
+} // namespace nbla_hip
+
+extern "C" {
+
+size_t nbla_hip_min_max_quantize_workspace_bytes(const int64_t *xshape, int ndim, const int64_t *qshape) {
+  const MinMaxPlan P = make_plan(xshape, ndim, qshape);
+  return P.params_bytes + P.partial_bytes;
+}
+
+int nbla_hip_min_max_quantize_f32(const float *x, float *y, const int64_t *xshape, int ndim, const int64_t *qshape,
+                                  float *qr_min, float *qr_max, const float *ql_min, const float *ql_max, float *scale,
+                                  float decay, int x_min_max, int ema, float eps, void *workspace,
+                                  size_t workspace_bytes, void *stream_) {
+  for (int i = 0; i < ndim; ++i)
+    if (qshape[i] != 1 && qshape[i] != xshape[i])
+      return fail(NBLA_HIP_ERR_VALUE,
+                  "x.shape and ql_min.shape must be same except for i-th dimension where ql_min.shape[i] == 1.");
+  const MinMaxPlan P = make_plan(xshape, ndim, qshape);
+  if (!P.L.ok)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED,
+                "kept axes separated by reduced axes (e.g. q shape (C,1,W)) are not supported by the HIP kernel.");
+  if (P.L.total == 0)
+    return NBLA_HIP_OK;
+  if (P.L.R0 * P.L.R1 > 0xffffffffll)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "reduction slices above 2^32 elements are not supported.");
+  if (workspace_bytes < P.params_bytes + P.partial_bytes || !aligned256(workspace))
+    return fail(NBLA_HIP_ERR_MEMORY, "min_max_quantize workspace too small or misaligned.");
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  hipStream_t stream = as_stream(stream_);
+  float4_t *params = static_cast<float4_t *>(workspace);
+  MinMaxPartial *partial = reinterpret_cast<MinMaxPartial *>(static_cast<char *>(workspace) + P.params_bytes);
+  const MinMaxLayout &L = P.L;
+  const bool vec_ok = aligned16(x) && (L.R1 % 4 == 0 || L.K == 1);
+  int nchunks = P.nchunks;
+
+  if (x_min_max) {
+    if (L.K == 1 && aligned16(x)) {
+      const size_t n4 = (size_t)L.total / 4;
+      size_t blocks = (n4 + kRedBlock * 4 - 1) / (kRedBlock * 4);
+      if (blocks > (size_t)nchunks)
+        blocks = nchunks;
+      if (blocks < 1)
+        blocks = 1;
+      nchunks = (int)blocks;
+      hipLaunchKernelGGL(minmax_reduce_flat, dim3((unsigned)blocks), dim3(kRedBlock), 0, stream, x, partial, n4,
+                         (size_t)L.total);
+    } else if (vec_ok && L.R1 % 4 == 0) {
+      hipLaunchKernelGGL(minmax_reduce_tiles<true>, dim3(nchunks, (unsigned)L.K), dim3(kRedBlock), 0, stream, x,
+                         partial, L.K, L.R1, P.tiles_per_row, P.tiles_per_k, nchunks);
+    } else {
+      hipLaunchKernelGGL(minmax_reduce_tiles<false>, dim3(nchunks, (unsigned)L.K), dim3(kRedBlock), 0, stream, x,
+                         partial, L.K, L.R1, P.tiles_per_row, P.tiles_per_k, nchunks);
+    }
+    NBLA_HIP_LAUNCH_CHECK("min_max_quantize reduction");
+  }
+  MinMaxScalars s;
+  s.decay = (float)decay;                            // (T)(decay_)        min_max_quantize.cpp:105
+  s.one_minus_decay = (float)(1.0 - (double)decay);  // (T)(1.0 - decay_)  :106
+  s.eps = eps;
+  s.x_min_max = x_min_max;
+  s.ema = ema;
+  hipLaunchKernelGGL(minmax_finalize, dim3((unsigned)L.K), dim3(64), 0, stream, partial, nchunks, qr_min, qr_max,
+                     ql_min, ql_max, scale, params, s);
+  NBLA_HIP_LAUNCH_CHECK("min_max_quantize finalize");
+
+  if (L.K == 1 && aligned16(x) && aligned16(y)) {
+    const size_t n4 = (size_t)L.total / 4;
+    const size_t blocks = n4 ? (n4 + kTile - 1) / kTile : 1;
+    hipLaunchKernelGGL(minmax_apply_flat, dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, y, n4, (size_t)L.total,
+                       params);
+  } else if (aligned16(x) && aligned16(y) && L.R1 % 4 == 0 && L.R1 >= 256 && L.R0 * L.K < 0x7fffffffll) {
+    int64_t ytiles = (L.R1 / 4 + kBlock - 1) / kBlock;
+    if (ytiles > 64)
+      ytiles = 64;
+    hipLaunchKernelGGL(minmax_apply_rows, dim3((unsigned)(L.R0 * L.K), (unsigned)ytiles), dim3(kBlock), 0, stream, x,
+                       y, L.K, L.R1, params);
+  } else {
+    int64_t blocks = (L.total + kBlock - 1) / kBlock;
+    if (blocks > 65536)
+      blocks = 65536;
+    hipLaunchKernelGGL(minmax_apply_generic, dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, y, L.total, L.K, L.R1,
+                       params);
+  }
+  NBLA_HIP_LAUNCH_CHECK("min_max_quantize apply");
+  return NBLA_HIP_OK;
+}
+
+} // extern "C"

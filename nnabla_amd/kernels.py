@@ -1,0 +1,202 @@
+"""ctypes binding of the kernel C-ABI (``include/nbla_hip_kernels.h``).
+
+Device memory and streams come from the caller; the helpers at the bottom accept
+``torch`` CUDA tensors purely as a convenient owner of device pointers.  Nothing
+here computes on the host and nothing falls back to the CPU: a missing library or
+a failing call raises ``KernelError``.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libnbla_hip_kernels.so")
+
+OK = 0
+ERR_NOT_IMPLEMENTED = -2
+ERR_VALUE = -3
+ERR_MEMORY = -5
+ERR_RUNTIME = -10
+
+#: every symbol declared in include/nbla_hip_kernels.h
+EXPORTED = (
+    "nbla_hip_init", "nbla_hip_last_error", "nbla_hip_version", "nbla_hip_cut_table",
+    "nbla_hip_fixed_point_quantize_f32", "nbla_hip_pow2_quantize_f32",
+    "nbla_hip_min_max_quantize_workspace_bytes", "nbla_hip_min_max_quantize_f32",
+    "nbla_hip_packed_bits_bytes", "nbla_hip_split_operand_bytes", "nbla_hip_binarize_workspace_bytes",
+    "nbla_hip_binarize_weights_f32", "nbla_hip_split_bf16x3_f32", "nbla_hip_gemm_bits_f32",
+    "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_weight_affine_f32",
+    "nbla_hip_binary_connect_affine_f32", "nbla_hip_affine_f32",
+)
+
+
+class KernelError(RuntimeError):
+    def __init__(self, code, message):
+        RuntimeError.__init__(self, "nbla_hip error %d: %s" % (code, message))
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    """The loaded kernel library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise KernelError(ERR_RUNTIME, "%s is missing: run `make -C nnabla_amd/csrc` (or "
+                              "__graft_entry__.build())" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        L.nbla_hip_last_error.restype = ctypes.c_char_p
+        L.nbla_hip_version.restype = ctypes.c_char_p
+        for name in ("nbla_hip_min_max_quantize_workspace_bytes", "nbla_hip_packed_bits_bytes",
+                     "nbla_hip_split_operand_bytes", "nbla_hip_binarize_workspace_bytes",
+                     "nbla_hip_binary_affine_workspace_bytes"):
+            getattr(L, name).restype = ctypes.c_size_t
+        _lib = L
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise KernelError(rc, lib().nbla_hip_last_error().decode())
+
+
+def _p(t):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _i64(v):
+    return ctypes.c_int64(int(v))
+
+
+def _shape(seq):
+    return (ctypes.c_int64 * len(seq))(*[int(s) for s in seq])
+
+
+def _stream(stream):
+    if stream is None:
+        import torch
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    return ctypes.c_void_p(int(stream))
+
+
+def _workspace(nbytes, like):
+    import torch
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=like.device)
+
+
+def init(device=0):
+    check(lib().nbla_hip_init(int(device)))
+
+
+def cut_table(which):
+    out = (ctypes.c_uint32 * 277)()
+    check(lib().nbla_hip_cut_table(int(which), out))
+    return list(out)
+
+
+# ------------------------------------------------------------------ tensor helpers
+
+def fixed_point_quantize(x, sign=True, n=8, delta=2.0 ** -4, out=None, stream=None):
+    import torch
+    y = torch.empty_like(x) if out is None else out
+    check(lib().nbla_hip_fixed_point_quantize_f32(_p(x), _p(y), ctypes.c_size_t(x.numel()), int(sign), int(n),
+                                                  ctypes.c_float(delta), _stream(stream)))
+    return y
+
+
+def pow2_quantize(x, sign=True, with_zero=True, n=8, m=1, out=None, stream=None):
+    import torch
+    y = torch.empty_like(x) if out is None else out
+    check(lib().nbla_hip_pow2_quantize_f32(_p(x), _p(y), ctypes.c_size_t(x.numel()), int(sign), int(with_zero),
+                                           int(n), int(m), _stream(stream)))
+    return y
+
+
+def min_max_quantize(x, qr_min, qr_max, ql_min, ql_max, decay=0.999, x_min_max=False, ema=False, eps=0.01,
+                     out=None, workspace=None, stream=None):
+    """Updates qr_min / qr_max in place; returns (y, scale)."""
+    import torch
+    y = torch.empty_like(x) if out is None else out
+    scale = torch.empty_like(qr_min)
+    xs, qs = _shape(x.shape), _shape(qr_min.shape)
+    need = lib().nbla_hip_min_max_quantize_workspace_bytes(xs, x.dim(), qs)
+    ws = _workspace(need, x) if workspace is None else workspace
+    check(lib().nbla_hip_min_max_quantize_f32(_p(x), _p(y), xs, x.dim(), qs, _p(qr_min), _p(qr_max), _p(ql_min),
+                                              _p(ql_max), _p(scale), ctypes.c_float(decay), int(x_min_max), int(ema),
+                                              ctypes.c_float(eps), _p(ws), ctypes.c_size_t(ws.numel()),
+                                              _stream(stream)))
+    return y, scale
+
+
+def binarize_weights(W, K, N, transposed=False, quantize_zero_to=1.0, want_alpha=True, stream=None):
+    """Returns (Wb, alpha or None, bits[uint32 tensor], zero_count tensor)."""
+    import torch
+    Wb = torch.empty_like(W)
+    alpha = torch.empty(N, dtype=torch.float32, device=W.device) if want_alpha else None
+    bits = torch.empty(lib().nbla_hip_packed_bits_bytes(_i64(K), _i64(N)) // 4, dtype=torch.int32, device=W.device)
+    zc = torch.empty(1, dtype=torch.int32, device=W.device)
+    ws = _workspace(lib().nbla_hip_binarize_workspace_bytes(_i64(K), _i64(N)), W)
+    check(lib().nbla_hip_binarize_weights_f32(_p(W), _p(Wb), _p(alpha), _p(bits), _i64(K), _i64(N), int(transposed),
+                                              ctypes.c_float(quantize_zero_to), _p(zc), _p(ws),
+                                              ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return Wb, alpha, bits, zc
+
+
+def split_bf16x3(x, M, K, ldx=None, stream=None):
+    import torch
+    out = torch.empty(lib().nbla_hip_split_operand_bytes(_i64(M), _i64(K)) // 2, dtype=torch.int16, device=x.device)
+    check(lib().nbla_hip_split_bf16x3_f32(_p(x), _i64(K if ldx is None else ldx), _p(out), _i64(M), _i64(K),
+                                          _stream(stream)))
+    return out
+
+
+def gemm_bits(xsplit, bits, alpha, bias, M, K, N, out=None, inner=1, outer_stride=None, n_stride=1, stream=None):
+    import torch
+    y = torch.empty((M, N), dtype=torch.float32, device=bits.device) if out is None else out
+    check(lib().nbla_hip_gemm_bits_f32(_p(xsplit), _p(bits), _p(alpha), _p(bias), _p(y), _i64(M), _i64(K), _i64(N),
+                                       _i64(inner), _i64(N if outer_stride is None else outer_stride), _i64(n_stride),
+                                       _stream(stream)))
+    return y
+
+
+def binary_affine_workspace(M, K, N, like):
+    return _workspace(lib().nbla_hip_binary_affine_workspace_bytes(_i64(M), _i64(K), _i64(N)), like)
+
+
+def binary_weight_affine(x, W, bias=None, quantize_zero_to=1.0, workspace=None, out=None, stream=None):
+    """x [M,K], W [K,N...] -> (y, Wb, alpha)."""
+    import torch
+    M, K = x.shape
+    N = W.numel() // K
+    Wb = torch.empty_like(W)
+    alpha = torch.empty(N, dtype=torch.float32, device=x.device)
+    y = torch.empty((M, N), dtype=torch.float32, device=x.device) if out is None else out
+    ws = binary_affine_workspace(M, K, N, x) if workspace is None else workspace
+    check(lib().nbla_hip_binary_weight_affine_f32(_p(x), _p(W), _p(Wb), _p(alpha), _p(bias), _p(y), _i64(M), _i64(K),
+                                                  _i64(N), ctypes.c_float(quantize_zero_to), _p(ws),
+                                                  ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return y, Wb, alpha
+
+
+def binary_connect_affine(x, W, bias=None, quantize_zero_to=1.0, workspace=None, out=None, stream=None):
+    """x [M,K], W [K,N...] -> (y, Wb)."""
+    import torch
+    M, K = x.shape
+    N = W.numel() // K
+    Wb = torch.empty_like(W)
+    y = torch.empty((M, N), dtype=torch.float32, device=x.device) if out is None else out
+    ws = binary_affine_workspace(M, K, N, x) if workspace is None else workspace
+    check(lib().nbla_hip_binary_connect_affine_f32(_p(x), _p(W), _p(Wb), _p(bias), _p(y), _i64(M), _i64(K), _i64(N),
+                                                   ctypes.c_float(quantize_zero_to), _p(ws),
+                                                   ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return y, Wb
+
+
+def affine(x, W, bias=None, out=None, stream=None):
+    import torch
+    M, K = x.shape
+    N = W.numel() // K
+    y = torch.empty((M, N), dtype=torch.float32, device=x.device) if out is None else out
+    check(lib().nbla_hip_affine_f32(_p(x), _p(W), _p(bias), _p(y), _i64(M), _i64(K), _i64(N), _stream(stream)))
+    return y

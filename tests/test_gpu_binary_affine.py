@@ -1,0 +1,187 @@
+"""BinaryWeightAffine / BinaryConnectAffine on the GPU against the CPU oracle.
+
+Bit-exact: Sign(W) (`Wb`) and the packed 1-bit operand.  At tolerance: alpha (rel 1e-6 against a float64
+mean; the reference's own fp32 summation order comes from Eigen and is unpinned) and y
+(max|y - y_ref| / max|y_ref| <= 1e-4 as the acceptance bar; the bf16x3 product is expected near 1e-6).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from nnabla_amd import kernels
+from util import bits_equal, first_mismatch, max_rel_err, to_np, unpack_bits
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-4         # north-star tolerance for GEMM outputs
+TIGHT = 5e-6       # what an fp32-faithful product should reach on these sizes
+
+
+def _dev(x, dev):
+    return torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+
+
+def _data(M, K, N, seed=313, wscale=0.02):
+    rng = np.random.RandomState(seed)
+    x = rng.randn(M, K).astype(np.float32)
+    W = (rng.randn(K, N) * wscale).astype(np.float32)
+    return x, W
+
+
+SHAPES = [(1, 32, 64), (2, 3, 4), (5, 17, 9), (8, 64, 64), (33, 100, 130), (64, 256, 256), (129, 96, 320),
+          (300, 1000, 257), (7, 4096, 70)]
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+def test_binarize_bits_and_alpha(dev, M, K, N):
+    _, W = _data(M, K, N)
+    W.ravel()[::7] = 0.0            # exact zeros take quantize_zero_to
+    W.ravel()[3::11] = -0.0
+    for q0 in (1.0, -1.0):
+        Wb, alpha, bits, zc = kernels.binarize_weights(_dev(W, dev), K, N, False, q0)
+        ref_Wb, ref_alpha = oracle.binary_weight_prepare(W, q0)
+        assert bits_equal(to_np(Wb), ref_Wb), first_mismatch(to_np(Wb), ref_Wb)
+        unpacked = unpack_bits(to_np(bits), K, N)
+        assert np.array_equal(unpacked, ref_Wb.astype(np.int8))
+        a64 = np.abs(W.astype(np.float64)).mean(0)
+        np.testing.assert_allclose(to_np(alpha), a64, rtol=2e-6, atol=1e-12)
+        np.testing.assert_allclose(ref_alpha, a64, rtol=2e-6, atol=1e-12)
+        assert int(to_np(zc)[0]) == int((W == 0).sum())
+
+
+@pytest.mark.parametrize("K,N", [(9, 6), (2304, 256), (75, 130)])
+def test_binarize_transposed_layout(dev, K, N):
+    """Convolution weights are stored [N(out channels), K]; bits must equal the [K, N] view's."""
+    rng = np.random.RandomState(1)
+    Wnk = (rng.randn(N, K) * 0.03).astype(np.float32)
+    Wnk.ravel()[::13] = 0.0
+    Wb, alpha, bits, zc = kernels.binarize_weights(_dev(Wnk, dev), K, N, True, 1.0)
+    ref_Wb = oracle.sign(Wnk, 1.0)
+    assert bits_equal(to_np(Wb), ref_Wb)
+    assert np.array_equal(unpack_bits(to_np(bits), K, N), ref_Wb.T.astype(np.int8))
+    np.testing.assert_allclose(to_np(alpha), np.abs(Wnk.astype(np.float64)).mean(1), rtol=2e-6)
+
+
+def test_split_is_exact(dev):
+    """hi + mid + lo == x exactly, in fragment order, zero padded."""
+    rng = np.random.RandomState(2)
+    M, K = 45, 70
+    x = (rng.randn(M, K) * np.exp(rng.randn(M, K) * 8)).astype(np.float32)
+    x[0, :6] = [0.0, -0.0, 1e-30, -3e38, 3.3e38, 1.0]
+    raw = to_np(kernels.split_bf16x3(_dev(x, dev), M, K)).view(np.uint16)
+    rb, kb = (M + 31) // 32, ((K + 31) // 32) * 2
+    frag = raw.reshape(rb, kb, 3, 64, 8).astype(np.uint32) << 16
+    planes = frag.view(np.float32)                       # [rb, kb, plane, lane, e]
+    total = planes[:, :, 0].astype(np.float64) + planes[:, :, 1] + planes[:, :, 2]
+    full = np.zeros((rb * 32, kb * 16), np.float64)
+    for lane in range(64):
+        for e in range(8):
+            full[(lane & 31)::32, ((lane >> 5) * 8 + e)::16] = total[:, :, lane, e]
+    assert np.array_equal(full[:M, :K], x.astype(np.float64))
+    assert not full[M:].any() and not full[:, K:].any()
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+@pytest.mark.parametrize("bias", [False, True])
+def test_binary_weight_affine_matches_oracle(dev, M, K, N, bias):
+    x, W = _data(M, K, N)
+    b = np.random.RandomState(9).randn(N).astype(np.float32) if bias else None
+    ref_y, ref_Wb, ref_alpha = oracle.binary_weight_affine(x, W, b, 1.0)
+    y, Wb, alpha = kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev), None if b is None else _dev(b, dev))
+    assert bits_equal(to_np(Wb), ref_Wb)
+    np.testing.assert_allclose(to_np(alpha), ref_alpha, rtol=2e-6)
+    y64 = x.astype(np.float64) @ (ref_Wb.astype(np.float64) * np.abs(W.astype(np.float64)).mean(0))
+    if b is not None:
+        y64 = y64 + b
+    assert max_rel_err(to_np(y), ref_y) <= TOL
+    assert max_rel_err(to_np(y), y64) <= TIGHT
+    assert max_rel_err(ref_y, y64) <= TIGHT
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+def test_binary_connect_affine_matches_oracle(dev, M, K, N):
+    x, W = _data(M, K, N, seed=7)
+    b = np.random.RandomState(3).randn(N).astype(np.float32)
+    ref_y, ref_Wb = oracle.binary_connect_affine(x, W, b, 1.0)
+    y, Wb = kernels.binary_connect_affine(_dev(x, dev), _dev(W, dev), _dev(b, dev))
+    assert bits_equal(to_np(Wb), ref_Wb)
+    y64 = x.astype(np.float64) @ ref_Wb.astype(np.float64) + b
+    assert max_rel_err(to_np(y), ref_y) <= TOL
+    assert max_rel_err(to_np(y), y64) <= TIGHT
+
+
+@pytest.mark.parametrize("q0", [0.0, 0.5, -1.0, 1.0])
+def test_quantize_zero_to_with_exact_zero_weights(dev, q0):
+    """Sign(0) = quantize_zero_to (test_binary_weight_affine.py:72 covers 0, -1, 1)."""
+    x, W = _data(40, 96, 72, seed=11)
+    W.ravel()[::5] = 0.0
+    ref_y, ref_Wb, ref_alpha = oracle.binary_weight_affine(x, W, None, q0)
+    y, Wb, alpha = kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev), None, q0)
+    assert bits_equal(to_np(Wb), ref_Wb)
+    assert max_rel_err(to_np(y), ref_y) <= TIGHT * 4
+    ref_y, ref_Wb = oracle.binary_connect_affine(x, W, None, q0)
+    y, Wb = kernels.binary_connect_affine(_dev(x, dev), _dev(W, dev), None, q0)
+    assert bits_equal(to_np(Wb), ref_Wb)
+    assert max_rel_err(to_np(y), ref_y) <= TIGHT * 4
+
+
+def test_plain_affine_f32(dev):
+    for (M, K, N) in [(2, 3, 4), (70, 130, 200), (256, 512, 384)]:
+        x, W = _data(M, K, N, seed=5, wscale=1.0)
+        b = np.random.RandomState(4).randn(N).astype(np.float32)
+        y = to_np(kernels.affine(_dev(x, dev), _dev(W, dev), _dev(b, dev)))
+        y64 = x.astype(np.float64) @ W.astype(np.float64) + b
+        assert max_rel_err(y, y64) <= TIGHT
+        assert max_rel_err(oracle.affine(x, W, b), y64) <= TIGHT
+
+
+@pytest.mark.parametrize("M", [1, 8, 64])
+def test_config3_full_width_small_m_vs_oracle(dev, M):
+    """BASELINE config 3 at K=4096, N=11008 for the M the CPU oracle finishes in seconds."""
+    rng = np.random.default_rng(313)
+    x = rng.standard_normal((M, 4096), dtype=np.float32)
+    W = rng.standard_normal((4096, 11008), dtype=np.float32) * np.float32(0.02)
+    ref_y, ref_Wb, ref_alpha = oracle.binary_weight_affine(x, W, None, 1.0)
+    y, Wb, alpha = kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev))
+    assert bits_equal(to_np(Wb), ref_Wb)
+    np.testing.assert_allclose(to_np(alpha), ref_alpha, rtol=2e-6)
+    assert max_rel_err(to_np(y), ref_y) <= TOL
+    yc, Wbc = kernels.binary_connect_affine(_dev(x, dev), _dev(W, dev))
+    ref_yc, _ = oracle.binary_connect_affine(x, W, None, 1.0)
+    assert bits_equal(to_np(Wbc), ref_Wb)
+    assert max_rel_err(to_np(yc), ref_yc) <= TOL
+
+
+@pytest.mark.parametrize("M", [512, 4096])
+def test_config3_full_size_properties(dev, M):
+    """At sizes the oracle cannot finish quickly: float64 dot products on sampled rows/columns,
+    linearity in x, and consistency between BinaryWeight and BinaryConnect (y_bw = y_bc * alpha)."""
+    rng = np.random.default_rng(7)
+    K, N = 4096, 11008
+    x = rng.standard_normal((M, K), dtype=np.float32)
+    W = rng.standard_normal((K, N), dtype=np.float32) * np.float32(0.02)
+    xd, Wd = _dev(x, dev), _dev(W, dev)
+    y, Wb, alpha = kernels.binary_weight_affine(xd, Wd)
+    yc, _ = kernels.binary_connect_affine(xd, Wd)
+    y, yc, alpha = to_np(y), to_np(yc), to_np(alpha)
+    assert bits_equal(to_np(Wb), oracle.sign(W, 1.0))
+    rows = rng.choice(M, 24, replace=False)
+    cols = rng.choice(N, 96, replace=False)
+    sgn = np.sign(W[:, cols]).astype(np.float64)
+    ref_c = x[rows].astype(np.float64) @ sgn
+    a64 = np.abs(W[:, cols].astype(np.float64)).mean(0)
+    assert np.abs(yc[np.ix_(rows, cols)] - ref_c).max() / np.abs(ref_c).max() <= TIGHT
+    assert np.abs(y[np.ix_(rows, cols)] - ref_c * a64).max() / np.abs(ref_c * a64).max() <= TIGHT
+    np.testing.assert_allclose(y, yc * alpha[None, :], rtol=1e-6, atol=1e-7)
+    # linearity: f(2x) == 2 f(x) exactly (power-of-two scaling commutes with every rounding)
+    y2, _, _ = kernels.binary_weight_affine(xd * 2, Wd)
+    assert bits_equal(to_np(y2), y * 2)
+
+
+def test_workspace_too_small_is_reported(dev):
+    x, W = _data(4, 64, 64)
+    ws = torch.empty(256, dtype=torch.uint8, device=dev)
+    with pytest.raises(kernels.KernelError) as ei:
+        kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev), workspace=ws)
+    assert ei.value.code == kernels.ERR_MEMORY

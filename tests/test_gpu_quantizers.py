@@ -1,0 +1,224 @@
+"""Bit-exact parity of the HIP quantizers (through the C-ABI) with the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from nnabla_amd import kernels
+from util import bits_equal, first_mismatch, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(x, dev):
+    return torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+
+
+# ------------------------------------------------------------- FixedPointQuantize
+
+FPQ_CASES = [
+    (True, 8, 2.0 ** -4), (False, 8, 2.0 ** -4), (True, 3, 0.1), (False, 5, 0.3), (True, 16, 1e-3),
+    (True, 2, 1.0), (False, 1, 0.5), (True, 12, 3.0), (True, 8, 2.0 ** -20), (True, 30, 2.0 ** -12),
+]
+
+
+@pytest.mark.parametrize("sign,n,delta", FPQ_CASES)
+def test_fixed_point_quantize_matches_oracle(dev, sign, n, delta):
+    rng = np.random.RandomState(313)
+    x = (rng.randn(257, 1031) * 2).astype(np.float32)
+    # values on and next to the rounding ties, the clip bounds, zeros, tiny negatives
+    nn = n - 1 if sign else n
+    mx = np.float32((2.0 ** nn - 1) * np.float32(delta))
+    ties = (np.arange(-40, 40, dtype=np.float32) + 0.5) * np.float32(delta)
+    special = np.concatenate([
+        ties, np.nextafter(ties, np.float32(np.inf)), np.nextafter(ties, np.float32(-np.inf)),
+        np.array([0.0, -0.0, 1e-30, -1e-30, 1e-45, -1e-45, mx, -mx, np.inf, -np.inf], np.float32),
+        np.nextafter(np.array([mx, -mx, mx, -mx], np.float32), np.array([np.inf, np.inf, -np.inf, -np.inf], np.float32)),
+    ]).astype(np.float32)
+    x.ravel()[:special.size] = special
+    ref = oracle.fixed_point_quantize(x, sign, n, delta)
+    y = to_np(kernels.fixed_point_quantize(_dev(x, dev), sign, n, delta))
+    assert bits_equal(y, ref), first_mismatch(y, ref)
+
+
+def test_fixed_point_quantize_config1_full_size(dev):
+    """BASELINE config 1: [256, 65536] ~ N(0, 2^2), sign, n=8, delta=2^-4, bit-exact."""
+    rng = np.random.default_rng(313)
+    x = (rng.standard_normal((256, 65536), dtype=np.float32) * np.float32(2.0))
+    ref = oracle.fixed_point_quantize(x, True, 8, 2.0 ** -4)
+    y = to_np(kernels.fixed_point_quantize(_dev(x, dev), True, 8, 2.0 ** -4))
+    assert bits_equal(y, ref), first_mismatch(y, ref)
+    # size-independent properties: idempotent (up to the sign of zero: the reference maps -0.0 to +0.0),
+    # on the delta grid, within bounds
+    yy = to_np(kernels.fixed_point_quantize(_dev(y, dev), True, 8, 2.0 ** -4))
+    assert np.array_equal(yy, y) and not np.signbit(yy[y == 0]).any() and np.signbit(y[(x < 0) & (y == 0)]).all()
+    assert np.all(np.abs(y) <= 7.9375) and np.all(y * 16 == np.round(y * 16))
+
+
+@pytest.mark.parametrize("size", [0, 1, 3, 4, 5, 1023, 1024, 1025, 4099])
+def test_fixed_point_quantize_ragged_and_unaligned(dev, size):
+    rng = np.random.RandomState(size + 1)
+    x = (rng.randn(size + 1) * 3).astype(np.float32)
+    xd = _dev(x, dev)
+    for off in (0, 1):  # off=1: pointer not 16-byte aligned -> scalar path
+        xs = xd[off:off + size]
+        y = torch.full((size + 2,), 7.0, device=dev)
+        kernels.fixed_point_quantize(xs, True, 8, 0.0625, out=y[off:off + size])
+        ref = oracle.fixed_point_quantize(x[off:off + size], True, 8, 0.0625)
+        got = to_np(y)
+        assert bits_equal(got[off:off + size], ref)
+        assert got[off + size] == 7.0 and (off == 0 or got[0] == 7.0)  # no write outside
+
+
+def test_fixed_point_quantize_in_place_and_errors(dev):
+    x = _dev((np.random.RandomState(1).randn(5000) * 2).astype(np.float32), dev)
+    ref = oracle.fixed_point_quantize(to_np(x), True, 8, 0.0625)
+    kernels.fixed_point_quantize(x, True, 8, 0.0625, out=x)
+    assert bits_equal(to_np(x), ref)
+    for sign, n, delta in [(True, 0, 0.1), (True, 8, 0.0), (True, 8, -1.0), (True, 1, 0.1)]:
+        with pytest.raises(kernels.KernelError) as ei:
+            kernels.fixed_point_quantize(x, sign, n, delta)
+        assert ei.value.code == kernels.ERR_VALUE
+        with pytest.raises(oracle.OracleError):
+            oracle.fixed_point_quantize(to_np(x), sign, n, delta)
+
+
+# ------------------------------------------------------------------ Pow2Quantize
+
+POW2_CASES = [
+    (True, True, 4, 1), (True, True, 8, 1), (True, False, 3, 0), (False, True, 4, 2), (False, False, 3, -2),
+    (True, True, 3, 0), (True, True, 6, 10), (False, False, 7, 100), (True, True, 9, 1), (False, False, 8, 120),
+]
+
+
+def _pow2_inputs(rng, shape, scale):
+    x = (rng.randn(*shape) * scale).astype(np.float32)
+    # every binade boundary region sqrt(2)*2^k (+-4 ulp), exact powers of two, zeros, subnormals, inf, nan
+    ks = np.arange(-149, 128)
+    cuts = (np.float64(2.0) ** (ks + 0.5))
+    cuts = cuts[(cuts > 1e-45) & (cuts < 3e38)].astype(np.float32)
+    near = []
+    for d in range(-4, 5):
+        near.append((cuts.view(np.uint32).astype(np.int64) + d).astype(np.uint32).view(np.float32))
+    pows = (np.float64(2.0) ** np.arange(-149, 128)).astype(np.float32)
+    special = np.concatenate(near + [pows, -pows, np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45,
+                                                             3.4e38, -3.4e38], np.float32)])
+    special = np.concatenate([special, -special]).astype(np.float32)
+    flat = x.ravel()
+    flat[:special.size] = special
+    return x
+
+
+@pytest.mark.parametrize("sign,with_zero,n,m", POW2_CASES)
+def test_pow2_quantize_matches_oracle(dev, sign, with_zero, n, m):
+    rng = np.random.RandomState(313)
+    x = _pow2_inputs(rng, (300, 1031), 2.0 ** (m - 2))
+    ref = oracle.pow2_quantize(x, sign, with_zero, n, m)
+    y = to_np(kernels.pow2_quantize(_dev(x, dev), sign, with_zero, n, m))
+    assert bits_equal(y, ref), first_mismatch(y, ref)
+
+
+def test_pow2_quantize_config2_weights(dev):
+    """BASELINE config 2b: [512,512,3,3] ~ N(0, 0.05^2), sign, with_zero, n=4, m=1."""
+    rng = np.random.default_rng(313)
+    w = (rng.standard_normal((512, 512, 3, 3), dtype=np.float32) * np.float32(0.05))
+    ref = oracle.pow2_quantize(w, True, True, 4, 1)
+    y = to_np(kernels.pow2_quantize(_dev(w, dev), True, True, 4, 1))
+    assert bits_equal(y, ref), first_mismatch(y, ref)
+    assert set(np.unique(np.abs(y)).tolist()) <= {0.0, 0.25, 0.5, 1.0, 2.0}
+
+
+def test_pow2_quantize_whole_binades_bruteforce(dev):
+    """Every fp32 value of three binades (2^23 patterns each) against the host libm path."""
+    for expo in (126, 127, 100):  # [0.5,1), [1,2), [2^-27, 2^-26)
+        u = (np.arange(1 << 23, dtype=np.uint32) | np.uint32(expo << 23))
+        x = u.view(np.float32)
+        ref = oracle.pow2_quantize(x, True, False, 8, 1)
+        y = to_np(kernels.pow2_quantize(_dev(x, dev), True, False, 8, 1))
+        assert bits_equal(y, ref), first_mismatch(y, ref)
+
+
+def test_pow2_quantize_errors(dev):
+    x = _dev(np.ones(16, np.float32), dev)
+    for sign, wz, n, m in [(True, True, 0, 1), (True, True, 2, 1), (True, False, 1, 1), (False, True, 1, 0)]:
+        with pytest.raises(kernels.KernelError) as ei:
+            kernels.pow2_quantize(x, sign, wz, n, m)
+        assert ei.value.code == kernels.ERR_VALUE
+        with pytest.raises(oracle.OracleError):
+            oracle.pow2_quantize(np.ones(16, np.float32), sign, wz, n, m)
+
+
+# ---------------------------------------------------------------- MinMaxQuantize
+
+def _mmq_both(dev, x, qshape, qr_min, qr_max, ql_min, ql_max, decay, x_min_max, ema, eps=0.01):
+    qmn = np.full(qshape, qr_min, np.float32) if np.isscalar(qr_min) else qr_min.astype(np.float32)
+    qmx = np.full(qshape, qr_max, np.float32) if np.isscalar(qr_max) else qr_max.astype(np.float32)
+    lmn = np.full(qshape, ql_min, np.float32)
+    lmx = np.full(qshape, ql_max, np.float32)
+    ref_y, ref_mn, ref_mx, ref_sc = oracle.min_max_quantize(x, qmn, qmx, lmn, lmx, decay, x_min_max, ema, eps)
+    dmn, dmx = _dev(qmn, dev), _dev(qmx, dev)
+    y, sc = kernels.min_max_quantize(_dev(x, dev), dmn, dmx, _dev(lmn, dev), _dev(lmx, dev), decay, x_min_max, ema,
+                                     eps)
+    return (to_np(y), to_np(dmn), to_np(dmx), to_np(sc)), (ref_y, ref_mn, ref_mx, ref_sc)
+
+
+MMQ_SHAPES = [
+    ((4, 8, 16, 16), (1, 1, 1, 1)), ((4, 8, 16, 16), (1, 8, 1, 1)), ((16, 8, 4, 4), (16, 1, 1, 1)),
+    ((6, 10), (1, 10)), ((6, 10), (6, 1)), ((3, 5, 7), (1, 5, 1)), ((2, 3, 4), (2, 3, 4)), ((5, 7, 9), (1, 1, 1)),
+    ((2, 64, 33, 32), (1, 64, 1, 1)), ((1, 1, 3000), (1, 1, 1)),
+]
+
+
+@pytest.mark.parametrize("xshape,qshape", MMQ_SHAPES)
+@pytest.mark.parametrize("x_min_max,ema", [(True, True), (True, False), (False, False), (False, True)])
+def test_min_max_quantize_matches_oracle(dev, xshape, qshape, x_min_max, ema):
+    rng = np.random.RandomState(313)
+    x = (rng.randn(*xshape) * 3).astype(np.float32)
+    got, ref = _mmq_both(dev, x, qshape, -6.0, 6.0, 0.0, 255.0, 0.999, x_min_max, ema)
+    for g, r, name in zip(got, ref, ("y", "qr_min", "qr_max", "scale")):
+        assert bits_equal(g, r), "%s: %s" % (name, first_mismatch(g, r))
+
+
+def test_min_max_quantize_signed_zero_and_limits(dev):
+    """The first of several equal extrema wins in the reference's scan (only visible for +0/-0);
+    values beyond +-1e8 and NaNs are ignored by Min/Max."""
+    x = np.abs(np.random.RandomState(0).randn(4, 8, 16, 16)).astype(np.float32) + 1.0
+    x[1, 2, 3, 4] = 0.0
+    x[0, 5, 0, 0] = -0.0      # earlier in scan order than the +0.0 above
+    x[3, 7, 1, 1] = 5e8       # ignored by Max (init -1e8, but > works) / beyond Min's 1e8 start
+    x[2, 0, 0, 0] = np.nan
+    for qshape in [(1, 1, 1, 1), (1, 8, 1, 1), (4, 1, 1, 1)]:
+        got, ref = _mmq_both(dev, x, qshape, 0.0, 0.0, 0.0, 255.0, 0.5, True, False)
+        for g, r, name in zip(got[1:], ref[1:], ("qr_min", "qr_max", "scale")):
+            assert bits_equal(g, r), "%s %s: %s" % (qshape, name, first_mismatch(g, r))
+    big = np.full((2, 3000), 3e8, np.float32)
+    got, ref = _mmq_both(dev, big, (1, 1), -1.0, 1.0, 0.0, 255.0, 0.9, True, False)
+    assert bits_equal(got[1], ref[1]) and bits_equal(got[2], ref[2]) and bits_equal(got[0], ref[0])
+
+
+def test_min_max_quantize_eps_nudge_and_zero_point_clamps(dev):
+    rng = np.random.RandomState(5)
+    x = rng.randn(8, 400).astype(np.float32)
+    for qr_min, qr_max in [(1.0, 1.001), (0.5, 0.4), (-3.0, -1.0), (2.0, 9.0), (-1.0, 1.0), (-0.37, 0.91)]:
+        got, ref = _mmq_both(dev, x, (1, 1), qr_min, qr_max, 0.0, 255.0, 0.999, False, False)
+        for g, r, name in zip(got, ref, ("y", "qr_min", "qr_max", "scale")):
+            assert bits_equal(g, r), "%s: %s" % (name, first_mismatch(g, r))
+    got, ref = _mmq_both(dev, x, (1, 1), -1.0, 1.0, -128.0, 127.0, 0.999, True, True)
+    assert bits_equal(got[0], ref[0])
+
+
+def test_min_max_quantize_config2_full_size(dev):
+    """BASELINE config 2a: post-ReLU activations [64,256,56,56], per-tensor, ema, decay .999."""
+    rng = np.random.default_rng(313)
+    x = np.abs(rng.standard_normal((64, 256, 56, 56), dtype=np.float32))
+    got, ref = _mmq_both(dev, x, (1, 1, 1, 1), -6.0, 6.0, 0.0, 255.0, 0.999, True, True)
+    for g, r, name in zip(got, ref, ("y", "qr_min", "qr_max", "scale")):
+        assert bits_equal(g, r), "%s: %s" % (name, first_mismatch(g, r))
+
+
+def test_min_max_quantize_shape_errors(dev):
+    x = _dev(np.zeros((4, 8, 2, 2), np.float32), dev)
+    q = _dev(np.zeros((1, 4, 1, 1), np.float32), dev)
+    with pytest.raises(kernels.KernelError) as ei:
+        kernels.min_max_quantize(x, q, q.clone(), q.clone(), q.clone())
+    assert ei.value.code == kernels.ERR_VALUE

@@ -1,0 +1,58 @@
+"""Shared helpers of the parity tests."""
+import numpy as np
+
+
+def bits_equal(a, b):
+    """Bit-for-bit equality of two fp32 arrays (distinguishes -0.0 from +0.0; NaNs equal when both NaN)."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    if a.shape != b.shape:
+        return False
+    ai, bi = a.view(np.uint32), b.view(np.uint32)
+    same = ai == bi
+    both_nan = np.isnan(a) & np.isnan(b)
+    return bool(np.all(same | both_nan))
+
+
+def first_mismatch(a, b):
+    a = np.ascontiguousarray(a, dtype=np.float32).ravel()
+    b = np.ascontiguousarray(b, dtype=np.float32).ravel()
+    bad = np.nonzero((a.view(np.uint32) != b.view(np.uint32)) & ~(np.isnan(a) & np.isnan(b)))[0]
+    if bad.size == 0:
+        return "identical"
+    i = int(bad[0])
+    return "%d mismatches, first at %d: %r (0x%08x) vs %r (0x%08x)" % (
+        bad.size, i, a[i], a.view(np.uint32)[i], b[i], b.view(np.uint32)[i])
+
+
+def max_rel_err(y, ref):
+    """max |y - ref| / max |ref|: the GEMM/conv acceptance metric (<= 1e-4)."""
+    ref = np.asarray(ref, dtype=np.float64)
+    y = np.asarray(y, dtype=np.float64)
+    denom = np.abs(ref).max()
+    return float(np.abs(y - ref).max() / (denom if denom > 0 else 1.0))
+
+
+def to_np(t):
+    return t.detach().cpu().numpy()
+
+
+def unpack_bits(bits_words, K, N):
+    """Packed 1-bit GEMM operand (uint32 words, [k_tiles][col_groups][64]) -> int8 [K, N] of +-1."""
+    w = np.ascontiguousarray(bits_words).view(np.uint32)
+    k_tiles = (K + 31) // 32
+    col_groups = (N + 63) // 64
+    w = w.reshape(k_tiles, col_groups, 64)
+    out = np.ones((k_tiles * 32, col_groups * 64), np.int8)
+    lane = np.arange(64)
+    for f in range(2):
+        for s in range(2):
+            for e in range(8):
+                p = 4 * (2 * f + s) + (e >> 1)
+                pos = 31 - p if (e & 1) else 15 - p
+                bit = (w >> np.uint32(pos)) & np.uint32(1)  # [kt, cg, lane]
+                k_off = s * 16 + (lane >> 5) * 8 + e        # per lane
+                n_off = f * 32 + (lane & 31)
+                for l in range(64):
+                    out[k_off[l]::32, n_off[l]::64][:k_tiles, :col_groups] = np.where(bit[:, :, l] == 1, -1, 1)
+    return out[:K, :N]
