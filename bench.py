@@ -1,0 +1,203 @@
+#!/usr/bin/env python
+"""Benchmark of the quantization hot path on one MI355X.
+
+One "step" is one BinaryWeightAffine forward at the headline shape (x [4096, 4096], W [4096, 11008]):
+sign/alpha/pack of W, bf16x3 split of x and the 1-bit-weight MFMA product, launched through the C-ABI on
+torch's current HIP stream with all inputs already resident in HBM.  The JSON line also carries the quantizer
+kernels' HBM figures (`quantizers`) and the small-M sweep (`sweep`).
+
+  value      whole-step fp32-equivalent TFLOP/s  (2*M*K*N / step time)
+  roofline   the dominant kernel (the MFMA product), timed with HIP events inside the timed steps
+  cpu_baseline  the CPU oracle (a port of nnabla's CPU arithmetic, 1 core) on a bounded row sample
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix
+PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X dense bf16 matrix
+PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
+
+
+def _events(n):
+    import torch
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def bench_binary_weight_affine(M, K, N, steps, warmup, dev):
+    import torch
+    from nnabla_amd import kernels as k
+    g = torch.Generator(device="cpu").manual_seed(313)
+    x = torch.randn(M, K, generator=g).to(dev)
+    W = (torch.randn(K, N, generator=g) * 0.02).to(dev)
+    Wb = torch.empty_like(W)
+    alpha = torch.empty(N, device=dev)
+    y = torch.empty(M, N, device=dev)
+    L = k.lib()
+    bits = torch.empty(L.nbla_hip_packed_bits_bytes(k._i64(K), k._i64(N)), dtype=torch.uint8, device=dev)
+    xs = torch.empty(L.nbla_hip_split_operand_bytes(k._i64(M), k._i64(K)), dtype=torch.uint8, device=dev)
+    pws = torch.empty(max(256, L.nbla_hip_binarize_workspace_bytes(k._i64(K), k._i64(N))), dtype=torch.uint8,
+                      device=dev)
+    st = k._stream(None)
+    import ctypes
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        k.check(L.nbla_hip_binarize_weights_f32(k._p(W), k._p(Wb), k._p(alpha), k._p(bits), k._i64(K), k._i64(N), 0,
+                                                ctypes.c_float(1.0), None, k._p(pws), ctypes.c_size_t(pws.numel()),
+                                                st))
+        if ev:
+            ev[1].record()
+        k.check(L.nbla_hip_split_bf16x3_f32(k._p(x), k._i64(K), k._p(xs), k._i64(M), k._i64(K), st))
+        if ev:
+            ev[2].record()
+        k.check(L.nbla_hip_gemm_bits_f32(k._p(xs), k._p(bits), k._p(alpha), None, k._p(y), k._i64(M), k._i64(K),
+                                         k._i64(N), k._i64(1), k._i64(N), k._i64(1), st))
+        if ev:
+            ev[3].record()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    evs = [_events(4) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(evs[i])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    prep = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
+    split = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+    gemm = sum(e[2].elapsed_time(e[3]) for e in evs) / steps
+    return {"ms_per_step": wall * 1e3 / steps, "prepare_ms": prep, "split_ms": split, "gemm_ms": gemm,
+            "flop": 2.0 * M * K * N}
+
+
+def time_kernel(fn, iters, warmup=3):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = _events(2)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def bench_quantizers(dev, iters):
+    import torch
+    from nnabla_amd import kernels as k
+    out = {}
+    g = torch.Generator(device="cpu").manual_seed(313)
+    x = (torch.randn(256, 65536, generator=g) * 2).to(dev)
+    y = torch.empty_like(x)
+    ms = time_kernel(lambda: k.fixed_point_quantize(x, True, 8, 2.0 ** -4, out=y), iters)
+    nbytes = 8.0 * x.numel()
+    out["fixed_point_quantize[256,65536]"] = {"ms": ms, "bytes": nbytes, "GBs": nbytes / ms / 1e6,
+                                              "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    ms = time_kernel(lambda: k.pow2_quantize(x, True, True, 4, 1, out=y), iters)
+    out["pow2_quantize[256,65536]"] = {"ms": ms, "bytes": nbytes, "GBs": nbytes / ms / 1e6,
+                                       "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    w = (torch.randn(512, 512, 3, 3, generator=g) * 0.05).to(dev)
+    wq = torch.empty_like(w)
+    ms = time_kernel(lambda: k.pow2_quantize(w, True, True, 4, 1, out=wq), iters)
+    nb = 8.0 * w.numel()
+    out["pow2_quantize[512,512,3,3]"] = {"ms": ms, "bytes": nb, "GBs": nb / ms / 1e6,
+                                         "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
+    del x, y
+    a = torch.randn(64, 256, 56, 56, generator=g).abs_().to(dev)
+    ya = torch.empty_like(a)
+    q = lambda v: torch.full((1, 1, 1, 1), v, device=dev)
+    qmn, qmx, lmn, lmx = q(-6.0), q(6.0), q(0.0), q(255.0)
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+    for name, xmm, bpe in (("min_max_quantize[64,256,56,56] x_min_max", True, 12.0),
+                           ("min_max_quantize[64,256,56,56] fixed range", False, 8.0)):
+        ms = time_kernel(lambda: k.min_max_quantize(a, qmn, qmx, lmn, lmx, 0.999, xmm, True, 0.01, out=ya,
+                                                    workspace=ws), iters)
+        nb = bpe * a.numel()
+        out[name] = {"ms": ms, "bytes": nb, "GBs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
+    return out
+
+
+def cpu_baseline(K, N, rows):
+    """The CPU oracle (port of the reference's CPU arithmetic, single thread) on `rows` rows of the workload."""
+    import numpy as np
+    import oracle
+    rng = np.random.default_rng(313)
+    x = rng.standard_normal((rows, K), dtype=np.float32)
+    W = rng.standard_normal((K, N), dtype=np.float32) * np.float32(0.02)
+    oracle.binary_weight_affine(x[:4], W[:, :64].copy(), None, 1.0)  # load the library
+    t0 = time.perf_counter()
+    oracle.binary_weight_affine(x, W, None, 1.0)
+    dt = time.perf_counter() - t0
+    return {"value": 2.0 * rows * K * N / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": "BinaryWeightAffine forward (sign/alpha passes over the full W + fp32 GEMM) on %d of 4096 "
+                      "rows of x, K=%d, N=%d, %.1f s" % (rows, K, N, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-rows", type=int, default=2048)
+    ap.add_argument("--section", choices=("all", "headline", "quantizers"), default="all",
+                    help="headline: only the timed BinaryWeightAffine steps (what the rocprofv3 summaries profile); "
+                         "quantizers: headline plus the quantizer kernels")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
+    import torch
+    from nnabla_amd import kernels
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    kernels.init(0)
+
+    M, K, N = 4096, 4096, 11008
+    r = bench_binary_weight_affine(M, K, N, args.steps, args.warmup, dev)
+    tflops = r["flop"] / (r["ms_per_step"] * 1e-3) / 1e12
+    gemm_tflops = r["flop"] / (r["gemm_ms"] * 1e-3) / 1e12
+    sweep = {}
+    for m in ((1, 8, 64, 512) if args.section == "all" else ()):
+        s = bench_binary_weight_affine(m, K, N, max(5, args.steps // 2), 2, dev)
+        packed_bytes = K * N / 8 + 6.0 * m * K + 4.0 * m * N + 4.0 * N
+        sweep["M=%d" % m] = {"ms_per_step": s["ms_per_step"], "gemm_ms": s["gemm_ms"], "prepare_ms": s["prepare_ms"],
+                             "gemm_TFLOPs": s["flop"] / s["gemm_ms"] / 1e9,
+                             "gemm_weight_GBs": packed_bytes / s["gemm_ms"] / 1e6}
+    quant = bench_quantizers(dev, max(10, args.steps)) if args.section != "headline" else {}
+    line = {
+        "metric": "binary-weight affine TFLOP/s + quantizer GB/s, % of MI355X roofline",
+        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 (bf16x3 MFMA operands, f32 accumulate)", "data": "synthetic",
+        "config": {"workload": "BinaryWeightAffine forward, x [4096,4096] ~ N(0,1), W [4096,11008] ~ N(0,0.02^2), "
+                               "quantize_zero_to=1, no bias; whole forward = sign/alpha/pack + split + MFMA product",
+                   "M": M, "K": K, "N": N},
+        "roofline": {"bound": "mfma", "achieved": gemm_tflops, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": gemm_tflops / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
+                     "kernel": "gemm_bits_kernel<256,256,4,2>", "kernel_ms": r["gemm_ms"],
+                     "note": "fp32-equivalent flops 2*M*K*N against the fp32 MFMA peak; the kernel issues 3x that "
+                             "in bf16 MFMA", "bf16_issue_frac": 3 * gemm_tflops / PEAK_BF16_MFMA_TFLOPS},
+        "step_breakdown_ms": {"prepare": r["prepare_ms"], "split": r["split_ms"], "gemm": r["gemm_ms"]},
+        "sweep": sweep,
+        "quantizers": quant,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(K, N, args.cpu_rows)
+    else:
+        line["cpu_baseline"] = None
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
