@@ -185,6 +185,47 @@ int nbla_hip_affine_f32(const float *x, const float *w, const float *bias,
                         float *y, int64_t M, int64_t K, int64_t N,
                         void *stream);
 
+/* ------------------------------------------------------ binary convolutions */
+
+/* Output spatial shape (i + 2p - (d(k-1)+1)) / s + 1 per dimension, as
+ * Convolution<T>::setup_impl, src/nbla/function/generic/convolution.cpp:91-104.
+ * NBLA_HIP_ERR_VALUE for a non-positive output size (the NBLA_CHECK at :99-103). */
+int nbla_hip_convolution_output_shape(int nd, const int64_t *in_sp,
+                                      const int64_t *kernel, const int64_t *pad,
+                                      const int64_t *stride,
+                                      const int64_t *dilation, int64_t *out_sp);
+
+size_t nbla_hip_binary_convolution_workspace_bytes(
+    int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
+    const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+    const int64_t *dilation, int64_t group, float quantize_zero_to);
+
+/* BinaryWeightConvolution forward, channel-first, nd = 1..3 spatial dimensions:
+ *   x [outer, C, in_sp...], W [O, C/group, kernel...] -> Wb (same shape as W),
+ *   alpha [O], y [outer, O, out_sp...]; bias [O] may be NULL.
+ * Replaces BinaryWeightConvolution<float>::forward_impl,
+ * src/nbla/function/generic/binary_weight_convolution.cpp:73-117 (alpha per
+ * output channel with the rounded reciprocal of col_w, :66) and the im2col +
+ * per-sample Eigen product of convolution.cpp:161-197 / unfold_to_patches.cpp.
+ * Argument errors as convolution.cpp:61-103.  Synchronises once when
+ * quantize_zero_to is neither +1 nor -1 (see nbla_hip_binary_weight_affine_f32). */
+int nbla_hip_binary_weight_convolution_f32(
+    const float *x, const float *W, float *Wb, float *alpha, const float *bias,
+    float *y, int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
+    const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+    const int64_t *dilation, int64_t group, float quantize_zero_to,
+    void *workspace, size_t workspace_bytes, void *stream);
+
+/* BinaryConnectConvolution forward (no alpha).  Replaces
+ * BinaryConnectConvolution<float>::forward_impl,
+ * src/nbla/function/generic/binary_connect_convolution.cpp:68-80. */
+int nbla_hip_binary_connect_convolution_f32(
+    const float *x, const float *W, float *Wb, const float *bias, float *y,
+    int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
+    const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+    const int64_t *dilation, int64_t group, float quantize_zero_to,
+    void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -2,12 +2,9 @@
 // preparation, activation split and the bit-weight product chained on one stream.
 #include "common.hpp"
 #include "gemm_layout.hpp"
+#include "internal.hpp"
 
 namespace nbla_hip {
-
-int launch_gemm_f32(const float *x, const float *w, const float *colscale, const float *bias, float *y, int64_t M,
-                    int64_t K, int64_t N, hipStream_t stream);
-
 namespace {
 
 struct AffineWorkspace {

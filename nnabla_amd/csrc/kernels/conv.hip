@@ -1,0 +1,308 @@
+// BinaryWeightConvolution / BinaryConnectConvolution forwards (channel-first, up
+// to three spatial dimensions, groups): the convolution is the product
+//   y'[pixel, o] = sum_k col[pixel, k] * Wb[o, k],   pixel = (sample, out position), k = (c, kernel tap)
+// The unfolded activations are never materialised in fp32: one kernel gathers
+// them straight into the bf16x3 fragment-ordered operand of the bit-weight MFMA
+// product, whose epilogue scatters into the [sample, O, out position] layout.
+#include "common.hpp"
+#include "gemm_layout.hpp"
+#include "internal.hpp"
+
+namespace nbla_hip {
+namespace {
+
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kMaxSpatial = 3;
+
+// Geometry normalised to three spatial dimensions (leading ones of size 1).
+struct ConvGeom {
+  int64_t outer, C, O, group;
+  int in_sp[kMaxSpatial], k[kMaxSpatial], pad[kMaxSpatial], stride[kMaxSpatial], dil[kMaxSpatial],
+      out_sp[kMaxSpatial];
+  int64_t in_sp_size, out_sp_size, k_size;
+  int64_t Cg, Og, Kg; // per group: input channels, output channels, contraction length
+  int64_t M;          // outer * out_sp_size
+};
+
+// convolution.cpp:41-160
+int make_geom(ConvGeom &g, int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O, const int64_t *kernel,
+              const int64_t *pad, const int64_t *stride, const int64_t *dil, int64_t group) {
+  if (nd < 1 || nd > kMaxSpatial)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "convolutions with %d spatial dimensions are not supported (1..3).", nd);
+  if (outer <= 0 || C <= 0 || O <= 0 || group <= 0)
+    return fail(NBLA_HIP_ERR_VALUE, "invalid convolution sizes.");
+  if (C % group != 0)
+    return fail(NBLA_HIP_ERR_VALUE, "Number of input channel needs to be divisible by group. Input channel: %lld, group: %lld.",
+                (long long)C, (long long)group);
+  if (O % group != 0)
+    return fail(NBLA_HIP_ERR_VALUE, "Number of output channel needs to be divisible by group. Output channel: %lld, group: %lld.",
+                (long long)O, (long long)group);
+  g.outer = outer;
+  g.C = C;
+  g.O = O;
+  g.group = group;
+  g.in_sp_size = g.out_sp_size = g.k_size = 1;
+  const int shift = kMaxSpatial - nd;
+  for (int i = 0; i < kMaxSpatial; ++i) {
+    g.in_sp[i] = g.k[i] = g.stride[i] = g.dil[i] = g.out_sp[i] = 1;
+    g.pad[i] = 0;
+  }
+  for (int i = 0; i < nd; ++i) {
+    if (kernel[i] <= 0 || stride[i] <= 0 || dil[i] <= 0 || pad[i] < 0 || in_sp[i] <= 0)
+      return fail(NBLA_HIP_ERR_VALUE, "invalid convolution parameter at spatial dimension %d.", i);
+    const int64_t ke = dil[i] * (kernel[i] - 1) + 1;
+    const int64_t span = in_sp[i] + 2 * pad[i] - ke;
+    const int64_t o = span / stride[i] + 1;
+    if (span < 0 || o <= 0)
+      return fail(NBLA_HIP_ERR_VALUE,
+                  "Invalid configuration of convolution at %d-th spatial dimension.  {input:%lld, kernel:%lld, "
+                  "pad:%lld, stride:%lld, dilation:%lld}.",
+                  i, (long long)in_sp[i], (long long)kernel[i], (long long)pad[i], (long long)stride[i],
+                  (long long)dil[i]);
+    g.in_sp[shift + i] = (int)in_sp[i];
+    g.k[shift + i] = (int)kernel[i];
+    g.pad[shift + i] = (int)pad[i];
+    g.stride[shift + i] = (int)stride[i];
+    g.dil[shift + i] = (int)dil[i];
+    g.out_sp[shift + i] = (int)o;
+    g.in_sp_size *= in_sp[i];
+    g.out_sp_size *= o;
+    g.k_size *= kernel[i];
+  }
+  g.Cg = C / group;
+  g.Og = O / group;
+  g.Kg = g.Cg * g.k_size;
+  g.M = outer * g.out_sp_size;
+  return NBLA_HIP_OK;
+}
+
+// Value of the unfolded matrix at (pixel m, column k) for group `grp`
+// (unfold_to_patches.cpp:103-194: zero where the tap falls into the padding).
+__device__ __forceinline__ float col_value(const float *__restrict__ x, const ConvGeom &g, int64_t grp, int64_t m,
+                                           int64_t k) {
+  const int64_t n = m / g.out_sp_size;
+  int64_t p = m - n * g.out_sp_size;
+  const int o2 = (int)(p % g.out_sp[2]);
+  p /= g.out_sp[2];
+  const int o1 = (int)(p % g.out_sp[1]);
+  const int o0 = (int)(p / g.out_sp[1]);
+  int64_t t = k;
+  const int k2 = (int)(t % g.k[2]);
+  t /= g.k[2];
+  const int k1 = (int)(t % g.k[1]);
+  t /= g.k[1];
+  const int k0 = (int)(t % g.k[0]);
+  const int64_t c = grp * g.Cg + t / g.k[0];
+  const int i0 = o0 * g.stride[0] + k0 * g.dil[0] - g.pad[0];
+  const int i1 = o1 * g.stride[1] + k1 * g.dil[1] - g.pad[1];
+  const int i2 = o2 * g.stride[2] + k2 * g.dil[2] - g.pad[2];
+  if ((unsigned)i0 >= (unsigned)g.in_sp[0] || (unsigned)i1 >= (unsigned)g.in_sp[1] ||
+      (unsigned)i2 >= (unsigned)g.in_sp[2])
+    return 0.0f;
+  return x[(n * g.C + c) * g.in_sp_size + ((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2] + i2];
+}
+
+__device__ __forceinline__ uint32_t bf16_rne(float v) {
+  const uint32_t u = __float_as_uint(v);
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+__device__ __forceinline__ void split3(float x, uint32_t &hi, uint32_t &mid, uint32_t &lo) {
+  const uint32_t u = __float_as_uint(x);
+  if ((u & 0x7f800000u) == 0x7f800000u) {
+    hi = (u >> 16) | ((u & 0xffffu) ? 0x40u : 0u);
+    mid = lo = 0u;
+    return;
+  }
+  hi = bf16_rne(x);
+  if ((hi & 0x7f80u) == 0x7f80u)
+    hi = u >> 16;
+  const float r1 = x - __uint_as_float(hi << 16);
+  mid = bf16_rne(r1);
+  const float r2 = r1 - __uint_as_float(mid << 16);
+  lo = bf16_rne(r2);
+}
+
+// One wavefront per (row block, k block) fragment of the split operand.
+__global__ __launch_bounds__(256) void im2col_split(const float *__restrict__ x, uint4_t *__restrict__ out, ConvGeom g,
+                                                    int64_t grp, int64_t k_blocks, int64_t frags) {
+  const int64_t frag = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (frag >= frags)
+    return;
+  const int lane = threadIdx.x & 63;
+  const int64_t rb = frag / k_blocks, kb = frag - rb * k_blocks;
+  const int64_t m = rb * kFragRows + (lane & 31);
+  const int64_t k0 = kb * kFragK + (lane >> 5) * 8;
+  uint32_t h[8], mi[8], l[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float v = (m < g.M && k0 + e < g.Kg) ? col_value(x, g, grp, m, k0 + e) : 0.0f;
+    split3(v, h[e], mi[e], l[e]);
+  }
+  uint4_t o;
+  uint4_t *dst = out + frag * 3 * 64 + lane;
+  o.x = h[0] | (h[1] << 16), o.y = h[2] | (h[3] << 16), o.z = h[4] | (h[5] << 16), o.w = h[6] | (h[7] << 16);
+  dst[0] = o;
+  o.x = mi[0] | (mi[1] << 16), o.y = mi[2] | (mi[3] << 16), o.z = mi[4] | (mi[5] << 16), o.w = mi[6] | (mi[7] << 16);
+  dst[64] = o;
+  o.x = l[0] | (l[1] << 16), o.y = l[2] | (l[3] << 16), o.z = l[4] | (l[5] << 16), o.w = l[6] | (l[7] << 16);
+  dst[128] = o;
+}
+
+// fp32 unfolded matrix [M, Kg] for the general (non bit-representable) path.
+__global__ __launch_bounds__(256) void im2col_f32(const float *__restrict__ x, float *__restrict__ col, ConvGeom g,
+                                                  int64_t grp) {
+  const int64_t total = g.M * g.Kg;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t m = i / g.Kg;
+    col[i] = col_value(x, g, grp, m, i - m * g.Kg);
+  }
+}
+
+struct ConvWorkspace {
+  size_t bits_off, bits_stride, split_off, prep_off, count_off, col_off, total;
+};
+
+ConvWorkspace plan_conv(const ConvGeom &g) {
+  ConvWorkspace w;
+  size_t off = 0;
+  w.bits_off = off;
+  w.bits_stride = round_up(nbla_hip_packed_bits_bytes(g.Kg, g.Og), 256);
+  off += w.bits_stride * g.group;
+  w.split_off = off;
+  off += round_up(nbla_hip_split_operand_bytes(g.M, g.Kg), 256);
+  w.prep_off = off;
+  off += round_up(nbla_hip_binarize_workspace_bytes(g.Kg, g.Og), 256);
+  w.count_off = off;
+  off += round_up(sizeof(int) * g.group, 256);
+  w.col_off = off; // fp32 unfolded matrix of the general path shares the split operand's space when it fits
+  w.total = off;
+  return w;
+}
+
+int binary_conv_forward(const float *x, const float *W, float *Wb, float *alpha, const float *bias, float *y,
+                        const ConvGeom &g, float zero_to, void *workspace, size_t workspace_bytes, void *stream_) {
+  const ConvWorkspace ws = plan_conv(g);
+  const bool representable = (zero_to == 1.0f || zero_to == -1.0f);
+  const size_t col_bytes = representable ? 0 : round_up((size_t)g.M * g.Kg * sizeof(float), 256);
+  if (workspace_bytes < ws.total + col_bytes || !aligned256(workspace))
+    return fail(NBLA_HIP_ERR_MEMORY, "binary convolution workspace too small (%zu < %zu) or misaligned.",
+                workspace_bytes, ws.total + col_bytes);
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  hipStream_t stream = as_stream(stream_);
+  char *base = static_cast<char *>(workspace);
+  int *counts = reinterpret_cast<int *>(base + ws.count_off);
+  // weights: per group a [Og, Kg] slab stored n-major -> packed [Kg, Og] bits, Sign, alpha
+  for (int64_t grp = 0; grp < g.group; ++grp) {
+    const int64_t woff = grp * g.Og * g.Kg;
+    rc = nbla_hip_binarize_weights_f32(W + woff, Wb + woff, alpha ? alpha + grp * g.Og : nullptr,
+                                       reinterpret_cast<uint32_t *>(base + ws.bits_off + grp * ws.bits_stride), g.Kg,
+                                       g.Og, 1, zero_to, representable ? nullptr : counts + grp, base + ws.prep_off,
+                                       nbla_hip_binarize_workspace_bytes(g.Kg, g.Og), stream_);
+    if (rc)
+      return rc;
+  }
+  bool use_bits = true;
+  if (!representable) {
+    int host_counts[64];
+    int total = 0;
+    for (int64_t g0 = 0; g0 < g.group; g0 += 64) {
+      const int64_t nb = (g.group - g0 < 64) ? g.group - g0 : 64;
+      hipError_t e = hipMemcpyAsync(host_counts, counts + g0, sizeof(int) * nb, hipMemcpyDeviceToHost, stream);
+      if (e == hipSuccess)
+        e = hipStreamSynchronize(stream);
+      if (e != hipSuccess)
+        return fail_hip(e, "reading the zero-weight count");
+      for (int64_t i = 0; i < nb; ++i)
+        total += host_counts[i];
+    }
+    use_bits = (total == 0);
+  }
+  const int64_t hw = g.out_sp_size;
+  for (int64_t grp = 0; grp < g.group; ++grp) {
+    float *yg = y + grp * g.Og * hw;
+    const float *ag = alpha ? alpha + grp * g.Og : nullptr;
+    const float *bg = bias ? bias + grp * g.Og : nullptr;
+    if (use_bits) {
+      const int64_t k_blocks = split_k_blocks(g.Kg);
+      const int64_t frags = split_row_blocks(g.M) * k_blocks;
+      hipLaunchKernelGGL(im2col_split, dim3((unsigned)ceil_div(frags, 4)), dim3(256), 0, stream, x,
+                         reinterpret_cast<uint4_t *>(base + ws.split_off), g, grp, k_blocks, frags);
+      NBLA_HIP_LAUNCH_CHECK("im2col_split");
+      rc = launch_gemm_bits(base + ws.split_off,
+                            reinterpret_cast<const uint32_t *>(base + ws.bits_off + grp * ws.bits_stride), ag, bg, yg,
+                            g.M, g.Kg, g.Og, hw, g.O * hw, hw, true, stream);
+    } else {
+      float *col = reinterpret_cast<float *>(base + ws.total);
+      int64_t blocks = ceil_div(g.M * g.Kg, 256);
+      if (blocks > 65536)
+        blocks = 65536;
+      hipLaunchKernelGGL(im2col_f32, dim3((unsigned)blocks), dim3(256), 0, stream, x, col, g, grp);
+      NBLA_HIP_LAUNCH_CHECK("im2col_f32");
+      rc = launch_gemm_f32_mapped(col, Wb + grp * g.Og * g.Kg, true, ag, bg, yg, g.M, g.Kg, g.Og, hw, g.O * hw, hw,
+                                  stream);
+    }
+    if (rc)
+      return rc;
+  }
+  return NBLA_HIP_OK;
+}
+
+} // namespace
+} // namespace nbla_hip
+
+using namespace nbla_hip;
+
+extern "C" {
+
+int nbla_hip_convolution_output_shape(int nd, const int64_t *in_sp, const int64_t *kernel, const int64_t *pad,
+                                      const int64_t *stride, const int64_t *dilation, int64_t *out_sp) {
+  ConvGeom g;
+  const int rc = make_geom(g, 1, 1, nd, in_sp, 1, kernel, pad, stride, dilation, 1);
+  if (rc)
+    return rc;
+  for (int i = 0; i < nd; ++i)
+    out_sp[i] = g.out_sp[kMaxSpatial - nd + i];
+  return NBLA_HIP_OK;
+}
+
+size_t nbla_hip_binary_convolution_workspace_bytes(int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
+                                                   const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+                                                   const int64_t *dilation, int64_t group, float quantize_zero_to) {
+  ConvGeom g;
+  if (make_geom(g, outer, C, nd, in_sp, O, kernel, pad, stride, dilation, group))
+    return 0;
+  const bool representable = (quantize_zero_to == 1.0f || quantize_zero_to == -1.0f);
+  return plan_conv(g).total + (representable ? 0 : round_up((size_t)g.M * g.Kg * sizeof(float), 256));
+}
+
+int nbla_hip_binary_weight_convolution_f32(const float *x, const float *W, float *Wb, float *alpha, const float *bias,
+                                           float *y, int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
+                                           const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+                                           const int64_t *dilation, int64_t group, float quantize_zero_to,
+                                           void *workspace, size_t workspace_bytes, void *stream) {
+  if (!alpha)
+    return fail(NBLA_HIP_ERR_VALUE, "BinaryWeightConvolution needs an alpha output of size channels_o.");
+  ConvGeom g;
+  const int rc = make_geom(g, outer, C, nd, in_sp, O, kernel, pad, stride, dilation, group);
+  if (rc)
+    return rc;
+  return binary_conv_forward(x, W, Wb, alpha, bias, y, g, quantize_zero_to, workspace, workspace_bytes, stream);
+}
+
+int nbla_hip_binary_connect_convolution_f32(const float *x, const float *W, float *Wb, const float *bias, float *y,
+                                            int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
+                                            const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+                                            const int64_t *dilation, int64_t group, float quantize_zero_to,
+                                            void *workspace, size_t workspace_bytes, void *stream) {
+  ConvGeom g;
+  const int rc = make_geom(g, outer, C, nd, in_sp, O, kernel, pad, stride, dilation, group);
+  if (rc)
+    return rc;
+  return binary_conv_forward(x, W, Wb, nullptr, bias, y, g, quantize_zero_to, workspace, workspace_bytes, stream);
+}
+
+} // extern "C"

@@ -14,6 +14,7 @@
 // VALU operations per register (shift, and-or).
 #include "common.hpp"
 #include "gemm_layout.hpp"
+#include "internal.hpp"
 
 namespace nbla_hip {
 namespace {
@@ -49,7 +50,9 @@ __device__ __forceinline__ int64_t xcd_remap(int64_t b, int64_t total) {
   return start + slot;
 }
 
-template <int BM, int BN, int kWavesM, int kWavesN>
+// kSwap exchanges the MFMA operand roles (the instruction computes the transposed 32x32 tile), which puts
+// consecutive m on consecutive lanes of the accumulator: the store pattern for outputs whose m index is contiguous.
+template <int BM, int BN, int kWavesM, int kWavesN, bool kSwap>
 __global__ __launch_bounds__(kWavesM *kWavesN * 64) void gemm_bits_kernel(GemmBitsArgs a) {
   constexpr int kThreads = kWavesM * kWavesN * 64;
   constexpr int MF = BM / kWavesM / 32;  // A fragments per wavefront (rows)
@@ -173,8 +176,12 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64) void gemm_bits_kernel(GemmBi
         for (int i = 0; i < MF; ++i)
 #pragma unroll
           for (int j = 0; j < NF; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[i][p]),
-                                                                __builtin_bit_cast(bf16x8_t, bf[j]), acc[i][j], 0, 0, 0);
+            acc[i][j] = kSwap ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[j]),
+                                                                        __builtin_bit_cast(bf16x8_t, af[i][p]),
+                                                                        acc[i][j], 0, 0, 0)
+                              : __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[i][p]),
+                                                                        __builtin_bit_cast(bf16x8_t, bf[j]),
+                                                                        acc[i][j], 0, 0, 0);
     }
 
     if (ks + 1 < a.k_steps)
@@ -183,40 +190,68 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64) void gemm_bits_kernel(GemmBi
   }
 
   // Epilogue.  Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
-  // column l%32 of the 32x32 fragment.
+  // column l%32 of the 32x32 fragment; rows are m and columns n, or the reverse
+  // under kSwap.
   const int col_in_frag = lane & 31, row_half = lane >> 5;
+  if (!kSwap) {
 #pragma unroll
-  for (int j = 0; j < NF; ++j) {
-    const int64_t n = bn * BN + (wn * NF + j) * 32 + col_in_frag;
-    if (n >= a.N)
-      continue;
-    const float al = a.alpha ? a.alpha[n] : 1.0f;
-    const float bi = a.bias ? a.bias[n] : 0.0f;
+    for (int j = 0; j < NF; ++j) {
+      const int64_t n = bn * BN + (wn * NF + j) * 32 + col_in_frag;
+      if (n >= a.N)
+        continue;
+      const float al = a.alpha ? a.alpha[n] : 1.0f;
+      const float bi = a.bias ? a.bias[n] : 0.0f;
+#pragma unroll
+      for (int i = 0; i < MF; ++i) {
+        const int64_t m0 = bm * BM + (wm * MF + i) * 32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t m = m0 + 8 * (r >> 2) + 4 * row_half + (r & 3);
+          if (m < a.M) {
+            float v = acc[i][j][r];
+            if (a.alpha)
+              v = v * al;
+            if (a.bias)
+              v = v + bi;
+            const int64_t off = (a.inner == 1) ? m * a.outer_stride : (m / a.inner) * a.outer_stride + (m % a.inner);
+            a.y[off + n * a.n_stride] = v;
+          }
+        }
+      }
+    }
+  } else {
 #pragma unroll
     for (int i = 0; i < MF; ++i) {
-      const int64_t m0 = bm * BM + (wm * MF + i) * 32;
+      const int64_t m = bm * BM + (wm * MF + i) * 32 + col_in_frag;
+      if (m >= a.M)
+        continue;
+      const int64_t off = (a.inner == 1) ? m * a.outer_stride : (m / a.inner) * a.outer_stride + (m % a.inner);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int64_t m = m0 + 8 * (r >> 2) + 4 * row_half + (r & 3);
-        if (m < a.M) {
-          float v = acc[i][j][r];
-          if (a.alpha)
-            v = v * al;
-          if (a.bias)
-            v = v + bi;
-          const int64_t off = (a.inner == 1) ? m * a.outer_stride : (m / a.inner) * a.outer_stride + (m % a.inner);
-          a.y[off + n * a.n_stride] = v;
+      for (int j = 0; j < NF; ++j) {
+        const int64_t n0 = bn * BN + (wn * NF + j) * 32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t n = n0 + 8 * (r >> 2) + 4 * row_half + (r & 3);
+          if (n < a.N) {
+            float v = acc[i][j][r];
+            if (a.alpha)
+              v = v * a.alpha[n];
+            if (a.bias)
+              v = v + a.bias[n];
+            a.y[off + n * a.n_stride] = v;
+          }
         }
       }
     }
   }
 }
 
-template <int BM, int BN, int kWavesM, int kWavesN> int launch_gemm_bits(const GemmBitsArgs &args, hipStream_t stream) {
+template <int BM, int BN, int kWavesM, int kWavesN, bool kSwap>
+int launch_tile(const GemmBitsArgs &args, hipStream_t stream) {
   constexpr int kThreads = kWavesM * kWavesN * 64;
   constexpr int kStageBytes = (BM / 32) * 6 * 64 * 16 + BN * 4;
   constexpr int kSmem = 2 * kStageBytes;
-  auto kernel = gemm_bits_kernel<BM, BN, kWavesM, kWavesN>;
+  auto kernel = gemm_bits_kernel<BM, BN, kWavesM, kWavesN, kSwap>;
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
@@ -232,16 +267,19 @@ template <int BM, int BN, int kWavesM, int kWavesN> int launch_gemm_bits(const G
   return NBLA_HIP_OK;
 }
 
+template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream) {
+  if (a.M > 128)
+    return launch_tile<256, 256, 4, 2, kSwap>(a, stream);
+  if (a.M > 32)
+    return launch_tile<128, 128, 4, 1, kSwap>(a, stream);
+  return launch_tile<32, 256, 1, 4, kSwap>(a, stream);
+}
+
 } // namespace
-} // namespace nbla_hip
 
-using namespace nbla_hip;
-
-extern "C" {
-
-int nbla_hip_gemm_bits_f32(const void *xsplit, const uint32_t *bits, const float *alpha, const float *bias, float *y,
-                           int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
-                           void *stream_) {
+int launch_gemm_bits(const void *xsplit, const uint32_t *bits, const float *alpha, const float *bias, float *y,
+                     int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
+                     bool swap_out, hipStream_t stream) {
   if (M <= 0 || K <= 0 || N <= 0 || inner <= 0)
     return fail(NBLA_HIP_ERR_VALUE, "invalid GEMM shape (M=%lld, K=%lld, N=%lld).", (long long)M, (long long)K,
                 (long long)N);
@@ -262,15 +300,21 @@ int nbla_hip_gemm_bits_f32(const void *xsplit, const uint32_t *bits, const float
   a.k_blocks = split_k_blocks(K);
   a.col_groups = bits_col_groups(N);
   a.k_steps = bits_k_tiles(K);
+  a.blocks_m = a.blocks_n = 0;
   a.inner = inner;
   a.outer_stride = outer_stride;
   a.n_stride = n_stride;
-  hipStream_t stream = as_stream(stream_);
-  if (M > 128)
-    return launch_gemm_bits<256, 256, 4, 2>(a, stream);
-  if (M > 32)
-    return launch_gemm_bits<128, 128, 4, 1>(a, stream);
-  return launch_gemm_bits<32, 256, 1, 4>(a, stream);
+  return swap_out ? dispatch<true>(a, stream) : dispatch<false>(a, stream);
 }
 
-} // extern "C"
+} // namespace nbla_hip
+
+using namespace nbla_hip;
+
+extern "C" int nbla_hip_gemm_bits_f32(const void *xsplit, const uint32_t *bits, const float *alpha, const float *bias,
+                                      float *y, int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride,
+                                      int64_t n_stride, void *stream) {
+  // m-contiguous outputs (n_stride != 1) store from the transposed accumulator tile
+  return launch_gemm_bits(xsplit, bits, alpha, bias, y, M, K, N, inner, outer_stride, n_stride, n_stride != 1,
+                          as_stream(stream));
+}

@@ -5,11 +5,9 @@
 // wavefronts each owning a 64x64 corner.
 #include "common.hpp"
 #include "gemm_layout.hpp"
+#include "internal.hpp"
 
 namespace nbla_hip {
-
-int launch_gemm_f32(const float *x, const float *w, const float *colscale, const float *bias, float *y, int64_t M,
-                    int64_t K, int64_t N, hipStream_t stream);
 
 namespace {
 
@@ -17,10 +15,14 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 constexpr int kBM = 128, kBN = 128, kBK = 16, kPad = 4;
 
+// w is [K, N] (kTransB == false) or [N, K] (kTransB == true).  Output element (m, n) goes to
+// y[(m / inner) * outer_stride + n * n_stride + (m % inner)].
+template <bool kTransB>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                        const float *__restrict__ colscale,
                                                        const float *__restrict__ bias, float *__restrict__ y,
-                                                       int64_t M, int64_t K, int64_t N) {
+                                                       int64_t M, int64_t K, int64_t N, int64_t inner,
+                                                       int64_t outer_stride, int64_t n_stride) {
   __shared__ float As[kBK][kBM + kPad]; // [k][m]
   __shared__ float Bs[kBK][kBN + kPad]; // [k][n]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -37,7 +39,8 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__
         acc[i][j][r] = 0.0f;
 
   const int a_row = tid >> 1, a_k = (tid & 1) * 8; // 128 rows x 2 halves of 8 k
-  const int b_k = tid >> 4, b_n = (tid & 15) * 8;  // 16 k x 16 groups of 8 n
+  const int b_k = tid >> 4, b_n = (tid & 15) * 8;  // [K,N] source: 16 k x 16 groups of 8 n
+  const int t_n = tid >> 1, t_k = (tid & 1) * 8;   // [N,K] source: 128 n x 2 halves of 8 k
 
   for (int64_t k0 = 0; k0 < K; k0 += kBK) {
     float av[8], bv[8];
@@ -48,16 +51,25 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int64_t k = k0 + b_k, n = n0 + b_n + e;
-      bv[e] = (k < K && n < N) ? w[k * N + n] : 0.0f;
+      if (kTransB) {
+        const int64_t n = n0 + t_n, k = k0 + t_k + e;
+        bv[e] = (k < K && n < N) ? w[n * K + k] : 0.0f;
+      } else {
+        const int64_t k = k0 + b_k, n = n0 + b_n + e;
+        bv[e] = (k < K && n < N) ? w[k * N + n] : 0.0f;
+      }
     }
     __syncthreads(); // previous tile fully consumed
 #pragma unroll
     for (int e = 0; e < 8; ++e)
       As[a_k + e][a_row] = av[e];
 #pragma unroll
-    for (int e = 0; e < 8; ++e)
-      Bs[b_k][b_n + e] = bv[e];
+    for (int e = 0; e < 8; ++e) {
+      if (kTransB)
+        Bs[t_k + e][t_n] = bv[e];
+      else
+        Bs[b_k][b_n + e] = bv[e];
+    }
     __syncthreads();
 #pragma unroll
     for (int kk = 0; kk < kBK; kk += 2) {
@@ -95,7 +107,8 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__
             v = v * sc;
           if (bias)
             v = v + bi;
-          y[m * N + n] = v;
+          const int64_t off = (inner == 1) ? m * outer_stride : (m / inner) * outer_stride + (m % inner);
+          y[off + n * n_stride] = v;
         }
       }
   }
@@ -103,12 +116,23 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__
 
 } // namespace
 
-int launch_gemm_f32(const float *x, const float *w, const float *colscale, const float *bias, float *y, int64_t M,
-                    int64_t K, int64_t N, hipStream_t stream) {
+int launch_gemm_f32_mapped(const float *x, const float *w, bool trans_b, const float *colscale, const float *bias,
+                           float *y, int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride,
+                           int64_t n_stride, hipStream_t stream) {
   const dim3 grid((unsigned)ceil_div(N, kBN), (unsigned)ceil_div(M, kBM));
-  hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, stream, x, w, colscale, bias, y, M, K, N);
+  if (trans_b)
+    hipLaunchKernelGGL(gemm_f32_kernel<true>, grid, dim3(256), 0, stream, x, w, colscale, bias, y, M, K, N, inner,
+                       outer_stride, n_stride);
+  else
+    hipLaunchKernelGGL(gemm_f32_kernel<false>, grid, dim3(256), 0, stream, x, w, colscale, bias, y, M, K, N, inner,
+                       outer_stride, n_stride);
   NBLA_HIP_LAUNCH_CHECK("gemm_f32");
   return NBLA_HIP_OK;
+}
+
+int launch_gemm_f32(const float *x, const float *w, const float *colscale, const float *bias, float *y, int64_t M,
+                    int64_t K, int64_t N, hipStream_t stream) {
+  return launch_gemm_f32_mapped(x, w, false, colscale, bias, y, M, K, N, 1, N, 1, stream);
 }
 
 } // namespace nbla_hip

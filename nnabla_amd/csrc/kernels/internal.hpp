@@ -1,0 +1,21 @@
+// Entry points shared between the translation units of the kernel library (not part of the C-ABI).
+#pragma once
+#include "common.hpp"
+
+namespace nbla_hip {
+
+// fp32 MFMA product y = (x . w) * colscale + bias; w is [K, N], or [N, K] when trans_b.  Output element (m, n) is
+// written at y[(m / inner) * outer_stride + n * n_stride + (m % inner)].
+int launch_gemm_f32_mapped(const float *x, const float *w, bool trans_b, const float *colscale, const float *bias,
+                           float *y, int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride,
+                           int64_t n_stride, hipStream_t stream);
+int launch_gemm_f32(const float *x, const float *w, const float *colscale, const float *bias, float *y, int64_t M,
+                    int64_t K, int64_t N, hipStream_t stream);
+
+// Bit-weight product with the choice of store orientation: swap_out makes consecutive lanes write consecutive m
+// (for outputs whose m index is the contiguous one, e.g. convolution results [batch, O, Ho*Wo]).
+int launch_gemm_bits(const void *xsplit, const uint32_t *bits, const float *alpha, const float *bias, float *y,
+                     int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
+                     bool swap_out, hipStream_t stream);
+
+} // namespace nbla_hip

@@ -26,6 +26,8 @@ EXPORTED = (
     "nbla_hip_binarize_weights_f32", "nbla_hip_split_bf16x3_f32", "nbla_hip_gemm_bits_f32",
     "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_weight_affine_f32",
     "nbla_hip_binary_connect_affine_f32", "nbla_hip_affine_f32",
+    "nbla_hip_convolution_output_shape", "nbla_hip_binary_convolution_workspace_bytes",
+    "nbla_hip_binary_weight_convolution_f32", "nbla_hip_binary_connect_convolution_f32",
 )
 
 
@@ -50,7 +52,7 @@ def lib():
         L.nbla_hip_version.restype = ctypes.c_char_p
         for name in ("nbla_hip_min_max_quantize_workspace_bytes", "nbla_hip_packed_bits_bytes",
                      "nbla_hip_split_operand_bytes", "nbla_hip_binarize_workspace_bytes",
-                     "nbla_hip_binary_affine_workspace_bytes"):
+                     "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_convolution_workspace_bytes"):
             getattr(L, name).restype = ctypes.c_size_t
         _lib = L
     return _lib
@@ -200,3 +202,53 @@ def affine(x, W, bias=None, out=None, stream=None):
     y = torch.empty((M, N), dtype=torch.float32, device=x.device) if out is None else out
     check(lib().nbla_hip_affine_f32(_p(x), _p(W), _p(bias), _p(y), _i64(M), _i64(K), _i64(N), _stream(stream)))
     return y
+
+
+def _conv_geometry(x, W, pad, stride, dilation, group):
+    nd = W.dim() - 2
+    outer = 1
+    for s in x.shape[:x.dim() - nd - 1]:
+        outer *= int(s)
+    C = int(x.shape[x.dim() - nd - 1])
+    in_sp = [int(s) for s in x.shape[x.dim() - nd:]]
+    O = int(W.shape[0])
+    kernel = [int(s) for s in W.shape[2:]]
+    pad = list(pad) if pad is not None else [0] * nd
+    stride = list(stride) if stride is not None else [1] * nd
+    dilation = list(dilation) if dilation is not None else [1] * nd
+    out_sp = (ctypes.c_int64 * nd)()
+    check(lib().nbla_hip_convolution_output_shape(nd, _shape(in_sp), _shape(kernel), _shape(pad), _shape(stride),
+                                                  _shape(dilation), out_sp))
+    geom = (_i64(outer), _i64(C), nd, _shape(in_sp), _i64(O), _shape(kernel), _shape(pad), _shape(stride),
+            _shape(dilation), _i64(group))
+    yshape = tuple(x.shape[:x.dim() - nd - 1]) + (O,) + tuple(int(v) for v in out_sp)
+    return geom, yshape
+
+
+def binary_weight_convolution(x, W, bias=None, pad=None, stride=None, dilation=None, group=1, quantize_zero_to=1.0,
+                              stream=None):
+    """x [..., C, spatial...], W [O, C/group, kernel...] -> (y, Wb, alpha)."""
+    import torch
+    geom, yshape = _conv_geometry(x, W, pad, stride, dilation, group)
+    q0 = ctypes.c_float(quantize_zero_to)
+    ws = _workspace(lib().nbla_hip_binary_convolution_workspace_bytes(*geom, q0), x)
+    Wb = torch.empty_like(W)
+    alpha = torch.empty(W.shape[0], dtype=torch.float32, device=x.device)
+    y = torch.empty(yshape, dtype=torch.float32, device=x.device)
+    check(lib().nbla_hip_binary_weight_convolution_f32(_p(x), _p(W), _p(Wb), _p(alpha), _p(bias), _p(y), *geom, q0,
+                                                       _p(ws), ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return y, Wb, alpha
+
+
+def binary_connect_convolution(x, W, bias=None, pad=None, stride=None, dilation=None, group=1, quantize_zero_to=1.0,
+                               stream=None):
+    """x [..., C, spatial...], W [O, C/group, kernel...] -> (y, Wb)."""
+    import torch
+    geom, yshape = _conv_geometry(x, W, pad, stride, dilation, group)
+    q0 = ctypes.c_float(quantize_zero_to)
+    ws = _workspace(lib().nbla_hip_binary_convolution_workspace_bytes(*geom, q0), x)
+    Wb = torch.empty_like(W)
+    y = torch.empty(yshape, dtype=torch.float32, device=x.device)
+    check(lib().nbla_hip_binary_connect_convolution_f32(_p(x), _p(W), _p(Wb), _p(bias), _p(y), *geom, q0, _p(ws),
+                                                        ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return y, Wb

@@ -1,0 +1,105 @@
+"""BinaryWeightConvolution / BinaryConnectConvolution on the GPU against the CPU oracle: Sign(W) bit-exact, alpha at
+rel 2e-6, outputs within max|y - y_ref| / max|y_ref| <= 1e-4 (expected ~1e-6)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from nnabla_amd import kernels
+from util import bits_equal, max_rel_err, to_np
+
+pytestmark = pytest.mark.gpu
+TOL, TIGHT = 1e-4, 5e-6
+
+
+def _dev(x, dev):
+    return torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+
+
+CASES = [
+    # (x shape, w shape, pad, stride, dilation, group)
+    ((2, 4, 7, 7), (6, 4, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((2, 4, 7, 7), (6, 2, 3, 3), (1, 0), (2, 1), (1, 2), 2),
+    ((1, 3, 9, 8), (5, 3, 2, 3), (0, 2), (1, 2), (2, 1), 1),
+    ((3, 2, 10), (4, 2, 3), (1,), (2,), (1,), 1),
+    ((2, 2, 4, 5, 6), (3, 2, 2, 3, 2), (1, 0, 1), (1, 2, 1), (1, 1, 2), 1),
+    ((2, 6, 5, 5), (6, 1, 3, 3), (1, 1), (1, 1), (1, 1), 6),
+    ((4, 8, 16, 16), (16, 8, 3, 3), (1, 1), (1, 1), (1, 1), 1),        # the reference tests' own size
+    ((2, 3, 4, 8, 16, 16), (16, 8, 3, 3), (1, 1), (2, 2), (1, 1), 1),  # base_axis = 3: leading axes fold into outer
+    ((3, 64, 14, 14), (96, 32, 3, 3), (1, 1), (1, 1), (1, 1), 2),
+]
+
+
+@pytest.mark.parametrize("xs,ws,pad,stride,dil,group", CASES)
+@pytest.mark.parametrize("bias", [False, True])
+def test_binary_weight_convolution_matches_oracle(dev, xs, ws, pad, stride, dil, group, bias):
+    rng = np.random.RandomState(313)
+    x = rng.randn(*xs).astype(np.float32)
+    W = (rng.randn(*ws) * 0.05).astype(np.float32)
+    b = rng.randn(ws[0]).astype(np.float32) if bias else None
+    ref_y, ref_Wb, ref_alpha = oracle.binary_weight_convolution(x, W, b, pad, stride, dil, group, 1.0)
+    y, Wb, alpha = kernels.binary_weight_convolution(_dev(x, dev), _dev(W, dev), None if b is None else _dev(b, dev),
+                                                     pad, stride, dil, group)
+    assert tuple(y.shape) == ref_y.shape
+    assert bits_equal(to_np(Wb), ref_Wb)
+    np.testing.assert_allclose(to_np(alpha), ref_alpha, rtol=2e-6)
+    assert max_rel_err(to_np(y), ref_y) <= TIGHT
+
+
+@pytest.mark.parametrize("xs,ws,pad,stride,dil,group", CASES)
+def test_binary_connect_convolution_matches_oracle(dev, xs, ws, pad, stride, dil, group):
+    rng = np.random.RandomState(7)
+    x = rng.randn(*xs).astype(np.float32)
+    W = (rng.randn(*ws) * 0.05).astype(np.float32)
+    b = rng.randn(ws[0]).astype(np.float32)
+    ref_y, ref_Wb = oracle.binary_connect_convolution(x, W, b, pad, stride, dil, group, 1.0)
+    y, Wb = kernels.binary_connect_convolution(_dev(x, dev), _dev(W, dev), _dev(b, dev), pad, stride, dil, group)
+    assert bits_equal(to_np(Wb), ref_Wb)
+    assert max_rel_err(to_np(y), ref_y) <= TIGHT
+
+
+@pytest.mark.parametrize("q0", [0.0, -1.0, 0.5])
+def test_convolution_quantize_zero_to_with_zero_weights(dev, q0):
+    rng = np.random.RandomState(3)
+    x = rng.randn(2, 4, 9, 9).astype(np.float32)
+    W = (rng.randn(6, 2, 3, 3) * 0.05).astype(np.float32)
+    W.ravel()[::4] = 0.0
+    ref_y, ref_Wb, ref_alpha = oracle.binary_weight_convolution(x, W, None, (1, 1), (1, 1), (1, 1), 2, q0)
+    y, Wb, alpha = kernels.binary_weight_convolution(_dev(x, dev), _dev(W, dev), None, (1, 1), (1, 1), (1, 1), 2, q0)
+    assert bits_equal(to_np(Wb), ref_Wb)
+    assert max_rel_err(to_np(y), ref_y) <= TIGHT * 4
+    ref_y, _ = oracle.binary_connect_convolution(x, W, None, (1, 1), (1, 1), (1, 1), 2, q0)
+    y, _ = kernels.binary_connect_convolution(_dev(x, dev), _dev(W, dev), None, (1, 1), (1, 1), (1, 1), 2, q0)
+    assert max_rel_err(to_np(y), ref_y) <= TIGHT * 4
+
+
+def test_config4_resnet_stage(dev):
+    """BASELINE config 4: x [32,256,14,14] ~ N(0,1), W [256,256,3,3] ~ N(0, 2/2304), stride 1, pad 1, zero bias.
+    The oracle is run on 4 of the 32 samples (convolution is independent per sample); all 32 are checked against
+    torch's float64 convolution on the same binarized weights."""
+    rng = np.random.default_rng(313)
+    x = rng.standard_normal((32, 256, 14, 14), dtype=np.float32)
+    W = rng.standard_normal((256, 256, 3, 3), dtype=np.float32) * np.float32(np.sqrt(2.0 / 2304))
+    b = np.zeros(256, np.float32)
+    y, Wb, alpha = kernels.binary_weight_convolution(_dev(x, dev), _dev(W, dev), _dev(b, dev), (1, 1), (1, 1), (1, 1))
+    yc, Wbc = kernels.binary_connect_convolution(_dev(x, dev), _dev(W, dev), _dev(b, dev), (1, 1), (1, 1), (1, 1))
+    ref_y, ref_Wb, ref_alpha = oracle.binary_weight_convolution(x[:4], W, b, (1, 1), (1, 1), (1, 1), 1, 1.0)
+    ref_yc, _ = oracle.binary_connect_convolution(x[:4], W, b, (1, 1), (1, 1), (1, 1), 1, 1.0)
+    assert bits_equal(to_np(Wb), ref_Wb) and bits_equal(to_np(Wbc), ref_Wb)
+    np.testing.assert_allclose(to_np(alpha), ref_alpha, rtol=2e-6)
+    assert max_rel_err(to_np(y)[:4], ref_y) <= TOL and max_rel_err(to_np(yc)[:4], ref_yc) <= TOL
+    s64 = torch.from_numpy(ref_Wb).double()
+    full = torch.nn.functional.conv2d(torch.from_numpy(x).double(), s64, None, 1, 1).numpy()
+    a64 = np.abs(W.astype(np.float64)).reshape(256, -1).mean(1).reshape(1, -1, 1, 1)
+    assert max_rel_err(to_np(yc), full) <= TIGHT
+    assert max_rel_err(to_np(y), full * a64) <= TIGHT
+
+
+def test_convolution_argument_errors(dev):
+    x = _dev(np.zeros((1, 4, 5, 5), np.float32), dev)
+    with pytest.raises(kernels.KernelError) as ei:
+        kernels.binary_weight_convolution(x, _dev(np.zeros((6, 4, 7, 7), np.float32), dev))
+    assert ei.value.code == kernels.ERR_VALUE
+    with pytest.raises(kernels.KernelError) as ei:
+        kernels.binary_connect_convolution(x, _dev(np.zeros((6, 2, 3, 3), np.float32), dev), group=3)
+    assert ei.value.code == kernels.ERR_VALUE
