@@ -226,6 +226,66 @@ int nbla_hip_binary_connect_convolution_f32(
     const int64_t *dilation, int64_t group, float quantize_zero_to,
     void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---------------------------------------------------------------------- INQ */
+
+/* INQ step selector (what the forward does to the indicators before quantizing):
+ *   -1  product only, weights untouched (recompute_impl, inq_affine.cpp:208-216)
+ *    0  no selection this minibatch
+ *    1  last entry of inq_iterations reached: every weight becomes fixed (:108-113)
+ *    2  fix half of the learnable weights, largest |w| first (:117-141); equal |w|
+ *       are taken in index order (the reference's order among equal keys is
+ *       whatever std::sort leaves)
+ *    3  fix each learnable weight with probability 1/2 (:143-149)
+ * The caller owns the minibatch counter and maps it to a step. */
+
+/* Bernoulli(0.5) source for step 3: must write `count` values (0 or 1) to `out`,
+ * advancing the caller's generator by exactly `count` draws -- the role of
+ * rdist_(rgen) with std::mt19937 in inq_affine.cpp:147. */
+typedef void (*nbla_hip_bernoulli_fn)(void *ctx, uint8_t *out, int64_t count);
+
+size_t nbla_hip_inq_workspace_bytes(int64_t size, int step);
+
+/* Steps A, B, C and F of INQAffine<float,int>::forward_impl,
+ * src/nbla/function/generic/inq_affine.cpp:95-190 and :203-204 (identical in
+ * inq_convolution.cpp:110-222): W and I (int32 indicators) are rewritten in
+ * place; old_W / old_I are the function's snapshot (read for the restore, then
+ * overwritten with the new W / I).  n1n2_out (device, 2 ints, may be NULL)
+ * receives the exponent range.  step 3 synchronises the stream once. */
+int nbla_hip_inq_update_weights_f32(float *W, int32_t *I, float *old_W,
+                                    int32_t *old_I, int64_t size, int num_bits,
+                                    int step, nbla_hip_bernoulli_fn draw,
+                                    void *draw_ctx, int32_t *n1n2_out,
+                                    void *workspace, size_t workspace_bytes,
+                                    void *stream);
+
+size_t nbla_hip_inq_affine_workspace_bytes(int64_t M, int64_t K, int64_t N,
+                                           int step);
+
+/* INQAffine forward: the weight update above, then y = x . W + bias with fp32
+ * accumulation of exact bf16-plane products.  Replaces
+ * INQAffine<float,int>::forward_impl, inq_affine.cpp:82-205. */
+int nbla_hip_inq_affine_f32(const float *x, float *W, int32_t *I, float *old_W,
+                            int32_t *old_I, const float *bias, float *y,
+                            int64_t M, int64_t K, int64_t N, int num_bits,
+                            int step, nbla_hip_bernoulli_fn draw,
+                            void *draw_ctx, void *workspace,
+                            size_t workspace_bytes, void *stream);
+
+size_t nbla_hip_inq_convolution_workspace_bytes(
+    int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
+    const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+    const int64_t *dilation, int64_t group, int step);
+
+/* INQConvolution forward.  Replaces INQConvolution<float,int>::forward_impl,
+ * src/nbla/function/generic/inq_convolution.cpp:104-238. */
+int nbla_hip_inq_convolution_f32(
+    const float *x, float *W, int32_t *I, float *old_W, int32_t *old_I,
+    const float *bias, float *y, int64_t outer, int64_t C, int nd,
+    const int64_t *in_sp, int64_t O, const int64_t *kernel, const int64_t *pad,
+    const int64_t *stride, const int64_t *dilation, int64_t group, int num_bits,
+    int step, nbla_hip_bernoulli_fn draw, void *draw_ctx, void *workspace,
+    size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

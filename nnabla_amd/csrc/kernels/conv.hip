@@ -7,23 +7,9 @@
 #include "common.hpp"
 #include "gemm_layout.hpp"
 #include "internal.hpp"
+#include "conv_geom.hpp"
 
 namespace nbla_hip {
-namespace {
-
-typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
-
-constexpr int kMaxSpatial = 3;
-
-// Geometry normalised to three spatial dimensions (leading ones of size 1).
-struct ConvGeom {
-  int64_t outer, C, O, group;
-  int in_sp[kMaxSpatial], k[kMaxSpatial], pad[kMaxSpatial], stride[kMaxSpatial], dil[kMaxSpatial],
-      out_sp[kMaxSpatial];
-  int64_t in_sp_size, out_sp_size, k_size;
-  int64_t Cg, Og, Kg; // per group: input channels, output channels, contraction length
-  int64_t M;          // outer * out_sp_size
-};
 
 // convolution.cpp:41-160
 int make_geom(ConvGeom &g, int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O, const int64_t *kernel,
@@ -76,6 +62,10 @@ int make_geom(ConvGeom &g, int64_t outer, int64_t C, int nd, const int64_t *in_s
   g.M = outer * g.out_sp_size;
   return NBLA_HIP_OK;
 }
+
+namespace {
+
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
 // Value of the unfolded matrix at (pixel m, column k) for group `grp`
 // (unfold_to_patches.cpp:103-194: zero where the tap falls into the padding).
@@ -160,6 +150,28 @@ __global__ __launch_bounds__(256) void im2col_f32(const float *__restrict__ x, f
   }
 }
 
+} // namespace
+
+int launch_im2col_split(const float *x, void *xsplit, const ConvGeom &g, int64_t grp, hipStream_t stream) {
+  const int64_t k_blocks = split_k_blocks(g.Kg);
+  const int64_t frags = split_row_blocks(g.M) * k_blocks;
+  hipLaunchKernelGGL(im2col_split, dim3((unsigned)ceil_div(frags, 4)), dim3(256), 0, stream, x,
+                     static_cast<uint4_t *>(xsplit), g, grp, k_blocks, frags);
+  NBLA_HIP_LAUNCH_CHECK("im2col_split");
+  return NBLA_HIP_OK;
+}
+
+int launch_im2col_f32(const float *x, float *col, const ConvGeom &g, int64_t grp, hipStream_t stream) {
+  int64_t blocks = ceil_div(g.M * g.Kg, 256);
+  if (blocks > 65536)
+    blocks = 65536;
+  hipLaunchKernelGGL(im2col_f32, dim3((unsigned)blocks), dim3(256), 0, stream, x, col, g, grp);
+  NBLA_HIP_LAUNCH_CHECK("im2col_f32");
+  return NBLA_HIP_OK;
+}
+
+namespace {
+
 struct ConvWorkspace {
   size_t bits_off, bits_stride, split_off, prep_off, count_off, col_off, total;
 };
@@ -227,21 +239,17 @@ int binary_conv_forward(const float *x, const float *W, float *Wb, float *alpha,
     const float *ag = alpha ? alpha + grp * g.Og : nullptr;
     const float *bg = bias ? bias + grp * g.Og : nullptr;
     if (use_bits) {
-      const int64_t k_blocks = split_k_blocks(g.Kg);
-      const int64_t frags = split_row_blocks(g.M) * k_blocks;
-      hipLaunchKernelGGL(im2col_split, dim3((unsigned)ceil_div(frags, 4)), dim3(256), 0, stream, x,
-                         reinterpret_cast<uint4_t *>(base + ws.split_off), g, grp, k_blocks, frags);
-      NBLA_HIP_LAUNCH_CHECK("im2col_split");
+      rc = launch_im2col_split(x, base + ws.split_off, g, grp, stream);
+      if (rc)
+        return rc;
       rc = launch_gemm_bits(base + ws.split_off,
                             reinterpret_cast<const uint32_t *>(base + ws.bits_off + grp * ws.bits_stride), ag, bg, yg,
                             g.M, g.Kg, g.Og, hw, g.O * hw, hw, true, stream);
     } else {
       float *col = reinterpret_cast<float *>(base + ws.total);
-      int64_t blocks = ceil_div(g.M * g.Kg, 256);
-      if (blocks > 65536)
-        blocks = 65536;
-      hipLaunchKernelGGL(im2col_f32, dim3((unsigned)blocks), dim3(256), 0, stream, x, col, g, grp);
-      NBLA_HIP_LAUNCH_CHECK("im2col_f32");
+      rc = launch_im2col_f32(x, col, g, grp, stream);
+      if (rc)
+        return rc;
       rc = launch_gemm_f32_mapped(col, Wb + grp * g.Og * g.Kg, true, ag, bg, yg, g.M, g.Kg, g.Og, hw, g.O * hw, hw,
                                   stream);
     }

@@ -28,6 +28,8 @@ EXPORTED = (
     "nbla_hip_binary_connect_affine_f32", "nbla_hip_affine_f32",
     "nbla_hip_convolution_output_shape", "nbla_hip_binary_convolution_workspace_bytes",
     "nbla_hip_binary_weight_convolution_f32", "nbla_hip_binary_connect_convolution_f32",
+    "nbla_hip_inq_workspace_bytes", "nbla_hip_inq_update_weights_f32", "nbla_hip_inq_affine_workspace_bytes",
+    "nbla_hip_inq_affine_f32", "nbla_hip_inq_convolution_workspace_bytes", "nbla_hip_inq_convolution_f32",
 )
 
 
@@ -52,7 +54,9 @@ def lib():
         L.nbla_hip_version.restype = ctypes.c_char_p
         for name in ("nbla_hip_min_max_quantize_workspace_bytes", "nbla_hip_packed_bits_bytes",
                      "nbla_hip_split_operand_bytes", "nbla_hip_binarize_workspace_bytes",
-                     "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_convolution_workspace_bytes"):
+                     "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_convolution_workspace_bytes",
+                     "nbla_hip_inq_workspace_bytes", "nbla_hip_inq_affine_workspace_bytes",
+                     "nbla_hip_inq_convolution_workspace_bytes"):
             getattr(L, name).restype = ctypes.c_size_t
         _lib = L
     return _lib
@@ -252,3 +256,61 @@ def binary_connect_convolution(x, W, bias=None, pad=None, stride=None, dilation=
     check(lib().nbla_hip_binary_connect_convolution_f32(_p(x), _p(W), _p(Wb), _p(bias), _p(y), *geom, q0, _p(ws),
                                                         ctypes.c_size_t(ws.numel()), _stream(stream)))
     return y, Wb
+
+
+# ---------------------------------------------------------------------------- INQ
+
+INQ_PRODUCT_ONLY, INQ_NO_SELECTION, INQ_FIX_ALL, INQ_LARGEST_ABS, INQ_RANDOM = -1, 0, 1, 2, 3
+BERNOULLI_FN = ctypes.CFUNCTYPE(None, ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint8), ctypes.c_int64)
+
+
+def _draw_callback(draw):
+    """Wraps a Python callable count -> sequence of 0/1 as the C callback of step 3."""
+    if draw is None:
+        return ctypes.cast(None, BERNOULLI_FN)
+
+    def cb(_ctx, out, count):
+        vals = draw(int(count))
+        for i in range(int(count)):
+            out[i] = int(vals[i])
+    return BERNOULLI_FN(cb)
+
+
+def inq_update_weights(W, I, old_W, old_I, num_bits, step, draw=None, stream=None):
+    """Steps A-C and F in place on W (fp32) and I (int32); returns a device tensor (n1, n2)."""
+    import torch
+    size = W.numel()
+    ws = _workspace(lib().nbla_hip_inq_workspace_bytes(_i64(size), int(step)), W)
+    n1n2 = torch.empty(2, dtype=torch.int32, device=W.device)
+    cb = _draw_callback(draw)
+    check(lib().nbla_hip_inq_update_weights_f32(_p(W), _p(I), _p(old_W), _p(old_I), _i64(size), int(num_bits),
+                                                int(step), cb, None, _p(n1n2), _p(ws), ctypes.c_size_t(ws.numel()),
+                                                _stream(stream)))
+    return n1n2
+
+
+def inq_affine(x, W, I, old_W, old_I, bias=None, num_bits=4, step=0, draw=None, stream=None):
+    """INQAffine forward; W, I, old_W, old_I are updated in place; returns y."""
+    import torch
+    M, K = x.shape
+    N = W.numel() // K
+    ws = _workspace(lib().nbla_hip_inq_affine_workspace_bytes(_i64(M), _i64(K), _i64(N), int(step)), x)
+    y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+    cb = _draw_callback(draw)
+    check(lib().nbla_hip_inq_affine_f32(_p(x), _p(W), _p(I), _p(old_W), _p(old_I), _p(bias), _p(y), _i64(M), _i64(K),
+                                        _i64(N), int(num_bits), int(step), cb, None, _p(ws),
+                                        ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return y
+
+
+def inq_convolution(x, W, I, old_W, old_I, bias=None, pad=None, stride=None, dilation=None, group=1, num_bits=4,
+                    step=0, draw=None, stream=None):
+    import torch
+    geom, yshape = _conv_geometry(x, W, pad, stride, dilation, group)
+    ws = _workspace(lib().nbla_hip_inq_convolution_workspace_bytes(*geom, int(step)), x)
+    y = torch.empty(yshape, dtype=torch.float32, device=x.device)
+    cb = _draw_callback(draw)
+    check(lib().nbla_hip_inq_convolution_f32(_p(x), _p(W), _p(I), _p(old_W), _p(old_I), _p(bias), _p(y), *geom,
+                                             int(num_bits), int(step), cb, None, _p(ws), ctypes.c_size_t(ws.numel()),
+                                             _stream(stream)))
+    return y

@@ -38,6 +38,7 @@ def lib():
             build()
         _lib = ctypes.CDLL(_LIB_PATH)
         _lib.orc_inq_create.restype = ctypes.c_void_p
+        _lib.orc_bernoulli_create.restype = ctypes.c_void_p
         _lib.orc_inq_counter.restype = ctypes.c_long
     return _lib
 
@@ -284,3 +285,20 @@ class Inq(object):
         y = np.empty(yshape, np.float32)
         _check(lib().orc_inq_convolution(self._h, _fp(x), _fp(W), _ip(I), _fp(b), _fp(y), *tail), "inq_convolution")
         return y
+
+
+class Bernoulli(object):
+    """std::mt19937(seed) + std::bernoulli_distribution(0.5): the draw stream of INQ's random selection."""
+
+    def __init__(self, seed):
+        self._h = ctypes.c_void_p(lib().orc_bernoulli_create(int(seed)))
+
+    def draw(self, count):
+        out = np.empty(int(count), np.uint8)
+        lib().orc_bernoulli_draw(self._h, out.ctypes.data_as(ctypes.POINTER(ctypes.c_ubyte)), ctypes.c_long(int(count)))
+        return out
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().orc_inq_destroy(self._h)
+            self._h = None

@@ -769,6 +769,21 @@ int orc_inq_commit(void *h, const float *weights, const int *indicators) {
   return ORC_OK;
 }
 
+// A stand-alone Bernoulli(0.5) stream identical to the one INQ's "random" selection consumes
+// (std::mt19937 + std::bernoulli_distribution, inq_affine.cpp:70-74,147): lets a test feed the same draws to
+// an implementation that takes them through a callback.
+void *orc_bernoulli_create(int seed) {
+  InqState *s = new InqState();
+  s->rgen = std::mt19937((unsigned)seed);
+  s->rdist = std::bernoulli_distribution(0.5);
+  return s;
+}
+void orc_bernoulli_draw(void *h, unsigned char *out, long count) {
+  InqState *s = static_cast<InqState *>(h);
+  for (long i = 0; i < count; ++i)
+    out[i] = s->rdist(s->rgen) ? 1 : 0;
+}
+
 // The two libm-dependent decisions of step C, exposed for table checks:
 // e(a) = floor(log2f(a)) + (frac >= (float)log2(1.5)) for a weight (:176-179)
 int orc_inq_exponent(float a) {

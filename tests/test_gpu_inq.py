@@ -1,0 +1,146 @@
+"""INQAffine / INQConvolution on the GPU against the CPU oracle: quantized weights and indicators bit-exact over a
+sequence of minibatches (restore, selection, quantization, snapshot), outputs within 1e-4 (expected ~1e-6)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from nnabla_amd import kernels
+from util import bits_equal, first_mismatch, max_rel_err, to_np
+
+pytestmark = pytest.mark.gpu
+TOL, TIGHT = 1e-4, 5e-6
+
+
+def _dev(x, dev):
+    return torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+
+
+def _step_for(counter, inq_iterations, algo):
+    """The host-side mapping of inq_affine.cpp:104-113 from the minibatch counter to the C-ABI's step."""
+    if counter in inq_iterations:
+        if inq_iterations[-1] == counter:
+            return kernels.INQ_FIX_ALL
+        return kernels.INQ_LARGEST_ABS if algo == "largest_abs" else kernels.INQ_RANDOM
+    return kernels.INQ_NO_SELECTION
+
+
+def _cut_point_values(n):
+    """Weights on and around the 1.5 * 2^k decision points and the pruning thresholds."""
+    ks = np.arange(-12, 3)
+    base = (1.5 * 2.0 ** ks).astype(np.float32)
+    vals = [base, np.nextafter(base, np.float32(0)), np.nextafter(base, np.float32(9)), (2.0 ** ks).astype(np.float32),
+            np.nextafter((2.0 ** ks).astype(np.float32), np.float32(0))]
+    v = np.concatenate(vals)
+    v = np.concatenate([v, -v, np.array([0.0, -0.0], np.float32)])
+    return np.resize(v, n).astype(np.float32)
+
+
+@pytest.mark.parametrize("num_bits", [2, 3, 4, 6])
+@pytest.mark.parametrize("algo", ["largest_abs", "random"])
+def test_inq_weight_sequence_matches_oracle(dev, num_bits, algo):
+    rng = np.random.RandomState(313)
+    shape = (70, 45)
+    W = (rng.randn(*shape) * 0.05).astype(np.float32)
+    W.ravel()[:200] = _cut_point_values(200) * 0.1
+    its = (0, 2, 3, 5)
+    seed = 11
+    inq = oracle.Inq(W.size, num_bits, its, algo, seed)
+    stream = oracle.Bernoulli(seed)
+    Wc, Ic = W.copy(), np.zeros(shape, np.int32)
+    Wd, Id = _dev(W, dev), torch.zeros(shape, dtype=torch.int32, device=dev)
+    oldW, oldI = torch.zeros_like(Wd), torch.zeros_like(Id)
+    for it in range(7):
+        n1, n2 = inq.quantize_weights(Wc, Ic)
+        inq.commit(Wc, Ic)
+        step = _step_for(it, its, algo)
+        n1n2 = kernels.inq_update_weights(Wd, Id, oldW, oldI, num_bits, step, draw=stream.draw)
+        assert tuple(to_np(n1n2)) == (n1, n2)
+        assert np.array_equal(to_np(Id), Ic), "indicators differ at minibatch %d" % it
+        assert bits_equal(to_np(Wd), Wc), "minibatch %d: %s" % (it, first_mismatch(to_np(Wd), Wc))
+        assert bits_equal(to_np(oldW), Wc) and np.array_equal(to_np(oldI), Ic)
+        # the "optimizer" moves every weight; fixed ones must come back on the next forward
+        upd = (rng.randn(*shape) * 0.01).astype(np.float32)
+        Wc += upd
+        Wd += _dev(upd, dev)
+    assert Ic.min() == 1
+
+
+def test_inq_largest_abs_tie_free_half_selection(dev):
+    """Exactly the num_learnable // 2 largest |w| become fixed, including the single-element quirk of the loop."""
+    for size in (1, 2, 3, 101, 4096):
+        rng = np.random.RandomState(size)
+        W = (rng.permutation(size).astype(np.float32) + 1) * np.where(rng.rand(size) < 0.5, -1, 1) * 0.001
+        W = W.astype(np.float32)
+        inq = oracle.Inq(size, 4, (0, 9), "largest_abs")
+        Wc, Ic = W.copy(), np.zeros(size, np.int32)
+        inq.quantize_weights(Wc, Ic)
+        Wd, Id = _dev(W, dev), torch.zeros(size, dtype=torch.int32, device=dev)
+        kernels.inq_update_weights(Wd, Id, torch.zeros_like(Wd), torch.zeros_like(Id), 4, kernels.INQ_LARGEST_ABS)
+        assert np.array_equal(to_np(Id), Ic) and bits_equal(to_np(Wd), Wc)
+        assert Ic.sum() == max(size // 2, 1)
+
+
+@pytest.mark.parametrize("M,K,N", [(2, 3, 4), (33, 100, 130), (64, 256, 192), (300, 520, 257)])
+def test_inq_affine_all_fixed_and_partially_fixed(dev, M, K, N):
+    rng = np.random.RandomState(5)
+    x = rng.randn(M, K).astype(np.float32)
+    W = (rng.randn(K, N) * 0.02).astype(np.float32)
+    b = rng.randn(N).astype(np.float32)
+    for its, nsteps in (((0,), 1), ((0, 5), 2)):        # all fixed at once / half fixed then a plain minibatch
+        inq = oracle.Inq(W.size, 4, its, "largest_abs")
+        Wc, Ic = W.copy(), np.zeros(W.shape, np.int32)
+        Wd, Id = _dev(W, dev), torch.zeros(W.shape, dtype=torch.int32, device=dev)
+        oldW, oldI = torch.zeros_like(Wd), torch.zeros_like(Id)
+        for it in range(nsteps):
+            ref_y = inq.affine(x, Wc, Ic, b)
+            y = kernels.inq_affine(_dev(x, dev), Wd, Id, oldW, oldI, _dev(b, dev), 4,
+                                   _step_for(it, its, "largest_abs"))
+            assert bits_equal(to_np(Wd), Wc) and np.array_equal(to_np(Id), Ic)
+            y64 = x.astype(np.float64) @ Wc.astype(np.float64) + b
+            assert max_rel_err(to_np(y), ref_y) <= TOL
+            assert max_rel_err(to_np(y), y64) <= TIGHT
+        # recompute: the product alone on the weights left by the forward
+        y2 = kernels.inq_affine(_dev(x, dev), Wd, Id, oldW, oldI, _dev(b, dev), 4, kernels.INQ_PRODUCT_ONLY)
+        assert bits_equal(to_np(y2), to_np(y)) and bits_equal(to_np(Wd), Wc)
+
+
+def test_inq_convolution_matches_oracle(dev):
+    rng = np.random.RandomState(9)
+    for xs, ws, pad, stride, group in [((2, 4, 9, 9), (6, 4, 3, 3), (1, 1), (1, 1), 1),
+                                       ((3, 6, 8, 7), (4, 3, 3, 2), (1, 0), (2, 1), 2)]:
+        x = rng.randn(*xs).astype(np.float32)
+        W = (rng.randn(*ws) * 0.05).astype(np.float32)
+        b = rng.randn(ws[0]).astype(np.float32)
+        its = (0, 1)
+        inq = oracle.Inq(W.size, 4, its, "largest_abs")
+        Wc, Ic = W.copy(), np.zeros(ws, np.int32)
+        Wd, Id = _dev(W, dev), torch.zeros(ws, dtype=torch.int32, device=dev)
+        oldW, oldI = torch.zeros_like(Wd), torch.zeros_like(Id)
+        for it in range(2):
+            ref_y = inq.convolution(x, Wc, Ic, b, pad, stride, None, group)
+            y = kernels.inq_convolution(_dev(x, dev), Wd, Id, oldW, oldI, _dev(b, dev), pad, stride, None, group, 4,
+                                        _step_for(it, its, "largest_abs"))
+            assert bits_equal(to_np(Wd), Wc) and np.array_equal(to_np(Id), Ic)
+            assert max_rel_err(to_np(y), ref_y) <= TIGHT
+
+
+def test_inq_config5_layer(dev):
+    """The INQAffine layer of BASELINE config 5: x [1024,4096], W [4096,4096] ~ N(0, 0.02^2), num_bits 4, every
+    weight fixed.  Weights bit-exact against the oracle; the output against float64 on sampled entries and against
+    the oracle's fp32 GEMM on the first 64 rows."""
+    rng = np.random.default_rng(313)
+    x = rng.standard_normal((1024, 4096), dtype=np.float32)
+    W = rng.standard_normal((4096, 4096), dtype=np.float32) * np.float32(0.02)
+    inq = oracle.Inq(W.size, 4, (0,), "largest_abs")
+    Wc, Ic = W.copy(), np.zeros(W.shape, np.int32)
+    ref_y = inq.affine(x[:64], Wc, Ic, None)
+    Wd, Id = _dev(W, dev), torch.zeros(W.shape, dtype=torch.int32, device=dev)
+    y = to_np(kernels.inq_affine(_dev(x, dev), Wd, Id, torch.zeros_like(Wd), torch.zeros_like(Id), None, 4,
+                                 kernels.INQ_FIX_ALL))
+    assert bits_equal(to_np(Wd), Wc), first_mismatch(to_np(Wd), Wc)
+    assert np.array_equal(to_np(Id), Ic) and Ic.min() == 1
+    assert max_rel_err(y[:64], ref_y) <= TOL
+    rows, cols = rng.choice(1024, 32, replace=False), rng.choice(4096, 64, replace=False)
+    ref = x[rows].astype(np.float64) @ Wc[:, cols].astype(np.float64)
+    assert np.abs(y[np.ix_(rows, cols)] - ref).max() / np.abs(ref).max() <= TIGHT
