@@ -286,6 +286,32 @@ int nbla_hip_inq_convolution_f32(
     int step, nbla_hip_bernoulli_fn draw, void *draw_ctx, void *workspace,
     size_t workspace_bytes, void *stream);
 
+/* ------------------------------------------- device memory and array storage */
+
+/* Thin wrappers the host layer (HipMemory, HipArray, the Hip backend singleton)
+ * uses so that it needs no HIP headers: the counterparts of malloc/free in
+ * src/nbla/memory/cpu_memory.cpp:49-80, of CpuArray::copy_from/zero/fill in
+ * src/nbla/array/cpu_array.cpp and of BackendBase::device_synchronize
+ * (include/nbla/backend_base.hpp:32-91).  `dtype` arguments are nbla::dtypes
+ * codes (include/nbla/dtypes.hpp:32-64).  memcpy kind: 1 = host to device,
+ * 2 = device to host (both complete before returning), 3 = device to device. */
+int nbla_hip_get_device_count(int *count);
+int nbla_hip_set_device(int device);
+int nbla_hip_malloc(void **ptr, size_t bytes, int device);
+int nbla_hip_free(void *ptr, int device);
+int nbla_hip_mem_info(int device, size_t *free_bytes, size_t *total_bytes);
+int nbla_hip_memcpy(void *dst, const void *src, size_t bytes, int kind,
+                    void *stream);
+int nbla_hip_device_synchronize(int device);
+int nbla_hip_stream_synchronize(void *stream);
+int nbla_hip_fill(void *dst, int dtype, size_t size, float value, void *stream);
+int nbla_hip_cast(const void *src, int src_dtype, void *dst, int dst_dtype,
+                  size_t size, void *stream);
+
+/* y = max(0, x).  Replaces ReLU<float>::forward_impl,
+ * src/nbla/function/generic/relu.cpp (std::max(T(0), x)). */
+int nbla_hip_relu_f32(const float *x, float *y, size_t size, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

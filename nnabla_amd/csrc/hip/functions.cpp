@@ -1,0 +1,219 @@
+// forward_impl of the "hip:float" Function classes: fetch device pointers through the Variable interface, obtain
+// scratch from the backend's caching allocator, call the kernel library.
+#include <nbla/hip/common.hpp>
+#include <nbla/hip/function/binary.hpp>
+#include <nbla/hip/function/inq.hpp>
+#include <nbla/hip/function/quantize.hpp>
+
+namespace nbla {
+
+namespace {
+vector<int64_t> to_i64(const Shape_t &s) { return vector<int64_t>(s.begin(), s.end()); }
+} // namespace
+
+// ---------------------------------------------------------------- quantizers
+template <typename T>
+void FixedPointQuantizeHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  NBLA_HIP_CALL(nbla_hip_fixed_point_quantize_f32(x, y, (size_t)inputs[0]->size(), this->sign_, this->n_, this->delta_,
+                                                  nullptr));
+}
+
+template <typename T> void Pow2QuantizeHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  NBLA_HIP_CALL(nbla_hip_pow2_quantize_f32(x, y, (size_t)inputs[0]->size(), this->sign_, this->with_zero_, this->n_,
+                                           this->m_, nullptr));
+}
+
+template <typename T> void MinMaxQuantizeHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const vector<int64_t> xshape = to_i64(inputs[0]->shape()), qshape = to_i64(inputs[1]->shape());
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  // qr_min / qr_max are running state: updated in place, as the reference updates its parameters
+  T *qr_min = inputs[1]->cast_data_and_get_pointer<T>(this->ctx_);
+  T *qr_max = inputs[2]->cast_data_and_get_pointer<T>(this->ctx_);
+  const T *ql_min = inputs[3]->get_data_pointer<T>(this->ctx_);
+  const T *ql_max = inputs[4]->get_data_pointer<T>(this->ctx_);
+  T *scale = this->scale_sptr_->template cast_data_and_get_pointer<T>(this->ctx_, true);
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  HipWorkspace ws(nbla_hip_min_max_quantize_workspace_bytes(xshape.data(), (int)xshape.size(), qshape.data()),
+                  this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_min_max_quantize_f32(x, y, xshape.data(), (int)xshape.size(), qshape.data(), qr_min, qr_max,
+                                              ql_min, ql_max, scale, this->decay_, this->x_min_max_, this->ema_,
+                                              this->eps_, ws.pointer(), ws.bytes(), nullptr));
+}
+
+// ------------------------------------------------------------- binary affine
+template <typename T>
+void BinaryWeightAffineHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const AffineShapes &s = this->shapes_;
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
+  T *wb = inputs[2]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  T *alpha = inputs[3]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  const T *b = inputs.size() == 5 ? inputs[4]->get_data_pointer<T>(this->ctx_) : nullptr;
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  HipWorkspace ws(nbla_hip_binary_affine_workspace_bytes(s.i_row, s.i_col, s.w_col), this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_binary_weight_affine_f32(x, w, wb, alpha, b, y, s.i_row, s.i_col, s.w_col,
+                                                  this->quantize_zero_to_, ws.pointer(), ws.bytes(), nullptr));
+}
+
+template <typename T>
+void BinaryConnectAffineHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const AffineShapes &s = this->shapes_;
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
+  T *wb = inputs[2]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  const T *b = inputs.size() == 4 ? inputs[3]->get_data_pointer<T>(this->ctx_) : nullptr;
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  HipWorkspace ws(nbla_hip_binary_affine_workspace_bytes(s.i_row, s.i_col, s.w_col), this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_binary_connect_affine_f32(x, w, wb, b, y, s.i_row, s.i_col, s.w_col, this->quantize_zero_to_,
+                                                   ws.pointer(), ws.bytes(), nullptr));
+}
+
+// -------------------------------------------------------- binary convolution
+template <typename T>
+void BinaryWeightConvolutionHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const ConvShapes &s = this->shapes_;
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
+  T *wb = inputs[2]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  T *alpha = inputs[3]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  const T *b = inputs.size() == 5 ? inputs[4]->get_data_pointer<T>(this->ctx_) : nullptr;
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  HipWorkspace ws(nbla_hip_binary_convolution_workspace_bytes(
+                      s.outer, s.channels_i, s.spatial_dims, s.spatial_i.data(), s.channels_o, s.kernel.data(),
+                      s.pad.data(), s.stride.data(), s.dilation.data(), s.group, this->quantize_zero_to_),
+                  this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_binary_weight_convolution_f32(
+      x, w, wb, alpha, b, y, s.outer, s.channels_i, s.spatial_dims, s.spatial_i.data(), s.channels_o, s.kernel.data(),
+      s.pad.data(), s.stride.data(), s.dilation.data(), s.group, this->quantize_zero_to_, ws.pointer(), ws.bytes(),
+      nullptr));
+}
+
+template <typename T>
+void BinaryConnectConvolutionHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const ConvShapes &s = this->shapes_;
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
+  T *wb = inputs[2]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  const T *b = inputs.size() == 4 ? inputs[3]->get_data_pointer<T>(this->ctx_) : nullptr;
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  HipWorkspace ws(nbla_hip_binary_convolution_workspace_bytes(
+                      s.outer, s.channels_i, s.spatial_dims, s.spatial_i.data(), s.channels_o, s.kernel.data(),
+                      s.pad.data(), s.stride.data(), s.dilation.data(), s.group, this->quantize_zero_to_),
+                  this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_binary_connect_convolution_f32(
+      x, w, wb, b, y, s.outer, s.channels_i, s.spatial_dims, s.spatial_i.data(), s.channels_o, s.kernel.data(),
+      s.pad.data(), s.stride.data(), s.dilation.data(), s.group, this->quantize_zero_to_, ws.pointer(), ws.bytes(),
+      nullptr));
+}
+
+// ----------------------------------------------------------------------- INQ
+namespace {
+// The Bernoulli stream of inq_affine.cpp:147: rdist_(rgen), one draw per learnable weight.
+void draw_bernoulli(void *ctx, uint8_t *out, int64_t count) {
+  InqState *s = static_cast<InqState *>(ctx);
+  std::mt19937 &gen = s->generator();
+  for (int64_t i = 0; i < count; ++i)
+    out[i] = s->rdist_(gen) ? 1 : 0;
+}
+} // namespace
+
+template <typename T, typename T1>
+void INQAffineHip<T, T1>::run(const Variables &inputs, const Variables &outputs, int step) {
+  hip_set_device(this->ctx_);
+  const AffineShapes &s = this->shapes_;
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  T *w = inputs[1]->cast_data_and_get_pointer<T>(this->ctx_);
+  T1 *ind = inputs[2]->cast_data_and_get_pointer<T1>(this->ctx_);
+  T *old_w = this->old_weights_.template cast_data_and_get_pointer<T>(this->ctx_);
+  T1 *old_i = this->old_indicators_.template cast_data_and_get_pointer<T1>(this->ctx_);
+  const T *b = inputs.size() == 4 ? inputs[3]->get_data_pointer<T>(this->ctx_) : nullptr;
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  HipWorkspace ws(nbla_hip_inq_affine_workspace_bytes(s.i_row, s.i_col, s.w_col, step), this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_inq_affine_f32(x, w, ind, old_w, old_i, b, y, s.i_row, s.i_col, s.w_col, this->num_bits_,
+                                        step, draw_bernoulli, static_cast<InqState *>(this), ws.pointer(), ws.bytes(),
+                                        nullptr));
+}
+template <typename T, typename T1>
+void INQAffineHip<T, T1>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  run(inputs, outputs, this->current_step());
+  this->minibatch_counter_++; // inq_affine.cpp:200
+}
+template <typename T, typename T1>
+void INQAffineHip<T, T1>::recompute_impl(const Variables &inputs, const Variables &outputs) {
+  run(inputs, outputs, -1); // inq_affine.cpp:208-216: the product alone
+}
+
+template <typename T, typename T1>
+void INQConvolutionHip<T, T1>::run(const Variables &inputs, const Variables &outputs, int step) {
+  hip_set_device(this->ctx_);
+  const ConvShapes &s = this->shapes_;
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  T *w = inputs[1]->cast_data_and_get_pointer<T>(this->ctx_);
+  T1 *ind = inputs[2]->cast_data_and_get_pointer<T1>(this->ctx_);
+  T *old_w = this->old_weights_.template cast_data_and_get_pointer<T>(this->ctx_);
+  T1 *old_i = this->old_indicators_.template cast_data_and_get_pointer<T1>(this->ctx_);
+  const T *b = inputs.size() == 4 ? inputs[3]->get_data_pointer<T>(this->ctx_) : nullptr;
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  HipWorkspace ws(nbla_hip_inq_convolution_workspace_bytes(s.outer, s.channels_i, s.spatial_dims, s.spatial_i.data(),
+                                                           s.channels_o, s.kernel.data(), s.pad.data(),
+                                                           s.stride.data(), s.dilation.data(), s.group, step),
+                  this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_inq_convolution_f32(x, w, ind, old_w, old_i, b, y, s.outer, s.channels_i, s.spatial_dims,
+                                             s.spatial_i.data(), s.channels_o, s.kernel.data(), s.pad.data(),
+                                             s.stride.data(), s.dilation.data(), s.group, this->num_bits_, step,
+                                             draw_bernoulli, static_cast<InqState *>(this), ws.pointer(), ws.bytes(),
+                                             nullptr));
+}
+template <typename T, typename T1>
+void INQConvolutionHip<T, T1>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  run(inputs, outputs, this->current_step());
+  this->minibatch_counter_++;
+}
+template <typename T, typename T1>
+void INQConvolutionHip<T, T1>::recompute_impl(const Variables &inputs, const Variables &outputs) {
+  run(inputs, outputs, -1);
+}
+
+// ------------------------------------------------------------ Affine and ReLU
+template <typename T> void AffineHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const AffineShapes &s = this->shapes_;
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
+  const T *b = inputs.size() == 3 ? inputs[2]->get_data_pointer<T>(this->ctx_) : nullptr;
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  NBLA_HIP_CALL(nbla_hip_affine_f32(x, w, b, y, s.i_row, s.i_col, s.w_col, nullptr));
+}
+
+template <typename T> void ReLUHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, !this->inplace_);
+  NBLA_HIP_CALL(nbla_hip_relu_f32(x, y, (size_t)inputs[0]->size(), nullptr));
+}
+
+// explicit instantiations for the "float" type config (function_types.yaml:483-509)
+template class FixedPointQuantizeHip<float>;
+template class Pow2QuantizeHip<float>;
+template class MinMaxQuantizeHip<float>;
+template class BinaryWeightAffineHip<float>;
+template class BinaryConnectAffineHip<float>;
+template class BinaryWeightConvolutionHip<float>;
+template class BinaryConnectConvolutionHip<float>;
+template class INQAffineHip<float, int>;
+template class INQConvolutionHip<float, int>;
+template class AffineHip<float>;
+template class ReLUHip<float>;
+
+} // namespace nbla

@@ -1,0 +1,56 @@
+// "hip:float" implementations of the binary-weight functions.
+#ifndef NBLA_HIP_FUNCTION_BINARY_HPP_
+#define NBLA_HIP_FUNCTION_BINARY_HPP_
+
+#include <nbla/function/binary_connect_affine.hpp>
+#include <nbla/function/binary_connect_convolution.hpp>
+#include <nbla/function/binary_weight_affine.hpp>
+#include <nbla/function/binary_weight_convolution.hpp>
+#include <nbla/hip/hip.hpp>
+
+namespace nbla {
+
+template <typename T> class BinaryWeightAffineHip : public BinaryWeightAffine<T> {
+public:
+  BinaryWeightAffineHip(const Context &ctx, int base_axis, float quantize_zero_to)
+      : BinaryWeightAffine<T>(ctx, base_axis, quantize_zero_to) {}
+  virtual vector<string> allowed_array_classes() { return SingletonManager::get<Hip>()->array_classes(); }
+
+protected:
+  virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+};
+
+template <typename T> class BinaryConnectAffineHip : public BinaryConnectAffine<T> {
+public:
+  BinaryConnectAffineHip(const Context &ctx, int base_axis, float quantize_zero_to)
+      : BinaryConnectAffine<T>(ctx, base_axis, quantize_zero_to) {}
+  virtual vector<string> allowed_array_classes() { return SingletonManager::get<Hip>()->array_classes(); }
+
+protected:
+  virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+};
+
+template <typename T> class BinaryWeightConvolutionHip : public BinaryWeightConvolution<T> {
+public:
+  BinaryWeightConvolutionHip(const Context &ctx, int base_axis, const vector<int> &pad, const vector<int> &stride,
+                             const vector<int> &dilation, int group, float quantize_zero_to)
+      : BinaryWeightConvolution<T>(ctx, base_axis, pad, stride, dilation, group, quantize_zero_to) {}
+  virtual vector<string> allowed_array_classes() { return SingletonManager::get<Hip>()->array_classes(); }
+
+protected:
+  virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+};
+
+template <typename T> class BinaryConnectConvolutionHip : public BinaryConnectConvolution<T> {
+public:
+  BinaryConnectConvolutionHip(const Context &ctx, int base_axis, const vector<int> &pad, const vector<int> &stride,
+                              const vector<int> &dilation, int group, float quantize_zero_to)
+      : BinaryConnectConvolution<T>(ctx, base_axis, pad, stride, dilation, group, quantize_zero_to) {}
+  virtual vector<string> allowed_array_classes() { return SingletonManager::get<Hip>()->array_classes(); }
+
+protected:
+  virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+};
+
+} // namespace nbla
+#endif

@@ -1,0 +1,234 @@
+// Device memory management and the storage-level array operations (fill, dtype
+// cast, ReLU) that the HipArray classes of the host layer are built on.
+#include "common.hpp"
+
+namespace nbla_hip {
+namespace {
+
+constexpr int kBlk = 256;
+
+unsigned grid_for(size_t size) {
+  size_t b = (size + kBlk - 1) / kBlk;
+  return (unsigned)(b > 16384 ? 16384 : (b < 1 ? 1 : b));
+}
+
+template <typename T> __global__ __launch_bounds__(kBlk) void fill_kernel(T *dst, size_t size, T value) {
+  for (size_t i = (size_t)blockIdx.x * kBlk + threadIdx.x; i < size; i += (size_t)gridDim.x * kBlk)
+    dst[i] = value;
+}
+
+template <typename Ta, typename Tb>
+__global__ __launch_bounds__(kBlk) void cast_kernel(const Ta *__restrict__ src, Tb *__restrict__ dst, size_t size) {
+  for (size_t i = (size_t)blockIdx.x * kBlk + threadIdx.x; i < size; i += (size_t)gridDim.x * kBlk)
+    dst[i] = static_cast<Tb>(src[i]);
+}
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(kBlk) void relu_kernel(const float *__restrict__ x, float *__restrict__ y, size_t n4,
+                                                    size_t size, int vec) {
+  if (vec) {
+    for (size_t i = (size_t)blockIdx.x * kBlk + threadIdx.x; i < n4; i += (size_t)gridDim.x * kBlk) {
+      float4_t v = reinterpret_cast<const float4_t *>(x)[i];
+      // std::max(T(0), x): zero for negatives and for NaN-free -0.0 keeps +0.0
+      v.x = v.x > 0.0f ? v.x : 0.0f;
+      v.y = v.y > 0.0f ? v.y : 0.0f;
+      v.z = v.z > 0.0f ? v.z : 0.0f;
+      v.w = v.w > 0.0f ? v.w : 0.0f;
+      reinterpret_cast<float4_t *>(y)[i] = v;
+    }
+    if (blockIdx.x == 0) {
+      const size_t i = 4 * n4 + threadIdx.x;
+      if (i < size)
+        y[i] = x[i] > 0.0f ? x[i] : 0.0f;
+    }
+  } else {
+    for (size_t i = (size_t)blockIdx.x * kBlk + threadIdx.x; i < size; i += (size_t)gridDim.x * kBlk)
+      y[i] = x[i] > 0.0f ? x[i] : 0.0f;
+  }
+}
+
+// nbla::dtypes codes (numpy compatible)
+enum { DT_BOOL = 0, DT_BYTE, DT_UBYTE, DT_SHORT, DT_USHORT, DT_INT, DT_UINT, DT_LONG, DT_ULONG, DT_LONGLONG,
+       DT_ULONGLONG, DT_FLOAT, DT_DOUBLE };
+
+template <typename Ta> int cast_from(const void *src, void *dst, int dst_dtype, size_t size, hipStream_t s) {
+  const Ta *p = static_cast<const Ta *>(src);
+  const dim3 g(grid_for(size)), b(kBlk);
+  switch (dst_dtype) {
+  case DT_BOOL: hipLaunchKernelGGL((cast_kernel<Ta, bool>), g, b, 0, s, p, static_cast<bool *>(dst), size); break;
+  case DT_BYTE: hipLaunchKernelGGL((cast_kernel<Ta, signed char>), g, b, 0, s, p, static_cast<signed char *>(dst), size); break;
+  case DT_UBYTE: hipLaunchKernelGGL((cast_kernel<Ta, unsigned char>), g, b, 0, s, p, static_cast<unsigned char *>(dst), size); break;
+  case DT_SHORT: hipLaunchKernelGGL((cast_kernel<Ta, short>), g, b, 0, s, p, static_cast<short *>(dst), size); break;
+  case DT_USHORT: hipLaunchKernelGGL((cast_kernel<Ta, unsigned short>), g, b, 0, s, p, static_cast<unsigned short *>(dst), size); break;
+  case DT_INT: hipLaunchKernelGGL((cast_kernel<Ta, int>), g, b, 0, s, p, static_cast<int *>(dst), size); break;
+  case DT_UINT: hipLaunchKernelGGL((cast_kernel<Ta, unsigned int>), g, b, 0, s, p, static_cast<unsigned int *>(dst), size); break;
+  case DT_LONG:
+  case DT_LONGLONG: hipLaunchKernelGGL((cast_kernel<Ta, long long>), g, b, 0, s, p, static_cast<long long *>(dst), size); break;
+  case DT_ULONG:
+  case DT_ULONGLONG: hipLaunchKernelGGL((cast_kernel<Ta, unsigned long long>), g, b, 0, s, p, static_cast<unsigned long long *>(dst), size); break;
+  case DT_FLOAT: hipLaunchKernelGGL((cast_kernel<Ta, float>), g, b, 0, s, p, static_cast<float *>(dst), size); break;
+  case DT_DOUBLE: hipLaunchKernelGGL((cast_kernel<Ta, double>), g, b, 0, s, p, static_cast<double *>(dst), size); break;
+  default: return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "unsupported destination dtype %d.", dst_dtype);
+  }
+  NBLA_HIP_LAUNCH_CHECK("cast");
+  return NBLA_HIP_OK;
+}
+
+template <typename T> int fill_as(void *dst, size_t size, float value, hipStream_t s) {
+  hipLaunchKernelGGL(fill_kernel<T>, dim3(grid_for(size)), dim3(kBlk), 0, s, static_cast<T *>(dst), size,
+                     static_cast<T>(value));
+  NBLA_HIP_LAUNCH_CHECK("fill");
+  return NBLA_HIP_OK;
+}
+
+size_t dtype_bytes(int dtype) {
+  switch (dtype) {
+  case DT_BOOL: case DT_BYTE: case DT_UBYTE: return 1;
+  case DT_SHORT: case DT_USHORT: return 2;
+  case DT_INT: case DT_UINT: case DT_FLOAT: return 4;
+  case DT_LONG: case DT_ULONG: case DT_LONGLONG: case DT_ULONGLONG: case DT_DOUBLE: return 8;
+  }
+  return 0;
+}
+
+} // namespace
+} // namespace nbla_hip
+
+using namespace nbla_hip;
+
+extern "C" {
+
+int nbla_hip_get_device_count(int *count) {
+  hipError_t e = hipGetDeviceCount(count);
+  if (e != hipSuccess) {
+    *count = 0;
+    return fail_hip(e, "hipGetDeviceCount");
+  }
+  return NBLA_HIP_OK;
+}
+
+int nbla_hip_set_device(int device) {
+  hipError_t e = hipSetDevice(device);
+  return e == hipSuccess ? NBLA_HIP_OK : fail_hip(e, "hipSetDevice");
+}
+
+int nbla_hip_malloc(void **ptr, size_t bytes, int device) {
+  hipError_t e = hipSetDevice(device);
+  if (e == hipSuccess)
+    e = hipMalloc(ptr, bytes ? bytes : 1);
+  if (e != hipSuccess) {
+    *ptr = nullptr;
+    (void)hipGetLastError(); // a failed allocation must not poison the next call
+    return fail_hip(e, "hipMalloc");
+  }
+  return NBLA_HIP_OK;
+}
+
+int nbla_hip_free(void *ptr, int device) {
+  if (!ptr)
+    return NBLA_HIP_OK;
+  hipError_t e = hipSetDevice(device);
+  if (e == hipSuccess)
+    e = hipFree(ptr);
+  return e == hipSuccess ? NBLA_HIP_OK : fail_hip(e, "hipFree");
+}
+
+int nbla_hip_mem_info(int device, size_t *free_bytes, size_t *total_bytes) {
+  hipError_t e = hipSetDevice(device);
+  if (e == hipSuccess)
+    e = hipMemGetInfo(free_bytes, total_bytes);
+  return e == hipSuccess ? NBLA_HIP_OK : fail_hip(e, "hipMemGetInfo");
+}
+
+int nbla_hip_memcpy(void *dst, const void *src, size_t bytes, int kind, void *stream) {
+  if (bytes == 0)
+    return NBLA_HIP_OK;
+  hipMemcpyKind k;
+  switch (kind) {
+  case 1: k = hipMemcpyHostToDevice; break;
+  case 2: k = hipMemcpyDeviceToHost; break;
+  case 3: k = hipMemcpyDeviceToDevice; break;
+  default: return fail(NBLA_HIP_ERR_VALUE, "invalid memcpy kind %d.", kind);
+  }
+  hipError_t e = hipMemcpyAsync(dst, src, bytes, k, as_stream(stream));
+  if (e == hipSuccess && k != hipMemcpyDeviceToDevice)
+    e = hipStreamSynchronize(as_stream(stream)); // host buffers are pageable: complete before returning
+  return e == hipSuccess ? NBLA_HIP_OK : fail_hip(e, "hipMemcpyAsync");
+}
+
+int nbla_hip_device_synchronize(int device) {
+  hipError_t e = hipSetDevice(device);
+  if (e == hipSuccess)
+    e = hipDeviceSynchronize();
+  return e == hipSuccess ? NBLA_HIP_OK : fail_hip(e, "hipDeviceSynchronize");
+}
+
+int nbla_hip_stream_synchronize(void *stream) {
+  hipError_t e = hipStreamSynchronize(as_stream(stream));
+  return e == hipSuccess ? NBLA_HIP_OK : fail_hip(e, "hipStreamSynchronize");
+}
+
+int nbla_hip_fill(void *dst, int dtype, size_t size, float value, void *stream_) {
+  if (size == 0)
+    return NBLA_HIP_OK;
+  hipStream_t s = as_stream(stream_);
+  if (value == 0.0f) { // all-zero bytes for every dtype
+    const size_t bytes = size * dtype_bytes(dtype);
+    if (bytes % 4 == 0)
+      return fill_as<unsigned int>(dst, bytes / 4, 0.0f, s);
+    return fill_as<unsigned char>(dst, bytes, 0.0f, s);
+  }
+  switch (dtype) {
+  case DT_BOOL: return fill_as<bool>(dst, size, value, s);
+  case DT_BYTE: return fill_as<signed char>(dst, size, value, s);
+  case DT_UBYTE: return fill_as<unsigned char>(dst, size, value, s);
+  case DT_SHORT: return fill_as<short>(dst, size, value, s);
+  case DT_USHORT: return fill_as<unsigned short>(dst, size, value, s);
+  case DT_INT: return fill_as<int>(dst, size, value, s);
+  case DT_UINT: return fill_as<unsigned int>(dst, size, value, s);
+  case DT_LONG: case DT_LONGLONG: return fill_as<long long>(dst, size, value, s);
+  case DT_ULONG: case DT_ULONGLONG: return fill_as<unsigned long long>(dst, size, value, s);
+  case DT_FLOAT: return fill_as<float>(dst, size, value, s);
+  case DT_DOUBLE: return fill_as<double>(dst, size, value, s);
+  }
+  return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "unsupported dtype %d.", dtype);
+}
+
+int nbla_hip_cast(const void *src, int src_dtype, void *dst, int dst_dtype, size_t size, void *stream_) {
+  if (size == 0)
+    return NBLA_HIP_OK;
+  hipStream_t s = as_stream(stream_);
+  const bool same = src_dtype == dst_dtype ||
+                    ((src_dtype == DT_LONG || src_dtype == DT_LONGLONG) && (dst_dtype == DT_LONG || dst_dtype == DT_LONGLONG)) ||
+                    ((src_dtype == DT_ULONG || src_dtype == DT_ULONGLONG) && (dst_dtype == DT_ULONG || dst_dtype == DT_ULONGLONG));
+  if (same) {
+    hipError_t e = hipMemcpyAsync(dst, src, size * dtype_bytes(src_dtype), hipMemcpyDeviceToDevice, s);
+    return e == hipSuccess ? NBLA_HIP_OK : fail_hip(e, "hipMemcpyAsync");
+  }
+  switch (src_dtype) {
+  case DT_BOOL: return cast_from<bool>(src, dst, dst_dtype, size, s);
+  case DT_BYTE: return cast_from<signed char>(src, dst, dst_dtype, size, s);
+  case DT_UBYTE: return cast_from<unsigned char>(src, dst, dst_dtype, size, s);
+  case DT_SHORT: return cast_from<short>(src, dst, dst_dtype, size, s);
+  case DT_USHORT: return cast_from<unsigned short>(src, dst, dst_dtype, size, s);
+  case DT_INT: return cast_from<int>(src, dst, dst_dtype, size, s);
+  case DT_UINT: return cast_from<unsigned int>(src, dst, dst_dtype, size, s);
+  case DT_LONG: case DT_LONGLONG: return cast_from<long long>(src, dst, dst_dtype, size, s);
+  case DT_ULONG: case DT_ULONGLONG: return cast_from<unsigned long long>(src, dst, dst_dtype, size, s);
+  case DT_FLOAT: return cast_from<float>(src, dst, dst_dtype, size, s);
+  case DT_DOUBLE: return cast_from<double>(src, dst, dst_dtype, size, s);
+  }
+  return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "unsupported source dtype %d.", src_dtype);
+}
+
+int nbla_hip_relu_f32(const float *x, float *y, size_t size, void *stream) {
+  if (size == 0)
+    return NBLA_HIP_OK;
+  const int vec = aligned16(x) && aligned16(y);
+  hipLaunchKernelGGL(relu_kernel, dim3(grid_for(vec ? size / 4 + 1 : size)), dim3(kBlk), 0, as_stream(stream), x, y,
+                     size / 4, size, vec);
+  NBLA_HIP_LAUNCH_CHECK("relu");
+  return NBLA_HIP_OK;
+}
+
+} // extern "C"

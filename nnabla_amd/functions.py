@@ -1,0 +1,101 @@
+"""``F.*``: the quantization functions (plus affine and relu) with nnabla's signatures
+(python/src/nnabla/functions.py:416-691 and the generated function_bases for functions.yaml:6735-7520)."""
+from .function import Function
+
+
+def _n_spatial(x, base_axis):
+    base_axis = base_axis if base_axis >= 0 else x.ndim + base_axis
+    return x.ndim - (base_axis + 1)
+
+
+def fixed_point_quantize(x, sign=True, n=8, delta=2 ** -4, quantize=True, ste_fine_grained=True, outputs=None):
+    """Fixed-point quantization of ``x`` (returns ``x`` itself when ``quantize`` is False)."""
+    if not quantize:
+        return x
+    f = Function("FixedPointQuantize", None, [int(sign), n, int(ste_fine_grained)], [delta])
+    return f(x, outputs=outputs)
+
+
+def pow2_quantize(x, sign=True, with_zero=True, n=8, m=1, quantize=True, ste_fine_grained=True, outputs=None):
+    """Power-of-two quantization of ``x`` (returns ``x`` itself when ``quantize`` is False)."""
+    if not quantize:
+        return x
+    f = Function("Pow2Quantize", None, [int(sign), int(with_zero), n, m, int(ste_fine_grained)])
+    return f(x, outputs=outputs)
+
+
+def min_max_quantize(x, qr_min, qr_max, ql_min, ql_max, decay=0.999, x_min_max=False, ema=False,
+                     ste_fine_grained=True, eps=0.01, quantize=True, outputs=None):
+    """Min-max quantization; ``qr_min`` / ``qr_max`` are updated in place when ``x_min_max`` is set."""
+    if not quantize:
+        return x
+    f = Function("MinMaxQuantize", None, [int(x_min_max), int(ema), int(ste_fine_grained)], [decay, eps])
+    return f(x, qr_min, qr_max, ql_min, ql_max, outputs=outputs)
+
+
+def binary_weight_affine(x, weight, binary_weight, alpha, bias=None, base_axis=1, quantize_zero_to=1.0,
+                         n_outputs=-1, outputs=None):
+    f = Function("BinaryWeightAffine", None, [base_axis], [quantize_zero_to])
+    ins = [x, weight, binary_weight, alpha] + ([bias] if bias is not None else [])
+    return f(*ins, outputs=outputs)
+
+
+def binary_connect_affine(x, weight, binary_weight, bias=None, base_axis=1, quantize_zero_to=1.0, n_outputs=-1,
+                          outputs=None):
+    f = Function("BinaryConnectAffine", None, [base_axis], [quantize_zero_to])
+    ins = [x, weight, binary_weight] + ([bias] if bias is not None else [])
+    return f(*ins, outputs=outputs)
+
+
+def _conv_iargs(x, base_axis, pad, stride, dilation, group):
+    nd = _n_spatial(x, base_axis)
+    pad = tuple(pad) if pad is not None else (0,) * nd
+    stride = tuple(stride) if stride is not None else (1,) * nd
+    dilation = tuple(dilation) if dilation is not None else (1,) * nd
+    return nd, list(pad) + list(stride) + list(dilation)
+
+
+def binary_weight_convolution(x, weight, binary_weight, alpha, bias=None, base_axis=1, pad=None, stride=None,
+                              dilation=None, group=1, quantize_zero_to=1.0, n_outputs=-1, outputs=None):
+    nd, geom = _conv_iargs(x, base_axis, pad, stride, dilation, group)
+    f = Function("BinaryWeightConvolution", None, [base_axis, group, nd] + geom, [quantize_zero_to])
+    ins = [x, weight, binary_weight, alpha] + ([bias] if bias is not None else [])
+    return f(*ins, outputs=outputs)
+
+
+def binary_connect_convolution(x, weight, binary_weight, bias=None, base_axis=1, pad=None, stride=None,
+                               dilation=None, group=1, quantize_zero_to=1.0, n_outputs=-1, outputs=None):
+    nd, geom = _conv_iargs(x, base_axis, pad, stride, dilation, group)
+    f = Function("BinaryConnectConvolution", None, [base_axis, group, nd] + geom, [quantize_zero_to])
+    ins = [x, weight, binary_weight] + ([bias] if bias is not None else [])
+    return f(*ins, outputs=outputs)
+
+
+def inq_affine(x, weight, indicator_fixedweights, bias=None, base_axis=1, num_bits=4, inq_iterations=(),
+               selection_algorithm='largest_abs', seed=-1, n_outputs=-1, outputs=None):
+    its = [int(i) for i in inq_iterations]
+    f = Function("INQAffine", None, [base_axis, num_bits, seed, len(its)] + its, [], selection_algorithm)
+    ins = [x, weight, indicator_fixedweights] + ([bias] if bias is not None else [])
+    return f(*ins, outputs=outputs)
+
+
+def inq_convolution(x, weight, indicator_fixedweights, bias=None, base_axis=1, pad=None, stride=None, dilation=None,
+                    group=1, num_bits=4, inq_iterations=(), selection_algorithm='largest_abs', seed=-1, n_outputs=-1,
+                    outputs=None):
+    nd, geom = _conv_iargs(x, base_axis, pad, stride, dilation, group)
+    its = [int(i) for i in inq_iterations]
+    f = Function("INQConvolution", None, [base_axis, group, num_bits, seed, nd] + geom + [len(its)] + its, [],
+                 selection_algorithm)
+    ins = [x, weight, indicator_fixedweights] + ([bias] if bias is not None else [])
+    return f(*ins, outputs=outputs)
+
+
+def affine(x, weight, bias=None, base_axis=1, n_outputs=-1, outputs=None):
+    f = Function("Affine", None, [base_axis])
+    ins = [x, weight] + ([bias] if bias is not None else [])
+    return f(*ins, outputs=outputs)
+
+
+def relu(x, inplace=False, n_outputs=-1, outputs=None):
+    f = Function("ReLU", None, [int(inplace)])
+    return f(x, outputs=outputs)

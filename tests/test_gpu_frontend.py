@@ -1,0 +1,270 @@
+"""The drop-in path end to end on the GPU: ``F.*`` under the hip extension context -> nbla function registry ->
+HipCachedArray storage -> C-ABI kernels, checked against the CPU oracle (the stand-in for nnabla's CPU context)."""
+import numpy as np
+import pytest
+
+import nnabla_amd as nn
+import nnabla_amd.functions as F
+import oracle
+from nnabla_amd import ext_hip
+from nnabla_amd.ext_utils import get_extension_context
+from util import bits_equal, first_mismatch, max_rel_err
+
+pytestmark = pytest.mark.gpu
+TOL, TIGHT = 1e-4, 5e-6
+
+
+@pytest.fixture()
+def ctx(dev):
+    c = get_extension_context('hip', device_id='0')
+    with nn.context_scope(c):
+        yield c
+
+
+def _var(a, dtype=None):
+    v = nn.Variable(a.shape)
+    if dtype is None:
+        v.d = a
+    else:
+        v.set_data(a, dtype)
+    return v
+
+
+def test_extension_module_api(ctx):
+    assert ext_hip.get_device_count() >= 1 and ext_hip.get_devices()[0] == '0'
+    ext_hip.device_synchronize('0')
+    ext_hip.synchronize(device_id='0')
+    ext_hip.clear_memory_cache()
+
+
+def test_fixed_point_and_pow2_quantize(ctx):
+    rng = np.random.RandomState(313)
+    x = (rng.randn(2, 3, 4) * 2).astype(np.float32)       # the reference tests' shape
+    xv = _var(x)
+    y = F.fixed_point_quantize(xv, True, 8, 2 ** -4)
+    assert y.parent.name == 'FixedPointQuantize'
+    y.forward()
+    assert y.head_array_class == 'HipCachedArray'          # computed and left on the device
+    assert bits_equal(y.d, oracle.fixed_point_quantize(x, True, 8, 2 ** -4))
+    big = (rng.randn(64, 4099) * 3).astype(np.float32)
+    for sign, n, delta in [(True, 8, 2 ** -4), (False, 5, 0.3), (True, 3, 0.1)]:
+        y = F.fixed_point_quantize(_var(big), sign, n, delta)
+        y.forward()
+        assert bits_equal(y.d, oracle.fixed_point_quantize(big, sign, n, delta))
+    w = (rng.randn(64, 32, 3, 3) * 0.05).astype(np.float32)
+    for sign, wz, n, m in [(True, True, 4, 1), (False, False, 3, 0), (True, False, 8, 2)]:
+        y = F.pow2_quantize(_var(w), sign, wz, n, m)
+        y.forward()
+        assert bits_equal(y.d, oracle.pow2_quantize(w, sign, wz, n, m))
+
+
+def test_reforward_after_input_update_and_reshape(ctx):
+    """The same graph re-run after the host rewrites the input (H2D sync again) and after a reshape (re-setup,
+    function.cpp:107-123)."""
+    rng = np.random.RandomState(1)
+    xv = nn.Variable((5, 7))
+    y = F.fixed_point_quantize(xv)
+    for _ in range(2):
+        x = (rng.randn(5, 7) * 2).astype(np.float32)
+        xv.d = x
+        y.forward()
+        assert bits_equal(y.d, oracle.fixed_point_quantize(x))
+    xv.reset_shape((3, 11), force=True)
+    x = (rng.randn(3, 11) * 2).astype(np.float32)
+    xv.d = x
+    y.forward()
+    assert y.shape == (3, 11) and bits_equal(y.d, oracle.fixed_point_quantize(x))
+
+
+@pytest.mark.parametrize("xshape,qshape", [((4, 8, 16, 16), (1, 1, 1, 1)), ((4, 8, 16, 16), (1, 8, 1, 1)),
+                                           ((16, 8, 3, 3), (16, 1, 1, 1))])
+@pytest.mark.parametrize("x_min_max,ema", [(True, True), (True, False), (False, False)])
+def test_min_max_quantize_updates_state_in_place(ctx, xshape, qshape, x_min_max, ema):
+    rng = np.random.RandomState(313)
+    qmn, qmx = np.full(qshape, -6, np.float32), np.full(qshape, 6, np.float32)
+    lmn, lmx = np.zeros(qshape, np.float32), np.full(qshape, 255, np.float32)
+    vmn, vmx = _var(qmn), _var(qmx)
+    xv = nn.Variable(xshape)
+    y = F.min_max_quantize(xv, vmn, vmx, _var(lmn), _var(lmx), 0.9, x_min_max, ema)
+    for _ in range(3):                                     # running min/max evolve over minibatches
+        x = (rng.randn(*xshape) * 2).astype(np.float32)
+        xv.d = x
+        y.forward()
+        ref_y, qmn, qmx, _ = oracle.min_max_quantize(x, qmn, qmx, lmn, lmx, 0.9, x_min_max, ema, 0.01)
+        assert bits_equal(y.d, ref_y), first_mismatch(y.d, ref_y)
+        assert bits_equal(vmn.d, qmn) and bits_equal(vmx.d, qmx)
+
+
+def test_binary_affines_write_their_parameters(ctx):
+    rng = np.random.RandomState(5)
+    x = rng.randn(6, 4, 20).astype(np.float32)             # base_axis = 2
+    W = (rng.randn(20, 3, 5) * 0.1).astype(np.float32)
+    b = rng.randn(3, 5).astype(np.float32)
+    wb, alpha = nn.Variable(W.shape), nn.Variable((15,))
+    y = F.binary_weight_affine(_var(x), _var(W), wb, alpha, _var(b), base_axis=2)
+    y.forward()
+    ref_y, ref_wb, ref_alpha = oracle.binary_weight_affine(x.reshape(24, 20), W.reshape(20, 15), b.ravel(), 1.0)
+    assert y.shape == (6, 4, 3, 5)
+    assert bits_equal(wb.d.reshape(20, 15), ref_wb)
+    np.testing.assert_allclose(alpha.d, ref_alpha, rtol=2e-6)
+    assert max_rel_err(y.d.reshape(24, 15), ref_y) <= TIGHT
+    wb2 = nn.Variable(W.shape)
+    y = F.binary_connect_affine(_var(x), _var(W), wb2, None, base_axis=2, quantize_zero_to=-1.0)
+    y.forward()
+    ref_y, ref_wb = oracle.binary_connect_affine(x.reshape(24, 20), W.reshape(20, 15), None, -1.0)
+    assert bits_equal(wb2.d.reshape(20, 15), ref_wb) and max_rel_err(y.d.reshape(24, 15), ref_y) <= TIGHT
+
+
+def test_binary_convolutions(ctx):
+    rng = np.random.RandomState(7)
+    x = rng.randn(4, 8, 16, 16).astype(np.float32)
+    W = (rng.randn(16, 8, 3, 3) * 0.05).astype(np.float32)
+    b = rng.randn(16).astype(np.float32)
+    wb, alpha = nn.Variable(W.shape), nn.Variable((16,))
+    y = F.binary_weight_convolution(_var(x), _var(W), wb, alpha, _var(b), pad=(1, 1), stride=(2, 1))
+    y.forward()
+    ref_y, ref_wb, ref_alpha = oracle.binary_weight_convolution(x, W, b, (1, 1), (2, 1), None, 1, 1.0)
+    assert y.shape == ref_y.shape and bits_equal(wb.d, ref_wb)
+    np.testing.assert_allclose(alpha.d, ref_alpha, rtol=2e-6)
+    assert max_rel_err(y.d, ref_y) <= TIGHT
+    wb2 = nn.Variable(W.shape)
+    y = F.binary_connect_convolution(_var(x), _var(W), wb2, None, pad=(1, 1), group=1)
+    y.forward()
+    ref_y, ref_wb = oracle.binary_connect_convolution(x, W, None, (1, 1), None, None, 1, 1.0)
+    assert bits_equal(wb2.d, ref_wb) and max_rel_err(y.d, ref_y) <= TIGHT
+
+
+@pytest.mark.parametrize("algo", ["largest_abs", "random"])
+def test_inq_affine_state_lives_in_the_function(ctx, algo):
+    """The minibatch counter, the snapshot and the generator belong to the function object (inq_affine.hpp:86-92);
+    float32 indicators written by the host are converted to int32 on first use, as in nnabla."""
+    rng = np.random.RandomState(3)
+    x = rng.randn(9, 40).astype(np.float32)
+    W = (rng.randn(40, 24) * 0.05).astype(np.float32)
+    its, seed = (0, 1, 3), 21
+    inq = oracle.Inq(W.size, 4, its, algo, seed)
+    Wc, Ic = W.copy(), np.zeros(W.shape, np.int32)
+    wv, iv = _var(W), _var(np.zeros(W.shape, np.float32))
+    y = F.inq_affine(_var(x), wv, iv, None, 1, 4, its, algo, seed)
+    for it in range(5):
+        ref_y = inq.affine(x, Wc, Ic, None)
+        y.forward()
+        assert np.array_equal(iv.d.astype(np.int32), Ic), "indicators differ at minibatch %d" % it
+        assert bits_equal(wv.d, Wc)
+        assert max_rel_err(y.d, ref_y) <= TIGHT
+        upd = (rng.randn(*W.shape) * 0.01).astype(np.float32)
+        Wc += upd
+        wv.d = wv.d + upd
+    y.forward()
+    before, w_before = y.d.copy(), wv.d.copy()
+    y.parent.recompute()                                    # product only: weights and counter stay as they are
+    assert bits_equal(y.d, before) and bits_equal(wv.d, w_before)
+
+
+def test_inq_convolution(ctx):
+    rng = np.random.RandomState(4)
+    x = rng.randn(2, 4, 9, 9).astype(np.float32)
+    W = (rng.randn(6, 4, 3, 3) * 0.05).astype(np.float32)
+    inq = oracle.Inq(W.size, 4, (0,), "largest_abs")
+    Wc, Ic = W.copy(), np.zeros(W.shape, np.int32)
+    ref_y = inq.convolution(x, Wc, Ic, None, (1, 1))
+    wv, iv = _var(W), _var(np.zeros(W.shape, np.int32), np.int32)
+    y = F.inq_convolution(_var(x), wv, iv, None, pad=(1, 1), num_bits=4, inq_iterations=(0,))
+    y.forward()
+    assert bits_equal(wv.d, Wc) and np.array_equal(iv.d, Ic) and max_rel_err(y.d, ref_y) <= TIGHT
+
+
+def test_auto_forward_and_relu(ctx):
+    x = (np.random.RandomState(2).randn(4, 9) * 2).astype(np.float32)
+    with nn.auto_forward():
+        y = F.relu(F.fixed_point_quantize(_var(x)))
+        got = y.d
+    ref = np.maximum(oracle.fixed_point_quantize(x), 0)
+    assert np.array_equal(got, ref) and not np.signbit(got).any()
+
+
+def test_device_memory_is_cached_and_released(ctx):
+    ext_hip.clear_memory_cache()
+    base = ext_hip.allocated_bytes('0')
+    x = np.ones((1024, 1024), np.float32)
+    y = F.fixed_point_quantize(_var(x))
+    y.forward()
+    _ = y.d
+    held = ext_hip.allocated_bytes('0')
+    assert held - base >= 2 * x.nbytes                      # input and output copies live on the device
+    y2 = F.fixed_point_quantize(_var(x))
+    y2.forward()
+    del y, y2
+    import gc
+    gc.collect()
+    ext_hip.clear_memory_cache()
+    assert ext_hip.allocated_bytes('0') <= base + (1 << 20)
+
+
+def test_config5_quantized_mlp_graph(ctx):
+    """BASELINE config 5: batch 1024; FixedPointQuantize -> INQAffine 4096x4096 (num_bits 4, every weight fixed)
+    -> 3 x [ReLU -> FixedPointQuantize -> BinaryWeightAffine 4096x4096]; x ~ N(0,1), W ~ N(0, 0.02^2).
+
+    Per layer, with the oracle fed the same input the GPU layer saw: quantizer outputs, Wb and INQ weights are
+    bit-exact, GEMM outputs within 1e-4.  End to end against the oracle-only chain: the quantizers are step
+    functions, so the ~1e-6 relative differences between two fp32 summation orders move a few activations across a
+    rounding tie by one level (2^-4); the whole-graph comparison therefore uses the reference's own comparison metric
+    (utils/cli/compare_with_cpu.py:46-52, std of the difference over the larger std) next to the max-norm figure."""
+    rng = np.random.default_rng(313)
+    B, D = 1024, 4096
+    x = rng.standard_normal((B, D), dtype=np.float32)
+    Ws = [rng.standard_normal((D, D), dtype=np.float32) * np.float32(0.02) for _ in range(4)]
+    # --- graph on the hip context
+    xv = _var(x)
+    w0, i0 = _var(Ws[0]), _var(np.zeros((D, D), np.float32))
+    h = F.fixed_point_quantize(xv, True, 8, 2 ** -4)
+    stages = [("fpq", h)]
+    h = F.inq_affine(h, w0, i0, None, 1, 4, (0,), 'largest_abs')
+    stages.append(("inq", h))
+    wbs, alphas, wvs = [], [], []
+    for l in range(1, 4):
+        h = F.relu(h)
+        stages.append(("relu", h))
+        h = F.fixed_point_quantize(h, True, 8, 2 ** -4)
+        stages.append(("fpq", h))
+        wv, wb, al = _var(Ws[l]), nn.Variable((D, D)), nn.Variable((D,))
+        wvs.append(wv), wbs.append(wb), alphas.append(al)
+        h = F.binary_weight_affine(h, wv, wb, al)
+        stages.append(("bwa", h))
+    h.forward()
+    gpu = [(kind, v.d) for kind, v in stages]
+    # --- per-layer parity on identical inputs, and the oracle-only chain
+    inq = oracle.Inq(D * D, 4, (0,), 'largest_abs')
+    Wq, Iq = Ws[0].copy(), np.zeros((D, D), np.int32)
+    cur_gpu_in, cur_ref = x, x
+    layer = 0
+    worst_gemm = 0.0
+    for kind, out in gpu:
+        if kind == "fpq":
+            assert bits_equal(out, oracle.fixed_point_quantize(cur_gpu_in, True, 8, 2 ** -4))
+            cur_ref = oracle.fixed_point_quantize(cur_ref, True, 8, 2 ** -4)
+        elif kind == "relu":
+            assert np.array_equal(out, np.maximum(cur_gpu_in, 0))
+            cur_ref = np.maximum(cur_ref, 0)
+        elif kind == "inq":
+            ref_same_in = inq.affine(cur_gpu_in, Wq, Iq, None)     # quantizes Wq in place
+            assert bits_equal(w0.d, Wq), first_mismatch(w0.d, Wq)
+            assert np.array_equal(i0.d.astype(np.int32), Iq)
+            worst_gemm = max(worst_gemm, max_rel_err(out, ref_same_in))
+            cur_ref = oracle.affine(cur_ref, Wq) if cur_ref is not cur_gpu_in else ref_same_in
+        else:
+            ref_same_in, ref_wb, ref_alpha = oracle.binary_weight_affine(cur_gpu_in, Ws[layer + 1], None, 1.0)
+            assert bits_equal(wbs[layer].d, ref_wb)
+            np.testing.assert_allclose(alphas[layer].d, ref_alpha, rtol=2e-6)
+            worst_gemm = max(worst_gemm, max_rel_err(out, ref_same_in))
+            cur_ref = oracle.affine(cur_ref, ref_wb * ref_alpha[None, :])
+            layer += 1
+        cur_gpu_in = out
+    assert worst_gemm <= TOL, worst_gemm
+    y_gpu, y_cpu = gpu[-1][1], cur_ref
+    std_metric = np.std(y_gpu.astype(np.float64) - y_cpu) / max(np.std(y_gpu), np.std(y_cpu))
+    max_metric = max_rel_err(y_gpu, y_cpu)
+    flipped_rows = np.mean(np.abs(y_gpu - y_cpu).max(1) > 1e-4 * np.abs(y_cpu).max())
+    print("config5: per-layer GEMM max rel err %.2e; end-to-end std metric %.2e, max-norm %.2e, rows touched by a "
+          "quantizer tie flip %.1f%%" % (worst_gemm, std_metric, max_metric, 100 * flipped_rows))
+    assert std_metric <= 2e-3 and max_metric <= 2e-2
