@@ -32,7 +32,8 @@ PrepPlan make_prep_plan(int64_t K, int64_t N, bool transposed) {
   P.k_tiles = bits_k_tiles(K);
   P.col_groups = bits_col_groups(N);
   P.Np = P.col_groups * kColGroup;
-  P.slices = transposed ? ceil_div(P.k_tiles, 4) : ceil_div(K, kKSlice);
+  // the [K, N] kernels cover 8 (vector path) or 16 (scalar path) k tiles per block; size for the finer one
+  P.slices = transposed ? ceil_div(P.k_tiles, 4) : ceil_div(P.k_tiles, 8);
   P.sums_bytes = round_up((size_t)P.slices * P.Np * sizeof(float), 256);
   P.zeros_bytes = round_up((size_t)P.slices * P.col_groups * sizeof(int), 256);
   return P;
@@ -124,6 +125,95 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_kn(const float *__restric
       acc += s_sum[r][threadIdx.x];
     sums[(int64_t)blockIdx.y * Np + cg * kColGroup + threadIdx.x] = acc;
   }
+  if (threadIdx.x == 0)
+    zeros[(int64_t)blockIdx.y * col_groups + cg] = s_zero[0] + s_zero[1] + s_zero[2] + s_zero[3];
+}
+
+// W stored [K, N], N % 4 == 0, 16-byte aligned: the streaming path.  A wavefront covers two k tiles of one column
+// group; lane = (kt_sub, g, f, nq): columns f*32 + 4*nq + {0..3}, k offsets s*16 + g*8 + e.  Each thread issues its
+// sixteen 128-bit loads up front (sixteen lanes cover 256 contiguous bytes of a row), builds the bits of its half
+// (f) of four packed words, and the two halves are OR-ed across lanes.  |W| column sums are folded in a fixed
+// order: over (g, kt_sub) by shuffles, over the block's wavefronts through LDS.
+__global__ __launch_bounds__(kPrepBlock) void binarize_kn_vec(const float *__restrict__ W, float *__restrict__ Wb,
+                                                              uint32_t *__restrict__ bits, float *__restrict__ sums,
+                                                              int *__restrict__ zeros, int64_t K, int64_t N,
+                                                              int64_t col_groups, int64_t Np, int64_t k_tiles,
+                                                              float zero_to) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nq = lane & 7, f = (lane >> 3) & 1, g = (lane >> 4) & 1, kt_sub = lane >> 5;
+  const int64_t cg = blockIdx.x;
+  const int64_t kt = ((int64_t)blockIdx.y * 4 + wave) * 2 + kt_sub;
+  const int64_t n0 = cg * kColGroup + f * 32 + 4 * nq;
+  const bool col_ok = n0 < N;
+  float4_t v[16];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int64_t k = kt * kTileK + s * 16 + g * 8 + e;
+      if (col_ok && k < K)
+        v[s * 8 + e] = *reinterpret_cast<const float4_t *>(W + k * N + n0);
+      else
+        v[s * 8 + e] = float4_t{1.0f, 1.0f, 1.0f, 1.0f};
+    }
+  uint32_t word[4] = {0u, 0u, 0u, 0u};
+  float asum[4] = {0.f, 0.f, 0.f, 0.f};
+  int nzero = 0;
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int64_t k = kt * kTileK + s * 16 + g * 8 + e;
+      const bool in = col_ok && k < K;
+      const float w[4] = {v[s * 8 + e].x, v[s * 8 + e].y, v[s * 8 + e].z, v[s * 8 + e].w};
+      float b[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        b[c] = sign_of(w[c], zero_to);
+        const bool is_zero = !(w[c] > 0.0f) && !(w[c] < 0.0f);
+        const bool neg = (w[c] < 0.0f) || (is_zero && zero_to < 0.0f);
+        // bit position of (f, s, e), with f a run-time value: p = 4*(2f+s) + e/2
+        const int pp = 4 * (2 * f + s) + (e >> 1);
+        const int pos = (e & 1) ? 31 - pp : 15 - pp;
+        word[c] |= (in && neg) ? (1u << pos) : 0u;
+        asum[c] += in ? fabsf(w[c]) : 0.0f;
+        nzero += (in && is_zero) ? 1 : 0;
+      }
+      if (in) {
+        float4_t o;
+        o.x = b[0], o.y = b[1], o.z = b[2], o.w = b[3];
+        __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(Wb + k * N + n0));
+      }
+    }
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+    word[c] |= __shfl_xor(word[c], 8); // the other half (f) of the same packed words
+  if (f == 0 && kt < k_tiles) {
+    uint4_t wv;
+    wv.x = word[0], wv.y = word[1], wv.z = word[2], wv.w = word[3];
+    *reinterpret_cast<uint4_t *>(bits + (kt * col_groups + cg) * 64 + g * 32 + 4 * nq) = wv;
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    asum[c] += __shfl_xor(asum[c], 16); // g
+    asum[c] += __shfl_xor(asum[c], 32); // kt_sub
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1)
+    nzero += __shfl_xor(nzero, off);
+  __shared__ float s_sum[kPrepBlock / 64][kColGroup];
+  __shared__ int s_zero[kPrepBlock / 64];
+  if (lane < 16) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      s_sum[wave][f * 32 + 4 * nq + c] = asum[c];
+  }
+  if (lane == 0)
+    s_zero[wave] = nzero;
+  __syncthreads();
+  if (threadIdx.x < kColGroup)
+    sums[(int64_t)blockIdx.y * Np + cg * kColGroup + threadIdx.x] =
+        ((s_sum[0][threadIdx.x] + s_sum[1][threadIdx.x]) + s_sum[2][threadIdx.x]) + s_sum[3][threadIdx.x];
   if (threadIdx.x == 0)
     zeros[(int64_t)blockIdx.y * col_groups + cg] = s_zero[0] + s_zero[1] + s_zero[2] + s_zero[3];
 }
@@ -270,6 +360,54 @@ __global__ __launch_bounds__(kPrepBlock) void split_bf16x3(const float *__restri
   dst[128] = o;
 }
 
+// Streaming variant for K % 64 == 0, 16-byte aligned rows: a wavefront converts a 32-row x 64-k patch (four
+// fragments).  Global loads are fully coalesced (16 lanes read 256 contiguous bytes of a row); the patch is turned
+// into fragment order through a padded LDS tile.
+__global__ __launch_bounds__(kPrepBlock) void split_bf16x3_tiled(const float *__restrict__ x, int64_t ldx,
+                                                                 uint4_t *__restrict__ out, int64_t M, int64_t K,
+                                                                 int64_t k_blocks, int64_t patches) {
+  constexpr int kRowStride = 68; // floats: 64 + 4 padding keeps the 128-bit column reads conflict-free
+  __shared__ float tile[kPrepBlock / 64][32 * kRowStride];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t patch = (int64_t)blockIdx.x * (kPrepBlock / 64) + wave;
+  if (patch >= patches)
+    return;
+  const int64_t patches_per_row = k_blocks / 4;
+  const int64_t rb = patch / patches_per_row, kq = patch - rb * patches_per_row;
+  float *t = tile[wave];
+  const int lr = lane >> 4, lc = (lane & 15) * 4;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int row = j * 4 + lr;
+    const int64_t m = rb * kFragRows + row;
+    float4_t v = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (m < M)
+      v = *reinterpret_cast<const float4_t *>(x + m * ldx + kq * 64 + lc);
+    *reinterpret_cast<float4_t *>(t + row * kRowStride + lc) = v;
+  }
+  // the tile is private to this wavefront: LDS operations of one wavefront complete in order
+  __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
+  const int r = lane & 31, g = lane >> 5;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float4_t a = *reinterpret_cast<const float4_t *>(t + r * kRowStride + q * 16 + g * 8);
+    const float4_t b = *reinterpret_cast<const float4_t *>(t + r * kRowStride + q * 16 + g * 8 + 4);
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    uint32_t h[8], mi[8], l[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      split3(v[e], h[e], mi[e], l[e]);
+    uint4_t o;
+    uint4_t *dst = out + ((rb * k_blocks + kq * 4 + q) * 3) * 64 + lane;
+    o.x = h[0] | (h[1] << 16), o.y = h[2] | (h[3] << 16), o.z = h[4] | (h[5] << 16), o.w = h[6] | (h[7] << 16);
+    __builtin_nontemporal_store(o, dst);
+    o.x = mi[0] | (mi[1] << 16), o.y = mi[2] | (mi[3] << 16), o.z = mi[4] | (mi[5] << 16), o.w = mi[6] | (mi[7] << 16);
+    __builtin_nontemporal_store(o, dst + 64);
+    o.x = l[0] | (l[1] << 16), o.y = l[2] | (l[3] << 16), o.z = l[4] | (l[5] << 16), o.w = l[6] | (l[7] << 16);
+    __builtin_nontemporal_store(o, dst + 128);
+  }
+}
+
 } // namespace
 } // namespace nbla_hip
 
@@ -307,14 +445,18 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint3
   hipStream_t stream = as_stream(stream_);
   float *sums = static_cast<float *>(workspace);
   int *zeros = reinterpret_cast<int *>(static_cast<char *>(workspace) + P.sums_bytes);
+  int64_t slices = P.slices;
   if (!transposed) {
-    const dim3 grid((unsigned)P.col_groups, (unsigned)P.slices);
-    if (N % 4 == 0 && aligned16(W) && aligned16(Wb))
-      hipLaunchKernelGGL(binarize_kn<true>, grid, dim3(kPrepBlock), 0, stream, W, Wb, bits, sums, zeros, K, N,
-                         P.col_groups, P.Np, quantize_zero_to);
-    else
+    if (N % 4 == 0 && aligned16(W) && aligned16(Wb)) {
+      const dim3 grid((unsigned)P.col_groups, (unsigned)P.slices);
+      hipLaunchKernelGGL(binarize_kn_vec, grid, dim3(kPrepBlock), 0, stream, W, Wb, bits, sums, zeros, K, N,
+                         P.col_groups, P.Np, P.k_tiles, quantize_zero_to);
+    } else {
+      slices = ceil_div(K, kKSlice);
+      const dim3 grid((unsigned)P.col_groups, (unsigned)slices);
       hipLaunchKernelGGL(binarize_kn<false>, grid, dim3(kPrepBlock), 0, stream, W, Wb, bits, sums, zeros, K, N,
                          P.col_groups, P.Np, quantize_zero_to);
+    }
   } else {
     const dim3 grid((unsigned)P.col_groups, (unsigned)P.slices);
     hipLaunchKernelGGL(binarize_nk, grid, dim3(kPrepBlock), 0, stream, W, Wb, bits, sums, zeros, K, N, P.col_groups,
@@ -324,7 +466,7 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint3
   if (alpha || zero_count) {
     const float inv_k = (float)1 / K;
     hipLaunchKernelGGL(binarize_finalize, dim3((unsigned)ceil_div(N, kPrepBlock)), dim3(kPrepBlock), 0, stream, sums,
-                       zeros, alpha, zero_count, N, P.Np, P.slices, P.slices * P.col_groups, inv_k);
+                       zeros, alpha, zero_count, N, P.Np, slices, slices * P.col_groups, inv_k);
     NBLA_HIP_LAUNCH_CHECK("binarize_finalize");
   }
   return NBLA_HIP_OK;
@@ -341,8 +483,14 @@ int nbla_hip_split_bf16x3_f32(const float *x, int64_t ldx, void *xsplit, int64_t
     return rc;
   const int64_t k_blocks = split_k_blocks(K);
   const int64_t frags = split_row_blocks(M) * k_blocks;
-  hipLaunchKernelGGL(split_bf16x3, dim3((unsigned)ceil_div(frags, kPrepBlock / 64)), dim3(kPrepBlock), 0,
-                     as_stream(stream_), x, ldx, static_cast<uint4_t *>(xsplit), M, K, k_blocks, frags);
+  if (K % 64 == 0 && ldx % 4 == 0 && aligned16(x)) {
+    const int64_t patches = frags / 4;
+    hipLaunchKernelGGL(split_bf16x3_tiled, dim3((unsigned)ceil_div(patches, kPrepBlock / 64)), dim3(kPrepBlock), 0,
+                       as_stream(stream_), x, ldx, static_cast<uint4_t *>(xsplit), M, K, k_blocks, patches);
+  } else {
+    hipLaunchKernelGGL(split_bf16x3, dim3((unsigned)ceil_div(frags, kPrepBlock / 64)), dim3(kPrepBlock), 0,
+                       as_stream(stream_), x, ldx, static_cast<uint4_t *>(xsplit), M, K, k_blocks, frags);
+  }
   NBLA_HIP_LAUNCH_CHECK("split_bf16x3");
   return NBLA_HIP_OK;
 }

@@ -134,59 +134,115 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64) void gemm_bits_kernel(GemmBi
       for (int r = 0; r < 16; ++r)
         acc[i][j][r] = 0.0f;
 
-  load_step(0);
-  store_step(0);
-  __syncthreads();
-
-  for (int64_t ks = 0; ks < a.k_steps; ++ks) {
-    const int buf = (int)(ks & 1);
-    if (ks + 1 < a.k_steps)
-      load_step(ks + 1);
-
+  // Fragment fetch and the MFMA block of one k16 sub-step (s = 0, 1) of a staged tile.
+  auto read_a = [&](int buf, int s, uint4_t (&af)[MF][3]) {
     const uint4_t *sa = reinterpret_cast<const uint4_t *>(smem + buf * kStageBytes);
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+      for (int p = 0; p < 3; ++p)
+        af[i][p] = sa[(wm * MF + i) * kASegVec + s * 192 + p * 64 + lane];
+  };
+  auto read_words = [&](int buf, uint32_t (&words)[NW]) {
     const uint32_t *sb = reinterpret_cast<const uint32_t *>(smem + buf * kStageBytes + kAVec * 16);
-    uint32_t words[NW];
 #pragma unroll
     for (int w = 0; w < NW; ++w)
       words[w] = sb[(wn * NW + w) * 64 + lane];
-
+  };
+  // Bits -> +-1.0 bf16 pairs: register i of fragment (f, s) is ((word << 4*(2f+s)+i) & 0x80008000) | 0x3F803F80.
+  // The two constants are kept in registers so that each register costs a shift and one v_and_or_b32.
+  uint32_t sign_mask = 0x80008000u, one_pair = 0x3F803F80u;
+  asm volatile("" : "+s"(sign_mask));
+  asm volatile("" : "+v"(one_pair));
+  auto expand = [&](int s, const uint32_t (&words)[NW], uint4_t (&bf)[NF]) {
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      uint4_t af[MF][3];
+    for (int j = 0; j < NF; ++j) {
+      const uint32_t w = words[j >> 1];
+      const int base = 4 * (2 * (j & 1) + s);
+      bf[j].x = ((w << (base + 0)) & sign_mask) | one_pair;
+      bf[j].y = ((w << (base + 1)) & sign_mask) | one_pair;
+      bf[j].z = ((w << (base + 2)) & sign_mask) | one_pair;
+      bf[j].w = ((w << (base + 3)) & sign_mask) | one_pair;
+    }
+  };
+  auto mma = [&](const uint4_t (&af)[MF][3], const uint4_t (&bf)[NF]) {
+    // smallest plane first: the low-order parts enter the accumulator before the leading one
+#pragma unroll
+    for (int p = 2; p >= 0; --p)
 #pragma unroll
       for (int i = 0; i < MF; ++i)
 #pragma unroll
-        for (int p = 0; p < 3; ++p)
-          af[i][p] = sa[(wm * MF + i) * kASegVec + s * 192 + p * 64 + lane];
-      uint4_t bf[NF];
+        for (int j = 0; j < NF; ++j) {
+          acc[i][j] = kSwap ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[j]),
+                                                                      __builtin_bit_cast(bf16x8_t, af[i][p]),
+                                                                      acc[i][j], 0, 0, 0)
+                            : __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[i][p]),
+                                                                      __builtin_bit_cast(bf16x8_t, bf[j]),
+                                                                      acc[i][j], 0, 0, 0);
+        }
+  };
+  // Asks the scheduler to issue the region just written as: one MFMA, then a few VALU / memory instructions in
+  // its shadow, repeated.  A wavefront issues in order and an MFMA occupies the matrix pipe for 32 cycles, so the
+  // expansion, fragment fetch and staging traffic of the next sub-step fit between consecutive MFMAs instead of
+  // in front of them (where wavefronts running in lockstep would all leave the matrix pipe idle together).
+  constexpr int kMfma = 3 * MF * NF;
+  constexpr int kValuPer = (NF * 8 + 8 + kMfma - 1) / kMfma + 1;
+  auto interleave_first = [&]() { // region: LDS reads of sub-step 1, expansion, MFMAs of sub-step 0, LDS staging writes
 #pragma unroll
-      for (int j = 0; j < NF; ++j) {
-        const uint32_t w = words[j >> 1];
-        const int base = 4 * (2 * (j & 1) + s);
-        bf[j].x = ((w << (base + 0)) & 0x80008000u) | 0x3F803F80u;
-        bf[j].y = ((w << (base + 1)) & 0x80008000u) | 0x3F803F80u;
-        bf[j].z = ((w << (base + 2)) & 0x80008000u) | 0x3F803F80u;
-        bf[j].w = ((w << (base + 3)) & 0x80008000u) | 0x3F803F80u;
-      }
-      // smallest plane first: the low-order parts enter the accumulator before the
-      // leading one
-#pragma unroll
-      for (int p = 2; p >= 0; --p)
-#pragma unroll
-        for (int i = 0; i < MF; ++i)
-#pragma unroll
-          for (int j = 0; j < NF; ++j)
-            acc[i][j] = kSwap ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[j]),
-                                                                        __builtin_bit_cast(bf16x8_t, af[i][p]),
-                                                                        acc[i][j], 0, 0, 0)
-                              : __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[i][p]),
-                                                                        __builtin_bit_cast(bf16x8_t, bf[j]),
-                                                                        acc[i][j], 0, 0, 0);
+    for (int g = 0; g < kMfma; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
+      if (g < MF * 3)
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
+      __builtin_amdgcn_sched_group_barrier(0x002, kValuPer, 0); // VALU
+      if (g >= kMfma - kAPasses - kBPasses)
+        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // DS write
     }
+  };
+  auto interleave_second = [&]() { // region: global loads, LDS reads of the next stage, expansion, MFMAs of sub-step 1
+#pragma unroll
+    for (int g = 0; g < kMfma; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
+      if (g < kAPasses + kBPasses)
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // VMEM read
+      if (g < MF * 3 + NW)
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
+      __builtin_amdgcn_sched_group_barrier(0x002, kValuPer, 0); // VALU
+    }
+  };
 
-    if (ks + 1 < a.k_steps)
-      store_step(buf ^ 1);
+  // Software pipeline.  Two LDS stages, one barrier per k step, no branches in the loop body (the last iterations
+  // re-load the final stage instead of skipping, so each half of the body is one scheduling region).  While the
+  // MFMA block of one k16 sub-step runs, the A fragments of the next sub-step are fetched from LDS and its B
+  // fragments are expanded; the global loads of stage ks+2 are issued a full step ahead of their use.
+  uint4_t af0[MF][3], af1[MF][3], bf0[NF], bf1[NF];
+  uint32_t wcur[NW], wnext[NW];
+  const int64_t last = a.k_steps - 1;
+  load_step(0);
+  store_step(0);
+  __syncthreads();
+  load_step(last < 1 ? last : 1);
+  read_words(0, wcur);
+  read_a(0, 0, af0);
+  expand(0, wcur, bf0);
+  for (int64_t ks = 0; ks <= last; ++ks) {
+    const int buf = (int)(ks & 1);
+    // sub-step 0 runs; sub-step 1 is prepared; the staged registers (stage ks+1) go to the other LDS buffer
+    read_a(buf, 1, af1);
+    expand(1, wcur, bf1);
+    mma(af0, bf0);
+    store_step(buf ^ 1);
+    interleave_first();
     __syncthreads();
+    // sub-step 1 runs; global loads of stage ks+2 are issued; sub-step 0 of stage ks+1 is prepared
+    load_step(ks + 2 < last ? ks + 2 : last);
+    read_words(buf ^ 1, wnext);
+    read_a(buf ^ 1, 0, af0);
+    expand(0, wnext, bf0);
+    mma(af1, bf1);
+    interleave_second();
+#pragma unroll
+    for (int w = 0; w < NW; ++w)
+      wcur[w] = wnext[w];
   }
 
   // Epilogue.  Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
@@ -267,11 +323,15 @@ int launch_tile(const GemmBitsArgs &args, hipStream_t stream) {
   return NBLA_HIP_OK;
 }
 
+// Tile choice by M (measured on MI355X at K = 4096, N = 11008): the wide 128x512 tile with sixteen wavefronts
+// wins once there are enough row blocks to fill the 256 CUs; smaller tiles keep more blocks in flight below that.
 template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream) {
-  if (a.M > 128)
-    return launch_tile<256, 256, 4, 2, kSwap>(a, stream);
+  if (a.M >= 3072)
+    return launch_tile<128, 512, 4, 4, kSwap>(a, stream);
+  if (a.M > 1024)
+    return launch_tile<128, 256, 2, 4, kSwap>(a, stream);
   if (a.M > 32)
-    return launch_tile<128, 128, 4, 1, kSwap>(a, stream);
+    return launch_tile<64, 256, 2, 4, kSwap>(a, stream);
   return launch_tile<32, 256, 1, 4, kSwap>(a, stream);
 }
 

@@ -11,23 +11,23 @@ namespace nbla_hip {
 namespace {
 
 constexpr int kBlock = 256;  // threads per block: 4 wavefronts
-constexpr int kUnroll = 4;   // float4 per thread per block tile
-constexpr int kTile = kBlock * kUnroll; // float4 per block
+constexpr int kUnroll = 4;   // float4 per thread per block tile (large inputs)
+constexpr int kTile = kBlock * kUnroll; // float4 per block at full unroll
 
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ float4_t load4(const float *p) {
-  return __builtin_nontemporal_load(reinterpret_cast<const float4_t *>(p));
-}
+// Streaming access pattern that measured best on MI355X for a read-once/write-once map: ordinary 128-bit loads,
+// nontemporal 128-bit stores.
+__device__ __forceinline__ float4_t load4(const float *p) { return *reinterpret_cast<const float4_t *>(p); }
 __device__ __forceinline__ void store4(float *p, float4_t v) {
   __builtin_nontemporal_store(v, reinterpret_cast<float4_t *>(p));
 }
 
 // Generic driver: applies `op` (a functor float -> float) to `size` elements.
 // The vector body covers size/4 float4s; the tail (size % 4) is done by block 0.
-template <typename Op> __global__ __launch_bounds__(kBlock) void map_vec4(const float *__restrict__ x, float *__restrict__ y, size_t n4, size_t size, Op op) {
+template <typename Op, int kUnroll> __global__ __launch_bounds__(kBlock) void map_vec4(const float *__restrict__ x, float *__restrict__ y, size_t n4, size_t size, Op op) {
   op.prepare();
-  const size_t base = (size_t)blockIdx.x * kTile + threadIdx.x;
+  const size_t base = (size_t)blockIdx.x * (kBlock * kUnroll) + threadIdx.x;
   float4_t v[kUnroll];
 #pragma unroll
   for (int j = 0; j < kUnroll; ++j) {
@@ -66,8 +66,15 @@ template <typename Op> int launch_map(const float *x, float *y, size_t size, Op 
     return NBLA_HIP_OK;
   if (aligned16(x) && aligned16(y)) {
     const size_t n4 = size / 4;
-    const size_t blocks = n4 ? (n4 + kTile - 1) / kTile : 1;
-    hipLaunchKernelGGL(map_vec4<Op>, dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, y, n4, size, op);
+    // inputs too small to give every CU several 4-deep blocks get one float4 per thread instead
+    if (n4 < (size_t)kBlock * kUnroll * 2048) {
+      const size_t blocks = n4 ? (n4 + kBlock - 1) / kBlock : 1;
+      hipLaunchKernelGGL((map_vec4<Op, 1>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, y, n4, size, op);
+    } else {
+      const size_t tile = (size_t)kBlock * kUnroll;
+      const size_t blocks = (n4 + tile - 1) / tile;
+      hipLaunchKernelGGL((map_vec4<Op, kUnroll>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, y, n4, size, op);
+    }
   } else {
     size_t blocks = (size + kBlock - 1) / kBlock;
     if (blocks > 65536)
@@ -146,6 +153,36 @@ struct Pow2Op {
   }
 };
 
+// Pow2Quantize with few levels (2^n' <= 8): |x| as a bit pattern is compared against the level boundaries
+// directly.  roundf(log2f(a)) is a non-decreasing step function of a, so level e starts at the calibrated cut of
+// binade e-1; the output exponent is e_min plus the number of boundaries at or below |x|.
+template <int kLevels> struct Pow2SmallOp {
+  uint32_t bound[kLevels]; // bound[0] = first |x| with r >= e_min, bound[j] = first |x| with r >= e_min + j
+  float p_min, thr;
+  int e_min;
+  int sign, with_zero;
+  __device__ __forceinline__ void prepare() {}
+  __device__ __forceinline__ float operator()(float x) const {
+    const uint32_t u = __float_as_uint(x) & 0x7fffffffu;
+    float q;
+    if (u > 0x7f800000u) {
+      q = __uint_as_float(u);
+    } else if (u < bound[0]) {
+      q = with_zero ? ((__uint_as_float(u) < thr) ? 0.0f : p_min) : p_min;
+    } else {
+      int up = 0;
+#pragma unroll
+      for (int j = 1; j < kLevels; ++j)
+        up += (u >= bound[j]) ? 1 : 0;
+      q = pow2_int(e_min + up);
+    }
+    const bool neg = x < 0.0f;
+    if (sign)
+      return neg ? -q : q;
+    return neg ? (with_zero ? 0.0f : p_min) : q;
+  }
+};
+
 } // namespace
 } // namespace nbla_hip
 
@@ -194,6 +231,43 @@ int nbla_hip_pow2_quantize_f32(const float *x, float *y, size_t size, int sign, 
   int rc = ensure_init();
   if (rc)
     return rc;
+  if (nn <= 3) { // up to eight levels: boundaries travel as kernel arguments
+    uint32_t table[kNumBinades];
+    rc = nbla_hip_cut_table(kCutPow2Round, table);
+    if (rc)
+      return rc;
+    const int levels = 1 << nn;
+    uint32_t bound[8];
+    for (int j = 0; j < levels; ++j) {
+      const int binade = (e_min + j - 1) + 149; // the cut where r steps from e_min+j-1 to e_min+j
+      // below the smallest subnormal binade every positive value already rounds to >= -149
+      bound[j] = binade >= 0 ? table[binade] : 1u;
+    }
+    const float p_min = (float)std::pow(2., e_min);
+    const float thr = (float)((float)p_min * std::pow(2., -0.5));
+    auto fill = [&](auto &op) {
+      for (int j = 0; j < levels; ++j)
+        op.bound[j] = bound[j];
+      op.p_min = p_min;
+      op.thr = thr;
+      op.e_min = e_min;
+      op.sign = sign;
+      op.with_zero = with_zero;
+    };
+    if (levels == 2) {
+      Pow2SmallOp<2> op;
+      fill(op);
+      return launch_map(x, y, size, op, as_stream(stream), "pow2_quantize");
+    }
+    if (levels == 4) {
+      Pow2SmallOp<4> op;
+      fill(op);
+      return launch_map(x, y, size, op, as_stream(stream), "pow2_quantize");
+    }
+    Pow2SmallOp<8> op;
+    fill(op);
+    return launch_map(x, y, size, op, as_stream(stream), "pow2_quantize");
+  }
   Pow2Op op;
   op.cuts = device_cut_table(kCutPow2Round);
   op.p_max = (float)std::pow(2., e_max);                 // pow2_quantize.cpp:37
@@ -257,7 +331,7 @@ MinMaxLayout collapse(const int64_t *xshape, int ndim, const int64_t *qshape) {
 
 constexpr int kRedBlock = 256;
 constexpr int kRedTile = kRedBlock * 4; // elements per block tile
-constexpr int kMaxChunks = 2048;
+constexpr int kMaxChunks = 1024;
 
 struct MinMaxPlan {
   MinMaxLayout L;
@@ -441,9 +515,17 @@ __global__ __launch_bounds__(64) void minmax_finalize(const MinMaxPartial *__res
   Extrema ex;
   ex.init();
   if (s.x_min_max) {
-    for (int c = threadIdx.x; c < nchunks; c += 64) {
-      const MinMaxPartial p = partial[k * nchunks + c];
-      ex.merge(p.vmin, p.imin, p.vmax, p.imax);
+    // four independent 16-byte loads in flight per lane before any merge
+    const float4_t *pp = reinterpret_cast<const float4_t *>(partial + k * nchunks);
+    for (int c = threadIdx.x; c < nchunks; c += 256) {
+      float4_t q[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        q[j] = (c + 64 * j < nchunks) ? pp[c + 64 * j] : float4_t{1e+8f, __uint_as_float(0xffffffffu), -1e+8f,
+                                                                   __uint_as_float(0xffffffffu)};
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        ex.merge(q[j].x, __float_as_uint(q[j].y), q[j].z, __float_as_uint(q[j].w));
     }
     ex.wave_reduce();
   }
