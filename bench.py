@@ -41,7 +41,7 @@ def bench_binary_weight_affine(M, K, N, steps, warmup, dev):
     y = torch.empty(M, N, device=dev)
     L = k.lib()
     bits = torch.empty(L.nbla_hip_packed_bits_bytes(k._i64(K), k._i64(N)), dtype=torch.uint8, device=dev)
-    xs = torch.empty(L.nbla_hip_split_operand_bytes(k._i64(M), k._i64(K)), dtype=torch.uint8, device=dev)
+    xs = torch.empty(L.nbla_hip_digit_operand_bytes(k._i64(M), k._i64(K)), dtype=torch.uint8, device=dev)
     pws = torch.empty(max(256, L.nbla_hip_binarize_workspace_bytes(k._i64(K), k._i64(N))), dtype=torch.uint8,
                       device=dev)
     st = k._stream(None)
@@ -55,7 +55,7 @@ def bench_binary_weight_affine(M, K, N, steps, warmup, dev):
                                                 st))
         if ev:
             ev[1].record()
-        k.check(L.nbla_hip_split_bf16x3_f32(k._p(x), k._i64(K), k._p(xs), k._i64(M), k._i64(K), st))
+        k.check(L.nbla_hip_split_digits_f32(k._p(x), k._i64(K), k._p(xs), k._i64(M), k._i64(K), st))
         if ev:
             ev[2].record()
         k.check(L.nbla_hip_gemm_bits_f32(k._p(xs), k._p(bits), k._p(alpha), None, k._p(y), k._i64(M), k._i64(K),
@@ -185,7 +185,7 @@ def main():
                    "M": M, "K": K, "N": N},
         "roofline": {"bound": "mfma", "achieved": gemm_tflops, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": gemm_tflops / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
-                     "kernel": "gemm_bits_kernel<256,256,4,2>", "kernel_ms": r["gemm_ms"],
+                     "kernel": "gemm_bits_kernel<128,512,4,4,false>", "kernel_ms": r["gemm_ms"],
                      "note": "fp32-equivalent flops 2*M*K*N against the fp32 MFMA peak; the kernel issues 3x that "
                              "in bf16 MFMA", "bf16_issue_frac": 3 * gemm_tflops / PEAK_BF16_MFMA_TFLOPS},
         "step_breakdown_ms": {"prepare": r["prepare_ms"], "split": r["split_ms"], "gemm": r["gemm_ms"]},

@@ -107,8 +107,12 @@ int nbla_hip_min_max_quantize_f32(const float *x, float *y,
 
 /* Bytes of the 1-bit packed GEMM operand for a [K, N] weight matrix. */
 size_t nbla_hip_packed_bits_bytes(int64_t K, int64_t N);
-/* Bytes of the bf16x3-split, fragment-ordered GEMM operand for x [M, K]. */
+/* Bytes of the bf16x3-split, fragment-ordered GEMM operand for x [M, K]
+ * (the operand of the plane x plane product used by the INQ forwards). */
 size_t nbla_hip_split_operand_bytes(int64_t M, int64_t K);
+/* Bytes of the int8 digit operand for x [M, K] (the operand of the bit-weight
+ * product): fragment-ordered digits, per-row sums and per-row shifts. */
+size_t nbla_hip_digit_operand_bytes(int64_t M, int64_t K);
 /* Scratch of nbla_hip_binarize_weights_f32 (column-sum partials, zero count). */
 size_t nbla_hip_binarize_workspace_bytes(int64_t K, int64_t N);
 
@@ -138,16 +142,27 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha,
 int nbla_hip_split_bf16x3_f32(const float *x, int64_t ldx, void *xsplit,
                               int64_t M, int64_t K, void *stream);
 
+/* Turn x [M, K] (row stride ldx elements) into the int8 digit operand: per
+ * row a power-of-two scale 2^s such that q = rint(x * 2^s) fits 24 bits for
+ * the row's largest magnitude, q as three balanced base-256 digits in MFMA
+ * fragment order, and the row sums of q.  A row holding NaN or infinity is
+ * marked and yields NaN outputs. */
+int nbla_hip_split_digits_f32(const float *x, int64_t ldx, void *xdigits,
+                              int64_t M, int64_t K, void *stream);
+
 /* y[m, n] = (sum_k x[m,k] * (+-1)[k,n]) * alpha[n] + bias[n]
- * with x given as the split operand and the weights as packed bits; alpha and
- * bias may be NULL.  fp32 accumulation of exact bf16 products on the MFMA
- * units.  Output addressing: element (m, n) is written at
+ * with x given as the digit operand and the weights as packed bits; alpha and
+ * bias may be NULL.  The sum is accumulated exactly in int32 on the int8 MFMA
+ * units and converted to fp32 once, so it does not depend on summation order;
+ * its error is the rounding of x to 24 bits relative to its row's largest
+ * magnitude (K above 16384 is processed in chunks whose fp32 results are added).
+ * Output addressing: element (m, n) is written at
  *   y[(m / inner) * outer_stride + n * n_stride + (m % inner)]
  * so a row-major [M, N] result is (inner=1, outer_stride=N, n_stride=1) and a
  * convolution result [batch, O, Ho*Wo] is (inner=Ho*Wo, outer_stride=O*Ho*Wo,
  * n_stride=Ho*Wo).  Replaces the Eigen product of affine.cpp:87-95 /
  * convolution.cpp:185-193 for binarised weights. */
-int nbla_hip_gemm_bits_f32(const void *xsplit, const uint32_t *bits,
+int nbla_hip_gemm_bits_f32(const void *xdigits, const uint32_t *bits,
                            const float *alpha, const float *bias, float *y,
                            int64_t M, int64_t K, int64_t N, int64_t inner,
                            int64_t outer_stride, int64_t n_stride,

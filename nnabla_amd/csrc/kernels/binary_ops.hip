@@ -17,7 +17,7 @@ AffineWorkspace plan_affine(int64_t M, int64_t K, int64_t N) {
   w.bits_off = off;
   off += round_up(nbla_hip_packed_bits_bytes(K, N), 256);
   w.split_off = off;
-  off += round_up(nbla_hip_split_operand_bytes(M, K), 256);
+  off += round_up(nbla_hip_digit_operand_bytes(M, K), 256);
   w.prep_off = off;
   off += round_up(nbla_hip_binarize_workspace_bytes(K, N), 256);
   w.count_off = off;
@@ -38,7 +38,7 @@ int binary_affine_forward(const float *x, const float *W, float *Wb, float *alph
                 ws.total);
   char *base = static_cast<char *>(workspace);
   uint32_t *bits = reinterpret_cast<uint32_t *>(base + ws.bits_off);
-  void *xsplit = base + ws.split_off;
+  void *xsplit = base + ws.split_off; // digit operand of x
   void *prep = base + ws.prep_off;
   int *count = reinterpret_cast<int *>(base + ws.count_off);
   const bool representable = (zero_to == 1.0f || zero_to == -1.0f);
@@ -59,7 +59,7 @@ int binary_affine_forward(const float *x, const float *W, float *Wb, float *alph
     if (host_count != 0)
       return launch_gemm_f32(x, Wb, alpha, bias, y, M, K, N, as_stream(stream_));
   }
-  rc = nbla_hip_split_bf16x3_f32(x, K, xsplit, M, K, stream_);
+  rc = nbla_hip_split_digits_f32(x, K, xsplit, M, K, stream_);
   if (rc)
     return rc;
   return nbla_hip_gemm_bits_f32(xsplit, bits, alpha, bias, y, M, K, N, 1, N, 1, stream_);

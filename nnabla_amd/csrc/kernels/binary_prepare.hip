@@ -41,9 +41,9 @@ PrepPlan make_prep_plan(int64_t K, int64_t N, bool transposed) {
 
 // W stored [K, N].  Block = 16 teams of 16 threads; team t handles k-tile
 // (slice * 16 + t) of column group blockIdx.x.  Thread (nq, g) of a team owns
-// columns f*32 + 4*nq + {0..3} (f = 0, 1) and k offsets s*16 + g*8 + {0..7}
-// (s = 0, 1): 32 bits for each of four packed words, which are exactly the
-// words of lanes g*32 + 4*nq + {0..3}.
+// columns f*32 + 4*nq + {0..3} (f = 0, 1) and k offsets g*16 + {0..15}:
+// 32 bits for each of four packed words, which are exactly the words of lanes
+// g*32 + 4*nq + {0..3}.
 template <bool kVec>
 __global__ __launch_bounds__(kPrepBlock) void binarize_kn(const float *__restrict__ W, float *__restrict__ Wb,
                                                           uint32_t *__restrict__ bits, float *__restrict__ sums,
@@ -60,11 +60,10 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_kn(const float *__restric
 #pragma unroll
     for (int f = 0; f < 2; ++f) {
       const int64_t n0 = cg * kColGroup + f * 32 + 4 * nq;
+      {
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int64_t k = kt * kTileK + s * 16 + g * 8 + e;
+        for (int j = 0; j < 16; ++j) {
+          const int64_t k = kt * kTileK + g * 16 + j;
           if (k >= K || n0 >= N)
             continue;
           float w[4];
@@ -77,7 +76,7 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_kn(const float *__restric
               w[c] = (n0 + c < N) ? W[k * N + n0 + c] : 1.0f;
           }
           float b[4];
-          const int pos = packed_bit_position(f, s, e);
+          const int pos = packed_bit_position(f, j);
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
             b[c] = sign_of(w[c], zero_to);
@@ -130,7 +129,7 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_kn(const float *__restric
 }
 
 // W stored [K, N], N % 4 == 0, 16-byte aligned: the streaming path.  A wavefront covers two k tiles of one column
-// group; lane = (kt_sub, g, f, nq): columns f*32 + 4*nq + {0..3}, k offsets s*16 + g*8 + e.  Each thread issues its
+// group; lane = (kt_sub, g, f, nq): columns f*32 + 4*nq + {0..3}, k offsets g*16 + j.  Each thread issues its
 // sixteen 128-bit loads up front (sixteen lanes cover 256 contiguous bytes of a row), builds the bits of its half
 // (f) of four packed words, and the two halves are OR-ed across lanes.  |W| column sums are folded in a fixed
 // order: over (g, kt_sub) by shuffles, over the block's wavefronts through LDS.
@@ -147,34 +146,28 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_kn_vec(const float *__res
   const bool col_ok = n0 < N;
   float4_t v[16];
 #pragma unroll
-  for (int s = 0; s < 2; ++s)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int64_t k = kt * kTileK + s * 16 + g * 8 + e;
-      if (col_ok && k < K)
-        v[s * 8 + e] = *reinterpret_cast<const float4_t *>(W + k * N + n0);
-      else
-        v[s * 8 + e] = float4_t{1.0f, 1.0f, 1.0f, 1.0f};
-    }
+  for (int j = 0; j < 16; ++j) {
+    const int64_t k = kt * kTileK + g * 16 + j;
+    if (col_ok && k < K)
+      v[j] = *reinterpret_cast<const float4_t *>(W + k * N + n0);
+    else
+      v[j] = float4_t{1.0f, 1.0f, 1.0f, 1.0f};
+  }
   uint32_t word[4] = {0u, 0u, 0u, 0u};
   float asum[4] = {0.f, 0.f, 0.f, 0.f};
   int nzero = 0;
 #pragma unroll
-  for (int s = 0; s < 2; ++s)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int64_t k = kt * kTileK + s * 16 + g * 8 + e;
+  for (int j = 0; j < 16; ++j) {
+      const int64_t k = kt * kTileK + g * 16 + j;
       const bool in = col_ok && k < K;
-      const float w[4] = {v[s * 8 + e].x, v[s * 8 + e].y, v[s * 8 + e].z, v[s * 8 + e].w};
+      const float w[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
       float b[4];
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         b[c] = sign_of(w[c], zero_to);
         const bool is_zero = !(w[c] > 0.0f) && !(w[c] < 0.0f);
         const bool neg = (w[c] < 0.0f) || (is_zero && zero_to < 0.0f);
-        // bit position of (f, s, e), with f a run-time value: p = 4*(2f+s) + e/2
-        const int pp = 4 * (2 * f + s) + (e >> 1);
-        const int pos = (e & 1) ? 31 - pp : 15 - pp;
+        const int pos = 4 * f + (j >> 2) + 8 * (j & 3); // packed_bit_position with f a run-time value
         word[c] |= (in && neg) ? (1u << pos) : 0u;
         asum[c] += in ? fabsf(w[c]) : 0.0f;
         nzero += (in && is_zero) ? 1 : 0;
@@ -220,7 +213,7 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_kn_vec(const float *__res
 
 // W stored [N, K] (convolution weights viewed [channels_o, col_w]).  Wavefront w
 // of the block handles k-tile blockIdx.y*4 + w of column group blockIdx.x; lane
-// l builds its own packed word from 4 runs of 8 consecutive k of rows n(f).
+// l builds its own packed word from 16 consecutive k of each of its two rows n(f).
 __global__ __launch_bounds__(kPrepBlock) void binarize_nk(const float *__restrict__ W, float *__restrict__ Wb,
                                                           uint32_t *__restrict__ bits, float *__restrict__ sums,
                                                           int *__restrict__ zeros, int64_t K, int64_t N,
@@ -237,17 +230,16 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_nk(const float *__restric
 #pragma unroll
     for (int f = 0; f < 2; ++f) {
       const int64_t n = cg * kColGroup + f * 32 + r;
+      {
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int64_t k = kt * kTileK + s * 16 + g * 8 + e;
+        for (int j = 0; j < 16; ++j) {
+          const int64_t k = kt * kTileK + g * 16 + j;
           if (n < N && k < K) {
             const float w = W[n * K + k];
             Wb[n * K + k] = sign_of(w, zero_to);
             const bool is_zero = !(w > 0.0f) && !(w < 0.0f);
             const bool neg = (w < 0.0f) || (is_zero && zero_to < 0.0f);
-            word |= neg ? (1u << packed_bit_position(f, s, e)) : 0u;
+            word |= neg ? (1u << packed_bit_position(f, j)) : 0u;
             asum[f] += fabsf(w);
             nzero += is_zero ? 1 : 0;
           }
@@ -408,6 +400,178 @@ __global__ __launch_bounds__(kPrepBlock) void split_bf16x3_tiled(const float *__
   }
 }
 
+// ------------------------------------------------------------ digit operand
+// Largest shift s with rint(amax * 2^s) <= kDigitMax, for amax > 0 finite given as its bit pattern.
+__device__ __forceinline__ int digit_shift(uint32_t amax_bits) {
+  const int e = binade_exponent(binade_of(amax_bits)); // amax in [2^e, 2^(e+1))
+  int s = 22 - e;                                      // amax * 2^s in [2^22, 2^23)
+  if (rintf(ldexpf(__uint_as_float(amax_bits), s)) > (float)kDigitMax)
+    --s;
+  return s;
+}
+__device__ __forceinline__ int to_fixed(float v, int s) { return (int)rintf(ldexpf(v, s)); }
+
+// q = d0 * 65536 + d1 * 256 + d2 with every digit in [-128, 127]
+__device__ __forceinline__ void balanced_digits(int q, uint32_t &d0, uint32_t &d1, uint32_t &d2) {
+  const int lo = (int)(int8_t)q;
+  const int q1 = (q - lo) >> 8;
+  const int mid = (int)(int8_t)q1;
+  const int hi = (q1 - mid) >> 8;
+  d0 = (uint32_t)hi & 0xffu;
+  d1 = (uint32_t)mid & 0xffu;
+  d2 = (uint32_t)lo & 0xffu;
+}
+
+// Sixteen fixed-point values of one lane -> its 16 bytes of each digit fragment.
+__device__ __forceinline__ void store_digits(const int (&q)[16], uint4_t *dst, bool streaming) {
+  uint32_t w[3][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    uint32_t d0, d1, d2;
+    balanced_digits(q[j], d0, d1, d2);
+    const int sh = 8 * (j & 3);
+    w[0][j >> 2] |= d0 << sh;
+    w[1][j >> 2] |= d1 << sh;
+    w[2][j >> 2] |= d2 << sh;
+  }
+#pragma unroll
+  for (int d = 0; d < 3; ++d) {
+    uint4_t o;
+    o.x = w[d][0], o.y = w[d][1], o.z = w[d][2], o.w = w[d][3];
+    if (streaming)
+      __builtin_nontemporal_store(o, dst + d * 64);
+    else
+      dst[d * 64] = o;
+  }
+}
+
+// One wavefront per (padded) row: the row's shift and, per chunk of kChunkK columns, the sum of its fixed-point
+// values.  The second sweep over the row is served by the caches.
+template <bool kVec>
+__global__ __launch_bounds__(kPrepBlock) void digit_row_scale(const float *__restrict__ x, int64_t ldx,
+                                                              int32_t *__restrict__ sum_hi, int32_t *__restrict__ sum_lo,
+                                                              int32_t *__restrict__ shift, int64_t M, int64_t K,
+                                                              int64_t rows, int64_t chunks) {
+  const int lane = threadIdx.x & 63;
+  const int64_t m = (int64_t)blockIdx.x * (kPrepBlock / 64) + (threadIdx.x >> 6);
+  if (m >= rows)
+    return;
+  if (m >= M) {
+    if (lane == 0)
+      shift[m] = 0;
+    for (int64_t c = lane; c < chunks; c += 64)
+      sum_hi[c * rows + m] = 0, sum_lo[c * rows + m] = 0;
+    return;
+  }
+  const float *row = x + m * ldx;
+  uint32_t amax = 0u;
+  if (kVec) {
+    for (int64_t k = 4 * lane; k < K; k += 256) { // K % 4 == 0
+      const float4_t v = *reinterpret_cast<const float4_t *>(row + k);
+      const uint32_t a = __float_as_uint(v.x) & 0x7fffffffu, b = __float_as_uint(v.y) & 0x7fffffffu;
+      const uint32_t c = __float_as_uint(v.z) & 0x7fffffffu, d = __float_as_uint(v.w) & 0x7fffffffu;
+      amax = max(max(amax, max(a, b)), max(c, d));
+    }
+  } else {
+    for (int64_t k = lane; k < K; k += 64)
+      amax = max(amax, __float_as_uint(row[k]) & 0x7fffffffu);
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1)
+    amax = max(amax, (uint32_t)__shfl_xor((int)amax, off));
+  const bool bad = amax >= 0x7f800000u;
+  const int s = (bad || amax == 0u) ? 0 : digit_shift(amax);
+  if (lane == 0)
+    shift[m] = bad ? kBadRow : s;
+  for (int64_t c = 0; c < chunks; ++c) {
+    const int64_t k_begin = c * kChunkK, k_end = (k_begin + kChunkK < K) ? k_begin + kChunkK : K;
+    long long acc = 0;
+    if (!bad) {
+      if (kVec) {
+        for (int64_t k = k_begin + 4 * lane; k < k_end; k += 256) {
+          const float4_t v = *reinterpret_cast<const float4_t *>(row + k);
+          acc += (long long)to_fixed(v.x, s) + to_fixed(v.y, s) + to_fixed(v.z, s) + to_fixed(v.w, s);
+        }
+      } else {
+        for (int64_t k = k_begin + lane; k < k_end; k += 64)
+          acc += to_fixed(row[k], s);
+      }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1)
+      acc += __shfl_xor(acc, off);
+    if (lane == 0) {
+      sum_hi[c * rows + m] = (int32_t)(acc >> 16);
+      sum_lo[c * rows + m] = (int32_t)(acc & 0xffff);
+    }
+  }
+}
+
+// One wavefront per (row block, k tile) fragment triple; lane l converts x[rb*32 + l%32][kt*32 + (l/32)*16 + 0..15].
+__global__ __launch_bounds__(kPrepBlock) void split_digits(const float *__restrict__ x, int64_t ldx,
+                                                           const int32_t *__restrict__ shift, uint4_t *__restrict__ out,
+                                                           int64_t M, int64_t K, int64_t k_tiles, int64_t frags) {
+  const int64_t frag = (int64_t)blockIdx.x * (kPrepBlock / 64) + (threadIdx.x >> 6);
+  if (frag >= frags)
+    return;
+  const int lane = threadIdx.x & 63;
+  const int64_t rb = frag / k_tiles, kt = frag - rb * k_tiles;
+  const int64_t m = rb * kFragRows + (lane & 31);
+  const int64_t k0 = kt * kTileK + (lane >> 5) * 16;
+  const int s = shift[m];
+  int q[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j)
+    q[j] = (m < M && k0 + j < K && s != kBadRow) ? to_fixed(x[m * ldx + k0 + j], s) : 0;
+  store_digits(q, out + frag * kDigits * 64 + lane, false);
+}
+
+// Streaming variant for K % 64 == 0, 16-byte aligned rows: a wavefront converts a 32-row x 64-k patch (two k tiles).
+// Global loads are fully coalesced (16 lanes read 256 contiguous bytes of a row); the patch is turned into fragment
+// order through a padded LDS tile.
+__global__ __launch_bounds__(kPrepBlock) void split_digits_tiled(const float *__restrict__ x, int64_t ldx,
+                                                                 const int32_t *__restrict__ shift,
+                                                                 uint4_t *__restrict__ out, int64_t M, int64_t K,
+                                                                 int64_t k_tiles, int64_t patches) {
+  constexpr int kRowStride = 68; // floats: 64 + 4 padding keeps the 128-bit column reads conflict-free
+  __shared__ float tile[kPrepBlock / 64][32 * kRowStride];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t patch = (int64_t)blockIdx.x * (kPrepBlock / 64) + wave;
+  if (patch >= patches)
+    return;
+  const int64_t patches_per_row = k_tiles / 2;
+  const int64_t rb = patch / patches_per_row, kq = patch - rb * patches_per_row;
+  float *t = tile[wave];
+  const int lr = lane >> 4, lc = (lane & 15) * 4;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int row = j * 4 + lr;
+    const int64_t m = rb * kFragRows + row;
+    float4_t v = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (m < M)
+      v = *reinterpret_cast<const float4_t *>(x + m * ldx + kq * 64 + lc);
+    *reinterpret_cast<float4_t *>(t + row * kRowStride + lc) = v;
+  }
+  const int r = lane & 31, g = lane >> 5;
+  const int s = shift[rb * kFragRows + r];
+  // the tile is private to this wavefront: LDS operations of one wavefront complete in order
+  __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    int q[16];
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+      const float4_t a = *reinterpret_cast<const float4_t *>(t + r * kRowStride + h * 32 + g * 16 + v4 * 4);
+      const bool ok = s != kBadRow;
+      q[v4 * 4 + 0] = ok ? to_fixed(a.x, s) : 0;
+      q[v4 * 4 + 1] = ok ? to_fixed(a.y, s) : 0;
+      q[v4 * 4 + 2] = ok ? to_fixed(a.z, s) : 0;
+      q[v4 * 4 + 3] = ok ? to_fixed(a.w, s) : 0;
+    }
+    store_digits(q, out + ((rb * k_tiles + kq * 2 + h) * kDigits) * 64 + lane, true);
+  }
+}
+
 } // namespace
 } // namespace nbla_hip
 
@@ -422,6 +586,8 @@ size_t nbla_hip_packed_bits_bytes(int64_t K, int64_t N) {
 size_t nbla_hip_split_operand_bytes(int64_t M, int64_t K) {
   return (size_t)split_row_blocks(M) * split_k_blocks(K) * 3 * kFragBytes;
 }
+
+size_t nbla_hip_digit_operand_bytes(int64_t M, int64_t K) { return digit_operand(M, K).total; }
 
 size_t nbla_hip_binarize_workspace_bytes(int64_t K, int64_t N) {
   const PrepPlan a = make_prep_plan(K, N, false), b = make_prep_plan(K, N, true);
@@ -492,6 +658,43 @@ int nbla_hip_split_bf16x3_f32(const float *x, int64_t ldx, void *xsplit, int64_t
                        as_stream(stream_), x, ldx, static_cast<uint4_t *>(xsplit), M, K, k_blocks, frags);
   }
   NBLA_HIP_LAUNCH_CHECK("split_bf16x3");
+  return NBLA_HIP_OK;
+}
+
+int nbla_hip_split_digits_f32(const float *x, int64_t ldx, void *xdigits, int64_t M, int64_t K, void *stream_) {
+  if (M <= 0 || K <= 0 || ldx < K)
+    return fail(NBLA_HIP_ERR_VALUE, "invalid digit operand shape (M=%lld, K=%lld, ldx=%lld).", (long long)M,
+                (long long)K, (long long)ldx);
+  if (!aligned16(xdigits))
+    return fail(NBLA_HIP_ERR_MEMORY, "digit operand buffer must be 16-byte aligned.");
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  hipStream_t stream = as_stream(stream_);
+  const DigitOperand d = digit_operand(M, K);
+  char *base = static_cast<char *>(xdigits);
+  int32_t *sum_hi = reinterpret_cast<int32_t *>(base + d.sum_hi_off);
+  int32_t *sum_lo = reinterpret_cast<int32_t *>(base + d.sum_lo_off);
+  int32_t *shift = reinterpret_cast<int32_t *>(base + d.shift_off);
+  const bool vec = K % 4 == 0 && ldx % 4 == 0 && aligned16(x);
+  const dim3 scale_grid((unsigned)ceil_div(d.rows, kPrepBlock / 64));
+  if (vec)
+    hipLaunchKernelGGL(digit_row_scale<true>, scale_grid, dim3(kPrepBlock), 0, stream, x, ldx, sum_hi, sum_lo, shift, M,
+                       K, d.rows, d.chunks);
+  else
+    hipLaunchKernelGGL(digit_row_scale<false>, scale_grid, dim3(kPrepBlock), 0, stream, x, ldx, sum_hi, sum_lo, shift,
+                       M, K, d.rows, d.chunks);
+  NBLA_HIP_LAUNCH_CHECK("digit_row_scale");
+  const int64_t frags = d.row_blocks * d.k_tiles;
+  if (K % 64 == 0 && ldx % 4 == 0 && aligned16(x)) {
+    const int64_t patches = frags / 2;
+    hipLaunchKernelGGL(split_digits_tiled, dim3((unsigned)ceil_div(patches, kPrepBlock / 64)), dim3(kPrepBlock), 0,
+                       stream, x, ldx, shift, static_cast<uint4_t *>(xdigits), M, K, d.k_tiles, patches);
+  } else {
+    hipLaunchKernelGGL(split_digits, dim3((unsigned)ceil_div(frags, kPrepBlock / 64)), dim3(kPrepBlock), 0, stream, x,
+                       ldx, shift, static_cast<uint4_t *>(xdigits), M, K, d.k_tiles, frags);
+  }
+  NBLA_HIP_LAUNCH_CHECK("split_digits");
   return NBLA_HIP_OK;
 }
 

@@ -1,8 +1,8 @@
 // BinaryWeightConvolution / BinaryConnectConvolution forwards (channel-first, up
 // to three spatial dimensions, groups): the convolution is the product
 //   y'[pixel, o] = sum_k col[pixel, k] * Wb[o, k],   pixel = (sample, out position), k = (c, kernel tap)
-// The unfolded activations are never materialised in fp32: one kernel gathers
-// them straight into the bf16x3 fragment-ordered operand of the bit-weight MFMA
+// The unfolded activations are never materialised in fp32: they are gathered
+// straight into the fragment-ordered digit operand of the bit-weight MFMA
 // product, whose epilogue scatters into the [sample, O, out position] layout.
 #include "common.hpp"
 #include "gemm_layout.hpp"
@@ -140,6 +140,80 @@ __global__ __launch_bounds__(256) void im2col_split(const float *__restrict__ x,
   dst[128] = o;
 }
 
+// ---- digit operand of the unfolded matrix (the int8 bit-weight product)
+__device__ __forceinline__ int to_fixed(float v, int s) { return (int)rintf(ldexpf(v, s)); }
+
+// One thread per (padded) row of the unfolded matrix: the row's shift and the per-chunk sums of its fixed-point
+// values.  Consecutive threads are consecutive output positions, so each tap is a coalesced read.
+__global__ __launch_bounds__(256) void im2col_row_scale(const float *__restrict__ x, int32_t *__restrict__ sum_hi,
+                                                        int32_t *__restrict__ sum_lo, int32_t *__restrict__ shift,
+                                                        ConvGeom g, int64_t grp, int64_t rows, int64_t chunks) {
+  const int64_t m = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (m >= rows)
+    return;
+  if (m >= g.M) {
+    shift[m] = 0;
+    for (int64_t c = 0; c < chunks; ++c)
+      sum_hi[c * rows + m] = 0, sum_lo[c * rows + m] = 0;
+    return;
+  }
+  uint32_t amax = 0u;
+  for (int64_t k = 0; k < g.Kg; ++k)
+    amax = max(amax, __float_as_uint(col_value(x, g, grp, m, k)) & 0x7fffffffu);
+  const bool bad = amax >= 0x7f800000u;
+  int s = 0;
+  if (!bad && amax != 0u) {
+    const int e = binade_exponent(binade_of(amax));
+    s = 22 - e;
+    if (rintf(ldexpf(__uint_as_float(amax), s)) > (float)kDigitMax)
+      --s;
+  }
+  shift[m] = bad ? kBadRow : s;
+  for (int64_t c = 0; c < chunks; ++c) {
+    const int64_t k_begin = c * kChunkK, k_end = (k_begin + kChunkK < g.Kg) ? k_begin + kChunkK : g.Kg;
+    long long acc = 0;
+    if (!bad)
+      for (int64_t k = k_begin; k < k_end; ++k)
+        acc += to_fixed(col_value(x, g, grp, m, k), s);
+    sum_hi[c * rows + m] = (int32_t)(acc >> 16);
+    sum_lo[c * rows + m] = (int32_t)(acc & 0xffff);
+  }
+}
+
+// One wavefront per (row block, k tile) fragment triple of the digit operand.
+__global__ __launch_bounds__(256) void im2col_digits(const float *__restrict__ x, const int32_t *__restrict__ shift,
+                                                     uint4_t *__restrict__ out, ConvGeom g, int64_t grp,
+                                                     int64_t k_tiles, int64_t frags) {
+  const int64_t frag = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (frag >= frags)
+    return;
+  const int lane = threadIdx.x & 63;
+  const int64_t rb = frag / k_tiles, kt = frag - rb * k_tiles;
+  const int64_t m = rb * kFragRows + (lane & 31);
+  const int64_t k0 = kt * kTileK + (lane >> 5) * 16;
+  const int s = shift[m];
+  uint32_t w[3][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const int q = (m < g.M && k0 + j < g.Kg && s != kBadRow) ? to_fixed(col_value(x, g, grp, m, k0 + j), s) : 0;
+    const int lo = (int)(int8_t)q;
+    const int q1 = (q - lo) >> 8;
+    const int mid = (int)(int8_t)q1;
+    const int hi = (q1 - mid) >> 8;
+    const int sh = 8 * (j & 3);
+    w[0][j >> 2] |= ((uint32_t)hi & 0xffu) << sh;
+    w[1][j >> 2] |= ((uint32_t)mid & 0xffu) << sh;
+    w[2][j >> 2] |= ((uint32_t)lo & 0xffu) << sh;
+  }
+  uint4_t *dst = out + frag * kDigits * 64 + lane;
+#pragma unroll
+  for (int d = 0; d < 3; ++d) {
+    uint4_t o;
+    o.x = w[d][0], o.y = w[d][1], o.z = w[d][2], o.w = w[d][3];
+    dst[d * 64] = o;
+  }
+}
+
 // fp32 unfolded matrix [M, Kg] for the general (non bit-representable) path.
 __global__ __launch_bounds__(256) void im2col_f32(const float *__restrict__ x, float *__restrict__ col, ConvGeom g,
                                                   int64_t grp) {
@@ -158,6 +232,21 @@ int launch_im2col_split(const float *x, void *xsplit, const ConvGeom &g, int64_t
   hipLaunchKernelGGL(im2col_split, dim3((unsigned)ceil_div(frags, 4)), dim3(256), 0, stream, x,
                      static_cast<uint4_t *>(xsplit), g, grp, k_blocks, frags);
   NBLA_HIP_LAUNCH_CHECK("im2col_split");
+  return NBLA_HIP_OK;
+}
+
+int launch_im2col_digits(const float *x, void *xdigits, const ConvGeom &g, int64_t grp, hipStream_t stream) {
+  const DigitOperand d = digit_operand(g.M, g.Kg);
+  char *base = static_cast<char *>(xdigits);
+  int32_t *shift = reinterpret_cast<int32_t *>(base + d.shift_off);
+  hipLaunchKernelGGL(im2col_row_scale, dim3((unsigned)ceil_div(d.rows, 256)), dim3(256), 0, stream, x,
+                     reinterpret_cast<int32_t *>(base + d.sum_hi_off), reinterpret_cast<int32_t *>(base + d.sum_lo_off),
+                     shift, g, grp, d.rows, d.chunks);
+  NBLA_HIP_LAUNCH_CHECK("im2col_row_scale");
+  const int64_t frags = d.row_blocks * d.k_tiles;
+  hipLaunchKernelGGL(im2col_digits, dim3((unsigned)ceil_div(frags, 4)), dim3(256), 0, stream, x, shift,
+                     reinterpret_cast<uint4_t *>(base), g, grp, d.k_tiles, frags);
+  NBLA_HIP_LAUNCH_CHECK("im2col_digits");
   return NBLA_HIP_OK;
 }
 
@@ -183,7 +272,7 @@ ConvWorkspace plan_conv(const ConvGeom &g) {
   w.bits_stride = round_up(nbla_hip_packed_bits_bytes(g.Kg, g.Og), 256);
   off += w.bits_stride * g.group;
   w.split_off = off;
-  off += round_up(nbla_hip_split_operand_bytes(g.M, g.Kg), 256);
+  off += round_up(nbla_hip_digit_operand_bytes(g.M, g.Kg), 256);
   w.prep_off = off;
   off += round_up(nbla_hip_binarize_workspace_bytes(g.Kg, g.Og), 256);
   w.count_off = off;
@@ -239,7 +328,7 @@ int binary_conv_forward(const float *x, const float *W, float *Wb, float *alpha,
     const float *ag = alpha ? alpha + grp * g.Og : nullptr;
     const float *bg = bias ? bias + grp * g.Og : nullptr;
     if (use_bits) {
-      rc = launch_im2col_split(x, base + ws.split_off, g, grp, stream);
+      rc = launch_im2col_digits(x, base + ws.split_off, g, grp, stream);
       if (rc)
         return rc;
       rc = launch_gemm_bits(base + ws.split_off,

@@ -1,17 +1,19 @@
-// y = (x . B) * alpha + bias for sign-binarised weights B, on the gfx950 matrix
-// cores.  x arrives as three bf16 planes (x == hi + mid + lo exactly) in MFMA
-// fragment order, B as one bit per weight.  Every product (bf16 plane element
-// times +-1) is exact, and v_mfma_f32_32x32x16_bf16 accumulates in fp32, so the
-// result carries fp32 accumulation error only ("bf16x3" fp32-faithful product).
+// y = (x . B) * alpha + bias for sign-binarised weights B, on the gfx950 matrix cores' int8 path.
 //
-// Work decomposition: a block of kWavesM x kWavesN wavefronts owns a
-// BM x BN output tile and walks K in steps of 32.  Per step it stages
-//   A: BM/32 row blocks x (2 k blocks x 3 planes) fragments = BM/32 * 6 KiB
-//   B: BN/64 column groups x 64 packed words               = BN * 4 B
-// from HBM/L2 into LDS through registers (double-buffered, one barrier per
-// step).  A fragments are read back with one conflict-free 128-bit LDS load per
-// lane; the packed words are expanded to +-1.0 bf16 pairs in registers with two
-// VALU operations per register (shift, and-or).
+// x arrives as the digit operand: per row a power-of-two scale and, per element, the integer q = rint(x * 2^s) as
+// three balanced base-256 digits (int8).  B arrives as one bit per weight and is expanded in registers to bytes
+// b in {0, 1}.  v_mfma_i32_32x32x32_i8 accumulates  sum_k digit * b  exactly in int32, one accumulator per digit, and
+// the epilogue forms  rowsum(q) - 2 * (acc0 * 65536 + acc1 * 256 + acc2)  =  sum_k q * (+-1)  in integer arithmetic
+// before the single conversion to fp32.  The result is therefore independent of tiling and summation order, and its
+// only error is the rounding of x to 24 significant bits relative to the largest magnitude of its row.
+//
+// Work decomposition: a block of kWavesM x kWavesN wavefronts owns a BM x BN output tile and walks K in steps of
+// 64 (two k tiles).  Per step it stages
+//   X: BM/32 row blocks x (2 k tiles x 3 digits) fragments = BM/32 * 6 KiB
+//   B: 2 k tiles x BN/64 column groups x 64 packed words   = BN * 8 B
+// from HBM/L2 straight into LDS (several steps ahead, one barrier per step).  X fragments are read back with one
+// conflict-free 128-bit LDS load per lane; a packed word becomes eight fragment registers with a shift and an AND each.
+// Every wavefront keeps 3 x MF x NF accumulator tiles, so blocks are sized for one wavefront per SIMD.
 #include "common.hpp"
 #include "gemm_layout.hpp"
 #include "internal.hpp"
@@ -19,27 +21,34 @@
 namespace nbla_hip {
 namespace {
 
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef int i32x16_t __attribute__((ext_vector_type(16)));
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
 struct GemmBitsArgs {
-  const uint4_t *xs;    // split operand
-  const uint32_t *bits; // packed weights
-  const float *alpha;   // may be null
-  const float *bias;    // may be null
+  const uint4_t *xd;      // digit fragments
+  const int32_t *sum_hi;  // row sums of this k chunk, high part
+  const int32_t *sum_lo;  // ... low 16 bits
+  const int32_t *shift;   // per-row scale exponents
+  const uint32_t *bits;   // packed weights
+  const float *alpha;     // may be null
+  const float *bias;      // may be null
   float *y;
   int64_t M, N;
-  int64_t row_blocks; // of the split operand
-  int64_t k_blocks;   // fragments along k (2 per k step)
-  int64_t col_groups; // of the packed operand
-  int64_t k_steps;
+  int64_t n_begin, n_end; // column range this launch produces (n_begin a multiple of 64)
+  int64_t row_blocks;     // of the digit operand
+  int64_t x_k_tiles;      // k tiles of the digit operand (even)
+  int64_t b_k_tiles;      // k tiles of the packed operand
+  int64_t col_groups;     // of the packed operand
+  int64_t step_begin, step_end; // k steps (of two k tiles) this launch covers
   int64_t blocks_m, blocks_n;
   int64_t inner, outer_stride, n_stride; // output addressing
+  int accumulate; // add to y instead of overwriting it (k chunks after the first)
+  int finish;     // apply alpha and bias (last k chunk)
 };
 
 // Blocks are handed to the 8 XCDs round-robin; give each XCD a contiguous run
-// of tiles (n fastest) so that blocks resident on one XCD share an A panel in
+// of tiles (n fastest) so that blocks resident on one XCD share an X panel in
 // that XCD's L2.
 __device__ __forceinline__ int64_t xcd_remap(int64_t b, int64_t total) {
   constexpr int64_t kXcds = 8;
@@ -50,228 +59,252 @@ __device__ __forceinline__ int64_t xcd_remap(int64_t b, int64_t total) {
   return start + slot;
 }
 
+// LDS buffers (k steps resident) per tile shape: as many as 160 KiB allow, at most four.
+constexpr int gemm_bits_stages(int BM, int BN) {
+  const int stage = (BM / 32) * 2 * kDigits * kFragBytes + 2 * BN * 4;
+  return 4 * stage <= 140 * 1024 ? 4 : 3;
+}
+
+// sum_k q_k * (+-1) as fp32 from the three digit accumulators and the row sum (hi * 65536 + lo), scaled by 2^-shift.
+// Integer arithmetic up to the last step: the high and low parts are combined by one fused multiply-add, whose
+// operands are exact (|hi part| < 2^24, low part reduced to 16 bits).
+__device__ __forceinline__ float finish_dot(int a0, int a1, int a2, int s_hi, int s_lo, int shift) {
+  int u = s_hi - 2 * a0;
+  int v = s_lo - 2 * (a1 * 256 + a2);
+  u += v >> 16;
+  v &= 0xffff;
+  const float r = fmaf((float)u, 65536.0f, (float)v);
+  return ldexpf(r, -shift);
+}
+
+// vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
+#define NBLA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xf) | (((n) >> 4) << 14) | (0x7 << 4) | (0xf << 8))
+
 // kSwap exchanges the MFMA operand roles (the instruction computes the transposed 32x32 tile), which puts
 // consecutive m on consecutive lanes of the accumulator: the store pattern for outputs whose m index is contiguous.
+//
+// Staging: global -> LDS copies bypass the registers (global_load_lds): one wavefront instruction moves one 1 KiB
+// digit fragment, or 64 packed words, to the same lane order in LDS.  kStages LDS buffers hold consecutive k steps;
+// the copy of step ks + kStages - 1 is issued while step ks is being multiplied.
 template <int BM, int BN, int kWavesM, int kWavesN, bool kSwap>
 __global__ __launch_bounds__(kWavesM *kWavesN * 64) void gemm_bits_kernel(GemmBitsArgs a) {
-  constexpr int kThreads = kWavesM * kWavesN * 64;
-  constexpr int MF = BM / kWavesM / 32;  // A fragments per wavefront (rows)
+#if defined(__HIP_DEVICE_COMPILE__) // the host pass only needs the launch stub; the body uses LDS address-space pointers
+  constexpr int kWaves = kWavesM * kWavesN;
+  constexpr int MF = BM / kWavesM / 32;  // X fragments per wavefront (rows)
   constexpr int NF = BN / kWavesN / 32;  // B fragments per wavefront (columns)
-  constexpr int NW = NF / 2;             // packed words per lane per k step
+  constexpr int NW = NF / 2;             // packed words per lane per k tile
   static_assert(NF % 2 == 0, "a packed word serves two column fragments");
-  constexpr int kASegs = BM / 32;        // row blocks per tile
-  constexpr int kASegVec = 6 * 64;       // uint4 per row block per k step (2 k blocks x 3 planes)
-  constexpr int kAVec = kASegs * kASegVec;
-  constexpr int kAPasses = (kAVec + kThreads - 1) / kThreads;
-  constexpr int kBWords = BN;            // BN/64 groups x 64 words
-  constexpr int kBPasses = (kBWords + kThreads - 1) / kThreads;
-  constexpr int kStageBytes = kAVec * 16 + kBWords * 4;
+  constexpr int kASegs = BM / 32;            // row blocks per tile
+  constexpr int kSegFrags = 2 * kDigits;     // fragments per row block per k step (2 k tiles x 3 digits)
+  constexpr int kAFrags = kASegs * kSegFrags;
+  constexpr int kBChunks = 2 * BN / 64;      // 64-word chunks per k step (2 k tiles x BN/64 column groups)
+  static_assert(kAFrags % kWaves == 0 && kBChunks % kWaves == 0, "every wavefront issues the same number of copies");
+  constexpr int kAPerWave = kAFrags / kWaves, kBPerWave = kBChunks / kWaves;
+  constexpr int kLoadsPerStage = kAPerWave + kBPerWave;
+  constexpr int kABytes = kAFrags * kFragBytes;
+  constexpr int kStageBytes = kABytes + kBChunks * 256;
+  constexpr int kStages = gemm_bits_stages(BM, BN);
+  constexpr int kDepth = kStages - 1; // k steps in flight ahead of the one being multiplied
+  static_assert(kDepth >= 1 && (kDepth - 1) * kLoadsPerStage < 64, "vmcnt is a 6-bit counter");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave % kWavesM, wn = wave / kWavesM;
 
   const int64_t tile = xcd_remap(blockIdx.x, a.blocks_m * a.blocks_n);
   const int64_t bm = tile / a.blocks_n, bn = tile - bm * a.blocks_n;
 
-  // Per-thread source pointers of the global -> LDS copy (constant over k but for
-  // a fixed advance per step).  Row blocks / column groups past the end of the
-  // operand are clamped: their products land in rows/columns that are not stored.
-  const uint4_t *a_src[kAPasses];
+  // Sources of this wavefront's copies (uniform bases; the lane adds its own 16 / 4 bytes).  Row blocks / column
+  // groups past the end of the operand are clamped: their products land in rows/columns that are not stored.
+  const uint4_t *a_src[kAPerWave];
 #pragma unroll
-  for (int p = 0; p < kAPasses; ++p) {
-    const int idx = p * kThreads + tid;
-    const int seg = idx / kASegVec, within = idx - seg * kASegVec;
+  for (int p = 0; p < kAPerWave; ++p) {
+    const int f = p * kWaves + wave;
+    const int seg = f / kSegFrags, rem = f - seg * kSegFrags;
     int64_t rb = bm * kASegs + seg;
     if (rb >= a.row_blocks)
       rb = a.row_blocks - 1;
-    a_src[p] = a.xs + rb * a.k_blocks * 192 + within;
+    a_src[p] = a.xd + (rb * a.x_k_tiles * kDigits + rem) * 64;
   }
-  const uint32_t *b_src[kBPasses];
+  const uint32_t *b_src[kBPerWave];
+  int b_tile[kBPerWave];
 #pragma unroll
-  for (int p = 0; p < kBPasses; ++p) {
-    const int idx = p * kThreads + tid;
-    int64_t cg = bn * (BN / 64) + idx / 64;
+  for (int p = 0; p < kBPerWave; ++p) {
+    const int c = p * kWaves + wave;
+    b_tile[p] = c / (BN / 64);
+    int64_t cg = a.n_begin / 64 + bn * (BN / 64) + (c - b_tile[p] * (BN / 64));
     if (cg >= a.col_groups)
       cg = a.col_groups - 1;
-    b_src[p] = a.bits + cg * 64 + (idx & 63);
+    b_src[p] = a.bits + cg * 64;
   }
-
-  uint4_t a_reg[kAPasses];
-  uint32_t b_reg[kBPasses];
-
-  auto load_step = [&](int64_t ks) {
+  typedef __attribute__((address_space(3))) void lds_void_t;
+  auto lds_at = [&](int byte_off) { return (lds_void_t *)(smem + byte_off); };
+  // issues the copies of k step `ks` into LDS buffer `buf`
+  auto copy_step = [&](int64_t ks, int buf) {
 #pragma unroll
-    for (int p = 0; p < kAPasses; ++p)
-      if (kAVec % kThreads == 0 || p * kThreads + tid < kAVec)
-        a_reg[p] = a_src[p][ks * kASegVec];
+    for (int p = 0; p < kAPerWave; ++p)
+      __builtin_amdgcn_global_load_lds(a_src[p] + ks * (kSegFrags * 64) + lane,
+                                       lds_at(buf * kStageBytes + (p * kWaves + wave) * kFragBytes), 16, 0, 0);
 #pragma unroll
-    for (int p = 0; p < kBPasses; ++p)
-      if (kBWords % kThreads == 0 || p * kThreads + tid < kBWords)
-        b_reg[p] = b_src[p][ks * a.col_groups * 64];
-  };
-  auto store_step = [&](int buf) {
-    uint4_t *sa = reinterpret_cast<uint4_t *>(smem + buf * kStageBytes);
-    uint32_t *sb = reinterpret_cast<uint32_t *>(smem + buf * kStageBytes + kAVec * 16);
-#pragma unroll
-    for (int p = 0; p < kAPasses; ++p)
-      if (kAVec % kThreads == 0 || p * kThreads + tid < kAVec)
-        sa[p * kThreads + tid] = a_reg[p];
-#pragma unroll
-    for (int p = 0; p < kBPasses; ++p)
-      if (kBWords % kThreads == 0 || p * kThreads + tid < kBWords)
-        sb[p * kThreads + tid] = b_reg[p];
+    for (int p = 0; p < kBPerWave; ++p) {
+      // an odd tile count leaves the second tile of the last step without words: any valid word will do, the
+      // digits it meets are zero
+      int64_t kt = 2 * ks + b_tile[p];
+      if (kt >= a.b_k_tiles)
+        kt = a.b_k_tiles - 1;
+      __builtin_amdgcn_global_load_lds(b_src[p] + kt * a.col_groups * 64 + lane,
+                                       lds_at(buf * kStageBytes + kABytes + (p * kWaves + wave) * 256), 4, 0, 0);
+    }
   };
 
-  f32x16_t acc[MF][NF];
+  i32x16_t acc[kDigits][MF][NF];
 #pragma unroll
-  for (int i = 0; i < MF; ++i)
+  for (int d = 0; d < kDigits; ++d)
 #pragma unroll
-    for (int j = 0; j < NF; ++j)
+    for (int i = 0; i < MF; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        acc[i][j][r] = 0.0f;
+      for (int j = 0; j < NF; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          acc[d][i][j][r] = 0;
 
-  // Fragment fetch and the MFMA block of one k16 sub-step (s = 0, 1) of a staged tile.
-  auto read_a = [&](int buf, int s, uint4_t (&af)[MF][3]) {
+  // Fragment fetch and the MFMA block of one k tile (t = 0, 1) of a staged step.
+  auto read_a = [&](int buf, int t, uint4_t (&af)[MF][kDigits]) {
     const uint4_t *sa = reinterpret_cast<const uint4_t *>(smem + buf * kStageBytes);
 #pragma unroll
     for (int i = 0; i < MF; ++i)
 #pragma unroll
-      for (int p = 0; p < 3; ++p)
-        af[i][p] = sa[(wm * MF + i) * kASegVec + s * 192 + p * 64 + lane];
+      for (int d = 0; d < kDigits; ++d)
+        af[i][d] = sa[((wm * MF + i) * kSegFrags + t * kDigits + d) * 64 + lane];
   };
-  auto read_words = [&](int buf, uint32_t (&words)[NW]) {
-    const uint32_t *sb = reinterpret_cast<const uint32_t *>(smem + buf * kStageBytes + kAVec * 16);
+  auto read_words = [&](int buf, int t, uint32_t (&words)[NW]) {
+    const uint32_t *sb = reinterpret_cast<const uint32_t *>(smem + buf * kStageBytes + kABytes);
 #pragma unroll
     for (int w = 0; w < NW; ++w)
-      words[w] = sb[(wn * NW + w) * 64 + lane];
+      words[w] = sb[t * BN + (wn * NW + w) * 64 + lane];
   };
-  // Bits -> +-1.0 bf16 pairs: register i of fragment (f, s) is ((word << 4*(2f+s)+i) & 0x80008000) | 0x3F803F80.
-  // The two constants are kept in registers so that each register costs a shift and one v_and_or_b32.
-  uint32_t sign_mask = 0x80008000u, one_pair = 0x3F803F80u;
-  asm volatile("" : "+s"(sign_mask));
-  asm volatile("" : "+v"(one_pair));
-  auto expand = [&](int s, const uint32_t (&words)[NW], uint4_t (&bf)[NF]) {
+  // Bits -> bytes in {0, 1}: register i of column half f is (word >> (4 f + i)) & 0x01010101.
+  uint32_t byte_ones = 0x01010101u;
+  asm volatile("" : "+s"(byte_ones));
+  auto mma = [&](const uint4_t (&af)[MF][kDigits], const uint32_t (&words)[NW]) {
 #pragma unroll
     for (int j = 0; j < NF; ++j) {
       const uint32_t w = words[j >> 1];
-      const int base = 4 * (2 * (j & 1) + s);
-      bf[j].x = ((w << (base + 0)) & sign_mask) | one_pair;
-      bf[j].y = ((w << (base + 1)) & sign_mask) | one_pair;
-      bf[j].z = ((w << (base + 2)) & sign_mask) | one_pair;
-      bf[j].w = ((w << (base + 3)) & sign_mask) | one_pair;
-    }
-  };
-  auto mma = [&](const uint4_t (&af)[MF][3], const uint4_t (&bf)[NF]) {
-    // smallest plane first: the low-order parts enter the accumulator before the leading one
+      const int base = 4 * (j & 1);
+      uint4_t bf;
+      bf.x = (w >> (base + 0)) & byte_ones;
+      bf.y = (w >> (base + 1)) & byte_ones;
+      bf.z = (w >> (base + 2)) & byte_ones;
+      bf.w = (w >> (base + 3)) & byte_ones;
 #pragma unroll
-    for (int p = 2; p >= 0; --p)
+      for (int d = 0; d < kDigits; ++d)
 #pragma unroll
-      for (int i = 0; i < MF; ++i)
-#pragma unroll
-        for (int j = 0; j < NF; ++j) {
-          acc[i][j] = kSwap ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[j]),
-                                                                      __builtin_bit_cast(bf16x8_t, af[i][p]),
-                                                                      acc[i][j], 0, 0, 0)
-                            : __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[i][p]),
-                                                                      __builtin_bit_cast(bf16x8_t, bf[j]),
-                                                                      acc[i][j], 0, 0, 0);
+        for (int i = 0; i < MF; ++i) {
+          acc[d][i][j] = kSwap ? __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, bf),
+                                                                       __builtin_bit_cast(i32x4_t, af[i][d]),
+                                                                       acc[d][i][j], 0, 0, 0)
+                               : __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, af[i][d]),
+                                                                       __builtin_bit_cast(i32x4_t, bf),
+                                                                       acc[d][i][j], 0, 0, 0);
         }
+    }
   };
   // Asks the scheduler to issue the region just written as: one MFMA, then a few VALU / memory instructions in
   // its shadow, repeated.  A wavefront issues in order and an MFMA occupies the matrix pipe for 32 cycles, so the
-  // expansion, fragment fetch and staging traffic of the next sub-step fit between consecutive MFMAs instead of
-  // in front of them (where wavefronts running in lockstep would all leave the matrix pipe idle together).
-  constexpr int kMfma = 3 * MF * NF;
+  // expansion, fragment fetch and copy issue of the next k tile fit between consecutive MFMAs instead of in front
+  // of them.
+  constexpr int kMfma = kDigits * MF * NF;
   constexpr int kValuPer = (NF * 8 + 8 + kMfma - 1) / kMfma + 1;
-  auto interleave_first = [&]() { // region: LDS reads of sub-step 1, expansion, MFMAs of sub-step 0, LDS staging writes
+  auto interleave = [&](bool with_copies) {
+#ifdef NBLA_NO_HINTS
+    return;
+#endif
 #pragma unroll
     for (int g = 0; g < kMfma; ++g) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
-      if (g < MF * 3)
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
-      __builtin_amdgcn_sched_group_barrier(0x002, kValuPer, 0); // VALU
-      if (g >= kMfma - kAPasses - kBPasses)
-        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // DS write
-    }
-  };
-  auto interleave_second = [&]() { // region: global loads, LDS reads of the next stage, expansion, MFMAs of sub-step 1
-#pragma unroll
-    for (int g = 0; g < kMfma; ++g) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
-      if (g < kAPasses + kBPasses)
+      if (with_copies && g < kLoadsPerStage)
         __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // VMEM read
-      if (g < MF * 3 + NW)
+      if (g < MF * kDigits + NW)
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
       __builtin_amdgcn_sched_group_barrier(0x002, kValuPer, 0); // VALU
     }
   };
 
-  // Software pipeline.  Two LDS stages, one barrier per k step, no branches in the loop body (the last iterations
-  // re-load the final stage instead of skipping, so each half of the body is one scheduling region).  While the
-  // MFMA block of one k16 sub-step runs, the A fragments of the next sub-step are fetched from LDS and its B
-  // fragments are expanded; the global loads of stage ks+2 are issued a full step ahead of their use.
-  uint4_t af0[MF][3], af1[MF][3], bf0[NF], bf1[NF];
-  uint32_t wcur[NW], wnext[NW];
-  const int64_t last = a.k_steps - 1;
-  load_step(0);
-  store_step(0);
-  __syncthreads();
-  load_step(last < 1 ? last : 1);
-  read_words(0, wcur);
-  read_a(0, 0, af0);
-  expand(0, wcur, bf0);
-  for (int64_t ks = 0; ks <= last; ++ks) {
-    const int buf = (int)(ks & 1);
-    // sub-step 0 runs; sub-step 1 is prepared; the staged registers (stage ks+1) go to the other LDS buffer
-    read_a(buf, 1, af1);
-    expand(1, wcur, bf1);
-    mma(af0, bf0);
-    store_step(buf ^ 1);
-    interleave_first();
-    __syncthreads();
-    // sub-step 1 runs; global loads of stage ks+2 are issued; sub-step 0 of stage ks+1 is prepared
-    load_step(ks + 2 < last ? ks + 2 : last);
-    read_words(buf ^ 1, wnext);
-    read_a(buf ^ 1, 0, af0);
-    expand(0, wnext, bf0);
-    mma(af1, bf1);
-    interleave_second();
+  // Software pipeline.  One barrier per k step, in the middle of it, no branches in the loop body (the last
+  // iterations copy the final step again instead of skipping).  While the MFMA block of one k tile runs, the
+  // fragments of the next one are fetched from LDS.
+  uint4_t af0[MF][kDigits], af1[MF][kDigits];
+  uint32_t w0[NW], w1[NW];
+  const int64_t first = a.step_begin, last = a.step_end - 1;
 #pragma unroll
-    for (int w = 0; w < NW; ++w)
-      wcur[w] = wnext[w];
+  for (int d = 0; d < kDepth; ++d)
+    copy_step(first + d < last ? first + d : last, d);
+  NBLA_WAIT_VMCNT((kDepth - 1) * kLoadsPerStage);
+  __syncthreads();
+  read_words(0, 0, w0);
+  read_a(0, 0, af0);
+  int buf = 0; // LDS buffer of step ks
+  for (int64_t ks = first; ks <= last; ++ks) {
+    const int buf_next = (buf + 1 == kStages) ? 0 : buf + 1;
+    const int buf_copy = (buf == 0) ? kStages - 1 : buf - 1; // the buffer step ks-1 occupied = that of step ks+kDepth
+    // tile 0 runs; tile 1 is fetched
+    read_a(buf, 1, af1);
+    read_words(buf, 1, w1);
+    mma(af0, w0);
+    interleave(false);
+    // step ks+1 has landed (the copies of later steps may still be in flight); every wavefront is done with the
+    // buffer of step ks-1
+    NBLA_WAIT_VMCNT((kDepth - 1) * kLoadsPerStage);
+    __syncthreads();
+    // tile 1 runs; the copy of step ks+kDepth is issued; tile 0 of step ks+1 is fetched
+    copy_step(ks + kDepth < last ? ks + kDepth : last, buf_copy);
+    read_words(buf_next, 0, w0);
+    read_a(buf_next, 0, af0);
+    mma(af1, w1);
+    interleave(true);
+    buf = buf_next;
   }
+  NBLA_WAIT_VMCNT(0);
 
   // Epilogue.  Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
   // column l%32 of the 32x32 fragment; rows are m and columns n, or the reverse
   // under kSwap.
   const int col_in_frag = lane & 31, row_half = lane >> 5;
+  auto emit = [&](int64_t m, int64_t n, float v, float al, float bi) {
+    const int64_t off = (a.inner == 1) ? m * a.outer_stride : (m / a.inner) * a.outer_stride + (m % a.inner);
+    float *dst = a.y + off + n * a.n_stride;
+    if (a.accumulate)
+      v = *dst + v;
+    if (a.finish) {
+      if (a.alpha)
+        v = v * al;
+      if (a.bias)
+        v = v + bi;
+    }
+    *dst = v;
+  };
   if (!kSwap) {
 #pragma unroll
-    for (int j = 0; j < NF; ++j) {
-      const int64_t n = bn * BN + (wn * NF + j) * 32 + col_in_frag;
-      if (n >= a.N)
-        continue;
-      const float al = a.alpha ? a.alpha[n] : 1.0f;
-      const float bi = a.bias ? a.bias[n] : 0.0f;
+    for (int i = 0; i < MF; ++i) {
+      const int64_t m0 = bm * BM + (wm * MF + i) * 32;
 #pragma unroll
-      for (int i = 0; i < MF; ++i) {
-        const int64_t m0 = bm * BM + (wm * MF + i) * 32;
+      for (int r = 0; r < 16; ++r) {
+        const int64_t m = m0 + 8 * (r >> 2) + 4 * row_half + (r & 3);
+        if (m >= a.M)
+          continue;
+        const int s_hi = a.sum_hi[m], s_lo = a.sum_lo[m], sh = a.shift[m];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int64_t m = m0 + 8 * (r >> 2) + 4 * row_half + (r & 3);
-          if (m < a.M) {
-            float v = acc[i][j][r];
-            if (a.alpha)
-              v = v * al;
-            if (a.bias)
-              v = v + bi;
-            const int64_t off = (a.inner == 1) ? m * a.outer_stride : (m / a.inner) * a.outer_stride + (m % a.inner);
-            a.y[off + n * a.n_stride] = v;
-          }
+        for (int j = 0; j < NF; ++j) {
+          const int64_t n = a.n_begin + bn * BN + (wn * NF + j) * 32 + col_in_frag;
+          if (n >= a.n_end)
+            continue;
+          float v = finish_dot(acc[0][i][j][r], acc[1][i][j][r], acc[2][i][j][r], s_hi, s_lo, sh);
+          if (sh == kBadRow)
+            v = __builtin_nanf("");
+          emit(m, n, v, a.alpha ? a.alpha[n] : 1.0f, a.bias ? a.bias[n] : 0.0f);
         }
       }
     }
@@ -281,32 +314,31 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64) void gemm_bits_kernel(GemmBi
       const int64_t m = bm * BM + (wm * MF + i) * 32 + col_in_frag;
       if (m >= a.M)
         continue;
-      const int64_t off = (a.inner == 1) ? m * a.outer_stride : (m / a.inner) * a.outer_stride + (m % a.inner);
+      const int s_hi = a.sum_hi[m], s_lo = a.sum_lo[m], sh = a.shift[m];
 #pragma unroll
       for (int j = 0; j < NF; ++j) {
-        const int64_t n0 = bn * BN + (wn * NF + j) * 32;
+        const int64_t n0 = a.n_begin + bn * BN + (wn * NF + j) * 32;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int64_t n = n0 + 8 * (r >> 2) + 4 * row_half + (r & 3);
-          if (n < a.N) {
-            float v = acc[i][j][r];
-            if (a.alpha)
-              v = v * a.alpha[n];
-            if (a.bias)
-              v = v + a.bias[n];
-            a.y[off + n * a.n_stride] = v;
-          }
+          if (n >= a.n_end)
+            continue;
+          float v = finish_dot(acc[0][i][j][r], acc[1][i][j][r], acc[2][i][j][r], s_hi, s_lo, sh);
+          if (sh == kBadRow)
+            v = __builtin_nanf("");
+          emit(m, n, v, a.alpha ? a.alpha[n] : 1.0f, a.bias ? a.bias[n] : 0.0f);
         }
       }
     }
   }
+#endif
 }
 
 template <int BM, int BN, int kWavesM, int kWavesN, bool kSwap>
 int launch_tile(const GemmBitsArgs &args, hipStream_t stream) {
   constexpr int kThreads = kWavesM * kWavesN * 64;
-  constexpr int kStageBytes = (BM / 32) * 6 * 64 * 16 + BN * 4;
-  constexpr int kSmem = 2 * kStageBytes;
+  constexpr int kStageBytes = (BM / 32) * 2 * kDigits * kFragBytes + 2 * BN * 4;
+  constexpr int kSmem = gemm_bits_stages(BM, BN) * kStageBytes;
   auto kernel = gemm_bits_kernel<BM, BN, kWavesM, kWavesN, kSwap>;
   static bool configured = false;
   if (!configured) {
@@ -317,64 +349,82 @@ int launch_tile(const GemmBitsArgs &args, hipStream_t stream) {
   }
   GemmBitsArgs a = args;
   a.blocks_m = ceil_div(a.M, BM);
-  a.blocks_n = ceil_div(a.N, BN);
+  a.blocks_n = ceil_div(a.n_end - a.n_begin, BN);
   hipLaunchKernelGGL(kernel, dim3((unsigned)(a.blocks_m * a.blocks_n)), dim3(kThreads), kSmem, stream, a);
   NBLA_HIP_LAUNCH_CHECK("gemm_bits");
   return NBLA_HIP_OK;
 }
 
-// Tile choice by M (measured on MI355X at K = 4096, N = 11008): the wide 128x512 tile with sixteen wavefronts
-// wins once there are enough row blocks to fill the 256 CUs; smaller tiles keep more blocks in flight below that.
+// Tile choice by M: four wavefronts of 64x128 (one per SIMD, the accumulators take most of the register file) on a
+// 128x256 tile once there are enough row blocks to fill the 256 CUs; smaller tiles keep more blocks in flight
+// below that.
 template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream) {
-  if (a.M >= 3072)
-    return launch_tile<128, 512, 4, 4, kSwap>(a, stream);
   if (a.M > 1024)
-    return launch_tile<128, 256, 2, 4, kSwap>(a, stream);
+    return launch_tile<128, 256, 4, 2, kSwap>(a, stream);
   if (a.M > 32)
-    return launch_tile<64, 256, 2, 4, kSwap>(a, stream);
-  return launch_tile<32, 256, 1, 4, kSwap>(a, stream);
+    return launch_tile<64, 256, 2, 2, kSwap>(a, stream);
+  return launch_tile<32, 256, 1, 2, kSwap>(a, stream);
 }
 
 } // namespace
 
-int launch_gemm_bits(const void *xsplit, const uint32_t *bits, const float *alpha, const float *bias, float *y,
+int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alpha, const float *bias, float *y,
                      int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
                      bool swap_out, hipStream_t stream) {
   if (M <= 0 || K <= 0 || N <= 0 || inner <= 0)
     return fail(NBLA_HIP_ERR_VALUE, "invalid GEMM shape (M=%lld, K=%lld, N=%lld).", (long long)M, (long long)K,
                 (long long)N);
-  if (!aligned16(xsplit) || !aligned16(bits))
+  if (!aligned16(xdigits) || !aligned16(bits))
     return fail(NBLA_HIP_ERR_MEMORY, "GEMM operands must be 16-byte aligned.");
   int rc = ensure_init();
   if (rc)
     return rc;
+  const DigitOperand d = digit_operand(M, K);
+  const char *base = static_cast<const char *>(xdigits);
   GemmBitsArgs a;
-  a.xs = static_cast<const uint4_t *>(xsplit);
+  a.xd = reinterpret_cast<const uint4_t *>(base);
+  a.shift = reinterpret_cast<const int32_t *>(base + d.shift_off);
   a.bits = bits;
   a.alpha = alpha;
   a.bias = bias;
   a.y = y;
   a.M = M;
   a.N = N;
-  a.row_blocks = split_row_blocks(M);
-  a.k_blocks = split_k_blocks(K);
+  a.n_begin = 0;
+  a.n_end = N;
+  a.row_blocks = d.row_blocks;
+  a.x_k_tiles = d.k_tiles;
+  a.b_k_tiles = bits_k_tiles(K);
   a.col_groups = bits_col_groups(N);
-  a.k_steps = bits_k_tiles(K);
   a.blocks_m = a.blocks_n = 0;
   a.inner = inner;
   a.outer_stride = outer_stride;
   a.n_stride = n_stride;
-  return swap_out ? dispatch<true>(a, stream) : dispatch<false>(a, stream);
+  // one launch per chunk of kChunkK columns of x: the int32 accumulators of a chunk cannot overflow, and the fp32
+  // partial results of the chunks are added up in y
+  const int64_t steps_per_chunk = kChunkK / (2 * kTileK), steps = d.k_tiles / 2;
+  for (int64_t c = 0; c < d.chunks; ++c) {
+    a.sum_hi = reinterpret_cast<const int32_t *>(base + d.sum_hi_off) + c * d.rows;
+    a.sum_lo = reinterpret_cast<const int32_t *>(base + d.sum_lo_off) + c * d.rows;
+    a.step_begin = c * steps_per_chunk;
+    a.step_end = (a.step_begin + steps_per_chunk < steps) ? a.step_begin + steps_per_chunk : steps;
+    a.accumulate = c > 0;
+    a.finish = c + 1 == d.chunks;
+    rc = swap_out ? dispatch<true>(a, stream) : dispatch<false>(a, stream);
+    if (rc)
+      return rc;
+  }
+  return NBLA_HIP_OK;
 }
 
 } // namespace nbla_hip
 
 using namespace nbla_hip;
 
-extern "C" int nbla_hip_gemm_bits_f32(const void *xsplit, const uint32_t *bits, const float *alpha, const float *bias,
+extern "C" int nbla_hip_gemm_bits_f32(const void *xdigits, const uint32_t *bits, const float *alpha, const float *bias,
                                       float *y, int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride,
                                       int64_t n_stride, void *stream) {
   // m-contiguous outputs (n_stride != 1) store from the transposed accumulator tile
-  return launch_gemm_bits(xsplit, bits, alpha, bias, y, M, K, N, inner, outer_stride, n_stride, n_stride != 1,
+  return launch_gemm_bits(xdigits, bits, alpha, bias, y, M, K, N, inner, outer_stride, n_stride, n_stride != 1,
                           as_stream(stream));
 }

@@ -14,15 +14,27 @@
 // Rows >= M and columns >= K are zero.  K is padded to a multiple of 32 (two
 // k blocks: one kernel k-step), M to a multiple of 32.
 //
+// (This operand feeds the plane x plane product used where both factors are real numbers.)
+//
+// The bit-weight product runs on v_mfma_i32_32x32x32_i8 instead.  One i8 operand fragment covers 32 rows by 32 k;
+// lane l holds row (l % 32) and sixteen bytes, byte j being k-slot (l / 32) * 16 + j of the k tile.
+//
+// X ("digit operand"): row m of an fp32 matrix is turned into integers q = rint(x * 2^s_m), |q| < 2^23, with one
+// power-of-two scale per row (s_m the largest shift that keeps the row's largest magnitude inside the digit range),
+// and q into three balanced base-256 digits q = d0 * 65536 + d1 * 256 + d2, each an int8:
+//     X'[row_block = m / 32][k_tile = k / 32][digit 0..2][lane][16 x int8]
+// followed, per chunk of kChunkK columns, by the row sums of q split as sum = hi * 65536 + lo (two int32 arrays of
+// row_blocks * 32 entries per chunk), and by the shifts s_m (one int32 array; kBadRow marks a row holding a
+// non-finite value).  Rows >= M and columns >= K are zero.  The number of k tiles is padded to an even count.
+//
 // B ("packed bits"): one bit per weight, set = negative (-1), clear = +1:
 //     B'[k_tile = k / 32][col_group = n / 64][lane] : one uint32 word
-// Lane l's word serves column n = col_group * 64 + f * 32 + (l % 32) for
-// f = 0, 1 and k = k_tile * 32 + s * 16 + (l / 32) * 8 + e for s = 0, 1 and
-// e = 0..7.  With j = 2 f + s, i = e / 2 and p = 4 j + i the bit sits at
-// position 15 - p (e even) or 31 - p (e odd), so that
-//     ((word << p) & 0x80008000) | 0x3F803F80
-// is directly the register holding the bf16 pair (+-1.0, +-1.0) for k = e, e+1
-// of fragment (f, s).  Bits outside [K, N] are clear.
+// Lane l's word serves column n = col_group * 64 + f * 32 + (l % 32) for f = 0, 1 and k-slots (l / 32) * 16 + j,
+// j = 0..15.  The bit of (f, j) sits at position 4 f + j / 4 + 8 (j % 4), so that
+//     (word >> (4 f + i)) & 0x01010101
+// is directly register i of the i8 fragment of column half f holding b = 1 for a negative weight and 0 otherwise
+// (bytes j = 4 i .. 4 i + 3).  With b in {0, 1} the signed product is  sum q * (1 - 2 b) = rowsum(q) - 2 sum q b.
+// Bits outside [K, N] are clear.
 #pragma once
 #include <stdint.h>
 
@@ -41,10 +53,33 @@ __host__ __device__ inline int64_t split_k_blocks(int64_t K) { return ceil_div(K
 __host__ __device__ inline int64_t bits_k_tiles(int64_t K) { return ceil_div(K, kTileK); }
 __host__ __device__ inline int64_t bits_col_groups(int64_t N) { return ceil_div(N, kColGroup); }
 
-// Bit position inside a packed word for fragment (f, s) and k-offset e.
-__host__ __device__ inline int packed_bit_position(int f, int s, int e) {
-  const int p = 4 * (2 * f + s) + (e >> 1);
-  return (e & 1) ? 31 - p : 15 - p;
+// Bit position inside a packed word for column half f and k-slot offset j (0..15) of the lane.
+__host__ __device__ inline int packed_bit_position(int f, int j) { return 4 * f + (j >> 2) + 8 * (j & 3); }
+
+// ---- digit operand geometry
+constexpr int kDigits = 3;
+constexpr int64_t kChunkK = 16384;        // columns whose i32 accumulators are folded together (keeps them < 2^31)
+constexpr int kDigitMax = 8355711;        // 127 * 65536 + 127 * 256 + 127: the largest q three balanced digits hold
+constexpr int kBadRow = -2147483647 - 1;  // shift value marking a row with a NaN or an infinity
+
+__host__ __device__ inline int64_t digit_k_tiles(int64_t K) { return ceil_div(K, 2 * kTileK) * 2; }
+__host__ __device__ inline int64_t digit_chunks(int64_t K) { return ceil_div(K, kChunkK); }
+// byte offsets of the sections of a digit operand
+struct DigitOperand {
+  int64_t row_blocks, k_tiles, rows, chunks;
+  size_t sum_hi_off, sum_lo_off, shift_off, total;
+};
+__host__ __device__ inline DigitOperand digit_operand(int64_t M, int64_t K) {
+  DigitOperand d;
+  d.row_blocks = split_row_blocks(M);
+  d.k_tiles = digit_k_tiles(K);
+  d.rows = d.row_blocks * kFragRows;
+  d.chunks = digit_chunks(K);
+  d.sum_hi_off = (size_t)d.row_blocks * d.k_tiles * kDigits * kFragBytes;
+  d.sum_lo_off = d.sum_hi_off + (size_t)d.chunks * d.rows * sizeof(int32_t);
+  d.shift_off = d.sum_lo_off + (size_t)d.chunks * d.rows * sizeof(int32_t);
+  d.total = d.shift_off + (size_t)d.rows * sizeof(int32_t);
+  return d;
 }
 
 } // namespace nbla_hip

@@ -22,8 +22,9 @@ EXPORTED = (
     "nbla_hip_init", "nbla_hip_last_error", "nbla_hip_version", "nbla_hip_cut_table",
     "nbla_hip_fixed_point_quantize_f32", "nbla_hip_pow2_quantize_f32",
     "nbla_hip_min_max_quantize_workspace_bytes", "nbla_hip_min_max_quantize_f32",
-    "nbla_hip_packed_bits_bytes", "nbla_hip_split_operand_bytes", "nbla_hip_binarize_workspace_bytes",
-    "nbla_hip_binarize_weights_f32", "nbla_hip_split_bf16x3_f32", "nbla_hip_gemm_bits_f32",
+    "nbla_hip_packed_bits_bytes", "nbla_hip_split_operand_bytes", "nbla_hip_digit_operand_bytes",
+    "nbla_hip_binarize_workspace_bytes", "nbla_hip_binarize_weights_f32", "nbla_hip_split_bf16x3_f32",
+    "nbla_hip_split_digits_f32", "nbla_hip_gemm_bits_f32",
     "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_weight_affine_f32",
     "nbla_hip_binary_connect_affine_f32", "nbla_hip_affine_f32",
     "nbla_hip_convolution_output_shape", "nbla_hip_binary_convolution_workspace_bytes",
@@ -56,7 +57,8 @@ def lib():
         L.nbla_hip_last_error.restype = ctypes.c_char_p
         L.nbla_hip_version.restype = ctypes.c_char_p
         for name in ("nbla_hip_min_max_quantize_workspace_bytes", "nbla_hip_packed_bits_bytes",
-                     "nbla_hip_split_operand_bytes", "nbla_hip_binarize_workspace_bytes",
+                     "nbla_hip_split_operand_bytes", "nbla_hip_digit_operand_bytes",
+                     "nbla_hip_binarize_workspace_bytes",
                      "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_convolution_workspace_bytes",
                      "nbla_hip_inq_workspace_bytes", "nbla_hip_inq_affine_workspace_bytes",
                      "nbla_hip_inq_convolution_workspace_bytes"):
@@ -156,6 +158,15 @@ def split_bf16x3(x, M, K, ldx=None, stream=None):
     import torch
     out = torch.empty(lib().nbla_hip_split_operand_bytes(_i64(M), _i64(K)) // 2, dtype=torch.int16, device=x.device)
     check(lib().nbla_hip_split_bf16x3_f32(_p(x), _i64(K if ldx is None else ldx), _p(out), _i64(M), _i64(K),
+                                          _stream(stream)))
+    return out
+
+
+def split_digits(x, M, K, ldx=None, stream=None):
+    """The int8 digit operand of x [M, K] (bytes): digit fragments, row sums, row shifts."""
+    import torch
+    out = torch.empty(lib().nbla_hip_digit_operand_bytes(_i64(M), _i64(K)), dtype=torch.uint8, device=x.device)
+    check(lib().nbla_hip_split_digits_f32(_p(x), _i64(K if ldx is None else ldx), _p(out), _i64(M), _i64(K),
                                           _stream(stream)))
     return out
 

@@ -10,7 +10,7 @@ import torch
 
 import oracle
 from nnabla_amd import kernels
-from util import bits_equal, first_mismatch, max_rel_err, to_np, unpack_bits
+from util import unpack_digits, bits_equal, first_mismatch, max_rel_err, to_np, unpack_bits
 
 pytestmark = pytest.mark.gpu
 
@@ -63,8 +63,58 @@ def test_binarize_transposed_layout(dev, K, N):
     np.testing.assert_allclose(to_np(alpha), np.abs(Wnk.astype(np.float64)).mean(1), rtol=2e-6)
 
 
+@pytest.mark.parametrize("M,K", [(45, 70), (45, 128), (64, 64), (100, 1024), (1, 4096), (3, 16384 + 40)])
+def test_digit_operand(dev, M, K):
+    """The int8 digit operand: q = rint(x * 2^s) with the largest power-of-two scale that keeps the row inside three
+    balanced base-256 digits, digits in fragment order, exact row sums per k chunk (K % 64 == 0 takes the LDS-tiled
+    kernel)."""
+    rng = np.random.RandomState(2)
+    x = (rng.randn(M, K) * np.exp(rng.randn(M, 1) * 8)).astype(np.float32)
+    x[0, :6] = [0.0, -0.0, 1e-30, -3e-5, 3.3e-7, 1.0]
+    if M > 2:
+        x[2] = 0.0
+    q, shift, sums = unpack_digits(to_np(kernels.split_digits(_dev(x, dev), M, K)), M, K)
+    x64 = x.astype(np.float64)
+    expect = np.rint(np.ldexp(x64, shift[:, None].astype(np.int64)))          # exact scaling, ties to even
+    assert np.array_equal(q, expect.astype(np.int64))
+    amax = np.abs(q).max(1)
+    assert (amax <= 8355711).all()
+    nz = np.abs(x).max(1) > 0
+    # the scale is maximal: one more doubling would leave the digit range
+    assert (np.rint(np.ldexp(np.abs(x64).max(1)[nz], shift[nz].astype(np.int64) + 1)) > 8355711).all()
+    assert (shift[~nz] == 0).all()
+    for c in range(sums.shape[0]):
+        assert np.array_equal(sums[c], q[:, c * 16384:(c + 1) * 16384].sum(1))
+    # value error: at most half a unit of the row's scale
+    assert (np.abs(np.ldexp(q.astype(np.float64), -shift[:, None].astype(np.int64)) - x64)
+            <= np.ldexp(0.5, -shift[:, None].astype(np.int64))).all()
+
+
+def test_digit_operand_marks_non_finite_rows(dev):
+    x = np.ones((5, 64), np.float32)
+    x[1, 3] = np.inf
+    x[3, 60] = np.nan
+    W = np.ones((64, 64), np.float32)
+    _, shift, _ = unpack_digits(to_np(kernels.split_digits(_dev(x, dev), 5, 64)), 5, 64)
+    assert shift[1] == -2 ** 31 and shift[3] == -2 ** 31 and shift[0] == shift[2] == shift[4]
+    y, _ = kernels.binary_connect_affine(_dev(x, dev), _dev(W, dev))
+    y = to_np(y)
+    assert np.isnan(y[[1, 3]]).all() and np.array_equal(y[[0, 2, 4]], np.full((3, 64), 64.0, np.float32))
+
+
+@pytest.mark.parametrize("M,K,N", [(3, 16384 + 40, 70), (40, 40000, 64)])
+def test_long_contraction_is_chunked(dev, M, K, N):
+    """K above 16384 is accumulated in int32 per chunk of 16384 columns and the chunks are added in fp32."""
+    x, W = _data(M, K, N, seed=3)
+    b = np.random.RandomState(4).randn(N).astype(np.float32)
+    y, Wb, alpha = kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev), _dev(b, dev))
+    sgn = np.where(W >= 0, 1.0, -1.0)
+    y64 = x.astype(np.float64) @ (sgn * np.abs(W.astype(np.float64)).mean(0)) + b
+    assert max_rel_err(to_np(y), y64) <= TIGHT
+
+
 def test_split_is_exact(dev):
-    """hi + mid + lo == x exactly, in fragment order, zero padded."""
+    """bf16x3 operand of the plane x plane product: hi + mid + lo == x exactly, in fragment order, zero padded."""
     rng = np.random.RandomState(2)
     M, K = 45, 70
     x = (rng.randn(M, K) * np.exp(rng.randn(M, K) * 8)).astype(np.float32)
@@ -109,6 +159,21 @@ def test_binary_connect_affine_matches_oracle(dev, M, K, N):
     y64 = x.astype(np.float64) @ ref_Wb.astype(np.float64) + b
     assert max_rel_err(to_np(y), ref_y) <= TOL
     assert max_rel_err(to_np(y), y64) <= TIGHT
+
+
+@pytest.mark.parametrize("M,K,N", [(3100, 96, 5732), (3072, 64, 11008)])
+def test_tall_m_column_divided_launch(dev, M, K, N):
+    """M >= 3072 with a tile count that is not a whole number of rounds: the columns are produced by two launches
+    with different tile widths; every output element is checked against float64."""
+    x, W = _data(M, K, N, seed=21)
+    b = np.random.RandomState(5).randn(N).astype(np.float32)
+    y, Wb, alpha = kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev), _dev(b, dev))
+    sgn = np.where(W >= 0, 1.0, -1.0)
+    assert bits_equal(to_np(Wb), sgn.astype(np.float32))
+    y64 = x.astype(np.float64) @ (sgn * np.abs(W.astype(np.float64)).mean(0)) + b
+    assert max_rel_err(to_np(y), y64) <= TIGHT
+    yc, _ = kernels.binary_connect_affine(_dev(x, dev), _dev(W, dev))
+    assert max_rel_err(to_np(yc), x.astype(np.float64) @ sgn) <= TIGHT
 
 
 @pytest.mark.parametrize("q0", [0.0, 0.5, -1.0, 1.0])
@@ -167,7 +232,7 @@ def test_config3_full_size_properties(dev, M):
     y, yc, alpha = to_np(y), to_np(yc), to_np(alpha)
     assert bits_equal(to_np(Wb), oracle.sign(W, 1.0))
     rows = rng.choice(M, 24, replace=False)
-    cols = rng.choice(N, 96, replace=False)
+    cols = np.union1d(rng.choice(N, 96, replace=False), [0, 8191, 8192, 8575, 8576, 10999, N - 1])
     sgn = np.sign(W[:, cols]).astype(np.float64)
     ref_c = x[rows].astype(np.float64) @ sgn
     a64 = np.abs(W[:, cols].astype(np.float64)).mean(0)

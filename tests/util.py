@@ -46,13 +46,32 @@ def unpack_bits(bits_words, K, N):
     out = np.ones((k_tiles * 32, col_groups * 64), np.int8)
     lane = np.arange(64)
     for f in range(2):
-        for s in range(2):
-            for e in range(8):
-                p = 4 * (2 * f + s) + (e >> 1)
-                pos = 31 - p if (e & 1) else 15 - p
-                bit = (w >> np.uint32(pos)) & np.uint32(1)  # [kt, cg, lane]
-                k_off = s * 16 + (lane >> 5) * 8 + e        # per lane
-                n_off = f * 32 + (lane & 31)
-                for l in range(64):
-                    out[k_off[l]::32, n_off[l]::64][:k_tiles, :col_groups] = np.where(bit[:, :, l] == 1, -1, 1)
+        for j in range(16):
+            pos = 4 * f + (j >> 2) + 8 * (j & 3)
+            bit = (w >> np.uint32(pos)) & np.uint32(1)  # [kt, cg, lane]
+            k_off = (lane >> 5) * 16 + j                # per lane
+            n_off = f * 32 + (lane & 31)
+            for l in range(64):
+                out[k_off[l]::32, n_off[l]::64][:k_tiles, :col_groups] = np.where(bit[:, :, l] == 1, -1, 1)
     return out[:K, :N]
+
+
+def unpack_digits(raw, M, K):
+    """Digit operand bytes -> (q int64 [M, K], shift int32 [M], row sums int64 [chunks, M]) as the kernels define it:
+    fragments [row_block][k_tile][digit][lane][16 x int8], then sum_hi, sum_lo ([chunks][rows] int32), then shifts."""
+    raw = np.ascontiguousarray(raw).view(np.uint8)
+    rb, kt = (M + 31) // 32, ((K + 63) // 64) * 2
+    rows, chunks = rb * 32, (K + 16383) // 16384
+    nfrag = rb * kt * 3 * 1024
+    d = raw[:nfrag].view(np.int8).reshape(rb, kt, 3, 64, 16).astype(np.int64)
+    qf = d[:, :, 0] * 65536 + d[:, :, 1] * 256 + d[:, :, 2]          # [rb, kt, lane, j]
+    q = np.zeros((rows, kt * 32), np.int64)
+    for lane in range(64):
+        for j in range(16):
+            q[(lane & 31)::32, ((lane >> 5) * 16 + j)::32] = qf[:, :, lane, j]
+    meta = raw[nfrag:].view(np.int32)
+    hi = meta[:chunks * rows].reshape(chunks, rows).astype(np.int64)
+    lo = meta[chunks * rows:2 * chunks * rows].reshape(chunks, rows).astype(np.int64)
+    shift = meta[2 * chunks * rows:2 * chunks * rows + rows]
+    assert not q[M:].any() and not q[:, K:].any()
+    return q[:M, :K], shift[:M].copy(), (hi * 65536 + lo)[:, :M]
