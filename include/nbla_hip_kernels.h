@@ -105,7 +105,8 @@ int nbla_hip_min_max_quantize_f32(const float *x, float *y,
 
 /* ------------------------------------------- binary weights: sign/alpha/pack */
 
-/* Bytes of the 1-bit packed GEMM operand for a [K, N] weight matrix. */
+/* Bytes of the 1-bit packed GEMM operand for a [K, N] weight matrix (K padded
+ * to 32, N to 256). */
 size_t nbla_hip_packed_bits_bytes(int64_t K, int64_t N);
 /* Bytes of the bf16x3-split, fragment-ordered GEMM operand for x [M, K]
  * (the operand of the plane x plane product used by the INQ forwards). */

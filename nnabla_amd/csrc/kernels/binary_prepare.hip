@@ -21,10 +21,10 @@ __device__ __forceinline__ float sign_of(float w, float zero_to) {
 }
 
 // Workspace: colsum partials [slices][Np] floats, then zero-count partials
-// [slices * col_groups] ints.  slices depends on the source layout.
+// [slices * col_groups] ints, then the pair words.  slices depends on the source layout.
 struct PrepPlan {
   int64_t k_tiles, col_groups, Np, slices;
-  size_t sums_bytes, zeros_bytes;
+  size_t sums_bytes, zeros_bytes, pairs_bytes;
 };
 
 PrepPlan make_prep_plan(int64_t K, int64_t N, bool transposed) {
@@ -36,6 +36,7 @@ PrepPlan make_prep_plan(int64_t K, int64_t N, bool transposed) {
   P.slices = transposed ? ceil_div(P.k_tiles, 4) : ceil_div(P.k_tiles, 8);
   P.sums_bytes = round_up((size_t)P.slices * P.Np * sizeof(float), 256);
   P.zeros_bytes = round_up((size_t)P.slices * P.col_groups * sizeof(int), 256);
+  P.pairs_bytes = round_up((size_t)P.k_tiles * P.col_groups * 64 * sizeof(uint32_t), 256);
   return P;
 }
 
@@ -296,6 +297,32 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_finalize(const float *__r
     if (threadIdx.x == 0)
       *zero_count = s_z[0] + s_z[1] + s_z[2] + s_z[3];
   }
+}
+
+// Pair words -> packed operand: thread (k tile, wide group, lane) interleaves the four pair groups of its wide group.
+__global__ __launch_bounds__(kPrepBlock) void widen_bits(const uint32_t *__restrict__ pairs, uint4_t *__restrict__ bits,
+                                                         int64_t col_groups, int64_t wide_groups, int64_t total) {
+  const int64_t idx = (int64_t)blockIdx.x * kPrepBlock + threadIdx.x;
+  if (idx >= total)
+    return;
+  const int lane = (int)(idx & 63);
+  const int64_t t = idx >> 6;
+  const int64_t kt = t / wide_groups, wg = t - kt * wide_groups;
+  uint32_t w[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+    w[q] = (4 * wg + q < col_groups) ? pairs[(kt * col_groups + 4 * wg + q) * 64 + lane] : 0u;
+  uint32_t o[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int f = 0; f < 2; ++f)
+        o[i] |= ((w[q] >> (4 * f + i)) & 0x01010101u) << (2 * q + f);
+  uint4_t v;
+  v.x = o[0], v.y = o[1], v.z = o[2], v.w = o[3];
+  bits[idx] = v;
 }
 
 // ------------------------------------------------------------------ bf16 split
@@ -580,7 +607,7 @@ using namespace nbla_hip;
 extern "C" {
 
 size_t nbla_hip_packed_bits_bytes(int64_t K, int64_t N) {
-  return (size_t)bits_k_tiles(K) * bits_col_groups(N) * 64 * sizeof(uint32_t);
+  return (size_t)bits_k_tiles(K) * bits_wide_groups(N) * 64 * 4 * sizeof(uint32_t);
 }
 
 size_t nbla_hip_split_operand_bytes(int64_t M, int64_t K) {
@@ -591,7 +618,7 @@ size_t nbla_hip_digit_operand_bytes(int64_t M, int64_t K) { return digit_operand
 
 size_t nbla_hip_binarize_workspace_bytes(int64_t K, int64_t N) {
   const PrepPlan a = make_prep_plan(K, N, false), b = make_prep_plan(K, N, true);
-  const size_t wa = a.sums_bytes + a.zeros_bytes, wb = b.sums_bytes + b.zeros_bytes;
+  const size_t wa = a.sums_bytes + a.zeros_bytes + a.pairs_bytes, wb = b.sums_bytes + b.zeros_bytes + b.pairs_bytes;
   return wa > wb ? wa : wb;
 }
 
@@ -601,7 +628,7 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint3
   if (K <= 0 || N <= 0)
     return fail(NBLA_HIP_ERR_VALUE, "weight matrix must not be empty (K=%lld, N=%lld).", (long long)K, (long long)N);
   const PrepPlan P = make_prep_plan(K, N, transposed != 0);
-  if (workspace_bytes < P.sums_bytes + P.zeros_bytes || !aligned256(workspace))
+  if (workspace_bytes < P.sums_bytes + P.zeros_bytes + P.pairs_bytes || !aligned256(workspace))
     return fail(NBLA_HIP_ERR_MEMORY, "binarize workspace too small or misaligned.");
   if (!aligned16(bits))
     return fail(NBLA_HIP_ERR_MEMORY, "packed-bit buffer must be 16-byte aligned.");
@@ -611,24 +638,31 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint3
   hipStream_t stream = as_stream(stream_);
   float *sums = static_cast<float *>(workspace);
   int *zeros = reinterpret_cast<int *>(static_cast<char *>(workspace) + P.sums_bytes);
+  uint32_t *pairs = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + P.sums_bytes + P.zeros_bytes);
   int64_t slices = P.slices;
   if (!transposed) {
     if (N % 4 == 0 && aligned16(W) && aligned16(Wb)) {
       const dim3 grid((unsigned)P.col_groups, (unsigned)P.slices);
-      hipLaunchKernelGGL(binarize_kn_vec, grid, dim3(kPrepBlock), 0, stream, W, Wb, bits, sums, zeros, K, N,
+      hipLaunchKernelGGL(binarize_kn_vec, grid, dim3(kPrepBlock), 0, stream, W, Wb, pairs, sums, zeros, K, N,
                          P.col_groups, P.Np, P.k_tiles, quantize_zero_to);
     } else {
       slices = ceil_div(K, kKSlice);
       const dim3 grid((unsigned)P.col_groups, (unsigned)slices);
-      hipLaunchKernelGGL(binarize_kn<false>, grid, dim3(kPrepBlock), 0, stream, W, Wb, bits, sums, zeros, K, N,
+      hipLaunchKernelGGL(binarize_kn<false>, grid, dim3(kPrepBlock), 0, stream, W, Wb, pairs, sums, zeros, K, N,
                          P.col_groups, P.Np, quantize_zero_to);
     }
   } else {
     const dim3 grid((unsigned)P.col_groups, (unsigned)P.slices);
-    hipLaunchKernelGGL(binarize_nk, grid, dim3(kPrepBlock), 0, stream, W, Wb, bits, sums, zeros, K, N, P.col_groups,
+    hipLaunchKernelGGL(binarize_nk, grid, dim3(kPrepBlock), 0, stream, W, Wb, pairs, sums, zeros, K, N, P.col_groups,
                        P.Np, P.k_tiles, quantize_zero_to);
   }
   NBLA_HIP_LAUNCH_CHECK("binarize_weights");
+  {
+    const int64_t wide_groups = bits_wide_groups(N), total = P.k_tiles * wide_groups * 64;
+    hipLaunchKernelGGL(widen_bits, dim3((unsigned)ceil_div(total, kPrepBlock)), dim3(kPrepBlock), 0, stream, pairs,
+                       reinterpret_cast<uint4_t *>(bits), P.col_groups, wide_groups, total);
+    NBLA_HIP_LAUNCH_CHECK("widen_bits");
+  }
   if (alpha || zero_count) {
     const float inv_k = (float)1 / K;
     hipLaunchKernelGGL(binarize_finalize, dim3((unsigned)ceil_div(N, kPrepBlock)), dim3(kPrepBlock), 0, stream, sums,

@@ -1,9 +1,9 @@
 // y = (x . B) * alpha + bias for sign-binarised weights B, on the gfx950 matrix cores' int8 path.
 //
 // x arrives as the digit operand: per row a power-of-two scale and, per element, the integer q = rint(x * 2^s) as
-// three balanced base-256 digits (int8).  B arrives as one bit per weight and is expanded in registers to bytes
-// b in {0, 1}.  v_mfma_i32_32x32x32_i8 accumulates  sum_k digit * b  exactly in int32, one accumulator per digit, and
-// the epilogue forms  rowsum(q) - 2 * (acc0 * 65536 + acc1 * 256 + acc2)  =  sum_k q * (+-1)  in integer arithmetic
+// three balanced base-256 digits (int8).  B arrives as one bit per weight and is expanded in registers (one AND per
+// register) to bytes b * 2^F, F the column fragment's index inside its 256-column group.  v_mfma_i32_32x32x32_i8 accumulates  sum_k digit * b  exactly in int32, one accumulator per digit, and
+// the epilogue divides the 2^F out and forms  rowsum(q) - 2 * (acc0 * 65536 + acc1 * 256 + acc2)  =  sum_k q * (+-1)  in integer arithmetic
 // before the single conversion to fp32.  The result is therefore independent of tiling and summation order, and its
 // only error is the rounding of x to 24 significant bits relative to the largest magnitude of its row.
 //
@@ -12,11 +12,14 @@
 //   X: BM/32 row blocks x (2 k tiles x 3 digits) fragments = BM/32 * 6 KiB
 //   B: 2 k tiles x BN/64 column groups x 64 packed words   = BN * 8 B
 // from HBM/L2 straight into LDS (several steps ahead, one barrier per step).  X fragments are read back with one
-// conflict-free 128-bit LDS load per lane; a packed word becomes eight fragment registers with a shift and an AND each.
+// conflict-free 128-bit LDS load per lane; four packed words become the four registers of any of eight column fragments
+// with one AND each.
 // Every wavefront keeps 3 x MF x NF accumulator tiles, so blocks are sized for one wavefront per SIMD.
 #include "common.hpp"
 #include "gemm_layout.hpp"
 #include "internal.hpp"
+
+#include <type_traits>
 
 namespace nbla_hip {
 namespace {
@@ -35,11 +38,11 @@ struct GemmBitsArgs {
   const float *bias;      // may be null
   float *y;
   int64_t M, N;
-  int64_t n_begin, n_end; // column range this launch produces (n_begin a multiple of 64)
+  int64_t n_begin, n_end; // column range this launch produces (n_begin a multiple of 256)
   int64_t row_blocks;     // of the digit operand
   int64_t x_k_tiles;      // k tiles of the digit operand (even)
   int64_t b_k_tiles;      // k tiles of the packed operand
-  int64_t col_groups;     // of the packed operand
+  int64_t wide_groups;    // 256-column groups of the packed operand
   int64_t step_begin, step_end; // k steps (of two k tiles) this launch covers
   int64_t blocks_m, blocks_n;
   int64_t inner, outer_stride, n_stride; // output addressing
@@ -68,7 +71,11 @@ constexpr int gemm_bits_stages(int BM, int BN) {
 // sum_k q_k * (+-1) as fp32 from the three digit accumulators and the row sum (hi * 65536 + lo), scaled by 2^-shift.
 // Integer arithmetic up to the last step: the high and low parts are combined by one fused multiply-add, whose
 // operands are exact (|hi part| < 2^24, low part reduced to 16 bits).
-__device__ __forceinline__ float finish_dot(int a0, int a1, int a2, int s_hi, int s_lo, int shift) {
+__device__ __forceinline__ float finish_dot(int a0, int a1, int a2, int s_hi, int s_lo, int shift, int frag) {
+  // accumulators of column fragment `frag` carry the factor 2^frag, or -128 for frag 7 (0x80 as int8)
+  a0 >>= frag, a1 >>= frag, a2 >>= frag;
+  if (frag == 7)
+    a0 = -a0, a1 = -a1, a2 = -a2;
   int u = s_hi - 2 * a0;
   int v = s_lo - 2 * (a1 * 256 + a2);
   u += v >> 16;
@@ -87,25 +94,25 @@ __device__ __forceinline__ float finish_dot(int a0, int a1, int a2, int s_hi, in
 // digit fragment, or 64 packed words, to the same lane order in LDS.  kStages LDS buffers hold consecutive k steps;
 // the copy of step ks + kStages - 1 is issued while step ks is being multiplied.
 template <int BM, int BN, int kWavesM, int kWavesN, bool kSwap>
-__global__ __launch_bounds__(kWavesM *kWavesN * 64) void gemm_bits_kernel(GemmBitsArgs a) {
+__global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 : 2)) void gemm_bits_kernel(GemmBitsArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__) // the host pass only needs the launch stub; the body uses LDS address-space pointers
   constexpr int kWaves = kWavesM * kWavesN;
   constexpr int MF = BM / kWavesM / 32;  // X fragments per wavefront (rows)
   constexpr int NF = BN / kWavesN / 32;  // B fragments per wavefront (columns)
-  constexpr int NW = NF / 2;             // packed words per lane per k tile
-  static_assert(NF % 2 == 0, "a packed word serves two column fragments");
+  static_assert(BN % kWideGroup == 0 && (kWideGroup / 32) % NF == 0, "a wavefront's fragments share one wide group");
   constexpr int kASegs = BM / 32;            // row blocks per tile
   constexpr int kSegFrags = 2 * kDigits;     // fragments per row block per k step (2 k tiles x 3 digits)
   constexpr int kAFrags = kASegs * kSegFrags;
-  constexpr int kBChunks = 2 * BN / 64;      // 64-word chunks per k step (2 k tiles x BN/64 column groups)
-  static_assert(kAFrags % kWaves == 0 && kBChunks % kWaves == 0, "every wavefront issues the same number of copies");
-  constexpr int kAPerWave = kAFrags / kWaves, kBPerWave = kBChunks / kWaves;
-  constexpr int kLoadsPerStage = kAPerWave + kBPerWave;
+  constexpr int kBChunks = 2 * BN / kWideGroup; // 1 KiB chunks of packed words per k step (2 k tiles x wide groups)
+  // One copy instruction moves 1 KiB (a fragment, or the words of one wide group); the kChunks copies of a k step
+  // are dealt round-robin, so wavefronts below kExtra issue one more than the others.
+  constexpr int kChunks = kAFrags + kBChunks;
+  constexpr int kPerWave = kChunks / kWaves, kExtra = kChunks % kWaves;
   constexpr int kABytes = kAFrags * kFragBytes;
-  constexpr int kStageBytes = kABytes + kBChunks * 256;
+  constexpr int kStageBytes = kABytes + kBChunks * kFragBytes;
   constexpr int kStages = gemm_bits_stages(BM, BN);
   constexpr int kDepth = kStages - 1; // k steps in flight ahead of the one being multiplied
-  static_assert(kDepth >= 1 && (kDepth - 1) * kLoadsPerStage < 64, "vmcnt is a 6-bit counter");
+  static_assert(kDepth >= 1 && (kDepth - 1) * (kPerWave + 1) < 64, "vmcnt is a 6-bit counter");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
@@ -117,47 +124,61 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64) void gemm_bits_kernel(GemmBi
   const int64_t tile = xcd_remap(blockIdx.x, a.blocks_m * a.blocks_n);
   const int64_t bm = tile / a.blocks_n, bn = tile - bm * a.blocks_n;
 
-  // Sources of this wavefront's copies (uniform bases; the lane adds its own 16 / 4 bytes).  Row blocks / column
-  // groups past the end of the operand are clamped: their products land in rows/columns that are not stored.
-  const uint4_t *a_src[kAPerWave];
+  // Sources of this wavefront's copies (uniform bases; the lane adds its own 16 bytes).  Row blocks / wide groups
+  // past the end of the operand are clamped: their products land in rows/columns that are not stored.
+  constexpr int kSlots = kPerWave + (kExtra ? 1 : 0);
+  const uint4_t *src[kSlots];
+  int64_t src_step[kSlots]; // advance per k step, in uint4
+  int b_tile[kSlots];       // -1 for a digit fragment, else the k tile (0, 1) of the packed words
 #pragma unroll
-  for (int p = 0; p < kAPerWave; ++p) {
-    const int f = p * kWaves + wave;
-    const int seg = f / kSegFrags, rem = f - seg * kSegFrags;
-    int64_t rb = bm * kASegs + seg;
-    if (rb >= a.row_blocks)
-      rb = a.row_blocks - 1;
-    a_src[p] = a.xd + (rb * a.x_k_tiles * kDigits + rem) * 64;
-  }
-  const uint32_t *b_src[kBPerWave];
-  int b_tile[kBPerWave];
-#pragma unroll
-  for (int p = 0; p < kBPerWave; ++p) {
+  for (int p = 0; p < kSlots; ++p) {
     const int c = p * kWaves + wave;
-    b_tile[p] = c / (BN / 64);
-    int64_t cg = a.n_begin / 64 + bn * (BN / 64) + (c - b_tile[p] * (BN / 64));
-    if (cg >= a.col_groups)
-      cg = a.col_groups - 1;
-    b_src[p] = a.bits + cg * 64;
+    if (c < kAFrags) {
+      const int seg = c / kSegFrags, rem = c - seg * kSegFrags;
+      int64_t rb = bm * kASegs + seg;
+      if (rb >= a.row_blocks)
+        rb = a.row_blocks - 1;
+      src[p] = a.xd + (rb * a.x_k_tiles * kDigits + rem) * 64;
+      src_step[p] = kSegFrags * 64;
+      b_tile[p] = -1;
+    } else {
+      const int cb = (c < kChunks) ? c - kAFrags : 0;
+      b_tile[p] = cb / (BN / kWideGroup);
+      int64_t wg = a.n_begin / kWideGroup + bn * (BN / kWideGroup) + (cb - b_tile[p] * (BN / kWideGroup));
+      if (wg >= a.wide_groups)
+        wg = a.wide_groups - 1;
+      src[p] = reinterpret_cast<const uint4_t *>(a.bits) + wg * 64;
+      src_step[p] = 2 * a.wide_groups * 64;
+    }
   }
   typedef __attribute__((address_space(3))) void lds_void_t;
   auto lds_at = [&](int byte_off) { return (lds_void_t *)(smem + byte_off); };
   // issues the copies of k step `ks` into LDS buffer `buf`
   auto copy_step = [&](int64_t ks, int buf) {
 #pragma unroll
-    for (int p = 0; p < kAPerWave; ++p)
-      __builtin_amdgcn_global_load_lds(a_src[p] + ks * (kSegFrags * 64) + lane,
-                                       lds_at(buf * kStageBytes + (p * kWaves + wave) * kFragBytes), 16, 0, 0);
-#pragma unroll
-    for (int p = 0; p < kBPerWave; ++p) {
-      // an odd tile count leaves the second tile of the last step without words: any valid word will do, the
-      // digits it meets are zero
-      int64_t kt = 2 * ks + b_tile[p];
-      if (kt >= a.b_k_tiles)
-        kt = a.b_k_tiles - 1;
-      __builtin_amdgcn_global_load_lds(b_src[p] + kt * a.col_groups * 64 + lane,
-                                       lds_at(buf * kStageBytes + kABytes + (p * kWaves + wave) * 256), 4, 0, 0);
+    for (int p = 0; p < kSlots; ++p) {
+      if (p == kPerWave && wave >= kExtra)
+        break;
+      // an odd tile count leaves the second tile of the last step without words: any valid words will do, the
+      // digits they meet are zero
+      int64_t adv = ks * src_step[p];
+      if (b_tile[p] >= 0) {
+        int64_t kt = 2 * ks + b_tile[p];
+        if (kt >= a.b_k_tiles)
+          kt = a.b_k_tiles - 1;
+        adv = kt * a.wide_groups * 64;
+      }
+      __builtin_amdgcn_global_load_lds(src[p] + adv + lane, lds_at(buf * kStageBytes + (p * kWaves + wave) * kFragBytes),
+                                       16, 0, 0);
     }
+  };
+  // waits until at most `steps` k steps of this wavefront's copies are in flight
+  auto wait_copies = [&](auto steps) {
+    constexpr int n = decltype(steps)::value;
+    if (kExtra && wave < kExtra)
+      NBLA_WAIT_VMCNT(n * (kPerWave + 1));
+    else
+      NBLA_WAIT_VMCNT(n * kPerWave);
   };
 
   i32x16_t acc[kDigits][MF][NF];
@@ -180,25 +201,26 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64) void gemm_bits_kernel(GemmBi
       for (int d = 0; d < kDigits; ++d)
         af[i][d] = sa[((wm * MF + i) * kSegFrags + t * kDigits + d) * 64 + lane];
   };
-  auto read_words = [&](int buf, int t, uint32_t (&words)[NW]) {
-    const uint32_t *sb = reinterpret_cast<const uint32_t *>(smem + buf * kStageBytes + kABytes);
-#pragma unroll
-    for (int w = 0; w < NW; ++w)
-      words[w] = sb[t * BN + (wn * NW + w) * 64 + lane];
+  const int frag0 = (wn * NF) % (kWideGroup / 32); // index of this wavefront's first column fragment in its group
+  auto read_words = [&](int buf, int t, uint4_t &words) {
+    const uint4_t *sb = reinterpret_cast<const uint4_t *>(smem + buf * kStageBytes + kABytes);
+    words = sb[(t * (BN / kWideGroup) + (wn * NF) / (kWideGroup / 32)) * 64 + lane];
   };
-  // Bits -> bytes in {0, 1}: register i of column half f is (word >> (4 f + i)) & 0x01010101.
-  uint32_t byte_ones = 0x01010101u;
-  asm volatile("" : "+s"(byte_ones));
-  auto mma = [&](const uint4_t (&af)[MF][kDigits], const uint32_t (&words)[NW]) {
+  // Bits -> bytes in {0, 2^F}: register i of column fragment F is word_i & (0x01010101 << F).
+  uint32_t frag_mask[NF];
+#pragma unroll
+  for (int j = 0; j < NF; ++j) {
+    frag_mask[j] = 0x01010101u << (frag0 + j);
+    asm volatile("" : "+s"(frag_mask[j]));
+  }
+  auto mma = [&](const uint4_t (&af)[MF][kDigits], const uint4_t &words) {
 #pragma unroll
     for (int j = 0; j < NF; ++j) {
-      const uint32_t w = words[j >> 1];
-      const int base = 4 * (j & 1);
       uint4_t bf;
-      bf.x = (w >> (base + 0)) & byte_ones;
-      bf.y = (w >> (base + 1)) & byte_ones;
-      bf.z = (w >> (base + 2)) & byte_ones;
-      bf.w = (w >> (base + 3)) & byte_ones;
+      bf.x = words.x & frag_mask[j];
+      bf.y = words.y & frag_mask[j];
+      bf.z = words.z & frag_mask[j];
+      bf.w = words.w & frag_mask[j];
 #pragma unroll
       for (int d = 0; d < kDigits; ++d)
 #pragma unroll
@@ -217,17 +239,14 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64) void gemm_bits_kernel(GemmBi
   // expansion, fragment fetch and copy issue of the next k tile fit between consecutive MFMAs instead of in front
   // of them.
   constexpr int kMfma = kDigits * MF * NF;
-  constexpr int kValuPer = (NF * 8 + 8 + kMfma - 1) / kMfma + 1;
+  constexpr int kValuPer = (NF * 4 + 8 + kMfma - 1) / kMfma + 1;
   auto interleave = [&](bool with_copies) {
-#ifdef NBLA_NO_HINTS
-    return;
-#endif
 #pragma unroll
     for (int g = 0; g < kMfma; ++g) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
-      if (with_copies && g < kLoadsPerStage)
+      if (with_copies && g < kSlots)
         __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // VMEM read
-      if (g < MF * kDigits + NW)
+      if (g < MF * kDigits + 1)
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
       __builtin_amdgcn_sched_group_barrier(0x002, kValuPer, 0); // VALU
     }
@@ -237,74 +256,115 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64) void gemm_bits_kernel(GemmBi
   // iterations copy the final step again instead of skipping).  While the MFMA block of one k tile runs, the
   // fragments of the next one are fetched from LDS.
   uint4_t af0[MF][kDigits], af1[MF][kDigits];
-  uint32_t w0[NW], w1[NW];
+  uint4_t w0, w1;
   const int64_t first = a.step_begin, last = a.step_end - 1;
 #pragma unroll
   for (int d = 0; d < kDepth; ++d)
     copy_step(first + d < last ? first + d : last, d);
-  NBLA_WAIT_VMCNT((kDepth - 1) * kLoadsPerStage);
+  wait_copies(std::integral_constant<int, kDepth - 1>());
   __syncthreads();
   read_words(0, 0, w0);
   read_a(0, 0, af0);
+  // A wavefront whose columns all lie past the end of the operand (last tile of a row of tiles) only takes part in
+  // the copies and barriers: the matrix pipe of its SIMD is left to the other wavefront.
+  const bool idle = a.n_begin + bn * BN + wn * NF * 32 >= a.n_end;
   int buf = 0; // LDS buffer of step ks
-  for (int64_t ks = first; ks <= last; ++ks) {
-    const int buf_next = (buf + 1 == kStages) ? 0 : buf + 1;
-    const int buf_copy = (buf == 0) ? kStages - 1 : buf - 1; // the buffer step ks-1 occupied = that of step ks+kDepth
-    // tile 0 runs; tile 1 is fetched
-    read_a(buf, 1, af1);
-    read_words(buf, 1, w1);
-    mma(af0, w0);
-    interleave(false);
-    // step ks+1 has landed (the copies of later steps may still be in flight); every wavefront is done with the
-    // buffer of step ks-1
-    NBLA_WAIT_VMCNT((kDepth - 1) * kLoadsPerStage);
-    __syncthreads();
-    // tile 1 runs; the copy of step ks+kDepth is issued; tile 0 of step ks+1 is fetched
-    copy_step(ks + kDepth < last ? ks + kDepth : last, buf_copy);
-    read_words(buf_next, 0, w0);
-    read_a(buf_next, 0, af0);
-    mma(af1, w1);
-    interleave(true);
-    buf = buf_next;
+  if (idle) {
+    for (int64_t ks = first; ks <= last; ++ks) {
+      const int buf_copy = (buf == 0) ? kStages - 1 : buf - 1;
+      wait_copies(std::integral_constant<int, kDepth - 1>());
+      __syncthreads();
+      copy_step(ks + kDepth < last ? ks + kDepth : last, buf_copy);
+      buf = (buf + 1 == kStages) ? 0 : buf + 1;
+    }
+  } else {
+    for (int64_t ks = first; ks <= last; ++ks) {
+      const int buf_next = (buf + 1 == kStages) ? 0 : buf + 1;
+      const int buf_copy = (buf == 0) ? kStages - 1 : buf - 1; // the buffer step ks-1 occupied = that of step ks+kDepth
+      // tile 0 runs; tile 1 is fetched
+      read_a(buf, 1, af1);
+      read_words(buf, 1, w1);
+      mma(af0, w0);
+      interleave(false);
+      // step ks+1 has landed (the copies of later steps may still be in flight); every wavefront is done with the
+      // buffer of step ks-1
+      wait_copies(std::integral_constant<int, kDepth - 1>());
+      __syncthreads();
+      // tile 1 runs; the copy of step ks+kDepth is issued; tile 0 of step ks+1 is fetched
+      copy_step(ks + kDepth < last ? ks + kDepth : last, buf_copy);
+      read_words(buf_next, 0, w0);
+      read_a(buf_next, 0, af0);
+      mma(af1, w1);
+      interleave(true);
+      buf = buf_next;
+    }
   }
   NBLA_WAIT_VMCNT(0);
 
   // Epilogue.  Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
   // column l%32 of the 32x32 fragment; rows are m and columns n, or the reverse
   // under kSwap.
+  // Everything an output element needs besides its accumulators (row sums and shift, alpha, bias) is loaded into
+  // registers before the stores of the group it belongs to: the compiler cannot move a load across a store to y.
   const int col_in_frag = lane & 31, row_half = lane >> 5;
-  auto emit = [&](int64_t m, int64_t n, float v, float al, float bi) {
-    const int64_t off = (a.inner == 1) ? m * a.outer_stride : (m / a.inner) * a.outer_stride + (m % a.inner);
-    float *dst = a.y + off + n * a.n_stride;
+  const bool use_alpha = a.finish && a.alpha, use_bias = a.finish && a.bias;
+  // start of output row m (32-bit division: M and inner are below 2^31)
+  auto row_ptr = [&](int64_t m) {
+    const uint32_t mu = (uint32_t)m, in = (uint32_t)a.inner;
+    const int64_t off = (in == 1u) ? m * a.outer_stride : (int64_t)(mu / in) * a.outer_stride + (mu % in);
+    return a.y + off;
+  };
+  auto finish = [&](float v, float prev, float al, float bi) {
     if (a.accumulate)
-      v = *dst + v;
-    if (a.finish) {
-      if (a.alpha)
-        v = v * al;
-      if (a.bias)
-        v = v + bi;
-    }
-    *dst = v;
+      v = prev + v;
+    if (use_alpha)
+      v = v * al;
+    if (use_bias)
+      v = v + bi;
+    return v;
   };
   if (!kSwap) {
+    const int64_t ncol0 = a.n_begin + bn * BN + wn * NF * 32 + col_in_frag;
+    float al[NF], bi[NF];
+#pragma unroll
+    for (int j = 0; j < NF; ++j) {
+      const int64_t n = (ncol0 + 32 * j < a.N) ? ncol0 + 32 * j : a.N - 1;
+      al[j] = use_alpha ? a.alpha[n] : 1.0f;
+      bi[j] = use_bias ? a.bias[n] : 0.0f;
+    }
 #pragma unroll
     for (int i = 0; i < MF; ++i) {
-      const int64_t m0 = bm * BM + (wm * MF + i) * 32;
+      const int64_t m0 = bm * BM + (wm * MF + i) * 32 + 4 * row_half;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int64_t m = m0 + 8 * (r >> 2) + 4 * row_half + (r & 3);
-        if (m >= a.M)
-          continue;
-        const int s_hi = a.sum_hi[m], s_lo = a.sum_lo[m], sh = a.shift[m];
+      for (int rq = 0; rq < 4; ++rq) {
+        // rows m0 + 8 rq + 0..3 (the metadata arrays are padded to whole row blocks)
+        const int64_t mq = m0 + 8 * rq;
+        const int64_t ml = (mq < a.row_blocks * kFragRows) ? mq : 0; // row blocks past the operand are not stored
+        const i32x4_t s_hi = *reinterpret_cast<const i32x4_t *>(a.sum_hi + ml);
+        const i32x4_t s_lo = *reinterpret_cast<const i32x4_t *>(a.sum_lo + ml);
+        const i32x4_t sh = *reinterpret_cast<const i32x4_t *>(a.shift + ml);
 #pragma unroll
-        for (int j = 0; j < NF; ++j) {
-          const int64_t n = a.n_begin + bn * BN + (wn * NF + j) * 32 + col_in_frag;
-          if (n >= a.n_end)
+        for (int e = 0; e < 4; ++e) {
+          const int r = 4 * rq + e;
+          if (mq + e >= a.M)
             continue;
-          float v = finish_dot(acc[0][i][j][r], acc[1][i][j][r], acc[2][i][j][r], s_hi, s_lo, sh);
-          if (sh == kBadRow)
-            v = __builtin_nanf("");
-          emit(m, n, v, a.alpha ? a.alpha[n] : 1.0f, a.bias ? a.bias[n] : 0.0f);
+          float *row = row_ptr(mq + e) + ncol0 * a.n_stride;
+          float prev[NF];
+          if (a.accumulate) {
+#pragma unroll
+            for (int j = 0; j < NF; ++j)
+              prev[j] = (ncol0 + 32 * j < a.n_end) ? row[32 * j * a.n_stride] : 0.0f;
+          }
+#pragma unroll
+          for (int j = 0; j < NF; ++j) {
+            float v = finish_dot(acc[0][i][j][r], acc[1][i][j][r], acc[2][i][j][r], s_hi[e], s_lo[e], sh[e],
+                                 frag0 + j);
+            if (sh[e] == kBadRow)
+              v = __builtin_nanf("");
+            v = finish(v, prev[j], al[j], bi[j]);
+            if (ncol0 + 32 * j < a.n_end)
+              __builtin_nontemporal_store(v, row + 32 * j * a.n_stride);
+          }
         }
       }
     }
@@ -315,18 +375,35 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64) void gemm_bits_kernel(GemmBi
       if (m >= a.M)
         continue;
       const int s_hi = a.sum_hi[m], s_lo = a.sum_lo[m], sh = a.shift[m];
+      float *row = row_ptr(m);
 #pragma unroll
       for (int j = 0; j < NF; ++j) {
-        const int64_t n0 = a.n_begin + bn * BN + (wn * NF + j) * 32;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int64_t n = n0 + 8 * (r >> 2) + 4 * row_half + (r & 3);
-          if (n >= a.n_end)
-            continue;
-          float v = finish_dot(acc[0][i][j][r], acc[1][i][j][r], acc[2][i][j][r], s_hi, s_lo, sh);
-          if (sh == kBadRow)
-            v = __builtin_nanf("");
-          emit(m, n, v, a.alpha ? a.alpha[n] : 1.0f, a.bias ? a.bias[n] : 0.0f);
+        for (int rq = 0; rq < 4; ++rq) {
+          const int64_t n0 = a.n_begin + bn * BN + (wn * NF + j) * 32 + 4 * row_half + 8 * rq;
+          float al[4], bi[4], prev[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int64_t n = (n0 + e < a.N) ? n0 + e : a.N - 1;
+            al[e] = use_alpha ? a.alpha[n] : 1.0f;
+            bi[e] = use_bias ? a.bias[n] : 0.0f;
+          }
+          float *p = row + n0 * a.n_stride;
+          if (a.accumulate) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              prev[e] = (n0 + e < a.n_end) ? p[e * a.n_stride] : 0.0f;
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int r = 4 * rq + e;
+            float v = finish_dot(acc[0][i][j][r], acc[1][i][j][r], acc[2][i][j][r], s_hi, s_lo, sh, frag0 + j);
+            if (sh == kBadRow)
+              v = __builtin_nanf("");
+            v = finish(v, prev[e], al[e], bi[e]);
+            if (n0 + e < a.n_end)
+              __builtin_nontemporal_store(v, p + e * a.n_stride);
+          }
         }
       }
     }
@@ -355,14 +432,17 @@ int launch_tile(const GemmBitsArgs &args, hipStream_t stream) {
   return NBLA_HIP_OK;
 }
 
-// Tile choice by M: four wavefronts of 64x128 (one per SIMD, the accumulators take most of the register file) on a
-// 128x256 tile once there are enough row blocks to fill the 256 CUs; smaller tiles keep more blocks in flight
-// below that.
+// Tile choice.  A wavefront owns 32x128 outputs (its three accumulator sets take 192 registers), so eight
+// wavefronts fill a CU.  Blocks of four wavefronts (one per SIMD), two blocks per CU, measured best: the barrier
+// couples only four wavefronts and one block's prologue / epilogue overlaps the other's main loop.  The packed
+// operand costs 1/24 of the digit operand's bytes per element, so the block tile is one row block high and wide
+// (32x512) to keep the global -> LDS traffic lowest; narrow outputs take 32x256 blocks of two wavefronts.
 template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream) {
-  if (a.M > 1024)
-    return launch_tile<128, 256, 4, 2, kSwap>(a, stream);
-  if (a.M > 32)
-    return launch_tile<64, 256, 2, 2, kSwap>(a, stream);
+#if defined(NBLA_DBG_TILE)
+  return launch_tile<NBLA_DBG_TILE, kSwap>(a, stream);
+#endif
+  if (a.N > 256 && a.M > 128)
+    return launch_tile<32, 512, 1, 4, kSwap>(a, stream);
   return launch_tile<32, 256, 1, 2, kSwap>(a, stream);
 }
 
@@ -371,7 +451,7 @@ template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream) {
 int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alpha, const float *bias, float *y,
                      int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
                      bool swap_out, hipStream_t stream) {
-  if (M <= 0 || K <= 0 || N <= 0 || inner <= 0)
+  if (M <= 0 || K <= 0 || N <= 0 || inner <= 0 || M > 0x7fffffffll || inner > 0x7fffffffll)
     return fail(NBLA_HIP_ERR_VALUE, "invalid GEMM shape (M=%lld, K=%lld, N=%lld).", (long long)M, (long long)K,
                 (long long)N);
   if (!aligned16(xdigits) || !aligned16(bits))
@@ -395,7 +475,7 @@ int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alp
   a.row_blocks = d.row_blocks;
   a.x_k_tiles = d.k_tiles;
   a.b_k_tiles = bits_k_tiles(K);
-  a.col_groups = bits_col_groups(N);
+  a.wide_groups = bits_wide_groups(N);
   a.blocks_m = a.blocks_n = 0;
   a.inner = inner;
   a.outer_stride = outer_stride;

@@ -27,14 +27,21 @@
 // row_blocks * 32 entries per chunk), and by the shifts s_m (one int32 array; kBadRow marks a row holding a
 // non-finite value).  Rows >= M and columns >= K are zero.  The number of k tiles is padded to an even count.
 //
-// B ("packed bits"): one bit per weight, set = negative (-1), clear = +1:
-//     B'[k_tile = k / 32][col_group = n / 64][lane] : one uint32 word
-// Lane l's word serves column n = col_group * 64 + f * 32 + (l % 32) for f = 0, 1 and k-slots (l / 32) * 16 + j,
-// j = 0..15.  The bit of (f, j) sits at position 4 f + j / 4 + 8 (j % 4), so that
-//     (word >> (4 f + i)) & 0x01010101
-// is directly register i of the i8 fragment of column half f holding b = 1 for a negative weight and 0 otherwise
-// (bytes j = 4 i .. 4 i + 3).  With b in {0, 1} the signed product is  sum q * (1 - 2 b) = rowsum(q) - 2 sum q b.
+// B ("packed bits"): one bit per weight, set = negative (-1), clear = +1, in groups of 256 columns (eight column
+// fragments F = 0..7 of 32 columns):
+//     B'[k_tile = k / 32][wide_group = n / 256][lane][4 x uint32]
+// Word i (0..3) of lane l serves column n = wide_group * 256 + F * 32 + (l % 32) and k-slots (l / 32) * 16 + 4 i + c,
+// c = 0..3; the bit of (F, c) sits at position F + 8 c, so that
+//     word_i & (0x01010101 << F)
+// is directly register i of the i8 fragment of column fragment F, holding 2^F (as int8: -128 for F = 7) for a
+// negative weight and 0 otherwise: the accumulators of fragment F come out scaled by that constant, which the
+// epilogue divides out exactly.  With b in {0, 1} the signed product is  sum q * (1 - 2 b) = rowsum(q) - 2 sum q b.
 // Bits outside [K, N] are clear.
+//
+// The kernels that binarise weights first emit "pair words" (an intermediate kept in their workspace):
+//     P[k_tile][pair_group = n / 64][lane] : one uint32, bit 4 f + j / 4 + 8 (j % 4) for column half f = 0, 1 and
+//     k-slot offset j = 0..15 of the lane
+// and a small relayout pass interleaves four pair groups into one wide group.
 #pragma once
 #include <stdint.h>
 
@@ -43,7 +50,7 @@ namespace nbla_hip {
 constexpr int kFragRows = 32;   // rows per MFMA fragment
 constexpr int kFragK = 16;      // k per MFMA fragment
 constexpr int kTileK = 32;      // k per kernel step (two fragments)
-constexpr int kColGroup = 64;   // columns per packed word group
+constexpr int kColGroup = 64;   // columns per pair-word group
 constexpr int kFragBytes = 1024;
 
 __host__ __device__ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -53,8 +60,11 @@ __host__ __device__ inline int64_t split_k_blocks(int64_t K) { return ceil_div(K
 __host__ __device__ inline int64_t bits_k_tiles(int64_t K) { return ceil_div(K, kTileK); }
 __host__ __device__ inline int64_t bits_col_groups(int64_t N) { return ceil_div(N, kColGroup); }
 
-// Bit position inside a packed word for column half f and k-slot offset j (0..15) of the lane.
+// Bit position inside a pair word for column half f and k-slot offset j (0..15) of the lane.
 __host__ __device__ inline int packed_bit_position(int f, int j) { return 4 * f + (j >> 2) + 8 * (j & 3); }
+
+constexpr int kWideGroup = 256; // columns per group of the packed operand
+__host__ __device__ inline int64_t bits_wide_groups(int64_t N) { return ceil_div(N, kWideGroup); }
 
 // ---- digit operand geometry
 constexpr int kDigits = 3;

@@ -56,7 +56,7 @@ def test_size_queries():
     L = kernels.lib()
     i64 = ctypes.c_int64
     assert L.nbla_hip_packed_bits_bytes(i64(4096), i64(11008)) == 4096 * 11008 // 8
-    assert L.nbla_hip_packed_bits_bytes(i64(33), i64(65)) == 2 * 2 * 64 * 4           # padded to 64 x 128
+    assert L.nbla_hip_packed_bits_bytes(i64(33), i64(65)) == 2 * 1 * 64 * 16          # padded to 64 x 256
     assert L.nbla_hip_split_operand_bytes(i64(4096), i64(4096)) == 4096 * 4096 * 6
     assert L.nbla_hip_split_operand_bytes(i64(1), i64(1)) == 32 * 32 * 6
     # int8 digit operand: 3 bytes per element (K padded to 64), then per row two int32 sums per 16384-column chunk

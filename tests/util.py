@@ -38,21 +38,20 @@ def to_np(t):
 
 
 def unpack_bits(bits_words, K, N):
-    """Packed 1-bit GEMM operand (uint32 words, [k_tiles][col_groups][64]) -> int8 [K, N] of +-1."""
+    """Packed 1-bit GEMM operand (uint32 words, [k_tiles][wide_groups][64 lanes][4]) -> int8 [K, N] of +-1.
+    Word i of lane l: bit F + 8 c is column wide_group * 256 + F * 32 + l % 32, k = k_tile * 32 + (l / 32) * 16 + 4 i + c."""
     w = np.ascontiguousarray(bits_words).view(np.uint32)
     k_tiles = (K + 31) // 32
-    col_groups = (N + 63) // 64
-    w = w.reshape(k_tiles, col_groups, 64)
-    out = np.ones((k_tiles * 32, col_groups * 64), np.int8)
-    lane = np.arange(64)
-    for f in range(2):
-        for j in range(16):
-            pos = 4 * f + (j >> 2) + 8 * (j & 3)
-            bit = (w >> np.uint32(pos)) & np.uint32(1)  # [kt, cg, lane]
-            k_off = (lane >> 5) * 16 + j                # per lane
-            n_off = f * 32 + (lane & 31)
-            for l in range(64):
-                out[k_off[l]::32, n_off[l]::64][:k_tiles, :col_groups] = np.where(bit[:, :, l] == 1, -1, 1)
+    groups = (N + 255) // 256
+    w = w.reshape(k_tiles, groups, 64, 4)
+    out = np.ones((k_tiles * 32, groups * 256), np.int8)
+    for lane in range(64):
+        for i in range(4):
+            for c in range(4):
+                k_off = (lane >> 5) * 16 + 4 * i + c
+                for F in range(8):
+                    bit = (w[:, :, lane, i] >> np.uint32(F + 8 * c)) & np.uint32(1)   # [kt, group]
+                    out[k_off::32, (F * 32 + (lane & 31))::256] = np.where(bit == 1, -1, 1)
     return out[:K, :N]
 
 
