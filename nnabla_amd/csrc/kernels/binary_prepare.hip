@@ -301,7 +301,8 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_finalize(const float *__r
 
 // Pair words -> packed operand: thread (k tile, wide group, lane) interleaves the four pair groups of its wide group.
 __global__ __launch_bounds__(kPrepBlock) void widen_bits(const uint32_t *__restrict__ pairs, uint4_t *__restrict__ bits,
-                                                         int64_t col_groups, int64_t wide_groups, int64_t total) {
+                                                         int64_t k_tiles, int64_t col_groups, int64_t wide_groups,
+                                                         int64_t total) {
   const int64_t idx = (int64_t)blockIdx.x * kPrepBlock + threadIdx.x;
   if (idx >= total)
     return;
@@ -311,7 +312,7 @@ __global__ __launch_bounds__(kPrepBlock) void widen_bits(const uint32_t *__restr
   uint32_t w[4];
 #pragma unroll
   for (int q = 0; q < 4; ++q)
-    w[q] = (4 * wg + q < col_groups) ? pairs[(kt * col_groups + 4 * wg + q) * 64 + lane] : 0u;
+    w[q] = (kt < k_tiles && 4 * wg + q < col_groups) ? pairs[(kt * col_groups + 4 * wg + q) * 64 + lane] : 0u;
   uint32_t o[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -607,7 +608,7 @@ using namespace nbla_hip;
 extern "C" {
 
 size_t nbla_hip_packed_bits_bytes(int64_t K, int64_t N) {
-  return (size_t)bits_k_tiles(K) * bits_wide_groups(N) * 64 * 4 * sizeof(uint32_t);
+  return (size_t)bits_packed_k_tiles(K) * bits_wide_groups(N) * 64 * 4 * sizeof(uint32_t);
 }
 
 size_t nbla_hip_split_operand_bytes(int64_t M, int64_t K) {
@@ -658,9 +659,9 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint3
   }
   NBLA_HIP_LAUNCH_CHECK("binarize_weights");
   {
-    const int64_t wide_groups = bits_wide_groups(N), total = P.k_tiles * wide_groups * 64;
+    const int64_t wide_groups = bits_wide_groups(N), total = bits_packed_k_tiles(K) * wide_groups * 64;
     hipLaunchKernelGGL(widen_bits, dim3((unsigned)ceil_div(total, kPrepBlock)), dim3(kPrepBlock), 0, stream, pairs,
-                       reinterpret_cast<uint4_t *>(bits), P.col_groups, wide_groups, total);
+                       reinterpret_cast<uint4_t *>(bits), P.k_tiles, P.col_groups, wide_groups, total);
     NBLA_HIP_LAUNCH_CHECK("widen_bits");
   }
   if (alpha || zero_count) {

@@ -41,7 +41,6 @@ struct GemmBitsArgs {
   int64_t n_begin, n_end; // column range this launch produces (n_begin a multiple of 256)
   int64_t row_blocks;     // of the digit operand
   int64_t x_k_tiles;      // k tiles of the digit operand (even)
-  int64_t b_k_tiles;      // k tiles of the packed operand
   int64_t wide_groups;    // 256-column groups of the packed operand
   int64_t step_begin, step_end; // k steps (of two k tiles) this launch covers
   int64_t blocks_m, blocks_n;
@@ -62,10 +61,14 @@ __device__ __forceinline__ int64_t xcd_remap(int64_t b, int64_t total) {
   return start + slot;
 }
 
-// LDS buffers (k steps resident) per tile shape: as many as 160 KiB allow, at most four.
-constexpr int gemm_bits_stages(int BM, int BN) {
+// LDS buffers (k steps resident) per tile shape: what fits the block's share of the CU's 160 KiB, at most six.
+constexpr int gemm_bits_stages(int BM, int BN, int waves) {
   const int stage = (BM / 32) * 2 * kDigits * kFragBytes + 2 * BN * 4;
-  return 4 * stage <= 140 * 1024 ? 4 : 3;
+  const int budget = (waves >= 8 ? 144 : 72) * 1024; // two blocks per CU below eight wavefronts
+#ifdef NBLA_DBG_STAGES
+  return NBLA_DBG_STAGES;
+#endif
+  return budget / stage >= 6 ? 6 : (budget / stage >= 3 ? budget / stage : 3);
 }
 
 // sum_k q_k * (+-1) as fp32 from the three digit accumulators and the row sum (hi * 65536 + lo), scaled by 2^-shift.
@@ -83,6 +86,16 @@ __device__ __forceinline__ float finish_dot(int a0, int a1, int a2, int s_hi, in
   const float r = fmaf((float)u, 65536.0f, (float)v);
   return ldexpf(r, -shift);
 }
+
+// Workgroup barrier without the memory fence of __syncthreads(): the fence would wait for every outstanding
+// global -> LDS copy, including those issued for later k steps.  The waits that matter are explicit (wait_copies);
+// the empty asm statements keep the compiler from moving LDS accesses across the barrier.
+#define NBLA_BARRIER()                                                                                                 \
+  do {                                                                                                                 \
+    asm volatile("" ::: "memory");                                                                                     \
+    __builtin_amdgcn_s_barrier();                                                                                      \
+    asm volatile("" ::: "memory");                                                                                     \
+  } while (0)
 
 // vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
 #define NBLA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xf) | (((n) >> 4) << 14) | (0x7 << 4) | (0xf << 8))
@@ -110,7 +123,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
   constexpr int kPerWave = kChunks / kWaves, kExtra = kChunks % kWaves;
   constexpr int kABytes = kAFrags * kFragBytes;
   constexpr int kStageBytes = kABytes + kBChunks * kFragBytes;
-  constexpr int kStages = gemm_bits_stages(BM, BN);
+  constexpr int kStages = gemm_bits_stages(BM, BN, kWaves);
   constexpr int kDepth = kStages - 1; // k steps in flight ahead of the one being multiplied
   static_assert(kDepth >= 1 && (kDepth - 1) * (kPerWave + 1) < 64, "vmcnt is a 6-bit counter");
 
@@ -129,7 +142,6 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
   constexpr int kSlots = kPerWave + (kExtra ? 1 : 0);
   const uint4_t *src[kSlots];
   int64_t src_step[kSlots]; // advance per k step, in uint4
-  int b_tile[kSlots];       // -1 for a digit fragment, else the k tile (0, 1) of the packed words
 #pragma unroll
   for (int p = 0; p < kSlots; ++p) {
     const int c = p * kWaves + wave;
@@ -140,14 +152,14 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
         rb = a.row_blocks - 1;
       src[p] = a.xd + (rb * a.x_k_tiles * kDigits + rem) * 64;
       src_step[p] = kSegFrags * 64;
-      b_tile[p] = -1;
     } else {
+      // packed words: chunk = (k tile of the step, wide group of the tile); the operand holds an even number of k tiles
       const int cb = (c < kChunks) ? c - kAFrags : 0;
-      b_tile[p] = cb / (BN / kWideGroup);
-      int64_t wg = a.n_begin / kWideGroup + bn * (BN / kWideGroup) + (cb - b_tile[p] * (BN / kWideGroup));
+      const int t = cb / (BN / kWideGroup);
+      int64_t wg = a.n_begin / kWideGroup + bn * (BN / kWideGroup) + (cb - t * (BN / kWideGroup));
       if (wg >= a.wide_groups)
         wg = a.wide_groups - 1;
-      src[p] = reinterpret_cast<const uint4_t *>(a.bits) + wg * 64;
+      src[p] = reinterpret_cast<const uint4_t *>(a.bits) + (t * a.wide_groups + wg) * 64;
       src_step[p] = 2 * a.wide_groups * 64;
     }
   }
@@ -159,17 +171,8 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
     for (int p = 0; p < kSlots; ++p) {
       if (p == kPerWave && wave >= kExtra)
         break;
-      // an odd tile count leaves the second tile of the last step without words: any valid words will do, the
-      // digits they meet are zero
-      int64_t adv = ks * src_step[p];
-      if (b_tile[p] >= 0) {
-        int64_t kt = 2 * ks + b_tile[p];
-        if (kt >= a.b_k_tiles)
-          kt = a.b_k_tiles - 1;
-        adv = kt * a.wide_groups * 64;
-      }
-      __builtin_amdgcn_global_load_lds(src[p] + adv + lane, lds_at(buf * kStageBytes + (p * kWaves + wave) * kFragBytes),
-                                       16, 0, 0);
+      __builtin_amdgcn_global_load_lds(src[p] + ks * src_step[p] + lane,
+                                       lds_at(buf * kStageBytes + (p * kWaves + wave) * kFragBytes), 16, 0, 0);
     }
   };
   // waits until at most `steps` k steps of this wavefront's copies are in flight
@@ -213,9 +216,9 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
     frag_mask[j] = 0x01010101u << (frag0 + j);
     asm volatile("" : "+s"(frag_mask[j]));
   }
-  auto mma = [&](const uint4_t (&af)[MF][kDigits], const uint4_t &words) {
+  auto mma = [&](const uint4_t (&af)[MF][kDigits], const uint4_t &words, auto j_begin, auto j_end) {
 #pragma unroll
-    for (int j = 0; j < NF; ++j) {
+    for (int j = decltype(j_begin)::value; j < decltype(j_end)::value; ++j) {
       uint4_t bf;
       bf.x = words.x & frag_mask[j];
       bf.y = words.y & frag_mask[j];
@@ -234,27 +237,13 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
         }
     }
   };
-  // Asks the scheduler to issue the region just written as: one MFMA, then a few VALU / memory instructions in
-  // its shadow, repeated.  A wavefront issues in order and an MFMA occupies the matrix pipe for 32 cycles, so the
-  // expansion, fragment fetch and copy issue of the next k tile fit between consecutive MFMAs instead of in front
-  // of them.
-  constexpr int kMfma = kDigits * MF * NF;
-  constexpr int kValuPer = (NF * 4 + 8 + kMfma - 1) / kMfma + 1;
-  auto interleave = [&](bool with_copies) {
-#pragma unroll
-    for (int g = 0; g < kMfma; ++g) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
-      if (with_copies && g < kSlots)
-        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // VMEM read
-      if (g < MF * kDigits + 1)
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
-      __builtin_amdgcn_sched_group_barrier(0x002, kValuPer, 0); // VALU
-    }
-  };
-
-  // Software pipeline.  One barrier per k step, in the middle of it, no branches in the loop body (the last
-  // iterations copy the final step again instead of skipping).  While the MFMA block of one k tile runs, the
-  // fragments of the next one are fetched from LDS.
+  // Software pipeline.  One barrier per k step, in the middle of it.  A wavefront issues in order and an MFMA keeps
+  // the matrix pipe busy for 32 cycles, so each half step is laid out by hand: the MFMAs of the first column
+  // fragment go first, the LDS reads of the next k tile (and the copies of a later k step) are issued in their
+  // shadow, and the remaining MFMAs cover the latency.  sched_barrier pins that order.
+  typedef std::integral_constant<int, 0> J0;
+  typedef std::integral_constant<int, 1> J1;
+  typedef std::integral_constant<int, NF> JN;
   uint4_t af0[MF][kDigits], af1[MF][kDigits];
   uint4_t w0, w1;
   const int64_t first = a.step_begin, last = a.step_end - 1;
@@ -262,7 +251,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
   for (int d = 0; d < kDepth; ++d)
     copy_step(first + d < last ? first + d : last, d);
   wait_copies(std::integral_constant<int, kDepth - 1>());
-  __syncthreads();
+  NBLA_BARRIER();
   read_words(0, 0, w0);
   read_a(0, 0, af0);
   // A wavefront whose columns all lie past the end of the operand (last tile of a row of tiles) only takes part in
@@ -273,7 +262,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
     for (int64_t ks = first; ks <= last; ++ks) {
       const int buf_copy = (buf == 0) ? kStages - 1 : buf - 1;
       wait_copies(std::integral_constant<int, kDepth - 1>());
-      __syncthreads();
+      NBLA_BARRIER();
       copy_step(ks + kDepth < last ? ks + kDepth : last, buf_copy);
       buf = (buf + 1 == kStages) ? 0 : buf + 1;
     }
@@ -282,20 +271,32 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
       const int buf_next = (buf + 1 == kStages) ? 0 : buf + 1;
       const int buf_copy = (buf == 0) ? kStages - 1 : buf - 1; // the buffer step ks-1 occupied = that of step ks+kDepth
       // tile 0 runs; tile 1 is fetched
+      mma(af0, w0, J0(), J1());
+      __builtin_amdgcn_sched_barrier(0);
       read_a(buf, 1, af1);
       read_words(buf, 1, w1);
-      mma(af0, w0);
-      interleave(false);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(af0, w0, J1(), JN());
+      __builtin_amdgcn_sched_barrier(0);
       // step ks+1 has landed (the copies of later steps may still be in flight); every wavefront is done with the
       // buffer of step ks-1
+#ifndef NBLA_DBG_NOWAIT
       wait_copies(std::integral_constant<int, kDepth - 1>());
-      __syncthreads();
+#endif
+#ifndef NBLA_DBG_NOBAR
+      NBLA_BARRIER();
+#endif
       // tile 1 runs; the copy of step ks+kDepth is issued; tile 0 of step ks+1 is fetched
+      mma(af1, w1, J0(), J1());
+      __builtin_amdgcn_sched_barrier(0);
+#ifndef NBLA_DBG_NOCOPY
       copy_step(ks + kDepth < last ? ks + kDepth : last, buf_copy);
+#endif
       read_words(buf_next, 0, w0);
       read_a(buf_next, 0, af0);
-      mma(af1, w1);
-      interleave(true);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(af1, w1, J1(), JN());
+      __builtin_amdgcn_sched_barrier(0);
       buf = buf_next;
     }
   }
@@ -415,7 +416,7 @@ template <int BM, int BN, int kWavesM, int kWavesN, bool kSwap>
 int launch_tile(const GemmBitsArgs &args, hipStream_t stream) {
   constexpr int kThreads = kWavesM * kWavesN * 64;
   constexpr int kStageBytes = (BM / 32) * 2 * kDigits * kFragBytes + 2 * BN * 4;
-  constexpr int kSmem = gemm_bits_stages(BM, BN) * kStageBytes;
+  constexpr int kSmem = gemm_bits_stages(BM, BN, kWavesM * kWavesN) * kStageBytes;
   auto kernel = gemm_bits_kernel<BM, BN, kWavesM, kWavesN, kSwap>;
   static bool configured = false;
   if (!configured) {
@@ -474,7 +475,6 @@ int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alp
   a.n_end = N;
   a.row_blocks = d.row_blocks;
   a.x_k_tiles = d.k_tiles;
-  a.b_k_tiles = bits_k_tiles(K);
   a.wide_groups = bits_wide_groups(N);
   a.blocks_m = a.blocks_n = 0;
   a.inner = inner;

@@ -36,7 +36,7 @@
 // is directly register i of the i8 fragment of column fragment F, holding 2^F (as int8: -128 for F = 7) for a
 // negative weight and 0 otherwise: the accumulators of fragment F come out scaled by that constant, which the
 // epilogue divides out exactly.  With b in {0, 1} the signed product is  sum q * (1 - 2 b) = rowsum(q) - 2 sum q b.
-// Bits outside [K, N] are clear.
+// Bits outside [K, N] are clear; the number of k tiles is padded to an even count.
 //
 // The kernels that binarise weights first emit "pair words" (an intermediate kept in their workspace):
 //     P[k_tile][pair_group = n / 64][lane] : one uint32, bit 4 f + j / 4 + 8 (j % 4) for column half f = 0, 1 and
@@ -65,6 +65,8 @@ __host__ __device__ inline int packed_bit_position(int f, int j) { return 4 * f 
 
 constexpr int kWideGroup = 256; // columns per group of the packed operand
 __host__ __device__ inline int64_t bits_wide_groups(int64_t N) { return ceil_div(N, kWideGroup); }
+// k tiles of the packed operand: an even count (one kernel k step is two tiles), the padding tile all clear
+__host__ __device__ inline int64_t bits_packed_k_tiles(int64_t K) { return ceil_div(K, 2 * kTileK) * 2; }
 
 // ---- digit operand geometry
 constexpr int kDigits = 3;

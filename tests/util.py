@@ -41,7 +41,7 @@ def unpack_bits(bits_words, K, N):
     """Packed 1-bit GEMM operand (uint32 words, [k_tiles][wide_groups][64 lanes][4]) -> int8 [K, N] of +-1.
     Word i of lane l: bit F + 8 c is column wide_group * 256 + F * 32 + l % 32, k = k_tile * 32 + (l / 32) * 16 + 4 i + c."""
     w = np.ascontiguousarray(bits_words).view(np.uint32)
-    k_tiles = (K + 31) // 32
+    k_tiles = ((K + 63) // 64) * 2          # padded to an even count
     groups = (N + 255) // 256
     w = w.reshape(k_tiles, groups, 64, 4)
     out = np.ones((k_tiles * 32, groups * 256), np.int8)
