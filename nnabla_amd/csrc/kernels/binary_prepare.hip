@@ -269,14 +269,43 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_nk(const float *__restric
     zeros[(int64_t)blockIdx.y * col_groups + cg] = s_zero[0] + s_zero[1] + s_zero[2] + s_zero[3];
 }
 
+// Pair words -> packed operand: thread (k tile, wide group, lane) interleaves the four pair groups of its wide group.
+__device__ __forceinline__ void widen_bits(const uint32_t *__restrict__ pairs, uint4_t *__restrict__ bits,
+                                           int64_t k_tiles, int64_t col_groups, int64_t wide_groups, int64_t idx) {
+  const int lane = (int)(idx & 63);
+  const int64_t t = idx >> 6;
+  const int64_t kt = t / wide_groups, wg = t - kt * wide_groups;
+  uint32_t w[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+    w[q] = (kt < k_tiles && 4 * wg + q < col_groups) ? pairs[(kt * col_groups + 4 * wg + q) * 64 + lane] : 0u;
+  uint32_t o[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int f = 0; f < 2; ++f)
+        o[i] |= ((w[q] >> (4 * f + i)) & 0x01010101u) << (2 * q + f);
+  uint4_t v;
+  v.x = o[0], v.y = o[1], v.z = o[2], v.w = o[3];
+  bits[idx] = v;
+}
+
 // alpha[n] = (sum over slices) * ((float)1 / K)   (binary_weight_affine.cpp:68,
 // binary_weight_convolution.cpp:66: a multiply by the rounded reciprocal), and
-// the total zero count.
+// the total zero count; the same launch turns the pair words into the packed operand (one thread per output uint4).
 __global__ __launch_bounds__(kPrepBlock) void binarize_finalize(const float *__restrict__ sums, const int *__restrict__ zeros,
                                                                 float *__restrict__ alpha, int *__restrict__ zero_count,
                                                                 int64_t N, int64_t Np, int64_t slices,
-                                                                int64_t zero_entries, float inv_k) {
+                                                                int64_t zero_entries, float inv_k,
+                                                                const uint32_t *__restrict__ pairs,
+                                                                uint4_t *__restrict__ bits, int64_t k_tiles,
+                                                                int64_t col_groups, int64_t wide_groups,
+                                                                int64_t widen_total) {
   const int64_t n = (int64_t)blockIdx.x * kPrepBlock + threadIdx.x;
+  if (n < widen_total)
+    widen_bits(pairs, bits, k_tiles, col_groups, wide_groups, n);
   if (alpha && n < N) {
     float acc = 0.0f;
     for (int64_t s = 0; s < slices; ++s)
@@ -297,33 +326,6 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_finalize(const float *__r
     if (threadIdx.x == 0)
       *zero_count = s_z[0] + s_z[1] + s_z[2] + s_z[3];
   }
-}
-
-// Pair words -> packed operand: thread (k tile, wide group, lane) interleaves the four pair groups of its wide group.
-__global__ __launch_bounds__(kPrepBlock) void widen_bits(const uint32_t *__restrict__ pairs, uint4_t *__restrict__ bits,
-                                                         int64_t k_tiles, int64_t col_groups, int64_t wide_groups,
-                                                         int64_t total) {
-  const int64_t idx = (int64_t)blockIdx.x * kPrepBlock + threadIdx.x;
-  if (idx >= total)
-    return;
-  const int lane = (int)(idx & 63);
-  const int64_t t = idx >> 6;
-  const int64_t kt = t / wide_groups, wg = t - kt * wide_groups;
-  uint32_t w[4];
-#pragma unroll
-  for (int q = 0; q < 4; ++q)
-    w[q] = (kt < k_tiles && 4 * wg + q < col_groups) ? pairs[(kt * col_groups + 4 * wg + q) * 64 + lane] : 0u;
-  uint32_t o[4] = {0u, 0u, 0u, 0u};
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-#pragma unroll
-      for (int f = 0; f < 2; ++f)
-        o[i] |= ((w[q] >> (4 * f + i)) & 0x01010101u) << (2 * q + f);
-  uint4_t v;
-  v.x = o[0], v.y = o[1], v.z = o[2], v.w = o[3];
-  bits[idx] = v;
 }
 
 // ------------------------------------------------------------------ bf16 split
@@ -493,7 +495,23 @@ __global__ __launch_bounds__(kPrepBlock) void digit_row_scale(const float *__res
   }
   const float *row = x + m * ldx;
   uint32_t amax = 0u;
-  if (kVec) {
+  // rows of up to 4096 values stay in registers between the two sweeps (16 float4 per lane)
+  constexpr int kKeep = 16;
+  const bool keep = kVec && K <= 256 * kKeep;
+  float4_t kept[kKeep];
+  if (keep) {
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i) {
+      const int64_t k = 4 * lane + 256 * i;
+      kept[i] = (k < K) ? *reinterpret_cast<const float4_t *>(row + k) : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i) {
+      const uint32_t a = __float_as_uint(kept[i].x) & 0x7fffffffu, b = __float_as_uint(kept[i].y) & 0x7fffffffu;
+      const uint32_t c = __float_as_uint(kept[i].z) & 0x7fffffffu, d = __float_as_uint(kept[i].w) & 0x7fffffffu;
+      amax = max(max(amax, max(a, b)), max(c, d));
+    }
+  } else if (kVec) {
     for (int64_t k = 4 * lane; k < K; k += 256) { // K % 4 == 0
       const float4_t v = *reinterpret_cast<const float4_t *>(row + k);
       const uint32_t a = __float_as_uint(v.x) & 0x7fffffffu, b = __float_as_uint(v.y) & 0x7fffffffu;
@@ -515,7 +533,13 @@ __global__ __launch_bounds__(kPrepBlock) void digit_row_scale(const float *__res
     const int64_t k_begin = c * kChunkK, k_end = (k_begin + kChunkK < K) ? k_begin + kChunkK : K;
     long long acc = 0;
     if (!bad) {
-      if (kVec) {
+      if (keep) { // a single chunk
+        int part = 0; // at most 64 values of magnitude < 2^23 per lane
+#pragma unroll
+        for (int i = 0; i < kKeep; ++i)
+          part += to_fixed(kept[i].x, s) + to_fixed(kept[i].y, s) + to_fixed(kept[i].z, s) + to_fixed(kept[i].w, s);
+        acc = part;
+      } else if (kVec) {
         for (int64_t k = k_begin + 4 * lane; k < k_end; k += 256) {
           const float4_t v = *reinterpret_cast<const float4_t *>(row + k);
           acc += (long long)to_fixed(v.x, s) + to_fixed(v.y, s) + to_fixed(v.z, s) + to_fixed(v.w, s);
@@ -660,14 +684,11 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint3
   NBLA_HIP_LAUNCH_CHECK("binarize_weights");
   {
     const int64_t wide_groups = bits_wide_groups(N), total = bits_packed_k_tiles(K) * wide_groups * 64;
-    hipLaunchKernelGGL(widen_bits, dim3((unsigned)ceil_div(total, kPrepBlock)), dim3(kPrepBlock), 0, stream, pairs,
-                       reinterpret_cast<uint4_t *>(bits), P.k_tiles, P.col_groups, wide_groups, total);
-    NBLA_HIP_LAUNCH_CHECK("widen_bits");
-  }
-  if (alpha || zero_count) {
     const float inv_k = (float)1 / K;
-    hipLaunchKernelGGL(binarize_finalize, dim3((unsigned)ceil_div(N, kPrepBlock)), dim3(kPrepBlock), 0, stream, sums,
-                       zeros, alpha, zero_count, N, P.Np, slices, slices * P.col_groups, inv_k);
+    const int64_t threads = total > N ? total : N;
+    hipLaunchKernelGGL(binarize_finalize, dim3((unsigned)ceil_div(threads, kPrepBlock)), dim3(kPrepBlock), 0, stream,
+                       sums, zeros, alpha, zero_count, N, P.Np, slices, slices * P.col_groups, inv_k, pairs,
+                       reinterpret_cast<uint4_t *>(bits), P.k_tiles, P.col_groups, wide_groups, total);
     NBLA_HIP_LAUNCH_CHECK("binarize_finalize");
   }
   return NBLA_HIP_OK;

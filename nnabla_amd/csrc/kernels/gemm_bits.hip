@@ -65,9 +65,6 @@ __device__ __forceinline__ int64_t xcd_remap(int64_t b, int64_t total) {
 constexpr int gemm_bits_stages(int BM, int BN, int waves) {
   const int stage = (BM / 32) * 2 * kDigits * kFragBytes + 2 * BN * 4;
   const int budget = (waves >= 8 ? 144 : 72) * 1024; // two blocks per CU below eight wavefronts
-#ifdef NBLA_DBG_STAGES
-  return NBLA_DBG_STAGES;
-#endif
   return budget / stage >= 6 ? 6 : (budget / stage >= 3 ? budget / stage : 3);
 }
 
@@ -134,8 +131,14 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave % kWavesM, wn = wave / kWavesM;
 
+  // Tiles are walked in bands of kBand block rows, column by column inside a band: the blocks resident on an XCD at
+  // one time then cover about kBand x kBand tiles, so its L2 serves each digit panel and each packed panel to
+  // several blocks instead of streaming the whole packed operand once per block row.
+  constexpr int64_t kBand = 8;
   const int64_t tile = xcd_remap(blockIdx.x, a.blocks_m * a.blocks_n);
-  const int64_t bm = tile / a.blocks_n, bn = tile - bm * a.blocks_n;
+  const int64_t band = tile / (kBand * a.blocks_n), in_band = tile - band * (kBand * a.blocks_n);
+  const int64_t band_rows = (a.blocks_m - band * kBand < kBand) ? a.blocks_m - band * kBand : kBand;
+  const int64_t bn = in_band / band_rows, bm = band * kBand + (in_band - bn * band_rows);
 
   // Sources of this wavefront's copies (uniform bases; the lane adds its own 16 bytes).  Row blocks / wide groups
   // past the end of the operand are clamped: their products land in rows/columns that are not stored.
@@ -280,18 +283,12 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
       __builtin_amdgcn_sched_barrier(0);
       // step ks+1 has landed (the copies of later steps may still be in flight); every wavefront is done with the
       // buffer of step ks-1
-#ifndef NBLA_DBG_NOWAIT
       wait_copies(std::integral_constant<int, kDepth - 1>());
-#endif
-#ifndef NBLA_DBG_NOBAR
       NBLA_BARRIER();
-#endif
       // tile 1 runs; the copy of step ks+kDepth is issued; tile 0 of step ks+1 is fetched
       mma(af1, w1, J0(), J1());
       __builtin_amdgcn_sched_barrier(0);
-#ifndef NBLA_DBG_NOCOPY
       copy_step(ks + kDepth < last ? ks + kDepth : last, buf_copy);
-#endif
       read_words(buf_next, 0, w0);
       read_a(buf_next, 0, af0);
       __builtin_amdgcn_sched_barrier(0);
@@ -439,9 +436,6 @@ int launch_tile(const GemmBitsArgs &args, hipStream_t stream) {
 // operand costs 1/24 of the digit operand's bytes per element, so the block tile is one row block high and wide
 // (32x512) to keep the global -> LDS traffic lowest; narrow outputs take 32x256 blocks of two wavefronts.
 template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream) {
-#if defined(NBLA_DBG_TILE)
-  return launch_tile<NBLA_DBG_TILE, kSwap>(a, stream);
-#endif
   if (a.N > 256 && a.M > 128)
     return launch_tile<32, 512, 1, 4, kSwap>(a, stream);
   return launch_tile<32, 256, 1, 2, kSwap>(a, stream);
