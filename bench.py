@@ -25,6 +25,10 @@ if ROOT not in sys.path:
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix
 PEAK_INT8_MFMA_TOPS = 5000.0    # MI355X dense int8 matrix
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
+# HBM-side bytes of one launch of the dominant kernel at the headline shape, from rocprofv3 FETCH_SIZE / WRITE_SIZE
+# runs of this same command (scaled by what a streaming kernel of known size reads on those counters):
+# 264.0 MB fetched + 180.2 MB written.
+GEMM_TRAFFIC_BYTES_PROFILED = 444.2e6
 
 
 def _events(n):
@@ -186,7 +190,9 @@ def main():
                                "quantize_zero_to=1, no bias; whole forward = sign/alpha/pack + split + MFMA product",
                    "M": M, "K": K, "N": N},
         "roofline": {"bound": "mfma", "achieved": 3 * gemm_tflops, "peak": PEAK_INT8_MFMA_TOPS, "unit": "TOP/s",
-                     "frac": 3 * gemm_tflops / PEAK_INT8_MFMA_TOPS, "traffic": None,
+                     "frac": 3 * gemm_tflops / PEAK_INT8_MFMA_TOPS, "traffic": GEMM_TRAFFIC_BYTES_PROFILED,
+                     "traffic_note": "bytes per launch between L2 and the memory side, profiled (not live); "
+                                     "algorithmic: 56.2 MB read + 180.4 MB written",
                      "kernel": "gemm_bits_kernel<32,512,1,4,false>", "kernel_ms": r["gemm_ms"],
                      "note": "int8 operations issued (3 digit planes x 2*M*K*N) against the int8 MFMA peak",
                      "fp32_equiv_TFLOPs": gemm_tflops, "fp32_equiv_over_fp32_mfma_peak": gemm_tflops / PEAK_FP32_MFMA_TFLOPS},
