@@ -134,6 +134,33 @@ def bench_quantizers(dev, iters):
     return out
 
 
+def bench_other_configs(dev, iters):
+    """Whole-op timings (workspace allocation outside the loop is not possible through the convenience wrappers, so
+    the caching allocator's hit is inside): binary convolutions of the ResNet-18 stage and the INQAffine layer."""
+    import torch
+    from nnabla_amd import kernels as k
+    out = {}
+    g = torch.Generator(device="cpu").manual_seed(7)
+    x = torch.randn(32, 256, 14, 14, generator=g).to(dev)
+    W = (torch.randn(256, 256, 3, 3, generator=g) * (2.0 / 2304) ** 0.5).to(dev)
+    flop = 2.0 * 32 * 14 * 14 * 256 * 2304
+    ms = time_kernel(lambda: k.binary_weight_convolution(x, W, None, (1, 1), (1, 1), (1, 1), 1), iters)
+    out["binary_weight_convolution[32,256,14,14]x[256,256,3,3]"] = {"ms": ms, "TFLOPs": flop / ms / 1e9}
+    ms = time_kernel(lambda: k.binary_connect_convolution(x, W, None, (1, 1), (1, 1), (1, 1), 1), iters)
+    out["binary_connect_convolution[32,256,14,14]x[256,256,3,3]"] = {"ms": ms, "TFLOPs": flop / ms / 1e9}
+    M, K, N = 1024, 4096, 4096
+    xa = torch.randn(M, K, generator=g).to(dev)
+    Wq = (torch.randn(K, N, generator=g) * 0.02).to(dev)
+    I = torch.zeros(K, N, dtype=torch.int32, device=dev)
+    oW, oI = Wq.clone(), I.clone()
+    k.inq_affine(xa, Wq, I, oW, oI, None, 4, k.INQ_FIX_ALL)          # every weight becomes a power of two
+    ms = time_kernel(lambda: k.inq_affine(xa, Wq, I, oW, oI, None, 4, k.INQ_NO_SELECTION), iters)
+    out["inq_affine[1024,4096]x[4096,4096] (restore+quantize+product)"] = {"ms": ms, "TFLOPs": 2.0 * M * K * N / ms / 1e9}
+    ms = time_kernel(lambda: k.inq_affine(xa, Wq, I, oW, oI, None, 4, k.INQ_PRODUCT_ONLY), iters)
+    out["inq_affine[1024,4096]x[4096,4096] (product only)"] = {"ms": ms, "TFLOPs": 2.0 * M * K * N / ms / 1e9}
+    return out
+
+
 def cpu_baseline(K, N, rows):
     """The CPU oracle (port of the reference's CPU arithmetic, single thread) on `rows` rows of the workload."""
     import numpy as np
@@ -181,6 +208,7 @@ def main():
                              "gemm_TFLOPs": s["flop"] / s["gemm_ms"] / 1e9,
                              "gemm_weight_GBs": packed_bytes / s["gemm_ms"] / 1e6}
     quant = bench_quantizers(dev, max(10, args.steps)) if args.section != "headline" else {}
+    other = bench_other_configs(dev, max(5, args.steps // 2)) if args.section == "all" else {}
     line = {
         "metric": "binary-weight affine TFLOP/s + quantizer GB/s, % of MI355X roofline",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -199,6 +227,7 @@ def main():
         "step_breakdown_ms": {"prepare": r["prepare_ms"], "split": r["split_ms"], "gemm": r["gemm_ms"]},
         "sweep": sweep,
         "quantizers": quant,
+        "other_configs": other,
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(K, N, args.cpu_rows)

@@ -479,7 +479,7 @@ __device__ __forceinline__ void store_digits(const int (&q)[16], uint4_t *dst, b
 // values.  The second sweep over the row is served by the caches.
 template <bool kVec>
 __global__ __launch_bounds__(kPrepBlock) void digit_row_scale(const float *__restrict__ x, int64_t ldx,
-                                                              int32_t *__restrict__ sum_hi, int32_t *__restrict__ sum_lo,
+                                                              long long *__restrict__ sums,
                                                               int32_t *__restrict__ shift, int64_t M, int64_t K,
                                                               int64_t rows, int64_t chunks) {
   const int lane = threadIdx.x & 63;
@@ -490,7 +490,7 @@ __global__ __launch_bounds__(kPrepBlock) void digit_row_scale(const float *__res
     if (lane == 0)
       shift[m] = 0;
     for (int64_t c = lane; c < chunks; c += 64)
-      sum_hi[c * rows + m] = 0, sum_lo[c * rows + m] = 0;
+      sums[c * rows + m] = 0;
     return;
   }
   const float *row = x + m * ldx;
@@ -552,10 +552,8 @@ __global__ __launch_bounds__(kPrepBlock) void digit_row_scale(const float *__res
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1)
       acc += __shfl_xor(acc, off);
-    if (lane == 0) {
-      sum_hi[c * rows + m] = (int32_t)(acc >> 16);
-      sum_lo[c * rows + m] = (int32_t)(acc & 0xffff);
-    }
+    if (lane == 0)
+      sums[c * rows + m] = acc;
   }
 }
 
@@ -729,17 +727,16 @@ int nbla_hip_split_digits_f32(const float *x, int64_t ldx, void *xdigits, int64_
   hipStream_t stream = as_stream(stream_);
   const DigitOperand d = digit_operand(M, K);
   char *base = static_cast<char *>(xdigits);
-  int32_t *sum_hi = reinterpret_cast<int32_t *>(base + d.sum_hi_off);
-  int32_t *sum_lo = reinterpret_cast<int32_t *>(base + d.sum_lo_off);
+  long long *sums = reinterpret_cast<long long *>(base + d.sum_off);
   int32_t *shift = reinterpret_cast<int32_t *>(base + d.shift_off);
   const bool vec = K % 4 == 0 && ldx % 4 == 0 && aligned16(x);
   const dim3 scale_grid((unsigned)ceil_div(d.rows, kPrepBlock / 64));
   if (vec)
-    hipLaunchKernelGGL(digit_row_scale<true>, scale_grid, dim3(kPrepBlock), 0, stream, x, ldx, sum_hi, sum_lo, shift, M,
-                       K, d.rows, d.chunks);
+    hipLaunchKernelGGL(digit_row_scale<true>, scale_grid, dim3(kPrepBlock), 0, stream, x, ldx, sums, shift, M, K, d.rows,
+                       d.chunks);
   else
-    hipLaunchKernelGGL(digit_row_scale<false>, scale_grid, dim3(kPrepBlock), 0, stream, x, ldx, sum_hi, sum_lo, shift,
-                       M, K, d.rows, d.chunks);
+    hipLaunchKernelGGL(digit_row_scale<false>, scale_grid, dim3(kPrepBlock), 0, stream, x, ldx, sums, shift, M, K, d.rows,
+                       d.chunks);
   NBLA_HIP_LAUNCH_CHECK("digit_row_scale");
   const int64_t frags = d.row_blocks * d.k_tiles;
   if (K % 64 == 0 && ldx % 4 == 0 && aligned16(x)) {

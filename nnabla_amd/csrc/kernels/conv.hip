@@ -143,75 +143,155 @@ __global__ __launch_bounds__(256) void im2col_split(const float *__restrict__ x,
 // ---- digit operand of the unfolded matrix (the int8 bit-weight product)
 __device__ __forceinline__ int to_fixed(float v, int s) { return (int)rintf(ldexpf(v, s)); }
 
-// One thread per (padded) row of the unfolded matrix: the row's shift and the per-chunk sums of its fixed-point
-// values.  Consecutive threads are consecutive output positions, so each tap is a coalesced read.
-__global__ __launch_bounds__(256) void im2col_row_scale(const float *__restrict__ x, int32_t *__restrict__ sum_hi,
-                                                        int32_t *__restrict__ sum_lo, int32_t *__restrict__ shift,
-                                                        ConvGeom g, int64_t grp, int64_t rows, int64_t chunks) {
+// Largest |x| over the channels of group `grp`, per (sample, input position), as a bit pattern (NaN/Inf show as
+// patterns >= 0x7f800000).  Consecutive threads are consecutive positions: coalesced for every channel.
+__global__ __launch_bounds__(256) void conv_channel_max(const float *__restrict__ x, uint32_t *__restrict__ cmax,
+                                                        ConvGeom g, int64_t grp) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= g.outer * g.in_sp_size)
+    return;
+  const int64_t n = i / g.in_sp_size, p = i - n * g.in_sp_size;
+  const float *src = x + (n * g.C + grp * g.Cg) * g.in_sp_size + p;
+  uint32_t m = 0u;
+  for (int64_t c = 0; c < g.Cg; ++c)
+    m = max(m, __float_as_uint(src[c * g.in_sp_size]) & 0x7fffffffu);
+  cmax[i] = m;
+}
+
+// One thread per (padded) row of the unfolded matrix: the largest magnitude of the row is the largest channel
+// maximum under the kernel window; sets the row's shift and clears its sums.
+__global__ __launch_bounds__(256) void conv_row_shift(const uint32_t *__restrict__ cmax, long long *__restrict__ sums,
+                                                      int32_t *__restrict__ shift, ConvGeom g, int64_t rows,
+                                                      int64_t chunks) {
   const int64_t m = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (m >= rows)
     return;
+  for (int64_t c = 0; c < chunks; ++c)
+    sums[c * rows + m] = 0;
   if (m >= g.M) {
     shift[m] = 0;
-    for (int64_t c = 0; c < chunks; ++c)
-      sum_hi[c * rows + m] = 0, sum_lo[c * rows + m] = 0;
     return;
   }
+  const int64_t n = m / g.out_sp_size;
+  int64_t p = m - n * g.out_sp_size;
+  const int o2 = (int)(p % g.out_sp[2]);
+  p /= g.out_sp[2];
+  const int o1 = (int)(p % g.out_sp[1]);
+  const int o0 = (int)(p / g.out_sp[1]);
   uint32_t amax = 0u;
-  for (int64_t k = 0; k < g.Kg; ++k)
-    amax = max(amax, __float_as_uint(col_value(x, g, grp, m, k)) & 0x7fffffffu);
-  const bool bad = amax >= 0x7f800000u;
+  for (int k0 = 0; k0 < g.k[0]; ++k0) {
+    const int i0 = o0 * g.stride[0] + k0 * g.dil[0] - g.pad[0];
+    if ((unsigned)i0 >= (unsigned)g.in_sp[0])
+      continue;
+    for (int k1 = 0; k1 < g.k[1]; ++k1) {
+      const int i1 = o1 * g.stride[1] + k1 * g.dil[1] - g.pad[1];
+      if ((unsigned)i1 >= (unsigned)g.in_sp[1])
+        continue;
+      for (int k2 = 0; k2 < g.k[2]; ++k2) {
+        const int i2 = o2 * g.stride[2] + k2 * g.dil[2] - g.pad[2];
+        if ((unsigned)i2 >= (unsigned)g.in_sp[2])
+          continue;
+        amax = max(amax, cmax[n * g.in_sp_size + ((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2] + i2]);
+      }
+    }
+  }
   int s = 0;
-  if (!bad && amax != 0u) {
-    const int e = binade_exponent(binade_of(amax));
-    s = 22 - e;
+  if (amax >= 0x7f800000u) {
+    s = kBadRow;
+  } else if (amax != 0u) {
+    s = 22 - binade_exponent(binade_of(amax));
     if (rintf(ldexpf(__uint_as_float(amax), s)) > (float)kDigitMax)
       --s;
   }
-  shift[m] = bad ? kBadRow : s;
-  for (int64_t c = 0; c < chunks; ++c) {
-    const int64_t k_begin = c * kChunkK, k_end = (k_begin + kChunkK < g.Kg) ? k_begin + kChunkK : g.Kg;
-    long long acc = 0;
-    if (!bad)
-      for (int64_t k = k_begin; k < k_end; ++k)
-        acc += to_fixed(col_value(x, g, grp, m, k), s);
-    sum_hi[c * rows + m] = (int32_t)(acc >> 16);
-    sum_lo[c * rows + m] = (int32_t)(acc & 0xffff);
-  }
+  shift[m] = s;
 }
 
-// One wavefront per (row block, k tile) fragment triple of the digit operand.
+// A wavefront converts kTilesPerWave consecutive k tiles of one row block: lane l owns row rb*32 + l%32 and the
+// k-slots (l/32)*16 + 0..15 of each tile.  The column index is decoded to (channel, tap) once per tile and then
+// stepped; the row's partial sum of fixed-point values goes to the row sums with one 64-bit atomic per lane.
+constexpr int kTilesPerWave = 8;
 __global__ __launch_bounds__(256) void im2col_digits(const float *__restrict__ x, const int32_t *__restrict__ shift,
-                                                     uint4_t *__restrict__ out, ConvGeom g, int64_t grp,
-                                                     int64_t k_tiles, int64_t frags) {
-  const int64_t frag = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (frag >= frags)
+                                                     long long *__restrict__ sums, uint4_t *__restrict__ out,
+                                                     ConvGeom g, int64_t grp, int64_t k_tiles, int64_t tile_groups,
+                                                     int64_t rows, int64_t jobs) {
+  const int64_t job = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (job >= jobs)
     return;
   const int lane = threadIdx.x & 63;
-  const int64_t rb = frag / k_tiles, kt = frag - rb * k_tiles;
+  const int64_t rb = job / tile_groups, tg = job - rb * tile_groups;
   const int64_t m = rb * kFragRows + (lane & 31);
-  const int64_t k0 = kt * kTileK + (lane >> 5) * 16;
   const int s = shift[m];
-  uint32_t w[3][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+  const bool row_ok = m < g.M && s != kBadRow;
+  // output position of the row
+  const int64_t n = m / g.out_sp_size;
+  int64_t p = m - n * g.out_sp_size;
+  const int o2 = (int)(p % g.out_sp[2]);
+  p /= g.out_sp[2];
+  const int o1 = (int)(p % g.out_sp[1]);
+  const int o0 = (int)(p / g.out_sp[1]);
+  const int b0 = o0 * g.stride[0] - g.pad[0], b1 = o1 * g.stride[1] - g.pad[1], b2 = o2 * g.stride[2] - g.pad[2];
+  const float *xn = x + (n * g.C + grp * g.Cg) * g.in_sp_size;
+  long long row_sum[2] = {0, 0}; // at most two chunks meet a group of 8 tiles
+  const int64_t kt_begin = tg * kTilesPerWave;
+  for (int t = 0; t < kTilesPerWave; ++t) {
+    const int64_t kt = kt_begin + t;
+    if (kt >= k_tiles)
+      break;
+    const int64_t k0 = kt * kTileK + (lane >> 5) * 16;
+    // decode k0 -> (channel, tap)
+    int64_t q = k0;
+    int k2 = (int)(q % g.k[2]);
+    q /= g.k[2];
+    int k1 = (int)(q % g.k[1]);
+    q /= g.k[1];
+    int kk0 = (int)(q % g.k[0]);
+    int64_t c = q / g.k[0];
+    uint32_t w[3][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+    int part = 0;
 #pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    const int q = (m < g.M && k0 + j < g.Kg && s != kBadRow) ? to_fixed(col_value(x, g, grp, m, k0 + j), s) : 0;
-    const int lo = (int)(int8_t)q;
-    const int q1 = (q - lo) >> 8;
-    const int mid = (int)(int8_t)q1;
-    const int hi = (q1 - mid) >> 8;
-    const int sh = 8 * (j & 3);
-    w[0][j >> 2] |= ((uint32_t)hi & 0xffu) << sh;
-    w[1][j >> 2] |= ((uint32_t)mid & 0xffu) << sh;
-    w[2][j >> 2] |= ((uint32_t)lo & 0xffu) << sh;
-  }
-  uint4_t *dst = out + frag * kDigits * 64 + lane;
+    for (int j = 0; j < 16; ++j) {
+      int qv = 0;
+      if (row_ok && k0 + j < g.Kg) {
+        const int i0 = b0 + kk0 * g.dil[0], i1 = b1 + k1 * g.dil[1], i2 = b2 + k2 * g.dil[2];
+        if ((unsigned)i0 < (unsigned)g.in_sp[0] && (unsigned)i1 < (unsigned)g.in_sp[1] &&
+            (unsigned)i2 < (unsigned)g.in_sp[2])
+          qv = to_fixed(xn[c * g.in_sp_size + ((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2] + i2], s);
+      }
+      part += qv;
+      const int lo = (int)(int8_t)qv;
+      const int q1 = (qv - lo) >> 8;
+      const int mid = (int)(int8_t)q1;
+      const int hi = (q1 - mid) >> 8;
+      const int sh = 8 * (j & 3);
+      w[0][j >> 2] |= ((uint32_t)hi & 0xffu) << sh;
+      w[1][j >> 2] |= ((uint32_t)mid & 0xffu) << sh;
+      w[2][j >> 2] |= ((uint32_t)lo & 0xffu) << sh;
+      // next column: tap index runs fastest, then the channel
+      if (++k2 == g.k[2]) {
+        k2 = 0;
+        if (++k1 == g.k[1]) {
+          k1 = 0;
+          if (++kk0 == g.k[0]) {
+            kk0 = 0;
+            ++c;
+          }
+        }
+      }
+    }
+    row_sum[(kt * kTileK) / kChunkK - (kt_begin * kTileK) / kChunkK] += part;
+    uint4_t *dst = out + ((rb * k_tiles + kt) * kDigits) * 64 + lane;
 #pragma unroll
-  for (int d = 0; d < 3; ++d) {
-    uint4_t o;
-    o.x = w[d][0], o.y = w[d][1], o.z = w[d][2], o.w = w[d][3];
-    dst[d * 64] = o;
+    for (int d = 0; d < 3; ++d) {
+      uint4_t o;
+      o.x = w[d][0], o.y = w[d][1], o.z = w[d][2], o.w = w[d][3];
+      dst[d * 64] = o;
+    }
   }
+  const int64_t chunk0 = (kt_begin * kTileK) / kChunkK;
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+    if (row_sum[h] != 0)
+      atomicAdd(reinterpret_cast<unsigned long long *>(sums + (chunk0 + h) * rows + m), (unsigned long long)row_sum[h]);
 }
 
 // fp32 unfolded matrix [M, Kg] for the general (non bit-representable) path.
@@ -235,17 +315,23 @@ int launch_im2col_split(const float *x, void *xsplit, const ConvGeom &g, int64_t
   return NBLA_HIP_OK;
 }
 
-int launch_im2col_digits(const float *x, void *xdigits, const ConvGeom &g, int64_t grp, hipStream_t stream) {
+// `scratch` holds outer * in_sp_size uint32 (the channel maxima).
+int launch_im2col_digits(const float *x, void *xdigits, void *scratch, const ConvGeom &g, int64_t grp,
+                         hipStream_t stream) {
   const DigitOperand d = digit_operand(g.M, g.Kg);
   char *base = static_cast<char *>(xdigits);
+  long long *sums = reinterpret_cast<long long *>(base + d.sum_off);
   int32_t *shift = reinterpret_cast<int32_t *>(base + d.shift_off);
-  hipLaunchKernelGGL(im2col_row_scale, dim3((unsigned)ceil_div(d.rows, 256)), dim3(256), 0, stream, x,
-                     reinterpret_cast<int32_t *>(base + d.sum_hi_off), reinterpret_cast<int32_t *>(base + d.sum_lo_off),
-                     shift, g, grp, d.rows, d.chunks);
-  NBLA_HIP_LAUNCH_CHECK("im2col_row_scale");
-  const int64_t frags = d.row_blocks * d.k_tiles;
-  hipLaunchKernelGGL(im2col_digits, dim3((unsigned)ceil_div(frags, 4)), dim3(256), 0, stream, x, shift,
-                     reinterpret_cast<uint4_t *>(base), g, grp, d.k_tiles, frags);
+  uint32_t *cmax = static_cast<uint32_t *>(scratch);
+  hipLaunchKernelGGL(conv_channel_max, dim3((unsigned)ceil_div(g.outer * g.in_sp_size, 256)), dim3(256), 0, stream, x,
+                     cmax, g, grp);
+  NBLA_HIP_LAUNCH_CHECK("conv_channel_max");
+  hipLaunchKernelGGL(conv_row_shift, dim3((unsigned)ceil_div(d.rows, 256)), dim3(256), 0, stream, cmax, sums, shift, g,
+                     d.rows, d.chunks);
+  NBLA_HIP_LAUNCH_CHECK("conv_row_shift");
+  const int64_t tile_groups = ceil_div(d.k_tiles, kTilesPerWave), jobs = d.row_blocks * tile_groups;
+  hipLaunchKernelGGL(im2col_digits, dim3((unsigned)ceil_div(jobs, 4)), dim3(256), 0, stream, x, shift, sums,
+                     reinterpret_cast<uint4_t *>(base), g, grp, d.k_tiles, tile_groups, d.rows, jobs);
   NBLA_HIP_LAUNCH_CHECK("im2col_digits");
   return NBLA_HIP_OK;
 }
@@ -262,7 +348,7 @@ int launch_im2col_f32(const float *x, float *col, const ConvGeom &g, int64_t grp
 namespace {
 
 struct ConvWorkspace {
-  size_t bits_off, bits_stride, split_off, prep_off, count_off, col_off, total;
+  size_t bits_off, bits_stride, split_off, cmax_off, prep_off, count_off, col_off, total;
 };
 
 ConvWorkspace plan_conv(const ConvGeom &g) {
@@ -273,6 +359,8 @@ ConvWorkspace plan_conv(const ConvGeom &g) {
   off += w.bits_stride * g.group;
   w.split_off = off;
   off += round_up(nbla_hip_digit_operand_bytes(g.M, g.Kg), 256);
+  w.cmax_off = off;
+  off += round_up((size_t)g.outer * g.in_sp_size * sizeof(uint32_t), 256);
   w.prep_off = off;
   off += round_up(nbla_hip_binarize_workspace_bytes(g.Kg, g.Og), 256);
   w.count_off = off;
@@ -328,7 +416,7 @@ int binary_conv_forward(const float *x, const float *W, float *Wb, float *alpha,
     const float *ag = alpha ? alpha + grp * g.Og : nullptr;
     const float *bg = bias ? bias + grp * g.Og : nullptr;
     if (use_bits) {
-      rc = launch_im2col_digits(x, base + ws.split_off, g, grp, stream);
+      rc = launch_im2col_digits(x, base + ws.split_off, base + ws.cmax_off, g, grp, stream);
       if (rc)
         return rc;
       rc = launch_gemm_bits(base + ws.split_off,

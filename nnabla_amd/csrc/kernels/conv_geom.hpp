@@ -22,7 +22,8 @@ int make_geom(ConvGeom &g, int64_t outer, int64_t C, int nd, const int64_t *in_s
 
 // Unfolded activations of group `grp`, as the bf16x3 split MFMA operand [M, Kg] or as plain fp32 [M, Kg].
 int launch_im2col_split(const float *x, void *xsplit, const ConvGeom &g, int64_t grp, hipStream_t stream);
-int launch_im2col_digits(const float *x, void *xdigits, const ConvGeom &g, int64_t grp, hipStream_t stream);
+int launch_im2col_digits(const float *x, void *xdigits, void *scratch, const ConvGeom &g, int64_t grp,
+                         hipStream_t stream);
 int launch_im2col_f32(const float *x, float *col, const ConvGeom &g, int64_t grp, hipStream_t stream);
 
 } // namespace nbla_hip

@@ -30,8 +30,7 @@ typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
 struct GemmBitsArgs {
   const uint4_t *xd;      // digit fragments
-  const int32_t *sum_hi;  // row sums of this k chunk, high part
-  const int32_t *sum_lo;  // ... low 16 bits
+  const long long *sums;  // row sums of this k chunk
   const int32_t *shift;   // per-row scale exponents
   const uint32_t *bits;   // packed weights
   const float *alpha;     // may be null
@@ -338,9 +337,18 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
         // rows m0 + 8 rq + 0..3 (the metadata arrays are padded to whole row blocks)
         const int64_t mq = m0 + 8 * rq;
         const int64_t ml = (mq < a.row_blocks * kFragRows) ? mq : 0; // row blocks past the operand are not stored
-        const i32x4_t s_hi = *reinterpret_cast<const i32x4_t *>(a.sum_hi + ml);
-        const i32x4_t s_lo = *reinterpret_cast<const i32x4_t *>(a.sum_lo + ml);
+        const i32x4_t sum01 = *reinterpret_cast<const i32x4_t *>(a.sums + ml); // two int64 as (lo, hi) words
+        const i32x4_t sum23 = *reinterpret_cast<const i32x4_t *>(a.sums + ml + 2);
         const i32x4_t sh = *reinterpret_cast<const i32x4_t *>(a.shift + ml);
+        // sum = s_hi * 65536 + s_lo with s_lo in [0, 65536)
+        const uint32_t lo_w[4] = {(uint32_t)sum01.x, (uint32_t)sum01.z, (uint32_t)sum23.x, (uint32_t)sum23.z};
+        const int hi_w[4] = {sum01.y, sum01.w, sum23.y, sum23.w};
+        int s_hi[4], s_lo[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s_hi[e] = (int)((lo_w[e] >> 16) | ((uint32_t)hi_w[e] << 16));
+          s_lo[e] = (int)(lo_w[e] & 0xffffu);
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int r = 4 * rq + e;
@@ -372,7 +380,8 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
       const int64_t m = bm * BM + (wm * MF + i) * 32 + col_in_frag;
       if (m >= a.M)
         continue;
-      const int s_hi = a.sum_hi[m], s_lo = a.sum_lo[m], sh = a.shift[m];
+      const long long sum = a.sums[m];
+      const int s_hi = (int)(sum >> 16), s_lo = (int)(sum & 0xffff), sh = a.shift[m];
       float *row = row_ptr(m);
 #pragma unroll
       for (int j = 0; j < NF; ++j) {
@@ -478,8 +487,7 @@ int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alp
   // partial results of the chunks are added up in y
   const int64_t steps_per_chunk = kChunkK / (2 * kTileK), steps = d.k_tiles / 2;
   for (int64_t c = 0; c < d.chunks; ++c) {
-    a.sum_hi = reinterpret_cast<const int32_t *>(base + d.sum_hi_off) + c * d.rows;
-    a.sum_lo = reinterpret_cast<const int32_t *>(base + d.sum_lo_off) + c * d.rows;
+    a.sums = reinterpret_cast<const long long *>(base + d.sum_off) + c * d.rows;
     a.step_begin = c * steps_per_chunk;
     a.step_end = (a.step_begin + steps_per_chunk < steps) ? a.step_begin + steps_per_chunk : steps;
     a.accumulate = c > 0;

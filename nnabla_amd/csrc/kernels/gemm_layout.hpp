@@ -23,9 +23,8 @@
 // power-of-two scale per row (s_m the largest shift that keeps the row's largest magnitude inside the digit range),
 // and q into three balanced base-256 digits q = d0 * 65536 + d1 * 256 + d2, each an int8:
 //     X'[row_block = m / 32][k_tile = k / 32][digit 0..2][lane][16 x int8]
-// followed, per chunk of kChunkK columns, by the row sums of q split as sum = hi * 65536 + lo (two int32 arrays of
-// row_blocks * 32 entries per chunk), and by the shifts s_m (one int32 array; kBadRow marks a row holding a
-// non-finite value).  Rows >= M and columns >= K are zero.  The number of k tiles is padded to an even count.
+// followed, per chunk of kChunkK columns, by the row sums of q (one int64 array of row_blocks * 32 entries per
+// chunk), and by the shifts s_m (one int32 array; kBadRow marks a row holding a non-finite value).  Rows >= M and columns >= K are zero.  The number of k tiles is padded to an even count.
 //
 // B ("packed bits"): one bit per weight, set = negative (-1), clear = +1, in groups of 256 columns (eight column
 // fragments F = 0..7 of 32 columns):
@@ -79,7 +78,7 @@ __host__ __device__ inline int64_t digit_chunks(int64_t K) { return ceil_div(K, 
 // byte offsets of the sections of a digit operand
 struct DigitOperand {
   int64_t row_blocks, k_tiles, rows, chunks;
-  size_t sum_hi_off, sum_lo_off, shift_off, total;
+  size_t sum_off, shift_off, total;
 };
 __host__ __device__ inline DigitOperand digit_operand(int64_t M, int64_t K) {
   DigitOperand d;
@@ -87,9 +86,8 @@ __host__ __device__ inline DigitOperand digit_operand(int64_t M, int64_t K) {
   d.k_tiles = digit_k_tiles(K);
   d.rows = d.row_blocks * kFragRows;
   d.chunks = digit_chunks(K);
-  d.sum_hi_off = (size_t)d.row_blocks * d.k_tiles * kDigits * kFragBytes;
-  d.sum_lo_off = d.sum_hi_off + (size_t)d.chunks * d.rows * sizeof(int32_t);
-  d.shift_off = d.sum_lo_off + (size_t)d.chunks * d.rows * sizeof(int32_t);
+  d.sum_off = (size_t)d.row_blocks * d.k_tiles * kDigits * kFragBytes;
+  d.shift_off = d.sum_off + (size_t)d.chunks * d.rows * sizeof(int64_t);
   d.total = d.shift_off + (size_t)d.rows * sizeof(int32_t);
   return d;
 }

@@ -2,7 +2,7 @@
 
 Bit-exact: Sign(W) (`Wb`) and the packed 1-bit operand.  At tolerance: alpha (rel 1e-6 against a float64
 mean; the reference's own fp32 summation order comes from Eigen and is unpinned) and y
-(max|y - y_ref| / max|y_ref| <= 1e-4 as the acceptance bar; the bf16x3 product is expected near 1e-6).
+(max|y - y_ref| / max|y_ref| <= 1e-4 as the acceptance bar; the int8-digit product is expected below 1e-6).
 """
 import numpy as np
 import pytest
@@ -162,9 +162,9 @@ def test_binary_connect_affine_matches_oracle(dev, M, K, N):
 
 
 @pytest.mark.parametrize("M,K,N", [(3100, 96, 5732), (3072, 64, 11008)])
-def test_tall_m_column_divided_launch(dev, M, K, N):
-    """M >= 3072 with a tile count that is not a whole number of rounds: the columns are produced by two launches
-    with different tile widths; every output element is checked against float64."""
+def test_tall_m_every_element(dev, M, K, N):
+    """Tall outputs with a ragged last column tile (idle wavefronts, clamped wide groups): every output element is
+    checked against float64."""
     x, W = _data(M, K, N, seed=21)
     b = np.random.RandomState(5).randn(N).astype(np.float32)
     y, Wb, alpha = kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev), _dev(b, dev))

@@ -57,7 +57,7 @@ def unpack_bits(bits_words, K, N):
 
 def unpack_digits(raw, M, K):
     """Digit operand bytes -> (q int64 [M, K], shift int32 [M], row sums int64 [chunks, M]) as the kernels define it:
-    fragments [row_block][k_tile][digit][lane][16 x int8], then sum_hi, sum_lo ([chunks][rows] int32), then shifts."""
+    fragments [row_block][k_tile][digit][lane][16 x int8], then the row sums ([chunks][rows] int64), then shifts."""
     raw = np.ascontiguousarray(raw).view(np.uint8)
     rb, kt = (M + 31) // 32, ((K + 63) // 64) * 2
     rows, chunks = rb * 32, (K + 16383) // 16384
@@ -68,9 +68,7 @@ def unpack_digits(raw, M, K):
     for lane in range(64):
         for j in range(16):
             q[(lane & 31)::32, ((lane >> 5) * 16 + j)::32] = qf[:, :, lane, j]
-    meta = raw[nfrag:].view(np.int32)
-    hi = meta[:chunks * rows].reshape(chunks, rows).astype(np.int64)
-    lo = meta[chunks * rows:2 * chunks * rows].reshape(chunks, rows).astype(np.int64)
-    shift = meta[2 * chunks * rows:2 * chunks * rows + rows]
+    sums = raw[nfrag:nfrag + chunks * rows * 8].view(np.int64).reshape(chunks, rows)
+    shift = raw[nfrag + chunks * rows * 8:nfrag + chunks * rows * 8 + rows * 4].view(np.int32)
     assert not q[M:].any() and not q[:, K:].any()
-    return q[:M, :K], shift[:M].copy(), (hi * 65536 + lo)[:, :M]
+    return q[:M, :K], shift[:M].copy(), sums[:, :M].copy()
