@@ -598,7 +598,7 @@ __global__ __launch_bounds__(kPrepBlock) void split_digits_tiled(const float *__
     const int row = j * 4 + lr;
     const int64_t m = rb * kFragRows + row;
     float4_t v = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (m < M)
+    if (m < M && kq * 64 + lc < K) // the k tiles are padded past K
       v = *reinterpret_cast<const float4_t *>(x + m * ldx + kq * 64 + lc);
     *reinterpret_cast<float4_t *>(t + row * kRowStride + lc) = v;
   }

@@ -143,19 +143,24 @@ __global__ __launch_bounds__(256) void im2col_split(const float *__restrict__ x,
 // ---- digit operand of the unfolded matrix (the int8 bit-weight product)
 __device__ __forceinline__ int to_fixed(float v, int s) { return (int)rintf(ldexpf(v, s)); }
 
-// Largest |x| over the channels of group `grp`, per (sample, input position), as a bit pattern (NaN/Inf show as
-// patterns >= 0x7f800000).  Consecutive threads are consecutive positions: coalesced for every channel.
+// Largest |x| over a slice of the channels of group `grp`, per (sample, input position), as a bit pattern (NaN/Inf
+// show as patterns >= 0x7f800000): cmax[slice][position].  Consecutive threads are consecutive positions (coalesced
+// for every channel); blockIdx.y is the channel slice.
+constexpr int kChannelSlices = 16;
 __global__ __launch_bounds__(256) void conv_channel_max(const float *__restrict__ x, uint32_t *__restrict__ cmax,
                                                         ConvGeom g, int64_t grp) {
+  const int64_t total = g.outer * g.in_sp_size;
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= g.outer * g.in_sp_size)
+  if (i >= total)
     return;
+  const int64_t per = ceil_div(g.Cg, kChannelSlices);
+  const int64_t c_begin = blockIdx.y * per, c_end = (c_begin + per < g.Cg) ? c_begin + per : g.Cg;
   const int64_t n = i / g.in_sp_size, p = i - n * g.in_sp_size;
   const float *src = x + (n * g.C + grp * g.Cg) * g.in_sp_size + p;
   uint32_t m = 0u;
-  for (int64_t c = 0; c < g.Cg; ++c)
+  for (int64_t c = c_begin; c < c_end; ++c)
     m = max(m, __float_as_uint(src[c * g.in_sp_size]) & 0x7fffffffu);
-  cmax[i] = m;
+  cmax[blockIdx.y * total + i] = m;
 }
 
 // One thread per (padded) row of the unfolded matrix: the largest magnitude of the row is the largest channel
@@ -191,7 +196,10 @@ __global__ __launch_bounds__(256) void conv_row_shift(const uint32_t *__restrict
         const int i2 = o2 * g.stride[2] + k2 * g.dil[2] - g.pad[2];
         if ((unsigned)i2 >= (unsigned)g.in_sp[2])
           continue;
-        amax = max(amax, cmax[n * g.in_sp_size + ((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2] + i2]);
+        const int64_t pos = n * g.in_sp_size + ((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2] + i2;
+#pragma unroll
+        for (int sl = 0; sl < kChannelSlices; ++sl)
+          amax = max(amax, cmax[sl * g.outer * g.in_sp_size + pos]);
       }
     }
   }
@@ -209,7 +217,7 @@ __global__ __launch_bounds__(256) void conv_row_shift(const uint32_t *__restrict
 // A wavefront converts kTilesPerWave consecutive k tiles of one row block: lane l owns row rb*32 + l%32 and the
 // k-slots (l/32)*16 + 0..15 of each tile.  The column index is decoded to (channel, tap) once per tile and then
 // stepped; the row's partial sum of fixed-point values goes to the row sums with one 64-bit atomic per lane.
-constexpr int kTilesPerWave = 8;
+constexpr int kTilesPerWave = 2;
 __global__ __launch_bounds__(256) void im2col_digits(const float *__restrict__ x, const int32_t *__restrict__ shift,
                                                      long long *__restrict__ sums, uint4_t *__restrict__ out,
                                                      ConvGeom g, int64_t grp, int64_t k_tiles, int64_t tile_groups,
@@ -231,7 +239,7 @@ __global__ __launch_bounds__(256) void im2col_digits(const float *__restrict__ x
   const int o0 = (int)(p / g.out_sp[1]);
   const int b0 = o0 * g.stride[0] - g.pad[0], b1 = o1 * g.stride[1] - g.pad[1], b2 = o2 * g.stride[2] - g.pad[2];
   const float *xn = x + (n * g.C + grp * g.Cg) * g.in_sp_size;
-  long long row_sum[2] = {0, 0}; // at most two chunks meet a group of 8 tiles
+  long long row_sum[2] = {0, 0}; // at most two chunks meet a group of tiles
   const int64_t kt_begin = tg * kTilesPerWave;
   for (int t = 0; t < kTilesPerWave; ++t) {
     const int64_t kt = kt_begin + t;
@@ -315,7 +323,7 @@ int launch_im2col_split(const float *x, void *xsplit, const ConvGeom &g, int64_t
   return NBLA_HIP_OK;
 }
 
-// `scratch` holds outer * in_sp_size uint32 (the channel maxima).
+// `scratch` holds kChannelSlices * outer * in_sp_size uint32 (the channel maxima).
 int launch_im2col_digits(const float *x, void *xdigits, void *scratch, const ConvGeom &g, int64_t grp,
                          hipStream_t stream) {
   const DigitOperand d = digit_operand(g.M, g.Kg);
@@ -323,8 +331,8 @@ int launch_im2col_digits(const float *x, void *xdigits, void *scratch, const Con
   long long *sums = reinterpret_cast<long long *>(base + d.sum_off);
   int32_t *shift = reinterpret_cast<int32_t *>(base + d.shift_off);
   uint32_t *cmax = static_cast<uint32_t *>(scratch);
-  hipLaunchKernelGGL(conv_channel_max, dim3((unsigned)ceil_div(g.outer * g.in_sp_size, 256)), dim3(256), 0, stream, x,
-                     cmax, g, grp);
+  hipLaunchKernelGGL(conv_channel_max, dim3((unsigned)ceil_div(g.outer * g.in_sp_size, 256), kChannelSlices), dim3(256),
+                     0, stream, x, cmax, g, grp);
   NBLA_HIP_LAUNCH_CHECK("conv_channel_max");
   hipLaunchKernelGGL(conv_row_shift, dim3((unsigned)ceil_div(d.rows, 256)), dim3(256), 0, stream, cmax, sums, shift, g,
                      d.rows, d.chunks);
@@ -360,7 +368,7 @@ ConvWorkspace plan_conv(const ConvGeom &g) {
   w.split_off = off;
   off += round_up(nbla_hip_digit_operand_bytes(g.M, g.Kg), 256);
   w.cmax_off = off;
-  off += round_up((size_t)g.outer * g.in_sp_size * sizeof(uint32_t), 256);
+  off += round_up((size_t)16 * g.outer * g.in_sp_size * sizeof(uint32_t), 256); // kChannelSlices slices
   w.prep_off = off;
   off += round_up(nbla_hip_binarize_workspace_bytes(g.Kg, g.Og), 256);
   w.count_off = off;

@@ -60,11 +60,20 @@ __device__ __forceinline__ int64_t xcd_remap(int64_t b, int64_t total) {
   return start + slot;
 }
 
-// LDS buffers (k steps resident) per tile shape: what fits the block's share of the CU's 160 KiB, at most six.
-constexpr int gemm_bits_stages(int BM, int BN, int waves) {
-  const int stage = (BM / 32) * 2 * kDigits * kFragBytes + 2 * BN * 4;
-  const int budget = (waves >= 8 ? 144 : 72) * 1024; // two blocks per CU below eight wavefronts
+// LDS buffers (stages resident) per tile shape: what fits the block's share of the CU's 160 KiB, at most six.
+constexpr int gemm_bits_stage_bytes(int BM, int BN, int waves_k) {
+  return ((BM / 32) * 2 * kDigits * kFragBytes + 2 * BN * 4) * waves_k;
+}
+constexpr int gemm_bits_stages(int BM, int BN, int waves_mn, int waves_k) {
+  const int stage = gemm_bits_stage_bytes(BM, BN, waves_k);
+  const int budget = (waves_mn * waves_k >= 8 ? 144 : 72) * 1024; // two blocks per CU below eight wavefronts
   return budget / stage >= 6 ? 6 : (budget / stage >= 3 ? budget / stage : 3);
+}
+// LDS bytes of a block: the stages, or the accumulator exchange of the k groups if that is larger
+constexpr int gemm_bits_lds_bytes(int BM, int BN, int waves_m, int waves_n, int waves_k) {
+  const int stages = gemm_bits_stages(BM, BN, waves_m * waves_n, waves_k) * gemm_bits_stage_bytes(BM, BN, waves_k);
+  const int exchange = (waves_k - 1) * (BM / 32) * (BN / 32) * 4096; // one digit: 32x32 int32 per fragment
+  return stages > exchange ? stages : exchange;
 }
 
 // sum_k q_k * (+-1) as fp32 from the three digit accumulators and the row sum (hi * 65536 + lo), scaled by 2^-shift.
@@ -102,10 +111,15 @@ __device__ __forceinline__ float finish_dot(int a0, int a1, int a2, int s_hi, in
 // Staging: global -> LDS copies bypass the registers (global_load_lds): one wavefront instruction moves one 1 KiB
 // digit fragment, or 64 packed words, to the same lane order in LDS.  kStages LDS buffers hold consecutive k steps;
 // the copy of step ks + kStages - 1 is issued while step ks is being multiplied.
-template <int BM, int BN, int kWavesM, int kWavesN, bool kSwap>
-__global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 : 2)) void gemm_bits_kernel(GemmBitsArgs a) {
+//
+// kWavesK > 1 splits the contraction inside the block: wavefront group wk multiplies k steps wk, wk + kWavesK, ...
+// of the same output tile (a stage then holds kWavesK consecutive k steps) and the groups' int32 accumulators are
+// added through LDS at the end, exactly.  Used when the output has too few tiles to occupy the CUs.
+template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, bool kSwap>
+__global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN * kWavesK >= 8 ? 1 : 2)) void gemm_bits_kernel(GemmBitsArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__) // the host pass only needs the launch stub; the body uses LDS address-space pointers
-  constexpr int kWaves = kWavesM * kWavesN;
+  constexpr int kWavesMN = kWavesM * kWavesN;
+  constexpr int kWaves = kWavesMN * kWavesK;
   constexpr int MF = BM / kWavesM / 32;  // X fragments per wavefront (rows)
   constexpr int NF = BN / kWavesN / 32;  // B fragments per wavefront (columns)
   static_assert(BN % kWideGroup == 0 && (kWideGroup / 32) % NF == 0, "a wavefront's fragments share one wide group");
@@ -115,11 +129,13 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
   constexpr int kBChunks = 2 * BN / kWideGroup; // 1 KiB chunks of packed words per k step (2 k tiles x wide groups)
   // One copy instruction moves 1 KiB (a fragment, or the words of one wide group); the kChunks copies of a k step
   // are dealt round-robin, so wavefronts below kExtra issue one more than the others.
-  constexpr int kChunks = kAFrags + kBChunks;
+  constexpr int kStepChunks = kAFrags + kBChunks;
+  constexpr int kChunks = kStepChunks * kWavesK; // a stage holds kWavesK consecutive k steps
   constexpr int kPerWave = kChunks / kWaves, kExtra = kChunks % kWaves;
   constexpr int kABytes = kAFrags * kFragBytes;
-  constexpr int kStageBytes = kABytes + kBChunks * kFragBytes;
-  constexpr int kStages = gemm_bits_stages(BM, BN, kWaves);
+  constexpr int kStepBytes = kStepChunks * kFragBytes;
+  constexpr int kStageBytes = kStepBytes * kWavesK;
+  constexpr int kStages = gemm_bits_stages(BM, BN, kWavesMN, kWavesK);
   constexpr int kDepth = kStages - 1; // k steps in flight ahead of the one being multiplied
   static_assert(kDepth >= 1 && (kDepth - 1) * (kPerWave + 1) < 64, "vmcnt is a 6-bit counter");
 
@@ -128,7 +144,8 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave % kWavesM, wn = wave / kWavesM;
+  const int wk = wave / kWavesMN, wmn = wave - wk * kWavesMN;
+  const int wm = wmn % kWavesM, wn = wmn / kWavesM;
 
   // Tiles are walked in bands of kBand block rows, column by column inside a band: the blocks resident on an XCD at
   // one time then cover about kBand x kBand tiles, so its L2 serves each digit panel and each packed panel to
@@ -146,28 +163,30 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
   int64_t src_step[kSlots]; // advance per k step, in uint4
 #pragma unroll
   for (int p = 0; p < kSlots; ++p) {
-    const int c = p * kWaves + wave;
+    const int cs = p * kWaves + wave;                 // chunk of the stage
+    const int kk = (cs / kStepChunks) % kWavesK;      // k step inside the stage
+    const int c = cs - (cs / kStepChunks) * kStepChunks;
     if (c < kAFrags) {
       const int seg = c / kSegFrags, rem = c - seg * kSegFrags;
       int64_t rb = bm * kASegs + seg;
       if (rb >= a.row_blocks)
         rb = a.row_blocks - 1;
-      src[p] = a.xd + (rb * a.x_k_tiles * kDigits + rem) * 64;
       src_step[p] = kSegFrags * 64;
+      src[p] = a.xd + (rb * a.x_k_tiles * kDigits + rem) * 64 + kk * src_step[p];
     } else {
-      // packed words: chunk = (k tile of the step, wide group of the tile); the operand holds an even number of k tiles
-      const int cb = (c < kChunks) ? c - kAFrags : 0;
+      // packed words: chunk = (k tile of the step, wide group of the tile)
+      const int cb = c - kAFrags;
       const int t = cb / (BN / kWideGroup);
       int64_t wg = a.n_begin / kWideGroup + bn * (BN / kWideGroup) + (cb - t * (BN / kWideGroup));
       if (wg >= a.wide_groups)
         wg = a.wide_groups - 1;
-      src[p] = reinterpret_cast<const uint4_t *>(a.bits) + (t * a.wide_groups + wg) * 64;
       src_step[p] = 2 * a.wide_groups * 64;
+      src[p] = reinterpret_cast<const uint4_t *>(a.bits) + (t * a.wide_groups + wg) * 64 + kk * src_step[p];
     }
   }
   typedef __attribute__((address_space(3))) void lds_void_t;
   auto lds_at = [&](int byte_off) { return (lds_void_t *)(smem + byte_off); };
-  // issues the copies of k step `ks` into LDS buffer `buf`
+  // issues the copies of the stage starting at k step `ks` into LDS buffer `buf`
   auto copy_step = [&](int64_t ks, int buf) {
 #pragma unroll
     for (int p = 0; p < kSlots; ++p) {
@@ -199,7 +218,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
 
   // Fragment fetch and the MFMA block of one k tile (t = 0, 1) of a staged step.
   auto read_a = [&](int buf, int t, uint4_t (&af)[MF][kDigits]) {
-    const uint4_t *sa = reinterpret_cast<const uint4_t *>(smem + buf * kStageBytes);
+    const uint4_t *sa = reinterpret_cast<const uint4_t *>(smem + buf * kStageBytes + wk * kStepBytes);
 #pragma unroll
     for (int i = 0; i < MF; ++i)
 #pragma unroll
@@ -208,7 +227,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
   };
   const int frag0 = (wn * NF) % (kWideGroup / 32); // index of this wavefront's first column fragment in its group
   auto read_words = [&](int buf, int t, uint4_t &words) {
-    const uint4_t *sb = reinterpret_cast<const uint4_t *>(smem + buf * kStageBytes + kABytes);
+    const uint4_t *sb = reinterpret_cast<const uint4_t *>(smem + buf * kStageBytes + wk * kStepBytes + kABytes);
     words = sb[(t * (BN / kWideGroup) + (wn * NF) / (kWideGroup / 32)) * 64 + lane];
   };
   // Bits -> bytes in {0, 2^F}: register i of column fragment F is word_i & (0x01010101 << F).
@@ -248,10 +267,12 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
   typedef std::integral_constant<int, NF> JN;
   uint4_t af0[MF][kDigits], af1[MF][kDigits];
   uint4_t w0, w1;
-  const int64_t first = a.step_begin, last = a.step_end - 1;
+  // stages are numbered by their first k step; the operands are padded so that the number of k steps is a multiple
+  // of kWavesK
+  const int64_t first = a.step_begin, last = a.step_end - kWavesK;
 #pragma unroll
   for (int d = 0; d < kDepth; ++d)
-    copy_step(first + d < last ? first + d : last, d);
+    copy_step(first + d * kWavesK < last ? first + d * kWavesK : last, d);
   wait_copies(std::integral_constant<int, kDepth - 1>());
   NBLA_BARRIER();
   read_words(0, 0, w0);
@@ -261,15 +282,15 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
   const bool idle = a.n_begin + bn * BN + wn * NF * 32 >= a.n_end;
   int buf = 0; // LDS buffer of step ks
   if (idle) {
-    for (int64_t ks = first; ks <= last; ++ks) {
+    for (int64_t ks = first; ks <= last; ks += kWavesK) {
       const int buf_copy = (buf == 0) ? kStages - 1 : buf - 1;
       wait_copies(std::integral_constant<int, kDepth - 1>());
       NBLA_BARRIER();
-      copy_step(ks + kDepth < last ? ks + kDepth : last, buf_copy);
+      copy_step(ks + kDepth * kWavesK < last ? ks + kDepth * kWavesK : last, buf_copy);
       buf = (buf + 1 == kStages) ? 0 : buf + 1;
     }
   } else {
-    for (int64_t ks = first; ks <= last; ++ks) {
+    for (int64_t ks = first; ks <= last; ks += kWavesK) {
       const int buf_next = (buf + 1 == kStages) ? 0 : buf + 1;
       const int buf_copy = (buf == 0) ? kStages - 1 : buf - 1; // the buffer step ks-1 occupied = that of step ks+kDepth
       // tile 0 runs; tile 1 is fetched
@@ -287,7 +308,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
       // tile 1 runs; the copy of step ks+kDepth is issued; tile 0 of step ks+1 is fetched
       mma(af1, w1, J0(), J1());
       __builtin_amdgcn_sched_barrier(0);
-      copy_step(ks + kDepth < last ? ks + kDepth : last, buf_copy);
+      copy_step(ks + kDepth * kWavesK < last ? ks + kDepth * kWavesK : last, buf_copy);
       read_words(buf_next, 0, w0);
       read_a(buf_next, 0, af0);
       __builtin_amdgcn_sched_barrier(0);
@@ -297,6 +318,51 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
     }
   }
   NBLA_WAIT_VMCNT(0);
+
+  if (kWavesK > 1) {
+    // Exact sum of the k groups' accumulators through LDS (the staging buffers are free now), one digit at a time:
+    // groups 1.. store, group 0 adds.
+    uint4_t *red = reinterpret_cast<uint4_t *>(smem);
+    constexpr int kRegs4 = MF * NF * 4; // uint4 per lane per digit
+#pragma unroll
+    for (int d = 0; d < kDigits; ++d) {
+      NBLA_BARRIER();
+      if (wk > 0 && !idle) {
+        uint4_t *dst = red + (size_t)((wk - 1) * kWavesMN + wmn) * kRegs4 * 64 + lane;
+#pragma unroll
+        for (int i = 0; i < MF; ++i)
+#pragma unroll
+          for (int j = 0; j < NF; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              uint4_t v;
+              v.x = acc[d][i][j][4 * q + 0], v.y = acc[d][i][j][4 * q + 1];
+              v.z = acc[d][i][j][4 * q + 2], v.w = acc[d][i][j][4 * q + 3];
+              dst[((i * NF + j) * 4 + q) * 64] = v;
+            }
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): the stores have reached LDS
+      NBLA_BARRIER();
+      if (wk == 0 && !idle) {
+#pragma unroll
+        for (int g = 1; g < kWavesK; ++g) {
+          const uint4_t *srcp = red + (size_t)((g - 1) * kWavesMN + wmn) * kRegs4 * 64 + lane;
+#pragma unroll
+          for (int i = 0; i < MF; ++i)
+#pragma unroll
+            for (int j = 0; j < NF; ++j)
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                const uint4_t v = srcp[((i * NF + j) * 4 + q) * 64];
+                acc[d][i][j][4 * q + 0] += (int)v.x, acc[d][i][j][4 * q + 1] += (int)v.y;
+                acc[d][i][j][4 * q + 2] += (int)v.z, acc[d][i][j][4 * q + 3] += (int)v.w;
+              }
+        }
+      }
+    }
+    if (wk > 0)
+      return;
+  }
 
   // Epilogue.  Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
   // column l%32 of the 32x32 fragment; rows are m and columns n, or the reverse
@@ -418,12 +484,11 @@ __global__ __launch_bounds__(kWavesM *kWavesN * 64, (kWavesM * kWavesN >= 8 ? 1 
 #endif
 }
 
-template <int BM, int BN, int kWavesM, int kWavesN, bool kSwap>
+template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, bool kSwap>
 int launch_tile(const GemmBitsArgs &args, hipStream_t stream) {
-  constexpr int kThreads = kWavesM * kWavesN * 64;
-  constexpr int kStageBytes = (BM / 32) * 2 * kDigits * kFragBytes + 2 * BN * 4;
-  constexpr int kSmem = gemm_bits_stages(BM, BN, kWavesM * kWavesN) * kStageBytes;
-  auto kernel = gemm_bits_kernel<BM, BN, kWavesM, kWavesN, kSwap>;
+  constexpr int kThreads = kWavesM * kWavesN * kWavesK * 64;
+  constexpr int kSmem = gemm_bits_lds_bytes(BM, BN, kWavesM, kWavesN, kWavesK);
+  auto kernel = gemm_bits_kernel<BM, BN, kWavesM, kWavesN, kWavesK, kSwap>;
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
@@ -443,11 +508,15 @@ int launch_tile(const GemmBitsArgs &args, hipStream_t stream) {
 // wavefronts fill a CU.  Blocks of four wavefronts (one per SIMD), two blocks per CU, measured best: the barrier
 // couples only four wavefronts and one block's prologue / epilogue overlaps the other's main loop.  The packed
 // operand costs 1/24 of the digit operand's bytes per element, so the block tile is one row block high and wide
-// (32x512) to keep the global -> LDS traffic lowest; narrow outputs take 32x256 blocks of two wavefronts.
+// (32x512) to keep the global -> LDS traffic lowest; narrow outputs take 32x256 blocks of two wavefronts, and
+// outputs of at most 256 such tiles use eight wavefronts per 32x256 tile, four k groups of two.
 template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream) {
-  if (a.N > 256 && a.M > 128)
-    return launch_tile<32, 512, 1, 4, kSwap>(a, stream);
-  return launch_tile<32, 256, 1, 2, kSwap>(a, stream);
+  const int64_t narrow_tiles = ceil_div(a.M, 32) * ceil_div(a.N, 256);
+  if (narrow_tiles <= 256) // too few tiles for the CUs: four k groups per tile
+    return launch_tile<32, 256, 1, 2, 4, kSwap>(a, stream);
+  if (a.N > 256)
+    return launch_tile<32, 512, 1, 4, 1, kSwap>(a, stream);
+  return launch_tile<32, 256, 1, 2, 1, kSwap>(a, stream);
 }
 
 } // namespace

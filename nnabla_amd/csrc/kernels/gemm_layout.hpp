@@ -24,7 +24,7 @@
 // and q into three balanced base-256 digits q = d0 * 65536 + d1 * 256 + d2, each an int8:
 //     X'[row_block = m / 32][k_tile = k / 32][digit 0..2][lane][16 x int8]
 // followed, per chunk of kChunkK columns, by the row sums of q (one int64 array of row_blocks * 32 entries per
-// chunk), and by the shifts s_m (one int32 array; kBadRow marks a row holding a non-finite value).  Rows >= M and columns >= K are zero.  The number of k tiles is padded to an even count.
+// chunk), and by the shifts s_m (one int32 array; kBadRow marks a row holding a non-finite value).  Rows >= M and columns >= K are zero.  The number of k tiles is padded to a multiple of 8.
 //
 // B ("packed bits"): one bit per weight, set = negative (-1), clear = +1, in groups of 256 columns (eight column
 // fragments F = 0..7 of 32 columns):
@@ -35,7 +35,7 @@
 // is directly register i of the i8 fragment of column fragment F, holding 2^F (as int8: -128 for F = 7) for a
 // negative weight and 0 otherwise: the accumulators of fragment F come out scaled by that constant, which the
 // epilogue divides out exactly.  With b in {0, 1} the signed product is  sum q * (1 - 2 b) = rowsum(q) - 2 sum q b.
-// Bits outside [K, N] are clear; the number of k tiles is padded to an even count.
+// Bits outside [K, N] are clear; the number of k tiles is padded to a multiple of 8.
 //
 // The kernels that binarise weights first emit "pair words" (an intermediate kept in their workspace):
 //     P[k_tile][pair_group = n / 64][lane] : one uint32, bit 4 f + j / 4 + 8 (j % 4) for column half f = 0, 1 and
@@ -64,8 +64,8 @@ __host__ __device__ inline int packed_bit_position(int f, int j) { return 4 * f 
 
 constexpr int kWideGroup = 256; // columns per group of the packed operand
 __host__ __device__ inline int64_t bits_wide_groups(int64_t N) { return ceil_div(N, kWideGroup); }
-// k tiles of the packed operand: an even count (one kernel k step is two tiles), the padding tile all clear
-__host__ __device__ inline int64_t bits_packed_k_tiles(int64_t K) { return ceil_div(K, 2 * kTileK) * 2; }
+// k tiles of the packed operand: padded like the digit operand's, the padding tiles all clear
+__host__ __device__ inline int64_t bits_packed_k_tiles(int64_t K) { return ceil_div(K, 8 * kTileK) * 8; }
 
 // ---- digit operand geometry
 constexpr int kDigits = 3;
@@ -73,7 +73,9 @@ constexpr int64_t kChunkK = 16384;        // columns whose i32 accumulators are 
 constexpr int kDigitMax = 8355711;        // 127 * 65536 + 127 * 256 + 127: the largest q three balanced digits hold
 constexpr int kBadRow = -2147483647 - 1;  // shift value marking a row with a NaN or an infinity
 
-__host__ __device__ inline int64_t digit_k_tiles(int64_t K) { return ceil_div(K, 2 * kTileK) * 2; }
+// k tiles of both bit-weight operands are padded (with zeros) to a multiple of 8: a kernel k step is two tiles and
+// a block may split the contraction over four wavefront groups
+__host__ __device__ inline int64_t digit_k_tiles(int64_t K) { return ceil_div(K, 8 * kTileK) * 8; }
 __host__ __device__ inline int64_t digit_chunks(int64_t K) { return ceil_div(K, kChunkK); }
 // byte offsets of the sections of a digit operand
 struct DigitOperand {

@@ -41,7 +41,7 @@ def unpack_bits(bits_words, K, N):
     """Packed 1-bit GEMM operand (uint32 words, [k_tiles][wide_groups][64 lanes][4]) -> int8 [K, N] of +-1.
     Word i of lane l: bit F + 8 c is column wide_group * 256 + F * 32 + l % 32, k = k_tile * 32 + (l / 32) * 16 + 4 i + c."""
     w = np.ascontiguousarray(bits_words).view(np.uint32)
-    k_tiles = ((K + 63) // 64) * 2          # padded to an even count
+    k_tiles = ((K + 255) // 256) * 8        # padded to a multiple of 8
     groups = (N + 255) // 256
     w = w.reshape(k_tiles, groups, 64, 4)
     out = np.ones((k_tiles * 32, groups * 256), np.int8)
@@ -59,7 +59,7 @@ def unpack_digits(raw, M, K):
     """Digit operand bytes -> (q int64 [M, K], shift int32 [M], row sums int64 [chunks, M]) as the kernels define it:
     fragments [row_block][k_tile][digit][lane][16 x int8], then the row sums ([chunks][rows] int64), then shifts."""
     raw = np.ascontiguousarray(raw).view(np.uint8)
-    rb, kt = (M + 31) // 32, ((K + 63) // 64) * 2
+    rb, kt = (M + 31) // 32, ((K + 255) // 256) * 8
     rows, chunks = rb * 32, (K + 16383) // 16384
     nfrag = rb * kt * 3 * 1024
     d = raw[:nfrag].view(np.int8).reshape(rb, kt, 3, 64, 16).astype(np.int64)
