@@ -155,31 +155,26 @@ struct Pow2Op {
 
 // Pow2Quantize with few levels (2^n' <= 8): |x| as a bit pattern is compared against the level boundaries
 // directly.  roundf(log2f(a)) is a non-decreasing step function of a, so level e starts at the calibrated cut of
-// binade e-1; the output exponent is e_min plus the number of boundaries at or below |x|.
+// binade e-1; with_zero adds the boundary p_min * 2^-0.5 below which the result is 0.  The result is the value of
+// the last boundary at or below |x| (positive floats order like their bit patterns).
 template <int kLevels> struct Pow2SmallOp {
-  uint32_t bound[kLevels]; // bound[0] = first |x| with r >= e_min, bound[j] = first |x| with r >= e_min + j
-  float p_min, thr;
-  int e_min;
-  int sign, with_zero;
+  uint32_t bound[kLevels]; // ascending; unused entries 0xffffffff
+  float value[kLevels];    // result from bound[j] on
+  float base;              // result below bound[0]
+  float neg_value;         // result for x < 0 when unsigned
+  int sign;
   __device__ __forceinline__ void prepare() {}
   __device__ __forceinline__ float operator()(float x) const {
     const uint32_t u = __float_as_uint(x) & 0x7fffffffu;
-    float q;
-    if (u > 0x7f800000u) {
-      q = __uint_as_float(u);
-    } else if (u < bound[0]) {
-      q = with_zero ? ((__uint_as_float(u) < thr) ? 0.0f : p_min) : p_min;
-    } else {
-      int up = 0;
+    float q = base;
 #pragma unroll
-      for (int j = 1; j < kLevels; ++j)
-        up += (u >= bound[j]) ? 1 : 0;
-      q = pow2_int(e_min + up);
-    }
+    for (int j = 0; j < kLevels; ++j)
+      q = (u >= bound[j]) ? value[j] : q;
+    q = (u > 0x7f800000u) ? __uint_as_float(u) : q; // NaN propagates through every comparison of the reference
     const bool neg = x < 0.0f;
     if (sign)
       return neg ? -q : q;
-    return neg ? (with_zero ? 0.0f : p_min) : q;
+    return neg ? neg_value : q;
   }
 };
 
@@ -231,35 +226,47 @@ int nbla_hip_pow2_quantize_f32(const float *x, float *y, size_t size, int sign, 
   int rc = ensure_init();
   if (rc)
     return rc;
-  if (nn <= 3) { // up to eight levels: boundaries travel as kernel arguments
+  if (nn <= 3) { // up to eight levels: boundaries and level values travel as kernel arguments
     uint32_t table[kNumBinades];
     rc = nbla_hip_cut_table(kCutPow2Round, table);
     if (rc)
       return rc;
     const int levels = 1 << nn;
+    const float p_min = (float)std::pow(2., e_min);
+    const float thr = (float)((float)p_min * std::pow(2., -0.5)); // pow2_quantize.cpp:39 (float member times double)
     uint32_t bound[8];
-    for (int j = 0; j < levels; ++j) {
+    float value[8];
+    int count = 0;
+    if (with_zero) { // p_min where r >= e_min (from the cut of binade e_min-1 on) or |x| >= thr; 0 below both
+      uint32_t thr_bits;
+      std::memcpy(&thr_bits, &thr, sizeof(thr_bits));
+      const int binade = (e_min - 1) + 149;
+      const uint32_t cut = binade >= 0 ? table[binade] : 1u;
+      bound[count] = thr_bits < cut ? thr_bits : cut;
+      value[count++] = p_min;
+    }
+    for (int j = 1; j < levels; ++j) {
       const int binade = (e_min + j - 1) + 149; // the cut where r steps from e_min+j-1 to e_min+j
       // below the smallest subnormal binade every positive value already rounds to >= -149
-      bound[j] = binade >= 0 ? table[binade] : 1u;
+      bound[count] = binade >= 0 ? table[binade] : 1u;
+      value[count++] = (float)std::pow(2., e_min + j);
     }
-    const float p_min = (float)std::pow(2., e_min);
-    const float thr = (float)((float)p_min * std::pow(2., -0.5));
     auto fill = [&](auto &op) {
-      for (int j = 0; j < levels; ++j)
-        op.bound[j] = bound[j];
-      op.p_min = p_min;
-      op.thr = thr;
-      op.e_min = e_min;
+      constexpr int cap = (int)(sizeof(op.bound) / sizeof(op.bound[0]));
+      for (int j = 0; j < cap; ++j) {
+        op.bound[j] = j < count ? bound[j] : 0xffffffffu;
+        op.value[j] = j < count ? value[j] : 0.0f;
+      }
+      op.base = with_zero ? 0.0f : p_min;
+      op.neg_value = with_zero ? 0.0f : p_min;
       op.sign = sign;
-      op.with_zero = with_zero;
     };
-    if (levels == 2) {
+    if (count <= 2) {
       Pow2SmallOp<2> op;
       fill(op);
       return launch_map(x, y, size, op, as_stream(stream), "pow2_quantize");
     }
-    if (levels == 4) {
+    if (count <= 4) {
       Pow2SmallOp<4> op;
       fill(op);
       return launch_map(x, y, size, op, as_stream(stream), "pow2_quantize");
@@ -359,55 +366,74 @@ MinMaxPlan make_plan(const int64_t *xshape, int ndim, const int64_t *qshape) {
   return P;
 }
 
+// min.cpp:29-41 / max.cpp:48-60 scan the slice in index order with strict comparisons starting from +-1e8; of
+// several equal extrema the first wins, which is only visible for +0 / -0.  Plain min / max give the value (NaN is
+// ignored by both formulations); beside them the first zero of the slice (index and sign) is tracked, and when the
+// extremum turns out to be zero it takes that element's sign.  Zeros are rare in most inputs, so their bookkeeping
+// sits behind a branch.
 struct MinMaxPartial {
   float vmin;
-  uint32_t imin;
   float vmax;
-  uint32_t imax;
+  uint32_t zidx;  // index of the first +-0 element, 0xffffffff if none
+  uint32_t zsign; // its sign bit
 };
 
-// min.cpp:29-41 / max.cpp:48-60 scan the slice in index order with strict
-// comparisons starting from +-1e8; the first of several equal extrema (which can
-// only differ for +0/-0) wins.  Tracking (value, first index) and combining with
-// "smaller value, then smaller index" reproduces that for any traversal order.
 struct Extrema {
   float vmin, vmax;
-  uint32_t imin, imax;
+  uint32_t zidx, zsign;
   __device__ __forceinline__ void init() {
     vmin = 1e+8f;
     vmax = -1e+8f;
-    imin = imax = 0xffffffffu;
+    zidx = 0xffffffffu;
+    zsign = 0u;
   }
   __device__ __forceinline__ void take(float v, uint32_t i) { // i increases per thread
-    if (v < vmin) {
-      vmin = v;
-      imin = i;
-    }
-    if (v > vmax) {
-      vmax = v;
-      imax = i;
+    vmin = __builtin_fminf(vmin, v);
+    vmax = __builtin_fmaxf(vmax, v);
+    const uint32_t u = __float_as_uint(v);
+    if ((u << 1) == 0u && zidx == 0xffffffffu) {
+      zidx = i;
+      zsign = u >> 31;
     }
   }
-  __device__ __forceinline__ void merge(float omin, uint32_t oimin, float omax, uint32_t oimax) {
-    if (omin < vmin || (omin == vmin && oimin < imin)) {
-      vmin = omin;
-      imin = oimin;
+  __device__ __forceinline__ void take4(float4_t v, uint32_t i) {
+    vmin = __builtin_fminf(__builtin_fminf(vmin, v.x), __builtin_fminf(v.y, __builtin_fminf(v.z, v.w)));
+    vmax = __builtin_fmaxf(__builtin_fmaxf(vmax, v.x), __builtin_fmaxf(v.y, __builtin_fmaxf(v.z, v.w)));
+    const uint32_t ux = __float_as_uint(v.x) << 1, uy = __float_as_uint(v.y) << 1;
+    const uint32_t uz = __float_as_uint(v.z) << 1, uw = __float_as_uint(v.w) << 1;
+    if (min(min(ux, uy), min(uz, uw)) == 0u && zidx == 0xffffffffu) {
+      const int c = (ux == 0u) ? 0 : (uy == 0u) ? 1 : (uz == 0u) ? 2 : 3;
+      const float z = (c == 0) ? v.x : (c == 1) ? v.y : (c == 2) ? v.z : v.w;
+      zidx = i + c;
+      zsign = __float_as_uint(z) >> 31;
     }
-    if (omax > vmax || (omax == vmax && oimax < imax)) {
-      vmax = omax;
-      imax = oimax;
+  }
+  __device__ __forceinline__ void merge(float omin, float omax, uint32_t ozidx, uint32_t ozsign) {
+    vmin = __builtin_fminf(vmin, omin);
+    vmax = __builtin_fmaxf(vmax, omax);
+    if (ozidx < zidx) {
+      zidx = ozidx;
+      zsign = ozsign;
     }
   }
   __device__ __forceinline__ void wave_reduce() {
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) {
       const float a = __shfl_xor(vmin, off);
-      const uint32_t ai = __shfl_xor(imin, off);
       const float b = __shfl_xor(vmax, off);
-      const uint32_t bi = __shfl_xor(imax, off);
-      merge(a, ai, b, bi);
+      const uint32_t zi = __shfl_xor(zidx, off);
+      const uint32_t zs = __shfl_xor(zsign, off);
+      merge(a, b, zi, zs);
     }
   }
+  // the extrema as the reference's scan would leave them
+  __device__ __forceinline__ float min_value() const {
+    return (vmin == 0.0f) ? __uint_as_float(zsign << 31) : vmin;
+  }
+  __device__ __forceinline__ float max_value() const {
+    return (vmax == 0.0f) ? __uint_as_float(zsign << 31) : vmax;
+  }
+  __device__ __forceinline__ MinMaxPartial pack() const { return MinMaxPartial{vmin, vmax, zidx, zsign}; }
 };
 
 // Stage 1: block (chunk c, channel k) scans tiles c, c+nchunks, ... of channel k.
@@ -427,10 +453,7 @@ __global__ __launch_bounds__(kRedBlock) void minmax_reduce_tiles(const float *__
     const uint32_t idx = (uint32_t)(r0 * R1 + r1);
     if (kVec) { // R1 % 4 == 0 and x 16-byte aligned
       const float4_t v = *reinterpret_cast<const float4_t *>(p);
-      ex.take(v.x, idx);
-      ex.take(v.y, idx + 1);
-      ex.take(v.z, idx + 2);
-      ex.take(v.w, idx + 3);
+      ex.take4(v, idx);
     } else {
       const int n = (R1 - r1) < 4 ? (int)(R1 - r1) : 4;
       for (int j = 0; j < n; ++j)
@@ -441,44 +464,39 @@ __global__ __launch_bounds__(kRedBlock) void minmax_reduce_tiles(const float *__
   __shared__ MinMaxPartial s_part[kRedBlock / 64];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   if (lane == 0)
-    s_part[wave] = MinMaxPartial{ex.vmin, ex.imin, ex.vmax, ex.imax};
+    s_part[wave] = ex.pack();
   __syncthreads();
   if (threadIdx.x == 0) {
     for (int w = 1; w < kRedBlock / 64; ++w)
-      ex.merge(s_part[w].vmin, s_part[w].imin, s_part[w].vmax, s_part[w].imax);
-    partial[k * nchunks + blockIdx.x] = MinMaxPartial{ex.vmin, ex.imin, ex.vmax, ex.imax};
+      ex.merge(s_part[w].vmin, s_part[w].vmax, s_part[w].zidx, s_part[w].zsign);
+    partial[k * nchunks + blockIdx.x] = ex.pack();
   }
 }
 
-// Per-tensor stage 1 (K == 1, 16-byte aligned): a flat grid-strided scan with
-// four independent 128-bit loads in flight per thread.
+// Per-tensor stage 1 (K == 1, 16-byte aligned): every block scans one contiguous range.
 __global__ __launch_bounds__(kRedBlock) void minmax_reduce_flat(const float *__restrict__ x, MinMaxPartial *__restrict__ partial,
                                                                 size_t n4, size_t size) {
   Extrema ex;
   ex.init();
-  const size_t stride = (size_t)gridDim.x * kRedBlock;
-  size_t i = (size_t)blockIdx.x * kRedBlock + threadIdx.x;
-  for (; i + 3 * stride < n4; i += 4 * stride) {
+  // block b streams the contiguous range [b * per, (b + 1) * per) of float4s, four 128-bit loads in flight per thread
+  const size_t per = (n4 + gridDim.x - 1) / gridDim.x;
+  const size_t begin = (size_t)blockIdx.x * per, end = (begin + per < n4) ? begin + per : n4;
+  size_t i = begin + threadIdx.x;
+  for (; i + 3 * kRedBlock < end; i += 4 * kRedBlock) {
     float4_t v[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      v[j] = load4(x + 4 * (i + j * stride));
+      v[j] = load4(x + 4 * (i + j * kRedBlock));
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t idx = (uint32_t)(4 * (i + j * stride));
-      ex.take(v[j].x, idx);
-      ex.take(v[j].y, idx + 1);
-      ex.take(v[j].z, idx + 2);
-      ex.take(v[j].w, idx + 3);
+      const uint32_t idx = (uint32_t)(4 * (i + j * kRedBlock));
+      ex.take4(v[j], idx);
     }
   }
-  for (; i < n4; i += stride) {
+  for (; i < end; i += kRedBlock) {
     const float4_t v = load4(x + 4 * i);
     const uint32_t idx = (uint32_t)(4 * i);
-    ex.take(v.x, idx);
-    ex.take(v.y, idx + 1);
-    ex.take(v.z, idx + 2);
-    ex.take(v.w, idx + 3);
+    ex.take4(v, idx);
   }
   if (blockIdx.x == gridDim.x - 1) { // tail elements, highest indices
     const size_t t = 4 * n4 + threadIdx.x;
@@ -489,12 +507,12 @@ __global__ __launch_bounds__(kRedBlock) void minmax_reduce_flat(const float *__r
   __shared__ MinMaxPartial s_part[kRedBlock / 64];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   if (lane == 0)
-    s_part[wave] = MinMaxPartial{ex.vmin, ex.imin, ex.vmax, ex.imax};
+    s_part[wave] = ex.pack();
   __syncthreads();
   if (threadIdx.x == 0) {
     for (int w = 1; w < kRedBlock / 64; ++w)
-      ex.merge(s_part[w].vmin, s_part[w].imin, s_part[w].vmax, s_part[w].imax);
-    partial[blockIdx.x] = MinMaxPartial{ex.vmin, ex.imin, ex.vmax, ex.imax};
+      ex.merge(s_part[w].vmin, s_part[w].vmax, s_part[w].zidx, s_part[w].zsign);
+    partial[blockIdx.x] = ex.pack();
   }
 }
 
@@ -515,17 +533,16 @@ __global__ __launch_bounds__(64) void minmax_finalize(const MinMaxPartial *__res
   Extrema ex;
   ex.init();
   if (s.x_min_max) {
-    // four independent 16-byte loads in flight per lane before any merge
+    // sixteen independent 16-byte loads in flight per lane before any merge: one round trip for 1024 partials
     const float4_t *pp = reinterpret_cast<const float4_t *>(partial + k * nchunks);
-    for (int c = threadIdx.x; c < nchunks; c += 256) {
-      float4_t q[4];
+    for (int c = threadIdx.x; c < nchunks; c += 1024) {
+      float4_t q[16];
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        q[j] = (c + 64 * j < nchunks) ? pp[c + 64 * j] : float4_t{1e+8f, __uint_as_float(0xffffffffu), -1e+8f,
-                                                                   __uint_as_float(0xffffffffu)};
+      for (int j = 0; j < 16; ++j)
+        q[j] = (c + 64 * j < nchunks) ? pp[c + 64 * j] : float4_t{1e+8f, -1e+8f, __uint_as_float(0xffffffffu), 0.0f};
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        ex.merge(q[j].x, __float_as_uint(q[j].y), q[j].z, __float_as_uint(q[j].w));
+      for (int j = 0; j < 16; ++j)
+        ex.merge(q[j].x, q[j].y, __float_as_uint(q[j].z), __float_as_uint(q[j].w));
     }
     ex.wave_reduce();
   }
@@ -533,15 +550,15 @@ __global__ __launch_bounds__(64) void minmax_finalize(const MinMaxPartial *__res
     return;
   float lo = qr_min[k], hi = qr_max[k];
   if (s.x_min_max && s.ema) {
-    const float a = ex.vmin * s.one_minus_decay;
+    const float a = ex.min_value() * s.one_minus_decay;
     lo = lo * s.decay;
     lo = lo + a;
-    const float b = ex.vmax * s.one_minus_decay;
+    const float b = ex.max_value() * s.one_minus_decay;
     hi = hi * s.decay;
     hi = hi + b;
   } else if (s.x_min_max) {
-    lo = ex.vmin;
-    hi = ex.vmax;
+    lo = ex.min_value();
+    hi = ex.max_value();
   }
   if (hi - lo < s.eps)
     hi = lo + s.eps;
