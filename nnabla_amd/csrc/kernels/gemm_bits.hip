@@ -186,14 +186,24 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
   }
   typedef __attribute__((address_space(3))) void lds_void_t;
   auto lds_at = [&](int byte_off) { return (lds_void_t *)(smem + byte_off); };
-  // issues the copies of the stage starting at k step `ks` into LDS buffer `buf`
-  auto copy_step = [&](int64_t ks, int buf) {
+  // Stages are copied in order; each slot keeps a cursor that advances by one stage per call and stops at the last
+  // stage (the final calls copy it again rather than run past the operand).
+  const uint4_t *cur[kSlots], *cur_last[kSlots];
+#pragma unroll
+  for (int p = 0; p < kSlots; ++p) {
+    cur[p] = src[p] + a.step_begin * src_step[p];
+    cur_last[p] = src[p] + (a.step_end - kWavesK) * src_step[p];
+  }
+  // issues the copies of the next stage into LDS buffer `buf`
+  auto copy_next = [&](int buf) {
 #pragma unroll
     for (int p = 0; p < kSlots; ++p) {
       if (p == kPerWave && wave >= kExtra)
         break;
-      __builtin_amdgcn_global_load_lds(src[p] + ks * src_step[p] + lane,
-                                       lds_at(buf * kStageBytes + (p * kWaves + wave) * kFragBytes), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(cur[p] + lane, lds_at(buf * kStageBytes + (p * kWaves + wave) * kFragBytes), 16,
+                                       0, 0);
+      const uint4_t *next = cur[p] + kWavesK * src_step[p];
+      cur[p] = next < cur_last[p] ? next : cur_last[p];
     }
   };
   // waits until at most `steps` k steps of this wavefront's copies are in flight
@@ -272,7 +282,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
   const int64_t first = a.step_begin, last = a.step_end - kWavesK;
 #pragma unroll
   for (int d = 0; d < kDepth; ++d)
-    copy_step(first + d * kWavesK < last ? first + d * kWavesK : last, d);
+    copy_next(d);
   wait_copies(std::integral_constant<int, kDepth - 1>());
   NBLA_BARRIER();
   read_words(0, 0, w0);
@@ -286,7 +296,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
       const int buf_copy = (buf == 0) ? kStages - 1 : buf - 1;
       wait_copies(std::integral_constant<int, kDepth - 1>());
       NBLA_BARRIER();
-      copy_step(ks + kDepth * kWavesK < last ? ks + kDepth * kWavesK : last, buf_copy);
+      copy_next(buf_copy);
       buf = (buf + 1 == kStages) ? 0 : buf + 1;
     }
   } else {
@@ -308,7 +318,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
       // tile 1 runs; the copy of step ks+kDepth is issued; tile 0 of step ks+1 is fetched
       mma(af1, w1, J0(), J1());
       __builtin_amdgcn_sched_barrier(0);
-      copy_step(ks + kDepth * kWavesK < last ? ks + kDepth * kWavesK : last, buf_copy);
+      copy_next(buf_copy);
       read_words(buf_next, 0, w0);
       read_a(buf_next, 0, af0);
       __builtin_amdgcn_sched_barrier(0);
