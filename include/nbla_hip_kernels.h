@@ -103,6 +103,48 @@ int nbla_hip_min_max_quantize_f32(const float *x, float *y,
                                   float eps, void *workspace,
                                   size_t workspace_bytes, void *stream);
 
+/* ------------------------------------------------ quantizers: backward (STE) */
+
+/* dx (+)= dy inside [min, max], 0 outside (an accumulated dx is left alone
+ * there); plain dx (+)= dy when ste_fine_grained == 0.  Replaces
+ * FixedPointQuantize<float>::backward_impl,
+ * src/nbla/function/generic/fixed_point_quantize.cpp:69-127.  accum != 0 adds to
+ * the existing dx. */
+int nbla_hip_fixed_point_quantize_backward_f32(const float *dy, const float *x,
+                                               float *dx, size_t size, int sign,
+                                               int n, float delta,
+                                               int ste_fine_grained, int accum,
+                                               void *stream);
+
+/* dx (+)= c * dy with c = 0 where 2^round(log2|x|) > 2^m and, unsigned, where
+ * x < 0.  Replaces Pow2Quantize<float>::backward_impl,
+ * src/nbla/function/generic/pow2_quantize.cpp:84-156. */
+int nbla_hip_pow2_quantize_backward_f32(const float *dy, const float *x,
+                                        float *dx, size_t size, int sign,
+                                        int with_zero, int n, int m,
+                                        int ste_fine_grained, int accum,
+                                        void *stream);
+
+size_t nbla_hip_min_max_quantize_backward_workspace_bytes(const int64_t *xshape,
+                                                          int ndim,
+                                                          const int64_t *qshape);
+
+/* Backward of MinMaxQuantize.  Replaces MinMaxQuantize<float>::backward_impl,
+ * src/nbla/function/generic/min_max_quantize.cpp:225-350: with [m', M'] the
+ * nudged range recomputed from qr_min, ql_min, ql_max and the forward's scale,
+ *   dx       (+)= (x >= m') * (x <= M') * dy        (dy alone if not fine grained)
+ *   g_qr_min (+)= sum over the reduced axes of (x < m') * dy
+ *   g_qr_max (+)= sum over the reduced axes of (x > M') * dy
+ * the range gradients only when neither x_min_max nor ema is set (:294-295).
+ * dx, g_qr_min, g_qr_max may be NULL (not propagated). */
+int nbla_hip_min_max_quantize_backward_f32(
+    const float *dy, const float *x, float *dx, const int64_t *xshape, int ndim,
+    const int64_t *qshape, const float *qr_min, const float *qr_max,
+    const float *ql_min, const float *ql_max, const float *scale,
+    float *g_qr_min, float *g_qr_max, int ste_fine_grained, int x_min_max,
+    int ema, int accum_x, int accum_min, int accum_max, void *workspace,
+    size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------- binary weights: sign/alpha/pack */
 
 /* Bytes of the 1-bit packed GEMM operand for a [K, N] weight matrix (K padded

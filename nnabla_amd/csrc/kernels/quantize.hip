@@ -3,6 +3,7 @@
 // operation rounded on its own (the file is compiled with -ffp-contract=off and
 // correctly rounded division), wavefront-shuffle reductions for the min/max.
 #include "common.hpp"
+#include "quantize_common.hpp"
 
 #include <cmath>
 #include <cstring>
@@ -14,7 +15,6 @@ constexpr int kBlock = 256;  // threads per block: 4 wavefronts
 constexpr int kUnroll = 4;   // float4 per thread per block tile (large inputs)
 constexpr int kTile = kBlock * kUnroll; // float4 per block at full unroll
 
-typedef float float4_t __attribute__((ext_vector_type(4)));
 
 // Streaming access pattern that measured best on MI355X for a read-once/write-once map: ordinary 128-bit loads,
 // nontemporal 128-bit stores.
@@ -293,48 +293,6 @@ int nbla_hip_pow2_quantize_f32(const float *x, float *y, size_t size, int sign, 
 // ---------------------------------------------------------------------- MinMax
 namespace nbla_hip {
 namespace {
-
-// (x shape, q shape) collapsed to element index = (r0 * K + k) * R1 + r1 with k
-// the kept (per-channel) index and r0, r1 the reduced ones.
-struct MinMaxLayout {
-  int64_t R0, K, R1, total;
-  bool ok;
-};
-
-MinMaxLayout collapse(const int64_t *xshape, int ndim, const int64_t *qshape) {
-  // runs of (kept?) axes, ignoring size-1 axes
-  int64_t sizes[3] = {1, 1, 1};
-  int stage = 0; // 0: leading reduced, 1: kept, 2: trailing reduced
-  MinMaxLayout L{1, 1, 1, 1, true};
-  for (int i = 0; i < ndim; ++i) {
-    const int64_t s = xshape[i];
-    L.total *= s;
-    if (s == 1)
-      continue;
-    const bool kept = qshape[i] != 1;
-    if (kept) {
-      if (stage == 0)
-        stage = 1;
-      else if (stage == 2) {
-        L.ok = false; // kept, reduced, kept: not a single (R0, K, R1) pattern
-        continue;
-      }
-      sizes[1] *= s;
-    } else {
-      if (stage == 1)
-        stage = 2;
-      sizes[stage == 0 ? 0 : 2] *= s;
-    }
-  }
-  L.R0 = sizes[0];
-  L.K = sizes[1];
-  L.R1 = sizes[2];
-  if (L.K == 1) { // per-tensor: one flat run
-    L.R1 = L.R0 * L.R1;
-    L.R0 = 1;
-  }
-  return L;
-}
 
 constexpr int kRedBlock = 256;
 constexpr int kRedTile = kRedBlock * 4; // elements per block tile

@@ -1,0 +1,340 @@
+// Backward passes (straight-through estimators) of FixedPointQuantize, Pow2Quantize and MinMaxQuantize:
+// HBM-bound elementwise kernels (128-bit accesses) and, for the MinMaxQuantize range gradients, masked sums with a
+// fixed summation order.
+#include "common.hpp"
+#include "quantize_common.hpp"
+
+#include <cmath>
+#include <cstring>
+
+namespace nbla_hip {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 4;
+
+__device__ __forceinline__ float4_t load4(const float *p) { return *reinterpret_cast<const float4_t *>(p); }
+__device__ __forceinline__ void store4(float *p, float4_t v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<float4_t *>(p));
+}
+
+// dx[i] = op(dy[i], x[i], i) (+ dx[i] when kAccum).  `op` returns the gradient contribution; kUseX tells whether x is
+// read at all.
+template <typename Op, bool kAccum, bool kUseX>
+__global__ __launch_bounds__(kBlock) void grad_vec4(const float *__restrict__ dy, const float *__restrict__ x,
+                                                    float *__restrict__ dx, size_t n4, size_t size, Op op) {
+  const size_t base = (size_t)blockIdx.x * (kBlock * kUnroll) + threadIdx.x;
+  float4_t g[kUnroll], v[kUnroll], o[kUnroll];
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const size_t i = base + (size_t)j * kBlock;
+    if (i < n4) {
+      g[j] = load4(dy + 4 * i);
+      if (kUseX)
+        v[j] = load4(x + 4 * i);
+      if (kAccum)
+        o[j] = load4(dx + 4 * i);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const size_t i = base + (size_t)j * kBlock;
+    if (i < n4) {
+      float4_t r;
+      r.x = op.template apply<kAccum>(g[j].x, kUseX ? v[j].x : 0.0f, kAccum ? o[j].x : 0.0f, 4 * i);
+      r.y = op.template apply<kAccum>(g[j].y, kUseX ? v[j].y : 0.0f, kAccum ? o[j].y : 0.0f, 4 * i + 1);
+      r.z = op.template apply<kAccum>(g[j].z, kUseX ? v[j].z : 0.0f, kAccum ? o[j].z : 0.0f, 4 * i + 2);
+      r.w = op.template apply<kAccum>(g[j].w, kUseX ? v[j].w : 0.0f, kAccum ? o[j].w : 0.0f, 4 * i + 3);
+      store4(dx + 4 * i, r);
+    }
+  }
+  if (blockIdx.x == 0) {
+    const size_t i = 4 * n4 + threadIdx.x;
+    if (i < size)
+      dx[i] = op.template apply<kAccum>(dy[i], kUseX ? x[i] : 0.0f, kAccum ? dx[i] : 0.0f, i);
+  }
+}
+
+template <typename Op, bool kAccum, bool kUseX>
+__global__ __launch_bounds__(kBlock) void grad_scalar(const float *__restrict__ dy, const float *__restrict__ x,
+                                                      float *__restrict__ dx, size_t size, Op op) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < size; i += (size_t)gridDim.x * kBlock)
+    dx[i] = op.template apply<kAccum>(dy[i], kUseX ? x[i] : 0.0f, kAccum ? dx[i] : 0.0f, i);
+}
+
+template <typename Op, bool kUseX>
+int launch_grad(const float *dy, const float *x, float *dx, size_t size, int accum, Op op, hipStream_t stream,
+                const char *what) {
+  if (size == 0)
+    return NBLA_HIP_OK;
+  if (aligned16(dy) && aligned16(dx) && (!kUseX || aligned16(x))) {
+    const size_t n4 = size / 4, tile = (size_t)kBlock * kUnroll;
+    const size_t blocks = n4 ? (n4 + tile - 1) / tile : 1;
+    if (accum)
+      hipLaunchKernelGGL((grad_vec4<Op, true, kUseX>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, dy, x, dx, n4,
+                         size, op);
+    else
+      hipLaunchKernelGGL((grad_vec4<Op, false, kUseX>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, dy, x, dx, n4,
+                         size, op);
+  } else {
+    size_t blocks = (size + kBlock - 1) / kBlock;
+    if (blocks > 65536)
+      blocks = 65536;
+    if (accum)
+      hipLaunchKernelGGL((grad_scalar<Op, true, kUseX>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, dy, x, dx,
+                         size, op);
+    else
+      hipLaunchKernelGGL((grad_scalar<Op, false, kUseX>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, dy, x, dx,
+                         size, op);
+  }
+  NBLA_HIP_LAUNCH_CHECK(what);
+  return NBLA_HIP_OK;
+}
+
+// Plain straight-through: dx (+)= dy  (fixed_point_quantize.cpp:69-78, pow2_quantize.cpp:84-93,
+// min_max_quantize.cpp:285-291).
+struct PassOp {
+  template <bool kAccum> __device__ __forceinline__ float apply(float dy, float, float old, size_t) const {
+    return kAccum ? dy + old : dy;
+  }
+};
+
+// fixed_point_quantize.cpp:81-99: gradient only inside [min, max]; outside, an accumulated dx is left as it is.
+struct FixedPointGradOp {
+  float max_, min_;
+  template <bool kAccum> __device__ __forceinline__ float apply(float dy, float x, float old, size_t) const {
+    if (x > max_ || x < min_)
+      return kAccum ? old : 0.0f;
+    return kAccum ? old + dy : dy;
+  }
+};
+
+// pow2_quantize.cpp:96-125: c = 0 where 2^round(log2|x|) > p_max (|x| at or above the calibrated cut of binade
+// log2(p_max), infinity included) and, unsigned, where x < 0; dx (+)= c * dy as a product.
+struct Pow2GradOp {
+  uint32_t cut; // first |x| pattern whose rounded exponent exceeds log2(p_max)
+  int sign;
+  template <bool kAccum> __device__ __forceinline__ float apply(float dy, float x, float old, size_t) const {
+    const uint32_t u = __float_as_uint(x) & 0x7fffffffu;
+    float c = (u >= cut && u <= 0x7f800000u) ? 0.0f : 1.0f; // NaN: q > p_max is false
+    if (!sign)
+      c = (x < 0.0f) ? 0.0f : c;
+    const float t = c * dy;
+    return kAccum ? old + t : t;
+  }
+};
+
+// min_max_quantize.cpp:262-284: mask = (x >= m') * (x <= M'), dx = mask * dy (+ dx); bounds per channel
+// (element i belongs to channel (i / R1) % K).
+struct MinMaxGradOp {
+  const float2 *bounds; // (m', M') per channel
+  int64_t K, R1;
+  template <bool kAccum> __device__ __forceinline__ float apply(float dy, float x, float old, size_t i) const {
+    const float2 b = bounds[K == 1 ? 0 : (int64_t)(i / R1) % K];
+    const float iv0 = (x >= b.x) ? 1.0f : 0.0f, iv1 = (x <= b.y) ? 1.0f : 0.0f;
+    float mask = iv0 * iv1;
+    mask = mask * dy;
+    return kAccum ? mask + old : mask;
+  }
+};
+
+// ---- MinMaxQuantize range gradients
+__global__ __launch_bounds__(64) void minmax_bounds(const float *__restrict__ qr_min, const float *__restrict__ ql_min,
+                                                    const float *__restrict__ ql_max, const float *__restrict__ scale,
+                                                    float2 *__restrict__ bounds, int64_t K) {
+  const int64_t k = (int64_t)blockIdx.x * 64 + threadIdx.x;
+  if (k >= K)
+    return;
+  float m_n, M_n;
+  nudge_qr_min_max(qr_min[k], ql_min[k], ql_max[k], scale[k], m_n, M_n);
+  bounds[k] = float2{m_n, M_n};
+}
+
+// Block (chunk c, channel k) adds mask * dy over tiles c, c + nchunks, ... of channel k, for both masks
+// (x < m' and x > M'): per thread in index order, then lanes, wavefronts in a fixed order.
+constexpr int kSumTile = kBlock * 4;
+__global__ __launch_bounds__(kBlock) void minmax_range_grad_partial(const float *__restrict__ dy,
+                                                                    const float *__restrict__ x,
+                                                                    const float2 *__restrict__ bounds,
+                                                                    float2 *__restrict__ partial, int64_t K, int64_t R1,
+                                                                    int64_t tiles_per_row, int64_t tiles_per_k,
+                                                                    int nchunks) {
+  const int64_t k = blockIdx.y;
+  const float2 b = bounds[k];
+  float lo = 0.0f, hi = 0.0f;
+  for (int64_t t = blockIdx.x; t < tiles_per_k; t += nchunks) {
+    const int64_t r0 = t / tiles_per_row, tr = t - r0 * tiles_per_row;
+    const int64_t base = (r0 * K + k) * R1;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t r1 = tr * kSumTile + j * kBlock + threadIdx.x;
+      if (r1 < R1) {
+        const float xv = x[base + r1], g = dy[base + r1];
+        lo += ((xv < b.x) ? 1.0f : 0.0f) * g;
+        hi += ((xv > b.y) ? 1.0f : 0.0f) * g;
+      }
+    }
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    lo += __shfl_xor(lo, off);
+    hi += __shfl_xor(hi, off);
+  }
+  __shared__ float2 s_part[kBlock / 64];
+  if ((threadIdx.x & 63) == 0)
+    s_part[threadIdx.x >> 6] = float2{lo, hi};
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float2 acc = s_part[0];
+    for (int w = 1; w < kBlock / 64; ++w)
+      acc.x += s_part[w].x, acc.y += s_part[w].y;
+    partial[k * nchunks + blockIdx.x] = acc;
+  }
+}
+
+__global__ __launch_bounds__(64) void minmax_range_grad_final(const float2 *__restrict__ partial, int nchunks,
+                                                              float *__restrict__ g_min, float *__restrict__ g_max,
+                                                              int accum_min, int accum_max, int64_t K) {
+  const int64_t k = (int64_t)blockIdx.x * 64 + threadIdx.x;
+  if (k >= K)
+    return;
+  float lo = 0.0f, hi = 0.0f;
+  for (int c = 0; c < nchunks; ++c) {
+    lo += partial[k * nchunks + c].x;
+    hi += partial[k * nchunks + c].y;
+  }
+  if (g_min)
+    g_min[k] = accum_min ? g_min[k] + lo : lo; // add2(g_qr_min, sum) :316-317
+  if (g_max)
+    g_max[k] = accum_max ? g_max[k] + hi : hi;
+}
+
+struct RangeGradPlan {
+  MinMaxLayout L;
+  int64_t tiles_per_row, tiles_per_k;
+  int nchunks;
+  size_t bounds_bytes, partial_bytes;
+};
+
+RangeGradPlan make_range_plan(const int64_t *xshape, int ndim, const int64_t *qshape) {
+  RangeGradPlan P;
+  P.L = collapse(xshape, ndim, qshape);
+  P.tiles_per_row = (P.L.R1 + kSumTile - 1) / kSumTile;
+  P.tiles_per_k = P.tiles_per_row * P.L.R0;
+  int64_t chunks = 1024 / (P.L.K < 1024 ? P.L.K : 1024);
+  if (chunks < 1)
+    chunks = 1;
+  if (chunks > P.tiles_per_k)
+    chunks = P.tiles_per_k;
+  if (chunks < 1)
+    chunks = 1;
+  P.nchunks = (int)chunks;
+  P.bounds_bytes = round_up((size_t)P.L.K * sizeof(float2), 256);
+  P.partial_bytes = round_up((size_t)P.L.K * P.nchunks * sizeof(float2), 256);
+  return P;
+}
+
+} // namespace
+} // namespace nbla_hip
+
+using namespace nbla_hip;
+
+extern "C" {
+
+int nbla_hip_fixed_point_quantize_backward_f32(const float *dy, const float *x, float *dx, size_t size, int sign, int n,
+                                               float delta, int ste_fine_grained, int accum, void *stream) {
+  if (!(n > 0 && delta > 0.))
+    return fail(NBLA_HIP_ERR_VALUE, "Both bit width and delta should be positive.");
+  const int nn = sign ? n - 1 : n;
+  if (!(nn > 0))
+    return fail(NBLA_HIP_ERR_VALUE, "bit width should be positive when considering sign (1bit).");
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  if (!ste_fine_grained)
+    return launch_grad<PassOp, false>(dy, x, dx, size, accum, PassOp(), as_stream(stream), "quantize backward");
+  const float max_ = (float)((std::pow(2, nn) - 1) * delta);
+  const float min_ = sign ? (float)(-max_) : 0.0f;
+  return launch_grad<FixedPointGradOp, true>(dy, x, dx, size, accum, FixedPointGradOp{max_, min_}, as_stream(stream),
+                                             "fixed_point_quantize backward");
+}
+
+int nbla_hip_pow2_quantize_backward_f32(const float *dy, const float *x, float *dx, size_t size, int sign,
+                                        int with_zero, int n, int m, int ste_fine_grained, int accum, void *stream) {
+  if (!(n > 0))
+    return fail(NBLA_HIP_ERR_VALUE, "bit width should be positive.");
+  int nn = sign ? n - 1 : n;
+  nn = with_zero ? nn - 1 : nn;
+  if (!(nn > 0))
+    return fail(NBLA_HIP_ERR_VALUE, "bit width should be positive when considering zero (1bit) and sign (1bit).");
+  if (m > 127 || m < -149)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "2^%d is outside the finite non-zero fp32 range.", m);
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  if (!ste_fine_grained)
+    return launch_grad<PassOp, false>(dy, x, dx, size, accum, PassOp(), as_stream(stream), "quantize backward");
+  uint32_t table[kNumBinades];
+  rc = nbla_hip_cut_table(kCutPow2Round, table);
+  if (rc)
+    return rc;
+  Pow2GradOp op;
+  op.cut = table[m + 149]; // round(log2 a) steps from m to m + 1 at the cut of binade m
+  op.sign = sign;
+  return launch_grad<Pow2GradOp, true>(dy, x, dx, size, accum, op, as_stream(stream), "pow2_quantize backward");
+}
+
+size_t nbla_hip_min_max_quantize_backward_workspace_bytes(const int64_t *xshape, int ndim, const int64_t *qshape) {
+  const RangeGradPlan P = make_range_plan(xshape, ndim, qshape);
+  return P.bounds_bytes + P.partial_bytes;
+}
+
+int nbla_hip_min_max_quantize_backward_f32(const float *dy, const float *x, float *dx, const int64_t *xshape, int ndim,
+                                           const int64_t *qshape, const float *qr_min, const float *qr_max,
+                                           const float *ql_min, const float *ql_max, const float *scale,
+                                           float *g_qr_min, float *g_qr_max, int ste_fine_grained, int x_min_max,
+                                           int ema, int accum_x, int accum_min, int accum_max, void *workspace,
+                                           size_t workspace_bytes, void *stream_) {
+  (void)qr_max;
+  for (int i = 0; i < ndim; ++i)
+    if (qshape[i] != 1 && qshape[i] != xshape[i])
+      return fail(NBLA_HIP_ERR_VALUE, "q tensors must have size 1 or the size of x along every axis (axis %d).", i);
+  const RangeGradPlan P = make_range_plan(xshape, ndim, qshape);
+  if (!P.L.ok)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "q shapes whose kept axes are separated by reduced axes are not supported.");
+  if (workspace_bytes < P.bounds_bytes + P.partial_bytes || !aligned256(workspace))
+    return fail(NBLA_HIP_ERR_MEMORY, "min_max_quantize backward workspace too small or misaligned.");
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  hipStream_t stream = as_stream(stream_);
+  const bool range_grads = !(x_min_max || ema) && (g_qr_min || g_qr_max);
+  float2 *bounds = static_cast<float2 *>(workspace);
+  float2 *partial = reinterpret_cast<float2 *>(static_cast<char *>(workspace) + P.bounds_bytes);
+  if ((dx && ste_fine_grained) || range_grads) {
+    hipLaunchKernelGGL(minmax_bounds, dim3((unsigned)((P.L.K + 63) / 64)), dim3(64), 0, stream, qr_min, ql_min, ql_max,
+                       scale, bounds, P.L.K);
+    NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward bounds");
+  }
+  if (dx) {
+    if (ste_fine_grained) {
+      MinMaxGradOp op{bounds, P.L.K, P.L.R1};
+      rc = launch_grad<MinMaxGradOp, true>(dy, x, dx, (size_t)P.L.total, accum_x, op, stream, "min_max_quantize backward");
+    } else {
+      rc = launch_grad<PassOp, false>(dy, x, dx, (size_t)P.L.total, accum_x, PassOp(), stream, "quantize backward");
+    }
+    if (rc)
+      return rc;
+  }
+  if (range_grads) {
+    hipLaunchKernelGGL(minmax_range_grad_partial, dim3((unsigned)P.nchunks, (unsigned)P.L.K), dim3(kBlock), 0, stream,
+                       dy, x, bounds, partial, P.L.K, P.L.R1, P.tiles_per_row, P.tiles_per_k, P.nchunks);
+    NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward range sums");
+    hipLaunchKernelGGL(minmax_range_grad_final, dim3((unsigned)((P.L.K + 63) / 64)), dim3(64), 0, stream, partial,
+                       P.nchunks, g_qr_min, g_qr_max, accum_min, accum_max, P.L.K);
+    NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward range gradients");
+  }
+  return NBLA_HIP_OK;
+}
+
+} // extern "C"

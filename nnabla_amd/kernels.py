@@ -22,6 +22,8 @@ EXPORTED = (
     "nbla_hip_init", "nbla_hip_last_error", "nbla_hip_version", "nbla_hip_cut_table",
     "nbla_hip_fixed_point_quantize_f32", "nbla_hip_pow2_quantize_f32",
     "nbla_hip_min_max_quantize_workspace_bytes", "nbla_hip_min_max_quantize_f32",
+    "nbla_hip_fixed_point_quantize_backward_f32", "nbla_hip_pow2_quantize_backward_f32",
+    "nbla_hip_min_max_quantize_backward_workspace_bytes", "nbla_hip_min_max_quantize_backward_f32",
     "nbla_hip_packed_bits_bytes", "nbla_hip_split_operand_bytes", "nbla_hip_digit_operand_bytes",
     "nbla_hip_binarize_workspace_bytes", "nbla_hip_binarize_weights_f32", "nbla_hip_split_bf16x3_f32",
     "nbla_hip_split_digits_f32", "nbla_hip_gemm_bits_f32",
@@ -57,6 +59,7 @@ def lib():
         L.nbla_hip_last_error.restype = ctypes.c_char_p
         L.nbla_hip_version.restype = ctypes.c_char_p
         for name in ("nbla_hip_min_max_quantize_workspace_bytes", "nbla_hip_packed_bits_bytes",
+                     "nbla_hip_min_max_quantize_backward_workspace_bytes",
                      "nbla_hip_split_operand_bytes", "nbla_hip_digit_operand_bytes",
                      "nbla_hip_binarize_workspace_bytes",
                      "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_convolution_workspace_bytes",
@@ -138,6 +141,46 @@ def min_max_quantize(x, qr_min, qr_max, ql_min, ql_max, decay=0.999, x_min_max=F
                                               ctypes.c_float(eps), _p(ws), ctypes.c_size_t(ws.numel()),
                                               _stream(stream)))
     return y, scale
+
+
+def _grad_out(dy, dx):
+    import torch
+    return (torch.empty_like(dy), 0) if dx is None else (dx, 1)
+
+
+def fixed_point_quantize_backward(dy, x, sign=True, n=8, delta=2.0 ** -4, ste_fine_grained=True, dx=None,
+                                  stream=None):
+    """dx = STE gradient; a dx passed in is accumulated onto (in place)."""
+    out, accum = _grad_out(dy, dx)
+    check(lib().nbla_hip_fixed_point_quantize_backward_f32(_p(dy), _p(x), _p(out), ctypes.c_size_t(dy.numel()),
+                                                           int(sign), int(n), ctypes.c_float(delta),
+                                                           int(ste_fine_grained), accum, _stream(stream)))
+    return out
+
+
+def pow2_quantize_backward(dy, x, sign=True, with_zero=True, n=8, m=1, ste_fine_grained=True, dx=None, stream=None):
+    out, accum = _grad_out(dy, dx)
+    check(lib().nbla_hip_pow2_quantize_backward_f32(_p(dy), _p(x), _p(out), ctypes.c_size_t(dy.numel()), int(sign),
+                                                    int(with_zero), int(n), int(m), int(ste_fine_grained), accum,
+                                                    _stream(stream)))
+    return out
+
+
+def min_max_quantize_backward(dy, x, qr_min, qr_max, ql_min, ql_max, scale, ste_fine_grained=True, x_min_max=False,
+                              ema=False, dx=None, g_qr_min=None, g_qr_max=None, want_x=True, want_min=True,
+                              want_max=True, stream=None):
+    """Returns (dx, g_qr_min, g_qr_max); gradients passed in are accumulated onto, None where not wanted."""
+    import torch
+    xs, qs = _shape(x.shape), _shape(qr_min.shape)
+    ws = _workspace(lib().nbla_hip_min_max_quantize_backward_workspace_bytes(xs, x.dim(), qs), x)
+    odx, ax = _grad_out(dy, dx) if want_x else (None, 0)
+    omin, amin = _grad_out(qr_min, g_qr_min) if want_min else (None, 0)
+    omax, amax = _grad_out(qr_max, g_qr_max) if want_max else (None, 0)
+    check(lib().nbla_hip_min_max_quantize_backward_f32(
+        _p(dy), _p(x), _p(odx), xs, x.dim(), qs, _p(qr_min), _p(qr_max), _p(ql_min), _p(ql_max), _p(scale), _p(omin),
+        _p(omax), int(ste_fine_grained), int(x_min_max), int(ema), ax, amin, amax, _p(ws),
+        ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return odx, omin, omax
 
 
 def binarize_weights(W, K, N, transposed=False, quantize_zero_to=1.0, want_alpha=True, stream=None):

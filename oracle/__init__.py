@@ -122,6 +122,43 @@ def min_max_quantize(x, qr_min, qr_max, ql_min, ql_max, decay=0.999, x_min_max=F
     return y, qr_min, qr_max, scale
 
 
+def fixed_point_quantize_backward(dy, x, sign=True, n=8, delta=2.0 ** -4, ste_fine_grained=True, dx=None):
+    """dx (accumulated onto the given dx when one is passed), fixed_point_quantize.cpp:69-127."""
+    dy, x = _f32(dy), _f32(x)
+    out = np.zeros_like(x) if dx is None else _f32(dx).copy()
+    _check(lib().orc_fixed_point_quantize_backward(_fp(dy), _fp(x), _fp(out), ctypes.c_long(x.size), int(sign), int(n),
+                                                   ctypes.c_float(delta), int(ste_fine_grained), int(dx is not None)),
+           "fixed_point_quantize_backward")
+    return out
+
+
+def pow2_quantize_backward(dy, x, sign=True, with_zero=True, n=8, m=1, ste_fine_grained=True, dx=None):
+    dy, x = _f32(dy), _f32(x)
+    out = np.zeros_like(x) if dx is None else _f32(dx).copy()
+    _check(lib().orc_pow2_quantize_backward(_fp(dy), _fp(x), _fp(out), ctypes.c_long(x.size), int(sign),
+                                            int(with_zero), int(n), int(m), int(ste_fine_grained),
+                                            int(dx is not None)), "pow2_quantize_backward")
+    return out
+
+
+def min_max_quantize_backward(dy, x, qr_min, qr_max, ql_min, ql_max, scale, ste_fine_grained=True, x_min_max=False,
+                              ema=False, dx=None, g_qr_min=None, g_qr_max=None, want_x=True, want_min=True,
+                              want_max=True):
+    """Returns (dx, g_qr_min, g_qr_max); a gradient passed in is accumulated onto, min_max_quantize.cpp:225-350."""
+    dy, x = _f32(dy), _f32(x)
+    qs = [_f32(q) for q in (qr_min, qr_max, ql_min, ql_max, scale)]
+    odx = (np.zeros_like(x) if dx is None else _f32(dx).copy()) if want_x else None
+    omin = (np.zeros_like(qs[0]) if g_qr_min is None else _f32(g_qr_min).copy()) if want_min else None
+    omax = (np.zeros_like(qs[0]) if g_qr_max is None else _f32(g_qr_max).copy()) if want_max else None
+    nul = ctypes.POINTER(ctypes.c_float)()
+    _check(lib().orc_min_max_quantize_backward(
+        _fp(dy), _fp(x), _fp(odx) if want_x else nul, _longs(x.shape), x.ndim, _longs(qs[0].shape), _fp(qs[0]),
+        _fp(qs[1]), _fp(qs[2]), _fp(qs[3]), _fp(qs[4]), _fp(omin) if want_min else nul,
+        _fp(omax) if want_max else nul, int(ste_fine_grained), int(x_min_max), int(ema), int(dx is not None),
+        int(g_qr_min is not None), int(g_qr_max is not None)), "min_max_quantize_backward")
+    return odx, omin, omax
+
+
 def sign(x, alpha0=1.0):
     x = _f32(x)
     y = np.empty_like(x)

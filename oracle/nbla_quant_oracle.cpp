@@ -510,6 +510,162 @@ int orc_min_max_quantize(const float *x, float *y, const long *xshape, int ndim,
 }
 
 // ---------------------------------------------------------------------------
+// Backward passes of the three quantizers (straight-through estimators).
+// ---------------------------------------------------------------------------
+
+// FixedPointQuantize<T>::backward_impl, fixed_point_quantize.cpp:69-127.
+int orc_fixed_point_quantize_backward(const float *dy, const float *x, float *dx,
+                                      long size, int sign, int n_bits, float delta,
+                                      int ste_fine_grained, int accum) {
+  if (!(n_bits > 0 && delta > 0.))
+    return ORC_ERR_VALUE;
+  const int n = sign ? n_bits - 1 : n_bits;
+  if (!(n > 0))
+    return ORC_ERR_VALUE;
+  const float max_ = (float)((std::pow(2, n) - 1) * delta);
+  const float min_ = sign ? (float)(-max_) : 0.0f;
+  for (long s = 0; s < size; ++s) {
+    if (!ste_fine_grained) { // :69-78
+      if (accum)
+        dx[s] += dy[s];
+      else
+        dx[s] = dy[s];
+    } else if (x[s] > max_) { // :84-99
+      if (!accum)
+        dx[s] = 0.0f;
+    } else if (x[s] < min_) {
+      if (!accum)
+        dx[s] = 0.0f;
+    } else {
+      if (accum)
+        dx[s] += dy[s];
+      else
+        dx[s] = dy[s];
+    }
+  }
+  return ORC_OK;
+}
+
+// Pow2Quantize<T>::backward_impl, pow2_quantize.cpp:84-156.
+int orc_pow2_quantize_backward(const float *dy, const float *x, float *dx, long size,
+                               int sign, int with_zero, int n_bits, int m,
+                               int ste_fine_grained, int accum) {
+  if (!(n_bits > 0))
+    return ORC_ERR_VALUE;
+  int n = sign ? n_bits - 1 : n_bits;
+  n = with_zero ? n - 1 : n;
+  if (!(n > 0))
+    return ORC_ERR_VALUE;
+  const float p_max = (float)std::pow(2., m);
+  for (long s = 0; s < size; ++s) {
+    float c = 1.0f;
+    if (ste_fine_grained) { // :97-125
+      const float x_abs = std::fabs(x[s]);
+      const float q = std::pow(2.0f, std::round(std::log2(x_abs)));
+      if (q > p_max)
+        c = 0.0f;
+      if (!sign)
+        c = (x[s] < 0.0) ? 0.0f : c;
+      if (accum)
+        dx[s] += c * dy[s];
+      else
+        dx[s] = c * dy[s];
+    } else {
+      if (accum)
+        dx[s] += dy[s];
+      else
+        dx[s] = dy[s];
+    }
+  }
+  return ORC_OK;
+}
+
+// MinMaxQuantize<T>::backward_impl, min_max_quantize.cpp:225-350.  qr_min / qr_max are the
+// values the forward pass left, `scale` its scale_sptr_.  dx / g_qr_min / g_qr_max may be
+// null (propagate_down false).  The Sum helper is a plain running sum here; the reference's
+// Eigen reduction order is not restated (results are compared at tolerance).
+int orc_min_max_quantize_backward(const float *dy, const float *x, float *dx,
+                                  const long *xshape, int ndim, const long *qshape,
+                                  const float *qr_min, const float *qr_max,
+                                  const float *ql_min, const float *ql_max,
+                                  const float *scale, float *g_qr_min, float *g_qr_max,
+                                  int ste_fine_grained, int x_min_max, int ema,
+                                  int accum_x, int accum_min, int accum_max) {
+  long total = 1, qsize = 1;
+  for (int i = 0; i < ndim; ++i) {
+    if (qshape[i] != 1 && qshape[i] != xshape[i])
+      return ORC_ERR_VALUE;
+    total *= xshape[i];
+    qsize *= qshape[i];
+  }
+  // nudge_qr_min_max :363-390 with the forward's scale
+  std::vector<float> m_n(qsize), M_n(qsize);
+  for (long i = 0; i < qsize; ++i) {
+    const float zero_point_from_min = ql_min[i] - qr_min[i] / scale[i];
+    float zero_point_nudged;
+    if (zero_point_from_min <= ql_min[i])
+      zero_point_nudged = ql_min[i];
+    else if (zero_point_from_min >= ql_max[i])
+      zero_point_nudged = ql_max[i];
+    else
+      zero_point_nudged = std::round(zero_point_from_min);
+    m_n[i] = (ql_min[i] - zero_point_nudged) * scale[i];
+    M_n[i] = (ql_max[i] - zero_point_nudged) * scale[i];
+  }
+  std::vector<long> qstride(ndim);
+  {
+    long s = 1;
+    for (int i = ndim - 1; i >= 0; --i) {
+      qstride[i] = (qshape[i] == 1) ? 0 : s;
+      s *= qshape[i];
+    }
+  }
+  std::vector<long> qidx(total);
+  for (long o = 0; o < total; ++o) {
+    long rem = o, qi = 0;
+    for (int i = ndim - 1; i >= 0; --i) {
+      qi += (rem % xshape[i]) * qstride[i];
+      rem /= xshape[i];
+    }
+    qidx[o] = qi;
+  }
+  if (dx) { // :259-292
+    for (long o = 0; o < total; ++o) {
+      if (ste_fine_grained) {
+        const float iv0 = (x[o] >= m_n[qidx[o]]) ? 1.0f : 0.0f; // greater_equal
+        const float iv1 = (x[o] <= M_n[qidx[o]]) ? 1.0f : 0.0f; // less_equal
+        float mask = iv0 * iv1;
+        mask = mask * dy[o];
+        dx[o] = accum_x ? mask + dx[o] : mask;
+      } else {
+        dx[o] = accum_x ? dy[o] + dx[o] : dy[o];
+      }
+    }
+  }
+  if (x_min_max || ema) // :294-295
+    return ORC_OK;
+  if (g_qr_min) { // :302-323
+    std::vector<float> acc(qsize, 0.0f);
+    for (long o = 0; o < total; ++o) {
+      const float mask = (x[o] < m_n[qidx[o]]) ? 1.0f : 0.0f;
+      acc[qidx[o]] += mask * dy[o];
+    }
+    for (long i = 0; i < qsize; ++i)
+      g_qr_min[i] = accum_min ? g_qr_min[i] + acc[i] : acc[i];
+  }
+  if (g_qr_max) { // :325-348
+    std::vector<float> acc(qsize, 0.0f);
+    for (long o = 0; o < total; ++o) {
+      const float mask = (x[o] > M_n[qidx[o]]) ? 1.0f : 0.0f;
+      acc[qidx[o]] += mask * dy[o];
+    }
+    for (long i = 0; i < qsize; ++i)
+      g_qr_max[i] = accum_max ? g_qr_max[i] + acc[i] : acc[i];
+  }
+  return ORC_OK;
+}
+
+// ---------------------------------------------------------------------------
 // Sign: include/nbla/function/sign.hpp:48-50
 // ---------------------------------------------------------------------------
 void orc_sign(const float *x, float *y, long size, float alpha0) {

@@ -1,0 +1,101 @@
+"""Pins of the oracle's backward restatements (CPU only): closed forms from the reference text
+(fixed_point_quantize.cpp:69-127, pow2_quantize.cpp:84-156, min_max_quantize.cpp:225-350) written independently in
+numpy, the accumulate/overwrite rules, and the cases the straight-through estimators special-case."""
+import numpy as np
+import pytest
+
+import oracle
+
+
+def _rand(shape, seed, scale=1.0):
+    return (np.random.RandomState(seed).randn(*shape) * scale).astype(np.float32)
+
+
+@pytest.mark.parametrize("sign,n,delta", [(True, 8, 2.0 ** -4), (False, 4, 0.1), (True, 3, 0.25)])
+def test_fixed_point_backward_mask(sign, n, delta):
+    x = _rand((5, 37), 1, 6.0)
+    dy = _rand((5, 37), 2)
+    nn = n - 1 if sign else n
+    hi = np.float32((2 ** nn - 1) * delta)
+    lo = np.float32(-hi) if sign else np.float32(0)
+    x.ravel()[:4] = [hi, lo, np.nextafter(hi, np.float32(np.inf)), np.nextafter(lo, np.float32(-np.inf))]
+    inside = (x <= hi) & (x >= lo)
+    assert np.array_equal(oracle.fixed_point_quantize_backward(dy, x, sign, n, delta, True), np.where(inside, dy, 0))
+    old = _rand((5, 37), 3)
+    # outside the range an accumulated gradient is left untouched; inside dy is added
+    assert np.array_equal(oracle.fixed_point_quantize_backward(dy, x, sign, n, delta, True, dx=old),
+                          np.where(inside, old + dy, old))
+    assert np.array_equal(oracle.fixed_point_quantize_backward(dy, x, sign, n, delta, False), dy)
+    assert np.array_equal(oracle.fixed_point_quantize_backward(dy, x, sign, n, delta, False, dx=old), old + dy)
+
+
+@pytest.mark.parametrize("sign,with_zero,n,m", [(True, True, 4, 1), (False, True, 4, 0), (True, False, 3, -2),
+                                                (False, False, 2, 3)])
+def test_pow2_backward_mask(sign, with_zero, n, m):
+    x = _rand((4, 50), 5, 2.0 ** m)
+    dy = _rand((4, 50), 6)
+    x.ravel()[:6] = [0.0, -0.0, 2.0 ** m, 2.0 ** m * 1.4, 2.0 ** m * 1.5, -(2.0 ** m) * 3]
+    # 2^round(log2|x|) > 2^m  <=>  round(log2|x|) > m; away from the sqrt(2) windows float64 decides it
+    with np.errstate(divide="ignore"):
+        r = np.round(np.log2(np.abs(x.astype(np.float64))))
+    c = np.where(r > m, 0.0, 1.0)
+    if not sign:
+        c = np.where(x < 0, 0.0, c)
+    got = oracle.pow2_quantize_backward(dy, x, sign, with_zero, n, m, True)
+    assert np.array_equal(got, (c * dy).astype(np.float32))
+    old = _rand((4, 50), 7)
+    got = oracle.pow2_quantize_backward(dy, x, sign, with_zero, n, m, True, dx=old)
+    assert np.array_equal(got, old + (c * dy).astype(np.float32))
+    assert np.array_equal(oracle.pow2_quantize_backward(dy, x, sign, with_zero, n, m, False), dy)
+
+
+def test_pow2_backward_product_keeps_ieee_cases():
+    """dx = c * dy is a product: a zero factor turns an infinite dy into NaN and keeps the sign of zero."""
+    x = np.array([100.0, 100.0, -100.0], np.float32)
+    dy = np.array([np.inf, -3.0, 2.0], np.float32)
+    got = oracle.pow2_quantize_backward(dy, x, True, True, 4, 1, True)
+    assert np.isnan(got[0]) and got[1] == 0 and np.signbit(got[1]) and got[2] == 0 and not np.signbit(got[2])
+
+
+@pytest.mark.parametrize("qshape", [(1, 1, 1, 1), (1, 6, 1, 1), (4, 1, 1, 1)])
+@pytest.mark.parametrize("fine", [True, False])
+def test_min_max_backward(qshape, fine):
+    x = _rand((4, 6, 5, 3), 11, 3.0)
+    dy = _rand((4, 6, 5, 3), 12)
+    qr_min = np.full(qshape, -2.0, np.float32) + _rand(qshape, 13, 0.1)
+    qr_max = np.full(qshape, 2.5, np.float32) + _rand(qshape, 14, 0.1)
+    ql_min = np.zeros(qshape, np.float32)
+    ql_max = np.full(qshape, 255.0, np.float32)
+    _, qmn, qmx, scale = oracle.min_max_quantize(x, qr_min, qr_max, ql_min, ql_max, 0.999, False, False, 0.01)
+    # nudged range in float64 (exact enough away from ties of the zero point)
+    zp = np.clip(np.round(ql_min - qmn.astype(np.float64) / scale), ql_min, ql_max)
+    m_n = ((ql_min - zp) * scale).astype(np.float32)
+    M_n = ((ql_max - zp) * scale).astype(np.float32)
+    dx, gmin, gmax = oracle.min_max_quantize_backward(dy, x, qmn, qmx, ql_min, ql_max, scale, fine, False, False)
+    inside = (x >= m_n) & (x <= M_n)
+    assert np.array_equal(dx, np.where(inside, dy, 0).astype(np.float32) if fine else dy)
+    axes = tuple(i for i in range(4) if qshape[i] == 1)
+    ref_min = np.where(x < m_n, dy, 0).astype(np.float64).sum(axis=axes, keepdims=True)
+    ref_max = np.where(x > M_n, dy, 0).astype(np.float64).sum(axis=axes, keepdims=True)
+    np.testing.assert_allclose(gmin, ref_min, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(gmax, ref_max, rtol=1e-5, atol=1e-5)
+    # accumulation onto given gradients
+    odx, omin, omax = _rand(x.shape, 15), _rand(qshape, 16), _rand(qshape, 17)
+    dx2, gmin2, gmax2 = oracle.min_max_quantize_backward(dy, x, qmn, qmx, ql_min, ql_max, scale, fine, False, False,
+                                                         dx=odx, g_qr_min=omin, g_qr_max=omax)
+    assert np.array_equal(dx2, dx + odx)
+    np.testing.assert_allclose(gmin2, omin + gmin, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(gmax2, omax + gmax, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("x_min_max,ema", [(True, False), (False, True), (True, True)])
+def test_min_max_backward_no_range_gradient_with_statistics(x_min_max, ema):
+    """min_max_quantize.cpp:294-295: with x_min_max or ema the range parameters receive no gradient."""
+    x = _rand((2, 3, 4, 4), 21)
+    dy = _rand((2, 3, 4, 4), 22)
+    q = lambda v: np.full((1, 1, 1, 1), v, np.float32)
+    _, qmn, qmx, scale = oracle.min_max_quantize(x, q(-1), q(1), q(0), q(255), 0.999, x_min_max, ema, 0.01)
+    sentinel = q(7.0)
+    dx, gmin, gmax = oracle.min_max_quantize_backward(dy, x, qmn, qmx, q(0), q(255), scale, True, x_min_max, ema,
+                                                      g_qr_min=sentinel, g_qr_max=sentinel)
+    assert gmin == 7.0 and gmax == 7.0 and dx.shape == x.shape
