@@ -261,6 +261,18 @@ NBLA_API int nblac_function_backward(void *f, void **inputs, int ni, void **outp
                                                  vector<bool>(ni, true), vector<bool>(ni, false));
   });
 }
+// flags[i] bit 0: propagate_down, bit 1: accum, one byte per input
+NBLA_API int nblac_function_backward_flags(void *f, void **inputs, int ni, void **outputs, int no,
+                                           const unsigned char *flags) {
+  return guarded([&] {
+    vector<bool> prop(ni), accum(ni);
+    for (int i = 0; i < ni; ++i) {
+      prop[i] = flags[i] & 1;
+      accum[i] = (flags[i] >> 1) & 1;
+    }
+    static_cast<FuncHandle *>(f)->func->backward(to_variables(inputs, ni), to_variables(outputs, no), prop, accum);
+  });
+}
 NBLA_API void *nblac_function_copy(void *f) {
   FuncHandle *h = nullptr;
   guarded([&] { h = new FuncHandle{static_cast<FuncHandle *>(f)->func->copy()}; });

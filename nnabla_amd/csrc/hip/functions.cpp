@@ -47,6 +47,64 @@ template <typename T> void MinMaxQuantizeHip<T>::forward_impl(const Variables &i
                                               this->eps_, ws.pointer(), ws.bytes(), nullptr));
 }
 
+// fixed_point_quantize.cpp:103-127
+template <typename T>
+void FixedPointQuantizeHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                             const vector<bool> &propagate_down, const vector<bool> &accum) {
+  if (!propagate_down[0])
+    return;
+  hip_set_device(this->ctx_);
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  T *dx = inputs[0]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[0]);
+  const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_fixed_point_quantize_backward_f32(dy, x, dx, (size_t)inputs[0]->size(), this->sign_, this->n_,
+                                                           this->delta_, this->ste_fine_grained_, accum[0], nullptr));
+}
+
+// pow2_quantize.cpp:127-156
+template <typename T>
+void Pow2QuantizeHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                       const vector<bool> &propagate_down, const vector<bool> &accum) {
+  if (!propagate_down[0])
+    return;
+  hip_set_device(this->ctx_);
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  T *dx = inputs[0]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[0]);
+  const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_pow2_quantize_backward_f32(dy, x, dx, (size_t)inputs[0]->size(), this->sign_,
+                                                    this->with_zero_, this->n_, this->m_, this->ste_fine_grained_,
+                                                    accum[0], nullptr));
+}
+
+// min_max_quantize.cpp:225-350
+template <typename T>
+void MinMaxQuantizeHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                         const vector<bool> &propagate_down, const vector<bool> &accum) {
+  NBLA_CHECK(!(propagate_down[3] || propagate_down[4]), error_code::value,
+             "Backward to x(inputs[0]), qr_min(inputs[1]), and/or qr_max(inputs[2])are only allowed.");
+  if (!(propagate_down[0] || propagate_down[1] || propagate_down[2]))
+    return;
+  hip_set_device(this->ctx_);
+  const vector<int64_t> xshape = to_i64(inputs[0]->shape()), qshape = to_i64(inputs[1]->shape());
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const T *qr_min = inputs[1]->get_data_pointer<T>(this->ctx_);
+  const T *qr_max = inputs[2]->get_data_pointer<T>(this->ctx_);
+  const T *ql_min = inputs[3]->get_data_pointer<T>(this->ctx_);
+  const T *ql_max = inputs[4]->get_data_pointer<T>(this->ctx_);
+  const T *scale = this->scale_sptr_->template get_data_pointer<T>(this->ctx_);
+  const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
+  const bool range = !(this->x_min_max_ || this->ema_);
+  T *dx = propagate_down[0] ? inputs[0]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[0]) : nullptr;
+  T *g_min = (range && propagate_down[1]) ? inputs[1]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[1]) : nullptr;
+  T *g_max = (range && propagate_down[2]) ? inputs[2]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[2]) : nullptr;
+  HipWorkspace ws(nbla_hip_min_max_quantize_backward_workspace_bytes(xshape.data(), (int)xshape.size(), qshape.data()),
+                  this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_min_max_quantize_backward_f32(
+      dy, x, dx, xshape.data(), (int)xshape.size(), qshape.data(), qr_min, qr_max, ql_min, ql_max, scale, g_min, g_max,
+      this->ste_fine_grained_, this->x_min_max_, this->ema_, accum[0], accum[1], accum[2], ws.pointer(), ws.bytes(),
+      nullptr));
+}
+
 // ------------------------------------------------------------- binary affine
 template <typename T>
 void BinaryWeightAffineHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {

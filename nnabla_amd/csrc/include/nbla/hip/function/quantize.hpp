@@ -1,5 +1,5 @@
 // "hip:float" implementations of the elementwise quantizers.  Each class reuses the argument checks and shape
-// inference of the generic class and replaces forward_impl by one call into the kernel library.
+// inference of the generic class and replaces forward_impl / backward_impl by calls into the kernel library.
 #ifndef NBLA_HIP_FUNCTION_QUANTIZE_HPP_
 #define NBLA_HIP_FUNCTION_QUANTIZE_HPP_
 
@@ -18,6 +18,8 @@ public:
 
 protected:
   virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+  virtual void backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                             const vector<bool> &accum);
 };
 
 template <typename T> class Pow2QuantizeHip : public Pow2Quantize<T> {
@@ -28,6 +30,8 @@ public:
 
 protected:
   virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+  virtual void backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                             const vector<bool> &accum);
 };
 
 template <typename T> class MinMaxQuantizeHip : public MinMaxQuantize<T> {
@@ -38,6 +42,8 @@ public:
 
 protected:
   virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+  virtual void backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                             const vector<bool> &accum);
 };
 
 } // namespace nbla

@@ -54,9 +54,15 @@ class Function(object):
         _capi.check(_capi.lib().nblac_function_recompute(self._h, _handles(inputs), len(inputs), _handles(outputs),
                                                          len(outputs)))
 
-    def backward(self, inputs, outputs):
-        _capi.check(_capi.lib().nblac_function_backward(self._h, _handles(inputs), len(inputs), _handles(outputs),
-                                                        len(outputs)))
+    def backward(self, inputs, outputs, propagate_down=None, accum=None):
+        """Function::backward: gradients of the outputs (their .g) -> gradients of the inputs flagged in
+        propagate_down, added to the existing ones where accum is set."""
+        n = len(inputs)
+        prop = [True] * n if propagate_down is None else list(propagate_down)
+        acc = [False] * n if accum is None else list(accum)
+        flags = (ctypes.c_ubyte * max(1, n))(*[(1 if prop[i] else 0) | (2 if acc[i] else 0) for i in range(n)])
+        _capi.check(_capi.lib().nblac_function_backward_flags(self._h, _handles(inputs), n, _handles(outputs),
+                                                              len(outputs), flags))
 
     def __call__(self, *inputs, **kw):
         """Connects the function to its inputs: creates outputs, runs setup (shape inference), executes at once in
@@ -102,3 +108,6 @@ class FunctionNode(object):
 
     def recompute(self):
         self.function.recompute(self.inputs, self.outputs)
+
+    def backward(self, propagate_down, accum):
+        self.function.backward(self.inputs, self.outputs, propagate_down, accum)

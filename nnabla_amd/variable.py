@@ -144,6 +144,12 @@ class Variable(object):
     def fill(self, v):
         _capi.check(_capi.lib().nblac_variable_fill(self._h, 0, ctypes.c_double(float(v))))
 
+    def _fill(self, which, v):
+        _capi.check(_capi.lib().nblac_variable_fill(self._h, which, ctypes.c_double(float(v))))
+
+    def zero_grad(self):
+        self._fill(1, 0.0)
+
     @property
     def head_array_class(self):
         buf = ctypes.create_string_buffer(64)
@@ -181,7 +187,42 @@ class Variable(object):
             node.forward()
 
     def backward(self, grad=1, clear_buffer=False):
-        raise _capi.NblaNotImplementedError("backward passes are not part of this build (forward-only hot path).")
+        """Back-propagates from this variable (CgVariable::backward): its gradient is filled with `grad` (a scalar or an
+        array; None keeps the current .g), then every function it depends on runs its backward in reverse order.
+        Gradients of leaf variables are accumulated onto (zero them beforehand, as with nnabla); intermediate
+        gradients are overwritten by their first contribution and accumulated by later ones."""
+        if grad is not None:
+            if np.isscalar(grad):
+                self._fill(1, float(grad))
+            else:
+                self.g = np.asarray(grad)
+        done, order = set(), []
+
+        def visit(v):
+            node = v.parent
+            if node is None or id(node) in done:
+                return
+            done.add(id(node))
+            for i in node.inputs:
+                visit(i)
+            order.append(node)
+        import sys
+        limit = sys.getrecursionlimit()
+        sys.setrecursionlimit(max(limit, 10000))
+        try:
+            visit(self)
+        finally:
+            sys.setrecursionlimit(limit)
+        written = set()
+        for node in reversed(order):
+            if not any(i.need_grad for i in node.inputs):
+                continue
+            prop = [bool(i.need_grad) for i in node.inputs]
+            accum = [(i.parent is None) or (id(i) in written) for i in node.inputs]
+            node.backward(prop, accum)
+            for i, p in zip(node.inputs, prop):
+                if p:
+                    written.add(id(i))
 
     def get_unlinked_variable(self, need_grad=None):
         v = self.reshape(self.shape, unlink=True)

@@ -268,3 +268,53 @@ def test_config5_quantized_mlp_graph(ctx):
     print("config5: per-layer GEMM max rel err %.2e; end-to-end std metric %.2e, max-norm %.2e, rows touched by a "
           "quantizer tie flip %.1f%%" % (worst_gemm, std_metric, max_metric, 100 * flipped_rows))
     assert std_metric <= 2e-3 and max_metric <= 2e-2
+
+
+# ------------------------------------------------------------------ backward
+def test_quantizer_backward_through_the_registry(ctx):
+    """F.* forward, Variable.backward(): the hip:float classes' backward_impl against the oracle, including the
+    accumulation of leaf gradients and propagate_down."""
+    rng = np.random.RandomState(5)
+    x = rng.randn(6, 50).astype(np.float32) * 4
+    gy = rng.randn(6, 50).astype(np.float32)
+    if True:
+        v = nn.Variable.from_numpy_array(x, need_grad=True)
+        v.zero_grad()
+        y = F.fixed_point_quantize(v, True, 4, 0.5, True)
+        y.forward()
+        y.backward(gy)
+        ref = oracle.fixed_point_quantize_backward(gy, x, True, 4, 0.5, True)
+        assert bits_equal(v.g, ref)
+        y.backward(gy)                       # leaf gradients accumulate
+        assert bits_equal(v.g, oracle.fixed_point_quantize_backward(gy, x, True, 4, 0.5, True, dx=ref))
+
+        w = nn.Variable.from_numpy_array(x, need_grad=True)
+        w.zero_grad()
+        z = F.pow2_quantize(w, True, True, 4, 1, True)
+        z.forward()
+        z.backward(gy)
+        # the leaf gradient was zero and is accumulated onto: 0 + (-0) = +0
+        assert bits_equal(w.g, oracle.pow2_quantize_backward(gy, x, True, True, 4, 1, True, dx=np.zeros_like(x)))
+
+
+def test_min_max_quantize_backward_through_the_registry(ctx):
+    rng = np.random.RandomState(6)
+    x = rng.randn(4, 3, 8, 8).astype(np.float32) * 3
+    gy = rng.randn(4, 3, 8, 8).astype(np.float32)
+    q = lambda v: np.full((1, 3, 1, 1), v, np.float32)
+    if True:
+        vx = nn.Variable.from_numpy_array(x, need_grad=True)
+        vmin = nn.Variable.from_numpy_array(q(-2.0), need_grad=True)
+        vmax = nn.Variable.from_numpy_array(q(2.0), need_grad=True)
+        vlmin, vlmax = nn.Variable.from_numpy_array(q(0.0)), nn.Variable.from_numpy_array(q(255.0))
+        for v in (vx, vmin, vmax):
+            v.zero_grad()
+        y = F.min_max_quantize(vx, vmin, vmax, vlmin, vlmax, 0.999, False, False, True, 0.01)
+        y.forward()
+        y.backward(gy)
+        _, qmn, qmx, scale = oracle.min_max_quantize(x, q(-2.0), q(2.0), q(0.0), q(255.0), 0.999, False, False, 0.01)
+        rdx, rmin, rmax = oracle.min_max_quantize_backward(gy, x, qmn, qmx, q(0.0), q(255.0), scale, True, False, False,
+                                                           dx=np.zeros_like(x))
+        assert bits_equal(vx.g, rdx)
+        np.testing.assert_allclose(vmin.g, rmin, rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(vmax.g, rmax, rtol=1e-5, atol=1e-5)
