@@ -193,6 +193,13 @@ int nbla_hip_split_bf16x3_f32(const float *x, int64_t ldx, void *xsplit,
 int nbla_hip_split_digits_f32(const float *x, int64_t ldx, void *xdigits,
                               int64_t M, int64_t K, void *stream);
 
+/* Same, for the matrix x[m,k] * colscale[k] (one rounded fp32 product per
+ * element; colscale may be NULL).  Used by the backward pass, where the
+ * gradient is scaled by alpha before it meets the transposed binary weights. */
+int nbla_hip_split_digits_scaled_f32(const float *x, int64_t ldx,
+                                     const float *colscale, void *xdigits,
+                                     int64_t M, int64_t K, void *stream);
+
 /* y[m, n] = (sum_k x[m,k] * (+-1)[k,n]) * alpha[n] + bias[n]
  * with x given as the digit operand and the weights as packed bits; alpha and
  * bias may be NULL.  The sum is accumulated exactly in int32 on the int8 MFMA
@@ -227,6 +234,40 @@ int nbla_hip_binary_weight_affine_f32(const float *x, const float *W,
                                       int64_t K, int64_t N,
                                       float quantize_zero_to, void *workspace,
                                       size_t workspace_bytes, void *stream);
+
+size_t nbla_hip_affine_backward_workspace_bytes(int64_t M, int64_t K, int64_t N);
+
+/* Backward of BinaryWeightAffine (alpha != NULL) / BinaryConnectAffine
+ * (alpha == NULL): with Ws[k,n] = Sign(W)[k,n] * alpha[n] (or Sign(W)),
+ *   dx[M,K] (+)= dy . Ws^T      dW[K,N] (+)= x^T . dy      db[N] (+)= sum_m dy
+ * The weight gradient passes straight through the binarisation (Sign backward
+ * is the identity, sign.hpp:48-50).  Replaces
+ * BinaryWeightAffine<float>::backward_impl, binary_weight_affine.cpp:124-146,
+ * BinaryConnectAffine<float>::backward_impl, binary_connect_affine.cpp:73-92
+ * and the Affine backward they call, affine.cpp:98-140.  dx runs on the
+ * bit-weight product (W is binarised again into its transposed packing); Wb
+ * (the forward's fp32 signs) is only read when quantize_zero_to is neither +1
+ * nor -1 and W holds exact zeros.  dx, dW, db may be NULL (not propagated);
+ * accum_* != 0 adds to the existing gradient. */
+int nbla_hip_binary_affine_backward_f32(const float *dy, const float *x,
+                                        const float *W, const float *Wb,
+                                        const float *alpha, float *dx,
+                                        float *dW, float *db, int64_t M,
+                                        int64_t K, int64_t N,
+                                        float quantize_zero_to, int accum_x,
+                                        int accum_w, int accum_b,
+                                        void *workspace, size_t workspace_bytes,
+                                        void *stream);
+
+/* Backward of Affine with real-valued weights (the product inside INQAffine):
+ *   dx (+)= dy . W^T      dW (+)= x^T . dy      db (+)= sum_m dy
+ * Replaces Affine<float>::backward_impl, affine.cpp:98-140, as called by
+ * INQAffine<float,int>::backward_impl, inq_affine.cpp:218-232. */
+int nbla_hip_affine_backward_f32(const float *dy, const float *x, const float *W,
+                                 float *dx, float *dW, float *db, int64_t M,
+                                 int64_t K, int64_t N, int accum_x, int accum_w,
+                                 int accum_b, void *workspace,
+                                 size_t workspace_bytes, void *stream);
 
 /* BinaryConnectAffine forward (no alpha).  Replaces
  * BinaryConnectAffine<float>::forward_impl,
@@ -369,6 +410,10 @@ int nbla_hip_cast(const void *src, int src_dtype, void *dst, int dst_dtype,
 /* y = max(0, x).  Replaces ReLU<float>::forward_impl,
  * src/nbla/function/generic/relu.cpp (std::max(T(0), x)). */
 int nbla_hip_relu_f32(const float *x, float *y, size_t size, void *stream);
+/* dx (+)= (y > 0 ? dy : 0) with y the forward output.  Replaces
+ * ReLU<float>::backward_impl, src/nbla/function/generic/relu.cpp:41-66. */
+int nbla_hip_relu_backward_f32(const float *dy, const float *y, float *dx,
+                               size_t size, int accum, void *stream);
 
 #ifdef __cplusplus
 }

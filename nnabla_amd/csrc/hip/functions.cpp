@@ -135,6 +135,57 @@ void BinaryConnectAffineHip<T>::forward_impl(const Variables &inputs, const Vari
                                                    ws.pointer(), ws.bytes(), nullptr));
 }
 
+namespace {
+// Shared body of the affine backward passes: `bias_index` is the position of the bias among the inputs (or -1).
+template <typename T, typename Call>
+void affine_backward_common(const Context &ctx, const AffineShapes &s, const Variables &inputs, const Variables &outputs,
+                            const vector<bool> &propagate_down, const vector<bool> &accum, int bias_index, Call call) {
+  const bool has_bias = bias_index >= 0 && (int)inputs.size() > bias_index;
+  const bool pb = has_bias && propagate_down[bias_index];
+  if (!(propagate_down[0] || propagate_down[1] || pb))
+    return;
+  hip_set_device(ctx);
+  const T *x = inputs[0]->get_data_pointer<T>(ctx);
+  const T *dy = outputs[0]->get_grad_pointer<T>(ctx);
+  T *dx = propagate_down[0] ? inputs[0]->cast_grad_and_get_pointer<T>(ctx, !accum[0]) : nullptr;
+  T *dw = propagate_down[1] ? inputs[1]->cast_grad_and_get_pointer<T>(ctx, !accum[1]) : nullptr;
+  T *db = pb ? inputs[bias_index]->cast_grad_and_get_pointer<T>(ctx, !accum[bias_index]) : nullptr;
+  HipWorkspace ws(nbla_hip_affine_backward_workspace_bytes(s.i_row, s.i_col, s.w_col), ctx);
+  call(dy, x, dx, dw, db, (int)accum[0], (int)accum[1], has_bias ? (int)accum[bias_index] : 0, ws);
+}
+} // namespace
+
+// binary_weight_affine.cpp:124-146
+template <typename T>
+void BinaryWeightAffineHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                             const vector<bool> &propagate_down, const vector<bool> &accum) {
+  const AffineShapes &s = this->shapes_;
+  affine_backward_common<T>(this->ctx_, s, inputs, outputs, propagate_down, accum, 4,
+                            [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
+                              const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
+                              const T *wb = inputs[2]->get_data_pointer<T>(this->ctx_);
+                              const T *alpha = inputs[3]->get_data_pointer<T>(this->ctx_);
+                              NBLA_HIP_CALL(nbla_hip_binary_affine_backward_f32(
+                                  dy, x, w, wb, alpha, dx, dw, db, s.i_row, s.i_col, s.w_col, this->quantize_zero_to_,
+                                  ax, aw, ab, ws.pointer(), ws.bytes(), nullptr));
+                            });
+}
+
+// binary_connect_affine.cpp:73-92
+template <typename T>
+void BinaryConnectAffineHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                              const vector<bool> &propagate_down, const vector<bool> &accum) {
+  const AffineShapes &s = this->shapes_;
+  affine_backward_common<T>(this->ctx_, s, inputs, outputs, propagate_down, accum, 3,
+                            [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
+                              const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
+                              const T *wb = inputs[2]->get_data_pointer<T>(this->ctx_);
+                              NBLA_HIP_CALL(nbla_hip_binary_affine_backward_f32(
+                                  dy, x, w, wb, nullptr, dx, dw, db, s.i_row, s.i_col, s.w_col,
+                                  this->quantize_zero_to_, ax, aw, ab, ws.pointer(), ws.bytes(), nullptr));
+                            });
+}
+
 // -------------------------------------------------------- binary convolution
 template <typename T>
 void BinaryWeightConvolutionHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
@@ -252,6 +303,45 @@ template <typename T> void AffineHip<T>::forward_impl(const Variables &inputs, c
   const T *b = inputs.size() == 3 ? inputs[2]->get_data_pointer<T>(this->ctx_) : nullptr;
   T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
   NBLA_HIP_CALL(nbla_hip_affine_f32(x, w, b, y, s.i_row, s.i_col, s.w_col, nullptr));
+}
+
+// inq_affine.cpp:218-232: Affine backward with the (quantized) weights
+template <typename T, typename T1>
+void INQAffineHip<T, T1>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                        const vector<bool> &propagate_down, const vector<bool> &accum) {
+  const AffineShapes &s = this->shapes_;
+  affine_backward_common<T>(this->ctx_, s, inputs, outputs, propagate_down, accum, 3,
+                            [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
+                              const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
+                              NBLA_HIP_CALL(nbla_hip_affine_backward_f32(dy, x, w, dx, dw, db, s.i_row, s.i_col, s.w_col,
+                                                                         ax, aw, ab, ws.pointer(), ws.bytes(), nullptr));
+                            });
+}
+
+// affine.cpp:98-140
+template <typename T>
+void AffineHip<T>::backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                                 const vector<bool> &accum) {
+  const AffineShapes &s = this->shapes_;
+  affine_backward_common<T>(this->ctx_, s, inputs, outputs, propagate_down, accum, 2,
+                            [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
+                              const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
+                              NBLA_HIP_CALL(nbla_hip_affine_backward_f32(dy, x, w, dx, dw, db, s.i_row, s.i_col, s.w_col,
+                                                                         ax, aw, ab, ws.pointer(), ws.bytes(), nullptr));
+                            });
+}
+
+// relu.cpp:51-66
+template <typename T>
+void ReLUHip<T>::backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                               const vector<bool> &accum) {
+  if (!propagate_down[0])
+    return;
+  hip_set_device(this->ctx_);
+  const T *y = outputs[0]->get_data_pointer<T>(this->ctx_);
+  T *dx = inputs[0]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[0]);
+  const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_relu_backward_f32(dy, y, dx, (size_t)inputs[0]->size(), accum[0], nullptr));
 }
 
 template <typename T> void ReLUHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {

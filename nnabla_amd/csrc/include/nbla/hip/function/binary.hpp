@@ -18,6 +18,8 @@ public:
 
 protected:
   virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+  virtual void backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                             const vector<bool> &accum);
 };
 
 template <typename T> class BinaryConnectAffineHip : public BinaryConnectAffine<T> {
@@ -28,6 +30,8 @@ public:
 
 protected:
   virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+  virtual void backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                             const vector<bool> &accum);
 };
 
 template <typename T> class BinaryWeightConvolutionHip : public BinaryWeightConvolution<T> {

@@ -20,6 +20,8 @@ public:
 protected:
   virtual void forward_impl(const Variables &inputs, const Variables &outputs);
   virtual void recompute_impl(const Variables &inputs, const Variables &outputs);
+  virtual void backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                             const vector<bool> &accum);
   void run(const Variables &inputs, const Variables &outputs, int step);
 };
 
@@ -45,6 +47,8 @@ public:
 
 protected:
   virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+  virtual void backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                             const vector<bool> &accum);
 };
 
 template <typename T> class ReLUHip : public ReLU<T> {
@@ -54,6 +58,8 @@ public:
 
 protected:
   virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+  virtual void backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                             const vector<bool> &accum);
 };
 
 } // namespace nbla

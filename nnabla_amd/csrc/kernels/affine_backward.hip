@@ -1,0 +1,233 @@
+// Backward passes of the affine products: BinaryWeightAffine / BinaryConnectAffine (gradient w.r.t. x on the
+// bit-weight product) and Affine with real-valued weights (INQAffine), plus the bias gradient.
+#include "common.hpp"
+#include "gemm_layout.hpp"
+#include "internal.hpp"
+
+namespace nbla_hip {
+namespace {
+
+constexpr int kRows = 256; // rows of dy per partial column sum
+
+// partial[s][n] = sum of dy[m][n] over the rows m of slice s, in row order; consecutive threads are consecutive columns.
+__global__ __launch_bounds__(256) void column_sum_partial(const float *__restrict__ dy, float *__restrict__ partial,
+                                                          int64_t M, int64_t N) {
+  const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (n >= N)
+    return;
+  const int64_t m0 = (int64_t)blockIdx.y * kRows, m1 = (m0 + kRows < M) ? m0 + kRows : M;
+  float acc = 0.0f;
+  for (int64_t m = m0; m < m1; ++m)
+    acc += dy[m * N + n];
+  partial[(int64_t)blockIdx.y * N + n] = acc;
+}
+
+__global__ __launch_bounds__(256) void column_sum_final(const float *__restrict__ partial, float *__restrict__ db,
+                                                        int64_t slices, int64_t N, int accumulate) {
+  const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (n >= N)
+    return;
+  float acc = 0.0f;
+  for (int64_t s = 0; s < slices; ++s)
+    acc += partial[s * N + n];
+  db[n] = accumulate ? db[n] + acc : acc;
+}
+
+// out[m][n] = dy[m][n] * alpha[n]  (general path only)
+__global__ __launch_bounds__(256) void scale_columns(const float *__restrict__ dy, const float *__restrict__ alpha,
+                                                     float *__restrict__ out, int64_t total, int64_t N) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256)
+    out[i] = dy[i] * alpha[i % N];
+}
+
+struct BackwardPlan {
+  size_t bits_off, digits_off, prep_off, count_off, a_planes_off, b_planes_off, flag_off, sums_off, scaled_off, total;
+};
+
+// One layout for all three backward entry points (the regions a call does not use are simply left alone).
+BackwardPlan plan_backward(int64_t M, int64_t K, int64_t N) {
+  BackwardPlan p;
+  size_t off = 0;
+  p.bits_off = off; // packed Sign(W) with the roles of k and n exchanged
+  off += round_up(nbla_hip_packed_bits_bytes(N, K), 256);
+  p.digits_off = off; // digit operand of dy (* alpha), M x N
+  off += round_up(nbla_hip_digit_operand_bytes(M, N), 256);
+  p.prep_off = off;
+  off += round_up(nbla_hip_binarize_workspace_bytes(N, K), 256);
+  p.count_off = off;
+  off += 256;
+  // bf16 planes: the larger of (x^T, dy) for dW and (dy, W^T) for dx
+  const size_t a1 = nbla_hip_split_operand_bytes(K, M), b1 = nbla_hip_split_operand_bytes(N, M);
+  const size_t a2 = nbla_hip_split_operand_bytes(M, N), b2 = nbla_hip_split_operand_bytes(K, N);
+  p.a_planes_off = off;
+  off += round_up(a1 > a2 ? a1 : a2, 256);
+  p.b_planes_off = off;
+  off += round_up(b1 > b2 ? b1 : b2, 256);
+  p.flag_off = off;
+  off += 256;
+  p.sums_off = off;
+  off += round_up(column_sums_workspace_bytes(M, N), 256);
+  p.scaled_off = off; // dy * alpha in fp32, general path only
+  off += round_up((size_t)M * N * sizeof(float), 256);
+  p.total = off;
+  return p;
+}
+
+// dW[K, N] (+)= x^T . dy on the plane x plane product (both factors are real numbers)
+int grad_weights(const float *x, const float *dy, float *dW, int64_t M, int64_t K, int64_t N, bool accumulate,
+                 char *base, const BackwardPlan &p, hipStream_t stream) {
+  int *flag = reinterpret_cast<int *>(base + p.flag_off);
+  // x^T as the row operand: rows k, contraction m.  The "weight plane" splitter produces exactly that layout.
+  int dummy_rc = launch_split_weights(x, base + p.a_planes_off, flag, M, K, false, stream);
+  if (dummy_rc)
+    return dummy_rc;
+  int rc = launch_split_weights(dy, base + p.b_planes_off, flag, M, N, false, stream);
+  if (rc)
+    return rc;
+  // the flag now tells whether dy needs its lower planes
+  return launch_gemm_planes(base + p.a_planes_off, base + p.b_planes_off, flag, nullptr, nullptr, dW, K, M, N, 1, N, 1,
+                            stream, accumulate);
+}
+
+// dx[M, K] (+)= dy' . W^T with real-valued weights, dy' [M, N]
+int grad_input_planes(const float *dyp, const float *W, float *dx, int64_t M, int64_t K, int64_t N, bool accumulate,
+                      char *base, const BackwardPlan &p, hipStream_t stream) {
+  int *flag = reinterpret_cast<int *>(base + p.flag_off);
+  int rc = nbla_hip_split_bf16x3_f32(dyp, N, base + p.a_planes_off, M, N, stream);
+  if (rc)
+    return rc;
+  // W stored [K, N] = [output column of dx][contraction]: the transposed weight layout
+  rc = launch_split_weights(W, base + p.b_planes_off, flag, N, K, true, stream);
+  if (rc)
+    return rc;
+  return launch_gemm_planes(base + p.a_planes_off, base + p.b_planes_off, flag, nullptr, nullptr, dx, M, N, K, 1, K, 1,
+                            stream, accumulate);
+}
+
+int check_args(int64_t M, int64_t K, int64_t N, void *workspace, size_t workspace_bytes, const BackwardPlan &p) {
+  if (M <= 0 || K <= 0 || N <= 0)
+    return fail(NBLA_HIP_ERR_VALUE, "invalid affine shape (M=%lld, K=%lld, N=%lld).", (long long)M, (long long)K,
+                (long long)N);
+  if (workspace_bytes < p.total || !aligned256(workspace))
+    return fail(NBLA_HIP_ERR_MEMORY, "affine backward workspace too small (%zu < %zu) or misaligned.", workspace_bytes,
+                p.total);
+  return ensure_init();
+}
+
+} // namespace
+
+size_t column_sums_workspace_bytes(int64_t M, int64_t N) { return (size_t)ceil_div(M, kRows) * N * sizeof(float); }
+
+int launch_column_sums(const float *dy, float *db, int64_t M, int64_t N, bool accumulate, void *partial,
+                       hipStream_t stream) {
+  const int64_t slices = ceil_div(M, kRows);
+  hipLaunchKernelGGL(column_sum_partial, dim3((unsigned)ceil_div(N, 256), (unsigned)slices), dim3(256), 0, stream, dy,
+                     static_cast<float *>(partial), M, N);
+  NBLA_HIP_LAUNCH_CHECK("column_sum_partial");
+  hipLaunchKernelGGL(column_sum_final, dim3((unsigned)ceil_div(N, 256)), dim3(256), 0, stream,
+                     static_cast<const float *>(partial), db, slices, N, accumulate ? 1 : 0);
+  NBLA_HIP_LAUNCH_CHECK("column_sum_final");
+  return NBLA_HIP_OK;
+}
+
+} // namespace nbla_hip
+
+using namespace nbla_hip;
+
+extern "C" {
+
+size_t nbla_hip_affine_backward_workspace_bytes(int64_t M, int64_t K, int64_t N) {
+  if (M <= 0 || K <= 0 || N <= 0)
+    return 0;
+  return plan_backward(M, K, N).total;
+}
+
+int nbla_hip_binary_affine_backward_f32(const float *dy, const float *x, const float *W, const float *Wb,
+                                        const float *alpha, float *dx, float *dW, float *db, int64_t M, int64_t K,
+                                        int64_t N, float quantize_zero_to, int accum_x, int accum_w, int accum_b,
+                                        void *workspace, size_t workspace_bytes, void *stream_) {
+  const BackwardPlan p = plan_backward(M, K, N);
+  int rc = check_args(M, K, N, workspace, workspace_bytes, p);
+  if (rc)
+    return rc;
+  hipStream_t stream = as_stream(stream_);
+  char *base = static_cast<char *>(workspace);
+  if (dx) {
+    const bool representable = (quantize_zero_to == 1.0f || quantize_zero_to == -1.0f);
+    uint32_t *bits = reinterpret_cast<uint32_t *>(base + p.bits_off);
+    int *count = reinterpret_cast<int *>(base + p.count_off);
+    // Sign(W) packed for the contraction over n: W is stored [K, N] = [output column of dx][contraction]
+    rc = nbla_hip_binarize_weights_f32(W, nullptr, nullptr, bits, N, K, 1, quantize_zero_to,
+                                       representable ? nullptr : count, base + p.prep_off,
+                                       nbla_hip_binarize_workspace_bytes(N, K), stream_);
+    if (rc)
+      return rc;
+    bool use_bits = true;
+    if (!representable) {
+      int host_count = 0;
+      hipError_t e = hipMemcpyAsync(&host_count, count, sizeof(int), hipMemcpyDeviceToHost, stream);
+      if (e == hipSuccess)
+        e = hipStreamSynchronize(stream);
+      if (e != hipSuccess)
+        return fail_hip(e, "reading the zero-weight count");
+      use_bits = host_count == 0;
+    }
+    if (use_bits) {
+      rc = nbla_hip_split_digits_scaled_f32(dy, N, alpha, base + p.digits_off, M, N, stream_);
+      if (rc)
+        return rc;
+      rc = launch_gemm_bits(base + p.digits_off, bits, nullptr, nullptr, dx, M, N, K, 1, K, 1, false, stream,
+                            accum_x != 0);
+    } else {
+      if (!Wb)
+        return fail(NBLA_HIP_ERR_VALUE, "the binarised weights are needed when Sign(0) is neither +1 nor -1.");
+      const float *dyp = dy;
+      if (alpha) {
+        float *scaled = reinterpret_cast<float *>(base + p.scaled_off);
+        int64_t blocks = ceil_div(M * N, 256);
+        if (blocks > 65536)
+          blocks = 65536;
+        hipLaunchKernelGGL(scale_columns, dim3((unsigned)blocks), dim3(256), 0, stream, dy, alpha, scaled, M * N, N);
+        NBLA_HIP_LAUNCH_CHECK("scale_columns");
+        dyp = scaled;
+      }
+      rc = grad_input_planes(dyp, Wb, dx, M, K, N, accum_x != 0, base, p, stream);
+    }
+    if (rc)
+      return rc;
+  }
+  if (dW) {
+    rc = grad_weights(x, dy, dW, M, K, N, accum_w != 0, base, p, stream);
+    if (rc)
+      return rc;
+  }
+  if (db)
+    return launch_column_sums(dy, db, M, N, accum_b != 0, base + p.sums_off, stream);
+  return NBLA_HIP_OK;
+}
+
+int nbla_hip_affine_backward_f32(const float *dy, const float *x, const float *W, float *dx, float *dW, float *db,
+                                 int64_t M, int64_t K, int64_t N, int accum_x, int accum_w, int accum_b,
+                                 void *workspace, size_t workspace_bytes, void *stream_) {
+  const BackwardPlan p = plan_backward(M, K, N);
+  int rc = check_args(M, K, N, workspace, workspace_bytes, p);
+  if (rc)
+    return rc;
+  hipStream_t stream = as_stream(stream_);
+  char *base = static_cast<char *>(workspace);
+  if (dx) {
+    rc = grad_input_planes(dy, W, dx, M, K, N, accum_x != 0, base, p, stream);
+    if (rc)
+      return rc;
+  }
+  if (dW) {
+    rc = grad_weights(x, dy, dW, M, K, N, accum_w != 0, base, p, stream);
+    if (rc)
+      return rc;
+  }
+  if (db)
+    return launch_column_sums(dy, db, M, N, accum_b != 0, base + p.sums_off, stream);
+  return NBLA_HIP_OK;
+}
+
+} // extern "C"

@@ -88,7 +88,8 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_kn(const float *__restric
             asum[f][c] += in ? fabsf(w[c]) : 0.0f;
             nzero += (in && is_zero) ? 1 : 0;
           }
-          if (kVec) {
+          if (!Wb) {
+          } else if (kVec) {
             float4_t o;
             o.x = b[0], o.y = b[1], o.z = b[2], o.w = b[3];
             *reinterpret_cast<float4_t *>(Wb + k * N + n0) = o;
@@ -173,7 +174,7 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_kn_vec(const float *__res
         asum[c] += in ? fabsf(w[c]) : 0.0f;
         nzero += (in && is_zero) ? 1 : 0;
       }
-      if (in) {
+      if (in && Wb) {
         float4_t o;
         o.x = b[0], o.y = b[1], o.z = b[2], o.w = b[3];
         __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(Wb + k * N + n0));
@@ -237,7 +238,8 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_nk(const float *__restric
           const int64_t k = kt * kTileK + g * 16 + j;
           if (n < N && k < K) {
             const float w = W[n * K + k];
-            Wb[n * K + k] = sign_of(w, zero_to);
+            if (Wb)
+              Wb[n * K + k] = sign_of(w, zero_to);
             const bool is_zero = !(w > 0.0f) && !(w < 0.0f);
             const bool neg = (w < 0.0f) || (is_zero && zero_to < 0.0f);
             word |= neg ? (1u << packed_bit_position(f, j)) : 0u;
@@ -477,8 +479,18 @@ __device__ __forceinline__ void store_digits(const int (&q)[16], uint4_t *dst, b
 
 // One wavefront per (padded) row: the row's shift and, per chunk of kChunkK columns, the sum of its fixed-point
 // values.  The second sweep over the row is served by the caches.
+// `cs` (may be null) scales column k of x by cs[k] before anything else: one rounded fp32 product per element.
+__device__ __forceinline__ float4_t scaled4(float4_t v, const float *__restrict__ cs, int64_t k) {
+  if (cs) {
+    const float4_t c = *reinterpret_cast<const float4_t *>(cs + k);
+    v.x = v.x * c.x, v.y = v.y * c.y, v.z = v.z * c.z, v.w = v.w * c.w;
+  }
+  return v;
+}
+
 template <bool kVec>
 __global__ __launch_bounds__(kPrepBlock) void digit_row_scale(const float *__restrict__ x, int64_t ldx,
+                                                              const float *__restrict__ cs,
                                                               long long *__restrict__ sums,
                                                               int32_t *__restrict__ shift, int64_t M, int64_t K,
                                                               int64_t rows, int64_t chunks) {
@@ -503,7 +515,7 @@ __global__ __launch_bounds__(kPrepBlock) void digit_row_scale(const float *__res
 #pragma unroll
     for (int i = 0; i < kKeep; ++i) {
       const int64_t k = 4 * lane + 256 * i;
-      kept[i] = (k < K) ? *reinterpret_cast<const float4_t *>(row + k) : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+      kept[i] = (k < K) ? scaled4(*reinterpret_cast<const float4_t *>(row + k), cs, k) : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
     }
 #pragma unroll
     for (int i = 0; i < kKeep; ++i) {
@@ -513,14 +525,14 @@ __global__ __launch_bounds__(kPrepBlock) void digit_row_scale(const float *__res
     }
   } else if (kVec) {
     for (int64_t k = 4 * lane; k < K; k += 256) { // K % 4 == 0
-      const float4_t v = *reinterpret_cast<const float4_t *>(row + k);
+      const float4_t v = scaled4(*reinterpret_cast<const float4_t *>(row + k), cs, k);
       const uint32_t a = __float_as_uint(v.x) & 0x7fffffffu, b = __float_as_uint(v.y) & 0x7fffffffu;
       const uint32_t c = __float_as_uint(v.z) & 0x7fffffffu, d = __float_as_uint(v.w) & 0x7fffffffu;
       amax = max(max(amax, max(a, b)), max(c, d));
     }
   } else {
     for (int64_t k = lane; k < K; k += 64)
-      amax = max(amax, __float_as_uint(row[k]) & 0x7fffffffu);
+      amax = max(amax, __float_as_uint(cs ? row[k] * cs[k] : row[k]) & 0x7fffffffu);
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1)
@@ -541,12 +553,12 @@ __global__ __launch_bounds__(kPrepBlock) void digit_row_scale(const float *__res
         acc = part;
       } else if (kVec) {
         for (int64_t k = k_begin + 4 * lane; k < k_end; k += 256) {
-          const float4_t v = *reinterpret_cast<const float4_t *>(row + k);
+          const float4_t v = scaled4(*reinterpret_cast<const float4_t *>(row + k), cs, k);
           acc += (long long)to_fixed(v.x, s) + to_fixed(v.y, s) + to_fixed(v.z, s) + to_fixed(v.w, s);
         }
       } else {
         for (int64_t k = k_begin + lane; k < k_end; k += 64)
-          acc += to_fixed(row[k], s);
+          acc += to_fixed(cs ? row[k] * cs[k] : row[k], s);
       }
     }
 #pragma unroll
@@ -559,6 +571,7 @@ __global__ __launch_bounds__(kPrepBlock) void digit_row_scale(const float *__res
 
 // One wavefront per (row block, k tile) fragment triple; lane l converts x[rb*32 + l%32][kt*32 + (l/32)*16 + 0..15].
 __global__ __launch_bounds__(kPrepBlock) void split_digits(const float *__restrict__ x, int64_t ldx,
+                                                           const float *__restrict__ cs,
                                                            const int32_t *__restrict__ shift, uint4_t *__restrict__ out,
                                                            int64_t M, int64_t K, int64_t k_tiles, int64_t frags) {
   const int64_t frag = (int64_t)blockIdx.x * (kPrepBlock / 64) + (threadIdx.x >> 6);
@@ -572,7 +585,9 @@ __global__ __launch_bounds__(kPrepBlock) void split_digits(const float *__restri
   int q[16];
 #pragma unroll
   for (int j = 0; j < 16; ++j)
-    q[j] = (m < M && k0 + j < K && s != kBadRow) ? to_fixed(x[m * ldx + k0 + j], s) : 0;
+    q[j] = (m < M && k0 + j < K && s != kBadRow)
+               ? to_fixed(cs ? x[m * ldx + k0 + j] * cs[k0 + j] : x[m * ldx + k0 + j], s)
+               : 0;
   store_digits(q, out + frag * kDigits * 64 + lane, false);
 }
 
@@ -580,6 +595,7 @@ __global__ __launch_bounds__(kPrepBlock) void split_digits(const float *__restri
 // Global loads are fully coalesced (16 lanes read 256 contiguous bytes of a row); the patch is turned into fragment
 // order through a padded LDS tile.
 __global__ __launch_bounds__(kPrepBlock) void split_digits_tiled(const float *__restrict__ x, int64_t ldx,
+                                                                 const float *__restrict__ cs,
                                                                  const int32_t *__restrict__ shift,
                                                                  uint4_t *__restrict__ out, int64_t M, int64_t K,
                                                                  int64_t k_tiles, int64_t patches) {
@@ -599,7 +615,7 @@ __global__ __launch_bounds__(kPrepBlock) void split_digits_tiled(const float *__
     const int64_t m = rb * kFragRows + row;
     float4_t v = {0.0f, 0.0f, 0.0f, 0.0f};
     if (m < M && kq * 64 + lc < K) // the k tiles are padded past K
-      v = *reinterpret_cast<const float4_t *>(x + m * ldx + kq * 64 + lc);
+      v = scaled4(*reinterpret_cast<const float4_t *>(x + m * ldx + kq * 64 + lc), cs, kq * 64 + lc);
     *reinterpret_cast<float4_t *>(t + row * kRowStride + lc) = v;
   }
   const int r = lane & 31, g = lane >> 5;
@@ -664,7 +680,7 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint3
   uint32_t *pairs = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + P.sums_bytes + P.zeros_bytes);
   int64_t slices = P.slices;
   if (!transposed) {
-    if (N % 4 == 0 && aligned16(W) && aligned16(Wb)) {
+    if (N % 4 == 0 && aligned16(W) && aligned16(Wb)) { // a null Wb (no fp32 signs wanted) counts as aligned
       const dim3 grid((unsigned)P.col_groups, (unsigned)P.slices);
       hipLaunchKernelGGL(binarize_kn_vec, grid, dim3(kPrepBlock), 0, stream, W, Wb, pairs, sums, zeros, K, N,
                          P.col_groups, P.Np, P.k_tiles, quantize_zero_to);
@@ -716,6 +732,12 @@ int nbla_hip_split_bf16x3_f32(const float *x, int64_t ldx, void *xsplit, int64_t
 }
 
 int nbla_hip_split_digits_f32(const float *x, int64_t ldx, void *xdigits, int64_t M, int64_t K, void *stream_) {
+  return nbla_hip_split_digits_scaled_f32(x, ldx, nullptr, xdigits, M, K, stream_);
+}
+
+int nbla_hip_split_digits_scaled_f32(const float *x, int64_t ldx, const float *colscale, void *xdigits, int64_t M,
+                                     int64_t K, void *stream_) {
+  const float *cs = colscale;
   if (M <= 0 || K <= 0 || ldx < K)
     return fail(NBLA_HIP_ERR_VALUE, "invalid digit operand shape (M=%lld, K=%lld, ldx=%lld).", (long long)M,
                 (long long)K, (long long)ldx);
@@ -729,23 +751,23 @@ int nbla_hip_split_digits_f32(const float *x, int64_t ldx, void *xdigits, int64_
   char *base = static_cast<char *>(xdigits);
   long long *sums = reinterpret_cast<long long *>(base + d.sum_off);
   int32_t *shift = reinterpret_cast<int32_t *>(base + d.shift_off);
-  const bool vec = K % 4 == 0 && ldx % 4 == 0 && aligned16(x);
+  const bool vec = K % 4 == 0 && ldx % 4 == 0 && aligned16(x) && aligned16(cs);
   const dim3 scale_grid((unsigned)ceil_div(d.rows, kPrepBlock / 64));
   if (vec)
-    hipLaunchKernelGGL(digit_row_scale<true>, scale_grid, dim3(kPrepBlock), 0, stream, x, ldx, sums, shift, M, K, d.rows,
-                       d.chunks);
+    hipLaunchKernelGGL(digit_row_scale<true>, scale_grid, dim3(kPrepBlock), 0, stream, x, ldx, cs, sums, shift, M, K,
+                       d.rows, d.chunks);
   else
-    hipLaunchKernelGGL(digit_row_scale<false>, scale_grid, dim3(kPrepBlock), 0, stream, x, ldx, sums, shift, M, K, d.rows,
-                       d.chunks);
+    hipLaunchKernelGGL(digit_row_scale<false>, scale_grid, dim3(kPrepBlock), 0, stream, x, ldx, cs, sums, shift, M, K,
+                       d.rows, d.chunks);
   NBLA_HIP_LAUNCH_CHECK("digit_row_scale");
   const int64_t frags = d.row_blocks * d.k_tiles;
-  if (K % 64 == 0 && ldx % 4 == 0 && aligned16(x)) {
+  if (K % 64 == 0 && ldx % 4 == 0 && aligned16(x) && aligned16(cs)) {
     const int64_t patches = frags / 2;
     hipLaunchKernelGGL(split_digits_tiled, dim3((unsigned)ceil_div(patches, kPrepBlock / 64)), dim3(kPrepBlock), 0,
-                       stream, x, ldx, shift, static_cast<uint4_t *>(xdigits), M, K, d.k_tiles, patches);
+                       stream, x, ldx, cs, shift, static_cast<uint4_t *>(xdigits), M, K, d.k_tiles, patches);
   } else {
     hipLaunchKernelGGL(split_digits, dim3((unsigned)ceil_div(frags, kPrepBlock / 64)), dim3(kPrepBlock), 0, stream, x,
-                       ldx, shift, static_cast<uint4_t *>(xdigits), M, K, d.k_tiles, frags);
+                       ldx, cs, shift, static_cast<uint4_t *>(xdigits), M, K, d.k_tiles, frags);
   }
   NBLA_HIP_LAUNCH_CHECK("split_digits");
   return NBLA_HIP_OK;

@@ -533,7 +533,7 @@ template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream) {
 
 int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alpha, const float *bias, float *y,
                      int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
-                     bool swap_out, hipStream_t stream) {
+                     bool swap_out, hipStream_t stream, bool accumulate) {
   if (M <= 0 || K <= 0 || N <= 0 || inner <= 0 || M > 0x7fffffffll || inner > 0x7fffffffll)
     return fail(NBLA_HIP_ERR_VALUE, "invalid GEMM shape (M=%lld, K=%lld, N=%lld).", (long long)M, (long long)K,
                 (long long)N);
@@ -569,7 +569,7 @@ int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alp
     a.sums = reinterpret_cast<const long long *>(base + d.sum_off) + c * d.rows;
     a.step_begin = c * steps_per_chunk;
     a.step_end = (a.step_begin + steps_per_chunk < steps) ? a.step_begin + steps_per_chunk : steps;
-    a.accumulate = c > 0;
+    a.accumulate = c > 0 || accumulate;
     a.finish = c + 1 == d.chunks;
     rc = swap_out ? dispatch<true>(a, stream) : dispatch<false>(a, stream);
     if (rc)

@@ -30,6 +30,7 @@ struct GemmPlanesArgs {
   float *y;
   int64_t M, N, row_blocks, col_blocks, k_blocks, k_steps, blocks_m, blocks_n;
   int64_t inner, outer_stride, n_stride;
+  int accumulate; // add to y instead of overwriting it
 };
 
 constexpr int kBM = 128, kBN = 128, kThreads = 256;
@@ -175,6 +176,8 @@ __global__ __launch_bounds__(kThreads) void gemm_planes_kernel(GemmPlanesArgs a)
           if (a.bias)
             v = v + bi;
           const int64_t off = (a.inner == 1) ? m * a.outer_stride : (m / a.inner) * a.outer_stride + (m % a.inner);
+          if (a.accumulate)
+            v = a.y[off + n * a.n_stride] + v;
           a.y[off + n * a.n_stride] = v;
         }
       }
@@ -249,7 +252,7 @@ int launch_split_weights(const float *w, void *planes, int *need_low, int64_t K,
 
 int launch_gemm_planes(const void *xsplit, const void *wplanes, const int *need_low, const float *colscale,
                        const float *bias, float *y, int64_t M, int64_t K, int64_t N, int64_t inner,
-                       int64_t outer_stride, int64_t n_stride, hipStream_t stream) {
+                       int64_t outer_stride, int64_t n_stride, hipStream_t stream, bool accumulate) {
   constexpr int kSmem = 2 * (kAStageBytes + kSegs * 2 * 3 * 64 * 16);
   static bool configured = false;
   if (!configured) {
@@ -277,6 +280,7 @@ int launch_gemm_planes(const void *xsplit, const void *wplanes, const int *need_
   a.inner = inner;
   a.outer_stride = outer_stride;
   a.n_stride = n_stride;
+  a.accumulate = accumulate ? 1 : 0;
   hipLaunchKernelGGL(gemm_planes_kernel, dim3((unsigned)(a.blocks_m * a.blocks_n)), dim3(kThreads), kSmem, stream, a);
   NBLA_HIP_LAUNCH_CHECK("gemm_planes");
   return NBLA_HIP_OK;

@@ -16,7 +16,7 @@ int launch_gemm_f32(const float *x, const float *w, const float *colscale, const
 // (for outputs whose m index is the contiguous one, e.g. convolution results [batch, O, Ho*Wo]).
 int launch_gemm_bits(const void *xsplit, const uint32_t *bits, const float *alpha, const float *bias, float *y,
                      int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
-                     bool swap_out, hipStream_t stream);
+                     bool swap_out, hipStream_t stream, bool accumulate = false);
 
 // Weight matrix w ([K, N], or [N, K] when transposed) as bf16x3 planes in fragment order; *need_low is set to
 // non-zero when some weight is not exactly a bf16 value (the product then needs the cross terms).
@@ -25,6 +25,11 @@ int launch_split_weights(const float *w, void *planes, int *need_low, int64_t K,
 // y = (x . w) * colscale + bias with both operands as bf16x3 planes.
 int launch_gemm_planes(const void *xsplit, const void *wplanes, const int *need_low, const float *colscale,
                        const float *bias, float *y, int64_t M, int64_t K, int64_t N, int64_t inner,
-                       int64_t outer_stride, int64_t n_stride, hipStream_t stream);
+                       int64_t outer_stride, int64_t n_stride, hipStream_t stream, bool accumulate = false);
+
+// db[n] (+)= sum over m of dy[m, n]; `partial` holds ceil(M / 256) * N floats.
+size_t column_sums_workspace_bytes(int64_t M, int64_t N);
+int launch_column_sums(const float *dy, float *db, int64_t M, int64_t N, bool accumulate, void *partial,
+                       hipStream_t stream);
 
 } // namespace nbla_hip

@@ -138,6 +138,14 @@ struct MinMaxGradOp {
   }
 };
 
+// relu.cpp:41-49: dx (+)= (y > 0 ? dy : 0), y the forward output
+struct ReluGradOp {
+  template <bool kAccum> __device__ __forceinline__ float apply(float dy, float y, float old, size_t) const {
+    const float t = (y > 0.0f) ? dy : 0.0f;
+    return kAccum ? old + t : t;
+  }
+};
+
 // ---- MinMaxQuantize range gradients
 __global__ __launch_bounds__(64) void minmax_bounds(const float *__restrict__ qr_min, const float *__restrict__ ql_min,
                                                     const float *__restrict__ ql_max, const float *__restrict__ scale,
@@ -282,6 +290,13 @@ int nbla_hip_pow2_quantize_backward_f32(const float *dy, const float *x, float *
   op.cut = table[m + 149]; // round(log2 a) steps from m to m + 1 at the cut of binade m
   op.sign = sign;
   return launch_grad<Pow2GradOp, true>(dy, x, dx, size, accum, op, as_stream(stream), "pow2_quantize backward");
+}
+
+int nbla_hip_relu_backward_f32(const float *dy, const float *y, float *dx, size_t size, int accum, void *stream) {
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  return launch_grad<ReluGradOp, true>(dy, y, dx, size, accum, ReluGradOp(), as_stream(stream), "relu backward");
 }
 
 size_t nbla_hip_min_max_quantize_backward_workspace_bytes(const int64_t *xshape, int ndim, const int64_t *qshape) {

@@ -28,14 +28,15 @@ EXPORTED = (
     "nbla_hip_binarize_workspace_bytes", "nbla_hip_binarize_weights_f32", "nbla_hip_split_bf16x3_f32",
     "nbla_hip_split_digits_f32", "nbla_hip_gemm_bits_f32",
     "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_weight_affine_f32",
-    "nbla_hip_binary_connect_affine_f32", "nbla_hip_affine_f32",
+    "nbla_hip_binary_connect_affine_f32", "nbla_hip_affine_f32", "nbla_hip_split_digits_scaled_f32",
+    "nbla_hip_affine_backward_workspace_bytes", "nbla_hip_binary_affine_backward_f32", "nbla_hip_affine_backward_f32",
     "nbla_hip_convolution_output_shape", "nbla_hip_binary_convolution_workspace_bytes",
     "nbla_hip_binary_weight_convolution_f32", "nbla_hip_binary_connect_convolution_f32",
     "nbla_hip_inq_workspace_bytes", "nbla_hip_inq_update_weights_f32", "nbla_hip_inq_affine_workspace_bytes",
     "nbla_hip_inq_affine_f32", "nbla_hip_inq_convolution_workspace_bytes", "nbla_hip_inq_convolution_f32",
     "nbla_hip_get_device_count", "nbla_hip_set_device", "nbla_hip_malloc", "nbla_hip_free", "nbla_hip_mem_info",
     "nbla_hip_memcpy", "nbla_hip_device_synchronize", "nbla_hip_stream_synchronize", "nbla_hip_fill",
-    "nbla_hip_cast", "nbla_hip_relu_f32",
+    "nbla_hip_cast", "nbla_hip_relu_f32", "nbla_hip_relu_backward_f32",
 )
 
 
@@ -60,6 +61,7 @@ def lib():
         L.nbla_hip_version.restype = ctypes.c_char_p
         for name in ("nbla_hip_min_max_quantize_workspace_bytes", "nbla_hip_packed_bits_bytes",
                      "nbla_hip_min_max_quantize_backward_workspace_bytes",
+                     "nbla_hip_affine_backward_workspace_bytes",
                      "nbla_hip_split_operand_bytes", "nbla_hip_digit_operand_bytes",
                      "nbla_hip_binarize_workspace_bytes",
                      "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_convolution_workspace_bytes",
@@ -254,6 +256,46 @@ def binary_connect_affine(x, W, bias=None, quantize_zero_to=1.0, workspace=None,
                                                    ctypes.c_float(quantize_zero_to), _p(ws),
                                                    ctypes.c_size_t(ws.numel()), _stream(stream)))
     return y, Wb
+
+
+def _grads(shapes, given, want, like):
+    import torch
+    outs, accum = [], []
+    for shp, g, w in zip(shapes, given, want):
+        if not w:
+            outs.append(None), accum.append(0)
+        elif g is None:
+            outs.append(torch.empty(shp, dtype=torch.float32, device=like.device)), accum.append(0)
+        else:
+            outs.append(g), accum.append(1)
+    return outs, accum
+
+
+def binary_affine_backward(dy, x, W, Wb=None, alpha=None, quantize_zero_to=1.0, dx=None, dW=None, db=None,
+                           want=(True, True, True), workspace=None, stream=None):
+    """(dx, dW, db) of BinaryWeightAffine (alpha given) / BinaryConnectAffine (alpha None); gradients passed in are
+    accumulated onto in place."""
+    M, K = x.shape
+    N = W.numel() // K
+    (odx, odw, odb), (ax, aw, ab) = _grads(((M, K), tuple(W.shape), (N,)), (dx, dW, db), want, x)
+    ws = workspace if workspace is not None else _workspace(
+        lib().nbla_hip_affine_backward_workspace_bytes(_i64(M), _i64(K), _i64(N)), x)
+    check(lib().nbla_hip_binary_affine_backward_f32(_p(dy), _p(x), _p(W), _p(Wb), _p(alpha), _p(odx), _p(odw), _p(odb),
+                                                    _i64(M), _i64(K), _i64(N), ctypes.c_float(quantize_zero_to), ax,
+                                                    aw, ab, _p(ws), ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return odx, odw, odb
+
+
+def affine_backward(dy, x, W, dx=None, dW=None, db=None, want=(True, True, True), workspace=None, stream=None):
+    """(dx, dW, db) of y = x.W + b with real-valued weights."""
+    M, K = x.shape
+    N = W.numel() // K
+    (odx, odw, odb), (ax, aw, ab) = _grads(((M, K), tuple(W.shape), (N,)), (dx, dW, db), want, x)
+    ws = workspace if workspace is not None else _workspace(
+        lib().nbla_hip_affine_backward_workspace_bytes(_i64(M), _i64(K), _i64(N)), x)
+    check(lib().nbla_hip_affine_backward_f32(_p(dy), _p(x), _p(W), _p(odx), _p(odw), _p(odb), _i64(M), _i64(K), _i64(N),
+                                             ax, aw, ab, _p(ws), ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return odx, odw, odb
 
 
 def affine(x, W, bias=None, out=None, stream=None):

@@ -122,6 +122,43 @@ def min_max_quantize(x, qr_min, qr_max, ql_min, ql_max, decay=0.999, x_min_max=F
     return y, qr_min, qr_max, scale
 
 
+def _opt(a, want, like_shape):
+    if not want:
+        return None
+    return np.zeros(like_shape, np.float32) if a is None else _f32(a).copy()
+
+
+def affine_backward(dy, x, W, dx=None, dW=None, db=None, want=(True, True, True)):
+    """(dx, dW, db) of y = x.W + b (affine.cpp:98-140); gradients passed in are accumulated onto."""
+    dy, x, W = _f32(dy), _f32(x), _f32(W)
+    M, K = x.shape
+    N = W.size // K
+    odx, odw, odb = _opt(dx, want[0], (M, K)), _opt(dW, want[1], W.shape), _opt(db, want[2], (N,))
+    nul = ctypes.POINTER(ctypes.c_float)()
+    _check(lib().orc_affine_backward(_fp(dy), _fp(x), _fp(W), _fp(odx) if want[0] else nul,
+                                     _fp(odw) if want[1] else nul, _fp(odb) if want[2] else nul, ctypes.c_long(M),
+                                     ctypes.c_long(K), ctypes.c_long(N), int(dx is not None), int(dW is not None),
+                                     int(db is not None)), "affine_backward")
+    return odx, odw, odb
+
+
+def binary_affine_backward(dy, x, W, alpha=None, quantize_zero_to=1.0, dx=None, dW=None, db=None,
+                           want=(True, True, True)):
+    """Backward of BinaryWeightAffine (alpha given) / BinaryConnectAffine (alpha None)."""
+    dy, x, W = _f32(dy), _f32(x), _f32(W)
+    M, K = x.shape
+    N = W.size // K
+    odx, odw, odb = _opt(dx, want[0], (M, K)), _opt(dW, want[1], W.shape), _opt(db, want[2], (N,))
+    nul = ctypes.POINTER(ctypes.c_float)()
+    al = _f32(alpha) if alpha is not None else None
+    _check(lib().orc_binary_affine_backward(_fp(dy), _fp(x), _fp(W), _fp(al) if al is not None else nul,
+                                            _fp(odx) if want[0] else nul, _fp(odw) if want[1] else nul,
+                                            _fp(odb) if want[2] else nul, ctypes.c_long(M), ctypes.c_long(K),
+                                            ctypes.c_long(N), ctypes.c_float(quantize_zero_to), int(dx is not None),
+                                            int(dW is not None), int(db is not None)), "binary_affine_backward")
+    return odx, odw, odb
+
+
 def fixed_point_quantize_backward(dy, x, sign=True, n=8, delta=2.0 ** -4, ste_fine_grained=True, dx=None):
     """dx (accumulated onto the given dx when one is passed), fixed_point_quantize.cpp:69-127."""
     dy, x = _f32(dy), _f32(x)

@@ -510,6 +510,67 @@ int orc_min_max_quantize(const float *x, float *y, const long *xshape, int ndim,
 }
 
 // ---------------------------------------------------------------------------
+// Affine<T>::backward_impl, affine.cpp:98-140 (plain loops in place of the Eigen
+// products; their summation order is not restated), and the two binary affine
+// backward passes built on it.
+// ---------------------------------------------------------------------------
+int orc_affine_backward(const float *dy, const float *x, const float *w, float *dx,
+                        float *dw, float *db, long M, long K, long N, int accum_x,
+                        int accum_w, int accum_b) {
+  if (dx) { // mdx (+)= mdy * mw.transpose()
+    for (long m = 0; m < M; ++m)
+      for (long k = 0; k < K; ++k) {
+        float acc = 0.0f;
+        for (long n = 0; n < N; ++n)
+          acc += dy[m * N + n] * w[k * N + n];
+        dx[m * K + k] = accum_x ? dx[m * K + k] + acc : acc;
+      }
+  }
+  if (dw) { // mdw (+)= mx.transpose() * mdy
+    for (long k = 0; k < K; ++k)
+      for (long n = 0; n < N; ++n) {
+        float acc = 0.0f;
+        for (long m = 0; m < M; ++m)
+          acc += x[m * K + k] * dy[m * N + n];
+        dw[k * N + n] = accum_w ? dw[k * N + n] + acc : acc;
+      }
+  }
+  if (db) { // mdb (+)= mdy.colwise().sum()
+    for (long n = 0; n < N; ++n) {
+      float acc = 0.0f;
+      for (long m = 0; m < M; ++m)
+        acc += dy[m * N + n];
+      db[n] = accum_b ? db[n] + acc : acc;
+    }
+  }
+  return ORC_OK;
+}
+
+// BinaryWeightAffine<T>::backward_impl, binary_weight_affine.cpp:124-146 (alpha != null) and
+// BinaryConnectAffine<T>::backward_impl, binary_connect_affine.cpp:73-92 (alpha == null): Affine backward with the
+// (scaled) binary weights, its weight gradient computed without accumulation and then passed through Sign's
+// backward (identity, sign.hpp:48-50) onto dW.
+int orc_binary_affine_backward(const float *dy, const float *x, const float *W,
+                               const float *alpha, float *dx, float *dW, float *db,
+                               long M, long K, long N, float quantize_zero_to,
+                               int accum_x, int accum_w, int accum_b) {
+  std::vector<float> ws((size_t)K * N), g;
+  for (long k = 0; k < K; ++k)
+    for (long n = 0; n < N; ++n) {
+      const float v = W[k * N + n];
+      const float b = (v > 0.0f) ? 1.0f : ((v < 0.0f) ? -1.0f : quantize_zero_to);
+      ws[k * N + n] = alpha ? b * alpha[n] : b;
+    }
+  if (dW)
+    g.resize((size_t)K * N);
+  orc_affine_backward(dy, x, ws.data(), dx, dW ? g.data() : nullptr, db, M, K, N, accum_x, 0, accum_b);
+  if (dW)
+    for (long i = 0; i < K * N; ++i)
+      dW[i] = accum_w ? dW[i] + g[i] : g[i];
+  return ORC_OK;
+}
+
+// ---------------------------------------------------------------------------
 // Backward passes of the three quantizers (straight-through estimators).
 // ---------------------------------------------------------------------------
 

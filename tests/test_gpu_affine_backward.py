@@ -1,0 +1,112 @@
+"""GPU parity of the affine backward passes (BinaryWeightAffine, BinaryConnectAffine, Affine/INQAffine) against the
+CPU oracle at the north-star tolerance and against float64 at the fp32-faithful one."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from nnabla_amd import kernels
+from util import max_rel_err, to_np
+
+pytestmark = pytest.mark.gpu
+TOL, TIGHT = 1e-4, 5e-6
+
+
+def _dev(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def _data(M, K, N, seed):
+    rng = np.random.RandomState(seed)
+    return (rng.randn(M, K).astype(np.float32), (rng.randn(K, N) * 0.02).astype(np.float32),
+            rng.randn(M, N).astype(np.float32))
+
+
+SHAPES = [(1, 32, 64), (5, 17, 9), (33, 100, 130), (64, 256, 256), (300, 520, 257), (40, 70, 4096)]
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+@pytest.mark.parametrize("with_alpha", [True, False])
+def test_binary_affine_backward(dev, M, K, N, with_alpha):
+    x, W, dy = _data(M, K, N, 31)
+    alpha = np.abs(W).mean(0).astype(np.float32) if with_alpha else None
+    rdx, rdw, rdb = oracle.binary_affine_backward(dy, x, W, alpha, 1.0)
+    d = lambda a: None if a is None else _dev(a, dev)
+    gdx, gdw, gdb = kernels.binary_affine_backward(d(dy), d(x), d(W), None, d(alpha), 1.0)
+    sgn = np.where(W >= 0, 1.0, -1.0) * (alpha.astype(np.float64) if with_alpha else 1.0)
+    dx64 = dy.astype(np.float64) @ sgn.T
+    dw64 = x.astype(np.float64).T @ dy.astype(np.float64)
+    db64 = dy.astype(np.float64).sum(0)
+    for got, ref, ref64 in ((gdx, rdx, dx64), (gdw, rdw, dw64), (gdb, rdb, db64)):
+        assert max_rel_err(to_np(got), ref) <= TOL
+        assert max_rel_err(to_np(got), ref64) <= TIGHT
+        assert max_rel_err(ref, ref64) <= TIGHT
+
+
+def test_binary_affine_backward_accumulates_and_skips(dev):
+    M, K, N = 37, 96, 200
+    x, W, dy = _data(M, K, N, 32)
+    alpha = np.abs(W).mean(0).astype(np.float32)
+    rng = np.random.RandomState(3)
+    odx, odw, odb = (rng.randn(M, K).astype(np.float32), rng.randn(K, N).astype(np.float32),
+                     rng.randn(N).astype(np.float32))
+    rdx, rdw, rdb = oracle.binary_affine_backward(dy, x, W, alpha, 1.0, dx=odx, dW=odw, db=odb)
+    d = lambda a: _dev(a, dev)
+    gdx, gdw, gdb = kernels.binary_affine_backward(d(dy), d(x), d(W), None, d(alpha), 1.0, dx=d(odx), dW=d(odw),
+                                                   db=d(odb))
+    assert max_rel_err(to_np(gdx), rdx) <= TIGHT
+    assert max_rel_err(to_np(gdw), rdw) <= TIGHT
+    assert max_rel_err(to_np(gdb), rdb) <= TIGHT
+    only = kernels.binary_affine_backward(d(dy), d(x), d(W), None, d(alpha), 1.0, want=(False, True, False))
+    assert only[0] is None and only[2] is None
+    assert max_rel_err(to_np(only[1]), x.astype(np.float64).T @ dy.astype(np.float64)) <= TIGHT
+
+
+@pytest.mark.parametrize("q0", [0.0, 0.5, -1.0])
+def test_binary_affine_backward_with_zero_weights(dev, q0):
+    """Sign(0) = quantize_zero_to: values other than +-1 cannot be packed to one bit and take the general product."""
+    M, K, N = 20, 64, 72
+    x, W, dy = _data(M, K, N, 33)
+    W.ravel()[::5] = 0.0
+    alpha = np.abs(W).mean(0).astype(np.float32)
+    Wb = oracle.sign(W, q0)
+    rdx, rdw, _ = oracle.binary_affine_backward(dy, x, W, alpha, q0)
+    d = lambda a: _dev(a, dev)
+    gdx, gdw, _ = kernels.binary_affine_backward(d(dy), d(x), d(W), d(Wb), d(alpha), q0)
+    assert max_rel_err(to_np(gdx), rdx) <= TIGHT * 4
+    assert max_rel_err(to_np(gdw), rdw) <= TIGHT * 4
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+def test_affine_backward_real_weights(dev, M, K, N):
+    """The product inside INQAffine: weights that are zero or signed powers of two, and arbitrary ones."""
+    x, W, dy = _data(M, K, N, 34)
+    for weights in (W, np.sign(W) * np.exp2(np.round(np.log2(np.abs(W) + 1e-9))).astype(np.float32)):
+        weights = weights.astype(np.float32)
+        rdx, rdw, rdb = oracle.affine_backward(dy, x, weights)
+        d = lambda a: _dev(a, dev)
+        gdx, gdw, gdb = kernels.affine_backward(d(dy), d(x), d(weights))
+        dx64 = dy.astype(np.float64) @ weights.astype(np.float64).T
+        assert max_rel_err(to_np(gdx), dx64) <= TIGHT and max_rel_err(to_np(gdx), rdx) <= TOL
+        assert max_rel_err(to_np(gdw), x.astype(np.float64).T @ dy.astype(np.float64)) <= TIGHT
+        assert max_rel_err(to_np(gdb), dy.astype(np.float64).sum(0)) <= TIGHT
+
+
+def test_backward_full_size_sample(dev):
+    """BinaryWeightAffine backward at K=4096, N=11008 with M=512: sampled rows / columns against float64."""
+    M, K, N = 512, 4096, 11008
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((M, K), dtype=np.float32)
+    W = rng.standard_normal((K, N), dtype=np.float32) * np.float32(0.02)
+    dy = rng.standard_normal((M, N), dtype=np.float32)
+    alpha = np.abs(W).mean(0).astype(np.float32)
+    d = lambda a: _dev(a, dev)
+    gdx, gdw, gdb = kernels.binary_affine_backward(d(dy), d(x), d(W), None, d(alpha), 1.0)
+    rows, cols = rng.choice(M, 16, replace=False), rng.choice(K, 64, replace=False)
+    ws = np.where(W[cols] >= 0, 1.0, -1.0) * alpha.astype(np.float64)
+    ref = dy[rows].astype(np.float64) @ ws.T
+    assert np.abs(to_np(gdx)[np.ix_(rows, cols)] - ref).max() / np.abs(ref).max() <= TIGHT
+    ks, ns = rng.choice(K, 32, replace=False), rng.choice(N, 64, replace=False)
+    ref = x[:, ks].astype(np.float64).T @ dy[:, ns].astype(np.float64)
+    assert np.abs(to_np(gdw)[np.ix_(ks, ns)] - ref).max() / np.abs(ref).max() <= TIGHT
+    assert max_rel_err(to_np(gdb), dy.astype(np.float64).sum(0)) <= TIGHT

@@ -318,3 +318,69 @@ def test_min_max_quantize_backward_through_the_registry(ctx):
         assert bits_equal(vx.g, rdx)
         np.testing.assert_allclose(vmin.g, rmin, rtol=1e-5, atol=1e-5)
         np.testing.assert_allclose(vmax.g, rmax, rtol=1e-5, atol=1e-5)
+
+
+def test_quantized_mlp_backward(ctx):
+    """Two quantized layers, forward and backward through the graph: gradients of the input and of both weight
+    matrices against the oracle's chain (quantizer STEs bit-exact given the same upstream gradient; products at
+    the fp32-faithful tolerance)."""
+    rng = np.random.RandomState(17)
+    B, D, H, O = 48, 96, 160, 40
+    x = rng.randn(B, D).astype(np.float32)
+    W1 = (rng.randn(D, H) * 0.05).astype(np.float32)
+    W2 = (rng.randn(H, O) * 0.05).astype(np.float32)
+    b2 = rng.randn(O).astype(np.float32)
+    gy = rng.randn(B, O).astype(np.float32)
+
+    vx = nn.Variable.from_numpy_array(x, need_grad=True)
+    vW1 = nn.Variable.from_numpy_array(W1, need_grad=True)
+    vW2 = nn.Variable.from_numpy_array(W2, need_grad=True)
+    vb2 = nn.Variable.from_numpy_array(b2, need_grad=True)
+    for v in (vx, vW1, vW2, vb2):
+        v.zero_grad()
+    q1 = F.fixed_point_quantize(vx, True, 8, 2.0 ** -4)
+    a1 = F.binary_weight_affine(q1, vW1, nn.Variable(W1.shape), nn.Variable((H,)))
+    h = F.relu(a1)
+    q2 = F.fixed_point_quantize(h, True, 8, 2.0 ** -4)
+    y = F.binary_connect_affine(q2, vW2, nn.Variable(W2.shape), vb2)
+    y.forward()
+    y.backward(gy)
+
+    # oracle chain on the values the GPU produced (so that quantizer ties cannot diverge the two chains)
+    oq1 = oracle.fixed_point_quantize(x, True, 8, 2.0 ** -4)
+    assert bits_equal(q1.d, oq1)
+    alpha1 = np.abs(W1).mean(0).astype(np.float32)
+    ha, hq = h.d, q2.d
+    g_q2, g_W2, g_b2 = oracle.binary_affine_backward(gy, hq, W2, None, 1.0)
+    g_h = oracle.fixed_point_quantize_backward(g_q2, ha, True, 8, 2.0 ** -4, True)
+    g_a1 = np.where(ha > 0, g_h, 0).astype(np.float32)
+    g_q1, g_W1, _ = oracle.binary_affine_backward(g_a1, oq1, W1, alpha1, 1.0, want=(True, True, False))
+    g_x = oracle.fixed_point_quantize_backward(g_q1, x, True, 8, 2.0 ** -4, True)
+    assert max_rel_err(vW2.g, g_W2) <= TIGHT
+    assert max_rel_err(vb2.g, g_b2) <= TIGHT
+    assert max_rel_err(vW1.g, g_W1) <= TIGHT * 2
+    assert max_rel_err(vx.g, g_x) <= TIGHT * 2
+    # the clipped inputs receive exactly zero gradient
+    clipped = (x > 7.9375) | (x < -7.9375)
+    assert not vx.g[clipped].any()
+
+
+def test_inq_affine_backward_through_the_registry(ctx):
+    rng = np.random.RandomState(18)
+    B, D, O = 20, 64, 96
+    x = rng.randn(B, D).astype(np.float32)
+    W = (rng.randn(D, O) * 0.05).astype(np.float32)
+    gy = rng.randn(B, O).astype(np.float32)
+    vx = nn.Variable.from_numpy_array(x, need_grad=True)
+    vW = nn.Variable.from_numpy_array(W, need_grad=True)
+    vI = nn.Variable(W.shape)
+    vI.set_data(np.ones(W.shape), np.int32)
+    vx.zero_grad()
+    vW.zero_grad()
+    y = F.inq_affine(vx, vW, vI, None, 1, 4, (), "largest_abs", -1)
+    y.forward()
+    y.backward(gy)
+    Wq = vW.d                                   # quantized in place by the forward pass
+    rdx, rdw, _ = oracle.affine_backward(gy, x, Wq, want=(True, True, False))
+    assert max_rel_err(vx.g, rdx) <= TIGHT
+    assert max_rel_err(vW.g, rdw) <= TIGHT

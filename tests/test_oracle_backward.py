@@ -99,3 +99,39 @@ def test_min_max_backward_no_range_gradient_with_statistics(x_min_max, ema):
     dx, gmin, gmax = oracle.min_max_quantize_backward(dy, x, qmn, qmx, q(0), q(255), scale, True, x_min_max, ema,
                                                       g_qr_min=sentinel, g_qr_max=sentinel)
     assert gmin == 7.0 and gmax == 7.0 and dx.shape == x.shape
+
+
+@pytest.mark.parametrize("M,K,N", [(3, 5, 4), (17, 33, 29)])
+def test_affine_backward_against_float64(M, K, N):
+    """affine.cpp:98-140: dx = dy.W^T, dW = x^T.dy, db = column sums; accumulation adds to what was there."""
+    rng = np.random.RandomState(41)
+    x, W, dy = rng.randn(M, K).astype(np.float32), rng.randn(K, N).astype(np.float32), rng.randn(M, N).astype(np.float32)
+    dx, dW, db = oracle.affine_backward(dy, x, W)
+    np.testing.assert_allclose(dx, dy.astype(np.float64) @ W.astype(np.float64).T, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(dW, x.astype(np.float64).T @ dy.astype(np.float64), rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(db, dy.astype(np.float64).sum(0), rtol=1e-5, atol=1e-5)
+    o = [rng.randn(*s).astype(np.float32) for s in ((M, K), (K, N), (N,))]
+    dx2, dW2, db2 = oracle.affine_backward(dy, x, W, dx=o[0], dW=o[1], db=o[2])
+    assert np.array_equal(dx2, o[0] + dx) and np.array_equal(dW2, o[1] + dW) and np.array_equal(db2, o[2] + db)
+    only = oracle.affine_backward(dy, x, W, want=(False, False, True))
+    assert only[0] is None and only[1] is None and np.array_equal(only[2], db)
+
+
+@pytest.mark.parametrize("q0", [1.0, 0.0, -1.0])
+def test_binary_affine_backward_uses_scaled_signs_and_full_ste(q0):
+    """binary_weight_affine.cpp:124-146: the input gradient sees Sign(W) * alpha, the weight gradient is x^T.dy
+    untouched by the binarisation (it does not depend on W at all)."""
+    rng = np.random.RandomState(42)
+    M, K, N = 6, 9, 7
+    x, W, dy = rng.randn(M, K).astype(np.float32), rng.randn(K, N).astype(np.float32), rng.randn(M, N).astype(np.float32)
+    W.ravel()[::4] = 0.0
+    alpha = np.abs(W).mean(0).astype(np.float32)
+    ws = np.where(W > 0, 1.0, np.where(W < 0, -1.0, q0)).astype(np.float32) * alpha
+    dx, dW, db = oracle.binary_affine_backward(dy, x, W, alpha, q0)
+    rdx, rdW, rdb = oracle.affine_backward(dy, x, ws)
+    assert np.array_equal(dx, rdx) and np.array_equal(dW, rdW) and np.array_equal(db, rdb)
+    dW_other = oracle.binary_affine_backward(dy, x, -3.0 * W + 1.0, alpha, q0)[1]
+    assert np.array_equal(dW_other, dW)
+    # BinaryConnect: no alpha
+    dxc = oracle.binary_affine_backward(dy, x, W, None, q0)[0]
+    assert np.array_equal(dxc, oracle.affine_backward(dy, x, np.where(W > 0, 1.0, np.where(W < 0, -1.0, q0)))[0])
