@@ -158,6 +158,28 @@ def bench_other_configs(dev, iters):
     out["inq_affine[1024,4096]x[4096,4096] (restore+quantize+product)"] = {"ms": ms, "TFLOPs": 2.0 * M * K * N / ms / 1e9}
     ms = time_kernel(lambda: k.inq_affine(xa, Wq, I, oW, oI, None, 4, k.INQ_PRODUCT_ONLY), iters)
     out["inq_affine[1024,4096]x[4096,4096] (product only)"] = {"ms": ms, "TFLOPs": 2.0 * M * K * N / ms / 1e9}
+    # backward passes (the next row of the scope table)
+    n = 1 << 24
+    xq = torch.randn(n, generator=g).to(dev) * 2
+    gq = torch.randn(n, generator=g).to(dev)
+    dq = torch.empty_like(xq)
+    ms = time_kernel(lambda: k.fixed_point_quantize_backward(gq, xq, True, 8, 2.0 ** -4, True, dx=None), iters)
+    out["fixed_point_quantize_backward[256,65536] fine-grained"] = {"ms": ms, "GBs": 12.0 * n / ms / 1e6,
+                                                                    "frac_hbm": 12.0 * n / ms / 1e6 / PEAK_HBM_GBS}
+    M, K, N = 4096, 4096, 11008
+    xb = torch.randn(M, K, generator=g).to(dev)
+    Wb_ = (torch.randn(K, N, generator=g) * 0.02).to(dev)
+    gyb = torch.randn(M, N, generator=g).to(dev)
+    alpha = Wb_.abs().mean(0)
+    ws = torch.empty(k.lib().nbla_hip_affine_backward_workspace_bytes(k._i64(M), k._i64(K), k._i64(N)),
+                     dtype=torch.uint8, device=dev)
+    dxb, dwb = torch.empty(M, K, device=dev), torch.empty(K, N, device=dev)
+    ms = time_kernel(lambda: k.binary_affine_backward(gyb, xb, Wb_, None, alpha, 1.0, dx=None, want=(True, False, False),
+                                                      workspace=ws), max(3, iters // 2))
+    out["binary_weight_affine_backward dx [4096,4096,11008]"] = {"ms": ms, "TFLOPs": 2.0 * M * K * N / ms / 1e9}
+    ms = time_kernel(lambda: k.binary_affine_backward(gyb, xb, Wb_, None, alpha, 1.0, want=(False, True, False),
+                                                      workspace=ws), max(3, iters // 2))
+    out["binary_weight_affine_backward dW [4096,4096,11008]"] = {"ms": ms, "TFLOPs": 2.0 * M * K * N / ms / 1e9}
     return out
 
 
