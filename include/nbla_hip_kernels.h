@@ -325,6 +325,45 @@ int nbla_hip_binary_connect_convolution_f32(
     const int64_t *dilation, int64_t group, float quantize_zero_to,
     void *workspace, size_t workspace_bytes, void *stream);
 
+/* Workspace of the two convolution backward entry points below. */
+size_t nbla_hip_convolution_backward_workspace_bytes(
+    int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
+    const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+    const int64_t *dilation, int64_t group);
+
+/* Backward of BinaryWeightConvolution (alpha != NULL, alpha[o] scales output
+ * channel o) / BinaryConnectConvolution (alpha == NULL): Convolution backward
+ * with the weights Ws = Sign(W) (* alpha),
+ *   dx (+)= fold(Ws_g^T . dy_g)    dW (+)= dy_g . unfold(x)_g^T    db (+)= sums of dy
+ * the weight gradient passing straight through the binarisation.  Replaces
+ * BinaryWeightConvolution<float>::backward_impl,
+ * binary_weight_convolution.cpp:119-142,
+ * BinaryConnectConvolution<float>::backward_impl,
+ * binary_connect_convolution.cpp:83-103, the Convolution backward they call,
+ * convolution.cpp:199-283, and fold_from_patches.cpp:95-170.  dy is
+ * [outer, O, out_sp...], x [outer, C, in_sp...], W and dW [O, C/group, kernel...].
+ * dx runs on the bit-weight product; Wb (the forward's fp32 signs) is only read
+ * when quantize_zero_to is neither +1 nor -1 and W holds exact zeros.  dx, dW,
+ * db may be NULL (not propagated); accum_* != 0 adds to the existing gradient. */
+int nbla_hip_binary_convolution_backward_f32(
+    const float *dy, const float *x, const float *W, const float *Wb,
+    const float *alpha, float *dx, float *dW, float *db, int64_t outer,
+    int64_t C, int nd, const int64_t *in_sp, int64_t O, const int64_t *kernel,
+    const int64_t *pad, const int64_t *stride, const int64_t *dilation,
+    int64_t group, float quantize_zero_to, int accum_x, int accum_w,
+    int accum_b, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Backward of Convolution with real-valued weights (the product inside
+ * INQConvolution).  Replaces Convolution<float>::backward_impl,
+ * convolution.cpp:199-283, as called by
+ * INQConvolution<float,int>::backward_impl, inq_convolution.cpp:220-232. */
+int nbla_hip_convolution_backward_f32(
+    const float *dy, const float *x, const float *W, float *dx, float *dW,
+    float *db, int64_t outer, int64_t C, int nd, const int64_t *in_sp,
+    int64_t O, const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+    const int64_t *dilation, int64_t group, int accum_x, int accum_w,
+    int accum_b, void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---------------------------------------------------------------------- INQ */
 
 /* INQ step selector (what the forward does to the indicators before quantizing):

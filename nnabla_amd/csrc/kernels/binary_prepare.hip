@@ -271,6 +271,85 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_nk(const float *__restric
     zeros[(int64_t)blockIdx.y * col_groups + cg] = s_zero[0] + s_zero[1] + s_zero[2] + s_zero[3];
 }
 
+// W stored [N, K], K % 4 == 0, 16-byte aligned: the streaming path of the layout above.  The block covers 64 rows
+// x 128 k (slice blockIdx.x of column group blockIdx.y); thread t reads four consecutive k (one 128-bit load, 32
+// lanes cover 512 contiguous bytes of a row) of rows i*8 + t/32, turns them into the four bits they occupy in the
+// packed word (bit 4f + jq + 8c for k quad jq, element c) and parks that partial word in LDS; wavefront w then ORs
+// the eight partial words (f, jq) of each packed word of k tile w.  |W| row sums: the four k of a thread in order,
+// then a butterfly over the 32 lanes of the row.
+constexpr int kPartStride = 36; // words per LDS row: 32 k quads + padding that keeps 16-byte alignment
+__global__ __launch_bounds__(kPrepBlock) void binarize_nk_vec(const float *__restrict__ W, float *__restrict__ Wb,
+                                                              uint32_t *__restrict__ bits, float *__restrict__ sums,
+                                                              int *__restrict__ zeros, int64_t K, int64_t N,
+                                                              int64_t col_groups, int64_t Np, int64_t k_tiles,
+                                                              float zero_to) {
+  __shared__ __attribute__((aligned(16))) uint32_t s_part[kColGroup * kPartStride];
+  __shared__ int s_zero[kPrepBlock / 64];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int kq = threadIdx.x & 31, rsub = threadIdx.x >> 5;
+  const int64_t slice = blockIdx.x, cg = blockIdx.y;
+  const int64_t k = slice * 128 + kq * 4;
+  float4_t v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int64_t n = cg * kColGroup + i * 8 + rsub;
+    if (n < N && k < K)
+      v[i] = __builtin_nontemporal_load(reinterpret_cast<const float4_t *>(W + n * K + k));
+    else
+      v[i] = float4_t{1.0f, 1.0f, 1.0f, 1.0f};
+  }
+  int nzero = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = i * 8 + rsub;
+    const int64_t n = cg * kColGroup + row;
+    const bool in = n < N && k < K;
+    const float w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+    float b[4];
+    uint32_t part = 0u;
+    float asum = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      b[c] = sign_of(w[c], zero_to);
+      const bool is_zero = !(w[c] > 0.0f) && !(w[c] < 0.0f);
+      const bool neg = (w[c] < 0.0f) || (is_zero && zero_to < 0.0f);
+      part |= (in && neg) ? (1u << (4 * (i >> 2) + (kq & 3) + 8 * c)) : 0u;
+      asum += in ? fabsf(w[c]) : 0.0f;
+      nzero += (in && is_zero) ? 1 : 0;
+    }
+    s_part[row * kPartStride + kq] = part;
+    if (in && Wb) {
+      float4_t o;
+      o.x = b[0], o.y = b[1], o.z = b[2], o.w = b[3];
+      __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(Wb + n * K + k));
+    }
+#pragma unroll
+    for (int off = 16; off >= 1; off >>= 1)
+      asum += __shfl_xor(asum, off);
+    if (kq == 0)
+      sums[slice * Np + cg * kColGroup + row] = asum;
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1)
+    nzero += __shfl_xor(nzero, off);
+  if (lane == 0)
+    s_zero[wave] = nzero;
+  __syncthreads();
+  const int64_t kt = slice * 4 + wave;
+  if (kt < k_tiles) {
+    const int g = lane >> 5, r = lane & 31;
+    uint32_t word = 0u;
+#pragma unroll
+    for (int f = 0; f < 2; ++f) {
+      const uint4_t q = *reinterpret_cast<const uint4_t *>(&s_part[(f * 32 + r) * kPartStride + wave * 8 + g * 4]);
+      word |= q.x | q.y | q.z | q.w;
+    }
+    bits[(kt * col_groups + cg) * 64 + lane] = word;
+  }
+  if (threadIdx.x == 0)
+    zeros[slice * col_groups + cg] = s_zero[0] + s_zero[1] + s_zero[2] + s_zero[3];
+}
+
 // Pair words -> packed operand: thread (k tile, wide group, lane) interleaves the four pair groups of its wide group.
 __device__ __forceinline__ void widen_bits(const uint32_t *__restrict__ pairs, uint4_t *__restrict__ bits,
                                            int64_t k_tiles, int64_t col_groups, int64_t wide_groups, int64_t idx) {
@@ -691,9 +770,14 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint3
                          P.col_groups, P.Np, quantize_zero_to);
     }
   } else {
-    const dim3 grid((unsigned)P.col_groups, (unsigned)P.slices);
-    hipLaunchKernelGGL(binarize_nk, grid, dim3(kPrepBlock), 0, stream, W, Wb, pairs, sums, zeros, K, N, P.col_groups,
-                       P.Np, P.k_tiles, quantize_zero_to);
+    if (K % 4 == 0 && aligned16(W) && aligned16(Wb) && P.col_groups <= 65535) {
+      hipLaunchKernelGGL(binarize_nk_vec, dim3((unsigned)P.slices, (unsigned)P.col_groups), dim3(kPrepBlock), 0, stream,
+                         W, Wb, pairs, sums, zeros, K, N, P.col_groups, P.Np, P.k_tiles, quantize_zero_to);
+    } else {
+      const dim3 grid((unsigned)P.col_groups, (unsigned)P.slices);
+      hipLaunchKernelGGL(binarize_nk, grid, dim3(kPrepBlock), 0, stream, W, Wb, pairs, sums, zeros, K, N, P.col_groups,
+                         P.Np, P.k_tiles, quantize_zero_to);
+    }
   }
   NBLA_HIP_LAUNCH_CHECK("binarize_weights");
   {

@@ -1,0 +1,290 @@
+// Backward passes of the convolutions: Binary{Weight,Connect}Convolution (gradient w.r.t. x on the bit-weight
+// product) and Convolution with real-valued weights (INQConvolution), plus weight and bias gradients.
+//
+// Per group the reference's sample loop (convolution.cpp:199-283) is folded into three matrix products over all
+// samples at once, with m = (sample, output position) as the long dimension:
+//   dyt [M, Og]          the output gradient of the group, transposed so that m is the row index
+//   colg[n][kk][l]       = sum over o of dyt[m, o] * w[o, kk]   (then folded into dx by a gather)
+//   dW  [Og, Kg]         = dyt^T . col(x)                        (col(x) [M, Kg] is the unfolded input)
+//   db  [Og]             = column sums of dyt
+#include "common.hpp"
+#include "conv_geom.hpp"
+#include "gemm_layout.hpp"
+#include "internal.hpp"
+
+namespace nbla_hip {
+namespace {
+
+// dyt[(n * L + l) * Og + o] = dy[(n * O + grp * Og + o) * L + l] * (scale ? scale[o] : 1): a 32 x 32 tile through LDS
+// so that both sides move contiguous runs.
+__global__ __launch_bounds__(256) void gather_dy(const float *__restrict__ dy, const float *__restrict__ scale,
+                                                 float *__restrict__ dyt, int64_t O, int64_t Og, int64_t L,
+                                                 int64_t grp) {
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const int64_t n = blockIdx.z, l0 = (int64_t)blockIdx.x * 32, o0 = (int64_t)blockIdx.y * 32;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t o = o0 + ty + 8 * i, l = l0 + tx;
+    tile[ty + 8 * i][tx] = (o < Og && l < L) ? dy[(n * O + grp * Og + o) * L + l] : 0.0f;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t l = l0 + ty + 8 * i, o = o0 + tx;
+    if (l < L && o < Og) {
+      const float v = tile[tx][ty + 8 * i];
+      dyt[(n * L + l) * Og + o] = scale ? v * scale[o] : v;
+    }
+  }
+}
+
+// dx element (n, c, position) (+)= sum of the unfolded gradient over the taps that read that position, in
+// ascending tap order (the order fold_from_patches.cpp:125-170 adds them in).  colg is [outer][Kg][L].
+__global__ __launch_bounds__(256) void col2im_gather(const float *__restrict__ colg, float *__restrict__ dx, ConvGeom g,
+                                                     int64_t grp, int accumulate) {
+  const int64_t total = g.outer * g.Cg * g.in_sp_size;
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+    int64_t t = idx;
+    const int i2 = (int)(t % g.in_sp[2]);
+    t /= g.in_sp[2];
+    const int i1 = (int)(t % g.in_sp[1]);
+    t /= g.in_sp[1];
+    const int i0 = (int)(t % g.in_sp[0]);
+    t /= g.in_sp[0];
+    const int64_t cc = t % g.Cg, n = t / g.Cg;
+    const float *src = colg + (n * g.Kg + cc * g.k_size) * g.out_sp_size;
+    float acc = 0.0f;
+    for (int k0 = 0; k0 < g.k[0]; ++k0) {
+      const int t0 = i0 + g.pad[0] - k0 * g.dil[0];
+      if (t0 < 0 || t0 % g.stride[0] != 0 || t0 / g.stride[0] >= g.out_sp[0])
+        continue;
+      for (int k1 = 0; k1 < g.k[1]; ++k1) {
+        const int t1 = i1 + g.pad[1] - k1 * g.dil[1];
+        if (t1 < 0 || t1 % g.stride[1] != 0 || t1 / g.stride[1] >= g.out_sp[1])
+          continue;
+        for (int k2 = 0; k2 < g.k[2]; ++k2) {
+          const int t2 = i2 + g.pad[2] - k2 * g.dil[2];
+          if (t2 < 0 || t2 % g.stride[2] != 0 || t2 / g.stride[2] >= g.out_sp[2])
+            continue;
+          const int64_t tap = ((int64_t)k0 * g.k[1] + k1) * g.k[2] + k2;
+          const int64_t l = ((int64_t)(t0 / g.stride[0]) * g.out_sp[1] + t1 / g.stride[1]) * g.out_sp[2] +
+                            t2 / g.stride[2];
+          acc += src[tap * g.out_sp_size + l];
+        }
+      }
+    }
+    const int64_t pos = ((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2] + i2;
+    float *dst = dx + (n * g.C + grp * g.Cg + cc) * g.in_sp_size + pos;
+    *dst = accumulate ? *dst + acc : acc;
+  }
+}
+
+struct ConvBackwardPlan {
+  size_t dyt_off, scaled_off, col_off, a_planes_off, b_planes_off, digits_off, bits_off, prep_off, count_off,
+      flag_off, sums_off, total;
+};
+
+size_t larger(size_t a, size_t b) { return a > b ? a : b; }
+
+// One layout for both entry points; every region is reused group after group.
+ConvBackwardPlan plan_conv_backward(const ConvGeom &g) {
+  ConvBackwardPlan p;
+  size_t off = 0;
+  const size_t dyt_bytes = round_up((size_t)g.M * g.Og * sizeof(float), 256);
+  p.dyt_off = off;
+  off += dyt_bytes;
+  p.scaled_off = off; // dyt * alpha in fp32 (only when Sign(0) is neither +1 nor -1)
+  off += dyt_bytes;
+  p.col_off = off; // unfolded input [M, Kg], and the unfolded gradient [outer][Kg][L]
+  off += round_up((size_t)g.M * g.Kg * sizeof(float), 256);
+  p.a_planes_off = off; // dyt^T for dW (rows o, contraction m) or dyt for dx (rows m, contraction o)
+  off += round_up(larger(nbla_hip_split_operand_bytes(g.Og, g.M), nbla_hip_split_operand_bytes(g.M, g.Og)), 256);
+  p.b_planes_off = off; // col(x) (columns kk, contraction m) or w (columns kk, contraction o)
+  off += round_up(larger(nbla_hip_split_operand_bytes(g.Kg, g.M), nbla_hip_split_operand_bytes(g.Kg, g.Og)), 256);
+  p.digits_off = off;
+  off += round_up(nbla_hip_digit_operand_bytes(g.M, g.Og), 256);
+  p.bits_off = off;
+  off += round_up(nbla_hip_packed_bits_bytes(g.Og, g.Kg), 256);
+  p.prep_off = off;
+  off += round_up(nbla_hip_binarize_workspace_bytes(g.Og, g.Kg), 256);
+  p.count_off = off;
+  off += 256;
+  p.flag_off = off;
+  off += 256;
+  p.sums_off = off;
+  off += round_up(column_sums_workspace_bytes(g.M, g.Og), 256);
+  p.total = off;
+  return p;
+}
+
+int launch_gather_dy(const float *dy, const float *scale, float *dyt, const ConvGeom &g, int64_t grp,
+                     hipStream_t stream) {
+  if (g.outer > 65535 || ceil_div(g.Og, 32) > 65535)
+    return fail(NBLA_HIP_ERR_VALUE, "convolution backward supports at most 65535 samples per call.");
+  const dim3 grid((unsigned)ceil_div(g.out_sp_size, 32), (unsigned)ceil_div(g.Og, 32), (unsigned)g.outer);
+  hipLaunchKernelGGL(gather_dy, grid, dim3(256), 0, stream, dy, scale, dyt, g.O, g.Og, g.out_sp_size, grp);
+  NBLA_HIP_LAUNCH_CHECK("gather_dy");
+  return NBLA_HIP_OK;
+}
+
+int launch_col2im(const float *colg, float *dx, const ConvGeom &g, int64_t grp, bool accumulate, hipStream_t stream) {
+  int64_t blocks = ceil_div(g.outer * g.Cg * g.in_sp_size, 256);
+  if (blocks > 262144)
+    blocks = 262144;
+  hipLaunchKernelGGL(col2im_gather, dim3((unsigned)blocks), dim3(256), 0, stream, colg, dx, g, grp,
+                     accumulate ? 1 : 0);
+  NBLA_HIP_LAUNCH_CHECK("col2im_gather");
+  return NBLA_HIP_OK;
+}
+
+// `binary`: the weights of the forward pass were Sign(W) (* alpha[o]); otherwise W itself.
+int conv_backward(const float *dy, const float *x, const float *W, const float *Wb, const float *alpha, float *dx,
+                  float *dW, float *db, const ConvGeom &g, bool binary, float zero_to, bool accum_x, bool accum_w,
+                  bool accum_b, void *workspace, size_t workspace_bytes, void *stream_) {
+  const ConvBackwardPlan p = plan_conv_backward(g);
+  if (workspace_bytes < p.total || !aligned256(workspace))
+    return fail(NBLA_HIP_ERR_MEMORY, "convolution backward workspace too small (%zu < %zu) or misaligned.",
+                workspace_bytes, p.total);
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  hipStream_t stream = as_stream(stream_);
+  char *base = static_cast<char *>(workspace);
+  float *dyt = reinterpret_cast<float *>(base + p.dyt_off);
+  float *scaled = reinterpret_cast<float *>(base + p.scaled_off);
+  float *col = reinterpret_cast<float *>(base + p.col_off);
+  int *flag = reinterpret_cast<int *>(base + p.flag_off);
+  int *count = reinterpret_cast<int *>(base + p.count_off);
+  uint32_t *bits = reinterpret_cast<uint32_t *>(base + p.bits_off);
+  const bool representable = (zero_to == 1.0f || zero_to == -1.0f);
+  const int64_t L = g.out_sp_size;
+  for (int64_t grp = 0; grp < g.group; ++grp) {
+    const float *Wg = W + grp * g.Og * g.Kg;
+    const float *ag = alpha ? alpha + grp * g.Og : nullptr;
+    rc = launch_gather_dy(dy, nullptr, dyt, g, grp, stream);
+    if (rc)
+      return rc;
+    if (dx) {
+      bool use_bits = binary;
+      if (binary) {
+        // Sign(W_g) packed for the contraction over o: W_g is stored [Og, Kg] = [contraction][column]
+        rc = nbla_hip_binarize_weights_f32(Wg, nullptr, nullptr, bits, g.Og, g.Kg, 0, zero_to,
+                                           representable ? nullptr : count, base + p.prep_off,
+                                           nbla_hip_binarize_workspace_bytes(g.Og, g.Kg), stream_);
+        if (rc)
+          return rc;
+        if (!representable) {
+          int host_count = 0;
+          hipError_t e = hipMemcpyAsync(&host_count, count, sizeof(int), hipMemcpyDeviceToHost, stream);
+          if (e == hipSuccess)
+            e = hipStreamSynchronize(stream);
+          if (e != hipSuccess)
+            return fail_hip(e, "reading the zero-weight count");
+          use_bits = host_count == 0;
+        }
+      }
+      if (use_bits) {
+        rc = nbla_hip_split_digits_scaled_f32(dyt, g.Og, ag, base + p.digits_off, g.M, g.Og, stream_);
+        if (rc)
+          return rc;
+        rc = launch_gemm_bits(base + p.digits_off, bits, nullptr, nullptr, col, g.M, g.Og, g.Kg, L, g.Kg * L, L, true,
+                              stream);
+      } else {
+        const float *wsrc = Wg;
+        const float *dsrc = dyt;
+        if (binary) {
+          if (!Wb)
+            return fail(NBLA_HIP_ERR_VALUE, "the binarised weights are needed when Sign(0) is neither +1 nor -1.");
+          wsrc = Wb + grp * g.Og * g.Kg;
+          if (ag) {
+            rc = launch_gather_dy(dy, ag, scaled, g, grp, stream);
+            if (rc)
+              return rc;
+            dsrc = scaled;
+          }
+        }
+        rc = nbla_hip_split_bf16x3_f32(dsrc, g.Og, base + p.a_planes_off, g.M, g.Og, stream_);
+        if (rc)
+          return rc;
+        rc = launch_split_weights(wsrc, base + p.b_planes_off, flag, g.Og, g.Kg, false, stream);
+        if (rc)
+          return rc;
+        rc = launch_gemm_planes(base + p.a_planes_off, base + p.b_planes_off, flag, nullptr, nullptr, col, g.M, g.Og,
+                                g.Kg, L, g.Kg * L, L, stream);
+      }
+      if (rc)
+        return rc;
+      rc = launch_col2im(col, dx, g, grp, accum_x, stream);
+      if (rc)
+        return rc;
+    }
+    if (dW) {
+      rc = launch_im2col_f32(x, col, g, grp, stream);
+      if (rc)
+        return rc;
+      // dyt^T as the row operand (rows o, contraction m) and col(x) as the column operand (columns kk)
+      rc = launch_split_weights(dyt, base + p.a_planes_off, flag, g.M, g.Og, false, stream);
+      if (rc)
+        return rc;
+      rc = launch_split_weights(col, base + p.b_planes_off, flag, g.M, g.Kg, false, stream);
+      if (rc)
+        return rc;
+      rc = launch_gemm_planes(base + p.a_planes_off, base + p.b_planes_off, flag, nullptr, nullptr,
+                              dW + grp * g.Og * g.Kg, g.Og, g.M, g.Kg, 1, g.Kg, 1, stream, accum_w);
+      if (rc)
+        return rc;
+    }
+    if (db) {
+      rc = launch_column_sums(dyt, db + grp * g.Og, g.M, g.Og, accum_b, base + p.sums_off, stream);
+      if (rc)
+        return rc;
+    }
+  }
+  return NBLA_HIP_OK;
+}
+
+} // namespace
+} // namespace nbla_hip
+
+using namespace nbla_hip;
+
+extern "C" {
+
+size_t nbla_hip_convolution_backward_workspace_bytes(int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
+                                                     const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+                                                     const int64_t *dilation, int64_t group) {
+  ConvGeom g;
+  if (make_geom(g, outer, C, nd, in_sp, O, kernel, pad, stride, dilation, group))
+    return 0;
+  return plan_conv_backward(g).total;
+}
+
+int nbla_hip_binary_convolution_backward_f32(const float *dy, const float *x, const float *W, const float *Wb,
+                                             const float *alpha, float *dx, float *dW, float *db, int64_t outer,
+                                             int64_t C, int nd, const int64_t *in_sp, int64_t O, const int64_t *kernel,
+                                             const int64_t *pad, const int64_t *stride, const int64_t *dilation,
+                                             int64_t group, float quantize_zero_to, int accum_x, int accum_w,
+                                             int accum_b, void *workspace, size_t workspace_bytes, void *stream) {
+  ConvGeom g;
+  const int rc = make_geom(g, outer, C, nd, in_sp, O, kernel, pad, stride, dilation, group);
+  if (rc)
+    return rc;
+  return conv_backward(dy, x, W, Wb, alpha, dx, dW, db, g, true, quantize_zero_to, accum_x != 0, accum_w != 0,
+                       accum_b != 0, workspace, workspace_bytes, stream);
+}
+
+int nbla_hip_convolution_backward_f32(const float *dy, const float *x, const float *W, float *dx, float *dW, float *db,
+                                      int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
+                                      const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+                                      const int64_t *dilation, int64_t group, int accum_x, int accum_w, int accum_b,
+                                      void *workspace, size_t workspace_bytes, void *stream) {
+  ConvGeom g;
+  const int rc = make_geom(g, outer, C, nd, in_sp, O, kernel, pad, stride, dilation, group);
+  if (rc)
+    return rc;
+  return conv_backward(dy, x, W, nullptr, nullptr, dx, dW, db, g, false, 1.0f, accum_x != 0, accum_w != 0,
+                       accum_b != 0, workspace, workspace_bytes, stream);
+}
+
+} // extern "C"

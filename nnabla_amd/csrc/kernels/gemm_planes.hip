@@ -231,7 +231,8 @@ __global__ __launch_bounds__(256) void split_weights(const float *__restrict__ w
   dst[64] = o;
   o.x = l[0] | (l[1] << 16), o.y = l[2] | (l[3] << 16), o.z = l[4] | (l[5] << 16), o.w = l[6] | (l[7] << 16);
   dst[128] = o;
-  if (__any(low != 0) && lane == 0)
+  // one flag for the whole grid: look before writing, or millions of wavefronts queue on one address
+  if (__any(low != 0) && lane == 0 && __hip_atomic_load(need_low, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
     atomicOr(need_low, 1);
 }
 

@@ -32,6 +32,8 @@ EXPORTED = (
     "nbla_hip_affine_backward_workspace_bytes", "nbla_hip_binary_affine_backward_f32", "nbla_hip_affine_backward_f32",
     "nbla_hip_convolution_output_shape", "nbla_hip_binary_convolution_workspace_bytes",
     "nbla_hip_binary_weight_convolution_f32", "nbla_hip_binary_connect_convolution_f32",
+    "nbla_hip_convolution_backward_workspace_bytes", "nbla_hip_binary_convolution_backward_f32",
+    "nbla_hip_convolution_backward_f32",
     "nbla_hip_inq_workspace_bytes", "nbla_hip_inq_update_weights_f32", "nbla_hip_inq_affine_workspace_bytes",
     "nbla_hip_inq_affine_f32", "nbla_hip_inq_convolution_workspace_bytes", "nbla_hip_inq_convolution_f32",
     "nbla_hip_get_device_count", "nbla_hip_set_device", "nbla_hip_malloc", "nbla_hip_free", "nbla_hip_mem_info",
@@ -62,6 +64,7 @@ def lib():
         for name in ("nbla_hip_min_max_quantize_workspace_bytes", "nbla_hip_packed_bits_bytes",
                      "nbla_hip_min_max_quantize_backward_workspace_bytes",
                      "nbla_hip_affine_backward_workspace_bytes",
+                     "nbla_hip_convolution_backward_workspace_bytes",
                      "nbla_hip_split_operand_bytes", "nbla_hip_digit_operand_bytes",
                      "nbla_hip_binarize_workspace_bytes",
                      "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_convolution_workspace_bytes",
@@ -355,6 +358,33 @@ def binary_connect_convolution(x, W, bias=None, pad=None, stride=None, dilation=
     check(lib().nbla_hip_binary_connect_convolution_f32(_p(x), _p(W), _p(Wb), _p(bias), _p(y), *geom, q0, _p(ws),
                                                         ctypes.c_size_t(ws.numel()), _stream(stream)))
     return y, Wb
+
+
+def binary_convolution_backward(dy, x, W, Wb=None, alpha=None, pad=None, stride=None, dilation=None, group=1,
+                                quantize_zero_to=1.0, dx=None, dW=None, db=None, want=(True, True, True),
+                                workspace=None, stream=None):
+    """(dx, dW, db) of BinaryWeightConvolution (alpha given) / BinaryConnectConvolution (alpha None); gradients
+    passed in are accumulated onto in place."""
+    geom, _ = _conv_geometry(x, W, pad, stride, dilation, group)
+    (odx, odw, odb), (ax, aw, ab) = _grads((tuple(x.shape), tuple(W.shape), (int(W.shape[0]),)), (dx, dW, db), want, x)
+    ws = workspace if workspace is not None else _workspace(
+        lib().nbla_hip_convolution_backward_workspace_bytes(*geom), x)
+    check(lib().nbla_hip_binary_convolution_backward_f32(_p(dy), _p(x), _p(W), _p(Wb), _p(alpha), _p(odx), _p(odw),
+                                                         _p(odb), *geom, ctypes.c_float(quantize_zero_to), ax, aw, ab,
+                                                         _p(ws), ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return odx, odw, odb
+
+
+def convolution_backward(dy, x, W, pad=None, stride=None, dilation=None, group=1, dx=None, dW=None, db=None,
+                         want=(True, True, True), workspace=None, stream=None):
+    """(dx, dW, db) of a convolution with real-valued weights."""
+    geom, _ = _conv_geometry(x, W, pad, stride, dilation, group)
+    (odx, odw, odb), (ax, aw, ab) = _grads((tuple(x.shape), tuple(W.shape), (int(W.shape[0]),)), (dx, dW, db), want, x)
+    ws = workspace if workspace is not None else _workspace(
+        lib().nbla_hip_convolution_backward_workspace_bytes(*geom), x)
+    check(lib().nbla_hip_convolution_backward_f32(_p(dy), _p(x), _p(W), _p(odx), _p(odw), _p(odb), *geom, ax, aw, ab,
+                                                  _p(ws), ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return odx, odw, odb
 
 
 # ---------------------------------------------------------------------------- INQ

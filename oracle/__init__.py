@@ -310,6 +310,37 @@ def binary_connect_convolution(x, W, b=None, pad=None, stride=None, dilation=Non
     return y, Wb
 
 
+def convolution_backward(dy, x, W, pad=None, stride=None, dilation=None, group=1, dx=None, dW=None, db=None,
+                         want=(True, True, True)):
+    """(dx, dW, db) of Convolution (convolution.cpp:199-283); gradients passed in are accumulated onto."""
+    x, W, tail, yshape = _conv_args(x, W, pad, stride, dilation, group)
+    dy = _f32(dy).reshape(yshape)
+    odx, odw, odb = _opt(dx, want[0], x.shape), _opt(dW, want[1], W.shape), _opt(db, want[2], (W.shape[0],))
+    nul = ctypes.POINTER(ctypes.c_float)()
+    _check(lib().orc_convolution_backward(_fp(dy), _fp(x), _fp(W), _fp(odx) if want[0] else nul,
+                                          _fp(odw) if want[1] else nul, _fp(odb) if want[2] else nul, *tail,
+                                          int(dx is not None), int(dW is not None), int(db is not None)),
+           "convolution_backward")
+    return odx, odw, odb
+
+
+def binary_convolution_backward(dy, x, W, alpha=None, pad=None, stride=None, dilation=None, group=1,
+                                quantize_zero_to=1.0, dx=None, dW=None, db=None, want=(True, True, True)):
+    """Backward of BinaryWeightConvolution (alpha given) / BinaryConnectConvolution (alpha None)."""
+    x, W, tail, yshape = _conv_args(x, W, pad, stride, dilation, group)
+    dy = _f32(dy).reshape(yshape)
+    odx, odw, odb = _opt(dx, want[0], x.shape), _opt(dW, want[1], W.shape), _opt(db, want[2], (W.shape[0],))
+    nul = ctypes.POINTER(ctypes.c_float)()
+    al = _f32(alpha) if alpha is not None else None
+    _check(lib().orc_binary_convolution_backward(_fp(dy), _fp(x), _fp(W), _fp(al) if al is not None else nul,
+                                                 _fp(odx) if want[0] else nul, _fp(odw) if want[1] else nul,
+                                                 _fp(odb) if want[2] else nul, *tail,
+                                                 ctypes.c_float(quantize_zero_to), int(dx is not None),
+                                                 int(dW is not None), int(db is not None)),
+           "binary_convolution_backward")
+    return odx, odw, odb
+
+
 class Inq(object):
     """Stateful INQ weight logic (one object per INQAffine / INQConvolution)."""
 

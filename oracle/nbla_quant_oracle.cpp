@@ -228,6 +228,95 @@ void conv_forward(const ConvGeom &g, const float *x, const float *w,
   }
 }
 
+// col2im of one sample, accumulating into dxs: fold_from_patches.cpp:22-170.
+// Each column row (c, kernel index) is added into the image in row order, so an
+// image element receives its taps in ascending kernel index.
+void col2im_add(const ConvGeom &g, const float *col, float *dxs) {
+  const long rows = g.C * g.k_size;
+  for (long r = 0; r < rows; ++r) {
+    long rem = r;
+    long kidx[3] = {0, 0, 0};
+    for (int i = g.nd - 1; i >= 0; --i) {
+      kidx[i] = rem % g.k[i];
+      rem /= g.k[i];
+    }
+    float *xc = dxs + rem * g.in_sp_size;
+    const float *src = col + r * g.out_sp_size;
+    for (long p = 0; p < g.out_sp_size; ++p) {
+      long prem = p;
+      long off = 0, mul = 1;
+      bool inside = true;
+      for (int i = g.nd - 1; i >= 0; --i) {
+        const long o = prem % g.out_sp[i];
+        prem /= g.out_sp[i];
+        const long pos = o * g.stride[i] + kidx[i] * g.dil[i] - g.pad[i];
+        if (pos < 0 || pos >= g.in_sp[i])
+          inside = false;
+        off += pos * mul;
+        mul *= g.in_sp[i];
+      }
+      if (inside)
+        xc[off] = xc[off] + src[p];
+    }
+  }
+}
+
+// Convolution<T>::backward_impl, convolution.cpp:199-283: the sample loop with
+//   col_g = W_g^T * dy_g, folded into dx;   dW_g += dy_g * col_g(x)^T;   db += row sums of dy.
+// Plain loops stand in for the Eigen products (their summation order is not restated).
+void conv_backward(const ConvGeom &g, const float *dy, const float *x, const float *w, float *dx,
+                   float *dw, float *db, int accum_x, int accum_w, int accum_b) {
+  const long row_w = g.O / g.group, col_w = g.col_rows, L = g.out_sp_size;
+  const long in_size = g.C * g.in_sp_size, out_size = g.O * L;
+  std::vector<float> col((size_t)g.C * g.k_size * L);
+  if (dx && !accum_x)
+    std::fill(dx, dx + g.outer * in_size, 0.0f);
+  if (dw && !accum_w)
+    std::fill(dw, dw + g.O * col_w, 0.0f);
+  if (db && !accum_b)
+    std::fill(db, db + g.O, 0.0f);
+  for (long n = 0; n < g.outer; ++n) {
+    const float *dyn = dy + n * out_size;
+    if (dx) {
+      for (long gi = 0; gi < g.group; ++gi) {
+        const float *wg = w + gi * row_w * col_w;
+        const float *dyg = dyn + gi * row_w * L;
+        float *cg = col.data() + gi * col_w * L;
+        for (long j = 0; j < col_w; ++j)
+          for (long p = 0; p < L; ++p) {
+            float acc = 0.0f;
+            for (long o = 0; o < row_w; ++o)
+              acc += wg[o * col_w + j] * dyg[o * L + p];
+            cg[j * L + p] = acc;
+          }
+      }
+      col2im_add(g, col.data(), dx + n * in_size);
+    }
+    if (dw) {
+      im2col(g, x + n * in_size, col.data());
+      for (long gi = 0; gi < g.group; ++gi) {
+        const float *dyg = dyn + gi * row_w * L;
+        const float *cg = col.data() + gi * col_w * L;
+        float *dwg = dw + gi * row_w * col_w;
+        for (long o = 0; o < row_w; ++o)
+          for (long j = 0; j < col_w; ++j) {
+            float acc = 0.0f;
+            for (long p = 0; p < L; ++p)
+              acc += dyg[o * L + p] * cg[j * L + p];
+            dwg[o * col_w + j] = dwg[o * col_w + j] + acc;
+          }
+      }
+    }
+    if (db)
+      for (long o = 0; o < g.O; ++o) {
+        float acc = 0.0f;
+        for (long p = 0; p < L; ++p)
+          acc += dyn[o * L + p];
+        db[o] = db[o] + acc;
+      }
+  }
+}
+
 // Steps B and C of inq_affine.cpp:104-190 (shared verbatim by
 // inq_convolution.cpp:119-205), plus step A (:95-102).
 struct InqState {
@@ -863,6 +952,51 @@ int orc_binary_connect_convolution(const float *x, const float *W, float *Wb,
     Wb[i] = sign_op(W[i], quantize_zero_to);
   if (y)
     conv_forward(g, x, Wb, b, y);
+  return ORC_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Convolution backward (also INQConvolution<T>::backward_impl, inq_convolution.cpp:220-232, which hands
+// its inputs to it unchanged) and the two binary convolution backward passes.
+// ---------------------------------------------------------------------------
+int orc_convolution_backward(const float *dy, const float *x, const float *w, float *dx, float *dw,
+                             float *db, long outer, long C, int nd, const long *in_sp, long O,
+                             const long *kernel, const long *pad, const long *stride, const long *dil,
+                             long group, int accum_x, int accum_w, int accum_b) {
+  ConvGeom g;
+  const int rc = make_geom(g, outer, C, nd, in_sp, O, kernel, pad, stride, dil, group);
+  if (rc)
+    return rc;
+  conv_backward(g, dy, x, w, dx, dw, db, accum_x, accum_w, accum_b);
+  return ORC_OK;
+}
+
+// BinaryWeightConvolution<T>::backward_impl, binary_weight_convolution.cpp:119-142 (alpha != null; alpha[o] scales
+// output channel o) and BinaryConnectConvolution<T>::backward_impl, binary_connect_convolution.cpp:83-103
+// (alpha == null): Convolution backward with the (scaled) binary weights, the weight gradient computed without
+// accumulation and then passed through Sign's backward (identity) onto dW.
+int orc_binary_convolution_backward(const float *dy, const float *x, const float *W, const float *alpha,
+                                    float *dx, float *dW, float *db, long outer, long C, int nd,
+                                    const long *in_sp, long O, const long *kernel, const long *pad,
+                                    const long *stride, const long *dil, long group,
+                                    float quantize_zero_to, int accum_x, int accum_w, int accum_b) {
+  ConvGeom g;
+  const int rc = make_geom(g, outer, C, nd, in_sp, O, kernel, pad, stride, dil, group);
+  if (rc)
+    return rc;
+  const long col_w = g.col_rows;
+  std::vector<float> ws((size_t)O * col_w), gw;
+  for (long o = 0; o < O; ++o)
+    for (long j = 0; j < col_w; ++j) {
+      const float b = sign_op(W[o * col_w + j], quantize_zero_to);
+      ws[o * col_w + j] = alpha ? b * alpha[o] : b;
+    }
+  if (dW)
+    gw.resize((size_t)O * col_w);
+  conv_backward(g, dy, x, ws.data(), dx, dW ? gw.data() : nullptr, db, accum_x, 0, accum_b);
+  if (dW)
+    for (long i = 0; i < O * col_w; ++i)
+      dW[i] = accum_w ? dW[i] + gw[i] : gw[i];
   return ORC_OK;
 }
 

@@ -135,3 +135,73 @@ def test_binary_affine_backward_uses_scaled_signs_and_full_ste(q0):
     # BinaryConnect: no alpha
     dxc = oracle.binary_affine_backward(dy, x, W, None, q0)[0]
     assert np.array_equal(dxc, oracle.affine_backward(dy, x, np.where(W > 0, 1.0, np.where(W < 0, -1.0, q0)))[0])
+
+
+CONV_CASES = [
+    # (x shape, W shape, pad, stride, dilation, group)
+    ((2, 4, 7, 6), (6, 4, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((3, 4, 9, 8), (4, 2, 3, 2), (2, 0), (2, 1), (1, 2), 2),
+    ((2, 6, 11), (3, 2, 4), (1,), (3,), (2,), 3),
+    ((1, 2, 5, 6, 4), (4, 2, 2, 3, 1), (1, 1, 0), (1, 2, 1), (1, 1, 1), 1),
+]
+
+
+def _torch_conv_grads(x, W, b, dy, pad, stride, dilation, group):
+    """Gradients by torch's CPU autograd in float64: an independent library routine for the same operator."""
+    import torch
+    import torch.nn.functional as tf
+    tx = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    tw = torch.tensor(W, dtype=torch.float64, requires_grad=True)
+    tb = torch.tensor(b, dtype=torch.float64, requires_grad=True)
+    conv = {1: tf.conv1d, 2: tf.conv2d, 3: tf.conv3d}[W.ndim - 2]
+    y = conv(tx, tw, tb, stride=stride, padding=pad, dilation=dilation, groups=group)
+    y.backward(torch.tensor(dy, dtype=torch.float64))
+    return tx.grad.numpy(), tw.grad.numpy(), tb.grad.numpy()
+
+
+@pytest.mark.parametrize("xs,ws,pad,stride,dil,group", CONV_CASES)
+def test_convolution_backward_against_autograd(xs, ws, pad, stride, dil, group):
+    x, W, b = _rand(xs, 11), _rand(ws, 12, 0.3), _rand((ws[0],), 13)
+    y = oracle.convolution(x, W, b, pad, stride, dil, group)
+    dy = _rand(y.shape, 14)
+    rdx, rdw, rdb = _torch_conv_grads(x, W, b, dy, pad, stride, dil, group)
+    dx, dw, db = oracle.convolution_backward(dy, x, W, pad, stride, dil, group)
+    np.testing.assert_allclose(dx, rdx, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(dw, rdw, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(db, rdb, rtol=2e-5, atol=2e-5)
+    # accumulation onto existing gradients, and outputs that are not asked for stay untouched
+    ox, ow, ob = _rand(xs, 15), _rand(ws, 16), _rand((ws[0],), 17)
+    ax, aw, ab = oracle.convolution_backward(dy, x, W, pad, stride, dil, group, dx=ox, dW=ow, db=ob)
+    np.testing.assert_allclose(ax, ox + rdx, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(aw, ow + rdw, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(ab, ob + rdb, rtol=2e-5, atol=2e-5)
+    only_w = oracle.convolution_backward(dy, x, W, pad, stride, dil, group, want=(False, True, False))
+    assert only_w[0] is None and only_w[2] is None and np.array_equal(only_w[1], dw)
+
+
+@pytest.mark.parametrize("xs,ws,pad,stride,dil,group", CONV_CASES[:3])
+@pytest.mark.parametrize("weight_scaled", [True, False])
+def test_binary_convolution_backward_is_convolution_backward_of_sign_weights(xs, ws, pad, stride, dil, group,
+                                                                             weight_scaled):
+    """dx and db are those of a convolution with Sign(W) (* alpha per output channel); the weight gradient is the
+    one w.r.t. those weights handed straight through onto W (no factor alpha, no mask)."""
+    x, W = _rand(xs, 21), _rand(ws, 22, 0.3)
+    W.ravel()[:3] = [0.0, -0.0, 1e-30]
+    q0 = -1.0
+    if weight_scaled:
+        _, Wb, alpha = oracle.binary_weight_convolution(x, W, None, pad, stride, dil, group, q0)
+        Ws = Wb * alpha.reshape((-1,) + (1,) * (W.ndim - 1))
+    else:
+        _, Wb = oracle.binary_connect_convolution(x, W, None, pad, stride, dil, group, q0)
+        alpha, Ws = None, Wb
+    assert Wb.ravel()[0] == -1.0 and Wb.ravel()[1] == -1.0 and Wb.ravel()[2] == 1.0
+    y = oracle.convolution(x, Ws, None, pad, stride, dil, group)
+    dy = _rand(y.shape, 23)
+    rdx, rdw, rdb = _torch_conv_grads(x, Ws, np.zeros(ws[0], np.float32), dy, pad, stride, dil, group)
+    dx, dw, db = oracle.binary_convolution_backward(dy, x, W, alpha, pad, stride, dil, group, q0)
+    np.testing.assert_allclose(dx, rdx, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(dw, rdw, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(db, rdb, rtol=2e-5, atol=2e-5)
+    ow = _rand(ws, 24)
+    _, aw, _ = oracle.binary_convolution_backward(dy, x, W, alpha, pad, stride, dil, group, q0, dW=ow)
+    np.testing.assert_allclose(aw, ow + rdw, rtol=2e-5, atol=2e-5)
