@@ -226,6 +226,65 @@ void BinaryConnectConvolutionHip<T>::forward_impl(const Variables &inputs, const
       nullptr));
 }
 
+namespace {
+// Shared body of the convolution backward passes: `bias_index` is the position of the bias among the inputs.
+template <typename T, typename Call>
+void conv_backward_common(const Context &ctx, const ConvShapes &s, const Variables &inputs, const Variables &outputs,
+                          const vector<bool> &propagate_down, const vector<bool> &accum, int bias_index, Call call) {
+  const bool has_bias = (int)inputs.size() > bias_index;
+  const bool pb = has_bias && propagate_down[bias_index];
+  if (!(propagate_down[0] || propagate_down[1] || pb))
+    return;
+  hip_set_device(ctx);
+  const T *x = inputs[0]->get_data_pointer<T>(ctx);
+  const T *dy = outputs[0]->get_grad_pointer<T>(ctx);
+  T *dx = propagate_down[0] ? inputs[0]->cast_grad_and_get_pointer<T>(ctx, !accum[0]) : nullptr;
+  T *dw = propagate_down[1] ? inputs[1]->cast_grad_and_get_pointer<T>(ctx, !accum[1]) : nullptr;
+  T *db = pb ? inputs[bias_index]->cast_grad_and_get_pointer<T>(ctx, !accum[bias_index]) : nullptr;
+  HipWorkspace ws(nbla_hip_convolution_backward_workspace_bytes(s.outer, s.channels_i, s.spatial_dims,
+                                                                s.spatial_i.data(), s.channels_o, s.kernel.data(),
+                                                                s.pad.data(), s.stride.data(), s.dilation.data(),
+                                                                s.group),
+                  ctx);
+  call(dy, x, dx, dw, db, (int)accum[0], (int)accum[1], has_bias ? (int)accum[bias_index] : 0, ws);
+}
+} // namespace
+
+// binary_weight_convolution.cpp:119-142
+template <typename T>
+void BinaryWeightConvolutionHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                                  const vector<bool> &propagate_down, const vector<bool> &accum) {
+  const ConvShapes &s = this->shapes_;
+  conv_backward_common<T>(
+      this->ctx_, s, inputs, outputs, propagate_down, accum, 4,
+      [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
+        const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
+        const T *wb = inputs[2]->get_data_pointer<T>(this->ctx_);
+        const T *alpha = inputs[3]->get_data_pointer<T>(this->ctx_);
+        NBLA_HIP_CALL(nbla_hip_binary_convolution_backward_f32(
+            dy, x, w, wb, alpha, dx, dw, db, s.outer, s.channels_i, s.spatial_dims, s.spatial_i.data(), s.channels_o,
+            s.kernel.data(), s.pad.data(), s.stride.data(), s.dilation.data(), s.group, this->quantize_zero_to_, ax, aw,
+            ab, ws.pointer(), ws.bytes(), nullptr));
+      });
+}
+
+// binary_connect_convolution.cpp:83-103
+template <typename T>
+void BinaryConnectConvolutionHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                                   const vector<bool> &propagate_down, const vector<bool> &accum) {
+  const ConvShapes &s = this->shapes_;
+  conv_backward_common<T>(
+      this->ctx_, s, inputs, outputs, propagate_down, accum, 3,
+      [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
+        const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
+        const T *wb = inputs[2]->get_data_pointer<T>(this->ctx_);
+        NBLA_HIP_CALL(nbla_hip_binary_convolution_backward_f32(
+            dy, x, w, wb, nullptr, dx, dw, db, s.outer, s.channels_i, s.spatial_dims, s.spatial_i.data(), s.channels_o,
+            s.kernel.data(), s.pad.data(), s.stride.data(), s.dilation.data(), s.group, this->quantize_zero_to_, ax, aw,
+            ab, ws.pointer(), ws.bytes(), nullptr));
+      });
+}
+
 // ----------------------------------------------------------------------- INQ
 namespace {
 // The Bernoulli stream of inq_affine.cpp:147: rdist_(rgen), one draw per learnable weight.
@@ -316,6 +375,22 @@ void INQAffineHip<T, T1>::backward_impl(const Variables &inputs, const Variables
                               NBLA_HIP_CALL(nbla_hip_affine_backward_f32(dy, x, w, dx, dw, db, s.i_row, s.i_col, s.w_col,
                                                                          ax, aw, ab, ws.pointer(), ws.bytes(), nullptr));
                             });
+}
+
+// inq_convolution.cpp:220-232
+template <typename T, typename T1>
+void INQConvolutionHip<T, T1>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                             const vector<bool> &propagate_down, const vector<bool> &accum) {
+  const ConvShapes &s = this->shapes_;
+  conv_backward_common<T>(
+      this->ctx_, s, inputs, outputs, propagate_down, accum, 3,
+      [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
+        const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
+        NBLA_HIP_CALL(nbla_hip_convolution_backward_f32(
+            dy, x, w, dx, dw, db, s.outer, s.channels_i, s.spatial_dims, s.spatial_i.data(), s.channels_o,
+            s.kernel.data(), s.pad.data(), s.stride.data(), s.dilation.data(), s.group, ax, aw, ab, ws.pointer(),
+            ws.bytes(), nullptr));
+      });
 }
 
 // affine.cpp:98-140

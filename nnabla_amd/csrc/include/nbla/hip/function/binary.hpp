@@ -43,6 +43,8 @@ public:
 
 protected:
   virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+  virtual void backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                             const vector<bool> &accum);
 };
 
 template <typename T> class BinaryConnectConvolutionHip : public BinaryConnectConvolution<T> {
@@ -54,6 +56,8 @@ public:
 
 protected:
   virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+  virtual void backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                             const vector<bool> &accum);
 };
 
 } // namespace nbla

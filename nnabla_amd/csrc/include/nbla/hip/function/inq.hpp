@@ -37,6 +37,8 @@ public:
 protected:
   virtual void forward_impl(const Variables &inputs, const Variables &outputs);
   virtual void recompute_impl(const Variables &inputs, const Variables &outputs);
+  virtual void backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                             const vector<bool> &accum);
   void run(const Variables &inputs, const Variables &outputs, int step);
 };
 

@@ -384,3 +384,38 @@ def test_inq_affine_backward_through_the_registry(ctx):
     rdx, rdw, _ = oracle.affine_backward(gy, x, Wq, want=(True, True, False))
     assert max_rel_err(vx.g, rdx) <= TIGHT
     assert max_rel_err(vW.g, rdw) <= TIGHT
+
+
+def test_convolution_backward_through_the_registry(ctx):
+    """BinaryWeightConvolution -> ReLU -> BinaryConnectConvolution -> INQConvolution, backward through the graph."""
+    rng = np.random.RandomState(19)
+    x = rng.randn(3, 4, 10, 9).astype(np.float32)
+    W1 = (rng.randn(8, 4, 3, 3) * 0.05).astype(np.float32)
+    b1 = rng.randn(8).astype(np.float32)
+    W2 = (rng.randn(6, 4, 3, 2) * 0.05).astype(np.float32)
+    W3 = (rng.randn(5, 6, 2, 2) * 0.05).astype(np.float32)
+    vx, vW1, vb1, vW2, vW3 = [nn.Variable.from_numpy_array(a, need_grad=True) for a in (x, W1, b1, W2, W3)]
+    for v in (vx, vW1, vb1, vW2, vW3):
+        v.zero_grad()
+    vI = nn.Variable(W3.shape)
+    vI.set_data(np.ones(W3.shape), np.int32)
+    alpha1 = nn.Variable((8,))
+    c1 = F.binary_weight_convolution(vx, vW1, nn.Variable(W1.shape), alpha1, vb1, pad=(1, 1), stride=(2, 1))
+    h = F.relu(c1)
+    c2 = F.binary_connect_convolution(h, vW2, nn.Variable(W2.shape), None, pad=(1, 0), group=2)
+    y = F.inq_convolution(c2, vW3, vI, None, num_bits=4, inq_iterations=())
+    y.forward()
+    gy = rng.randn(*y.shape).astype(np.float32)
+    y.backward(gy)
+
+    hv, c2v, W3q = h.d, c2.d, vW3.d
+    g_c2, g_W3, _ = oracle.convolution_backward(gy, c2v, W3q, want=(True, True, False))
+    g_h, g_W2, _ = oracle.binary_convolution_backward(g_c2, hv, W2, None, (1, 0), None, None, 2, 1.0,
+                                                      want=(True, True, False))
+    g_c1 = np.where(hv > 0, g_h, 0).astype(np.float32)
+    g_x, g_W1, g_b1 = oracle.binary_convolution_backward(g_c1, x, W1, alpha1.d, (1, 1), (2, 1), None, 1, 1.0)
+    assert max_rel_err(vW3.g, g_W3) <= TIGHT
+    assert max_rel_err(vW2.g, g_W2) <= TIGHT * 2
+    assert max_rel_err(vW1.g, g_W1) <= TIGHT * 4
+    assert max_rel_err(vb1.g, g_b1) <= TIGHT * 4
+    assert max_rel_err(vx.g, g_x) <= TIGHT * 4
