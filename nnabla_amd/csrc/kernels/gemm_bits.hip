@@ -48,18 +48,6 @@ struct GemmBitsArgs {
   int finish;     // apply alpha and bias (last k chunk)
 };
 
-// Blocks are handed to the 8 XCDs round-robin; give each XCD a contiguous run
-// of tiles (n fastest) so that blocks resident on one XCD share an X panel in
-// that XCD's L2.
-__device__ __forceinline__ int64_t xcd_remap(int64_t b, int64_t total) {
-  constexpr int64_t kXcds = 8;
-  const int64_t per = total / kXcds, rem = total % kXcds;
-  const int64_t xcd = b % kXcds, slot = b / kXcds;
-  // XCDs [0, rem) own per+1 tiles, the rest own per tiles.
-  const int64_t start = xcd * per + (xcd < rem ? xcd : rem);
-  return start + slot;
-}
-
 // LDS buffers (stages resident) per tile shape: what fits the block's share of the CU's 160 KiB, at most six.
 constexpr int gemm_bits_stage_bytes(int BM, int BN, int waves_k) {
   return ((BM / 32) * 2 * kDigits * kFragBytes + 2 * BN * 4) * waves_k;
@@ -150,11 +138,8 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
   // Tiles are walked in bands of kBand block rows, column by column inside a band: the blocks resident on an XCD at
   // one time then cover about kBand x kBand tiles, so its L2 serves each digit panel and each packed panel to
   // several blocks instead of streaming the whole packed operand once per block row.
-  constexpr int64_t kBand = 8;
-  const int64_t tile = xcd_remap(blockIdx.x, a.blocks_m * a.blocks_n);
-  const int64_t band = tile / (kBand * a.blocks_n), in_band = tile - band * (kBand * a.blocks_n);
-  const int64_t band_rows = (a.blocks_m - band * kBand < kBand) ? a.blocks_m - band * kBand : kBand;
-  const int64_t bn = in_band / band_rows, bm = band * kBand + (in_band - bn * band_rows);
+  int64_t bm, bn;
+  band_tile<8>(blockIdx.x, a.blocks_m, a.blocks_n, bm, bn);
 
   // Sources of this wavefront's copies (uniform bases; the lane adds its own 16 bytes).  Row blocks / wide groups
   // past the end of the operand are clamped: their products land in rows/columns that are not stored.

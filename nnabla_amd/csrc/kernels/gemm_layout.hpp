@@ -94,4 +94,30 @@ __host__ __device__ inline DigitOperand digit_operand(int64_t M, int64_t K) {
   return d;
 }
 
+#if defined(__HIPCC__)
+// Blocks are handed to the 8 XCDs round-robin; give each XCD a contiguous run
+// of tiles (n fastest) so that blocks resident on one XCD share an X panel in
+// that XCD's L2.
+__device__ __forceinline__ int64_t xcd_remap(int64_t b, int64_t total) {
+  constexpr int64_t kXcds = 8;
+  const int64_t per = total / kXcds, rem = total % kXcds;
+  const int64_t xcd = b % kXcds, slot = b / kXcds;
+  // XCDs [0, rem) own per+1 tiles, the rest own per tiles.
+  const int64_t start = xcd * per + (xcd < rem ? xcd : rem);
+  return start + slot;
+}
+
+// Tile (bm, bn) of block b: an XCD's run of tiles is walked in bands of kBand tile rows, column by column inside a
+// band, so the blocks resident on an XCD at one time cover a compact patch of tiles and its L2 serves each row
+// panel and each column panel to several of them.
+template <int kBand>
+__device__ __forceinline__ void band_tile(int64_t b, int64_t blocks_m, int64_t blocks_n, int64_t &bm, int64_t &bn) {
+  const int64_t tile = xcd_remap(b, blocks_m * blocks_n);
+  const int64_t band = tile / (kBand * blocks_n), in_band = tile - band * (kBand * blocks_n);
+  const int64_t band_rows = (blocks_m - band * kBand < kBand) ? blocks_m - band * kBand : kBand;
+  bn = in_band / band_rows;
+  bm = band * kBand + (in_band - bn * band_rows);
+}
+#endif
+
 } // namespace nbla_hip

@@ -141,7 +141,9 @@ __global__ __launch_bounds__(kThreads) void gemm_planes_kernel(GemmPlanesArgs a)
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave & 1, wn = wave >> 1;
-  const int64_t bm = blockIdx.x / a.blocks_n, bn = blockIdx.x - bm * a.blocks_n;
+  // one block per CU (98 KiB of LDS): the 32 blocks resident on an XCD cover 4 x 8 tiles
+  int64_t bm, bn;
+  band_tile<4>(blockIdx.x, a.blocks_m, a.blocks_n, bm, bn);
   f32x16_t acc[2][2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
