@@ -364,6 +364,57 @@ int nbla_hip_convolution_backward_f32(
     const int64_t *dilation, int64_t group, int accum_x, int accum_w,
     int accum_b, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ------------------------------------------ QuantizeLinear / DequantizeLinear / Prune */
+
+#define NBLA_HIP_DTYPE_BYTE 1  /* nbla::dtypes::BYTE  (int8 range)  */
+#define NBLA_HIP_DTYPE_UBYTE 2 /* nbla::dtypes::UBYTE (uint8 range) */
+
+/* y = saturate(round(x / scale) + zp') with zp' = saturate(round(zero_point))
+ * written back into zero_point, every step rounded in fp32 on its own;
+ * round is std::round (half_to_even == 0, "HALF_AWAY_FROM_ZERO") or round-half-
+ * to-even ("HALF_TO_EVEN"); the range is [-128,127] / [0,255] for BYTE / UBYTE,
+ * [-127,127] / [1,255] with narrow_range.  scale and zero_point have x's number
+ * of dimensions with each size 1 (broadcast) or equal to x's.  Replaces
+ * QuantizeLinear<float>::forward_impl, quantize_linear.cpp:25-117 (setup checks
+ * :28-46 -> NBLA_HIP_ERR_VALUE). */
+int nbla_hip_quantize_linear_f32(const float *x, const float *scale,
+                                 float *zero_point, float *y,
+                                 const int64_t *xshape,
+                                 const int64_t *scale_shape,
+                                 const int64_t *zero_point_shape, int ndim,
+                                 int half_to_even, int narrow_range, int dtype,
+                                 void *stream);
+/* dx (+)= dy / scale.  Replaces the x branch of
+ * QuantizeLinear<float>::backward_impl, quantize_linear.cpp:119-156 (gradients
+ * of scale and zero point are not_implemented there too). */
+int nbla_hip_quantize_linear_backward_f32(const float *dy, const float *scale,
+                                          float *dx, const int64_t *xshape,
+                                          const int64_t *scale_shape, int ndim,
+                                          int accum, void *stream);
+
+/* y = (x - zero_point) * scale.  Replaces
+ * DequantizeLinear<float>::forward_impl, dequantize_linear.cpp:25-67. */
+int nbla_hip_dequantize_linear_f32(const float *x, const float *scale,
+                                   const float *zero_point, float *y,
+                                   const int64_t *xshape,
+                                   const int64_t *scale_shape,
+                                   const int64_t *zero_point_shape, int ndim,
+                                   void *stream);
+/* dx (+)= dy * scale.  dequantize_linear.cpp:69-108. */
+int nbla_hip_dequantize_linear_backward_f32(const float *dy, const float *scale,
+                                            float *dx, const int64_t *xshape,
+                                            const int64_t *scale_shape,
+                                            int ndim, int accum, void *stream);
+
+/* Prune: y = (|x| < t) ? 0 : x with t = the (int)((size-1)*rate)-th smallest
+ * |x| (+1 when rate == 1).  Replaces Prune<float>::forward_impl,
+ * prune.cpp:27-70 (the full sort there is replaced by a radix select of that
+ * one order statistic).  Its backward is the identity (prune.cpp:72-90):
+ * use nbla_hip_fixed_point_quantize_backward_f32 with ste_fine_grained = 0. */
+size_t nbla_hip_prune_workspace_bytes(void);
+int nbla_hip_prune_f32(const float *x, float *y, size_t size, float rate,
+                       void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---------------------------------------------------------------------- INQ */
 
 /* INQ step selector (what the forward does to the indicators before quantizing):

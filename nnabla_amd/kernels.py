@@ -34,6 +34,8 @@ EXPORTED = (
     "nbla_hip_binary_weight_convolution_f32", "nbla_hip_binary_connect_convolution_f32",
     "nbla_hip_convolution_backward_workspace_bytes", "nbla_hip_binary_convolution_backward_f32",
     "nbla_hip_convolution_backward_f32",
+    "nbla_hip_quantize_linear_f32", "nbla_hip_quantize_linear_backward_f32", "nbla_hip_dequantize_linear_f32",
+    "nbla_hip_dequantize_linear_backward_f32", "nbla_hip_prune_workspace_bytes", "nbla_hip_prune_f32",
     "nbla_hip_inq_workspace_bytes", "nbla_hip_inq_update_weights_f32", "nbla_hip_inq_affine_workspace_bytes",
     "nbla_hip_inq_affine_f32", "nbla_hip_inq_convolution_workspace_bytes", "nbla_hip_inq_convolution_f32",
     "nbla_hip_get_device_count", "nbla_hip_set_device", "nbla_hip_malloc", "nbla_hip_free", "nbla_hip_mem_info",
@@ -64,7 +66,7 @@ def lib():
         for name in ("nbla_hip_min_max_quantize_workspace_bytes", "nbla_hip_packed_bits_bytes",
                      "nbla_hip_min_max_quantize_backward_workspace_bytes",
                      "nbla_hip_affine_backward_workspace_bytes",
-                     "nbla_hip_convolution_backward_workspace_bytes",
+                     "nbla_hip_convolution_backward_workspace_bytes", "nbla_hip_prune_workspace_bytes",
                      "nbla_hip_split_operand_bytes", "nbla_hip_digit_operand_bytes",
                      "nbla_hip_binarize_workspace_bytes",
                      "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_convolution_workspace_bytes",
@@ -385,6 +387,49 @@ def convolution_backward(dy, x, W, pad=None, stride=None, dilation=None, group=1
     check(lib().nbla_hip_convolution_backward_f32(_p(dy), _p(x), _p(W), _p(odx), _p(odw), _p(odb), *geom, ax, aw, ab,
                                                   _p(ws), ctypes.c_size_t(ws.numel()), _stream(stream)))
     return odx, odw, odb
+
+
+# ------------------------------------------------------- QuantizeLinear / DequantizeLinear / Prune
+
+DTYPE_BYTE, DTYPE_UBYTE = 1, 2
+
+
+def quantize_linear(x, scale, zero_point, round_mode="HALF_AWAY_FROM_ZERO", narrow_range=False, dtype=DTYPE_BYTE,
+                    stream=None):
+    """y = saturate(round(x / scale) + zero_point); ``zero_point`` is rounded and saturated in place."""
+    import torch
+    y = torch.empty_like(x)
+    check(lib().nbla_hip_quantize_linear_f32(_p(x), _p(scale), _p(zero_point), _p(y), _shape(x.shape),
+                                             _shape(scale.shape), _shape(zero_point.shape), x.dim(),
+                                             int(round_mode == "HALF_TO_EVEN"), int(narrow_range), int(dtype),
+                                             _stream(stream)))
+    return y
+
+
+def dequantize_linear(x, scale, zero_point, stream=None):
+    import torch
+    y = torch.empty_like(x)
+    check(lib().nbla_hip_dequantize_linear_f32(_p(x), _p(scale), _p(zero_point), _p(y), _shape(x.shape),
+                                               _shape(scale.shape), _shape(zero_point.shape), x.dim(),
+                                               _stream(stream)))
+    return y
+
+
+def linear_quantize_backward(dy, scale, dequantize=False, dx=None, stream=None):
+    """dx (+)= dy / scale (QuantizeLinear) or dy * scale (DequantizeLinear)."""
+    out, accum = _grad_out(dy, dx)
+    fn = lib().nbla_hip_dequantize_linear_backward_f32 if dequantize else lib().nbla_hip_quantize_linear_backward_f32
+    check(fn(_p(dy), _p(scale), _p(out), _shape(dy.shape), _shape(scale.shape), dy.dim(), accum, _stream(stream)))
+    return out
+
+
+def prune(x, rate=0.9, workspace=None, stream=None):
+    import torch
+    y = torch.empty_like(x)
+    ws = workspace if workspace is not None else _workspace(lib().nbla_hip_prune_workspace_bytes(), x)
+    check(lib().nbla_hip_prune_f32(_p(x), _p(y), ctypes.c_size_t(x.numel()), ctypes.c_float(rate), _p(ws),
+                                   ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return y
 
 
 # ---------------------------------------------------------------------------- INQ

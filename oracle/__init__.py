@@ -341,6 +341,48 @@ def binary_convolution_backward(dy, x, W, alpha=None, pad=None, stride=None, dil
     return odx, odw, odb
 
 
+def _bshapes(x, scale, zero_point):
+    x, scale, zero_point = _f32(x), _f32(scale), _f32(zero_point)
+    assert x.ndim == scale.ndim == zero_point.ndim
+    return x, scale, zero_point
+
+
+def quantize_linear(x, scale, zero_point, round_mode="HALF_AWAY_FROM_ZERO", narrow_range=False, dtype=1):
+    """Returns (y, zero_point after its in-place rounding); quantize_linear.cpp:97-117."""
+    x, scale, zero_point = _bshapes(x, scale, zero_point)
+    zp = zero_point.copy()
+    y = np.empty_like(x)
+    _check(lib().orc_quantize_linear(_fp(x), _fp(scale), _fp(zp), _fp(y), _longs(x.shape), _longs(scale.shape),
+                                     _longs(zp.shape), x.ndim, int(round_mode == "HALF_TO_EVEN"), int(narrow_range),
+                                     int(dtype)), "quantize_linear")
+    return y, zp
+
+
+def dequantize_linear(x, scale, zero_point):
+    x, scale, zero_point = _bshapes(x, scale, zero_point)
+    y = np.empty_like(x)
+    _check(lib().orc_dequantize_linear(_fp(x), _fp(scale), _fp(zero_point), _fp(y), _longs(x.shape),
+                                       _longs(scale.shape), _longs(zero_point.shape), x.ndim), "dequantize_linear")
+    return y
+
+
+def linear_quantize_backward(dy, scale, dequantize=False, dx=None):
+    """dx (+)= dy / scale (QuantizeLinear) or dy * scale (DequantizeLinear)."""
+    dy, scale = _f32(dy), _f32(scale)
+    out = np.zeros_like(dy) if dx is None else _f32(dx).copy()
+    _check(lib().orc_linear_quantize_backward(_fp(dy), _fp(scale), _fp(out), _longs(dy.shape), _longs(scale.shape),
+                                              dy.ndim, int(dequantize), int(dx is not None)),
+           "linear_quantize_backward")
+    return out
+
+
+def prune(x, rate=0.9):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _check(lib().orc_prune(_fp(x), _fp(y), ctypes.c_long(x.size), ctypes.c_float(rate)), "prune")
+    return y
+
+
 class Inq(object):
     """Stateful INQ weight logic (one object per INQAffine / INQConvolution)."""
 

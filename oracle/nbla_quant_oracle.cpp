@@ -1001,6 +1001,116 @@ int orc_binary_convolution_backward(const float *dy, const float *x, const float
 }
 
 // ---------------------------------------------------------------------------
+// QuantizeLinear / DequantizeLinear / Prune.
+// ---------------------------------------------------------------------------
+namespace {
+// Offset into a broadcast parameter (sizes 1 or equal to x's) of x's flat index i.
+long bcast_offset(long i, const long *xshape, const long *pshape, int ndim) {
+  long off = 0, mul = 1;
+  for (int d = ndim - 1; d >= 0; --d) {
+    const long c = i % xshape[d];
+    i /= xshape[d];
+    if (pshape[d] != 1) {
+      off += c * mul;
+      mul *= pshape[d];
+    }
+  }
+  return off;
+}
+// QuantizeLinear<T>::round, quantize_linear.cpp:78-95.
+float ql_round(float v, int half_to_even) {
+  if (!half_to_even)
+    return std::round(v);
+  const float t = std::round(v);
+  if (std::abs(v - t) == 0.5)
+    return (float)(std::round(v * 0.5) * 2);
+  return t;
+}
+float ql_saturate(float v, int lo, int hi) { return v < lo ? (float)lo : (v > hi ? (float)hi : v); }
+} // namespace
+
+// QuantizeLinear<T>::forward_impl, quantize_linear.cpp:97-117 with the ranges of setup_impl :52-60; dtype 1 = BYTE,
+// 2 = UBYTE.  zero_point is rounded and saturated in place, as the reference does to its input.
+int orc_quantize_linear(const float *x, const float *scale, float *zero_point, float *y,
+                        const long *xshape, const long *sshape, const long *zshape, int ndim,
+                        int half_to_even, int narrow_range, int dtype) {
+  int lo, hi;
+  if (dtype == 1) {
+    lo = narrow_range ? -127 : -128, hi = 127;
+  } else if (dtype == 2) {
+    lo = narrow_range ? 1 : 0, hi = 255;
+  } else {
+    return ORC_ERR_VALUE;
+  }
+  long size = 1, zsize = 1;
+  for (int d = 0; d < ndim; ++d) {
+    if ((sshape[d] != 1 && sshape[d] != xshape[d]) || (zshape[d] != 1 && zshape[d] != xshape[d]))
+      return ORC_ERR_VALUE;
+    size *= xshape[d];
+    zsize *= zshape[d];
+  }
+  for (long i = 0; i < size; ++i)
+    y[i] = x[i] / scale[bcast_offset(i, xshape, sshape, ndim)]; // Div2
+  for (long i = 0; i < size; ++i)
+    y[i] = ql_round(y[i], half_to_even);
+  for (long i = 0; i < zsize; ++i)
+    zero_point[i] = ql_saturate(ql_round(zero_point[i], half_to_even), lo, hi);
+  for (long i = 0; i < size; ++i)
+    y[i] = y[i] + zero_point[bcast_offset(i, xshape, zshape, ndim)]; // Add2
+  for (long i = 0; i < size; ++i)
+    y[i] = ql_saturate(y[i], lo, hi);
+  return ORC_OK;
+}
+
+// DequantizeLinear<T>::forward_impl, dequantize_linear.cpp:55-67: Sub2 then Mul2.
+int orc_dequantize_linear(const float *x, const float *scale, const float *zero_point, float *y,
+                          const long *xshape, const long *sshape, const long *zshape, int ndim) {
+  long size = 1;
+  for (int d = 0; d < ndim; ++d) {
+    if ((sshape[d] != 1 && sshape[d] != xshape[d]) || (zshape[d] != 1 && zshape[d] != xshape[d]))
+      return ORC_ERR_VALUE;
+    size *= xshape[d];
+  }
+  for (long i = 0; i < size; ++i)
+    y[i] = x[i] - zero_point[bcast_offset(i, xshape, zshape, ndim)];
+  for (long i = 0; i < size; ++i)
+    y[i] = y[i] * scale[bcast_offset(i, xshape, sshape, ndim)];
+  return ORC_OK;
+}
+
+// x branch of the two backward passes (quantize_linear.cpp:137-147: dy / scale; dequantize_linear.cpp:88-98:
+// dy * scale), added to dx when accum.
+int orc_linear_quantize_backward(const float *dy, const float *scale, float *dx, const long *xshape,
+                                 const long *sshape, int ndim, int dequantize, int accum) {
+  long size = 1;
+  for (int d = 0; d < ndim; ++d)
+    size *= xshape[d];
+  for (long i = 0; i < size; ++i) {
+    const float s = scale[bcast_offset(i, xshape, sshape, ndim)];
+    const float g = dequantize ? dy[i] * s : dy[i] / s;
+    dx[i] = accum ? dx[i] + g : g;
+  }
+  return ORC_OK;
+}
+
+// Prune<T>::setup_impl / forward_impl, prune.cpp:27-70.
+int orc_prune(const float *x, float *y, long size, float rate) {
+  if (!(rate >= 0 && rate <= 1))
+    return ORC_ERR_VALUE;
+  if (size == 0)
+    return ORC_OK;
+  const int x_size = (int)size;
+  const int thresh_idx = (int)((x_size - 1) * rate);
+  std::vector<float> buffer(x, x + size);
+  std::sort(buffer.begin(), buffer.end(), [](float i, float j) { return std::abs(i) < std::abs(j); });
+  float thresh_val = std::abs(buffer[thresh_idx]);
+  thresh_val += rate == 1.0 ? 1.0 : 0.0;
+  for (long s = 0; s < size; ++s)
+    y[s] = (std::abs(x[s]) < thresh_val) ? 0.0f : x[s];
+  return ORC_OK;
+}
+
+// ---------------------------------------------------------------------------
 // INQ (INQAffine / INQConvolution share the weight logic).
 //   inq_affine.cpp:34-79 (setup), :82-205 (forward), inq_convolution.cpp:35-238.
 // ---------------------------------------------------------------------------

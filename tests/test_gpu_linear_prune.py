@@ -1,0 +1,103 @@
+"""QuantizeLinear / DequantizeLinear / Prune on the GPU against the CPU oracle: bit-exact (every step of the
+reference chain is a separately rounded fp32 operation; Prune's threshold is an order statistic)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from nnabla_amd import kernels
+from util import bits_equal, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def _rand(shape, seed, scale=1.0):
+    return (np.random.RandomState(seed).randn(*shape) * scale).astype(np.float32)
+
+
+SHAPES = [
+    # (x shape, scale shape, zero-point shape)
+    ((3, 5, 7), (1, 1, 1), (1, 1, 1)),
+    ((3, 5, 7), (1, 5, 1), (1, 5, 1)),
+    ((3, 5, 8), (3, 1, 1), (1, 1, 8)),
+    ((3, 5, 8), (3, 5, 8), (1, 5, 1)),
+    ((4, 16, 6, 6), (1, 16, 1, 1), (1, 16, 1, 1)),
+    ((2, 3, 4, 5, 6, 8), (2, 1, 4, 1, 6, 1), (1, 3, 1, 5, 1, 8)),
+    ((64, 4096), (1, 1), (1, 1)),
+    ((64, 4096), (1, 4096), (1, 1)),
+    ((1000,), (1,), (1,)),
+    ((1, 1), (1, 1), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("xs,ss,zs", SHAPES)
+@pytest.mark.parametrize("mode,narrow,dtype", [("HALF_AWAY_FROM_ZERO", False, 1), ("HALF_TO_EVEN", True, 1),
+                                               ("HALF_TO_EVEN", False, 2), ("HALF_AWAY_FROM_ZERO", True, 2)])
+def test_quantize_linear(dev, xs, ss, zs, mode, narrow, dtype):
+    x = _rand(xs, 1, 60.0)
+    x.ravel()[:6] = [0.5, 1.5, 2.5, -0.5, -1.5, -2.5][:min(6, x.size)]
+    scale = (np.abs(_rand(ss, 2)) + 0.25).astype(np.float32)
+    if int(np.prod(ss)) == 1:
+        scale[...] = 0.5
+    zp = _rand(zs, 3, 40.0)
+    ref, ref_zp = oracle.quantize_linear(x, scale, zp, mode, narrow, dtype)
+    dzp = _dev(zp, dev)
+    y = kernels.quantize_linear(_dev(x, dev), _dev(scale, dev), dzp, mode, narrow, dtype)
+    assert bits_equal(to_np(y), ref)
+    assert bits_equal(to_np(dzp), ref_zp)                          # rounded and saturated in place
+
+
+@pytest.mark.parametrize("xs,ss,zs", SHAPES)
+def test_dequantize_linear_and_backward(dev, xs, ss, zs):
+    x = np.rint(_rand(xs, 4, 50.0)).astype(np.float32)
+    scale = (np.abs(_rand(ss, 5)) + 0.1).astype(np.float32)
+    zp = np.rint(_rand(zs, 6, 5.0)).astype(np.float32)
+    y = kernels.dequantize_linear(_dev(x, dev), _dev(scale, dev), _dev(zp, dev))
+    assert bits_equal(to_np(y), oracle.dequantize_linear(x, scale, zp))
+    dy, old = _rand(xs, 7), _rand(xs, 8)
+    for deq in (False, True):
+        g = kernels.linear_quantize_backward(_dev(dy, dev), _dev(scale, dev), deq)
+        assert bits_equal(to_np(g), oracle.linear_quantize_backward(dy, scale, deq))
+        acc = _dev(old, dev)
+        kernels.linear_quantize_backward(_dev(dy, dev), _dev(scale, dev), deq, dx=acc)
+        assert bits_equal(to_np(acc), oracle.linear_quantize_backward(dy, scale, deq, dx=old))
+
+
+def test_quantize_linear_rejects_bad_arguments(dev):
+    x, one = _dev(np.zeros((2, 3), np.float32), dev), _dev(np.ones((1, 1), np.float32), dev)
+    with pytest.raises(kernels.KernelError) as e:
+        kernels.quantize_linear(x, one, one.clone(), dtype=5)
+    assert e.value.code == kernels.ERR_VALUE
+    with pytest.raises(kernels.KernelError) as e:
+        kernels.quantize_linear(x, _dev(np.ones((2, 2), np.float32), dev), one.clone())
+    assert e.value.code == kernels.ERR_VALUE
+
+
+@pytest.mark.parametrize("size", [1, 7, 1000, 4097, 1 << 20])
+@pytest.mark.parametrize("rate", [0.0, 0.33, 0.5, 0.9, 1.0])
+def test_prune(dev, size, rate):
+    x = _rand((size,), 9, 3.0)
+    if size > 20:
+        x[::7] = x[3]
+        x[::14] = -x[3]
+        x[5] = 0.0
+        x[6] = -0.0
+    y = kernels.prune(_dev(x, dev), rate)
+    assert bits_equal(to_np(y), oracle.prune(x, rate))
+
+
+def test_prune_large_and_special_values(dev):
+    """16.8 M elements (the FixedPointQuantize bench shape) with denormals and infinities; the radix select must land
+    on exactly the element a full sort would."""
+    rng = np.random.default_rng(313)
+    x = (rng.standard_normal((256, 65536)) * 2).astype(np.float32)
+    x.ravel()[:4] = [np.inf, -np.inf, 1e-42, -1e-42]
+    for rate in (0.5, 0.999):
+        y = kernels.prune(_dev(x, dev), rate)
+        assert bits_equal(to_np(y), oracle.prune(x, rate))
+    with pytest.raises(kernels.KernelError):
+        kernels.prune(_dev(x[:1], dev), 1.5)
