@@ -12,6 +12,7 @@
 #include <nbla/function/inq_convolution.hpp>
 #include <nbla/function/min_max_quantize.hpp>
 #include <nbla/function/pow2_quantize.hpp>
+#include <nbla/function/quantize_linear.hpp>
 #include <nbla/hip/init.hpp>
 #include <nbla/init.hpp>
 
@@ -125,6 +126,16 @@ FunctionPtr create_by_name(const string &name, const Context &ctx, const int64_t
   if (name == "ReLU") {
     need(1, 0);
     return create_ReLU(ctx, ia[0] != 0);
+  }
+  if (name == "QuantizeLinear") {
+    need(2, 0);
+    return create_QuantizeLinear(ctx, sarg, ia[0] != 0, (int)ia[1]);
+  }
+  if (name == "DequantizeLinear")
+    return create_DequantizeLinear(ctx);
+  if (name == "Prune") {
+    need(0, 1);
+    return create_Prune(ctx, (float)fa[0]);
   }
   NBLA_ERROR(error_code::value, "Unknown function '%s'.", name.c_str());
 }

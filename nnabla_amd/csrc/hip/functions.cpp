@@ -4,6 +4,7 @@
 #include <nbla/hip/function/binary.hpp>
 #include <nbla/hip/function/inq.hpp>
 #include <nbla/hip/function/quantize.hpp>
+#include <nbla/hip/function/quantize_linear.hpp>
 
 namespace nbla {
 
@@ -426,6 +427,99 @@ template <typename T> void ReLUHip<T>::forward_impl(const Variables &inputs, con
   NBLA_HIP_CALL(nbla_hip_relu_f32(x, y, (size_t)inputs[0]->size(), nullptr));
 }
 
+// ------------------------------------------- QuantizeLinear / DequantizeLinear / Prune
+namespace {
+vector<int64_t> shape64(const Variable *v) {
+  const Shape_t s = v->shape();
+  return vector<int64_t>(s.begin(), s.end());
+}
+} // namespace
+
+// quantize_linear.cpp:97-117
+template <typename T> void QuantizeLinearHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const T *scale = inputs[1]->get_data_pointer<T>(this->ctx_);
+  T *zp = inputs[2]->cast_data_and_get_pointer<T>(this->ctx_, false); // rounded and saturated in place
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  const vector<int64_t> xs = shape64(inputs[0]), ss = shape64(inputs[1]), zs = shape64(inputs[2]);
+  NBLA_HIP_CALL(nbla_hip_quantize_linear_f32(x, scale, zp, y, xs.data(), ss.data(), zs.data(), (int)xs.size(),
+                                             this->round_mode_ == "HALF_TO_EVEN", this->narrow_range_, this->dtype_,
+                                             nullptr));
+}
+
+// quantize_linear.cpp:119-156
+template <typename T>
+void QuantizeLinearHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                         const vector<bool> &propagate_down, const vector<bool> &accum) {
+  if (!(propagate_down[0] || propagate_down[1] || propagate_down[2]))
+    return;
+  if (propagate_down[0]) {
+    hip_set_device(this->ctx_);
+    const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
+    const T *scale = inputs[1]->get_data_pointer<T>(this->ctx_);
+    T *dx = inputs[0]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[0]);
+    const vector<int64_t> xs = shape64(inputs[0]), ss = shape64(inputs[1]);
+    NBLA_HIP_CALL(nbla_hip_quantize_linear_backward_f32(dy, scale, dx, xs.data(), ss.data(), (int)xs.size(), accum[0],
+                                                        nullptr));
+  }
+  NBLA_CHECK(!propagate_down[1], error_code::not_implemented, "Backward w.r.t. the scale is not supported now.");
+  NBLA_CHECK(!propagate_down[2], error_code::not_implemented, "Backward w.r.t. the zero point is not supported now.");
+}
+
+// dequantize_linear.cpp:55-67
+template <typename T> void DequantizeLinearHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const T *scale = inputs[1]->get_data_pointer<T>(this->ctx_);
+  const T *zp = inputs[2]->get_data_pointer<T>(this->ctx_);
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  const vector<int64_t> xs = shape64(inputs[0]), ss = shape64(inputs[1]), zs = shape64(inputs[2]);
+  NBLA_HIP_CALL(nbla_hip_dequantize_linear_f32(x, scale, zp, y, xs.data(), ss.data(), zs.data(), (int)xs.size(),
+                                               nullptr));
+}
+
+// dequantize_linear.cpp:69-108
+template <typename T>
+void DequantizeLinearHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                           const vector<bool> &propagate_down, const vector<bool> &accum) {
+  if (!(propagate_down[0] || propagate_down[1] || propagate_down[2]))
+    return;
+  if (propagate_down[0]) {
+    hip_set_device(this->ctx_);
+    const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
+    const T *scale = inputs[1]->get_data_pointer<T>(this->ctx_);
+    T *dx = inputs[0]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[0]);
+    const vector<int64_t> xs = shape64(inputs[0]), ss = shape64(inputs[1]);
+    NBLA_HIP_CALL(nbla_hip_dequantize_linear_backward_f32(dy, scale, dx, xs.data(), ss.data(), (int)xs.size(),
+                                                          accum[0], nullptr));
+  }
+  NBLA_CHECK(!propagate_down[1], error_code::not_implemented, "Backward w.r.t. the scale is not supported now.");
+  NBLA_CHECK(!propagate_down[2], error_code::not_implemented, "Backward w.r.t. the zero point is not supported now.");
+}
+
+// prune.cpp:39-70
+template <typename T> void PruneHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  HipWorkspace ws(nbla_hip_prune_workspace_bytes(), this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_prune_f32(x, y, (size_t)inputs[0]->size(), this->rate_, ws.pointer(), ws.bytes(), nullptr));
+}
+
+// prune.cpp:72-90: the gradient passes through unchanged
+template <typename T>
+void PruneHip<T>::backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                                const vector<bool> &accum) {
+  if (!propagate_down[0])
+    return;
+  hip_set_device(this->ctx_);
+  const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
+  T *dx = inputs[0]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[0]);
+  NBLA_HIP_CALL(nbla_hip_fixed_point_quantize_backward_f32(dy, dy, dx, (size_t)inputs[0]->size(), 1, 8, 1.0f, 0,
+                                                           accum[0], nullptr));
+}
+
 // explicit instantiations for the "float" type config (function_types.yaml:483-509)
 template class FixedPointQuantizeHip<float>;
 template class Pow2QuantizeHip<float>;
@@ -438,5 +532,8 @@ template class INQAffineHip<float, int>;
 template class INQConvolutionHip<float, int>;
 template class AffineHip<float>;
 template class ReLUHip<float>;
+template class QuantizeLinearHip<float>;
+template class DequantizeLinearHip<float>;
+template class PruneHip<float>;
 
 } // namespace nbla

@@ -7,6 +7,7 @@
 #include <nbla/hip/function/binary.hpp>
 #include <nbla/hip/function/inq.hpp>
 #include <nbla/hip/function/quantize.hpp>
+#include <nbla/hip/function/quantize_linear.hpp>
 #include <nbla/hip/init.hpp>
 #include <nbla/init.hpp>
 
@@ -64,6 +65,9 @@ void init_hip() {
                               int);
   NBLA_REGISTER_FUNCTION_IMPL(Affine, AffineHip<float>, "hip:float", int);
   NBLA_REGISTER_FUNCTION_IMPL(ReLU, ReLUHip<float>, "hip:float", bool);
+  NBLA_REGISTER_FUNCTION_IMPL(QuantizeLinear, QuantizeLinearHip<float>, "hip:float", const string &, bool, int);
+  NBLA_REGISTER_FUNCTION_IMPL(DequantizeLinear, DequantizeLinearHip<float>, "hip:float");
+  NBLA_REGISTER_FUNCTION_IMPL(Prune, PruneHip<float>, "hip:float", float);
 }
 
 } // namespace nbla

@@ -1,5 +1,5 @@
 // QuantizeLinear, DequantizeLinear (broadcast scale / zero point, each arithmetic step rounded on its own as the
-// reference's chain of Div2 / round / Add2 / saturate does) and Prune (k-th smallest |x| by a three-pass radix
+// reference's chain of Div2 / round / Add2 / saturate does) and Prune (k-th smallest |x| by a four-pass radix
 // select over the magnitude bits, then a masked copy).  All HBM-bound; 128-bit accesses where the layout allows.
 #include "common.hpp"
 #include "gemm_layout.hpp"
@@ -54,15 +54,16 @@ bool make_broadcast(Broadcast &b, const int64_t *xshape, const int64_t *sshape, 
   return true;
 }
 
-__device__ __forceinline__ void offsets(const Broadcast &b, int64_t i, int64_t &so, int64_t &zo) {
+template <typename Index>
+__device__ __forceinline__ void offsets(const Broadcast &b, Index i, int64_t &so, int64_t &zo) {
   so = zo = 0;
 #pragma unroll
   for (int d = kMaxDims - 1; d >= 0; --d) {
     if (d < b.nd) {
-      const int64_t q = (d == 0) ? 0 : i / b.size[d];
-      const int64_t c = (d == 0) ? i : i - q * b.size[d];
-      so += c * b.sstride[d];
-      zo += c * b.zstride[d];
+      const Index q = (d == 0) ? 0 : i / (Index)b.size[d];
+      const Index c = (d == 0) ? i : i - q * (Index)b.size[d];
+      so += (int64_t)c * b.sstride[d];
+      zo += (int64_t)c * b.zstride[d];
       i = q;
     }
   }
@@ -77,11 +78,20 @@ __device__ __forceinline__ float round_mode(float v, int half_to_even) {
 }
 __device__ __forceinline__ float saturate(float v, float lo, float hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
+// x / s.  A scale that is a power of two with a normal reciprocal is divided by multiplying with that reciprocal:
+// both are the one correct rounding of the same real number.
+__device__ __forceinline__ float divide(float x, float s) {
+  const uint32_t u = __float_as_uint(s), e = u >> 23;
+  if ((u & 0x807fffffu) == 0u && e >= 1u && e <= 253u)
+    return x * __uint_as_float((254u - e) << 23);
+  return x / s;
+}
+
 struct QuantizeOp {
   int half_to_even;
   float lo, hi;
   __device__ __forceinline__ float operator()(float x, float scale, float zp) const {
-    const float t = round_mode(x / scale, half_to_even);
+    const float t = round_mode(divide(x, scale), half_to_even);
     return saturate(t + zp, lo, hi);
   }
 };
@@ -90,38 +100,66 @@ struct DequantizeOp {
 };
 // dx (+)= dy / scale  and  dx (+)= dy * scale  (the zero point is not read)
 struct DivGradOp {
-  __device__ __forceinline__ float operator()(float dy, float scale, float) const { return dy / scale; }
+  __device__ __forceinline__ float operator()(float dy, float scale, float) const { return divide(dy, scale); }
 };
 struct MulGradOp {
   __device__ __forceinline__ float operator()(float dy, float scale, float) const { return dy * scale; }
 };
 
-// y[i] = op(x[i], scale[...], zp[...]) (+ y[i] when kAccum).  kVec: four consecutive elements per thread, all inside
-// the innermost dimension (its size is a multiple of four).
-template <typename Op, bool kVec, bool kAccum>
+// y[i] = op(x[i], scale[...], zp[...]) (+ y[i] when kAccum).  kVec: four float4 per thread (loads issued together),
+// each float4 inside the innermost dimension (its size is a multiple of four).  Index: uint32_t when the element
+// count fits, so the index decomposition divides in 32 bits.
+constexpr int kUnroll = 4;
+template <typename Op, bool kVec, bool kAccum, typename Index>
 __global__ __launch_bounds__(kBlock) void broadcast_map(const float *__restrict__ x, const float *__restrict__ scale,
                                                         const float *__restrict__ zp, float *__restrict__ y,
                                                         int64_t count, Broadcast b, Op op) {
-  const int64_t step = (int64_t)gridDim.x * kBlock;
-  for (int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x; t < count; t += step) {
-    int64_t so, zo;
-    if (kVec) {
-      const int64_t i = 4 * t;
-      offsets(b, i, so, zo);
-      const int64_t ss = b.sstride[b.nd - 1], zs = b.zstride[b.nd - 1];
-      const float4_t v = *reinterpret_cast<const float4_t *>(x + i);
-      float4_t o;
-      o.x = op(v.x, scale[so], zp ? zp[zo] : 0.0f);
-      o.y = op(v.y, scale[so + ss], zp ? zp[zo + zs] : 0.0f);
-      o.z = op(v.z, scale[so + 2 * ss], zp ? zp[zo + 2 * zs] : 0.0f);
-      o.w = op(v.w, scale[so + 3 * ss], zp ? zp[zo + 3 * zs] : 0.0f);
-      if (kAccum) {
-        const float4_t old = *reinterpret_cast<const float4_t *>(y + i);
-        o.x = old.x + o.x, o.y = old.y + o.y, o.z = old.z + o.z, o.w = old.w + o.w;
+  if (kVec) {
+    const int64_t base = (int64_t)blockIdx.x * (kBlock * kUnroll) + threadIdx.x;
+    float4_t v[kUnroll], old[kUnroll];
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      const int64_t t = base + (int64_t)j * kBlock;
+      if (t < count) {
+        v[j] = *reinterpret_cast<const float4_t *>(x + 4 * t);
+        if (kAccum)
+          old[j] = *reinterpret_cast<const float4_t *>(y + 4 * t);
       }
-      __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(y + i));
-    } else {
-      offsets(b, t, so, zo);
+    }
+    const int64_t ss = b.sstride[b.nd - 1], zs = b.zstride[b.nd - 1];
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      const int64_t t = base + (int64_t)j * kBlock;
+      if (t < count) {
+        int64_t so, zo;
+        offsets<Index>(b, (Index)(4 * t), so, zo);
+        // innermost stride 0: one value for the four elements; stride 1: four consecutive values
+        float4_t sv, zv;
+        if (ss == 0)
+          sv.x = sv.y = sv.z = sv.w = scale[so];
+        else
+          sv = *reinterpret_cast<const float4_t *>(scale + so);
+        if (!zp)
+          zv.x = zv.y = zv.z = zv.w = 0.0f;
+        else if (zs == 0)
+          zv.x = zv.y = zv.z = zv.w = zp[zo];
+        else
+          zv = *reinterpret_cast<const float4_t *>(zp + zo);
+        float4_t o;
+        o.x = op(v[j].x, sv.x, zv.x);
+        o.y = op(v[j].y, sv.y, zv.y);
+        o.z = op(v[j].z, sv.z, zv.z);
+        o.w = op(v[j].w, sv.w, zv.w);
+        if (kAccum)
+          o.x = old[j].x + o.x, o.y = old[j].y + o.y, o.z = old[j].z + o.z, o.w = old[j].w + o.w;
+        __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(y + 4 * t));
+      }
+    }
+  } else {
+    const int64_t step = (int64_t)gridDim.x * kBlock;
+    for (int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x; t < count; t += step) {
+      int64_t so, zo;
+      offsets<Index>(b, (Index)t, so, zo);
       const float o = op(x[t], scale[so], zp ? zp[zo] : 0.0f);
       y[t] = kAccum ? y[t] + o : o;
     }
@@ -154,22 +192,31 @@ int launch_broadcast(const float *x, const float *scale, const float *zp, float 
   int rc = ensure_init();
   if (rc)
     return rc;
-  const bool vec = b.size[b.nd - 1] % 4 == 0 && aligned16(x) && aligned16(y);
+  const bool vec = b.size[b.nd - 1] % 4 == 0 && aligned16(x) && aligned16(y) && aligned16(scale) && aligned16(zp);
+  const bool narrow = total < ((int64_t)1 << 31);
   const int64_t count = vec ? total / 4 : total;
-  int64_t blocks = ceil_div(count, (int64_t)kBlock);
-  if (blocks > 1048576)
-    blocks = 1048576;
-#define NBLA_LAUNCH_MAP(V, A)                                                                                          \
-  hipLaunchKernelGGL((broadcast_map<Op, V, A>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, scale, zp, y,      \
+  int64_t blocks = ceil_div(count, (int64_t)kBlock * (vec ? kUnroll : 1));
+  if (!vec && blocks > 1048576)
+    blocks = 1048576; // grid-stride loop
+#define NBLA_LAUNCH_MAP(V, A, I)                                                                                       \
+  hipLaunchKernelGGL((broadcast_map<Op, V, A, I>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, scale, zp, y,   \
                      count, b, op)
+#define NBLA_LAUNCH_MAP_I(V, A)                                                                                        \
+  do {                                                                                                                 \
+    if (narrow)                                                                                                        \
+      NBLA_LAUNCH_MAP(V, A, uint32_t);                                                                                 \
+    else                                                                                                               \
+      NBLA_LAUNCH_MAP(V, A, int64_t);                                                                                  \
+  } while (0)
   if (vec && accum)
-    NBLA_LAUNCH_MAP(true, true);
+    NBLA_LAUNCH_MAP_I(true, true);
   else if (vec)
-    NBLA_LAUNCH_MAP(true, false);
+    NBLA_LAUNCH_MAP_I(true, false);
   else if (accum)
-    NBLA_LAUNCH_MAP(false, true);
+    NBLA_LAUNCH_MAP_I(false, true);
   else
-    NBLA_LAUNCH_MAP(false, false);
+    NBLA_LAUNCH_MAP_I(false, false);
+#undef NBLA_LAUNCH_MAP_I
 #undef NBLA_LAUNCH_MAP
   NBLA_HIP_LAUNCH_CHECK(what);
   return NBLA_HIP_OK;
@@ -189,95 +236,129 @@ int quantize_range(int dtype, int narrow_range, float &lo, float &hi) {
 
 // ------------------------------------------------------------------------------------------------------ Prune
 
-constexpr int kBins = 2048;
+// Radix select of the rank-th smallest magnitude: four passes over the 31 magnitude bits (8, 8, 8, 7), each
+// histogramming the digit of the elements that share the digits chosen so far.  LDS holds 32 copies of the 256
+// counters, copy = lane % 32 at address bin * 32 + copy: the 32 lanes served together never meet in a counter or a
+// bank.  No separate selection kernels: every block re-derives the chosen digits from the finished histograms of
+// the earlier passes (a 256-entry scan each).
+constexpr int kPasses = 4, kBins = 256, kCopies = 32;
+constexpr int kBinStride = 16; // words between the global counters of two bins: one 64-byte line each
 struct SelectState {
-  uint32_t prefix; // magnitude bits fixed so far (already shifted into place)
-  uint32_t rank;   // rank of the wanted element among those sharing the prefix
-  uint32_t hist[kBins];
+  uint32_t hist[kPasses][kBins * kBinStride];
 };
+__device__ __forceinline__ int pass_shift(int p) { return p == 0 ? 23 : (p == 1 ? 15 : (p == 2 ? 7 : 0)); }
+__device__ __forceinline__ int pass_bits(int p) { return p == 3 ? 7 : 8; }
 
-// Histogram of `bits` bits at `shift` of the magnitudes whose bits above shift + bits equal the prefix.
-__global__ __launch_bounds__(kBlock) void prune_histogram(const float *__restrict__ x, int64_t n,
-                                                          SelectState *__restrict__ st, int shift, int bits,
-                                                          int first) {
-  __shared__ uint32_t h[kBins];
-  for (int i = threadIdx.x; i < kBins; i += kBlock)
-    h[i] = 0u;
-  __syncthreads();
-  const uint32_t prefix = first ? 0u : st->prefix;
-  const uint32_t mask = (1u << bits) - 1u;
-  const int above = shift + bits;
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
-    const uint32_t key = __float_as_uint(x[i]) & 0x7fffffffu;
-    if (first || (key >> above) == (prefix >> above))
-      atomicAdd(&h[(key >> shift) & mask], 1u);
+// Digits of passes [0, upto) and the rank left inside the chosen bins; all threads of the block take part and get
+// the same answer.  `scratch` holds kBlock / 64 + 2 words.
+__device__ __forceinline__ void chosen_prefix(const SelectState *st, int upto, uint32_t rank0, uint32_t *scratch,
+                                              uint32_t &prefix, uint32_t &rank) {
+  prefix = 0u;
+  rank = rank0;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int p = 0; p < upto; ++p) {
+    const uint32_t c = st->hist[p][threadIdx.x * kBinStride]; // kBlock == kBins
+    uint32_t incl = c;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const uint32_t up = __shfl_up(incl, off);
+      if (lane >= off)
+        incl += up;
+    }
+    if (lane == 63)
+      scratch[wave] = incl;
+    __syncthreads();
+    uint32_t before = 0;
+    for (int w = 0; w < wave; ++w)
+      before += scratch[w];
+    const uint32_t excl = before + incl - c;
+    if (c != 0 && excl <= rank && rank < excl + c) {
+      scratch[kBlock / 64] = (uint32_t)threadIdx.x;
+      scratch[kBlock / 64 + 1] = rank - excl;
+    }
+    __syncthreads();
+    prefix |= scratch[kBlock / 64] << pass_shift(p);
+    rank = scratch[kBlock / 64 + 1];
+    __syncthreads();
   }
-  __syncthreads();
-  for (int i = threadIdx.x; i < kBins; i += kBlock)
-    if (h[i])
-      atomicAdd(&st->hist[i], h[i]);
 }
 
-// One block: find the bin holding the wanted rank, extend the prefix, clear the histogram for the next pass.
-__global__ __launch_bounds__(kBlock) void prune_pick(SelectState *__restrict__ st, int shift, int bits, int first,
-                                                     uint32_t rank0) {
-  __shared__ uint32_t part[kBlock];
-  const int per = kBins / kBlock; // 8 consecutive bins per thread
-  uint32_t local[per];
-  uint32_t sum = 0;
-  for (int j = 0; j < per; ++j) {
-    local[j] = st->hist[threadIdx.x * per + j];
-    sum += local[j];
-  }
-  part[threadIdx.x] = sum;
+__global__ __launch_bounds__(kBlock) void prune_histogram(const float *__restrict__ x, int64_t n4, int64_t n,
+                                                          SelectState *__restrict__ st, int pass, uint32_t rank0) {
+  __shared__ uint32_t h[kBins * kCopies];
+  __shared__ uint32_t scratch[kBlock / 64 + 2];
+  for (int i = threadIdx.x; i < kBins * kCopies; i += kBlock)
+    h[i] = 0u;
+  uint32_t prefix, rank;
+  chosen_prefix(st, pass, rank0, scratch, prefix, rank);
   __syncthreads();
-  if (threadIdx.x == 0) {
-    const uint32_t rank = first ? rank0 : st->rank;
-    uint32_t before = 0;
-    int t = 0;
-    while (t < kBlock - 1 && before + part[t] <= rank)
-      before += part[t++];
-    part[0] = (uint32_t)t; // owning thread
-    part[1] = before;
-    part[2] = rank;
+  const int shift = pass_shift(pass), above = shift + pass_bits(pass);
+  const uint32_t mask = (1u << pass_bits(pass)) - 1u, want = prefix >> above;
+  const int copy = threadIdx.x & (kCopies - 1);
+  auto count = [&](float v) {
+    const uint32_t key = __float_as_uint(v) & 0x7fffffffu;
+    if (pass == 0 || (key >> above) == want)
+      atomicAdd(&h[((key >> shift) & mask) * kCopies + copy], 1u);
+  };
+  // four loads in flight per thread before the counters are touched
+  const int64_t tiles = (n4 + kBlock * 4 - 1) / (kBlock * 4);
+  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    const int64_t base = tile * (kBlock * 4) + threadIdx.x;
+    float4_t v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (base + j * kBlock < n4)
+        v[j] = *reinterpret_cast<const float4_t *>(x + 4 * (base + j * kBlock));
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (base + j * kBlock < n4)
+        count(v[j].x), count(v[j].y), count(v[j].z), count(v[j].w);
+  }
+  if (blockIdx.x == 0) {
+    const int64_t i = 4 * n4 + threadIdx.x;
+    if (i < n)
+      count(x[i]);
   }
   __syncthreads();
-  const uint32_t owner = part[0], before = part[1], rank = part[2];
-  __syncthreads();
-  if (threadIdx.x == owner) {
-    uint32_t acc = before;
-    int j = 0;
-    while (j < per - 1 && acc + local[j] <= rank)
-      acc += local[j++];
-    const uint32_t bin = owner * per + j;
-    st->prefix = (first ? 0u : st->prefix) | (bin << shift);
-    st->rank = rank - acc;
-  }
-  for (int j = 0; j < per; ++j)
-    st->hist[threadIdx.x * per + j] = 0u;
-  (void)bits;
+  uint32_t total = 0;
+#pragma unroll 8
+  for (int c = 0; c < kCopies; ++c)
+    total += h[threadIdx.x * kCopies + ((c + threadIdx.x) & (kCopies - 1))]; // rotated: one bank per lane
+  if (total)
+    atomicAdd(&st->hist[pass][threadIdx.x * kBinStride], total);
 }
 
 __global__ __launch_bounds__(kBlock) void clear_select(SelectState *st) {
-  for (int i = threadIdx.x; i < kBins; i += kBlock)
-    st->hist[i] = 0u;
-  if (threadIdx.x == 0)
-    st->prefix = st->rank = 0u;
+  for (int p = 0; p < kPasses; ++p)
+    st->hist[p][threadIdx.x * kBinStride] = 0u;
 }
 
-// y = (|x| < thresh) ? 0 : x with thresh = |k-th smallest| (+ 1 when rate == 1), prune.cpp:62-69
+// y = (|x| < thresh) ? 0 : x with thresh = |rank-th smallest| (+ 1 when rate == 1), prune.cpp:62-69
 __global__ __launch_bounds__(kBlock) void prune_apply(const float *__restrict__ x, float *__restrict__ y, int64_t n4,
-                                                      int64_t n, const SelectState *__restrict__ st, float add) {
-  const float thresh = __uint_as_float(st->prefix) + add;
-  const int64_t step = (int64_t)gridDim.x * kBlock;
-  for (int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x; t < n4; t += step) {
-    const float4_t v = *reinterpret_cast<const float4_t *>(x + 4 * t);
-    float4_t o;
-    o.x = fabsf(v.x) < thresh ? 0.0f : v.x;
-    o.y = fabsf(v.y) < thresh ? 0.0f : v.y;
-    o.z = fabsf(v.z) < thresh ? 0.0f : v.z;
-    o.w = fabsf(v.w) < thresh ? 0.0f : v.w;
-    __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(y + 4 * t));
+                                                      int64_t n, const SelectState *__restrict__ st, uint32_t rank0,
+                                                      float add) {
+  __shared__ uint32_t scratch[kBlock / 64 + 2];
+  uint32_t prefix, rank;
+  chosen_prefix(st, kPasses, rank0, scratch, prefix, rank);
+  const float thresh = __uint_as_float(prefix) + add;
+  const int64_t tiles = (n4 + kBlock * 4 - 1) / (kBlock * 4);
+  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    const int64_t base = tile * (kBlock * 4) + threadIdx.x;
+    float4_t v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (base + j * kBlock < n4)
+        v[j] = *reinterpret_cast<const float4_t *>(x + 4 * (base + j * kBlock));
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (base + j * kBlock < n4) {
+        float4_t o;
+        o.x = fabsf(v[j].x) < thresh ? 0.0f : v[j].x;
+        o.y = fabsf(v[j].y) < thresh ? 0.0f : v[j].y;
+        o.z = fabsf(v[j].z) < thresh ? 0.0f : v[j].z;
+        o.w = fabsf(v[j].w) < thresh ? 0.0f : v[j].w;
+        __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(y + 4 * (base + j * kBlock)));
+      }
   }
   if (blockIdx.x == 0) {
     const int64_t i = 4 * n4 + threadIdx.x;
@@ -372,24 +453,20 @@ int nbla_hip_prune_f32(const float *x, float *y, size_t size, float rate, void *
   const int x_size = (int)size;
   const uint32_t rank = (uint32_t)(int)((x_size - 1) * rate);
   const int64_t n = (int64_t)size;
-  int64_t blocks = ceil_div(n, (int64_t)kBlock * 16);
-  if (blocks > 2048)
-    blocks = 2048;
-  if (blocks < 1)
-    blocks = 1;
+  const int64_t n4 = n / 4;
+  int64_t blocks = ceil_div(n4 ? n4 : 1, (int64_t)kBlock * 4);
+  if (blocks > 1024)
+    blocks = 1024; // every block ends with up to 256 global counter updates
   hipLaunchKernelGGL(clear_select, dim3(1), dim3(kBlock), 0, stream, st);
   NBLA_HIP_LAUNCH_CHECK("clear_select");
-  const int shifts[3] = {20, 10, 0}, widths[3] = {11, 10, 10};
-  for (int p = 0; p < 3; ++p) {
-    hipLaunchKernelGGL(prune_histogram, dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, n, st, shifts[p],
-                       widths[p], p == 0 ? 1 : 0);
+  for (int p = 0; p < kPasses; ++p) {
+    hipLaunchKernelGGL(prune_histogram, dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, n4, n, st, p, rank);
     NBLA_HIP_LAUNCH_CHECK("prune_histogram");
-    hipLaunchKernelGGL(prune_pick, dim3(1), dim3(kBlock), 0, stream, st, shifts[p], widths[p], p == 0 ? 1 : 0, rank);
-    NBLA_HIP_LAUNCH_CHECK("prune_pick");
   }
-  const int64_t n4 = n / 4;
   int64_t ablocks = ceil_div(n4 ? n4 : 1, (int64_t)kBlock * 4);
-  hipLaunchKernelGGL(prune_apply, dim3((unsigned)ablocks), dim3(kBlock), 0, stream, x, y, n4, n, st,
+  if (ablocks > 4096)
+    ablocks = 4096; // every block re-derives the threshold, so keep their number bounded
+  hipLaunchKernelGGL(prune_apply, dim3((unsigned)ablocks), dim3(kBlock), 0, stream, x, y, n4, n, st, rank,
                      rate == 1.0f ? 1.0f : 0.0f);
   NBLA_HIP_LAUNCH_CHECK("prune_apply");
   return NBLA_HIP_OK;

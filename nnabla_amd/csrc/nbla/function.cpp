@@ -10,6 +10,7 @@
 #include <nbla/function/inq_convolution.hpp>
 #include <nbla/function/min_max_quantize.hpp>
 #include <nbla/function/pow2_quantize.hpp>
+#include <nbla/function/quantize_linear.hpp>
 
 #include <algorithm>
 
@@ -95,6 +96,9 @@ NBLA_REGISTER_FUNCTION_SOURCE(INQConvolution, int, const vector<int> &, const ve
                               int, const vector<int> &, const string &, int);
 NBLA_REGISTER_FUNCTION_SOURCE(Affine, int);
 NBLA_REGISTER_FUNCTION_SOURCE(ReLU, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(QuantizeLinear, const string &, bool, int);
+NBLA_REGISTER_FUNCTION_SOURCE(DequantizeLinear);
+NBLA_REGISTER_FUNCTION_SOURCE(Prune, float);
 
 // ------------------------------------------------------------- shape inference
 AffineShapes infer_affine_shapes(int base_axis, Variable *x, Variable *w, Variable *bias) {

@@ -99,3 +99,34 @@ def affine(x, weight, bias=None, base_axis=1, n_outputs=-1, outputs=None):
 def relu(x, inplace=False, n_outputs=-1, outputs=None):
     f = Function("ReLU", None, [int(inplace)])
     return f(x, outputs=outputs)
+
+
+def quantize_linear(x, scale, zero_point, round_mode='HALF_AWAY_FROM_ZERO', narrow_range=False, dtype=1,
+                    n_outputs=-1, outputs=None):
+    """``saturate(round(x / scale) + zero_point)`` to the int8 (``dtype`` 1 or ``numpy.int8``) or uint8 (2 or
+    ``numpy.uint8``) range; ``zero_point`` is rounded and saturated in place (functions.yaml:7556-7601)."""
+    f = Function("QuantizeLinear", None, [int(narrow_range), _dtype_code(dtype)], [], round_mode)
+    return f(x, scale, zero_point, outputs=outputs)
+
+
+def dequantize_linear(x, scale, zero_point, n_outputs=-1, outputs=None):
+    """``(x - zero_point) * scale`` (functions.yaml:7602-7640)."""
+    f = Function("DequantizeLinear", None, [], [])
+    return f(x, scale, zero_point, outputs=outputs)
+
+
+def prune(x, rate=0.9, n_outputs=-1, outputs=None):
+    """Zero the ``rate`` fraction of smallest magnitudes (functions.yaml:7521-7555)."""
+    f = Function("Prune", None, [], [rate])
+    return f(x, outputs=outputs)
+
+
+def _dtype_code(dtype):
+    """nbla::dtypes code of a numpy dtype (int8 -> 1, uint8 -> 2); integers pass through."""
+    if isinstance(dtype, int):
+        return dtype
+    import numpy as np
+    code = {np.dtype(np.int8): 1, np.dtype(np.uint8): 2}.get(np.dtype(dtype))
+    if code is None:
+        raise ValueError("quantize_linear: dtype must be int8 or uint8, not %r" % (dtype,))
+    return code

@@ -5,8 +5,9 @@
 
 Functions are created through the registry for the *current* context, so a graph loaded under the ``hip`` extension
 context runs on the hip:float classes (the dispatch nnp_impl_create_function.cpp.tmpl:51-117 performs for every
-function; here for the nine quantization functions, Affine and ReLU).  Network definitions are read from protobuf
-text (``.nntxt`` / ``.prototxt``), parameters from ``parameter.protobuf`` or from ``parameter`` entries of the text.
+function; here for the nine quantization functions, QuantizeLinear, DequantizeLinear, Prune, Affine and ReLU).
+Network definitions are read from protobuf text (``.nntxt`` / ``.prototxt``), parameters from
+``parameter.protobuf`` or from ``parameter`` entries of the text.
 """
 import io
 import os
@@ -73,6 +74,11 @@ _BUILDERS = {
         i[0], i[1], i[2], _opt(i, 3), **dict(_conv_kwargs(p), **_inq_kwargs(p)))),
     "Affine": ("affine_param", 2, lambda p, i: F.affine(i[0], i[1], _opt(i, 2), base_axis=int(p.get("base_axis", 1)))),
     "ReLU": ("relu_param", 1, lambda p, i: F.relu(i[0], inplace=bool(p.get("inplace", False)))),
+    "QuantizeLinear": ("quantize_linear_param", 3, lambda p, i: F.quantize_linear(
+        i[0], i[1], i[2], round_mode=str(p.get("round_mode", "HALF_AWAY_FROM_ZERO")),
+        narrow_range=bool(p.get("narrow_range", False)), dtype=int(p.get("dtype", 1)))),
+    "DequantizeLinear": ("dequantize_linear_param", 3, lambda p, i: F.dequantize_linear(i[0], i[1], i[2])),
+    "Prune": ("prune_param", 1, lambda p, i: F.prune(i[0], rate=float(p.get("rate", 0.9)))),
 }
 
 SUPPORTED_FUNCTIONS = tuple(sorted(_BUILDERS))

@@ -419,3 +419,32 @@ def test_convolution_backward_through_the_registry(ctx):
     assert max_rel_err(vW1.g, g_W1) <= TIGHT * 4
     assert max_rel_err(vb1.g, g_b1) <= TIGHT * 4
     assert max_rel_err(vx.g, g_x) <= TIGHT * 4
+
+
+def test_quantize_dequantize_linear_and_prune_through_the_registry(ctx):
+    rng = np.random.RandomState(23)
+    x = (rng.randn(4, 6, 5, 5) * 3).astype(np.float32)
+    scale = (np.abs(rng.randn(1, 6, 1, 1)) + 0.05).astype(np.float32)
+    zp = (rng.randn(1, 6, 1, 1) * 4).astype(np.float32)
+    vx = nn.Variable.from_numpy_array(x, need_grad=True)
+    vx.zero_grad()
+    vs, vz = _var(scale), _var(zp)
+    p = F.prune(vx, rate=0.4)
+    q = F.quantize_linear(p, vs, vz, 'HALF_TO_EVEN', True, np.int8)
+    y = F.dequantize_linear(q, vs, vz)
+    y.forward()
+    rp = oracle.prune(x, 0.4)
+    rq, rzp = oracle.quantize_linear(rp, scale, zp, 'HALF_TO_EVEN', True, 1)
+    assert bits_equal(p.d, rp) and bits_equal(q.d, rq)
+    assert bits_equal(vz.d, rzp)                                   # the zero point was rounded in place ...
+    assert bits_equal(y.d, oracle.dequantize_linear(rq, scale, rzp))   # ... and the dequantizer sees the rounded one
+    gy = rng.randn(*x.shape).astype(np.float32)
+    y.backward(gy)
+    g = oracle.linear_quantize_backward(oracle.linear_quantize_backward(gy, scale, True), scale, False)
+    assert bits_equal(vx.g, g)                                     # Prune passes the gradient through
+    with pytest.raises(ValueError):
+        F.quantize_linear(vx, vs, vz, 'HALF_UP')
+    with pytest.raises(ValueError):
+        F.quantize_linear(vx, vs, _var(np.zeros((1, 5, 1, 1), np.float32)))
+    with pytest.raises(ValueError):
+        F.prune(vx, rate=1.5)

@@ -191,3 +191,21 @@ def test_graph_errors(hip_ctx):
     assert set(SUPPORTED_FUNCTIONS) >= {"FixedPointQuantize", "Pow2Quantize", "MinMaxQuantize", "BinaryWeightAffine",
                                         "BinaryConnectAffine", "BinaryWeightConvolution",
                                         "BinaryConnectConvolution", "INQAffine", "INQConvolution"}
+
+
+def test_linear_quantizer_and_prune_builders(hip_ctx):
+    text = '''network { name: "q" batch_size: 2
+      variable { name: "x" type: "Buffer" shape: { dim: -1 dim: 3 dim: 4 } }
+      variable { name: "s" type: "Parameter" shape: { dim: 1 dim: 3 dim: 1 } initializer { type: "Constant" multiplier: 0.5 } }
+      variable { name: "z" type: "Parameter" shape: { dim: 1 dim: 1 dim: 1 } }
+      function { name: "p" type: "Prune" input: "x" output: "xp" prune_param { rate: 0.25 } }
+      function { name: "q" type: "QuantizeLinear" input: "xp" input: "s" input: "z" output: "xq"
+                 quantize_linear_param { round_mode: "HALF_TO_EVEN" narrow_range: true dtype: 2 } }
+      function { name: "d" type: "DequantizeLinear" input: "xq" input: "s" input: "z" output: "y" }
+    }'''
+    net = NnpLoader(io.BytesIO(text.encode()), extension=".nntxt").get_network("q")
+    v = net.variables
+    assert list(net.outputs) == ["y"] and v["y"].shape == (2, 3, 4)
+    assert v["xp"].parent.info == {"type": "Prune", "iargs": (), "fargs": (0.25,), "sarg": None}
+    assert v["xq"].parent.info == {"type": "QuantizeLinear", "iargs": (1, 2), "fargs": (), "sarg": "HALF_TO_EVEN"}
+    assert v["y"].parent.info["type"] == "DequantizeLinear"
