@@ -325,6 +325,21 @@ int nbla_hip_binary_connect_convolution_f32(
     const int64_t *dilation, int64_t group, float quantize_zero_to,
     void *workspace, size_t workspace_bytes, void *stream);
 
+/* Convolution with real-valued weights, y = conv(x, W) + bias on the bf16-plane
+ * product (three planes per operand, fp32 accumulate).  Replaces
+ * Convolution<float>::forward_impl, convolution.cpp:161-197. */
+size_t nbla_hip_convolution_workspace_bytes(
+    int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
+    const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+    const int64_t *dilation, int64_t group);
+int nbla_hip_convolution_f32(const float *x, const float *W, const float *bias,
+                             float *y, int64_t outer, int64_t C, int nd,
+                             const int64_t *in_sp, int64_t O,
+                             const int64_t *kernel, const int64_t *pad,
+                             const int64_t *stride, const int64_t *dilation,
+                             int64_t group, void *workspace,
+                             size_t workspace_bytes, void *stream);
+
 /* Workspace of the two convolution backward entry points below. */
 size_t nbla_hip_convolution_backward_workspace_bytes(
     int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,

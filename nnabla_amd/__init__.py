@@ -16,4 +16,6 @@ There is no CPU fallback: without the built HIP libraries every front-end call r
 __version__ = "0.1.0"
 
 from .context import Context, context_scope, get_current_context, set_default_context  # noqa: F401
-from .variable import Variable, auto_forward, get_auto_forward, set_auto_forward  # noqa: F401
+from .variable import NdArray, Variable, auto_forward, get_auto_forward, set_auto_forward  # noqa: F401
+from .parameter import (clear_parameters, get_parameter, get_parameter_or_create, get_parameters,  # noqa: F401
+                        parameter_scope, pop_parameter, set_parameter)

@@ -7,6 +7,7 @@
 #include <nbla/function/binary_connect_convolution.hpp>
 #include <nbla/function/binary_weight_affine.hpp>
 #include <nbla/function/binary_weight_convolution.hpp>
+#include <nbla/function/convolution.hpp>
 #include <nbla/function/fixed_point_quantize.hpp>
 #include <nbla/function/inq_affine.hpp>
 #include <nbla/function/inq_convolution.hpp>
@@ -127,6 +128,14 @@ FunctionPtr create_by_name(const string &name, const Context &ctx, const int64_t
     need(1, 0);
     return create_ReLU(ctx, ia[0] != 0);
   }
+  if (name == "Convolution") {
+    need(4, 0);
+    const int64_t *p = ia;
+    const int base_axis = (int)*p++, group = (int)*p++, channel_last = (int)*p++, nd = (int)*p++;
+    NBLA_CHECK(ni >= 4 + 3 * nd, error_code::value, "Convolution: pad/stride/dilation arguments missing.");
+    const vector<int> pad = take_ints(p, nd), stride = take_ints(p, nd), dilation = take_ints(p, nd);
+    return create_Convolution(ctx, base_axis, pad, stride, dilation, group, channel_last != 0);
+  }
   if (name == "QuantizeLinear") {
     need(2, 0);
     return create_QuantizeLinear(ctx, sarg, ia[0] != 0, (int)ia[1]);
@@ -233,6 +242,17 @@ NBLA_API int nblac_variable_share(void *dst, void *src) {
     VarHandle *d = static_cast<VarHandle *>(dst), *s = static_cast<VarHandle *>(src);
     d->var->set_data(s->var->data()->view(d->var->shape()));
     d->var->set_grad(s->var->grad()->view(d->var->shape()));
+  });
+}
+
+// dst's data (which = 0) or grad (which = 1) becomes a view of src's: `outputs=[param.data]` of the front-end.
+NBLA_API int nblac_variable_share_array(void *dst, void *src, int which) {
+  return guarded([&] {
+    VarHandle *d = static_cast<VarHandle *>(dst), *s = static_cast<VarHandle *>(src);
+    if (which == 0)
+      d->var->set_data(s->var->data()->view(d->var->shape()));
+    else
+      d->var->set_grad(s->var->grad()->view(d->var->shape()));
   });
 }
 

@@ -394,6 +394,39 @@ void INQConvolutionHip<T, T1>::backward_impl(const Variables &inputs, const Vari
       });
 }
 
+// convolution.cpp:161-197
+template <typename T> void ConvolutionHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const ConvShapes &s = this->shapes_;
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
+  const T *b = inputs.size() == 3 ? inputs[2]->get_data_pointer<T>(this->ctx_) : nullptr;
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  HipWorkspace ws(nbla_hip_convolution_workspace_bytes(s.outer, s.channels_i, s.spatial_dims, s.spatial_i.data(),
+                                                       s.channels_o, s.kernel.data(), s.pad.data(), s.stride.data(),
+                                                       s.dilation.data(), s.group),
+                  this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_convolution_f32(x, w, b, y, s.outer, s.channels_i, s.spatial_dims, s.spatial_i.data(),
+                                         s.channels_o, s.kernel.data(), s.pad.data(), s.stride.data(),
+                                         s.dilation.data(), s.group, ws.pointer(), ws.bytes(), nullptr));
+}
+
+// convolution.cpp:199-283
+template <typename T>
+void ConvolutionHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                      const vector<bool> &propagate_down, const vector<bool> &accum) {
+  const ConvShapes &s = this->shapes_;
+  conv_backward_common<T>(
+      this->ctx_, s, inputs, outputs, propagate_down, accum, 2,
+      [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
+        const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
+        NBLA_HIP_CALL(nbla_hip_convolution_backward_f32(
+            dy, x, w, dx, dw, db, s.outer, s.channels_i, s.spatial_dims, s.spatial_i.data(), s.channels_o,
+            s.kernel.data(), s.pad.data(), s.stride.data(), s.dilation.data(), s.group, ax, aw, ab, ws.pointer(),
+            ws.bytes(), nullptr));
+      });
+}
+
 // affine.cpp:98-140
 template <typename T>
 void AffineHip<T>::backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
@@ -532,6 +565,7 @@ template class INQAffineHip<float, int>;
 template class INQConvolutionHip<float, int>;
 template class AffineHip<float>;
 template class ReLUHip<float>;
+template class ConvolutionHip<float>;
 template class QuantizeLinearHip<float>;
 template class DequantizeLinearHip<float>;
 template class PruneHip<float>;

@@ -65,6 +65,8 @@ void init_hip() {
                               int);
   NBLA_REGISTER_FUNCTION_IMPL(Affine, AffineHip<float>, "hip:float", int);
   NBLA_REGISTER_FUNCTION_IMPL(ReLU, ReLUHip<float>, "hip:float", bool);
+  NBLA_REGISTER_FUNCTION_IMPL(Convolution, ConvolutionHip<float>, "hip:float", int, const vector<int> &,
+                              const vector<int> &, const vector<int> &, int, bool);
   NBLA_REGISTER_FUNCTION_IMPL(QuantizeLinear, QuantizeLinearHip<float>, "hip:float", const string &, bool, int);
   NBLA_REGISTER_FUNCTION_IMPL(DequantizeLinear, DequantizeLinearHip<float>, "hip:float");
   NBLA_REGISTER_FUNCTION_IMPL(Prune, PruneHip<float>, "hip:float", float);

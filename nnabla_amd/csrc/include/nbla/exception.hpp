@@ -52,7 +52,9 @@ inline string format_string(const string &fmt) { return fmt; }
 
 #define NBLA_CHECK(condition, code, msg, ...)                                                                          \
   if (!(condition)) {                                                                                                  \
-    NBLA_ERROR(code, ::nbla::string("Failed `" #condition "`: ") + msg, ##__VA_ARGS__);                                \
+    /* the condition text is appended after formatting: it may itself contain '%' */                                  \
+    throw ::nbla::Exception(code, ::nbla::string("Failed `" #condition "`: ") + ::nbla::format_string(msg, ##__VA_ARGS__), \
+                            __func__, __FILE__, __LINE__);                                                             \
   }
 
 } // namespace nbla

@@ -6,6 +6,7 @@
 #include <nbla/function/affine.hpp>
 #include <nbla/function/inq_affine.hpp>
 #include <nbla/function/inq_convolution.hpp>
+#include <nbla/function/convolution.hpp>
 #include <nbla/hip/hip.hpp>
 
 namespace nbla {
@@ -45,6 +46,19 @@ protected:
 template <typename T> class AffineHip : public Affine<T> {
 public:
   AffineHip(const Context &ctx, int base_axis) : Affine<T>(ctx, base_axis) {}
+  virtual vector<string> allowed_array_classes() { return SingletonManager::get<Hip>()->array_classes(); }
+
+protected:
+  virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+  virtual void backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                             const vector<bool> &accum);
+};
+
+template <typename T> class ConvolutionHip : public Convolution<T> {
+public:
+  ConvolutionHip(const Context &ctx, int base_axis, const vector<int> &pad, const vector<int> &stride,
+                 const vector<int> &dilation, int group, bool channel_last)
+      : Convolution<T>(ctx, base_axis, pad, stride, dilation, group, channel_last) {}
   virtual vector<string> allowed_array_classes() { return SingletonManager::get<Hip>()->array_classes(); }
 
 protected:

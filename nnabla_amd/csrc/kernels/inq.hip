@@ -456,4 +456,20 @@ int nbla_hip_inq_convolution_f32(const float *x, float *W, int32_t *I, float *ol
   return NBLA_HIP_OK;
 }
 
+size_t nbla_hip_convolution_workspace_bytes(int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
+                                            const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+                                            const int64_t *dilation, int64_t group) {
+  return nbla_hip_inq_convolution_workspace_bytes(outer, C, nd, in_sp, O, kernel, pad, stride, dilation, group, -1);
+}
+
+// Convolution with real-valued weights: the product-only step of the INQ entry point (the weights are only read).
+int nbla_hip_convolution_f32(const float *x, const float *W, const float *bias, float *y, int64_t outer, int64_t C,
+                             int nd, const int64_t *in_sp, int64_t O, const int64_t *kernel, const int64_t *pad,
+                             const int64_t *stride, const int64_t *dilation, int64_t group, void *workspace,
+                             size_t workspace_bytes, void *stream) {
+  return nbla_hip_inq_convolution_f32(x, const_cast<float *>(W), nullptr, nullptr, nullptr, bias, y, outer, C, nd, in_sp,
+                                      O, kernel, pad, stride, dilation, group, 0, -1, nullptr, nullptr, workspace,
+                                      workspace_bytes, stream);
+}
+
 } // extern "C"

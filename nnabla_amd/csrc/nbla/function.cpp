@@ -5,6 +5,7 @@
 #include <nbla/function/binary_connect_convolution.hpp>
 #include <nbla/function/binary_weight_affine.hpp>
 #include <nbla/function/binary_weight_convolution.hpp>
+#include <nbla/function/convolution.hpp>
 #include <nbla/function/fixed_point_quantize.hpp>
 #include <nbla/function/inq_affine.hpp>
 #include <nbla/function/inq_convolution.hpp>
@@ -96,6 +97,7 @@ NBLA_REGISTER_FUNCTION_SOURCE(INQConvolution, int, const vector<int> &, const ve
                               int, const vector<int> &, const string &, int);
 NBLA_REGISTER_FUNCTION_SOURCE(Affine, int);
 NBLA_REGISTER_FUNCTION_SOURCE(ReLU, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(Convolution, int, const vector<int> &, const vector<int> &, const vector<int> &, int, bool);
 NBLA_REGISTER_FUNCTION_SOURCE(QuantizeLinear, const string &, bool, int);
 NBLA_REGISTER_FUNCTION_SOURCE(DequantizeLinear);
 NBLA_REGISTER_FUNCTION_SOURCE(Prune, float);

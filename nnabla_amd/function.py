@@ -3,7 +3,7 @@ import ctypes
 
 from . import _capi
 from .context import get_current_context
-from .variable import Variable, get_auto_forward
+from .variable import NdArray, Variable, get_auto_forward
 
 
 def _handles(variables):
@@ -73,8 +73,14 @@ class Function(object):
         n = self.min_outputs if n_outputs < 0 else n_outputs
         outs = []
         for i in range(n):
-            if outputs is not None and i < len(outputs) and outputs[i] is not None:
-                outs.append(outputs[i])
+            given = outputs[i] if outputs is not None and i < len(outputs) else None
+            if isinstance(given, NdArray):
+                # a fresh output variable writing into the given array (function.pyx.tmpl:318-326)
+                v = Variable(given.shape)
+                v._share_array(given._var, given._which)
+                outs.append(v)
+            elif given is not None:
+                outs.append(given)
             else:
                 outs.append(Variable(()))
         self.setup(inputs, outs)

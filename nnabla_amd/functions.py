@@ -96,6 +96,14 @@ def affine(x, weight, bias=None, base_axis=1, n_outputs=-1, outputs=None):
     return f(*ins, outputs=outputs)
 
 
+def convolution(x, weight, bias=None, base_axis=1, pad=None, stride=None, dilation=None, group=1, channel_last=False,
+                n_outputs=-1, outputs=None):
+    nd, geom = _conv_iargs(x, base_axis, pad, stride, dilation, group)
+    f = Function("Convolution", None, [base_axis, group, int(channel_last), nd] + geom)
+    ins = [x, weight] + ([bias] if bias is not None else [])
+    return f(*ins, outputs=outputs)
+
+
 def relu(x, inplace=False, n_outputs=-1, outputs=None):
     f = Function("ReLU", None, [int(inplace)])
     return f(x, outputs=outputs)

@@ -33,7 +33,7 @@ EXPORTED = (
     "nbla_hip_convolution_output_shape", "nbla_hip_binary_convolution_workspace_bytes",
     "nbla_hip_binary_weight_convolution_f32", "nbla_hip_binary_connect_convolution_f32",
     "nbla_hip_convolution_backward_workspace_bytes", "nbla_hip_binary_convolution_backward_f32",
-    "nbla_hip_convolution_backward_f32",
+    "nbla_hip_convolution_backward_f32", "nbla_hip_convolution_workspace_bytes", "nbla_hip_convolution_f32",
     "nbla_hip_quantize_linear_f32", "nbla_hip_quantize_linear_backward_f32", "nbla_hip_dequantize_linear_f32",
     "nbla_hip_dequantize_linear_backward_f32", "nbla_hip_prune_workspace_bytes", "nbla_hip_prune_f32",
     "nbla_hip_inq_workspace_bytes", "nbla_hip_inq_update_weights_f32", "nbla_hip_inq_affine_workspace_bytes",
@@ -67,6 +67,7 @@ def lib():
                      "nbla_hip_min_max_quantize_backward_workspace_bytes",
                      "nbla_hip_affine_backward_workspace_bytes",
                      "nbla_hip_convolution_backward_workspace_bytes", "nbla_hip_prune_workspace_bytes",
+                     "nbla_hip_convolution_workspace_bytes",
                      "nbla_hip_split_operand_bytes", "nbla_hip_digit_operand_bytes",
                      "nbla_hip_binarize_workspace_bytes",
                      "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_convolution_workspace_bytes",

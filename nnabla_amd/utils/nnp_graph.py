@@ -73,6 +73,8 @@ _BUILDERS = {
     "INQConvolution": ("inq_convolution_param", 3, lambda p, i: F.inq_convolution(
         i[0], i[1], i[2], _opt(i, 3), **dict(_conv_kwargs(p), **_inq_kwargs(p)))),
     "Affine": ("affine_param", 2, lambda p, i: F.affine(i[0], i[1], _opt(i, 2), base_axis=int(p.get("base_axis", 1)))),
+    "Convolution": ("convolution_param", 2, lambda p, i: F.convolution(
+        i[0], i[1], _opt(i, 2), channel_last=bool(p.get("channel_last", False)), **_conv_kwargs(p))),
     "ReLU": ("relu_param", 1, lambda p, i: F.relu(i[0], inplace=bool(p.get("inplace", False)))),
     "QuantizeLinear": ("quantize_linear_param", 3, lambda p, i: F.quantize_linear(
         i[0], i[1], i[2], round_mode=str(p.get("round_mode", "HALF_AWAY_FROM_ZERO")),

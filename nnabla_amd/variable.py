@@ -43,6 +43,33 @@ def _shape_arr(shape):
     return (ctypes.c_int64 * len(shape))(*[int(s) for s in shape])
 
 
+class NdArray(object):
+    """The data (``which`` 0) or grad (``which`` 1) array of a variable: what ``v.data`` / ``v.grad`` return.  Passing
+    one as ``outputs=[param.data]`` makes a function write its result into that array."""
+
+    def __init__(self, var, which):
+        self._var = var
+        self._which = which
+
+    @property
+    def shape(self):
+        return self._var.shape
+
+    @property
+    def data(self):
+        return self._var._get(self._which)
+
+    @data.setter
+    def data(self, value):
+        self._var._set(self._which, value)
+
+    def zero(self):
+        self._var._fill(self._which, 0.0)
+
+    def fill(self, v):
+        self._var._fill(self._which, v)
+
+
 class Variable(object):
     """An N-d array with data and grad, living wherever it was last written (host or device)."""
 
@@ -115,6 +142,18 @@ class Variable(object):
         dt = value.dtype if keep_dtype and value.dtype in _NP2DT else self._dtype(which)
         arr = np.ascontiguousarray(np.broadcast_to(value, self.shape), dtype=dt)
         _capi.check(_capi.lib().nblac_variable_set(self._h, which, arr.ctypes.data_as(ctypes.c_void_p), _NP2DT[dt]))
+
+    @property
+    def data(self):
+        return NdArray(self, 0)
+
+    @property
+    def grad(self):
+        return NdArray(self, 1)
+
+    def _share_array(self, other, which):
+        """This variable's data or grad becomes a view of ``other``'s."""
+        _capi.check(_capi.lib().nblac_variable_share_array(self._h, other._h, which))
 
     @property
     def d(self):
