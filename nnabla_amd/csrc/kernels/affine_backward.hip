@@ -40,6 +40,8 @@ __global__ __launch_bounds__(256) void scale_columns(const float *__restrict__ d
     out[i] = dy[i] * alpha[i % N];
 }
 
+size_t max3(size_t a, size_t b, size_t c) { return a > b ? (a > c ? a : c) : (b > c ? b : c); }
+
 struct BackwardPlan {
   size_t bits_off, digits_off, prep_off, count_off, a_planes_off, b_planes_off, flag_off, sums_off, scaled_off, total;
 };
@@ -59,10 +61,12 @@ BackwardPlan plan_backward(int64_t M, int64_t K, int64_t N) {
   // bf16 planes: the larger of (x^T, dy) for dW and (dy, W^T) for dx
   const size_t a1 = nbla_hip_split_operand_bytes(K, M), b1 = nbla_hip_split_operand_bytes(N, M);
   const size_t a2 = nbla_hip_split_operand_bytes(M, N), b2 = nbla_hip_split_operand_bytes(K, N);
+  // ... and the digit operands of x^T and dy^T for dW share the same two regions
+  const size_t a3 = nbla_hip_digit_operand_bytes(K, M), b3 = nbla_hip_digit_operand_bytes(N, M);
   p.a_planes_off = off;
-  off += round_up(a1 > a2 ? a1 : a2, 256);
+  off += round_up(max3(a1, a2, a3), 256);
   p.b_planes_off = off;
-  off += round_up(b1 > b2 ? b1 : b2, 256);
+  off += round_up(max3(b1, b2, b3), 256);
   p.flag_off = off;
   off += 256;
   p.sums_off = off;
@@ -73,20 +77,17 @@ BackwardPlan plan_backward(int64_t M, int64_t K, int64_t N) {
   return p;
 }
 
-// dW[K, N] (+)= x^T . dy on the plane x plane product (both factors are real numbers)
+// dW[K, N] (+)= x^T . dy on the digit x digit product (both factors are real numbers): the operand rows are the
+// columns of x and of dy, the contraction runs over the M samples.
 int grad_weights(const float *x, const float *dy, float *dW, int64_t M, int64_t K, int64_t N, bool accumulate,
                  char *base, const BackwardPlan &p, hipStream_t stream) {
-  int *flag = reinterpret_cast<int *>(base + p.flag_off);
-  // x^T as the row operand: rows k, contraction m.  The "weight plane" splitter produces exactly that layout.
-  int dummy_rc = launch_split_weights(x, base + p.a_planes_off, flag, M, K, false, stream);
-  if (dummy_rc)
-    return dummy_rc;
-  int rc = launch_split_weights(dy, base + p.b_planes_off, flag, M, N, false, stream);
+  int rc = launch_split_digits_columns(x, K, base + p.a_planes_off, M, K, stream);
   if (rc)
     return rc;
-  // the flag now tells whether dy needs its lower planes
-  return launch_gemm_planes(base + p.a_planes_off, base + p.b_planes_off, flag, nullptr, nullptr, dW, K, M, N, 1, N, 1,
-                            stream, accumulate);
+  rc = launch_split_digits_columns(dy, N, base + p.b_planes_off, M, N, stream);
+  if (rc)
+    return rc;
+  return launch_gemm_digits(base + p.a_planes_off, base + p.b_planes_off, dW, K, M, N, 1, N, 1, stream, accumulate);
 }
 
 // dx[M, K] (+)= dy' . W^T with real-valued weights, dy' [M, N]

@@ -3,6 +3,7 @@
 // bf16x3 split of the activations.
 #include "common.hpp"
 #include "gemm_layout.hpp"
+#include "internal.hpp"
 
 #include <cmath>
 
@@ -717,8 +718,131 @@ __global__ __launch_bounds__(kPrepBlock) void split_digits_tiled(const float *__
   }
 }
 
+// ---- digit operand of a transposed source: the operand's rows are the columns c of src [R, C] (row stride ld) and
+// its contraction index runs over src's rows, so x^T or dy^T feed the digit x digit product without a transposed
+// copy.  One scale per column: column maxima by integer atomicMax on the magnitude bits (order-independent).
+__global__ __launch_bounds__(kPrepBlock) void clear_words(uint32_t *__restrict__ p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * kPrepBlock + threadIdx.x;
+  if (i < n)
+    p[i] = 0u;
+}
+
+// Block = 64 column quads x 4 row groups over a slab of 64 rows; 128-bit loads where the layout allows, four in
+// flight per thread; the row groups are folded through LDS before the atomics.
+template <bool kVec>
+__global__ __launch_bounds__(kPrepBlock) void column_absmax(const float *__restrict__ src, int64_t ld, int64_t R,
+                                                            int64_t C, uint32_t *__restrict__ cmax) {
+  __shared__ uint32_t part[4][256];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int64_t c0 = ((int64_t)blockIdx.x * 64 + tx) * 4;
+  const int64_t r0 = (int64_t)blockIdx.y * 64;
+  uint32_t m[4] = {0u, 0u, 0u, 0u};
+  if (c0 < C) {
+#pragma unroll 4
+    for (int i = 0; i < 16; ++i) {
+      const int64_t r = r0 + ty + 4 * i;
+      if (r >= R)
+        break;
+      float v[4];
+      if (kVec) {
+        const float4_t q = *reinterpret_cast<const float4_t *>(src + r * ld + c0);
+        v[0] = q.x, v[1] = q.y, v[2] = q.z, v[3] = q.w;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          v[j] = (c0 + j < C) ? src[r * ld + c0 + j] : 0.0f;
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t u = __float_as_uint(v[j]) & 0x7fffffffu;
+        m[j] = u > m[j] ? u : m[j];
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    part[ty][tx * 4 + j] = m[j];
+  __syncthreads();
+  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (c < C) {
+    uint32_t a = part[0][threadIdx.x], b = part[1][threadIdx.x], d = part[2][threadIdx.x], e = part[3][threadIdx.x];
+    a = a > b ? a : b;
+    d = d > e ? d : e;
+    a = a > d ? a : d;
+    if (a)
+      atomicMax(&cmax[c], a);
+  }
+}
+
+// shift of every (padded) operand row from its column maximum; a NaN or an infinity marks the row
+__global__ __launch_bounds__(kPrepBlock) void column_shift(const uint32_t *__restrict__ cmax,
+                                                           int32_t *__restrict__ shift, int64_t C, int64_t rows) {
+  const int64_t c = (int64_t)blockIdx.x * kPrepBlock + threadIdx.x;
+  if (c >= rows)
+    return;
+  const uint32_t m = c < C ? cmax[c] : 0u;
+  shift[c] = m >= 0x7f800000u ? kBadRow : (m == 0u ? 0 : digit_shift(m));
+}
+
+// One wavefront per fragment (32 operand rows = columns of src, 32 contraction steps = rows of src); fragments are
+// numbered with the column block fastest so that a block's four wavefronts read 512 contiguous bytes of each row.
+__global__ __launch_bounds__(kPrepBlock) void split_digits_columns(const float *__restrict__ src, int64_t ld,
+                                                                   const int32_t *__restrict__ shift,
+                                                                   uint4_t *__restrict__ out, int64_t R, int64_t C,
+                                                                   int64_t k_tiles, int64_t col_blocks,
+                                                                   int64_t frags) {
+  const int64_t frag = (int64_t)blockIdx.x * (kPrepBlock / 64) + (threadIdx.x >> 6);
+  if (frag >= frags)
+    return;
+  const int lane = threadIdx.x & 63;
+  const int64_t mt = frag / col_blocks, cb = frag - mt * col_blocks;
+  const int64_t c = cb * kFragRows + (lane & 31);
+  const int64_t r0 = mt * kTileK + (lane >> 5) * 16;
+  const int s = shift[c];
+  const bool live = c < C && s != kBadRow;
+  float v[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j)
+    v[j] = (live && r0 + j < R) ? src[(r0 + j) * ld + c] : 0.0f;
+  int q[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j)
+    q[j] = to_fixed(v[j], s == kBadRow ? 0 : s);
+  store_digits(q, out + (cb * k_tiles + mt) * kDigits * 64 + lane, true);
+}
+
 } // namespace
+
+// Digit operand (rows = the C columns of src, contraction over its R rows); `digits` holds
+// nbla_hip_digit_operand_bytes(C, R).  The operand's row-sum section serves as scratch for the column maxima (the
+// digit x digit product does not read row sums).
+int launch_split_digits_columns(const float *src, int64_t ld, void *digits, int64_t R, int64_t C,
+                                hipStream_t stream) {
+  const DigitOperand d = digit_operand(C, R);
+  char *base = static_cast<char *>(digits);
+  uint32_t *cmax = reinterpret_cast<uint32_t *>(base + d.sum_off);
+  int32_t *shift = reinterpret_cast<int32_t *>(base + d.shift_off);
+  hipLaunchKernelGGL(clear_words, dim3((unsigned)ceil_div(d.rows, kPrepBlock)), dim3(kPrepBlock), 0, stream, cmax,
+                     d.rows);
+  NBLA_HIP_LAUNCH_CHECK("clear_words");
+  const dim3 grid((unsigned)ceil_div(C, 256), (unsigned)ceil_div(R, 64));
+  if (C % 4 == 0 && ld % 4 == 0 && aligned16(src))
+    hipLaunchKernelGGL(column_absmax<true>, grid, dim3(kPrepBlock), 0, stream, src, ld, R, C, cmax);
+  else
+    hipLaunchKernelGGL(column_absmax<false>, grid, dim3(kPrepBlock), 0, stream, src, ld, R, C, cmax);
+  NBLA_HIP_LAUNCH_CHECK("column_absmax");
+  hipLaunchKernelGGL(column_shift, dim3((unsigned)ceil_div(d.rows, kPrepBlock)), dim3(kPrepBlock), 0, stream, cmax,
+                     shift, C, d.rows);
+  NBLA_HIP_LAUNCH_CHECK("column_shift");
+  const int64_t frags = d.k_tiles * d.row_blocks;
+  hipLaunchKernelGGL(split_digits_columns, dim3((unsigned)ceil_div(frags, kPrepBlock / 64)), dim3(kPrepBlock), 0,
+                     stream, src, ld, shift, reinterpret_cast<uint4_t *>(base), R, C, d.k_tiles, d.row_blocks, frags);
+  NBLA_HIP_LAUNCH_CHECK("split_digits_columns");
+  return NBLA_HIP_OK;
+}
+
 } // namespace nbla_hip
+
 
 using namespace nbla_hip;
 

@@ -5,7 +5,7 @@
 // samples at once, with m = (sample, output position) as the long dimension:
 //   dyt [M, Og]          the output gradient of the group, transposed so that m is the row index
 //   colg[n][kk][l]       = sum over o of dyt[m, o] * w[o, kk]   (then folded into dx by a gather)
-//   dW  [Og, Kg]         = dyt^T . col(x)                        (col(x) [M, Kg] is the unfolded input)
+//   dW  [Og, Kg]         = dyt^T . col(x)                        (col(x) [M, Kg] is the unfolded input; digit x digit)
 //   db  [Og]             = column sums of dyt
 #include "common.hpp"
 #include "conv_geom.hpp"
@@ -99,9 +99,13 @@ ConvBackwardPlan plan_conv_backward(const ConvGeom &g) {
   p.col_off = off; // unfolded input [M, Kg], and the unfolded gradient [outer][Kg][L]
   off += round_up((size_t)g.M * g.Kg * sizeof(float), 256);
   p.a_planes_off = off; // dyt^T for dW (rows o, contraction m) or dyt for dx (rows m, contraction o)
-  off += round_up(larger(nbla_hip_split_operand_bytes(g.Og, g.M), nbla_hip_split_operand_bytes(g.M, g.Og)), 256);
+  off += round_up(larger(larger(nbla_hip_split_operand_bytes(g.Og, g.M), nbla_hip_split_operand_bytes(g.M, g.Og)),
+                         nbla_hip_digit_operand_bytes(g.Og, g.M)),
+                  256);
   p.b_planes_off = off; // col(x) (columns kk, contraction m) or w (columns kk, contraction o)
-  off += round_up(larger(nbla_hip_split_operand_bytes(g.Kg, g.M), nbla_hip_split_operand_bytes(g.Kg, g.Og)), 256);
+  off += round_up(larger(larger(nbla_hip_split_operand_bytes(g.Kg, g.M), nbla_hip_split_operand_bytes(g.Kg, g.Og)),
+                         nbla_hip_digit_operand_bytes(g.Kg, g.M)),
+                  256);
   p.digits_off = off;
   off += round_up(nbla_hip_digit_operand_bytes(g.M, g.Og), 256);
   p.bits_off = off;
@@ -223,15 +227,15 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
       rc = launch_im2col_f32(x, col, g, grp, stream);
       if (rc)
         return rc;
-      // dyt^T as the row operand (rows o, contraction m) and col(x) as the column operand (columns kk)
-      rc = launch_split_weights(dyt, base + p.a_planes_off, flag, g.M, g.Og, false, stream);
+      // digit operands of dyt^T (rows o) and col(x)^T (rows kk), contraction over the pixels m
+      rc = launch_split_digits_columns(dyt, g.Og, base + p.a_planes_off, g.M, g.Og, stream);
       if (rc)
         return rc;
-      rc = launch_split_weights(col, base + p.b_planes_off, flag, g.M, g.Kg, false, stream);
+      rc = launch_split_digits_columns(col, g.Kg, base + p.b_planes_off, g.M, g.Kg, stream);
       if (rc)
         return rc;
-      rc = launch_gemm_planes(base + p.a_planes_off, base + p.b_planes_off, flag, nullptr, nullptr,
-                              dW + grp * g.Og * g.Kg, g.Og, g.M, g.Kg, 1, g.Kg, 1, stream, accum_w);
+      rc = launch_gemm_digits(base + p.a_planes_off, base + p.b_planes_off, dW + grp * g.Og * g.Kg, g.Og, g.M, g.Kg, 1,
+                              g.Kg, 1, stream, accum_w);
       if (rc)
         return rc;
     }

@@ -1,0 +1,216 @@
+// Product of two real-valued matrices on the int8 matrix cores: y[m, n] = sum_k A[m, k] * B[n, k] with both
+// operands as digit operands (per row a power-of-two scale and three balanced base-256 int8 digits, see
+// gemm_layout.hpp).  With qa = a0 * 2^16 + a1 * 2^8 + a2 and qb likewise,
+//     qa * qb = a0 b0 * 2^32 + (a0 b1 + a1 b0) * 2^24 + (a0 b2 + a1 b1 + a2 b0) * 2^16 + (lower terms)
+// and the six leading digit products are accumulated exactly in three int32 accumulators per output (one per power
+// of 256); the dropped terms are below 2^-23 of |row max| * |column max| per k.  The epilogue combines the three
+// sums in 64-bit integers, converts once and applies the two scales, so the result does not depend on the order of
+// summation.  Used for the weight gradients (x^T . dy), where neither factor is a sign matrix.
+//
+// Tiling: 128 x 128 outputs per block of four wavefronts (2 x 2, 64 x 64 each: 2 x 2 fragments x 3 accumulators =
+// 192 registers), k in tiles of 32 (one v_mfma_i32_32x32x32_i8 fragment).
+#include "common.hpp"
+#include "gemm_layout.hpp"
+#include "internal.hpp"
+
+namespace nbla_hip {
+namespace {
+
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+struct GemmDigitsArgs {
+  const uint4_t *ad, *bd; // [row blocks][k tiles][3][64] uint4 each
+  const int32_t *ashift, *bshift;
+  float *y;
+  int64_t M, N, a_row_blocks, b_row_blocks, k_tiles, step_begin, step_end, blocks_m, blocks_n;
+  int64_t inner, outer_stride, n_stride;
+  int accumulate;
+};
+
+constexpr int kBM = 128, kBN = 128, kThreads = 256, kWaves = 4;
+constexpr int kSegs = 4;               // 32-row fragments per tile side
+constexpr int kSegVec = kDigits * 64;  // uint4 per fragment and k step
+constexpr int kSideVec = kSegs * kSegVec;
+constexpr int kStageBytes = 2 * kSideVec * 16; // 24 KiB: the A and B fragments of one k tile
+constexpr int kStages = 3;
+constexpr int kChunks = 2 * kSegs * kDigits;   // 1 KiB copies per k tile
+constexpr int kPerWave = kChunks / kWaves;     // 6
+constexpr int kSmemBytes = kStages * kStageBytes;
+
+// Workgroup barrier without the memory fence of __syncthreads() (which would wait for every global -> LDS copy in
+// flight, including those of later k tiles); the waits that matter are explicit.
+#define NBLA_BARRIER()                                                                                                 \
+  do {                                                                                                                 \
+    asm volatile("" ::: "memory");                                                                                     \
+    __builtin_amdgcn_s_barrier();                                                                                      \
+    asm volatile("" ::: "memory");                                                                                     \
+  } while (0)
+// vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
+#define NBLA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xf) | (((n) >> 4) << 14) | (0x7 << 4) | (0xf << 8))
+
+// Staging: global -> LDS copies bypass the registers (one wavefront instruction moves one 1 KiB fragment); three
+// LDS buffers hold consecutive k tiles and the copy of tile t + 2 is issued while tile t is multiplied.  Two blocks
+// share a CU (256 registers per lane: 192 accumulators + the 12 operand quads of a tile), so one block's LDS reads
+// and barrier waits are covered by the other's MFMAs.
+__global__ __launch_bounds__(kThreads, 2) void gemm_digits_kernel(GemmDigitsArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__) // the host pass only needs the launch stub; the body uses LDS address-space pointers
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave & 1, wn = wave >> 1;
+  int64_t bm, bn;
+  band_tile<4>(blockIdx.x, a.blocks_m, a.blocks_n, bm, bn);
+
+  // this wavefront's copies: chunk c = p * kWaves + wave of the stage; chunks [0, 12) are A fragments (row block,
+  // digit), [12, 24) B fragments
+  const uint4_t *cur[kPerWave], *cur_last[kPerWave];
+#pragma unroll
+  for (int p = 0; p < kPerWave; ++p) {
+    const int c = p * kWaves + wave;
+    const int side = c / (kSegs * kDigits), r = c - side * (kSegs * kDigits);
+    const int seg = r / kDigits, d = r - seg * kDigits;
+    int64_t rb = (side ? bn : bm) * kSegs + seg;
+    const int64_t limit = side ? a.b_row_blocks : a.a_row_blocks;
+    if (rb >= limit)
+      rb = limit - 1; // clamped: those rows / columns are not stored
+    const uint4_t *base = (side ? a.bd : a.ad) + (rb * a.k_tiles * kDigits + d) * 64;
+    cur[p] = base + a.step_begin * kSegVec;
+    cur_last[p] = base + (a.step_end - 1) * kSegVec;
+  }
+  typedef __attribute__((address_space(3))) void lds_void_t;
+  auto copy_next = [&](int buf) {
+#pragma unroll
+    for (int p = 0; p < kPerWave; ++p) {
+      __builtin_amdgcn_global_load_lds(cur[p] + lane,
+                                       (lds_void_t *)(smem + buf * kStageBytes + (p * kWaves + wave) * kFragBytes), 16,
+                                       0, 0);
+      const uint4_t *next = cur[p] + kSegVec;
+      cur[p] = next < cur_last[p] ? next : cur_last[p]; // the last calls copy the final tile again
+    }
+  };
+
+  i32x16_t acc[2][2][3];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int t = 0; t < 3; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          acc[i][j][t][r] = 0;
+
+  copy_next(0);
+  copy_next(1);
+  int buf = 0;
+  for (int64_t kt = a.step_begin; kt < a.step_end; ++kt) {
+    // tile kt has landed (the copies of tile kt + 1 may still be in flight) and every wavefront is done with the
+    // buffer tile kt - 1 occupied, which tile kt + 2 takes over
+    NBLA_WAIT_VMCNT(kPerWave);
+    NBLA_BARRIER();
+    copy_next(buf == 0 ? kStages - 1 : buf - 1);
+    const uint4_t *sa = reinterpret_cast<const uint4_t *>(smem + buf * kStageBytes);
+    const uint4_t *sb = sa + kSideVec;
+    i32x4_t af[2][3], bf[2][3];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int d = 0; d < 3; ++d) {
+        af[i][d] = __builtin_bit_cast(i32x4_t, sa[((wm * 2 + i) * kDigits + d) * 64 + lane]);
+        bf[i][d] = __builtin_bit_cast(i32x4_t, sb[((wn * 2 + i) * kDigits + d) * 64 + lane]);
+      }
+    // digit pairs (a digit, b digit) -> accumulator a + b
+    constexpr int da[6] = {0, 0, 1, 0, 1, 2};
+    constexpr int db[6] = {0, 1, 0, 2, 1, 0};
+#pragma unroll
+    for (int t = 0; t < 6; ++t)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j][da[t] + db[t]] =
+              __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i][da[t]], bf[j][db[t]], acc[i][j][da[t] + db[t]], 0, 0, 0);
+    buf = (buf + 1 == kStages) ? 0 : buf + 1;
+  }
+  NBLA_WAIT_VMCNT(0);
+
+  // y = (acc0 * 2^16 + acc1 * 2^8 + acc2) * 2^(16 - sa - sb)
+  const int col_in_frag = lane & 31, row_half = lane >> 5;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int64_t n = bn * kBN + (wn * 2 + j) * 32 + col_in_frag;
+    if (n >= a.N)
+      continue;
+    const int32_t sb_n = a.bshift[n];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int64_t m0 = bm * kBM + (wm * 2 + i) * 32;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int64_t m = m0 + 8 * (r >> 2) + 4 * row_half + (r & 3);
+        if (m < a.M) {
+          const int32_t sa_m = a.ashift[m];
+          float v;
+          if (sa_m == kBadRow || sb_n == kBadRow) {
+            v = __uint_as_float(0x7fc00000u);
+          } else {
+            const long long t = ((long long)acc[i][j][0][r] << 16) + ((long long)acc[i][j][1][r] << 8) +
+                                (long long)acc[i][j][2][r];
+            // the two shifts are applied one after the other: each stays inside ldexpf's exponent range
+            v = ldexpf(ldexpf((float)t, 16 - sa_m), -sb_n);
+          }
+          const int64_t off = (a.inner == 1) ? m * a.outer_stride : (m / a.inner) * a.outer_stride + (m % a.inner);
+          float *dst = a.y + off + n * a.n_stride;
+          *dst = a.accumulate ? *dst + v : v;
+        }
+      }
+    }
+  }
+#endif
+}
+
+} // namespace
+
+int launch_gemm_digits(const void *adigits, const void *bdigits, float *y, int64_t M, int64_t K, int64_t N,
+                       int64_t inner, int64_t outer_stride, int64_t n_stride, hipStream_t stream, bool accumulate) {
+  const DigitOperand da = digit_operand(M, K), db = digit_operand(N, K);
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_digits_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
+    if (e != hipSuccess)
+      return fail_hip(e, "hipFuncSetAttribute(gemm_digits LDS size)");
+    configured = true;
+  }
+  GemmDigitsArgs a;
+  a.ad = static_cast<const uint4_t *>(adigits);
+  a.bd = static_cast<const uint4_t *>(bdigits);
+  a.ashift = reinterpret_cast<const int32_t *>(static_cast<const char *>(adigits) + da.shift_off);
+  a.bshift = reinterpret_cast<const int32_t *>(static_cast<const char *>(bdigits) + db.shift_off);
+  a.y = y;
+  a.M = M;
+  a.N = N;
+  a.a_row_blocks = da.row_blocks;
+  a.b_row_blocks = db.row_blocks;
+  a.k_tiles = da.k_tiles;
+  a.blocks_m = ceil_div(M, kBM);
+  a.blocks_n = ceil_div(N, kBN);
+  a.inner = inner;
+  a.outer_stride = outer_stride;
+  a.n_stride = n_stride;
+  // chunks of kChunkK contraction elements keep the int32 sums below 2^31; their fp32 results are added up
+  const int64_t tiles_per_chunk = kChunkK / kTileK;
+  for (int64_t t0 = 0, chunk = 0; t0 < a.k_tiles; t0 += tiles_per_chunk, ++chunk) {
+    a.step_begin = t0;
+    a.step_end = (t0 + tiles_per_chunk < a.k_tiles) ? t0 + tiles_per_chunk : a.k_tiles;
+    a.accumulate = (accumulate || chunk > 0) ? 1 : 0;
+    hipLaunchKernelGGL(gemm_digits_kernel, dim3((unsigned)(a.blocks_m * a.blocks_n)), dim3(kThreads), kSmemBytes, stream,
+                       a);
+    NBLA_HIP_LAUNCH_CHECK("gemm_digits");
+  }
+  return NBLA_HIP_OK;
+}
+
+} // namespace nbla_hip

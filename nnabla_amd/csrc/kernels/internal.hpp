@@ -27,6 +27,13 @@ int launch_gemm_planes(const void *xsplit, const void *wplanes, const int *need_
                        const float *bias, float *y, int64_t M, int64_t K, int64_t N, int64_t inner,
                        int64_t outer_stride, int64_t n_stride, hipStream_t stream, bool accumulate = false);
 
+// Digit operand whose rows are the C columns of src [R, C] (row stride ld), contraction over src's rows.
+int launch_split_digits_columns(const float *src, int64_t ld, void *digits, int64_t R, int64_t C, hipStream_t stream);
+// y[m, n] (+)= sum_k A[m, k] * B[n, k], both factors real-valued digit operands (rows M x K and N x K).
+int launch_gemm_digits(const void *adigits, const void *bdigits, float *y, int64_t M, int64_t K, int64_t N,
+                       int64_t inner, int64_t outer_stride, int64_t n_stride, hipStream_t stream,
+                       bool accumulate = false);
+
 // db[n] (+)= sum over m of dy[m, n]; `partial` holds ceil(M / 256) * N floats.
 size_t column_sums_workspace_bytes(int64_t M, int64_t N);
 int launch_column_sums(const float *dy, float *db, int64_t M, int64_t N, bool accumulate, void *partial,
