@@ -81,13 +81,14 @@ BackwardPlan plan_backward(int64_t M, int64_t K, int64_t N) {
 // columns of x and of dy, the contraction runs over the M samples.
 int grad_weights(const float *x, const float *dy, float *dW, int64_t M, int64_t K, int64_t N, bool accumulate,
                  char *base, const BackwardPlan &p, hipStream_t stream) {
-  int rc = launch_split_digits_columns(x, K, base + p.a_planes_off, M, K, stream);
+  int rc = launch_split_digits_columns(x, K, base + p.a_planes_off, M, K, false, stream);
   if (rc)
     return rc;
-  rc = launch_split_digits_columns(dy, N, base + p.b_planes_off, M, N, stream);
+  rc = launch_split_digits_columns(dy, N, base + p.b_planes_off, M, N, false, stream);
   if (rc)
     return rc;
-  return launch_gemm_digits(base + p.a_planes_off, base + p.b_planes_off, dW, K, M, N, 1, N, 1, stream, accumulate);
+  return launch_gemm_digits(base + p.a_planes_off, base + p.b_planes_off, nullptr, dW, K, M, N, 1, N, 1, stream,
+                            accumulate);
 }
 
 // dx[M, K] (+)= dy' . W^T with real-valued weights, dy' [M, N]

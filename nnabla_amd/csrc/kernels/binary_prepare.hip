@@ -719,24 +719,39 @@ __global__ __launch_bounds__(kPrepBlock) void split_digits_tiled(const float *__
 }
 
 // ---- digit operand of a transposed source: the operand's rows are the columns c of src [R, C] (row stride ld) and
-// its contraction index runs over src's rows, so x^T or dy^T feed the digit x digit product without a transposed
-// copy.  One scale per column: column maxima by integer atomicMax on the magnitude bits (order-independent).
-__global__ __launch_bounds__(kPrepBlock) void clear_words(uint32_t *__restrict__ p, int64_t n) {
+// its contraction index runs over src's rows, so x^T, dy^T or W^T feed the digit x digit product without a
+// transposed copy.  One scale per column: column maxima by integer atomicMax on the magnitude bits
+// (order-independent).
+//
+// With `detect` the pass also finds out whether every element is zero or a signed power of two no more than six
+// binades below its column's largest (INQ weights once they are fixed): then the scale is chosen so that each
+// value is an integer of magnitude <= 64 and sits in the lowest digit alone ("narrow" operand, flag word 0), and
+// the product needs three digit products instead of six and drops nothing.
+__global__ __launch_bounds__(kPrepBlock) void clear_column_scratch(uint32_t *__restrict__ cmax,
+                                                                   uint32_t *__restrict__ cmin, int64_t n,
+                                                                   int32_t *__restrict__ flag, int flag_value) {
   const int64_t i = (int64_t)blockIdx.x * kPrepBlock + threadIdx.x;
-  if (i < n)
-    p[i] = 0u;
+  if (i < n) {
+    cmax[i] = 0u;
+    cmin[i] = 0xffffffffu;
+  }
+  if (i == 0)
+    *flag = flag_value;
 }
 
 // Block = 64 column quads x 4 row groups over a slab of 64 rows; 128-bit loads where the layout allows, four in
 // flight per thread; the row groups are folded through LDS before the atomics.
-template <bool kVec>
+template <bool kVec, bool kDetect>
 __global__ __launch_bounds__(kPrepBlock) void column_absmax(const float *__restrict__ src, int64_t ld, int64_t R,
-                                                            int64_t C, uint32_t *__restrict__ cmax) {
+                                                            int64_t C, uint32_t *__restrict__ cmax,
+                                                            uint32_t *__restrict__ cmin, int32_t *__restrict__ flag) {
   __shared__ uint32_t part[4][256];
+  __shared__ uint32_t part_min[kDetect ? 4 : 1][256];
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   const int64_t c0 = ((int64_t)blockIdx.x * 64 + tx) * 4;
   const int64_t r0 = (int64_t)blockIdx.y * 64;
-  uint32_t m[4] = {0u, 0u, 0u, 0u};
+  uint32_t m[4] = {0u, 0u, 0u, 0u}, mn[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+  bool other = false; // an element that is neither zero nor a normal power of two
   if (c0 < C) {
 #pragma unroll 4
     for (int i = 0; i < 16; ++i) {
@@ -756,12 +771,22 @@ __global__ __launch_bounds__(kPrepBlock) void column_absmax(const float *__restr
       for (int j = 0; j < 4; ++j) {
         const uint32_t u = __float_as_uint(v[j]) & 0x7fffffffu;
         m[j] = u > m[j] ? u : m[j];
+        if (kDetect && u) {
+          mn[j] = u < mn[j] ? u : mn[j];
+          other |= (u & 0x007fffffu) != 0u || (u >> 23) == 0u;
+        }
       }
     }
   }
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+  for (int j = 0; j < 4; ++j) {
     part[ty][tx * 4 + j] = m[j];
+    if (kDetect)
+      part_min[ty][tx * 4 + j] = mn[j];
+  }
+  if (kDetect && __any(other) && (threadIdx.x & 63) == 0 &&
+      __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
+    atomicOr(flag, 1);
   __syncthreads();
   const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (c < C) {
@@ -771,23 +796,51 @@ __global__ __launch_bounds__(kPrepBlock) void column_absmax(const float *__restr
     a = a > d ? a : d;
     if (a)
       atomicMax(&cmax[c], a);
+    if (kDetect) {
+      a = part_min[0][threadIdx.x], b = part_min[1][threadIdx.x], d = part_min[2][threadIdx.x];
+      e = part_min[3][threadIdx.x];
+      a = a < b ? a : b;
+      d = d < e ? d : e;
+      a = a < d ? a : d;
+      if (a != 0xffffffffu)
+        atomicMin(&cmin[c], a);
+    }
   }
 }
 
-// shift of every (padded) operand row from its column maximum; a NaN or an infinity marks the row
-__global__ __launch_bounds__(kPrepBlock) void column_shift(const uint32_t *__restrict__ cmax,
-                                                           int32_t *__restrict__ shift, int64_t C, int64_t rows) {
+// Shift of every (padded) operand row from its column maximum; a NaN or an infinity marks the row.  The narrow
+// shift (largest element -> 64) replaces the maximum in `cmax`; a column spanning more than six binades raises the
+// flag.
+__global__ __launch_bounds__(kPrepBlock) void column_shift(uint32_t *__restrict__ cmax,
+                                                           const uint32_t *__restrict__ cmin,
+                                                           int32_t *__restrict__ shift, int64_t C, int64_t rows,
+                                                           int32_t *__restrict__ flag, int detect) {
   const int64_t c = (int64_t)blockIdx.x * kPrepBlock + threadIdx.x;
   if (c >= rows)
     return;
   const uint32_t m = c < C ? cmax[c] : 0u;
-  shift[c] = m >= 0x7f800000u ? kBadRow : (m == 0u ? 0 : digit_shift(m));
+  const bool bad = m >= 0x7f800000u;
+  shift[c] = bad ? kBadRow : (m == 0u ? 0 : digit_shift(m));
+  if (detect) {
+    int narrow = 0;
+    if (bad) {
+      narrow = kBadRow;
+    } else if (m != 0u) {
+      const int e_max = (int)(m >> 23) - 127, e_min = (int)(cmin[c] >> 23) - 127;
+      narrow = 6 - e_max;
+      if (e_max - e_min > 6 && __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
+        atomicOr(flag, 1);
+    }
+    cmax[c] = (uint32_t)narrow;
+  }
 }
 
 // One wavefront per fragment (32 operand rows = columns of src, 32 contraction steps = rows of src); fragments are
 // numbered with the column block fastest so that a block's four wavefronts read 512 contiguous bytes of each row.
 __global__ __launch_bounds__(kPrepBlock) void split_digits_columns(const float *__restrict__ src, int64_t ld,
                                                                    const int32_t *__restrict__ shift,
+                                                                   const int32_t *__restrict__ narrow_shift,
+                                                                   const int32_t *__restrict__ flag,
                                                                    uint4_t *__restrict__ out, int64_t R, int64_t C,
                                                                    int64_t k_tiles, int64_t col_blocks,
                                                                    int64_t frags) {
@@ -798,7 +851,7 @@ __global__ __launch_bounds__(kPrepBlock) void split_digits_columns(const float *
   const int64_t mt = frag / col_blocks, cb = frag - mt * col_blocks;
   const int64_t c = cb * kFragRows + (lane & 31);
   const int64_t r0 = mt * kTileK + (lane >> 5) * 16;
-  const int s = shift[c];
+  const int s = (*flag == 0) ? narrow_shift[c] : shift[c];
   const bool live = c < C && s != kBadRow;
   float v[16];
 #pragma unroll
@@ -814,29 +867,40 @@ __global__ __launch_bounds__(kPrepBlock) void split_digits_columns(const float *
 } // namespace
 
 // Digit operand (rows = the C columns of src, contraction over its R rows); `digits` holds
-// nbla_hip_digit_operand_bytes(C, R).  The operand's row-sum section serves as scratch for the column maxima (the
-// digit x digit product does not read row sums).
-int launch_split_digits_columns(const float *src, int64_t ld, void *digits, int64_t R, int64_t C,
+// nbla_hip_digit_operand_bytes(C, R).  The operand's row-sum section serves as scratch (column maxima, then the
+// narrow shifts, and the column minima); the digit x digit product does not read row sums.
+int launch_split_digits_columns(const float *src, int64_t ld, void *digits, int64_t R, int64_t C, bool detect_narrow,
                                 hipStream_t stream) {
   const DigitOperand d = digit_operand(C, R);
   char *base = static_cast<char *>(digits);
   uint32_t *cmax = reinterpret_cast<uint32_t *>(base + d.sum_off);
+  uint32_t *cmin = cmax + d.rows;
   int32_t *shift = reinterpret_cast<int32_t *>(base + d.shift_off);
-  hipLaunchKernelGGL(clear_words, dim3((unsigned)ceil_div(d.rows, kPrepBlock)), dim3(kPrepBlock), 0, stream, cmax,
-                     d.rows);
-  NBLA_HIP_LAUNCH_CHECK("clear_words");
+  int32_t *flag = reinterpret_cast<int32_t *>(base + d.flag_off);
+  hipLaunchKernelGGL(clear_column_scratch, dim3((unsigned)ceil_div(d.rows, kPrepBlock)), dim3(kPrepBlock), 0, stream,
+                     cmax, cmin, d.rows, flag, detect_narrow ? 0 : 1);
+  NBLA_HIP_LAUNCH_CHECK("clear_column_scratch");
   const dim3 grid((unsigned)ceil_div(C, 256), (unsigned)ceil_div(R, 64));
-  if (C % 4 == 0 && ld % 4 == 0 && aligned16(src))
-    hipLaunchKernelGGL(column_absmax<true>, grid, dim3(kPrepBlock), 0, stream, src, ld, R, C, cmax);
+  const bool vec = C % 4 == 0 && ld % 4 == 0 && aligned16(src);
+#define NBLA_LAUNCH_ABSMAX(V, D)                                                                                       \
+  hipLaunchKernelGGL((column_absmax<V, D>), grid, dim3(kPrepBlock), 0, stream, src, ld, R, C, cmax, cmin, flag)
+  if (vec && detect_narrow)
+    NBLA_LAUNCH_ABSMAX(true, true);
+  else if (vec)
+    NBLA_LAUNCH_ABSMAX(true, false);
+  else if (detect_narrow)
+    NBLA_LAUNCH_ABSMAX(false, true);
   else
-    hipLaunchKernelGGL(column_absmax<false>, grid, dim3(kPrepBlock), 0, stream, src, ld, R, C, cmax);
+    NBLA_LAUNCH_ABSMAX(false, false);
+#undef NBLA_LAUNCH_ABSMAX
   NBLA_HIP_LAUNCH_CHECK("column_absmax");
   hipLaunchKernelGGL(column_shift, dim3((unsigned)ceil_div(d.rows, kPrepBlock)), dim3(kPrepBlock), 0, stream, cmax,
-                     shift, C, d.rows);
+                     cmin, shift, C, d.rows, flag, detect_narrow ? 1 : 0);
   NBLA_HIP_LAUNCH_CHECK("column_shift");
   const int64_t frags = d.k_tiles * d.row_blocks;
   hipLaunchKernelGGL(split_digits_columns, dim3((unsigned)ceil_div(frags, kPrepBlock / 64)), dim3(kPrepBlock), 0,
-                     stream, src, ld, shift, reinterpret_cast<uint4_t *>(base), R, C, d.k_tiles, d.row_blocks, frags);
+                     stream, src, ld, shift, reinterpret_cast<const int32_t *>(cmax), flag,
+                     reinterpret_cast<uint4_t *>(base), R, C, d.k_tiles, d.row_blocks, frags);
   NBLA_HIP_LAUNCH_CHECK("split_digits_columns");
   return NBLA_HIP_OK;
 }

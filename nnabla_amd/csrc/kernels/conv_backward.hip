@@ -228,14 +228,14 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
       if (rc)
         return rc;
       // digit operands of dyt^T (rows o) and col(x)^T (rows kk), contraction over the pixels m
-      rc = launch_split_digits_columns(dyt, g.Og, base + p.a_planes_off, g.M, g.Og, stream);
+      rc = launch_split_digits_columns(dyt, g.Og, base + p.a_planes_off, g.M, g.Og, false, stream);
       if (rc)
         return rc;
-      rc = launch_split_digits_columns(col, g.Kg, base + p.b_planes_off, g.M, g.Kg, stream);
+      rc = launch_split_digits_columns(col, g.Kg, base + p.b_planes_off, g.M, g.Kg, false, stream);
       if (rc)
         return rc;
-      rc = launch_gemm_digits(base + p.a_planes_off, base + p.b_planes_off, dW + grp * g.Og * g.Kg, g.Og, g.M, g.Kg, 1,
-                              g.Kg, 1, stream, accum_w);
+      rc = launch_gemm_digits(base + p.a_planes_off, base + p.b_planes_off, nullptr, dW + grp * g.Og * g.Kg, g.Og, g.M,
+                              g.Kg, 1, g.Kg, 1, stream, accum_w);
       if (rc)
         return rc;
     }

@@ -22,11 +22,13 @@ typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
 struct GemmDigitsArgs {
   const uint4_t *ad, *bd; // [row blocks][k tiles][3][64] uint4 each
-  const int32_t *ashift, *bshift;
+  const int32_t *ashift, *bshift, *bshift_narrow, *bflag;
+  const float *bias;
   float *y;
   int64_t M, N, a_row_blocks, b_row_blocks, k_tiles, step_begin, step_end, blocks_m, blocks_n;
   int64_t inner, outer_stride, n_stride;
-  int accumulate;
+  int accumulate; // add to y instead of overwriting it
+  int finish;     // last chunk of the contraction: add the bias
 };
 
 constexpr int kBM = 128, kBN = 128, kThreads = 256, kWaves = 4;
@@ -54,9 +56,11 @@ constexpr int kSmemBytes = kStages * kStageBytes;
 // LDS buffers hold consecutive k tiles and the copy of tile t + 2 is issued while tile t is multiplied.  Two blocks
 // share a CU (256 registers per lane: 192 accumulators + the 12 operand quads of a tile), so one block's LDS reads
 // and barrier waits are covered by the other's MFMAs.
-__global__ __launch_bounds__(kThreads, 2) void gemm_digits_kernel(GemmDigitsArgs a) {
+// kNarrow: the B operand holds every value in its lowest digit alone (a small integer): three products
+// a_t x b2 -> accumulator t, nothing dropped, and only the lowest-digit fragments of B are copied.
+template <bool kNarrow>
+__device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsigned char *smem) {
 #if defined(__HIP_DEVICE_COMPILE__) // the host pass only needs the launch stub; the body uses LDS address-space pointers
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave & 1, wn = wave >> 1;
@@ -80,9 +84,13 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_digits_kernel(GemmDigitsArgs
     cur_last[p] = base + (a.step_end - 1) * kSegVec;
   }
   typedef __attribute__((address_space(3))) void lds_void_t;
+  // narrow: of a wavefront's six chunks the three A fragments and exactly one B fragment (digit 2) are needed
+  constexpr int kCopies = kNarrow ? 4 : kPerWave;
   auto copy_next = [&](int buf) {
 #pragma unroll
     for (int p = 0; p < kPerWave; ++p) {
+      if (kNarrow && p >= 3 && ((p * kWaves + wave) - kSegs * kDigits) % kDigits != 2)
+        continue;
       __builtin_amdgcn_global_load_lds(cur[p] + lane,
                                        (lds_void_t *)(smem + buf * kStageBytes + (p * kWaves + wave) * kFragBytes), 16,
                                        0, 0);
@@ -108,7 +116,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_digits_kernel(GemmDigitsArgs
   for (int64_t kt = a.step_begin; kt < a.step_end; ++kt) {
     // tile kt has landed (the copies of tile kt + 1 may still be in flight) and every wavefront is done with the
     // buffer tile kt - 1 occupied, which tile kt + 2 takes over
-    NBLA_WAIT_VMCNT(kPerWave);
+    NBLA_WAIT_VMCNT(kCopies);
     NBLA_BARRIER();
     copy_next(buf == 0 ? kStages - 1 : buf - 1);
     const uint4_t *sa = reinterpret_cast<const uint4_t *>(smem + buf * kStageBytes);
@@ -119,31 +127,44 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_digits_kernel(GemmDigitsArgs
 #pragma unroll
       for (int d = 0; d < 3; ++d) {
         af[i][d] = __builtin_bit_cast(i32x4_t, sa[((wm * 2 + i) * kDigits + d) * 64 + lane]);
-        bf[i][d] = __builtin_bit_cast(i32x4_t, sb[((wn * 2 + i) * kDigits + d) * 64 + lane]);
+        if (!kNarrow || d == 2)
+          bf[i][d] = __builtin_bit_cast(i32x4_t, sb[((wn * 2 + i) * kDigits + d) * 64 + lane]);
       }
-    // digit pairs (a digit, b digit) -> accumulator a + b
-    constexpr int da[6] = {0, 0, 1, 0, 1, 2};
-    constexpr int db[6] = {0, 1, 0, 2, 1, 0};
+    if (kNarrow) {
 #pragma unroll
-    for (int t = 0; t < 6; ++t)
+      for (int t = 0; t < 3; ++t)
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j][da[t] + db[t]] =
-              __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i][da[t]], bf[j][db[t]], acc[i][j][da[t] + db[t]], 0, 0, 0);
+          for (int j = 0; j < 2; ++j)
+            acc[i][j][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i][t], bf[j][2], acc[i][j][t], 0, 0, 0);
+    } else {
+      // digit pairs (a digit, b digit) -> accumulator a + b
+      constexpr int da[6] = {0, 0, 1, 0, 1, 2};
+      constexpr int db[6] = {0, 1, 0, 2, 1, 0};
+#pragma unroll
+      for (int t = 0; t < 6; ++t)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc[i][j][da[t] + db[t]] =
+                __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i][da[t]], bf[j][db[t]], acc[i][j][da[t] + db[t]], 0, 0, 0);
+    }
     buf = (buf + 1 == kStages) ? 0 : buf + 1;
   }
   NBLA_WAIT_VMCNT(0);
 
-  // y = (acc0 * 2^16 + acc1 * 2^8 + acc2) * 2^(16 - sa - sb)
+  // y = (acc0 * 2^16 + acc1 * 2^8 + acc2) * 2^(16 - sa - sb); the narrow form has no factor 2^16 (b is its low digit)
   const int col_in_frag = lane & 31, row_half = lane >> 5;
+  const int32_t *bshift = kNarrow ? a.bshift_narrow : a.bshift;
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int64_t n = bn * kBN + (wn * 2 + j) * 32 + col_in_frag;
     if (n >= a.N)
       continue;
-    const int32_t sb_n = a.bshift[n];
+    const int32_t sb_n = bshift[n];
+    const float bias = (a.bias && a.finish) ? a.bias[n] : 0.0f;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int64_t m0 = bm * kBM + (wm * 2 + i) * 32;
@@ -159,11 +180,15 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_digits_kernel(GemmDigitsArgs
             const long long t = ((long long)acc[i][j][0][r] << 16) + ((long long)acc[i][j][1][r] << 8) +
                                 (long long)acc[i][j][2][r];
             // the two shifts are applied one after the other: each stays inside ldexpf's exponent range
-            v = ldexpf(ldexpf((float)t, 16 - sa_m), -sb_n);
+            v = ldexpf(ldexpf((float)t, (kNarrow ? 0 : 16) - sa_m), -sb_n);
           }
           const int64_t off = (a.inner == 1) ? m * a.outer_stride : (m / a.inner) * a.outer_stride + (m % a.inner);
           float *dst = a.y + off + n * a.n_stride;
-          *dst = a.accumulate ? *dst + v : v;
+          if (a.accumulate)
+            v = *dst + v;
+          if (a.bias && a.finish)
+            v = v + bias;
+          *dst = v;
         }
       }
     }
@@ -171,10 +196,19 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_digits_kernel(GemmDigitsArgs
 #endif
 }
 
+__global__ __launch_bounds__(kThreads, 2) void gemm_digits_kernel(GemmDigitsArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  if (*a.bflag == 0) // uniform over the grid
+    gemm_digits_tile<true>(a, smem);
+  else
+    gemm_digits_tile<false>(a, smem);
+}
+
 } // namespace
 
-int launch_gemm_digits(const void *adigits, const void *bdigits, float *y, int64_t M, int64_t K, int64_t N,
-                       int64_t inner, int64_t outer_stride, int64_t n_stride, hipStream_t stream, bool accumulate) {
+int launch_gemm_digits(const void *adigits, const void *bdigits, const float *bias, float *y, int64_t M, int64_t K,
+                       int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride, hipStream_t stream,
+                       bool accumulate) {
   const DigitOperand da = digit_operand(M, K), db = digit_operand(N, K);
   static bool configured = false;
   if (!configured) {
@@ -189,6 +223,9 @@ int launch_gemm_digits(const void *adigits, const void *bdigits, float *y, int64
   a.bd = static_cast<const uint4_t *>(bdigits);
   a.ashift = reinterpret_cast<const int32_t *>(static_cast<const char *>(adigits) + da.shift_off);
   a.bshift = reinterpret_cast<const int32_t *>(static_cast<const char *>(bdigits) + db.shift_off);
+  a.bshift_narrow = reinterpret_cast<const int32_t *>(static_cast<const char *>(bdigits) + db.sum_off);
+  a.bflag = reinterpret_cast<const int32_t *>(static_cast<const char *>(bdigits) + db.flag_off);
+  a.bias = bias;
   a.y = y;
   a.M = M;
   a.N = N;
@@ -206,6 +243,7 @@ int launch_gemm_digits(const void *adigits, const void *bdigits, float *y, int64
     a.step_begin = t0;
     a.step_end = (t0 + tiles_per_chunk < a.k_tiles) ? t0 + tiles_per_chunk : a.k_tiles;
     a.accumulate = (accumulate || chunk > 0) ? 1 : 0;
+    a.finish = a.step_end == a.k_tiles ? 1 : 0;
     hipLaunchKernelGGL(gemm_digits_kernel, dim3((unsigned)(a.blocks_m * a.blocks_n)), dim3(kThreads), kSmemBytes, stream,
                        a);
     NBLA_HIP_LAUNCH_CHECK("gemm_digits");

@@ -24,7 +24,9 @@
 // and q into three balanced base-256 digits q = d0 * 65536 + d1 * 256 + d2, each an int8:
 //     X'[row_block = m / 32][k_tile = k / 32][digit 0..2][lane][16 x int8]
 // followed, per chunk of kChunkK columns, by the row sums of q (one int64 array of row_blocks * 32 entries per
-// chunk), and by the shifts s_m (one int32 array; kBadRow marks a row holding a non-finite value).  Rows >= M and columns >= K are zero.  The number of k tiles is padded to a multiple of 8.
+// chunk), by the shifts s_m (one int32 array; kBadRow marks a row holding a non-finite value) and by a 256-byte tail
+// whose first word is the mode flag of column-scaled operands (0: every row is held in its lowest digit alone).
+// Rows >= M and columns >= K are zero.  The number of k tiles is padded to a multiple of 8.
 //
 // B ("packed bits"): one bit per weight, set = negative (-1), clear = +1, in groups of 256 columns (eight column
 // fragments F = 0..7 of 32 columns):
@@ -80,7 +82,7 @@ __host__ __device__ inline int64_t digit_chunks(int64_t K) { return ceil_div(K, 
 // byte offsets of the sections of a digit operand
 struct DigitOperand {
   int64_t row_blocks, k_tiles, rows, chunks;
-  size_t sum_off, shift_off, total;
+  size_t sum_off, shift_off, flag_off, total;
 };
 __host__ __device__ inline DigitOperand digit_operand(int64_t M, int64_t K) {
   DigitOperand d;
@@ -90,7 +92,8 @@ __host__ __device__ inline DigitOperand digit_operand(int64_t M, int64_t K) {
   d.chunks = digit_chunks(K);
   d.sum_off = (size_t)d.row_blocks * d.k_tiles * kDigits * kFragBytes;
   d.shift_off = d.sum_off + (size_t)d.chunks * d.rows * sizeof(int64_t);
-  d.total = d.shift_off + (size_t)d.rows * sizeof(int32_t);
+  d.flag_off = d.shift_off + (size_t)d.rows * sizeof(int32_t); // one word: see launch_split_digits_columns
+  d.total = d.flag_off + 256;
   return d;
 }
 

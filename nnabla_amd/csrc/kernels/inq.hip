@@ -74,18 +74,55 @@ InqWorkspace plan_inq(int64_t size, int selection) {
 
 // Step A (inq_affine.cpp:95-102) fused with the max|w| scan of step C (:153-158).
 __global__ __launch_bounds__(kBlk) void inq_restore_absmax(float *__restrict__ W, const float *__restrict__ old_W,
-                                                           const int *__restrict__ old_I, int64_t size,
+                                                           const int *__restrict__ old_I, int64_t size, int vec,
                                                            uint32_t *__restrict__ partial) {
+  typedef float f4_t __attribute__((ext_vector_type(4)));
+  typedef int i4_t __attribute__((ext_vector_type(4)));
   uint32_t mx = 0u; // bits of a non-negative float order like the float
-  for (int64_t i = (int64_t)blockIdx.x * kBlk + threadIdx.x; i < size; i += (int64_t)gridDim.x * kBlk) {
+  auto take = [&](float w) {
+    const uint32_t u = __float_as_uint(w) & 0x7fffffffu;
+    if (u <= 0x7f800000u && u > mx) // NaN never compares greater
+      mx = u;
+  };
+  const int64_t stride = (int64_t)gridDim.x * kBlk;
+  int64_t done = 0;
+  if (vec) { // 16-byte aligned arrays: four weights per lane and access, two accesses in flight
+    const int64_t n4 = size / 4;
+    for (int64_t i = (int64_t)blockIdx.x * kBlk + threadIdx.x; i < n4; i += 2 * stride) {
+      const int64_t j = i + stride;
+      const bool second = j < n4;
+      f4_t w0 = reinterpret_cast<const f4_t *>(W)[i], w1 = w0;
+      i4_t f0 = reinterpret_cast<const i4_t *>(old_I)[i], f1 = f0;
+      if (second) {
+        w1 = reinterpret_cast<const f4_t *>(W)[j];
+        f1 = reinterpret_cast<const i4_t *>(old_I)[j];
+      }
+      if (f0.x == 1 || f0.y == 1 || f0.z == 1 || f0.w == 1) {
+        const f4_t o = reinterpret_cast<const f4_t *>(old_W)[i];
+        w0.x = f0.x == 1 ? o.x : w0.x, w0.y = f0.y == 1 ? o.y : w0.y;
+        w0.z = f0.z == 1 ? o.z : w0.z, w0.w = f0.w == 1 ? o.w : w0.w;
+        reinterpret_cast<f4_t *>(W)[i] = w0;
+      }
+      take(w0.x), take(w0.y), take(w0.z), take(w0.w);
+      if (second) {
+        if (f1.x == 1 || f1.y == 1 || f1.z == 1 || f1.w == 1) {
+          const f4_t o = reinterpret_cast<const f4_t *>(old_W)[j];
+          w1.x = f1.x == 1 ? o.x : w1.x, w1.y = f1.y == 1 ? o.y : w1.y;
+          w1.z = f1.z == 1 ? o.z : w1.z, w1.w = f1.w == 1 ? o.w : w1.w;
+          reinterpret_cast<f4_t *>(W)[j] = w1;
+        }
+        take(w1.x), take(w1.y), take(w1.z), take(w1.w);
+      }
+    }
+    done = n4 * 4;
+  }
+  for (int64_t i = done + (int64_t)blockIdx.x * kBlk + threadIdx.x; i < size; i += stride) {
     float w = W[i];
     if (old_I[i] == 1) {
       w = old_W[i];
       W[i] = w;
     }
-    const uint32_t u = __float_as_uint(w) & 0x7fffffffu;
-    if (u <= 0x7f800000u && u > mx) // NaN never compares greater
-      mx = u;
+    take(w);
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) {
@@ -256,7 +293,8 @@ int update_weights(float *W, int *I, float *old_W, int *old_I, int64_t size, int
   if (nparts > (unsigned)kMaxPartials)
     nparts = kMaxPartials;
 
-  hipLaunchKernelGGL(inq_restore_absmax, dim3(nparts), dim3(kBlk), 0, stream, W, old_W, old_I, size, partial);
+  hipLaunchKernelGGL(inq_restore_absmax, dim3(nparts), dim3(kBlk), 0, stream, W, old_W, old_I, size,
+                     (aligned16(W) && aligned16(old_W) && aligned16(old_I)) ? 1 : 0, partial);
   NBLA_HIP_LAUNCH_CHECK("inq_restore_absmax");
 
   if (selection == 1) {
@@ -338,10 +376,13 @@ ProductWorkspace plan_product(int64_t wsize, int64_t M, int64_t K, int64_t N, in
   size_t off = 0;
   p.update_off = off;
   off += round_up(plan_inq(wsize, step == 2 ? 1 : (step == 3 ? 2 : 0)).total, 256);
+  // activations and weights as bf16 planes (convolution) or as digit operands (affine)
+  const size_t xa = nbla_hip_split_operand_bytes(M, K), xb = nbla_hip_digit_operand_bytes(M, K);
+  const size_t wa = nbla_hip_split_operand_bytes(N, K), wb = nbla_hip_digit_operand_bytes(N, K);
   p.split_off = off;
-  off += round_up(nbla_hip_split_operand_bytes(M, K), 256);
+  off += round_up(xa > xb ? xa : xb, 256);
   p.planes_off = off;
-  off += round_up(nbla_hip_split_operand_bytes(N, K), 256);
+  off += round_up(wa > wb ? wa : wb, 256);
   p.flag_off = off;
   off += 256;
   p.total = off;
@@ -394,14 +435,16 @@ int nbla_hip_inq_affine_f32(const float *x, float *W, int32_t *I, float *old_W, 
     if (rc)
       return rc;
   }
-  int *flag = reinterpret_cast<int *>(base + p.flag_off);
-  rc = nbla_hip_split_bf16x3_f32(x, K, base + p.split_off, M, K, stream_);
+  // The product runs on the int8 digit kernels: x as a row-scaled digit operand, W^T as a column-scaled one.  Once
+  // every weight is zero or a power of two (all fixed) and a column spans at most six binades, each weight is a small
+  // integer in one digit and three exact digit products give the result; otherwise six (weights still being learnt).
+  rc = nbla_hip_split_digits_f32(x, K, base + p.split_off, M, K, stream_);
   if (rc)
     return rc;
-  rc = launch_split_weights(W, base + p.planes_off, flag, K, N, false, stream);
+  rc = launch_split_digits_columns(W, N, base + p.planes_off, K, N, true, stream);
   if (rc)
     return rc;
-  return launch_gemm_planes(base + p.split_off, base + p.planes_off, flag, nullptr, bias, y, M, K, N, 1, N, 1, stream);
+  return launch_gemm_digits(base + p.split_off, base + p.planes_off, bias, y, M, K, N, 1, N, 1, stream);
 }
 
 size_t nbla_hip_inq_convolution_workspace_bytes(int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,

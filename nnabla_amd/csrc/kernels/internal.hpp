@@ -27,11 +27,15 @@ int launch_gemm_planes(const void *xsplit, const void *wplanes, const int *need_
                        const float *bias, float *y, int64_t M, int64_t K, int64_t N, int64_t inner,
                        int64_t outer_stride, int64_t n_stride, hipStream_t stream, bool accumulate = false);
 
-// Digit operand whose rows are the C columns of src [R, C] (row stride ld), contraction over src's rows.
-int launch_split_digits_columns(const float *src, int64_t ld, void *digits, int64_t R, int64_t C, hipStream_t stream);
-// y[m, n] (+)= sum_k A[m, k] * B[n, k], both factors real-valued digit operands (rows M x K and N x K).
-int launch_gemm_digits(const void *adigits, const void *bdigits, float *y, int64_t M, int64_t K, int64_t N,
-                       int64_t inner, int64_t outer_stride, int64_t n_stride, hipStream_t stream,
+// Digit operand whose rows are the C columns of src [R, C] (row stride ld), contraction over src's rows.  With
+// detect_narrow the operand comes out in its one-digit form when every element is zero or a power of two within six
+// binades of its column's largest (its flag word tells the product which form it got).
+int launch_split_digits_columns(const float *src, int64_t ld, void *digits, int64_t R, int64_t C, bool detect_narrow,
+                                hipStream_t stream);
+// y[m, n] (+)= sum_k A[m, k] * B[n, k] (+ bias[n]), both factors real-valued digit operands (rows M x K and N x K);
+// A is a row-scaled operand, B a row- or column-scaled one whose flag word selects the six- or three-product form.
+int launch_gemm_digits(const void *adigits, const void *bdigits, const float *bias, float *y, int64_t M, int64_t K,
+                       int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride, hipStream_t stream,
                        bool accumulate = false);
 
 // db[n] (+)= sum over m of dy[m, n]; `partial` holds ceil(M / 256) * N floats.

@@ -61,9 +61,9 @@ def test_size_queries():
     assert L.nbla_hip_split_operand_bytes(i64(1), i64(1)) == 32 * 32 * 6
     # int8 digit operand: 3 bytes per element (K padded to 256), then per row one int64 sum per 16384-column chunk
     # and one int32 shift
-    assert L.nbla_hip_digit_operand_bytes(i64(4096), i64(4096)) == 4096 * 4096 * 3 + 4096 * 12
-    assert L.nbla_hip_digit_operand_bytes(i64(1), i64(1)) == 32 * 256 * 3 + 32 * 12
-    assert L.nbla_hip_digit_operand_bytes(i64(32), i64(16385)) == 32 * 16640 * 3 + 32 * (2 * 8 + 4)
+    assert L.nbla_hip_digit_operand_bytes(i64(4096), i64(4096)) == 4096 * 4096 * 3 + 4096 * 12 + 256
+    assert L.nbla_hip_digit_operand_bytes(i64(1), i64(1)) == 32 * 256 * 3 + 32 * 12 + 256
+    assert L.nbla_hip_digit_operand_bytes(i64(32), i64(16385)) == 32 * 16640 * 3 + 32 * (2 * 8 + 4) + 256
     assert L.nbla_hip_binary_affine_workspace_bytes(i64(64), i64(256), i64(256)) % 256 == 0
 
 
