@@ -284,6 +284,17 @@ int nbla_hip_affine_f32(const float *x, const float *w, const float *bias,
                         float *y, int64_t M, int64_t K, int64_t N,
                         void *stream);
 
+/* The same product on the int8 digit kernels (x row-scaled, w column-scaled,
+ * three int8 digits each, six exact digit products per output; three when every
+ * weight is zero or a power of two within six binades of its column's largest):
+ * several times the fp32 MFMA rate at fp32-faithful accuracy (each operand is
+ * rounded to 24 bits relative to its row / column maximum). */
+size_t nbla_hip_affine_workspace_bytes(int64_t M, int64_t K, int64_t N);
+int nbla_hip_affine_digits_f32(const float *x, const float *w, const float *bias,
+                               float *y, int64_t M, int64_t K, int64_t N,
+                               void *workspace, size_t workspace_bytes,
+                               void *stream);
+
 /* ------------------------------------------------------ binary convolutions */
 
 /* Output spatial shape (i + 2p - (d(k-1)+1)) / s + 1 per dimension, as

@@ -362,7 +362,8 @@ template <typename T> void AffineHip<T>::forward_impl(const Variables &inputs, c
   const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
   const T *b = inputs.size() == 3 ? inputs[2]->get_data_pointer<T>(this->ctx_) : nullptr;
   T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
-  NBLA_HIP_CALL(nbla_hip_affine_f32(x, w, b, y, s.i_row, s.i_col, s.w_col, nullptr));
+  HipWorkspace ws(nbla_hip_affine_workspace_bytes(s.i_row, s.i_col, s.w_col), this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_affine_digits_f32(x, w, b, y, s.i_row, s.i_col, s.w_col, ws.pointer(), ws.bytes(), nullptr));
 }
 
 // inq_affine.cpp:218-232: Affine backward with the (quantized) weights

@@ -63,10 +63,12 @@ BackwardPlan plan_backward(int64_t M, int64_t K, int64_t N) {
   const size_t a2 = nbla_hip_split_operand_bytes(M, N), b2 = nbla_hip_split_operand_bytes(K, N);
   // ... and the digit operands of x^T and dy^T for dW share the same two regions
   const size_t a3 = nbla_hip_digit_operand_bytes(K, M), b3 = nbla_hip_digit_operand_bytes(N, M);
+  // ... and those of dy and W for the real-weight dx
+  const size_t a4 = nbla_hip_digit_operand_bytes(M, N), b4 = nbla_hip_digit_operand_bytes(K, N);
   p.a_planes_off = off;
-  off += round_up(max3(a1, a2, a3), 256);
+  off += round_up(max3(max3(a1, a2, a3), a4, 0), 256);
   p.b_planes_off = off;
-  off += round_up(max3(b1, b2, b3), 256);
+  off += round_up(max3(max3(b1, b2, b3), b4, 0), 256);
   p.flag_off = off;
   off += 256;
   p.sums_off = off;
@@ -91,19 +93,18 @@ int grad_weights(const float *x, const float *dy, float *dW, int64_t M, int64_t 
                             accumulate);
 }
 
-// dx[M, K] (+)= dy' . W^T with real-valued weights, dy' [M, N]
+// dx[M, K] (+)= dy' . W^T with real-valued weights, dy' [M, N], on the digit x digit product: both operands are
+// row-scaled (rows m of dy', rows k of W, contraction over n)
 int grad_input_planes(const float *dyp, const float *W, float *dx, int64_t M, int64_t K, int64_t N, bool accumulate,
                       char *base, const BackwardPlan &p, hipStream_t stream) {
-  int *flag = reinterpret_cast<int *>(base + p.flag_off);
-  int rc = nbla_hip_split_bf16x3_f32(dyp, N, base + p.a_planes_off, M, N, stream);
+  int rc = nbla_hip_split_digits_f32(dyp, N, base + p.a_planes_off, M, N, stream);
   if (rc)
     return rc;
-  // W stored [K, N] = [output column of dx][contraction]: the transposed weight layout
-  rc = launch_split_weights(W, base + p.b_planes_off, flag, N, K, true, stream);
+  rc = nbla_hip_split_digits_f32(W, N, base + p.b_planes_off, K, N, stream);
   if (rc)
     return rc;
-  return launch_gemm_planes(base + p.a_planes_off, base + p.b_planes_off, flag, nullptr, nullptr, dx, M, N, K, 1, K, 1,
-                            stream, accumulate);
+  return launch_gemm_digits(base + p.a_planes_off, base + p.b_planes_off, nullptr, dx, M, N, K, 1, K, 1, stream,
+                            accumulate);
 }
 
 int check_args(int64_t M, int64_t K, int64_t N, void *workspace, size_t workspace_bytes, const BackwardPlan &p) {
@@ -230,6 +231,34 @@ int nbla_hip_affine_backward_f32(const float *dy, const float *x, const float *W
   if (db)
     return launch_column_sums(dy, db, M, N, accum_b != 0, base + p.sums_off, stream);
   return NBLA_HIP_OK;
+}
+
+size_t nbla_hip_affine_workspace_bytes(int64_t M, int64_t K, int64_t N) {
+  if (M <= 0 || K <= 0 || N <= 0)
+    return 0;
+  return round_up(nbla_hip_digit_operand_bytes(M, K), 256) + round_up(nbla_hip_digit_operand_bytes(N, K), 256);
+}
+
+int nbla_hip_affine_digits_f32(const float *x, const float *W, const float *bias, float *y, int64_t M, int64_t K,
+                               int64_t N, void *workspace, size_t workspace_bytes, void *stream_) {
+  if (M <= 0 || K <= 0 || N <= 0)
+    return fail(NBLA_HIP_ERR_VALUE, "invalid affine shape (M=%lld, K=%lld, N=%lld).", (long long)M, (long long)K,
+                (long long)N);
+  if (workspace_bytes < nbla_hip_affine_workspace_bytes(M, K, N) || !aligned256(workspace))
+    return fail(NBLA_HIP_ERR_MEMORY, "affine workspace too small or misaligned.");
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  hipStream_t stream = as_stream(stream_);
+  char *xd = static_cast<char *>(workspace);
+  char *wd = xd + round_up(nbla_hip_digit_operand_bytes(M, K), 256);
+  rc = nbla_hip_split_digits_f32(x, K, xd, M, K, stream_);
+  if (rc)
+    return rc;
+  rc = launch_split_digits_columns(W, N, wd, K, N, true, stream);
+  if (rc)
+    return rc;
+  return launch_gemm_digits(xd, wd, bias, y, M, K, N, 1, N, 1, stream);
 }
 
 } // extern "C"

@@ -578,6 +578,8 @@ __global__ __launch_bounds__(kPrepBlock) void digit_row_scale(const float *__res
   const int64_t m = (int64_t)blockIdx.x * (kPrepBlock / 64) + (threadIdx.x >> 6);
   if (m >= rows)
     return;
+  if (m == 0 && lane == 0)
+    shift[rows] = 1; // the operand's flag word (behind the shifts): a row-scaled operand is never in the narrow form
   if (m >= M) {
     if (lane == 0)
       shift[m] = 0;

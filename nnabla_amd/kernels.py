@@ -29,6 +29,7 @@ EXPORTED = (
     "nbla_hip_split_digits_f32", "nbla_hip_gemm_bits_f32",
     "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_weight_affine_f32",
     "nbla_hip_binary_connect_affine_f32", "nbla_hip_affine_f32", "nbla_hip_split_digits_scaled_f32",
+    "nbla_hip_affine_workspace_bytes", "nbla_hip_affine_digits_f32",
     "nbla_hip_affine_backward_workspace_bytes", "nbla_hip_binary_affine_backward_f32", "nbla_hip_affine_backward_f32",
     "nbla_hip_convolution_output_shape", "nbla_hip_binary_convolution_workspace_bytes",
     "nbla_hip_binary_weight_convolution_f32", "nbla_hip_binary_connect_convolution_f32",
@@ -67,7 +68,7 @@ def lib():
                      "nbla_hip_min_max_quantize_backward_workspace_bytes",
                      "nbla_hip_affine_backward_workspace_bytes",
                      "nbla_hip_convolution_backward_workspace_bytes", "nbla_hip_prune_workspace_bytes",
-                     "nbla_hip_convolution_workspace_bytes",
+                     "nbla_hip_convolution_workspace_bytes", "nbla_hip_affine_workspace_bytes",
                      "nbla_hip_split_operand_bytes", "nbla_hip_digit_operand_bytes",
                      "nbla_hip_binarize_workspace_bytes",
                      "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_convolution_workspace_bytes",
@@ -302,6 +303,19 @@ def affine_backward(dy, x, W, dx=None, dW=None, db=None, want=(True, True, True)
     check(lib().nbla_hip_affine_backward_f32(_p(dy), _p(x), _p(W), _p(odx), _p(odw), _p(odb), _i64(M), _i64(K), _i64(N),
                                              ax, aw, ab, _p(ws), ctypes.c_size_t(ws.numel()), _stream(stream)))
     return odx, odw, odb
+
+
+def affine_digits(x, W, bias=None, out=None, workspace=None, stream=None):
+    """y = x.W + b on the int8 digit kernels."""
+    import torch
+    M, K = x.shape
+    N = W.numel() // K
+    y = torch.empty((M, N), dtype=torch.float32, device=x.device) if out is None else out
+    ws = workspace if workspace is not None else _workspace(
+        lib().nbla_hip_affine_workspace_bytes(_i64(M), _i64(K), _i64(N)), x)
+    check(lib().nbla_hip_affine_digits_f32(_p(x), _p(W), _p(bias), _p(y), _i64(M), _i64(K), _i64(N), _p(ws),
+                                           ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return y
 
 
 def affine(x, W, bias=None, out=None, stream=None):

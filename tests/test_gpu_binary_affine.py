@@ -199,6 +199,36 @@ def test_plain_affine_f32(dev):
         y64 = x.astype(np.float64) @ W.astype(np.float64) + b
         assert max_rel_err(y, y64) <= TIGHT
         assert max_rel_err(oracle.affine(x, W, b), y64) <= TIGHT
+        # the same product on the int8 digit kernels (what the Affine function class runs)
+        yd = to_np(kernels.affine_digits(_dev(x, dev), _dev(W, dev), _dev(b, dev)))
+        assert max_rel_err(yd, y64) <= TIGHT
+
+
+def test_affine_digits_special_rows_and_narrow_weights(dev):
+    """Rows of x or columns of W holding NaN / Inf give NaN outputs for that row / column only; weights that are all
+    zero or powers of two within six binades per column take the three-product form and are multiplied exactly."""
+    rng = np.random.RandomState(8)
+    x = rng.randn(70, 200).astype(np.float32)
+    W = (rng.randn(200, 90) * 0.1).astype(np.float32)
+    x[3, 5] = np.inf
+    W[7, 11] = np.nan
+    y = to_np(kernels.affine_digits(_dev(x, dev), _dev(W, dev)))
+    assert np.isnan(y[3]).all() and np.isnan(y[:, 11]).all()
+    ok = np.ones_like(y, bool)
+    ok[3], ok[:, 11] = False, False
+    xf, Wf = x.copy(), W.copy()
+    xf[3, 5], Wf[7, 11] = 0, 0
+    ref = xf.astype(np.float64) @ Wf.astype(np.float64)
+    assert np.isfinite(y[ok]).all() and np.abs(y - ref)[ok].max() / np.abs(ref[ok]).max() <= TIGHT
+    # powers of two: exponents within 6 of the column's largest, some zeros, both signs
+    e = rng.randint(-9, -3, size=(200, 90))
+    Wp = (np.where(rng.rand(200, 90) < 0.2, 0.0, 2.0 ** e) * rng.choice([-1.0, 1.0], size=(200, 90))).astype(np.float32)
+    xi = np.rint(rng.randn(70, 200) * 64).astype(np.float32) / 64          # exactly representable rows
+    yp = to_np(kernels.affine_digits(_dev(xi, dev), _dev(Wp, dev)))
+    assert np.array_equal(yp, (xi.astype(np.float64) @ Wp.astype(np.float64)).astype(np.float32))
+    Wp[0, 0] = 2.0 ** -20                                                  # one column now spans too many binades
+    yw = to_np(kernels.affine_digits(_dev(xi, dev), _dev(Wp, dev)))
+    assert max_rel_err(yw, xi.astype(np.float64) @ Wp.astype(np.float64)) <= TIGHT
 
 
 @pytest.mark.parametrize("M", [1, 8, 64])
