@@ -218,8 +218,9 @@ def cpu_baseline(K, N, rows):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=30,
+                    help="untimed steps; the first few dozen launches after idle run at ramping clocks")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=2048)
     ap.add_argument("--section", choices=("all", "headline", "quantizers"), default="all",
@@ -259,7 +260,7 @@ def main():
                      "frac": 3 * gemm_tflops / PEAK_INT8_MFMA_TOPS, "traffic": GEMM_TRAFFIC_BYTES_PROFILED,
                      "traffic_note": "bytes per launch between L2 and the memory side, profiled (not live); "
                                      "algorithmic: 56.2 MB read + 180.4 MB written",
-                     "kernel": "gemm_bits_kernel<32,512,1,4,false>", "kernel_ms": r["gemm_ms"],
+                     "kernel": "gemm_bits_kernel<32,512,1,4,1,false>", "kernel_ms": r["gemm_ms"],
                      "note": "int8 operations issued (3 digit planes x 2*M*K*N) against the int8 MFMA peak",
                      "fp32_equiv_TFLOPs": gemm_tflops, "fp32_equiv_over_fp32_mfma_peak": gemm_tflops / PEAK_FP32_MFMA_TFLOPS},
         "step_breakdown_ms": {"prepare": r["prepare_ms"], "split": r["split_ms"], "gemm": r["gemm_ms"]},

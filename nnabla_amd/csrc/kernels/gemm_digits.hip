@@ -65,7 +65,7 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave & 1, wn = wave >> 1;
   int64_t bm, bn;
-  band_tile<4>(blockIdx.x, a.blocks_m, a.blocks_n, bm, bn);
+  band_tile<8>(blockIdx.x, a.blocks_m, a.blocks_n, bm, bn); // two blocks per CU: 64 resident tiles per XCD = 8 x 8
 
   // this wavefront's copies: chunk c = p * kWaves + wave of the stage; chunks [0, 12) are A fragments (row block,
   // digit), [12, 24) B fragments
