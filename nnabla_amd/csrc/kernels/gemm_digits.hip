@@ -36,10 +36,12 @@ constexpr int kSegs = 4;               // 32-row fragments per tile side
 constexpr int kSegVec = kDigits * 64;  // uint4 per fragment and k step
 constexpr int kSideVec = kSegs * kSegVec;
 constexpr int kStageBytes = 2 * kSideVec * 16; // 24 KiB: the A and B fragments of one k tile
-constexpr int kStages = 3;
 constexpr int kChunks = 2 * kSegs * kDigits;   // 1 KiB copies per k tile
 constexpr int kPerWave = kChunks / kWaves;     // 6
-constexpr int kSmemBytes = kStages * kStageBytes;
+// Three LDS stages when two blocks share a CU; six (the whole LDS) when the output has so few tiles that a CU holds
+// one block anyway: with one wavefront per SIMD a k tile is multiplied in a few hundred cycles and the copies need
+// the longer head start to cover the memory latency.
+constexpr int kStagesShared = 3, kStagesAlone = 6;
 
 // Workgroup barrier without the memory fence of __syncthreads() (which would wait for every global -> LDS copy in
 // flight, including those of later k tiles); the waits that matter are explicit.
@@ -52,13 +54,13 @@ constexpr int kSmemBytes = kStages * kStageBytes;
 // vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
 #define NBLA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xf) | (((n) >> 4) << 14) | (0x7 << 4) | (0xf << 8))
 
-// Staging: global -> LDS copies bypass the registers (one wavefront instruction moves one 1 KiB fragment); three
-// LDS buffers hold consecutive k tiles and the copy of tile t + 2 is issued while tile t is multiplied.  Two blocks
+// Staging: global -> LDS copies bypass the registers (one wavefront instruction moves one 1 KiB fragment); kStages
+// LDS buffers hold consecutive k tiles and the copy of tile t + kStages - 1 is issued while tile t is multiplied.  Two blocks
 // share a CU (256 registers per lane: 192 accumulators + the 12 operand quads of a tile), so one block's LDS reads
 // and barrier waits are covered by the other's MFMAs.
 // kNarrow: the B operand holds every value in its lowest digit alone (a small integer): three products
 // a_t x b2 -> accumulator t, nothing dropped, and only the lowest-digit fragments of B are copied.
-template <bool kNarrow>
+template <bool kNarrow, int kStages>
 __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsigned char *smem) {
 #if defined(__HIP_DEVICE_COMPILE__) // the host pass only needs the launch stub; the body uses LDS address-space pointers
   const int tid = threadIdx.x, lane = tid & 63;
@@ -110,13 +112,15 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
         for (int r = 0; r < 16; ++r)
           acc[i][j][t][r] = 0;
 
-  copy_next(0);
-  copy_next(1);
+  static_assert((kStages - 2) * kPerWave < 64, "vmcnt is a 6-bit counter");
+#pragma unroll
+  for (int d = 0; d < kStages - 1; ++d)
+    copy_next(d);
   int buf = 0;
   for (int64_t kt = a.step_begin; kt < a.step_end; ++kt) {
-    // tile kt has landed (the copies of tile kt + 1 may still be in flight) and every wavefront is done with the
-    // buffer tile kt - 1 occupied, which tile kt + 2 takes over
-    NBLA_WAIT_VMCNT(kCopies);
+    // tile kt has landed (the copies of the kStages - 2 tiles after it may still be in flight) and every wavefront
+    // is done with the buffer tile kt - 1 occupied, which tile kt + kStages - 1 takes over
+    NBLA_WAIT_VMCNT((kStages - 2) * kCopies);
     NBLA_BARRIER();
     copy_next(buf == 0 ? kStages - 1 : buf - 1);
     const uint4_t *sa = reinterpret_cast<const uint4_t *>(smem + buf * kStageBytes);
@@ -155,53 +159,71 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
   }
   NBLA_WAIT_VMCNT(0);
 
-  // y = (acc0 * 2^16 + acc1 * 2^8 + acc2) * 2^(16 - sa - sb); the narrow form has no factor 2^16 (b is its low digit)
+  // y = (acc0 * 2^16 + acc1 * 2^8 + acc2) * 2^(16 - sa - sb); the narrow form has no factor 2^16 (b is its low digit).
+  // Row by row: the row's offset (one 32-bit division when m is folded into two output indices) and shift are
+  // formed once and serve both column fragments.
   const int col_in_frag = lane & 31, row_half = lane >> 5;
   const int32_t *bshift = kNarrow ? a.bshift_narrow : a.bshift;
+  int64_t n_col[2];
+  int32_t sb_n[2];
+  float bias_n[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    const int64_t n = bn * kBN + (wn * 2 + j) * 32 + col_in_frag;
-    if (n >= a.N)
-      continue;
-    const int32_t sb_n = bshift[n];
-    const float bias = (a.bias && a.finish) ? a.bias[n] : 0.0f;
+    n_col[j] = bn * kBN + (wn * 2 + j) * 32 + col_in_frag;
+    const bool in = n_col[j] < a.N;
+    sb_n[j] = in ? bshift[n_col[j]] : 0;
+    bias_n[j] = (in && a.bias && a.finish) ? a.bias[n_col[j]] : 0.0f;
+  }
+  const bool add_bias = a.bias && a.finish;
+  const uint32_t inner = (uint32_t)a.inner;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int64_t m0 = bm * kBM + (wm * 2 + i) * 32;
+  for (int i = 0; i < 2; ++i) {
+    const int64_t m0 = bm * kBM + (wm * 2 + i) * 32;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int64_t m = m0 + 8 * (r >> 2) + 4 * row_half + (r & 3);
-        if (m < a.M) {
-          const int32_t sa_m = a.ashift[m];
-          float v;
-          if (sa_m == kBadRow || sb_n == kBadRow) {
-            v = __uint_as_float(0x7fc00000u);
-          } else {
-            const long long t = ((long long)acc[i][j][0][r] << 16) + ((long long)acc[i][j][1][r] << 8) +
-                                (long long)acc[i][j][2][r];
-            // the two shifts are applied one after the other: each stays inside ldexpf's exponent range
-            v = ldexpf(ldexpf((float)t, (kNarrow ? 0 : 16) - sa_m), -sb_n);
-          }
-          const int64_t off = (a.inner == 1) ? m * a.outer_stride : (m / a.inner) * a.outer_stride + (m % a.inner);
-          float *dst = a.y + off + n * a.n_stride;
-          if (a.accumulate)
-            v = *dst + v;
-          if (a.bias && a.finish)
-            v = v + bias;
-          *dst = v;
+    for (int r = 0; r < 16; ++r) {
+      const int64_t m = m0 + 8 * (r >> 2) + 4 * row_half + (r & 3);
+      if (m >= a.M)
+        continue;
+      const int32_t sa_m = a.ashift[m];
+      int64_t off;
+      if (inner == 1u) {
+        off = m * a.outer_stride;
+      } else {
+        const uint32_t mu = (uint32_t)m, q = mu / inner; // m < 2^31: operand rows are counted in 32 bits
+        off = (int64_t)q * a.outer_stride + (mu - q * inner);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (n_col[j] >= a.N)
+          continue;
+        float v;
+        if (sa_m == kBadRow || sb_n[j] == kBadRow) {
+          v = __uint_as_float(0x7fc00000u);
+        } else {
+          const long long t = ((long long)acc[i][j][0][r] << 16) + ((long long)acc[i][j][1][r] << 8) +
+                              (long long)acc[i][j][2][r];
+          // the two shifts are applied one after the other: each stays inside ldexpf's exponent range
+          v = ldexpf(ldexpf((float)t, (kNarrow ? 0 : 16) - sa_m), -sb_n[j]);
         }
+        float *dst = a.y + off + n_col[j] * a.n_stride;
+        if (a.accumulate)
+          v = *dst + v;
+        if (add_bias)
+          v = v + bias_n[j];
+        *dst = v;
       }
     }
   }
 #endif
 }
 
+template <int kStages>
 __global__ __launch_bounds__(kThreads, 2) void gemm_digits_kernel(GemmDigitsArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   if (*a.bflag == 0) // uniform over the grid
-    gemm_digits_tile<true>(a, smem);
+    gemm_digits_tile<true, kStages>(a, smem);
   else
-    gemm_digits_tile<false>(a, smem);
+    gemm_digits_tile<false, kStages>(a, smem);
 }
 
 } // namespace
@@ -209,11 +231,16 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_digits_kernel(GemmDigitsArgs
 int launch_gemm_digits(const void *adigits, const void *bdigits, const float *bias, float *y, int64_t M, int64_t K,
                        int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride, hipStream_t stream,
                        bool accumulate) {
+  if (M >= ((int64_t)1 << 31) || N >= ((int64_t)1 << 31))
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "digit product: more than 2^31 - 1 rows or columns.");
   const DigitOperand da = digit_operand(M, K), db = digit_operand(N, K);
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_digits_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_digits_kernel<kStagesShared>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kStagesShared * kStageBytes);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_digits_kernel<kStagesAlone>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kStagesAlone * kStageBytes);
     if (e != hipSuccess)
       return fail_hip(e, "hipFuncSetAttribute(gemm_digits LDS size)");
     configured = true;
@@ -244,8 +271,13 @@ int launch_gemm_digits(const void *adigits, const void *bdigits, const float *bi
     a.step_end = (t0 + tiles_per_chunk < a.k_tiles) ? t0 + tiles_per_chunk : a.k_tiles;
     a.accumulate = (accumulate || chunk > 0) ? 1 : 0;
     a.finish = a.step_end == a.k_tiles ? 1 : 0;
-    hipLaunchKernelGGL(gemm_digits_kernel, dim3((unsigned)(a.blocks_m * a.blocks_n)), dim3(kThreads), kSmemBytes, stream,
-                       a);
+    const unsigned blocks = (unsigned)(a.blocks_m * a.blocks_n);
+    if (blocks <= 384) // fewer than 1.5 blocks per CU
+      hipLaunchKernelGGL(gemm_digits_kernel<kStagesAlone>, dim3(blocks), dim3(kThreads), kStagesAlone * kStageBytes,
+                         stream, a);
+    else
+      hipLaunchKernelGGL(gemm_digits_kernel<kStagesShared>, dim3(blocks), dim3(kThreads), kStagesShared * kStageBytes,
+                         stream, a);
     NBLA_HIP_LAUNCH_CHECK("gemm_digits");
   }
   return NBLA_HIP_OK;
