@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
   constexpr int kStageBytes = kStepBytes * kWavesK;
   constexpr int kStages = gemm_bits_stages(BM, BN, kWavesMN, kWavesK);
   constexpr int kDepth = kStages - 1; // k steps in flight ahead of the one being multiplied
-  static_assert(kDepth >= 1 && (kDepth - 1) * (kPerWave + 1) < 64, "vmcnt is a 6-bit counter");
+  static_assert(kDepth >= 2 && (kDepth - 1) * (kPerWave + 1) < 64, "vmcnt is a 6-bit counter");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
@@ -279,7 +279,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
   if (idle) {
     for (int64_t ks = first; ks <= last; ks += kWavesK) {
       const int buf_copy = (buf == 0) ? kStages - 1 : buf - 1;
-      wait_copies(std::integral_constant<int, kDepth - 1>());
+      wait_copies(std::integral_constant<int, kDepth - 2>());
       NBLA_BARRIER();
       copy_next(buf_copy);
       buf = (buf + 1 == kStages) ? 0 : buf + 1;
@@ -296,9 +296,9 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
       __builtin_amdgcn_sched_barrier(0);
       mma(af0, w0, J1(), JN());
       __builtin_amdgcn_sched_barrier(0);
-      // step ks+1 has landed (the copies of later steps may still be in flight); every wavefront is done with the
-      // buffer of step ks-1
-      wait_copies(std::integral_constant<int, kDepth - 1>());
+      // step ks+1 has landed: the copies issued so far reach step ks+kDepth-1, so at most the kDepth-2 steps behind
+      // ks+1 may still be in flight; every wavefront is done with the buffer of step ks-1
+      wait_copies(std::integral_constant<int, kDepth - 2>());
       NBLA_BARRIER();
       // tile 1 runs; the copy of step ks+kDepth is issued; tile 0 of step ks+1 is fetched
       mma(af1, w1, J0(), J1());

@@ -4,8 +4,8 @@
 //     qa * qb = a0 b0 * 2^32 + (a0 b1 + a1 b0) * 2^24 + (a0 b2 + a1 b1 + a2 b0) * 2^16 + (lower terms)
 // and the six leading digit products are accumulated exactly in three int32 accumulators per output (one per power
 // of 256); the dropped terms are below 2^-23 of |row max| * |column max| per k.  The epilogue combines the three
-// sums in 64-bit integers, converts once and applies the two scales, so the result does not depend on the order of
-// summation.  Used for the weight gradients (x^T . dy), where neither factor is a sign matrix.
+// sums in integer arithmetic, converts once and applies the two scales, so the result does not depend on the order
+// of summation.  Used for the weight gradients (x^T . dy), where neither factor is a sign matrix.
 //
 // Tiling: 128 x 128 outputs per block of four wavefronts (2 x 2, 64 x 64 each: 2 x 2 fragments x 3 accumulators =
 // 192 registers), k in tiles of 32 (one v_mfma_i32_32x32x32_i8 fragment).
@@ -176,15 +176,25 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
   }
   const bool add_bias = a.bias && a.finish;
   const uint32_t inner = (uint32_t)a.inner;
+  // the 32 row shifts of each row fragment: one coalesced load up front (lane l holds row l % 32), handed out by
+  // shuffles, instead of a dependent global load per row inside the store loop
+  int32_t row_shift[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    int64_t m = bm * kBM + (wm * 2 + i) * 32 + (lane & 31);
+    const int64_t last = a.a_row_blocks * kFragRows - 1;
+    row_shift[i] = a.ashift[m < last ? m : last];
+  }
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int64_t m0 = bm * kBM + (wm * 2 + i) * 32;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int64_t m = m0 + 8 * (r >> 2) + 4 * row_half + (r & 3);
+      const int row = 8 * (r >> 2) + 4 * row_half + (r & 3);
+      const int32_t sa_m = __shfl(row_shift[i], row);
+      const int64_t m = m0 + row;
       if (m >= a.M)
         continue;
-      const int32_t sa_m = a.ashift[m];
       int64_t off;
       if (inner == 1u) {
         off = m * a.outer_stride;
@@ -200,10 +210,14 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
         if (sa_m == kBadRow || sb_n[j] == kBadRow) {
           v = __uint_as_float(0x7fc00000u);
         } else {
-          const long long t = ((long long)acc[i][j][0][r] << 16) + ((long long)acc[i][j][1][r] << 8) +
-                              (long long)acc[i][j][2][r];
+          // t = acc0 * 2^16 + acc1 * 2^8 + acc2 regrouped as hi * 2^16 + lo with 0 <= lo < 2^17 and |hi| < 2^30 (32-bit
+          // integer steps only), then one fused multiply-add: exact while |hi| < 2^24, else rounded twice (2^-24 of t)
+          const int a0 = acc[i][j][0][r], a1 = acc[i][j][1][r], a2 = acc[i][j][2][r];
+          const int hi = a0 + (a1 >> 8) + (a2 >> 16);
+          const int lo = ((a1 & 0xff) << 8) + (a2 & 0xffff);
+          const float t = fmaf((float)hi, 65536.0f, (float)lo);
           // the two shifts are applied one after the other: each stays inside ldexpf's exponent range
-          v = ldexpf(ldexpf((float)t, (kNarrow ? 0 : 16) - sa_m), -sb_n[j]);
+          v = ldexpf(ldexpf(t, (kNarrow ? 0 : 16) - sa_m), -sb_n[j]);
         }
         float *dst = a.y + off + n_col[j] * a.n_stride;
         if (a.accumulate)
