@@ -81,6 +81,28 @@ def test_inq_largest_abs_tie_free_half_selection(dev):
         assert Ic.sum() == max(size // 2, 1)
 
 
+@pytest.mark.parametrize("num_bits,top", [(4, 1.9), (6, 1.4)])
+def test_inq_every_weight_of_the_level_range(dev, num_bits, top):
+    """Every fp32 value from below the pruning threshold up to max|w| (whole binades, both signs), all fixed:
+    the quantized weights follow the host libm's log2f cut for cut (inq_affine.cpp:153-190)."""
+    lo_exp, hi_exp = (-6, 0) if num_bits == 4 else (-18, 0)
+    for e in range(lo_exp, hi_exp + 1):
+        u = np.arange(1 << 23, dtype=np.uint32) | np.uint32((e + 127) << 23)
+        w = u.view(np.float32).copy()
+        w[1::2] *= -1
+        w[0] = np.float32(top)  # the same max|w| (hence n1, n2) for every binade
+        w = w[np.abs(w) <= np.float32(top)]
+        inq = oracle.Inq(w.size, num_bits, (0,), "largest_abs")
+        Wc, Ic = w.copy(), np.zeros(w.size, np.int32)
+        n1, n2 = inq.quantize_weights(Wc, Ic)
+        Wd, Id = _dev(w, dev), torch.zeros(w.size, dtype=torch.int32, device=dev)
+        n1n2 = kernels.inq_update_weights(Wd, Id, torch.zeros_like(Wd), torch.zeros_like(Id), num_bits,
+                                          kernels.INQ_FIX_ALL)
+        assert tuple(to_np(n1n2)) == (n1, n2)
+        assert bits_equal(to_np(Wd), Wc), "binade 2^%d: %s" % (e, first_mismatch(to_np(Wd), Wc))
+        assert int(to_np(Id).min()) == 1
+
+
 @pytest.mark.parametrize("M,K,N", [(2, 3, 4), (33, 100, 130), (64, 256, 192), (300, 520, 257)])
 def test_inq_affine_all_fixed_and_partially_fixed(dev, M, K, N):
     rng = np.random.RandomState(5)

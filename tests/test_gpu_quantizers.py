@@ -55,6 +55,31 @@ def test_fixed_point_quantize_config1_full_size(dev):
     assert np.all(np.abs(y) <= 7.9375) and np.all(y * 16 == np.round(y * 16))
 
 
+@pytest.mark.parametrize("sign,n,delta", [(True, 8, 2.0 ** -4), (False, 6, 0.1)])
+def test_fixed_point_quantize_every_fp32_value(dev, sign, n, delta):
+    """All 2^32 bit patterns except NaNs against fixed_point_quantize.cpp:52-65 restated with torch operations:
+    fp32 compare and divide, the +0.5 and the truncation in float64 (exact), one fp32 multiply, negation for x < 0."""
+    nn = n - 1 if sign else n
+    d32 = np.float32(delta)
+    mx = np.float32((2.0 ** nn - 1) * float(d32))
+    mn = np.float32(-mx if sign else 0.0)
+    dd = torch.tensor(float(d32), dtype=torch.float32, device=dev)  # a device operand: a true fp32 divide
+    chunk = 1 << 27
+    for start in range(0, 1 << 32, chunk):
+        lo = start - (1 << 32) if start >= (1 << 31) else start  # the same bit patterns as signed 32-bit integers
+        x = torch.arange(lo, lo + chunk, dtype=torch.int32, device=dev).view(torch.float32)
+        y = kernels.fixed_point_quantize(x, sign, n, delta)
+        q = (x.abs() / dd).double()
+        k = torch.trunc(q + 0.5).float() * dd
+        ref = torch.where(x < 0, -k, k)
+        ref = torch.where(x > float(mx), torch.full_like(ref, float(mx)), ref)
+        ref = torch.where(x < float(mn), torch.full_like(ref, float(mn)), ref)
+        ok = (y.view(torch.int32) == ref.view(torch.int32)) | torch.isnan(x)
+        if not bool(ok.all()):
+            i = int((~ok).nonzero()[0])
+            raise AssertionError("x=%r (bits %#x): got %r want %r" % (float(x[i]), start + i, float(y[i]), float(ref[i])))
+
+
 @pytest.mark.parametrize("size", [0, 1, 3, 4, 5, 1023, 1024, 1025, 4099])
 def test_fixed_point_quantize_ragged_and_unaligned(dev, size):
     rng = np.random.RandomState(size + 1)
