@@ -720,6 +720,95 @@ __global__ __launch_bounds__(kPrepBlock) void split_digits_tiled(const float *__
   }
 }
 
+// Scale and digits in one pass for rows of up to 4096 values (K % 4 == 0, 16-byte aligned rows): a block of eight
+// wavefronts keeps 16 rows in registers in fragment order.  Wavefront w owns the k tiles [w * kTiles, (w + 1) * kTiles);
+// lane r + 16 * q holds, for row r, the 16 values of fragment half g = q & 1 of the tiles 2 * t + (q >> 1).  Row maxima
+// and row sums cross the wavefronts through LDS; every store instruction then writes four 256-byte runs of one
+// fragment (the other 16 rows of the row block come from the neighbouring block).  x is read once.
+constexpr int kFusedWaves = 8, kFusedRows = 16;
+template <int kTiles>
+__global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const float *__restrict__ x, int64_t ldx,
+                                                                       const float *__restrict__ cs,
+                                                                       long long *__restrict__ sums,
+                                                                       int32_t *__restrict__ shift,
+                                                                       uint4_t *__restrict__ out, int64_t M, int64_t K,
+                                                                       int64_t k_tiles, int64_t rows) {
+  static_assert(kTiles % 2 == 0, "a lane walks its wavefront's tiles in pairs");
+  constexpr int kPairs = kTiles / 2;
+  __shared__ uint32_t s_max[kFusedWaves][kFusedRows];
+  __shared__ long long s_sum[kFusedWaves][kFusedRows];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = lane & 15, g = (lane >> 4) & 1, th = lane >> 5;
+  const int64_t m = (int64_t)blockIdx.x * kFusedRows + r;
+  if (blockIdx.x == 0 && threadIdx.x == 0)
+    shift[rows] = 1; // the operand's flag word: a row-scaled operand is never in the narrow form
+  const float *row = x + m * ldx;
+  float4_t v[kPairs][4];
+  uint32_t amax = 0u;
+#pragma unroll
+  for (int t = 0; t < kPairs; ++t) {
+    const int64_t k0 = ((int64_t)wave * kTiles + 2 * t + th) * kTileK + g * 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t k = k0 + 4 * i;
+      v[t][i] = (m < M && k < K) ? scaled4(*reinterpret_cast<const float4_t *>(row + k), cs, k)
+                                 : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < kPairs; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t a = __float_as_uint(v[t][i].x) & 0x7fffffffu, b = __float_as_uint(v[t][i].y) & 0x7fffffffu;
+      const uint32_t c = __float_as_uint(v[t][i].z) & 0x7fffffffu, d = __float_as_uint(v[t][i].w) & 0x7fffffffu;
+      amax = max(max(amax, max(a, b)), max(c, d));
+    }
+  amax = max(amax, (uint32_t)__shfl_xor((int)amax, 16));
+  amax = max(amax, (uint32_t)__shfl_xor((int)amax, 32));
+  if (lane < kFusedRows)
+    s_max[wave][lane] = amax;
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < kFusedWaves; ++w)
+    amax = max(amax, s_max[w][r]);
+  const bool bad = amax >= 0x7f800000u;
+  const int s = (bad || amax == 0u) ? 0 : digit_shift(amax);
+  int part = 0; // at most 128 values of magnitude < 2^23 per lane
+#pragma unroll
+  for (int t = 0; t < kPairs; ++t) {
+    int q[16];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      q[4 * i + 0] = bad ? 0 : to_fixed(v[t][i].x, s);
+      q[4 * i + 1] = bad ? 0 : to_fixed(v[t][i].y, s);
+      q[4 * i + 2] = bad ? 0 : to_fixed(v[t][i].z, s);
+      q[4 * i + 3] = bad ? 0 : to_fixed(v[t][i].w, s);
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      part += q[j];
+    const int64_t kt = (int64_t)wave * kTiles + 2 * t + th;
+    if (kt < k_tiles) {
+      const int64_t rb = m / kFragRows;
+      store_digits(q, out + ((rb * k_tiles + kt) * kDigits) * 64 + (int)(m % kFragRows) + 32 * g, true);
+    }
+  }
+  long long acc = part;
+  acc += __shfl_xor(acc, 16);
+  acc += __shfl_xor(acc, 32);
+  if (lane < kFusedRows)
+    s_sum[wave][lane] = acc;
+  __syncthreads();
+  if (threadIdx.x < kFusedRows) {
+    long long total = 0;
+#pragma unroll
+    for (int w = 0; w < kFusedWaves; ++w)
+      total += s_sum[w][threadIdx.x];
+    sums[m] = total; // a single chunk: K <= 4096 < kChunkK
+    shift[m] = bad ? kBadRow : s;
+  }
+}
+
 // ---- digit operand of a transposed source: the operand's rows are the columns c of src [R, C] (row stride ld) and
 // its contraction index runs over src's rows, so x^T, dy^T or W^T feed the digit x digit product without a
 // transposed copy.  One scale per column: column maxima by integer atomicMax on the magnitude bits
@@ -1026,6 +1115,24 @@ int nbla_hip_split_digits_scaled_f32(const float *x, int64_t ldx, const float *c
   long long *sums = reinterpret_cast<long long *>(base + d.sum_off);
   int32_t *shift = reinterpret_cast<int32_t *>(base + d.shift_off);
   const bool vec = K % 4 == 0 && ldx % 4 == 0 && aligned16(x) && aligned16(cs);
+  if (vec && d.k_tiles <= kFusedWaves * 16) { // rows of up to 4096 values: one pass, rows held in registers
+    const dim3 grid((unsigned)(d.rows / kFusedRows)), block(kFusedWaves * 64);
+    uint4_t *out = static_cast<uint4_t *>(xdigits);
+    if (d.k_tiles <= kFusedWaves * 2)
+      hipLaunchKernelGGL(split_digits_rows<2>, grid, block, 0, stream, x, ldx, cs, sums, shift, out, M, K, d.k_tiles,
+                         d.rows);
+    else if (d.k_tiles <= kFusedWaves * 4)
+      hipLaunchKernelGGL(split_digits_rows<4>, grid, block, 0, stream, x, ldx, cs, sums, shift, out, M, K, d.k_tiles,
+                         d.rows);
+    else if (d.k_tiles <= kFusedWaves * 8)
+      hipLaunchKernelGGL(split_digits_rows<8>, grid, block, 0, stream, x, ldx, cs, sums, shift, out, M, K, d.k_tiles,
+                         d.rows);
+    else
+      hipLaunchKernelGGL(split_digits_rows<16>, grid, block, 0, stream, x, ldx, cs, sums, shift, out, M, K, d.k_tiles,
+                         d.rows);
+    NBLA_HIP_LAUNCH_CHECK("split_digits_rows");
+    return NBLA_HIP_OK;
+  }
   const dim3 scale_grid((unsigned)ceil_div(d.rows, kPrepBlock / 64));
   if (vec)
     hipLaunchKernelGGL(digit_row_scale<true>, scale_grid, dim3(kPrepBlock), 0, stream, x, ldx, cs, sums, shift, M, K,
