@@ -720,34 +720,36 @@ __global__ __launch_bounds__(kPrepBlock) void split_digits_tiled(const float *__
   }
 }
 
-// Scale and digits in one pass for rows of up to 4096 values (K % 4 == 0, 16-byte aligned rows): a block of eight
-// wavefronts keeps 16 rows in registers in fragment order.  Wavefront w owns the k tiles [w * kTiles, (w + 1) * kTiles);
-// lane r + 16 * q holds, for row r, the 16 values of fragment half g = q & 1 of the tiles 2 * t + (q >> 1).  Row maxima
-// and row sums cross the wavefronts through LDS; every store instruction then writes four 256-byte runs of one
-// fragment (the other 16 rows of the row block come from the neighbouring block).  x is read once.
-constexpr int kFusedWaves = 8, kFusedRows = 16;
-template <int kTiles>
+// Scale and digits in one pass for rows of up to 16384 values (K % 4 == 0, 16-byte aligned rows): a block of eight
+// wavefronts keeps kRows rows in registers in fragment order.  Wavefront w owns the k tiles
+// [w * kSlots * kPer, (w + 1) * kSlots * kPer), kSlots = 32 / kRows; lane r + kRows * (g + 2 * ts) holds, for row r,
+// the 16 values of fragment half g of the tiles kSlots * t + ts, t < kPer.  Row maxima and row sums cross the
+// wavefronts through LDS; every store instruction then writes runs of kRows * 16 bytes of a fragment (the other rows
+// of the row block come from neighbouring blocks).  x is read once.
+constexpr int kFusedWaves = 8;
+template <int kRows, int kPer>
 __global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const float *__restrict__ x, int64_t ldx,
                                                                        const float *__restrict__ cs,
                                                                        long long *__restrict__ sums,
                                                                        int32_t *__restrict__ shift,
                                                                        uint4_t *__restrict__ out, int64_t M, int64_t K,
                                                                        int64_t k_tiles, int64_t rows) {
-  static_assert(kTiles % 2 == 0, "a lane walks its wavefront's tiles in pairs");
-  constexpr int kPairs = kTiles / 2;
-  __shared__ uint32_t s_max[kFusedWaves][kFusedRows];
-  __shared__ long long s_sum[kFusedWaves][kFusedRows];
+  static_assert(kRows == 4 || kRows == 8 || kRows == 16, "rows per block");
+  static_assert(kPer * 16 < 256, "a lane's partial sum of kPer * 16 values below 2^23 fits an int");
+  constexpr int kSlots = 32 / kRows;
+  __shared__ uint32_t s_max[kFusedWaves][kRows];
+  __shared__ long long s_sum[kFusedWaves][kRows];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int r = lane & 15, g = (lane >> 4) & 1, th = lane >> 5;
-  const int64_t m = (int64_t)blockIdx.x * kFusedRows + r;
+  const int r = lane % kRows, g = (lane / kRows) & 1, ts = lane / (2 * kRows);
+  const int64_t m = (int64_t)blockIdx.x * kRows + r;
   if (blockIdx.x == 0 && threadIdx.x == 0)
     shift[rows] = 1; // the operand's flag word: a row-scaled operand is never in the narrow form
   const float *row = x + m * ldx;
-  float4_t v[kPairs][4];
+  float4_t v[kPer][4];
   uint32_t amax = 0u;
 #pragma unroll
-  for (int t = 0; t < kPairs; ++t) {
-    const int64_t k0 = ((int64_t)wave * kTiles + 2 * t + th) * kTileK + g * 16;
+  for (int t = 0; t < kPer; ++t) {
+    const int64_t k0 = (((int64_t)wave * kPer + t) * kSlots + ts) * kTileK + g * 16;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int64_t k = k0 + 4 * i;
@@ -756,16 +758,17 @@ __global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const floa
     }
   }
 #pragma unroll
-  for (int t = 0; t < kPairs; ++t)
+  for (int t = 0; t < kPer; ++t)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t a = __float_as_uint(v[t][i].x) & 0x7fffffffu, b = __float_as_uint(v[t][i].y) & 0x7fffffffu;
       const uint32_t c = __float_as_uint(v[t][i].z) & 0x7fffffffu, d = __float_as_uint(v[t][i].w) & 0x7fffffffu;
       amax = max(max(amax, max(a, b)), max(c, d));
     }
-  amax = max(amax, (uint32_t)__shfl_xor((int)amax, 16));
-  amax = max(amax, (uint32_t)__shfl_xor((int)amax, 32));
-  if (lane < kFusedRows)
+#pragma unroll
+  for (int off = kRows; off < 64; off <<= 1)
+    amax = max(amax, (uint32_t)__shfl_xor((int)amax, off));
+  if (lane < kRows)
     s_max[wave][lane] = amax;
   __syncthreads();
 #pragma unroll
@@ -773,9 +776,9 @@ __global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const floa
     amax = max(amax, s_max[w][r]);
   const bool bad = amax >= 0x7f800000u;
   const int s = (bad || amax == 0u) ? 0 : digit_shift(amax);
-  int part = 0; // at most 128 values of magnitude < 2^23 per lane
+  int part = 0;
 #pragma unroll
-  for (int t = 0; t < kPairs; ++t) {
+  for (int t = 0; t < kPer; ++t) {
     int q[16];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -787,26 +790,34 @@ __global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const floa
 #pragma unroll
     for (int j = 0; j < 16; ++j)
       part += q[j];
-    const int64_t kt = (int64_t)wave * kTiles + 2 * t + th;
+    const int64_t kt = ((int64_t)wave * kPer + t) * kSlots + ts;
     if (kt < k_tiles) {
       const int64_t rb = m / kFragRows;
       store_digits(q, out + ((rb * k_tiles + kt) * kDigits) * 64 + (int)(m % kFragRows) + 32 * g, true);
     }
   }
   long long acc = part;
-  acc += __shfl_xor(acc, 16);
-  acc += __shfl_xor(acc, 32);
-  if (lane < kFusedRows)
+#pragma unroll
+  for (int off = kRows; off < 64; off <<= 1)
+    acc += __shfl_xor(acc, off);
+  if (lane < kRows)
     s_sum[wave][lane] = acc;
   __syncthreads();
-  if (threadIdx.x < kFusedRows) {
+  if (threadIdx.x < kRows) {
     long long total = 0;
 #pragma unroll
     for (int w = 0; w < kFusedWaves; ++w)
       total += s_sum[w][threadIdx.x];
-    sums[m] = total; // a single chunk: K <= 4096 < kChunkK
+    sums[m] = total; // a single chunk: K <= kChunkK
     shift[m] = bad ? kBadRow : s;
   }
+}
+
+template <int kRows, int kPer>
+void launch_split_digits_rows(const float *x, int64_t ldx, const float *cs, long long *sums, int32_t *shift,
+                              uint4_t *out, int64_t M, int64_t K, const DigitOperand &d, hipStream_t stream) {
+  hipLaunchKernelGGL((split_digits_rows<kRows, kPer>), dim3((unsigned)(d.rows / kRows)), dim3(kFusedWaves * 64), 0,
+                     stream, x, ldx, cs, sums, shift, out, M, K, d.k_tiles, d.rows);
 }
 
 // ---- digit operand of a transposed source: the operand's rows are the columns c of src [R, C] (row stride ld) and
@@ -1115,21 +1126,25 @@ int nbla_hip_split_digits_scaled_f32(const float *x, int64_t ldx, const float *c
   long long *sums = reinterpret_cast<long long *>(base + d.sum_off);
   int32_t *shift = reinterpret_cast<int32_t *>(base + d.shift_off);
   const bool vec = K % 4 == 0 && ldx % 4 == 0 && aligned16(x) && aligned16(cs);
-  if (vec && d.k_tiles <= kFusedWaves * 16) { // rows of up to 4096 values: one pass, rows held in registers
-    const dim3 grid((unsigned)(d.rows / kFusedRows)), block(kFusedWaves * 64);
+  if (vec && d.k_tiles <= 512) { // rows of up to 16384 values: one pass, rows held in registers
     uint4_t *out = static_cast<uint4_t *>(xdigits);
-    if (d.k_tiles <= kFusedWaves * 2)
-      hipLaunchKernelGGL(split_digits_rows<2>, grid, block, 0, stream, x, ldx, cs, sums, shift, out, M, K, d.k_tiles,
-                         d.rows);
-    else if (d.k_tiles <= kFusedWaves * 4)
-      hipLaunchKernelGGL(split_digits_rows<4>, grid, block, 0, stream, x, ldx, cs, sums, shift, out, M, K, d.k_tiles,
-                         d.rows);
-    else if (d.k_tiles <= kFusedWaves * 8)
-      hipLaunchKernelGGL(split_digits_rows<8>, grid, block, 0, stream, x, ldx, cs, sums, shift, out, M, K, d.k_tiles,
-                         d.rows);
+    const int64_t kt = d.k_tiles; // tiles a block covers: 8 wavefronts x (32 / rows) x tiles per lane
+    if (kt <= 16)
+      launch_split_digits_rows<16, 1>(x, ldx, cs, sums, shift, out, M, K, d, stream);
+    else if (kt <= 32)
+      launch_split_digits_rows<16, 2>(x, ldx, cs, sums, shift, out, M, K, d, stream);
+    else if (kt <= 64)
+      launch_split_digits_rows<16, 4>(x, ldx, cs, sums, shift, out, M, K, d, stream);
+    else if (kt <= 128)
+      launch_split_digits_rows<16, 8>(x, ldx, cs, sums, shift, out, M, K, d, stream);
+    else if (kt <= 192)
+      launch_split_digits_rows<8, 6>(x, ldx, cs, sums, shift, out, M, K, d, stream);
+    else if (kt <= 256)
+      launch_split_digits_rows<8, 8>(x, ldx, cs, sums, shift, out, M, K, d, stream);
+    else if (kt <= 384)
+      launch_split_digits_rows<4, 6>(x, ldx, cs, sums, shift, out, M, K, d, stream);
     else
-      hipLaunchKernelGGL(split_digits_rows<16>, grid, block, 0, stream, x, ldx, cs, sums, shift, out, M, K, d.k_tiles,
-                         d.rows);
+      launch_split_digits_rows<4, 8>(x, ldx, cs, sums, shift, out, M, K, d, stream);
     NBLA_HIP_LAUNCH_CHECK("split_digits_rows");
     return NBLA_HIP_OK;
   }

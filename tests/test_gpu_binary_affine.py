@@ -63,11 +63,12 @@ def test_binarize_transposed_layout(dev, K, N):
     np.testing.assert_allclose(to_np(alpha), np.abs(Wnk.astype(np.float64)).mean(1), rtol=2e-6)
 
 
-@pytest.mark.parametrize("M,K", [(45, 70), (45, 128), (64, 64), (100, 1024), (1, 4096), (3, 16384 + 40)])
+@pytest.mark.parametrize("M,K", [(45, 70), (45, 128), (64, 64), (100, 1024), (37, 2048), (1, 4096), (19, 5000), (33, 8192),
+                                 (21, 11008), (9, 16384), (3, 16384 + 40)])
 def test_digit_operand(dev, M, K):
     """The int8 digit operand: q = rint(x * 2^s) with the largest power-of-two scale that keeps the row inside three
-    balanced base-256 digits, digits in fragment order, exact row sums per k chunk (K % 64 == 0 takes the LDS-tiled
-    kernel)."""
+    balanced base-256 digits, digits in fragment order, exact row sums per k chunk (rows of up to 16384 values with
+    K % 4 == 0 take the one-pass kernel in its eight shapes, the others the two-pass kernels)."""
     rng = np.random.RandomState(2)
     x = (rng.randn(M, K) * np.exp(rng.randn(M, 1) * 8)).astype(np.float32)
     x[0, :6] = [0.0, -0.0, 1e-30, -3e-5, 3.3e-7, 1.0]
