@@ -1128,23 +1128,56 @@ int nbla_hip_split_digits_scaled_f32(const float *x, int64_t ldx, const float *c
   const bool vec = K % 4 == 0 && ldx % 4 == 0 && aligned16(x) && aligned16(cs);
   if (vec && d.k_tiles <= 512) { // rows of up to 16384 values: one pass, rows held in registers
     uint4_t *out = static_cast<uint4_t *>(xdigits);
-    const int64_t kt = d.k_tiles; // tiles a block covers: 8 wavefronts x (32 / rows) x tiles per lane
-    if (kt <= 16)
-      launch_split_digits_rows<16, 1>(x, ldx, cs, sums, shift, out, M, K, d, stream);
-    else if (kt <= 32)
-      launch_split_digits_rows<16, 2>(x, ldx, cs, sums, shift, out, M, K, d, stream);
-    else if (kt <= 64)
-      launch_split_digits_rows<16, 4>(x, ldx, cs, sums, shift, out, M, K, d, stream);
-    else if (kt <= 128)
-      launch_split_digits_rows<16, 8>(x, ldx, cs, sums, shift, out, M, K, d, stream);
-    else if (kt <= 192)
-      launch_split_digits_rows<8, 6>(x, ldx, cs, sums, shift, out, M, K, d, stream);
-    else if (kt <= 256)
-      launch_split_digits_rows<8, 8>(x, ldx, cs, sums, shift, out, M, K, d, stream);
-    else if (kt <= 384)
-      launch_split_digits_rows<4, 6>(x, ldx, cs, sums, shift, out, M, K, d, stream);
-    else
-      launch_split_digits_rows<4, 8>(x, ldx, cs, sums, shift, out, M, K, d, stream);
+    // A block covers 8 wavefronts x (32 / rows) x (tiles per lane) k tiles.  Most rows per block (longest store runs)
+    // among the shapes that hold the row and still give every CU a block; the fewest rows otherwise.
+    const int64_t kt = d.k_tiles;
+    int rows_per_block = 0;
+    for (int rows : {16, 8, 4}) {
+      const int64_t per = ceil_div(kt, kFusedWaves * (32 / rows));
+      if (per > (rows == 8 ? 11 : 8))
+        continue;
+      rows_per_block = rows;
+      if (d.rows / rows >= 256)
+        break;
+    }
+    const int64_t per = ceil_div(kt, kFusedWaves * (32 / rows_per_block));
+#define NBLA_SPLIT_ROWS(R, P)                                                                                          \
+  launch_split_digits_rows<R, P>(x, ldx, cs, sums, shift, out, M, K, d, stream)
+    if (rows_per_block == 16) {
+      if (per <= 1)
+        NBLA_SPLIT_ROWS(16, 1);
+      else if (per <= 2)
+        NBLA_SPLIT_ROWS(16, 2);
+      else if (per <= 4)
+        NBLA_SPLIT_ROWS(16, 4);
+      else
+        NBLA_SPLIT_ROWS(16, 8);
+    } else if (rows_per_block == 8) {
+      if (per <= 1)
+        NBLA_SPLIT_ROWS(8, 1);
+      else if (per <= 2)
+        NBLA_SPLIT_ROWS(8, 2);
+      else if (per <= 4)
+        NBLA_SPLIT_ROWS(8, 4);
+      else if (per <= 6)
+        NBLA_SPLIT_ROWS(8, 6);
+      else if (per <= 8)
+        NBLA_SPLIT_ROWS(8, 8);
+      else
+        NBLA_SPLIT_ROWS(8, 11);
+    } else {
+      if (per <= 1)
+        NBLA_SPLIT_ROWS(4, 1);
+      else if (per <= 2)
+        NBLA_SPLIT_ROWS(4, 2);
+      else if (per <= 4)
+        NBLA_SPLIT_ROWS(4, 4);
+      else if (per <= 6)
+        NBLA_SPLIT_ROWS(4, 6);
+      else
+        NBLA_SPLIT_ROWS(4, 8);
+    }
+#undef NBLA_SPLIT_ROWS
     NBLA_HIP_LAUNCH_CHECK("split_digits_rows");
     return NBLA_HIP_OK;
   }

@@ -91,6 +91,27 @@ def test_digit_operand(dev, M, K):
             <= np.ldexp(0.5, -shift[:, None].astype(np.int64))).all()
 
 
+@pytest.mark.parametrize("M,K", [(4100, 128), (4100, 512), (4100, 2048), (2100, 64), (2100, 4096), (2100, 6000),
+                                 (2100, 8192), (2100, 11008), (1100, 4096), (1100, 100)])
+def test_digit_operand_block_shapes(dev, M, K):
+    """Row counts that give every CU a block select the one-pass kernel's 16- and 8-row shapes; the operand must not
+    depend on the shape."""
+    rng = np.random.RandomState(M + K)
+    x = (rng.randn(M, K) * np.exp(rng.randn(M, 1) * 4)).astype(np.float32)
+    x[5] = 0.0
+    x[7, K // 2] = np.inf
+    q, shift, sums = unpack_digits(to_np(kernels.split_digits(_dev(x, dev), M, K)), M, K)
+    assert shift[7] == -2 ** 31 and not q[7].any() and sums[0, 7] == 0 and shift[5] == 0
+    ok = np.ones(M, bool)
+    ok[7] = False
+    amax = np.abs(x[ok]).max(1).astype(np.float64)
+    want = np.where(amax > 0, 22 - np.floor(np.log2(np.where(amax > 0, amax, 1.0))), 0).astype(np.int64)
+    want -= (np.rint(np.ldexp(amax, want)) > 8355711)
+    assert np.array_equal(shift[ok], want)
+    assert np.array_equal(q[ok], np.rint(np.ldexp(x[ok].astype(np.float64), want[:, None])).astype(np.int64))
+    assert np.array_equal(sums[0], q.sum(1))
+
+
 def test_digit_operand_marks_non_finite_rows(dev):
     x = np.ones((5, 64), np.float32)
     x[1, 3] = np.inf
