@@ -1,5 +1,5 @@
 // QuantizeLinear, DequantizeLinear (broadcast scale / zero point, each arithmetic step rounded on its own as the
-// reference's chain of Div2 / round / Add2 / saturate does) and Prune (k-th smallest |x| by a four-pass radix
+// reference's chain of Div2 / round / Add2 / saturate does) and Prune (k-th smallest |x| by a three-pass radix
 // select over the magnitude bits, then a masked copy).  All HBM-bound; 128-bit accesses where the layout allows.
 #include "common.hpp"
 #include "gemm_layout.hpp"
@@ -9,6 +9,8 @@
 
 namespace nbla_hip {
 namespace {
+
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kBlock = 256;
 constexpr int kMaxDims = 6;
@@ -236,69 +238,51 @@ int quantize_range(int dtype, int narrow_range, float &lo, float &hi) {
 
 // ------------------------------------------------------------------------------------------------------ Prune
 
-// Radix select of the rank-th smallest magnitude: four passes over the 31 magnitude bits (8, 8, 8, 7), each
-// histogramming the digit of the elements that share the digits chosen so far.  LDS holds 32 copies of the 256
-// counters, copy = lane % 32 at address bin * 32 + copy: the 32 lanes served together never meet in a counter or a
-// bank.  No separate selection kernels: every block re-derives the chosen digits from the finished histograms of
-// the earlier passes (a 256-entry scan each).
-constexpr int kPasses = 4, kBins = 256, kCopies = 32;
-constexpr int kBinStride = 16; // words between the global counters of two bins: one 64-byte line each
+// Radix select of the rank-th smallest magnitude: three passes over the 31 magnitude bits (11, 10, 10), each
+// histogramming the digit of the elements that share the digits chosen so far.  A block counts in LDS (four copies
+// of the counters, copy = lane % 4), adds its non-zero counters to one of eight global copies (a counter that every
+// block of the grid updates is a serial chain of device-wide atomics, 15 ns each: the dominant cost with a single
+// copy) and takes a ticket; the block holding the last ticket scans the finished histogram and records the chosen
+// digit and the rank left inside it for the next pass.
+constexpr int kPasses = 3, kMaxBins = 2048, kLdsCopies = 4, kGlobalCopies = 8;
+constexpr int kSelectBlocks = 512;
 struct SelectState {
-  uint32_t hist[kPasses][kBins * kBinStride];
+  uint32_t hist[kPasses][kGlobalCopies][kMaxBins];
+  uint32_t done[kPasses];       // blocks of pass p that have added their counters
+  uint32_t prefix[kPasses + 1]; // magnitude bits chosen before pass p (entry kPasses: the selected magnitude)
+  uint32_t rank[kPasses + 1];   // rank among the elements that share them
 };
-__device__ __forceinline__ int pass_shift(int p) { return p == 0 ? 23 : (p == 1 ? 15 : (p == 2 ? 7 : 0)); }
-__device__ __forceinline__ int pass_bits(int p) { return p == 3 ? 7 : 8; }
+__device__ __forceinline__ int pass_shift(int p) { return p == 0 ? 20 : (p == 1 ? 10 : 0); }
+__device__ __forceinline__ int pass_bits(int p) { return p == 0 ? 11 : 10; }
 
-// Digits of passes [0, upto) and the rank left inside the chosen bins; all threads of the block take part and get
-// the same answer.  `scratch` holds kBlock / 64 + 2 words.
-__device__ __forceinline__ void chosen_prefix(const SelectState *st, int upto, uint32_t rank0, uint32_t *scratch,
-                                              uint32_t &prefix, uint32_t &rank) {
-  prefix = 0u;
-  rank = rank0;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int p = 0; p < upto; ++p) {
-    const uint32_t c = st->hist[p][threadIdx.x * kBinStride]; // kBlock == kBins
-    uint32_t incl = c;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-      const uint32_t up = __shfl_up(incl, off);
-      if (lane >= off)
-        incl += up;
-    }
-    if (lane == 63)
-      scratch[wave] = incl;
-    __syncthreads();
-    uint32_t before = 0;
-    for (int w = 0; w < wave; ++w)
-      before += scratch[w];
-    const uint32_t excl = before + incl - c;
-    if (c != 0 && excl <= rank && rank < excl + c) {
-      scratch[kBlock / 64] = (uint32_t)threadIdx.x;
-      scratch[kBlock / 64 + 1] = rank - excl;
-    }
-    __syncthreads();
-    prefix |= scratch[kBlock / 64] << pass_shift(p);
-    rank = scratch[kBlock / 64 + 1];
-    __syncthreads();
+__global__ __launch_bounds__(kBlock) void clear_select(SelectState *st, uint32_t rank0) {
+  uint32_t *h = &st->hist[0][0][0];
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < kPasses * kGlobalCopies * kMaxBins)
+    h[i] = 0u;
+  if (i < kPasses)
+    st->done[i] = 0u;
+  if (i == 0) {
+    st->prefix[0] = 0u;
+    st->rank[0] = rank0;
   }
 }
 
 __global__ __launch_bounds__(kBlock) void prune_histogram(const float *__restrict__ x, int64_t n4, int64_t n,
-                                                          SelectState *__restrict__ st, int pass, uint32_t rank0) {
-  __shared__ uint32_t h[kBins * kCopies];
-  __shared__ uint32_t scratch[kBlock / 64 + 2];
-  for (int i = threadIdx.x; i < kBins * kCopies; i += kBlock)
+                                                          SelectState *__restrict__ st, int pass) {
+  __shared__ uint32_t h[kMaxBins * kLdsCopies];
+  __shared__ uint32_t scratch[kBlock / 64 + 1];
+  for (int i = threadIdx.x; i < kMaxBins * kLdsCopies; i += kBlock)
     h[i] = 0u;
-  uint32_t prefix, rank;
-  chosen_prefix(st, pass, rank0, scratch, prefix, rank);
+  const uint32_t prefix = st->prefix[pass], rank = st->rank[pass];
   __syncthreads();
-  const int shift = pass_shift(pass), above = shift + pass_bits(pass);
-  const uint32_t mask = (1u << pass_bits(pass)) - 1u, want = prefix >> above;
-  const int copy = threadIdx.x & (kCopies - 1);
+  const int shift = pass_shift(pass), above = shift + pass_bits(pass), bins = 1 << pass_bits(pass);
+  const uint32_t mask = (uint32_t)bins - 1u, want = prefix >> above;
+  const int copy = threadIdx.x & (kLdsCopies - 1);
   auto count = [&](float v) {
     const uint32_t key = __float_as_uint(v) & 0x7fffffffu;
     if (pass == 0 || (key >> above) == want)
-      atomicAdd(&h[((key >> shift) & mask) * kCopies + copy], 1u);
+      atomicAdd(&h[((key >> shift) & mask) * kLdsCopies + copy], 1u);
   };
   // four loads in flight per thread before the counters are touched
   const int64_t tiles = (n4 + kBlock * 4 - 1) / (kBlock * 4);
@@ -320,27 +304,70 @@ __global__ __launch_bounds__(kBlock) void prune_histogram(const float *__restric
       count(x[i]);
   }
   __syncthreads();
-  uint32_t total = 0;
-#pragma unroll 8
-  for (int c = 0; c < kCopies; ++c)
-    total += h[threadIdx.x * kCopies + ((c + threadIdx.x) & (kCopies - 1))]; // rotated: one bank per lane
-  if (total)
-    atomicAdd(&st->hist[pass][threadIdx.x * kBinStride], total);
-}
-
-__global__ __launch_bounds__(kBlock) void clear_select(SelectState *st) {
-  for (int p = 0; p < kPasses; ++p)
-    st->hist[p][threadIdx.x * kBinStride] = 0u;
+  uint32_t *g = st->hist[pass][blockIdx.x % kGlobalCopies];
+  for (int b = threadIdx.x; b < bins; b += kBlock) {
+    const uint4_t c = *reinterpret_cast<const uint4_t *>(&h[b * kLdsCopies]);
+    const uint32_t total = c.x + c.y + c.z + c.w;
+    if (total)
+      atomicAdd(&g[b], total);
+  }
+  // The ticket follows this block's counter updates: the barrier waits until every one of them has been performed
+  // (device-wide atomics act on memory itself, past the per-XCD L2), so whoever draws the last ticket finds all
+  // blocks' counts there and reads them the same way, with atomic loads.  No cache write-back or invalidation is
+  // involved, which a fence in every block would cost.
+  __syncthreads();
+  if (threadIdx.x == 0)
+    scratch[kBlock / 64] = atomicAdd(&st->done[pass], 1u);
+  __syncthreads();
+  if (scratch[kBlock / 64] != gridDim.x - 1)
+    return;
+  // thread t owns the bins [t * per, (t + 1) * per), per = 8 or 4
+  const int per = bins / kBlock, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint32_t c[kMaxBins / kBlock];
+#pragma unroll
+  for (int i = 0; i < kMaxBins / kBlock; ++i)
+    c[i] = 0u;
+  for (int k = 0; k < kGlobalCopies; ++k) {
+    const unsigned long long *src = reinterpret_cast<const unsigned long long *>(&st->hist[pass][k][threadIdx.x * per]);
+#pragma unroll
+    for (int i = 0; i < kMaxBins / kBlock / 2; ++i)
+      if (2 * i < per) {
+        const unsigned long long two = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        c[2 * i] += (uint32_t)two;
+        c[2 * i + 1] += (uint32_t)(two >> 32);
+      }
+  }
+  uint32_t mine = 0;
+#pragma unroll
+  for (int i = 0; i < kMaxBins / kBlock; ++i)
+    mine += c[i];
+  uint32_t incl = mine;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t up = __shfl_up(incl, off);
+    if (lane >= off)
+      incl += up;
+  }
+  if (lane == 63)
+    scratch[wave] = incl;
+  __syncthreads();
+  uint32_t excl = incl - mine;
+  for (int w = 0; w < wave; ++w)
+    excl += scratch[w];
+#pragma unroll
+  for (int i = 0; i < kMaxBins / kBlock; ++i) {
+    if (c[i] != 0u && excl <= rank && rank < excl + c[i]) {
+      st->prefix[pass + 1] = prefix | ((uint32_t)(threadIdx.x * per + i) << shift);
+      st->rank[pass + 1] = rank - excl;
+    }
+    excl += c[i];
+  }
 }
 
 // y = (|x| < thresh) ? 0 : x with thresh = |rank-th smallest| (+ 1 when rate == 1), prune.cpp:62-69
 __global__ __launch_bounds__(kBlock) void prune_apply(const float *__restrict__ x, float *__restrict__ y, int64_t n4,
-                                                      int64_t n, const SelectState *__restrict__ st, uint32_t rank0,
-                                                      float add) {
-  __shared__ uint32_t scratch[kBlock / 64 + 2];
-  uint32_t prefix, rank;
-  chosen_prefix(st, kPasses, rank0, scratch, prefix, rank);
-  const float thresh = __uint_as_float(prefix) + add;
+                                                      int64_t n, const SelectState *__restrict__ st, float add) {
+  const float thresh = __uint_as_float(st->prefix[kPasses]) + add;
   const int64_t tiles = (n4 + kBlock * 4 - 1) / (kBlock * 4);
   for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
     const int64_t base = tile * (kBlock * 4) + threadIdx.x;
@@ -455,18 +482,19 @@ int nbla_hip_prune_f32(const float *x, float *y, size_t size, float rate, void *
   const int64_t n = (int64_t)size;
   const int64_t n4 = n / 4;
   int64_t blocks = ceil_div(n4 ? n4 : 1, (int64_t)kBlock * 4);
-  if (blocks > 1024)
-    blocks = 1024; // every block ends with up to 256 global counter updates
-  hipLaunchKernelGGL(clear_select, dim3(1), dim3(kBlock), 0, stream, st);
+  if (blocks > kSelectBlocks)
+    blocks = kSelectBlocks;
+  hipLaunchKernelGGL(clear_select, dim3((unsigned)ceil_div(kPasses * kGlobalCopies * kMaxBins, kBlock)), dim3(kBlock), 0,
+                     stream, st, rank);
   NBLA_HIP_LAUNCH_CHECK("clear_select");
   for (int p = 0; p < kPasses; ++p) {
-    hipLaunchKernelGGL(prune_histogram, dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, n4, n, st, p, rank);
+    hipLaunchKernelGGL(prune_histogram, dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, n4, n, st, p);
     NBLA_HIP_LAUNCH_CHECK("prune_histogram");
   }
   int64_t ablocks = ceil_div(n4 ? n4 : 1, (int64_t)kBlock * 4);
   if (ablocks > 4096)
-    ablocks = 4096; // every block re-derives the threshold, so keep their number bounded
-  hipLaunchKernelGGL(prune_apply, dim3((unsigned)ablocks), dim3(kBlock), 0, stream, x, y, n4, n, st, rank,
+    ablocks = 4096;
+  hipLaunchKernelGGL(prune_apply, dim3((unsigned)ablocks), dim3(kBlock), 0, stream, x, y, n4, n, st,
                      rate == 1.0f ? 1.0f : 0.0f);
   NBLA_HIP_LAUNCH_CHECK("prune_apply");
   return NBLA_HIP_OK;

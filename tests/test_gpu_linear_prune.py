@@ -101,3 +101,15 @@ def test_prune_large_and_special_values(dev):
         assert bits_equal(to_np(y), oracle.prune(x, rate))
     with pytest.raises(kernels.KernelError):
         kernels.prune(_dev(x[:1], dev), 1.5)
+
+
+def test_prune_reuses_its_workspace(dev):
+    """Back-to-back calls on one workspace (histograms, tickets and chosen digits of the previous call are left in
+    it), with changing sizes and rates."""
+    import torch
+    ws = torch.empty(kernels.lib().nbla_hip_prune_workspace_bytes(), dtype=torch.uint8, device=dev)
+    ws.fill_(0xff)
+    for i, (size, rate) in enumerate([(300000, 0.9), (1000, 0.2), (2100000, 0.75), (5, 1.0), (300000, 0.9)]):
+        x = _rand((size,), 20 + i, 2.0)
+        y = kernels.prune(_dev(x, dev), rate, workspace=ws)
+        assert bits_equal(to_np(y), oracle.prune(x, rate)), (size, rate)
