@@ -841,25 +841,24 @@ __global__ __launch_bounds__(kPrepBlock) void clear_column_scratch(uint32_t *__r
     *flag = flag_value;
 }
 
-// Block = 64 column quads x 4 row groups over a slab of 64 rows; 128-bit loads where the layout allows, four in
-// flight per thread; the row groups are folded through LDS before the atomics.
+// Block = 64 column quads x 4 row groups over a slab of `slab` rows (a multiple of 4); 128-bit loads where the
+// layout allows, eight in flight per thread; the row groups are folded through LDS before the atomics.
 template <bool kVec, bool kDetect>
 __global__ __launch_bounds__(kPrepBlock) void column_absmax(const float *__restrict__ src, int64_t ld, int64_t R,
                                                             int64_t C, uint32_t *__restrict__ cmax,
-                                                            uint32_t *__restrict__ cmin, int32_t *__restrict__ flag) {
+                                                            uint32_t *__restrict__ cmin, int32_t *__restrict__ flag,
+                                                            int slab) {
   __shared__ uint32_t part[4][256];
   __shared__ uint32_t part_min[kDetect ? 4 : 1][256];
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   const int64_t c0 = ((int64_t)blockIdx.x * 64 + tx) * 4;
-  const int64_t r0 = (int64_t)blockIdx.y * 64;
+  const int64_t r0 = (int64_t)blockIdx.y * slab;
+  const int64_t r_end = r0 + slab < R ? r0 + slab : R;
   uint32_t m[4] = {0u, 0u, 0u, 0u}, mn[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
   bool other = false; // an element that is neither zero nor a normal power of two
   if (c0 < C) {
-#pragma unroll 4
-    for (int i = 0; i < 16; ++i) {
-      const int64_t r = r0 + ty + 4 * i;
-      if (r >= R)
-        break;
+#pragma unroll 8
+    for (int64_t r = r0 + ty; r < r_end; r += 4) {
       float v[4];
       if (kVec) {
         const float4_t q = *reinterpret_cast<const float4_t *>(src + r * ld + c0);
@@ -982,10 +981,13 @@ int launch_split_digits_columns(const float *src, int64_t ld, void *digits, int6
   hipLaunchKernelGGL(clear_column_scratch, dim3((unsigned)ceil_div(d.rows, kPrepBlock)), dim3(kPrepBlock), 0, stream,
                      cmax, cmin, d.rows, flag, detect_narrow ? 0 : 1);
   NBLA_HIP_LAUNCH_CHECK("clear_column_scratch");
-  const dim3 grid((unsigned)ceil_div(C, 256), (unsigned)ceil_div(R, 64));
+  int slab = 64; // taller slabs (fewer atomics per column) while a thousand blocks remain
+  while (slab < 256 && ceil_div(C, 256) * ceil_div(R, 2 * slab) >= 1024)
+    slab *= 2;
+  const dim3 grid((unsigned)ceil_div(C, 256), (unsigned)ceil_div(R, slab));
   const bool vec = C % 4 == 0 && ld % 4 == 0 && aligned16(src);
 #define NBLA_LAUNCH_ABSMAX(V, D)                                                                                       \
-  hipLaunchKernelGGL((column_absmax<V, D>), grid, dim3(kPrepBlock), 0, stream, src, ld, R, C, cmax, cmin, flag)
+  hipLaunchKernelGGL((column_absmax<V, D>), grid, dim3(kPrepBlock), 0, stream, src, ld, R, C, cmax, cmin, flag, slab)
   if (vec && detect_narrow)
     NBLA_LAUNCH_ABSMAX(true, true);
   else if (vec)
