@@ -113,3 +113,32 @@ def test_prune_reuses_its_workspace(dev):
         x = _rand((size,), 20 + i, 2.0)
         y = kernels.prune(_dev(x, dev), rate, workspace=ws)
         assert bits_equal(to_np(y), oracle.prune(x, rate)), (size, rate)
+
+
+@pytest.mark.parametrize("scale,zp,mode", [(0.3, 3.0, "HALF_AWAY_FROM_ZERO"), (0.0123, -7.0, "HALF_TO_EVEN"),
+                                           (1.9999999, 0.0, "HALF_AWAY_FROM_ZERO"), (0.125, 1.0, "HALF_TO_EVEN"),
+                                           (3e-39, 0.0, "HALF_AWAY_FROM_ZERO"), (1e30, 100.0, "HALF_AWAY_FROM_ZERO"),
+                                           (-0.7, 5.0, "HALF_TO_EVEN")])
+def test_quantize_linear_every_fp32_value(dev, scale, zp, mode):
+    """All 2^32 bit patterns of x for a few scales (ordinary, all-ones significand, power of two, subnormal, huge,
+    negative) against quantize_linear.cpp:78-111 restated with torch operations: an fp32 divide by a device operand,
+    rounding in float64 (exact), fp32 add, clamp.  The kernel estimates most quotients with a reciprocal; this pins
+    that no estimate changes an output."""
+    import torch
+    s = torch.tensor([scale], dtype=torch.float32, device=dev)
+    z = torch.tensor([zp], dtype=torch.float32, device=dev)
+    chunk = 1 << 27
+    for start in range(0, 1 << 32, chunk):
+        lo = start - (1 << 32) if start >= (1 << 31) else start
+        x = torch.arange(lo, lo + chunk, dtype=torch.int32, device=dev).view(torch.float32)
+        y = kernels.quantize_linear(x, s, z.clone(), round_mode=mode)
+        q = (x / s).double()
+        if mode == "HALF_TO_EVEN":
+            t = torch.round(q)
+        else:
+            t = torch.copysign(torch.floor(q.abs() + 0.5), q)
+        ref = torch.clamp(t.float() + z, -128.0, 127.0)
+        same = (y == ref) | (torch.isnan(y) & torch.isnan(ref))
+        if not bool(same.all()):
+            i = int((~same).nonzero()[0])
+            raise AssertionError("x=%r (bits %#x): got %r want %r" % (float(x[i]), start + i, float(y[i]), float(ref[i])))
