@@ -118,12 +118,13 @@ POW2_CASES = [
 
 def _pow2_inputs(rng, shape, scale):
     x = (rng.randn(*shape) * scale).astype(np.float32)
-    # every binade boundary region sqrt(2)*2^k (+-4 ulp), exact powers of two, zeros, subnormals, inf, nan
+    # every binade boundary region sqrt(2)*2^k (+-64 ulp: log2f's own rounding moves the decision by up to 44 ulp of x
+    # in the outer binades), exact powers of two, zeros, subnormals, inf, nan
     ks = np.arange(-149, 128)
     cuts = (np.float64(2.0) ** (ks + 0.5))
     cuts = cuts[(cuts > 1e-45) & (cuts < 3e38)].astype(np.float32)
     near = []
-    for d in range(-4, 5):
+    for d in range(-64, 65):
         near.append((cuts.view(np.uint32).astype(np.int64) + d).astype(np.uint32).view(np.float32))
     pows = (np.float64(2.0) ** np.arange(-149, 128)).astype(np.float32)
     special = np.concatenate(near + [pows, -pows, np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45,
@@ -161,6 +162,38 @@ def test_pow2_quantize_whole_binades_bruteforce(dev):
         ref = oracle.pow2_quantize(x, True, False, 8, 1)
         y = to_np(kernels.pow2_quantize(_dev(x, dev), True, False, 8, 1))
         assert bits_equal(y, ref), first_mismatch(y, ref)
+
+
+@pytest.mark.parametrize("sign,with_zero,n,m", [(True, True, 4, 1), (False, False, 7, 60), (True, False, 8, -20)])
+def test_pow2_quantize_every_normal_fp32_value(dev, sign, with_zero, n, m):
+    """Every normal fp32 input farther than 64 ulp from a cut 2^(k + 1/2) (nearer ones depend on how log2f rounds,
+    up to 44 ulp of x away in the outer binades; they and the subnormals are compared with the host libm above)
+    against pow2_quantize.cpp:55-81 restated in float64 torch operations, where round(log2|x|) is unambiguous."""
+    nn = n - (1 if sign else 0) - (1 if with_zero else 0)
+    p_max, p_min = float(2.0 ** m), float(2.0 ** (m - (2 ** nn - 1)))
+    thr = float(np.float32(p_min * 2.0 ** -0.5))
+    chunk = 1 << 27
+    for start in range(0, 1 << 32, chunk):
+        lo = start - (1 << 32) if start >= (1 << 31) else start
+        bits = torch.arange(lo, lo + chunk, dtype=torch.int32, device=dev)
+        x = bits.view(torch.float32)
+        y = kernels.pow2_quantize(x, sign, with_zero, n, m)
+        ax = x.abs()
+        q = torch.exp2(torch.round(torch.log2(ax.double())))
+        q = torch.clamp(q, max=p_max)
+        low = torch.where(ax < thr, torch.zeros_like(q), torch.full_like(q, p_min)) if with_zero else \
+            torch.full_like(q, p_min)
+        q = torch.where(q < p_min, low, q).float()
+        if sign:
+            ref = torch.where(x < 0, -q, q)
+        else:
+            ref = torch.where(x < 0, torch.full_like(q, 0.0 if with_zero else p_min), q)
+        mant, expo = bits & 0x7fffff, (bits >> 23) & 0xff
+        checked = (expo > 0) & (expo < 255) & ((mant - 0x3504f3).abs() > 64)
+        same = (y == ref) | ~checked
+        if not bool(same.all()):
+            i = int((~same).nonzero()[0])
+            raise AssertionError("x=%r (bits %#x): got %r want %r" % (float(x[i]), start + i, float(y[i]), float(ref[i])))
 
 
 def test_pow2_quantize_errors(dev):
@@ -247,3 +280,38 @@ def test_min_max_quantize_shape_errors(dev):
     with pytest.raises(kernels.KernelError) as ei:
         kernels.min_max_quantize(x, q, q.clone(), q.clone(), q.clone())
     assert ei.value.code == kernels.ERR_VALUE
+
+
+@pytest.mark.parametrize("qr_min,qr_max,ql_min,ql_max", [(-6.0, 6.0, 0.0, 255.0), (-0.37, 1.9, -128.0, 127.0),
+                                                         (0.0, 1e-3, 0.0, 15.0)])
+def test_min_max_quantize_every_fp32_value(dev, qr_min, qr_max, ql_min, ql_max):
+    """All 2^32 bit patterns of x except NaNs through the element-wise chain of min_max_quantize.cpp:188-222, restated
+    with one torch operation per reference function (fp32 each; the fp32 divide takes a device operand; the rounding
+    is done in float64, exactly), for fixed ranges (x_min_max off).  The nudged range follows :353-390 in numpy fp32."""
+    f = np.float32
+    mn, mx, lmn, lmx, eps = f(qr_min), f(qr_max), f(ql_min), f(ql_max), f(0.01)
+    if f(mx - mn) < eps:
+        mx = f(mn + eps)
+    scale = f(f(mx - mn) / f(lmx - lmn))
+    zp_from_min = f(lmn - f(mn / scale))
+    zp = lmn if zp_from_min <= lmn else (lmx if zp_from_min >= lmx else f(np.round(zp_from_min)))
+    m_, M_ = f(f(lmn - zp) * scale), f(f(lmx - zp) * scale)
+    q = lambda v: torch.full((1,), float(v), dtype=torch.float32, device=dev)
+    qmn, qmx = q(qr_min), q(qr_max)
+    sc, lo, hi = q(scale), q(m_), q(M_)
+    chunk = 1 << 27
+    for start in range(0, 1 << 32, chunk):
+        b0 = start - (1 << 32) if start >= (1 << 31) else start
+        x = torch.arange(b0, b0 + chunk, dtype=torch.int32, device=dev).view(torch.float32)
+        y, s_out = kernels.min_max_quantize(x, qmn, qmx, q(ql_min), q(ql_max), 0.999, False, False, 0.01)
+        if start == 0:
+            assert float(s_out) == float(scale) and float(qmn) == float(f(qr_min))
+        t = torch.where(x > lo, x, lo)
+        t = torch.where(t < hi, t, hi)
+        t = (t - lo) / sc
+        t = torch.floor(t.double() + 0.5).float()   # roundf of a non-negative value
+        ref = t * sc + lo
+        same = (y.view(torch.int32) == ref.view(torch.int32)) | torch.isnan(x)
+        if not bool(same.all()):
+            i = int((~same).nonzero()[0])
+            raise AssertionError("x=%r (bits %#x): got %r want %r" % (float(x[i]), start + i, float(y[i]), float(ref[i])))
