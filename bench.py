@@ -13,6 +13,7 @@ kernels' HBM figures (`quantizers`) and the small-M sweep (`sweep`).
   cpu_baseline  the CPU oracle (a port of nnabla's CPU arithmetic, 1 core) on a bounded row sample
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -158,6 +159,26 @@ def bench_other_configs(dev, iters):
     out["inq_affine[1024,4096]x[4096,4096] (restore+quantize+product)"] = {"ms": ms, "TFLOPs": 2.0 * M * K * N / ms / 1e9}
     ms = time_kernel(lambda: k.inq_affine(xa, Wq, I, oW, oI, None, 4, k.INQ_PRODUCT_ONLY), iters)
     out["inq_affine[1024,4096]x[4096,4096] (product only)"] = {"ms": ms, "TFLOPs": 2.0 * M * K * N / ms / 1e9}
+    # the 4-layer quantized MLP, batch 1024: FixedPointQuantize -> INQAffine (every weight fixed, steady-state forward:
+    # restore + quantize + product) -> 3 x [ReLU -> FixedPointQuantize -> BinaryWeightAffine], all 4096 x 4096
+    L = k.lib()
+    Wm = [(torch.randn(K, N, generator=g) * 0.02).to(dev) for _ in range(3)]
+    act = [torch.empty(M, N, device=dev) for _ in range(2)]
+    ws_b = k.binary_affine_workspace(M, K, N, xa)
+
+    def relu_(t):
+        k.check(L.nbla_hip_relu_f32(k._p(t), k._p(t), ctypes.c_size_t(t.numel()), k._stream(None)))
+
+    def mlp():
+        k.fixed_point_quantize(xa, True, 8, 2.0 ** -4, out=act[0])
+        h = k.inq_affine(act[0], Wq, I, oW, oI, None, 4, k.INQ_NO_SELECTION)
+        for l in range(3):
+            relu_(h)
+            k.fixed_point_quantize(h, True, 8, 2.0 ** -4, out=act[0])
+            h, _, _ = k.binary_weight_affine(act[0], Wm[l], None, 1.0, workspace=ws_b, out=act[1])
+        return h
+    ms = time_kernel(mlp, iters)
+    out["quantized_mlp[1024 x 4096, 4 layers] forward"] = {"ms": ms, "TFLOPs": 4 * 2.0 * M * K * N / ms / 1e9}
     # backward passes (the next row of the scope table)
     n = 1 << 24
     xq = torch.randn(n, generator=g).to(dev) * 2

@@ -504,11 +504,15 @@ int launch_tile(const GemmBitsArgs &args, hipStream_t stream) {
 // couples only four wavefronts and one block's prologue / epilogue overlaps the other's main loop.  The packed
 // operand costs 1/24 of the digit operand's bytes per element, so the block tile is one row block high and wide
 // (32x512) to keep the global -> LDS traffic lowest; narrow outputs take 32x256 blocks of two wavefronts, and
-// outputs of at most 256 such tiles use eight wavefronts per 32x256 tile, four k groups of two.
+// outputs of at most 256 such tiles use eight wavefronts per 32x256 tile, four k groups of two; outputs of at most
+// 256 wide tiles (every CU would hold a single block of four wavefronts) eight wavefronts per 32x512 tile, two k
+// groups of four.
 template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream) {
   const int64_t narrow_tiles = ceil_div(a.M, 32) * ceil_div(a.N, 256);
   if (narrow_tiles <= 256) // too few tiles for the CUs: four k groups per tile
     return launch_tile<32, 256, 1, 2, 4, kSwap>(a, stream);
+  if (a.N > 256 && ceil_div(a.M, 32) * ceil_div(a.N, 512) <= 256) // one wide tile per CU at most: two k groups
+    return launch_tile<32, 512, 1, 4, 2, kSwap>(a, stream);
   if (a.N > 256)
     return launch_tile<32, 512, 1, 4, 1, kSwap>(a, stream);
   return launch_tile<32, 256, 1, 2, 1, kSwap>(a, stream);

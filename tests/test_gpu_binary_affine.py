@@ -30,7 +30,7 @@ def _data(M, K, N, seed=313, wscale=0.02):
 
 
 SHAPES = [(1, 32, 64), (2, 3, 4), (5, 17, 9), (8, 64, 64), (33, 100, 130), (64, 256, 256), (129, 96, 320),
-          (300, 1000, 257), (7, 4096, 70)]
+          (300, 1000, 257), (7, 4096, 70), (1000, 200, 2100)]  # the last: 160 wide tiles, two k groups per block
 
 
 @pytest.mark.parametrize("M,K,N", SHAPES)
