@@ -60,43 +60,62 @@ constexpr int kStagesShared = 3, kStagesAlone = 6;
 // and barrier waits are covered by the other's MFMAs.
 // kNarrow: the B operand holds every value in its lowest digit alone (a small integer): three products
 // a_t x b2 -> accumulator t, nothing dropped, and only the lowest-digit fragments of B are copied.
-template <bool kNarrow, int kStages>
+// kGroups = 2 (outputs of at most one tile per CU): eight wavefronts, two groups of four; group g multiplies the k
+// tiles g, g + 2, ... of the same output tile (a stage then holds two consecutive k tiles), so every SIMD has a second
+// wavefront to issue from while the first waits.  At the end the groups swap halves of their int32 accumulators
+// through LDS (exactly) and group g finishes row fragment g of each wavefront tile.
+template <bool kNarrow, int kStages, int kGroups>
 __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsigned char *smem) {
 #if defined(__HIP_DEVICE_COMPILE__) // the host pass only needs the launch stub; the body uses LDS address-space pointers
+  static_assert(kGroups == 1 || kGroups == 2, "k groups per block");
+  constexpr int kAllWaves = kWaves * kGroups;
+  constexpr int kGroupStageBytes = kGroups * kStageBytes;
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int group = wave_all / kWaves, wave = wave_all % kWaves;
   const int wm = wave & 1, wn = wave >> 1;
   int64_t bm, bn;
   band_tile<8>(blockIdx.x, a.blocks_m, a.blocks_n, bm, bn); // two blocks per CU: 64 resident tiles per XCD = 8 x 8
 
-  // this wavefront's copies: chunk c = p * kWaves + wave of the stage; chunks [0, 12) are A fragments (row block,
-  // digit), [12, 24) B fragments
+  // This wavefront's copies.  The 24 fragments of a k tile are numbered u: [0, 12) the A fragments (row block,
+  // digit), [12, 16) the lowest-digit B fragments, [16, 24) the other B fragments; wavefront w takes
+  // u = q * kAllWaves + w, so each takes the same number (two thirds of its list) of the sixteen that the narrow form
+  // needs.  Copy p of a wavefront is fragment q = p % kPerTile of k tile p / kPerTile of the stage.
+  constexpr int kPerTile = kChunks / kAllWaves; // 6 or 3
   const uint4_t *cur[kPerWave], *cur_last[kPerWave];
+  int dest[kPerWave]; // byte offset inside a stage
 #pragma unroll
   for (int p = 0; p < kPerWave; ++p) {
-    const int c = p * kWaves + wave;
-    const int side = c / (kSegs * kDigits), r = c - side * (kSegs * kDigits);
-    const int seg = r / kDigits, d = r - seg * kDigits;
+    const int sub = p / kPerTile, q = p - sub * kPerTile;
+    const int u = q * kAllWaves + wave_all;
+    int side, seg, d;
+    if (u < kSegs * kDigits)
+      side = 0, seg = u / kDigits, d = u - seg * kDigits;
+    else if (u < kSegs * kDigits + kSegs)
+      side = 1, seg = u - kSegs * kDigits, d = kDigits - 1;
+    else
+      side = 1, seg = (u - kSegs * kDigits - kSegs) / (kDigits - 1), d = (u - kSegs * kDigits - kSegs) % (kDigits - 1);
+    dest[p] = sub * kStageBytes + ((side * kSegs + seg) * kDigits + d) * kFragBytes;
     int64_t rb = (side ? bn : bm) * kSegs + seg;
     const int64_t limit = side ? a.b_row_blocks : a.a_row_blocks;
     if (rb >= limit)
       rb = limit - 1; // clamped: those rows / columns are not stored
     const uint4_t *base = (side ? a.bd : a.ad) + (rb * a.k_tiles * kDigits + d) * 64;
-    cur[p] = base + a.step_begin * kSegVec;
-    cur_last[p] = base + (a.step_end - 1) * kSegVec;
+    cur[p] = base + (a.step_begin + sub) * kSegVec;
+    cur_last[p] = base + (a.step_end - kGroups + sub) * kSegVec;
   }
   typedef __attribute__((address_space(3))) void lds_void_t;
-  // narrow: of a wavefront's six chunks the three A fragments and exactly one B fragment (digit 2) are needed
-  constexpr int kCopies = kNarrow ? 4 : kPerWave;
+  // narrow: the first two thirds of each k tile's list (A fragments and lowest-digit B fragments)
+  constexpr int kNeeded = (kSegs * kDigits + kSegs) / kAllWaves; // 4 or 2 per k tile
+  constexpr int kCopies = kNarrow ? kNeeded * kGroups : kPerWave;
   auto copy_next = [&](int buf) {
 #pragma unroll
     for (int p = 0; p < kPerWave; ++p) {
-      if (kNarrow && p >= 3 && ((p * kWaves + wave) - kSegs * kDigits) % kDigits != 2)
+      if (kNarrow && p % kPerTile >= kNeeded)
         continue;
-      __builtin_amdgcn_global_load_lds(cur[p] + lane,
-                                       (lds_void_t *)(smem + buf * kStageBytes + (p * kWaves + wave) * kFragBytes), 16,
-                                       0, 0);
-      const uint4_t *next = cur[p] + kSegVec;
+      __builtin_amdgcn_global_load_lds(cur[p] + lane, (lds_void_t *)(smem + buf * kGroupStageBytes + dest[p]), 16, 0,
+                                       0);
+      const uint4_t *next = cur[p] + kGroups * kSegVec;
       cur[p] = next < cur_last[p] ? next : cur_last[p]; // the last calls copy the final tile again
     }
   };
@@ -117,13 +136,13 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
   for (int d = 0; d < kStages - 1; ++d)
     copy_next(d);
   int buf = 0;
-  for (int64_t kt = a.step_begin; kt < a.step_end; ++kt) {
+  for (int64_t kt = a.step_begin; kt < a.step_end; kt += kGroups) {
     // tile kt has landed (the copies of the kStages - 2 tiles after it may still be in flight) and every wavefront
     // is done with the buffer tile kt - 1 occupied, which tile kt + kStages - 1 takes over
     NBLA_WAIT_VMCNT((kStages - 2) * kCopies);
     NBLA_BARRIER();
     copy_next(buf == 0 ? kStages - 1 : buf - 1);
-    const uint4_t *sa = reinterpret_cast<const uint4_t *>(smem + buf * kStageBytes);
+    const uint4_t *sa = reinterpret_cast<const uint4_t *>(smem + buf * kGroupStageBytes + group * kStageBytes);
     const uint4_t *sb = sa + kSideVec;
     i32x4_t af[2][3], bf[2][3];
 #pragma unroll
@@ -159,6 +178,36 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
   }
   NBLA_WAIT_VMCNT(0);
 
+  if (kGroups == 2) {
+    // swap: every wavefront hands the row fragment it does not finish to its partner in the other group, one
+    // accumulator set at a time (8 wavefronts x 2 fragments x 16 registers x 64 lanes x 4 B = 64 KiB per round)
+    int *xs = reinterpret_cast<int *>(smem);
+    const int partner = wave_all ^ kWaves;
+#pragma unroll
+    for (int t = 0; t < 3; ++t) {
+      __syncthreads(); // the stages (first round) or the previous round's values have been read
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        if (i != group) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              xs[((wave_all * 2 + j) * 16 + r) * 64 + lane] = acc[i][j][t][r];
+        }
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        if (i == group) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              acc[i][j][t][r] += xs[((partner * 2 + j) * 16 + r) * 64 + lane];
+        }
+    }
+  }
+
   // y = (acc0 * 2^16 + acc1 * 2^8 + acc2) * 2^(16 - sa - sb); the narrow form has no factor 2^16 (b is its low digit).
   // Row by row: the row's offset (one 32-bit division when m is folded into two output indices) and shift are
   // formed once and serve both column fragments.
@@ -187,6 +236,8 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
   }
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
+    if (kGroups == 2 && i != group)
+      continue;
     const int64_t m0 = bm * kBM + (wm * 2 + i) * 32;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -231,13 +282,13 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
 #endif
 }
 
-template <int kStages>
-__global__ __launch_bounds__(kThreads, 2) void gemm_digits_kernel(GemmDigitsArgs a) {
+template <int kStages, int kGroups>
+__global__ __launch_bounds__(kThreads * kGroups, kGroups == 1 ? 2 : 1) void gemm_digits_kernel(GemmDigitsArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   if (*a.bflag == 0) // uniform over the grid
-    gemm_digits_tile<true, kStages>(a, smem);
+    gemm_digits_tile<true, kStages, kGroups>(a, smem);
   else
-    gemm_digits_tile<false, kStages>(a, smem);
+    gemm_digits_tile<false, kStages, kGroups>(a, smem);
 }
 
 } // namespace
@@ -250,11 +301,14 @@ int launch_gemm_digits(const void *adigits, const void *bdigits, const float *bi
   const DigitOperand da = digit_operand(M, K), db = digit_operand(N, K);
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_digits_kernel<kStagesShared>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_digits_kernel<kStagesShared, 1>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kStagesShared * kStageBytes);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_digits_kernel<kStagesAlone>),
+      e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_digits_kernel<kStagesAlone, 1>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, kStagesAlone * kStageBytes);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_digits_kernel<kStagesShared, 2>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kStagesShared * 2 * kStageBytes);
     if (e != hipSuccess)
       return fail_hip(e, "hipFuncSetAttribute(gemm_digits LDS size)");
     configured = true;
@@ -286,12 +340,16 @@ int launch_gemm_digits(const void *adigits, const void *bdigits, const float *bi
     a.accumulate = (accumulate || chunk > 0) ? 1 : 0;
     a.finish = a.step_end == a.k_tiles ? 1 : 0;
     const unsigned blocks = (unsigned)(a.blocks_m * a.blocks_n);
-    if (blocks <= 384) // fewer than 1.5 blocks per CU
-      hipLaunchKernelGGL(gemm_digits_kernel<kStagesAlone>, dim3(blocks), dim3(kThreads), kStagesAlone * kStageBytes,
-                         stream, a);
+    if (blocks <= 256 && (a.step_end - a.step_begin) % 2 == 0) // at most one block per CU: eight wavefronts, two k
+                                                               // groups (k tiles come in multiples of 8)
+      hipLaunchKernelGGL((gemm_digits_kernel<kStagesShared, 2>), dim3(blocks), dim3(2 * kThreads),
+                         kStagesShared * 2 * kStageBytes, stream, a);
+    else if (blocks <= 384) // fewer than 1.5 blocks per CU
+      hipLaunchKernelGGL((gemm_digits_kernel<kStagesAlone, 1>), dim3(blocks), dim3(kThreads),
+                         kStagesAlone * kStageBytes, stream, a);
     else
-      hipLaunchKernelGGL(gemm_digits_kernel<kStagesShared>, dim3(blocks), dim3(kThreads), kStagesShared * kStageBytes,
-                         stream, a);
+      hipLaunchKernelGGL((gemm_digits_kernel<kStagesShared, 1>), dim3(blocks), dim3(kThreads),
+                         kStagesShared * kStageBytes, stream, a);
     NBLA_HIP_LAUNCH_CHECK("gemm_digits");
   }
   return NBLA_HIP_OK;
