@@ -215,56 +215,77 @@ __global__ __launch_bounds__(256) void conv_row_shift(const uint32_t *__restrict
 }
 
 // A wavefront converts kTilesPerWave consecutive k tiles of one row block: lane l owns row rb*32 + l%32 and the
-// k-slots (l/32)*16 + 0..15 of each tile.  The column index is decoded to (channel, tap) once per tile and then
-// stepped; the row's partial sum of fixed-point values goes to the row sums with one 64-bit atomic per lane.
+// k-slots (l/32)*16 + 0..15 of each tile.  The wavefront first decodes its 64 column indices k -> (channel, tap),
+// one per lane, into a wavefront-private LDS table {offset of the tap relative to the window origin, tap
+// displacements per dimension, k < Kg}; an element then costs one broadcast table read, three bound checks and one
+// load, issued unconditionally from a clamped address and masked afterwards.  Offsets inside one sample's channel
+// group are 32-bit (the host checks that they fit).  The row's partial sum of fixed-point values goes to the row sums
+// with one 64-bit atomic per lane.
 constexpr int kTilesPerWave = 2;
+static_assert(kTilesPerWave * kTileK == 64, "one table entry per lane");
 __global__ __launch_bounds__(256) void im2col_digits(const float *__restrict__ x, const int32_t *__restrict__ shift,
                                                      long long *__restrict__ sums, uint4_t *__restrict__ out,
                                                      ConvGeom g, int64_t grp, int64_t k_tiles, int64_t tile_groups,
                                                      int64_t rows, int64_t jobs) {
+  typedef int i32x4_t __attribute__((ext_vector_type(4)));
+  __shared__ i32x4_t table[4][64];
   const int64_t job = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (job >= jobs)
     return;
-  const int lane = threadIdx.x & 63;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t rb = job / tile_groups, tg = job - rb * tile_groups;
   const int64_t m = rb * kFragRows + (lane & 31);
   const int s = shift[m];
   const bool row_ok = m < g.M && s != kBadRow;
-  // output position of the row
-  const int64_t n = m / g.out_sp_size;
-  int64_t p = m - n * g.out_sp_size;
-  const int o2 = (int)(p % g.out_sp[2]);
+  const int in0 = g.in_sp[0], in1 = g.in_sp[1], in2 = g.in_sp[2], plane = (int)g.in_sp_size;
+  const int64_t kt_begin = tg * kTilesPerWave;
+  {
+    const int K0 = g.k[0], K1 = g.k[1], K2 = g.k[2];
+    const int kk = (int)(kt_begin * kTileK) + lane;
+    int q = kk;
+    const int k2 = q % K2;
+    q /= K2;
+    const int k1 = q % K1;
+    q /= K1;
+    const int k0 = q % K0, c = q / K0;
+    const int e0 = k0 * g.dil[0], e1 = k1 * g.dil[1], e2 = k2 * g.dil[2];
+    i32x4_t e;
+    e.x = c * plane + (e0 * in1 + e1) * in2 + e2;
+    e.y = e0 | (e1 << 16);
+    e.z = e2;
+    e.w = kk < (int)g.Kg ? 1 : 0;
+    table[wave][lane] = e; // read back by this wavefront only: LDS operations of one wavefront complete in order
+  }
+  // output position of the row (rows past the end read sample 0 and are masked)
+  const int64_t n = m < g.M ? m / g.out_sp_size : 0;
+  int p = m < g.M ? (int)(m - n * g.out_sp_size) : 0;
+  const int o2 = p % g.out_sp[2];
   p /= g.out_sp[2];
-  const int o1 = (int)(p % g.out_sp[1]);
-  const int o0 = (int)(p / g.out_sp[1]);
+  const int o1 = p % g.out_sp[1];
+  const int o0 = p / g.out_sp[1];
   const int b0 = o0 * g.stride[0] - g.pad[0], b1 = o1 * g.stride[1] - g.pad[1], b2 = o2 * g.stride[2] - g.pad[2];
+  const int origin = (b0 * in1 + b1) * in2 + b2; // may be negative; origin + table offset is checked per element
   const float *xn = x + (n * g.C + grp * g.Cg) * g.in_sp_size;
   long long row_sum[2] = {0, 0}; // at most two chunks meet a group of tiles
-  const int64_t kt_begin = tg * kTilesPerWave;
   for (int t = 0; t < kTilesPerWave; ++t) {
     const int64_t kt = kt_begin + t;
     if (kt >= k_tiles)
       break;
-    const int64_t k0 = kt * kTileK + (lane >> 5) * 16;
-    // decode k0 -> (channel, tap)
-    int64_t q = k0;
-    int k2 = (int)(q % g.k[2]);
-    q /= g.k[2];
-    int k1 = (int)(q % g.k[1]);
-    q /= g.k[1];
-    int kk0 = (int)(q % g.k[0]);
-    int64_t c = q / g.k[0];
+    float v[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const i32x4_t e = table[wave][t * kTileK + (lane >> 5) * 16 + j];
+      const int i0 = b0 + (e.y & 0xffff), i1 = b1 + (int)((uint32_t)e.y >> 16), i2 = b2 + e.z;
+      const bool ok = row_ok && e.w != 0 && (unsigned)i0 < (unsigned)in0 && (unsigned)i1 < (unsigned)in1 &&
+                      (unsigned)i2 < (unsigned)in2;
+      const float xv = xn[ok ? origin + e.x : 0];
+      v[j] = ok ? xv : 0.0f;
+    }
     uint32_t w[3][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
     int part = 0;
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
-      int qv = 0;
-      if (row_ok && k0 + j < g.Kg) {
-        const int i0 = b0 + kk0 * g.dil[0], i1 = b1 + k1 * g.dil[1], i2 = b2 + k2 * g.dil[2];
-        if ((unsigned)i0 < (unsigned)g.in_sp[0] && (unsigned)i1 < (unsigned)g.in_sp[1] &&
-            (unsigned)i2 < (unsigned)g.in_sp[2])
-          qv = to_fixed(xn[c * g.in_sp_size + ((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2] + i2], s);
-      }
+      const int qv = to_fixed(v[j], s); // masked values are 0.0f -> 0 whatever the shift
       part += qv;
       const int lo = (int)(int8_t)qv;
       const int q1 = (qv - lo) >> 8;
@@ -274,17 +295,6 @@ __global__ __launch_bounds__(256) void im2col_digits(const float *__restrict__ x
       w[0][j >> 2] |= ((uint32_t)hi & 0xffu) << sh;
       w[1][j >> 2] |= ((uint32_t)mid & 0xffu) << sh;
       w[2][j >> 2] |= ((uint32_t)lo & 0xffu) << sh;
-      // next column: tap index runs fastest, then the channel
-      if (++k2 == g.k[2]) {
-        k2 = 0;
-        if (++k1 == g.k[1]) {
-          k1 = 0;
-          if (++kk0 == g.k[0]) {
-            kk0 = 0;
-            ++c;
-          }
-        }
-      }
     }
     row_sum[(kt * kTileK) / kChunkK - (kt_begin * kTileK) / kChunkK] += part;
     uint4_t *dst = out + ((rb * k_tiles + kt) * kDigits) * 64 + lane;
@@ -326,6 +336,14 @@ int launch_im2col_split(const float *x, void *xsplit, const ConvGeom &g, int64_t
 // `scratch` holds kChannelSlices * outer * in_sp_size uint32 (the channel maxima).
 int launch_im2col_digits(const float *x, void *xdigits, void *scratch, const ConvGeom &g, int64_t grp,
                          hipStream_t stream) {
+  // the unfold kernel keeps offsets inside one sample's channel group, output positions and k in 32 bits
+  bool fits = g.Cg * g.in_sp_size < ((int64_t)1 << 31) && g.out_sp_size < ((int64_t)1 << 31) &&
+              g.Kg + 2 * kTileK * kTilesPerWave < ((int64_t)1 << 31);
+  for (int i = 0; i < kMaxSpatial; ++i)
+    fits = fits && (int64_t)(g.k[i] - 1) * g.dil[i] < 65536; // tap displacements travel as 16-bit fields
+  if (!fits)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "convolution: a sample's channel group, its output map or the unfolded "
+                                              "row has 2^31 elements or more, or a dilated kernel spans 65536.");
   const DigitOperand d = digit_operand(g.M, g.Kg);
   char *base = static_cast<char *>(xdigits);
   long long *sums = reinterpret_cast<long long *>(base + d.sum_off);
