@@ -91,24 +91,32 @@ __global__ __launch_bounds__(kBlk) void inq_restore_absmax(float *__restrict__ W
     for (int64_t i = (int64_t)blockIdx.x * kBlk + threadIdx.x; i < n4; i += 2 * stride) {
       const int64_t j = i + stride;
       const bool second = j < n4;
-      f4_t w0 = reinterpret_cast<const f4_t *>(W)[i], w1 = w0;
-      i4_t f0 = reinterpret_cast<const i4_t *>(old_I)[i], f1 = f0;
-      if (second) {
+      // the indicators first: a quad whose four weights are all fixed is taken from the snapshot without reading W
+      const i4_t f0 = reinterpret_cast<const i4_t *>(old_I)[i];
+      const i4_t f1 = second ? reinterpret_cast<const i4_t *>(old_I)[j] : f0;
+      const bool all0 = f0.x == 1 && f0.y == 1 && f0.z == 1 && f0.w == 1;
+      const bool any0 = f0.x == 1 || f0.y == 1 || f0.z == 1 || f0.w == 1;
+      const bool all1 = f1.x == 1 && f1.y == 1 && f1.z == 1 && f1.w == 1;
+      const bool any1 = f1.x == 1 || f1.y == 1 || f1.z == 1 || f1.w == 1;
+      f4_t w0 = {0.0f, 0.0f, 0.0f, 0.0f}, w1 = w0, o0 = w0, o1 = w0;
+      if (!all0)
+        w0 = reinterpret_cast<const f4_t *>(W)[i];
+      if (any0)
+        o0 = reinterpret_cast<const f4_t *>(old_W)[i];
+      if (second && !all1)
         w1 = reinterpret_cast<const f4_t *>(W)[j];
-        f1 = reinterpret_cast<const i4_t *>(old_I)[j];
-      }
-      if (f0.x == 1 || f0.y == 1 || f0.z == 1 || f0.w == 1) {
-        const f4_t o = reinterpret_cast<const f4_t *>(old_W)[i];
-        w0.x = f0.x == 1 ? o.x : w0.x, w0.y = f0.y == 1 ? o.y : w0.y;
-        w0.z = f0.z == 1 ? o.z : w0.z, w0.w = f0.w == 1 ? o.w : w0.w;
+      if (second && any1)
+        o1 = reinterpret_cast<const f4_t *>(old_W)[j];
+      if (any0) {
+        w0.x = f0.x == 1 ? o0.x : w0.x, w0.y = f0.y == 1 ? o0.y : w0.y;
+        w0.z = f0.z == 1 ? o0.z : w0.z, w0.w = f0.w == 1 ? o0.w : w0.w;
         reinterpret_cast<f4_t *>(W)[i] = w0;
       }
       take(w0.x), take(w0.y), take(w0.z), take(w0.w);
       if (second) {
-        if (f1.x == 1 || f1.y == 1 || f1.z == 1 || f1.w == 1) {
-          const f4_t o = reinterpret_cast<const f4_t *>(old_W)[j];
-          w1.x = f1.x == 1 ? o.x : w1.x, w1.y = f1.y == 1 ? o.y : w1.y;
-          w1.z = f1.z == 1 ? o.z : w1.z, w1.w = f1.w == 1 ? o.w : w1.w;
+        if (any1) {
+          w1.x = f1.x == 1 ? o1.x : w1.x, w1.y = f1.y == 1 ? o1.y : w1.y;
+          w1.z = f1.z == 1 ? o1.z : w1.z, w1.w = f1.w == 1 ? o1.w : w1.w;
           reinterpret_cast<f4_t *>(W)[j] = w1;
         }
         take(w1.x), take(w1.y), take(w1.z), take(w1.w);
@@ -217,7 +225,8 @@ __global__ __launch_bounds__(kBlk) void inq_quantize(float *__restrict__ W, int 
       // zero with a zero threshold, infinities and NaN: outside the reference's defined behaviour; left as they are
     }
     W[i] = w;
-    I[i] = ind;
+    if (fix_all)
+      I[i] = ind; // otherwise unchanged
     old_W[i] = w;
     old_I[i] = ind;
   }
