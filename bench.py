@@ -231,9 +231,19 @@ def cpu_baseline(K, N, rows):
     t0 = time.perf_counter()
     oracle.binary_weight_affine(x, W, None, 1.0)
     dt = time.perf_counter() - t0
-    return {"value": 2.0 * rows * K * N / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
-            "sample": "BinaryWeightAffine forward (sign/alpha passes over the full W + fp32 GEMM) on %d of 4096 "
-                      "rows of x, K=%d, N=%d, %.1f s" % (rows, K, N, dt)}
+    out = {"value": 2.0 * rows * K * N / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+           "sample": "BinaryWeightAffine forward (sign/alpha passes over the full W + fp32 GEMM) on %d of 4096 "
+                     "rows of x, K=%d, N=%d, %.1f s" % (rows, K, N, dt)}
+    # a second, separately labelled figure: the same fp32 product alone with the host BLAS on all cores
+    import torch
+    xt, wt = torch.from_numpy(x), torch.from_numpy(W)
+    torch.matmul(xt[:64], wt)
+    t0 = time.perf_counter()
+    torch.matmul(xt, wt)
+    dt = time.perf_counter() - t0
+    out["host_blas_sgemm"] = {"TFLOPs": 2.0 * rows * K * N / dt / 1e12, "threads": torch.get_num_threads(),
+                              "note": "torch.matmul fp32 of the same rows, product only (no sign / alpha passes)"}
+    return out
 
 
 def main():
