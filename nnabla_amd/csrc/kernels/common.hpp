@@ -5,6 +5,8 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <atomic>
+
 #include "nbla_hip_kernels.h"
 
 namespace nbla_hip {
@@ -25,6 +27,23 @@ enum CutTable { kCutPow2Round = 0, kCutInqExponent = 1, kCutInqN1 = 2, kNumCutTa
 const uint32_t *device_cut_table(int which);
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Raises a kernel's dynamic LDS limit on the current device, once per device (`done` holds one bit per device; the
+// attribute belongs to the device that is current when it is set).
+inline int allow_dynamic_lds(const void *kernel, int bytes, std::atomic<uint64_t> &done, const char *what) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess)
+    return fail_hip(e, "hipGetDevice");
+  const uint64_t bit = 1ull << (dev & 63);
+  if (done.load(std::memory_order_acquire) & bit)
+    return NBLA_HIP_OK;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess)
+    return fail_hip(e, what);
+  done.fetch_or(bit, std::memory_order_release);
+  return NBLA_HIP_OK;
+}
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline bool aligned256(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 255u) == 0; }

@@ -484,13 +484,11 @@ int launch_tile(const GemmBitsArgs &args, hipStream_t stream) {
   constexpr int kThreads = kWavesM * kWavesN * kWavesK * 64;
   constexpr int kSmem = gemm_bits_lds_bytes(BM, BN, kWavesM, kWavesN, kWavesK);
   auto kernel = gemm_bits_kernel<BM, BN, kWavesM, kWavesN, kWavesK, kSwap>;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
-    if (e != hipSuccess)
-      return fail_hip(e, "hipFuncSetAttribute(gemm_bits LDS size)");
-    configured = true;
-  }
+  static std::atomic<uint64_t> configured{0};
+  const int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), kSmem, configured,
+                                   "hipFuncSetAttribute(gemm_bits LDS size)");
+  if (rc)
+    return rc;
   GemmBitsArgs a = args;
   a.blocks_m = ceil_div(a.M, BM);
   a.blocks_n = ceil_div(a.n_end - a.n_begin, BN);

@@ -299,20 +299,17 @@ int launch_gemm_digits(const void *adigits, const void *bdigits, const float *bi
   if (M >= ((int64_t)1 << 31) || N >= ((int64_t)1 << 31))
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "digit product: more than 2^31 - 1 rows or columns.");
   const DigitOperand da = digit_operand(M, K), db = digit_operand(N, K);
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_digits_kernel<kStagesShared, 1>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kStagesShared * kStageBytes);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_digits_kernel<kStagesAlone, 1>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, kStagesAlone * kStageBytes);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_digits_kernel<kStagesShared, 2>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, kStagesShared * 2 * kStageBytes);
-    if (e != hipSuccess)
-      return fail_hip(e, "hipFuncSetAttribute(gemm_digits LDS size)");
-    configured = true;
-  }
+  static std::atomic<uint64_t> configured[3];
+  int rc = allow_dynamic_lds(reinterpret_cast<const void *>(gemm_digits_kernel<kStagesShared, 1>),
+                             kStagesShared * kStageBytes, configured[0], "hipFuncSetAttribute(gemm_digits LDS size)");
+  if (!rc)
+    rc = allow_dynamic_lds(reinterpret_cast<const void *>(gemm_digits_kernel<kStagesAlone, 1>),
+                           kStagesAlone * kStageBytes, configured[1], "hipFuncSetAttribute(gemm_digits LDS size)");
+  if (!rc)
+    rc = allow_dynamic_lds(reinterpret_cast<const void *>(gemm_digits_kernel<kStagesShared, 2>),
+                           kStagesShared * 2 * kStageBytes, configured[2], "hipFuncSetAttribute(gemm_digits LDS size)");
+  if (rc)
+    return rc;
   GemmDigitsArgs a;
   a.ad = static_cast<const uint4_t *>(adigits);
   a.bd = static_cast<const uint4_t *>(bdigits);

@@ -257,14 +257,11 @@ int launch_gemm_planes(const void *xsplit, const void *wplanes, const int *need_
                        const float *bias, float *y, int64_t M, int64_t K, int64_t N, int64_t inner,
                        int64_t outer_stride, int64_t n_stride, hipStream_t stream, bool accumulate) {
   constexpr int kSmem = 2 * (kAStageBytes + kSegs * 2 * 3 * 64 * 16);
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_planes_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
-    if (e != hipSuccess)
-      return fail_hip(e, "hipFuncSetAttribute(gemm_planes LDS size)");
-    configured = true;
-  }
+  static std::atomic<uint64_t> configured{0};
+  const int rc_lds = allow_dynamic_lds(reinterpret_cast<const void *>(gemm_planes_kernel), kSmem, configured,
+                                       "hipFuncSetAttribute(gemm_planes LDS size)");
+  if (rc_lds)
+    return rc_lds;
   GemmPlanesArgs a;
   a.xs = static_cast<const uint4_t *>(xsplit);
   a.ws = static_cast<const uint4_t *>(wplanes);
