@@ -149,6 +149,13 @@ def bench_other_configs(dev, iters):
     out["binary_weight_convolution[32,256,14,14]x[256,256,3,3]"] = {"ms": ms, "TFLOPs": flop / ms / 1e9}
     ms = time_kernel(lambda: k.binary_connect_convolution(x, W, None, (1, 1), (1, 1), (1, 1), 1), iters)
     out["binary_connect_convolution[32,256,14,14]x[256,256,3,3]"] = {"ms": ms, "TFLOPs": flop / ms / 1e9}
+    # backward of the same stage: dx, dW (db is a column sum) in one call
+    dyc = torch.randn(32, 256, 14, 14, generator=g).to(dev)
+    gx, gw, gb = torch.zeros_like(x), torch.zeros_like(W), torch.zeros(256, device=dev)
+    ms = time_kernel(lambda: k.binary_convolution_backward(dyc, x, W, None, None, (1, 1), (1, 1), (1, 1), 1, 1.0,
+                                                           dx=gx, dW=gw, db=gb), iters)
+    out["binary_connect_convolution_backward[32,256,14,14]x[256,256,3,3] dx+dW+db"] = {
+        "ms": ms, "TFLOPs": 2 * flop / ms / 1e9}
     M, K, N = 1024, 4096, 4096
     xa = torch.randn(M, K, generator=g).to(dev)
     Wq = (torch.randn(K, N, generator=g) * 0.02).to(dev)

@@ -7,19 +7,31 @@
 namespace nbla_hip {
 namespace {
 
-constexpr int kRows = 256; // rows of dy per partial column sum
+// Column sums (bias gradients) in a fixed order: slices of `rows` rows (256, or 64 when that leaves fewer than a
+// thousand blocks), inside a slice four interleaved row groups per column, folded through LDS in group order; then
+// the slices in slice order.
+constexpr int kSumCols = 64;
+inline int column_sum_rows(int64_t M, int64_t N) {
+  return ceil_div(N, kSumCols) * ceil_div(M, 256) >= 1024 ? 256 : 64;
+}
 
-// partial[s][n] = sum of dy[m][n] over the rows m of slice s, in row order; consecutive threads are consecutive columns.
+// partial[s][n] = sum of dy[m][n] over the rows m of slice s; block = 64 columns x 4 row groups.
 __global__ __launch_bounds__(256) void column_sum_partial(const float *__restrict__ dy, float *__restrict__ partial,
-                                                          int64_t M, int64_t N) {
-  const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (n >= N)
-    return;
-  const int64_t m0 = (int64_t)blockIdx.y * kRows, m1 = (m0 + kRows < M) ? m0 + kRows : M;
+                                                          int64_t M, int64_t N, int rows) {
+  __shared__ float part[4][kSumCols];
+  const int c = threadIdx.x & (kSumCols - 1), rg = threadIdx.x >> 6;
+  const int64_t n = (int64_t)blockIdx.x * kSumCols + c;
+  const int64_t m0 = (int64_t)blockIdx.y * rows, m1 = (m0 + rows < M) ? m0 + rows : M;
   float acc = 0.0f;
-  for (int64_t m = m0; m < m1; ++m)
-    acc += dy[m * N + n];
-  partial[(int64_t)blockIdx.y * N + n] = acc;
+  if (n < N) {
+#pragma unroll 8
+    for (int64_t m = m0 + rg; m < m1; m += 4)
+      acc += dy[m * N + n];
+  }
+  part[rg][c] = acc;
+  __syncthreads();
+  if (rg == 0 && n < N)
+    partial[(int64_t)blockIdx.y * N + n] = ((part[0][c] + part[1][c]) + part[2][c]) + part[3][c];
 }
 
 __global__ __launch_bounds__(256) void column_sum_final(const float *__restrict__ partial, float *__restrict__ db,
@@ -28,6 +40,7 @@ __global__ __launch_bounds__(256) void column_sum_final(const float *__restrict_
   if (n >= N)
     return;
   float acc = 0.0f;
+#pragma unroll 8
   for (int64_t s = 0; s < slices; ++s)
     acc += partial[s * N + n];
   db[n] = accumulate ? db[n] + acc : acc;
@@ -119,13 +132,14 @@ int check_args(int64_t M, int64_t K, int64_t N, void *workspace, size_t workspac
 
 } // namespace
 
-size_t column_sums_workspace_bytes(int64_t M, int64_t N) { return (size_t)ceil_div(M, kRows) * N * sizeof(float); }
+size_t column_sums_workspace_bytes(int64_t M, int64_t N) { return (size_t)ceil_div(M, 64) * N * sizeof(float); }
 
 int launch_column_sums(const float *dy, float *db, int64_t M, int64_t N, bool accumulate, void *partial,
                        hipStream_t stream) {
-  const int64_t slices = ceil_div(M, kRows);
-  hipLaunchKernelGGL(column_sum_partial, dim3((unsigned)ceil_div(N, 256), (unsigned)slices), dim3(256), 0, stream, dy,
-                     static_cast<float *>(partial), M, N);
+  const int rows = column_sum_rows(M, N);
+  const int64_t slices = ceil_div(M, rows);
+  hipLaunchKernelGGL(column_sum_partial, dim3((unsigned)ceil_div(N, kSumCols), (unsigned)slices), dim3(256), 0, stream,
+                     dy, static_cast<float *>(partial), M, N, rows);
   NBLA_HIP_LAUNCH_CHECK("column_sum_partial");
   hipLaunchKernelGGL(column_sum_final, dim3((unsigned)ceil_div(N, 256)), dim3(256), 0, stream,
                      static_cast<const float *>(partial), db, slices, N, accumulate ? 1 : 0);
