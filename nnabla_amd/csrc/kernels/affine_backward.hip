@@ -56,7 +56,8 @@ __global__ __launch_bounds__(256) void scale_columns(const float *__restrict__ d
 size_t max3(size_t a, size_t b, size_t c) { return a > b ? (a > c ? a : c) : (b > c ? b : c); }
 
 struct BackwardPlan {
-  size_t bits_off, digits_off, prep_off, count_off, a_planes_off, b_planes_off, flag_off, sums_off, scaled_off, total;
+  size_t bits_off, digits_off, prep_off, count_off, a_planes_off, b_planes_off, flag_off, sums_off, scaled_off, split_off,
+      split_bytes, total;
 };
 
 // One layout for all three backward entry points (the regions a call does not use are simply left alone).
@@ -88,6 +89,10 @@ BackwardPlan plan_backward(int64_t M, int64_t K, int64_t N) {
   off += round_up(column_sums_workspace_bytes(M, N), 256);
   p.scaled_off = off; // dy * alpha in fp32, general path only
   off += round_up((size_t)M * N * sizeof(float), 256);
+  p.split_off = off; // partial results of a digit product whose contraction is spread over the CUs (small outputs)
+  const size_t s1 = gemm_digits_split_bytes(K, M, N), s2 = gemm_digits_split_bytes(M, N, K);
+  p.split_bytes = s1 > s2 ? s1 : s2;
+  off += round_up(p.split_bytes, 256);
   p.total = off;
   return p;
 }
@@ -103,7 +108,7 @@ int grad_weights(const float *x, const float *dy, float *dW, int64_t M, int64_t 
   if (rc)
     return rc;
   return launch_gemm_digits(base + p.a_planes_off, base + p.b_planes_off, nullptr, dW, K, M, N, 1, N, 1, stream,
-                            accumulate);
+                            accumulate, base + p.split_off, p.split_bytes);
 }
 
 // dx[M, K] (+)= dy' . W^T with real-valued weights, dy' [M, N], on the digit x digit product: both operands are
@@ -117,7 +122,7 @@ int grad_input_planes(const float *dyp, const float *W, float *dx, int64_t M, in
   if (rc)
     return rc;
   return launch_gemm_digits(base + p.a_planes_off, base + p.b_planes_off, nullptr, dx, M, N, K, 1, K, 1, stream,
-                            accumulate);
+                            accumulate, base + p.split_off, p.split_bytes);
 }
 
 int check_args(int64_t M, int64_t K, int64_t N, void *workspace, size_t workspace_bytes, const BackwardPlan &p) {

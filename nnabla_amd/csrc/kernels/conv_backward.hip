@@ -234,8 +234,9 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
       rc = launch_split_digits_columns(col, g.Kg, base + p.b_planes_off, g.M, g.Kg, false, stream);
       if (rc)
         return rc;
+      // the unfolded fp32 matrix has been consumed: its buffer takes the partial results of a split contraction
       rc = launch_gemm_digits(base + p.a_planes_off, base + p.b_planes_off, nullptr, dW + grp * g.Og * g.Kg, g.Og, g.M,
-                              g.Kg, 1, g.Kg, 1, stream, accum_w);
+                              g.Kg, 1, g.Kg, 1, stream, accum_w, col, (size_t)g.M * g.Kg * sizeof(float));
       if (rc)
         return rc;
     }

@@ -29,6 +29,9 @@ struct GemmDigitsArgs {
   int64_t inner, outer_stride, n_stride;
   int accumulate; // add to y instead of overwriting it
   int finish;     // last chunk of the contraction: add the bias
+  // contraction split over blockIdx.y (outputs of few tiles): split z multiplies the k tiles
+  // [step_begin + z * split_tiles, + split_tiles) and writes its own dense [M, N] partial result at y + z * M * N
+  int64_t split_tiles; // 0: no split
 };
 
 constexpr int kBM = 128, kBN = 128, kThreads = 256, kWaves = 4;
@@ -285,17 +288,60 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
 template <int kStages, int kGroups>
 __global__ __launch_bounds__(kThreads * kGroups, kGroups == 1 ? 2 : 1) void gemm_digits_kernel(GemmDigitsArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  if (a.split_tiles > 0) {
+    const int64_t begin = a.step_begin + (int64_t)blockIdx.y * a.split_tiles;
+    a.step_end = begin + a.split_tiles < a.step_end ? begin + a.split_tiles : a.step_end;
+    a.step_begin = begin;
+    a.y += (int64_t)blockIdx.y * a.M * a.N;
+  }
   if (*a.bflag == 0) // uniform over the grid
     gemm_digits_tile<true, kStages, kGroups>(a, smem);
   else
     gemm_digits_tile<false, kStages, kGroups>(a, smem);
 }
 
+// y (+)= sum over the splits of their partial results, in split order, then the bias: what the single-launch epilogue
+// does with one value.
+__global__ __launch_bounds__(256) void gemm_digits_split_sum(const float *__restrict__ partial, int splits, int64_t M,
+                                                             int64_t N, float *__restrict__ y, int64_t inner,
+                                                             int64_t outer_stride, int64_t n_stride,
+                                                             const float *__restrict__ bias, int accumulate) {
+  const int64_t total = M * N;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t m = i / N, n = i - m * N;
+    float v = partial[i];
+    for (int z = 1; z < splits; ++z)
+      v += partial[(int64_t)z * total + i];
+    const int64_t q = m / inner;
+    float *dst = y + q * outer_stride + (m - q * inner) + n * n_stride;
+    if (accumulate)
+      v = *dst + v;
+    if (bias)
+      v = v + bias[n];
+    *dst = v;
+  }
+}
+
+// Splits of the contraction for an output of `tiles` 128 x 128 tiles and `k_tiles` k tiles: as many as fill the CUs
+// with one block each, at least 16 k tiles per split; 1 = no split.
+inline int64_t digit_product_splits(int64_t tiles, int64_t k_tiles) {
+  if (tiles * 2 > 256 || k_tiles < 32)
+    return 1;
+  const int64_t by_cus = 256 / tiles, by_k = k_tiles / 16;
+  return by_cus < by_k ? by_cus : by_k;
+}
+
 } // namespace
+
+size_t gemm_digits_split_bytes(int64_t M, int64_t K, int64_t N) {
+  const int64_t k_tiles = digit_k_tiles(K) < kChunkK / kTileK ? digit_k_tiles(K) : kChunkK / kTileK;
+  const int64_t s = digit_product_splits(ceil_div(M, kBM) * ceil_div(N, kBN), k_tiles);
+  return s > 1 ? (size_t)s * M * N * sizeof(float) : 0;
+}
 
 int launch_gemm_digits(const void *adigits, const void *bdigits, const float *bias, float *y, int64_t M, int64_t K,
                        int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride, hipStream_t stream,
-                       bool accumulate) {
+                       bool accumulate, void *split_ws, size_t split_ws_bytes) {
   if (M >= ((int64_t)1 << 31) || N >= ((int64_t)1 << 31))
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "digit product: more than 2^31 - 1 rows or columns.");
   const DigitOperand da = digit_operand(M, K), db = digit_operand(N, K);
@@ -336,9 +382,34 @@ int launch_gemm_digits(const void *adigits, const void *bdigits, const float *bi
     a.step_end = (t0 + tiles_per_chunk < a.k_tiles) ? t0 + tiles_per_chunk : a.k_tiles;
     a.accumulate = (accumulate || chunk > 0) ? 1 : 0;
     a.finish = a.step_end == a.k_tiles ? 1 : 0;
+    a.split_tiles = 0;
     const unsigned blocks = (unsigned)(a.blocks_m * a.blocks_n);
-    if (blocks <= 256 && (a.step_end - a.step_begin) % 2 == 0) // at most one block per CU: eight wavefronts, two k
-                                                               // groups (k tiles come in multiples of 8)
+    const int64_t chunk_tiles = a.step_end - a.step_begin;
+    int64_t splits = split_ws ? digit_product_splits(blocks, chunk_tiles) : 1;
+    while (splits > 1 && (size_t)splits * M * N * sizeof(float) > split_ws_bytes)
+      --splits;
+    if (splits > 1) {
+      // few output tiles, long contraction: every split writes a dense partial result, summed in split order
+      GemmDigitsArgs part = a;
+      part.split_tiles = ceil_div(ceil_div(chunk_tiles, splits), 8) * 8;
+      splits = ceil_div(chunk_tiles, part.split_tiles);
+      part.y = static_cast<float *>(split_ws);
+      part.inner = 1, part.outer_stride = N, part.n_stride = 1;
+      part.accumulate = 0, part.bias = nullptr;
+      hipLaunchKernelGGL((gemm_digits_kernel<kStagesShared, 2>), dim3(blocks, (unsigned)splits), dim3(2 * kThreads),
+                         kStagesShared * 2 * kStageBytes, stream, part);
+      NBLA_HIP_LAUNCH_CHECK("gemm_digits");
+      int64_t sum_blocks = ceil_div(M * N, 256);
+      if (sum_blocks > 4096)
+        sum_blocks = 4096;
+      hipLaunchKernelGGL(gemm_digits_split_sum, dim3((unsigned)sum_blocks), dim3(256), 0, stream,
+                         static_cast<const float *>(split_ws), (int)splits, M, N, y, inner, outer_stride, n_stride,
+                         a.finish ? bias : nullptr, a.accumulate);
+      NBLA_HIP_LAUNCH_CHECK("gemm_digits_split_sum");
+      continue;
+    }
+    if (blocks <= 256 && chunk_tiles % 2 == 0) // at most one block per CU: eight wavefronts, two k groups (k tiles
+                                               // come in multiples of 8)
       hipLaunchKernelGGL((gemm_digits_kernel<kStagesShared, 2>), dim3(blocks), dim3(2 * kThreads),
                          kStagesShared * 2 * kStageBytes, stream, a);
     else if (blocks <= 384) // fewer than 1.5 blocks per CU

@@ -34,9 +34,12 @@ int launch_split_digits_columns(const float *src, int64_t ld, void *digits, int6
                                 hipStream_t stream);
 // y[m, n] (+)= sum_k A[m, k] * B[n, k] (+ bias[n]), both factors real-valued digit operands (rows M x K and N x K);
 // A is a row-scaled operand, B a row- or column-scaled one whose flag word selects the six- or three-product form.
+// `split_ws` (may be null; gemm_digits_split_bytes(M, K, N) bytes make every split possible) lets an output of few
+// tiles with a long contraction spread the contraction over the CUs: dense partial results, summed in a fixed order.
 int launch_gemm_digits(const void *adigits, const void *bdigits, const float *bias, float *y, int64_t M, int64_t K,
                        int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride, hipStream_t stream,
-                       bool accumulate = false);
+                       bool accumulate = false, void *split_ws = nullptr, size_t split_ws_bytes = 0);
+size_t gemm_digits_split_bytes(int64_t M, int64_t K, int64_t N);
 
 // db[n] (+)= sum over m of dy[m, n]; `partial` holds ceil(M / 256) * N floats.
 size_t column_sums_workspace_bytes(int64_t M, int64_t N);
