@@ -312,6 +312,136 @@ __global__ __launch_bounds__(256) void im2col_digits(const float *__restrict__ x
       atomicAdd(reinterpret_cast<unsigned long long *>(sums + (chunk0 + h) * rows + m), (unsigned long long)row_sum[h]);
 }
 
+// ---- the unfolded matrix as the *transposed* digit operand (rows = unfolded columns kk = (channel, tap), contraction
+// over the output positions m of all samples): the second factor of the weight gradient dyt^T . col(x).
+//
+// One shift per channel: the largest |x| of the channel over all samples and positions bounds every unfolded column
+// of that channel (a scale only has to bound its row).  Block per channel.
+__global__ __launch_bounds__(256) void conv_channel_shift(const float *__restrict__ x, int32_t *__restrict__ shift,
+                                                          ConvGeom g, int64_t grp, int64_t rows) {
+  __shared__ uint32_t s_max[4];
+  const int64_t c = blockIdx.x;
+  const int taps = (int)g.k_size;
+  uint32_t amax = 0u;
+  for (int64_t n = 0; n < g.outer; ++n) {
+    const float *src = x + (n * g.C + grp * g.Cg + c) * g.in_sp_size;
+    for (int64_t p = threadIdx.x; p < g.in_sp_size; p += 256)
+      amax = max(amax, __float_as_uint(src[p]) & 0x7fffffffu);
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1)
+    amax = max(amax, (uint32_t)__shfl_xor((int)amax, off));
+  if ((threadIdx.x & 63) == 0)
+    s_max[threadIdx.x >> 6] = amax;
+  __syncthreads();
+  amax = max(max(s_max[0], s_max[1]), max(s_max[2], s_max[3]));
+  int s = 0;
+  if (amax >= 0x7f800000u) {
+    s = kBadRow;
+  } else if (amax != 0u) {
+    s = 22 - binade_exponent(binade_of(amax));
+    if (rintf(ldexpf(__uint_as_float(amax), s)) > (float)kDigitMax)
+      --s;
+  }
+  for (int t = threadIdx.x; t < taps; t += 256)
+    shift[c * taps + t] = s;
+  if (c == 0) { // padding rows of the operand and its flag word (1: all three digits are in use)
+    for (int64_t r = g.Kg + threadIdx.x; r < rows; r += 256)
+      shift[r] = 0;
+    if (threadIdx.x == 0)
+      shift[rows] = 1;
+  }
+}
+
+// A wavefront converts two k tiles (64 output positions m) of one row block (32 unfolded columns): lane l owns column
+// rb*32 + l%32 and the positions (l/32)*16 + 0..15 of each tile.  The 64 positions are decoded once, one per lane,
+// into a wavefront-private LDS table {sample base offset (64-bit), window origin per dimension}; the lane's own
+// column is decoded once into its tap displacements and channel offset.
+__global__ __launch_bounds__(256) void im2col_digits_columns(const float *__restrict__ x,
+                                                             const int32_t *__restrict__ shift,
+                                                             uint4_t *__restrict__ out, ConvGeom g, int64_t grp,
+                                                             int64_t k_tiles, int64_t tile_groups, int64_t jobs) {
+  typedef int i32x4_t __attribute__((ext_vector_type(4)));
+  __shared__ i32x4_t table[4][64];
+  __shared__ int table_b2[4][64];
+  const int64_t job = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (job >= jobs)
+    return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t rb = job / tile_groups, tg = job - rb * tile_groups;
+  const int in0 = g.in_sp[0], in1 = g.in_sp[1], in2 = g.in_sp[2], plane = (int)g.in_sp_size;
+  const int64_t kt_begin = tg * kTilesPerWave;
+  { // this lane's table entry: output position m = kt_begin * 32 + lane
+    const int64_t m = kt_begin * kTileK + lane;
+    const bool in = m < g.M;
+    const int64_t n = in ? m / g.out_sp_size : 0;
+    int p = in ? (int)(m - n * g.out_sp_size) : 0;
+    const int o2 = p % g.out_sp[2];
+    p /= g.out_sp[2];
+    const int o1 = p % g.out_sp[1];
+    const int o0 = p / g.out_sp[1];
+    const int b0 = o0 * g.stride[0] - g.pad[0], b1 = o1 * g.stride[1] - g.pad[1], b2 = o2 * g.stride[2] - g.pad[2];
+    const int64_t base = (n * g.C + grp * g.Cg) * g.in_sp_size + ((int64_t)b0 * in1 + b1) * in2 + b2;
+    i32x4_t e;
+    e.x = (int)(uint32_t)(uint64_t)base;
+    e.y = (int)(uint32_t)((uint64_t)base >> 32);
+    e.z = in ? b0 : -(1 << 30); // a position past the end fails every bound check
+    e.w = b1;
+    table[wave][lane] = e;
+    table_b2[wave][lane] = b2; // read back by this wavefront only: LDS operations of one wavefront complete in order
+  }
+  // this lane's column kk -> (channel, tap)
+  const int64_t kk = rb * kFragRows + (lane & 31);
+  const int s = shift[kk];
+  const bool row_ok = kk < g.Kg && s != kBadRow;
+  int q = row_ok ? (int)kk : 0;
+  const int t2 = q % g.k[2];
+  q /= g.k[2];
+  const int t1 = q % g.k[1];
+  q /= g.k[1];
+  const int t0 = q % g.k[0], c = q / g.k[0];
+  const int e0 = t0 * g.dil[0], e1 = t1 * g.dil[1], e2 = t2 * g.dil[2];
+  const int delta = c * plane + (e0 * in1 + e1) * in2 + e2; // offset of the tap relative to the window origin
+  for (int t = 0; t < kTilesPerWave; ++t) {
+    const int64_t kt = kt_begin + t;
+    if (kt >= k_tiles)
+      break;
+    float v[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int idx = t * kTileK + (lane >> 5) * 16 + j;
+      const i32x4_t e = table[wave][idx];
+      const int b2 = table_b2[wave][idx];
+      const int i0 = e.z + e0, i1 = e.w + e1, i2 = b2 + e2;
+      const bool ok = row_ok && (unsigned)i0 < (unsigned)in0 && (unsigned)i1 < (unsigned)in1 &&
+                      (unsigned)i2 < (unsigned)in2;
+      const int64_t base = (int64_t)(((uint64_t)(uint32_t)e.y << 32) | (uint32_t)e.x);
+      const float xv = x[ok ? base + delta : 0];
+      v[j] = ok ? xv : 0.0f;
+    }
+    uint32_t w[3][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int qv = to_fixed(v[j], s);
+      const int lo = (int)(int8_t)qv;
+      const int q1 = (qv - lo) >> 8;
+      const int mid = (int)(int8_t)q1;
+      const int hi = (q1 - mid) >> 8;
+      const int sh = 8 * (j & 3);
+      w[0][j >> 2] |= ((uint32_t)hi & 0xffu) << sh;
+      w[1][j >> 2] |= ((uint32_t)mid & 0xffu) << sh;
+      w[2][j >> 2] |= ((uint32_t)lo & 0xffu) << sh;
+    }
+    uint4_t *dst = out + ((rb * k_tiles + kt) * kDigits) * 64 + lane;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+      uint4_t o;
+      o.x = w[d][0], o.y = w[d][1], o.z = w[d][2], o.w = w[d][3];
+      dst[d * 64] = o;
+    }
+  }
+}
+
 // fp32 unfolded matrix [M, Kg] for the general (non bit-representable) path.
 __global__ __launch_bounds__(256) void im2col_f32(const float *__restrict__ x, float *__restrict__ col, ConvGeom g,
                                                   int64_t grp) {
@@ -359,6 +489,27 @@ int launch_im2col_digits(const float *x, void *xdigits, void *scratch, const Con
   hipLaunchKernelGGL(im2col_digits, dim3((unsigned)ceil_div(jobs, 4)), dim3(256), 0, stream, x, shift, sums,
                      reinterpret_cast<uint4_t *>(base), g, grp, d.k_tiles, tile_groups, d.rows, jobs);
   NBLA_HIP_LAUNCH_CHECK("im2col_digits");
+  return NBLA_HIP_OK;
+}
+
+// Digit operand of col(x)^T: rows = the Kg unfolded columns, contraction over the M output positions.
+int launch_im2col_digits_columns(const float *x, void *digits, const ConvGeom &g, int64_t grp, hipStream_t stream) {
+  bool fits = g.Cg * g.in_sp_size < ((int64_t)1 << 31) && g.out_sp_size < ((int64_t)1 << 31) &&
+              g.Kg < ((int64_t)1 << 31);
+  for (int i = 0; i < kMaxSpatial; ++i)
+    fits = fits && (int64_t)g.in_sp[i] + g.pad[i] + (int64_t)g.k[i] * g.dil[i] < ((int64_t)1 << 30);
+  if (!fits)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "convolution backward: a sample's channel group, its output map or a "
+                                              "padded input extent has 2^30 elements or more.");
+  const DigitOperand d = digit_operand(g.Kg, g.M);
+  char *base = static_cast<char *>(digits);
+  int32_t *shift = reinterpret_cast<int32_t *>(base + d.shift_off);
+  hipLaunchKernelGGL(conv_channel_shift, dim3((unsigned)g.Cg), dim3(256), 0, stream, x, shift, g, grp, d.rows);
+  NBLA_HIP_LAUNCH_CHECK("conv_channel_shift");
+  const int64_t tile_groups = ceil_div(d.k_tiles, kTilesPerWave), jobs = d.row_blocks * tile_groups;
+  hipLaunchKernelGGL(im2col_digits_columns, dim3((unsigned)ceil_div(jobs, 4)), dim3(256), 0, stream, x, shift,
+                     reinterpret_cast<uint4_t *>(base), g, grp, d.k_tiles, tile_groups, jobs);
+  NBLA_HIP_LAUNCH_CHECK("im2col_digits_columns");
   return NBLA_HIP_OK;
 }
 

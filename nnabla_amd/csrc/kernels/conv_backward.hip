@@ -224,17 +224,15 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
         return rc;
     }
     if (dW) {
-      rc = launch_im2col_f32(x, col, g, grp, stream);
-      if (rc)
-        return rc;
-      // digit operands of dyt^T (rows o) and col(x)^T (rows kk), contraction over the pixels m
+      // digit operands of dyt^T (rows o) and col(x)^T (rows kk, gathered straight from x), contraction over the
+      // pixels m
       rc = launch_split_digits_columns(dyt, g.Og, base + p.a_planes_off, g.M, g.Og, false, stream);
       if (rc)
         return rc;
-      rc = launch_split_digits_columns(col, g.Kg, base + p.b_planes_off, g.M, g.Kg, false, stream);
+      rc = launch_im2col_digits_columns(x, base + p.b_planes_off, g, grp, stream);
       if (rc)
         return rc;
-      // the unfolded fp32 matrix has been consumed: its buffer takes the partial results of a split contraction
+      // the buffer of the unfolded gradient is free here: it takes the partial results of a split contraction
       rc = launch_gemm_digits(base + p.a_planes_off, base + p.b_planes_off, nullptr, dW + grp * g.Og * g.Kg, g.Og, g.M,
                               g.Kg, 1, g.Kg, 1, stream, accum_w, col, (size_t)g.M * g.Kg * sizeof(float));
       if (rc)

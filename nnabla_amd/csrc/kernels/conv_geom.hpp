@@ -25,5 +25,8 @@ int launch_im2col_split(const float *x, void *xsplit, const ConvGeom &g, int64_t
 int launch_im2col_digits(const float *x, void *xdigits, void *scratch, const ConvGeom &g, int64_t grp,
                          hipStream_t stream);
 int launch_im2col_f32(const float *x, float *col, const ConvGeom &g, int64_t grp, hipStream_t stream);
+// col(x)^T (rows = unfolded columns, contraction over the output positions) as a digit operand with one scale per
+// input channel.
+int launch_im2col_digits_columns(const float *x, void *digits, const ConvGeom &g, int64_t grp, hipStream_t stream);
 
 } // namespace nbla_hip
