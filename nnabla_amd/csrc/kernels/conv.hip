@@ -323,10 +323,12 @@ __global__ __launch_bounds__(256) void conv_channel_shift(const float *__restric
   const int64_t c = blockIdx.x;
   const int taps = (int)g.k_size;
   uint32_t amax = 0u;
-  for (int64_t n = 0; n < g.outer; ++n) {
-    const float *src = x + (n * g.C + grp * g.Cg + c) * g.in_sp_size;
-    for (int64_t p = threadIdx.x; p < g.in_sp_size; p += 256)
-      amax = max(amax, __float_as_uint(src[p]) & 0x7fffffffu);
+  const float *src = x + (grp * g.Cg + c) * g.in_sp_size;
+  const int64_t total = g.outer * g.in_sp_size, sample_stride = g.C * g.in_sp_size;
+#pragma unroll 4
+  for (int64_t i = threadIdx.x; i < total; i += 256) { // (sample, position) pairs, independent loads
+    const int64_t n = i / g.in_sp_size;
+    amax = max(amax, __float_as_uint(src[n * sample_stride + (i - n * g.in_sp_size)]) & 0x7fffffffu);
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1)

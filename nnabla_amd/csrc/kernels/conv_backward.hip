@@ -41,41 +41,50 @@ __global__ __launch_bounds__(256) void gather_dy(const float *__restrict__ dy, c
 
 // dx element (n, c, position) (+)= sum of the unfolded gradient over the taps that read that position, in
 // ascending tap order (the order fold_from_patches.cpp:125-170 adds them in).  colg is [outer][Kg][L].
+// One thread per element of a sample's channel group; 32-bit arithmetic inside the sample (the host checks that it
+// fits); kUnitStride drops the divisions of the general case.
+template <bool kUnitStride>
 __global__ __launch_bounds__(256) void col2im_gather(const float *__restrict__ colg, float *__restrict__ dx, ConvGeom g,
                                                      int64_t grp, int accumulate) {
-  const int64_t total = g.outer * g.Cg * g.in_sp_size;
-  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
-    int64_t t = idx;
-    const int i2 = (int)(t % g.in_sp[2]);
-    t /= g.in_sp[2];
-    const int i1 = (int)(t % g.in_sp[1]);
-    t /= g.in_sp[1];
-    const int i0 = (int)(t % g.in_sp[0]);
-    t /= g.in_sp[0];
-    const int64_t cc = t % g.Cg, n = t / g.Cg;
-    const float *src = colg + (n * g.Kg + cc * g.k_size) * g.out_sp_size;
+  const int in0 = g.in_sp[0], in1 = g.in_sp[1], in2 = g.in_sp[2], plane = (int)g.in_sp_size, Cg = (int)g.Cg;
+  const int out0 = g.out_sp[0], out1 = g.out_sp[1], out2 = g.out_sp[2], L = (int)g.out_sp_size;
+  const int K0 = g.k[0], K1 = g.k[1], K2 = g.k[2], taps = (int)g.k_size;
+  const int s0 = g.stride[0], s1 = g.stride[1], s2 = g.stride[2];
+  const int per_sample = Cg * plane;
+  const int64_t n = blockIdx.y;
+  const float *sample = colg + n * g.Kg * g.out_sp_size;
+  float *dst_sample = dx + (n * g.C + grp * g.Cg) * g.in_sp_size;
+  for (int idx = blockIdx.x * 256 + threadIdx.x; idx < per_sample; idx += gridDim.x * 256) {
+    int t = idx;
+    const int i2 = t % in2;
+    t /= in2;
+    const int i1 = t % in1;
+    t /= in1;
+    const int i0 = t % in0;
+    const int cc = t / in0;
+    const float *src = sample + (int64_t)cc * taps * L;
     float acc = 0.0f;
-    for (int k0 = 0; k0 < g.k[0]; ++k0) {
+    for (int k0 = 0; k0 < K0; ++k0) {
       const int t0 = i0 + g.pad[0] - k0 * g.dil[0];
-      if (t0 < 0 || t0 % g.stride[0] != 0 || t0 / g.stride[0] >= g.out_sp[0])
+      const int q0 = kUnitStride ? t0 : t0 / s0;
+      if (t0 < 0 || (!kUnitStride && t0 - q0 * s0 != 0) || q0 >= out0)
         continue;
-      for (int k1 = 0; k1 < g.k[1]; ++k1) {
+      for (int k1 = 0; k1 < K1; ++k1) {
         const int t1 = i1 + g.pad[1] - k1 * g.dil[1];
-        if (t1 < 0 || t1 % g.stride[1] != 0 || t1 / g.stride[1] >= g.out_sp[1])
+        const int q1 = kUnitStride ? t1 : t1 / s1;
+        if (t1 < 0 || (!kUnitStride && t1 - q1 * s1 != 0) || q1 >= out1)
           continue;
-        for (int k2 = 0; k2 < g.k[2]; ++k2) {
+        for (int k2 = 0; k2 < K2; ++k2) {
           const int t2 = i2 + g.pad[2] - k2 * g.dil[2];
-          if (t2 < 0 || t2 % g.stride[2] != 0 || t2 / g.stride[2] >= g.out_sp[2])
+          const int q2 = kUnitStride ? t2 : t2 / s2;
+          if (t2 < 0 || (!kUnitStride && t2 - q2 * s2 != 0) || q2 >= out2)
             continue;
-          const int64_t tap = ((int64_t)k0 * g.k[1] + k1) * g.k[2] + k2;
-          const int64_t l = ((int64_t)(t0 / g.stride[0]) * g.out_sp[1] + t1 / g.stride[1]) * g.out_sp[2] +
-                            t2 / g.stride[2];
-          acc += src[tap * g.out_sp_size + l];
+          const int tap = (k0 * K1 + k1) * K2 + k2;
+          acc += src[(int64_t)tap * L + (q0 * out1 + q1) * out2 + q2];
         }
       }
     }
-    const int64_t pos = ((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2] + i2;
-    float *dst = dx + (n * g.C + grp * g.Cg + cc) * g.in_sp_size + pos;
+    float *dst = dst_sample + idx;
     *dst = accumulate ? *dst + acc : acc;
   }
 }
@@ -133,11 +142,18 @@ int launch_gather_dy(const float *dy, const float *scale, float *dyt, const Conv
 }
 
 int launch_col2im(const float *colg, float *dx, const ConvGeom &g, int64_t grp, bool accumulate, hipStream_t stream) {
-  int64_t blocks = ceil_div(g.outer * g.Cg * g.in_sp_size, 256);
-  if (blocks > 262144)
-    blocks = 262144;
-  hipLaunchKernelGGL(col2im_gather, dim3((unsigned)blocks), dim3(256), 0, stream, colg, dx, g, grp,
-                     accumulate ? 1 : 0);
+  if (g.Cg * g.in_sp_size >= ((int64_t)1 << 31) || g.k_size * g.out_sp_size >= ((int64_t)1 << 31) || g.outer > 65535)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "convolution backward: a sample's channel group or unfolded channel has "
+                                              "2^31 elements or more, or more than 65535 samples.");
+  int64_t bx = ceil_div(g.Cg * g.in_sp_size, 256);
+  if (bx > 65536)
+    bx = 65536;
+  const dim3 grid((unsigned)bx, (unsigned)g.outer);
+  const bool unit = g.stride[0] == 1 && g.stride[1] == 1 && g.stride[2] == 1;
+  if (unit)
+    hipLaunchKernelGGL(col2im_gather<true>, grid, dim3(256), 0, stream, colg, dx, g, grp, accumulate ? 1 : 0);
+  else
+    hipLaunchKernelGGL(col2im_gather<false>, grid, dim3(256), 0, stream, colg, dx, g, grp, accumulate ? 1 : 0);
   NBLA_HIP_LAUNCH_CHECK("col2im_gather");
   return NBLA_HIP_OK;
 }
