@@ -156,6 +156,12 @@ def bench_other_configs(dev, iters):
                                                            dx=gx, dW=gw, db=gb), iters)
     out["binary_connect_convolution_backward[32,256,14,14]x[256,256,3,3] dx+dW+db"] = {
         "ms": ms, "TFLOPs": 2 * flop / ms / 1e9}
+    # the same stage with real-valued weights (plain Convolution / INQConvolution's product)
+    Ic = torch.zeros(W.shape, dtype=torch.int32, device=dev)
+    Wc, oWc, oIc = W.clone(), W.clone(), Ic.clone()
+    ms = time_kernel(lambda: k.inq_convolution(x, Wc, Ic, oWc, oIc, None, (1, 1), (1, 1), (1, 1), 1, 4,
+                                               k.INQ_PRODUCT_ONLY), iters)
+    out["convolution[32,256,14,14]x[256,256,3,3] real weights"] = {"ms": ms, "TFLOPs": flop / ms / 1e9}
     M, K, N = 1024, 4096, 4096
     xa = torch.randn(M, K, generator=g).to(dev)
     Wq = (torch.randn(K, N, generator=g) * 0.02).to(dev)

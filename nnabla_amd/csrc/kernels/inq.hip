@@ -377,10 +377,11 @@ int update_weights(float *W, int *I, float *old_W, int *old_I, int64_t size, int
 }
 
 struct ProductWorkspace {
-  size_t update_off, split_off, planes_off, flag_off, total;
+  size_t update_off, split_off, planes_off, flag_off, extra_off, total;
 };
 
-ProductWorkspace plan_product(int64_t wsize, int64_t M, int64_t K, int64_t N, int step) {
+// `extra`: further scratch behind the operands (the convolution's channel maxima and split partial results)
+ProductWorkspace plan_product(int64_t wsize, int64_t M, int64_t K, int64_t N, int step, size_t extra = 0) {
   ProductWorkspace p;
   size_t off = 0;
   p.update_off = off;
@@ -394,8 +395,19 @@ ProductWorkspace plan_product(int64_t wsize, int64_t M, int64_t K, int64_t N, in
   off += round_up(wa > wb ? wa : wb, 256);
   p.flag_off = off;
   off += 256;
+  p.extra_off = off;
+  off += round_up(extra, 256);
   p.total = off;
   return p;
+}
+
+// scratch of the convolution product: the unfold's channel maxima (16 slices per input position), then the partial
+// results of a split contraction
+size_t conv_channel_max_bytes(const ConvGeom &g) {
+  return round_up((size_t)16 * g.outer * g.in_sp_size * sizeof(uint32_t), 256);
+}
+size_t conv_product_extra(const ConvGeom &g) {
+  return conv_channel_max_bytes(g) + gemm_digits_split_bytes(g.M, g.Kg, g.Og);
 }
 
 } // namespace
@@ -462,7 +474,7 @@ size_t nbla_hip_inq_convolution_workspace_bytes(int64_t outer, int64_t C, int nd
   ConvGeom g;
   if (make_geom(g, outer, C, nd, in_sp, O, kernel, pad, stride, dilation, group))
     return 0;
-  return plan_product(g.O * g.Kg, g.M, g.Kg, g.Og, step).total;
+  return plan_product(g.O * g.Kg, g.M, g.Kg, g.Og, step, conv_product_extra(g)).total;
 }
 
 int nbla_hip_inq_convolution_f32(const float *x, float *W, int32_t *I, float *old_W, int32_t *old_I, const float *bias,
@@ -475,7 +487,7 @@ int nbla_hip_inq_convolution_f32(const float *x, float *W, int32_t *I, float *ol
   int rc = make_geom(g, outer, C, nd, in_sp, O, kernel, pad, stride, dilation, group);
   if (rc)
     return rc;
-  const ProductWorkspace p = plan_product(g.O * g.Kg, g.M, g.Kg, g.Og, step);
+  const ProductWorkspace p = plan_product(g.O * g.Kg, g.M, g.Kg, g.Og, step, conv_product_extra(g));
   if (workspace_bytes < p.total || !aligned256(workspace))
     return fail(NBLA_HIP_ERR_MEMORY, "INQ convolution workspace too small (%zu < %zu) or misaligned.", workspace_bytes,
                 p.total);
@@ -491,17 +503,20 @@ int nbla_hip_inq_convolution_f32(const float *x, float *W, int32_t *I, float *ol
     if (rc)
       return rc;
   }
-  int *flag = reinterpret_cast<int *>(base + p.flag_off);
+  // The product runs on the int8 digit kernels: the unfolded input goes straight into a row-scaled digit operand
+  // (rows = output positions), the weights [Og, Kg] into another (rows = output channels); six exact digit products.
   const int64_t hw = g.out_sp_size;
+  const size_t cmax_bytes = conv_channel_max_bytes(g);
   for (int64_t grp = 0; grp < g.group; ++grp) {
-    rc = launch_im2col_split(x, base + p.split_off, g, grp, stream);
+    rc = launch_im2col_digits(x, base + p.split_off, base + p.extra_off, g, grp, stream);
     if (rc)
       return rc;
-    rc = launch_split_weights(W + grp * g.Og * g.Kg, base + p.planes_off, flag, g.Kg, g.Og, true, stream);
+    rc = nbla_hip_split_digits_f32(W + grp * g.Og * g.Kg, g.Kg, base + p.planes_off, g.Og, g.Kg, stream_);
     if (rc)
       return rc;
-    rc = launch_gemm_planes(base + p.split_off, base + p.planes_off, flag, nullptr, bias ? bias + grp * g.Og : nullptr,
-                            y + grp * g.Og * hw, g.M, g.Kg, g.Og, hw, g.O * hw, hw, stream);
+    rc = launch_gemm_digits(base + p.split_off, base + p.planes_off, bias ? bias + grp * g.Og : nullptr,
+                            y + grp * g.Og * hw, g.M, g.Kg, g.Og, hw, g.O * hw, hw, stream, false,
+                            base + p.extra_off + cmax_bytes, gemm_digits_split_bytes(g.M, g.Kg, g.Og));
     if (rc)
       return rc;
   }
