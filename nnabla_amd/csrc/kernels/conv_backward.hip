@@ -108,13 +108,9 @@ ConvBackwardPlan plan_conv_backward(const ConvGeom &g) {
   p.col_off = off; // unfolded input [M, Kg], and the unfolded gradient [outer][Kg][L]
   off += round_up((size_t)g.M * g.Kg * sizeof(float), 256);
   p.a_planes_off = off; // dyt^T for dW (rows o, contraction m) or dyt for dx (rows m, contraction o)
-  off += round_up(larger(larger(nbla_hip_split_operand_bytes(g.Og, g.M), nbla_hip_split_operand_bytes(g.M, g.Og)),
-                         nbla_hip_digit_operand_bytes(g.Og, g.M)),
-                  256);
+  off += round_up(larger(nbla_hip_digit_operand_bytes(g.M, g.Og), nbla_hip_digit_operand_bytes(g.Og, g.M)), 256);
   p.b_planes_off = off; // col(x) (columns kk, contraction m) or w (columns kk, contraction o)
-  off += round_up(larger(larger(nbla_hip_split_operand_bytes(g.Kg, g.M), nbla_hip_split_operand_bytes(g.Kg, g.Og)),
-                         nbla_hip_digit_operand_bytes(g.Kg, g.M)),
-                  256);
+  off += round_up(larger(nbla_hip_digit_operand_bytes(g.Kg, g.M), nbla_hip_digit_operand_bytes(g.Kg, g.Og)), 256);
   p.digits_off = off;
   off += round_up(nbla_hip_digit_operand_bytes(g.M, g.Og), 256);
   p.bits_off = off;
@@ -174,7 +170,6 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
   float *dyt = reinterpret_cast<float *>(base + p.dyt_off);
   float *scaled = reinterpret_cast<float *>(base + p.scaled_off);
   float *col = reinterpret_cast<float *>(base + p.col_off);
-  int *flag = reinterpret_cast<int *>(base + p.flag_off);
   int *count = reinterpret_cast<int *>(base + p.count_off);
   uint32_t *bits = reinterpret_cast<uint32_t *>(base + p.bits_off);
   const bool representable = (zero_to == 1.0f || zero_to == -1.0f);
@@ -224,14 +219,16 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
             dsrc = scaled;
           }
         }
-        rc = nbla_hip_split_bf16x3_f32(dsrc, g.Og, base + p.a_planes_off, g.M, g.Og, stream_);
+        // real x real on the digit product: dyt rows m (row-scaled), the weights' columns kk (column-scaled; signs and
+        // zeros take the one-digit form), contraction over the output channels o
+        rc = nbla_hip_split_digits_f32(dsrc, g.Og, base + p.a_planes_off, g.M, g.Og, stream_);
         if (rc)
           return rc;
-        rc = launch_split_weights(wsrc, base + p.b_planes_off, flag, g.Og, g.Kg, false, stream);
+        rc = launch_split_digits_columns(wsrc, g.Kg, base + p.b_planes_off, g.Og, g.Kg, binary, stream);
         if (rc)
           return rc;
-        rc = launch_gemm_planes(base + p.a_planes_off, base + p.b_planes_off, flag, nullptr, nullptr, col, g.M, g.Og,
-                                g.Kg, L, g.Kg * L, L, stream);
+        rc = launch_gemm_digits(base + p.a_planes_off, base + p.b_planes_off, nullptr, col, g.M, g.Og, g.Kg, L,
+                                g.Kg * L, L, stream);
       }
       if (rc)
         return rc;
