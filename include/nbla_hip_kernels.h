@@ -150,9 +150,6 @@ int nbla_hip_min_max_quantize_backward_f32(
 /* Bytes of the 1-bit packed GEMM operand for a [K, N] weight matrix (K padded
  * to 32, N to 256). */
 size_t nbla_hip_packed_bits_bytes(int64_t K, int64_t N);
-/* Bytes of the bf16x3-split, fragment-ordered GEMM operand for x [M, K]
- * (the operand of the plane x plane product used by the INQ forwards). */
-size_t nbla_hip_split_operand_bytes(int64_t M, int64_t K);
 /* Bytes of the int8 digit operand for x [M, K] (the operand of the bit-weight
  * product): fragment-ordered digits, per-row sums and per-row shifts. */
 size_t nbla_hip_digit_operand_bytes(int64_t M, int64_t K);
@@ -179,11 +176,6 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha,
                                   int transposed, float quantize_zero_to,
                                   int *zero_count, void *workspace,
                                   size_t workspace_bytes, void *stream);
-
-/* Split x [M, K] (row stride ldx elements) into three bf16 planes
- * (x == hi + mid + lo exactly) stored in MFMA fragment order. */
-int nbla_hip_split_bf16x3_f32(const float *x, int64_t ldx, void *xsplit,
-                              int64_t M, int64_t K, void *stream);
 
 /* Turn x [M, K] (row stride ldx elements) into the int8 digit operand: per
  * row a power-of-two scale 2^s such that q = rint(x * 2^s) fits 24 bits for
@@ -336,8 +328,8 @@ int nbla_hip_binary_connect_convolution_f32(
     const int64_t *dilation, int64_t group, float quantize_zero_to,
     void *workspace, size_t workspace_bytes, void *stream);
 
-/* Convolution with real-valued weights, y = conv(x, W) + bias on the bf16-plane
- * product (three planes per operand, fp32 accumulate).  Replaces
+/* Convolution with real-valued weights, y = conv(x, W) + bias on the int8 digit
+ * product (three digits per operand, exact int32 accumulation).  Replaces
  * Convolution<float>::forward_impl, convolution.cpp:161-197. */
 size_t nbla_hip_convolution_workspace_bytes(
     int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
@@ -476,8 +468,8 @@ int nbla_hip_inq_update_weights_f32(float *W, int32_t *I, float *old_W,
 size_t nbla_hip_inq_affine_workspace_bytes(int64_t M, int64_t K, int64_t N,
                                            int step);
 
-/* INQAffine forward: the weight update above, then y = x . W + bias with fp32
- * accumulation of exact bf16-plane products.  Replaces
+/* INQAffine forward: the weight update above, then y = x . W + bias on the int8
+ * digit product (exact int32 accumulation of digit products).  Replaces
  * INQAffine<float,int>::forward_impl, inq_affine.cpp:82-205. */
 int nbla_hip_inq_affine_f32(const float *x, float *W, int32_t *I, float *old_W,
                             int32_t *old_I, const float *bias, float *y,

@@ -53,8 +53,6 @@ __global__ __launch_bounds__(256) void scale_columns(const float *__restrict__ d
     out[i] = dy[i] * alpha[i % N];
 }
 
-size_t max3(size_t a, size_t b, size_t c) { return a > b ? (a > c ? a : c) : (b > c ? b : c); }
-
 struct BackwardPlan {
   size_t bits_off, digits_off, prep_off, count_off, a_planes_off, b_planes_off, flag_off, sums_off, scaled_off, split_off,
       split_bytes, total;
@@ -72,17 +70,13 @@ BackwardPlan plan_backward(int64_t M, int64_t K, int64_t N) {
   off += round_up(nbla_hip_binarize_workspace_bytes(N, K), 256);
   p.count_off = off;
   off += 256;
-  // bf16 planes: the larger of (x^T, dy) for dW and (dy, W^T) for dx
-  const size_t a1 = nbla_hip_split_operand_bytes(K, M), b1 = nbla_hip_split_operand_bytes(N, M);
-  const size_t a2 = nbla_hip_split_operand_bytes(M, N), b2 = nbla_hip_split_operand_bytes(K, N);
-  // ... and the digit operands of x^T and dy^T for dW share the same two regions
+  // digit operands of x^T and dy^T for dW, and of dy and W for the real-weight dx, share two regions
   const size_t a3 = nbla_hip_digit_operand_bytes(K, M), b3 = nbla_hip_digit_operand_bytes(N, M);
-  // ... and those of dy and W for the real-weight dx
   const size_t a4 = nbla_hip_digit_operand_bytes(M, N), b4 = nbla_hip_digit_operand_bytes(K, N);
   p.a_planes_off = off;
-  off += round_up(max3(max3(a1, a2, a3), a4, 0), 256);
+  off += round_up(a3 > a4 ? a3 : a4, 256);
   p.b_planes_off = off;
-  off += round_up(max3(max3(b1, b2, b3), b4, 0), 256);
+  off += round_up(b3 > b4 ? b3 : b4, 256);
   p.flag_off = off;
   off += 256;
   p.sums_off = off;

@@ -1,6 +1,6 @@
 // Operand preparation for the binary-weight products: one pass over W that
 // writes Sign(W), the 1-bit packed MFMA operand and the |W| column sums, and the
-// bf16x3 split of the activations.
+// int8 digit operands of the activations.
 #include "common.hpp"
 #include "gemm_layout.hpp"
 #include "internal.hpp"
@@ -407,108 +407,6 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_finalize(const float *__r
     __syncthreads();
     if (threadIdx.x == 0)
       *zero_count = s_z[0] + s_z[1] + s_z[2] + s_z[3];
-  }
-}
-
-// ------------------------------------------------------------------ bf16 split
-__device__ __forceinline__ uint32_t bf16_rne(float v) { // finite v
-  const uint32_t u = __float_as_uint(v);
-  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-}
-__device__ __forceinline__ float bf16_to_float(uint32_t h) { return __uint_as_float(h << 16); }
-
-// x == hi + mid + lo with each part a bf16: the residuals are exact in fp32.
-// Non-finite x keeps its class in `hi` alone.
-__device__ __forceinline__ void split3(float x, uint32_t &hi, uint32_t &mid, uint32_t &lo) {
-  const uint32_t u = __float_as_uint(x);
-  if ((u & 0x7f800000u) == 0x7f800000u) {
-    hi = (u >> 16) | ((u & 0xffffu) ? 0x40u : 0u);
-    mid = lo = 0u;
-    return;
-  }
-  hi = bf16_rne(x);
-  if ((hi & 0x7f80u) == 0x7f80u)
-    hi = u >> 16; // rounding up would overflow to infinity: truncate instead
-  const float r1 = x - bf16_to_float(hi);
-  mid = bf16_rne(r1);
-  const float r2 = r1 - bf16_to_float(mid);
-  lo = bf16_rne(r2);
-}
-
-// One wavefront per (row block, k block) fragment; lane l converts the eight
-// values x[rb*32 + l%32][kb*16 + (l/32)*8 + 0..7].
-__global__ __launch_bounds__(kPrepBlock) void split_bf16x3(const float *__restrict__ x, int64_t ldx, uint4_t *__restrict__ out,
-                                                           int64_t M, int64_t K, int64_t k_blocks, int64_t frags) {
-  const int64_t frag = (int64_t)blockIdx.x * (kPrepBlock / 64) + (threadIdx.x >> 6);
-  if (frag >= frags)
-    return;
-  const int lane = threadIdx.x & 63;
-  const int64_t rb = frag / k_blocks, kb = frag - rb * k_blocks;
-  const int64_t m = rb * kFragRows + (lane & 31);
-  const int64_t k0 = kb * kFragK + (lane >> 5) * 8;
-  float v[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e)
-    v[e] = (m < M && k0 + e < K) ? x[m * ldx + k0 + e] : 0.0f;
-  uint32_t h[8], mi[8], l[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e)
-    split3(v[e], h[e], mi[e], l[e]);
-  uint4_t o;
-  uint4_t *dst = out + frag * 3 * 64 + lane;
-  o.x = h[0] | (h[1] << 16), o.y = h[2] | (h[3] << 16), o.z = h[4] | (h[5] << 16), o.w = h[6] | (h[7] << 16);
-  dst[0] = o;
-  o.x = mi[0] | (mi[1] << 16), o.y = mi[2] | (mi[3] << 16), o.z = mi[4] | (mi[5] << 16), o.w = mi[6] | (mi[7] << 16);
-  dst[64] = o;
-  o.x = l[0] | (l[1] << 16), o.y = l[2] | (l[3] << 16), o.z = l[4] | (l[5] << 16), o.w = l[6] | (l[7] << 16);
-  dst[128] = o;
-}
-
-// Streaming variant for K % 64 == 0, 16-byte aligned rows: a wavefront converts a 32-row x 64-k patch (four
-// fragments).  Global loads are fully coalesced (16 lanes read 256 contiguous bytes of a row); the patch is turned
-// into fragment order through a padded LDS tile.
-__global__ __launch_bounds__(kPrepBlock) void split_bf16x3_tiled(const float *__restrict__ x, int64_t ldx,
-                                                                 uint4_t *__restrict__ out, int64_t M, int64_t K,
-                                                                 int64_t k_blocks, int64_t patches) {
-  constexpr int kRowStride = 68; // floats: 64 + 4 padding keeps the 128-bit column reads conflict-free
-  __shared__ float tile[kPrepBlock / 64][32 * kRowStride];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int64_t patch = (int64_t)blockIdx.x * (kPrepBlock / 64) + wave;
-  if (patch >= patches)
-    return;
-  const int64_t patches_per_row = k_blocks / 4;
-  const int64_t rb = patch / patches_per_row, kq = patch - rb * patches_per_row;
-  float *t = tile[wave];
-  const int lr = lane >> 4, lc = (lane & 15) * 4;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int row = j * 4 + lr;
-    const int64_t m = rb * kFragRows + row;
-    float4_t v = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (m < M)
-      v = *reinterpret_cast<const float4_t *>(x + m * ldx + kq * 64 + lc);
-    *reinterpret_cast<float4_t *>(t + row * kRowStride + lc) = v;
-  }
-  // the tile is private to this wavefront: LDS operations of one wavefront complete in order
-  __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
-  const int r = lane & 31, g = lane >> 5;
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const float4_t a = *reinterpret_cast<const float4_t *>(t + r * kRowStride + q * 16 + g * 8);
-    const float4_t b = *reinterpret_cast<const float4_t *>(t + r * kRowStride + q * 16 + g * 8 + 4);
-    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-    uint32_t h[8], mi[8], l[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e)
-      split3(v[e], h[e], mi[e], l[e]);
-    uint4_t o;
-    uint4_t *dst = out + ((rb * k_blocks + kq * 4 + q) * 3) * 64 + lane;
-    o.x = h[0] | (h[1] << 16), o.y = h[2] | (h[3] << 16), o.z = h[4] | (h[5] << 16), o.w = h[6] | (h[7] << 16);
-    __builtin_nontemporal_store(o, dst);
-    o.x = mi[0] | (mi[1] << 16), o.y = mi[2] | (mi[3] << 16), o.z = mi[4] | (mi[5] << 16), o.w = mi[6] | (mi[7] << 16);
-    __builtin_nontemporal_store(o, dst + 64);
-    o.x = l[0] | (l[1] << 16), o.y = l[2] | (l[3] << 16), o.z = l[4] | (l[5] << 16), o.w = l[6] | (l[7] << 16);
-    __builtin_nontemporal_store(o, dst + 128);
   }
 }
 
@@ -1020,10 +918,6 @@ size_t nbla_hip_packed_bits_bytes(int64_t K, int64_t N) {
   return (size_t)bits_packed_k_tiles(K) * bits_wide_groups(N) * 64 * 4 * sizeof(uint32_t);
 }
 
-size_t nbla_hip_split_operand_bytes(int64_t M, int64_t K) {
-  return (size_t)split_row_blocks(M) * split_k_blocks(K) * 3 * kFragBytes;
-}
-
 size_t nbla_hip_digit_operand_bytes(int64_t M, int64_t K) { return digit_operand(M, K).total; }
 
 size_t nbla_hip_binarize_workspace_bytes(int64_t K, int64_t N) {
@@ -1081,29 +975,6 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint3
                        reinterpret_cast<uint4_t *>(bits), P.k_tiles, P.col_groups, wide_groups, total);
     NBLA_HIP_LAUNCH_CHECK("binarize_finalize");
   }
-  return NBLA_HIP_OK;
-}
-
-int nbla_hip_split_bf16x3_f32(const float *x, int64_t ldx, void *xsplit, int64_t M, int64_t K, void *stream_) {
-  if (M <= 0 || K <= 0 || ldx < K)
-    return fail(NBLA_HIP_ERR_VALUE, "invalid split operand shape (M=%lld, K=%lld, ldx=%lld).", (long long)M,
-                (long long)K, (long long)ldx);
-  if (!aligned16(xsplit))
-    return fail(NBLA_HIP_ERR_MEMORY, "split operand buffer must be 16-byte aligned.");
-  int rc = ensure_init();
-  if (rc)
-    return rc;
-  const int64_t k_blocks = split_k_blocks(K);
-  const int64_t frags = split_row_blocks(M) * k_blocks;
-  if (K % 64 == 0 && ldx % 4 == 0 && aligned16(x)) {
-    const int64_t patches = frags / 4;
-    hipLaunchKernelGGL(split_bf16x3_tiled, dim3((unsigned)ceil_div(patches, kPrepBlock / 64)), dim3(kPrepBlock), 0,
-                       as_stream(stream_), x, ldx, static_cast<uint4_t *>(xsplit), M, K, k_blocks, patches);
-  } else {
-    hipLaunchKernelGGL(split_bf16x3, dim3((unsigned)ceil_div(frags, kPrepBlock / 64)), dim3(kPrepBlock), 0,
-                       as_stream(stream_), x, ldx, static_cast<uint4_t *>(xsplit), M, K, k_blocks, frags);
-  }
-  NBLA_HIP_LAUNCH_CHECK("split_bf16x3");
   return NBLA_HIP_OK;
 }
 

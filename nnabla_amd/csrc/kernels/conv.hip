@@ -93,53 +93,6 @@ __device__ __forceinline__ float col_value(const float *__restrict__ x, const Co
   return x[(n * g.C + c) * g.in_sp_size + ((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2] + i2];
 }
 
-__device__ __forceinline__ uint32_t bf16_rne(float v) {
-  const uint32_t u = __float_as_uint(v);
-  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-}
-
-__device__ __forceinline__ void split3(float x, uint32_t &hi, uint32_t &mid, uint32_t &lo) {
-  const uint32_t u = __float_as_uint(x);
-  if ((u & 0x7f800000u) == 0x7f800000u) {
-    hi = (u >> 16) | ((u & 0xffffu) ? 0x40u : 0u);
-    mid = lo = 0u;
-    return;
-  }
-  hi = bf16_rne(x);
-  if ((hi & 0x7f80u) == 0x7f80u)
-    hi = u >> 16;
-  const float r1 = x - __uint_as_float(hi << 16);
-  mid = bf16_rne(r1);
-  const float r2 = r1 - __uint_as_float(mid << 16);
-  lo = bf16_rne(r2);
-}
-
-// One wavefront per (row block, k block) fragment of the split operand.
-__global__ __launch_bounds__(256) void im2col_split(const float *__restrict__ x, uint4_t *__restrict__ out, ConvGeom g,
-                                                    int64_t grp, int64_t k_blocks, int64_t frags) {
-  const int64_t frag = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (frag >= frags)
-    return;
-  const int lane = threadIdx.x & 63;
-  const int64_t rb = frag / k_blocks, kb = frag - rb * k_blocks;
-  const int64_t m = rb * kFragRows + (lane & 31);
-  const int64_t k0 = kb * kFragK + (lane >> 5) * 8;
-  uint32_t h[8], mi[8], l[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const float v = (m < g.M && k0 + e < g.Kg) ? col_value(x, g, grp, m, k0 + e) : 0.0f;
-    split3(v, h[e], mi[e], l[e]);
-  }
-  uint4_t o;
-  uint4_t *dst = out + frag * 3 * 64 + lane;
-  o.x = h[0] | (h[1] << 16), o.y = h[2] | (h[3] << 16), o.z = h[4] | (h[5] << 16), o.w = h[6] | (h[7] << 16);
-  dst[0] = o;
-  o.x = mi[0] | (mi[1] << 16), o.y = mi[2] | (mi[3] << 16), o.z = mi[4] | (mi[5] << 16), o.w = mi[6] | (mi[7] << 16);
-  dst[64] = o;
-  o.x = l[0] | (l[1] << 16), o.y = l[2] | (l[3] << 16), o.z = l[4] | (l[5] << 16), o.w = l[6] | (l[7] << 16);
-  dst[128] = o;
-}
-
 // ---- digit operand of the unfolded matrix (the int8 bit-weight product)
 __device__ __forceinline__ int to_fixed(float v, int s) { return (int)rintf(ldexpf(v, s)); }
 
@@ -455,15 +408,6 @@ __global__ __launch_bounds__(256) void im2col_f32(const float *__restrict__ x, f
 }
 
 } // namespace
-
-int launch_im2col_split(const float *x, void *xsplit, const ConvGeom &g, int64_t grp, hipStream_t stream) {
-  const int64_t k_blocks = split_k_blocks(g.Kg);
-  const int64_t frags = split_row_blocks(g.M) * k_blocks;
-  hipLaunchKernelGGL(im2col_split, dim3((unsigned)ceil_div(frags, 4)), dim3(256), 0, stream, x,
-                     static_cast<uint4_t *>(xsplit), g, grp, k_blocks, frags);
-  NBLA_HIP_LAUNCH_CHECK("im2col_split");
-  return NBLA_HIP_OK;
-}
 
 // `scratch` holds kChannelSlices * outer * in_sp_size uint32 (the channel maxima).
 int launch_im2col_digits(const float *x, void *xdigits, void *scratch, const ConvGeom &g, int64_t grp,

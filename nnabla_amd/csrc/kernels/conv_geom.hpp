@@ -20,8 +20,7 @@ struct ConvGeom {
 int make_geom(ConvGeom &g, int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O, const int64_t *kernel,
               const int64_t *pad, const int64_t *stride, const int64_t *dil, int64_t group);
 
-// Unfolded activations of group `grp`, as the bf16x3 split MFMA operand [M, Kg] or as plain fp32 [M, Kg].
-int launch_im2col_split(const float *x, void *xsplit, const ConvGeom &g, int64_t grp, hipStream_t stream);
+// Unfolded activations of group `grp`, as the int8 digit MFMA operand [M, Kg] or as plain fp32 [M, Kg].
 int launch_im2col_digits(const float *x, void *xdigits, void *scratch, const ConvGeom &g, int64_t grp,
                          hipStream_t stream);
 int launch_im2col_f32(const float *x, float *col, const ConvGeom &g, int64_t grp, hipStream_t stream);

@@ -1,7 +1,6 @@
 // General fp32 product y = (x . w) * colscale + bias on v_mfma_f32_32x32x2_f32:
-// the path for weights that are not representable as +-1 bits or bf16 planes
-// (plain Affine, BinaryWeight* with an arbitrary quantize_zero_to and exact zero
-// weights, INQ with learnable weights left).  LDS-tiled 128x128x16, four
+// the fallback for binary layers whose Sign(W) is not representable as +-1 bits (an arbitrary quantize_zero_to
+// with exact zero weights) and the reference product of nbla_hip_affine_f32.  LDS-tiled 128x128x16, four
 // wavefronts each owning a 64x64 corner.
 #include "common.hpp"
 #include "gemm_layout.hpp"

@@ -1,23 +1,9 @@
-// Operand layouts shared by the kernels that produce GEMM operands (sign
-// binarisation, bf16x3 split, im2col, INQ) and the MFMA kernels that consume
-// them.
+// Operand layouts shared by the kernels that produce GEMM operands (sign binarisation, digit split, im2col, INQ) and
+// the MFMA kernels that consume them.
 //
-// The contraction is y[m, n] = sum_k A[m, k] * B[k, n] on
-// v_mfma_f32_32x32x16_bf16.  One MFMA operand fragment covers 32 rows (m for
-// A, n for B) by 16 k; lane l of the wavefront holds row (l % 32) and the eight
-// k values (l / 32) * 8 + 0..7, i.e. 16 bytes of bf16.
-//
-// A ("split operand"): an fp32 matrix is stored as three bf16 planes
-// hi/mid/lo with x == hi + mid + lo exactly, already in fragment order:
-//     A'[row_block = m / 32][k_block = k / 16][plane][lane][8 x bf16]
-// so a fragment is 1 KiB of consecutive bytes, read by lane l at offset 16 * l.
-// Rows >= M and columns >= K are zero.  K is padded to a multiple of 32 (two
-// k blocks: one kernel k-step), M to a multiple of 32.
-//
-// (This operand feeds the plane x plane product used where both factors are real numbers.)
-//
-// The bit-weight product runs on v_mfma_i32_32x32x32_i8 instead.  One i8 operand fragment covers 32 rows by 32 k;
-// lane l holds row (l % 32) and sixteen bytes, byte j being k-slot (l / 32) * 16 + j of the k tile.
+// The contraction is y[m, n] = sum_k A[m, k] * B[k, n] on v_mfma_i32_32x32x32_i8.  One i8 operand fragment covers
+// 32 rows (m for A, n for B) by 32 k; lane l holds row (l % 32) and sixteen bytes, byte j being k-slot
+// (l / 32) * 16 + j of the k tile: a fragment is 1 KiB of consecutive bytes, read by lane l at offset 16 * l.
 //
 // X ("digit operand"): row m of an fp32 matrix is turned into integers q = rint(x * 2^s_m), |q| < 2^23, with one
 // power-of-two scale per row (s_m the largest shift that keeps the row's largest magnitude inside the digit range),
@@ -49,15 +35,13 @@
 namespace nbla_hip {
 
 constexpr int kFragRows = 32;   // rows per MFMA fragment
-constexpr int kFragK = 16;      // k per MFMA fragment
-constexpr int kTileK = 32;      // k per kernel step (two fragments)
+constexpr int kTileK = 32;      // k per i8 MFMA fragment and k tile
 constexpr int kColGroup = 64;   // columns per pair-word group
 constexpr int kFragBytes = 1024;
 
 __host__ __device__ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 __host__ __device__ inline int64_t split_row_blocks(int64_t M) { return ceil_div(M, kFragRows); }
-__host__ __device__ inline int64_t split_k_blocks(int64_t K) { return ceil_div(K, kTileK) * 2; }
 __host__ __device__ inline int64_t bits_k_tiles(int64_t K) { return ceil_div(K, kTileK); }
 __host__ __device__ inline int64_t bits_col_groups(int64_t N) { return ceil_div(N, kColGroup); }
 

@@ -386,13 +386,11 @@ ProductWorkspace plan_product(int64_t wsize, int64_t M, int64_t K, int64_t N, in
   size_t off = 0;
   p.update_off = off;
   off += round_up(plan_inq(wsize, step == 2 ? 1 : (step == 3 ? 2 : 0)).total, 256);
-  // activations and weights as bf16 planes (convolution) or as digit operands (affine)
-  const size_t xa = nbla_hip_split_operand_bytes(M, K), xb = nbla_hip_digit_operand_bytes(M, K);
-  const size_t wa = nbla_hip_split_operand_bytes(N, K), wb = nbla_hip_digit_operand_bytes(N, K);
+  // activations and weights as digit operands
   p.split_off = off;
-  off += round_up(xa > xb ? xa : xb, 256);
+  off += round_up(nbla_hip_digit_operand_bytes(M, K), 256);
   p.planes_off = off;
-  off += round_up(wa > wb ? wa : wb, 256);
+  off += round_up(nbla_hip_digit_operand_bytes(N, K), 256);
   p.flag_off = off;
   off += 256;
   p.extra_off = off;

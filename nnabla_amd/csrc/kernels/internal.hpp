@@ -18,15 +18,6 @@ int launch_gemm_bits(const void *xsplit, const uint32_t *bits, const float *alph
                      int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
                      bool swap_out, hipStream_t stream, bool accumulate = false);
 
-// Weight matrix w ([K, N], or [N, K] when transposed) as bf16x3 planes in fragment order; *need_low is set to
-// non-zero when some weight is not exactly a bf16 value (the product then needs the cross terms).
-int launch_split_weights(const float *w, void *planes, int *need_low, int64_t K, int64_t N, bool transposed,
-                         hipStream_t stream);
-// y = (x . w) * colscale + bias with both operands as bf16x3 planes.
-int launch_gemm_planes(const void *xsplit, const void *wplanes, const int *need_low, const float *colscale,
-                       const float *bias, float *y, int64_t M, int64_t K, int64_t N, int64_t inner,
-                       int64_t outer_stride, int64_t n_stride, hipStream_t stream, bool accumulate = false);
-
 // Digit operand whose rows are the C columns of src [R, C] (row stride ld), contraction over src's rows.  With
 // detect_narrow the operand comes out in its one-digit form when every element is zero or a power of two within six
 // binades of its column's largest (its flag word tells the product which form it got).

@@ -24,8 +24,8 @@ EXPORTED = (
     "nbla_hip_min_max_quantize_workspace_bytes", "nbla_hip_min_max_quantize_f32",
     "nbla_hip_fixed_point_quantize_backward_f32", "nbla_hip_pow2_quantize_backward_f32",
     "nbla_hip_min_max_quantize_backward_workspace_bytes", "nbla_hip_min_max_quantize_backward_f32",
-    "nbla_hip_packed_bits_bytes", "nbla_hip_split_operand_bytes", "nbla_hip_digit_operand_bytes",
-    "nbla_hip_binarize_workspace_bytes", "nbla_hip_binarize_weights_f32", "nbla_hip_split_bf16x3_f32",
+    "nbla_hip_packed_bits_bytes", "nbla_hip_digit_operand_bytes",
+    "nbla_hip_binarize_workspace_bytes", "nbla_hip_binarize_weights_f32",
     "nbla_hip_split_digits_f32", "nbla_hip_gemm_bits_f32",
     "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_weight_affine_f32",
     "nbla_hip_binary_connect_affine_f32", "nbla_hip_affine_f32", "nbla_hip_split_digits_scaled_f32",
@@ -69,7 +69,7 @@ def lib():
                      "nbla_hip_affine_backward_workspace_bytes",
                      "nbla_hip_convolution_backward_workspace_bytes", "nbla_hip_prune_workspace_bytes",
                      "nbla_hip_convolution_workspace_bytes", "nbla_hip_affine_workspace_bytes",
-                     "nbla_hip_split_operand_bytes", "nbla_hip_digit_operand_bytes",
+                     "nbla_hip_digit_operand_bytes",
                      "nbla_hip_binarize_workspace_bytes",
                      "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_convolution_workspace_bytes",
                      "nbla_hip_inq_workspace_bytes", "nbla_hip_inq_affine_workspace_bytes",
@@ -204,14 +204,6 @@ def binarize_weights(W, K, N, transposed=False, quantize_zero_to=1.0, want_alpha
                                               ctypes.c_float(quantize_zero_to), _p(zc), _p(ws),
                                               ctypes.c_size_t(ws.numel()), _stream(stream)))
     return Wb, alpha, bits, zc
-
-
-def split_bf16x3(x, M, K, ldx=None, stream=None):
-    import torch
-    out = torch.empty(lib().nbla_hip_split_operand_bytes(_i64(M), _i64(K)) // 2, dtype=torch.int16, device=x.device)
-    check(lib().nbla_hip_split_bf16x3_f32(_p(x), _i64(K if ldx is None else ldx), _p(out), _i64(M), _i64(K),
-                                          _stream(stream)))
-    return out
 
 
 def split_digits(x, M, K, ldx=None, stream=None):

@@ -57,8 +57,6 @@ def test_size_queries():
     i64 = ctypes.c_int64
     assert L.nbla_hip_packed_bits_bytes(i64(4096), i64(11008)) == 4096 * 11008 // 8
     assert L.nbla_hip_packed_bits_bytes(i64(33), i64(65)) == 8 * 1 * 64 * 16          # padded to 256 x 256
-    assert L.nbla_hip_split_operand_bytes(i64(4096), i64(4096)) == 4096 * 4096 * 6
-    assert L.nbla_hip_split_operand_bytes(i64(1), i64(1)) == 32 * 32 * 6
     # int8 digit operand: 3 bytes per element (K padded to 256), then per row one int64 sum per 16384-column chunk
     # and one int32 shift
     assert L.nbla_hip_digit_operand_bytes(i64(4096), i64(4096)) == 4096 * 4096 * 3 + 4096 * 12 + 256

@@ -135,25 +135,6 @@ def test_long_contraction_is_chunked(dev, M, K, N):
     assert max_rel_err(to_np(y), y64) <= TIGHT
 
 
-def test_split_is_exact(dev):
-    """bf16x3 operand of the plane x plane product: hi + mid + lo == x exactly, in fragment order, zero padded."""
-    rng = np.random.RandomState(2)
-    M, K = 45, 70
-    x = (rng.randn(M, K) * np.exp(rng.randn(M, K) * 8)).astype(np.float32)
-    x[0, :6] = [0.0, -0.0, 1e-30, -3e38, 3.3e38, 1.0]
-    raw = to_np(kernels.split_bf16x3(_dev(x, dev), M, K)).view(np.uint16)
-    rb, kb = (M + 31) // 32, ((K + 31) // 32) * 2
-    frag = raw.reshape(rb, kb, 3, 64, 8).astype(np.uint32) << 16
-    planes = frag.view(np.float32)                       # [rb, kb, plane, lane, e]
-    total = planes[:, :, 0].astype(np.float64) + planes[:, :, 1] + planes[:, :, 2]
-    full = np.zeros((rb * 32, kb * 16), np.float64)
-    for lane in range(64):
-        for e in range(8):
-            full[(lane & 31)::32, ((lane >> 5) * 8 + e)::16] = total[:, :, lane, e]
-    assert np.array_equal(full[:M, :K], x.astype(np.float64))
-    assert not full[M:].any() and not full[:, K:].any()
-
-
 @pytest.mark.parametrize("M,K,N", SHAPES)
 @pytest.mark.parametrize("bias", [False, True])
 def test_binary_weight_affine_matches_oracle(dev, M, K, N, bias):
