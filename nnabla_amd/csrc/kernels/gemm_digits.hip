@@ -322,6 +322,43 @@ __global__ __launch_bounds__(256) void gemm_digits_split_sum(const float *__rest
   }
 }
 
+// The same for outputs whose consecutive elements in memory are consecutive rows m (n_stride != 1: convolution
+// results [sample, channel, position]): a 32 x 32 tile is read along n and, through LDS, written along m.
+__global__ __launch_bounds__(256) void gemm_digits_split_sum_rows(const float *__restrict__ partial, int splits,
+                                                                  int64_t M, int64_t N, float *__restrict__ y,
+                                                                  int64_t inner, int64_t outer_stride, int64_t n_stride,
+                                                                  const float *__restrict__ bias, int accumulate) {
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5; // ty: 0..7
+  const int64_t n0 = (int64_t)blockIdx.x * 32, m0 = (int64_t)blockIdx.y * 32, total = M * N;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t m = m0 + ty + 8 * i, n = n0 + tx;
+    float v = 0.0f;
+    if (m < M && n < N) {
+      v = partial[m * N + n];
+      for (int z = 1; z < splits; ++z)
+        v += partial[(int64_t)z * total + m * N + n];
+    }
+    tile[ty + 8 * i][tx] = v;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t m = m0 + tx, n = n0 + ty + 8 * i;
+    if (m < M && n < N) {
+      float v = tile[tx][ty + 8 * i];
+      const int64_t q = m / inner;
+      float *dst = y + q * outer_stride + (m - q * inner) + n * n_stride;
+      if (accumulate)
+        v = *dst + v;
+      if (bias)
+        v = v + bias[n];
+      *dst = v;
+    }
+  }
+}
+
 // Splits of the contraction for an output of `tiles` 128 x 128 tiles and `k_tiles` k tiles: as many as fill the CUs
 // with one block each, at least 16 k tiles per split; 1 = no split.
 inline int64_t digit_product_splits(int64_t tiles, int64_t k_tiles) {
@@ -399,12 +436,18 @@ int launch_gemm_digits(const void *adigits, const void *bdigits, const float *bi
       hipLaunchKernelGGL((gemm_digits_kernel<kStagesShared, 2>), dim3(blocks, (unsigned)splits), dim3(2 * kThreads),
                          kStagesShared * 2 * kStageBytes, stream, part);
       NBLA_HIP_LAUNCH_CHECK("gemm_digits");
-      int64_t sum_blocks = ceil_div(M * N, 256);
-      if (sum_blocks > 4096)
-        sum_blocks = 4096;
-      hipLaunchKernelGGL(gemm_digits_split_sum, dim3((unsigned)sum_blocks), dim3(256), 0, stream,
-                         static_cast<const float *>(split_ws), (int)splits, M, N, y, inner, outer_stride, n_stride,
-                         a.finish ? bias : nullptr, a.accumulate);
+      if (n_stride != 1 && ceil_div(M, 32) <= 65535) {
+        hipLaunchKernelGGL(gemm_digits_split_sum_rows, dim3((unsigned)ceil_div(N, 32), (unsigned)ceil_div(M, 32)),
+                           dim3(256), 0, stream, static_cast<const float *>(split_ws), (int)splits, M, N, y, inner,
+                           outer_stride, n_stride, a.finish ? bias : nullptr, a.accumulate);
+      } else {
+        int64_t sum_blocks = ceil_div(M * N, 256);
+        if (sum_blocks > 4096)
+          sum_blocks = 4096;
+        hipLaunchKernelGGL(gemm_digits_split_sum, dim3((unsigned)sum_blocks), dim3(256), 0, stream,
+                           static_cast<const float *>(split_ws), (int)splits, M, N, y, inner, outer_stride, n_stride,
+                           a.finish ? bias : nullptr, a.accumulate);
+      }
       NBLA_HIP_LAUNCH_CHECK("gemm_digits_split_sum");
       continue;
     }
