@@ -6,7 +6,7 @@ import torch
 
 import oracle
 from nnabla_amd import kernels
-from util import max_rel_err, to_np
+from util import bits_equal, max_rel_err, to_np
 
 pytestmark = pytest.mark.gpu
 TOL, TIGHT = 1e-4, 5e-6
@@ -60,6 +60,26 @@ def test_binary_affine_backward_accumulates_and_skips(dev):
     only = kernels.binary_affine_backward(d(dy), d(x), d(W), None, d(alpha), 1.0, want=(False, True, False))
     assert only[0] is None and only[2] is None
     assert max_rel_err(to_np(only[1]), x.astype(np.float64).T @ dy.astype(np.float64)) <= TIGHT
+
+
+@pytest.mark.parametrize("M,K,N", [(2048, 96, 130), (3000, 200, 64), (1500, 40, 520)])
+def test_backward_small_outputs_long_batch(dev, M, K, N):
+    """Few output tiles and a long contraction over the samples: the weight-gradient product spreads the contraction
+    over the CUs (partial results summed in a fixed order), here onto gradients that are already there; so does the
+    input gradient of a real-weight layer when N is the long index."""
+    x, W, dy = _data(M, K, N, 35)
+    rng = np.random.RandomState(5)
+    odw = rng.randn(K, N).astype(np.float32)
+    d = lambda a: _dev(a, dev)
+    _, gdw, _ = kernels.binary_affine_backward(d(dy), d(x), d(W), None, None, 1.0, dW=d(odw), want=(False, True, False))
+    dw64 = odw.astype(np.float64) + x.astype(np.float64).T @ dy.astype(np.float64)
+    assert max_rel_err(to_np(gdw), dw64) <= TIGHT
+    again = kernels.binary_affine_backward(d(dy), d(x), d(W), None, None, 1.0, dW=d(odw), want=(False, True, False))[1]
+    assert bits_equal(to_np(again), to_np(gdw))                      # deterministic
+    # real-weight dx with the roles exchanged: [N', K'] weights, contraction over the long index
+    x2, W2, dy2 = _data(K, N, M, 36)                                 # dy2 [K, M], W2 [N, M]
+    gdx = kernels.affine_backward(d(dy2), d(x2), d(W2), want=(True, False, False))[0]
+    assert max_rel_err(to_np(gdx), dy2.astype(np.float64) @ W2.astype(np.float64).T) <= TIGHT
 
 
 @pytest.mark.parametrize("q0", [0.0, 0.5, -1.0])
