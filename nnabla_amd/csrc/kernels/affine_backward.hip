@@ -249,7 +249,9 @@ int nbla_hip_affine_backward_f32(const float *dy, const float *x, const float *W
 size_t nbla_hip_affine_workspace_bytes(int64_t M, int64_t K, int64_t N) {
   if (M <= 0 || K <= 0 || N <= 0)
     return 0;
-  return round_up(nbla_hip_digit_operand_bytes(M, K), 256) + round_up(nbla_hip_digit_operand_bytes(N, K), 256);
+  // the two digit operands, then the partial results of a contraction spread over the CUs (small outputs)
+  return round_up(nbla_hip_digit_operand_bytes(M, K), 256) + round_up(nbla_hip_digit_operand_bytes(N, K), 256) +
+         round_up(gemm_digits_split_bytes(M, K, N), 256);
 }
 
 int nbla_hip_affine_digits_f32(const float *x, const float *W, const float *bias, float *y, int64_t M, int64_t K,
@@ -271,7 +273,8 @@ int nbla_hip_affine_digits_f32(const float *x, const float *W, const float *bias
   rc = launch_split_digits_columns(W, N, wd, K, N, true, stream);
   if (rc)
     return rc;
-  return launch_gemm_digits(xd, wd, bias, y, M, K, N, 1, N, 1, stream);
+  char *split = wd + round_up(nbla_hip_digit_operand_bytes(N, K), 256);
+  return launch_gemm_digits(xd, wd, bias, y, M, K, N, 1, N, 1, stream, false, split, gemm_digits_split_bytes(M, K, N));
 }
 
 } // extern "C"

@@ -427,7 +427,7 @@ int nbla_hip_inq_update_weights_f32(float *W, int32_t *I, float *old_W, int32_t 
 }
 
 size_t nbla_hip_inq_affine_workspace_bytes(int64_t M, int64_t K, int64_t N, int step) {
-  return plan_product(K * N, M, K, N, step).total;
+  return plan_product(K * N, M, K, N, step, gemm_digits_split_bytes(M, K, N)).total;
 }
 
 int nbla_hip_inq_affine_f32(const float *x, float *W, int32_t *I, float *old_W, int32_t *old_I, const float *bias,
@@ -437,7 +437,7 @@ int nbla_hip_inq_affine_f32(const float *x, float *W, int32_t *I, float *old_W, 
   if (M <= 0 || K <= 0 || N <= 0)
     return fail(NBLA_HIP_ERR_VALUE, "invalid affine shape (M=%lld, K=%lld, N=%lld).", (long long)M, (long long)K,
                 (long long)N);
-  const ProductWorkspace p = plan_product(K * N, M, K, N, step);
+  const ProductWorkspace p = plan_product(K * N, M, K, N, step, gemm_digits_split_bytes(M, K, N));
   if (workspace_bytes < p.total || !aligned256(workspace))
     return fail(NBLA_HIP_ERR_MEMORY, "INQ affine workspace too small (%zu < %zu) or misaligned.", workspace_bytes,
                 p.total);
@@ -463,7 +463,8 @@ int nbla_hip_inq_affine_f32(const float *x, float *W, int32_t *I, float *old_W, 
   rc = launch_split_digits_columns(W, N, base + p.planes_off, K, N, true, stream);
   if (rc)
     return rc;
-  return launch_gemm_digits(base + p.split_off, base + p.planes_off, bias, y, M, K, N, 1, N, 1, stream);
+  return launch_gemm_digits(base + p.split_off, base + p.planes_off, bias, y, M, K, N, 1, N, 1, stream, false,
+                            base + p.extra_off, gemm_digits_split_bytes(M, K, N));
 }
 
 size_t nbla_hip_inq_convolution_workspace_bytes(int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
