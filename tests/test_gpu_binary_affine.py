@@ -283,3 +283,39 @@ def test_workspace_too_small_is_reported(dev):
     with pytest.raises(kernels.KernelError) as ei:
         kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev), workspace=ws)
     assert ei.value.code == kernels.ERR_MEMORY
+
+
+def test_forward_replays_in_a_hip_graph(dev):
+    """BinaryWeightAffine and a FixedPointQuantize in front of it, captured once and replayed with new inputs: the
+    entry points allocate nothing, never synchronise on this path and clear their scratch with kernels, so every
+    replay must reproduce the eager result bit for bit (eager work and synchronisations run between the replays)."""
+    M, K, N = 96, 512, 768
+    rng = np.random.RandomState(77)
+    W = _dev((rng.randn(K, N) * 0.02).astype(np.float32), dev)
+    x = torch.empty(M, K, device=dev)
+    xq, y = torch.empty_like(x), torch.empty(M, N, device=dev)
+    ws = kernels.binary_affine_workspace(M, K, N, x)
+
+    def step():
+        kernels.fixed_point_quantize(x, True, 8, 2.0 ** -4, out=xq)
+        return kernels.binary_weight_affine(xq, W, None, 1.0, workspace=ws, out=y)
+
+    x.copy_(_dev(rng.randn(M, K).astype(np.float32), dev))
+    step()                                            # first call outside the capture (one-time kernel attributes)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _, Wb, alpha = step()
+    for i in range(4):
+        xi = _dev((rng.randn(M, K) * (i + 1)).astype(np.float32), dev)
+        x.copy_(xi)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = to_np(y).copy()
+        y.zero_()                                     # eager work between the replays
+        step()
+        torch.cuda.synchronize()
+        assert bits_equal(got, to_np(y)), "replay %d differs from the eager result" % i
+        ref, _, _ = oracle.binary_weight_affine(oracle.fixed_point_quantize(to_np(xi), True, 8, 2.0 ** -4),
+                                                to_np(W), None, 1.0)
+        assert max_rel_err(got, ref) <= TOL
