@@ -868,16 +868,39 @@ __global__ __launch_bounds__(kPrepBlock) void split_digits_columns(const float *
 // Digit operand (rows = the C columns of src, contraction over its R rows); `digits` holds
 // nbla_hip_digit_operand_bytes(C, R).  The operand's row-sum section serves as scratch (column maxima, then the
 // narrow shifts, and the column minima); the digit x digit product does not read row sums.
-int launch_split_digits_columns(const float *src, int64_t ld, void *digits, int64_t R, int64_t C, bool detect_narrow,
-                                hipStream_t stream) {
+ColumnScratch column_scratch(void *digits, int64_t R, int64_t C) {
   const DigitOperand d = digit_operand(C, R);
   char *base = static_cast<char *>(digits);
-  uint32_t *cmax = reinterpret_cast<uint32_t *>(base + d.sum_off);
-  uint32_t *cmin = cmax + d.rows;
+  ColumnScratch s;
+  s.cmax = reinterpret_cast<uint32_t *>(base + d.sum_off);
+  s.cmin = s.cmax + d.rows;
+  s.flag = reinterpret_cast<int32_t *>(base + d.flag_off);
+  s.rows = d.rows;
+  return s;
+}
+
+int launch_split_digits_columns_from_stats(const float *src, int64_t ld, void *digits, int64_t R, int64_t C,
+                                           bool detect_narrow, hipStream_t stream) {
+  const DigitOperand d = digit_operand(C, R);
+  char *base = static_cast<char *>(digits);
+  const ColumnScratch cs = column_scratch(digits, R, C);
   int32_t *shift = reinterpret_cast<int32_t *>(base + d.shift_off);
-  int32_t *flag = reinterpret_cast<int32_t *>(base + d.flag_off);
-  hipLaunchKernelGGL(clear_column_scratch, dim3((unsigned)ceil_div(d.rows, kPrepBlock)), dim3(kPrepBlock), 0, stream,
-                     cmax, cmin, d.rows, flag, detect_narrow ? 0 : 1);
+  hipLaunchKernelGGL(column_shift, dim3((unsigned)ceil_div(d.rows, kPrepBlock)), dim3(kPrepBlock), 0, stream, cs.cmax,
+                     cs.cmin, shift, C, d.rows, cs.flag, detect_narrow ? 1 : 0);
+  NBLA_HIP_LAUNCH_CHECK("column_shift");
+  const int64_t frags = d.k_tiles * d.row_blocks;
+  hipLaunchKernelGGL(split_digits_columns, dim3((unsigned)ceil_div(frags, kPrepBlock / 64)), dim3(kPrepBlock), 0,
+                     stream, src, ld, shift, reinterpret_cast<const int32_t *>(cs.cmax), cs.flag,
+                     reinterpret_cast<uint4_t *>(base), R, C, d.k_tiles, d.row_blocks, frags);
+  NBLA_HIP_LAUNCH_CHECK("split_digits_columns");
+  return NBLA_HIP_OK;
+}
+
+int launch_split_digits_columns(const float *src, int64_t ld, void *digits, int64_t R, int64_t C, bool detect_narrow,
+                                hipStream_t stream) {
+  const ColumnScratch cs = column_scratch(digits, R, C);
+  hipLaunchKernelGGL(clear_column_scratch, dim3((unsigned)ceil_div(cs.rows, kPrepBlock)), dim3(kPrepBlock), 0, stream,
+                     cs.cmax, cs.cmin, cs.rows, cs.flag, detect_narrow ? 0 : 1);
   NBLA_HIP_LAUNCH_CHECK("clear_column_scratch");
   int slab = 64; // taller slabs (fewer atomics per column) while a thousand blocks remain
   while (slab < 256 && ceil_div(C, 256) * ceil_div(R, 2 * slab) >= 1024)
@@ -885,7 +908,8 @@ int launch_split_digits_columns(const float *src, int64_t ld, void *digits, int6
   const dim3 grid((unsigned)ceil_div(C, 256), (unsigned)ceil_div(R, slab));
   const bool vec = C % 4 == 0 && ld % 4 == 0 && aligned16(src);
 #define NBLA_LAUNCH_ABSMAX(V, D)                                                                                       \
-  hipLaunchKernelGGL((column_absmax<V, D>), grid, dim3(kPrepBlock), 0, stream, src, ld, R, C, cmax, cmin, flag, slab)
+  hipLaunchKernelGGL((column_absmax<V, D>), grid, dim3(kPrepBlock), 0, stream, src, ld, R, C, cs.cmax, cs.cmin,       \
+                     cs.flag, slab)
   if (vec && detect_narrow)
     NBLA_LAUNCH_ABSMAX(true, true);
   else if (vec)
@@ -896,15 +920,7 @@ int launch_split_digits_columns(const float *src, int64_t ld, void *digits, int6
     NBLA_LAUNCH_ABSMAX(false, false);
 #undef NBLA_LAUNCH_ABSMAX
   NBLA_HIP_LAUNCH_CHECK("column_absmax");
-  hipLaunchKernelGGL(column_shift, dim3((unsigned)ceil_div(d.rows, kPrepBlock)), dim3(kPrepBlock), 0, stream, cmax,
-                     cmin, shift, C, d.rows, flag, detect_narrow ? 1 : 0);
-  NBLA_HIP_LAUNCH_CHECK("column_shift");
-  const int64_t frags = d.k_tiles * d.row_blocks;
-  hipLaunchKernelGGL(split_digits_columns, dim3((unsigned)ceil_div(frags, kPrepBlock / 64)), dim3(kPrepBlock), 0,
-                     stream, src, ld, shift, reinterpret_cast<const int32_t *>(cmax), flag,
-                     reinterpret_cast<uint4_t *>(base), R, C, d.k_tiles, d.row_blocks, frags);
-  NBLA_HIP_LAUNCH_CHECK("split_digits_columns");
-  return NBLA_HIP_OK;
+  return launch_split_digits_columns_from_stats(src, ld, digits, R, C, detect_narrow, stream);
 }
 
 } // namespace nbla_hip

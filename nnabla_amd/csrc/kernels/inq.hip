@@ -151,7 +151,18 @@ __global__ __launch_bounds__(kBlk) void inq_restore_absmax(float *__restrict__ W
 // n1, n2 and the pruning threshold (inq_affine.cpp:157-166).  `levels` is the
 // host's (int)pow(2, num_bits - 2).
 __global__ __launch_bounds__(64) void inq_finalize(const uint32_t *__restrict__ partial, int nparts, int levels,
-                                                   const uint32_t *__restrict__ n1_cuts, InqParams *__restrict__ params) {
+                                                   const uint32_t *__restrict__ n1_cuts, InqParams *__restrict__ params,
+                                                   ColumnScratch cols) {
+  // the column statistics that the quantize pass will gather (cols.cmax null: none wanted) start from their neutral
+  // values
+  if (cols.cmax) {
+    for (int64_t i = threadIdx.x; i < cols.rows; i += 64) {
+      cols.cmax[i] = 0u;
+      cols.cmin[i] = 0xffffffffu;
+    }
+    if (threadIdx.x == 0)
+      *cols.flag = 0;
+  }
   uint32_t mx = 0u;
   for (int i = threadIdx.x; i < nparts; i += 64)
     mx = partial[i] > mx ? partial[i] : mx;
@@ -188,6 +199,32 @@ __global__ __launch_bounds__(64) void inq_finalize(const uint32_t *__restrict__ 
   *params = p;
 }
 
+// Step C for one fixed weight (:168-190).
+__device__ __forceinline__ float inq_quantize_value(float w, const InqParams &p, const uint32_t *s_cut) {
+  const uint32_t u = __float_as_uint(w) & 0x7fffffffu;
+  const float a = __uint_as_float(u);
+  if (a < p.thr)
+    return 0.0f;
+  if (u < 0x7f800000u && u != 0u) {
+    const int idx = binade_of(u);
+    int e = binade_exponent(idx) + (u >= s_cut[idx] ? 1 : 0);
+    if (e > p.n1)
+      e = p.n1;
+    if (e < p.n2)
+      e = p.n2;
+    float q;
+    if (e > 127)
+      q = __uint_as_float(0x7f800000u);
+    else if (e < -149)
+      q = 0.0f;
+    else
+      q = pow2_int(e);
+    return (w < 0.0f) ? -q : q;
+  }
+  // zero with a zero threshold, infinities and NaN: outside the reference's defined behaviour; left as they are
+  return w;
+}
+
 // Step C for the fixed weights (:168-190) and step F (:203-204).
 __global__ __launch_bounds__(kBlk) void inq_quantize(float *__restrict__ W, int *__restrict__ I, float *__restrict__ old_W,
                                                      int *__restrict__ old_I, int64_t size, int fix_all,
@@ -200,35 +237,88 @@ __global__ __launch_bounds__(kBlk) void inq_quantize(float *__restrict__ W, int 
   const InqParams p = *params;
   for (int64_t i = (int64_t)blockIdx.x * kBlk + threadIdx.x; i < size; i += (int64_t)gridDim.x * kBlk) {
     float w = W[i];
-    int ind = fix_all ? 1 : I[i];
-    if (ind == 1) {
-      const uint32_t u = __float_as_uint(w) & 0x7fffffffu;
-      const float a = __uint_as_float(u);
-      if (a < p.thr) {
-        w = 0.0f;
-      } else if (u < 0x7f800000u && u != 0u) {
-        const int idx = binade_of(u);
-        int e = binade_exponent(idx) + (u >= s_cut[idx] ? 1 : 0);
-        if (e > p.n1)
-          e = p.n1;
-        if (e < p.n2)
-          e = p.n2;
-        float q;
-        if (e > 127)
-          q = __uint_as_float(0x7f800000u);
-        else if (e < -149)
-          q = 0.0f;
-        else
-          q = pow2_int(e);
-        w = (w < 0.0f) ? -q : q;
-      }
-      // zero with a zero threshold, infinities and NaN: outside the reference's defined behaviour; left as they are
-    }
+    const int ind = fix_all ? 1 : I[i];
+    if (ind == 1)
+      w = inq_quantize_value(w, p, s_cut);
     W[i] = w;
     if (fix_all)
       I[i] = ind; // otherwise unchanged
     old_W[i] = w;
     old_I[i] = ind;
+  }
+}
+
+// The same for a weight matrix [R, C] (C % 4 == 0, 16-byte aligned) that is about to become the column-scaled digit
+// operand of the product: the pass also gathers that operand's column statistics (largest / smallest non-zero
+// magnitude per column, the flag for elements that are neither zero nor a normal power of two) from the values it
+// writes, so the operand needs no pass of its own over W for them.  Block = 64 column quads x 4 row groups over a
+// slab of rows, as in the stand-alone statistics kernel.
+__global__ __launch_bounds__(kBlk) void inq_quantize_columns(float *__restrict__ W, int *__restrict__ I,
+                                                             float *__restrict__ old_W, int *__restrict__ old_I,
+                                                             int64_t R, int64_t C, int slab, int fix_all,
+                                                             const InqParams *__restrict__ params,
+                                                             const uint32_t *__restrict__ e_cuts, ColumnScratch cols) {
+  typedef float f4_t __attribute__((ext_vector_type(4)));
+  typedef int i4_t __attribute__((ext_vector_type(4)));
+  static_assert(kBlk == 256, "64 column quads x 4 row groups");
+  __shared__ uint32_t s_cut[kNumBinades];
+  __shared__ uint32_t part[4][256], part_min[4][256];
+  for (int i = threadIdx.x; i < kNumBinades; i += kBlk)
+    s_cut[i] = e_cuts[i];
+  __syncthreads();
+  const InqParams p = *params;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int64_t c0 = ((int64_t)blockIdx.x * 64 + tx) * 4;
+  const int64_t r0 = (int64_t)blockIdx.y * slab, r_end = r0 + slab < R ? r0 + slab : R;
+  uint32_t m[4] = {0u, 0u, 0u, 0u}, mn[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+  bool other = false;
+  if (c0 < C) {
+#pragma unroll 2
+    for (int64_t r = r0 + ty; r < r_end; r += 4) {
+      const int64_t i = r * C + c0;
+      f4_t w = *reinterpret_cast<const f4_t *>(W + i);
+      i4_t ind = {1, 1, 1, 1};
+      if (!fix_all)
+        ind = *reinterpret_cast<const i4_t *>(I + i);
+      w.x = ind.x == 1 ? inq_quantize_value(w.x, p, s_cut) : w.x;
+      w.y = ind.y == 1 ? inq_quantize_value(w.y, p, s_cut) : w.y;
+      w.z = ind.z == 1 ? inq_quantize_value(w.z, p, s_cut) : w.z;
+      w.w = ind.w == 1 ? inq_quantize_value(w.w, p, s_cut) : w.w;
+      *reinterpret_cast<f4_t *>(W + i) = w;
+      if (fix_all)
+        *reinterpret_cast<i4_t *>(I + i) = ind;
+      *reinterpret_cast<f4_t *>(old_W + i) = w;
+      *reinterpret_cast<i4_t *>(old_I + i) = ind;
+      const float v[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t u = __float_as_uint(v[j]) & 0x7fffffffu;
+        m[j] = u > m[j] ? u : m[j];
+        if (u) {
+          mn[j] = u < mn[j] ? u : mn[j];
+          other |= (u & 0x007fffffu) != 0u || (u >> 23) == 0u;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    part[ty][tx * 4 + j] = m[j];
+    part_min[ty][tx * 4 + j] = mn[j];
+  }
+  if (__any(other) && (threadIdx.x & 63) == 0 &&
+      __hip_atomic_load(cols.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
+    atomicOr(cols.flag, 1);
+  __syncthreads();
+  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (c < C) {
+    uint32_t a = max(max(part[0][threadIdx.x], part[1][threadIdx.x]), max(part[2][threadIdx.x], part[3][threadIdx.x]));
+    if (a)
+      atomicMax(&cols.cmax[c], a);
+    a = min(min(part_min[0][threadIdx.x], part_min[1][threadIdx.x]),
+            min(part_min[2][threadIdx.x], part_min[3][threadIdx.x]));
+    if (a != 0xffffffffu)
+      atomicMin(&cols.cmin[c], a);
   }
 }
 
@@ -277,9 +367,12 @@ unsigned grid_for(int64_t size) {
   return (unsigned)(b > 8192 ? 8192 : (b < 1 ? 1 : b));
 }
 
+// `cols` (may be null) with `columns` > 0: W is a [size / columns, columns] matrix about to become a column-scaled
+// digit operand; the quantize pass then fills that operand's column statistics and *cols_done is set.
 int update_weights(float *W, int *I, float *old_W, int *old_I, int64_t size, int num_bits, int step,
                    nbla_hip_bernoulli_fn draw, void *draw_ctx, int *n1n2_out, void *workspace, size_t workspace_bytes,
-                   hipStream_t stream) {
+                   hipStream_t stream, const ColumnScratch *cols = nullptr, int64_t columns = 0,
+                   bool *cols_done = nullptr) {
   if (size <= 0)
     return fail(NBLA_HIP_ERR_VALUE, "INQ weight tensor must not be empty.");
   if (size > 0x7fffffffll)
@@ -362,12 +455,28 @@ int update_weights(float *W, int *I, float *old_W, int *old_I, int64_t size, int
   }
 
   const int levels = (int)std::pow(2, num_bits - 2); // inq_affine.cpp:165
+  const bool with_cols = cols && columns > 0 && columns % 4 == 0 && size % columns == 0 && aligned16(W) &&
+                         aligned16(I) && aligned16(old_W) && aligned16(old_I);
+  ColumnScratch none;
+  none.cmax = none.cmin = nullptr, none.flag = nullptr, none.rows = 0;
   hipLaunchKernelGGL(inq_finalize, dim3(1), dim3(64), 0, stream, partial, (int)nparts, levels,
-                     device_cut_table(kCutInqN1), params);
+                     device_cut_table(kCutInqN1), params, with_cols ? *cols : none);
   NBLA_HIP_LAUNCH_CHECK("inq_finalize");
-  hipLaunchKernelGGL(inq_quantize, dim3(grid_for(size)), dim3(kBlk), 0, stream, W, I, old_W, old_I, size,
-                     step == 1 ? 1 : 0, params, device_cut_table(kCutInqExponent));
+  if (with_cols) {
+    const int64_t R = size / columns;
+    int slab = 64;
+    while (slab < 256 && ceil_div(columns, 256) * ceil_div(R, 2 * slab) >= 1024)
+      slab *= 2;
+    hipLaunchKernelGGL(inq_quantize_columns, dim3((unsigned)ceil_div(columns, 256), (unsigned)ceil_div(R, slab)),
+                       dim3(kBlk), 0, stream, W, I, old_W, old_I, R, columns, slab, step == 1 ? 1 : 0, params,
+                       device_cut_table(kCutInqExponent), *cols);
+  } else {
+    hipLaunchKernelGGL(inq_quantize, dim3(grid_for(size)), dim3(kBlk), 0, stream, W, I, old_W, old_I, size,
+                       step == 1 ? 1 : 0, params, device_cut_table(kCutInqExponent));
+  }
   NBLA_HIP_LAUNCH_CHECK("inq_quantize");
+  if (cols_done)
+    *cols_done = with_cols;
   if (n1n2_out) {
     hipError_t e = hipMemcpyAsync(n1n2_out, params, 2 * sizeof(int), hipMemcpyDeviceToDevice, stream);
     if (e != hipSuccess)
@@ -444,9 +553,15 @@ int nbla_hip_inq_affine_f32(const float *x, float *W, int32_t *I, float *old_W, 
   hipStream_t stream = as_stream(stream_);
   char *base = static_cast<char *>(workspace);
   int rc;
+  // The product runs on the int8 digit kernels: x as a row-scaled digit operand, W^T as a column-scaled one.  Once
+  // every weight is zero or a power of two (all fixed) and a column spans at most six binades, each weight is a small
+  // integer in one digit and three exact digit products give the result; otherwise six (weights still being learnt).
+  // The weight update's last pass gathers the column statistics of that operand on the way.
+  bool cols_done = false;
   if (step >= 0) {
+    const ColumnScratch cols = column_scratch(base + p.planes_off, K, N);
     rc = update_weights(W, I, old_W, old_I, K * N, num_bits, step, draw, draw_ctx, nullptr, base + p.update_off,
-                        p.split_off - p.update_off, stream);
+                        p.split_off - p.update_off, stream, &cols, N, &cols_done);
     if (rc)
       return rc;
   } else {
@@ -454,13 +569,11 @@ int nbla_hip_inq_affine_f32(const float *x, float *W, int32_t *I, float *old_W, 
     if (rc)
       return rc;
   }
-  // The product runs on the int8 digit kernels: x as a row-scaled digit operand, W^T as a column-scaled one.  Once
-  // every weight is zero or a power of two (all fixed) and a column spans at most six binades, each weight is a small
-  // integer in one digit and three exact digit products give the result; otherwise six (weights still being learnt).
   rc = nbla_hip_split_digits_f32(x, K, base + p.split_off, M, K, stream_);
   if (rc)
     return rc;
-  rc = launch_split_digits_columns(W, N, base + p.planes_off, K, N, true, stream);
+  rc = cols_done ? launch_split_digits_columns_from_stats(W, N, base + p.planes_off, K, N, true, stream)
+                 : launch_split_digits_columns(W, N, base + p.planes_off, K, N, true, stream);
   if (rc)
     return rc;
   return launch_gemm_digits(base + p.split_off, base + p.planes_off, bias, y, M, K, N, 1, N, 1, stream, false,

@@ -23,6 +23,18 @@ int launch_gemm_bits(const void *xsplit, const uint32_t *bits, const float *alph
 // binades of its column's largest (its flag word tells the product which form it got).
 int launch_split_digits_columns(const float *src, int64_t ld, void *digits, int64_t R, int64_t C, bool detect_narrow,
                                 hipStream_t stream);
+// The statistics that pass gathers, kept in the operand's own row-sum area: per column the largest and the smallest
+// non-zero magnitude (bit patterns, by atomicMax / atomicMin from 0 / 0xffffffff) and a flag word raised when an
+// element is neither zero nor a normal power of two.  A kernel that touches every element of src anyway may fill them
+// itself (clearing them first) and call the second half of the pass.
+struct ColumnScratch {
+  uint32_t *cmax, *cmin;
+  int32_t *flag;
+  int64_t rows; // entries of cmax / cmin (columns padded to whole fragments)
+};
+ColumnScratch column_scratch(void *digits, int64_t R, int64_t C);
+int launch_split_digits_columns_from_stats(const float *src, int64_t ld, void *digits, int64_t R, int64_t C,
+                                           bool detect_narrow, hipStream_t stream);
 // y[m, n] (+)= sum_k A[m, k] * B[n, k] (+ bias[n]), both factors real-valued digit operands (rows M x K and N x K);
 // A is a row-scaled operand, B a row- or column-scaled one whose flag word selects the six- or three-product form.
 // `split_ws` (may be null; gemm_digits_split_bytes(M, K, N) bytes make every split possible) lets an output of few
