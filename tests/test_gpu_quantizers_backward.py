@@ -120,3 +120,43 @@ def test_min_max_backward_statistics_modes_leave_range_gradients(dev, x_min_max,
     rdx, _, _ = oracle.min_max_quantize_backward(dy, x, qmn, qmx, q(0), q(255), scale, True, x_min_max, ema)
     assert bits_equal(to_np(gdx), rdx)
     assert to_np(gmin).item() == 7.0 and to_np(gmax).item() == 9.0
+
+
+@pytest.mark.parametrize("sign,n,delta", [(True, 8, 2.0 ** -4), (False, 5, 0.3)])
+def test_fixed_point_backward_every_fp32_value(dev, sign, n, delta):
+    """The fine-grained STE mask of fixed_point_quantize.cpp:84-99 for all 2^32 bit patterns of x (dy = 3): dx = dy
+    inside [min, max] (and for NaN, which fails both comparisons), 0 outside."""
+    nn = n - 1 if sign else n
+    mx = float(np.float32((2.0 ** nn - 1) * float(np.float32(delta))))
+    mn = -mx if sign else 0.0
+    chunk = 1 << 27
+    dy = torch.full((chunk,), 3.0, device=dev)
+    for start in range(0, 1 << 32, chunk):
+        lo = start - (1 << 32) if start >= (1 << 31) else start
+        x = torch.arange(lo, lo + chunk, dtype=torch.int32, device=dev).view(torch.float32)
+        dx = kernels.fixed_point_quantize_backward(dy, x, sign, n, delta, True)
+        ref = torch.where((x > mx) | (x < mn), torch.zeros_like(dy), dy)
+        assert bool((dx == ref).all()), "chunk starting at bits %#x" % start
+
+
+@pytest.mark.parametrize("sign,with_zero,n,m", [(True, True, 4, 1), (False, False, 6, 3)])
+def test_pow2_backward_every_normal_fp32_value(dev, sign, with_zero, n, m):
+    """The fine-grained STE mask of pow2_quantize.cpp:97-125 for every normal x farther than 64 ulp from a cut
+    2^(k + 1/2) (the neighbourhoods of the cuts are compared with the host libm in the test above): 0 where
+    2^round(log2|x|) exceeds 2^m, and for negative x of the unsigned form."""
+    p_max = float(2.0 ** m)
+    chunk = 1 << 27
+    dy = torch.full((chunk,), -2.5, device=dev)
+    for start in range(0, 1 << 32, chunk):
+        lo = start - (1 << 32) if start >= (1 << 31) else start
+        bits = torch.arange(lo, lo + chunk, dtype=torch.int32, device=dev)
+        x = bits.view(torch.float32)
+        dx = kernels.pow2_quantize_backward(dy, x, sign, with_zero, n, m, True)
+        q = torch.exp2(torch.round(torch.log2(x.abs().double())))
+        c = q <= p_max
+        if not sign:
+            c = c & ~(x < 0)
+        ref = torch.where(c, dy, torch.zeros_like(dy))
+        mant, expo = bits & 0x7fffff, (bits >> 23) & 0xff
+        checked = (expo > 0) & (expo < 255) & ((mant - 0x3504f3).abs() > 64)
+        assert bool(((dx == ref) | ~checked).all()), "chunk starting at bits %#x" % start
