@@ -52,6 +52,8 @@ def bench_binary_weight_affine(M, K, N, steps, warmup, dev):
     pws = torch.empty(max(256, L.nbla_hip_binarize_workspace_bytes(k._i64(K), k._i64(N))), dtype=torch.uint8,
                       device=dev)
     st = k._stream(None)
+    gws = torch.empty(max(256, L.nbla_hip_gemm_bits_workspace_bytes(k._i64(M), k._i64(K), k._i64(N))), dtype=torch.uint8,
+                      device=dev)
     import ctypes
 
     def step(ev=None):
@@ -66,7 +68,8 @@ def bench_binary_weight_affine(M, K, N, steps, warmup, dev):
         if ev:
             ev[2].record()
         k.check(L.nbla_hip_gemm_bits_f32(k._p(xs), k._p(bits), k._p(alpha), None, k._p(y), k._i64(M), k._i64(K),
-                                         k._i64(N), k._i64(1), k._i64(N), k._i64(1), st))
+                                         k._i64(N), k._i64(1), k._i64(N), k._i64(1), k._p(gws),
+                                         ctypes.c_size_t(gws.numel()), st))
         if ev:
             ev[3].record()
 

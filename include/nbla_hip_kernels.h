@@ -203,11 +203,16 @@ int nbla_hip_split_digits_scaled_f32(const float *x, int64_t ldx,
  * so a row-major [M, N] result is (inner=1, outer_stride=N, n_stride=1) and a
  * convolution result [batch, O, Ho*Wo] is (inner=Ho*Wo, outer_stride=O*Ho*Wo,
  * n_stride=Ho*Wo).  Replaces the Eigen product of affine.cpp:87-95 /
- * convolution.cpp:185-193 for binarised weights. */
+ * convolution.cpp:185-193 for binarised weights.
+ * `workspace` (may be NULL; nbla_hip_gemm_bits_workspace_bytes(M, K, N) bytes,
+ * 256-byte aligned) lets an output of very few tiles (M up to 64 or so) spread
+ * its contraction over the CUs: fp32 partial results, summed in a fixed order. */
+size_t nbla_hip_gemm_bits_workspace_bytes(int64_t M, int64_t K, int64_t N);
 int nbla_hip_gemm_bits_f32(const void *xdigits, const uint32_t *bits,
                            const float *alpha, const float *bias, float *y,
                            int64_t M, int64_t K, int64_t N, int64_t inner,
                            int64_t outer_stride, int64_t n_stride,
+                           void *workspace, size_t workspace_bytes,
                            void *stream);
 
 /* ------------------------------------------------------- whole-op forwards */

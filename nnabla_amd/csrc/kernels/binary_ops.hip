@@ -8,7 +8,7 @@ namespace nbla_hip {
 namespace {
 
 struct AffineWorkspace {
-  size_t bits_off, split_off, prep_off, count_off, total;
+  size_t bits_off, split_off, prep_off, count_off, gemm_off, gemm_bytes, total;
 };
 
 AffineWorkspace plan_affine(int64_t M, int64_t K, int64_t N) {
@@ -22,6 +22,9 @@ AffineWorkspace plan_affine(int64_t M, int64_t K, int64_t N) {
   off += round_up(nbla_hip_binarize_workspace_bytes(K, N), 256);
   w.count_off = off;
   off += 256;
+  w.gemm_off = off; // partial results of a product whose contraction is spread over the CUs (very small M)
+  w.gemm_bytes = nbla_hip_gemm_bits_workspace_bytes(M, K, N);
+  off += w.gemm_bytes;
   w.total = off;
   return w;
 }
@@ -62,7 +65,8 @@ int binary_affine_forward(const float *x, const float *W, float *Wb, float *alph
   rc = nbla_hip_split_digits_f32(x, K, xsplit, M, K, stream_);
   if (rc)
     return rc;
-  return nbla_hip_gemm_bits_f32(xsplit, bits, alpha, bias, y, M, K, N, 1, N, 1, stream_);
+  return nbla_hip_gemm_bits_f32(xsplit, bits, alpha, bias, y, M, K, N, 1, N, 1, base + ws.gemm_off, ws.gemm_bytes,
+                                stream_);
 }
 
 } // namespace

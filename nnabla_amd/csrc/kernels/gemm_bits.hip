@@ -46,6 +46,11 @@ struct GemmBitsArgs {
   int64_t inner, outer_stride, n_stride; // output addressing
   int accumulate; // add to y instead of overwriting it (k chunks after the first)
   int finish;     // apply alpha and bias (last k chunk)
+  // contraction split over blockIdx.y (outputs of very few tiles): split z multiplies the k steps
+  // [step_begin + z * split_steps, + split_steps) and writes a dense [M, N] partial result at y + z * M * N; only
+  // split 0 adds the row sums
+  int64_t split_steps; // 0: no split
+  int use_sums;
 };
 
 // LDS buffers (stages resident) per tile shape: what fits the block's share of the CU's 160 KiB, at most six.
@@ -129,6 +134,13 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
+  if (a.split_steps > 0) {
+    const int64_t begin = a.step_begin + (int64_t)blockIdx.y * a.split_steps;
+    a.step_end = begin + a.split_steps < a.step_end ? begin + a.split_steps : a.step_end;
+    a.step_begin = begin;
+    a.y += (int64_t)blockIdx.y * a.M * a.N;
+    a.use_sums = blockIdx.y == 0;
+  }
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -398,8 +410,11 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
         // rows m0 + 8 rq + 0..3 (the metadata arrays are padded to whole row blocks)
         const int64_t mq = m0 + 8 * rq;
         const int64_t ml = (mq < a.row_blocks * kFragRows) ? mq : 0; // row blocks past the operand are not stored
-        const i32x4_t sum01 = *reinterpret_cast<const i32x4_t *>(a.sums + ml); // two int64 as (lo, hi) words
-        const i32x4_t sum23 = *reinterpret_cast<const i32x4_t *>(a.sums + ml + 2);
+        i32x4_t sum01 = {0, 0, 0, 0}, sum23 = {0, 0, 0, 0};
+        if (a.use_sums) {
+          sum01 = *reinterpret_cast<const i32x4_t *>(a.sums + ml); // two int64 as (lo, hi) words
+          sum23 = *reinterpret_cast<const i32x4_t *>(a.sums + ml + 2);
+        }
         const i32x4_t sh = *reinterpret_cast<const i32x4_t *>(a.shift + ml);
         // sum = s_hi * 65536 + s_lo with s_lo in [0, 65536)
         const uint32_t lo_w[4] = {(uint32_t)sum01.x, (uint32_t)sum01.z, (uint32_t)sum23.x, (uint32_t)sum23.z};
@@ -441,7 +456,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
       const int64_t m = bm * BM + (wm * MF + i) * 32 + col_in_frag;
       if (m >= a.M)
         continue;
-      const long long sum = a.sums[m];
+      const long long sum = a.use_sums ? a.sums[m] : 0;
       const int s_hi = (int)(sum >> 16), s_lo = (int)(sum & 0xffff), sh = a.shift[m];
       float *row = row_ptr(m);
 #pragma unroll
@@ -480,7 +495,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
 }
 
 template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, bool kSwap>
-int launch_tile(const GemmBitsArgs &args, hipStream_t stream) {
+int launch_tile(const GemmBitsArgs &args, hipStream_t stream, unsigned splits = 1) {
   constexpr int kThreads = kWavesM * kWavesN * kWavesK * 64;
   constexpr int kSmem = gemm_bits_lds_bytes(BM, BN, kWavesM, kWavesN, kWavesK);
   auto kernel = gemm_bits_kernel<BM, BN, kWavesM, kWavesN, kWavesK, kSwap>;
@@ -492,7 +507,7 @@ int launch_tile(const GemmBitsArgs &args, hipStream_t stream) {
   GemmBitsArgs a = args;
   a.blocks_m = ceil_div(a.M, BM);
   a.blocks_n = ceil_div(a.n_end - a.n_begin, BN);
-  hipLaunchKernelGGL(kernel, dim3((unsigned)(a.blocks_m * a.blocks_n)), dim3(kThreads), kSmem, stream, a);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(a.blocks_m * a.blocks_n), splits), dim3(kThreads), kSmem, stream, a);
   NBLA_HIP_LAUNCH_CHECK("gemm_bits");
   return NBLA_HIP_OK;
 }
@@ -505,8 +520,65 @@ int launch_tile(const GemmBitsArgs &args, hipStream_t stream) {
 // outputs of at most 256 such tiles use eight wavefronts per 32x256 tile, four k groups of two; outputs of at most
 // 256 wide tiles (every CU would hold a single block of four wavefronts) eight wavefronts per 32x512 tile, two k
 // groups of four.
-template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream) {
+// Splits of the contraction over blocks for an output of `tiles` 32x256 tiles and `steps` k steps: as many as give
+// every CU a block, at least eight k steps (two rounds of the four k groups) each; 1 = no split.
+inline int64_t bit_product_splits(int64_t tiles, int64_t steps) {
+  if (tiles * 2 > 256 || steps < 16)
+    return 1;
+  const int64_t by_cus = 256 / tiles, by_k = steps / 8;
+  return by_cus < by_k ? by_cus : by_k;
+}
+
+// y (+)= (sum over the splits, in split order) (* alpha) (+ bias): the order of operations of the kernel's epilogue.
+__global__ __launch_bounds__(256) void gemm_bits_split_sum(const float *__restrict__ partial, int splits, int64_t M,
+                                                           int64_t N, float *__restrict__ y, int64_t inner,
+                                                           int64_t outer_stride, int64_t n_stride,
+                                                           const float *__restrict__ alpha,
+                                                           const float *__restrict__ bias, int accumulate) {
+  const int64_t total = M * N;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t m = i / N, n = i - m * N;
+    float v = partial[i];
+    for (int z = 1; z < splits; ++z)
+      v += partial[(int64_t)z * total + i];
+    const int64_t q = m / inner;
+    float *dst = y + q * outer_stride + (m - q * inner) + n * n_stride;
+    if (accumulate)
+      v = *dst + v;
+    if (alpha)
+      v = v * alpha[n];
+    if (bias)
+      v = v + bias[n];
+    *dst = v;
+  }
+}
+
+template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream, void *split_ws, size_t split_ws_bytes) {
   const int64_t narrow_tiles = ceil_div(a.M, 32) * ceil_div(a.N, 256);
+  if (!kSwap && split_ws) {
+    int64_t splits = bit_product_splits(narrow_tiles, a.step_end - a.step_begin);
+    while (splits > 1 && (size_t)splits * a.M * a.N * sizeof(float) > split_ws_bytes)
+      --splits;
+    if (splits > 1) {
+      GemmBitsArgs part = a;
+      part.split_steps = ceil_div(ceil_div(a.step_end - a.step_begin, splits), 4) * 4; // whole rounds of the k groups
+      splits = ceil_div(a.step_end - a.step_begin, part.split_steps);
+      part.y = static_cast<float *>(split_ws);
+      part.inner = 1, part.outer_stride = a.N, part.n_stride = 1;
+      part.accumulate = 0, part.finish = 0;
+      int rc = launch_tile<32, 256, 1, 2, 4, kSwap>(part, stream, (unsigned)splits);
+      if (rc)
+        return rc;
+      int64_t blocks = ceil_div(a.M * a.N, 256);
+      if (blocks > 4096)
+        blocks = 4096;
+      hipLaunchKernelGGL(gemm_bits_split_sum, dim3((unsigned)blocks), dim3(256), 0, stream,
+                         static_cast<const float *>(split_ws), (int)splits, a.M, a.N, a.y, a.inner, a.outer_stride,
+                         a.n_stride, a.finish ? a.alpha : nullptr, a.finish ? a.bias : nullptr, a.accumulate);
+      NBLA_HIP_LAUNCH_CHECK("gemm_bits_split_sum");
+      return NBLA_HIP_OK;
+    }
+  }
   if (narrow_tiles <= 256) // too few tiles for the CUs: four k groups per tile
     return launch_tile<32, 256, 1, 2, 4, kSwap>(a, stream);
   if (a.N > 256 && ceil_div(a.M, 32) * ceil_div(a.N, 512) <= 256) // one wide tile per CU at most: two k groups
@@ -520,7 +592,7 @@ template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream) {
 
 int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alpha, const float *bias, float *y,
                      int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
-                     bool swap_out, hipStream_t stream, bool accumulate) {
+                     bool swap_out, hipStream_t stream, bool accumulate, void *split_ws, size_t split_ws_bytes) {
   if (M <= 0 || K <= 0 || N <= 0 || inner <= 0 || M > 0x7fffffffll || inner > 0x7fffffffll)
     return fail(NBLA_HIP_ERR_VALUE, "invalid GEMM shape (M=%lld, K=%lld, N=%lld).", (long long)M, (long long)K,
                 (long long)N);
@@ -546,6 +618,8 @@ int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alp
   a.x_k_tiles = d.k_tiles;
   a.wide_groups = bits_wide_groups(N);
   a.blocks_m = a.blocks_n = 0;
+  a.split_steps = 0;
+  a.use_sums = 1;
   a.inner = inner;
   a.outer_stride = outer_stride;
   a.n_stride = n_stride;
@@ -558,21 +632,31 @@ int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alp
     a.step_end = (a.step_begin + steps_per_chunk < steps) ? a.step_begin + steps_per_chunk : steps;
     a.accumulate = c > 0 || accumulate;
     a.finish = c + 1 == d.chunks;
-    rc = swap_out ? dispatch<true>(a, stream) : dispatch<false>(a, stream);
+    rc = swap_out ? dispatch<true>(a, stream, nullptr, 0) : dispatch<false>(a, stream, split_ws, split_ws_bytes);
     if (rc)
       return rc;
   }
   return NBLA_HIP_OK;
 }
 
+size_t gemm_bits_split_bytes(int64_t M, int64_t K, int64_t N) {
+  const int64_t steps = digit_k_tiles(K < kChunkK ? K : kChunkK) / 2;
+  const int64_t s = bit_product_splits(ceil_div(M, 32) * ceil_div(N, 256), steps);
+  return s > 1 ? (size_t)s * M * N * sizeof(float) : 0;
+}
+
 } // namespace nbla_hip
 
 using namespace nbla_hip;
 
+extern "C" size_t nbla_hip_gemm_bits_workspace_bytes(int64_t M, int64_t K, int64_t N) {
+  return M > 0 && K > 0 && N > 0 ? round_up(gemm_bits_split_bytes(M, K, N), 256) : 0;
+}
+
 extern "C" int nbla_hip_gemm_bits_f32(const void *xdigits, const uint32_t *bits, const float *alpha, const float *bias,
                                       float *y, int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride,
-                                      int64_t n_stride, void *stream) {
+                                      int64_t n_stride, void *workspace, size_t workspace_bytes, void *stream) {
   // m-contiguous outputs (n_stride != 1) store from the transposed accumulator tile
   return launch_gemm_bits(xdigits, bits, alpha, bias, y, M, K, N, inner, outer_stride, n_stride, n_stride != 1,
-                          as_stream(stream));
+                          as_stream(stream), false, workspace, workspace_bytes);
 }

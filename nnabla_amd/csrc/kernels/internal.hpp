@@ -16,7 +16,10 @@ int launch_gemm_f32(const float *x, const float *w, const float *colscale, const
 // (for outputs whose m index is the contiguous one, e.g. convolution results [batch, O, Ho*Wo]).
 int launch_gemm_bits(const void *xsplit, const uint32_t *bits, const float *alpha, const float *bias, float *y,
                      int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
-                     bool swap_out, hipStream_t stream, bool accumulate = false);
+                     bool swap_out, hipStream_t stream, bool accumulate = false, void *split_ws = nullptr,
+                     size_t split_ws_bytes = 0);
+// Scratch that lets launch_gemm_bits spread the contraction of a very small output (M <= 64 or so) over the CUs.
+size_t gemm_bits_split_bytes(int64_t M, int64_t K, int64_t N);
 
 // Digit operand whose rows are the C columns of src [R, C] (row stride ld), contraction over src's rows.  With
 // detect_narrow the operand comes out in its one-digit form when every element is zero or a power of two within six

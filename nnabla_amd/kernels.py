@@ -26,7 +26,7 @@ EXPORTED = (
     "nbla_hip_min_max_quantize_backward_workspace_bytes", "nbla_hip_min_max_quantize_backward_f32",
     "nbla_hip_packed_bits_bytes", "nbla_hip_digit_operand_bytes",
     "nbla_hip_binarize_workspace_bytes", "nbla_hip_binarize_weights_f32",
-    "nbla_hip_split_digits_f32", "nbla_hip_gemm_bits_f32",
+    "nbla_hip_split_digits_f32", "nbla_hip_gemm_bits_workspace_bytes", "nbla_hip_gemm_bits_f32",
     "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_weight_affine_f32",
     "nbla_hip_binary_connect_affine_f32", "nbla_hip_affine_f32", "nbla_hip_split_digits_scaled_f32",
     "nbla_hip_affine_workspace_bytes", "nbla_hip_affine_digits_f32",
@@ -69,7 +69,7 @@ def lib():
                      "nbla_hip_affine_backward_workspace_bytes",
                      "nbla_hip_convolution_backward_workspace_bytes", "nbla_hip_prune_workspace_bytes",
                      "nbla_hip_convolution_workspace_bytes", "nbla_hip_affine_workspace_bytes",
-                     "nbla_hip_digit_operand_bytes",
+                     "nbla_hip_digit_operand_bytes", "nbla_hip_gemm_bits_workspace_bytes",
                      "nbla_hip_binarize_workspace_bytes",
                      "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_convolution_workspace_bytes",
                      "nbla_hip_inq_workspace_bytes", "nbla_hip_inq_affine_workspace_bytes",
@@ -215,12 +215,15 @@ def split_digits(x, M, K, ldx=None, stream=None):
     return out
 
 
-def gemm_bits(xsplit, bits, alpha, bias, M, K, N, out=None, inner=1, outer_stride=None, n_stride=1, stream=None):
+def gemm_bits(xsplit, bits, alpha, bias, M, K, N, out=None, inner=1, outer_stride=None, n_stride=1, workspace=None,
+              stream=None):
     import torch
     y = torch.empty((M, N), dtype=torch.float32, device=bits.device) if out is None else out
+    ws = workspace if workspace is not None else _workspace(
+        lib().nbla_hip_gemm_bits_workspace_bytes(_i64(M), _i64(K), _i64(N)), bits)
     check(lib().nbla_hip_gemm_bits_f32(_p(xsplit), _p(bits), _p(alpha), _p(bias), _p(y), _i64(M), _i64(K), _i64(N),
                                        _i64(inner), _i64(N if outer_stride is None else outer_stride), _i64(n_stride),
-                                       _stream(stream)))
+                                       _p(ws), ctypes.c_size_t(ws.numel()), _stream(stream)))
     return y
 
 
