@@ -236,7 +236,7 @@ def test_affine_digits_special_rows_and_narrow_weights(dev):
 
 @pytest.mark.parametrize("M", [1, 8, 64])
 def test_config3_full_width_small_m_vs_oracle(dev, M):
-    """BASELINE config 3 at K=4096, N=11008 for the M the CPU oracle finishes in seconds."""
+    """Benchmark configuration 3 at K=4096, N=11008 for the M the CPU oracle finishes in seconds."""
     rng = np.random.default_rng(313)
     x = rng.standard_normal((M, 4096), dtype=np.float32)
     W = rng.standard_normal((4096, 11008), dtype=np.float32) * np.float32(0.02)

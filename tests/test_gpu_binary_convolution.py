@@ -74,7 +74,7 @@ def test_convolution_quantize_zero_to_with_zero_weights(dev, q0):
 
 
 def test_config4_resnet_stage(dev):
-    """BASELINE config 4: x [32,256,14,14] ~ N(0,1), W [256,256,3,3] ~ N(0, 2/2304), stride 1, pad 1, zero bias.
+    """Benchmark configuration 4: x [32,256,14,14] ~ N(0,1), W [256,256,3,3] ~ N(0, 2/2304), stride 1, pad 1, zero bias.
     The oracle is run on 4 of the 32 samples (convolution is independent per sample); all 32 are checked against
     torch's float64 convolution on the same binarized weights."""
     rng = np.random.default_rng(313)

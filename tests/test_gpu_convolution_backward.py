@@ -96,7 +96,7 @@ def test_convolution_backward_accumulates_and_skips(dev):
 
 
 def test_config4_backward(dev):
-    """BASELINE config 4 shape (x [32,256,14,14], W [256,256,3,3], stride 1, pad 1): the oracle covers 2 of the 32
+    """Benchmark configuration 4 shape (x [32,256,14,14], W [256,256,3,3], stride 1, pad 1): the oracle covers 2 of the 32
     samples for dx (samples are independent); dW and db of all 32 are checked against torch's float64 autograd on
     the CPU."""
     import torch.nn.functional as tf

@@ -202,7 +202,7 @@ def test_device_memory_is_cached_and_released(ctx):
 
 
 def test_config5_quantized_mlp_graph(ctx):
-    """BASELINE config 5: batch 1024; FixedPointQuantize -> INQAffine 4096x4096 (num_bits 4, every weight fixed)
+    """Benchmark configuration 5: batch 1024; FixedPointQuantize -> INQAffine 4096x4096 (num_bits 4, every weight fixed)
     -> 3 x [ReLU -> FixedPointQuantize -> BinaryWeightAffine 4096x4096]; x ~ N(0,1), W ~ N(0, 0.02^2).
 
     Per layer, with the oracle fed the same input the GPU layer saw: quantizer outputs, Wb and INQ weights are

@@ -148,7 +148,7 @@ def test_inq_convolution_matches_oracle(dev):
 
 
 def test_inq_config5_layer(dev):
-    """The INQAffine layer of BASELINE config 5: x [1024,4096], W [4096,4096] ~ N(0, 0.02^2), num_bits 4, every
+    """The INQAffine layer of benchmark configuration 5: x [1024,4096], W [4096,4096] ~ N(0, 0.02^2), num_bits 4, every
     weight fixed.  Weights bit-exact against the oracle; the output against float64 on sampled entries and against
     the oracle's fp32 GEMM on the first 64 rows."""
     rng = np.random.default_rng(313)

@@ -42,7 +42,7 @@ def test_fixed_point_quantize_matches_oracle(dev, sign, n, delta):
 
 
 def test_fixed_point_quantize_config1_full_size(dev):
-    """BASELINE config 1: [256, 65536] ~ N(0, 2^2), sign, n=8, delta=2^-4, bit-exact."""
+    """Benchmark configuration 1: [256, 65536] ~ N(0, 2^2), sign, n=8, delta=2^-4, bit-exact."""
     rng = np.random.default_rng(313)
     x = (rng.standard_normal((256, 65536), dtype=np.float32) * np.float32(2.0))
     ref = oracle.fixed_point_quantize(x, True, 8, 2.0 ** -4)
@@ -145,7 +145,7 @@ def test_pow2_quantize_matches_oracle(dev, sign, with_zero, n, m):
 
 
 def test_pow2_quantize_config2_weights(dev):
-    """BASELINE config 2b: [512,512,3,3] ~ N(0, 0.05^2), sign, with_zero, n=4, m=1."""
+    """Benchmark configuration 2b: [512,512,3,3] ~ N(0, 0.05^2), sign, with_zero, n=4, m=1."""
     rng = np.random.default_rng(313)
     w = (rng.standard_normal((512, 512, 3, 3), dtype=np.float32) * np.float32(0.05))
     ref = oracle.pow2_quantize(w, True, True, 4, 1)
@@ -266,7 +266,7 @@ def test_min_max_quantize_eps_nudge_and_zero_point_clamps(dev):
 
 
 def test_min_max_quantize_config2_full_size(dev):
-    """BASELINE config 2a: post-ReLU activations [64,256,56,56], per-tensor, ema, decay .999."""
+    """Benchmark configuration 2a: post-ReLU activations [64,256,56,56], per-tensor, ema, decay .999."""
     rng = np.random.default_rng(313)
     x = np.abs(rng.standard_normal((64, 256, 56, 56), dtype=np.float32))
     got, ref = _mmq_both(dev, x, (1, 1, 1, 1), -6.0, 6.0, 0.0, 255.0, 0.999, True, True)
