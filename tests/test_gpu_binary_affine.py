@@ -112,6 +112,20 @@ def test_digit_operand_block_shapes(dev, M, K):
     assert np.array_equal(sums[0], q.sum(1))
 
 
+@pytest.mark.parametrize("M,K,ldx", [(70, 256, 260), (2100, 1024, 1100), (33, 4096, 4100), (40, 90, 97), (64, 8192, 8200)])
+def test_digit_operand_of_a_strided_matrix(dev, M, K, ldx):
+    """Row stride larger than the row length (a slice of a wider matrix): the operand only depends on the M x K view."""
+    rng = np.random.RandomState(K)
+    wide = rng.randn(M, ldx).astype(np.float32)
+    view = np.ascontiguousarray(wide[:, :K])
+    a = to_np(kernels.split_digits(_dev(wide, dev), M, K, ldx=ldx))
+    b = to_np(kernels.split_digits(_dev(view, dev), M, K))
+    qa, sa, ma = unpack_digits(a, M, K)
+    qb, sb, mb = unpack_digits(b, M, K)
+    assert np.array_equal(qa, qb) and np.array_equal(sa, sb) and np.array_equal(ma, mb)
+    assert np.array_equal(qa, np.rint(np.ldexp(view.astype(np.float64), sa[:, None].astype(np.int64))).astype(np.int64))
+
+
 def test_digit_operand_marks_non_finite_rows(dev):
     x = np.ones((5, 64), np.float32)
     x[1, 3] = np.inf
