@@ -195,6 +195,8 @@ def bench_other_configs(dev, iters):
         return h
     ms = time_kernel(mlp, iters)
     out["quantized_mlp[1024 x 4096, 4 layers] forward"] = {"ms": ms, "TFLOPs": 4 * 2.0 * M * K * N / ms / 1e9}
+    out["quantized_mlp[1024 x 4096, 4 layers] forward, through the function registry"] = bench_frontend_mlp(
+        max(5, iters // 2))
     # backward passes (the next row of the scope table)
     n = 1 << 24
     xq = torch.randn(n, generator=g).to(dev) * 2
@@ -234,6 +236,41 @@ def bench_other_configs(dev, iters):
                                                       workspace=ws), max(3, iters // 2))
     out["binary_weight_affine_backward dW [4096,4096,11008]"] = {"ms": ms, "TFLOPs": 2.0 * M * K * N / ms / 1e9}
     return out
+
+
+def bench_frontend_mlp(iters):
+    """The same 4-layer quantized MLP built with the Python front-end (F.* on the hip context -> C API -> the
+    "hip:float" Function classes -> C-ABI), forward() of the graph timed on the host between device synchronisations."""
+    import numpy as np
+    import nnabla_amd as nn
+    import nnabla_amd.functions as F
+    from nnabla_amd import ext_hip
+    from nnabla_amd.ext_utils import get_extension_context
+    rng = np.random.default_rng(313)
+    B, D = 1024, 4096
+
+    def var(a):
+        v = nn.Variable(a.shape)
+        v.d = a
+        return v
+    with nn.context_scope(get_extension_context('hip')):
+        x = var(rng.standard_normal((B, D), dtype=np.float32))
+        Ws = [var(rng.standard_normal((D, D), dtype=np.float32) * np.float32(0.02)) for _ in range(4)]
+        h = F.fixed_point_quantize(x, True, 8, 2 ** -4)
+        h = F.inq_affine(h, Ws[0], var(np.zeros((D, D), np.float32)), None, 1, 4, (0,), 'largest_abs')
+        for l in range(1, 4):
+            h = F.relu(h)
+            h = F.fixed_point_quantize(h, True, 8, 2 ** -4)
+            h = F.binary_weight_affine(h, Ws[l], nn.Variable((D, D)), nn.Variable((D,)))
+        for _ in range(5):
+            h.forward()
+        ext_hip.device_synchronize('0')
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            h.forward()
+        ext_hip.device_synchronize('0')
+        ms = (time.perf_counter() - t0) / iters * 1e3
+    return {"ms": ms, "TFLOPs": 4 * 2.0 * B * D * D / ms / 1e9}
 
 
 def cpu_baseline(K, N, rows):
