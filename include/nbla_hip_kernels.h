@@ -438,6 +438,24 @@ size_t nbla_hip_prune_workspace_bytes(void);
 int nbla_hip_prune_f32(const float *x, float *y, size_t size, float rate,
                        void *workspace, size_t workspace_bytes, void *stream);
 
+/* Range recorders of quantization-aware training: y = x (skipped when y == x)
+ * and, when `training`, the one-element statistics m / M updated from this
+ * batch.  Replaces the forward_impl of the five recorder PythonFunctions,
+ * python/src/nnabla/utils/qnn.py:73-84 (mode 0, MinMaxMinMaxRecorder: m =
+ * min(m, min x), M = max(M, max x)), :178-188 (1, AbsMaxRecorder: M = max(M,
+ * max|x|)), :289-300 (2, MinMaxMvaRecorder: m = decay*m + (1-decay)*min x, M
+ * likewise), :411-420 (3, MaxMaxRecorder) and :509-518 (4, MaxMvaRecorder); the
+ * chains of Min / Max / Abs / Maximum2 / MulScalar / Add2 / Identity helper
+ * functions there become one scan and one update.  `m` is unused in modes 1, 3
+ * and 4.  `decay` is the Python float of the reference: decay and 1 - decay
+ * are each rounded to fp32 once, as its MulScalar functions do.  Their backward passes the gradient through: use
+ * nbla_hip_fixed_point_quantize_backward_f32 with ste_fine_grained = 0. */
+size_t nbla_hip_range_recorder_workspace_bytes(void);
+int nbla_hip_range_recorder_f32(const float *x, float *y, size_t size, float *m,
+                                float *M, int mode, double decay, int training,
+                                void *workspace, size_t workspace_bytes,
+                                void *stream);
+
 /* ---------------------------------------------------------------------- INQ */
 
 /* INQ step selector (what the forward does to the indicators before quantizing):

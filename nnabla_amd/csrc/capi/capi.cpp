@@ -14,6 +14,7 @@
 #include <nbla/function/min_max_quantize.hpp>
 #include <nbla/function/pow2_quantize.hpp>
 #include <nbla/function/quantize_linear.hpp>
+#include <nbla/function/range_recorder.hpp>
 #include <nbla/hip/init.hpp>
 #include <nbla/init.hpp>
 
@@ -145,6 +146,14 @@ FunctionPtr create_by_name(const string &name, const Context &ctx, const int64_t
   if (name == "Prune") {
     need(0, 1);
     return create_Prune(ctx, (float)fa[0]);
+  }
+  if (name == "Sink") {
+    need(1, 0);
+    return create_Sink(ctx, ia[0] != 0);
+  }
+  if (name == "RangeRecorder") {
+    need(2, 1);
+    return create_RangeRecorder(ctx, (int)ia[0], fa[0], ia[1] != 0);
   }
   NBLA_ERROR(error_code::value, "Unknown function '%s'.", name.c_str());
 }

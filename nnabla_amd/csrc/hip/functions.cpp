@@ -5,6 +5,7 @@
 #include <nbla/hip/function/inq.hpp>
 #include <nbla/hip/function/quantize.hpp>
 #include <nbla/hip/function/quantize_linear.hpp>
+#include <nbla/hip/function/range_recorder.hpp>
 
 namespace nbla {
 
@@ -554,6 +555,39 @@ void PruneHip<T>::backward_impl(const Variables &inputs, const Variables &output
                                                            accum[0], nullptr));
 }
 
+// The recorder PythonFunctions' forward_impl (qnn.py:73-84, :178-188, :289-300, :411-420, :509-518): y.copy_from(x),
+// then the statistics take this batch's extrema.
+template <typename T> void RangeRecorderHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  T *m = nullptr, *M = nullptr;
+  if (this->training_) {
+    if (this->two_sided())
+      m = inputs[1]->cast_data_and_get_pointer<T>(this->ctx_, false);
+    Variable *stat = inputs[this->two_sided() ? 2 : 1];
+    M = stat->cast_data_and_get_pointer<T>(this->ctx_, false);
+  }
+  HipWorkspace ws(nbla_hip_range_recorder_workspace_bytes(), this->ctx_);
+  NBLA_HIP_CALL(nbla_hip_range_recorder_f32(x, y, (size_t)inputs[0]->size(), m, M, this->mode_, this->decay_,
+                                            this->training_, ws.pointer(), ws.bytes(), nullptr));
+}
+
+// The gradient passes through unchanged.  (The reference's backward_impl, e.g. qnn.py:86-95, first copies the input
+// gradient over the output gradient and so hands the input gradient back to itself; the recorders are identity
+// functions and this is their gradient.)
+template <typename T>
+void RangeRecorderHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                        const vector<bool> &propagate_down, const vector<bool> &accum) {
+  if (!propagate_down[0])
+    return;
+  hip_set_device(this->ctx_);
+  const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
+  T *dx = inputs[0]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[0]);
+  NBLA_HIP_CALL(nbla_hip_fixed_point_quantize_backward_f32(dy, dy, dx, (size_t)inputs[0]->size(), 1, 8, 1.0f, 0,
+                                                           accum[0], nullptr));
+}
+
 // explicit instantiations for the "float" type config (function_types.yaml:483-509)
 template class FixedPointQuantizeHip<float>;
 template class Pow2QuantizeHip<float>;
@@ -570,5 +604,7 @@ template class ConvolutionHip<float>;
 template class QuantizeLinearHip<float>;
 template class DequantizeLinearHip<float>;
 template class PruneHip<float>;
+template class SinkHip<float>;
+template class RangeRecorderHip<float>;
 
 } // namespace nbla

@@ -8,6 +8,7 @@
 #include <nbla/hip/function/inq.hpp>
 #include <nbla/hip/function/quantize.hpp>
 #include <nbla/hip/function/quantize_linear.hpp>
+#include <nbla/hip/function/range_recorder.hpp>
 #include <nbla/hip/init.hpp>
 #include <nbla/init.hpp>
 
@@ -70,6 +71,8 @@ void init_hip() {
   NBLA_REGISTER_FUNCTION_IMPL(QuantizeLinear, QuantizeLinearHip<float>, "hip:float", const string &, bool, int);
   NBLA_REGISTER_FUNCTION_IMPL(DequantizeLinear, DequantizeLinearHip<float>, "hip:float");
   NBLA_REGISTER_FUNCTION_IMPL(Prune, PruneHip<float>, "hip:float", float);
+  NBLA_REGISTER_FUNCTION_IMPL(Sink, SinkHip<float>, "hip:float", bool);
+  NBLA_REGISTER_FUNCTION_IMPL(RangeRecorder, RangeRecorderHip<float>, "hip:float", int, double, bool);
 }
 
 } // namespace nbla

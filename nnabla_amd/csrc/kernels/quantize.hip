@@ -708,3 +708,160 @@ int nbla_hip_min_max_quantize_f32(const float *x, float *y, const int64_t *xshap
 }
 
 } // extern "C"
+
+// ------------------------------------------------------------------ range recorders
+// The recorders of quantization-aware training (python/src/nnabla/utils/qnn.py:42-560) are identity functions that
+// keep running statistics of what passes through them: y = x, and while training the one-element arrays m / M take
+//   kMinMaxMinMax  m = minimum2(m, min x), M = maximum2(M, max x)                     (qnn.py:73-84)
+//   kAbsMax        M = maximum2(M, max |x|)                                           (qnn.py:178-188)
+//   kMinMaxMva     m = decay * m + (1 - decay) * min x, M likewise with max x         (qnn.py:289-300)
+//   kMaxMax        M = maximum2(M, max x)                                             (qnn.py:411-420)
+//   kMaxMva        M = decay * M + (1 - decay) * max x                                (qnn.py:509-518)
+// with min / max as max.cpp / min.cpp compute them (see Extrema above).  One pass copies x to y and scans it.
+namespace nbla_hip {
+namespace {
+
+enum RecorderMode { kMinMaxMinMax = 0, kAbsMax = 1, kMinMaxMva = 2, kMaxMax = 3, kMaxMva = 4, kRecorderModes = 5 };
+
+template <bool kAbs, bool kCopy>
+__global__ __launch_bounds__(kRedBlock) void record_scan(const float *__restrict__ x, float *__restrict__ y,
+                                                         MinMaxPartial *__restrict__ partial, size_t n4, size_t size) {
+  Extrema ex;
+  ex.init();
+  const size_t per = (n4 + gridDim.x - 1) / gridDim.x;
+  const size_t begin = (size_t)blockIdx.x * per, end = (begin + per < n4) ? begin + per : n4;
+  size_t i = begin + threadIdx.x;
+  for (; i + 3 * kRedBlock < end; i += 4 * kRedBlock) {
+    float4_t v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      v[j] = load4(x + 4 * (i + j * kRedBlock));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (kCopy)
+        store4(y + 4 * (i + j * kRedBlock), v[j]);
+      if (kAbs)
+        v[j] = float4_t{__builtin_fabsf(v[j].x), __builtin_fabsf(v[j].y), __builtin_fabsf(v[j].z),
+                        __builtin_fabsf(v[j].w)};
+      ex.take4(v[j], (uint32_t)(4 * (i + j * kRedBlock)));
+    }
+  }
+  for (; i < end; i += kRedBlock) {
+    float4_t v = load4(x + 4 * i);
+    if (kCopy)
+      store4(y + 4 * i, v);
+    if (kAbs)
+      v = float4_t{__builtin_fabsf(v.x), __builtin_fabsf(v.y), __builtin_fabsf(v.z), __builtin_fabsf(v.w)};
+    ex.take4(v, (uint32_t)(4 * i));
+  }
+  if (blockIdx.x == gridDim.x - 1) { // the elements past the last float4 (all of them when n4 is 0), highest indices
+    for (size_t t = 4 * n4 + threadIdx.x; t < size; t += kRedBlock) {
+      const float v = x[t];
+      if (kCopy)
+        y[t] = v;
+      ex.take(kAbs ? __builtin_fabsf(v) : v, (uint32_t)t);
+    }
+  }
+  ex.wave_reduce();
+  __shared__ MinMaxPartial s_part[kRedBlock / 64];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0)
+    s_part[wave] = ex.pack();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kRedBlock / 64; ++w)
+      ex.merge(s_part[w].vmin, s_part[w].vmax, s_part[w].zidx, s_part[w].zsign);
+    partial[blockIdx.x] = ex.pack();
+  }
+}
+
+__global__ __launch_bounds__(64) void record_update(const MinMaxPartial *__restrict__ partial, int nchunks,
+                                                    float *__restrict__ m, float *__restrict__ M, int mode,
+                                                    float decay, float one_minus_decay) {
+  Extrema ex;
+  ex.init();
+  for (int c = threadIdx.x; c < nchunks; c += 64)
+    ex.merge(partial[c].vmin, partial[c].vmax, partial[c].zidx, partial[c].zsign);
+  ex.wave_reduce();
+  if (threadIdx.x != 0)
+    return;
+  const float mb = ex.min_value(), Mb = ex.max_value();
+  if (mode == kMinMaxMinMax) {
+    const float lo = *m, hi = *M;
+    *m = (lo < mb) ? lo : mb; // minimum2.hpp:41
+    *M = (hi > Mb) ? hi : Mb; // maximum2.hpp:41
+  } else if (mode == kAbsMax || mode == kMaxMax) {
+    const float hi = *M;
+    *M = (hi > Mb) ? hi : Mb;
+  } else if (mode == kMinMaxMva) {
+    // MulScalar, MulScalar, Add2: three roundings per statistic
+    const float a = decay * *m, b = one_minus_decay * mb;
+    *m = a + b;
+    const float c = decay * *M, d = one_minus_decay * Mb;
+    *M = c + d;
+  } else {
+    const float c = decay * *M, d = one_minus_decay * Mb;
+    *M = c + d;
+  }
+}
+
+} // namespace
+} // namespace nbla_hip
+
+extern "C" {
+
+size_t nbla_hip_range_recorder_workspace_bytes(void) { return (size_t)kMaxChunks * sizeof(MinMaxPartial); }
+
+int nbla_hip_range_recorder_f32(const float *x, float *y, size_t size, float *m, float *M, int mode, double decay,
+                                int training, void *workspace, size_t workspace_bytes, void *stream_) {
+  if (mode < 0 || mode >= kRecorderModes)
+    return fail(NBLA_HIP_ERR_VALUE, "range recorder: unknown mode %d.", mode);
+  if (size > 0xffffffffull)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "range recorder: arrays above 2^32 elements are not supported.");
+  hipStream_t stream = as_stream(stream_);
+  if (!training) { // y.copy_from(x) only
+    if (size && y != x) {
+      hipError_t e = hipMemcpyAsync(y, x, size * sizeof(float), hipMemcpyDeviceToDevice, stream);
+      if (e != hipSuccess)
+        return fail_hip(e, "range recorder copy");
+    }
+    return NBLA_HIP_OK;
+  }
+  const bool two = (mode == kMinMaxMinMax || mode == kMinMaxMva);
+  if (M == nullptr || (two && m == nullptr))
+    return fail(NBLA_HIP_ERR_VALUE, "range recorder: the statistics arrays are missing.");
+  if (workspace_bytes < nbla_hip_range_recorder_workspace_bytes() || !aligned16(workspace))
+    return fail(NBLA_HIP_ERR_MEMORY, "range recorder workspace too small or misaligned.");
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  MinMaxPartial *partial = static_cast<MinMaxPartial *>(workspace);
+  const bool copy = (y != x);
+  const size_t n4 = (aligned16(x) && (!copy || aligned16(y))) ? size / 4 : 0;
+  size_t blocks = (n4 + kRedBlock * 4 - 1) / (kRedBlock * 4);
+  if (blocks > (size_t)kMaxChunks)
+    blocks = kMaxChunks;
+  if (blocks < 1)
+    blocks = 1;
+  const dim3 grid((unsigned)blocks), block(kRedBlock);
+  if (mode == kAbsMax) {
+    if (copy)
+      hipLaunchKernelGGL((record_scan<true, true>), grid, block, 0, stream, x, y, partial, n4, size);
+    else
+      hipLaunchKernelGGL((record_scan<true, false>), grid, block, 0, stream, x, y, partial, n4, size);
+  } else {
+    if (copy)
+      hipLaunchKernelGGL((record_scan<false, true>), grid, block, 0, stream, x, y, partial, n4, size);
+    else
+      hipLaunchKernelGGL((record_scan<false, false>), grid, block, 0, stream, x, y, partial, n4, size);
+  }
+  NBLA_HIP_LAUNCH_CHECK("range recorder scan");
+  // `decay * m` and `(1 - decay) * mb` of the reference are MulScalar functions: each takes the Python float (a
+  // double) and rounds it to fp32 once
+  hipLaunchKernelGGL(record_update, dim3(1), dim3(64), 0, stream, partial, (int)blocks, m, M, mode, (float)decay,
+                     (float)(1.0 - decay));
+  NBLA_HIP_LAUNCH_CHECK("range recorder update");
+  return NBLA_HIP_OK;
+}
+
+} // extern "C"

@@ -12,6 +12,7 @@
 #include <nbla/function/min_max_quantize.hpp>
 #include <nbla/function/pow2_quantize.hpp>
 #include <nbla/function/quantize_linear.hpp>
+#include <nbla/function/range_recorder.hpp>
 
 #include <algorithm>
 
@@ -101,6 +102,8 @@ NBLA_REGISTER_FUNCTION_SOURCE(Convolution, int, const vector<int> &, const vecto
 NBLA_REGISTER_FUNCTION_SOURCE(QuantizeLinear, const string &, bool, int);
 NBLA_REGISTER_FUNCTION_SOURCE(DequantizeLinear);
 NBLA_REGISTER_FUNCTION_SOURCE(Prune, float);
+NBLA_REGISTER_FUNCTION_SOURCE(Sink, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(RangeRecorder, int, double, bool);
 
 // ------------------------------------------------------------- shape inference
 AffineShapes infer_affine_shapes(int base_axis, Variable *x, Variable *w, Variable *bias) {

@@ -1,5 +1,6 @@
 """Function objects and graph nodes (the subset of python/src/nnabla/function.pyx.tmpl the path needs)."""
 import ctypes
+import weakref
 
 from . import _capi
 from .context import get_current_context
@@ -10,10 +11,21 @@ def _handles(variables):
     return (ctypes.c_void_p * len(variables))(*[v._h for v in variables])
 
 
+class Info(dict):
+    """What a function was created from: the registry name with the packed integer / float / string arguments (the
+    dict items), plus ``type_name`` (the name the function reports, as ``nnabla.function.Info.type_name``) and
+    ``args`` (the keyword arguments of the ``F.*`` call, as ``Info.args``)."""
+
+    def __init__(self, name, iargs, fargs, sarg, args=None, type_name=None):
+        dict.__init__(self, type=name, iargs=tuple(iargs), fargs=tuple(fargs), sarg=sarg)
+        self.args = dict(args or {})
+        self.type_name = type_name or name
+
+
 class Function(object):
     """A function instance created through the nbla registry for the current (or given) context."""
 
-    def __init__(self, name, ctx=None, iargs=(), fargs=(), sarg=None):
+    def __init__(self, name, ctx=None, iargs=(), fargs=(), sarg=None, args=None):
         L = _capi.lib()
         ctx = ctx or get_current_context()
         self.ctx = ctx
@@ -24,7 +36,15 @@ class Function(object):
                                     str(ctx.device_id).encode(), ia, len(iargs), fa, len(fargs),
                                     None if sarg is None else sarg.encode())
         self._h = _capi.check_handle(h)
-        self.info = {"type": name, "iargs": tuple(iargs), "fargs": tuple(fargs), "sarg": sarg}
+        self.info = Info(name, iargs, fargs, sarg, args)
+        if name == "RangeRecorder":
+            self.info.type_name = self.name
+
+    def clone(self, ctx=None):
+        """A new function of the same type and arguments (what the graph converters' ``_modify_as_same`` builds by
+        evaluating ``F.<type_name>(ctx, **args)``, graph_converter.py:138-151)."""
+        i = self.info
+        return Function(i["type"], ctx, i["iargs"], i["fargs"], i["sarg"], i.args)
 
     def __del__(self):
         h = getattr(self, "_h", None)
@@ -100,6 +120,14 @@ class FunctionNode(object):
         self.function = function
         self.inputs = inputs
         self.outputs = outputs
+        ref = weakref.ref(self)
+        for v in {id(i): i for i in inputs}.values():
+            v._consumers.append(ref)
+
+    @property
+    def rank(self):
+        """Longest path from a leaf variable (CgFunction::rank, computation_graph.cpp:28-35)."""
+        return max([i.rank for i in self.inputs] or [0])
 
     @property
     def name(self):

@@ -37,6 +37,7 @@ EXPORTED = (
     "nbla_hip_convolution_backward_f32", "nbla_hip_convolution_workspace_bytes", "nbla_hip_convolution_f32",
     "nbla_hip_quantize_linear_f32", "nbla_hip_quantize_linear_backward_f32", "nbla_hip_dequantize_linear_f32",
     "nbla_hip_dequantize_linear_backward_f32", "nbla_hip_prune_workspace_bytes", "nbla_hip_prune_f32",
+    "nbla_hip_range_recorder_workspace_bytes", "nbla_hip_range_recorder_f32",
     "nbla_hip_inq_workspace_bytes", "nbla_hip_inq_update_weights_f32", "nbla_hip_inq_affine_workspace_bytes",
     "nbla_hip_inq_affine_f32", "nbla_hip_inq_convolution_workspace_bytes", "nbla_hip_inq_convolution_f32",
     "nbla_hip_get_device_count", "nbla_hip_set_device", "nbla_hip_malloc", "nbla_hip_free", "nbla_hip_mem_info",
@@ -68,6 +69,7 @@ def lib():
                      "nbla_hip_min_max_quantize_backward_workspace_bytes",
                      "nbla_hip_affine_backward_workspace_bytes",
                      "nbla_hip_convolution_backward_workspace_bytes", "nbla_hip_prune_workspace_bytes",
+                     "nbla_hip_range_recorder_workspace_bytes",
                      "nbla_hip_convolution_workspace_bytes", "nbla_hip_affine_workspace_bytes",
                      "nbla_hip_digit_operand_bytes", "nbla_hip_gemm_bits_workspace_bytes",
                      "nbla_hip_binarize_workspace_bytes",
@@ -439,6 +441,23 @@ def prune(x, rate=0.9, workspace=None, stream=None):
     ws = workspace if workspace is not None else _workspace(lib().nbla_hip_prune_workspace_bytes(), x)
     check(lib().nbla_hip_prune_f32(_p(x), _p(y), ctypes.c_size_t(x.numel()), ctypes.c_float(rate), _p(ws),
                                    ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return y
+
+
+RECORDER_MODES = {"MinMaxMinMaxRecorder": 0, "AbsMaxRecorder": 1, "MinMaxMvaRecorder": 2, "MaxMaxRecorder": 3,
+                  "MaxMvaRecorder": 4}
+
+
+def range_recorder(x, m, M, mode, decay=0.99, training=True, y=None, workspace=None, stream=None):
+    """y = x; m / M (one-element tensors, updated in place; m may be None for the one-sided recorders) take this
+    batch's statistics.  `mode` is a key or value of RECORDER_MODES."""
+    import torch
+    mode = RECORDER_MODES.get(mode, mode)
+    y = torch.empty_like(x) if y is None else y
+    ws = workspace if workspace is not None else _workspace(lib().nbla_hip_range_recorder_workspace_bytes(), x)
+    check(lib().nbla_hip_range_recorder_f32(_p(x), _p(y), ctypes.c_size_t(x.numel()), _p(m) if m is not None else None,
+                                            _p(M), int(mode), ctypes.c_double(decay), int(bool(training)), _p(ws),
+                                            ctypes.c_size_t(ws.numel()), _stream(stream)))
     return y
 
 

@@ -79,6 +79,7 @@ class Variable(object):
         self._h = _capi.check_handle(L.nblac_variable_new(_shape_arr(shape), len(shape)))
         self.need_grad = need_grad
         self.parent = None        # the FunctionNode that produces this variable
+        self._consumers = []      # weak references to the FunctionNodes that take this variable as an input
         self.name = ''
         self.persistent = False
 
@@ -203,27 +204,61 @@ class Variable(object):
         return p
 
     # ------------------------------------------------------------------- graph
+    def _function_order(self):
+        """The functions this variable depends on, each after the producers of its inputs."""
+        done, order = set(), []
+        stack = [(self.parent, 0)] if self.parent is not None else []
+        if stack:
+            done.add(id(self.parent))
+        while stack:
+            node, k = stack.pop()
+            if k < len(node.inputs):
+                stack.append((node, k + 1))
+                nxt = node.inputs[k].parent
+                if nxt is not None and id(nxt) not in done:
+                    done.add(id(nxt))
+                    stack.append((nxt, 0))
+            else:
+                order.append(node)
+        return order
+
     def forward(self, clear_buffer=False, clear_no_need_grad=False):
         """Runs every function this variable depends on, in dependency order (CgVariable::forward)."""
-        done, order = set(), []
-
-        def visit(v):
-            node = v.parent
-            if node is None or id(node) in done:
-                return
-            done.add(id(node))
-            for i in node.inputs:
-                visit(i)
-            order.append(node)
-        import sys
-        limit = sys.getrecursionlimit()
-        sys.setrecursionlimit(max(limit, 10000))
-        try:
-            visit(self)
-        finally:
-            sys.setrecursionlimit(limit)
-        for node in order:
+        for node in self._function_order():
             node.forward()
+
+    def visit(self, f):
+        """Calls ``f(function)`` for every function this variable depends on, in forward order
+        (python/src/nnabla/_variable.pyx, ``Variable.visit``)."""
+        for node in self._function_order():
+            f(node)
+
+    @property
+    def function_references(self):
+        """The live functions that take this variable as an input, oldest first."""
+        alive = [r for r in self._consumers if r() is not None]
+        self._consumers = alive
+        return [r() for r in alive]
+
+    @property
+    def rank(self):
+        """0 for a leaf, else one more than the producing function's rank (function.cpp:109)."""
+        ranks = {}
+        for node in self._function_order():
+            ranks[id(node)] = max([ranks.get(id(i.parent), -1) + 1 for i in node.inputs] or [0])
+        return 0 if self.parent is None else ranks[id(self.parent)] + 1
+
+    def rewire_on(self, var):
+        """This variable takes over ``var``'s arrays and producing function, so that everything built on this variable
+        now follows ``var``'s graph; ``var`` loses its parent (``Variable.rewire_on``, _variable.pyx:435-475)."""
+        if tuple(var.shape) != tuple(self.shape):
+            raise ValueError("rewire_on: shapes differ, %r and %r" % (self.shape, var.shape))
+        _capi.check(_capi.lib().nblac_variable_share(self._h, var._h))
+        node = var.parent
+        self.parent = node
+        if node is not None:
+            node.outputs = [self if o is var else o for o in node.outputs]
+            var.parent = None
 
     def backward(self, grad=1, clear_buffer=False):
         """Back-propagates from this variable (CgVariable::backward): its gradient is filled with `grad` (a scalar or an
@@ -235,23 +270,7 @@ class Variable(object):
                 self._fill(1, float(grad))
             else:
                 self.g = np.asarray(grad)
-        done, order = set(), []
-
-        def visit(v):
-            node = v.parent
-            if node is None or id(node) in done:
-                return
-            done.add(id(node))
-            for i in node.inputs:
-                visit(i)
-            order.append(node)
-        import sys
-        limit = sys.getrecursionlimit()
-        sys.setrecursionlimit(max(limit, 10000))
-        try:
-            visit(self)
-        finally:
-            sys.setrecursionlimit(limit)
+        order = self._function_order()
         written = set()
         for node in reversed(order):
             if not any(i.need_grad for i in node.inputs):

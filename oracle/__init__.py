@@ -4,7 +4,9 @@ TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by ``__graft_entry__.smoke()``
 and by the CPU-baseline leg of ``bench.py``.  The product package never imports
 this module.  Every function takes and returns numpy arrays (fp32 / int32,
 C-contiguous) and maps one-to-one onto an ``orc_*`` entry point, which in turn
-cites the nnabla file:line it restates.
+cites the nnabla file:line it restates; ``range_recorder`` and ``recorder_scale``
+(scalar bookkeeping of quantization-aware training) are numpy restatements
+written here.
 """
 import ctypes
 import os
@@ -381,6 +383,49 @@ def prune(x, rate=0.9):
     y = np.empty_like(x)
     _check(lib().orc_prune(_fp(x), _fp(y), ctypes.c_long(x.size), ctypes.c_float(rate)), "prune")
     return y
+
+
+RECORDERS = ("MinMaxMinMaxRecorder", "AbsMaxRecorder", "MinMaxMvaRecorder", "MaxMaxRecorder", "MaxMvaRecorder")
+
+
+def range_recorder(x, m, M, kind, decay=0.99):
+    """One training-mode forward of a QAT range recorder: returns (m_new, M_new) as fp32 scalars (m_new is m unchanged
+    for the one-sided kinds).  numpy restatement (no ``orc_*`` entry point) of python/src/nnabla/utils/qnn.py
+    forward_impl :73-84 (MinMaxMinMax), :178-188 (AbsMax), :289-300 (MinMaxMva), :411-420 (MaxMax), :509-518
+    (MaxMva), with Min / Max as ``min_max_reduce``, Minimum2 / Maximum2 as include/nbla/function/minimum2.hpp:41 /
+    maximum2.hpp:41, and ``decay * m + (1 - decay) * mb`` as MulScalar, MulScalar, Add2 in fp32."""
+    assert kind in RECORDERS
+    f = np.float32
+    x = _f32(x)
+    src = np.abs(x) if kind == "AbsMaxRecorder" else x
+    mb, Mb = min_max_reduce(src, (1,) * x.ndim)
+    mb, Mb = f(mb.reshape(-1)[0]), f(Mb.reshape(-1)[0])
+    m = None if m is None else f(np.asarray(m, np.float32).reshape(-1)[0])
+    M = f(np.asarray(M, np.float32).reshape(-1)[0])
+    if kind == "MinMaxMinMaxRecorder":
+        return (m if m < mb else mb), (M if M > Mb else Mb)
+    if kind in ("AbsMaxRecorder", "MaxMaxRecorder"):
+        return m, (M if M > Mb else Mb)
+    d, e = f(decay), f(1.0 - decay)
+    if kind == "MinMaxMvaRecorder":
+        return f(f(d * m) + f(e * mb)), f(f(d * M) + f(e * Mb))
+    return m, f(f(d * M) + f(e * Mb))
+
+
+def recorder_scale(m, M, kind, narrow_range=False, round_method="NOTROUND"):
+    """QuantizeLinear scale from recorded statistics: qnn.py:126-139 for the two-sided recorders ((M - m) / levels,
+    floored at 1e-24), :229-240 / :460-469 / :543-552 for the one-sided ones (2 M / levels); levels = 255, or 254
+    with ``narrow_range``; then optionally moved to a power of two with the exponent rounded as asked."""
+    levels = 254 if narrow_range else 255
+    M = np.asarray(M, np.float32)
+    if kind in ("MinMaxMinMaxRecorder", "MinMaxMvaRecorder"):
+        scale = np.maximum(M - np.asarray(m, np.float32), np.float32(1e-24)) / np.float32(levels)
+    else:
+        scale = (np.float32(2) * M) / np.float32(levels)
+    rnd = {"CEIL": np.ceil, "ROUND": np.round, "FLOOR": np.floor, "NOTROUND": None}[round_method]
+    if rnd is not None:
+        scale = np.float32(2) ** rnd(np.log(scale) / np.log(2))
+    return np.asarray(scale, np.float32)
 
 
 class Inq(object):

@@ -1,0 +1,372 @@
+"""Quantization-aware training on the GPU: the range-recorder kernel against the CPU oracle (bit-exact), the recorder
+functions through the registry, and the converted graphs end to end (recording graph == float graph; simulated-
+quantization graph against the same chain computed with the oracle's functions)."""
+import numpy as np
+import pytest
+import torch
+
+import nnabla_amd as nn
+import nnabla_amd.experimental.graph_converters as GC
+import nnabla_amd.functions as F
+import nnabla_amd.parametric_functions as PF
+import oracle
+from nnabla_amd import kernels as K
+from nnabla_amd.ext_utils import get_extension_context
+from nnabla_amd.utils import qnn
+from nnabla_amd.utils.qnn import FunctionsRankRecorder, QATConfig, QATScheduler, QNNState
+from util import bits_equal, first_mismatch, max_rel_err, to_np
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+@pytest.fixture()
+def ctx(dev):
+    nn.clear_parameters()
+    with nn.context_scope(get_extension_context('hip', device_id='0')):
+        yield
+    nn.clear_parameters()
+
+
+def _var(a):
+    v = nn.Variable(a.shape)
+    v.d = a
+    return v
+
+
+def _f32_bits(a):
+    return np.asarray(a, np.float32).reshape(-1).view(np.uint32)
+
+
+# ----------------------------------------------------------------------------------------------- kernel vs oracle
+@pytest.mark.parametrize("kind", oracle.RECORDERS)
+@pytest.mark.parametrize("shape", [(1,), (3,), (7, 9), (4, 16, 16), (1000, 1031), (2, 3, 1024, 1024)])
+def test_recorder_kernel_bit_exact(dev, kind, shape):
+    """Three consecutive batches: statistics and the copied output against the oracle, bit for bit."""
+    rng = np.random.default_rng(1000 * oracle.RECORDERS.index(kind) + len(shape) + sum(shape))
+    two = kind in ("MinMaxMinMaxRecorder", "MinMaxMvaRecorder")
+    m_ref, M_ref = np.float32(0.0), np.float32(0.0)
+    m = torch.zeros(1, device=dev) if two else None
+    M = torch.zeros(1, device=dev)
+    for it in range(3):
+        x = (rng.standard_normal(shape) * (it + 1) + 0.25 * it).astype(np.float32)
+        xt = torch.from_numpy(x).to(dev)
+        y = K.range_recorder(xt, m, M, kind, decay=0.99)
+        assert bits_equal(to_np(y), x), first_mismatch(to_np(y), x)
+        m_ref, M_ref = oracle.range_recorder(x, m_ref if two else None, M_ref, kind, 0.99)
+        assert _f32_bits(to_np(M))[0] == _f32_bits(M_ref)[0], (it, to_np(M), M_ref)
+        if two:
+            assert _f32_bits(to_np(m))[0] == _f32_bits(m_ref)[0], (it, to_np(m), m_ref)
+
+
+def test_recorder_kernel_edge_cases(dev):
+    """Signed zeros, NaNs, values beyond the +-1e8 the reductions start from, unaligned views, in-place, training off."""
+    cases = [np.array([-0.0, 0.0, -0.0], np.float32), np.array([0.0, -0.0], np.float32),
+             np.array([np.nan, 1.0, -2.0, np.nan], np.float32), np.full(5, np.nan, np.float32),
+             np.array([3e8, -3e8], np.float32), np.array([-3e8, -2e8], np.float32),
+             np.array([np.inf, -np.inf, 1.0], np.float32), np.zeros(1031, np.float32)]
+    for x in cases:
+        for kind in oracle.RECORDERS:
+            two = kind in ("MinMaxMinMaxRecorder", "MinMaxMvaRecorder")
+            for start in (0.0, -1.5, 2.5):
+                m = torch.full((1,), start, device=dev) if two else None
+                M = torch.full((1,), start, device=dev)
+                K.range_recorder(torch.from_numpy(x).to(dev), m, M, kind, decay=0.9)
+                m_ref, M_ref = oracle.range_recorder(x, start if two else None, start, kind, 0.9)
+                assert bits_equal(to_np(M), [M_ref]), (x, kind, start, to_np(M), M_ref)
+                if two:
+                    assert bits_equal(to_np(m), [m_ref]), (x, kind, start, to_np(m), m_ref)
+    rng = np.random.default_rng(3)
+    base = torch.from_numpy(rng.standard_normal(4099).astype(np.float32)).to(dev)
+    for off, n in [(1, 4096), (3, 1001), (2, 5)]:          # not 16-byte aligned
+        view = base[off:off + n]
+        M = torch.zeros(1, device=dev)
+        y = torch.empty(n + 1, device=dev)[1:]
+        K.range_recorder(view, None, M, "AbsMaxRecorder", y=y)
+        assert bits_equal(to_np(y), to_np(view))
+        assert to_np(M)[0] == np.abs(to_np(view)).max()
+    x = base.clone()
+    M = torch.zeros(1, device=dev)
+    K.range_recorder(x, None, M, "MaxMaxRecorder", y=x)    # in place: no copy, statistics only
+    assert bits_equal(to_np(x), to_np(base)) and to_np(M)[0] == to_np(base).max()
+    M = torch.full((1,), 7.0, device=dev)
+    y = K.range_recorder(base, None, M, "MaxMaxRecorder", training=False)
+    assert bits_equal(to_np(y), to_np(base)) and to_np(M)[0] == 7.0
+    with pytest.raises(K.KernelError):
+        K.range_recorder(base, None, M, 9)
+    with pytest.raises(K.KernelError):
+        K.range_recorder(base, None, M, "MinMaxMinMaxRecorder")      # the minimum array is missing
+
+
+def test_recorder_invariants_at_benchmark_size(dev):
+    """Properties that hold whatever the data: running extrema equal the extrema of everything seen (and of the
+    starting zero); a moving average fed a constant batch maximum c follows c (1 - decay^n)."""
+    g = torch.Generator(device=dev)
+    g.manual_seed(11)
+    m, M = torch.zeros(1, device=dev), torch.zeros(1, device=dev)
+    A = torch.zeros(1, device=dev)
+    lo, hi, amax = 0.0, 0.0, 0.0
+    for it in range(3):
+        x = torch.randn((256, 65536), device=dev, generator=g) * (1 + it)
+        y = K.range_recorder(x, m, M, "MinMaxMinMaxRecorder")
+        K.range_recorder(x, None, A, "AbsMaxRecorder", y=x)
+        assert torch.equal(y, x)
+        lo, hi, amax = min(lo, x.min().item()), max(hi, x.max().item()), max(amax, x.abs().max().item())
+        assert (m.item(), M.item(), A.item()) == (lo, hi, amax)
+    x = torch.rand((64, 4096), device=dev, generator=g)
+    x[17, 33] = 5.0
+    V = torch.zeros(1, device=dev)
+    for n in range(1, 40):
+        K.range_recorder(x, None, V, "MaxMvaRecorder", decay=0.9, y=x)
+        assert abs(V.item() - 5.0 * (1 - 0.9 ** n)) < 5e-6 * n
+    lo_v, hi_v = torch.zeros(1, device=dev), torch.zeros(1, device=dev)
+    x[3, 5] = -2.0
+    for n in range(1, 20):
+        K.range_recorder(x, lo_v, hi_v, "MinMaxMvaRecorder", decay=0.75, y=x)
+        assert abs(lo_v.item() + 2.0 * (1 - 0.75 ** n)) < 5e-6 * n and abs(hi_v.item() - 5.0 * (1 - 0.75 ** n)) < 5e-6 * n
+
+
+# ------------------------------------------------------------------------------------- functions through the registry
+def test_recorder_functions_forward_backward(ctx):
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((4, 5, 6)).astype(np.float32)
+    for kind, call in (("MinMaxMinMaxRecorder", qnn.minmax_minmax_recorder), ("AbsMaxRecorder", qnn.abs_max_recorder),
+                       ("MinMaxMvaRecorder", qnn.minmax_mva_recorder), ("MaxMaxRecorder", qnn.max_max_recorder),
+                       ("MaxMvaRecorder", qnn.max_mva_recorder)):
+        two = kind.startswith("MinMax")
+        xv = _var(x)
+        xv.need_grad = True
+        stats = [_var(np.zeros((1, 1, 1), np.float32)) for _ in range(2 if two else 1)]
+        y = call(xv, *stats)
+        assert y.parent.info.type_name == kind
+        m_ref, M_ref = np.float32(0), np.float32(0)
+        for _ in range(2):
+            y.forward()
+            m_ref, M_ref = oracle.range_recorder(x, m_ref if two else None, M_ref, kind, 0.99)
+        assert bits_equal(y.d, x)
+        assert bits_equal(stats[-1].d, np.full((1, 1, 1), M_ref))
+        if two:
+            assert bits_equal(stats[0].d, np.full((1, 1, 1), m_ref))
+        # the gradient passes through; accumulated onto a leaf's existing gradient
+        dy = rng.standard_normal(x.shape).astype(np.float32)
+        xv.g = np.ones_like(x)
+        y.backward(dy)
+        assert bits_equal(xv.g, dy + 1)
+        # training=False: identity, statistics untouched
+        frozen = call(xv, *stats, training=False)
+        before = [s.d.copy() for s in stats]
+        frozen.forward()
+        assert bits_equal(frozen.d, x) and all(bits_equal(s.d, b) for s, b in zip(stats, before))
+
+
+def test_sink(ctx):
+    a, b = _var(np.ones((2, 3), np.float32)), _var(np.ones((4,), np.float32))
+    a.need_grad = b.need_grad = True
+    h = F.relu(a)
+    end = F.sink(h, b)
+    end.forward()
+    a.g, b.g = 0, 0
+    end.backward(None)
+    assert np.array_equal(b.g, np.ones(4, np.float32)) and np.array_equal(a.g, np.ones((2, 3), np.float32))
+
+
+# ------------------------------------------------------------------------------------------------ converted graphs
+def small_net(x):
+    h = F.relu(PF.convolution(x, 8, (3, 3), pad=(1, 1), name='c1'))
+    h = F.relu(PF.convolution(h, 8, (3, 3), stride=(2, 2), name='c2'))
+    h = F.relu(PF.affine(h, 32, name='f1'))
+    return PF.affine(h, 10, name='f2')
+
+
+def randomise_parameters(rng):
+    for k, v in nn.get_parameters(grad_only=False).items():
+        v.d = (rng.standard_normal(v.shape) * (0.2 if k.endswith('W') else 0.05)).astype(np.float32)
+
+
+def oracle_training_graph(x, cfg):
+    """small_net's simulated-quantization graph computed with the oracle: D -> function -> Q along the chain, weights
+    and biases through Q -> D, scales read from the registered parameters."""
+    rm, nr = cfg.round_mode, cfg.narrow_range
+    P = {k: v.d for k, v in nn.get_parameters(grad_only=False).items()}
+
+    def sz(scope, name, nd):
+        return P['%s/scale-%s' % (scope, name)].reshape((1,) * nd), P['%s/zeropoint-%s' % (scope, name)].reshape((1,) * nd)
+
+    def qdq(v, scope, name):
+        s, z = sz(scope, name, v.ndim)
+        q, z2 = oracle.quantize_linear(v, s, z, rm, nr, 1)
+        return oracle.dequantize_linear(q, s, z2)
+
+    h = oracle.convolution(x, P['c1/conv/W'], P['c1/conv/b'], pad=(1, 1))
+    h = np.maximum(qdq(h, 'ReLU-1', 'x0'), 0)
+    h = qdq(h, 'Convolution-2', 'x0')
+    h = oracle.convolution(h, qdq(P['c2/conv/W'], 'Convolution-2', 'w0'), qdq(P['c2/conv/b'], 'Convolution-2', 'b'),
+                           stride=(2, 2))
+    h = np.maximum(qdq(h, 'ReLU-3', 'x0'), 0)
+    h = qdq(h, 'Affine-4', 'x0')
+    h = oracle.affine(h.reshape(h.shape[0], -1), qdq(P['f1/affine/W'], 'Affine-4', 'w0'),
+                      qdq(P['f1/affine/b'], 'Affine-4', 'b'))
+    h = np.maximum(qdq(h, 'ReLU-5', 'x0'), 0)
+    return oracle.affine(h, P['f2/affine/W'], P['f2/affine/b'])
+
+
+def check_every_function(y):
+    """Each function of y's graph against the oracle fed the inputs the device function read: the quantize /
+    dequantize / ReLU / recorder steps bit for bit, the products within the acceptance tolerance."""
+    counts = {}
+
+    def check(f):
+        t = f.info.type_name
+        ins = [i.d for i in f.inputs]
+        out = f.outputs[0].d
+        a = f.info.args
+        if t == 'Convolution':
+            want = oracle.convolution(ins[0], ins[1], ins[2] if len(ins) > 2 else None, pad=a['pad'],
+                                      stride=a['stride'], dilation=a['dilation'], group=a['group'])
+            assert max_rel_err(out, want) < TOL, (t, max_rel_err(out, want))
+        elif t == 'Affine':
+            want = oracle.affine(ins[0].reshape(ins[0].shape[0], -1), ins[1], ins[2] if len(ins) > 2 else None)
+            assert max_rel_err(out, want) < TOL, (t, max_rel_err(out, want))
+        elif t == 'ReLU':
+            assert bits_equal(out, np.maximum(ins[0], 0))
+        elif t == 'QuantizeLinear':
+            want, _ = oracle.quantize_linear(ins[0], ins[1], ins[2], a['round_mode'], a['narrow_range'], a['dtype'])
+            assert bits_equal(out, want), (t, first_mismatch(out, want))
+            assert np.array_equal(out, np.round(out)) and out.min() >= -128 and out.max() <= 127
+        elif t == 'DequantizeLinear':
+            want = oracle.dequantize_linear(ins[0], ins[1], ins[2])
+            assert bits_equal(out, want), (t, first_mismatch(out, want))
+        elif t.endswith('Recorder'):
+            assert bits_equal(out, ins[0])
+        else:
+            raise AssertionError("unexpected function %s" % t)
+        counts[t] = counts.get(t, 0) + 1
+    y.visit(check)
+    return counts
+
+
+def test_scheduler_end_to_end(ctx):
+    rng = np.random.default_rng(2024)
+    x = nn.Variable((16, 3, 16, 16))
+    y = small_net(x)
+    randomise_parameters(rng)
+    float_net = GC.GraphConverter([GC.FunctionModifier()]).convert(y)      # an untouched copy to compare with
+    float_in = float_net
+    while float_in.parent is not None:
+        float_in = float_in.parent.inputs[0]
+    cfg = QATConfig()
+    # the activation recorders average from zero with decay 0.99: they need a few hundred batches to settle
+    n_rec = 400
+    cfg.niter_to_recording, cfg.niter_to_training = 1, 1 + n_rec
+    sched = QATScheduler(cfg)
+    sched(y)
+
+    batches = [rng.standard_normal(x.shape).astype(np.float32) * (1 + 0.1 * (i % 5)) for i in range(n_rec + 3)]
+    seen_max = {}
+    for i, data in enumerate(batches):
+        sched.step()
+        x.d = data
+        float_in.d = data
+        y.forward()
+        float_net.forward()
+        if sched.state != QNNState.TRAINING and i < 8:
+            # the recorders are identity functions: the recording graph computes what the float graph computes
+            assert bits_equal(y.d, float_net.d), (i, first_mismatch(y.d, float_net.d))
+        if sched.state == QNNState.RECORDING and i < 5:
+            seen_max[i] = nn.get_parameter('Affine-4/M-w0').d.ravel()[0]
+            if i == 2:
+                assert check_every_function(y) == {'Convolution': 2, 'Affine': 2, 'ReLU': 3, 'MaxMvaRecorder': 5,
+                                                   'MinMaxMinMaxRecorder': 4}
+    assert sched.state == QNNState.TRAINING
+    # weights did not change while recording: their running maximum is the weight maximum from the first batch on
+    W = nn.get_parameter('f1/affine/W').d
+    assert all(v == W.max() for v in seen_max.values()) and len(seen_max) == 4
+    assert nn.get_parameter('Affine-4/m-w0').d.ravel()[0] == W.min()
+    # the activation statistic of four recorded batches is the moving average of their maxima, from zero
+    h = np.maximum(oracle.convolution(batches[1], nn.get_parameter('c1/conv/W').d, nn.get_parameter('c1/conv/b').d,
+                                      pad=(1, 1)), 0)
+    first = np.float32(np.float32(1.0 - 0.99) * h.max())
+    settled = nn.get_parameter('Convolution-2/M-x0').d.ravel()[0]
+    assert first < settled < 1.5 * h.max() and settled > 0.5 * h.max()
+
+    # the simulated-quantization graph, function by function, against the oracle
+    counts = check_every_function(y)
+    assert counts == {'Convolution': 2, 'Affine': 2, 'ReLU': 3, 'QuantizeLinear': 9, 'DequantizeLinear': 9}
+    # and as a whole against the same chain computed on the oracle alone; a value that sits on a rounding boundary
+    # may fall to the other side there, which moves it by one quantization step
+    want = oracle_training_graph(batches[-1], cfg)
+    got = y.d
+    assert got.shape == want.shape == (16, 10)
+    assert max_rel_err(got, want) < 0.05, max_rel_err(got, want)
+    # and it is a quantized network: close to the float one, not equal to it
+    err = max_rel_err(got, float_net.d)
+    assert 0 < err < 0.3, err
+
+    # gradients flow through the Q / DQ pairs (straight-through: dy / scale * scale)
+    for v in nn.get_parameters().values():
+        v.g = 0
+    y.backward(np.ones((16, 10), np.float32))
+    gW = nn.get_parameter('f1/affine/W').g
+    relu5 = y.parent.inputs[0]
+    dpre = (relu5.d > 0).astype(np.float32) * (np.ones((16, 10), np.float32) @ nn.get_parameter('f2/affine/W').d.T)
+    h_in = y.parent.inputs[0].parent.inputs[0].parent.inputs[0].parent.inputs[0].parent.inputs[0]   # Affine-4's input
+    assert h_in.parent.info.type_name == 'DequantizeLinear'
+    want_gW = h_in.d.reshape(16, -1).astype(np.float64).T @ dpre.astype(np.float64)
+    assert max_rel_err(gW, want_gW) < 1e-3, max_rel_err(gW, want_gW)
+    assert np.abs(nn.get_parameter('c1/conv/W').g).max() > 0
+
+
+def test_recording_with_other_recorders_matches_oracle(ctx):
+    """MinMaxMva activations / AbsMax weights on an MLP: every registered statistic against the oracle's recorders fed
+    the same tensors."""
+    rng = np.random.default_rng(77)
+    x = nn.Variable((32, 64))
+    h = F.relu(PF.affine(x, 48, name='a'))
+    y = PF.affine(F.relu(PF.affine(h, 40, name='b')), 8, name='c')
+    randomise_parameters(rng)
+    cfg = QATConfig()
+    cfg.skip_inputs_layers, cfg.skip_outputs_layers = [], []
+    cfg.record_layers = ['Affine']
+    cfg.recorder_activation = qnn.MinMaxMvaRecorderCallback
+    cfg.recorder_weight = qnn.AbsMaxRecorderCallback
+    ranks = FunctionsRankRecorder()
+    y.visit(ranks)
+    y_rec = GC.GraphConverter([GC.QuantizeNonQNNToRecordingModifier(ranks.functions_ranks, config=cfg)]).convert(y)
+    x_rec = y_rec
+    while x_rec.parent is not None:
+        x_rec = x_rec.parent.inputs[0]
+    P = {k: v.d for k, v in nn.get_parameters(grad_only=False).items()}
+    ref = {}
+    for it in range(3):
+        data = rng.standard_normal(x.shape).astype(np.float32) * (it + 1)
+        x_rec.d = data
+        y_rec.forward()
+        acts = {'Affine-0': data}
+        acts['Affine-2'] = np.maximum(oracle.affine(data, P['a/affine/W'], P['a/affine/b']), 0)
+        acts['Affine-4'] = np.maximum(oracle.affine(acts['Affine-2'], P['b/affine/W'], P['b/affine/b']), 0)
+        for scope, pre in (('Affine-0', 'a'), ('Affine-2', 'b'), ('Affine-4', 'c')):
+            act = to_np_device(y_rec, scope)
+            lo, hi = ref.get(scope + 'x', (np.float32(0), np.float32(0)))
+            # the recorded activation is the device's own (its fp32 sums differ from the oracle's in the last bits)
+            ref[scope + 'x'] = oracle.range_recorder(act, lo, hi, 'MinMaxMvaRecorder', 0.99)
+            assert max_rel_err(act, acts[scope]) < TOL
+            for j, leaf in enumerate(('W', 'b')):
+                _, Mw = oracle.range_recorder(P['%s/affine/%s' % (pre, leaf)], None,
+                                              ref.get(scope + leaf, np.float32(0)), 'AbsMaxRecorder')
+                ref[scope + leaf] = Mw
+                assert nn.get_parameter('%s/M-w%d' % (scope, j)).d.ravel()[0] == Mw
+            assert bits_equal(nn.get_parameter(scope + '/m-x0').d.ravel(), [ref[scope + 'x'][0]])
+            assert bits_equal(nn.get_parameter(scope + '/M-x0').d.ravel(), [ref[scope + 'x'][1]])
+
+
+def to_np_device(y_rec, scope):
+    """The tensor that entered the activation recorder registered under ``scope`` in the graph of ``y_rec``."""
+    target = nn.get_parameter(scope + '/M-x0')
+    found = []
+
+    def look(f):
+        if f.info.type_name == 'MinMaxMvaRecorder' and f.inputs[2] is target:
+            found.append(f.inputs[0].d)
+    y_rec.visit(look)
+    assert len(found) == 1
+    return found[0]
