@@ -221,6 +221,16 @@ def bench_other_configs(dev, iters):
     ms = time_kernel(lambda: k.prune(xq, 0.9, workspace=pws), iters)
     out["prune[256,65536] rate 0.9"] = {"ms": ms, "GBs": 20.0 * n / ms / 1e6,
                                         "frac_hbm": 20.0 * n / ms / 1e6 / PEAK_HBM_GBS}
+    # range recorders of quantization-aware training: copy + scan (8 B/elem), or the scan alone when the output
+    # aliases the input (4 B/elem)
+    rws = torch.empty(k.lib().nbla_hip_range_recorder_workspace_bytes(), dtype=torch.uint8, device=dev)
+    rm_, rM_, ry = torch.zeros(1, device=dev), torch.zeros(1, device=dev), torch.empty_like(x2)
+    ms = time_kernel(lambda: k.range_recorder(x2, rm_, rM_, "MinMaxMvaRecorder", y=ry, workspace=rws), iters)
+    out["min_max_mva_recorder[256,65536]"] = {"ms": ms, "GBs": 8.0 * n / ms / 1e6,
+                                              "frac_hbm": 8.0 * n / ms / 1e6 / PEAK_HBM_GBS}
+    ms = time_kernel(lambda: k.range_recorder(x2, None, rM_, "AbsMaxRecorder", y=x2, workspace=rws), iters)
+    out["abs_max_recorder[256,65536] in place"] = {"ms": ms, "GBs": 4.0 * n / ms / 1e6,
+                                                   "frac_hbm": 4.0 * n / ms / 1e6 / PEAK_HBM_GBS}
     M, K, N = 4096, 4096, 11008
     xb = torch.randn(M, K, generator=g).to(dev)
     Wb_ = (torch.randn(K, N, generator=g) * 0.02).to(dev)

@@ -780,8 +780,17 @@ __global__ __launch_bounds__(64) void record_update(const MinMaxPartial *__restr
                                                     float decay, float one_minus_decay) {
   Extrema ex;
   ex.init();
-  for (int c = threadIdx.x; c < nchunks; c += 64)
-    ex.merge(partial[c].vmin, partial[c].vmax, partial[c].zidx, partial[c].zsign);
+  // sixteen independent 16-byte loads in flight per lane: one round trip for up to 1024 partials
+  const float4_t *pp = reinterpret_cast<const float4_t *>(partial);
+  for (int c = threadIdx.x; c < nchunks; c += 1024) {
+    float4_t q[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      q[j] = (c + 64 * j < nchunks) ? pp[c + 64 * j] : float4_t{1e+8f, -1e+8f, __uint_as_float(0xffffffffu), 0.0f};
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      ex.merge(q[j].x, q[j].y, __float_as_uint(q[j].z), __float_as_uint(q[j].w));
+  }
   ex.wave_reduce();
   if (threadIdx.x != 0)
     return;

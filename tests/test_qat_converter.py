@@ -425,3 +425,42 @@ def test_scheduler_argument_checks():
     cfg.precision_mode = qnn.PrecisionMode.QNN
     with pytest.raises(NotImplementedError):
         GC.QuantizeRecordingToTrainingModifier({}, config=cfg)
+
+
+# ------------------------------------------------------------------------------------------- pins of the oracle
+def test_oracle_recorder_pins():
+    """What fixes ``oracle.range_recorder`` independently of its own text: running extrema are the extrema of
+    everything seen (and of the starting value), a moving average fed a constant follows c (1 - decay^n) -- swapped
+    weights or a dropped term fail it at n = 1 -- and one step from zero gives the fp32 nearest to the double
+    1 - decay (MulScalar casts its Python float once, mul_scalar.hpp), not 1 minus the fp32 decay."""
+    rng = np.random.default_rng(9)
+    batches = [rng.standard_normal((5, 7, 3)).astype(np.float32) * (k + 1) for k in range(4)]
+    m = M = A = X = np.float32(0)
+    for k, x in enumerate(batches):
+        m, M = oracle.range_recorder(x, m, M, 'MinMaxMinMaxRecorder')
+        _, A = oracle.range_recorder(x, None, A, 'AbsMaxRecorder')
+        _, X = oracle.range_recorder(x, None, X, 'MaxMaxRecorder')
+        seen = np.concatenate([b.ravel() for b in batches[:k + 1]] + [np.zeros(1, np.float32)])
+        assert (m, M, A, X) == (seen.min(), seen.max(), np.abs(seen).max(), seen.max())
+    neg = -np.abs(batches[0]) - 1
+    assert oracle.range_recorder(neg, None, np.float32(0), 'MaxMaxRecorder')[1] == 0       # the start value wins
+    assert oracle.range_recorder(neg, None, np.float32(-9), 'MaxMaxRecorder')[1] == neg.max()
+    assert oracle.range_recorder(neg, None, np.float32(0), 'AbsMaxRecorder')[1] == -neg.min()
+
+    x = np.full((3, 4), 0.25, np.float32)
+    x[1, 2], x[2, 0] = 5.0, -2.0
+    for decay in (0.9, 0.75, 0.99):
+        lo = hi = one = np.float32(0)
+        for n in range(1, 30):
+            lo, hi = oracle.range_recorder(x, lo, hi, 'MinMaxMvaRecorder', decay)
+            _, one = oracle.range_recorder(x, None, one, 'MaxMvaRecorder', decay)
+            assert abs(hi - 5.0 * (1 - decay ** n)) < 2e-6 * n and abs(lo + 2.0 * (1 - decay ** n)) < 2e-6 * n
+            assert one == hi
+    unit = np.ones((2, 2), np.float32)
+    got = oracle.range_recorder(unit, None, np.float32(0), 'MaxMvaRecorder', 0.99)[1]
+    assert np.float32(got).view(np.uint32) == 0x3c23d70a                 # fp32(0.01); 1 - fp32(0.99) is 0x3c23d700
+    assert np.float32(1) - np.float32(0.99) != got
+    # from a non-zero start: two products rounded to fp32, then their sum
+    got = oracle.range_recorder(3 * unit, None, np.float32(7), 'MaxMvaRecorder', 0.9)[1]
+    assert got == np.float32(np.float32(np.float32(0.9) * np.float32(7)) + np.float32(np.float32(1.0 - 0.9) * np.float32(3)))
+    assert abs(got - 6.6) < 1e-6
