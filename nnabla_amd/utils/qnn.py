@@ -7,9 +7,9 @@ function ``RangeRecorder`` of the hip extension (one scan kernel), reporting the
 the graph converters recognise it by ``info.type_name``.
 
 Not carried over: batch-normalisation folding (``bn_folding`` / ``bn_self_folding`` are accepted and have nothing to
-act on, since no BatchNormalization function exists on this path), re-registering parameters with a solver, and
-``QATScheduler.save``.
+act on, since no BatchNormalization function exists on this path) and re-registering parameters with a solver.
 """
+from collections import OrderedDict
 from enum import Enum
 
 import numpy as np
@@ -308,4 +308,19 @@ class QATScheduler(object):
         self.counter += 1
 
     def save(self, fname, inputs, batch_size=1, net_name='net', deploy=False):
-        raise NotImplementedError("QATScheduler.save: writing NNP files is not part of this package.")
+        """Writes the registered evaluation network(s) (those registered with ``training=False``) as an NNP file with
+        inputs 'x0', 'x1', ... and outputs 'y0', 'y1', ... (qnn.py:927-1000).  ``deploy=True`` is not available (it
+        is not in the reference either)."""
+        if deploy:
+            raise NotImplementedError("QATScheduler.save: deployment conversion is not supported.")
+        from .save import save
+        inputs = list(inputs) if isinstance(inputs, (list, tuple)) else [inputs]
+        for pred, training in self.registry:
+            if training:
+                continue
+            outputs = list(pred) if isinstance(pred, (list, tuple)) else [pred]
+            names = OrderedDict(('x{}'.format(i), v) for i, v in enumerate(inputs))
+            outs = OrderedDict(('y{}'.format(i), v) for i, v in enumerate(outputs))
+            save(fname, {'networks': [{'name': net_name, 'batch_size': batch_size, 'outputs': outs, 'names': names}],
+                         'executors': [{'name': 'runtime', 'network': net_name, 'data': list(names),
+                                        'output': list(outs)}]})

@@ -80,6 +80,7 @@ class Variable(object):
         self.need_grad = need_grad
         self.parent = None        # the FunctionNode that produces this variable
         self._consumers = []      # weak references to the FunctionNodes that take this variable as an input
+        self._viewed = None       # the variable whose arrays this one views (set by reshape / unlink / rewire_on)
         self.name = ''
         self.persistent = False
 
@@ -88,6 +89,12 @@ class Variable(object):
         if h and _capi._lib is not None:
             _capi._lib.nblac_variable_free(h)
             self._h = None
+
+    @property
+    def _origin(self):
+        """The variable that owns the arrays this one views; itself for an ordinary variable (kept as None inside, so
+        that a variable does not refer to itself and is freed as soon as it is dropped)."""
+        return self if self._viewed is None else self._viewed
 
     @staticmethod
     def from_numpy_array(data, grad=None, need_grad=None):
@@ -122,6 +129,7 @@ class Variable(object):
         """A variable sharing this one's arrays under another shape."""
         v = Variable(shape, self.need_grad)
         _capi.check(_capi.lib().nblac_variable_share(v._h, self._h))
+        v._viewed = self._origin
         if not unlink:
             v.parent = self.parent
         return v
@@ -254,6 +262,7 @@ class Variable(object):
         if tuple(var.shape) != tuple(self.shape):
             raise ValueError("rewire_on: shapes differ, %r and %r" % (self.shape, var.shape))
         _capi.check(_capi.lib().nblac_variable_share(self._h, var._h))
+        self._viewed = var._origin
         node = var.parent
         self.parent = node
         if node is not None:

@@ -370,3 +370,73 @@ def to_np_device(y_rec, scope):
     y_rec.visit(look)
     assert len(found) == 1
     return found[0]
+
+
+# ------------------------------------------------------------------------------------------------- saving as NNP
+def test_scheduler_save_and_reload(ctx, tmp_path):
+    """The evaluation network of a finished schedule written with QATScheduler.save, read back with NnpLoader and
+    executed: the same bits as the graph it was written from."""
+    from nnabla_amd.utils.nnp_graph import NnpLoader
+    rng = np.random.default_rng(5)
+    x = nn.Variable((8, 3, 16, 16))
+    y = small_net(x)
+    randomise_parameters(rng)
+    vx = nn.Variable((4, 3, 16, 16))
+    vy = small_net(vx)                                  # shares the parameters
+    cfg = QATConfig()
+    cfg.recorder_activation = qnn.MaxMaxRecorderCallback
+    cfg.niter_to_recording, cfg.niter_to_training = 0, 3
+    sched = QATScheduler(cfg)
+    sched(y)
+    sched(vy, training=False)
+    for i in range(5):
+        sched.step()
+        x.d = rng.standard_normal(x.shape).astype(np.float32)
+        y.forward()
+    assert sched.state == QNNState.TRAINING
+    data = rng.standard_normal(vx.shape).astype(np.float32)
+    vx.d = data
+    vy.forward()
+    counts = check_every_function(vy)
+    assert counts['QuantizeLinear'] == 9
+
+    path = str(tmp_path / 'qnn.nnp')
+    sched.save(path, vx, batch_size=4)
+    loader = NnpLoader(path)
+    ex = loader.get_executor('runtime')
+    assert list(ex.data_variables) == ['x0'] and list(ex.output_variables) == ['y0']
+    ex.data_variables['x0'].d = data
+    ex.execute()
+    assert bits_equal(ex.output_variables['y0'].d, vy.d), first_mismatch(ex.output_variables['y0'].d, vy.d)
+    names = []
+    ex.output_variables['y0'].visit(lambda f: names.append(f.info.type_name))
+    mine = []
+    vy.visit(lambda f: mine.append(f.info.type_name))
+    assert names == mine
+    assert np.array_equal(loader.get_parameters()['ReLU-1/scale-x0'].d, nn.get_parameter('ReLU-1/scale-x0').d)
+    with pytest.raises(NotImplementedError):
+        sched.save(path, vx, deploy=True)
+
+
+def test_every_function_saved_and_reloaded(ctx, tmp_path):
+    from nnabla_amd.utils.nnp_graph import NnpLoader
+    from nnabla_amd.utils.save import save
+    from test_nnp_save import contents_of, every_function_net
+    x = nn.Variable((6, 3, 6, 6))
+    y = every_function_net(x)
+    for k, v in nn.get_parameters(grad_only=False).items():
+        if k in ('mmq/ql_min', 'ql/z'):
+            v.d = 0
+        elif k == 'mmq/ql_max':
+            v.d = 255
+        elif k == 'ql/s':
+            v.d = 0.05
+    path = str(tmp_path / 'all.nnp')
+    save(path, contents_of(x, y, 6))                   # before any forward: INQ / min-max state as initialised
+    data = np.random.default_rng(1).standard_normal(x.shape).astype(np.float32)
+    x.d = data
+    y.forward()
+    ex = NnpLoader(path).get_executor('runtime')
+    ex.data_variables['x'].d = data
+    ex.execute()
+    assert bits_equal(ex.output_variables['y'].d, y.d), first_mismatch(ex.output_variables['y'].d, y.d)
