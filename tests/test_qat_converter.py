@@ -128,6 +128,21 @@ def test_identity_conversion_copies_the_graph_and_shares_parameters():
     assert all(q is not p and q.parent is None and q.shape == p.shape for p, q in zip(old[0].inputs, new[0].inputs))
 
 
+def test_identity_modifier_replaces_inputs():
+    x = nn.Variable((2, 3, 8, 8))
+    y = small_net(x)
+    x2 = nn.Variable((5, 3, 8, 8))
+    y2 = GC.GraphConverter([GC.IdentityModifier({x: x2})]).convert(y)
+    assert names(y2) == names(y) and y2.shape == (5, 5)
+    first = []
+    y2.visit(first.append)
+    assert first[0].inputs[0] is x2
+    with pytest.raises(ValueError):
+        GC.GraphConverter([GC.IdentityModifier({x: x2}, copy_value=True)]).convert(y)
+    y3 = GC.GraphConverter([GC.IdentityModifier()]).convert(y)
+    assert graph_info(y3) == graph_info(y)
+
+
 def test_modifier_replacing_a_function_and_list_outputs():
     class ReluToPrune(GC.FunctionModifier):
         def modify(self, f, inputs):
