@@ -98,9 +98,9 @@ __device__ __forceinline__ float rounded_quotient(float x, float s, int half_to_
   const float a = fabsf(s);
   if (a >= 0x1p-100f && a <= 0x1p100f) {
     const float q = x * __builtin_amdgcn_rcpf(s);
-    const float t = round_half_away(q);
+    const float t = rintf(q); // away from a tie every rounding mode gives this integer (and the same signed zero)
     const float m = fabsf(q);
-    const float d = fabsf(fabsf(q - t) - 0.5f); // distance from the nearest tie; q - t is exact below 2^23
+    const float d = 0.5f - fabsf(q - t); // distance from the nearest tie; q - t is exact below 2^23
     if (m >= 4096.0f || d > fmaxf(m, 0.5f) * 0x1p-20f)
       return t;
   }
@@ -108,20 +108,76 @@ __device__ __forceinline__ float rounded_quotient(float x, float s, int half_to_
 }
 
 struct QuantizeOp {
+  static constexpr bool kRoundsZeroPoint = false;
+  static constexpr bool kUniform = false;
   int half_to_even;
   float lo, hi;
   __device__ __forceinline__ float operator()(float x, float scale, float zp) const {
     return saturate(rounded_quotient(x, scale, half_to_even) + zp, lo, hi);
   }
 };
+// The same with a one-element zero point that has not been rounded yet: every thread rounds it for itself and one
+// thread stores the rounded value back (quantize_linear.cpp:109-111 rounds the zero point in place).  Threads that
+// read it after that store find a value rounding leaves unchanged.
+struct QuantizeRoundingOp {
+  static constexpr bool kRoundsZeroPoint = true;
+  static constexpr bool kUniform = false;
+  int half_to_even;
+  float lo, hi;
+  __device__ __forceinline__ float zero_point(float zp) const { return saturate(round_mode(zp, half_to_even), lo, hi); }
+  // zp: already rounded by the caller (once per thread)
+  __device__ __forceinline__ float operator()(float x, float scale, float zp) const {
+    return saturate(rounded_quotient(x, scale, half_to_even) + zp, lo, hi);
+  }
+};
+// One scale and one zero point for the whole tensor (what per-tensor quantization-aware training produces): the
+// reciprocal, the range check of the scale and the rounded zero point are worked out once per thread, and no
+// broadcast offsets are computed.
+struct QuantizeUniformOp {
+  static constexpr bool kRoundsZeroPoint = false;
+  static constexpr bool kUniform = true;
+  int half_to_even;
+  float lo, hi;
+  struct State {
+    float s, inv, zp;
+    bool fast;
+  };
+  __device__ __forceinline__ State prepare(float s, float zp_raw) const {
+    State st;
+    const float a = fabsf(s);
+    st.s = s;
+    st.fast = a >= 0x1p-100f && a <= 0x1p100f;
+    st.inv = st.fast ? __builtin_amdgcn_rcpf(s) : 0.0f;
+    st.zp = saturate(round_mode(zp_raw, half_to_even), lo, hi);
+    return st;
+  }
+  __device__ __forceinline__ float apply(float x, const State &st) const { // rounded_quotient with the shared parts
+    if (st.fast) {
+      const float q = x * st.inv;
+      const float t = rintf(q);
+      const float m = fabsf(q);
+      const float d = 0.5f - fabsf(q - t);
+      if (m >= 4096.0f || d > fmaxf(m, 0.5f) * 0x1p-20f)
+        return saturate(t + st.zp, lo, hi);
+    }
+    return saturate(round_mode(divide(x, st.s), half_to_even) + st.zp, lo, hi);
+  }
+  __device__ __forceinline__ float operator()(float x, float scale, float zp) const { return 0.0f; } // not used
+};
 struct DequantizeOp {
+  static constexpr bool kRoundsZeroPoint = false;
+  static constexpr bool kUniform = false;
   __device__ __forceinline__ float operator()(float x, float scale, float zp) const { return (x - zp) * scale; }
 };
 // dx (+)= dy / scale  and  dx (+)= dy * scale  (the zero point is not read)
 struct DivGradOp {
+  static constexpr bool kRoundsZeroPoint = false;
+  static constexpr bool kUniform = false;
   __device__ __forceinline__ float operator()(float dy, float scale, float) const { return divide(dy, scale); }
 };
 struct MulGradOp {
+  static constexpr bool kRoundsZeroPoint = false;
+  static constexpr bool kUniform = false;
   __device__ __forceinline__ float operator()(float dy, float scale, float) const { return dy * scale; }
 };
 
@@ -133,6 +189,39 @@ template <typename Op, bool kVec, bool kAccum, typename Index>
 __global__ __launch_bounds__(kBlock) void broadcast_map(const float *__restrict__ x, const float *__restrict__ scale,
                                                         const float *__restrict__ zp, float *__restrict__ y,
                                                         int64_t count, Broadcast b, Op op) {
+  if constexpr (Op::kUniform) {
+    const auto st = op.prepare(scale[0], zp[0]);
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+      const_cast<float *>(zp)[0] = st.zp;
+    if (kVec) {
+      const int64_t base = (int64_t)blockIdx.x * (kBlock * kUnroll) + threadIdx.x;
+      float4_t v[kUnroll];
+#pragma unroll
+      for (int j = 0; j < kUnroll; ++j)
+        if (base + (int64_t)j * kBlock < count)
+          v[j] = *reinterpret_cast<const float4_t *>(x + 4 * (base + (int64_t)j * kBlock));
+#pragma unroll
+      for (int j = 0; j < kUnroll; ++j) {
+        const int64_t t = base + (int64_t)j * kBlock;
+        if (t < count) {
+          float4_t o;
+          o.x = op.apply(v[j].x, st), o.y = op.apply(v[j].y, st), o.z = op.apply(v[j].z, st), o.w = op.apply(v[j].w, st);
+          __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(y + 4 * t));
+        }
+      }
+    } else {
+      const int64_t step = (int64_t)gridDim.x * kBlock;
+      for (int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x; t < count; t += step)
+        y[t] = op.apply(x[t], st);
+    }
+    return;
+  }
+  float rounded_zp = 0.0f;
+  if constexpr (Op::kRoundsZeroPoint) {
+    rounded_zp = op.zero_point(zp[0]);
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+      const_cast<float *>(zp)[0] = rounded_zp;
+  }
   if (kVec) {
     const int64_t base = (int64_t)blockIdx.x * (kBlock * kUnroll) + threadIdx.x;
     float4_t v[kUnroll], old[kUnroll];
@@ -158,7 +247,9 @@ __global__ __launch_bounds__(kBlock) void broadcast_map(const float *__restrict_
           sv.x = sv.y = sv.z = sv.w = scale[so];
         else
           sv = *reinterpret_cast<const float4_t *>(scale + so);
-        if (!zp)
+        if (Op::kRoundsZeroPoint)
+          zv.x = zv.y = zv.z = zv.w = rounded_zp;
+        else if (!zp)
           zv.x = zv.y = zv.z = zv.w = 0.0f;
         else if (zs == 0)
           zv.x = zv.y = zv.z = zv.w = zp[zo];
@@ -179,7 +270,7 @@ __global__ __launch_bounds__(kBlock) void broadcast_map(const float *__restrict_
     for (int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x; t < count; t += step) {
       int64_t so, zo;
       offsets<Index>(b, (Index)t, so, zo);
-      const float o = op(x[t], scale[so], zp ? zp[zo] : 0.0f);
+      const float o = op(x[t], scale[so], Op::kRoundsZeroPoint ? rounded_zp : (zp ? zp[zo] : 0.0f));
       y[t] = kAccum ? y[t] + o : o;
     }
   }
@@ -432,6 +523,22 @@ int nbla_hip_quantize_linear_f32(const float *x, const float *scale, float *zero
   int64_t zsize = 1;
   for (int i = 0; i < ndim; ++i)
     zsize *= zero_point_shape[i];
+  int64_t xsize = 1;
+  for (int i = 0; i < ndim; ++i)
+    xsize *= xshape[i];
+  int64_t ssize = 1;
+  for (int i = 0; i < ndim; ++i)
+    ssize *= scale_shape[i];
+  if (zsize == 1 && ssize == 1 && xsize > 0) {
+    QuantizeUniformOp op{half_to_even ? 1 : 0, lo, hi};
+    return launch_broadcast(x, scale, zero_point, y, xshape, scale_shape, zero_point_shape, ndim, false, op, stream,
+                            "QuantizeLinear");
+  }
+  if (zsize == 1 && xsize > 0) { // no separate launch for the zero point
+    QuantizeRoundingOp op{half_to_even ? 1 : 0, lo, hi};
+    return launch_broadcast(x, scale, zero_point, y, xshape, scale_shape, zero_point_shape, ndim, false, op, stream,
+                            "QuantizeLinear");
+  }
   if (zsize > 0) {
     int64_t blocks = ceil_div(zsize, (int64_t)kBlock);
     if (blocks > 65536)

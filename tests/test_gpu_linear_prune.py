@@ -6,7 +6,7 @@ import torch
 
 import oracle
 from nnabla_amd import kernels
-from util import bits_equal, to_np
+from util import bits_equal, first_mismatch, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -49,6 +49,24 @@ def test_quantize_linear(dev, xs, ss, zs, mode, narrow, dtype):
     y = kernels.quantize_linear(_dev(x, dev), _dev(scale, dev), dzp, mode, narrow, dtype)
     assert bits_equal(to_np(y), ref)
     assert bits_equal(to_np(dzp), ref_zp)                          # rounded and saturated in place
+
+
+@pytest.mark.parametrize("mode", ["HALF_AWAY_FROM_ZERO", "HALF_TO_EVEN"])
+@pytest.mark.parametrize("scale,zp", [(0.3, 2.5), (0.0371, -3.5), (7.0, 300.0), (1e-30, 0.49), (3e38, -0.5)])
+@pytest.mark.parametrize("n", [1, 5, 4096, 1 << 18, (1 << 18) + 3])
+def test_quantize_linear_one_scale_one_zero_point(dev, mode, scale, zp, n):
+    """Per-tensor parameters (one scale, one unrounded zero point, handled inside the main launch): ties of the zero
+    point, saturating zero points, scales at the ends of the range, vector and element-wise sizes."""
+    with np.errstate(over='ignore'):                       # the largest scale takes some inputs to infinity
+        x = _rand((n,), n % 97, 40.0 * scale if scale < 1e30 else 1e38)
+        x[:min(n, 4)] = np.array([0.5, -0.5, 1.5, 2.5], np.float32)[:min(n, 4)] * np.float32(scale)
+    s, z = np.full((1,), scale, np.float32), np.full((1,), zp, np.float32)
+    for dtype, narrow in ((1, False), (2, True)):
+        ref, ref_zp = oracle.quantize_linear(x, s, z, mode, narrow, dtype)
+        dz = _dev(z, dev)
+        y = kernels.quantize_linear(_dev(x, dev), _dev(s, dev), dz, mode, narrow, dtype)
+        assert bits_equal(to_np(y), ref), first_mismatch(to_np(y), ref)
+        assert bits_equal(to_np(dz), ref_zp)
 
 
 @pytest.mark.parametrize("xs,ss,zs", SHAPES)
