@@ -1,1 +1,2 @@
-"""Utilities around the function path: NNP / nntxt graph files."""
+"""Utilities around the function path: NNP / nntxt graph files (``nnp_graph``, ``nnp_format``, ``save``) and
+quantization-aware training (``qnn``)."""
