@@ -353,7 +353,10 @@ int quantize_range(int dtype, int narrow_range, float &lo, float &hi) {
 // copy) and takes a ticket; the block holding the last ticket scans the finished histogram and records the chosen
 // digit and the rank left inside it for the next pass.
 constexpr int kPasses = 3, kMaxBins = 2048, kLdsCopies = 4, kGlobalCopies = 8;
-constexpr int kSelectBlocks = 512;
+constexpr int kSelectBlocks = 256;
+// 256 histogram blocks of 1024 threads: one per CU; the block that finishes a pass scans the bins with all its
+// threads, and fewer blocks mean fewer counter updates (measured against 512 x 256, 512 x 512, 1024 x 512, 512 x 1024)
+constexpr int kHistBlock = 1024;
 struct SelectState {
   uint32_t hist[kPasses][kGlobalCopies][kMaxBins];
   uint32_t done[kPasses];       // blocks of pass p that have added their counters
@@ -376,11 +379,11 @@ __global__ __launch_bounds__(kBlock) void clear_select(SelectState *st, uint32_t
   }
 }
 
-__global__ __launch_bounds__(kBlock) void prune_histogram(const float *__restrict__ x, int64_t n4, int64_t n,
+__global__ __launch_bounds__(kHistBlock) void prune_histogram(const float *__restrict__ x, int64_t n4, int64_t n,
                                                           SelectState *__restrict__ st, int pass) {
   __shared__ uint32_t h[kMaxBins * kLdsCopies];
-  __shared__ uint32_t scratch[kBlock / 64 + 1];
-  for (int i = threadIdx.x; i < kMaxBins * kLdsCopies; i += kBlock)
+  __shared__ uint32_t scratch[kHistBlock / 64 + 1];
+  for (int i = threadIdx.x; i < kMaxBins * kLdsCopies; i += kHistBlock)
     h[i] = 0u;
   const uint32_t prefix = st->prefix[pass], rank = st->rank[pass];
   __syncthreads();
@@ -393,17 +396,17 @@ __global__ __launch_bounds__(kBlock) void prune_histogram(const float *__restric
       atomicAdd(&h[((key >> shift) & mask) * kLdsCopies + copy], 1u);
   };
   // four loads in flight per thread before the counters are touched
-  const int64_t tiles = (n4 + kBlock * 4 - 1) / (kBlock * 4);
+  const int64_t tiles = (n4 + kHistBlock * 4 - 1) / (kHistBlock * 4);
   for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-    const int64_t base = tile * (kBlock * 4) + threadIdx.x;
+    const int64_t base = tile * (kHistBlock * 4) + threadIdx.x;
     float4_t v[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      if (base + j * kBlock < n4)
-        v[j] = *reinterpret_cast<const float4_t *>(x + 4 * (base + j * kBlock));
+      if (base + j * kHistBlock < n4)
+        v[j] = *reinterpret_cast<const float4_t *>(x + 4 * (base + j * kHistBlock));
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      if (base + j * kBlock < n4)
+      if (base + j * kHistBlock < n4)
         count(v[j].x), count(v[j].y), count(v[j].z), count(v[j].w);
   }
   if (blockIdx.x == 0) {
@@ -413,7 +416,7 @@ __global__ __launch_bounds__(kBlock) void prune_histogram(const float *__restric
   }
   __syncthreads();
   uint32_t *g = st->hist[pass][blockIdx.x % kGlobalCopies];
-  for (int b = threadIdx.x; b < bins; b += kBlock) {
+  for (int b = threadIdx.x; b < bins; b += kHistBlock) {
     const uint4_t c = *reinterpret_cast<const uint4_t *>(&h[b * kLdsCopies]);
     const uint32_t total = c.x + c.y + c.z + c.w;
     if (total)
@@ -425,20 +428,24 @@ __global__ __launch_bounds__(kBlock) void prune_histogram(const float *__restric
   // involved, which a fence in every block would cost.
   __syncthreads();
   if (threadIdx.x == 0)
-    scratch[kBlock / 64] = atomicAdd(&st->done[pass], 1u);
+    scratch[kHistBlock / 64] = atomicAdd(&st->done[pass], 1u);
   __syncthreads();
-  if (scratch[kBlock / 64] != gridDim.x - 1)
+  if (scratch[kHistBlock / 64] != gridDim.x - 1)
     return;
-  // thread t owns the bins [t * per, (t + 1) * per), per = 8 or 4
-  const int per = bins / kBlock, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  uint32_t c[kMaxBins / kBlock];
+  // thread t owns the bins [t * per, (t + 1) * per), per = 2 or 1
+  const int per = bins / kHistBlock, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint32_t c[kMaxBins / kHistBlock];
 #pragma unroll
-  for (int i = 0; i < kMaxBins / kBlock; ++i)
+  for (int i = 0; i < kMaxBins / kHistBlock; ++i)
     c[i] = 0u;
   for (int k = 0; k < kGlobalCopies; ++k) {
     const unsigned long long *src = reinterpret_cast<const unsigned long long *>(&st->hist[pass][k][threadIdx.x * per]);
+    if (per == 1) {
+      c[0] += __hip_atomic_load(&st->hist[pass][k][threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      continue;
+    }
 #pragma unroll
-    for (int i = 0; i < kMaxBins / kBlock / 2; ++i)
+    for (int i = 0; i < kMaxBins / kHistBlock / 2; ++i)
       if (2 * i < per) {
         const unsigned long long two = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         c[2 * i] += (uint32_t)two;
@@ -447,7 +454,7 @@ __global__ __launch_bounds__(kBlock) void prune_histogram(const float *__restric
   }
   uint32_t mine = 0;
 #pragma unroll
-  for (int i = 0; i < kMaxBins / kBlock; ++i)
+  for (int i = 0; i < kMaxBins / kHistBlock; ++i)
     mine += c[i];
   uint32_t incl = mine;
 #pragma unroll
@@ -463,7 +470,7 @@ __global__ __launch_bounds__(kBlock) void prune_histogram(const float *__restric
   for (int w = 0; w < wave; ++w)
     excl += scratch[w];
 #pragma unroll
-  for (int i = 0; i < kMaxBins / kBlock; ++i) {
+  for (int i = 0; i < kMaxBins / kHistBlock; ++i) {
     if (c[i] != 0u && excl <= rank && rank < excl + c[i]) {
       st->prefix[pass + 1] = prefix | ((uint32_t)(threadIdx.x * per + i) << shift);
       st->rank[pass + 1] = rank - excl;
@@ -605,14 +612,14 @@ int nbla_hip_prune_f32(const float *x, float *y, size_t size, float rate, void *
   const uint32_t rank = (uint32_t)(int)((x_size - 1) * rate);
   const int64_t n = (int64_t)size;
   const int64_t n4 = n / 4;
-  int64_t blocks = ceil_div(n4 ? n4 : 1, (int64_t)kBlock * 4);
+  int64_t blocks = ceil_div(n4 ? n4 : 1, (int64_t)kHistBlock * 4);
   if (blocks > kSelectBlocks)
     blocks = kSelectBlocks;
   hipLaunchKernelGGL(clear_select, dim3((unsigned)ceil_div(kPasses * kGlobalCopies * kMaxBins, kBlock)), dim3(kBlock), 0,
                      stream, st, rank);
   NBLA_HIP_LAUNCH_CHECK("clear_select");
   for (int p = 0; p < kPasses; ++p) {
-    hipLaunchKernelGGL(prune_histogram, dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, n4, n, st, p);
+    hipLaunchKernelGGL(prune_histogram, dim3((unsigned)blocks), dim3(kHistBlock), 0, stream, x, n4, n, st, p);
     NBLA_HIP_LAUNCH_CHECK("prune_histogram");
   }
   int64_t ablocks = ceil_div(n4 ? n4 : 1, (int64_t)kBlock * 4);
