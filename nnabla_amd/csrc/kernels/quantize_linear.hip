@@ -348,11 +348,11 @@ int quantize_range(int dtype, int narrow_range, float &lo, float &hi) {
 
 // Radix select of the rank-th smallest magnitude: three passes over the 31 magnitude bits (11, 10, 10), each
 // histogramming the digit of the elements that share the digits chosen so far.  A block counts in LDS (four copies
-// of the counters, copy = lane % 4), adds its non-zero counters to one of eight global copies (a counter that every
+// of the counters, copy = lane % 4), adds its non-zero counters to one of four global copies (a counter that every
 // block of the grid updates is a serial chain of device-wide atomics, 15 ns each: the dominant cost with a single
 // copy) and takes a ticket; the block holding the last ticket scans the finished histogram and records the chosen
 // digit and the rank left inside it for the next pass.
-constexpr int kPasses = 3, kMaxBins = 2048, kLdsCopies = 4, kGlobalCopies = 8;
+constexpr int kPasses = 3, kMaxBins = 2048, kLdsCopies = 4, kGlobalCopies = 4;
 constexpr int kSelectBlocks = 256;
 // 256 histogram blocks of 1024 threads: one per CU; the block that finishes a pass scans the bins with all its
 // threads, and fewer blocks mean fewer counter updates (measured against 512 x 256, 512 x 512, 1024 x 512, 512 x 1024)
