@@ -103,6 +103,29 @@ int nbla_hip_min_max_quantize_f32(const float *x, float *y,
                                   float eps, void *workspace,
                                   size_t workspace_bytes, void *stream);
 
+/* The same forward for callers that cannot allocate device memory or carry a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  It has no counterpart in the reference.  The reduction
+ * partials and the nudged-range table live in a fixed array of
+ * NBLA_HIP_STATIC_SCRATCH_BYTES inside the library, one copy per device, held
+ * until the process ends; nbla_hip_init(device) must have run for the current
+ * device (it resolves that device's copy), and the call itself allocates
+ * nothing.  Shapes whose scratch (nbla_hip_min_max_quantize_workspace_bytes)
+ * exceeds the array -- more than 8192 quantization ranges -- return
+ * NBLA_HIP_ERR_MEMORY.  All calls on one device share the array: calls that
+ * overlap on one device (different streams or threads) race; calls on one
+ * stream are ordered.  Nothing in the array has to be cleared between calls
+ * (every word read is written earlier in the same call).  Results are
+ * bit-identical to nbla_hip_min_max_quantize_f32. */
+#define NBLA_HIP_STATIC_SCRATCH_BYTES (256 * 1024)
+int nbla_hip_min_max_quantize_static_f32(const float *x, float *y,
+                                         const int64_t *xshape, int ndim,
+                                         const int64_t *qshape, float *qr_min,
+                                         float *qr_max, const float *ql_min,
+                                         const float *ql_max, float *scale,
+                                         float decay, int x_min_max, int ema,
+                                         float eps, void *stream);
+
 /* ------------------------------------------------ quantizers: backward (STE) */
 
 /* dx (+)= dy inside [min, max], 0 outside (an accumulated dx is left alone

@@ -18,6 +18,10 @@ int fail_hip(hipError_t err, const char *what);
 // Makes sure the current device has been initialised (tables uploaded).
 int ensure_init();
 
+// Resolves, once per device and with that device current, the address of the fixed scratch array behind
+// nbla_hip_min_max_quantize_static_f32 (defined beside that array).  Called by nbla_hip_init.
+int register_static_scratch(int device);
+
 // Number of binades a positive finite fp32 value can fall into: 23 subnormal
 // binades (leading bit 0..22) followed by exponent fields 1..254.
 constexpr int kNumBinades = 277;

@@ -157,6 +157,9 @@ int nbla_hip_init(int device) {
   if (e != hipSuccess)
     return fail_hip(e, "hipMemcpy(cut tables)");
   g_device_tables[device] = static_cast<const uint32_t *>(sym);
+  const int rc_scratch = register_static_scratch(device);
+  if (rc_scratch)
+    return rc_scratch;
   g_device_ready[device] = true;
   return NBLA_HIP_OK;
 }

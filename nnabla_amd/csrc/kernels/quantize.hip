@@ -7,6 +7,7 @@
 
 #include <cmath>
 #include <cstring>
+#include <mutex>
 
 namespace nbla_hip {
 namespace {
@@ -617,20 +618,14 @@ __global__ __launch_bounds__(kBlock) void minmax_apply_generic(const float *__re
   }
 }
 
-} // namespace
-} // namespace nbla_hip
 
-extern "C" {
-
-size_t nbla_hip_min_max_quantize_workspace_bytes(const int64_t *xshape, int ndim, const int64_t *qshape) {
-  const MinMaxPlan P = make_plan(xshape, ndim, qshape);
-  return P.params_bytes + P.partial_bytes;
-}
-
-int nbla_hip_min_max_quantize_f32(const float *x, float *y, const int64_t *xshape, int ndim, const int64_t *qshape,
-                                  float *qr_min, float *qr_max, const float *ql_min, const float *ql_max, float *scale,
-                                  float decay, int x_min_max, int ema, float eps, void *workspace,
-                                  size_t workspace_bytes, void *stream_) {
+// The whole forward on caller-provided scratch (`workspace`: the nudged-range table, then the reduction partials).
+// Every word of the scratch that a launch reads has been written earlier in the same call, so nothing has to start
+// at zero.  `scratch_limit` != 0 marks the fixed-size scratch of the allocation-free entry point.
+int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, int ndim, const int64_t *qshape,
+                             float *qr_min, float *qr_max, const float *ql_min, const float *ql_max, float *scale,
+                             float decay, int x_min_max, int ema, float eps, void *workspace, size_t workspace_bytes,
+                             size_t scratch_limit, void *stream_) {
   for (int i = 0; i < ndim; ++i)
     if (qshape[i] != 1 && qshape[i] != xshape[i])
       return fail(NBLA_HIP_ERR_VALUE,
@@ -643,6 +638,11 @@ int nbla_hip_min_max_quantize_f32(const float *x, float *y, const int64_t *xshap
     return NBLA_HIP_OK;
   if (P.L.R0 * P.L.R1 > 0xffffffffll)
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "reduction slices above 2^32 elements are not supported.");
+  if (scratch_limit && P.params_bytes + P.partial_bytes > scratch_limit)
+    return fail(NBLA_HIP_ERR_MEMORY,
+                "min_max_quantize: %lld quantization ranges need %zu bytes of scratch, above the %zu bytes of the "
+                "allocation-free entry point; use nbla_hip_min_max_quantize_f32 with a workspace.",
+                (long long)P.L.K, P.params_bytes + P.partial_bytes, scratch_limit);
   if (workspace_bytes < P.params_bytes + P.partial_bytes || !aligned256(workspace))
     return fail(NBLA_HIP_ERR_MEMORY, "min_max_quantize workspace too small or misaligned.");
   int rc = ensure_init();
@@ -705,6 +705,77 @@ int nbla_hip_min_max_quantize_f32(const float *x, float *y, const int64_t *xshap
   }
   NBLA_HIP_LAUNCH_CHECK("min_max_quantize apply");
   return NBLA_HIP_OK;
+}
+
+// ---- scratch of the allocation-free entry point: one copy per device that loads this library, held until the
+// process ends.  Host code never uses the array's name as an address: the per-device address comes from
+// hipGetSymbolAddress, once per device, and is what the kernels receive.
+constexpr size_t kStaticScratchBytes = NBLA_HIP_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxScratchDevices = 64;
+std::mutex g_scratch_mutex;
+std::atomic<void *> g_scratch_ptr[kMaxScratchDevices] = {};
+
+} // namespace
+
+int register_static_scratch(int device) {
+  if (device < 0 || device >= kMaxScratchDevices)
+    return fail(NBLA_HIP_ERR_VALUE, "device index %d out of range", device);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device].load(std::memory_order_acquire))
+    return NBLA_HIP_OK;
+  int current = -1;
+  hipError_t e = hipGetDevice(&current);
+  if (e != hipSuccess)
+    return fail_hip(e, "hipGetDevice");
+  if (current != device)
+    return fail(NBLA_HIP_ERR_RUNTIME, "static scratch of device %d asked for while device %d is current", device,
+                current);
+  void *ptr = nullptr;
+  e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess)
+    return fail_hip(e, "hipGetSymbolAddress(static scratch)");
+  if (!ptr || !aligned256(ptr))
+    return fail(NBLA_HIP_ERR_RUNTIME, "static scratch of device %d resolved to a null or misaligned address", device);
+  g_scratch_ptr[device].store(ptr, std::memory_order_release);
+  return NBLA_HIP_OK;
+}
+
+} // namespace nbla_hip
+
+extern "C" {
+
+size_t nbla_hip_min_max_quantize_workspace_bytes(const int64_t *xshape, int ndim, const int64_t *qshape) {
+  const MinMaxPlan P = make_plan(xshape, ndim, qshape);
+  return P.params_bytes + P.partial_bytes;
+}
+
+int nbla_hip_min_max_quantize_f32(const float *x, float *y, const int64_t *xshape, int ndim, const int64_t *qshape,
+                                  float *qr_min, float *qr_max, const float *ql_min, const float *ql_max, float *scale,
+                                  float decay, int x_min_max, int ema, float eps, void *workspace,
+                                  size_t workspace_bytes, void *stream_) {
+  return min_max_quantize_forward(x, y, xshape, ndim, qshape, qr_min, qr_max, ql_min, ql_max, scale, decay, x_min_max,
+                                  ema, eps, workspace, workspace_bytes, 0, stream_);
+}
+
+int nbla_hip_min_max_quantize_static_f32(const float *x, float *y, const int64_t *xshape, int ndim,
+                                         const int64_t *qshape, float *qr_min, float *qr_max, const float *ql_min,
+                                         const float *ql_max, float *scale, float decay, int x_min_max, int ema,
+                                         float eps, void *stream_) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess)
+    return fail_hip(e, "hipGetDevice");
+  if (dev < 0 || dev >= kMaxScratchDevices)
+    return fail(NBLA_HIP_ERR_VALUE, "device index %d out of range", dev);
+  void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr)
+    return fail(NBLA_HIP_ERR_RUNTIME,
+                "nbla_hip_min_max_quantize_static_f32: call nbla_hip_init(%d) first (it resolves the device's "
+                "scratch address; this entry point does no set-up of its own).", dev);
+  return min_max_quantize_forward(x, y, xshape, ndim, qshape, qr_min, qr_max, ql_min, ql_max, scale, decay, x_min_max,
+                                  ema, eps, ptr, kStaticScratchBytes, kStaticScratchBytes, stream_);
 }
 
 } // extern "C"

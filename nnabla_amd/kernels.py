@@ -22,6 +22,7 @@ EXPORTED = (
     "nbla_hip_init", "nbla_hip_last_error", "nbla_hip_version", "nbla_hip_cut_table",
     "nbla_hip_fixed_point_quantize_f32", "nbla_hip_pow2_quantize_f32",
     "nbla_hip_min_max_quantize_workspace_bytes", "nbla_hip_min_max_quantize_f32",
+    "nbla_hip_min_max_quantize_static_f32",
     "nbla_hip_fixed_point_quantize_backward_f32", "nbla_hip_pow2_quantize_backward_f32",
     "nbla_hip_min_max_quantize_backward_workspace_bytes", "nbla_hip_min_max_quantize_backward_f32",
     "nbla_hip_packed_bits_bytes", "nbla_hip_digit_operand_bytes",
@@ -151,6 +152,17 @@ def min_max_quantize(x, qr_min, qr_max, ql_min, ql_max, decay=0.999, x_min_max=F
                                               _p(ql_max), _p(scale), ctypes.c_float(decay), int(x_min_max), int(ema),
                                               ctypes.c_float(eps), _p(ws), ctypes.c_size_t(ws.numel()),
                                               _stream(stream)))
+    return y, scale
+
+
+def min_max_quantize_static(x, qr_min, qr_max, ql_min, ql_max, scale, y, decay=0.999, x_min_max=False, ema=False,
+                            eps=0.01, stream=None):
+    """The allocation-free variant: every buffer, outputs included, comes from the caller; the library's fixed
+    per-device scratch replaces the workspace.  ``init(device)`` must have run."""
+    xs, qs = _shape(x.shape), _shape(qr_min.shape)
+    check(lib().nbla_hip_min_max_quantize_static_f32(_p(x), _p(y), xs, x.dim(), qs, _p(qr_min), _p(qr_max),
+                                                     _p(ql_min), _p(ql_max), _p(scale), ctypes.c_float(decay),
+                                                     int(x_min_max), int(ema), ctypes.c_float(eps), _stream(stream)))
     return y, scale
 
 
