@@ -422,10 +422,15 @@ __global__ __launch_bounds__(kHistBlock) void prune_histogram(const float *__res
     if (total)
       atomicAdd(&g[b], total);
   }
-  // The ticket follows this block's counter updates: the barrier waits until every one of them has been performed
-  // (device-wide atomics act on memory itself, past the per-XCD L2), so whoever draws the last ticket finds all
-  // blocks' counts there and reads them the same way, with atomic loads.  No cache write-back or invalidation is
-  // involved, which a fence in every block would cost.
+  // The ticket must follow this block's counter updates.  A workgroup barrier alone does not order that: it makes no
+  // wavefront wait for its own outstanding no-return atomics.  So every wavefront first waits until the memory system
+  // has acknowledged all of its vector memory operations (vmcnt(0): a device-scope atomic is acknowledged once it has
+  // been performed at the device's coherence point, past the per-XCD L2), then the barrier collects the wavefronts,
+  // and only then the ticket is drawn.  Whoever draws the last ticket therefore finds every block's counts in place
+  // and reads them with device-scope atomic loads.  No cache write-back or invalidation is involved (the payload is
+  // atomics only), which a release / acquire fence per block would cost.
+  __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0), expcnt / lgkmcnt untouched
+  asm volatile("" ::: "memory");
   __syncthreads();
   if (threadIdx.x == 0)
     scratch[kHistBlock / 64] = atomicAdd(&st->done[pass], 1u);
