@@ -8,13 +8,17 @@
 #include <nbla/function/binary_weight_affine.hpp>
 #include <nbla/function/binary_weight_convolution.hpp>
 #include <nbla/function/convolution.hpp>
+#include <nbla/function/dequantize_linear.hpp>
 #include <nbla/function/fixed_point_quantize.hpp>
 #include <nbla/function/inq_affine.hpp>
 #include <nbla/function/inq_convolution.hpp>
 #include <nbla/function/min_max_quantize.hpp>
 #include <nbla/function/pow2_quantize.hpp>
+#include <nbla/function/prune.hpp>
 #include <nbla/function/quantize_linear.hpp>
-#include <nbla/function/range_recorder.hpp>
+#include <nbla/function/relu.hpp>
+#include <nbla/function/sink.hpp>
+#include <nbla/hip/function/range_recorder.hpp>
 #include <nbla/hip/init.hpp>
 #include <nbla/init.hpp>
 

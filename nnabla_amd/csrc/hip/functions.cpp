@@ -6,8 +6,14 @@
 #include <nbla/hip/function/quantize.hpp>
 #include <nbla/hip/function/quantize_linear.hpp>
 #include <nbla/hip/function/range_recorder.hpp>
+#include <nbla/random_manager.hpp>
+
+#include <algorithm>
+#include <random>
 
 namespace nbla {
+
+NBLA_REGISTER_FUNCTION_SOURCE(RangeRecorder, int, double, bool);
 
 namespace {
 vector<int64_t> to_i64(const Shape_t &s) { return vector<int64_t>(s.begin(), s.end()); }
@@ -29,6 +35,24 @@ template <typename T> void Pow2QuantizeHip<T>::forward_impl(const Variables &inp
   T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
   NBLA_HIP_CALL(nbla_hip_pow2_quantize_f32(x, y, (size_t)inputs[0]->size(), this->sign_, this->with_zero_, this->n_,
                                            this->m_, nullptr));
+}
+
+// min_max_quantize.cpp:45-127: the shape checks; none of the helper functions the CPU class creates is needed.
+template <typename T> void MinMaxQuantizeHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
+  auto x = inputs[0];
+  auto qr_min = inputs[1], qr_max = inputs[2], ql_min = inputs[3], ql_max = inputs[4];
+  NBLA_CHECK(ql_min->ndim() == ql_max->ndim() && ql_max->ndim() == qr_min->ndim() && qr_min->ndim() == qr_max->ndim(),
+             error_code::value, "All input dimensions must be same.");
+  NBLA_CHECK(ql_min->shape() == ql_max->shape() && ql_max->shape() == qr_min->shape() &&
+                 qr_min->shape() == qr_max->shape(),
+             error_code::value, "All shapes among ql_min, ql_max, qr_min, and qr_max must be same.");
+  NBLA_CHECK(x->ndim() == ql_min->ndim(), error_code::value, "x and ql_min must have the same number of dimensions.");
+  for (Size_t i = 0; i < ql_min->ndim(); i++) {
+    NBLA_CHECK(ql_min->shape()[i] == 1 || x->shape()[i] == ql_min->shape()[i], error_code::value,
+               "x.shape and ql_min.shape must be same except for i-th dimension where ql_min.shape[i] == 1.");
+  }
+  outputs[0]->reshape(x->shape(), true);
+  this->scale_sptr_ = make_shared<Variable>(ql_min->shape());
 }
 
 template <typename T> void MinMaxQuantizeHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
@@ -108,10 +132,31 @@ void MinMaxQuantizeHip<T>::backward_impl(const Variables &inputs, const Variable
 }
 
 // ------------------------------------------------------------- binary affine
+// binary_weight_affine.cpp:32-72
+template <typename T> void BinaryWeightAffineHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
+  shapes_ = infer_affine_shapes(this->base_axis_, inputs[0], inputs[1], inputs.size() == 5 ? inputs[4] : nullptr);
+  this->base_axis_ = shapes_.base_axis;
+  this->w_row_ = shapes_.w_row;
+  this->w_col_ = shapes_.w_col;
+  NBLA_CHECK(inputs[1]->shape() == inputs[2]->shape(), error_code::value,
+             "Binary and float weights must have same size.");
+  NBLA_CHECK(inputs[3]->size() == shapes_.w_col, error_code::value, "Size of alpha must be equal to output size.");
+  outputs[0]->reshape(shapes_.out_shape, true);
+}
+
+// binary_connect_affine.cpp:29-57
+template <typename T> void BinaryConnectAffineHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
+  shapes_ = infer_affine_shapes(this->base_axis_, inputs[0], inputs[1], inputs.size() == 4 ? inputs[3] : nullptr);
+  this->base_axis_ = shapes_.base_axis;
+  NBLA_CHECK(inputs[1]->shape() == inputs[2]->shape(), error_code::value,
+             "Binary and float weights must have same size.");
+  outputs[0]->reshape(shapes_.out_shape, true);
+}
+
 template <typename T>
 void BinaryWeightAffineHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
   hip_set_device(this->ctx_);
-  const AffineShapes &s = this->shapes_;
+  const AffineShapes &s = shapes_;
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
   const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
   T *wb = inputs[2]->cast_data_and_get_pointer<T>(this->ctx_, true);
@@ -126,7 +171,7 @@ void BinaryWeightAffineHip<T>::forward_impl(const Variables &inputs, const Varia
 template <typename T>
 void BinaryConnectAffineHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
   hip_set_device(this->ctx_);
-  const AffineShapes &s = this->shapes_;
+  const AffineShapes &s = shapes_;
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
   const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
   T *wb = inputs[2]->cast_data_and_get_pointer<T>(this->ctx_, true);
@@ -161,7 +206,7 @@ void affine_backward_common(const Context &ctx, const AffineShapes &s, const Var
 template <typename T>
 void BinaryWeightAffineHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
                                              const vector<bool> &propagate_down, const vector<bool> &accum) {
-  const AffineShapes &s = this->shapes_;
+  const AffineShapes &s = shapes_;
   affine_backward_common<T>(this->ctx_, s, inputs, outputs, propagate_down, accum, 4,
                             [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
                               const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
@@ -177,7 +222,7 @@ void BinaryWeightAffineHip<T>::backward_impl(const Variables &inputs, const Vari
 template <typename T>
 void BinaryConnectAffineHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
                                               const vector<bool> &propagate_down, const vector<bool> &accum) {
-  const AffineShapes &s = this->shapes_;
+  const AffineShapes &s = shapes_;
   affine_backward_common<T>(this->ctx_, s, inputs, outputs, propagate_down, accum, 3,
                             [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
                               const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
@@ -189,10 +234,36 @@ void BinaryConnectAffineHip<T>::backward_impl(const Variables &inputs, const Var
 }
 
 // -------------------------------------------------------- binary convolution
+// binary_weight_convolution.cpp:33-70
+template <typename T>
+void BinaryWeightConvolutionHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
+  shapes_ = infer_conv_shapes(this->base_axis_, this->pad_, this->stride_, this->dilation_, this->group_, inputs[0],
+                              inputs[1], inputs.size() == 5 ? inputs[4] : nullptr);
+  this->base_axis_ = shapes_.base_axis;
+  this->channels_o_ = (int)shapes_.channels_o;
+  this->col_w_ = (int)shapes_.inner_size_k;
+  NBLA_CHECK(inputs[1]->shape() == inputs[2]->shape(), error_code::value,
+             "Binary and float weights must have same size.");
+  NBLA_CHECK(inputs[3]->size() == shapes_.channels_o, error_code::value,
+             "Size of alpha must be equal to the number of output channels.");
+  outputs[0]->reshape(shapes_.out_shape, true);
+}
+
+// binary_connect_convolution.cpp:35-65
+template <typename T>
+void BinaryConnectConvolutionHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
+  shapes_ = infer_conv_shapes(this->base_axis_, this->pad_, this->stride_, this->dilation_, this->group_, inputs[0],
+                              inputs[1], inputs.size() == 4 ? inputs[3] : nullptr);
+  this->base_axis_ = shapes_.base_axis;
+  NBLA_CHECK(inputs[1]->shape() == inputs[2]->shape(), error_code::value,
+             "Binary and float weights must have same size.");
+  outputs[0]->reshape(shapes_.out_shape, true);
+}
+
 template <typename T>
 void BinaryWeightConvolutionHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
   hip_set_device(this->ctx_);
-  const ConvShapes &s = this->shapes_;
+  const ConvShapes &s = shapes_;
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
   const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
   T *wb = inputs[2]->cast_data_and_get_pointer<T>(this->ctx_, true);
@@ -212,7 +283,7 @@ void BinaryWeightConvolutionHip<T>::forward_impl(const Variables &inputs, const 
 template <typename T>
 void BinaryConnectConvolutionHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
   hip_set_device(this->ctx_);
-  const ConvShapes &s = this->shapes_;
+  const ConvShapes &s = shapes_;
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
   const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
   T *wb = inputs[2]->cast_data_and_get_pointer<T>(this->ctx_, true);
@@ -256,7 +327,7 @@ void conv_backward_common(const Context &ctx, const ConvShapes &s, const Variabl
 template <typename T>
 void BinaryWeightConvolutionHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
                                                   const vector<bool> &propagate_down, const vector<bool> &accum) {
-  const ConvShapes &s = this->shapes_;
+  const ConvShapes &s = shapes_;
   conv_backward_common<T>(
       this->ctx_, s, inputs, outputs, propagate_down, accum, 4,
       [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
@@ -274,7 +345,7 @@ void BinaryWeightConvolutionHip<T>::backward_impl(const Variables &inputs, const
 template <typename T>
 void BinaryConnectConvolutionHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
                                                    const vector<bool> &propagate_down, const vector<bool> &accum) {
-  const ConvShapes &s = this->shapes_;
+  const ConvShapes &s = shapes_;
   conv_backward_common<T>(
       this->ctx_, s, inputs, outputs, propagate_down, accum, 3,
       [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
@@ -289,19 +360,78 @@ void BinaryConnectConvolutionHip<T>::backward_impl(const Variables &inputs, cons
 
 // ----------------------------------------------------------------------- INQ
 namespace {
-// The Bernoulli stream of inq_affine.cpp:147: rdist_(rgen), one draw per learnable weight.
+// Steps A, B, D and F of INQAffine<T, T1>::setup_impl (inq_affine.cpp:34-79; the same in inq_convolution.cpp:35-102):
+// indicator shape, selection algorithm, the generator of the "random" selection, counter and snapshots.
+void inq_setup_state(Variable *weights, Variable *indicators, const string &selection_algorithm, int seed,
+                     std::mt19937 &rgen, std::bernoulli_distribution &rdist, int &minibatch_counter,
+                     Variable &old_weights, Variable &old_indicators) {
+  NBLA_CHECK(weights->shape().size() == indicators->shape().size(), error_code::value,
+             "Indicators and weights must have same size. Ndim of weights: %d != ndim of indicators: %d.",
+             (int)weights->shape().size(), (int)indicators->shape().size());
+  NBLA_CHECK(weights->shape() == indicators->shape(), error_code::value,
+             "Indicators and weights must have same size.");
+  NBLA_CHECK(selection_algorithm == "largest_abs" || selection_algorithm == "random", error_code::value,
+             "Provided value for selection algorithm not valid: %s. Valid values are \"largest_abs\" and \"random\".",
+             selection_algorithm.c_str());
+  if (selection_algorithm == "random") {
+    std::random_device rdev;
+    rgen = std::mt19937(seed == -1 ? rdev() : (unsigned)seed);
+    rdist = std::bernoulli_distribution(0.5);
+  }
+  minibatch_counter = 0;
+  old_weights.reshape(weights->shape(), true);
+  old_indicators.reshape(weights->shape(), true);
+  old_indicators.data()->zero();
+}
+
+// The indicator update the current minibatch calls for (inq_affine.cpp:104-113): 0 none, 1 fix all, 2 largest_abs,
+// 3 random.
+int inq_current_step(const vector<int> &inq_iterations, int minibatch_counter, const string &selection_algorithm) {
+  if (std::find(inq_iterations.begin(), inq_iterations.end(), minibatch_counter) == inq_iterations.end())
+    return 0;
+  if (inq_iterations.back() == minibatch_counter)
+    return 1;
+  return selection_algorithm == "largest_abs" ? 2 : 3;
+}
+
+// The Bernoulli stream of inq_affine.cpp:84-86,147: rdist_(rgen), one draw per learnable weight, from the
+// process-wide generator when the seed is -1.
+struct InqDraw {
+  std::mt19937 *gen;
+  std::bernoulli_distribution *dist;
+};
 void draw_bernoulli(void *ctx, uint8_t *out, int64_t count) {
-  InqState *s = static_cast<InqState *>(ctx);
-  std::mt19937 &gen = s->generator();
+  InqDraw *d = static_cast<InqDraw *>(ctx);
   for (int64_t i = 0; i < count; ++i)
-    out[i] = s->rdist_(gen) ? 1 : 0;
+    out[i] = (*d->dist)(*d->gen) ? 1 : 0;
 }
 } // namespace
+
+// inq_affine.cpp:34-79
+template <typename T, typename T1>
+void INQAffineHip<T, T1>::setup_impl(const Variables &inputs, const Variables &outputs) {
+  shapes_ = infer_affine_shapes(this->base_axis_, inputs[0], inputs[1], inputs.size() == 4 ? inputs[3] : nullptr);
+  this->base_axis_ = shapes_.base_axis;
+  outputs[0]->reshape(shapes_.out_shape, true);
+  inq_setup_state(inputs[1], inputs[2], this->selection_algorithm_, this->seed_, this->rgen_, this->rdist_,
+                  this->minibatch_counter_, this->old_weights_, this->old_indicators_);
+}
+
+// inq_convolution.cpp:35-102
+template <typename T, typename T1>
+void INQConvolutionHip<T, T1>::setup_impl(const Variables &inputs, const Variables &outputs) {
+  shapes_ = infer_conv_shapes(this->base_axis_, this->pad_, this->stride_, this->dilation_, this->group_, inputs[0],
+                              inputs[1], inputs.size() == 4 ? inputs[3] : nullptr);
+  this->base_axis_ = shapes_.base_axis;
+  outputs[0]->reshape(shapes_.out_shape, true);
+  inq_setup_state(inputs[1], inputs[2], this->selection_algorithm_, this->seed_, this->rgen_, this->rdist_,
+                  this->minibatch_counter_, this->old_weights_, this->old_indicators_);
+}
 
 template <typename T, typename T1>
 void INQAffineHip<T, T1>::run(const Variables &inputs, const Variables &outputs, int step) {
   hip_set_device(this->ctx_);
-  const AffineShapes &s = this->shapes_;
+  const AffineShapes &s = shapes_;
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
   T *w = inputs[1]->cast_data_and_get_pointer<T>(this->ctx_);
   T1 *ind = inputs[2]->cast_data_and_get_pointer<T1>(this->ctx_);
@@ -310,13 +440,15 @@ void INQAffineHip<T, T1>::run(const Variables &inputs, const Variables &outputs,
   const T *b = inputs.size() == 4 ? inputs[3]->get_data_pointer<T>(this->ctx_) : nullptr;
   T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
   HipWorkspace ws(nbla_hip_inq_affine_workspace_bytes(s.i_row, s.i_col, s.w_col, step), this->ctx_);
+  InqDraw draw{this->seed_ == -1 ? &SingletonManager::get<RandomManager>()->get_rand_generator() : &this->rgen_,
+               &this->rdist_};
   NBLA_HIP_CALL(nbla_hip_inq_affine_f32(x, w, ind, old_w, old_i, b, y, s.i_row, s.i_col, s.w_col, this->num_bits_,
-                                        step, draw_bernoulli, static_cast<InqState *>(this), ws.pointer(), ws.bytes(),
-                                        nullptr));
+                                        step, draw_bernoulli, &draw, ws.pointer(), ws.bytes(), nullptr));
 }
 template <typename T, typename T1>
 void INQAffineHip<T, T1>::forward_impl(const Variables &inputs, const Variables &outputs) {
-  run(inputs, outputs, this->current_step());
+  run(inputs, outputs,
+      inq_current_step(this->inq_iterations_, this->minibatch_counter_, this->selection_algorithm_));
   this->minibatch_counter_++; // inq_affine.cpp:200
 }
 template <typename T, typename T1>
@@ -327,7 +459,7 @@ void INQAffineHip<T, T1>::recompute_impl(const Variables &inputs, const Variable
 template <typename T, typename T1>
 void INQConvolutionHip<T, T1>::run(const Variables &inputs, const Variables &outputs, int step) {
   hip_set_device(this->ctx_);
-  const ConvShapes &s = this->shapes_;
+  const ConvShapes &s = shapes_;
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
   T *w = inputs[1]->cast_data_and_get_pointer<T>(this->ctx_);
   T1 *ind = inputs[2]->cast_data_and_get_pointer<T1>(this->ctx_);
@@ -339,15 +471,17 @@ void INQConvolutionHip<T, T1>::run(const Variables &inputs, const Variables &out
                                                            s.channels_o, s.kernel.data(), s.pad.data(),
                                                            s.stride.data(), s.dilation.data(), s.group, step),
                   this->ctx_);
+  InqDraw draw{this->seed_ == -1 ? &SingletonManager::get<RandomManager>()->get_rand_generator() : &this->rgen_,
+               &this->rdist_};
   NBLA_HIP_CALL(nbla_hip_inq_convolution_f32(x, w, ind, old_w, old_i, b, y, s.outer, s.channels_i, s.spatial_dims,
                                              s.spatial_i.data(), s.channels_o, s.kernel.data(), s.pad.data(),
                                              s.stride.data(), s.dilation.data(), s.group, this->num_bits_, step,
-                                             draw_bernoulli, static_cast<InqState *>(this), ws.pointer(), ws.bytes(),
-                                             nullptr));
+                                             draw_bernoulli, &draw, ws.pointer(), ws.bytes(), nullptr));
 }
 template <typename T, typename T1>
 void INQConvolutionHip<T, T1>::forward_impl(const Variables &inputs, const Variables &outputs) {
-  run(inputs, outputs, this->current_step());
+  run(inputs, outputs,
+      inq_current_step(this->inq_iterations_, this->minibatch_counter_, this->selection_algorithm_));
   this->minibatch_counter_++;
 }
 template <typename T, typename T1>
@@ -356,9 +490,38 @@ void INQConvolutionHip<T, T1>::recompute_impl(const Variables &inputs, const Var
 }
 
 // ------------------------------------------------------------ Affine and ReLU
+// affine.cpp:29-78
+template <typename T> void AffineHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
+  shapes_ = infer_affine_shapes(this->base_axis_, inputs[0], inputs[1], inputs.size() == 3 ? inputs[2] : nullptr);
+  this->base_axis_ = shapes_.base_axis;
+  this->i_row_ = shapes_.i_row;
+  this->i_col_ = shapes_.i_col;
+  this->w_row_ = shapes_.w_row;
+  this->w_col_ = shapes_.w_col;
+  this->o_row_ = shapes_.i_row;
+  this->o_col_ = shapes_.w_col;
+  outputs[0]->reshape(shapes_.out_shape, true);
+}
+
+// convolution.cpp:41-160
+template <typename T> void ConvolutionHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
+  NBLA_CHECK(!this->channel_last_, error_code::not_implemented,
+             "The passed argument channel_last_=true is not supported in Convolution.");
+  shapes_ = infer_conv_shapes(this->base_axis_, this->pad_, this->stride_, this->dilation_, this->group_, inputs[0],
+                              inputs[1], inputs.size() == 3 ? inputs[2] : nullptr);
+  this->base_axis_ = shapes_.base_axis;
+  this->channels_i_ = shapes_.channels_i;
+  this->channels_o_ = shapes_.channels_o;
+  this->channels_g_ = shapes_.channels_g;
+  this->spatial_dims_ = shapes_.spatial_dims;
+  this->outer_size_ = shapes_.outer;
+  this->inner_size_k_ = shapes_.inner_size_k;
+  outputs[0]->reshape(shapes_.out_shape, true);
+}
+
 template <typename T> void AffineHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
   hip_set_device(this->ctx_);
-  const AffineShapes &s = this->shapes_;
+  const AffineShapes &s = shapes_;
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
   const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
   const T *b = inputs.size() == 3 ? inputs[2]->get_data_pointer<T>(this->ctx_) : nullptr;
@@ -371,7 +534,7 @@ template <typename T> void AffineHip<T>::forward_impl(const Variables &inputs, c
 template <typename T, typename T1>
 void INQAffineHip<T, T1>::backward_impl(const Variables &inputs, const Variables &outputs,
                                         const vector<bool> &propagate_down, const vector<bool> &accum) {
-  const AffineShapes &s = this->shapes_;
+  const AffineShapes &s = shapes_;
   affine_backward_common<T>(this->ctx_, s, inputs, outputs, propagate_down, accum, 3,
                             [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
                               const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
@@ -384,7 +547,7 @@ void INQAffineHip<T, T1>::backward_impl(const Variables &inputs, const Variables
 template <typename T, typename T1>
 void INQConvolutionHip<T, T1>::backward_impl(const Variables &inputs, const Variables &outputs,
                                              const vector<bool> &propagate_down, const vector<bool> &accum) {
-  const ConvShapes &s = this->shapes_;
+  const ConvShapes &s = shapes_;
   conv_backward_common<T>(
       this->ctx_, s, inputs, outputs, propagate_down, accum, 3,
       [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
@@ -399,7 +562,7 @@ void INQConvolutionHip<T, T1>::backward_impl(const Variables &inputs, const Vari
 // convolution.cpp:161-197
 template <typename T> void ConvolutionHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
   hip_set_device(this->ctx_);
-  const ConvShapes &s = this->shapes_;
+  const ConvShapes &s = shapes_;
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
   const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
   const T *b = inputs.size() == 3 ? inputs[2]->get_data_pointer<T>(this->ctx_) : nullptr;
@@ -417,7 +580,7 @@ template <typename T> void ConvolutionHip<T>::forward_impl(const Variables &inpu
 template <typename T>
 void ConvolutionHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
                                       const vector<bool> &propagate_down, const vector<bool> &accum) {
-  const ConvShapes &s = this->shapes_;
+  const ConvShapes &s = shapes_;
   conv_backward_common<T>(
       this->ctx_, s, inputs, outputs, propagate_down, accum, 2,
       [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
@@ -433,7 +596,7 @@ void ConvolutionHip<T>::backward_impl(const Variables &inputs, const Variables &
 template <typename T>
 void AffineHip<T>::backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
                                  const vector<bool> &accum) {
-  const AffineShapes &s = this->shapes_;
+  const AffineShapes &s = shapes_;
   affine_backward_common<T>(this->ctx_, s, inputs, outputs, propagate_down, accum, 2,
                             [&](const T *dy, const T *x, T *dx, T *dw, T *db, int ax, int aw, int ab, HipWorkspace &ws) {
                               const T *w = inputs[1]->get_data_pointer<T>(this->ctx_);
@@ -458,7 +621,7 @@ void ReLUHip<T>::backward_impl(const Variables &inputs, const Variables &outputs
 template <typename T> void ReLUHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
   hip_set_device(this->ctx_);
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
-  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, !this->inplace_);
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
   NBLA_HIP_CALL(nbla_hip_relu_f32(x, y, (size_t)inputs[0]->size(), nullptr));
 }
 
@@ -469,6 +632,51 @@ vector<int64_t> shape64(const Variable *v) {
   return vector<int64_t>(s.begin(), s.end());
 }
 } // namespace
+
+// quantize_linear.cpp:28-46 and dequantize_linear.cpp:27-45: scale and zero point have x's rank, sizes 1 or x's.
+namespace {
+void check_linear_quantize_shapes(const Variables &inputs) {
+  NBLA_CHECK((inputs[0]->ndim() == inputs[1]->ndim()) && (inputs[0]->ndim() == inputs[2]->ndim()), error_code::value,
+             "Dimensions of inputs must be same (%d, %d, %d).", (int)inputs[0]->ndim(), (int)inputs[1]->ndim(),
+             (int)inputs[2]->ndim());
+  for (int i = 0; i < (int)inputs[0]->ndim(); ++i) {
+    const auto s0 = inputs[0]->shape()[i], s1 = inputs[1]->shape()[i], s2 = inputs[2]->shape()[i];
+    NBLA_CHECK(s1 == 1 || s1 == s0, error_code::value,
+               "Size at %d-th dimension of inputs[1] (%d) should be 1 or match the size at %d-th dimension of "
+               "inputs[0] (%d).",
+               i, (int)s1, i, (int)s0);
+    NBLA_CHECK(s2 == 1 || s2 == s0, error_code::value,
+               "Size at %d-th dimension of inputs[2] (%d) should be 1 or match the size at %d-th dimension of "
+               "inputs[0] (%d).",
+               i, (int)s2, i, (int)s0);
+  }
+}
+} // namespace
+
+// quantize_linear.cpp:25-95
+template <typename T> void QuantizeLinearHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
+  check_linear_quantize_shapes(inputs);
+  NBLA_CHECK(this->round_mode_ == "HALF_AWAY_FROM_ZERO" || this->round_mode_ == "HALF_TO_EVEN", error_code::value,
+             "round_mode must be HALF_AWAY_FROM_ZERO or HALF_TO_EVEN, not '%s'.", this->round_mode_.c_str());
+  outputs[0]->reshape(inputs[0]->shape(), true);
+  const dtypes dtype = static_cast<dtypes>(this->dtype_);
+  if (dtype == dtypes::BYTE) {
+    this->min_range_ = this->narrow_range_ ? -127 : -128;
+    this->max_range_ = 127;
+  } else if (dtype == dtypes::UBYTE) {
+    this->min_range_ = this->narrow_range_ ? 1 : 0;
+    this->max_range_ = 255;
+  } else {
+    NBLA_ERROR(error_code::value, "dtype must be BYTE (%d) or UBYTE (%d), not %d.", (int)dtypes::BYTE,
+               (int)dtypes::UBYTE, this->dtype_);
+  }
+}
+
+// dequantize_linear.cpp:25-53
+template <typename T> void DequantizeLinearHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
+  check_linear_quantize_shapes(inputs);
+  outputs[0]->reshape(inputs[0]->shape(), true);
+}
 
 // quantize_linear.cpp:97-117
 template <typename T> void QuantizeLinearHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {

@@ -54,7 +54,7 @@ HipMemory::HipMemory(size_t bytes, const string &device_id, void *ptr) : Memory(
 HipMemory::~HipMemory() {}
 
 bool HipMemory::alloc_impl() {
-  const int dev = hip_device_index(device_id_);
+  const int dev = hip_device_index(this->device_id());
   void *p = nullptr;
   if (nbla_hip_malloc(&p, bytes_, dev) != 0)
     return false;
@@ -64,7 +64,7 @@ bool HipMemory::alloc_impl() {
   return true;
 }
 shared_ptr<Memory> HipMemory::divide_impl(size_t second_start) {
-  HipMemory *second = new HipMemory(bytes_ - second_start, device_id_, static_cast<char *>(ptr_) + second_start);
+  HipMemory *second = new HipMemory(bytes_ - second_start, this->device_id(), static_cast<char *>(ptr_) + second_start);
   second->root_ = root_;
   return shared_ptr<Memory>(second);
 }
@@ -72,13 +72,14 @@ void HipMemory::merge_next_impl(Memory *) {}
 void HipMemory::merge_prev_impl(Memory *from) { ptr_ = from->pointer(); }
 
 // -------------------------------------------------------------------- HipArray
-HipArray::HipArray(Size_t size, dtypes dtype, const Context &ctx)
+HipArray::HipArray(const Size_t size, dtypes dtype, const Context &ctx, const AllocatorMemoryPtr mem,
+                   const Size_t offset)
     : Array(size, dtype, ctx,
-            make_shared<AllocatorMemory>(SingletonManager::get<Hip>()->naive_allocator()->alloc(
-                Array::size_as_bytes(size, dtype), ctx.device_id))),
+            mem ? mem
+                : SingletonManager::get<Hip>()->naive_allocator()->alloc(Array::size_as_bytes(size, dtype),
+                                                                         ctx.device_id),
+            offset),
       device_(hip_device_index(ctx.device_id)) {}
-HipArray::HipArray(Size_t size, dtypes dtype, const Context &ctx, AllocatorMemoryPtr mem, Size_t offset)
-    : Array(size, dtype, ctx, mem, offset), device_(hip_device_index(ctx.device_id)) {}
 HipArray::~HipArray() {}
 
 void HipArray::copy_from(const Array *src_array) {
@@ -97,10 +98,13 @@ void HipArray::fill(float value) {
 }
 Context HipArray::filter_context(const Context &ctx) { return Context({}, "HipArray", ctx.device_id); }
 
-HipCachedArray::HipCachedArray(Size_t size, dtypes dtype, const Context &ctx)
+HipCachedArray::HipCachedArray(const Size_t size, dtypes dtype, const Context &ctx, const AllocatorMemoryPtr mem,
+                               const Size_t offset)
     : HipArray(size, dtype, ctx,
-               make_shared<AllocatorMemory>(SingletonManager::get<Hip>()->caching_allocator()->alloc(
-                   Array::size_as_bytes(size, dtype), ctx.device_id))) {}
+               mem ? mem
+                   : SingletonManager::get<Hip>()->caching_allocator()->alloc(Array::size_as_bytes(size, dtype),
+                                                                              ctx.device_id),
+               offset) {}
 HipCachedArray::~HipCachedArray() {}
 Context HipCachedArray::filter_context(const Context &ctx) { return Context({}, "HipCachedArray", ctx.device_id); }
 

@@ -17,7 +17,8 @@ protected:
   Size_t offset_; // elements into mem_ (narrowed views)
 
 public:
-  Array(Size_t size, dtypes dtype, const Context &ctx, AllocatorMemoryPtr mem, Size_t offset = 0);
+  Array(const Size_t size, dtypes dtype, const Context &ctx, const AllocatorMemoryPtr mem = nullptr,
+        const Size_t offset = 0);
   virtual ~Array();
   Array(const Array &) = delete;
   Array &operator=(const Array &) = delete;
@@ -33,7 +34,7 @@ public:
   Size_t size() const { return size_; }
   Size_t offset() const { return offset_; }
   const Context &context() const { return ctx_; }
-  AllocatorMemoryPtr memory() { return mem_; }
+  AllocatorMemoryPtr memory() const { return mem_; }
 
   // Element-wise copy with dtype conversion from an array of the same class family.
   virtual void copy_from(const Array *src_array) = 0;

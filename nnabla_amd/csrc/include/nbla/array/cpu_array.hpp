@@ -9,8 +9,9 @@ namespace nbla {
 // Host array backed by the naive (uncached) host allocator.
 class NBLA_API CpuArray : public Array {
 public:
-  CpuArray(Size_t size, dtypes dtype, const Context &ctx);
-  CpuArray(Size_t size, dtypes dtype, const Context &ctx, AllocatorMemoryPtr mem, Size_t offset = 0);
+  // Without `mem` the array takes its memory from the backend's allocator (cpu_array.cpp:25-31).
+  CpuArray(const Size_t size, dtypes dtype, const Context &ctx, const AllocatorMemoryPtr mem = nullptr,
+           const Size_t offset = 0);
   virtual ~CpuArray();
   void copy_from(const Array *src_array) override;
   void zero() override;
@@ -21,7 +22,8 @@ public:
 // Host array backed by the caching host allocator.
 class NBLA_API CpuCachedArray : public CpuArray {
 public:
-  CpuCachedArray(Size_t size, dtypes dtype, const Context &ctx);
+  CpuCachedArray(const Size_t size, dtypes dtype, const Context &ctx, const AllocatorMemoryPtr mem = nullptr,
+                 const Size_t offset = 0);
   virtual ~CpuCachedArray();
   static Context filter_context(const Context &ctx);
 };

@@ -12,9 +12,10 @@ namespace nbla {
 
 class NBLA_API ArrayCreator {
 public:
-  typedef std::function<Array *(Size_t, dtypes, const Context &)> Creator;
+  typedef std::function<Array *(const Size_t, dtypes, const Context &, const AllocatorMemoryPtr, const Size_t)> Creator;
   typedef std::function<Context(const Context &)> FilterContext;
-  static Array *create(Size_t size, dtypes dtype, const Context &ctx);
+  static Array *create(const Size_t size, dtypes dtype, const Context &ctx, const AllocatorMemoryPtr mem = nullptr,
+                       const Size_t offset = 0);
   static Context filter_context(const Context &ctx);
   static void add_creator(const string &name, Creator creator, FilterContext filter_context);
   static vector<string> get_array_classes();
@@ -47,8 +48,10 @@ private:
 
 #define NBLA_REGISTER_ARRAY_CREATOR(CLS)                                                                               \
   ::nbla::ArrayCreator::add_creator(                                                                                   \
-      #CLS, [](::nbla::Size_t size, ::nbla::dtypes dtype, const ::nbla::Context &ctx) -> ::nbla::Array * {             \
-        return new CLS(size, dtype, ctx);                                                                              \
+      #CLS,                                                                                                            \
+      [](const ::nbla::Size_t size, ::nbla::dtypes dtype, const ::nbla::Context &ctx,                                  \
+         const ::nbla::AllocatorMemoryPtr mem, const ::nbla::Size_t offset) -> ::nbla::Array * {                       \
+        return new CLS(size, dtype, ctx, mem, offset);                                                                 \
       },                                                                                                               \
       CLS::filter_context)
 #define NBLA_REGISTER_ARRAY_SYNCHRONIZER(SRC_CLASS, DST_CLASS, SYNCHRONIZER)                                           \

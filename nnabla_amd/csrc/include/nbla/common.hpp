@@ -83,8 +83,6 @@ template <typename T> inline string string_join(const vector<T> &v, const string
   return oss.str();
 }
 
-// Negative axes count from the end (common.hpp refine_axis).
-void refine_axis(int &axis, int ndim);
 
 } // namespace nbla
 #endif

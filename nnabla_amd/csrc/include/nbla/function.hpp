@@ -45,10 +45,13 @@ public:
   virtual string name() = 0;
   virtual vector<string> allowed_array_classes() = 0;
   virtual bool grad_depends_output_data(int i, int o) const { return true; }
-  virtual bool grad_depends_input_data(int i, int j) const { return grad_depends_input_data_impl(i, j); }
+  virtual bool grad_depends_input_data(int i, int j) const final { return grad_depends_input_data_impl(i, j); }
   virtual int inplace_data(int i) const { return NOT_INPLACE; }
   virtual int inplace_data_with(int i) const { NBLA_ERROR(error_code::not_implemented, "not in-place"); }
-  virtual bool overwrite_input_data_in_forward(int i) const { return overwrite_input_data_in_forward_impl(i); }
+  virtual bool overwrite_input_data_in_forward(int i) const final { return overwrite_input_data_in_forward_impl(i); }
+  // A function that keeps its inputs' buffers (Sink) tells the graph engine not to clear or zero them.
+  virtual bool prohibit_clear_input_buffers() const { return false; }
+  virtual bool prohibit_zero_input_grad() const { return false; }
   virtual bool need_setup_recompute(int o) const { return false; }
   virtual shared_ptr<Function> copy() const = 0;
   bool ask_if_used_and_use() {

@@ -1,22 +1,23 @@
-// Affine and ReLU: the two plain functions the quantized graphs of this build need beside the quantization family
-// (mirrors include/nbla/function/affine.hpp and relu.hpp).
+// Affine: the class a "hip:float" implementation derives from.  Constructor, argument types, member
+// names are those of include/nbla/function/affine.hpp:50-107.
+// This build has no CPU arithmetic: a generic *_impl method without a body of its own raises not_implemented.
 #ifndef NBLA_FUNCTION_AFFINE_HPP_
 #define NBLA_FUNCTION_AFFINE_HPP_
 
 #include <nbla/cpu.hpp>
-#include <nbla/function/utils_shapes.hpp>
+#include <nbla/function.hpp>
+#include <nbla/function/no_cpu_impl.hpp>
 #include <nbla/function_registry.hpp>
 
 namespace nbla {
 
 NBLA_REGISTER_FUNCTION_HEADER(Affine, int);
-NBLA_REGISTER_FUNCTION_HEADER(ReLU, bool);
 
 // Inputs: x, weight, [bias].
 template <typename T> class Affine : public BaseFunction<int> {
 protected:
   int base_axis_;
-  AffineShapes shapes_;
+  Size_t i_row_, i_col_, w_row_, w_col_, o_row_, o_col_;
 
 public:
   Affine(const Context &ctx, int base_axis) : BaseFunction(ctx, base_axis), base_axis_(base_axis) {}
@@ -31,41 +32,12 @@ public:
   virtual bool grad_depends_output_data(int i, int o) const { return false; }
 
 protected:
-  virtual void setup_impl(const Variables &inputs, const Variables &outputs) {
-    shapes_ = infer_affine_shapes(base_axis_, inputs[0], inputs[1], inputs.size() == 3 ? inputs[2] : nullptr);
-    base_axis_ = shapes_.base_axis;
-    outputs[0]->reshape(shapes_.out_shape, true);
-  }
+  virtual void setup_impl(const Variables &, const Variables &) { NBLA_NO_CPU_IMPL("Affine"); }
   virtual void forward_impl(const Variables &, const Variables &) { NBLA_NO_CPU_IMPL("Affine"); }
   virtual void backward_impl(const Variables &, const Variables &, const vector<bool> &, const vector<bool> &) {
     NBLA_NO_CPU_IMPL("Affine backward");
   }
-};
-
-template <typename T> class ReLU : public BaseFunction<bool> {
-protected:
-  bool inplace_;
-
-public:
-  ReLU(const Context &ctx, bool inplace) : BaseFunction(ctx, inplace), inplace_(inplace) {}
-  virtual ~ReLU() {}
-  virtual shared_ptr<Function> copy() const { return create_ReLU(ctx_, inplace_); }
-  virtual vector<dtypes> in_types() { return vector<dtypes>{get_dtype<T>()}; }
-  virtual vector<dtypes> out_types() { return vector<dtypes>{get_dtype<T>()}; }
-  virtual int min_inputs() { return 1; }
-  virtual int min_outputs() { return 1; }
-  virtual string name() { return "ReLU"; }
-  virtual vector<string> allowed_array_classes() { return SingletonManager::get<Cpu>()->array_classes(); }
-  virtual bool grad_depends_input_data(int i, int j) const { return false; }
-
-protected:
-  virtual void setup_impl(const Variables &inputs, const Variables &outputs) {
-    outputs[0]->reshape(inputs[0]->shape(), true);
-  }
-  virtual void forward_impl(const Variables &, const Variables &) { NBLA_NO_CPU_IMPL("ReLU"); }
-  virtual void backward_impl(const Variables &, const Variables &, const vector<bool> &, const vector<bool> &) {
-    NBLA_NO_CPU_IMPL("ReLU backward");
-  }
+  virtual bool grad_depends_input_data_impl(int i, int j) const { return (i == 0 && j == 1) || (i == 1 && j == 0); }
 };
 
 } // namespace nbla

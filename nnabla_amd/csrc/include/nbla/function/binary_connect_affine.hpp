@@ -1,9 +1,12 @@
-// BinaryConnectAffine (mirrors include/nbla/function/binary_connect_affine.hpp:78-125).
+// BinaryConnectAffine: the class a "hip:float" implementation derives from.  Constructor, argument types, member
+// names are those of include/nbla/function/binary_connect_affine.hpp:78-125.
+// This build has no CPU arithmetic: a generic *_impl method without a body of its own raises not_implemented.
 #ifndef NBLA_FUNCTION_BINARY_CONNECT_AFFINE_HPP_
 #define NBLA_FUNCTION_BINARY_CONNECT_AFFINE_HPP_
 
 #include <nbla/cpu.hpp>
-#include <nbla/function/utils_shapes.hpp>
+#include <nbla/function.hpp>
+#include <nbla/function/no_cpu_impl.hpp>
 #include <nbla/function_registry.hpp>
 
 namespace nbla {
@@ -15,16 +18,14 @@ template <typename T> class BinaryConnectAffine : public BaseFunction<int, float
 protected:
   int base_axis_;
   float quantize_zero_to_;
-  AffineShapes shapes_;
 
 public:
   BinaryConnectAffine(const Context &ctx, int base_axis, float quantize_zero_to)
-      : BaseFunction(ctx, base_axis, quantize_zero_to), base_axis_(base_axis), quantize_zero_to_(quantize_zero_to) {}
+        : BaseFunction(ctx, base_axis, quantize_zero_to), base_axis_(base_axis), quantize_zero_to_(quantize_zero_to) {}
   virtual ~BinaryConnectAffine() {}
   virtual shared_ptr<Function> copy() const { return create_BinaryConnectAffine(ctx_, base_axis_, quantize_zero_to_); }
-  virtual vector<dtypes> in_types() {
-    return vector<dtypes>{get_dtype<T>(), get_dtype<T>(), get_dtype<T>(), get_dtype<T>()};
-  }
+  virtual vector<dtypes> in_types() { return vector<dtypes>{get_dtype<T>(), get_dtype<T>(), get_dtype<T>(),
+      get_dtype<T>()}; }
   virtual vector<dtypes> out_types() { return vector<dtypes>{get_dtype<T>()}; }
   virtual int min_inputs() { return 3; }
   virtual int min_outputs() { return 1; }
@@ -33,19 +34,12 @@ public:
   virtual bool grad_depends_output_data(int i, int o) const { return false; }
 
 protected:
-  // binary_connect_affine.cpp:29-57
-  virtual void setup_impl(const Variables &inputs, const Variables &outputs) {
-    shapes_ = infer_affine_shapes(base_axis_, inputs[0], inputs[1], inputs.size() == 4 ? inputs[3] : nullptr);
-    base_axis_ = shapes_.base_axis;
-    NBLA_CHECK(inputs[1]->shape() == inputs[2]->shape(), error_code::value,
-               "Binary and float weights must have same size.");
-    outputs[0]->reshape(shapes_.out_shape, true);
-  }
+  virtual void setup_impl(const Variables &, const Variables &) { NBLA_NO_CPU_IMPL("BinaryConnectAffine"); }
   virtual void forward_impl(const Variables &, const Variables &) { NBLA_NO_CPU_IMPL("BinaryConnectAffine"); }
   virtual void backward_impl(const Variables &, const Variables &, const vector<bool> &, const vector<bool> &) {
     NBLA_NO_CPU_IMPL("BinaryConnectAffine backward");
   }
-  virtual bool overwrite_input_data_in_forward_impl(int i) const { return i == 2; }
+  virtual bool grad_depends_input_data_impl(int i, int j) const { return (i == 0 && j == 2) || (i == 2 && j == 0); }
 };
 
 } // namespace nbla

@@ -1,39 +1,41 @@
-// BinaryConnectConvolution (mirrors include/nbla/function/binary_connect_convolution.hpp:91-153).
+// BinaryConnectConvolution: the class a "hip:float" implementation derives from.  Constructor, argument types, member
+// names are those of include/nbla/function/binary_connect_convolution.hpp:91-153.
+// This build has no CPU arithmetic: a generic *_impl method without a body of its own raises not_implemented.
 #ifndef NBLA_FUNCTION_BINARY_CONNECT_CONVOLUTION_HPP_
 #define NBLA_FUNCTION_BINARY_CONNECT_CONVOLUTION_HPP_
 
 #include <nbla/cpu.hpp>
-#include <nbla/function/utils_shapes.hpp>
+#include <nbla/function.hpp>
+#include <nbla/function/no_cpu_impl.hpp>
 #include <nbla/function_registry.hpp>
 
 namespace nbla {
 
 NBLA_REGISTER_FUNCTION_HEADER(BinaryConnectConvolution, int, const vector<int> &, const vector<int> &,
-                              const vector<int> &, int, float);
+    const vector<int> &, int, float);
 
 // Inputs: x, weight, binary_weight (written), [bias].
 template <typename T>
-class BinaryConnectConvolution
-    : public BaseFunction<int, const vector<int> &, const vector<int> &, const vector<int> &, int, float> {
+class BinaryConnectConvolution : public BaseFunction<int, const vector<int> &,
+    const vector<int> &, const vector<int> &, int, float> {
 protected:
   int base_axis_;
-  vector<int> pad_, stride_, dilation_;
+  vector<int> pad_;
+  vector<int> stride_;
+  vector<int> dilation_;
   int group_;
   float quantize_zero_to_;
-  ConvShapes shapes_;
 
 public:
   BinaryConnectConvolution(const Context &ctx, int base_axis, const vector<int> &pad, const vector<int> &stride,
-                           const vector<int> &dilation, int group, float quantize_zero_to)
-      : BaseFunction(ctx, base_axis, pad, stride, dilation, group, quantize_zero_to), base_axis_(base_axis), pad_(pad),
-        stride_(stride), dilation_(dilation), group_(group), quantize_zero_to_(quantize_zero_to) {}
+        const vector<int> &dilation, int group, float quantize_zero_to) : BaseFunction(ctx, base_axis, pad, stride,
+        dilation, group, quantize_zero_to), base_axis_(base_axis), pad_(pad), stride_(stride), dilation_(dilation),
+        group_(group), quantize_zero_to_(quantize_zero_to) {}
   virtual ~BinaryConnectConvolution() {}
-  virtual shared_ptr<Function> copy() const {
-    return create_BinaryConnectConvolution(ctx_, base_axis_, pad_, stride_, dilation_, group_, quantize_zero_to_);
-  }
-  virtual vector<dtypes> in_types() {
-    return vector<dtypes>{get_dtype<T>(), get_dtype<T>(), get_dtype<T>(), get_dtype<T>()};
-  }
+  virtual shared_ptr<Function> copy() const { return create_BinaryConnectConvolution(ctx_, base_axis_, pad_, stride_,
+      dilation_, group_, quantize_zero_to_); }
+  virtual vector<dtypes> in_types() { return vector<dtypes>{get_dtype<T>(), get_dtype<T>(), get_dtype<T>(),
+      get_dtype<T>()}; }
   virtual vector<dtypes> out_types() { return vector<dtypes>{get_dtype<T>()}; }
   virtual int min_inputs() { return 3; }
   virtual int min_outputs() { return 1; }
@@ -42,20 +44,12 @@ public:
   virtual bool grad_depends_output_data(int i, int o) const { return false; }
 
 protected:
-  // binary_connect_convolution.cpp:35-65
-  virtual void setup_impl(const Variables &inputs, const Variables &outputs) {
-    shapes_ = infer_conv_shapes(base_axis_, pad_, stride_, dilation_, group_, inputs[0], inputs[1],
-                                inputs.size() == 4 ? inputs[3] : nullptr);
-    base_axis_ = shapes_.base_axis;
-    NBLA_CHECK(inputs[1]->shape() == inputs[2]->shape(), error_code::value,
-               "Binary and float weights must have same size.");
-    outputs[0]->reshape(shapes_.out_shape, true);
-  }
+  virtual void setup_impl(const Variables &, const Variables &) { NBLA_NO_CPU_IMPL("BinaryConnectConvolution"); }
   virtual void forward_impl(const Variables &, const Variables &) { NBLA_NO_CPU_IMPL("BinaryConnectConvolution"); }
   virtual void backward_impl(const Variables &, const Variables &, const vector<bool> &, const vector<bool> &) {
     NBLA_NO_CPU_IMPL("BinaryConnectConvolution backward");
   }
-  virtual bool overwrite_input_data_in_forward_impl(int i) const { return i == 2; }
+  virtual bool grad_depends_input_data_impl(int i, int j) const { return (i == 0 && j == 2) || (i == 2 && j == 0); }
 };
 
 } // namespace nbla

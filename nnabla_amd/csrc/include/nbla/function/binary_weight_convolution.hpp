@@ -1,39 +1,42 @@
-// BinaryWeightConvolution (mirrors include/nbla/function/binary_weight_convolution.hpp:85-150).
+// BinaryWeightConvolution: the class a "hip:float" implementation derives from.  Constructor, argument types, member
+// names are those of include/nbla/function/binary_weight_convolution.hpp:85-150.
+// This build has no CPU arithmetic: a generic *_impl method without a body of its own raises not_implemented.
 #ifndef NBLA_FUNCTION_BINARY_WEIGHT_CONVOLUTION_HPP_
 #define NBLA_FUNCTION_BINARY_WEIGHT_CONVOLUTION_HPP_
 
 #include <nbla/cpu.hpp>
-#include <nbla/function/utils_shapes.hpp>
+#include <nbla/function.hpp>
+#include <nbla/function/no_cpu_impl.hpp>
 #include <nbla/function_registry.hpp>
 
 namespace nbla {
 
 NBLA_REGISTER_FUNCTION_HEADER(BinaryWeightConvolution, int, const vector<int> &, const vector<int> &,
-                              const vector<int> &, int, float);
+    const vector<int> &, int, float);
 
 // Inputs: x, weight, binary_weight (written), alpha (written), [bias].
 template <typename T>
-class BinaryWeightConvolution
-    : public BaseFunction<int, const vector<int> &, const vector<int> &, const vector<int> &, int, float> {
+class BinaryWeightConvolution : public BaseFunction<int, const vector<int> &,
+    const vector<int> &, const vector<int> &, int, float> {
 protected:
   int base_axis_;
-  vector<int> pad_, stride_, dilation_;
+  const vector<int> pad_;
+  const vector<int> stride_;
+  const vector<int> dilation_;
   int group_;
   float quantize_zero_to_;
-  ConvShapes shapes_;
+  int channels_o_, col_w_;
 
 public:
   BinaryWeightConvolution(const Context &ctx, int base_axis, const vector<int> &pad, const vector<int> &stride,
-                          const vector<int> &dilation, int group, float quantize_zero_to)
-      : BaseFunction(ctx, base_axis, pad, stride, dilation, group, quantize_zero_to), base_axis_(base_axis), pad_(pad),
-        stride_(stride), dilation_(dilation), group_(group), quantize_zero_to_(quantize_zero_to) {}
+        const vector<int> &dilation, int group, float quantize_zero_to) : BaseFunction(ctx, base_axis, pad, stride,
+        dilation, group, quantize_zero_to), base_axis_(base_axis), pad_(pad), stride_(stride), dilation_(dilation),
+        group_(group), quantize_zero_to_(quantize_zero_to) {}
   virtual ~BinaryWeightConvolution() {}
-  virtual shared_ptr<Function> copy() const {
-    return create_BinaryWeightConvolution(ctx_, base_axis_, pad_, stride_, dilation_, group_, quantize_zero_to_);
-  }
-  virtual vector<dtypes> in_types() {
-    return vector<dtypes>{get_dtype<T>(), get_dtype<T>(), get_dtype<T>(), get_dtype<T>(), get_dtype<T>()};
-  }
+  virtual shared_ptr<Function> copy() const { return create_BinaryWeightConvolution(ctx_, base_axis_, pad_, stride_,
+      dilation_, group_, quantize_zero_to_); }
+  virtual vector<dtypes> in_types() { return vector<dtypes>{get_dtype<T>(), get_dtype<T>(), get_dtype<T>(),
+      get_dtype<T>(), get_dtype<T>()}; }
   virtual vector<dtypes> out_types() { return vector<dtypes>{get_dtype<T>()}; }
   virtual int min_inputs() { return 4; }
   virtual int min_outputs() { return 1; }
@@ -42,22 +45,12 @@ public:
   virtual bool grad_depends_output_data(int i, int o) const { return false; }
 
 protected:
-  // binary_weight_convolution.cpp:33-70
-  virtual void setup_impl(const Variables &inputs, const Variables &outputs) {
-    shapes_ = infer_conv_shapes(base_axis_, pad_, stride_, dilation_, group_, inputs[0], inputs[1],
-                                inputs.size() == 5 ? inputs[4] : nullptr);
-    base_axis_ = shapes_.base_axis;
-    NBLA_CHECK(inputs[1]->shape() == inputs[2]->shape(), error_code::value,
-               "Binary and float weights must have same size.");
-    NBLA_CHECK(inputs[3]->size() == shapes_.channels_o, error_code::value,
-               "Size of alpha must be equal to the number of output channels.");
-    outputs[0]->reshape(shapes_.out_shape, true);
-  }
+  virtual void setup_impl(const Variables &, const Variables &) { NBLA_NO_CPU_IMPL("BinaryWeightConvolution"); }
   virtual void forward_impl(const Variables &, const Variables &) { NBLA_NO_CPU_IMPL("BinaryWeightConvolution"); }
   virtual void backward_impl(const Variables &, const Variables &, const vector<bool> &, const vector<bool> &) {
     NBLA_NO_CPU_IMPL("BinaryWeightConvolution backward");
   }
-  virtual bool overwrite_input_data_in_forward_impl(int i) const { return i == 2 || i == 3; }
+  virtual bool grad_depends_input_data_impl(int i, int j) const { return i == 1 && j == 0; }
 };
 
 } // namespace nbla

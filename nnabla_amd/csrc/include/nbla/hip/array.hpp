@@ -13,8 +13,9 @@ protected:
   int device_;
 
 public:
-  HipArray(Size_t size, dtypes dtype, const Context &ctx);
-  HipArray(Size_t size, dtypes dtype, const Context &ctx, AllocatorMemoryPtr mem, Size_t offset = 0);
+  // Without `mem` the array takes its memory from the hip backend's allocator, as CpuArray does from the host's.
+  HipArray(const Size_t size, dtypes dtype, const Context &ctx, const AllocatorMemoryPtr mem = nullptr,
+           const Size_t offset = 0);
   virtual ~HipArray();
   void copy_from(const Array *src_array) override;
   void zero() override;
@@ -25,7 +26,8 @@ public:
 // Device array backed by the caching device allocator (the default array class of the hip context).
 class NBLA_API HipCachedArray : public HipArray {
 public:
-  HipCachedArray(Size_t size, dtypes dtype, const Context &ctx);
+  HipCachedArray(const Size_t size, dtypes dtype, const Context &ctx, const AllocatorMemoryPtr mem = nullptr,
+                 const Size_t offset = 0);
   virtual ~HipCachedArray();
   static Context filter_context(const Context &ctx);
 };

@@ -1,5 +1,6 @@
-// "hip:float" implementations of the elementwise quantizers.  Each class reuses the argument checks and shape
-// inference of the generic class and replaces forward_impl / backward_impl by calls into the kernel library.
+// "hip:float" implementations of the elementwise quantizers.  FixedPointQuantize and Pow2Quantize reuse the generic
+// setup_impl (argument checks and the derived bounds); MinMaxQuantize replaces it, because the generic one also builds
+// the chain of CPU helper functions that its forward pass runs.
 #ifndef NBLA_HIP_FUNCTION_QUANTIZE_HPP_
 #define NBLA_HIP_FUNCTION_QUANTIZE_HPP_
 
@@ -41,6 +42,7 @@ public:
   virtual vector<string> allowed_array_classes() { return SingletonManager::get<Hip>()->array_classes(); }
 
 protected:
+  virtual void setup_impl(const Variables &inputs, const Variables &outputs);
   virtual void forward_impl(const Variables &inputs, const Variables &outputs);
   virtual void backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
                              const vector<bool> &accum);

@@ -1,13 +1,15 @@
-// Shape inference shared by the affine- and convolution-shaped functions.
-#ifndef NBLA_FUNCTION_UTILS_SHAPES_HPP_
-#define NBLA_FUNCTION_UTILS_SHAPES_HPP_
+// Shape inference of the affine- and convolution-shaped "hip:float" functions.  The generic classes of nnabla infer
+// these inside setup_impl bodies that also build chains of CPU helper functions; the hip classes replace those
+// bodies, so they carry the inferred geometry themselves, in the form the kernel library takes it.
+#ifndef NBLA_HIP_FUNCTION_SHAPES_HPP_
+#define NBLA_HIP_FUNCTION_SHAPES_HPP_
 
 #include <nbla/function.hpp>
 
 namespace nbla {
 
 // Affine<T>::setup_impl (src/nbla/function/generic/affine.cpp:29-78): x [.., i_col] viewed [i_row, i_col],
-// W [w_row, ...] viewed [w_row, w_col]; output shape x.shape[:base_axis] + W.shape[1:].
+// W [w_row, ...] viewed [w_row, w_col]; output shape x.shape[:base_axis] + W.shape[1:].  Same checks and messages.
 struct AffineShapes {
   int base_axis;
   Size_t i_row, i_col, w_row, w_col;
@@ -24,10 +26,6 @@ struct ConvShapes {
 };
 NBLA_API ConvShapes infer_conv_shapes(int base_axis, const vector<int> &pad, const vector<int> &stride,
                                       const vector<int> &dilation, int group, Variable *x, Variable *w, Variable *bias);
-
-#define NBLA_NO_CPU_IMPL(NAME)                                                                                         \
-  NBLA_ERROR(::nbla::error_code::not_implemented,                                                                      \
-             NAME " has no CPU implementation in this build; create it with a 'hip:float' context.")
 
 } // namespace nbla
 #endif

@@ -3,6 +3,7 @@
 #ifndef NBLA_HIP_MEMORY_HPP_
 #define NBLA_HIP_MEMORY_HPP_
 
+#include <nbla/exception.hpp>
 #include <nbla/memory/memory.hpp>
 
 namespace nbla {
@@ -13,6 +14,9 @@ public:
   ~HipMemory();
 
 protected:
+  // Owner of the hipMalloc'ed block this memory was carved from; every fragment shares it, so the block goes back
+  // to the device when the last fragment is destroyed, in whatever order the allocator drops them.
+  shared_ptr<void> root_;
   HipMemory(size_t bytes, const string &device_id, void *ptr);
   bool alloc_impl() override;
   shared_ptr<Memory> divide_impl(size_t second_start) override;

@@ -28,7 +28,7 @@ public:
   AllocatorMemory &operator=(const AllocatorMemory &) = delete;
   shared_ptr<Memory> memory() { return memory_; }
   size_t bytes() const { return memory_ ? memory_->bytes() : 0; }
-  const string &device_id() const { return memory_->device_id(); }
+  string device_id() const { return memory_->device_id(); }
   void *pointer() { return memory_ ? memory_->pointer() : nullptr; }
   const void *const_pointer() const { return memory_ ? memory_->const_pointer() : nullptr; }
 
@@ -42,7 +42,7 @@ public:
   Allocator() {}
   virtual ~Allocator() {}
   // Requests at least `bytes` on `device_id` (zero-byte requests get the minimum block).
-  AllocatorMemory alloc(size_t bytes, const string &device_id);
+  AllocatorMemoryPtr alloc(size_t bytes, const string &device_id);
   // Called by AllocatorMemory's destructor.
   void free(shared_ptr<Memory> memory);
   // Releases cached, currently unused blocks back to the device; returns the bytes freed.

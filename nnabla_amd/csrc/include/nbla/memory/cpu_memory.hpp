@@ -12,6 +12,9 @@ public:
   ~CpuMemory();
 
 protected:
+  // Owner of the allocation this block was carved from; shared by all of its fragments, so the allocation is
+  // returned when the last fragment goes away, in whatever order that happens.
+  shared_ptr<void> root_;
   CpuMemory(size_t bytes, const string &device_id, void *ptr);
   bool alloc_impl() override;
   shared_ptr<Memory> divide_impl(size_t second_start) override;

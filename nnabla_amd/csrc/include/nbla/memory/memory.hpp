@@ -8,6 +8,12 @@
 namespace nbla {
 
 class NBLA_API Memory {
+  string device_id_;
+  bool locked_ = false;
+  Memory *next_ = nullptr;
+  Memory *prev_ = nullptr;
+  void disable() { ptr_ = nullptr; }
+
 public:
   Memory(size_t bytes, const string &device_id);
   virtual ~Memory();
@@ -15,7 +21,7 @@ public:
   Memory &operator=(const Memory &) = delete;
 
   size_t bytes() const { return bytes_; }
-  const string &device_id() const { return device_id_; }
+  string device_id() const { return device_id_; }
   void *pointer() { return ptr_; }
   const void *const_pointer() const { return ptr_; }
   bool locked() const { return locked_; }
@@ -25,7 +31,7 @@ public:
   Memory *next() const { return next_; }
   // Neighbour blocks carved from the same allocation are held weakly through raw
   // pointers; the owning allocator keeps them alive.
-  bool disabled() const { return bytes_ == 0; }
+  bool disabled() { return !ptr_; }
 
   // Obtains the memory from the device; throws error_code::memory on failure.
   void alloc();
@@ -36,22 +42,10 @@ public:
   static void associate_consecutive(Memory *left, Memory *right);
 
 protected:
-  size_t bytes_;
-  string device_id_;
+  size_t bytes_ = 0;
   void *ptr_ = nullptr;
-  // Owner of the device allocation this block was carved from; shared by all of its fragments, so the allocation
-  // is returned to the device when the last fragment goes away, in whatever order that happens.
-  shared_ptr<void> root_;
-  bool locked_ = false;
-  Memory *prev_ = nullptr;
-  Memory *next_ = nullptr;
-
-  void disable() {
-    ptr_ = nullptr;
-    bytes_ = 0;
-    root_.reset();
-  }
-  // Backend hooks.
+  // Backend hooks.  An implementation keeps whatever owns the underlying allocation itself (CpuMemory and HipMemory
+  // share one owner between all fragments carved from an allocation).
   virtual bool alloc_impl() = 0;
   virtual shared_ptr<Memory> divide_impl(size_t second_start) = 0;
   virtual void merge_next_impl(Memory *from) = 0;

@@ -8,7 +8,7 @@
 
 namespace nbla {
 
-Array::Array(Size_t size, dtypes dtype, const Context &ctx, AllocatorMemoryPtr mem, Size_t offset)
+Array::Array(const Size_t size, dtypes dtype, const Context &ctx, const AllocatorMemoryPtr mem, const Size_t offset)
     : size_(size), dtype_(dtype), ctx_(ctx), mem_(mem), offset_(offset) {}
 Array::~Array() {}
 void Array::wait_event(const Context &, int) {}
@@ -97,12 +97,11 @@ void cpu_fill(void *dst, dtypes dtype, Size_t size, float value) {
 }
 
 // -------------------------------------------------------------------- CpuArray
-CpuArray::CpuArray(Size_t size, dtypes dtype, const Context &ctx)
+CpuArray::CpuArray(const Size_t size, dtypes dtype, const Context &ctx, const AllocatorMemoryPtr mem,
+                   const Size_t offset)
     : Array(size, dtype, ctx,
-            make_shared<AllocatorMemory>(SingletonManager::get<Cpu>()->naive_allocator()->alloc(
-                Array::size_as_bytes(size, dtype), ""))) {}
-CpuArray::CpuArray(Size_t size, dtypes dtype, const Context &ctx, AllocatorMemoryPtr mem, Size_t offset)
-    : Array(size, dtype, ctx, mem, offset) {}
+            mem ? mem : SingletonManager::get<Cpu>()->naive_allocator()->alloc(Array::size_as_bytes(size, dtype), ""),
+            offset) {}
 CpuArray::~CpuArray() {}
 
 void CpuArray::copy_from(const Array *src_array) {
@@ -113,10 +112,12 @@ void CpuArray::zero() { std::memset(pointer<void>(), 0, size_ * sizeof_dtype(dty
 void CpuArray::fill(float value) { cpu_fill(pointer<void>(), dtype_, size_, value); }
 Context CpuArray::filter_context(const Context &) { return Context({}, "CpuArray", ""); }
 
-CpuCachedArray::CpuCachedArray(Size_t size, dtypes dtype, const Context &ctx)
+CpuCachedArray::CpuCachedArray(const Size_t size, dtypes dtype, const Context &ctx, const AllocatorMemoryPtr mem,
+                               const Size_t offset)
     : CpuArray(size, dtype, ctx,
-               make_shared<AllocatorMemory>(SingletonManager::get<Cpu>()->caching_allocator()->alloc(
-                   Array::size_as_bytes(size, dtype), ""))) {}
+               mem ? mem
+                   : SingletonManager::get<Cpu>()->caching_allocator()->alloc(Array::size_as_bytes(size, dtype), ""),
+               offset) {}
 CpuCachedArray::~CpuCachedArray() {}
 Context CpuCachedArray::filter_context(const Context &) { return Context({}, "CpuCachedArray", ""); }
 
@@ -130,14 +131,15 @@ std::map<string, std::pair<ArrayCreator::Creator, ArrayCreator::FilterContext>> 
 void ArrayCreator::add_creator(const string &name, Creator creator, FilterContext filter_context) {
   registry()[name] = {creator, filter_context};
 }
-Array *ArrayCreator::create(Size_t size, dtypes dtype, const Context &ctx) {
+Array *ArrayCreator::create(const Size_t size, dtypes dtype, const Context &ctx, const AllocatorMemoryPtr mem,
+                            const Size_t offset) {
   auto it = registry().find(ctx.array_class);
   if (it == registry().end()) {
     vector<string> have = get_array_classes();
     NBLA_ERROR(error_code::unclassified, "'%s' could not be found in [%s]", ctx.array_class.c_str(),
                string_join(have, ", ").c_str());
   }
-  return it->second.first(size, dtype, ctx);
+  return it->second.first(size, dtype, ctx, mem, offset);
 }
 Context ArrayCreator::filter_context(const Context &ctx) {
   auto it = registry().find(ctx.array_class);

@@ -53,12 +53,6 @@ string dtype_to_string(dtypes dtype) {
   return "UNKNOWN";
 }
 
-void refine_axis(int &axis, int ndim) {
-  NBLA_CHECK(axis < ndim && ndim + axis >= 0, error_code::value, "axis must be in the range of [-ndim, ndim). axis : %d, ndim: %d.", axis, ndim);
-  if (axis < 0)
-    axis += ndim;
-}
-
 // ------------------------------------------------------------------- Context
 Context::Context(const vector<string> &backend, const string &array_class, const string &device_id)
     : backend(backend), array_class(array_class), device_id(device_id) {}

@@ -8,7 +8,7 @@
 namespace nbla {
 
 // ---------------------------------------------------------------------- Memory
-Memory::Memory(size_t bytes, const string &device_id) : bytes_(bytes), device_id_(device_id) {}
+Memory::Memory(size_t bytes, const string &device_id) : device_id_(device_id), bytes_(bytes) {}
 
 Memory::~Memory() {
   // Unlink from the chain of blocks carved from the same allocation.
@@ -81,11 +81,11 @@ AllocatorMemory &AllocatorMemory::operator=(AllocatorMemory &&rhs) {
 }
 
 // ------------------------------------------------------------------- Allocator
-AllocatorMemory Allocator::alloc(size_t bytes, const string &device_id) {
+AllocatorMemoryPtr Allocator::alloc(size_t bytes, const string &device_id) {
   std::lock_guard<std::mutex> lock(mutex_);
   shared_ptr<Memory> mem = alloc_impl(bytes, device_id);
   mem->lock();
-  return AllocatorMemory(mem, shared_from_this());
+  return make_shared<AllocatorMemory>(mem, shared_from_this());
 }
 
 void Allocator::free(shared_ptr<Memory> memory) {
@@ -236,7 +236,7 @@ bool CpuMemory::alloc_impl() {
   return true;
 }
 shared_ptr<Memory> CpuMemory::divide_impl(size_t second_start) {
-  CpuMemory *second = new CpuMemory(bytes_ - second_start, device_id_, static_cast<char *>(ptr_) + second_start);
+  CpuMemory *second = new CpuMemory(bytes_ - second_start, device_id(), static_cast<char *>(ptr_) + second_start);
   second->root_ = root_;
   return shared_ptr<Memory>(second);
 }
