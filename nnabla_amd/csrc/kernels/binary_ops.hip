@@ -26,6 +26,10 @@ AffineWorkspace plan_affine(int64_t M, int64_t K, int64_t N) {
   w.gemm_bytes = nbla_hip_gemm_bits_workspace_bytes(M, K, N);
   off += w.gemm_bytes;
   w.total = off;
+  // the one-pass form for very few rows keeps its slab partials at the start of the same buffer
+  const size_t small = round_up(small_m_affine_workspace_bytes(M, K, N), 256);
+  if (small > w.total)
+    w.total = small;
   return w;
 }
 
@@ -40,6 +44,13 @@ int binary_affine_forward(const float *x, const float *W, float *Wb, float *alph
     return fail(NBLA_HIP_ERR_MEMORY, "binary affine workspace too small (%zu < %zu) or misaligned.", workspace_bytes,
                 ws.total);
   char *base = static_cast<char *>(workspace);
+  if (small_m_affine_applies(x, W, Wb, alpha, bias, y, M, K, N)) {
+    const int rc = ensure_init();
+    if (rc)
+      return rc;
+    return launch_small_m_affine(x, W, Wb, alpha, bias, y, M, K, N, zero_to, base, workspace_bytes,
+                                 as_stream(stream_));
+  }
   uint32_t *bits = reinterpret_cast<uint32_t *>(base + ws.bits_off);
   void *xsplit = base + ws.split_off; // digit operand of x
   void *prep = base + ws.prep_off;

@@ -25,6 +25,7 @@ __device__ __forceinline__ float sign_of(float w, float zero_to) {
 // [slices * col_groups] ints, then the pair words.  slices depends on the source layout.
 struct PrepPlan {
   int64_t k_tiles, col_groups, Np, slices;
+  int64_t wide_groups, Npw, slabs; // the streaming [K, N] kernel: 256-column groups, padded columns, slabs of 256 rows
   size_t sums_bytes, zeros_bytes, pairs_bytes;
 };
 
@@ -33,9 +34,13 @@ PrepPlan make_prep_plan(int64_t K, int64_t N, bool transposed) {
   P.k_tiles = bits_k_tiles(K);
   P.col_groups = bits_col_groups(N);
   P.Np = P.col_groups * kColGroup;
-  // the [K, N] kernels cover 8 (vector path) or 16 (scalar path) k tiles per block; size for the finer one
+  // the scalar [K, N] kernel covers 16 k tiles per block, the [N, K] kernels 4; size for the finer one
   P.slices = transposed ? ceil_div(P.k_tiles, 4) : ceil_div(P.k_tiles, 8);
-  P.sums_bytes = round_up((size_t)P.slices * P.Np * sizeof(float), 256);
+  P.wide_groups = bits_wide_groups(N);
+  P.Npw = P.wide_groups * kWideGroup;
+  P.slabs = bits_packed_k_tiles(K) / 8;
+  const size_t sums_a = (size_t)P.slices * P.Np, sums_b = transposed ? 0 : (size_t)P.slabs * P.Npw;
+  P.sums_bytes = round_up((sums_a > sums_b ? sums_a : sums_b) * sizeof(float), 256);
   P.zeros_bytes = round_up((size_t)P.slices * P.col_groups * sizeof(int), 256);
   P.pairs_bytes = round_up((size_t)P.k_tiles * P.col_groups * 64 * sizeof(uint32_t), 256);
   return P;
@@ -131,87 +136,147 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_kn(const float *__restric
     zeros[(int64_t)blockIdx.y * col_groups + cg] = s_zero[0] + s_zero[1] + s_zero[2] + s_zero[3];
 }
 
-// W stored [K, N], N % 4 == 0, 16-byte aligned: the streaming path.  A wavefront covers two k tiles of one column
-// group; lane = (kt_sub, g, f, nq): columns f*32 + 4*nq + {0..3}, k offsets g*16 + j.  Each thread issues its
-// sixteen 128-bit loads up front (sixteen lanes cover 256 contiguous bytes of a row), builds the bits of its half
-// (f) of four packed words, and the two halves are OR-ed across lanes.  |W| column sums are folded in a fixed
-// order: over (g, kt_sub) by shuffles, over the block's wavefronts through LDS.
-__global__ __launch_bounds__(kPrepBlock) void binarize_kn_vec(const float *__restrict__ W, float *__restrict__ Wb,
-                                                              uint32_t *__restrict__ bits, float *__restrict__ sums,
-                                                              int *__restrict__ zeros, int64_t K, int64_t N,
-                                                              int64_t col_groups, int64_t Np, int64_t k_tiles,
-                                                              float zero_to) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int nq = lane & 7, f = (lane >> 3) & 1, g = (lane >> 4) & 1, kt_sub = lane >> 5;
-  const int64_t cg = blockIdx.x;
-  const int64_t kt = ((int64_t)blockIdx.y * 4 + wave) * 2 + kt_sub;
-  const int64_t n0 = cg * kColGroup + f * 32 + 4 * nq;
-  const bool col_ok = n0 < N;
-  float4_t v[16];
-#pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    const int64_t k = kt * kTileK + g * 16 + j;
-    if (col_ok && k < K)
-      v[j] = *reinterpret_cast<const float4_t *>(W + k * N + n0);
-    else
-      v[j] = float4_t{1.0f, 1.0f, 1.0f, 1.0f};
-  }
+// W stored [K, N], N % 4 == 0, 16-byte aligned: the streaming path.  A block of four wavefronts covers 256 rows of one
+// 256-column group, wavefront w rows 64 w .. 64 w + 63 (two k tiles); a lane owns four consecutive columns, so every
+// load and store instruction of a wavefront moves 1 KiB of one row.  Four rows are in flight while four are consumed
+// (128 registers per lane: sixteen wavefronts per CU).
+// Per element: Sign -> Wb (nontemporal store), |w| into the lane's column sums, the sign bit shifted into a 32-bit
+// word per column (bit k = row k of the k tile).  After 32 rows the wavefront transposes those words through LDS into
+// the packed operand's own layout (lane l: columns F * 32 + l % 32, k slots (l / 32) * 16 + j; bit F + 8 c of word i
+// for k slot 4 i + c) and writes the k tile's 1 KiB straight into the packed operand.  No intermediate pair words and
+// no relayout pass.  Column sums: lanes in row order, then the block's four wavefronts through LDS in wavefront order.
+constexpr int kWideWaveRows = 64, kWideBatch = 4;
+constexpr int kWideTileBatches = kTileK / kWideBatch; // batches per k tile
+template <bool kFull, bool kCountZeros>
+__device__ __forceinline__ void binarize_wide_walk(const float *__restrict__ W, float *__restrict__ Wb,
+                                                   uint4_t *__restrict__ bits_out, int64_t tile_stride, uint32_t *s_x,
+                                                   int64_t K, int64_t N, int64_t k_wave, int64_t n0, int lane,
+                                                   float zero_to,
+                                                   float (&cs)[4], int &nzero) {
+  const bool col_ok = kFull || n0 < N;
+  const int64_t n_ld = col_ok ? n0 : N - 4; // loads are unconditional: a clamped address, masked afterwards
+  const uint32_t lane_bytes = (uint32_t)(n_ld * 4);
+  float4_t va[kWideBatch], vb[kWideBatch];
   uint32_t word[4] = {0u, 0u, 0u, 0u};
-  float asum[4] = {0.f, 0.f, 0.f, 0.f};
-  int nzero = 0;
+  auto load_batch = [&](int b, float4_t (&dst)[kWideBatch]) {
 #pragma unroll
-  for (int j = 0; j < 16; ++j) {
-      const int64_t k = kt * kTileK + g * 16 + j;
-      const bool in = col_ok && k < K;
-      const float w[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
-      float b[4];
+    for (int j = 0; j < kWideBatch; ++j) {
+      int64_t k = k_wave + b * kWideBatch + j;
+      if (!kFull && k >= K)
+        k = K - 1;
+      const char *row = reinterpret_cast<const char *>(W + k * N); // uniform base + 32-bit lane offset
+      dst[j] = *reinterpret_cast<const float4_t *>(row + lane_bytes);
+    }
+  };
+  auto consume_batch = [&](int b, const float4_t (&src)[kWideBatch]) {
+#pragma unroll
+    for (int j = 0; j < kWideBatch; ++j) {
+      const int64_t k = k_wave + b * kWideBatch + j;
+      const bool in = kFull || (col_ok && k < K);
+      const float w[4] = {src[j].x, src[j].y, src[j].z, src[j].w};
+      float sg[4];
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        b[c] = sign_of(w[c], zero_to);
-        const bool is_zero = !(w[c] > 0.0f) && !(w[c] < 0.0f);
-        const bool neg = (w[c] < 0.0f) || (is_zero && zero_to < 0.0f);
-        const int pos = 4 * f + (j >> 2) + 8 * (j & 3); // packed_bit_position with f a run-time value
-        word[c] |= (in && neg) ? (1u << pos) : 0u;
-        asum[c] += in ? fabsf(w[c]) : 0.0f;
-        nzero += (in && is_zero) ? 1 : 0;
+        // sign.hpp:48-50; +-0 and NaN are exactly the inputs that are neither less nor greater than zero
+        const bool nonzero = __builtin_islessgreater(w[c], 0.0f);
+        const float one = __uint_as_float((__float_as_uint(w[c]) & 0x80000000u) | 0x3f800000u);
+        sg[c] = nonzero ? one : zero_to;
+        // the sign of Sign(w) is the packed bit: rows enter at bit 31 and move down one place per row
+        const uint32_t bit = in ? (__float_as_uint(sg[c]) & 0x80000000u) : 0u;
+        word[c] = (word[c] >> 1) | bit;
+        cs[c] += in ? fabsf(w[c]) : 0.0f;
+        if (kCountZeros)
+          nzero += (in && !nonzero) ? 1 : 0;
       }
       if (in && Wb) {
         float4_t o;
-        o.x = b[0], o.y = b[1], o.z = b[2], o.w = b[3];
-        __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(Wb + k * N + n0));
+        o.x = sg[0], o.y = sg[1], o.z = sg[2], o.w = sg[3];
+        char *row = reinterpret_cast<char *>(Wb + k * N);
+        __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(row + lane_bytes));
       }
     }
+  };
+  // 32 rows are in `word`: transpose them into the packed layout and write the k tile
+  auto emit_tile = [&](int t) {
+    uint4_t mine;
+    mine.x = word[0], mine.y = word[1], mine.z = word[2], mine.w = word[3];
+    *reinterpret_cast<uint4_t *>(s_x + 4 * lane) = mine;
+    __builtin_amdgcn_wave_barrier(); // the wavefront's own LDS traffic stays in program order
+    const int q = (lane & 31) >> 2, c = lane & 3, half = (lane >> 5) * 16;
+    uint32_t out[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
-  for (int c = 0; c < 4; ++c)
-    word[c] |= __shfl_xor(word[c], 8); // the other half (f) of the same packed words
-  if (f == 0 && kt < k_tiles) {
-    uint4_t wv;
-    wv.x = word[0], wv.y = word[1], wv.z = word[2], wv.w = word[3];
-    *reinterpret_cast<uint4_t *>(bits + (kt * col_groups + cg) * 64 + g * 32 + 4 * nq) = wv;
+    for (int F = 0; F < 8; ++F) {
+      const uint32_t col = s_x[(F * 8 + q) * 4 + c]; // column F * 32 + lane % 32, bit k = row k
+      const uint32_t h = (col >> half) & 0xffffu;    // this lane's sixteen k slots
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t nib = (h >> (4 * i)) & 0xfu;
+        // bits 0..3 of nib to bit positions 0, 8, 16, 24 (the sixteen partial products land on distinct bits)
+        out[i] |= ((nib * 0x00204081u) & 0x01010101u) << F;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    uint4_t o;
+    o.x = out[0], o.y = out[1], o.z = out[2], o.w = out[3];
+    bits_out[(size_t)t * tile_stride] = o; // bits_out: this lane's slot in the wavefront's first k tile
+  };
+  constexpr int kBatches = kWideWaveRows / kWideBatch;
+  load_batch(0, va);
+#pragma clang loop unroll(disable)
+  for (int b = 0; b < kBatches; b += 2) {
+    load_batch(b + 1, vb);
+    consume_batch(b, va);
+    if (b + 2 < kBatches)
+      load_batch(b + 2, va);
+    consume_batch(b + 1, vb);
+    if ((b + 2) % kWideTileBatches == 0) {
+      emit_tile(b / kWideTileBatches);
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        word[c] = 0u;
+    }
   }
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    asum[c] += __shfl_xor(asum[c], 16); // g
-    asum[c] += __shfl_xor(asum[c], 32); // kt_sub
-  }
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1)
-    nzero += __shfl_xor(nzero, off);
-  __shared__ float s_sum[kPrepBlock / 64][kColGroup];
+}
+
+template <bool kCountZeros>
+__global__ __launch_bounds__(kPrepBlock, 4) void binarize_kn_wide(const float *__restrict__ W, float *__restrict__ Wb,
+                                                                 uint4_t *__restrict__ bits, float *__restrict__ sums,
+                                                                 int *__restrict__ zeros, int64_t K, int64_t N,
+                                                                 int64_t wide_groups, int64_t Npw, float zero_to) {
+  __shared__ __attribute__((aligned(16))) uint32_t s_x[kPrepBlock / 64][256];
+  __shared__ float s_sum[kPrepBlock / 64][kWideGroup];
   __shared__ int s_zero[kPrepBlock / 64];
-  if (lane < 16) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // uniform: row indices stay in scalar registers
+  const int64_t wg = blockIdx.x, slab = blockIdx.y;
+  const int64_t k_wave = (slab * (kPrepBlock / 64) + wave) * kWideWaveRows;
+  const int64_t n0 = wg * kWideGroup + 4 * lane;
+  float cs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  int nzero = 0;
+  // consecutive k tiles of one wide group lie wide_groups * 64 uint4 apart
+  uint4_t *tile0 = bits + ((k_wave / kTileK) * wide_groups + wg) * 64 + lane;
+  const int64_t tile_stride = wide_groups * 64;
+  const bool full = k_wave + kWideWaveRows <= K && (wg + 1) * kWideGroup <= N;
+  if (full)
+    binarize_wide_walk<true, kCountZeros>(W, Wb, tile0, tile_stride, s_x[wave], K, N, k_wave, n0, lane, zero_to, cs,
+                                          nzero);
+  else
+    binarize_wide_walk<false, kCountZeros>(W, Wb, tile0, tile_stride, s_x[wave], K, N, k_wave, n0, lane, zero_to, cs,
+                                           nzero);
+  // column sums of the block's 256 rows, wavefronts in order
+  *reinterpret_cast<float4_t *>(&s_sum[wave][4 * lane]) = float4_t{cs[0], cs[1], cs[2], cs[3]};
+  if (kCountZeros) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
-      s_sum[wave][f * 32 + 4 * nq + c] = asum[c];
+    for (int off = 32; off >= 1; off >>= 1)
+      nzero += __shfl_xor(nzero, off);
+    if (lane == 0)
+      s_zero[wave] = nzero;
   }
-  if (lane == 0)
-    s_zero[wave] = nzero;
   __syncthreads();
-  if (threadIdx.x < kColGroup)
-    sums[(int64_t)blockIdx.y * Np + cg * kColGroup + threadIdx.x] =
-        ((s_sum[0][threadIdx.x] + s_sum[1][threadIdx.x]) + s_sum[2][threadIdx.x]) + s_sum[3][threadIdx.x];
-  if (threadIdx.x == 0)
-    zeros[(int64_t)blockIdx.y * col_groups + cg] = s_zero[0] + s_zero[1] + s_zero[2] + s_zero[3];
+  sums[slab * Npw + wg * kWideGroup + threadIdx.x] =
+      ((s_sum[0][threadIdx.x] + s_sum[1][threadIdx.x]) + s_sum[2][threadIdx.x]) + s_sum[3][threadIdx.x];
+  if (kCountZeros && threadIdx.x == 0)
+    zeros[slab * wide_groups + wg] = s_zero[0] + s_zero[1] + s_zero[2] + s_zero[3];
 }
 
 // W stored [N, K] (convolution weights viewed [channels_o, col_w]).  Wavefront w
@@ -295,7 +360,7 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_nk_vec(const float *__res
   for (int i = 0; i < 8; ++i) {
     const int64_t n = cg * kColGroup + i * 8 + rsub;
     if (n < N && k < K)
-      v[i] = __builtin_nontemporal_load(reinterpret_cast<const float4_t *>(W + n * K + k));
+      v[i] = *reinterpret_cast<const float4_t *>(W + n * K + k);
     else
       v[i] = float4_t{1.0f, 1.0f, 1.0f, 1.0f};
   }
@@ -390,8 +455,17 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_finalize(const float *__r
     widen_bits(pairs, bits, k_tiles, col_groups, wide_groups, n);
   if (alpha && n < N) {
     float acc = 0.0f;
-    for (int64_t s = 0; s < slices; ++s)
-      acc += sums[s * Np + n];
+    // eight slices' loads are issued before the first is added (the adds keep slice order)
+    for (int64_t s0 = 0; s0 < slices; s0 += 8) {
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        v[j] = sums[((s0 + j < slices) ? s0 + j : slices - 1) * Np + n];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (s0 + j < slices)
+          acc += v[j];
+    }
     alpha[n] = acc * inv_k;
   }
   if (zero_count && blockIdx.x == 0) {
@@ -961,10 +1035,25 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint3
   uint32_t *pairs = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + P.sums_bytes + P.zeros_bytes);
   int64_t slices = P.slices;
   if (!transposed) {
-    if (N % 4 == 0 && aligned16(W) && aligned16(Wb)) { // a null Wb (no fp32 signs wanted) counts as aligned
-      const dim3 grid((unsigned)P.col_groups, (unsigned)P.slices);
-      hipLaunchKernelGGL(binarize_kn_vec, grid, dim3(kPrepBlock), 0, stream, W, Wb, pairs, sums, zeros, K, N,
-                         P.col_groups, P.Np, P.k_tiles, quantize_zero_to);
+    if (N % 4 == 0 && N >= 4 && aligned16(W) && aligned16(Wb) && P.slabs <= 65535 &&
+        (uint64_t)N * 4 < (1ull << 32)) { // a null Wb (no fp32 signs wanted) counts as aligned
+      // writes the packed operand itself (padding k tiles included): nothing is left for the relayout below
+      const dim3 grid((unsigned)P.wide_groups, (unsigned)P.slabs);
+      uint4_t *packed = reinterpret_cast<uint4_t *>(bits);
+      if (zero_count)
+        hipLaunchKernelGGL(binarize_kn_wide<true>, grid, dim3(kPrepBlock), 0, stream, W, Wb, packed, sums, zeros, K, N,
+                           P.wide_groups, P.Npw, quantize_zero_to);
+      else
+        hipLaunchKernelGGL(binarize_kn_wide<false>, grid, dim3(kPrepBlock), 0, stream, W, Wb, packed, sums, zeros, K,
+                           N, P.wide_groups, P.Npw, quantize_zero_to);
+      NBLA_HIP_LAUNCH_CHECK("binarize_kn_wide");
+      if (alpha || zero_count) {
+        hipLaunchKernelGGL(binarize_finalize, dim3((unsigned)ceil_div(N, kPrepBlock)), dim3(kPrepBlock), 0, stream, sums,
+                           zeros, alpha, zero_count, N, P.Npw, P.slabs, P.slabs * P.wide_groups, (float)1 / K, pairs,
+                           reinterpret_cast<uint4_t *>(bits), P.k_tiles, P.col_groups, P.wide_groups, (int64_t)0);
+        NBLA_HIP_LAUNCH_CHECK("binarize_finalize");
+      }
+      return NBLA_HIP_OK;
     } else {
       slices = ceil_div(K, kKSlice);
       const dim3 grid((unsigned)P.col_groups, (unsigned)slices);

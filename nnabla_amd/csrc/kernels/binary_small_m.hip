@@ -1,0 +1,294 @@
+// BinaryWeightAffine / BinaryConnectAffine forward for a handful of input rows (M <= 16), in ONE pass over W.
+//
+// With so few rows the product is bound by the weights: 4 B read and 4 B written (the fp32 signs Wb are an output of
+// the function) per weight, against 2 M flop.  The general path walks W once to binarise it and then runs the packed
+// bits through the matrix cores in further launches; here the same walk that writes Sign(W) and sums |W| per column
+// also forms the dot products, on the vector ALUs: every weight a thread has in registers is turned into its sign s
+// and added to  acc[m] += s * x[m, k]  for each of the M rows.  W is read in 1 KiB runs (a wavefront covers 256
+// consecutive columns of a row) with a second batch of rows in flight while the first is consumed.
+//
+// The rows of x are the same for every lane: they are fetched with scalar loads and never occupy vector registers.
+//
+// Work decomposition: block = kWavesK wavefronts stacked in K; wavefront wk walks kRowsPerWave rows of the block's
+// 256-column strip.  The block's wavefronts fold their accumulators over wk through LDS (fixed order), and the block writes one
+// partial row per input row, plus the |W| column sums, for its slab of K.  A second, tiny launch adds the slabs in
+// slab order, forms alpha = colsum * ((float)1 / K) and scales: y = (sum_k s * x) * alpha + bias.  Every sum runs in a
+// fixed order, so results do not change from run to run.
+#include "common.hpp"
+#include "gemm_layout.hpp"
+#include "internal.hpp"
+
+namespace nbla_hip {
+namespace {
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+// Four wavefronts stacked in K over one 256-column strip; four such blocks per CU (128 registers per lane), so the
+// whole of a 4096 x 11008 weight matrix (688 blocks) is resident at once and no second round of blocks trails behind.
+constexpr int kWavesK = 4, kWavesN = 1;
+constexpr int kThreads = 64 * kWavesK * kWavesN;
+constexpr int blocks_per_cu(int MT) { return MT >= 16 ? 2 : 4; } // sixteen rows need more than 128 registers
+constexpr int kRowsPerWave = 64;                     // rows of W one wavefront walks
+constexpr int kSlabRows = kWavesK * kRowsPerWave;    // rows of W per block
+constexpr int kWaveCols = 256;                       // 64 lanes x float4
+constexpr int kStripCols = kWavesN * kWaveCols;      // columns per block
+
+// sign.hpp:48-50: w > 0 ? 1 : (w < 0 ? -1 : zero_to).  +-0 and NaN are exactly the inputs that are neither less nor
+// greater than zero; every other input takes 1 with its own sign bit.
+__device__ __forceinline__ float sign_of(float w, float zero_to) {
+  const float one = __uint_as_float((__float_as_uint(w) & 0x80000000u) | 0x3f800000u);
+  return __builtin_islessgreater(w, 0.0f) ? one : zero_to;
+}
+
+__host__ __device__ inline int64_t small_m_slabs(int64_t K) { return ceil_div(K, kSlabRows); }
+__host__ __device__ inline int64_t small_m_padded_cols(int64_t N) { return ceil_div(N, kStripCols) * kStripCols; }
+
+// partial[slab][r][Npad]: r < MT the dot products of input row r over the slab, r == MT the |W| column sums.
+//
+// The activations never enter vector registers: x[m, k] is the same for every lane, so it is read with scalar loads
+// and enters the multiply-add as a scalar operand.  kFull (decided per block) is the interior of W, where no row or
+// column test is needed; edge blocks run the same code with clamped loads and guarded stores.
+template <int MT, int kBatch, bool kFull>
+__device__ __forceinline__ void small_m_walk(const float *__restrict__ W, float *__restrict__ Wb,
+                                             const float *__restrict__ x, int64_t M, int64_t K, int64_t N,
+                                             int64_t k_wave, int64_t n0, float zero_to, float (&acc)[MT][4],
+                                             float (&cs)[4]) {
+  constexpr int kBatches = kRowsPerWave / kBatch;
+  static_assert(kBatches % 2 == 0, "the loop below consumes two batches per trip");
+  constexpr int kXRows = (32 / MT) < 1 ? 1 : ((32 / MT) > kBatch ? kBatch : (32 / MT)); // rows whose x is fetched at once
+  const bool col_ok = kFull || n0 < N;
+  const int64_t n_ld = col_ok ? n0 : N - 4; // loads are unconditional: a clamped address, masked afterwards
+  const uint32_t lane_bytes = (uint32_t)(n_ld * 4);
+  float4_t va[kBatch], vb[kBatch];
+  auto load_batch = [&](int b, float4_t (&dst)[kBatch]) {
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      int64_t k = k_wave + b * kBatch + j;
+      if (!kFull && k >= K)
+        k = K - 1;
+      const char *row = reinterpret_cast<const char *>(W + k * N); // uniform base + 32-bit lane offset
+      // ordinary loads, nontemporal stores: the combination that streams fastest here (nontemporal loads cost a fifth)
+      dst[j] = *reinterpret_cast<const float4_t *>(row + lane_bytes);
+    }
+  };
+  auto consume_batch = [&](int b, const float4_t (&src)[kBatch]) {
+#pragma unroll
+    for (int j0 = 0; j0 < kBatch; j0 += kXRows) {
+      float xv[kXRows][MT];
+#pragma unroll
+      for (int jj = 0; jj < kXRows; ++jj)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          const int64_t k = k_wave + b * kBatch + j0 + jj;
+          const bool ok = m < M && (kFull || k < K); // uniform
+          xv[jj][m] = ok ? x[(int64_t)m * K + k] : 0.0f;
+        }
+#pragma unroll
+      for (int jj = 0; jj < kXRows; ++jj) {
+        const int j = j0 + jj;
+        const int64_t k = k_wave + b * kBatch + j;
+        float4_t w = src[j];
+        if (!kFull && k >= K)
+          w = float4_t{0.0f, 0.0f, 0.0f, 0.0f}; // |0| adds nothing, and the row's x reads as zero
+        float s[4];
+        s[0] = sign_of(w.x, zero_to), s[1] = sign_of(w.y, zero_to);
+        s[2] = sign_of(w.z, zero_to), s[3] = sign_of(w.w, zero_to);
+        if (kFull || (col_ok && k < K)) {
+          float4_t o;
+          o.x = s[0], o.y = s[1], o.z = s[2], o.w = s[3];
+          char *row = reinterpret_cast<char *>(Wb + k * N);
+          __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(row + lane_bytes));
+        }
+        cs[0] += fabsf(w.x), cs[1] += fabsf(w.y), cs[2] += fabsf(w.z), cs[3] += fabsf(w.w);
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+          for (int c = 0; c < 4; ++c)
+            acc[m][c] = __builtin_fmaf(s[c], xv[jj][m], acc[m][c]);
+      }
+    }
+  };
+  // Two batches of rows are in registers at any time: one being consumed, one in flight.  The loop is kept rolled
+  // so that the compiler does not hoist further batches (their registers would spill).
+  load_batch(0, va);
+#pragma clang loop unroll(disable)
+  for (int b = 0; b < kBatches; b += 2) {
+    load_batch(b + 1, vb);
+    consume_batch(b, va);
+    if (b + 2 < kBatches)
+      load_batch(b + 2, va);
+    consume_batch(b + 1, vb);
+  }
+}
+
+template <int MT, int kBatch>
+__global__ __launch_bounds__(kThreads, blocks_per_cu(MT)) void binary_affine_small_m(const float *__restrict__ W, float *__restrict__ Wb,
+                                                                  const float *__restrict__ x,
+                                                                  float *__restrict__ partial, int64_t M, int64_t K,
+                                                                  int64_t N, int64_t Npad, float zero_to) {
+  constexpr int kVals = (MT + 1) * 4; // accumulators per lane
+  __shared__ __attribute__((aligned(16))) float red[2 * kWavesN * kVals * 64];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // uniform: row indices stay in scalar registers
+  const int wn = wave % kWavesN, wk = wave / kWavesN;
+  const int64_t slab = blockIdx.y;
+  const int64_t k_slab = slab * kSlabRows;
+  const int64_t n0 = (int64_t)blockIdx.x * kStripCols + wn * kWaveCols + 4 * lane;
+  const int64_t k_wave = k_slab + wk * kRowsPerWave;
+
+  float acc[MT][4];
+  float cs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      acc[m][c] = 0.0f;
+
+  const bool full = k_slab + kSlabRows <= K && ((int64_t)blockIdx.x + 1) * kStripCols <= N && M == MT;
+  if (full)
+    small_m_walk<MT, kBatch, true>(W, Wb, x, M, K, N, k_wave, n0, zero_to, acc, cs);
+  else
+    small_m_walk<MT, kBatch, false>(W, Wb, x, M, K, N, k_wave, n0, zero_to, acc, cs);
+
+  // Fold over wk in a fixed order: (wk0 + wk2) + (wk1 + wk3), through LDS.
+  auto slot = [&](int s) { return red + ((size_t)(s * kWavesN + wn) * kVals) * 64 + lane; };
+  auto put = [&](float *dst) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        dst[(m * 4 + c) * 64] = acc[m][c];
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      dst[(MT * 4 + c) * 64] = cs[c];
+  };
+  auto add = [&](const float *src) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        acc[m][c] += src[(m * 4 + c) * 64];
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      cs[c] += src[(MT * 4 + c) * 64];
+  };
+  if (wk >= 2)
+    put(slot(wk - 2));
+  __syncthreads();
+  if (wk < 2)
+    add(slot(wk));
+  __syncthreads();
+  if (wk == 1)
+    put(slot(1));
+  __syncthreads();
+  if (wk != 0)
+    return;
+  add(slot(1));
+  float *out = partial + (size_t)slab * (MT + 1) * Npad + n0; // n0 < Npad always
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    float4_t o;
+    o.x = acc[m][0], o.y = acc[m][1], o.z = acc[m][2], o.w = acc[m][3];
+    *reinterpret_cast<float4_t *>(out + (size_t)m * Npad) = o;
+  }
+  float4_t o;
+  o.x = cs[0], o.y = cs[1], o.z = cs[2], o.w = cs[3];
+  *reinterpret_cast<float4_t *>(out + (size_t)MT * Npad) = o;
+}
+
+// Thread (m, four columns): the slabs in slab order, alpha (binary_weight_affine.cpp:68: the column sum times the
+// rounded reciprocal of K), scale, bias.
+template <int MT>
+__global__ __launch_bounds__(256) void binary_affine_small_m_finish(const float *__restrict__ partial,
+                                                                    float *__restrict__ alpha,
+                                                                    const float *__restrict__ bias,
+                                                                    float *__restrict__ y, int64_t M, int64_t N,
+                                                                    int64_t Npad, int64_t slabs, float inv_k) {
+  const int64_t n0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  const int m = blockIdx.y;
+  if (n0 >= N)
+    return;
+  float4_t dot = {0.0f, 0.0f, 0.0f, 0.0f}, cs = {0.0f, 0.0f, 0.0f, 0.0f};
+  // eight slabs' loads are issued before the first is added (the adds keep slab order)
+  constexpr int kAhead = 8;
+  const size_t slab_stride = (size_t)(MT + 1) * Npad;
+  for (int64_t s0 = 0; s0 < slabs; s0 += kAhead) {
+    float4_t d[kAhead], c[kAhead];
+#pragma unroll
+    for (int j = 0; j < kAhead; ++j) {
+      const int64_t s = (s0 + j < slabs) ? s0 + j : slabs - 1; // clamped loads, masked below
+      const float *p = partial + (size_t)s * slab_stride + n0;
+      d[j] = *reinterpret_cast<const float4_t *>(p + (size_t)m * Npad);
+      if (alpha)
+        c[j] = *reinterpret_cast<const float4_t *>(p + (size_t)MT * Npad);
+    }
+#pragma unroll
+    for (int j = 0; j < kAhead; ++j) {
+      if (s0 + j >= slabs)
+        break;
+      dot.x += d[j].x, dot.y += d[j].y, dot.z += d[j].z, dot.w += d[j].w;
+      if (alpha)
+        cs.x += c[j].x, cs.y += c[j].y, cs.z += c[j].z, cs.w += c[j].w;
+    }
+  }
+  if (alpha) {
+    float4_t a;
+    a.x = cs.x * inv_k, a.y = cs.y * inv_k, a.z = cs.z * inv_k, a.w = cs.w * inv_k;
+    if (m == 0)
+      *reinterpret_cast<float4_t *>(alpha + n0) = a;
+    dot.x = dot.x * a.x, dot.y = dot.y * a.y, dot.z = dot.z * a.z, dot.w = dot.w * a.w;
+  }
+  if (bias) {
+    const float4_t b = *reinterpret_cast<const float4_t *>(bias + n0);
+    dot.x = dot.x + b.x, dot.y = dot.y + b.y, dot.z = dot.z + b.z, dot.w = dot.w + b.w;
+  }
+  *reinterpret_cast<float4_t *>(y + (size_t)m * N + n0) = dot;
+}
+
+template <int MT, int kBatch>
+int launch_small_m(const float *x, const float *W, float *Wb, float *alpha, const float *bias, float *y, int64_t M,
+                   int64_t K, int64_t N, float zero_to, float *partial, hipStream_t stream) {
+  const int64_t Npad = small_m_padded_cols(N), slabs = small_m_slabs(K);
+  hipLaunchKernelGGL((binary_affine_small_m<MT, kBatch>), dim3((unsigned)(Npad / kStripCols), (unsigned)slabs),
+                     dim3(kThreads), 0, stream, W, Wb, x, partial, M, K, N, Npad, zero_to);
+  NBLA_HIP_LAUNCH_CHECK("binary_affine_small_m");
+  hipLaunchKernelGGL(binary_affine_small_m_finish<MT>, dim3((unsigned)ceil_div(N / 4, 256), (unsigned)M), dim3(256), 0,
+                     stream, partial, alpha, bias, y, M, N, Npad, slabs, (float)1 / K);
+  NBLA_HIP_LAUNCH_CHECK("binary_affine_small_m_finish");
+  return NBLA_HIP_OK;
+}
+
+} // namespace
+
+bool small_m_affine_applies(const float *x, const float *W, const float *Wb, const float *alpha, const float *bias,
+                            const float *y, int64_t M, int64_t K, int64_t N) {
+  return M >= 1 && M <= kSmallMMaxRows && N % 4 == 0 && Wb && aligned16(W) && aligned16(Wb) && aligned16(y) &&
+         aligned16(alpha) && aligned16(bias) && small_m_slabs(K) <= 65535;
+}
+
+size_t small_m_affine_workspace_bytes(int64_t M, int64_t K, int64_t N) {
+  if (M < 1 || M > kSmallMMaxRows)
+    return 0;
+  const int64_t mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
+  return (size_t)small_m_slabs(K) * (mt + 1) * small_m_padded_cols(N) * sizeof(float);
+}
+
+int launch_small_m_affine(const float *x, const float *W, float *Wb, float *alpha, const float *bias, float *y,
+                          int64_t M, int64_t K, int64_t N, float zero_to, void *workspace, size_t workspace_bytes,
+                          hipStream_t stream) {
+  if (workspace_bytes < small_m_affine_workspace_bytes(M, K, N) || !aligned16(workspace))
+    return fail(NBLA_HIP_ERR_MEMORY, "small-M binary affine workspace too small or misaligned.");
+  float *partial = static_cast<float *>(workspace);
+  if (M <= 1)
+    return launch_small_m<1, 4>(x, W, Wb, alpha, bias, y, M, K, N, zero_to, partial, stream);
+  if (M <= 2)
+    return launch_small_m<2, 4>(x, W, Wb, alpha, bias, y, M, K, N, zero_to, partial, stream);
+  if (M <= 4)
+    return launch_small_m<4, 4>(x, W, Wb, alpha, bias, y, M, K, N, zero_to, partial, stream);
+  if (M <= 8)
+    return launch_small_m<8, 4>(x, W, Wb, alpha, bias, y, M, K, N, zero_to, partial, stream);
+  return launch_small_m<16, 4>(x, W, Wb, alpha, bias, y, M, K, N, zero_to, partial, stream);
+}
+
+} // namespace nbla_hip

@@ -127,15 +127,37 @@ def test_digit_operand_of_a_strided_matrix(dev, M, K, ldx):
 
 
 def test_digit_operand_marks_non_finite_rows(dev):
-    x = np.ones((5, 64), np.float32)
+    x = np.ones((40, 64), np.float32)
     x[1, 3] = np.inf
     x[3, 60] = np.nan
     W = np.ones((64, 64), np.float32)
-    _, shift, _ = unpack_digits(to_np(kernels.split_digits(_dev(x, dev), 5, 64)), 5, 64)
+    _, shift, _ = unpack_digits(to_np(kernels.split_digits(_dev(x, dev), 40, 64)), 40, 64)
     assert shift[1] == -2 ** 31 and shift[3] == -2 ** 31 and shift[0] == shift[2] == shift[4]
+    y, _ = kernels.binary_connect_affine(_dev(x, dev), _dev(W, dev))      # 40 rows: the digit-operand product
+    y = to_np(y)
+    ok = np.ones(40, bool)
+    ok[[1, 3]] = False
+    assert np.isnan(y[[1, 3]]).all() and np.array_equal(y[ok], np.full((38, 64), 64.0, np.float32))
+
+
+def test_few_rows_propagate_non_finite_values_per_element(dev):
+    """The one-pass product for a handful of rows multiplies and adds in fp32, so Inf and NaN spread exactly as in
+    the reference's product (affine.cpp:87-95): per output element."""
+    rng = np.random.RandomState(11)
+    x = rng.randn(5, 64).astype(np.float32)
+    x[1, 3] = np.inf
+    x[2, 7] = -np.inf
+    x[2, 9] = np.inf
+    x[3, 60] = np.nan
+    W = rng.randn(64, 64).astype(np.float32)
     y, _ = kernels.binary_connect_affine(_dev(x, dev), _dev(W, dev))
     y = to_np(y)
-    assert np.isnan(y[[1, 3]]).all() and np.array_equal(y[[0, 2, 4]], np.full((3, 64), 64.0, np.float32))
+    ref, _ = oracle.binary_connect_affine(x, W, None, 1.0)
+    assert np.array_equal(np.isnan(y), np.isnan(ref)) and np.array_equal(np.isposinf(y), np.isposinf(ref))
+    assert np.array_equal(np.isneginf(y), np.isneginf(ref))
+    fin = np.isfinite(ref)
+    assert fin[[0, 4]].all() and np.abs(y[fin] - ref[fin]).max() <= 1e-4 * np.abs(ref[fin]).max()
+    assert np.isinf(y[1]).all() and np.isnan(y[3]).all()
 
 
 @pytest.mark.parametrize("M,K,N", [(3, 16384 + 40, 70), (40, 40000, 64)])
@@ -176,6 +198,33 @@ def test_binary_connect_affine_matches_oracle(dev, M, K, N):
     y64 = x.astype(np.float64) @ ref_Wb.astype(np.float64) + b
     assert max_rel_err(to_np(y), ref_y) <= TOL
     assert max_rel_err(to_np(y), y64) <= TIGHT
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 9, 16])
+@pytest.mark.parametrize("K,N", [(300, 1028), (256, 256), (1000, 516), (64, 4), (4097, 260)])
+def test_few_rows_one_pass_product(dev, M, K, N):
+    """M <= 16 with N % 4 == 0 runs the one-pass form (signs, column sums and dot products in a single walk over W):
+    ragged last slab of K, ragged last strip of N, every row count the templates round up from; Wb bit-exact, alpha
+    and y against the oracle and float64.  Weights include exact zeros of both signs and a NaN (Sign -> zero_to)."""
+    x, W = _data(M, K, N, seed=M * 1000 + K)
+    W.ravel()[::7] = 0.0
+    W.ravel()[3::11] = -0.0
+    W[K // 2, N // 2] = np.nan
+    b = np.random.RandomState(2).randn(N).astype(np.float32)
+    for q0 in (1.0, -1.0, 0.0, 0.5):
+        ref_y, ref_Wb, ref_alpha = oracle.binary_weight_affine(x, W, b, q0)
+        y, Wb, alpha = kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev), _dev(b, dev), q0)
+        assert bits_equal(to_np(Wb), ref_Wb), first_mismatch(to_np(Wb), ref_Wb)
+        col_ok = ~np.isnan(ref_alpha)                       # the NaN weight's column has a NaN mean in both
+        assert np.array_equal(np.isnan(to_np(alpha)), ~col_ok)
+        np.testing.assert_allclose(to_np(alpha)[col_ok], ref_alpha[col_ok], rtol=2e-6)
+        assert max_rel_err(to_np(y)[:, col_ok], ref_y[:, col_ok]) <= TIGHT * 4
+        assert np.isnan(to_np(y)[:, ~col_ok]).all()
+        ref_y, ref_Wb = oracle.binary_connect_affine(x, W, None, q0)
+        y, Wb = kernels.binary_connect_affine(_dev(x, dev), _dev(W, dev), None, q0)
+        assert bits_equal(to_np(Wb), ref_Wb)
+        y64 = x.astype(np.float64) @ ref_Wb.astype(np.float64)
+        assert max_rel_err(to_np(y), y64) <= TIGHT and max_rel_err(to_np(y), ref_y) <= TIGHT * 4
 
 
 @pytest.mark.parametrize("M,K,N", [(3100, 96, 5732), (3072, 64, 11008)])
