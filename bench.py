@@ -26,10 +26,39 @@ if ROOT not in sys.path:
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix
 PEAK_INT8_MFMA_TOPS = 5000.0    # MI355X dense int8 matrix
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
-# HBM-side bytes of one launch of the dominant kernel at the headline shape, from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# runs of this same command (scaled by what a streaming kernel of known size reads on those counters):
-# 264.0 MB fetched + 180.2 MB written.
-GEMM_TRAFFIC_BYTES_PROFILED = 452.7e6
+HEADLINE_PROFILE = os.path.join(ROOT, "profiles", "binary_weight_affine_4096x4096x11008.md")
+KERNEL_SOURCES = ("gemm_bits.hip", "gemm_layout.hpp")
+
+
+def kernel_source_sha():
+    """sha256 over the sources of the dominant kernel: what a committed profile is stamped with."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "nnabla_amd", "csrc", "kernels", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def profiled_traffic():
+    """HBM-side bytes of one launch of the dominant kernel, read from the committed rocprofv3 summary (its line
+    `traffic: fetch_bytes=... write_bytes=... source_sha=...`, FETCH_SIZE / WRITE_SIZE scaled by what a streaming kernel
+    of known size reads on those counters).  Only reported while the kernel's sources are the ones that were profiled."""
+    import re
+    try:
+        text = open(HEADLINE_PROFILE).read()
+    except OSError:
+        return None, "no committed profile"
+    m = re.search(r"traffic: fetch_bytes=([0-9.e+]+) write_bytes=([0-9.e+]+) source_sha=([0-9a-f]+)", text)
+    if not m:
+        return None, "the committed profile carries no traffic line"
+    if m.group(3) != kernel_source_sha():
+        return None, "kernel sources changed since the committed profile (%s): traffic not carried over" % m.group(3)
+    return float(m.group(1)) + float(m.group(2)), ("bytes per launch between L2 and the memory side: %.1f MB fetched + "
+                                                   "%.1f MB written, rocprofv3 counters of the profile under profiles/ "
+                                                   "taken on these kernel sources (%s); algorithmic: 56.2 MB read + "
+                                                   "180.4 MB written" % (float(m.group(1)) / 1e6,
+                                                                         float(m.group(2)) / 1e6, m.group(3)))
 
 
 def _events(n):
@@ -40,9 +69,11 @@ def _events(n):
 def bench_binary_weight_affine(M, K, N, steps, warmup, dev):
     import torch
     from nnabla_amd import kernels as k
-    g = torch.Generator(device="cpu").manual_seed(313)
-    x = torch.randn(M, K, generator=g).to(dev)
-    W = (torch.randn(K, N, generator=g) * 0.02).to(dev)
+    # drawn on the device: host-side generation of 60 M values would leave the GPU idle for seconds right before the
+    # timed steps, and the first launches after idle run on ramping clocks
+    g = torch.Generator(device=dev).manual_seed(313)
+    x = torch.randn(M, K, generator=g, device=dev)
+    W = torch.randn(K, N, generator=g, device=dev) * 0.02
     Wb = torch.empty_like(W)
     alpha = torch.empty(N, device=dev)
     y = torch.empty(M, N, device=dev)
@@ -87,6 +118,22 @@ def bench_binary_weight_affine(M, K, N, steps, warmup, dev):
     gemm = sum(e[2].elapsed_time(e[3]) for e in evs) / steps
     return {"ms_per_step": wall * 1e3 / steps, "prepare_ms": prep, "split_ms": split, "gemm_ms": gemm,
             "flop": 2.0 * M * K * N}
+
+
+def bench_whole_forward(M, K, N, steps, warmup, dev):
+    """BinaryWeightAffine forward through the whole-function entry point (what the Function class calls)."""
+    import torch
+    from nnabla_amd import kernels as k
+    g = torch.Generator(device="cpu").manual_seed(313)
+    x = torch.randn(M, K, generator=g).to(dev)
+    W = (torch.randn(K, N, generator=g) * 0.02).to(dev)
+    ws = k.binary_affine_workspace(M, K, N, x)
+    y, Wb, alpha = torch.empty(M, N, device=dev), torch.empty_like(W), torch.empty(N, device=dev)
+    ms = time_kernel(lambda: k.binary_weight_affine(x, W, None, 1.0, workspace=ws, out=y, Wb=Wb, alpha=alpha), steps,
+                     warmup)
+    nbytes = 8.0 * K * N + 4.0 * M * K + 4.0 * M * N + 4.0 * N   # read W, write Wb; x, y, alpha
+    return {"ms_per_step": ms, "forward_bytes_model": nbytes, "forward_GBs": nbytes / ms / 1e6,
+            "forward_frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
 
 
 def time_kernel(fn, iters, warmup=3):
@@ -330,18 +377,26 @@ def main():
     kernels.init(0)
 
     M, K, N = 4096, 4096, 11008
+    # The other sections run first: the headline steps are then timed on a device that is already at its working
+    # clocks (the first dozens of launches after idle run on ramping clocks).  With --section headline there is
+    # nothing before them and the figure is a cold one.
+    sweep = {}
+    for m in ((1, 8, 16, 64, 512) if args.section == "all" else ()):
+        s = bench_whole_forward(m, K, N, max(10, args.steps), 5, dev)
+        if m > 16:   # the product runs on the matrix cores from packed bits: its share, timed between events
+            t = bench_binary_weight_affine(m, K, N, max(5, args.steps // 2), 2, dev)
+            packed_bytes = K * N / 8 + 3.0 * m * K + 4.0 * m * N + 4.0 * N
+            s.update({"gemm_ms": t["gemm_ms"], "prepare_ms": t["prepare_ms"], "gemm_TFLOPs": t["flop"] / t["gemm_ms"] / 1e9,
+                      "gemm_weight_GBs": packed_bytes / t["gemm_ms"] / 1e6})
+        else:
+            s["path"] = "one pass over W on the vector ALUs (no packed bits, no separate product launch)"
+        sweep["M=%d" % m] = s
+    quant = bench_quantizers(dev, max(10, args.steps)) if args.section != "headline" else {}
+    other = bench_other_configs(dev, max(5, args.steps // 2)) if args.section == "all" else {}
     r = bench_binary_weight_affine(M, K, N, args.steps, args.warmup, dev)
     tflops = r["flop"] / (r["ms_per_step"] * 1e-3) / 1e12
     gemm_tflops = r["flop"] / (r["gemm_ms"] * 1e-3) / 1e12
-    sweep = {}
-    for m in ((1, 8, 64, 512) if args.section == "all" else ()):
-        s = bench_binary_weight_affine(m, K, N, max(5, args.steps // 2), 2, dev)
-        packed_bytes = K * N / 8 + 3.0 * m * K + 4.0 * m * N + 4.0 * N
-        sweep["M=%d" % m] = {"ms_per_step": s["ms_per_step"], "gemm_ms": s["gemm_ms"], "prepare_ms": s["prepare_ms"],
-                             "gemm_TFLOPs": s["flop"] / s["gemm_ms"] / 1e9,
-                             "gemm_weight_GBs": packed_bytes / s["gemm_ms"] / 1e6}
-    quant = bench_quantizers(dev, max(10, args.steps)) if args.section != "headline" else {}
-    other = bench_other_configs(dev, max(5, args.steps // 2)) if args.section == "all" else {}
+    traffic, traffic_note = profiled_traffic()
     line = {
         "metric": "binary-weight affine TFLOP/s + quantizer GB/s, % of MI355X roofline",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -351,9 +406,7 @@ def main():
                                "quantize_zero_to=1, no bias; whole forward = sign/alpha/pack + split + MFMA product",
                    "M": M, "K": K, "N": N},
         "roofline": {"bound": "mfma", "achieved": 3 * gemm_tflops, "peak": PEAK_INT8_MFMA_TOPS, "unit": "TOP/s",
-                     "frac": 3 * gemm_tflops / PEAK_INT8_MFMA_TOPS, "traffic": GEMM_TRAFFIC_BYTES_PROFILED,
-                     "traffic_note": "bytes per launch between L2 and the memory side, profiled (not live); "
-                                     "algorithmic: 56.2 MB read + 180.4 MB written",
+                     "frac": 3 * gemm_tflops / PEAK_INT8_MFMA_TOPS, "traffic": traffic, "traffic_note": traffic_note,
                      "kernel": "gemm_bits_kernel<32,512,1,4,1,false>", "kernel_ms": r["gemm_ms"],
                      "note": "int8 operations issued (3 digit planes x 2*M*K*N) against the int8 MFMA peak",
                      "fp32_equiv_TFLOPs": gemm_tflops, "fp32_equiv_over_fp32_mfma_peak": gemm_tflops / PEAK_FP32_MFMA_TFLOPS},

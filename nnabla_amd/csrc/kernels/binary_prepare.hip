@@ -710,12 +710,13 @@ __global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const floa
   static_assert(kPer * 16 < 256, "a lane's partial sum of kPer * 16 values below 2^23 fits an int");
   constexpr int kSlots = 32 / kRows;
   __shared__ uint32_t s_max[kFusedWaves][kRows];
+  __shared__ uint32_t s_low[kFusedWaves][kRows];
   __shared__ long long s_sum[kFusedWaves][kRows];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane % kRows, g = (lane / kRows) & 1, ts = lane / (2 * kRows);
   const int64_t m = (int64_t)blockIdx.x * kRows + r;
   if (blockIdx.x == 0 && threadIdx.x == 0)
-    shift[rows] = 1; // the operand's flag word: a row-scaled operand is never in the narrow form
+    shift[rows] = 1; // the operand's flag word: a row-scaled operand is never in the column operands' narrow form
   const float *row = x + m * ldx;
   float4_t v[kPer][4];
   uint32_t amax = 0u;
@@ -748,6 +749,7 @@ __global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const floa
     amax = max(amax, s_max[w][r]);
   const bool bad = amax >= 0x7f800000u;
   const int s = (bad || amax == 0u) ? 0 : digit_shift(amax);
+  uint32_t low = 0u; // OR of the two lower digits of the row's values: zero for a one-digit row
   int part = 0;
 #pragma unroll
   for (int t = 0; t < kPer; ++t) {
@@ -760,8 +762,10 @@ __global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const floa
       q[4 * i + 3] = bad ? 0 : to_fixed(v[t][i].w, s);
     }
 #pragma unroll
-    for (int j = 0; j < 16; ++j)
+    for (int j = 0; j < 16; ++j) {
       part += q[j];
+      low |= (uint32_t)q[j] & 0xffffu; // q = d0 * 65536 + d1 * 256 + d2: d1 = d2 = 0 exactly when this is zero
+    }
     const int64_t kt = ((int64_t)wave * kPer + t) * kSlots + ts;
     if (kt < k_tiles) {
       const int64_t rb = m / kFragRows;
@@ -770,18 +774,26 @@ __global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const floa
   }
   long long acc = part;
 #pragma unroll
-  for (int off = kRows; off < 64; off <<= 1)
+  for (int off = kRows; off < 64; off <<= 1) {
     acc += __shfl_xor(acc, off);
-  if (lane < kRows)
+    low |= (uint32_t)__shfl_xor((int)low, off);
+  }
+  if (lane < kRows) {
     s_sum[wave][lane] = acc;
+    s_low[wave][lane] = low;
+  }
   __syncthreads();
   if (threadIdx.x < kRows) {
     long long total = 0;
+    uint32_t any_low = 0u;
 #pragma unroll
-    for (int w = 0; w < kFusedWaves; ++w)
+    for (int w = 0; w < kFusedWaves; ++w) {
       total += s_sum[w][threadIdx.x];
+      any_low |= s_low[w][threadIdx.x];
+    }
     sums[m] = total; // a single chunk: K <= kChunkK
-    shift[m] = bad ? kBadRow : s;
+    // one-digit row: every value sits in the top digit alone (all-zero and padding rows included)
+    shift[m] = bad ? kBadRow : (any_low == 0u ? s + kOneDigitBias : s);
   }
 }
 

@@ -108,16 +108,23 @@ __device__ __forceinline__ float finish_dot(int a0, int a1, int a2, int s_hi, in
 // kWavesK > 1 splits the contraction inside the block: wavefront group wk multiplies k steps wk, wk + kWavesK, ...
 // of the same output tile (a stage then holds kWavesK consecutive k steps) and the groups' int32 accumulators are
 // added through LDS at the end, exactly.  Used when the output has too few tiles to occupy the CUs.
-template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, bool kSwap>
-__global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN * kWavesK >= 8 ? 1 : 2)) void gemm_bits_kernel(GemmBitsArgs a) {
+//
+// kUsed = 1: every row of the block's row blocks is a one-digit row (gemm_layout.hpp: the two lower digits are zero).
+// Only the top-digit fragments are copied and multiplied, into the top accumulator; the lower accumulators stay
+// zero and the epilogue is the same.  A third of the MFMAs and a third of the digit traffic, same bits.
+template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, bool kSwap, int kUsed>
+__device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *smem) {
 #if defined(__HIP_DEVICE_COMPILE__) // the host pass only needs the launch stub; the body uses LDS address-space pointers
+  static_assert(kUsed == 1 || kUsed == kDigits, "digits multiplied");
+  constexpr int kFirst = 0; // first digit (and accumulator) in use: digits kFirst .. kFirst + kUsed - 1
   constexpr int kWavesMN = kWavesM * kWavesN;
   constexpr int kWaves = kWavesMN * kWavesK;
   constexpr int MF = BM / kWavesM / 32;  // X fragments per wavefront (rows)
   constexpr int NF = BN / kWavesN / 32;  // B fragments per wavefront (columns)
   static_assert(BN % kWideGroup == 0 && (kWideGroup / 32) % NF == 0, "a wavefront's fragments share one wide group");
   constexpr int kASegs = BM / 32;            // row blocks per tile
-  constexpr int kSegFrags = 2 * kDigits;     // fragments per row block per k step (2 k tiles x 3 digits)
+  constexpr int kSegFrags = 2 * kUsed;       // fragments copied per row block per k step (2 k tiles x digits in use)
+  constexpr int kSrcSegFrags = 2 * kDigits;  // fragments per row block per k step in the operand
   constexpr int kAFrags = kASegs * kSegFrags;
   constexpr int kBChunks = 2 * BN / kWideGroup; // 1 KiB chunks of packed words per k step (2 k tiles x wide groups)
   // One copy instruction moves 1 KiB (a fragment, or the words of one wide group); the kChunks copies of a k step
@@ -131,8 +138,6 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
   constexpr int kStages = gemm_bits_stages(BM, BN, kWavesMN, kWavesK);
   constexpr int kDepth = kStages - 1; // k steps in flight ahead of the one being multiplied
   static_assert(kDepth >= 2 && (kDepth - 1) * (kPerWave + 1) < 64, "vmcnt is a 6-bit counter");
-
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
   if (a.split_steps > 0) {
     const int64_t begin = a.step_begin + (int64_t)blockIdx.y * a.split_steps;
@@ -164,12 +169,13 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
     const int kk = (cs / kStepChunks) % kWavesK;      // k step inside the stage
     const int c = cs - (cs / kStepChunks) * kStepChunks;
     if (c < kAFrags) {
-      const int seg = c / kSegFrags, rem = c - seg * kSegFrags;
+      const int seg = c / kSegFrags, rem = c - seg * kSegFrags; // rem = (k tile of the step, digit in use)
+      const int t = rem / kUsed, d = kFirst + rem - t * kUsed;
       int64_t rb = bm * kASegs + seg;
       if (rb >= a.row_blocks)
         rb = a.row_blocks - 1;
-      src_step[p] = kSegFrags * 64;
-      src[p] = a.xd + (rb * a.x_k_tiles * kDigits + rem) * 64 + kk * src_step[p];
+      src_step[p] = kSrcSegFrags * 64;
+      src[p] = a.xd + (rb * a.x_k_tiles * kDigits + t * kDigits + d) * 64 + kk * src_step[p];
     } else {
       // packed words: chunk = (k tile of the step, wide group of the tile)
       const int cb = c - kAFrags;
@@ -224,13 +230,13 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
           acc[d][i][j][r] = 0;
 
   // Fragment fetch and the MFMA block of one k tile (t = 0, 1) of a staged step.
-  auto read_a = [&](int buf, int t, uint4_t (&af)[MF][kDigits]) {
+  auto read_a = [&](int buf, int t, uint4_t (&af)[MF][kUsed]) {
     const uint4_t *sa = reinterpret_cast<const uint4_t *>(smem + buf * kStageBytes + wk * kStepBytes);
 #pragma unroll
     for (int i = 0; i < MF; ++i)
 #pragma unroll
-      for (int d = 0; d < kDigits; ++d)
-        af[i][d] = sa[((wm * MF + i) * kSegFrags + t * kDigits + d) * 64 + lane];
+      for (int d = 0; d < kUsed; ++d)
+        af[i][d] = sa[((wm * MF + i) * kSegFrags + t * kUsed + d) * 64 + lane];
   };
   const int frag0 = (wn * NF) % (kWideGroup / 32); // index of this wavefront's first column fragment in its group
   auto read_words = [&](int buf, int t, uint4_t &words) {
@@ -244,7 +250,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
     frag_mask[j] = 0x01010101u << (frag0 + j);
     asm volatile("" : "+s"(frag_mask[j]));
   }
-  auto mma = [&](const uint4_t (&af)[MF][kDigits], const uint4_t &words, auto j_begin, auto j_end) {
+  auto mma = [&](const uint4_t (&af)[MF][kUsed], const uint4_t &words, auto j_begin, auto j_end) {
 #pragma unroll
     for (int j = decltype(j_begin)::value; j < decltype(j_end)::value; ++j) {
       uint4_t bf;
@@ -253,15 +259,15 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
       bf.z = words.z & frag_mask[j];
       bf.w = words.w & frag_mask[j];
 #pragma unroll
-      for (int d = 0; d < kDigits; ++d)
+      for (int d = 0; d < kUsed; ++d)
 #pragma unroll
         for (int i = 0; i < MF; ++i) {
-          acc[d][i][j] = kSwap ? __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, bf),
-                                                                       __builtin_bit_cast(i32x4_t, af[i][d]),
-                                                                       acc[d][i][j], 0, 0, 0)
-                               : __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, af[i][d]),
-                                                                       __builtin_bit_cast(i32x4_t, bf),
-                                                                       acc[d][i][j], 0, 0, 0);
+          acc[kFirst + d][i][j] = kSwap ? __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, bf),
+                                                                                __builtin_bit_cast(i32x4_t, af[i][d]),
+                                                                                acc[kFirst + d][i][j], 0, 0, 0)
+                                        : __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, af[i][d]),
+                                                                                __builtin_bit_cast(i32x4_t, bf),
+                                                                                acc[kFirst + d][i][j], 0, 0, 0);
         }
     }
   };
@@ -272,7 +278,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
   typedef std::integral_constant<int, 0> J0;
   typedef std::integral_constant<int, 1> J1;
   typedef std::integral_constant<int, NF> JN;
-  uint4_t af0[MF][kDigits], af1[MF][kDigits];
+  uint4_t af0[MF][kUsed], af1[MF][kUsed];
   uint4_t w0, w1;
   // stages are numbered by their first k step; the operands are padded so that the number of k steps is a multiple
   // of kWavesK
@@ -332,7 +338,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
     uint4_t *red = reinterpret_cast<uint4_t *>(smem);
     constexpr int kRegs4 = MF * NF * 4; // uint4 per lane per digit
 #pragma unroll
-    for (int d = 0; d < kDigits; ++d) {
+    for (int d = kFirst; d < kFirst + kUsed; ++d) {
       NBLA_BARRIER();
       if (wk > 0 && !idle) {
         uint4_t *dst = red + (size_t)((wk - 1) * kWavesMN + wmn) * kRegs4 * 64 + lane;
@@ -415,7 +421,10 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
           sum01 = *reinterpret_cast<const i32x4_t *>(a.sums + ml); // two int64 as (lo, hi) words
           sum23 = *reinterpret_cast<const i32x4_t *>(a.sums + ml + 2);
         }
-        const i32x4_t sh = *reinterpret_cast<const i32x4_t *>(a.shift + ml);
+        i32x4_t sh = *reinterpret_cast<const i32x4_t *>(a.shift + ml);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          sh[e] = plain_shift(sh[e]); // one-digit rows store their shift with a bias (kBadRow is negative: unchanged)
         // sum = s_hi * 65536 + s_lo with s_lo in [0, 65536)
         const uint32_t lo_w[4] = {(uint32_t)sum01.x, (uint32_t)sum01.z, (uint32_t)sum23.x, (uint32_t)sum23.z};
         const int hi_w[4] = {sum01.y, sum01.w, sum23.y, sum23.w};
@@ -457,7 +466,7 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
       if (m >= a.M)
         continue;
       const long long sum = a.use_sums ? a.sums[m] : 0;
-      const int s_hi = (int)(sum >> 16), s_lo = (int)(sum & 0xffff), sh = a.shift[m];
+      const int s_hi = (int)(sum >> 16), s_lo = (int)(sum & 0xffff), sh = plain_shift(a.shift[m]);
       float *row = row_ptr(m);
 #pragma unroll
       for (int j = 0; j < NF; ++j) {
@@ -492,6 +501,25 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
     }
   }
 #endif
+}
+
+template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, bool kSwap>
+__global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN * kWavesK >= 8 ? 1 : 2)) void gemm_bits_kernel(GemmBitsArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  // Are all rows of this block's row blocks one-digit rows?  (Same tile mapping as the body; rows past the operand
+  // are clamped to its last row, as the copies are.)
+  int64_t bm, bn;
+  band_tile<8>(blockIdx.x, a.blocks_m, a.blocks_n, bm, bn);
+  const int64_t rows = a.row_blocks * kFragRows;
+  bool one = true;
+  for (int r = threadIdx.x; r < BM; r += kWavesM * kWavesN * kWavesK * 64) {
+    const int64_t m = bm * BM + r;
+    one = one && one_digit_row(a.shift[m < rows ? m : rows - 1]);
+  }
+  if (__syncthreads_and(one))
+    gemm_bits_body<BM, BN, kWavesM, kWavesN, kWavesK, kSwap, 1>(a, smem);
+  else
+    gemm_bits_body<BM, BN, kWavesM, kWavesN, kWavesK, kSwap, kDigits>(a, smem);
 }
 
 template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, bool kSwap>

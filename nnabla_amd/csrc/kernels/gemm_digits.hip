@@ -63,14 +63,19 @@ constexpr int kStagesShared = 3, kStagesAlone = 6;
 // and barrier waits are covered by the other's MFMAs.
 // kNarrow: the B operand holds every value in its lowest digit alone (a small integer): three products
 // a_t x b2 -> accumulator t, nothing dropped, and only the lowest-digit fragments of B are copied.
+// kOneA (only with kNarrow): every row of the tile's A row blocks is a one-digit row (gemm_layout.hpp: its value sits
+// in the top digit): a single product a0 x b2 -> accumulator 0, and only the top-digit fragments of A and the
+// lowest-digit fragments of B are copied (eight per k tile, dealt evenly over the wavefronts).  Same bits as the other
+// forms: the other digits are zero.
 // kGroups = 2 (outputs of at most one tile per CU): eight wavefronts, two groups of four; group g multiplies the k
 // tiles g, g + 2, ... of the same output tile (a stage then holds two consecutive k tiles), so every SIMD has a second
 // wavefront to issue from while the first waits.  At the end the groups swap halves of their int32 accumulators
 // through LDS (exactly) and group g finishes row fragment g of each wavefront tile.
-template <bool kNarrow, int kStages, int kGroups>
+template <bool kNarrow, bool kOneA, int kStages, int kGroups>
 __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsigned char *smem) {
 #if defined(__HIP_DEVICE_COMPILE__) // the host pass only needs the launch stub; the body uses LDS address-space pointers
   static_assert(kGroups == 1 || kGroups == 2, "k groups per block");
+  static_assert(!kOneA || kNarrow, "the one-digit A form is implemented for one-digit B operands");
   constexpr int kAllWaves = kWaves * kGroups;
   constexpr int kGroupStageBytes = kGroups * kStageBytes;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -85,19 +90,32 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
   // u = q * kAllWaves + w, so each takes the same number (two thirds of its list) of the sixteen that the narrow form
   // needs.  Copy p of a wavefront is fragment q = p % kPerTile of k tile p / kPerTile of the stage.
   constexpr int kPerTile = kChunks / kAllWaves; // 6 or 3
+  // kOneA: the eight fragments f of a k tile that hold anything ([0, 4) A top digit, [4, 8) B lowest digit);
+  // wavefront w takes f = q * kAllWaves + w
+  constexpr int kOnePerTile = 2 * kSegs / kAllWaves; // 2 or 1
   const uint4_t *cur[kPerWave], *cur_last[kPerWave];
   int dest[kPerWave]; // byte offset inside a stage
 #pragma unroll
   for (int p = 0; p < kPerWave; ++p) {
-    const int sub = p / kPerTile, q = p - sub * kPerTile;
-    const int u = q * kAllWaves + wave_all;
-    int side, seg, d;
-    if (u < kSegs * kDigits)
-      side = 0, seg = u / kDigits, d = u - seg * kDigits;
-    else if (u < kSegs * kDigits + kSegs)
-      side = 1, seg = u - kSegs * kDigits, d = kDigits - 1;
-    else
-      side = 1, seg = (u - kSegs * kDigits - kSegs) / (kDigits - 1), d = (u - kSegs * kDigits - kSegs) % (kDigits - 1);
+    int sub, side, seg, d;
+    if (kOneA) {
+      sub = p / kOnePerTile;
+      const int f = (p - sub * kOnePerTile) * kAllWaves + wave_all;
+      side = f / kSegs, seg = f % kSegs, d = side ? kDigits - 1 : 0;
+      if (p >= kOnePerTile * kGroups)
+        sub = 0, side = 0, seg = 0; // unused slot
+    } else {
+      sub = p / kPerTile;
+      const int q = p - sub * kPerTile;
+      const int u = q * kAllWaves + wave_all;
+      if (u < kSegs * kDigits)
+        side = 0, seg = u / kDigits, d = u - seg * kDigits;
+      else if (u < kSegs * kDigits + kSegs)
+        side = 1, seg = u - kSegs * kDigits, d = kDigits - 1;
+      else
+        side = 1, seg = (u - kSegs * kDigits - kSegs) / (kDigits - 1),
+        d = (u - kSegs * kDigits - kSegs) % (kDigits - 1);
+    }
     dest[p] = sub * kStageBytes + ((side * kSegs + seg) * kDigits + d) * kFragBytes;
     int64_t rb = (side ? bn : bm) * kSegs + seg;
     const int64_t limit = side ? a.b_row_blocks : a.a_row_blocks;
@@ -110,11 +128,11 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
   typedef __attribute__((address_space(3))) void lds_void_t;
   // narrow: the first two thirds of each k tile's list (A fragments and lowest-digit B fragments)
   constexpr int kNeeded = (kSegs * kDigits + kSegs) / kAllWaves; // 4 or 2 per k tile
-  constexpr int kCopies = kNarrow ? kNeeded * kGroups : kPerWave;
+  constexpr int kCopies = kOneA ? kOnePerTile * kGroups : (kNarrow ? kNeeded * kGroups : kPerWave);
   auto copy_next = [&](int buf) {
 #pragma unroll
     for (int p = 0; p < kPerWave; ++p) {
-      if (kNarrow && p % kPerTile >= kNeeded)
+      if (kOneA ? p >= kOnePerTile * kGroups : (kNarrow && p % kPerTile >= kNeeded))
         continue;
       __builtin_amdgcn_global_load_lds(cur[p] + lane, (lds_void_t *)(smem + buf * kGroupStageBytes + dest[p]), 16, 0,
                                        0);
@@ -152,11 +170,18 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int d = 0; d < 3; ++d) {
-        af[i][d] = __builtin_bit_cast(i32x4_t, sa[((wm * 2 + i) * kDigits + d) * 64 + lane]);
+        if (!kOneA || d == 0)
+          af[i][d] = __builtin_bit_cast(i32x4_t, sa[((wm * 2 + i) * kDigits + d) * 64 + lane]);
         if (!kNarrow || d == 2)
           bf[i][d] = __builtin_bit_cast(i32x4_t, sb[((wn * 2 + i) * kDigits + d) * 64 + lane]);
       }
-    if (kNarrow) {
+    if (kOneA) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i][0], bf[j][2], acc[i][j][0], 0, 0, 0);
+    } else if (kNarrow) {
 #pragma unroll
       for (int t = 0; t < 3; ++t)
 #pragma unroll
@@ -187,7 +212,7 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
     int *xs = reinterpret_cast<int *>(smem);
     const int partner = wave_all ^ kWaves;
 #pragma unroll
-    for (int t = 0; t < 3; ++t) {
+    for (int t = 0; t < (kOneA ? 1 : 3); ++t) {
       __syncthreads(); // the stages (first round) or the previous round's values have been read
 #pragma unroll
       for (int i = 0; i < 2; ++i)
@@ -223,7 +248,7 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
   for (int j = 0; j < 2; ++j) {
     n_col[j] = bn * kBN + (wn * 2 + j) * 32 + col_in_frag;
     const bool in = n_col[j] < a.N;
-    sb_n[j] = in ? bshift[n_col[j]] : 0;
+    sb_n[j] = in ? plain_shift(bshift[n_col[j]]) : 0; // one-digit rows store their shift with a bias
     bias_n[j] = (in && a.bias && a.finish) ? a.bias[n_col[j]] : 0.0f;
   }
   const bool add_bias = a.bias && a.finish;
@@ -235,7 +260,7 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
   for (int i = 0; i < 2; ++i) {
     int64_t m = bm * kBM + (wm * 2 + i) * 32 + (lane & 31);
     const int64_t last = a.a_row_blocks * kFragRows - 1;
-    row_shift[i] = a.ashift[m < last ? m : last];
+    row_shift[i] = plain_shift(a.ashift[m < last ? m : last]);
   }
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
@@ -294,10 +319,23 @@ __global__ __launch_bounds__(kThreads * kGroups, kGroups == 1 ? 2 : 1) void gemm
     a.step_begin = begin;
     a.y += (int64_t)blockIdx.y * a.M * a.N;
   }
-  if (*a.bflag == 0) // uniform over the grid
-    gemm_digits_tile<true, kStages, kGroups>(a, smem);
-  else
-    gemm_digits_tile<false, kStages, kGroups>(a, smem);
+  if (*a.bflag == 0) { // uniform over the grid
+    // are all rows of this tile's A row blocks one-digit rows?  (rows past the operand clamp to its last row)
+    int64_t bm, bn;
+    band_tile<8>(blockIdx.x, a.blocks_m, a.blocks_n, bm, bn);
+    const int64_t rows = a.a_row_blocks * kFragRows;
+    bool one = true;
+    for (int r = threadIdx.x; r < kBM; r += kThreads * kGroups) {
+      const int64_t m = bm * kBM + r;
+      one = one && one_digit_row(a.ashift[m < rows ? m : rows - 1]);
+    }
+    if (__syncthreads_and(one))
+      gemm_digits_tile<true, true, kStages, kGroups>(a, smem);
+    else
+      gemm_digits_tile<true, false, kStages, kGroups>(a, smem);
+  } else {
+    gemm_digits_tile<false, false, kStages, kGroups>(a, smem);
+  }
 }
 
 // y (+)= sum over the splits of their partial results, in split order, then the bias: what the single-launch epilogue

@@ -58,6 +58,16 @@ constexpr int kDigits = 3;
 constexpr int64_t kChunkK = 16384;        // columns whose i32 accumulators are folded together (keeps them < 2^31)
 constexpr int kDigitMax = 8355711;        // 127 * 65536 + 127 * 256 + 127: the largest q three balanced digits hold
 constexpr int kBadRow = -2147483647 - 1;  // shift value marking a row with a NaN or an infinity
+// A row whose values all have zero lower digits d1 = d2 = 0 under the row's ordinary scale is a "one-digit row": this
+// is what rows of small fixed-point numbers look like (outputs of a fixed-point quantizer: multiples of one power of
+// two, at most seven bits from the unit to the largest magnitude -- the scale puts the largest magnitude into the top
+// digit and every other value is a whole number of top-digit units).  The producer marks such a row by storing its
+// shift with kOneDigitBias added (plain shifts lie in [-105, 171]); a product whose tile holds only such rows skips
+// the lower digits' fragments.  Nothing else changes -- digits, scale and row sums are the ordinary ones -- so both
+// forms of the product give the same bits.
+constexpr int kOneDigitBias = 1024;
+__host__ __device__ inline bool one_digit_row(int shift) { return shift >= kOneDigitBias / 2; }
+__host__ __device__ inline int plain_shift(int shift) { return one_digit_row(shift) ? shift - kOneDigitBias : shift; }
 
 // k tiles of both bit-weight operands are padded (with zeros) to a multiple of 8: a kernel k step is two tiles and
 // a block may split the contraction over four wavefront groups

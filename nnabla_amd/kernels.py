@@ -245,13 +245,14 @@ def binary_affine_workspace(M, K, N, like):
     return _workspace(lib().nbla_hip_binary_affine_workspace_bytes(_i64(M), _i64(K), _i64(N)), like)
 
 
-def binary_weight_affine(x, W, bias=None, quantize_zero_to=1.0, workspace=None, out=None, stream=None):
+def binary_weight_affine(x, W, bias=None, quantize_zero_to=1.0, workspace=None, out=None, stream=None, Wb=None,
+                         alpha=None):
     """x [M,K], W [K,N...] -> (y, Wb, alpha)."""
     import torch
     M, K = x.shape
     N = W.numel() // K
-    Wb = torch.empty_like(W)
-    alpha = torch.empty(N, dtype=torch.float32, device=x.device)
+    Wb = torch.empty_like(W) if Wb is None else Wb
+    alpha = torch.empty(N, dtype=torch.float32, device=x.device) if alpha is None else alpha
     y = torch.empty((M, N), dtype=torch.float32, device=x.device) if out is None else out
     ws = binary_affine_workspace(M, K, N, x) if workspace is None else workspace
     check(lib().nbla_hip_binary_weight_affine_f32(_p(x), _p(W), _p(Wb), _p(alpha), _p(bias), _p(y), _i64(M), _i64(K),

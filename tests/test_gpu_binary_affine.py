@@ -297,6 +297,80 @@ def test_affine_digits_special_rows_and_narrow_weights(dev):
     assert max_rel_err(yw, xi.astype(np.float64) @ Wp.astype(np.float64)) <= TIGHT
 
 
+def _fixed_point_rows(rng, M, K, delta=2.0 ** -4, n=8):
+    """Rows as FixedPointQuantize (sign, n bits, step delta) leaves them: integers in [-127, 127] times delta."""
+    return (rng.randint(-(2 ** (n - 1) - 1), 2 ** (n - 1), size=(M, K)) * delta).astype(np.float32)
+
+
+def test_digit_operand_of_fixed_point_rows_is_one_digit(dev):
+    """Rows whose values are multiples of one power of two and span at most seven bits land in the top digit alone
+    under the ordinary row scale (lower digits zero) and are marked as one-digit rows; the scale is the ordinary one."""
+    rng = np.random.RandomState(3)
+    M, K = 70, 1024
+    x = _fixed_point_rows(rng, M, K)
+    x[5] = rng.randn(K)                               # a general row
+    x[6] = 0.0                                        # all zero: one digit
+    x[7] = _fixed_point_rows(rng, 1, K)[0] * 2.0 ** 40   # the unit may be any power of two
+    x[8, 3] = 2.0 ** -9                               # one value 32 times finer than the rest: nine bits, not one digit
+    x[9] = np.where(rng.rand(K) < 0.5, 32.0, -0.25)   # 128 units of 2^-2: one past the edge
+    x[10] = np.where(rng.rand(K) < 0.5, 31.75, -0.25)  # 127 units of 2^-2: the edge
+    q, shift, sums, one = unpack_digits(to_np(kernels.split_digits(_dev(x, dev), M, K)), M, K, with_one_digit=True)
+    expect = np.ones(M, bool)
+    expect[[5, 8, 9]] = False
+    assert np.array_equal(one, expect), np.nonzero(one != expect)
+    assert np.array_equal(q, np.rint(np.ldexp(x.astype(np.float64), shift[:, None].astype(np.int64))).astype(np.int64))
+    assert np.abs(q[one]).max() <= 127 * 65536 and not (q[one] % 65536).any()
+    assert shift[0] == 20 and shift[7] == 20 - 40 and shift[10] == 18
+    assert np.array_equal(sums[0], q.sum(1))
+
+
+@pytest.mark.parametrize("M,K,N", [(256, 1024, 640), (1024, 512, 2048), (96, 4096, 300), (2100, 256, 1100)])
+def test_one_digit_rows_give_the_bits_of_the_three_digit_product(dev, M, K, N):
+    """A tile whose rows are all one-digit rows multiplies the lowest digit only.  The same rows inside tiles that
+    also hold a general row (so the tile takes the three-digit path) must give identical bits: both are the exact
+    integer sum, converted once.  Also against float64."""
+    rng = np.random.RandomState(M + K)
+    x = _fixed_point_rows(rng, M, K)
+    W = (rng.randn(K, N) * 0.02).astype(np.float32)
+    b = rng.randn(N).astype(np.float32)
+    y1, Wb, alpha = kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev), _dev(b, dev))
+    y1 = to_np(y1)
+    x3 = x.copy()
+    x3[::32] = rng.randn(len(x3[::32]), K)            # one general row in every 32-row block
+    y3, _, _ = kernels.binary_weight_affine(_dev(x3, dev), _dev(W, dev), _dev(b, dev))
+    y3 = to_np(y3)
+    same = np.ones(M, bool)
+    same[::32] = False
+    assert bits_equal(y1[same], y3[same]), first_mismatch(y1[same], y3[same])
+    sgn = np.where(W >= 0, 1.0, -1.0)
+    y64 = x.astype(np.float64) @ (sgn * np.abs(W.astype(np.float64)).mean(0)) + b
+    assert max_rel_err(y1, y64) <= TIGHT
+    ref_y, _, _ = oracle.binary_weight_affine(x[:64], W, b, 1.0)
+    assert max_rel_err(y1[:64], ref_y) <= TOL
+
+
+@pytest.mark.parametrize("M,K,N", [(256, 512, 384), (1024, 1024, 1024), (130, 4096, 200)])
+def test_one_digit_rows_times_one_digit_weights(dev, M, K, N):
+    """Real-weight product with fixed-point rows of x and power-of-two weights (an INQ layer behind a fixed-point
+    quantizer): a single digit product per tile.  Exact, hence equal to the float64 product rounded once, and
+    bit-identical to the rows' results inside tiles that take the three-product path."""
+    rng = np.random.RandomState(K)
+    x = _fixed_point_rows(rng, M, K)
+    e = rng.randint(-9, -3, size=(K, N))
+    W = (np.where(rng.rand(K, N) < 0.2, 0.0, 2.0 ** e) * rng.choice([-1.0, 1.0], size=(K, N))).astype(np.float32)
+    y1 = to_np(kernels.affine_digits(_dev(x, dev), _dev(W, dev)))
+    assert np.array_equal(y1, (x.astype(np.float64) @ W.astype(np.float64)).astype(np.float32))
+    x3 = x.copy()
+    x3[::128] = rng.randn(len(x3[::128]), K)          # one general row in every 128-row tile
+    y3 = to_np(kernels.affine_digits(_dev(x3, dev), _dev(W, dev)))
+    same = np.ones(M, bool)
+    same[::128] = False
+    assert bits_equal(y1[same], y3[same])
+    Wg = (rng.randn(K, N) * 0.05).astype(np.float32)  # general weights: six products, one-digit rows as three digits
+    yg = to_np(kernels.affine_digits(_dev(x, dev), _dev(Wg, dev)))
+    assert max_rel_err(yg, x.astype(np.float64) @ Wg.astype(np.float64)) <= TIGHT
+
+
 @pytest.mark.parametrize("M", [1, 8, 64])
 def test_config3_full_width_small_m_vs_oracle(dev, M):
     """Benchmark configuration 3 at K=4096, N=11008 for the M the CPU oracle finishes in seconds."""

@@ -55,9 +55,13 @@ def unpack_bits(bits_words, K, N):
     return out[:K, :N]
 
 
-def unpack_digits(raw, M, K):
+ONE_DIGIT_BIAS = 1024   # gemm_layout.hpp: a one-digit row stores its shift with this added
+
+
+def unpack_digits(raw, M, K, with_one_digit=False):
     """Digit operand bytes -> (q int64 [M, K], shift int32 [M], row sums int64 [chunks, M]) as the kernels define it:
-    fragments [row_block][k_tile][digit][lane][16 x int8], then the row sums ([chunks][rows] int64), then shifts."""
+    fragments [row_block][k_tile][digit][lane][16 x int8], then the row sums ([chunks][rows] int64), then shifts.
+    Shifts come back without the one-digit bias; with_one_digit appends the boolean mask of one-digit rows."""
     raw = np.ascontiguousarray(raw).view(np.uint8)
     rb, kt = (M + 31) // 32, ((K + 255) // 256) * 8
     rows, chunks = rb * 32, (K + 16383) // 16384
@@ -71,4 +75,11 @@ def unpack_digits(raw, M, K):
     sums = raw[nfrag:nfrag + chunks * rows * 8].view(np.int64).reshape(chunks, rows)
     shift = raw[nfrag + chunks * rows * 8:nfrag + chunks * rows * 8 + rows * 4].view(np.int32)
     assert not q[M:].any() and not q[:, K:].any()
-    return q[:M, :K], shift[:M].copy(), sums[:, :M].copy()
+    shift = shift[:M].copy()
+    one = shift >= ONE_DIGIT_BIAS // 2
+    shift[one] -= ONE_DIGIT_BIAS
+    if with_one_digit:
+        lower = d[:, :, 1:].reshape(rb, kt, 2, 2, 32, 16).any(axis=(1, 2, 3, 5)).reshape(-1)[:M]   # per row
+        assert not (lower & one).any(), "one-digit rows keep their value in the top digit"
+        return q[:M, :K], shift, sums[:, :M].copy(), one
+    return q[:M, :K], shift, sums[:, :M].copy()
