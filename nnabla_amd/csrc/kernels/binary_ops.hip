@@ -7,6 +7,31 @@
 namespace nbla_hip {
 namespace {
 
+// Rows of x holding a NaN or an infinity cannot be scaled to integers: the digit operand marks them (shift == kBadRow)
+// and the matrix-core product leaves NaN in their whole output row.  The reference's product propagates such values
+// element by element (affine.cpp:87-95: Inf * w = +-Inf, Inf - Inf = NaN, NaN anywhere = NaN), so those rows -- rare --
+// are recomputed here as plain fp32 dot products over the materialised weights Wb (* alpha).  Block b looks at rows
+// b, b + gridDim.x, ...; a launch that finds no marked row costs its launch only.
+__global__ __launch_bounds__(256) void affine_redo_marked_rows(const float *__restrict__ x, const float *__restrict__ Wb,
+                                                               const float *__restrict__ alpha,
+                                                               const float *__restrict__ bias, float *__restrict__ y,
+                                                               const int32_t *__restrict__ shift, int64_t M, int64_t K,
+                                                               int64_t N) {
+  for (int64_t m = blockIdx.x; m < M; m += gridDim.x) {
+    if (shift[m] != kBadRow) // uniform over the block
+      continue;
+    for (int64_t n = threadIdx.x; n < N; n += 256) {
+      const float a = alpha ? alpha[n] : 1.0f;
+      float acc = 0.0f;
+      for (int64_t k = 0; k < K; ++k) {
+        const float w = alpha ? Wb[k * N + n] * a : Wb[k * N + n]; // the scaled weight the reference multiplies with
+        acc = acc + x[m * K + k] * w;
+      }
+      y[m * N + n] = bias ? acc + bias[n] : acc;
+    }
+  }
+}
+
 struct AffineWorkspace {
   size_t bits_off, split_off, prep_off, count_off, gemm_off, gemm_bytes, total;
 };
@@ -76,8 +101,16 @@ int binary_affine_forward(const float *x, const float *W, float *Wb, float *alph
   rc = nbla_hip_split_digits_f32(x, K, xsplit, M, K, stream_);
   if (rc)
     return rc;
-  return nbla_hip_gemm_bits_f32(xsplit, bits, alpha, bias, y, M, K, N, 1, N, 1, base + ws.gemm_off, ws.gemm_bytes,
-                                stream_);
+  rc = nbla_hip_gemm_bits_f32(xsplit, bits, alpha, bias, y, M, K, N, 1, N, 1, base + ws.gemm_off, ws.gemm_bytes,
+                              stream_);
+  if (rc)
+    return rc;
+  const int32_t *shift = reinterpret_cast<const int32_t *>(static_cast<const char *>(xsplit) + digit_operand(M, K).shift_off);
+  const unsigned blocks = (unsigned)(M < 256 ? M : 256);
+  hipLaunchKernelGGL(affine_redo_marked_rows, dim3(blocks), dim3(256), 0, as_stream(stream_), x, Wb, alpha, bias, y,
+                     shift, M, K, N);
+  NBLA_HIP_LAUNCH_CHECK("affine_redo_marked_rows");
+  return NBLA_HIP_OK;
 }
 
 } // namespace

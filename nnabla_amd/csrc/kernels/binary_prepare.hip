@@ -39,7 +39,8 @@ PrepPlan make_prep_plan(int64_t K, int64_t N, bool transposed) {
   P.wide_groups = bits_wide_groups(N);
   P.Npw = P.wide_groups * kWideGroup;
   P.slabs = bits_packed_k_tiles(K) / 8;
-  const size_t sums_a = (size_t)P.slices * P.Np, sums_b = transposed ? 0 : (size_t)P.slabs * P.Npw;
+  // (matrices of few blocks use slabs of 128 rows: twice the partial sums)
+  const size_t sums_a = (size_t)P.slices * P.Np, sums_b = transposed ? 0 : (size_t)2 * P.slabs * P.Npw;
   P.sums_bytes = round_up((sums_a > sums_b ? sums_a : sums_b) * sizeof(float), 256);
   P.zeros_bytes = round_up((size_t)P.slices * P.col_groups * sizeof(int), 256);
   P.pairs_bytes = round_up((size_t)P.k_tiles * P.col_groups * 64 * sizeof(uint32_t), 256);
@@ -145,9 +146,9 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_kn(const float *__restric
 // the packed operand's own layout (lane l: columns F * 32 + l % 32, k slots (l / 32) * 16 + j; bit F + 8 c of word i
 // for k slot 4 i + c) and writes the k tile's 1 KiB straight into the packed operand.  No intermediate pair words and
 // no relayout pass.  Column sums: lanes in row order, then the block's four wavefronts through LDS in wavefront order.
-constexpr int kWideWaveRows = 64, kWideBatch = 4;
+constexpr int kWideBatch = 4;
 constexpr int kWideTileBatches = kTileK / kWideBatch; // batches per k tile
-template <bool kFull, bool kCountZeros>
+template <int kWideWaveRows, bool kFull, bool kCountZeros>
 __device__ __forceinline__ void binarize_wide_walk(const float *__restrict__ W, float *__restrict__ Wb,
                                                    uint4_t *__restrict__ bits_out, int64_t tile_stride, uint32_t *s_x,
                                                    int64_t K, int64_t N, int64_t k_wave, int64_t n0, int lane,
@@ -238,7 +239,8 @@ __device__ __forceinline__ void binarize_wide_walk(const float *__restrict__ W, 
   }
 }
 
-template <bool kCountZeros>
+// kWideWaveRows: 64 (two k tiles per wavefront), or 32 for matrices that would otherwise give the CUs too few blocks.
+template <int kWideWaveRows, bool kCountZeros>
 __global__ __launch_bounds__(kPrepBlock, 4) void binarize_kn_wide(const float *__restrict__ W, float *__restrict__ Wb,
                                                                  uint4_t *__restrict__ bits, float *__restrict__ sums,
                                                                  int *__restrict__ zeros, int64_t K, int64_t N,
@@ -258,10 +260,10 @@ __global__ __launch_bounds__(kPrepBlock, 4) void binarize_kn_wide(const float *_
   const int64_t tile_stride = wide_groups * 64;
   const bool full = k_wave + kWideWaveRows <= K && (wg + 1) * kWideGroup <= N;
   if (full)
-    binarize_wide_walk<true, kCountZeros>(W, Wb, tile0, tile_stride, s_x[wave], K, N, k_wave, n0, lane, zero_to, cs,
+    binarize_wide_walk<kWideWaveRows, true, kCountZeros>(W, Wb, tile0, tile_stride, s_x[wave], K, N, k_wave, n0, lane, zero_to, cs,
                                           nzero);
   else
-    binarize_wide_walk<false, kCountZeros>(W, Wb, tile0, tile_stride, s_x[wave], K, N, k_wave, n0, lane, zero_to, cs,
+    binarize_wide_walk<kWideWaveRows, false, kCountZeros>(W, Wb, tile0, tile_stride, s_x[wave], K, N, k_wave, n0, lane, zero_to, cs,
                                            nzero);
   // column sums of the block's 256 rows, wavefronts in order
   *reinterpret_cast<float4_t *>(&s_sum[wave][4 * lane]) = float4_t{cs[0], cs[1], cs[2], cs[3]};
@@ -1050,18 +1052,27 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint3
     if (N % 4 == 0 && N >= 4 && aligned16(W) && aligned16(Wb) && P.slabs <= 65535 &&
         (uint64_t)N * 4 < (1ull << 32)) { // a null Wb (no fp32 signs wanted) counts as aligned
       // writes the packed operand itself (padding k tiles included): nothing is left for the relayout below
-      const dim3 grid((unsigned)P.wide_groups, (unsigned)P.slabs);
+      // fewer than four blocks per CU with 256-row slabs: halve the slabs
+      const bool fine = P.wide_groups * P.slabs < 1024 && 2 * P.slabs <= 65535;
+      const int64_t slabs = fine ? 2 * P.slabs : P.slabs;
+      const dim3 grid((unsigned)P.wide_groups, (unsigned)slabs);
       uint4_t *packed = reinterpret_cast<uint4_t *>(bits);
-      if (zero_count)
-        hipLaunchKernelGGL(binarize_kn_wide<true>, grid, dim3(kPrepBlock), 0, stream, W, Wb, packed, sums, zeros, K, N,
-                           P.wide_groups, P.Npw, quantize_zero_to);
+#define NBLA_BINARIZE_WIDE(ROWS, COUNT)                                                                                \
+  hipLaunchKernelGGL((binarize_kn_wide<ROWS, COUNT>), grid, dim3(kPrepBlock), 0, stream, W, Wb, packed, sums, zeros, K,  \
+                     N, P.wide_groups, P.Npw, quantize_zero_to)
+      if (fine && zero_count)
+        NBLA_BINARIZE_WIDE(32, true);
+      else if (fine)
+        NBLA_BINARIZE_WIDE(32, false);
+      else if (zero_count)
+        NBLA_BINARIZE_WIDE(64, true);
       else
-        hipLaunchKernelGGL(binarize_kn_wide<false>, grid, dim3(kPrepBlock), 0, stream, W, Wb, packed, sums, zeros, K,
-                           N, P.wide_groups, P.Npw, quantize_zero_to);
+        NBLA_BINARIZE_WIDE(64, false);
+#undef NBLA_BINARIZE_WIDE
       NBLA_HIP_LAUNCH_CHECK("binarize_kn_wide");
       if (alpha || zero_count) {
         hipLaunchKernelGGL(binarize_finalize, dim3((unsigned)ceil_div(N, kPrepBlock)), dim3(kPrepBlock), 0, stream, sums,
-                           zeros, alpha, zero_count, N, P.Npw, P.slabs, P.slabs * P.wide_groups, (float)1 / K, pairs,
+                           zeros, alpha, zero_count, N, P.Npw, slabs, slabs * P.wide_groups, (float)1 / K, pairs,
                            reinterpret_cast<uint4_t *>(bits), P.k_tiles, P.col_groups, P.wide_groups, (int64_t)0);
         NBLA_HIP_LAUNCH_CHECK("binarize_finalize");
       }

@@ -135,7 +135,14 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
   constexpr int kABytes = kAFrags * kFragBytes;
   constexpr int kStepBytes = kStepChunks * kFragBytes;
   constexpr int kStageBytes = kStepBytes * kWavesK;
-  constexpr int kStages = gemm_bits_stages(BM, BN, kWavesMN, kWavesK);
+  // The LDS is sized for the three-digit stages.  One-digit stages are smaller, so more of them fit: the copies then
+  // run further ahead, which is what a block that multiplies a third as much per k step needs to stay fed (at most
+  // twelve stages, and few enough copies in flight for the 6-bit vmcnt).
+  constexpr int kStagesFull = gemm_bits_stages(BM, BN, kWavesMN, kWavesK);
+  constexpr int kLdsForStages = kStagesFull * gemm_bits_stage_bytes(BM, BN, kWavesK);
+  constexpr int kStagesFit = kLdsForStages / kStageBytes < 12 ? kLdsForStages / kStageBytes : 12;
+  constexpr int kStagesCnt = 63 / (kPerWave + 1) + 2; // (kStages - 2) * (kPerWave + 1) < 64
+  constexpr int kStages = kUsed == kDigits ? kStagesFull : (kStagesFit < kStagesCnt ? kStagesFit : kStagesCnt);
   constexpr int kDepth = kStages - 1; // k steps in flight ahead of the one being multiplied
   static_assert(kDepth >= 2 && (kDepth - 1) * (kPerWave + 1) < 64, "vmcnt is a 6-bit counter");
 

@@ -133,11 +133,43 @@ def test_digit_operand_marks_non_finite_rows(dev):
     W = np.ones((64, 64), np.float32)
     _, shift, _ = unpack_digits(to_np(kernels.split_digits(_dev(x, dev), 40, 64)), 40, 64)
     assert shift[1] == -2 ** 31 and shift[3] == -2 ** 31 and shift[0] == shift[2] == shift[4]
+    # the whole function: marked rows are recomputed element by element, as the reference's product leaves them
     y, _ = kernels.binary_connect_affine(_dev(x, dev), _dev(W, dev))      # 40 rows: the digit-operand product
     y = to_np(y)
     ok = np.ones(40, bool)
     ok[[1, 3]] = False
-    assert np.isnan(y[[1, 3]]).all() and np.array_equal(y[ok], np.full((38, 64), 64.0, np.float32))
+    assert np.isposinf(y[1]).all() and np.isnan(y[3]).all()
+    assert np.array_equal(y[ok], np.full((38, 64), 64.0, np.float32))
+    # the product alone leaves NaN in a marked row
+    _, _, bits, _ = kernels.binarize_weights(_dev(W, dev), 64, 64, want_alpha=False)
+    yp = to_np(kernels.gemm_bits(kernels.split_digits(_dev(x, dev), 40, 64), bits, None, None, 40, 64, 64))
+    assert np.isnan(yp[[1, 3]]).all() and np.array_equal(yp[ok], y[ok])
+
+
+@pytest.mark.parametrize("weight", [True, False])
+def test_many_rows_propagate_non_finite_values_per_element(dev, weight):
+    """Above sixteen rows the product runs on integer digits; rows holding Inf / NaN are recomputed in fp32 so that
+    every output element is what the reference's product gives (affine.cpp:87-95)."""
+    rng = np.random.RandomState(12)
+    M, K, N = 70, 96, 130
+    x = rng.randn(M, K).astype(np.float32)
+    x[1, 3] = np.inf
+    x[2, 7], x[2, 9] = -np.inf, np.inf
+    x[40, 60] = np.nan
+    x[69, 0] = -np.inf
+    W = rng.randn(K, N).astype(np.float32)
+    b = rng.randn(N).astype(np.float32)
+    if weight:
+        y, _, _ = kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev), _dev(b, dev))
+        ref, _, _ = oracle.binary_weight_affine(x, W, b, 1.0)
+    else:
+        y, _ = kernels.binary_connect_affine(_dev(x, dev), _dev(W, dev), _dev(b, dev))
+        ref, _ = oracle.binary_connect_affine(x, W, b, 1.0)
+    y = to_np(y)
+    assert np.array_equal(np.isnan(y), np.isnan(ref)) and np.array_equal(np.isposinf(y), np.isposinf(ref))
+    assert np.array_equal(np.isneginf(y), np.isneginf(ref))
+    fin = np.isfinite(ref)
+    assert fin.sum() >= 66 * N and np.abs(y[fin] - ref[fin]).max() <= 1e-4 * np.abs(ref[fin]).max()
 
 
 def test_few_rows_propagate_non_finite_values_per_element(dev):
