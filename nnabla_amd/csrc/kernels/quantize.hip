@@ -319,6 +319,8 @@ MinMaxPlan make_plan(const int64_t *xshape, int ndim, const int64_t *qshape) {
     want = P.tiles_per_k;
   if (want < 1)
     want = 1;
+  if (!P.L.ok)
+    want = 1; // the strided kernels fold a whole slice per block
   P.nchunks = (int)want;
   P.params_bytes = round_up((size_t)P.L.K * 16, 256);
   P.partial_bytes = round_up((size_t)P.L.K * P.nchunks * 16, 256);
@@ -619,6 +621,51 @@ __global__ __launch_bounds__(kBlock) void minmax_apply_generic(const float *__re
 }
 
 
+// Any pattern of kept and reduced axes (e.g. q shape (C, 1, W)): block k scans the slice of kept index k in the order
+// the reference's Min / Max scan it (reduced axes row-major), one element per thread and step.
+__device__ __forceinline__ int64_t strided_offset(int64_t idx, int n, const int64_t *size, const int64_t *stride) {
+  int64_t off = 0;
+  for (int d = n - 1; d >= 0; --d) {
+    const int64_t q = idx / size[d];
+    off += (idx - q * size[d]) * stride[d];
+    idx = q;
+  }
+  return off;
+}
+__global__ __launch_bounds__(kRedBlock) void minmax_reduce_strided(const float *__restrict__ x,
+                                                                   MinMaxPartial *__restrict__ partial, MinMaxAxes A,
+                                                                   int64_t R) {
+  const int64_t k = blockIdx.x;
+  const float *base = x + strided_offset(k, A.nkept, A.ksize, A.kstride);
+  Extrema ex;
+  ex.init();
+  for (int64_t r = threadIdx.x; r < R; r += kRedBlock)
+    ex.take(base[strided_offset(r, A.nred, A.rsize, A.rstride)], (uint32_t)r);
+  ex.wave_reduce();
+  __shared__ MinMaxPartial s_part[kRedBlock / 64];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0)
+    s_part[wave] = ex.pack();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kRedBlock / 64; ++w)
+      ex.merge(s_part[w].vmin, s_part[w].vmax, s_part[w].zidx, s_part[w].zsign);
+    partial[k] = ex.pack();
+  }
+}
+// Element i of x (dense, row-major) belongs to the kept index formed by its coordinates along the kept axes.
+__global__ __launch_bounds__(kBlock) void minmax_apply_strided(const float *__restrict__ x, float *__restrict__ y,
+                                                               int64_t total, MinMaxAxes A,
+                                                               const float4_t *__restrict__ params) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
+    int64_t k = 0;
+    for (int d = 0; d < A.nkept; ++d)
+      k = k * A.ksize[d] + (i / A.kstride[d]) % A.ksize[d];
+    const float4_t pr = params[k];
+    y[i] = minmax_apply(x[i], pr.x, pr.y, pr.z);
+  }
+}
+
 // The whole forward on caller-provided scratch (`workspace`: the nudged-range table, then the reduction partials).
 // Every word of the scratch that a launch reads has been written earlier in the same call, so nothing has to start
 // at zero.  `scratch_limit` != 0 marks the fixed-size scratch of the allocation-free entry point.
@@ -631,9 +678,9 @@ int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, in
       return fail(NBLA_HIP_ERR_VALUE,
                   "x.shape and ql_min.shape must be same except for i-th dimension where ql_min.shape[i] == 1.");
   const MinMaxPlan P = make_plan(xshape, ndim, qshape);
-  if (!P.L.ok)
-    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED,
-                "kept axes separated by reduced axes (e.g. q shape (C,1,W)) are not supported by the HIP kernel.");
+  MinMaxAxes axes;
+  if (!P.L.ok && !split_axes(xshape, ndim, qshape, axes))
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than eight kept or eight reduced axes of size above one.");
   if (P.L.total == 0)
     return NBLA_HIP_OK;
   if (P.L.R0 * P.L.R1 > 0xffffffffll)
@@ -654,6 +701,32 @@ int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, in
   const MinMaxLayout &L = P.L;
   const bool vec_ok = aligned16(x) && (L.R1 % 4 == 0 || L.K == 1);
   int nchunks = P.nchunks;
+
+  if (!L.ok) { // kept axes separated by reduced ones: the strided kernels
+    if (L.K > 0x7fffffffll)
+      return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than 2^31 - 1 quantization ranges.");
+    if (x_min_max) {
+      hipLaunchKernelGGL(minmax_reduce_strided, dim3((unsigned)L.K), dim3(kRedBlock), 0, stream, x, partial, axes,
+                         L.R1);
+      NBLA_HIP_LAUNCH_CHECK("min_max_quantize reduction");
+    }
+    MinMaxScalars sc;
+    sc.decay = (float)decay;
+    sc.one_minus_decay = (float)(1.0 - (double)decay);
+    sc.eps = eps;
+    sc.x_min_max = x_min_max;
+    sc.ema = ema;
+    hipLaunchKernelGGL(minmax_finalize, dim3((unsigned)L.K), dim3(64), 0, stream, partial, 1, qr_min, qr_max, ql_min,
+                       ql_max, scale, params, sc);
+    NBLA_HIP_LAUNCH_CHECK("min_max_quantize finalize");
+    int64_t blocks = (L.total + kBlock - 1) / kBlock;
+    if (blocks > 65536)
+      blocks = 65536;
+    hipLaunchKernelGGL(minmax_apply_strided, dim3((unsigned)blocks), dim3(kBlock), 0, stream, x, y, L.total, axes,
+                       params);
+    NBLA_HIP_LAUNCH_CHECK("min_max_quantize apply");
+    return NBLA_HIP_OK;
+  }
 
   if (x_min_max) {
     if (L.K == 1 && aligned16(x)) {

@@ -138,6 +138,23 @@ struct MinMaxGradOp {
   }
 };
 
+// The same mask for any pattern of kept and reduced axes: element i belongs to the kept index formed by its
+// coordinates along the kept axes.
+struct MinMaxGradStridedOp {
+  const float2 *bounds;
+  MinMaxAxes A;
+  template <bool kAccum> __device__ __forceinline__ float apply(float dy, float x, float old, size_t i) const {
+    int64_t k = 0;
+    for (int d = 0; d < A.nkept; ++d)
+      k = k * A.ksize[d] + ((int64_t)i / A.kstride[d]) % A.ksize[d];
+    const float2 b = bounds[k];
+    const float iv0 = (x >= b.x) ? 1.0f : 0.0f, iv1 = (x <= b.y) ? 1.0f : 0.0f;
+    float mask = iv0 * iv1;
+    mask = mask * dy;
+    return kAccum ? mask + old : mask;
+  }
+};
+
 // relu.cpp:41-49: dx (+)= (y > 0 ? dy : 0), y the forward output
 struct ReluGradOp {
   template <bool kAccum> __device__ __forceinline__ float apply(float dy, float y, float old, size_t) const {
@@ -200,6 +217,49 @@ __global__ __launch_bounds__(kBlock) void minmax_range_grad_partial(const float 
   }
 }
 
+// Any pattern of kept and reduced axes: block k walks the slice of kept index k, reduced axes row-major.
+__global__ __launch_bounds__(kBlock) void minmax_range_grad_strided(const float *__restrict__ dy,
+                                                                    const float *__restrict__ x,
+                                                                    const float2 *__restrict__ bounds,
+                                                                    float2 *__restrict__ partial, MinMaxAxes A,
+                                                                    int64_t R) {
+  const int64_t k = blockIdx.x;
+  const float2 b = bounds[k];
+  int64_t base = 0, idx = k;
+  for (int d = A.nkept - 1; d >= 0; --d) {
+    const int64_t q = idx / A.ksize[d];
+    base += (idx - q * A.ksize[d]) * A.kstride[d];
+    idx = q;
+  }
+  float lo = 0.0f, hi = 0.0f;
+  for (int64_t r = threadIdx.x; r < R; r += kBlock) {
+    int64_t off = base, rem = r;
+    for (int d = A.nred - 1; d >= 0; --d) {
+      const int64_t q = rem / A.rsize[d];
+      off += (rem - q * A.rsize[d]) * A.rstride[d];
+      rem = q;
+    }
+    const float xv = x[off], g = dy[off];
+    lo += ((xv < b.x) ? 1.0f : 0.0f) * g;
+    hi += ((xv > b.y) ? 1.0f : 0.0f) * g;
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    lo += __shfl_xor(lo, off);
+    hi += __shfl_xor(hi, off);
+  }
+  __shared__ float2 s_part[kBlock / 64];
+  if ((threadIdx.x & 63) == 0)
+    s_part[threadIdx.x >> 6] = float2{lo, hi};
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float2 acc = s_part[0];
+    for (int w = 1; w < kBlock / 64; ++w)
+      acc.x += s_part[w].x, acc.y += s_part[w].y;
+    partial[k] = acc;
+  }
+}
+
 __global__ __launch_bounds__(64) void minmax_range_grad_final(const float2 *__restrict__ partial, int nchunks,
                                                               float *__restrict__ g_min, float *__restrict__ g_max,
                                                               int accum_min, int accum_max, int64_t K) {
@@ -236,6 +296,8 @@ RangeGradPlan make_range_plan(const int64_t *xshape, int ndim, const int64_t *qs
     chunks = P.tiles_per_k;
   if (chunks < 1)
     chunks = 1;
+  if (!P.L.ok)
+    chunks = 1; // the strided kernel folds a whole slice per block
   P.nchunks = (int)chunks;
   P.bounds_bytes = round_up((size_t)P.L.K * sizeof(float2), 256);
   P.partial_bytes = round_up((size_t)P.L.K * P.nchunks * sizeof(float2), 256);
@@ -315,8 +377,13 @@ int nbla_hip_min_max_quantize_backward_f32(const float *dy, const float *x, floa
     if (qshape[i] != 1 && qshape[i] != xshape[i])
       return fail(NBLA_HIP_ERR_VALUE, "q tensors must have size 1 or the size of x along every axis (axis %d).", i);
   const RangeGradPlan P = make_range_plan(xshape, ndim, qshape);
-  if (!P.L.ok)
-    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "q shapes whose kept axes are separated by reduced axes are not supported.");
+  MinMaxAxes axes;
+  if (!P.L.ok && !split_axes(xshape, ndim, qshape, axes))
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than eight kept or eight reduced axes of size above one.");
+  if (!P.L.ok && P.L.K > 0x7fffffffll)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than 2^31 - 1 quantization ranges.");
+  if (P.L.total == 0)
+    return NBLA_HIP_OK;
   if (workspace_bytes < P.bounds_bytes + P.partial_bytes || !aligned256(workspace))
     return fail(NBLA_HIP_ERR_MEMORY, "min_max_quantize backward workspace too small or misaligned.");
   int rc = ensure_init();
@@ -332,7 +399,11 @@ int nbla_hip_min_max_quantize_backward_f32(const float *dy, const float *x, floa
     NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward bounds");
   }
   if (dx) {
-    if (ste_fine_grained) {
+    if (ste_fine_grained && !P.L.ok) {
+      MinMaxGradStridedOp op{bounds, axes};
+      rc = launch_grad<MinMaxGradStridedOp, true>(dy, x, dx, (size_t)P.L.total, accum_x, op, stream,
+                                                  "min_max_quantize backward");
+    } else if (ste_fine_grained) {
       MinMaxGradOp op{bounds, P.L.K, P.L.R1};
       rc = launch_grad<MinMaxGradOp, true>(dy, x, dx, (size_t)P.L.total, accum_x, op, stream, "min_max_quantize backward");
     } else {
@@ -341,7 +412,14 @@ int nbla_hip_min_max_quantize_backward_f32(const float *dy, const float *x, floa
     if (rc)
       return rc;
   }
-  if (range_grads) {
+  if (range_grads && !P.L.ok) {
+    hipLaunchKernelGGL(minmax_range_grad_strided, dim3((unsigned)P.L.K), dim3(kBlock), 0, stream, dy, x, bounds, partial,
+                       axes, P.L.R1);
+    NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward range sums");
+    hipLaunchKernelGGL(minmax_range_grad_final, dim3((unsigned)((P.L.K + 63) / 64)), dim3(64), 0, stream, partial, 1,
+                       g_qr_min, g_qr_max, accum_min, accum_max, P.L.K);
+    NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward range gradients");
+  } else if (range_grads) {
     hipLaunchKernelGGL(minmax_range_grad_partial, dim3((unsigned)P.nchunks, (unsigned)P.L.K), dim3(kBlock), 0, stream,
                        dy, x, bounds, partial, P.L.K, P.L.R1, P.tiles_per_row, P.tiles_per_k, P.nchunks);
     NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward range sums");

@@ -13,6 +13,39 @@ struct MinMaxLayout {
   bool ok;
 };
 
+// Any pattern of kept and reduced axes, for the strided kernels: the kept axes (row-major, as the q tensors are laid
+// out) and the reduced axes (row-major: the order in which Sum / Min / Max scan a slice once the reduced axes have
+// been moved to the back, sum.cpp:44-75) with their element strides in x.
+struct MinMaxAxes {
+  int nkept, nred;
+  int64_t ksize[8], kstride[8], rsize[8], rstride[8];
+};
+inline bool split_axes(const int64_t *xshape, int ndim, const int64_t *qshape, MinMaxAxes &A) {
+  A.nkept = A.nred = 0;
+  int64_t stride = 1;
+  int64_t strides[32];
+  if (ndim > 32)
+    return false;
+  for (int i = ndim - 1; i >= 0; --i) {
+    strides[i] = stride;
+    stride *= xshape[i];
+  }
+  for (int i = 0; i < ndim; ++i) {
+    if (xshape[i] == 1)
+      continue;
+    if (qshape[i] != 1) {
+      if (A.nkept == 8)
+        return false;
+      A.ksize[A.nkept] = xshape[i], A.kstride[A.nkept++] = strides[i];
+    } else {
+      if (A.nred == 8)
+        return false;
+      A.rsize[A.nred] = xshape[i], A.rstride[A.nred++] = strides[i];
+    }
+  }
+  return true;
+}
+
 inline MinMaxLayout collapse(const int64_t *xshape, int ndim, const int64_t *qshape) {
   // runs of (kept?) axes, ignoring size-1 axes
   int64_t sizes[3] = {1, 1, 1};
@@ -27,10 +60,8 @@ inline MinMaxLayout collapse(const int64_t *xshape, int ndim, const int64_t *qsh
     if (kept) {
       if (stage == 0)
         stage = 1;
-      else if (stage == 2) {
+      else if (stage == 2)
         L.ok = false; // kept, reduced, kept: not a single (R0, K, R1) pattern
-        continue;
-      }
       sizes[1] *= s;
     } else {
       if (stage == 1)
@@ -41,6 +72,10 @@ inline MinMaxLayout collapse(const int64_t *xshape, int ndim, const int64_t *qsh
   L.R0 = sizes[0];
   L.K = sizes[1];
   L.R1 = sizes[2];
+  if (!L.ok) { // general pattern (strided kernels): K kept indices, each with R1 reduced elements
+    L.R1 = L.R0 * L.R1;
+    L.R0 = 1;
+  }
   if (L.K == 1) { // per-tensor: one flat run
     L.R1 = L.R0 * L.R1;
     L.R0 = 1;

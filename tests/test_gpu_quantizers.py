@@ -224,6 +224,9 @@ MMQ_SHAPES = [
     ((4, 8, 16, 16), (1, 1, 1, 1)), ((4, 8, 16, 16), (1, 8, 1, 1)), ((16, 8, 4, 4), (16, 1, 1, 1)),
     ((6, 10), (1, 10)), ((6, 10), (6, 1)), ((3, 5, 7), (1, 5, 1)), ((2, 3, 4), (2, 3, 4)), ((5, 7, 9), (1, 1, 1)),
     ((2, 64, 33, 32), (1, 64, 1, 1)), ((1, 1, 3000), (1, 1, 1)),
+    # kept axes separated by reduced ones (the reference moves the reduced axes to the back, sum.cpp:44-75)
+    ((5, 7, 9), (5, 1, 9)), ((3, 4, 5, 6), (1, 4, 1, 6)), ((3, 4, 5, 6), (3, 1, 5, 1)), ((2, 3, 1, 4, 5), (2, 1, 1, 4, 1)),
+    ((6, 300, 7), (6, 1, 7)),
 ]
 
 
@@ -235,6 +238,21 @@ def test_min_max_quantize_matches_oracle(dev, xshape, qshape, x_min_max, ema):
     got, ref = _mmq_both(dev, x, qshape, -6.0, 6.0, 0.0, 255.0, 0.999, x_min_max, ema)
     for g, r, name in zip(got, ref, ("y", "qr_min", "qr_max", "scale")):
         assert bits_equal(g, r), "%s: %s" % (name, first_mismatch(g, r))
+
+
+def test_min_max_quantize_general_axes_first_zero_wins(dev):
+    """q shape (C, 1, W): the slice of (c, w) is scanned along the reduced axis in order, and of several zeros the
+    first one's sign is the extremum's (min.cpp:29-41 / max.cpp:48-60 keep the first of equals)."""
+    x = np.full((3, 6, 4), 0.0, np.float32)
+    x[0, :, 0] = [0.0, -0.0, 0.0, -0.0, 0.0, 0.0]      # max and min are zeros: first is +0
+    x[1, :, 2] = [-0.0, 0.0, 0.0, 0.0, 0.0, 0.0]       # first is -0
+    x[2, :, 1] = [-1.0, -0.0, 0.0, -3.0, -0.0, -2.0]   # max is a zero: the first zero is -0; min is -3
+    x[2, :, 3] = [5.0, 0.0, -0.0, 2.0, 0.0, 1.0]       # min is a zero: the first zero is +0
+    got, ref = _mmq_both(dev, x, (3, 1, 4), -6.0, 6.0, 0.0, 255.0, 0.999, True, False)
+    for g, r, name in zip(got, ref, ("y", "qr_min", "qr_max", "scale")):
+        assert bits_equal(g, r), "%s: %s" % (name, first_mismatch(g, r))
+    # (qr_max of an all-zero slice is moved to qr_min + eps, so the sign is looked at on qr_min)
+    assert np.signbit(got[1][1, 0, 2]) and not np.signbit(got[1][0, 0, 0])
 
 
 def test_min_max_quantize_signed_zero_and_limits(dev):

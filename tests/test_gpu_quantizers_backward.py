@@ -75,7 +75,9 @@ def test_pow2_backward_all_binade_cuts(dev):
 
 @pytest.mark.parametrize("xshape,qshape", [((4, 6, 5, 3), (1, 1, 1, 1)), ((4, 6, 5, 3), (1, 6, 1, 1)),
                                            ((4, 6, 5, 3), (4, 1, 1, 1)), ((16, 8, 32, 32), (1, 8, 1, 1)),
-                                           ((2, 3, 7), (1, 1, 1)), ((64, 1000), (1, 1000))])
+                                           ((2, 3, 7), (1, 1, 1)), ((64, 1000), (1, 1000)),
+                                           ((5, 7, 9), (5, 1, 9)), ((3, 4, 5, 6), (1, 4, 1, 6)),
+                                           ((6, 300, 7), (6, 1, 7)), ((2, 3, 1, 4, 5), (2, 1, 1, 4, 1))])
 @pytest.mark.parametrize("fine", [True, False])
 def test_min_max_backward(dev, xshape, qshape, fine):
     x, dy = _rand(xshape, 11, 3.0), _rand(xshape, 12)
