@@ -10,9 +10,7 @@
 #include "conv_geom.hpp"
 #include "gemm_layout.hpp"
 #include "internal.hpp"
-
-#include <cstring> // rocprim's texture iterator calls memset without including it
-#include <rocprim/rocprim.hpp>
+#include "radix_select.hpp"
 
 #include <cmath>
 #include <vector>
@@ -29,19 +27,29 @@ struct InqParams {
   int pad;
 };
 
-struct InqWorkspace {
-  size_t params_off, partial_off, keys_in_off, keys_out_off, vals_in_off, vals_out_off, scan_off, temp_off, temp_bytes,
-      draws_off, total;
+// Both selections rank weights in index order inside chunks of whole tiles: one block per chunk, the number of
+// ranked weights per chunk in `counts`, turned into each chunk's starting rank by a one-block scan.
+constexpr int kSelTile = kBlk * 4;   // weights per block and step: four consecutive ones per thread
+constexpr int kMaxChunks = 2048;
+struct ChunkPlan {
+  int nchunks;
+  int64_t chunk; // weights per chunk, a multiple of kSelTile
 };
-
-size_t rocprim_temp_bytes(int64_t size) {
-  size_t sort_bytes = 0, scan_bytes = 0;
-  uint32_t *k = nullptr;
-  int *f = nullptr;
-  (void)rocprim::radix_sort_pairs_desc(nullptr, sort_bytes, k, k, k, k, (size_t)size, 0, 32, (hipStream_t)0);
-  (void)rocprim::inclusive_scan(nullptr, scan_bytes, f, f, (size_t)size, rocprim::plus<int>(), (hipStream_t)0);
-  return sort_bytes > scan_bytes ? sort_bytes : scan_bytes;
+ChunkPlan plan_chunks(int64_t size) {
+  ChunkPlan c;
+  int64_t n = ceil_div(size, kSelTile);
+  if (n > kMaxChunks)
+    n = kMaxChunks;
+  if (n < 1)
+    n = 1;
+  c.chunk = ceil_div(ceil_div(size, n), kSelTile) * kSelTile;
+  c.nchunks = (int)ceil_div(size, c.chunk);
+  return c;
 }
+
+struct InqWorkspace {
+  size_t params_off, partial_off, state_off, counts_off, draws_off, total;
+};
 
 InqWorkspace plan_inq(int64_t size, int selection) {
   InqWorkspace w;
@@ -50,22 +58,12 @@ InqWorkspace plan_inq(int64_t size, int selection) {
   off += 256;
   w.partial_off = off;
   off += round_up(kMaxPartials * sizeof(uint32_t), 256);
-  const size_t arr = round_up((size_t)size * 4, 256);
-  w.keys_in_off = w.keys_out_off = w.vals_in_off = w.vals_out_off = w.scan_off = w.temp_off = w.draws_off = off;
-  w.temp_bytes = 0;
-  if (selection == 1) { // largest_abs: sort pairs + scan
-    w.keys_in_off = off, off += arr;
-    w.keys_out_off = off, off += arr;
-    w.vals_in_off = off, off += arr;
-    w.vals_out_off = off, off += arr;
-    w.scan_off = off, off += arr;
-    w.temp_bytes = round_up(rocprim_temp_bytes(size), 256);
-    w.temp_off = off, off += w.temp_bytes;
-  } else if (selection == 2) { // random: scan + uploaded draws
-    w.keys_in_off = off, off += arr; // learnable flags
-    w.scan_off = off, off += arr;
-    w.temp_bytes = round_up(rocprim_temp_bytes(size), 256);
-    w.temp_off = off, off += w.temp_bytes;
+  w.state_off = w.counts_off = w.draws_off = off;
+  if (selection == 1) { // largest_abs: radix select, then the ties in index order
+    w.state_off = off, off += round_up(sizeof(SelectState), 256);
+    w.counts_off = off, off += round_up((kMaxChunks + 1) * sizeof(uint32_t), 256);
+  } else if (selection == 2) { // random: ranks of the learnable weights + uploaded draws
+    w.counts_off = off, off += round_up((kMaxChunks + 1) * sizeof(uint32_t), 256);
     w.draws_off = off, off += round_up((size_t)size, 256);
   }
   w.total = off;
@@ -323,43 +321,217 @@ __global__ __launch_bounds__(kBlk) void inq_quantize_columns(float *__restrict__
 }
 
 // ---- selection: "largest_abs" (:117-141)
-__global__ __launch_bounds__(kBlk) void sel_keys(const float *__restrict__ W, uint32_t *__restrict__ keys,
-                                                 uint32_t *__restrict__ vals, int64_t size) {
-  for (int64_t i = (int64_t)blockIdx.x * kBlk + threadIdx.x; i < size; i += (int64_t)gridDim.x * kBlk) {
-    keys[i] = __float_as_uint(W[i]) & 0x7fffffffu;
-    vals[i] = (uint32_t)i;
+// The reference sorts all indices by falling |w| and then fixes learnable weights in that order until T =
+// num_learnable / 2 of them are fixed: the T learnable weights of largest magnitude.  Here: a radix select over the
+// learnable weights finds the T-th largest magnitude t (keys are the complemented magnitude bits, so "largest" is
+// "smallest key"; a NaN orders above every number, as its bits do) and how many of the weights of magnitude exactly t
+// belong to the T; those are taken in index order (the order a stable sort gives; the reference's std::sort leaves
+// the order of equal magnitudes to the library).  When T == 0 the reference's loop still runs once: it fixes the
+// first index of the sorted order, whatever its magnitude rank among learnable weights, if that one is learnable.
+__device__ __forceinline__ uint32_t inq_key(float w) { return 0x7fffffffu - (__float_as_uint(w) & 0x7fffffffu); }
+
+__global__ __launch_bounds__(kHistBlock) void inq_select_histogram(const float *__restrict__ W,
+                                                                   const int *__restrict__ I, int64_t n4, int64_t n,
+                                                                   SelectState *__restrict__ st, int pass) {
+  typedef float f4_t __attribute__((ext_vector_type(4)));
+  typedef int i4_t __attribute__((ext_vector_type(4)));
+  __shared__ uint32_t h[kMaxBins * kLdsCopies];
+  __shared__ uint32_t scratch[kHistBlock / 64 + 1];
+  const SelectPass sp = select_begin(h, st, pass);
+  // pass 0 also finds the first index of the sorted order: the largest magnitude of all weights, lowest index first
+  unsigned long long top = 0ull;
+  auto count = [&](float w, int ind, int64_t i) {
+    const uint32_t key = inq_key(w);
+    if (ind == 0)
+      select_count(h, sp, key);
+    if (pass == 0) {
+      const unsigned long long cand =
+          ((unsigned long long)(0x7fffffffu - key) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)i);
+      top = cand > top ? cand : top;
+    }
+  };
+  const int64_t tiles = (n4 + kHistBlock * 2 - 1) / (kHistBlock * 2);
+  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    const int64_t base = tile * (kHistBlock * 2) + threadIdx.x;
+    f4_t v[2];
+    i4_t f[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      if (base + j * kHistBlock < n4) {
+        v[j] = reinterpret_cast<const f4_t *>(W)[base + j * kHistBlock];
+        f[j] = reinterpret_cast<const i4_t *>(I)[base + j * kHistBlock];
+      }
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      if (base + j * kHistBlock < n4) {
+        const int64_t i = 4 * (base + j * kHistBlock);
+        count(v[j].x, f[j].x, i), count(v[j].y, f[j].y, i + 1), count(v[j].z, f[j].z, i + 2),
+            count(v[j].w, f[j].w, i + 3);
+      }
+  }
+  // what the 16-byte accesses leave: up to three weights, or all of them when the arrays are not aligned
+  for (int64_t i = 4 * n4 + (int64_t)blockIdx.x * kHistBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kHistBlock)
+    count(W[i], I[i], i);
+  if (pass == 0) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      const unsigned long long o = __shfl_xor(top, off);
+      top = o > top ? o : top;
+    }
+    if ((threadIdx.x & 63) == 0 && top != 0ull)
+      atomicMax(&st->top, top);
+    select_finish<true>(h, scratch, st, sp);
+  } else {
+    select_finish<false>(h, scratch, st, sp);
   }
 }
-__global__ __launch_bounds__(kBlk) void sel_flags_sorted(const int *__restrict__ I, const uint32_t *__restrict__ order,
-                                                         int *__restrict__ flags, int64_t size) {
-  for (int64_t j = (int64_t)blockIdx.x * kBlk + threadIdx.x; j < size; j += (int64_t)gridDim.x * kBlk)
-    flags[j] = (I[order[j]] == 0) ? 1 : 0;
+
+// What a selection ranks: kTies -- the learnable weights of the selected magnitude; otherwise every learnable weight.
+template <bool kTies>
+__device__ __forceinline__ uint32_t sel_ranked(const float *__restrict__ W, const int *__restrict__ I, int64_t i,
+                                               int64_t size, uint32_t key) {
+  if (i >= size || I[i] != 0)
+    return 0u;
+  return kTies ? (inq_key(W[i]) == key ? 1u : 0u) : 1u;
 }
-// Walks the reference's loop in closed form: with c[j] the number of learnable weights among the first j+1 of the
-// sorted order and T = num_learnable / 2, position j is fixed iff it is learnable and c[j] <= T; when T == 0 the
-// loop stops after its first iteration, which fixes position 0 if it is learnable.
-__global__ __launch_bounds__(kBlk) void sel_mark_sorted(int *__restrict__ I, const uint32_t *__restrict__ order,
-                                                        const int *__restrict__ c, int64_t size) {
-  const int T = c[size - 1] / 2;
-  for (int64_t j = (int64_t)blockIdx.x * kBlk + threadIdx.x; j < size; j += (int64_t)gridDim.x * kBlk) {
-    const int before = j ? c[j - 1] : 0;
-    const bool learnable = c[j] != before;
-    if (learnable && ((T >= 1 && c[j] <= T) || (T == 0 && j == 0)))
-      I[order[j]] = 1;
+
+template <bool kTies>
+__global__ __launch_bounds__(kBlk) void sel_count_chunks(const float *__restrict__ W, const int *__restrict__ I,
+                                                         int64_t size, int64_t chunk,
+                                                         const SelectState *__restrict__ st,
+                                                         uint32_t *__restrict__ counts) {
+  uint32_t key = 0u;
+  if (kTies) {
+    if (st->rank[kPasses] == kNoRank) { // nothing to rank
+      if (threadIdx.x == 0)
+        counts[blockIdx.x] = 0u;
+      return;
+    }
+    key = st->prefix[kPasses];
+  }
+  const int64_t begin = (int64_t)blockIdx.x * chunk;
+  uint32_t c = 0u;
+  for (int64_t t = begin; t < begin + chunk && t < size; t += kSelTile)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      c += sel_ranked<kTies>(W, I, t + j * kBlk + threadIdx.x, size, key);
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1)
+    c += __shfl_xor(c, off);
+  __shared__ uint32_t s_part[kBlk / 64];
+  if ((threadIdx.x & 63) == 0)
+    s_part[threadIdx.x >> 6] = c;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kBlk / 64; ++w)
+      c += s_part[w];
+    counts[blockIdx.x] = c;
   }
 }
-// ---- selection: "random" (:143-149)
-__global__ __launch_bounds__(kBlk) void sel_flags(const int *__restrict__ I, int *__restrict__ flags, int64_t size) {
-  for (int64_t i = (int64_t)blockIdx.x * kBlk + threadIdx.x; i < size; i += (int64_t)gridDim.x * kBlk)
-    flags[i] = (I[i] == 0) ? 1 : 0;
-}
-__global__ __launch_bounds__(kBlk) void sel_apply_draws(int *__restrict__ I, const int *__restrict__ c,
-                                                        const uint8_t *__restrict__ draws, int64_t size) {
-  for (int64_t i = (int64_t)blockIdx.x * kBlk + threadIdx.x; i < size; i += (int64_t)gridDim.x * kBlk) {
-    const int before = i ? c[i - 1] : 0;
-    if (c[i] != before) // learnable: its rank among the learnable weights is `before`
-      I[i] = draws[before];
+
+// counts[0 .. n) -> exclusive prefix sums in place, the total in counts[n]
+__global__ __launch_bounds__(kBlk) void sel_scan_counts(uint32_t *__restrict__ counts, int n) {
+  __shared__ uint32_t s_wave[kBlk / 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint32_t carry = 0u;
+  for (int base = 0; base < n; base += kBlk) {
+    const int i = base + threadIdx.x;
+    const uint32_t v = i < n ? counts[i] : 0u;
+    uint32_t incl = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const uint32_t up = __shfl_up(incl, off);
+      if (lane >= off)
+        incl += up;
+    }
+    __syncthreads(); // the previous step's s_wave has been read
+    if (lane == 63)
+      s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t before = carry, total = 0u;
+    for (int w = 0; w < kBlk / 64; ++w) {
+      before += w < wave ? s_wave[w] : 0u;
+      total += s_wave[w];
+    }
+    if (i < n)
+      counts[i] = before + incl - v;
+    carry += total;
   }
+  if (threadIdx.x == 0)
+    counts[n] = carry;
+}
+
+// Walks a chunk in index order handing every ranked weight its rank (its number among all ranked weights before it);
+// thread t of a step owns the four consecutive weights 4 t .. 4 t + 3 of the step's tile.
+template <bool kTies, class Apply>
+__device__ __forceinline__ void sel_walk_ranks(const float *__restrict__ W, const int *__restrict__ I, int64_t size,
+                                               int64_t chunk, uint32_t key, uint32_t start, Apply apply) {
+  __shared__ uint32_t s_wave[kBlk / 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t begin = (int64_t)blockIdx.x * chunk;
+  uint32_t carry = start;
+  for (int64_t t = begin; t < begin + chunk && t < size; t += kSelTile) {
+    const int64_t i0 = t + 4 * threadIdx.x;
+    uint32_t f[4], mine = 0u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f[j] = sel_ranked<kTies>(W, I, i0 + j, size, key);
+      mine += f[j];
+    }
+    uint32_t incl = mine;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const uint32_t up = __shfl_up(incl, off);
+      if (lane >= off)
+        incl += up;
+    }
+    __syncthreads();
+    if (lane == 63)
+      s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t before = carry, total = 0u;
+    for (int w = 0; w < kBlk / 64; ++w) {
+      before += w < wave ? s_wave[w] : 0u;
+      total += s_wave[w];
+    }
+    uint32_t r = before + incl - mine;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      apply(i0 + j, f[j] != 0u, r);
+      r += f[j];
+    }
+    carry += total;
+  }
+}
+
+__global__ __launch_bounds__(kBlk) void sel_mark_largest(const float *__restrict__ W, int *__restrict__ I, int64_t size,
+                                                         int64_t chunk, const SelectState *__restrict__ st,
+                                                         const uint32_t *__restrict__ starts) {
+  const uint32_t key = st->prefix[kPasses], last = st->rank[kPasses];
+  if (last == kNoRank) { // T == 0: only the first index of the sorted order is looked at
+    if (blockIdx.x == 0 && threadIdx.x == 0 && st->top != 0ull) {
+      const uint32_t i = 0xffffffffu - (uint32_t)st->top;
+      if (I[i] == 0)
+        I[i] = 1;
+    }
+    return;
+  }
+  sel_walk_ranks<true>(W, I, size, chunk, key, starts[blockIdx.x], [&](int64_t i, bool tie, uint32_t r) {
+    if (i >= size || I[i] != 0)
+      return;
+    if (inq_key(W[i]) < key || (tie && r <= last))
+      I[i] = 1;
+  });
+}
+
+// ---- selection: "random" (:143-149): learnable weight number r (in index order) takes draw r
+__global__ __launch_bounds__(kBlk) void sel_apply_draws(int *__restrict__ I, int64_t size, int64_t chunk,
+                                                        const uint32_t *__restrict__ starts,
+                                                        const uint8_t *__restrict__ draws) {
+  sel_walk_ranks<false>(nullptr, I, size, chunk, 0u, starts[blockIdx.x], [&](int64_t i, bool learnable, uint32_t r) {
+    if (learnable)
+      I[i] = draws[r];
+  });
 }
 
 unsigned grid_for(int64_t size) {
@@ -399,44 +571,41 @@ int update_weights(float *W, int *I, float *old_W, int *old_I, int64_t size, int
                      (aligned16(W) && aligned16(old_W) && aligned16(old_I)) ? 1 : 0, partial);
   NBLA_HIP_LAUNCH_CHECK("inq_restore_absmax");
 
+  const ChunkPlan cp = plan_chunks(size);
+  uint32_t *counts = reinterpret_cast<uint32_t *>(base + ws.counts_off);
   if (selection == 1) {
-    uint32_t *keys_in = reinterpret_cast<uint32_t *>(base + ws.keys_in_off);
-    uint32_t *keys_out = reinterpret_cast<uint32_t *>(base + ws.keys_out_off);
-    uint32_t *vals_in = reinterpret_cast<uint32_t *>(base + ws.vals_in_off);
-    uint32_t *vals_out = reinterpret_cast<uint32_t *>(base + ws.vals_out_off);
-    int *scan = reinterpret_cast<int *>(base + ws.scan_off);
-    int *flags = reinterpret_cast<int *>(keys_in); // keys_in is free once the sort has run
-    size_t temp_bytes = ws.temp_bytes;
-    hipLaunchKernelGGL(sel_keys, dim3(grid_for(size)), dim3(kBlk), 0, stream, W, keys_in, vals_in, size);
-    NBLA_HIP_LAUNCH_CHECK("inq selection keys");
-    hipError_t e = rocprim::radix_sort_pairs_desc(base + ws.temp_off, temp_bytes, keys_in, keys_out, vals_in, vals_out,
-                                                  (size_t)size, 0, 32, stream);
-    if (e != hipSuccess)
-      return fail_hip(e, "rocprim::radix_sort_pairs_desc");
-    hipLaunchKernelGGL(sel_flags_sorted, dim3(grid_for(size)), dim3(kBlk), 0, stream, I, vals_out, flags, size);
-    NBLA_HIP_LAUNCH_CHECK("inq selection flags");
-    temp_bytes = ws.temp_bytes;
-    e = rocprim::inclusive_scan(base + ws.temp_off, temp_bytes, flags, scan, (size_t)size, rocprim::plus<int>(),
-                                stream);
-    if (e != hipSuccess)
-      return fail_hip(e, "rocprim::inclusive_scan");
-    hipLaunchKernelGGL(sel_mark_sorted, dim3(grid_for(size)), dim3(kBlk), 0, stream, I, vals_out, scan, size);
+    SelectState *st = reinterpret_cast<SelectState *>(base + ws.state_off);
+    const bool vec = aligned16(W) && aligned16(I);
+    const int64_t n4 = vec ? size / 4 : 0;
+    int64_t blocks = vec ? ceil_div(n4 ? n4 : 1, (int64_t)kHistBlock * 2) : ceil_div(size, (int64_t)kHistBlock);
+    if (blocks > kSelectBlocks)
+      blocks = kSelectBlocks;
+    hipLaunchKernelGGL(clear_select, dim3(clear_select_blocks()), dim3(256), 0, stream, st, kNoRank);
+    NBLA_HIP_LAUNCH_CHECK("inq selection clear");
+    for (int p = 0; p < kPasses; ++p) {
+      hipLaunchKernelGGL(inq_select_histogram, dim3((unsigned)blocks), dim3(kHistBlock), 0, stream, W, I, n4, size, st,
+                         p);
+      NBLA_HIP_LAUNCH_CHECK("inq selection histogram");
+    }
+    hipLaunchKernelGGL(sel_count_chunks<true>, dim3((unsigned)cp.nchunks), dim3(kBlk), 0, stream, W, I, size, cp.chunk,
+                       st, counts);
+    NBLA_HIP_LAUNCH_CHECK("inq selection tie counts");
+    hipLaunchKernelGGL(sel_scan_counts, dim3(1), dim3(kBlk), 0, stream, counts, cp.nchunks);
+    NBLA_HIP_LAUNCH_CHECK("inq selection scan");
+    hipLaunchKernelGGL(sel_mark_largest, dim3((unsigned)cp.nchunks), dim3(kBlk), 0, stream, W, I, size, cp.chunk, st,
+                       counts);
     NBLA_HIP_LAUNCH_CHECK("inq selection mark");
   } else if (selection == 2) {
-    int *flags = reinterpret_cast<int *>(base + ws.keys_in_off);
-    int *scan = reinterpret_cast<int *>(base + ws.scan_off);
     uint8_t *draws = reinterpret_cast<uint8_t *>(base + ws.draws_off);
-    size_t temp_bytes = ws.temp_bytes;
-    hipLaunchKernelGGL(sel_flags, dim3(grid_for(size)), dim3(kBlk), 0, stream, I, flags, size);
-    NBLA_HIP_LAUNCH_CHECK("inq selection flags");
-    hipError_t e = rocprim::inclusive_scan(base + ws.temp_off, temp_bytes, flags, scan, (size_t)size,
-                                           rocprim::plus<int>(), stream);
-    if (e != hipSuccess)
-      return fail_hip(e, "rocprim::inclusive_scan");
+    hipLaunchKernelGGL(sel_count_chunks<false>, dim3((unsigned)cp.nchunks), dim3(kBlk), 0, stream, nullptr, I, size,
+                       cp.chunk, nullptr, counts);
+    NBLA_HIP_LAUNCH_CHECK("inq selection counts");
+    hipLaunchKernelGGL(sel_scan_counts, dim3(1), dim3(kBlk), 0, stream, counts, cp.nchunks);
+    NBLA_HIP_LAUNCH_CHECK("inq selection scan");
     // The generator lives on the host (as the reference's std::mt19937 does) and advances by exactly one draw per
     // learnable weight, so their number has to come back first.
     int learnable = 0;
-    e = hipMemcpyAsync(&learnable, scan + (size - 1), sizeof(int), hipMemcpyDeviceToHost, stream);
+    hipError_t e = hipMemcpyAsync(&learnable, counts + cp.nchunks, sizeof(int), hipMemcpyDeviceToHost, stream);
     if (e == hipSuccess)
       e = hipStreamSynchronize(stream);
     if (e != hipSuccess)
@@ -449,7 +618,8 @@ int update_weights(float *W, int *I, float *old_W, int *old_I, int64_t size, int
         e = hipStreamSynchronize(stream); // `host` goes out of scope below
       if (e != hipSuccess)
         return fail_hip(e, "uploading the Bernoulli draws");
-      hipLaunchKernelGGL(sel_apply_draws, dim3(grid_for(size)), dim3(kBlk), 0, stream, I, scan, draws, size);
+      hipLaunchKernelGGL(sel_apply_draws, dim3((unsigned)cp.nchunks), dim3(kBlk), 0, stream, I, size, cp.chunk, counts,
+                         draws);
       NBLA_HIP_LAUNCH_CHECK("inq selection apply");
     }
   }

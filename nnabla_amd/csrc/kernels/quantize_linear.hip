@@ -4,6 +4,7 @@
 #include "common.hpp"
 #include "gemm_layout.hpp"
 #include "quantize_common.hpp"
+#include "radix_select.hpp"
 
 #include <cmath>
 
@@ -346,55 +347,13 @@ int quantize_range(int dtype, int narrow_range, float &lo, float &hi) {
 
 // ------------------------------------------------------------------------------------------------------ Prune
 
-// Radix select of the rank-th smallest magnitude: three passes over the 31 magnitude bits (11, 10, 10), each
-// histogramming the digit of the elements that share the digits chosen so far.  A block counts in LDS (four copies
-// of the counters, copy = lane % 4), adds its non-zero counters to one of four global copies (a counter that every
-// block of the grid updates is a serial chain of device-wide atomics, 15 ns each: the dominant cost with a single
-// copy) and takes a ticket; the block holding the last ticket scans the finished histogram and records the chosen
-// digit and the rank left inside it for the next pass.
-constexpr int kPasses = 3, kMaxBins = 2048, kLdsCopies = 4, kGlobalCopies = 4;
-constexpr int kSelectBlocks = 256;
-// 256 histogram blocks of 1024 threads: one per CU; the block that finishes a pass scans the bins with all its
-// threads, and fewer blocks mean fewer counter updates (measured against 512 x 256, 512 x 512, 1024 x 512, 512 x 1024)
-constexpr int kHistBlock = 1024;
-struct SelectState {
-  uint32_t hist[kPasses][kGlobalCopies][kMaxBins];
-  uint32_t done[kPasses];       // blocks of pass p that have added their counters
-  uint32_t prefix[kPasses + 1]; // magnitude bits chosen before pass p (entry kPasses: the selected magnitude)
-  uint32_t rank[kPasses + 1];   // rank among the elements that share them
-};
-__device__ __forceinline__ int pass_shift(int p) { return p == 0 ? 20 : (p == 1 ? 10 : 0); }
-__device__ __forceinline__ int pass_bits(int p) { return p == 0 ? 11 : 10; }
-
-__global__ __launch_bounds__(kBlock) void clear_select(SelectState *st, uint32_t rank0) {
-  uint32_t *h = &st->hist[0][0][0];
-  const int i = blockIdx.x * kBlock + threadIdx.x;
-  if (i < kPasses * kGlobalCopies * kMaxBins)
-    h[i] = 0u;
-  if (i < kPasses)
-    st->done[i] = 0u;
-  if (i == 0) {
-    st->prefix[0] = 0u;
-    st->rank[0] = rank0;
-  }
-}
-
+// The rank-th smallest magnitude by the radix select of radix_select.hpp: keys are the 31 magnitude bits of x.
 __global__ __launch_bounds__(kHistBlock) void prune_histogram(const float *__restrict__ x, int64_t n4, int64_t n,
                                                           SelectState *__restrict__ st, int pass) {
   __shared__ uint32_t h[kMaxBins * kLdsCopies];
   __shared__ uint32_t scratch[kHistBlock / 64 + 1];
-  for (int i = threadIdx.x; i < kMaxBins * kLdsCopies; i += kHistBlock)
-    h[i] = 0u;
-  const uint32_t prefix = st->prefix[pass], rank = st->rank[pass];
-  __syncthreads();
-  const int shift = pass_shift(pass), above = shift + pass_bits(pass), bins = 1 << pass_bits(pass);
-  const uint32_t mask = (uint32_t)bins - 1u, want = prefix >> above;
-  const int copy = threadIdx.x & (kLdsCopies - 1);
-  auto count = [&](float v) {
-    const uint32_t key = __float_as_uint(v) & 0x7fffffffu;
-    if (pass == 0 || (key >> above) == want)
-      atomicAdd(&h[((key >> shift) & mask) * kLdsCopies + copy], 1u);
-  };
+  const SelectPass sp = select_begin(h, st, pass);
+  auto count = [&](float v) { select_count(h, sp, __float_as_uint(v) & 0x7fffffffu); };
   // four loads in flight per thread before the counters are touched
   const int64_t tiles = (n4 + kHistBlock * 4 - 1) / (kHistBlock * 4);
   for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
@@ -414,74 +373,7 @@ __global__ __launch_bounds__(kHistBlock) void prune_histogram(const float *__res
     if (i < n)
       count(x[i]);
   }
-  __syncthreads();
-  uint32_t *g = st->hist[pass][blockIdx.x % kGlobalCopies];
-  for (int b = threadIdx.x; b < bins; b += kHistBlock) {
-    const uint4_t c = *reinterpret_cast<const uint4_t *>(&h[b * kLdsCopies]);
-    const uint32_t total = c.x + c.y + c.z + c.w;
-    if (total)
-      atomicAdd(&g[b], total);
-  }
-  // The ticket must follow this block's counter updates.  A workgroup barrier alone does not order that: it makes no
-  // wavefront wait for its own outstanding no-return atomics.  So every wavefront first waits until the memory system
-  // has acknowledged all of its vector memory operations (vmcnt(0): a device-scope atomic is acknowledged once it has
-  // been performed at the device's coherence point, past the per-XCD L2), then the barrier collects the wavefronts,
-  // and only then the ticket is drawn.  Whoever draws the last ticket therefore finds every block's counts in place
-  // and reads them with device-scope atomic loads.  No cache write-back or invalidation is involved (the payload is
-  // atomics only), which a release / acquire fence per block would cost.
-  __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0), expcnt / lgkmcnt untouched
-  asm volatile("" ::: "memory");
-  __syncthreads();
-  if (threadIdx.x == 0)
-    scratch[kHistBlock / 64] = atomicAdd(&st->done[pass], 1u);
-  __syncthreads();
-  if (scratch[kHistBlock / 64] != gridDim.x - 1)
-    return;
-  // thread t owns the bins [t * per, (t + 1) * per), per = 2 or 1
-  const int per = bins / kHistBlock, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  uint32_t c[kMaxBins / kHistBlock];
-#pragma unroll
-  for (int i = 0; i < kMaxBins / kHistBlock; ++i)
-    c[i] = 0u;
-  for (int k = 0; k < kGlobalCopies; ++k) {
-    const unsigned long long *src = reinterpret_cast<const unsigned long long *>(&st->hist[pass][k][threadIdx.x * per]);
-    if (per == 1) {
-      c[0] += __hip_atomic_load(&st->hist[pass][k][threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      continue;
-    }
-#pragma unroll
-    for (int i = 0; i < kMaxBins / kHistBlock / 2; ++i)
-      if (2 * i < per) {
-        const unsigned long long two = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        c[2 * i] += (uint32_t)two;
-        c[2 * i + 1] += (uint32_t)(two >> 32);
-      }
-  }
-  uint32_t mine = 0;
-#pragma unroll
-  for (int i = 0; i < kMaxBins / kHistBlock; ++i)
-    mine += c[i];
-  uint32_t incl = mine;
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    const uint32_t up = __shfl_up(incl, off);
-    if (lane >= off)
-      incl += up;
-  }
-  if (lane == 63)
-    scratch[wave] = incl;
-  __syncthreads();
-  uint32_t excl = incl - mine;
-  for (int w = 0; w < wave; ++w)
-    excl += scratch[w];
-#pragma unroll
-  for (int i = 0; i < kMaxBins / kHistBlock; ++i) {
-    if (c[i] != 0u && excl <= rank && rank < excl + c[i]) {
-      st->prefix[pass + 1] = prefix | ((uint32_t)(threadIdx.x * per + i) << shift);
-      st->rank[pass + 1] = rank - excl;
-    }
-    excl += c[i];
-  }
+  select_finish<false>(h, scratch, st, sp);
 }
 
 // y = (|x| < thresh) ? 0 : x with thresh = |rank-th smallest| (+ 1 when rate == 1), prune.cpp:62-69
@@ -620,8 +512,7 @@ int nbla_hip_prune_f32(const float *x, float *y, size_t size, float rate, void *
   int64_t blocks = ceil_div(n4 ? n4 : 1, (int64_t)kHistBlock * 4);
   if (blocks > kSelectBlocks)
     blocks = kSelectBlocks;
-  hipLaunchKernelGGL(clear_select, dim3((unsigned)ceil_div(kPasses * kGlobalCopies * kMaxBins, kBlock)), dim3(kBlock), 0,
-                     stream, st, rank);
+  hipLaunchKernelGGL(clear_select, dim3(clear_select_blocks()), dim3(256), 0, stream, st, rank);
   NBLA_HIP_LAUNCH_CHECK("clear_select");
   for (int p = 0; p < kPasses; ++p) {
     hipLaunchKernelGGL(prune_histogram, dim3((unsigned)blocks), dim3(kHistBlock), 0, stream, x, n4, n, st, p);

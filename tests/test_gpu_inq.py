@@ -81,6 +81,87 @@ def test_inq_largest_abs_tie_free_half_selection(dev):
         assert Ic.sum() == max(size // 2, 1)
 
 
+@pytest.mark.parametrize("size,offset", [(7, 0), (1000, 0), (4099, 1), (70001, 0), (262147, 3), (1 << 21, 0)])
+@pytest.mark.parametrize("distinct", [1, 3, 40])
+def test_inq_largest_abs_with_many_equal_magnitudes(dev, size, offset, distinct):
+    """Weights drawn from a handful of magnitudes, part of them already fixed: std::sort leaves the order of equal
+    magnitudes to the library (inq_affine.cpp:121-123), so the comparison with the oracle is per magnitude -- the
+    number of newly fixed weights of every magnitude -- plus what the selection itself promises: num_learnable // 2
+    are fixed, none of them smaller than a weight left learnable, and among the weights of the magnitude where the
+    selection stops the lowest indices are taken.  `offset` moves the arrays off 16-byte alignment."""
+    rng = np.random.RandomState(size + distinct)
+    mags = (0.001 * (1 + np.arange(distinct))).astype(np.float32)
+    W = (mags[rng.randint(0, distinct, size)] * np.where(rng.rand(size) < 0.5, -1, 1)).astype(np.float32)
+    I0 = (rng.rand(size) < 0.3).astype(np.int32)
+    inq = oracle.Inq(size, 4, (0, 9), "largest_abs")
+    Wc, Ic = W.copy(), I0.copy()
+    inq.quantize_weights(Wc, Ic)
+    Wd = torch.zeros(size + offset, dtype=torch.float32, device=dev)[offset:]
+    Id = torch.zeros(size + offset, dtype=torch.int32, device=dev)[offset:]
+    Wd.copy_(_dev(W, dev)), Id.copy_(_dev(I0, dev))
+    kernels.inq_update_weights(Wd, Id, torch.zeros_like(Wd), torch.zeros_like(Id), 4, kernels.INQ_LARGEST_ABS)
+    Ig = to_np(Id)
+    learnable = I0 == 0
+    T = int(learnable.sum()) // 2
+    new_g, new_c = (Ig == 1) & learnable, (Ic == 1) & learnable
+    assert np.array_equal(Ig[~learnable], I0[~learnable])
+    assert new_g.sum() == new_c.sum() == max(T, int(new_c.sum()))
+    a = np.abs(W)
+    for m in mags:
+        assert (new_g & (a == m)).sum() == (new_c & (a == m)).sum(), "magnitude %g" % m
+    if new_g.any() and (learnable & ~new_g).any():
+        stop = a[new_g].min()
+        assert stop >= a[learnable & ~new_g].max()
+        ties = np.flatnonzero(learnable & (a == stop))
+        taken = int(new_g[ties].sum())
+        assert new_g[ties[:taken]].all() and not new_g[ties[taken:]].any()
+    # the weights fixed by both are quantized alike
+    both = (Ig == 1) & (Ic == 1)
+    assert bits_equal(to_np(Wd)[both], Wc[both])
+
+
+def test_inq_largest_abs_with_one_learnable_weight(dev):
+    """num_learnable // 2 == 0: the loop of inq_affine.cpp:133-141 still looks at the first index of the sorted
+    order and fixes it if it is learnable, i.e. only when the one learnable weight has the largest magnitude."""
+    for size, where, largest in ((1, 0, True), (5, 3, True), (5, 3, False), (3000, 2999, True), (3000, 17, False)):
+        W = np.linspace(0.01, 0.02, size).astype(np.float32)
+        W[where] = 0.5 if largest else 0.001
+        I0 = np.ones(size, np.int32)
+        I0[where] = 0
+        inq = oracle.Inq(size, 4, (0, 9), "largest_abs")
+        Wc, Ic = W.copy(), I0.copy()
+        inq.quantize_weights(Wc, Ic)
+        Wd, Id = _dev(W, dev), _dev(I0, dev)
+        kernels.inq_update_weights(Wd, Id, torch.zeros_like(Wd), torch.zeros_like(Id), 4, kernels.INQ_LARGEST_ABS)
+        assert Ic[where] == int(largest)
+        assert np.array_equal(to_np(Id), Ic), (size, where, largest)
+        assert bits_equal(to_np(Wd), Wc)
+    # nothing learnable at all
+    W, I0 = np.full(9, 0.3, np.float32), np.ones(9, np.int32)
+    Wd, Id = _dev(W, dev), _dev(I0, dev)
+    kernels.inq_update_weights(Wd, Id, torch.zeros_like(Wd), torch.zeros_like(Id), 4, kernels.INQ_LARGEST_ABS)
+    assert to_np(Id).min() == 1
+
+
+@pytest.mark.parametrize("size,offset", [(5, 0), (4099, 1), (300001, 0)])
+def test_inq_random_selection_draw_order(dev, size, offset):
+    """Learnable weight number r in index order takes draw r of the stream (inq_affine.cpp:143-149), for any
+    alignment and for sizes above one chunk of the ranking kernels."""
+    rng = np.random.RandomState(size)
+    W = (rng.randn(size) * 0.05).astype(np.float32)
+    I0 = (rng.rand(size) < 0.4).astype(np.int32)
+    inq = oracle.Inq(size, 4, (0, 9), "random", 5)
+    stream = oracle.Bernoulli(5)
+    Wc, Ic = W.copy(), I0.copy()
+    inq.quantize_weights(Wc, Ic)
+    Wd = torch.zeros(size + offset, dtype=torch.float32, device=dev)[offset:]
+    Id = torch.zeros(size + offset, dtype=torch.int32, device=dev)[offset:]
+    Wd.copy_(_dev(W, dev)), Id.copy_(_dev(I0, dev))
+    kernels.inq_update_weights(Wd, Id, torch.zeros_like(Wd), torch.zeros_like(Id), 4, kernels.INQ_RANDOM,
+                               draw=stream.draw)
+    assert np.array_equal(to_np(Id), Ic) and bits_equal(to_np(Wd), Wc)
+
+
 @pytest.mark.parametrize("num_bits,top", [(4, 1.9), (6, 1.4)])
 def test_inq_every_weight_of_the_level_range(dev, num_bits, top):
     """Every fp32 value from below the pruning threshold up to max|w| (whole binades, both signs), all fixed:
