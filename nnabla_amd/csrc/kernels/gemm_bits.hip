@@ -16,6 +16,7 @@
 // with one AND each.
 // Every wavefront keeps 3 x MF x NF accumulator tiles, so blocks are sized for one wavefront per SIMD.
 #include "common.hpp"
+#include "copy_pipeline.hpp"
 #include "gemm_layout.hpp"
 #include "internal.hpp"
 
@@ -144,7 +145,14 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
   constexpr int kStagesCnt = 63 / (kPerWave + 1) + 2; // (kStages - 2) * (kPerWave + 1) < 64
   constexpr int kStages = kUsed == kDigits ? kStagesFull : (kStagesFit < kStagesCnt ? kStagesFit : kStagesCnt);
   constexpr int kDepth = kStages - 1; // k steps in flight ahead of the one being multiplied
-  static_assert(kDepth >= 2 && (kDepth - 1) * (kPerWave + 1) < 64, "vmcnt is a 6-bit counter");
+  // How many of the most recently issued k steps each wait may leave in flight: taken from the model of this loop's
+  // order of copies, waits, barriers and LDS reads (copy_pipeline.hpp), which is also asserted safe as a whole.
+  constexpr int kPrologueWait = pipeline::two_tile_prologue_wait(kStages, kDepth);
+  constexpr int kLoopWait = pipeline::two_tile_loop_wait(kStages, kDepth);
+  static_assert(kPrologueWait >= 0 && kLoopWait >= 0 &&
+                    pipeline::two_tile_safe(kStages, kDepth, kPrologueWait, kLoopWait),
+                "the copy pipeline hands a buffer over too early");
+  static_assert(pipeline::counter_fits(kPrologueWait, kPerWave + (kExtra ? 1 : 0)), "vmcnt is a 6-bit counter");
 
   if (a.split_steps > 0) {
     const int64_t begin = a.step_begin + (int64_t)blockIdx.y * a.split_steps;
@@ -293,7 +301,7 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
 #pragma unroll
   for (int d = 0; d < kDepth; ++d)
     copy_next(d);
-  wait_copies(std::integral_constant<int, kDepth - 1>());
+  wait_copies(std::integral_constant<int, kPrologueWait>());
   NBLA_BARRIER();
   read_words(0, 0, w0);
   read_a(0, 0, af0);
@@ -304,7 +312,7 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
   if (idle) {
     for (int64_t ks = first; ks <= last; ks += kWavesK) {
       const int buf_copy = (buf == 0) ? kStages - 1 : buf - 1;
-      wait_copies(std::integral_constant<int, kDepth - 2>());
+      wait_copies(std::integral_constant<int, kLoopWait>());
       NBLA_BARRIER();
       copy_next(buf_copy);
       buf = (buf + 1 == kStages) ? 0 : buf + 1;
@@ -321,9 +329,9 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
       __builtin_amdgcn_sched_barrier(0);
       mma(af0, w0, J1(), JN());
       __builtin_amdgcn_sched_barrier(0);
-      // step ks+1 has landed: the copies issued so far reach step ks+kDepth-1, so at most the kDepth-2 steps behind
-      // ks+1 may still be in flight; every wavefront is done with the buffer of step ks-1
-      wait_copies(std::integral_constant<int, kDepth - 2>());
+      // step ks+1 has landed: the copies issued so far reach step ks+kDepth-1, so at most the kDepth-2 (= kLoopWait)
+      // steps behind ks+1 may still be in flight; every wavefront is done with the buffer of step ks-1
+      wait_copies(std::integral_constant<int, kLoopWait>());
       NBLA_BARRIER();
       // tile 1 runs; the copy of step ks+kDepth is issued; tile 0 of step ks+1 is fetched
       mma(af1, w1, J0(), J1());

@@ -10,6 +10,7 @@
 // Tiling: 128 x 128 outputs per block of four wavefronts (2 x 2, 64 x 64 each: 2 x 2 fragments x 3 accumulators =
 // 192 registers), k in tiles of 32 (one v_mfma_i32_32x32x32_i8 fragment).
 #include "common.hpp"
+#include "copy_pipeline.hpp"
 #include "gemm_layout.hpp"
 #include "internal.hpp"
 
@@ -45,6 +46,21 @@ constexpr int kPerWave = kChunks / kWaves;     // 6
 // one block anyway: with one wavefront per SIMD a k tile is multiplied in a few hundred cycles and the copies need
 // the longer head start to cover the memory latency.
 constexpr int kStagesShared = 3, kStagesAlone = 6;
+
+// Which of a wavefront's kPerWave copy slots a call of copy_next issues (the list of a k tile is ordered so that
+// every form of the product needs a prefix of each wavefront's share), and how many that makes: the unit in which the
+// loop's wait counts copies in flight.
+constexpr bool copy_slot_used(int p, bool one_a, bool narrow, int groups) {
+  const int all_waves = kWaves * groups, per_tile = kChunks / all_waves;
+  return one_a ? p < (2 * kSegs / all_waves) * groups
+               : !(narrow && p % per_tile >= (kSegs * kDigits + kSegs) / all_waves);
+}
+constexpr int copies_per_call(bool one_a, bool narrow, int groups) {
+  int n = 0;
+  for (int p = 0; p < kPerWave; ++p)
+    n += copy_slot_used(p, one_a, narrow, groups) ? 1 : 0;
+  return n;
+}
 
 // Workgroup barrier without the memory fence of __syncthreads() (which would wait for every global -> LDS copy in
 // flight, including those of later k tiles); the waits that matter are explicit.
@@ -132,7 +148,7 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
   auto copy_next = [&](int buf) {
 #pragma unroll
     for (int p = 0; p < kPerWave; ++p) {
-      if (kOneA ? p >= kOnePerTile * kGroups : (kNarrow && p % kPerTile >= kNeeded))
+      if (!copy_slot_used(p, kOneA, kNarrow, kGroups))
         continue;
       __builtin_amdgcn_global_load_lds(cur[p] + lane, (lds_void_t *)(smem + buf * kGroupStageBytes + dest[p]), 16, 0,
                                        0);
@@ -152,7 +168,13 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
         for (int r = 0; r < 16; ++r)
           acc[i][j][t][r] = 0;
 
-  static_assert((kStages - 2) * kPerWave < 64, "vmcnt is a 6-bit counter");
+  // The number of most recently issued k tiles the wait at the top of a tile may leave in flight, from the model of
+  // this loop's order of copies, waits, barriers and LDS reads (copy_pipeline.hpp)
+  constexpr int kLoopWait = pipeline::one_tile_loop_wait(kStages, kStages - 1);
+  static_assert(kLoopWait >= 0 && pipeline::one_tile_safe(kStages, kStages - 1, kLoopWait),
+                "the copy pipeline hands a buffer over too early");
+  static_assert(pipeline::counter_fits(kLoopWait, kPerWave), "vmcnt is a 6-bit counter");
+  static_assert(copies_per_call(kOneA, kNarrow, kGroups) == kCopies, "the wait counts the copies a call issues");
 #pragma unroll
   for (int d = 0; d < kStages - 1; ++d)
     copy_next(d);
@@ -160,7 +182,7 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
   for (int64_t kt = a.step_begin; kt < a.step_end; kt += kGroups) {
     // tile kt has landed (the copies of the kStages - 2 tiles after it may still be in flight) and every wavefront
     // is done with the buffer tile kt - 1 occupied, which tile kt + kStages - 1 takes over
-    NBLA_WAIT_VMCNT((kStages - 2) * kCopies);
+    NBLA_WAIT_VMCNT(kLoopWait * kCopies);
     NBLA_BARRIER();
     copy_next(buf == 0 ? kStages - 1 : buf - 1);
     const uint4_t *sa = reinterpret_cast<const uint4_t *>(smem + buf * kGroupStageBytes + group * kStageBytes);
