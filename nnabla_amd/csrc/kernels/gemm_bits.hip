@@ -21,6 +21,7 @@
 #include "internal.hpp"
 
 #include <type_traits>
+#include <utility>
 
 namespace nbla_hip {
 namespace {
@@ -173,24 +174,33 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
   int64_t bm, bn;
   band_tile<8>(blockIdx.x, a.blocks_m, a.blocks_n, bm, bn);
 
-  // Sources of this wavefront's copies (uniform bases; the lane adds its own 16 bytes).  Row blocks / wide groups
-  // past the end of the operand are clamped: their products land in rows/columns that are not stored.
+  // Sources of this wavefront's copies.  Slot p of wavefront w copies chunk p * kWaves + w of every stage; the chunk is
+  // described by a buffer resource that starts at the chunk's bytes in the first stage of this launch and ends with
+  // its bytes in the last one, and by a scalar byte offset that advances by one stage per copy (the lane adds its own
+  // 16 bytes).  The hardware range check (it covers the scalar offset too) turns a copy past the end (the copies run kDepth stages ahead of the last multiplication) into
+  // zeros in LDS: no address is clamped in the loop.  Row blocks / wide groups past the end of the operand are
+  // clamped here: their products land in rows / columns that are not stored.
   constexpr int kSlots = kPerWave + (kExtra ? 1 : 0);
-  const uint4_t *src[kSlots];
-  int64_t src_step[kSlots]; // advance per k step, in uint4
+  const int nstages = (int)((a.step_end - a.step_begin) / kWavesK);
+  __amdgpu_buffer_rsrc_t rsrc[kSlots];
+  uint32_t stage_bytes[kSlots]; // advance per stage
+  uint32_t soff[kSlots];        // offset of the next stage inside the resource
+  const uint32_t lane_bytes = lane * 16;
 #pragma unroll
   for (int p = 0; p < kSlots; ++p) {
     const int cs = p * kWaves + wave;                 // chunk of the stage
     const int kk = (cs / kStepChunks) % kWavesK;      // k step inside the stage
     const int c = cs - (cs / kStepChunks) * kStepChunks;
+    const uint4_t *src;
+    int64_t src_step; // advance per k step, in uint4
     if (c < kAFrags) {
       const int seg = c / kSegFrags, rem = c - seg * kSegFrags; // rem = (k tile of the step, digit in use)
       const int t = rem / kUsed, d = kFirst + rem - t * kUsed;
       int64_t rb = bm * kASegs + seg;
       if (rb >= a.row_blocks)
         rb = a.row_blocks - 1;
-      src_step[p] = kSrcSegFrags * 64;
-      src[p] = a.xd + (rb * a.x_k_tiles * kDigits + t * kDigits + d) * 64 + kk * src_step[p];
+      src_step = kSrcSegFrags * 64;
+      src = a.xd + (rb * a.x_k_tiles * kDigits + t * kDigits + d) * 64 + kk * src_step;
     } else {
       // packed words: chunk = (k tile of the step, wide group of the tile)
       const int cb = c - kAFrags;
@@ -198,39 +208,37 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
       int64_t wg = a.n_begin / kWideGroup + bn * (BN / kWideGroup) + (cb - t * (BN / kWideGroup));
       if (wg >= a.wide_groups)
         wg = a.wide_groups - 1;
-      src_step[p] = 2 * a.wide_groups * 64;
-      src[p] = reinterpret_cast<const uint4_t *>(a.bits) + (t * a.wide_groups + wg) * 64 + kk * src_step[p];
+      src_step = 2 * a.wide_groups * 64;
+      src = reinterpret_cast<const uint4_t *>(a.bits) + (t * a.wide_groups + wg) * 64 + kk * src_step;
     }
+    stage_bytes[p] = (uint32_t)(src_step * kWavesK * 16); // the host checks that a launch's stages span < 4 GiB
+    const uint32_t span = (uint32_t)(nstages - 1) * stage_bytes[p] + kFragBytes;
+    // (every input is uniform; reading the address through the first lane tells the compiler so, which keeps the
+    // resource in scalar registers)
+    const uint64_t first = reinterpret_cast<uint64_t>(src + a.step_begin * src_step);
+    const uint64_t base = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first >> 32)) << 32) |
+                          (uint32_t)__builtin_amdgcn_readfirstlane((int)first);
+    rsrc[p] = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>(base), 0,
+                                                __builtin_amdgcn_readfirstlane((int)span), 0x00020000);
+    stage_bytes[p] = __builtin_amdgcn_readfirstlane((int)stage_bytes[p]);
+    soff[p] = 0;
   }
   typedef __attribute__((address_space(3))) void lds_void_t;
-  auto lds_at = [&](int byte_off) { return (lds_void_t *)(smem + byte_off); };
-  // Stages are copied in order; each slot keeps a cursor that advances by one stage per call and stops at the last
-  // stage (the final calls copy it again rather than run past the operand).
-  const uint4_t *cur[kSlots], *cur_last[kSlots];
+  const int wave_lds = wave * kFragBytes;
+  // issues this wavefront's kCount copies of the next stage into the LDS buffer at byte offset `buf_bytes`
+  auto copy_next = [&](int buf_bytes, auto count_c) __attribute__((always_inline)) {
+    constexpr int kCount = decltype(count_c)::value;
 #pragma unroll
-  for (int p = 0; p < kSlots; ++p) {
-    cur[p] = src[p] + a.step_begin * src_step[p];
-    cur_last[p] = src[p] + (a.step_end - kWavesK) * src_step[p];
-  }
-  // issues the copies of the next stage into LDS buffer `buf`
-  auto copy_next = [&](int buf) {
-#pragma unroll
-    for (int p = 0; p < kSlots; ++p) {
-      if (p == kPerWave && wave >= kExtra)
-        break;
-      __builtin_amdgcn_global_load_lds(cur[p] + lane, lds_at(buf * kStageBytes + (p * kWaves + wave) * kFragBytes), 16,
-                                       0, 0);
-      const uint4_t *next = cur[p] + kWavesK * src_step[p];
-      cur[p] = next < cur_last[p] ? next : cur_last[p];
+    for (int p = 0; p < kCount; ++p) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc[p], (lds_void_t *)(smem + (wave_lds + buf_bytes) + p * kWaves * kFragBytes), 16, lane_bytes, soff[p], 0,
+          0);
+      soff[p] += stage_bytes[p];
     }
   };
-  // waits until at most `steps` k steps of this wavefront's copies are in flight
-  auto wait_copies = [&](auto steps) {
-    constexpr int n = decltype(steps)::value;
-    if (kExtra && wave < kExtra)
-      NBLA_WAIT_VMCNT(n * (kPerWave + 1));
-    else
-      NBLA_WAIT_VMCNT(n * kPerWave);
+  // waits until at most `steps` stages of this wavefront's copies (kCount each) are in flight
+  auto wait_copies = [&](auto steps, auto count_c) __attribute__((always_inline)) {
+    NBLA_WAIT_VMCNT(decltype(steps)::value * decltype(count_c)::value);
   };
 
   i32x16_t acc[kDigits][MF][NF];
@@ -245,8 +253,8 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
           acc[d][i][j][r] = 0;
 
   // Fragment fetch and the MFMA block of one k tile (t = 0, 1) of a staged step.
-  auto read_a = [&](int buf, int t, uint4_t (&af)[MF][kUsed]) {
-    const uint4_t *sa = reinterpret_cast<const uint4_t *>(smem + buf * kStageBytes + wk * kStepBytes);
+  auto read_a = [&](int buf_bytes, int t, uint4_t (&af)[MF][kUsed]) __attribute__((always_inline)) {
+    const uint4_t *sa = reinterpret_cast<const uint4_t *>(smem + buf_bytes + wk * kStepBytes);
 #pragma unroll
     for (int i = 0; i < MF; ++i)
 #pragma unroll
@@ -254,8 +262,8 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
         af[i][d] = sa[((wm * MF + i) * kSegFrags + t * kUsed + d) * 64 + lane];
   };
   const int frag0 = (wn * NF) % (kWideGroup / 32); // index of this wavefront's first column fragment in its group
-  auto read_words = [&](int buf, int t, uint4_t &words) {
-    const uint4_t *sb = reinterpret_cast<const uint4_t *>(smem + buf * kStageBytes + wk * kStepBytes + kABytes);
+  auto read_words = [&](int buf_bytes, int t, uint4_t &words) __attribute__((always_inline)) {
+    const uint4_t *sb = reinterpret_cast<const uint4_t *>(smem + buf_bytes + wk * kStepBytes + kABytes);
     words = sb[(t * (BN / kWideGroup) + (wn * NF) / (kWideGroup / 32)) * 64 + lane];
   };
   // Bits -> bytes in {0, 2^F}: register i of column fragment F is word_i & (0x01010101 << F).
@@ -265,7 +273,7 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
     frag_mask[j] = 0x01010101u << (frag0 + j);
     asm volatile("" : "+s"(frag_mask[j]));
   }
-  auto mma = [&](const uint4_t (&af)[MF][kUsed], const uint4_t &words, auto j_begin, auto j_end) {
+  auto mma = [&](const uint4_t (&af)[MF][kUsed], const uint4_t &words, auto j_begin, auto j_end) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = decltype(j_begin)::value; j < decltype(j_end)::value; ++j) {
       uint4_t bf;
@@ -277,12 +285,9 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
       for (int d = 0; d < kUsed; ++d)
 #pragma unroll
         for (int i = 0; i < MF; ++i) {
-          acc[kFirst + d][i][j] = kSwap ? __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, bf),
-                                                                                __builtin_bit_cast(i32x4_t, af[i][d]),
-                                                                                acc[kFirst + d][i][j], 0, 0, 0)
-                                        : __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, af[i][d]),
-                                                                                __builtin_bit_cast(i32x4_t, bf),
-                                                                                acc[kFirst + d][i][j], 0, 0, 0);
+          const i32x4_t va = __builtin_bit_cast(i32x4_t, af[i][d]), vb = __builtin_bit_cast(i32x4_t, bf);
+          acc[kFirst + d][i][j] =
+              __builtin_amdgcn_mfma_i32_32x32x32_i8(kSwap ? vb : va, kSwap ? va : vb, acc[kFirst + d][i][j], 0, 0, 0);
         }
     }
   };
@@ -290,61 +295,70 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
   // the matrix pipe busy for 32 cycles, so each half step is laid out by hand: the MFMAs of the first column
   // fragment go first, the LDS reads of the next k tile (and the copies of a later k step) are issued in their
   // shadow, and the remaining MFMAs cover the latency.  sched_barrier pins that order.
+  // Everything that is not an MFMA is kept short, because a wavefront cannot feed the matrix pipe while it works
+  // through scalar and address instructions: the copies are bounds-checked buffer loads whose addresses advance by
+  // one scalar add each; the number of copies a wavefront issues per stage (kPerWave, or one more for the first
+  // kExtra wavefronts) is a compile-time constant of its copy of the loop; the ring position is kept as three byte
+  // offsets that rotate; the loop counter is 32 bits wide.
   typedef std::integral_constant<int, 0> J0;
   typedef std::integral_constant<int, 1> J1;
   typedef std::integral_constant<int, NF> JN;
   uint4_t af0[MF][kUsed], af1[MF][kUsed];
   uint4_t w0, w1;
-  // stages are numbered by their first k step; the operands are padded so that the number of k steps is a multiple
-  // of kWavesK
-  const int64_t first = a.step_begin, last = a.step_end - kWavesK;
-#pragma unroll
-  for (int d = 0; d < kDepth; ++d)
-    copy_next(d);
-  wait_copies(std::integral_constant<int, kPrologueWait>());
-  NBLA_BARRIER();
-  read_words(0, 0, w0);
-  read_a(0, 0, af0);
   // A wavefront whose columns all lie past the end of the operand (last tile of a row of tiles) only takes part in
   // the copies and barriers: the matrix pipe of its SIMD is left to the other wavefront.
   const bool idle = a.n_begin + bn * BN + wn * NF * 32 >= a.n_end;
-  int buf = 0; // LDS buffer of step ks
-  if (idle) {
-    for (int64_t ks = first; ks <= last; ks += kWavesK) {
-      const int buf_copy = (buf == 0) ? kStages - 1 : buf - 1;
-      wait_copies(std::integral_constant<int, kLoopWait>());
-      NBLA_BARRIER();
-      copy_next(buf_copy);
-      buf = (buf + 1 == kStages) ? 0 : buf + 1;
+  auto run = [&](auto count_c) __attribute__((always_inline)) {
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d)
+      copy_next(d * kStageBytes, count_c);
+    wait_copies(std::integral_constant<int, kPrologueWait>(), count_c);
+    NBLA_BARRIER();
+    read_words(0, 0, w0);
+    read_a(0, 0, af0);
+    // byte offsets of the LDS buffers of step ks (`cur`), of step ks-1 = that of step ks+kDepth (`prev`)
+    int cur = 0, prev = (kStages - 1) * kStageBytes;
+    if (idle) {
+      for (int left = nstages; left > 0; --left) {
+        wait_copies(std::integral_constant<int, kLoopWait>(), count_c);
+        NBLA_BARRIER();
+        copy_next(prev, count_c);
+        prev = cur;
+        cur = (cur + kStageBytes == kStages * kStageBytes) ? 0 : cur + kStageBytes;
+      }
+      return;
     }
-  } else {
-    for (int64_t ks = first; ks <= last; ks += kWavesK) {
-      const int buf_next = (buf + 1 == kStages) ? 0 : buf + 1;
-      const int buf_copy = (buf == 0) ? kStages - 1 : buf - 1; // the buffer step ks-1 occupied = that of step ks+kDepth
+    for (int left = nstages; left > 0; --left) {
+      const int next = (cur + kStageBytes == kStages * kStageBytes) ? 0 : cur + kStageBytes;
       // tile 0 runs; tile 1 is fetched
       mma(af0, w0, J0(), J1());
       __builtin_amdgcn_sched_barrier(0);
-      read_a(buf, 1, af1);
-      read_words(buf, 1, w1);
+      read_a(cur, 1, af1);
+      read_words(cur, 1, w1);
       __builtin_amdgcn_sched_barrier(0);
       mma(af0, w0, J1(), JN());
       __builtin_amdgcn_sched_barrier(0);
       // step ks+1 has landed: the copies issued so far reach step ks+kDepth-1, so at most the kDepth-2 (= kLoopWait)
       // steps behind ks+1 may still be in flight; every wavefront is done with the buffer of step ks-1
-      wait_copies(std::integral_constant<int, kLoopWait>());
+      wait_copies(std::integral_constant<int, kLoopWait>(), count_c);
       NBLA_BARRIER();
       // tile 1 runs; the copy of step ks+kDepth is issued; tile 0 of step ks+1 is fetched
       mma(af1, w1, J0(), J1());
       __builtin_amdgcn_sched_barrier(0);
-      copy_next(buf_copy);
-      read_words(buf_next, 0, w0);
-      read_a(buf_next, 0, af0);
+      copy_next(prev, count_c);
+      read_words(next, 0, w0);
+      read_a(next, 0, af0);
       __builtin_amdgcn_sched_barrier(0);
       mma(af1, w1, J1(), JN());
       __builtin_amdgcn_sched_barrier(0);
-      buf = buf_next;
+      prev = cur;
+      cur = next;
     }
-  }
+  };
+  if (kExtra && wave < kExtra)
+    run(std::integral_constant<int, kPerWave + 1>());
+  else
+    run(std::integral_constant<int, kPerWave>());
   NBLA_WAIT_VMCNT(0);
 
   if (kWavesK > 1) {
@@ -641,6 +655,10 @@ int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alp
                 (long long)N);
   if (!aligned16(xdigits) || !aligned16(bits))
     return fail(NBLA_HIP_ERR_MEMORY, "GEMM operands must be 16-byte aligned.");
+  // the copies address one launch's share of the packed operand (at most kChunkK / 32 k tiles) with 32-bit offsets
+  if (bits_wide_groups(N) * kFragBytes * (kChunkK / kTileK) >= (int64_t)0xffffffffll)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "bit-weight product: more than %lld output columns are not supported.",
+                (long long)(0xffffffffll / (kFragBytes * (kChunkK / kTileK)) * kWideGroup));
   int rc = ensure_init();
   if (rc)
     return rc;
