@@ -538,7 +538,11 @@ int binary_conv_forward(const float *x, const float *W, float *Wb, float *alpha,
     float *yg = y + grp * g.Og * hw;
     const float *ag = alpha ? alpha + grp * g.Og : nullptr;
     const float *bg = bias ? bias + grp * g.Og : nullptr;
-    if (use_bits) {
+    if (use_bits && gemm_bits_unfold_applies(g)) {
+      rc = launch_gemm_bits_unfold(x, g, grp,
+                                   reinterpret_cast<const uint32_t *>(base + ws.bits_off + grp * ws.bits_stride), ag, bg,
+                                   yg, stream);
+    } else if (use_bits) {
       rc = launch_im2col_digits(x, base + ws.split_off, base + ws.cmax_off, g, grp, stream);
       if (rc)
         return rc;

@@ -16,6 +16,7 @@
 // with one AND each.
 // Every wavefront keeps 3 x MF x NF accumulator tiles, so blocks are sized for one wavefront per SIMD.
 #include "common.hpp"
+#include "conv_geom.hpp"
 #include "copy_pipeline.hpp"
 #include "gemm_layout.hpp"
 #include "internal.hpp"
@@ -53,6 +54,11 @@ struct GemmBitsArgs {
   // split 0 adds the row sums
   int64_t split_steps; // 0: no split
   int use_sums;
+  // unfolding product (gemm_bits_unfold_kernel): the rows are the unfolded windows of x, converted to digits in the
+  // kernel; xd, sums and shift are unused
+  const float *ux;
+  ConvGeom ug;
+  int64_t ugrp;
 };
 
 // LDS buffers (stages resident) per tile shape: what fits the block's share of the CU's 160 KiB, at most six.
@@ -114,10 +120,273 @@ __device__ __forceinline__ float finish_dot(int a0, int a1, int a2, int s_hi, in
 // kUsed = 1: every row of the block's row blocks is a one-digit row (gemm_layout.hpp: the two lower digits are zero).
 // Only the top-digit fragments are copied and multiplied, into the top accumulator; the lower accumulators stay
 // zero and the epilogue is the same.  A third of the MFMAs and a third of the digit traffic, same bits.
-template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, bool kSwap, int kUsed>
+// The unfolding product keeps two buffers of kUnfoldSteps stages of the plain kernel each; past them (and past the
+// k groups' exchange area, which reuses the buffers at the end) the LDS holds the row sums, row maxima and row shifts,
+// then the table of decoded unfolded columns (16 bytes each).
+constexpr int kUnfoldSteps = 2;
+constexpr int kUnfoldMetaBytes = 512 + 64 * 16 + 2 * 256 * 4; // sums, maxima, shifts; the taps' table; alpha, bias
+constexpr int unfold_meta_off(int BM, int BN, int waves_m, int waves_n, int waves_k) {
+  const int stages = 2 * kUnfoldSteps * gemm_bits_stage_bytes(BM, BN, waves_k);
+  const int exchange = (waves_k - 1) * (BM / 32) * (BN / 32) * 4096;
+  return stages > exchange ? stages : exchange;
+}
+
+// Main loop of the unfolding product: the block's 32 rows are unfolded windows of x (rows m = (sample, output
+// position), columns kk = (channel, kernel tap), as im2col lays them out) that are never written to memory.  The block
+//  1. decodes every column kk once into an LDS table {offset of (channel, tap) relative to the window origin, one-hot
+//     64-bit mask of the tap (zero for kk >= Kg)}, and the taps (at most 64) into {offset, displacements};
+//  2. finds for each row which taps fall inside the input (a 64-bit mask: an element of the row is then read iff
+//     its column's mask meets the row's) and the row's largest magnitude (over its taps and channels: 16 channel
+//     slices per row, combined by an LDS maximum), and from that the row's power-of-two scale, exactly as the
+//     stand-alone unfold kernels do;
+//  3. walks the contraction in stages of eight k tiles with two LDS buffers.  Wavefront w produces k tile w of a
+//     stage: lane l gathers the sixteen values of row l % 32, k slots (l / 32) * 16 + 0..15, turns them into digits,
+//     writes them where the fragment's lane l holds them and adds their sum to the row's sum; it also moves the
+//     packed words of the tile to LDS.  Everything is loaded into registers two stages ahead (the loads of stage s+2
+//     are in flight while stage s is multiplied and stage s+1 converted and stored), one barrier per stage.  (Plain
+//     loads, not global -> LDS copies: with such a copy outstanding the compiler makes every LDS read wait for all
+//     loads, the gathered ones included.)
+// `multiply(buffer offset)` runs the wavefront's MFMAs of one stage of the plain kernel (kWavesK k steps).
+template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, int kStageBytes, int kStepBytes, int kABytes,
+          class Multiply>
+__device__ __forceinline__ void unfold_main_loop(const GemmBitsArgs &a, unsigned char *smem, int64_t bm, int64_t bn,
+                                                 int wave, int lane, bool idle, Multiply multiply) {
+  static_assert(BM == 32 && BN == kWideGroup && kWavesM * kWavesN * kWavesK == 8 && kWavesK == 2 && kUnfoldSteps == 2,
+                "thread mapping of the unfolding product: eight wavefronts, eight k tiles per stage");
+  constexpr int kThreads = 512, kStageTiles = 2 * kWavesK * kUnfoldSteps, kStageK = kStageTiles * kTileK;
+  constexpr int kBufBytes = kUnfoldSteps * kStageBytes;
+  constexpr int kMetaOff = unfold_meta_off(BM, BN, kWavesM, kWavesN, kWavesK);
+  typedef __attribute__((address_space(3))) void lds_void_t;
+  const ConvGeom &g = a.ug;
+  long long *s_sums = reinterpret_cast<long long *>(smem + kMetaOff);
+  uint32_t *s_amax = reinterpret_cast<uint32_t *>(smem + kMetaOff + 256);
+  int32_t *s_shift = reinterpret_cast<int32_t *>(smem + kMetaOff + 384);
+  i32x4_t *table = reinterpret_cast<i32x4_t *>(smem + kMetaOff + kUnfoldMetaBytes);
+  float *s_alpha = reinterpret_cast<float *>(smem + kMetaOff + 512 + 64 * 16), *s_bias = s_alpha + 256;
+  const int tid = threadIdx.x;
+  const int in0 = g.in_sp[0], in1 = g.in_sp[1], in2 = g.in_sp[2], plane = (int)g.in_sp_size;
+  const int k_tiles = (int)a.x_k_tiles, nstages = k_tiles / kStageTiles;
+
+  // 1. the decoded columns and taps
+  i32x4_t *taps_table = reinterpret_cast<i32x4_t *>(smem + kMetaOff + 512);
+  const int taps = (int)g.k_size;
+  {
+    const int K0 = g.k[0], K1 = g.k[1], K2 = g.k[2];
+    for (int kk = tid; kk < k_tiles * kTileK; kk += kThreads) {
+      int q = kk;
+      const int k2 = q % K2;
+      q /= K2;
+      const int k1 = q % K1;
+      q /= K1;
+      const int k0 = q % K0, c = q / K0;
+      const int e0 = k0 * g.dil[0], e1 = k1 * g.dil[1], e2 = k2 * g.dil[2];
+      const int tap = (k0 * K1 + k1) * K2 + k2;
+      const unsigned long long bit = kk < (int)g.Kg ? 1ull << tap : 0ull;
+      i32x4_t e;
+      e.x = c * plane + (e0 * in1 + e1) * in2 + e2;
+      e.y = 0;
+      e.z = (int)(uint32_t)bit;
+      e.w = (int)(uint32_t)(bit >> 32);
+      table[kk] = e;
+      if (kk < taps) { // channel 0: kk is the tap
+        i32x4_t t;
+        t.x = e.x;
+        t.y = e0 | (e1 << 16);
+        t.z = e2;
+        t.w = 0;
+        taps_table[kk] = t;
+      }
+    }
+    if (tid < 32) {
+      s_amax[tid] = 0u;
+      s_sums[tid] = 0;
+    }
+    if (tid < 256) { // the block's columns' alpha and bias: the epilogue reads them from LDS
+      const int64_t col = a.n_begin + bn * BN + tid;
+      const int64_t nc = col < a.N ? col : a.N - 1;
+      s_alpha[tid] = (a.finish && a.alpha) ? a.alpha[nc] : 1.0f;
+      s_bias[tid] = (a.finish && a.bias) ? a.bias[nc] : 0.0f;
+    }
+  }
+  // this thread's row (the same for both of its roles: lane % 32)
+  const int r = lane & 31, half = lane >> 5;
+  const int64_t m = bm * BM + r;
+  const bool in_range = m < a.M;
+  const int64_t n = in_range ? m / g.out_sp_size : 0;
+  int p = in_range ? (int)(m - n * g.out_sp_size) : 0;
+  const int o2 = p % g.out_sp[2];
+  p /= g.out_sp[2];
+  const int o1 = p % g.out_sp[1];
+  const int o0 = p / g.out_sp[1];
+  const int b0 = o0 * g.stride[0] - g.pad[0], b1 = o1 * g.stride[1] - g.pad[1], b2 = o2 * g.stride[2] - g.pad[2];
+  const int origin = (b0 * in1 + b1) * in2 + b2; // may be negative; only added to the offsets of taps inside the input
+  const float *xn = a.ux + (n * g.C + a.ugrp * g.Cg) * g.in_sp_size;
+  __syncthreads();
+
+  // 2. the row's taps inside the input, and its largest magnitude: channel slice = (wavefront, half); per tap the
+  // sixteen channels c = slice + 16 j of a round of 256 channels are in flight together
+  uint32_t mask_lo = 0u, mask_hi = 0u;
+  {
+    uint32_t amax = 0u;
+    const int slice = wave * 2 + half, Cg = (int)g.Cg;
+    // (tap, round of 256 channels) pairs, the loads of one pair in flight while the previous one is reduced
+    const int rounds = (Cg + 255) / 256, pairs = taps * rounds;
+    float v[2][16];
+    bool okv[2];
+    int c0v[2];
+    auto issue = [&](int pair, int slot) __attribute__((always_inline)) {
+      const int t = pair / rounds, c0 = slice + (pair - t * rounds) * 256;
+      const i32x4_t e = taps_table[t];
+      const int i0 = b0 + (e.y & 0xffff), i1 = b1 + (int)((uint32_t)e.y >> 16), i2 = b2 + e.z;
+      const bool ok = in_range && (unsigned)i0 < (unsigned)in0 && (unsigned)i1 < (unsigned)in1 &&
+                      (unsigned)i2 < (unsigned)in2;
+      if (ok) {
+        if (t < 32)
+          mask_lo |= 1u << t;
+        else
+          mask_hi |= 1u << (t - 32);
+      }
+      const float *src = xn + (ok ? origin + e.x : 0);
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int c = c0 + 16 * j;
+        v[slot][j] = src[(int64_t)(c < Cg ? c : slice) * plane];
+      }
+      okv[slot] = ok;
+      c0v[slot] = c0;
+    };
+    auto reduce = [&](int slot) __attribute__((always_inline)) {
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        if (okv[slot] && c0v[slot] + 16 * j < Cg)
+          amax = max(amax, __float_as_uint(v[slot][j]) & 0x7fffffffu);
+    };
+    issue(0, 0);
+    for (int pair = 0; pair < pairs; pair += 2) {
+      if (pair + 1 < pairs)
+        issue(pair + 1, 1);
+      reduce(0);
+      if (pair + 2 < pairs)
+        issue(pair + 2, 0);
+      if (pair + 1 < pairs)
+        reduce(1);
+    }
+    if (amax)
+      atomicMax(&s_amax[r], amax);
+  }
+  __syncthreads();
+  if (tid < 32) {
+    const uint32_t amax = s_amax[tid];
+    int s = 0;
+    if (amax >= 0x7f800000u) {
+      s = kBadRow;
+    } else if (amax != 0u) {
+      s = 22 - binade_exponent(binade_of(amax));
+      if (rintf(ldexpf(__uint_as_float(amax), s)) > (float)kDigitMax)
+        --s;
+    }
+    s_shift[tid] = s;
+  }
+  __syncthreads();
+
+  // 3. the stages
+  const int s_row = s_shift[r];
+  if (s_row == kBadRow) // a row holding a NaN or an infinity is not read: its outputs become NaN in the epilogue
+    mask_lo = mask_hi = 0u;
+  // k tile `wave` of a stage sits in stage wave / 4 of the buffer, k step (wave % 4) / 2, tile wave % 2 of the step
+  const int tile_off = (wave >> 2) * kStageBytes + ((wave & 3) >> 1) * kStepBytes;
+  int64_t wg = a.n_begin / kWideGroup + bn;
+  if (wg >= a.wide_groups)
+    wg = a.wide_groups - 1;
+  const uint4_t *words_src = reinterpret_cast<const uint4_t *>(a.bits) + wg * 64 + lane;
+  auto gather = [&](int stage, float (&v)[16], uint4_t &words) __attribute__((always_inline)) {
+    words = words_src[(int64_t)(stage * kStageTiles + wave) * a.wide_groups * 64];
+    const int kb = stage * kStageK + wave * kTileK + half * 16;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const i32x4_t e = table[kb + j];
+      const bool ok = (((uint32_t)e.z & mask_lo) | ((uint32_t)e.w & mask_hi)) != 0u;
+      const float xv = xn[ok ? origin + e.x : 0];
+      v[j] = ok ? xv : 0.0f;
+    }
+  };
+  // The three balanced base-256 digits of q (|q| <= kDigitMax) are the low three bytes of q + 0x808080, each with its
+  // top bit flipped: adding 128 per digit position makes every digit a plain byte.
+  auto emit = [&](int stage, const float (&v)[16], const uint4_t &words) __attribute__((always_inline)) {
+    uint32_t w[3][4];
+    int part = 0;
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4) {
+      uint32_t d[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int qv = (int)rintf(ldexpf(v[4 * g4 + j], s_row)); // masked values are 0.0f -> 0 whatever the shift
+        part += qv;
+        d[j] = ((uint32_t)qv + 0x808080u) ^ 0x808080u; // bytes: lowest, middle, top digit, unused
+      }
+      // byte transpose: word of a digit = that digit of the four values, value j in byte j
+      const uint32_t t01 = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u); // d0.b0 d1.b0 d0.b1 d1.b1
+      const uint32_t t23 = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u);
+      const uint32_t u01 = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u); // d0.b2 d1.b2 d0.b3 d1.b3
+      const uint32_t u23 = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
+      w[2][g4] = __builtin_amdgcn_perm(t23, t01, 0x05040100u); // lowest digits
+      w[1][g4] = __builtin_amdgcn_perm(t23, t01, 0x07060302u); // middle digits
+      w[0][g4] = __builtin_amdgcn_perm(u23, u01, 0x05040100u); // top digits
+    }
+    uint4_t *dst = reinterpret_cast<uint4_t *>(smem + (stage & 1) * kBufBytes + tile_off +
+                                               (wave & 1) * kDigits * kFragBytes) + lane;
+#pragma unroll
+    for (int d = 0; d < kDigits; ++d) {
+      uint4_t o;
+      o.x = w[d][0], o.y = w[d][1], o.z = w[d][2], o.w = w[d][3];
+      dst[d * 64] = o;
+    }
+    *(reinterpret_cast<uint4_t *>(smem + (stage & 1) * kBufBytes + tile_off + kABytes + (wave & 1) * kFragBytes) +
+      lane) = words;
+    if (part != 0)
+      atomicAdd(reinterpret_cast<unsigned long long *>(&s_sums[r]), (unsigned long long)(long long)part);
+  };
+  // one stage: `ahead` receives the loads of stage s+2, `next` holds those of stage s+1
+  auto stage_step = [&](int s, float (&ahead)[16], uint4_t &words_ahead, const float (&next)[16],
+                        const uint4_t &words_next) __attribute__((always_inline)) {
+    if (s + 2 < nstages)
+      gather(s + 2, ahead, words_ahead);
+    // Multiplying stage s (reads one buffer) and converting stage s+1 (writes the other) are independent.  The two
+    // wavefronts of a SIMD (w and w + 4) take them in opposite orders, so one's MFMAs run beside the other's vector
+    // instructions instead of both queueing for the same pipe after every barrier.
+    if (wave >= 4 && s + 1 < nstages)
+      emit(s + 1, next, words_next);
+    if (!idle) {
+#pragma unroll
+      for (int u = 0; u < kUnfoldSteps; ++u)
+        multiply((s & 1) * kBufBytes + u * kStageBytes);
+    }
+    if (wave < 4 && s + 1 < nstages)
+      emit(s + 1, next, words_next);
+    // this wavefront's digits, words and row sums have reached LDS; no memory fence: it would wait for the loads of
+    // stage s+2
+    __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
+    NBLA_BARRIER();
+  };
+  float va[16], vb[16];
+  uint4_t wa, wb;
+  gather(0, va, wa);
+  if (nstages > 1)
+    gather(1, vb, wb);
+  emit(0, va, wa);
+  __syncthreads();
+  for (int s = 0; s < nstages; s += 2) {
+    stage_step(s, va, wa, vb, wb);
+    if (s + 1 < nstages)
+      stage_step(s + 1, vb, wb, va, wa);
+  }
+}
+
+template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, bool kSwap, int kUsed, bool kUnfold = false>
 __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *smem) {
 #if defined(__HIP_DEVICE_COMPILE__) // the host pass only needs the launch stub; the body uses LDS address-space pointers
   static_assert(kUsed == 1 || kUsed == kDigits, "digits multiplied");
+  static_assert(!kUnfold || (kSwap && kUsed == kDigits), "the unfolding product stores one lane per row, three digits");
   constexpr int kFirst = 0; // first digit (and accumulator) in use: digits kFirst .. kFirst + kUsed - 1
   constexpr int kWavesMN = kWavesM * kWavesN;
   constexpr int kWaves = kWavesMN * kWavesK;
@@ -174,73 +443,6 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
   int64_t bm, bn;
   band_tile<8>(blockIdx.x, a.blocks_m, a.blocks_n, bm, bn);
 
-  // Sources of this wavefront's copies.  Slot p of wavefront w copies chunk p * kWaves + w of every stage; the chunk is
-  // described by a buffer resource that starts at the chunk's bytes in the first stage of this launch and ends with
-  // its bytes in the last one, and by a scalar byte offset that advances by one stage per copy (the lane adds its own
-  // 16 bytes).  The hardware range check (it covers the scalar offset too) turns a copy past the end (the copies run kDepth stages ahead of the last multiplication) into
-  // zeros in LDS: no address is clamped in the loop.  Row blocks / wide groups past the end of the operand are
-  // clamped here: their products land in rows / columns that are not stored.
-  constexpr int kSlots = kPerWave + (kExtra ? 1 : 0);
-  const int nstages = (int)((a.step_end - a.step_begin) / kWavesK);
-  __amdgpu_buffer_rsrc_t rsrc[kSlots];
-  uint32_t stage_bytes[kSlots]; // advance per stage
-  uint32_t soff[kSlots];        // offset of the next stage inside the resource
-  const uint32_t lane_bytes = lane * 16;
-#pragma unroll
-  for (int p = 0; p < kSlots; ++p) {
-    const int cs = p * kWaves + wave;                 // chunk of the stage
-    const int kk = (cs / kStepChunks) % kWavesK;      // k step inside the stage
-    const int c = cs - (cs / kStepChunks) * kStepChunks;
-    const uint4_t *src;
-    int64_t src_step; // advance per k step, in uint4
-    if (c < kAFrags) {
-      const int seg = c / kSegFrags, rem = c - seg * kSegFrags; // rem = (k tile of the step, digit in use)
-      const int t = rem / kUsed, d = kFirst + rem - t * kUsed;
-      int64_t rb = bm * kASegs + seg;
-      if (rb >= a.row_blocks)
-        rb = a.row_blocks - 1;
-      src_step = kSrcSegFrags * 64;
-      src = a.xd + (rb * a.x_k_tiles * kDigits + t * kDigits + d) * 64 + kk * src_step;
-    } else {
-      // packed words: chunk = (k tile of the step, wide group of the tile)
-      const int cb = c - kAFrags;
-      const int t = cb / (BN / kWideGroup);
-      int64_t wg = a.n_begin / kWideGroup + bn * (BN / kWideGroup) + (cb - t * (BN / kWideGroup));
-      if (wg >= a.wide_groups)
-        wg = a.wide_groups - 1;
-      src_step = 2 * a.wide_groups * 64;
-      src = reinterpret_cast<const uint4_t *>(a.bits) + (t * a.wide_groups + wg) * 64 + kk * src_step;
-    }
-    stage_bytes[p] = (uint32_t)(src_step * kWavesK * 16); // the host checks that a launch's stages span < 4 GiB
-    const uint32_t span = (uint32_t)(nstages - 1) * stage_bytes[p] + kFragBytes;
-    // (every input is uniform; reading the address through the first lane tells the compiler so, which keeps the
-    // resource in scalar registers)
-    const uint64_t first = reinterpret_cast<uint64_t>(src + a.step_begin * src_step);
-    const uint64_t base = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first >> 32)) << 32) |
-                          (uint32_t)__builtin_amdgcn_readfirstlane((int)first);
-    rsrc[p] = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>(base), 0,
-                                                __builtin_amdgcn_readfirstlane((int)span), 0x00020000);
-    stage_bytes[p] = __builtin_amdgcn_readfirstlane((int)stage_bytes[p]);
-    soff[p] = 0;
-  }
-  typedef __attribute__((address_space(3))) void lds_void_t;
-  const int wave_lds = wave * kFragBytes;
-  // issues this wavefront's kCount copies of the next stage into the LDS buffer at byte offset `buf_bytes`
-  auto copy_next = [&](int buf_bytes, auto count_c) __attribute__((always_inline)) {
-    constexpr int kCount = decltype(count_c)::value;
-#pragma unroll
-    for (int p = 0; p < kCount; ++p) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rsrc[p], (lds_void_t *)(smem + (wave_lds + buf_bytes) + p * kWaves * kFragBytes), 16, lane_bytes, soff[p], 0,
-          0);
-      soff[p] += stage_bytes[p];
-    }
-  };
-  // waits until at most `steps` stages of this wavefront's copies (kCount each) are in flight
-  auto wait_copies = [&](auto steps, auto count_c) __attribute__((always_inline)) {
-    NBLA_WAIT_VMCNT(decltype(steps)::value * decltype(count_c)::value);
-  };
-
   i32x16_t acc[kDigits][MF][NF];
 #pragma unroll
   for (int d = 0; d < kDigits; ++d)
@@ -291,15 +493,6 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
         }
     }
   };
-  // Software pipeline.  One barrier per k step, in the middle of it.  A wavefront issues in order and an MFMA keeps
-  // the matrix pipe busy for 32 cycles, so each half step is laid out by hand: the MFMAs of the first column
-  // fragment go first, the LDS reads of the next k tile (and the copies of a later k step) are issued in their
-  // shadow, and the remaining MFMAs cover the latency.  sched_barrier pins that order.
-  // Everything that is not an MFMA is kept short, because a wavefront cannot feed the matrix pipe while it works
-  // through scalar and address instructions: the copies are bounds-checked buffer loads whose addresses advance by
-  // one scalar add each; the number of copies a wavefront issues per stage (kPerWave, or one more for the first
-  // kExtra wavefronts) is a compile-time constant of its copy of the loop; the ring position is kept as three byte
-  // offsets that rotate; the loop counter is 32 bits wide.
   typedef std::integral_constant<int, 0> J0;
   typedef std::integral_constant<int, 1> J1;
   typedef std::integral_constant<int, NF> JN;
@@ -308,57 +501,145 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
   // A wavefront whose columns all lie past the end of the operand (last tile of a row of tiles) only takes part in
   // the copies and barriers: the matrix pipe of its SIMD is left to the other wavefront.
   const bool idle = a.n_begin + bn * BN + wn * NF * 32 >= a.n_end;
-  auto run = [&](auto count_c) __attribute__((always_inline)) {
-#pragma unroll
-    for (int d = 0; d < kDepth; ++d)
-      copy_next(d * kStageBytes, count_c);
-    wait_copies(std::integral_constant<int, kPrologueWait>(), count_c);
-    NBLA_BARRIER();
-    read_words(0, 0, w0);
-    read_a(0, 0, af0);
-    // byte offsets of the LDS buffers of step ks (`cur`), of step ks-1 = that of step ks+kDepth (`prev`)
-    int cur = 0, prev = (kStages - 1) * kStageBytes;
-    if (idle) {
+  if constexpr (kUnfold) {
+    unfold_main_loop<BM, BN, kWavesM, kWavesN, kWavesK, kStageBytes, kStepBytes, kABytes>(
+        a, smem, bm, bn, wave, lane, idle, [&](int buf_bytes) __attribute__((always_inline)) {
+          read_a(buf_bytes, 0, af0);
+          read_words(buf_bytes, 0, w0);
+          read_a(buf_bytes, 1, af1);
+          read_words(buf_bytes, 1, w1);
+          mma(af0, w0, J0(), JN());
+          mma(af1, w1, J0(), JN());
+        });
+  } else {
+    // Sources of this wavefront's copies.  Slot p of wavefront w copies chunk p * kWaves + w of every stage; the chunk is
+    // described by a buffer resource that starts at the chunk's bytes in the first stage of this launch and ends with
+    // its bytes in the last one, and by a scalar byte offset that advances by one stage per copy (the lane adds its own
+    // 16 bytes).  The hardware range check (it covers the scalar offset too) turns a copy past the end (the copies run kDepth stages ahead of the last multiplication) into
+    // zeros in LDS: no address is clamped in the loop.  Row blocks / wide groups past the end of the operand are
+    // clamped here: their products land in rows / columns that are not stored.
+    constexpr int kSlots = kPerWave + (kExtra ? 1 : 0);
+    const int nstages = (int)((a.step_end - a.step_begin) / kWavesK);
+    __amdgpu_buffer_rsrc_t rsrc[kSlots];
+    uint32_t stage_bytes[kSlots]; // advance per stage
+    uint32_t soff[kSlots];        // offset of the next stage inside the resource
+    const uint32_t lane_bytes = lane * 16;
+  #pragma unroll
+    for (int p = 0; p < kSlots; ++p) {
+      const int cs = p * kWaves + wave;                 // chunk of the stage
+      const int kk = (cs / kStepChunks) % kWavesK;      // k step inside the stage
+      const int c = cs - (cs / kStepChunks) * kStepChunks;
+      const uint4_t *src;
+      int64_t src_step; // advance per k step, in uint4
+      if (c < kAFrags) {
+        const int seg = c / kSegFrags, rem = c - seg * kSegFrags; // rem = (k tile of the step, digit in use)
+        const int t = rem / kUsed, d = kFirst + rem - t * kUsed;
+        int64_t rb = bm * kASegs + seg;
+        if (rb >= a.row_blocks)
+          rb = a.row_blocks - 1;
+        src_step = kSrcSegFrags * 64;
+        src = a.xd + (rb * a.x_k_tiles * kDigits + t * kDigits + d) * 64 + kk * src_step;
+      } else {
+        // packed words: chunk = (k tile of the step, wide group of the tile)
+        const int cb = c - kAFrags;
+        const int t = cb / (BN / kWideGroup);
+        int64_t wg = a.n_begin / kWideGroup + bn * (BN / kWideGroup) + (cb - t * (BN / kWideGroup));
+        if (wg >= a.wide_groups)
+          wg = a.wide_groups - 1;
+        src_step = 2 * a.wide_groups * 64;
+        src = reinterpret_cast<const uint4_t *>(a.bits) + (t * a.wide_groups + wg) * 64 + kk * src_step;
+      }
+      stage_bytes[p] = (uint32_t)(src_step * kWavesK * 16); // the host checks that a launch's stages span < 4 GiB
+      const uint32_t span = (uint32_t)(nstages - 1) * stage_bytes[p] + kFragBytes;
+      // (every input is uniform; reading the address through the first lane tells the compiler so, which keeps the
+      // resource in scalar registers)
+      const uint64_t first = reinterpret_cast<uint64_t>(src + a.step_begin * src_step);
+      const uint64_t base = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first >> 32)) << 32) |
+                            (uint32_t)__builtin_amdgcn_readfirstlane((int)first);
+      rsrc[p] = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>(base), 0,
+                                                  __builtin_amdgcn_readfirstlane((int)span), 0x00020000);
+      stage_bytes[p] = __builtin_amdgcn_readfirstlane((int)stage_bytes[p]);
+      soff[p] = 0;
+    }
+    typedef __attribute__((address_space(3))) void lds_void_t;
+    const int wave_lds = wave * kFragBytes;
+    // issues this wavefront's kCount copies of the next stage into the LDS buffer at byte offset `buf_bytes`
+    auto copy_next = [&](int buf_bytes, auto count_c) __attribute__((always_inline)) {
+      constexpr int kCount = decltype(count_c)::value;
+  #pragma unroll
+      for (int p = 0; p < kCount; ++p) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rsrc[p], (lds_void_t *)(smem + (wave_lds + buf_bytes) + p * kWaves * kFragBytes), 16, lane_bytes, soff[p], 0,
+            0);
+        soff[p] += stage_bytes[p];
+      }
+    };
+    // waits until at most `steps` stages of this wavefront's copies (kCount each) are in flight
+    auto wait_copies = [&](auto steps, auto count_c) __attribute__((always_inline)) {
+      NBLA_WAIT_VMCNT(decltype(steps)::value * decltype(count_c)::value);
+    };
+
+    // Software pipeline.  One barrier per k step, in the middle of it.  A wavefront issues in order and an MFMA keeps
+    // the matrix pipe busy for 32 cycles, so each half step is laid out by hand: the MFMAs of the first column
+    // fragment go first, the LDS reads of the next k tile (and the copies of a later k step) are issued in their
+    // shadow, and the remaining MFMAs cover the latency.  sched_barrier pins that order.
+    // Everything that is not an MFMA is kept short, because a wavefront cannot feed the matrix pipe while it works
+    // through scalar and address instructions: the copies are bounds-checked buffer loads whose addresses advance by
+    // one scalar add each; the number of copies a wavefront issues per stage (kPerWave, or one more for the first
+    // kExtra wavefronts) is a compile-time constant of its copy of the loop; the ring position is kept as three byte
+    // offsets that rotate; the loop counter is 32 bits wide.
+    auto run = [&](auto count_c) __attribute__((always_inline)) {
+  #pragma unroll
+      for (int d = 0; d < kDepth; ++d)
+        copy_next(d * kStageBytes, count_c);
+      wait_copies(std::integral_constant<int, kPrologueWait>(), count_c);
+      NBLA_BARRIER();
+      read_words(0, 0, w0);
+      read_a(0, 0, af0);
+      // byte offsets of the LDS buffers of step ks (`cur`), of step ks-1 = that of step ks+kDepth (`prev`)
+      int cur = 0, prev = (kStages - 1) * kStageBytes;
+      if (idle) {
+        for (int left = nstages; left > 0; --left) {
+          wait_copies(std::integral_constant<int, kLoopWait>(), count_c);
+          NBLA_BARRIER();
+          copy_next(prev, count_c);
+          prev = cur;
+          cur = (cur + kStageBytes == kStages * kStageBytes) ? 0 : cur + kStageBytes;
+        }
+        return;
+      }
       for (int left = nstages; left > 0; --left) {
+        const int next = (cur + kStageBytes == kStages * kStageBytes) ? 0 : cur + kStageBytes;
+        // tile 0 runs; tile 1 is fetched
+        mma(af0, w0, J0(), J1());
+        __builtin_amdgcn_sched_barrier(0);
+        read_a(cur, 1, af1);
+        read_words(cur, 1, w1);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(af0, w0, J1(), JN());
+        __builtin_amdgcn_sched_barrier(0);
+        // step ks+1 has landed: the copies issued so far reach step ks+kDepth-1, so at most the kDepth-2 (= kLoopWait)
+        // steps behind ks+1 may still be in flight; every wavefront is done with the buffer of step ks-1
         wait_copies(std::integral_constant<int, kLoopWait>(), count_c);
         NBLA_BARRIER();
+        // tile 1 runs; the copy of step ks+kDepth is issued; tile 0 of step ks+1 is fetched
+        mma(af1, w1, J0(), J1());
+        __builtin_amdgcn_sched_barrier(0);
         copy_next(prev, count_c);
+        read_words(next, 0, w0);
+        read_a(next, 0, af0);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(af1, w1, J1(), JN());
+        __builtin_amdgcn_sched_barrier(0);
         prev = cur;
-        cur = (cur + kStageBytes == kStages * kStageBytes) ? 0 : cur + kStageBytes;
+        cur = next;
       }
-      return;
-    }
-    for (int left = nstages; left > 0; --left) {
-      const int next = (cur + kStageBytes == kStages * kStageBytes) ? 0 : cur + kStageBytes;
-      // tile 0 runs; tile 1 is fetched
-      mma(af0, w0, J0(), J1());
-      __builtin_amdgcn_sched_barrier(0);
-      read_a(cur, 1, af1);
-      read_words(cur, 1, w1);
-      __builtin_amdgcn_sched_barrier(0);
-      mma(af0, w0, J1(), JN());
-      __builtin_amdgcn_sched_barrier(0);
-      // step ks+1 has landed: the copies issued so far reach step ks+kDepth-1, so at most the kDepth-2 (= kLoopWait)
-      // steps behind ks+1 may still be in flight; every wavefront is done with the buffer of step ks-1
-      wait_copies(std::integral_constant<int, kLoopWait>(), count_c);
-      NBLA_BARRIER();
-      // tile 1 runs; the copy of step ks+kDepth is issued; tile 0 of step ks+1 is fetched
-      mma(af1, w1, J0(), J1());
-      __builtin_amdgcn_sched_barrier(0);
-      copy_next(prev, count_c);
-      read_words(next, 0, w0);
-      read_a(next, 0, af0);
-      __builtin_amdgcn_sched_barrier(0);
-      mma(af1, w1, J1(), JN());
-      __builtin_amdgcn_sched_barrier(0);
-      prev = cur;
-      cur = next;
-    }
-  };
-  if (kExtra && wave < kExtra)
-    run(std::integral_constant<int, kPerWave + 1>());
-  else
-    run(std::integral_constant<int, kPerWave>());
+    };
+    if (kExtra && wave < kExtra)
+      run(std::integral_constant<int, kPerWave + 1>());
+    else
+      run(std::integral_constant<int, kPerWave>());
+  }
   NBLA_WAIT_VMCNT(0);
 
   if (kWavesK > 1) {
@@ -494,8 +775,17 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
       const int64_t m = bm * BM + (wm * MF + i) * 32 + col_in_frag;
       if (m >= a.M)
         continue;
-      const long long sum = a.use_sums ? a.sums[m] : 0;
-      const int s_hi = (int)(sum >> 16), s_lo = (int)(sum & 0xffff), sh = plain_shift(a.shift[m]);
+      long long sum;
+      int sh;
+      if constexpr (kUnfold) { // the block's own rows, left in LDS by unfold_main_loop
+        constexpr int kMetaOff = unfold_meta_off(BM, BN, kWavesM, kWavesN, kWavesK);
+        sum = reinterpret_cast<const long long *>(smem + kMetaOff)[m - bm * BM];
+        sh = reinterpret_cast<const int32_t *>(smem + kMetaOff + 384)[m - bm * BM];
+      } else {
+        sum = a.use_sums ? a.sums[m] : 0;
+        sh = plain_shift(a.shift[m]);
+      }
+      const int s_hi = (int)(sum >> 16), s_lo = (int)(sum & 0xffff);
       float *row = row_ptr(m);
 #pragma unroll
       for (int j = 0; j < NF; ++j) {
@@ -505,9 +795,17 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
           float al[4], bi[4], prev[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const int64_t n = (n0 + e < a.N) ? n0 + e : a.N - 1;
-            al[e] = use_alpha ? a.alpha[n] : 1.0f;
-            bi[e] = use_bias ? a.bias[n] : 0.0f;
+            if constexpr (kUnfold) { // left in LDS by unfold_main_loop (1 and 0 where there is no alpha / bias)
+              constexpr int kMetaOff = unfold_meta_off(BM, BN, kWavesM, kWavesN, kWavesK);
+              const float *s_alpha = reinterpret_cast<const float *>(smem + kMetaOff + 512 + 64 * 16);
+              const int col = (int)(n0 + e - a.n_begin - bn * BN);
+              al[e] = s_alpha[col];
+              bi[e] = s_alpha[256 + col];
+            } else {
+              const int64_t n = (n0 + e < a.N) ? n0 + e : a.N - 1;
+              al[e] = use_alpha ? a.alpha[n] : 1.0f;
+              bi[e] = use_bias ? a.bias[n] : 0.0f;
+            }
           }
           float *p = row + n0 * a.n_stride;
           if (a.accumulate) {
@@ -549,6 +847,13 @@ __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN 
     gemm_bits_body<BM, BN, kWavesM, kWavesN, kWavesK, kSwap, 1>(a, smem);
   else
     gemm_bits_body<BM, BN, kWavesM, kWavesN, kWavesK, kSwap, kDigits>(a, smem);
+}
+
+// The convolution's product with the unfold fused in (unfold_main_loop): one block per 32 windows and 256 output
+// channels, eight wavefronts (four column pairs x two k groups).
+__global__ __launch_bounds__(512, 1) void gemm_bits_unfold_kernel(GemmBitsArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  gemm_bits_body<32, 256, 1, 4, 2, true, kDigits, true>(a, smem);
 }
 
 template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, bool kSwap>
@@ -681,6 +986,8 @@ int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alp
   a.blocks_m = a.blocks_n = 0;
   a.split_steps = 0;
   a.use_sums = 1;
+  a.ux = nullptr;
+  a.ugrp = 0;
   a.inner = inner;
   a.outer_stride = outer_stride;
   a.n_stride = n_stride;
@@ -697,6 +1004,72 @@ int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alp
     if (rc)
       return rc;
   }
+  return NBLA_HIP_OK;
+}
+
+// LDS of the unfolding product: two stage buffers (or the k groups' exchange), the rows' metadata, the column table
+static size_t unfold_lds_bytes(int64_t Kg) {
+  return (size_t)unfold_meta_off(32, 256, 1, 4, 2) + kUnfoldMetaBytes + (size_t)bits_packed_k_tiles(Kg) * kTileK * 16;
+}
+static_assert(kUnfoldSteps * 2 * 2 == 8, "the packed operand's k tiles come in multiples of eight: whole stages");
+
+bool gemm_bits_unfold_applies(const ConvGeom &g) {
+  // 32-bit offsets inside one sample's channel group and one output map, 16-bit tap displacements (as the stand-alone
+  // unfold kernel), one k chunk, and a column table that fits the LDS beside the stages
+  bool fits = g.Cg * g.in_sp_size < ((int64_t)1 << 31) && g.out_sp_size < ((int64_t)1 << 31) && g.Kg <= kChunkK &&
+              g.M < ((int64_t)1 << 31) - 64;
+  for (int i = 0; i < kMaxSpatial; ++i)
+    fits = fits && (int64_t)(g.k[i] - 1) * g.dil[i] < 65536;
+  return fits && g.k_size <= 64 && unfold_lds_bytes(g.Kg) <= 144 * 1024; // the taps of a row are a 64-bit mask
+}
+
+int launch_gemm_bits_unfold(const float *x, const ConvGeom &g, int64_t grp, const uint32_t *bits, const float *alpha,
+                            const float *bias, float *y, hipStream_t stream) {
+  if (!gemm_bits_unfold_applies(g))
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "the fused unfold product does not cover this geometry.");
+  if (!aligned16(bits))
+    return fail(NBLA_HIP_ERR_MEMORY, "GEMM operands must be 16-byte aligned.");
+  int rc = ensure_init();
+  if (rc)
+    return rc;
+  const size_t lds = unfold_lds_bytes(g.Kg);
+  static std::atomic<uint64_t> configured{0};
+  rc = allow_dynamic_lds(reinterpret_cast<const void *>(gemm_bits_unfold_kernel), 144 * 1024, configured,
+                         "hipFuncSetAttribute(gemm_bits_unfold LDS size)");
+  if (rc)
+    return rc;
+  const int64_t hw = g.out_sp_size;
+  GemmBitsArgs a;
+  a.xd = nullptr;
+  a.sums = nullptr;
+  a.shift = nullptr;
+  a.bits = bits;
+  a.alpha = alpha;
+  a.bias = bias;
+  a.y = y;
+  a.M = g.M;
+  a.N = g.Og;
+  a.n_begin = 0;
+  a.n_end = g.Og;
+  a.row_blocks = split_row_blocks(g.M);
+  a.x_k_tiles = bits_packed_k_tiles(g.Kg);
+  a.wide_groups = bits_wide_groups(g.Og);
+  a.step_begin = 0;
+  a.step_end = a.x_k_tiles / 2;
+  a.blocks_m = a.row_blocks;
+  a.blocks_n = a.wide_groups;
+  a.inner = hw;
+  a.outer_stride = g.O * hw;
+  a.n_stride = hw;
+  a.accumulate = 0;
+  a.finish = 1;
+  a.split_steps = 0;
+  a.use_sums = 1;
+  a.ux = x;
+  a.ug = g;
+  a.ugrp = grp;
+  hipLaunchKernelGGL(gemm_bits_unfold_kernel, dim3((unsigned)(a.blocks_m * a.blocks_n)), dim3(512), lds, stream, a);
+  NBLA_HIP_LAUNCH_CHECK("gemm_bits_unfold");
   return NBLA_HIP_OK;
 }
 

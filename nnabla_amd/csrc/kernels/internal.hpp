@@ -18,6 +18,13 @@ int launch_gemm_bits(const void *xsplit, const uint32_t *bits, const float *alph
                      int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
                      bool swap_out, hipStream_t stream, bool accumulate = false, void *split_ws = nullptr,
                      size_t split_ws_bytes = 0);
+// The same product for a convolution with the unfold fused in: the rows are the unfolded windows of x (group `grp`),
+// converted to digits inside the kernel; y is [sample, O, output position].  gemm_bits_unfold_applies tells whether
+// the geometry is covered (otherwise: launch_im2col_digits + launch_gemm_bits).
+struct ConvGeom;
+bool gemm_bits_unfold_applies(const ConvGeom &g);
+int launch_gemm_bits_unfold(const float *x, const ConvGeom &g, int64_t grp, const uint32_t *bits, const float *alpha,
+                            const float *bias, float *y, hipStream_t stream);
 // Scratch that lets launch_gemm_bits spread the contraction of a very small output (M <= 64 or so) over the CUs.
 size_t gemm_bits_split_bytes(int64_t M, int64_t K, int64_t N);
 

@@ -27,6 +27,14 @@ CASES = [
     ((4, 8, 16, 16), (16, 8, 3, 3), (1, 1), (1, 1), (1, 1), 1),        # the reference tests' own size
     ((2, 3, 4, 8, 16, 16), (16, 8, 3, 3), (1, 1), (2, 2), (1, 1), 1),  # base_axis = 3: leading axes fold into outer
     ((3, 64, 14, 14), (96, 32, 3, 3), (1, 1), (1, 1), (1, 1), 2),
+    # more than 256 output channels (two column groups of the fused unfold product, the second partly empty)
+    ((2, 16, 9, 9), (300, 16, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    # images of four positions: a block of 32 windows spans eight samples
+    ((40, 5, 2, 2), (7, 5, 2, 2), (1, 1), (1, 1), (1, 1), 1),
+    # 125 kernel taps: above the 64 the fused product's tap mask holds, so the stand-alone unfold runs
+    ((1, 2, 6, 6, 6), (4, 2, 5, 5, 5), (2, 2, 2), (1, 1, 1), (1, 1, 1), 1),
+    # 7 x 7 kernel, stride 2 (49 taps: the upper half of the tap mask)
+    ((2, 3, 20, 20), (8, 3, 7, 7), (3, 3), (2, 2), (1, 1), 1),
 ]
 
 
@@ -71,6 +79,26 @@ def test_convolution_quantize_zero_to_with_zero_weights(dev, q0):
     ref_y, _ = oracle.binary_connect_convolution(x, W, None, (1, 1), (1, 1), (1, 1), 2, q0)
     y, _ = kernels.binary_connect_convolution(_dev(x, dev), _dev(W, dev), None, (1, 1), (1, 1), (1, 1), 2, q0)
     assert max_rel_err(to_np(y), ref_y) <= TIGHT * 4
+
+
+def test_window_with_a_non_finite_value(dev):
+    """An Inf or NaN in x: every output whose window holds it is non-finite in the reference (Inf - Inf and 0 * Inf
+    give NaN, convolution.cpp's gemm); here the digit form gives NaN for all output channels of such a window.  All
+    other outputs are unaffected."""
+    rng = np.random.RandomState(5)
+    x = rng.randn(2, 8, 9, 9).astype(np.float32)
+    W = (rng.randn(6, 8, 3, 3) * 0.05).astype(np.float32)
+    clean, _, _ = kernels.binary_weight_convolution(_dev(x, dev), _dev(W, dev), None, (1, 1), (1, 1), (1, 1), 1)
+    x[1, 3, 4, 5] = np.inf
+    x[0, 0, 0, 0] = np.nan
+    y, _, _ = kernels.binary_weight_convolution(_dev(x, dev), _dev(W, dev), None, (1, 1), (1, 1), (1, 1), 1)
+    y, clean = to_np(y), to_np(clean)
+    hit = np.zeros((2, 9, 9), bool)
+    hit[1, 3:6, 4:7] = True
+    hit[0, 0:2, 0:2] = True
+    for o in range(6):
+        assert not np.isfinite(y[:, o][hit]).any()
+        assert bits_equal(y[:, o][~hit], clean[:, o][~hit])
 
 
 def test_config4_resnet_stage(dev):
