@@ -5,6 +5,8 @@
 #include "common.hpp"
 #include "quantize_common.hpp"
 
+#include <atomic>
+
 #include <cmath>
 #include <cstring>
 #include <mutex>
@@ -867,77 +869,9 @@ namespace {
 
 enum RecorderMode { kMinMaxMinMax = 0, kAbsMax = 1, kMinMaxMva = 2, kMaxMax = 3, kMaxMva = 4, kRecorderModes = 5 };
 
-template <bool kAbs, bool kCopy>
-__global__ __launch_bounds__(kRedBlock) void record_scan(const float *__restrict__ x, float *__restrict__ y,
-                                                         MinMaxPartial *__restrict__ partial, size_t n4, size_t size) {
-  Extrema ex;
-  ex.init();
-  const size_t per = (n4 + gridDim.x - 1) / gridDim.x;
-  const size_t begin = (size_t)blockIdx.x * per, end = (begin + per < n4) ? begin + per : n4;
-  size_t i = begin + threadIdx.x;
-  for (; i + 3 * kRedBlock < end; i += 4 * kRedBlock) {
-    float4_t v[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      v[j] = load4(x + 4 * (i + j * kRedBlock));
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      if (kCopy)
-        store4(y + 4 * (i + j * kRedBlock), v[j]);
-      if (kAbs)
-        v[j] = float4_t{__builtin_fabsf(v[j].x), __builtin_fabsf(v[j].y), __builtin_fabsf(v[j].z),
-                        __builtin_fabsf(v[j].w)};
-      ex.take4(v[j], (uint32_t)(4 * (i + j * kRedBlock)));
-    }
-  }
-  for (; i < end; i += kRedBlock) {
-    float4_t v = load4(x + 4 * i);
-    if (kCopy)
-      store4(y + 4 * i, v);
-    if (kAbs)
-      v = float4_t{__builtin_fabsf(v.x), __builtin_fabsf(v.y), __builtin_fabsf(v.z), __builtin_fabsf(v.w)};
-    ex.take4(v, (uint32_t)(4 * i));
-  }
-  if (blockIdx.x == gridDim.x - 1) { // the elements past the last float4 (all of them when n4 is 0), highest indices
-    for (size_t t = 4 * n4 + threadIdx.x; t < size; t += kRedBlock) {
-      const float v = x[t];
-      if (kCopy)
-        y[t] = v;
-      ex.take(kAbs ? __builtin_fabsf(v) : v, (uint32_t)t);
-    }
-  }
-  ex.wave_reduce();
-  __shared__ MinMaxPartial s_part[kRedBlock / 64];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  if (lane == 0)
-    s_part[wave] = ex.pack();
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    for (int w = 1; w < kRedBlock / 64; ++w)
-      ex.merge(s_part[w].vmin, s_part[w].vmax, s_part[w].zidx, s_part[w].zsign);
-    partial[blockIdx.x] = ex.pack();
-  }
-}
-
-__global__ __launch_bounds__(64) void record_update(const MinMaxPartial *__restrict__ partial, int nchunks,
-                                                    float *__restrict__ m, float *__restrict__ M, int mode,
-                                                    float decay, float one_minus_decay) {
-  Extrema ex;
-  ex.init();
-  // sixteen independent 16-byte loads in flight per lane: one round trip for up to 1024 partials
-  const float4_t *pp = reinterpret_cast<const float4_t *>(partial);
-  for (int c = threadIdx.x; c < nchunks; c += 1024) {
-    float4_t q[16];
-#pragma unroll
-    for (int j = 0; j < 16; ++j)
-      q[j] = (c + 64 * j < nchunks) ? pp[c + 64 * j] : float4_t{1e+8f, -1e+8f, __uint_as_float(0xffffffffu), 0.0f};
-#pragma unroll
-    for (int j = 0; j < 16; ++j)
-      ex.merge(q[j].x, q[j].y, __float_as_uint(q[j].z), __float_as_uint(q[j].w));
-  }
-  ex.wave_reduce();
-  if (threadIdx.x != 0)
-    return;
+// The statistic's update from the extrema of the whole array: what runs after the scan.
+__device__ __forceinline__ void record_apply(const Extrema &ex, float *__restrict__ m, float *__restrict__ M, int mode,
+                                             float decay, float one_minus_decay) {
   const float mb = ex.min_value(), Mb = ex.max_value();
   if (mode == kMinMaxMinMax) {
     const float lo = *m, hi = *M;
@@ -956,6 +890,139 @@ __global__ __launch_bounds__(64) void record_update(const MinMaxPartial *__restr
     const float c = decay * *M, d = one_minus_decay * Mb;
     *M = c + d;
   }
+}
+
+// Counters that tell a block whether it is the last of its launch to finish; one set per launch in flight (the host
+// hands the slots out in turn).  Two levels, because a counter that every block of a grid updates is a serial chain
+// of device-wide atomics (about 15 ns each): block b draws a ticket from counter b % kTicketGroups, and the block
+// that draws the last ticket of a counter draws one from the set's final counter.  Zero when the module is loaded;
+// the last block puts the zeros back.
+// (Counters sit 256 bytes apart: atomics on one cache line queue up behind each other whatever their address.)
+constexpr int kRecorderTickets = 16, kTicketGroups = 32, kTicketStride = 64;
+__device__ unsigned g_recorder_tickets[kRecorderTickets][(kTicketGroups + 1) * kTicketStride];
+
+// One launch scans (and copies) the array and updates the statistic.  Every block publishes its extrema with
+// device-scope atomic stores, waits until the memory system has acknowledged them (vmcnt(0)) and draws a ticket;
+// the block that draws the last one reads all the partial results back with atomic loads (they are complete: every
+// other block's stores were acknowledged before its ticket), merges them in block order and applies the update.
+// Only atomics carry the hand-over, so no cache is written back or invalidated.
+template <bool kAbs, bool kCopy>
+__global__ __launch_bounds__(kRedBlock) void record_scan(const float *__restrict__ x, float *__restrict__ y,
+                                                         MinMaxPartial *__restrict__ partial, size_t n4, size_t size,
+                                                         float *__restrict__ m, float *__restrict__ M, int mode,
+                                                         float decay, float one_minus_decay, int slot) {
+  Extrema ex;
+  ex.init();
+  const size_t per = (n4 + gridDim.x - 1) / gridDim.x;
+  const size_t begin = (size_t)blockIdx.x * per, end = (begin + per < n4) ? begin + per : n4;
+  size_t i = begin + threadIdx.x;
+  auto absolute = [](float4_t v) {
+    return float4_t{__builtin_fabsf(v.x), __builtin_fabsf(v.y), __builtin_fabsf(v.z), __builtin_fabsf(v.w)};
+  };
+  // four 16-byte loads per thread in flight while the previous four are consumed
+  if (i + 3 * kRedBlock < end) {
+    float4_t cur[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      cur[j] = load4(x + 4 * (i + j * kRedBlock));
+#pragma clang loop unroll(disable)
+    for (;;) {
+      const size_t nx = i + 4 * kRedBlock;
+      const bool more = nx + 3 * kRedBlock < end;
+      float4_t nxt[4];
+      if (more) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          nxt[j] = load4(x + 4 * (nx + j * kRedBlock));
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (kCopy)
+          store4(y + 4 * (i + j * kRedBlock), cur[j]);
+        ex.take4(kAbs ? absolute(cur[j]) : cur[j], (uint32_t)(4 * (i + j * kRedBlock)));
+      }
+      i = nx;
+      if (!more)
+        break;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        cur[j] = nxt[j];
+    }
+  }
+  for (; i < end; i += kRedBlock) {
+    float4_t v = load4(x + 4 * i);
+    if (kCopy)
+      store4(y + 4 * i, v);
+    ex.take4(kAbs ? absolute(v) : v, (uint32_t)(4 * i));
+  }
+  if (blockIdx.x == gridDim.x - 1) { // the elements past the last float4 (all of them when n4 is 0), highest indices
+    for (size_t t = 4 * n4 + threadIdx.x; t < size; t += kRedBlock) {
+      const float v = x[t];
+      if (kCopy)
+        y[t] = v;
+      ex.take(kAbs ? __builtin_fabsf(v) : v, (uint32_t)t);
+    }
+  }
+  ex.wave_reduce();
+  __shared__ MinMaxPartial s_part[kRedBlock / 64];
+  __shared__ unsigned s_ticket;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0)
+    s_part[wave] = ex.pack();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kRedBlock / 64; ++w)
+      ex.merge(s_part[w].vmin, s_part[w].vmax, s_part[w].zidx, s_part[w].zsign);
+    unsigned long long *dst = reinterpret_cast<unsigned long long *>(&partial[blockIdx.x]);
+    const unsigned long long lo = (unsigned long long)__float_as_uint(ex.vmin) |
+                                  ((unsigned long long)__float_as_uint(ex.vmax) << 32);
+    const unsigned long long hi = (unsigned long long)ex.zidx | ((unsigned long long)ex.zsign << 32);
+    __hip_atomic_store(dst, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(dst + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): the two stores have been performed
+    asm volatile("" ::: "memory");
+    // 1 = this block is the last of the launch
+    unsigned *tickets = g_recorder_tickets[slot];
+    const unsigned groups = gridDim.x < (unsigned)kTicketGroups ? gridDim.x : (unsigned)kTicketGroups;
+    const unsigned group = blockIdx.x % groups, members = (gridDim.x - group + groups - 1) / groups;
+    unsigned last = 0u;
+    if (atomicAdd(&tickets[group * kTicketStride], 1u) == members - 1u)
+      last = atomicAdd(&tickets[kTicketGroups * kTicketStride], 1u) == groups - 1u ? 1u : 0u;
+    s_ticket = last;
+  }
+  __syncthreads();
+  if (s_ticket == 0u)
+    return;
+  // the last block: every thread takes the partial results c = thread, thread + 256, ... four at a time (eight loads
+  // in flight: one round trip for up to 1024 blocks); the merge does not depend on the order
+  Extrema all;
+  all.init();
+  for (unsigned c0 = threadIdx.x; c0 < gridDim.x; c0 += 4 * kRedBlock) {
+    unsigned long long lo[4], hi[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const unsigned c = c0 + j * kRedBlock;
+      const unsigned long long *src = reinterpret_cast<const unsigned long long *>(&partial[c < gridDim.x ? c : c0]);
+      lo[j] = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      hi[j] = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      all.merge(__uint_as_float((uint32_t)lo[j]), __uint_as_float((uint32_t)(lo[j] >> 32)), (uint32_t)hi[j],
+                (uint32_t)(hi[j] >> 32));
+  }
+  all.wave_reduce();
+  if (lane == 0)
+    s_part[wave] = all.pack();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kRedBlock / 64; ++w)
+      all.merge(s_part[w].vmin, s_part[w].vmax, s_part[w].zidx, s_part[w].zsign);
+    record_apply(all, m, M, mode, decay, one_minus_decay);
+  }
+  if (threadIdx.x <= kTicketGroups)
+    __hip_atomic_store(&g_recorder_tickets[slot][threadIdx.x * kTicketStride], 0u, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
 }
 
 } // namespace
@@ -997,23 +1064,27 @@ int nbla_hip_range_recorder_f32(const float *x, float *y, size_t size, float *m,
   if (blocks < 1)
     blocks = 1;
   const dim3 grid((unsigned)blocks), block(kRedBlock);
-  if (mode == kAbsMax) {
-    if (copy)
-      hipLaunchKernelGGL((record_scan<true, true>), grid, block, 0, stream, x, y, partial, n4, size);
-    else
-      hipLaunchKernelGGL((record_scan<true, false>), grid, block, 0, stream, x, y, partial, n4, size);
-  } else {
-    if (copy)
-      hipLaunchKernelGGL((record_scan<false, true>), grid, block, 0, stream, x, y, partial, n4, size);
-    else
-      hipLaunchKernelGGL((record_scan<false, false>), grid, block, 0, stream, x, y, partial, n4, size);
-  }
-  NBLA_HIP_LAUNCH_CHECK("range recorder scan");
   // `decay * m` and `(1 - decay) * mb` of the reference are MulScalar functions: each takes the Python float (a
   // double) and rounds it to fp32 once
-  hipLaunchKernelGGL(record_update, dim3(1), dim3(64), 0, stream, partial, (int)blocks, m, M, mode, (float)decay,
-                     (float)(1.0 - decay));
-  NBLA_HIP_LAUNCH_CHECK("range recorder update");
+  const float dec = (float)decay, omd = (float)(1.0 - decay);
+  static std::atomic<unsigned> next_slot{0};
+  const int slot = (int)(next_slot.fetch_add(1u) % (unsigned)kRecorderTickets);
+  if (mode == kAbsMax) {
+    if (copy)
+      hipLaunchKernelGGL((record_scan<true, true>), grid, block, 0, stream, x, y, partial, n4, size, m, M, mode, dec,
+                         omd, slot);
+    else
+      hipLaunchKernelGGL((record_scan<true, false>), grid, block, 0, stream, x, y, partial, n4, size, m, M, mode, dec,
+                         omd, slot);
+  } else {
+    if (copy)
+      hipLaunchKernelGGL((record_scan<false, true>), grid, block, 0, stream, x, y, partial, n4, size, m, M, mode, dec,
+                         omd, slot);
+    else
+      hipLaunchKernelGGL((record_scan<false, false>), grid, block, 0, stream, x, y, partial, n4, size, m, M, mode, dec,
+                         omd, slot);
+  }
+  NBLA_HIP_LAUNCH_CHECK("range recorder scan");
   return NBLA_HIP_OK;
 }
 

@@ -354,19 +354,33 @@ __global__ __launch_bounds__(kHistBlock) void prune_histogram(const float *__res
   __shared__ uint32_t scratch[kHistBlock / 64 + 1];
   const SelectPass sp = select_begin(h, st, pass);
   auto count = [&](float v) { select_count(h, sp, __float_as_uint(v) & 0x7fffffffu); };
-  // four loads in flight per thread before the counters are touched
+  // four 16-byte loads per thread in flight while the previous four are counted
   const int64_t tiles = (n4 + kHistBlock * 4 - 1) / (kHistBlock * 4);
-  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+  auto fetch = [&](int64_t tile, float4_t (&v)[4]) __attribute__((always_inline)) {
     const int64_t base = tile * (kHistBlock * 4) + threadIdx.x;
-    float4_t v[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       if (base + j * kHistBlock < n4)
         v[j] = *reinterpret_cast<const float4_t *>(x + 4 * (base + j * kHistBlock));
+  };
+  if ((int64_t)blockIdx.x < tiles) {
+    float4_t cur[4];
+    fetch(blockIdx.x, cur);
+#pragma clang loop unroll(disable)
+    for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+      const int64_t next = tile + gridDim.x;
+      float4_t nxt[4];
+      if (next < tiles)
+        fetch(next, nxt);
+      const int64_t base = tile * (kHistBlock * 4) + threadIdx.x;
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (base + j * kHistBlock < n4)
-        count(v[j].x), count(v[j].y), count(v[j].z), count(v[j].w);
+      for (int j = 0; j < 4; ++j)
+        if (base + j * kHistBlock < n4)
+          count(cur[j].x), count(cur[j].y), count(cur[j].z), count(cur[j].w);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        cur[j] = nxt[j];
+    }
   }
   if (blockIdx.x == 0) {
     const int64_t i = 4 * n4 + threadIdx.x;
