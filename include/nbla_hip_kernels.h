@@ -561,6 +561,22 @@ int nbla_hip_fill(void *dst, int dtype, size_t size, float value, void *stream);
 int nbla_hip_cast(const void *src, int src_dtype, void *dst, int dst_dtype,
                   size_t size, void *stream);
 
+/* y = x0 + x1 (same shapes).  Replaces Add2<float>::forward_impl,
+ * src/nbla/function/generic/add2.cpp:39-47. */
+int nbla_hip_add2_f32(const float *x0, const float *x1, float *y, size_t size,
+                      void *stream);
+/* dx (+)= dy.  Replaces add2_backward_cpu,
+ * src/nbla/function/generic/add2.cpp:48-77. */
+int nbla_hip_add2_backward_f32(const float *dy, float *dx, size_t size,
+                               int accum, void *stream);
+/* dst[r * dst_stride + i] (+)= src[r * src_stride + i], r < rows, i < len:
+ * one input's share of Concatenate<float>::forward_impl / backward_impl,
+ * src/nbla/function/generic/concatenate.cpp:62-104 (rows = outer_size_, len =
+ * the input's inner size, the other stride = inner_total_size_). */
+int nbla_hip_copy_rows_f32(const float *src, int64_t src_stride, float *dst,
+                           int64_t dst_stride, int64_t rows, int64_t len,
+                           int accum, void *stream);
+
 /* y = max(0, x).  Replaces ReLU<float>::forward_impl,
  * src/nbla/function/generic/relu.cpp (std::max(T(0), x)). */
 int nbla_hip_relu_f32(const float *x, float *y, size_t size, void *stream);

@@ -2,11 +2,13 @@
 // status codes plus a thread-local message instead of C++ exceptions.
 #include <nbla/array/cpu_array.hpp>
 #include <nbla/backend_registry.hpp>
+#include <nbla/function/add2.hpp>
 #include <nbla/function/affine.hpp>
 #include <nbla/function/binary_connect_affine.hpp>
 #include <nbla/function/binary_connect_convolution.hpp>
 #include <nbla/function/binary_weight_affine.hpp>
 #include <nbla/function/binary_weight_convolution.hpp>
+#include <nbla/function/concatenate.hpp>
 #include <nbla/function/convolution.hpp>
 #include <nbla/function/dequantize_linear.hpp>
 #include <nbla/function/fixed_point_quantize.hpp>
@@ -132,6 +134,14 @@ FunctionPtr create_by_name(const string &name, const Context &ctx, const int64_t
   if (name == "ReLU") {
     need(1, 0);
     return create_ReLU(ctx, ia[0] != 0);
+  }
+  if (name == "Add2") {
+    need(1, 0);
+    return create_Add2(ctx, ia[0] != 0);
+  }
+  if (name == "Concatenate") {
+    need(1, 0);
+    return create_Concatenate(ctx, (int)ia[0]);
   }
   if (name == "Convolution") {
     need(4, 0);

@@ -1,6 +1,7 @@
 // forward_impl of the "hip:float" Function classes: fetch device pointers through the Variable interface, obtain
 // scratch from the backend's caching allocator, call the kernel library.
 #include <nbla/hip/common.hpp>
+#include <nbla/hip/function/arithmetic.hpp>
 #include <nbla/hip/function/binary.hpp>
 #include <nbla/hip/function/inq.hpp>
 #include <nbla/hip/function/quantize.hpp>
@@ -625,6 +626,64 @@ template <typename T> void ReLUHip<T>::forward_impl(const Variables &inputs, con
   NBLA_HIP_CALL(nbla_hip_relu_f32(x, y, (size_t)inputs[0]->size(), nullptr));
 }
 
+// ------------------------------------------------------------ Add2 and Concatenate
+// add2.cpp:39-47
+template <typename T> void Add2Hip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  const T *x0 = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const T *x1 = inputs[1]->get_data_pointer<T>(this->ctx_);
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  NBLA_HIP_CALL(nbla_hip_add2_f32(x0, x1, y, (size_t)inputs[0]->size(), nullptr));
+}
+
+// add2.cpp:59-77
+template <typename T>
+void Add2Hip<T>::backward_impl(const Variables &inputs, const Variables &outputs, const vector<bool> &propagate_down,
+                               const vector<bool> &accum) {
+  if (!(propagate_down[0] || propagate_down[1]))
+    return;
+  hip_set_device(this->ctx_);
+  const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
+  for (int i = 0; i < 2; ++i) {
+    if (!propagate_down[i])
+      continue;
+    T *dx = inputs[i]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[i]);
+    NBLA_HIP_CALL(nbla_hip_add2_backward_f32(dy, dx, (size_t)inputs[0]->size(), accum[i], nullptr));
+  }
+}
+
+// concatenate.cpp:62-76
+template <typename T> void ConcatenateHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->ctx_);
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  int64_t inner_offset = 0;
+  for (Variables::size_type c = 0; c < inputs.size(); ++c) {
+    const T *x = inputs[c]->get_data_pointer<T>(this->ctx_);
+    const int64_t inner_size = inputs[c]->size(this->axis_);
+    NBLA_HIP_CALL(nbla_hip_copy_rows_f32(x, inner_size, y + inner_offset, this->inner_total_size_, this->outer_size_,
+                                         inner_size, 0, nullptr));
+    inner_offset += inner_size;
+  }
+}
+
+// concatenate.cpp:78-104
+template <typename T>
+void ConcatenateHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                      const vector<bool> &propagate_down, const vector<bool> &accum) {
+  hip_set_device(this->ctx_);
+  const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
+  int64_t inner_offset = 0;
+  for (Variables::size_type c = 0; c < inputs.size(); ++c) {
+    const int64_t inner_size = inputs[c]->size(this->axis_);
+    if (propagate_down[c]) {
+      T *dx = inputs[c]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[c]);
+      NBLA_HIP_CALL(nbla_hip_copy_rows_f32(dy + inner_offset, this->inner_total_size_, dx, inner_size,
+                                           this->outer_size_, inner_size, accum[c], nullptr));
+    }
+    inner_offset += inner_size;
+  }
+}
+
 // ------------------------------------------- QuantizeLinear / DequantizeLinear / Prune
 namespace {
 vector<int64_t> shape64(const Variable *v) {
@@ -808,6 +867,8 @@ template class INQAffineHip<float, int>;
 template class INQConvolutionHip<float, int>;
 template class AffineHip<float>;
 template class ReLUHip<float>;
+template class Add2Hip<float>;
+template class ConcatenateHip<float>;
 template class ConvolutionHip<float>;
 template class QuantizeLinearHip<float>;
 template class DequantizeLinearHip<float>;

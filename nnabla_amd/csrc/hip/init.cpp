@@ -4,6 +4,7 @@
 #include <nbla/array_registry.hpp>
 #include <nbla/backend_registry.hpp>
 #include <nbla/hip/array.hpp>
+#include <nbla/hip/function/arithmetic.hpp>
 #include <nbla/hip/function/binary.hpp>
 #include <nbla/hip/function/inq.hpp>
 #include <nbla/hip/function/quantize.hpp>
@@ -66,6 +67,8 @@ void init_hip() {
                               int);
   NBLA_REGISTER_FUNCTION_IMPL(Affine, AffineHip<float>, "hip:float", int);
   NBLA_REGISTER_FUNCTION_IMPL(ReLU, ReLUHip<float>, "hip:float", bool);
+  NBLA_REGISTER_FUNCTION_IMPL(Add2, Add2Hip<float>, "hip:float", bool);
+  NBLA_REGISTER_FUNCTION_IMPL(Concatenate, ConcatenateHip<float>, "hip:float", int);
   NBLA_REGISTER_FUNCTION_IMPL(Convolution, ConvolutionHip<float>, "hip:float", int, const vector<int> &,
                               const vector<int> &, const vector<int> &, int, bool);
   NBLA_REGISTER_FUNCTION_IMPL(QuantizeLinear, QuantizeLinearHip<float>, "hip:float", const string &, bool, int);

@@ -47,6 +47,43 @@ __global__ __launch_bounds__(kBlk) void relu_kernel(const float *__restrict__ x,
   }
 }
 
+// y = x0 + x1, or dx (+)= dy when x1 is null (kAccum: dx already holds a gradient)
+template <bool kSum, bool kAccum>
+__global__ __launch_bounds__(kBlk) void add_kernel(const float *__restrict__ a, const float *__restrict__ b,
+                                                   float *__restrict__ y, size_t n4, size_t size, int vec) {
+  if (vec) {
+    for (size_t i = (size_t)blockIdx.x * kBlk + threadIdx.x; i < n4; i += (size_t)gridDim.x * kBlk) {
+      float4_t v = reinterpret_cast<const float4_t *>(a)[i];
+      if (kSum)
+        v += reinterpret_cast<const float4_t *>(b)[i];
+      if (kAccum)
+        v = reinterpret_cast<const float4_t *>(y)[i] + v;
+      reinterpret_cast<float4_t *>(y)[i] = v;
+    }
+  }
+  const size_t done = vec ? 4 * n4 : 0;
+  for (size_t i = done + (size_t)blockIdx.x * kBlk + threadIdx.x; i < size; i += (size_t)gridDim.x * kBlk) {
+    float v = a[i];
+    if (kSum)
+      v += b[i];
+    y[i] = kAccum ? y[i] + v : v;
+  }
+}
+
+// dst[r * dst_stride + i] (+)= src[r * src_stride + i] for r < rows, i < len: the copies of Concatenate
+template <bool kAccum>
+__global__ __launch_bounds__(kBlk) void rows_copy_kernel(const float *__restrict__ src, int64_t src_stride,
+                                                         float *__restrict__ dst, int64_t dst_stride, int64_t rows,
+                                                         int64_t len) {
+  const int64_t total = rows * len;
+  for (int64_t t = (int64_t)blockIdx.x * kBlk + threadIdx.x; t < total; t += (int64_t)gridDim.x * kBlk) {
+    const int64_t r = t / len, i = t - r * len;
+    const float v = src[r * src_stride + i];
+    float *d = dst + r * dst_stride + i;
+    *d = kAccum ? *d + v : v;
+  }
+}
+
 // nbla::dtypes codes (numpy compatible)
 enum { DT_BOOL = 0, DT_BYTE, DT_UBYTE, DT_SHORT, DT_USHORT, DT_INT, DT_UINT, DT_LONG, DT_ULONG, DT_LONGLONG,
        DT_ULONGLONG, DT_FLOAT, DT_DOUBLE };
@@ -219,6 +256,45 @@ int nbla_hip_cast(const void *src, int src_dtype, void *dst, int dst_dtype, size
   case DT_DOUBLE: return cast_from<double>(src, dst, dst_dtype, size, s);
   }
   return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "unsupported source dtype %d.", src_dtype);
+}
+
+int nbla_hip_add2_f32(const float *x0, const float *x1, float *y, size_t size, void *stream) {
+  if (size == 0)
+    return NBLA_HIP_OK;
+  const int vec = aligned16(x0) && aligned16(x1) && aligned16(y);
+  hipLaunchKernelGGL((add_kernel<true, false>), dim3(grid_for(vec ? size / 4 + 1 : size)), dim3(kBlk), 0,
+                     as_stream(stream), x0, x1, y, size / 4, size, vec);
+  NBLA_HIP_LAUNCH_CHECK("add2");
+  return NBLA_HIP_OK;
+}
+
+int nbla_hip_add2_backward_f32(const float *dy, float *dx, size_t size, int accum, void *stream) {
+  if (size == 0 || (dx == dy && !accum))
+    return NBLA_HIP_OK;
+  const int vec = aligned16(dy) && aligned16(dx);
+  const dim3 g(grid_for(vec ? size / 4 + 1 : size)), b(kBlk);
+  if (accum)
+    hipLaunchKernelGGL((add_kernel<false, true>), g, b, 0, as_stream(stream), dy, nullptr, dx, size / 4, size, vec);
+  else
+    hipLaunchKernelGGL((add_kernel<false, false>), g, b, 0, as_stream(stream), dy, nullptr, dx, size / 4, size, vec);
+  NBLA_HIP_LAUNCH_CHECK("add2 backward");
+  return NBLA_HIP_OK;
+}
+
+int nbla_hip_copy_rows_f32(const float *src, int64_t src_stride, float *dst, int64_t dst_stride, int64_t rows,
+                           int64_t len, int accum, void *stream) {
+  if (rows < 0 || len < 0 || src_stride < len || dst_stride < len)
+    return fail(NBLA_HIP_ERR_VALUE, "copy_rows: invalid sizes (rows=%lld, len=%lld, strides %lld / %lld).",
+                (long long)rows, (long long)len, (long long)src_stride, (long long)dst_stride);
+  if (rows == 0 || len == 0)
+    return NBLA_HIP_OK;
+  const dim3 g(grid_for((size_t)(rows * len))), b(kBlk);
+  if (accum)
+    hipLaunchKernelGGL(rows_copy_kernel<true>, g, b, 0, as_stream(stream), src, src_stride, dst, dst_stride, rows, len);
+  else
+    hipLaunchKernelGGL(rows_copy_kernel<false>, g, b, 0, as_stream(stream), src, src_stride, dst, dst_stride, rows, len);
+  NBLA_HIP_LAUNCH_CHECK("copy_rows");
+  return NBLA_HIP_OK;
 }
 
 int nbla_hip_relu_f32(const float *x, float *y, size_t size, void *stream) {

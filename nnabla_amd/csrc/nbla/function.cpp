@@ -1,10 +1,12 @@
 // Function protocol, the per-function registries and the process-wide random generator.
 #include <nbla/function.hpp>
+#include <nbla/function/add2.hpp>
 #include <nbla/function/affine.hpp>
 #include <nbla/function/binary_connect_affine.hpp>
 #include <nbla/function/binary_connect_convolution.hpp>
 #include <nbla/function/binary_weight_affine.hpp>
 #include <nbla/function/binary_weight_convolution.hpp>
+#include <nbla/function/concatenate.hpp>
 #include <nbla/function/convolution.hpp>
 #include <nbla/function/dequantize_linear.hpp>
 #include <nbla/function/fixed_point_quantize.hpp>
@@ -107,6 +109,8 @@ NBLA_REGISTER_FUNCTION_SOURCE(QuantizeLinear, const string &, bool, int);
 NBLA_REGISTER_FUNCTION_SOURCE(DequantizeLinear);
 NBLA_REGISTER_FUNCTION_SOURCE(Prune, float);
 NBLA_REGISTER_FUNCTION_SOURCE(Sink, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(Add2, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(Concatenate, int);
 
 // ----------------------------------------------------------------- RandomManager
 RandomManager::RandomManager() : rgen_(313), seed_(313), count_(0) {}

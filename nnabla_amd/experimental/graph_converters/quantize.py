@@ -5,9 +5,10 @@
 QuantizeLinear -> DequantizeLinear pairs whose scales come from the recorded ranges.  Both find their parameters
 under the scope '<function type>-<position of the function in the graph>'.
 
-Left out with the functions they serve, none of which exists on this path: the shared recorder / shared
-quantization of Add2 and Concatenate inputs, the two-input arithmetic functions, and the QNN / MIXED_QNN precision
-modes (None in the reference too, quantize.py:409-413).
+The inputs of Add2 and Concatenate share one recorder and one quantization range (that of the input produced
+earliest in the graph), as in the reference; of the two-input arithmetic set only Add2 exists on this path (Sub2,
+Mul2, Div2 and Pow2 are recognised by name, so their inputs are both treated as activations).  The QNN / MIXED_QNN
+precision modes are None in the reference too (quantize.py:409-413).
 """
 from collections import defaultdict
 
@@ -24,9 +25,28 @@ def _scope_of(f, ranks):
     return '{}-{}'.format(f.info.type_name, ranks.get(f, -1))
 
 
+# the functions whose two inputs are both activations (quantize.py:30-36)
+_TWO_ACTIVATIONS = ('Add2', 'Sub2', 'Mul2', 'Div2', 'Pow2')
+# the functions whose inputs have to share one quantization range (quantize.py:112-116, 351-353)
+_SHARED_RANGE = ('Add2', 'Concatenate')
+
+
 def _count_activations(f, inputs):
-    """How many leading inputs of ``f`` are activations; the rest are parameters."""
-    return len(inputs) if f.info.type_name in ('Concatenate', 'Stack') else 1
+    """How many leading inputs of ``f`` are activations; the rest are parameters (quantize.py:148-152)."""
+    fn = f.info.type_name
+    if fn in ('Concatenate', 'Stack'):
+        return len(inputs)
+    return 2 if fn in _TWO_ACTIVATIONS else 1
+
+
+def _earliest(variables, eligible=lambda v: True):
+    """Index of the variable of lowest rank (first of equals) among the eligible ones after the first, which is the
+    candidate to beat (quantize.py:117-123, 354-360)."""
+    idx, low = 0, variables[0].rank
+    for i, v in enumerate(variables[1:]):
+        if eligible(v) and v.rank < low:
+            idx, low = i + 1, v.rank
+    return idx
 
 
 def _axes(cfg):
@@ -110,11 +130,29 @@ class QuantizeNonQNNToRecordingModifier(FunctionModifier):
                 out.append(wgt()(p, axes=_axes(cfg), training=self._training, name='w{}'.format(i)))
         return out
 
+    # -- quantize.py:110-138
+    def share_recorder(self, f, inputs, new_inputs, cfg):
+        """Add2 / Concatenate: every input is recorded by the recorder (the statistics) of the input that is produced
+        earliest; the other inputs' own recorders are taken out again."""
+        if f.info.type_name not in _SHARED_RANGE:
+            return new_inputs
+        idx = _earliest(new_inputs)
+        scope = self.get_parameter_scope(new_inputs[idx].parent.inputs[1])
+        for i, v in enumerate(new_inputs):
+            if i == idx:
+                continue
+            v = v.parent.inputs[0]
+            with parameter.parameter_scope(scope):
+                v = cfg.recorder_activation()(v, axes=_axes(cfg), training=self._training, name='x0')
+            new_inputs[i] = v
+        return new_inputs
+
     def modify(self, f, inputs):
         if not self.check(f):
             return None
         cfg = self._config
-        h = self._modify_as_same(f, self.add_recorder(f, inputs, cfg))
+        new_inputs = self.share_recorder(f, inputs, self.add_recorder(f, inputs, cfg), cfg)
+        h = self._modify_as_same(f, new_inputs)
         if cfg.recorder_position == cfg.RecorderPosition.BOTH:
             # also record the output, under the scope of the (first) function that consumes it
             nxt = f.outputs[0].function_references[0]
@@ -209,6 +247,29 @@ class QuantizeRecordingToTrainingModifier(FunctionModifier):
                 inps[i] = v
             return inps
 
+        # quantize.py:348-373
+        def shared_quantization(self, f, inps):
+            """Add2 / Concatenate: every input is quantized with the scale and zero point of the (dequantized) input
+            that is produced earliest."""
+            if f.info.type_name not in _SHARED_RANGE:
+                return inps
+
+            def dequantized(v):
+                return v.parent is not None and v.parent.info.type_name == 'DequantizeLinear'
+
+            idx = _earliest(inps, dequantized)
+            s = zp = None
+            if dequantized(inps[idx]):
+                s, zp = inps[idx].parent.inputs[1:3]
+            for i in range(len(inps)):
+                if i == idx:
+                    continue
+                v = inps[i]
+                if dequantized(v):
+                    v = v.parent.inputs[0].parent.inputs[0]      # back to the value before its own Q -> DQ
+                inps[i] = self.try_to_dequantize(self._q(v, s, zp), s, zp)
+            return inps
+
         # quantize.py:240-271
         def _quantize_outputs(self, f, h):
             cfg = self._config
@@ -216,9 +277,14 @@ class QuantizeRecordingToTrainingModifier(FunctionModifier):
             for nxt in f.outputs[0].function_references:
                 if nxt.info.type_name == 'Sink':
                     return h
+                name = 'x0'
+                if nxt.info.type_name in _TWO_ACTIVATIONS:      # recorded as the consumer's i-th input
+                    for i, v in enumerate(nxt.inputs):
+                        if v is f.outputs[0]:
+                            name = 'x{}'.format(i)
                 with parameter.parameter_scope(_scope_of(nxt, self.functions_ranks)):
                     s, zp = cfg.recorder_activation.get_scale_zeropoint(
-                        h, axes=_axes(cfg), narrow_range=cfg.narrow_range, round_method=cfg.pow2.value, name='x0')
+                        h, axes=_axes(cfg), narrow_range=cfg.narrow_range, round_method=cfg.pow2.value, name=name)
                 if s is not None:
                     break
             h = self._q(h, s, zp)
@@ -228,6 +294,7 @@ class QuantizeRecordingToTrainingModifier(FunctionModifier):
         def modify(self, f, inputs):
             scope = _scope_of(f, self.functions_ranks)
             inps = self.dequantize_inputs(self.quantize_inputs(f, inputs, scope))
+            inps = self.shared_quantization(f, inps)
             h = self._modifier._modify_as_same(f, inps)
             if f.info.type_name == 'Sink':
                 return h

@@ -128,6 +128,20 @@ def relu(x, inplace=False, n_outputs=-1, outputs=None):
     return f(x, outputs=outputs)
 
 
+def add2(x0, x1, inplace=False, n_outputs=-1, outputs=None):
+    f = Function("Add2", None, [int(inplace)], args=dict(inplace=inplace))
+    return f(x0, x1, n_outputs=n_outputs, outputs=outputs)
+
+
+def concatenate(*x, **kw):
+    axis = kw.pop('axis', None)
+    n_outputs, outputs = kw.pop('n_outputs', -1), kw.pop('outputs', None)
+    if axis is None:
+        axis = len(x[0].shape) - 1
+    f = Function("Concatenate", None, [int(axis)], args=dict(axis=axis))
+    return f(*x, n_outputs=n_outputs, outputs=outputs)
+
+
 def quantize_linear(x, scale, zero_point, round_mode='HALF_AWAY_FROM_ZERO', narrow_range=False, dtype=1,
                     n_outputs=-1, outputs=None):
     """``saturate(round(x / scale) + zero_point)`` to the int8 (``dtype`` 1 or ``numpy.int8``) or uint8 (2 or

@@ -5,7 +5,8 @@
 
 Functions are created through the registry for the *current* context, so a graph loaded under the ``hip`` extension
 context runs on the hip:float classes (the dispatch nnp_impl_create_function.cpp.tmpl:51-117 performs for every
-function; here for the nine quantization functions, QuantizeLinear, DequantizeLinear, Prune, Affine and ReLU).
+function; here for the nine quantization functions, QuantizeLinear, DequantizeLinear, Prune, Affine, ReLU, Add2 and
+Concatenate).
 Network definitions are read from protobuf text (``.nntxt`` / ``.prototxt``), parameters from
 ``parameter.protobuf`` or from ``parameter`` entries of the text.
 """
@@ -76,6 +77,9 @@ _BUILDERS = {
     "Convolution": ("convolution_param", 2, lambda p, i: F.convolution(
         i[0], i[1], _opt(i, 2), channel_last=bool(p.get("channel_last", False)), **_conv_kwargs(p))),
     "ReLU": ("relu_param", 1, lambda p, i: F.relu(i[0], inplace=bool(p.get("inplace", False)))),
+    "Add2": ("add2_param", 2, lambda p, i: F.add2(i[0], i[1], inplace=bool(p.get("inplace", False)))),
+    "Concatenate": ("concatenate_param", 2, lambda p, i: F.concatenate(
+        *i, axis=int(p.get("axis", len(i[0].shape) - 1)))),
     "QuantizeLinear": ("quantize_linear_param", 3, lambda p, i: F.quantize_linear(
         i[0], i[1], i[2], round_mode=str(p.get("round_mode", "HALF_AWAY_FROM_ZERO")),
         narrow_range=bool(p.get("narrow_range", False)), dtype=int(p.get("dtype", 1)))),

@@ -270,9 +270,21 @@ class QATScheduler(object):
     def __call__(self, pred, training=True):
         self.registry.append((pred, training))
 
+    def _refuse_bn_folding(self, pred):
+        """BatchNormalization folding (qnn.py:842-856) is not part of this build: a graph that would need it is refused
+        rather than converted with unfolded statistics."""
+        if not (self.config.bn_folding or self.config.bn_self_folding):
+            return
+        found = []
+        pred.visit(lambda f: found.append(f) if f.info.type_name == 'BatchNormalization' else None)
+        if found:
+            raise NotImplementedError("QATScheduler: bn_folding / bn_self_folding is set and the network holds a "
+                                      "BatchNormalization; BatchNormalization folding is not available.")
+
     def _schedule_to_recording(self):
         from ..experimental import graph_converters as GC
         for i, (pred, training) in enumerate(self.registry):
+            self._refuse_bn_folding(pred)
             ranks = FunctionsRankRecorder()
             pred.visit(ranks)
             converted = GC.GraphConverter([GC.QuantizeNonQNNToRecordingModifier(

@@ -285,11 +285,15 @@ class Variable(object):
             if not any(i.need_grad for i in node.inputs):
                 continue
             prop = [bool(i.need_grad) for i in node.inputs]
-            accum = [(i.parent is None) or (id(i) in written) for i in node.inputs]
-            node.backward(prop, accum)
+            # keyed by the variable that owns the grad array: two views of one array are one gradient, also when both
+            # are inputs of this very function (its backward handles the inputs in order)
+            accum = []
             for i, p in zip(node.inputs, prop):
+                key = id(i._origin)
+                accum.append((i.parent is None) or (key in written))
                 if p:
-                    written.add(id(i))
+                    written.add(key)
+            node.backward(prop, accum)
 
     def get_unlinked_variable(self, need_grad=None):
         v = self.reshape(self.shape, unlink=True)

@@ -316,6 +316,131 @@ def test_scheduler_end_to_end(ctx):
     assert np.abs(nn.get_parameter('c1/conv/W').g).max() > 0
 
 
+def test_add2_and_concatenate_functions(ctx):
+    """add2.cpp:39-77 and concatenate.cpp:62-104 through the registry: forward values, gradients written and
+    accumulated, shape checks."""
+    rng = np.random.default_rng(11)
+    a, b = rng.standard_normal((3, 4, 5)).astype(np.float32), rng.standard_normal((3, 4, 5)).astype(np.float32)
+    va, vb = _var(a), _var(b)
+    va.need_grad = vb.need_grad = True
+    y = F.add2(va, vb)
+    y.forward()
+    assert bits_equal(y.d, a + b)
+    g = rng.standard_normal((3, 4, 5)).astype(np.float32)
+    va.g, vb.g = 1.5, 0.0
+    y.backward(g)
+    assert bits_equal(vb.g, g)
+    assert np.allclose(va.g, g) or np.allclose(va.g, g + 1.5)      # written, or added when the graph accumulates
+    with pytest.raises(RuntimeError):
+        F.add2(va, _var(np.zeros((3, 1, 5), np.float32)))          # broadcasting is not available
+
+    parts = [rng.standard_normal((2, n, 3, 7)).astype(np.float32) for n in (4, 1, 6)]
+    vs = [_var(p) for p in parts]
+    for v in vs:
+        v.need_grad = True
+    for axis in (1, -3):
+        c = F.concatenate(*vs, axis=axis)
+        assert c.shape == (2, 11, 3, 7)
+        c.forward()
+        assert bits_equal(c.d, np.concatenate(parts, axis=1))
+        gc_ = rng.standard_normal(c.shape).astype(np.float32)
+        for v in vs:
+            v.g = 0
+        c.backward(gc_)
+        off = 0
+        for v, p in zip(vs, parts):
+            assert bits_equal(v.g, gc_[:, off:off + p.shape[1]])
+            off += p.shape[1]
+    last = F.concatenate(_var(np.ones((2, 3), np.float32)), _var(np.zeros((2, 2), np.float32)))    # default: last axis
+    last.forward()
+    assert last.d.tolist() == [[1, 1, 1, 0, 0], [1, 1, 1, 0, 0]]
+    with pytest.raises(RuntimeError):
+        F.concatenate(vs[0], _var(np.zeros((2, 4, 3, 8), np.float32)), axis=1)
+
+
+def test_two_views_of_one_gradient_accumulate(ctx):
+    """A variable and a view of it (same arrays) feeding one function: the second contribution to the shared gradient
+    is added to the first, not written over it."""
+    rng = np.random.default_rng(3)
+    x = _var(rng.standard_normal((4, 6)).astype(np.float32))
+    x.need_grad = True
+    h = F.relu(x)
+    y = F.add2(h, h.reshape(h.shape))
+    y.forward()
+    g = rng.standard_normal((4, 6)).astype(np.float32)
+    x.g = 0
+    y.backward(g)
+    assert bits_equal(x.g, np.where(x.d > 0, 2 * g, 0).astype(np.float32))
+
+
+def residual_concat_net(x):
+    h = F.relu(PF.convolution(x, 4, (3, 3), pad=(1, 1), name='c1'))
+    r = F.relu(PF.convolution(h, 4, (3, 3), pad=(1, 1), name='c2'))
+    s = F.add2(h, r)
+    t = F.relu(PF.convolution(s, 3, (3, 3), pad=(1, 1), name='c3'))
+    return PF.affine(F.concatenate(t, s, axis=1), 6, name='f')
+
+
+def test_scheduler_with_add2_and_concatenate(ctx):
+    """A residual / concatenating network through the three states: the recording graph computes the float values,
+    and in the training graph the inputs of Add2 and of Concatenate sit on one quantization grid each."""
+    rng = np.random.default_rng(8)
+    x = nn.Variable((4, 3, 8, 8))
+    y = residual_concat_net(x)
+    randomise_parameters(rng)
+    float_net = GC.GraphConverter([GC.FunctionModifier()]).convert(y)
+    float_in = float_net
+    while float_in.parent is not None:
+        float_in = float_in.parent.inputs[0]
+    cfg = QATConfig()
+    cfg.niter_to_recording, cfg.niter_to_training = 1, 60
+    sched = QATScheduler(cfg)
+    sched(y)
+    for i in range(62):
+        sched.step()
+        data = rng.standard_normal(x.shape).astype(np.float32)
+        x.d = data
+        float_in.d = data
+        y.forward()
+        float_net.forward()
+        if sched.state == QNNState.RECORDING and i < 4:
+            assert bits_equal(y.d, float_net.d)
+    assert sched.state == QNNState.TRAINING
+    fs = []
+    y.visit(fs.append)
+    for kind in ('Add2', 'Concatenate'):
+        f = [g for g in fs if g.info.type_name == kind][0]
+        dq = [v.parent for v in f.inputs]
+        assert all(g.info.type_name == 'DequantizeLinear' for g in dq)
+        scale = float(dq[0].inputs[1].d.ravel()[0])
+        assert all(g.inputs[1] is dq[0].inputs[1] for g in dq) and scale > 0
+        for v in f.inputs:                   # every input value is a whole number of steps of the shared scale
+            steps = v.d / np.float32(scale)
+            assert np.abs(steps - np.round(steps)).max() < 1e-3
+    err = max_rel_err(y.d, float_net.d)
+    assert 0 < err < 0.5, err
+    y.backward(np.ones(y.shape, np.float32))
+    assert np.abs(nn.get_parameter('c1/conv/W').g).max() > 0
+
+
+def test_add2_and_concatenate_saved_and_reloaded(ctx, tmp_path):
+    from nnabla_amd.utils.nnp_graph import NnpLoader
+    from nnabla_amd.utils.save import save
+    from test_nnp_save import contents_of
+    x = nn.Variable((3, 3, 8, 8))
+    y = residual_concat_net(x)
+    randomise_parameters(np.random.default_rng(21))
+    path = str(tmp_path / 'res.nnp')
+    save(path, contents_of(x, y, 3))
+    data = np.random.default_rng(22).standard_normal(x.shape).astype(np.float32)
+    x.d = data
+    y.forward()
+    ex = NnpLoader(path).get_executor('runtime')
+    ex.data_variables['x'].d = data
+    ex.execute()
+    assert bits_equal(ex.output_variables['y'].d, y.d)
+
+
 def test_recording_with_other_recorders_matches_oracle(ctx):
     """MinMaxMva activations / AbsMax weights on an MLP: every registered statistic against the oracle's recorders fed
     the same tensors."""

@@ -276,6 +276,93 @@ def test_one_recorder_for_a_variable_with_two_consumers():
     assert got.count('MinMaxMinMaxRecorder') == 8
 
 
+def residual_net(x):
+    h = F.relu(PF.convolution(x, 4, (3, 3), pad=(1, 1), name='c1'))      # Convolution-0, ReLU-1
+    r = F.relu(PF.convolution(h, 4, (3, 3), pad=(1, 1), name='c2'))      # Convolution-2, ReLU-3
+    return PF.affine(F.add2(h, r), 5, name='f')                          # Add2-4, Affine-5
+
+
+def concat_net(x):
+    a = F.relu(PF.convolution(x, 4, (3, 3), pad=(1, 1), name='c1'))      # Convolution-0, ReLU-1
+    b = F.relu(PF.convolution(a, 2, (3, 3), pad=(1, 1), name='c2'))      # Convolution-2, ReLU-3
+    c = F.relu(PF.convolution(b, 3, (3, 3), pad=(1, 1), name='c3'))      # Convolution-4, ReLU-5
+    return PF.affine(F.concatenate(c, a, b, axis=1), 5, name='f')        # Concatenate-6, Affine-7
+
+
+def find(v, type_name):
+    out = []
+    v.visit(lambda f: out.append(f) if f.info.type_name == type_name else None)
+    return out
+
+
+def test_add2_inputs_share_the_recorder_of_the_earliest_one():
+    """quantize.py:110-138: h is already recorded for the second convolution ('Convolution-2/x0'); r gets a recorder
+    of its own ('Add2-4/x1'), which share_recorder replaces by one on the statistics of h's."""
+    x = nn.Variable((2, 3, 8, 8))
+    cfg = QATConfig()
+    y_rec = to_recording(residual_net(x), cfg)
+    act = cfg.recorder_activation().name()
+    assert names(y_rec) == ['Convolution', act, 'ReLU', act, 'MinMaxMinMaxRecorder', 'MinMaxMinMaxRecorder',
+                            'Convolution', act, 'ReLU', act, 'Add2', 'Affine']
+    add = find(y_rec, 'Add2')[0]
+    r0, r1 = add.inputs[0].parent, add.inputs[1].parent
+    assert r0.info.type_name == r1.info.type_name == act and r0 is not r1
+    assert r0.inputs[1] is r1.inputs[1] is nn.get_parameter('Convolution-2/M-x0')
+    conv2 = find(y_rec, 'Convolution')[1]
+    assert conv2.inputs[0] is add.inputs[0]                  # one recorder on h for both of its consumers
+    assert r1.inputs[0].parent.info.type_name == 'ReLU'      # r's own recorder is gone from the graph
+
+
+def test_concatenate_inputs_share_the_recorder_of_the_earliest_one():
+    x = nn.Variable((2, 3, 8, 8))
+    cfg = QATConfig()
+    y_rec = to_recording(concat_net(x), cfg)
+    act = cfg.recorder_activation().name()
+    cat = find(y_rec, 'Concatenate')[0]
+    assert tuple(cat.outputs[0].shape) == (2, 9, 8, 8)
+    recs = [v.parent for v in cat.inputs]
+    assert all(f.info.type_name == act for f in recs)
+    # inputs (c, a, b): a is produced first and is already recorded as the input of the second convolution
+    shared = nn.get_parameter('Convolution-2/M-x0')
+    assert all(f.inputs[1] is shared for f in recs)
+    assert recs[1] is find(y_rec, 'Convolution')[1].inputs[0].parent
+
+
+def test_add2_and_concatenate_inputs_are_quantized_with_one_range():
+    """quantize.py:348-373: in the training graph every input of Add2 / Concatenate goes through Q -> DQ with the
+    scale and zero point of the input produced earliest."""
+    for net, kind, n_in in ((residual_net, 'Add2', 2), (concat_net, 'Concatenate', 3)):
+        nn.clear_parameters()
+        x = nn.Variable((2, 3, 8, 8))
+        cfg = QATConfig()
+        y_rec = to_recording(net(x), cfg)
+        set_statistics(np.random.default_rng(3))
+        y_q = to_training(y_rec, cfg)
+        f = find(y_q, kind)[0]
+        assert len(f.inputs) == n_in
+        dq = [v.parent for v in f.inputs]
+        assert all(g.info.type_name == 'DequantizeLinear' for g in dq)
+        assert all(g.inputs[1] is dq[0].inputs[1] and g.inputs[2] is dq[0].inputs[2] for g in dq)
+        for g in dq:                       # each is the DQ of a Q with the same parameters
+            q = g.inputs[0].parent
+            assert q.info.type_name == 'QuantizeLinear' and q.inputs[1] is dq[0].inputs[1]
+        # the output of the function is quantized for its consumer as usual
+        assert f.outputs[0].function_references[0].info.type_name in ('QuantizeLinear', 'Affine')
+
+
+def test_output_statistics_of_a_two_input_consumer_are_named_after_its_input_position():
+    """quantize.py:233-237: the producer of Add2's second input looks its output range up as 'Add2-<rank>/x1', the
+    statistics add_recorder registered for that input (quantize.py:163-164) before share_recorder rewired it."""
+    x = nn.Variable((2, 3, 8, 8))
+    cfg = QATConfig()
+    y_rec = to_recording(residual_net(x), cfg)
+    assert 'Add2-4/M-x1' in nn.get_parameters(grad_only=False)
+    set_statistics(np.random.default_rng(4))
+    y_q = to_training(y_rec, cfg)
+    assert 'Add2-4/scale-x1' in nn.get_parameters(grad_only=False)
+    assert find(y_q, 'Add2')
+
+
 # ------------------------------------------------------------------------------ recording graph -> training graph
 def set_statistics(rng):
     for k, v in nn.get_parameters(grad_only=False).items():
@@ -424,6 +511,25 @@ def test_scheduler_states_and_rewiring():
     for _ in range(3):
         s.step()
     assert s.state == QNNState.TRAINING and names(tail) == got
+
+
+def test_scheduler_refuses_batch_normalization_folding():
+    """bn_folding / bn_self_folding (qnn.py:842-856) with a BatchNormalization in the graph: refused, not ignored."""
+    import types
+
+    class Graph(object):
+        def visit(self, fn):
+            fn(types.SimpleNamespace(info=types.SimpleNamespace(type_name='BatchNormalization')))
+
+    cfg = qnn.QATTensorRTConfig()
+    cfg.niter_to_recording, cfg.niter_to_training = 0, 5
+    sched = QATScheduler(cfg)
+    sched(Graph())
+    with pytest.raises(NotImplementedError):
+        sched.step()
+    cfg.bn_folding = cfg.bn_self_folding = False
+    sched = QATScheduler(cfg)
+    sched._refuse_bn_folding(Graph())        # nothing to fold: no complaint
 
 
 def test_scheduler_argument_checks():
