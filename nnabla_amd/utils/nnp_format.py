@@ -301,3 +301,161 @@ def encode_parameters(params):
 
 def pack_float(v):
     return struct.pack("<f", v)
+
+
+# ------------------------------------------------------------------- wire format of the network definition
+# The messages of nnabla.proto.tmpl a network definition uses, as {field name: (number, type)}; a type is a scalar kind
+# ('string', 'int64', 'bool', 'float'), the name of another message of this table, or ('repeated', type).
+# Function.<type>_param has the number 1001 + the position of the function in functions.yaml, and the fields of a
+# <Type>Parameter message are the function's arguments in the order of functions.yaml, numbered from 1
+# (nnabla.proto.tmpl:300-323); the positions below are those of build-tools/code_generator/functions.yaml.
+_CONV = [("base_axis", "int64"), ("pad", "Shape"), ("stride", "Shape"), ("dilation", "Shape"), ("group", "int64")]
+_FUNCTION_PARAMS = OrderedDict([
+    # snake name: (position in functions.yaml, arguments)
+    ("affine", (0, [("base_axis", "int64")])),
+    ("convolution", (4, _CONV + [("channel_last", "bool")])),
+    ("relu", (21, [("inplace", "bool")])),
+    ("add2", (64, [("inplace", "bool")])),
+    ("concatenate", (132, [("axis", "int64")])),
+    ("binary_connect_affine", (201, [("base_axis", "int64"), ("quantize_zero_to", "float")])),
+    ("binary_connect_convolution", (202, _CONV + [("quantize_zero_to", "float")])),
+    ("binary_weight_affine", (203, [("base_axis", "int64"), ("quantize_zero_to", "float")])),
+    ("binary_weight_convolution", (204, _CONV + [("quantize_zero_to", "float")])),
+    ("inq_affine", (205, [("base_axis", "int64"), ("num_bits", "int64"), ("inq_iterations", ("repeated", "int64")),
+                          ("selection_algorithm", "string"), ("seed", "int64")])),
+    ("inq_convolution", (206, _CONV + [("num_bits", "int64"), ("inq_iterations", ("repeated", "int64")),
+                                       ("selection_algorithm", "string"), ("seed", "int64")])),
+    ("fixed_point_quantize", (207, [("sign", "bool"), ("n", "int64"), ("delta", "float"),
+                                    ("ste_fine_grained", "bool")])),
+    ("min_max_quantize", (208, [("decay", "float"), ("x_min_max", "bool"), ("ema", "bool"),
+                                ("ste_fine_grained", "bool"), ("eps", "float")])),
+    ("pow2_quantize", (209, [("sign", "bool"), ("with_zero", "bool"), ("n", "int64"), ("m", "int64"),
+                             ("ste_fine_grained", "bool")])),
+    ("prune", (210, [("rate", "float")])),
+    ("quantize_linear", (211, [("round_mode", "string"), ("narrow_range", "bool"), ("dtype", "int64")])),
+])
+
+
+def _build_schema():
+    rep = lambda t: ("repeated", t)
+    s = {
+        "Shape": {"dim": (1, rep("int64"))},
+        "Context": {"backends": (1, rep("string")), "array_class": (2, "string"), "device_id": (3, "string"),
+                    "backend": (4, "string"), "compute_backend": (5, "string")},
+        "GlobalConfig": {"default_context": (1, "Context")},
+        "NNablaProtoBuf": {"version": (1, "string"), "global_config": (2, "GlobalConfig"),
+                           "network": (100, rep("Network")), "parameter": (200, rep("Parameter")),
+                           "executor": (600, rep("Executor"))},
+        "Network": {"name": (1, "string"), "batch_size": (10, "int64"), "repeat_info": (11, rep("RepeatInfo")),
+                    "variable": (100, rep("Variable")), "function": (200, rep("Function"))},
+        "RepeatInfo": {"id": (1, "string"), "times": (2, "int64")},
+        "RepeatParameter": {"repeat_id": (1, "string"), "times": (2, "int64")},
+        "RecurrentParameter": {"repeat_id": (1, "string"), "length": (2, "int64"), "axis": (3, "int64")},
+        "Variable": {"name": (1, "string"), "type": (2, "string"), "repeat_id": (3, rep("string")),
+                     "shape": (20, "Shape"), "initializer": (100, "Initializer")},
+        "Initializer": {"type": (2, "string"), "multiplier": (10, "float")},
+        "Parameter": {"variable_name": (1, "string"), "shape": (20, "Shape"), "data": (100, rep("float")),
+                      "need_grad": (101, "bool")},
+        "Executor": {"name": (1, "string"), "network_name": (10, "string"), "num_evaluations": (20, "int64"),
+                     "repeat_evaluation_type": (21, "string"), "need_back_propagation": (30, "bool"),
+                     "data_variable": (50, rep("DataVariable")), "generator_variable": (60, rep("GeneratorVariable")),
+                     "loss_variable": (70, rep("LossVariable")), "output_variable": (80, rep("OutputVariable")),
+                     "parameter_variable": (90, rep("ParameterVariable")), "no_image_normalization": (101, "bool")},
+        "DataVariable": {"variable_name": (1, "string"), "data_name": (3, "string")},
+        "GeneratorVariable": {"variable_name": (1, "string"), "type": (2, "string"), "multiplier": (3, "float")},
+        "LossVariable": {"variable_name": (1, "string")},
+        "OutputVariable": {"variable_name": (1, "string"), "type": (2, "string"), "data_name": (3, "string")},
+        "ParameterVariable": {"variable_name": (1, "string"), "learning_rate_multiplier": (2, "float")},
+        "Function": {"name": (1, "string"), "type": (2, "string"), "repeat_id": (3, rep("string")),
+                     "context": (10, "Context"), "input": (20, rep("string")), "output": (30, rep("string")),
+                     "repeat_param": (100, "RepeatParameter"), "recurrent_param": (101, "RecurrentParameter")},
+    }
+    for snake, (position, args) in _FUNCTION_PARAMS.items():
+        msg = "".join(p.capitalize() for p in snake.split("_")) + "Parameter"
+        s["Function"][snake + "_param"] = (1001 + position, msg)
+        s[msg] = {name: (i + 1, kind) for i, (name, kind) in enumerate(args)}
+    return s
+
+
+WIRE_SCHEMA = _build_schema()
+_SCALAR_WIRE = {"string": 2, "int64": 0, "bool": 0, "float": 5}
+
+
+def _decode_scalar(kind, wt, val, where):
+    if kind == "string" and wt == 2:
+        return bytes(val).decode("utf-8")
+    if kind == "int64" and wt == 0:
+        return _signed64(val)
+    if kind == "bool" and wt == 0:
+        return bool(val)
+    if kind == "float" and wt == 5:
+        return struct.unpack("<f", val)[0]
+    raise NnpFormatError("%s: wire type %d does not fit a %s" % (where, wt, kind))
+
+
+def decode_message(buf, message="NNablaProtoBuf", skip=()):
+    """Wire-format bytes of a message of WIRE_SCHEMA -> the :class:`Message` tree the text parser would give (same
+    field names; fields the schema does not list, e.g. the parameter messages of functions outside this path, are
+    left out, and so are the fields named in ``skip``)."""
+    fields = WIRE_SCHEMA[message]
+    by_number = {num: (name, kind) for name, (num, kind) in fields.items()}
+    out = Message()
+    for num, wt, val in _fields(buf):
+        if num not in by_number:
+            continue
+        name, kind = by_number[num]
+        if name in skip:
+            continue
+        where = "%s.%s" % (message, name)
+        repeated = isinstance(kind, tuple)
+        if repeated:
+            kind = kind[1]
+        if kind in WIRE_SCHEMA:
+            if wt != 2:
+                raise NnpFormatError("%s: wire type %d for a message" % (where, wt))
+            out.add(name, decode_message(val, kind))
+        elif repeated and wt == 2 and kind != "string":      # packed
+            if kind == "float":
+                if len(val) % 4:
+                    raise NnpFormatError("%s: packed floats of %d bytes" % (where, len(val)))
+                for f in np.frombuffer(val, dtype="<f4"):
+                    out.add(name, float(f))
+            else:
+                pos = 0
+                while pos < len(val):
+                    v, pos = _varint(val, pos)
+                    out.add(name, bool(v) if kind == "bool" else _signed64(v))
+        else:
+            out.add(name, _decode_scalar(kind, wt, val, where))
+    return out
+
+
+def encode_message(msg, message="NNablaProtoBuf"):
+    """Inverse of :func:`decode_message` (repeated numbers are written packed, as proto3 writers do)."""
+    fields = WIRE_SCHEMA[message]
+    out = []
+    for name, values in msg.fields.items():
+        if name not in fields:
+            raise NnpFormatError("%s has no field %r in the wire schema" % (message, name))
+        num, kind = fields[name]
+        repeated = isinstance(kind, tuple)
+        if repeated:
+            kind = kind[1]
+        if kind in WIRE_SCHEMA:
+            for v in values:
+                out.append(_enc_field(num, encode_message(v, kind)))
+        elif repeated and kind != "string":
+            if kind == "float":
+                body = np.asarray([float(v) for v in values], dtype="<f4").tobytes()
+            else:
+                body = b"".join(_enc_varint(int(v)) for v in values)
+            out.append(_enc_field(num, body))
+        else:
+            for v in values:
+                if kind == "string":
+                    out.append(_enc_field(num, str(v).encode("utf-8")))
+                elif kind == "float":
+                    out.append(_enc_varint((num << 3) | 5) + struct.pack("<f", float(v)))
+                else:
+                    out.append(_enc_varint((num << 3) | 0) + _enc_varint(int(v)))
+    return b"".join(out)

@@ -7,8 +7,8 @@ Functions are created through the registry for the *current* context, so a graph
 context runs on the hip:float classes (the dispatch nnp_impl_create_function.cpp.tmpl:51-117 performs for every
 function; here for the nine quantization functions, QuantizeLinear, DequantizeLinear, Prune, Affine, ReLU, Add2 and
 Concatenate).
-Network definitions are read from protobuf text (``.nntxt`` / ``.prototxt``), parameters from
-``parameter.protobuf`` or from ``parameter`` entries of the text.
+Network definitions are read from protobuf text (``.nntxt`` / ``.prototxt``) or from binary protobuf
+(``.protobuf``, load.py:492-494), parameters from ``parameter.protobuf`` or from ``parameter`` entries of either.
 """
 import io
 import os
@@ -224,8 +224,10 @@ class NnpLoader(object):
         if ext in (".nntxt", ".prototxt"):
             self._load_text(data.decode("utf-8") if isinstance(data, bytes) else data)
         elif ext == ".protobuf":
+            # parameters, and (load.py:492-494) possibly the networks and executors as well
             for pname, (arr, need_grad) in nnp_format.decode_parameters(data).items():
                 self._set_param(pname, arr, need_grad)
+            self._register(nnp_format.decode_message(data, skip=("parameter",)))
         elif ext == ".h5":
             raise NnpError("%s: HDF5 parameter files are not supported here (h5py is absent); save the parameters "
                            "as parameter.protobuf" % name)
@@ -246,6 +248,9 @@ class NnpLoader(object):
                 raise NnpError("parameter %r: %d values for shape %s" % (p.get("variable_name"), data.size, shape))
             self._set_param(str(p.get("variable_name")), data.reshape(shape) if shape else data,
                             bool(p.get("need_grad", False)))
+        self._register(root)
+
+    def _register(self, root):
         for n in root.all("network"):
             self._networks[str(n.get("name"))] = n
         for e in root.all("executor"):

@@ -209,3 +209,110 @@ def test_linear_quantizer_and_prune_builders(hip_ctx):
     assert v["xp"].parent.info == {"type": "Prune", "iargs": (), "fargs": (0.25,), "sarg": None}
     assert v["xq"].parent.info == {"type": "QuantizeLinear", "iargs": (1, 2), "fargs": (), "sarg": "HALF_TO_EVEN"}
     assert v["y"].parent.info["type"] == "DequantizeLinear"
+
+
+# ------------------------------------------------------------------------------- networks in binary protobuf
+def _pb_network_classes():
+    """google.protobuf message classes for every message of nnp_format.WIRE_SCHEMA, built without protoc."""
+    from google.protobuf import descriptor_pb2, descriptor_pool, message_factory
+    T = descriptor_pb2.FieldDescriptorProto
+    kinds = {"string": T.TYPE_STRING, "int64": T.TYPE_INT64, "bool": T.TYPE_BOOL, "float": T.TYPE_FLOAT}
+    fd = descriptor_pb2.FileDescriptorProto(name="nnabla_networks.proto", syntax="proto3")
+    for mname, fields in nnp_format.WIRE_SCHEMA.items():
+        m = fd.message_type.add(name=mname)
+        for fname, (num, kind) in fields.items():
+            label = T.LABEL_OPTIONAL
+            if isinstance(kind, tuple):
+                label, kind = T.LABEL_REPEATED, kind[1]
+            if kind in kinds:
+                m.field.add(name=fname, number=num, type=kinds[kind], label=label)
+            else:
+                m.field.add(name=fname, number=num, type=T.TYPE_MESSAGE, type_name="." + kind, label=label)
+    pool = descriptor_pool.DescriptorPool()
+    pool.Add(fd)
+    return message_factory.GetMessageClass(pool.FindMessageTypeByName("NNablaProtoBuf"))
+
+
+def _tree(msg):
+    """A Message tree as nested plain data, floats at float32 precision."""
+    out = []
+    for name, values in msg.fields.items():
+        for v in values:
+            if isinstance(v, nnp_format.Message):
+                out.append((name, _tree(v)))
+            elif isinstance(v, float):
+                out.append((name, float(np.float32(v))))
+            else:
+                out.append((name, str(v) if isinstance(v, str) else v))
+    return out
+
+
+def test_function_message_known_bytes():
+    """Function { name = 1; type = 2; input = 20; output = 30; relu_param = 1001 + 21 } with
+    ReLUParameter { inplace = 1 }: the bytes written out by hand (nnabla.proto.tmpl:291-323; ReLU is the 22nd
+    function of functions.yaml)."""
+    want = (b"\x0a\x01f" b"\x12\x04ReLU" b"\xa2\x01\x01x" b"\xf2\x01\x01y"
+            b"\xf2\x3f\x02\x08\x01")        # key (1022 << 3 | 2) = 8178 = f2 3f, length 2, inplace = true
+    f = nnp_format.parse_text('name: "f" type: "ReLU" input: "x" output: "y" relu_param { inplace: true }')
+    assert nnp_format.encode_message(f, "Function") == want
+    back = nnp_format.decode_message(want, "Function")
+    assert _tree(back) == _tree(f)
+    # the field numbers of the quantization functions: positions 201..211 of functions.yaml
+    nums = {k: v[0] for k, v in nnp_format.WIRE_SCHEMA["Function"].items() if k.endswith("_param")}
+    assert nums["binary_connect_affine_param"] == 1202 and nums["quantize_linear_param"] == 1212
+    assert nums["fixed_point_quantize_param"] == 1208 and nums["affine_param"] == 1001
+    assert nums["add2_param"] == 1065 and nums["concatenate_param"] == 1133 and nums["convolution_param"] == 1005
+
+
+def test_binary_network_round_trip_and_against_protobuf():
+    root = nnp_format.parse_text(NET)
+    wire = nnp_format.encode_message(root)
+    assert _tree(nnp_format.decode_message(wire)) == _tree(root)
+    Root = _pb_network_classes()
+    pb = Root()
+    pb.ParseFromString(wire)                      # google.protobuf reads what the encoder writes
+    net = pb.network[0]
+    assert net.name == "net" and net.batch_size == 4 and [v.name for v in net.variable][:2] == ["x", "W"]
+    assert list(net.variable[0].shape.dim) == [-1, 8]
+    f = net.function[0]
+    assert f.type == "FixedPointQuantize" and list(f.input) == ["x"] and list(f.output) == ["q"]
+    assert f.fixed_point_quantize_param.n == 8 and f.fixed_point_quantize_param.delta == 0.0625
+    assert f.fixed_point_quantize_param.sign is True
+    assert net.function[1].binary_weight_affine_param.base_axis == 1
+    assert pb.executor[0].output_variable[0].variable_name == "r"
+    assert abs(net.variable[1].initializer.multiplier - 0.5) < 1e-7
+    # and the decoder reads what google.protobuf writes (packed repeated fields, default values left out)
+    again = nnp_format.decode_message(pb.SerializeToString())
+    a, b = _tree(again), _tree(root)
+    # proto3 writers omit zeros and false, and write the fields in the order of their numbers
+    drop = lambda t: sorted([(k, drop(v) if isinstance(v, list) else v) for k, v in t
+                             if not (v is False or v == 0 or v == 0.0) or isinstance(v, list)], key=lambda kv: kv[0])
+    assert drop(a) == drop(b)
+
+
+def test_graph_from_binary_protobuf(tmp_path, hip_ctx):
+    """An archive whose network definition is binary (load.py:492-494): the same graph as from the text."""
+    rng = np.random.RandomState(1)
+    params = {"W": rng.randn(8, 6).astype(np.float32), "alpha": np.ones(6, np.float32)}
+    root = nnp_format.parse_text(NET)
+    path = str(tmp_path / "binary.nnp")
+    with zipfile.ZipFile(path, "w") as z:
+        z.writestr("nnp_version.txt", "0.1\n")
+        z.writestr("network.protobuf", nnp_format.encode_message(root))
+        z.writestr("parameter.protobuf", nnp_format.encode_parameters(params))
+    text_path = str(tmp_path / "text.nnp")
+    save_nnp(text_path, NET, params)
+    for p in (path, text_path):
+        L = NnpLoader(p)
+        assert L.get_network_names() == ["net"] and L.get_executor_names() == ["run"]
+        net = L.get_network("net", batch_size=3)
+        assert net.variables["r"].shape == (3, 6) and list(net.inputs) == ["x"] and list(net.outputs) == ["r"]
+        assert np.array_equal(L.get_parameters()["W"].d, params["W"])
+    # one .protobuf holding networks and parameters together
+    both = nnp_format.encode_message(root) + nnp_format.encode_parameters(params)
+    single = str(tmp_path / "all.protobuf")
+    with open(single, "wb") as fh:
+        fh.write(both)
+    L = NnpLoader(single)
+    assert L.get_network_names() == ["net"] and set(L.get_parameters()) >= {"W", "alpha"}
+    assert L.get_network("net").variables["y"].shape == (4, 6)
