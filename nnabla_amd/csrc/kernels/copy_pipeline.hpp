@@ -83,6 +83,28 @@ constexpr Program one_tile_program(int depth, int loop_wait, int steps) {
   return p;
 }
 
+// Bit-weight kernel, one-digit rows: a step's operands are few enough to be read one whole step ahead.
+//   prologue: issue steps 0 .. depth-1; wait(prologue_wait); barrier; read step 0
+//   step ks:  wait(loop_wait); barrier; read ks+1; (multiply step ks from registers); issue ks+depth
+constexpr Program read_ahead_program(int depth, int prologue_wait, int loop_wait, int steps) {
+  Program p{};
+  p.n = 0;
+  p.steps = steps;
+  for (int d = 0; d < depth; ++d)
+    push(p, kIssue, d);
+  push(p, kWait, prologue_wait);
+  push(p, kBarrier, 0);
+  push(p, kRead, 0);
+  for (int ks = 0; ks < steps; ++ks) {
+    push(p, kWait, loop_wait);
+    push(p, kBarrier, 0);
+    if (ks + 1 < steps)
+      push(p, kRead, ks + 1);
+    push(p, kIssue, ks + depth);
+  }
+  return p;
+}
+
 // 0: safe; 1: a buffer is read before the step has landed for every wavefront; 2: a copy may overwrite a buffer that
 // is still being read; 3: the program does not fit the model's tables; 4: a step is issued out of order
 constexpr int check(const Program &p, int stages) {
@@ -158,6 +180,17 @@ constexpr int two_tile_prologue_wait(int stages, int depth) {
   int best = -1;
   for (int w = 0; w <= depth; ++w)
     if (two_tile_safe(stages, depth, w, 0))
+      best = w;
+  return best;
+}
+constexpr bool read_ahead_safe(int stages, int depth, int prologue_wait, int loop_wait) {
+  return depth >= 1 &&
+         check(read_ahead_program(depth, prologue_wait, loop_wait, model_steps(stages)), stages) == 0;
+}
+constexpr int read_ahead_loop_wait(int stages, int depth) {
+  int best = -1;
+  for (int w = 0; w <= depth; ++w)
+    if (read_ahead_safe(stages, depth, depth - 1, w))
       best = w;
   return best;
 }

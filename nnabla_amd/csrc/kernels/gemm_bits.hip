@@ -77,6 +77,11 @@ constexpr int gemm_bits_lds_bytes(int BM, int BN, int waves_m, int waves_n, int 
   return stages > exchange ? stages : exchange;
 }
 
+// Past the stages (and the exchange area) the LDS holds what the epilogue needs besides the accumulators: the block's
+// row sums (int64) and shifts, and its columns' alpha and bias.  They are loaded while the first copies are in flight
+// and read back from LDS at the end, so the epilogue starts without a round trip to memory.
+constexpr int gemm_bits_epilogue_bytes(int BM, int BN) { return (BM * 12 + BN * 8 + 255) / 256 * 256; }
+
 // sum_k q_k * (+-1) as fp32 from the three digit accumulators and the row sum (hi * 65536 + lo), scaled by 2^-shift.
 // Integer arithmetic up to the last step: the high and low parts are combined by one fused multiply-add, whose
 // operands are exact (|hi part| < 2^24, low part reduced to 16 bits).
@@ -419,6 +424,7 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
   // order of copies, waits, barriers and LDS reads (copy_pipeline.hpp), which is also asserted safe as a whole.
   constexpr int kPrologueWait = pipeline::two_tile_prologue_wait(kStages, kDepth);
   constexpr int kLoopWait = pipeline::two_tile_loop_wait(kStages, kDepth);
+  constexpr int kAheadWait = pipeline::read_ahead_loop_wait(kStages, kDepth); // the loop of one-digit rows
   static_assert(kPrologueWait >= 0 && kLoopWait >= 0 &&
                     pipeline::two_tile_safe(kStages, kDepth, kPrologueWait, kLoopWait),
                 "the copy pipeline hands a buffer over too early");
@@ -501,6 +507,43 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
   // A wavefront whose columns all lie past the end of the operand (last tile of a row of tiles) only takes part in
   // the copies and barriers: the matrix pipe of its SIMD is left to the other wavefront.
   const bool idle = a.n_begin + bn * BN + wn * NF * 32 >= a.n_end;
+  // the epilogue's metadata (plain product): loaded here, written to LDS once the first copies have been issued
+  constexpr int kThreadsAll = kWaves * 64;
+  constexpr int kEpiOff = gemm_bits_lds_bytes(BM, BN, kWavesM, kWavesN, kWavesK);
+  constexpr int kEpiCols = (BN + kThreadsAll - 1) / kThreadsAll;
+  long long *epi_sums = reinterpret_cast<long long *>(smem + kEpiOff);
+  int32_t *epi_shift = reinterpret_cast<int32_t *>(smem + kEpiOff + BM * 8);
+  float *epi_alpha = reinterpret_cast<float *>(smem + kEpiOff + BM * 12), *epi_bias = epi_alpha + BN;
+  long long meta_sum = 0;
+  int32_t meta_shift = 0;
+  float meta_alpha[kEpiCols], meta_bias[kEpiCols];
+  if constexpr (!kUnfold) {
+    if (tid < BM) {
+      const int64_t m = bm * BM + tid;
+      const int64_t ml = (m < a.row_blocks * kFragRows) ? m : 0; // row blocks past the operand are not stored
+      meta_sum = a.use_sums ? a.sums[ml] : 0;
+      meta_shift = a.shift[ml];
+    }
+#pragma unroll
+    for (int c = 0; c < kEpiCols; ++c) {
+      const int64_t n = a.n_begin + bn * BN + c * kThreadsAll + tid;
+      const int64_t nc = n < a.N ? n : a.N - 1;
+      meta_alpha[c] = (a.finish && a.alpha) ? a.alpha[nc] : 1.0f;
+      meta_bias[c] = (a.finish && a.bias) ? a.bias[nc] : 0.0f;
+    }
+  }
+  auto store_epilogue_metadata = [&]() __attribute__((always_inline)) {
+    if (tid < BM) {
+      epi_sums[tid] = meta_sum;
+      epi_shift[tid] = meta_shift;
+    }
+#pragma unroll
+    for (int c = 0; c < kEpiCols; ++c)
+      if (c * kThreadsAll + tid < BN) {
+        epi_alpha[c * kThreadsAll + tid] = meta_alpha[c];
+        epi_bias[c * kThreadsAll + tid] = meta_bias[c];
+      }
+  };
   if constexpr (kUnfold) {
     unfold_main_loop<BM, BN, kWavesM, kWavesN, kWavesK, kStageBytes, kStepBytes, kABytes>(
         a, smem, bm, bn, wave, lane, idle, [&](int buf_bytes) __attribute__((always_inline)) {
@@ -592,12 +635,53 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
   #pragma unroll
       for (int d = 0; d < kDepth; ++d)
         copy_next(d * kStageBytes, count_c);
+      store_epilogue_metadata(); // its loads were issued before the copies: waiting for them leaves the copies in flight
       wait_copies(std::integral_constant<int, kPrologueWait>(), count_c);
       NBLA_BARRIER();
       read_words(0, 0, w0);
       read_a(0, 0, af0);
       // byte offsets of the LDS buffers of step ks (`cur`), of step ks-1 = that of step ks+kDepth (`prev`)
       int cur = 0, prev = (kStages - 1) * kStageBytes;
+      if (kUsed == 1 && !idle) {
+        // One-digit rows: a step has a third of the MFMAs, too few to cover an LDS read issued in the same step, and
+        // a third of the operand registers.  So both k tiles of step ks+1 are read at the top of step ks (after the
+        // barrier that says they have landed everywhere) and multiplied one step later, from registers.
+        static_assert(pipeline::read_ahead_safe(kStages, kDepth, kPrologueWait, kAheadWait),
+                      "the copy pipeline hands a buffer over too early");
+        read_words(0, 1, w1);
+        read_a(0, 1, af1);
+        for (int left = nstages; left > 0; --left) {
+          const int next = (cur + kStageBytes == kStages * kStageBytes) ? 0 : cur + kStageBytes;
+          uint4_t an0[MF][kUsed], an1[MF][kUsed], wn0, wn1;
+          wait_copies(std::integral_constant<int, kAheadWait>(), count_c);
+          // this wavefront's reads of step ks (issued a step ago) have returned: after the barrier another wavefront
+          // may send a copy into a buffer that holds an older step only, but the wait costs nothing here
+          __builtin_amdgcn_s_waitcnt(0xc07f);
+          NBLA_BARRIER();
+          if (left > 1) {
+            read_words(next, 0, wn0);
+            read_a(next, 0, an0);
+            read_words(next, 1, wn1);
+            read_a(next, 1, an1);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          mma(af0, w0, J0(), JN());
+          mma(af1, w1, J0(), JN());
+          __builtin_amdgcn_sched_barrier(0);
+          copy_next(prev, count_c);
+          if (left > 1) {
+#pragma unroll
+            for (int i = 0; i < MF; ++i)
+#pragma unroll
+              for (int d = 0; d < kUsed; ++d)
+                af0[i][d] = an0[i][d], af1[i][d] = an1[i][d];
+            w0 = wn0, w1 = wn1;
+          }
+          prev = cur;
+          cur = next;
+        }
+        return;
+      }
       if (idle) {
         for (int left = nstages; left > 0; --left) {
           wait_copies(std::integral_constant<int, kLoopWait>(), count_c);
@@ -700,132 +784,149 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
     const int64_t off = (in == 1u) ? m * a.outer_stride : (int64_t)(mu / in) * a.outer_stride + (mu % in);
     return a.y + off;
   };
-  auto finish = [&](float v, float prev, float al, float bi) {
-    if (a.accumulate)
-      v = prev + v;
-    if (use_alpha)
-      v = v * al;
-    if (use_bias)
-      v = v + bi;
-    return v;
-  };
-  if (!kSwap) {
-    const int64_t ncol0 = a.n_begin + bn * BN + wn * NF * 32 + col_in_frag;
-    float al[NF], bi[NF];
-#pragma unroll
-    for (int j = 0; j < NF; ++j) {
-      const int64_t n = (ncol0 + 32 * j < a.N) ? ncol0 + 32 * j : a.N - 1;
-      al[j] = use_alpha ? a.alpha[n] : 1.0f;
-      bi[j] = use_bias ? a.bias[n] : 0.0f;
-    }
-#pragma unroll
-    for (int i = 0; i < MF; ++i) {
-      const int64_t m0 = bm * BM + (wm * MF + i) * 32 + 4 * row_half;
-#pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        // rows m0 + 8 rq + 0..3 (the metadata arrays are padded to whole row blocks)
-        const int64_t mq = m0 + 8 * rq;
-        const int64_t ml = (mq < a.row_blocks * kFragRows) ? mq : 0; // row blocks past the operand are not stored
-        i32x4_t sum01 = {0, 0, 0, 0}, sum23 = {0, 0, 0, 0};
-        if (a.use_sums) {
-          sum01 = *reinterpret_cast<const i32x4_t *>(a.sums + ml); // two int64 as (lo, hi) words
-          sum23 = *reinterpret_cast<const i32x4_t *>(a.sums + ml + 2);
-        }
-        i32x4_t sh = *reinterpret_cast<const i32x4_t *>(a.shift + ml);
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          sh[e] = plain_shift(sh[e]); // one-digit rows store their shift with a bias (kBadRow is negative: unchanged)
-        // sum = s_hi * 65536 + s_lo with s_lo in [0, 65536)
-        const uint32_t lo_w[4] = {(uint32_t)sum01.x, (uint32_t)sum01.z, (uint32_t)sum23.x, (uint32_t)sum23.z};
-        const int hi_w[4] = {sum01.y, sum01.w, sum23.y, sum23.w};
-        int s_hi[4], s_lo[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          s_hi[e] = (int)((lo_w[e] >> 16) | ((uint32_t)hi_w[e] << 16));
-          s_lo[e] = (int)(lo_w[e] & 0xffffu);
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = 4 * rq + e;
-          if (mq + e >= a.M)
-            continue;
-          float *row = row_ptr(mq + e) + ncol0 * a.n_stride;
-          float prev[NF];
-          if (a.accumulate) {
-#pragma unroll
-            for (int j = 0; j < NF; ++j)
-              prev[j] = (ncol0 + 32 * j < a.n_end) ? row[32 * j * a.n_stride] : 0.0f;
-          }
-#pragma unroll
-          for (int j = 0; j < NF; ++j) {
-            float v = finish_dot(acc[0][i][j][r], acc[1][i][j][r], acc[2][i][j][r], s_hi[e], s_lo[e], sh[e],
-                                 frag0 + j);
-            if (sh[e] == kBadRow)
-              v = __builtin_nanf("");
-            v = finish(v, prev[j], al[j], bi[j]);
-            if (ncol0 + 32 * j < a.n_end)
-              __builtin_nontemporal_store(v, row + 32 * j * a.n_stride);
-          }
-        }
-      }
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < MF; ++i) {
-      const int64_t m = bm * BM + (wm * MF + i) * 32 + col_in_frag;
-      if (m >= a.M)
-        continue;
-      long long sum;
-      int sh;
-      if constexpr (kUnfold) { // the block's own rows, left in LDS by unfold_main_loop
-        constexpr int kMetaOff = unfold_meta_off(BM, BN, kWavesM, kWavesN, kWavesK);
-        sum = reinterpret_cast<const long long *>(smem + kMetaOff)[m - bm * BM];
-        sh = reinterpret_cast<const int32_t *>(smem + kMetaOff + 384)[m - bm * BM];
-      } else {
-        sum = a.use_sums ? a.sums[m] : 0;
-        sh = plain_shift(a.shift[m]);
-      }
-      const int s_hi = (int)(sum >> 16), s_lo = (int)(sum & 0xffff);
-      float *row = row_ptr(m);
-#pragma unroll
+  // The stores run in two copies, with and without reading y back first (k chunks after the first add to it): with
+  // the loads of the accumulating form anywhere in the same code the compiler waits for all outstanding memory
+  // operations before every output (the loads might be pending), and stores are outstanding memory operations, so
+  // each store would wait for the one before it.  Likewise with and without the bound checks a block on the edge
+  // of the output needs (a branch on the execution mask per store).
+  auto store_tile = [&](auto accumulate_c, auto inside_c) __attribute__((always_inline)) {
+    constexpr bool kAcc = decltype(accumulate_c)::value;
+    constexpr bool kInside = decltype(inside_c)::value; // every row and column of the block is stored: no checks
+    auto finish = [&](float v, float prev, float al, float bi) {
+      if (kAcc)
+        v = prev + v;
+      if (use_alpha)
+        v = v * al;
+      if (use_bias)
+        v = v + bi;
+      return v;
+    };
+    if (!kSwap) {
+      const int64_t ncol0 = a.n_begin + bn * BN + wn * NF * 32 + col_in_frag;
+      float al[NF], bi[NF];
+  #pragma unroll
       for (int j = 0; j < NF; ++j) {
-#pragma unroll
+        al[j] = epi_alpha[wn * NF * 32 + col_in_frag + 32 * j];
+        bi[j] = epi_bias[wn * NF * 32 + col_in_frag + 32 * j];
+      }
+  #pragma unroll
+      for (int i = 0; i < MF; ++i) {
+        const int64_t m0 = bm * BM + (wm * MF + i) * 32 + 4 * row_half;
+  #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
-          const int64_t n0 = a.n_begin + bn * BN + (wn * NF + j) * 32 + 4 * row_half + 8 * rq;
-          float al[4], bi[4], prev[4];
-#pragma unroll
+          // rows m0 + 8 rq + 0..3 (the metadata arrays are padded to whole row blocks)
+          const int64_t mq = m0 + 8 * rq;
+          const int rl = (wm * MF + i) * 32 + 4 * row_half + 8 * rq; // the same rows inside the block
+          const i32x4_t sum01 = *reinterpret_cast<const i32x4_t *>(epi_sums + rl); // two int64 as (lo, hi) words
+          const i32x4_t sum23 = *reinterpret_cast<const i32x4_t *>(epi_sums + rl + 2);
+          i32x4_t sh = *reinterpret_cast<const i32x4_t *>(epi_shift + rl);
+  #pragma unroll
+          for (int e = 0; e < 4; ++e)
+            sh[e] = plain_shift(sh[e]); // one-digit rows store their shift with a bias (kBadRow is negative: unchanged)
+          // sum = s_hi * 65536 + s_lo with s_lo in [0, 65536)
+          const uint32_t lo_w[4] = {(uint32_t)sum01.x, (uint32_t)sum01.z, (uint32_t)sum23.x, (uint32_t)sum23.z};
+          const int hi_w[4] = {sum01.y, sum01.w, sum23.y, sum23.w};
+          int s_hi[4], s_lo[4];
+  #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            if constexpr (kUnfold) { // left in LDS by unfold_main_loop (1 and 0 where there is no alpha / bias)
-              constexpr int kMetaOff = unfold_meta_off(BM, BN, kWavesM, kWavesN, kWavesK);
-              const float *s_alpha = reinterpret_cast<const float *>(smem + kMetaOff + 512 + 64 * 16);
-              const int col = (int)(n0 + e - a.n_begin - bn * BN);
-              al[e] = s_alpha[col];
-              bi[e] = s_alpha[256 + col];
-            } else {
-              const int64_t n = (n0 + e < a.N) ? n0 + e : a.N - 1;
-              al[e] = use_alpha ? a.alpha[n] : 1.0f;
-              bi[e] = use_bias ? a.bias[n] : 0.0f;
-            }
+            s_hi[e] = (int)((lo_w[e] >> 16) | ((uint32_t)hi_w[e] << 16));
+            s_lo[e] = (int)(lo_w[e] & 0xffffu);
           }
-          float *p = row + n0 * a.n_stride;
-          if (a.accumulate) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              prev[e] = (n0 + e < a.n_end) ? p[e * a.n_stride] : 0.0f;
-          }
-#pragma unroll
+  #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int r = 4 * rq + e;
-            float v = finish_dot(acc[0][i][j][r], acc[1][i][j][r], acc[2][i][j][r], s_hi, s_lo, sh, frag0 + j);
-            if (sh == kBadRow)
-              v = __builtin_nanf("");
-            v = finish(v, prev[e], al[e], bi[e]);
-            if (n0 + e < a.n_end)
-              __builtin_nontemporal_store(v, p + e * a.n_stride);
+            if (!kInside && mq + e >= a.M)
+              continue;
+            float *row = row_ptr(mq + e) + ncol0 * a.n_stride;
+            float prev[NF];
+            if (kAcc) {
+  #pragma unroll
+              for (int j = 0; j < NF; ++j)
+                prev[j] = (kInside || ncol0 + 32 * j < a.n_end) ? row[32 * j * a.n_stride] : 0.0f;
+            }
+  #pragma unroll
+            for (int j = 0; j < NF; ++j) {
+              float v = finish_dot(acc[0][i][j][r], acc[1][i][j][r], acc[2][i][j][r], s_hi[e], s_lo[e], sh[e],
+                                   frag0 + j);
+              if (sh[e] == kBadRow)
+                v = __builtin_nanf("");
+              v = finish(v, prev[j], al[j], bi[j]);
+              if (kInside || ncol0 + 32 * j < a.n_end)
+                __builtin_nontemporal_store(v, row + 32 * j * a.n_stride);
+            }
+          }
+        }
+      }
+    } else {
+  #pragma unroll
+      for (int i = 0; i < MF; ++i) {
+        const int64_t m = bm * BM + (wm * MF + i) * 32 + col_in_frag;
+        if (!kInside && m >= a.M)
+          continue;
+        long long sum;
+        int sh;
+        if constexpr (kUnfold) { // the block's own rows, left in LDS by unfold_main_loop
+          constexpr int kMetaOff = unfold_meta_off(BM, BN, kWavesM, kWavesN, kWavesK);
+          sum = reinterpret_cast<const long long *>(smem + kMetaOff)[m - bm * BM];
+          sh = reinterpret_cast<const int32_t *>(smem + kMetaOff + 384)[m - bm * BM];
+        } else {
+          sum = epi_sums[m - bm * BM];
+          sh = plain_shift(epi_shift[m - bm * BM]);
+        }
+        const int s_hi = (int)(sum >> 16), s_lo = (int)(sum & 0xffff);
+        float *row = row_ptr(m);
+  #pragma unroll
+        for (int j = 0; j < NF; ++j) {
+  #pragma unroll
+          for (int rq = 0; rq < 4; ++rq) {
+            const int64_t n0 = a.n_begin + bn * BN + (wn * NF + j) * 32 + 4 * row_half + 8 * rq;
+            float al[4], bi[4], prev[4];
+  #pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if constexpr (kUnfold) { // left in LDS by unfold_main_loop (1 and 0 where there is no alpha / bias)
+                constexpr int kMetaOff = unfold_meta_off(BM, BN, kWavesM, kWavesN, kWavesK);
+                const float *s_alpha = reinterpret_cast<const float *>(smem + kMetaOff + 512 + 64 * 16);
+                const int col = (int)(n0 + e - a.n_begin - bn * BN);
+                al[e] = s_alpha[col];
+                bi[e] = s_alpha[256 + col];
+              } else {
+                const int col = (wn * NF + j) * 32 + 4 * row_half + 8 * rq + e;
+                al[e] = epi_alpha[col];
+                bi[e] = epi_bias[col];
+              }
+            }
+            float *p = row + n0 * a.n_stride;
+            if (kAcc) {
+  #pragma unroll
+              for (int e = 0; e < 4; ++e)
+                prev[e] = (kInside || n0 + e < a.n_end) ? p[e * a.n_stride] : 0.0f;
+            }
+  #pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int r = 4 * rq + e;
+              float v = finish_dot(acc[0][i][j][r], acc[1][i][j][r], acc[2][i][j][r], s_hi, s_lo, sh, frag0 + j);
+              if (sh == kBadRow)
+                v = __builtin_nanf("");
+              v = finish(v, prev[e], al[e], bi[e]);
+              if (kInside || n0 + e < a.n_end)
+                __builtin_nontemporal_store(v, p + e * a.n_stride);
+            }
           }
         }
       }
     }
+  };
+  const bool inside = (bm + 1) * BM <= a.M && a.n_begin + (bn + 1) * BN <= a.n_end;
+  if (a.accumulate) {
+    if (inside)
+      store_tile(std::true_type(), std::true_type());
+    else
+      store_tile(std::true_type(), std::false_type());
+  } else {
+    if (inside)
+      store_tile(std::false_type(), std::true_type());
+    else
+      store_tile(std::false_type(), std::false_type());
   }
 #endif
 }
@@ -859,7 +960,7 @@ __global__ __launch_bounds__(512, 1) void gemm_bits_unfold_kernel(GemmBitsArgs a
 template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, bool kSwap>
 int launch_tile(const GemmBitsArgs &args, hipStream_t stream, unsigned splits = 1) {
   constexpr int kThreads = kWavesM * kWavesN * kWavesK * 64;
-  constexpr int kSmem = gemm_bits_lds_bytes(BM, BN, kWavesM, kWavesN, kWavesK);
+  constexpr int kSmem = gemm_bits_lds_bytes(BM, BN, kWavesM, kWavesN, kWavesK) + gemm_bits_epilogue_bytes(BM, BN);
   auto kernel = gemm_bits_kernel<BM, BN, kWavesM, kWavesN, kWavesK, kSwap>;
   static std::atomic<uint64_t> configured{0};
   const int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), kSmem, configured,

@@ -71,6 +71,10 @@ int main() {
     // one step of prefetch more than the ring has buffers for
     printf(" %d", check(two_tile_program(stages + 1, stages, 0, steps), stages));
     printf("\n");
+    printf("read_ahead %d %d %d %d %d\n", stages, read_ahead_loop_wait(stages, depth),
+           check(read_ahead_program(depth, depth - 1, depth - 2 < 0 ? 0 : depth - 2, steps), stages),
+           check(read_ahead_program(depth, depth - 1, depth - 1, steps), stages),
+           check(read_ahead_program(stages + 1, stages, 0, steps), stages));
     printf("one_tile %d %d %d %d %d\n", stages, one_tile_loop_wait(stages, depth),
            check(one_tile_program(depth, depth - 1, steps), stages), check(one_tile_program(depth, depth, steps), stages),
            check(one_tile_program(stages, 0, steps), stages));
@@ -123,6 +127,18 @@ def test_digit_loop_allowances(table):
         assert full_ring == 2  # a ring with no spare buffer: the copy lands in the buffer being multiplied
 
 
+def test_one_digit_loop_allowances(table):
+    """The bit-weight kernel's loop for one-digit rows reads step ks+1 at the top of step ks: before that read the
+    copies reach step ks + depth - 1, so depth - 2 steps may stay in flight; one step more in flight than the ring
+    has buffers overwrites the step being read."""
+    for stages, loop, shipped, one_more, too_deep in table["read_ahead"]:
+        depth = stages - 1
+        if stages == 2:
+            assert loop == -1
+            continue
+        assert loop == depth - 2 and shipped == 0 and one_more == 1 and too_deep == 2
+
+
 def test_counter_width(table):
     assert table["fits"] == [[1, 0, 1]]
 
@@ -131,7 +147,8 @@ def test_kernels_take_their_waits_from_the_model():
     bits = open(os.path.join(KERNELS, "gemm_bits.hip")).read()
     digits = open(os.path.join(KERNELS, "gemm_digits.hip")).read()
     waits = re.findall(r"wait_copies\(std::integral_constant<int, ([^>]+)>", bits)
-    assert waits and set(waits) <= {"kPrologueWait", "kLoopWait"}, waits
+    assert waits and set(waits) <= {"kPrologueWait", "kLoopWait", "kAheadWait"}, waits
+    assert "pipeline::read_ahead_safe(kStages, kDepth, kPrologueWait, kAheadWait)" in bits
     assert "pipeline::two_tile_safe(kStages, kDepth, kPrologueWait, kLoopWait)" in bits
     loop_waits = [w for w in re.findall(r"^ +NBLA_WAIT_VMCNT\(([^;\n]+)\);", digits, re.M) if w.strip() != "0"]
     assert loop_waits == ["kLoopWait * kCopies"], loop_waits
