@@ -14,6 +14,8 @@
 #include "gemm_layout.hpp"
 #include "internal.hpp"
 
+#include <type_traits>
+
 namespace nbla_hip {
 namespace {
 
@@ -284,51 +286,61 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
     const int64_t last = a.a_row_blocks * kFragRows - 1;
     row_shift[i] = plain_shift(a.ashift[m < last ? m : last]);
   }
+  // Two copies of the stores, with and without reading y back first: with that load anywhere in the loop the
+  // compiler waits for all outstanding memory operations before every output, and the stores before it are
+  // outstanding memory operations -- each store would wait for the previous one.
+  auto store_rows = [&](auto accumulate_c) __attribute__((always_inline)) {
+    constexpr bool kAcc = decltype(accumulate_c)::value;
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    if (kGroups == 2 && i != group)
-      continue;
-    const int64_t m0 = bm * kBM + (wm * 2 + i) * 32;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = 8 * (r >> 2) + 4 * row_half + (r & 3);
-      const int32_t sa_m = __shfl(row_shift[i], row);
-      const int64_t m = m0 + row;
-      if (m >= a.M)
+    for (int i = 0; i < 2; ++i) {
+      if (kGroups == 2 && i != group)
         continue;
-      int64_t off;
-      if (inner == 1u) {
-        off = m * a.outer_stride;
-      } else {
-        const uint32_t mu = (uint32_t)m, q = mu / inner; // m < 2^31: operand rows are counted in 32 bits
-        off = (int64_t)q * a.outer_stride + (mu - q * inner);
-      }
+      const int64_t m0 = bm * kBM + (wm * 2 + i) * 32;
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        if (n_col[j] >= a.N)
+      for (int r = 0; r < 16; ++r) {
+        const int row = 8 * (r >> 2) + 4 * row_half + (r & 3);
+        const int32_t sa_m = __shfl(row_shift[i], row);
+        const int64_t m = m0 + row;
+        if (m >= a.M)
           continue;
-        float v;
-        if (sa_m == kBadRow || sb_n[j] == kBadRow) {
-          v = __uint_as_float(0x7fc00000u);
+        int64_t off;
+        if (inner == 1u) {
+          off = m * a.outer_stride;
         } else {
-          // t = acc0 * 2^16 + acc1 * 2^8 + acc2 regrouped as hi * 2^16 + lo with 0 <= lo < 2^17 and |hi| < 2^30 (32-bit
-          // integer steps only), then one fused multiply-add: exact while |hi| < 2^24, else rounded twice (2^-24 of t)
-          const int a0 = acc[i][j][0][r], a1 = acc[i][j][1][r], a2 = acc[i][j][2][r];
-          const int hi = a0 + (a1 >> 8) + (a2 >> 16);
-          const int lo = ((a1 & 0xff) << 8) + (a2 & 0xffff);
-          const float t = fmaf((float)hi, 65536.0f, (float)lo);
-          // the two shifts are applied one after the other: each stays inside ldexpf's exponent range
-          v = ldexpf(ldexpf(t, (kNarrow ? 0 : 16) - sa_m), -sb_n[j]);
+          const uint32_t mu = (uint32_t)m, q = mu / inner; // m < 2^31: operand rows are counted in 32 bits
+          off = (int64_t)q * a.outer_stride + (mu - q * inner);
         }
-        float *dst = a.y + off + n_col[j] * a.n_stride;
-        if (a.accumulate)
-          v = *dst + v;
-        if (add_bias)
-          v = v + bias_n[j];
-        *dst = v;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          if (n_col[j] >= a.N)
+            continue;
+          float v;
+          if (sa_m == kBadRow || sb_n[j] == kBadRow) {
+            v = __uint_as_float(0x7fc00000u);
+          } else {
+            // t = acc0 * 2^16 + acc1 * 2^8 + acc2 regrouped as hi * 2^16 + lo with 0 <= lo < 2^17 and |hi| < 2^30 (32-bit
+            // integer steps only), then one fused multiply-add: exact while |hi| < 2^24, else rounded twice (2^-24 of t)
+            const int a0 = acc[i][j][0][r], a1 = acc[i][j][1][r], a2 = acc[i][j][2][r];
+            const int hi = a0 + (a1 >> 8) + (a2 >> 16);
+            const int lo = ((a1 & 0xff) << 8) + (a2 & 0xffff);
+            const float t = fmaf((float)hi, 65536.0f, (float)lo);
+            // the two shifts are applied one after the other: each stays inside ldexpf's exponent range
+            v = ldexpf(ldexpf(t, (kNarrow ? 0 : 16) - sa_m), -sb_n[j]);
+          }
+          float *dst = a.y + off + n_col[j] * a.n_stride;
+          if (kAcc)
+            v = *dst + v;
+          if (add_bias)
+            v = v + bias_n[j];
+          *dst = v;
+        }
       }
     }
-  }
+  };
+  if (a.accumulate)
+    store_rows(std::true_type());
+  else
+    store_rows(std::false_type());
 #endif
 }
 
