@@ -148,13 +148,14 @@ __global__ __launch_bounds__(kBlk) void inq_restore_absmax(float *__restrict__ W
 
 // n1, n2 and the pruning threshold (inq_affine.cpp:157-166).  `levels` is the
 // host's (int)pow(2, num_bits - 2).
-__global__ __launch_bounds__(64) void inq_finalize(const uint32_t *__restrict__ partial, int nparts, int levels,
+constexpr int kFinalizeThreads = 1024; // one round trip for the up to kMaxPartials partial maxima
+__global__ __launch_bounds__(kFinalizeThreads) void inq_finalize(const uint32_t *__restrict__ partial, int nparts, int levels,
                                                    const uint32_t *__restrict__ n1_cuts, InqParams *__restrict__ params,
                                                    ColumnScratch cols) {
   // the column statistics that the quantize pass will gather (cols.cmax null: none wanted) start from their neutral
   // values
   if (cols.cmax) {
-    for (int64_t i = threadIdx.x; i < cols.rows; i += 64) {
+    for (int64_t i = threadIdx.x; i < cols.rows; i += kFinalizeThreads) {
       cols.cmax[i] = 0u;
       cols.cmin[i] = 0xffffffffu;
     }
@@ -162,15 +163,21 @@ __global__ __launch_bounds__(64) void inq_finalize(const uint32_t *__restrict__ 
       *cols.flag = 0;
   }
   uint32_t mx = 0u;
-  for (int i = threadIdx.x; i < nparts; i += 64)
+  for (int i = threadIdx.x; i < nparts; i += kFinalizeThreads)
     mx = partial[i] > mx ? partial[i] : mx;
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) {
     const uint32_t o = __shfl_xor(mx, off);
     mx = o > mx ? o : mx;
   }
+  __shared__ uint32_t s_mx[kFinalizeThreads / 64];
+  if ((threadIdx.x & 63) == 0)
+    s_mx[threadIdx.x >> 6] = mx;
+  __syncthreads();
   if (threadIdx.x != 0)
     return;
+  for (int w = 1; w < kFinalizeThreads / 64; ++w)
+    mx = s_mx[w] > mx ? s_mx[w] : mx;
   if (mx == 0u)
     mx = 0x3f800000u; // max_absval == 0 -> 1
   int n1;
@@ -629,7 +636,7 @@ int update_weights(float *W, int *I, float *old_W, int *old_I, int64_t size, int
                          aligned16(I) && aligned16(old_W) && aligned16(old_I);
   ColumnScratch none;
   none.cmax = none.cmin = nullptr, none.flag = nullptr, none.rows = 0;
-  hipLaunchKernelGGL(inq_finalize, dim3(1), dim3(64), 0, stream, partial, (int)nparts, levels,
+  hipLaunchKernelGGL(inq_finalize, dim3(1), dim3(kFinalizeThreads), 0, stream, partial, (int)nparts, levels,
                      device_cut_table(kCutInqN1), params, with_cols ? *cols : none);
   NBLA_HIP_LAUNCH_CHECK("inq_finalize");
   if (with_cols) {
