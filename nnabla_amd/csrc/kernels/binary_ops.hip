@@ -10,8 +10,9 @@ namespace {
 // Rows of x holding a NaN or an infinity cannot be scaled to integers: the digit operand marks them (shift == kBadRow)
 // and the matrix-core product leaves NaN in their whole output row.  The reference's product propagates such values
 // element by element (affine.cpp:87-95: Inf * w = +-Inf, Inf - Inf = NaN, NaN anywhere = NaN), so those rows -- rare --
-// are recomputed here as plain fp32 dot products over the materialised weights Wb (* alpha).  Block b looks at rows
-// b, b + gridDim.x, ...; a launch that finds no marked row costs its launch only.
+// are recomputed as plain fp32 dot products over the materialised weights Wb (* alpha): by the kernel that splits x
+// into digits where that kernel is the one-pass form (the product then leaves the rows alone), by this kernel after
+// the product otherwise.  Block b looks at rows b, b + gridDim.x, ...
 __global__ __launch_bounds__(256) void affine_redo_marked_rows(const float *__restrict__ x, const float *__restrict__ Wb,
                                                                const float *__restrict__ alpha,
                                                                const float *__restrict__ bias, float *__restrict__ y,
@@ -98,18 +99,24 @@ int binary_affine_forward(const float *x, const float *W, float *Wb, float *alph
     if (host_count != 0)
       return launch_gemm_f32(x, Wb, alpha, bias, y, M, K, N, as_stream(stream_));
   }
-  rc = nbla_hip_split_digits_f32(x, K, xsplit, M, K, stream_);
+  // rows of x with a NaN or an infinity: computed by the splitting kernel where it can, else after the product
+  const RowRedo redo{Wb, alpha, bias, y, N};
+  bool redone = false;
+  rc = launch_split_digits_rows_redo(x, K, nullptr, xsplit, M, K, &redo, &redone, as_stream(stream_));
   if (rc)
     return rc;
-  rc = nbla_hip_gemm_bits_f32(xsplit, bits, alpha, bias, y, M, K, N, 1, N, 1, base + ws.gemm_off, ws.gemm_bytes,
-                              stream_);
+  rc = launch_gemm_bits(xsplit, bits, alpha, bias, y, M, K, N, 1, N, 1, false, as_stream(stream_), false,
+                        base + ws.gemm_off, ws.gemm_bytes, redone);
   if (rc)
     return rc;
-  const int32_t *shift = reinterpret_cast<const int32_t *>(static_cast<const char *>(xsplit) + digit_operand(M, K).shift_off);
-  const unsigned blocks = (unsigned)(M < 256 ? M : 256);
-  hipLaunchKernelGGL(affine_redo_marked_rows, dim3(blocks), dim3(256), 0, as_stream(stream_), x, Wb, alpha, bias, y,
-                     shift, M, K, N);
-  NBLA_HIP_LAUNCH_CHECK("affine_redo_marked_rows");
+  if (!redone) {
+    const int32_t *shift =
+        reinterpret_cast<const int32_t *>(static_cast<const char *>(xsplit) + digit_operand(M, K).shift_off);
+    const unsigned blocks = (unsigned)(M < 256 ? M : 256);
+    hipLaunchKernelGGL(affine_redo_marked_rows, dim3(blocks), dim3(256), 0, as_stream(stream_), x, Wb, alpha, bias, y,
+                       shift, M, K, N);
+    NBLA_HIP_LAUNCH_CHECK("affine_redo_marked_rows");
+  }
   return NBLA_HIP_OK;
 }
 

@@ -694,6 +694,24 @@ __global__ __launch_bounds__(kPrepBlock) void split_digits_tiled(const float *__
   }
 }
 
+// A row of x holding a NaN or an infinity cannot be scaled to integers: its shift becomes kBadRow and a matrix-core
+// product can only leave NaN in its whole output row.  The reference's affine propagates such values element by
+// element (affine.cpp:87-95: Inf * w = +-Inf, Inf - Inf = NaN, NaN anywhere = NaN), so a caller that has the
+// materialised weights at hand lets the kernel that finds such a row -- rare -- compute its outputs right away, as
+// plain fp32 dot products in the reference's order, and tells the product to leave the row alone.
+__device__ __noinline__ void redo_marked_row(const float *__restrict__ xrow, const RowRedo &redo, int64_t m, int64_t K,
+                                             int threads) {
+  for (int64_t n = threadIdx.x; n < redo.N; n += threads) {
+    const float a = redo.alpha ? redo.alpha[n] : 1.0f;
+    float acc = 0.0f;
+    for (int64_t k = 0; k < K; ++k) {
+      const float w = redo.alpha ? redo.Wb[k * redo.N + n] * a : redo.Wb[k * redo.N + n]; // the weight as multiplied
+      acc = acc + xrow[k] * w;
+    }
+    redo.y[m * redo.N + n] = redo.bias ? acc + redo.bias[n] : acc;
+  }
+}
+
 // Scale and digits in one pass for rows of up to 16384 values (K % 4 == 0, 16-byte aligned rows): a block of eight
 // wavefronts keeps kRows rows in registers in fragment order.  Wavefront w owns the k tiles
 // [w * kSlots * kPer, (w + 1) * kSlots * kPer), kSlots = 32 / kRows; lane r + kRows * (g + 2 * ts) holds, for row r,
@@ -707,7 +725,7 @@ __global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const floa
                                                                        long long *__restrict__ sums,
                                                                        int32_t *__restrict__ shift,
                                                                        uint4_t *__restrict__ out, int64_t M, int64_t K,
-                                                                       int64_t k_tiles, int64_t rows) {
+                                                                       int64_t k_tiles, int64_t rows, RowRedo redo) {
   static_assert(kRows == 4 || kRows == 8 || kRows == 16, "rows per block");
   static_assert(kPer * 16 < 256, "a lane's partial sum of kPer * 16 values below 2^23 fits an int");
   constexpr int kSlots = 32 / kRows;
@@ -797,13 +815,23 @@ __global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const floa
     // one-digit row: every value sits in the top digit alone (all-zero and padding rows included)
     shift[m] = bad ? kBadRow : (any_low == 0u ? s + kOneDigitBias : s);
   }
+  if (redo.y) {
+    // lane rr of every wavefront holds row rr's verdict, the same in all wavefronts: the loop is uniform over the block
+    const unsigned long long marked = __ballot(bad);
+    for (int rr = 0; rr < kRows; ++rr) {
+      const int64_t mr = (int64_t)blockIdx.x * kRows + rr;
+      if (((marked >> rr) & 1ull) && mr < M)
+        redo_marked_row(x + mr * ldx, redo, mr, K, kFusedWaves * 64);
+    }
+  }
 }
 
 template <int kRows, int kPer>
 void launch_split_digits_rows(const float *x, int64_t ldx, const float *cs, long long *sums, int32_t *shift,
-                              uint4_t *out, int64_t M, int64_t K, const DigitOperand &d, hipStream_t stream) {
+                              uint4_t *out, int64_t M, int64_t K, const DigitOperand &d, const RowRedo &redo,
+                              hipStream_t stream) {
   hipLaunchKernelGGL((split_digits_rows<kRows, kPer>), dim3((unsigned)(d.rows / kRows)), dim3(kFusedWaves * 64), 0,
-                     stream, x, ldx, cs, sums, shift, out, M, K, d.k_tiles, d.rows);
+                     stream, x, ldx, cs, sums, shift, out, M, K, d.k_tiles, d.rows, redo);
 }
 
 // ---- digit operand of a transposed source: the operand's rows are the columns c of src [R, C] (row stride ld) and
@@ -1112,7 +1140,19 @@ int nbla_hip_split_digits_f32(const float *x, int64_t ldx, void *xdigits, int64_
 
 int nbla_hip_split_digits_scaled_f32(const float *x, int64_t ldx, const float *colscale, void *xdigits, int64_t M,
                                      int64_t K, void *stream_) {
+  return launch_split_digits_rows_redo(x, ldx, colscale, xdigits, M, K, nullptr, nullptr, as_stream(stream_));
+}
+
+} // extern "C"
+
+namespace nbla_hip {
+
+int launch_split_digits_rows_redo(const float *x, int64_t ldx, const float *colscale, void *xdigits, int64_t M,
+                                  int64_t K, const RowRedo *redo_in, bool *redone, hipStream_t stream) {
   const float *cs = colscale;
+  const RowRedo redo = (redo_in && !colscale) ? *redo_in : RowRedo{nullptr, nullptr, nullptr, nullptr, 0};
+  if (redone)
+    *redone = false;
   if (M <= 0 || K <= 0 || ldx < K)
     return fail(NBLA_HIP_ERR_VALUE, "invalid digit operand shape (M=%lld, K=%lld, ldx=%lld).", (long long)M,
                 (long long)K, (long long)ldx);
@@ -1121,7 +1161,6 @@ int nbla_hip_split_digits_scaled_f32(const float *x, int64_t ldx, const float *c
   int rc = ensure_init();
   if (rc)
     return rc;
-  hipStream_t stream = as_stream(stream_);
   const DigitOperand d = digit_operand(M, K);
   char *base = static_cast<char *>(xdigits);
   long long *sums = reinterpret_cast<long long *>(base + d.sum_off);
@@ -1143,7 +1182,7 @@ int nbla_hip_split_digits_scaled_f32(const float *x, int64_t ldx, const float *c
     }
     const int64_t per = ceil_div(kt, kFusedWaves * (32 / rows_per_block));
 #define NBLA_SPLIT_ROWS(R, P)                                                                                          \
-  launch_split_digits_rows<R, P>(x, ldx, cs, sums, shift, out, M, K, d, stream)
+  launch_split_digits_rows<R, P>(x, ldx, cs, sums, shift, out, M, K, d, redo, stream)
     if (rows_per_block == 16) {
       if (per <= 1)
         NBLA_SPLIT_ROWS(16, 1);
@@ -1180,6 +1219,8 @@ int nbla_hip_split_digits_scaled_f32(const float *x, int64_t ldx, const float *c
     }
 #undef NBLA_SPLIT_ROWS
     NBLA_HIP_LAUNCH_CHECK("split_digits_rows");
+    if (redone)
+      *redone = redo.y != nullptr;
     return NBLA_HIP_OK;
   }
   const dim3 scale_grid((unsigned)ceil_div(d.rows, kPrepBlock / 64));
@@ -1203,4 +1244,4 @@ int nbla_hip_split_digits_scaled_f32(const float *x, int64_t ldx, const float *c
   return NBLA_HIP_OK;
 }
 
-} // extern "C"
+} // namespace nbla_hip

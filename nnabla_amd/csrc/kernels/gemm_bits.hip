@@ -54,6 +54,7 @@ struct GemmBitsArgs {
   // split 0 adds the row sums
   int64_t split_steps; // 0: no split
   int use_sums;
+  int keep_bad_rows; // rows marked kBadRow are left as they are in y (the caller has computed them) instead of NaN
   // unfolding product (gemm_bits_unfold_kernel): the rows are the unfolded windows of x, converted to digits in the
   // kernel; xd, sums and shift are unused
   const float *ux;
@@ -851,7 +852,7 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
               if (sh[e] == kBadRow)
                 v = __builtin_nanf("");
               v = finish(v, prev[j], al[j], bi[j]);
-              if (kInside || ncol0 + 32 * j < a.n_end)
+              if ((kInside || ncol0 + 32 * j < a.n_end) && !(sh[e] == kBadRow && a.keep_bad_rows))
                 __builtin_nontemporal_store(v, row + 32 * j * a.n_stride);
             }
           }
@@ -908,7 +909,7 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
               if (sh == kBadRow)
                 v = __builtin_nanf("");
               v = finish(v, prev[e], al[e], bi[e]);
-              if (kInside || n0 + e < a.n_end)
+              if ((kInside || n0 + e < a.n_end) && !(sh == kBadRow && a.keep_bad_rows))
                 __builtin_nontemporal_store(v, p + e * a.n_stride);
             }
           }
@@ -997,10 +998,13 @@ __global__ __launch_bounds__(256) void gemm_bits_split_sum(const float *__restri
                                                            int64_t N, float *__restrict__ y, int64_t inner,
                                                            int64_t outer_stride, int64_t n_stride,
                                                            const float *__restrict__ alpha,
-                                                           const float *__restrict__ bias, int accumulate) {
+                                                           const float *__restrict__ bias, int accumulate,
+                                                           const int32_t *__restrict__ keep_shift) {
   const int64_t total = M * N;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
     const int64_t m = i / N, n = i - m * N;
+    if (keep_shift && keep_shift[m] == kBadRow) // the caller has computed this row
+      continue;
     float v = partial[i];
     for (int z = 1; z < splits; ++z)
       v += partial[(int64_t)z * total + i];
@@ -1028,7 +1032,7 @@ template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream, vo
       splits = ceil_div(a.step_end - a.step_begin, part.split_steps);
       part.y = static_cast<float *>(split_ws);
       part.inner = 1, part.outer_stride = a.N, part.n_stride = 1;
-      part.accumulate = 0, part.finish = 0;
+      part.accumulate = 0, part.finish = 0, part.keep_bad_rows = 0;
       int rc = launch_tile<32, 256, 1, 2, 4, kSwap>(part, stream, (unsigned)splits);
       if (rc)
         return rc;
@@ -1037,7 +1041,8 @@ template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream, vo
         blocks = 4096;
       hipLaunchKernelGGL(gemm_bits_split_sum, dim3((unsigned)blocks), dim3(256), 0, stream,
                          static_cast<const float *>(split_ws), (int)splits, a.M, a.N, a.y, a.inner, a.outer_stride,
-                         a.n_stride, a.finish ? a.alpha : nullptr, a.finish ? a.bias : nullptr, a.accumulate);
+                         a.n_stride, a.finish ? a.alpha : nullptr, a.finish ? a.bias : nullptr, a.accumulate,
+                         a.keep_bad_rows ? a.shift : nullptr);
       NBLA_HIP_LAUNCH_CHECK("gemm_bits_split_sum");
       return NBLA_HIP_OK;
     }
@@ -1055,7 +1060,8 @@ template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream, vo
 
 int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alpha, const float *bias, float *y,
                      int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
-                     bool swap_out, hipStream_t stream, bool accumulate, void *split_ws, size_t split_ws_bytes) {
+                     bool swap_out, hipStream_t stream, bool accumulate, void *split_ws, size_t split_ws_bytes,
+                     bool keep_bad_rows) {
   if (M <= 0 || K <= 0 || N <= 0 || inner <= 0 || M > 0x7fffffffll || inner > 0x7fffffffll)
     return fail(NBLA_HIP_ERR_VALUE, "invalid GEMM shape (M=%lld, K=%lld, N=%lld).", (long long)M, (long long)K,
                 (long long)N);
@@ -1087,6 +1093,7 @@ int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alp
   a.blocks_m = a.blocks_n = 0;
   a.split_steps = 0;
   a.use_sums = 1;
+  a.keep_bad_rows = keep_bad_rows ? 1 : 0;
   a.ux = nullptr;
   a.ugrp = 0;
   a.inner = inner;
@@ -1166,6 +1173,7 @@ int launch_gemm_bits_unfold(const float *x, const ConvGeom &g, int64_t grp, cons
   a.finish = 1;
   a.split_steps = 0;
   a.use_sums = 1;
+  a.keep_bad_rows = 0;
   a.ux = x;
   a.ug = g;
   a.ugrp = grp;

@@ -13,11 +13,12 @@ int launch_gemm_f32(const float *x, const float *w, const float *colscale, const
                     int64_t K, int64_t N, hipStream_t stream);
 
 // Bit-weight product with the choice of store orientation: swap_out makes consecutive lanes write consecutive m
-// (for outputs whose m index is the contiguous one, e.g. convolution results [batch, O, Ho*Wo]).
+// (for outputs whose m index is the contiguous one, e.g. convolution results [batch, O, Ho*Wo]).  keep_bad_rows: rows
+// of the digit operand marked as holding a non-finite value are left as they are in y instead of being set to NaN.
 int launch_gemm_bits(const void *xsplit, const uint32_t *bits, const float *alpha, const float *bias, float *y,
                      int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
                      bool swap_out, hipStream_t stream, bool accumulate = false, void *split_ws = nullptr,
-                     size_t split_ws_bytes = 0);
+                     size_t split_ws_bytes = 0, bool keep_bad_rows = false);
 // The same product for a convolution with the unfold fused in: the rows are the unfolded windows of x (group `grp`),
 // converted to digits inside the kernel; y is [sample, O, output position].  gemm_bits_unfold_applies tells whether
 // the geometry is covered (otherwise: launch_im2col_digits + launch_gemm_bits).
@@ -25,6 +26,18 @@ struct ConvGeom;
 bool gemm_bits_unfold_applies(const ConvGeom &g);
 int launch_gemm_bits_unfold(const float *x, const ConvGeom &g, int64_t grp, const uint32_t *bits, const float *alpha,
                             const float *bias, float *y, hipStream_t stream);
+// Digit operand of the rows of x (nbla_hip_split_digits_scaled_f32) for a caller that holds materialised weights
+// Wb [K, N] (* alpha[n], + bias[n]): rows holding a NaN or an infinity get their outputs y[m, :] computed by the
+// splitting kernel itself, as fp32 dot products in the reference's order.  *redone tells whether that happened (only
+// the one-pass kernel for rows of up to 16384 values does it, and only without a column scale); the product is then
+// launched with keep_bad_rows, otherwise the caller recomputes those rows after the product.
+struct RowRedo {
+  const float *Wb, *alpha, *bias;
+  float *y;
+  int64_t N;
+};
+int launch_split_digits_rows_redo(const float *x, int64_t ldx, const float *colscale, void *xdigits, int64_t M,
+                                  int64_t K, const RowRedo *redo, bool *redone, hipStream_t stream);
 // Scratch that lets launch_gemm_bits spread the contraction of a very small output (M <= 64 or so) over the CUs.
 size_t gemm_bits_split_bytes(int64_t M, int64_t K, int64_t N);
 
