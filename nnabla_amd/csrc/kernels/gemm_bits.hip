@@ -86,18 +86,36 @@ constexpr int gemm_bits_epilogue_bytes(int BM, int BN) { return (BM * 12 + BN * 
 // sum_k q_k * (+-1) as fp32 from the three digit accumulators and the row sum (hi * 65536 + lo), scaled by 2^-shift.
 // Integer arithmetic up to the last step: the high and low parts are combined by one fused multiply-add, whose
 // operands are exact (|hi part| < 2^24, low part reduced to 16 bits).
-__device__ __forceinline__ float finish_dot(int a0, int a1, int a2, int s_hi, int s_lo, int shift, int frag) {
-  // accumulators of column fragment `frag` carry the factor 2^frag, or -128 for frag 7 (0x80 as int8)
-  a0 >>= frag, a1 >>= frag, a2 >>= frag;
-  if (frag == 7)
-    a0 = -a0, a1 = -a1, a2 = -a2;
-  int u = s_hi - 2 * a0;
-  int v = s_lo - 2 * (a1 * 256 + a2);
+//
+// The accumulators of column fragment `frag` carry the factor 2^frag (-128 for frag 7: 0x80 as int8); without it a
+// digit sum m_d is below 2^21 in magnitude (at most kChunkK products of magnitude 128), so the sign of the factor and
+// the weights -2, -512, -2 of  rowsum - 2 (m_0 65536 + m_1 256 + m_2)  go into 24-bit multiply-adds.
+// A row that holds a non-finite value gets hi_scale = NaN instead of 65536 (its digits are all zero): NaN comes out.
+struct FragScale {
+  int shift;             // frag
+  int c_hi, c_mid, c_lo; // -2, -512, -2, negated for frag 7
+};
+__device__ __forceinline__ FragScale frag_scale(int frag) {
+  const int sgn = frag == 7 ? -1 : 1;
+  FragScale f{frag, -2 * sgn, -512 * sgn, -2 * sgn};
+  // kept in scalar registers as values the compiler does not see through: a known multiplier makes it expand the
+  // 24-bit multiply-add into shifts with a sign extension of the other factor, three instructions for one
+  asm volatile("" : "+s"(f.c_hi), "+s"(f.c_mid), "+s"(f.c_lo));
+  return f;
+}
+__device__ __forceinline__ float finish_dot(int a0, int a1, int a2, int s_hi, int s_lo, int neg_shift, float hi_scale,
+                                            const FragScale &f) {
+  const int m0 = a0 >> f.shift, m1 = a1 >> f.shift, m2 = a2 >> f.shift;
+  int u = __mul24(m0, f.c_hi) + s_hi;
+  int v = __mul24(m1, f.c_mid) + (__mul24(m2, f.c_lo) + s_lo);
   u += v >> 16;
   v &= 0xffff;
-  const float r = fmaf((float)u, 65536.0f, (float)v);
-  return ldexpf(r, -shift);
+  const float r = fmaf((float)u, hi_scale, (float)v);
+  return ldexpf(r, neg_shift);
 }
+// per row: the exponent and the high part's scale
+__device__ __forceinline__ int row_neg_shift(int shift) { return shift == kBadRow ? 0 : -shift; }
+__device__ __forceinline__ float row_hi_scale(int shift) { return shift == kBadRow ? __builtin_nanf("") : 65536.0f; }
 
 // Workgroup barrier without the memory fence of __syncthreads(): the fence would wait for every outstanding
 // global -> LDS copy, including those issued for later k steps.  The waits that matter are explicit (wait_copies);
@@ -211,7 +229,7 @@ __device__ __forceinline__ void unfold_main_loop(const GemmBitsArgs &a, unsigned
       const int64_t col = a.n_begin + bn * BN + tid;
       const int64_t nc = col < a.N ? col : a.N - 1;
       s_alpha[tid] = (a.finish && a.alpha) ? a.alpha[nc] : 1.0f;
-      s_bias[tid] = (a.finish && a.bias) ? a.bias[nc] : 0.0f;
+      s_bias[tid] = (a.finish && a.bias) ? a.bias[nc] : -0.0f;
     }
   }
   // this thread's row (the same for both of its roles: lane % 32)
@@ -530,7 +548,7 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
       const int64_t n = a.n_begin + bn * BN + c * kThreadsAll + tid;
       const int64_t nc = n < a.N ? n : a.N - 1;
       meta_alpha[c] = (a.finish && a.alpha) ? a.alpha[nc] : 1.0f;
-      meta_bias[c] = (a.finish && a.bias) ? a.bias[nc] : 0.0f;
+      meta_bias[c] = (a.finish && a.bias) ? a.bias[nc] : -0.0f;
     }
   }
   auto store_epilogue_metadata = [&]() __attribute__((always_inline)) {
@@ -778,7 +796,6 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
   // Everything an output element needs besides its accumulators (row sums and shift, alpha, bias) is loaded into
   // registers before the stores of the group it belongs to: the compiler cannot move a load across a store to y.
   const int col_in_frag = lane & 31, row_half = lane >> 5;
-  const bool use_alpha = a.finish && a.alpha, use_bias = a.finish && a.bias;
   // start of output row m (32-bit division: M and inner are below 2^31)
   auto row_ptr = [&](int64_t m) {
     const uint32_t mu = (uint32_t)m, in = (uint32_t)a.inner;
@@ -793,15 +810,18 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
   auto store_tile = [&](auto accumulate_c, auto inside_c) __attribute__((always_inline)) {
     constexpr bool kAcc = decltype(accumulate_c)::value;
     constexpr bool kInside = decltype(inside_c)::value; // every row and column of the block is stored: no checks
+    // al is 1 and bi is -0 where there is no alpha / bias (or this is not the last k chunk): exact identities
     auto finish = [&](float v, float prev, float al, float bi) {
       if (kAcc)
         v = prev + v;
-      if (use_alpha)
-        v = v * al;
-      if (use_bias)
-        v = v + bi;
+      v = v * al;
+      v = v + bi;
       return v;
     };
+    FragScale fs[NF];
+  #pragma unroll
+    for (int j = 0; j < NF; ++j)
+      fs[j] = frag_scale(frag0 + j);
     if (!kSwap) {
       const int64_t ncol0 = a.n_begin + bn * BN + wn * NF * 32 + col_in_frag;
       float al[NF], bi[NF];
@@ -827,16 +847,21 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
           // sum = s_hi * 65536 + s_lo with s_lo in [0, 65536)
           const uint32_t lo_w[4] = {(uint32_t)sum01.x, (uint32_t)sum01.z, (uint32_t)sum23.x, (uint32_t)sum23.z};
           const int hi_w[4] = {sum01.y, sum01.w, sum23.y, sum23.w};
-          int s_hi[4], s_lo[4];
+          int s_hi[4], s_lo[4], neg_sh[4];
+          float hi_scale[4];
   #pragma unroll
           for (int e = 0; e < 4; ++e) {
             s_hi[e] = (int)((lo_w[e] >> 16) | ((uint32_t)hi_w[e] << 16));
             s_lo[e] = (int)(lo_w[e] & 0xffffu);
+            neg_sh[e] = row_neg_shift(sh[e]);
+            hi_scale[e] = row_hi_scale(sh[e]);
           }
   #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int r = 4 * rq + e;
             if (!kInside && mq + e >= a.M)
+              continue;
+            if (sh[e] == kBadRow && a.keep_bad_rows) // the caller has computed this row
               continue;
             float *row = row_ptr(mq + e) + ncol0 * a.n_stride;
             float prev[NF];
@@ -847,12 +872,10 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
             }
   #pragma unroll
             for (int j = 0; j < NF; ++j) {
-              float v = finish_dot(acc[0][i][j][r], acc[1][i][j][r], acc[2][i][j][r], s_hi[e], s_lo[e], sh[e],
-                                   frag0 + j);
-              if (sh[e] == kBadRow)
-                v = __builtin_nanf("");
+              float v = finish_dot(acc[0][i][j][r], acc[1][i][j][r], acc[2][i][j][r], s_hi[e], s_lo[e], neg_sh[e],
+                                   hi_scale[e], fs[j]);
               v = finish(v, prev[j], al[j], bi[j]);
-              if ((kInside || ncol0 + 32 * j < a.n_end) && !(sh[e] == kBadRow && a.keep_bad_rows))
+              if (kInside || ncol0 + 32 * j < a.n_end)
                 __builtin_nontemporal_store(v, row + 32 * j * a.n_stride);
             }
           }
@@ -875,6 +898,10 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
           sh = plain_shift(epi_shift[m - bm * BM]);
         }
         const int s_hi = (int)(sum >> 16), s_lo = (int)(sum & 0xffff);
+        if (sh == kBadRow && a.keep_bad_rows) // the caller has computed this row
+          continue;
+        const int neg_sh = row_neg_shift(sh);
+        const float hi_scale = row_hi_scale(sh);
         float *row = row_ptr(m);
   #pragma unroll
         for (int j = 0; j < NF; ++j) {
@@ -884,7 +911,7 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
             float al[4], bi[4], prev[4];
   #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              if constexpr (kUnfold) { // left in LDS by unfold_main_loop (1 and 0 where there is no alpha / bias)
+              if constexpr (kUnfold) { // left in LDS by unfold_main_loop (1 and -0 where there is no alpha / bias)
                 constexpr int kMetaOff = unfold_meta_off(BM, BN, kWavesM, kWavesN, kWavesK);
                 const float *s_alpha = reinterpret_cast<const float *>(smem + kMetaOff + 512 + 64 * 16);
                 const int col = (int)(n0 + e - a.n_begin - bn * BN);
@@ -905,11 +932,10 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
   #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int r = 4 * rq + e;
-              float v = finish_dot(acc[0][i][j][r], acc[1][i][j][r], acc[2][i][j][r], s_hi, s_lo, sh, frag0 + j);
-              if (sh == kBadRow)
-                v = __builtin_nanf("");
+              float v = finish_dot(acc[0][i][j][r], acc[1][i][j][r], acc[2][i][j][r], s_hi, s_lo, neg_sh, hi_scale,
+                                   fs[j]);
               v = finish(v, prev[e], al[e], bi[e]);
-              if ((kInside || n0 + e < a.n_end) && !(sh == kBadRow && a.keep_bad_rows))
+              if (kInside || n0 + e < a.n_end)
                 __builtin_nontemporal_store(v, p + e * a.n_stride);
             }
           }
