@@ -456,7 +456,10 @@ int nbla_hip_dequantize_linear_backward_f32(const float *dy, const float *scale,
  * |x| (+1 when rate == 1).  Replaces Prune<float>::forward_impl,
  * prune.cpp:27-70 (the full sort there is replaced by a radix select of that
  * one order statistic).  Its backward is the identity (prune.cpp:72-90):
- * use nbla_hip_fixed_point_quantize_backward_f32 with ste_fine_grained = 0. */
+ * use nbla_hip_fixed_point_quantize_backward_f32 with ste_fine_grained = 0.
+ * The workspace (about 8 MiB, independent of size; contents need not be
+ * cleared or kept between calls) holds the selection's histograms and the
+ * candidate keys its second pass hands to its third. */
 size_t nbla_hip_prune_workspace_bytes(void);
 int nbla_hip_prune_f32(const float *x, float *y, size_t size, float rate,
                        void *workspace, size_t workspace_bytes, void *stream);

@@ -343,7 +343,7 @@ __global__ __launch_bounds__(kHistBlock) void inq_select_histogram(const float *
   typedef float f4_t __attribute__((ext_vector_type(4)));
   typedef int i4_t __attribute__((ext_vector_type(4)));
   __shared__ uint32_t h[kMaxBins * kLdsCopies];
-  __shared__ uint32_t scratch[kHistBlock / 64 + 1];
+  __shared__ uint32_t scratch[kSelectScratch];
   const SelectPass sp = select_begin(h, st, pass);
   // pass 0 also finds the first index of the sorted order: the largest magnitude of all weights, lowest index first
   unsigned long long top = 0ull;

@@ -347,71 +347,183 @@ int quantize_range(int dtype, int narrow_range, float &lo, float &hi) {
 
 // ------------------------------------------------------------------------------------------------------ Prune
 
-// The rank-th smallest magnitude by the radix select of radix_select.hpp: keys are the 31 magnitude bits of x.
-__global__ __launch_bounds__(kHistBlock) void prune_histogram(const float *__restrict__ x, int64_t n4, int64_t n,
-                                                          SelectState *__restrict__ st, int pass) {
-  __shared__ uint32_t h[kMaxBins * kLdsCopies];
-  __shared__ uint32_t scratch[kHistBlock / 64 + 1];
-  const SelectPass sp = select_begin(h, st, pass);
-  auto count = [&](float v) { select_count(h, sp, __float_as_uint(v) & 0x7fffffffu); };
-  // four 16-byte loads per thread in flight while the previous four are counted
-  const int64_t tiles = (n4 + kHistBlock * 4 - 1) / (kHistBlock * 4);
-  auto fetch = [&](int64_t tile, float4_t (&v)[4]) __attribute__((always_inline)) {
-    const int64_t base = tile * (kHistBlock * 4) + threadIdx.x;
+// The rank-th smallest magnitude by the radix select of radix_select.hpp: keys are the 31 magnitude bits of x.  The
+// launches form a chain (three histogram passes, then the pass that writes y); each resolves the histogram its
+// predecessor left behind, every block for itself, while its first loads are already under way.
+//
+// The second pass also keeps the keys it counts -- those that share the first digit with the rank-th smallest, a few
+// percent of the data at most unless the magnitudes crowd into one binade -- in a per-block region of the workspace,
+// and the third pass reads those instead of x.  A block whose region is too small for its share (values of one
+// magnitude range clustered in one stretch of x) raises a flag, and the third pass then reads x as the others do.
+constexpr int kPruneLoads = 4;          // 16-byte loads per thread in flight
+constexpr int kCandPerBlock = 8192;     // candidate keys a block can keep
+struct PruneState {
+  SelectState sel;
+  uint32_t overflow;                    // some block found more candidates than its region holds
+  uint32_t counts[kSelectBlocks];       // candidates kept by each block of the second pass
+  uint32_t pad[3];
+  uint32_t cand[kSelectBlocks][kCandPerBlock];
+};
+
+__device__ __forceinline__ void prune_fetch(const float *__restrict__ x, int64_t n4, int64_t tile,
+                                            float4_t (&v)[kPruneLoads]) {
+  const int64_t base = tile * (kHistBlock * kPruneLoads) + threadIdx.x;
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (base + j * kHistBlock < n4)
-        v[j] = *reinterpret_cast<const float4_t *>(x + 4 * (base + j * kHistBlock));
+  for (int j = 0; j < kPruneLoads; ++j)
+    if (base + j * kHistBlock < n4)
+      v[j] = *reinterpret_cast<const float4_t *>(x + 4 * (base + j * kHistBlock));
+}
+
+__global__ __launch_bounds__(kHistBlock) void prune_histogram(const float *__restrict__ x, int64_t n4, int64_t n,
+                                                          PruneState *__restrict__ ps, int pass) {
+  __shared__ uint32_t h[kMaxBins * kLdsCopies];
+  __shared__ uint32_t scratch[kSelectScratch];
+  __shared__ uint32_t s_kept;
+  SelectState *st = &ps->sel;
+  const int64_t tiles = (n4 + kHistBlock * kPruneLoads - 1) / (kHistBlock * kPruneLoads);
+  const bool from_cand = pass == 2 && ps->overflow == 0u; // uniform over the grid
+  const bool any = (int64_t)blockIdx.x < tiles && !from_cand;
+  float4_t cur[kPruneLoads];
+  if (any)
+    prune_fetch(x, n4, blockIdx.x, cur);
+  if (threadIdx.x == 0) {
+    s_kept = 0u;
+    if (pass == 0 && blockIdx.x == 0)
+      ps->overflow = 0u;
+  }
+  const SelectPass sp = select_begin_at(h, select_resolve(scratch, st, pass), pass);
+  uint32_t *mine = ps->cand[blockIdx.x];
+  auto count = [&](float v) {
+    const uint32_t key = __float_as_uint(v) & 0x7fffffffu;
+    if (pass == 1) { // (only the few elements behind the last whole 16 bytes come this way in the second pass)
+      if ((key >> sp.above) == sp.want) {
+        atomicAdd(&h[((key >> sp.shift) & sp.mask) * kLdsCopies + sp.copy], 1u);
+        const uint32_t i = atomicAdd(&s_kept, 1u);
+        if (i < (uint32_t)kCandPerBlock)
+          mine[i] = key;
+      }
+    } else {
+      select_count(h, sp, key);
+    }
   };
-  if ((int64_t)blockIdx.x < tiles) {
-    float4_t cur[4];
-    fetch(blockIdx.x, cur);
+  // Second pass, one tile: count the keys that share the first digit and keep them.  Nearly all keys do not, so
+  // they are found without branches; a wavefront reserves room in the block's region for all its keys of the tile
+  // with one LDS atomic (a counter bumped once per key is a serial chain).
+  auto count_and_keep = [&](const float4_t (&v)[kPruneLoads], int64_t base) __attribute__((always_inline)) {
+    uint32_t found = 0u; // bit 4 j + e: element e of load j shares the digit
+#pragma unroll
+    for (int j = 0; j < kPruneLoads; ++j) {
+      const float e4[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+      const bool live = base + j * kHistBlock < n4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t key = __float_as_uint(e4[e]) & 0x7fffffffu;
+        found |= (live && (key >> sp.above) == sp.want) ? 1u << (4 * j + e) : 0u;
+      }
+    }
+    if (__ballot(found != 0u) == 0ull)
+      return;
+    const int lane = threadIdx.x & 63;
+    const uint32_t c = (uint32_t)__popc(found);
+    uint32_t incl = c;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const uint32_t up = __shfl_up(incl, off);
+      if (lane >= off)
+        incl += up;
+    }
+    uint32_t start = 0u;
+    if (lane == 63)
+      start = atomicAdd(&s_kept, incl);
+    uint32_t at = (uint32_t)__shfl((int)start, 63) + incl - c;
+#pragma unroll
+    for (int j = 0; j < kPruneLoads; ++j) {
+      const float e4[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (found & (1u << (4 * j + e))) {
+          const uint32_t key = __float_as_uint(e4[e]) & 0x7fffffffu;
+          atomicAdd(&h[((key >> sp.shift) & sp.mask) * kLdsCopies + sp.copy], 1u);
+          if (at < (uint32_t)kCandPerBlock)
+            mine[at] = key;
+          ++at;
+        }
+    }
+  };
+  if (from_cand) {
+    const uint32_t kept = ps->counts[blockIdx.x];
+    for (uint32_t i = threadIdx.x; i < kept; i += kHistBlock)
+      select_count(h, sp, mine[i]);
+  }
+  if (any) {
 #pragma clang loop unroll(disable)
     for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
       const int64_t next = tile + gridDim.x;
-      float4_t nxt[4];
+      float4_t nxt[kPruneLoads];
       if (next < tiles)
-        fetch(next, nxt);
-      const int64_t base = tile * (kHistBlock * 4) + threadIdx.x;
+        prune_fetch(x, n4, next, nxt);
+      const int64_t base = tile * (kHistBlock * kPruneLoads) + threadIdx.x;
+      if (pass == 1) {
+        count_and_keep(cur, base);
+      } else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (base + j * kHistBlock < n4)
-          count(cur[j].x), count(cur[j].y), count(cur[j].z), count(cur[j].w);
+        for (int j = 0; j < kPruneLoads; ++j)
+          if (base + j * kHistBlock < n4)
+            count(cur[j].x), count(cur[j].y), count(cur[j].z), count(cur[j].w);
+      }
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < kPruneLoads; ++j)
         cur[j] = nxt[j];
     }
   }
-  if (blockIdx.x == 0) {
+  if (blockIdx.x == 0 && !from_cand) {
     const int64_t i = 4 * n4 + threadIdx.x;
     if (i < n)
       count(x[i]);
   }
-  select_finish<false>(h, scratch, st, sp);
+  select_flush(h, st, sp); // (starts with a barrier: s_kept is final after it)
+  if (pass == 1 && threadIdx.x == 0) {
+    const uint32_t kept = s_kept;
+    ps->counts[blockIdx.x] = kept < (uint32_t)kCandPerBlock ? kept : (uint32_t)kCandPerBlock;
+    if (kept > (uint32_t)kCandPerBlock)
+      ps->overflow = 1u;
+  }
 }
 
 // y = (|x| < thresh) ? 0 : x with thresh = |rank-th smallest| (+ 1 when rate == 1), prune.cpp:62-69
-__global__ __launch_bounds__(kBlock) void prune_apply(const float *__restrict__ x, float *__restrict__ y, int64_t n4,
-                                                      int64_t n, const SelectState *__restrict__ st, float add) {
-  const float thresh = __uint_as_float(st->prefix[kPasses]) + add;
-  const int64_t tiles = (n4 + kBlock * 4 - 1) / (kBlock * 4);
-  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-    const int64_t base = tile * (kBlock * 4) + threadIdx.x;
-    float4_t v[4];
+__global__ __launch_bounds__(kHistBlock) void prune_apply(const float *__restrict__ x, float *__restrict__ y,
+                                                          int64_t n4, int64_t n, PruneState *__restrict__ ps,
+                                                          float add) {
+  __shared__ uint32_t scratch[kSelectScratch];
+  SelectState *st = &ps->sel;
+  const int64_t tiles = (n4 + kHistBlock * kPruneLoads - 1) / (kHistBlock * kPruneLoads);
+  const bool any = (int64_t)blockIdx.x < tiles;
+  float4_t cur[kPruneLoads];
+  if (any)
+    prune_fetch(x, n4, blockIdx.x, cur);
+  const float thresh = __uint_as_float(select_resolve(scratch, st, kPasses).prefix) + add;
+  if (any) {
+#pragma clang loop unroll(disable)
+    for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+      const int64_t next = tile + gridDim.x;
+      float4_t nxt[kPruneLoads];
+      if (next < tiles)
+        prune_fetch(x, n4, next, nxt);
+      const int64_t base = tile * (kHistBlock * kPruneLoads) + threadIdx.x;
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (base + j * kBlock < n4)
-        v[j] = *reinterpret_cast<const float4_t *>(x + 4 * (base + j * kBlock));
+      for (int j = 0; j < kPruneLoads; ++j)
+        if (base + j * kHistBlock < n4) {
+          float4_t o;
+          o.x = fabsf(cur[j].x) < thresh ? 0.0f : cur[j].x;
+          o.y = fabsf(cur[j].y) < thresh ? 0.0f : cur[j].y;
+          o.z = fabsf(cur[j].z) < thresh ? 0.0f : cur[j].z;
+          o.w = fabsf(cur[j].w) < thresh ? 0.0f : cur[j].w;
+          __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(y + 4 * (base + j * kHistBlock)));
+        }
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (base + j * kBlock < n4) {
-        float4_t o;
-        o.x = fabsf(v[j].x) < thresh ? 0.0f : v[j].x;
-        o.y = fabsf(v[j].y) < thresh ? 0.0f : v[j].y;
-        o.z = fabsf(v[j].z) < thresh ? 0.0f : v[j].z;
-        o.w = fabsf(v[j].w) < thresh ? 0.0f : v[j].w;
-        __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(y + 4 * (base + j * kBlock)));
-      }
+      for (int j = 0; j < kPruneLoads; ++j)
+        cur[j] = nxt[j];
+    }
   }
   if (blockIdx.x == 0) {
     const int64_t i = 4 * n4 + threadIdx.x;
@@ -499,7 +611,7 @@ int nbla_hip_dequantize_linear_backward_f32(const float *dy, const float *scale,
                           as_stream(stream_), "DequantizeLinear backward");
 }
 
-size_t nbla_hip_prune_workspace_bytes(void) { return round_up(sizeof(SelectState), 256); }
+size_t nbla_hip_prune_workspace_bytes(void) { return round_up(sizeof(PruneState), 256); }
 
 int nbla_hip_prune_f32(const float *x, float *y, size_t size, float rate, void *workspace, size_t workspace_bytes,
                        void *stream_) {
@@ -509,7 +621,7 @@ int nbla_hip_prune_f32(const float *x, float *y, size_t size, float rate, void *
     return NBLA_HIP_OK;
   if (size > 0x7fffffffu)
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "Prune: more than 2^31 - 1 elements (the reference indexes with int).");
-  if (workspace_bytes < sizeof(SelectState) || !aligned256(workspace))
+  if (workspace_bytes < sizeof(PruneState) || !aligned256(workspace))
     return fail(NBLA_HIP_ERR_MEMORY, "Prune workspace too small or misaligned.");
   if (!aligned16(x) || !aligned16(y))
     return fail(NBLA_HIP_ERR_MEMORY, "Prune: x and y must be 16-byte aligned.");
@@ -517,25 +629,27 @@ int nbla_hip_prune_f32(const float *x, float *y, size_t size, float rate, void *
   if (rc)
     return rc;
   hipStream_t stream = as_stream(stream_);
-  SelectState *st = static_cast<SelectState *>(workspace);
+  PruneState *ps = static_cast<PruneState *>(workspace);
+  SelectState *st = &ps->sel;
   // prune.cpp:33-34: thresh_idx_ = (int)((x_size - 1) * rate_), an int times a float
   const int x_size = (int)size;
   const uint32_t rank = (uint32_t)(int)((x_size - 1) * rate);
   const int64_t n = (int64_t)size;
   const int64_t n4 = n / 4;
-  int64_t blocks = ceil_div(n4 ? n4 : 1, (int64_t)kHistBlock * 4);
+  int64_t blocks = ceil_div(n4 ? n4 : 1, (int64_t)kHistBlock * kPruneLoads);
   if (blocks > kSelectBlocks)
     blocks = kSelectBlocks;
   hipLaunchKernelGGL(clear_select, dim3(clear_select_blocks()), dim3(256), 0, stream, st, rank);
   NBLA_HIP_LAUNCH_CHECK("clear_select");
   for (int p = 0; p < kPasses; ++p) {
-    hipLaunchKernelGGL(prune_histogram, dim3((unsigned)blocks), dim3(kHistBlock), 0, stream, x, n4, n, st, p);
+    hipLaunchKernelGGL(prune_histogram, dim3((unsigned)blocks), dim3(kHistBlock), 0, stream, x, n4, n, ps, p);
     NBLA_HIP_LAUNCH_CHECK("prune_histogram");
   }
-  int64_t ablocks = ceil_div(n4 ? n4 : 1, (int64_t)kBlock * 4);
-  if (ablocks > 4096)
-    ablocks = 4096;
-  hipLaunchKernelGGL(prune_apply, dim3((unsigned)ablocks), dim3(kBlock), 0, stream, x, y, n4, n, st,
+  // every block of this launch resolves the last histogram first: two blocks per CU at most
+  int64_t ablocks = ceil_div(n4 ? n4 : 1, (int64_t)kHistBlock * kPruneLoads);
+  if (ablocks > 2 * kSelectBlocks)
+    ablocks = 2 * kSelectBlocks;
+  hipLaunchKernelGGL(prune_apply, dim3((unsigned)ablocks), dim3(kHistBlock), 0, stream, x, y, n4, n, ps,
                      rate == 1.0f ? 1.0f : 0.0f);
   NBLA_HIP_LAUNCH_CHECK("prune_apply");
   return NBLA_HIP_OK;

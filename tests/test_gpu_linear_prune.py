@@ -121,6 +121,22 @@ def test_prune_large_and_special_values(dev):
         kernels.prune(_dev(x[:1], dev), 1.5)
 
 
+@pytest.mark.parametrize("rate", [0.3, 0.6, 0.97])
+def test_prune_magnitudes_clustered_in_one_stretch(dev, rate):
+    """The second selection pass keeps the keys that share the first digit with the threshold in per-block regions of
+    the workspace; when those keys sit in one stretch of x (here: 1.3 M values of one binade in a row, far more than
+    the blocks that read that stretch can keep) the third pass has to fall back to reading x.  Same result either
+    way; the first rate puts the threshold outside the stretch, the others inside it."""
+    rng = np.random.default_rng(77)
+    n = 1 << 22
+    x = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    lo = n // 3
+    x[lo:lo + 1300000] = (1.0 + rng.random(1300000) * 0.12).astype(np.float32) * rng.choice([-1.0, 1.0], 1300000).astype(np.float32)
+    x[lo + 1300000:] *= 1000.0
+    y = kernels.prune(_dev(x, dev), rate)
+    assert bits_equal(to_np(y), oracle.prune(x, rate))
+
+
 def test_prune_reuses_its_workspace(dev):
     """Back-to-back calls on one workspace (histograms, tickets and chosen digits of the previous call are left in
     it), with changing sizes and rates."""
