@@ -190,6 +190,13 @@ __device__ __forceinline__ void unfold_main_loop(const GemmBitsArgs &a, unsigned
   const int tid = threadIdx.x;
   const int in0 = g.in_sp[0], in1 = g.in_sp[1], in2 = g.in_sp[2], plane = (int)g.in_sp_size;
   const int k_tiles = (int)a.x_k_tiles, nstages = k_tiles / kStageTiles;
+  // scratch of step 2, in the space of the stage buffers (unused until step 3): per-pixel channel maxima of the
+  // input positions the block's windows touch, and the runs of consecutive rows that lie in one sample ("segments")
+  constexpr int kPixCap = 4096, kPixPerLane = 8; // pixels in all segments / 64-pixel rounds of one segment
+  static_assert(kPixCap * 4 + 4 * 32 * 4 + 4 <= kMetaOff, "the scratch of step 2 fits the stage buffers");
+  uint32_t *s_pix = reinterpret_cast<uint32_t *>(smem);
+  int *seg_lo = reinterpret_cast<int *>(smem + kPixCap * 4), *seg_hi = seg_lo + 32, *seg_n = seg_lo + 64;
+  int *row_seg = seg_lo + 96, *seg_count = seg_lo + 128;
 
   // 1. the decoded columns and taps
   i32x4_t *taps_table = reinterpret_cast<i32x4_t *>(smem + kMetaOff + 512);
@@ -224,7 +231,11 @@ __device__ __forceinline__ void unfold_main_loop(const GemmBitsArgs &a, unsigned
     if (tid < 32) {
       s_amax[tid] = 0u;
       s_sums[tid] = 0;
+      seg_lo[tid] = 0x7fffffff;
+      seg_hi[tid] = -1;
     }
+    for (int i = tid; i < kPixCap; i += kThreads)
+      s_pix[i] = 0u;
     if (tid < 256) { // the block's columns' alpha and bias: the epilogue reads them from LDS
       const int64_t col = a.n_begin + bn * BN + tid;
       const int64_t nc = col < a.N ? col : a.N - 1;
@@ -247,19 +258,77 @@ __device__ __forceinline__ void unfold_main_loop(const GemmBitsArgs &a, unsigned
   const float *xn = a.ux + (n * g.C + a.ugrp * g.Cg) * g.in_sp_size;
   __syncthreads();
 
-  // 2. the row's taps inside the input, and its largest magnitude: channel slice = (wavefront, half); per tap the
-  // sixteen channels c = slice + 16 j of a round of 256 channels are in flight together
+  // 2. the row's taps inside the input (a 64-bit mask), and its largest magnitude.  The rows of a block are
+  // consecutive output positions, so their windows overlap: instead of gathering every row's window (taps x channels
+  // loads per row, a few values per cache line), the block first takes the maximum over the channels of every input
+  // position its windows can touch -- per segment one run [lo, hi] of the flattened plane, read with consecutive
+  // lanes on consecutive positions -- and a row's maximum is then the maximum of its taps' positions.
+  if (tid < 32) {
+    // segments: wavefront 0, lanes 0..31 hold rows 0..31
+    const unsigned long long starts = __ballot(in_range && (r == 0 || m / g.out_sp_size != (m - 1) / g.out_sp_size));
+    const int seg = __popcll(starts & ((2ull << r) - 1ull)) - 1;
+    row_seg[r] = in_range ? seg : 0;
+    if (in_range) {
+      int last = 0; // the largest tap offset
+      for (int t = 0; t < taps; ++t)
+        last = max(last, taps_table[t].x);
+      const int lo = origin > 0 ? origin : 0, hi = origin + last < plane - 1 ? origin + last : plane - 1;
+      atomicMin(&seg_lo[seg], lo);
+      atomicMax(&seg_hi[seg], hi);
+      seg_n[seg] = (int)n;
+    }
+    if (r == 0)
+      *seg_count = __popcll(starts & 0xffffffffull);
+  }
+  __syncthreads();
   uint32_t mask_lo = 0u, mask_hi = 0u;
-  {
+  const int nseg = *seg_count;
+  // blocks whose positions do not fit the scratch take the gathering form
+  bool by_pixels = true;
+  int my_base = 0, total = 0;
+  for (int sgm = 0; sgm < (by_pixels ? nseg : 0); ++sgm) {
+    const int len = seg_hi[sgm] - seg_lo[sgm] + 1;
+    if (sgm == row_seg[r])
+      my_base = total;
+    total += len > 0 ? len : 0;
+    by_pixels = by_pixels && len <= 64 * kPixPerLane;
+  }
+  by_pixels = by_pixels && total <= kPixCap;
+  if (by_pixels) {
+    const int Cg = (int)g.Cg;
+    int base = 0;
+    for (int sgm = 0; sgm < nseg; ++sgm) {
+      const int lo = seg_lo[sgm], len = seg_hi[sgm] - lo + 1;
+      if (len <= 0)
+        continue;
+      const float *xs = a.ux + ((int64_t)seg_n[sgm] * g.C + a.ugrp * g.Cg) * g.in_sp_size + lo;
+      for (int p0 = 0; p0 < len; p0 += 64) {
+        const int pix = p0 + lane;
+        const bool live = pix < len;
+        const float *src = xs + (live ? pix : 0);
+        uint32_t amax = 0u;
+        // channels wave, wave + 8, ...: sixteen loads in flight
+        for (int c0 = wave; c0 < Cg; c0 += 8 * 16) {
+          float v[16];
+#pragma unroll
+          for (int j = 0; j < 16; ++j) {
+            const int c = c0 + 8 * j;
+            v[j] = src[(int64_t)(c < Cg ? c : wave) * plane];
+          }
+#pragma unroll
+          for (int j = 0; j < 16; ++j)
+            if (c0 + 8 * j < Cg)
+              amax = max(amax, __float_as_uint(v[j]) & 0x7fffffffu);
+        }
+        if (live && amax)
+          atomicMax(&s_pix[base + pix], amax);
+      }
+      base += len;
+    }
+    __syncthreads();
     uint32_t amax = 0u;
-    const int slice = wave * 2 + half, Cg = (int)g.Cg;
-    // (tap, round of 256 channels) pairs, the loads of one pair in flight while the previous one is reduced
-    const int rounds = (Cg + 255) / 256, pairs = taps * rounds;
-    float v[2][16];
-    bool okv[2];
-    int c0v[2];
-    auto issue = [&](int pair, int slot) __attribute__((always_inline)) {
-      const int t = pair / rounds, c0 = slice + (pair - t * rounds) * 256;
+    const int rel = my_base + origin - seg_lo[row_seg[r]];
+    for (int t = 0; t < taps; ++t) {
       const i32x4_t e = taps_table[t];
       const int i0 = b0 + (e.y & 0xffff), i1 = b1 + (int)((uint32_t)e.y >> 16), i2 = b2 + e.z;
       const bool ok = in_range && (unsigned)i0 < (unsigned)in0 && (unsigned)i1 < (unsigned)in1 &&
@@ -269,34 +338,60 @@ __device__ __forceinline__ void unfold_main_loop(const GemmBitsArgs &a, unsigned
           mask_lo |= 1u << t;
         else
           mask_hi |= 1u << (t - 32);
+        amax = max(amax, s_pix[rel + e.x]);
       }
-      const float *src = xn + (ok ? origin + e.x : 0);
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const int c = c0 + 16 * j;
-        v[slot][j] = src[(int64_t)(c < Cg ? c : slice) * plane];
-      }
-      okv[slot] = ok;
-      c0v[slot] = c0;
-    };
-    auto reduce = [&](int slot) __attribute__((always_inline)) {
-#pragma unroll
-      for (int j = 0; j < 16; ++j)
-        if (okv[slot] && c0v[slot] + 16 * j < Cg)
-          amax = max(amax, __float_as_uint(v[slot][j]) & 0x7fffffffu);
-    };
-    issue(0, 0);
-    for (int pair = 0; pair < pairs; pair += 2) {
-      if (pair + 1 < pairs)
-        issue(pair + 1, 1);
-      reduce(0);
-      if (pair + 2 < pairs)
-        issue(pair + 2, 0);
-      if (pair + 1 < pairs)
-        reduce(1);
     }
-    if (amax)
-      atomicMax(&s_amax[r], amax);
+    if (tid < 32)
+      s_amax[r] = amax;
+  } else {
+    {
+      uint32_t amax = 0u;
+      const int slice = wave * 2 + half, Cg = (int)g.Cg;
+      // (tap, round of 256 channels) pairs, the loads of one pair in flight while the previous one is reduced
+      const int rounds = (Cg + 255) / 256, pairs = taps * rounds;
+      float v[2][16];
+      bool okv[2];
+      int c0v[2];
+      auto issue = [&](int pair, int slot) __attribute__((always_inline)) {
+        const int t = pair / rounds, c0 = slice + (pair - t * rounds) * 256;
+        const i32x4_t e = taps_table[t];
+        const int i0 = b0 + (e.y & 0xffff), i1 = b1 + (int)((uint32_t)e.y >> 16), i2 = b2 + e.z;
+        const bool ok = in_range && (unsigned)i0 < (unsigned)in0 && (unsigned)i1 < (unsigned)in1 &&
+                        (unsigned)i2 < (unsigned)in2;
+        if (ok) {
+          if (t < 32)
+            mask_lo |= 1u << t;
+          else
+            mask_hi |= 1u << (t - 32);
+        }
+        const float *src = xn + (ok ? origin + e.x : 0);
+  #pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const int c = c0 + 16 * j;
+          v[slot][j] = src[(int64_t)(c < Cg ? c : slice) * plane];
+        }
+        okv[slot] = ok;
+        c0v[slot] = c0;
+      };
+      auto reduce = [&](int slot) __attribute__((always_inline)) {
+  #pragma unroll
+        for (int j = 0; j < 16; ++j)
+          if (okv[slot] && c0v[slot] + 16 * j < Cg)
+            amax = max(amax, __float_as_uint(v[slot][j]) & 0x7fffffffu);
+      };
+      issue(0, 0);
+      for (int pair = 0; pair < pairs; pair += 2) {
+        if (pair + 1 < pairs)
+          issue(pair + 1, 1);
+        reduce(0);
+        if (pair + 2 < pairs)
+          issue(pair + 2, 0);
+        if (pair + 1 < pairs)
+          reduce(1);
+      }
+      if (amax)
+        atomicMax(&s_amax[r], amax);
+    }
   }
   __syncthreads();
   if (tid < 32) {

@@ -35,6 +35,13 @@ CASES = [
     ((1, 2, 6, 6, 6), (4, 2, 5, 5, 5), (2, 2, 2), (1, 1, 1), (1, 1, 1), 1),
     # 7 x 7 kernel, stride 2 (49 taps: the upper half of the tap mask)
     ((2, 3, 20, 20), (8, 3, 7, 7), (3, 3), (2, 2), (1, 1), 1),
+    # one output position per sample: every row of a block is a segment of its own (32 per block)
+    ((70, 3, 3, 3), (5, 3, 3, 3), (0, 0), (1, 1), (1, 1), 1),
+    # a wide image: the input positions under a block's 32 windows (three rows of 300) exceed what the per-position
+    # maxima of the fused product hold, so its rows' maxima are gathered window by window
+    ((1, 2, 5, 300), (4, 2, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    # padding larger than the kernel: windows that lie wholly outside the input
+    ((2, 3, 6, 6), (4, 3, 2, 2), (3, 3), (1, 1), (1, 1), 1),
 ]
 
 
