@@ -81,6 +81,9 @@ constexpr int copies_per_call(bool one_a, bool narrow, int groups) {
 // and barrier waits are covered by the other's MFMAs.
 // kNarrow: the B operand holds every value in its lowest digit alone (a small integer): three products
 // a_t x b2 -> accumulator t, nothing dropped, and only the lowest-digit fragments of B are copied.
+// kTopB (a form of kNarrow): every row of the tile's B row blocks is a one-digit row of a row-scaled operand (its value
+// sits in the top digit: power-of-two weights once INQ has fixed them): the same three products with b0 in place of
+// b2, and the factor 2^16 of the top digit in the epilogue.
 // kOneA (only with kNarrow): every row of the tile's A row blocks is a one-digit row (gemm_layout.hpp: its value sits
 // in the top digit): a single product a0 x b2 -> accumulator 0, and only the top-digit fragments of A and the
 // lowest-digit fragments of B are copied (eight per k tile, dealt evenly over the wavefronts).  Same bits as the other
@@ -89,11 +92,13 @@ constexpr int copies_per_call(bool one_a, bool narrow, int groups) {
 // tiles g, g + 2, ... of the same output tile (a stage then holds two consecutive k tiles), so every SIMD has a second
 // wavefront to issue from while the first waits.  At the end the groups swap halves of their int32 accumulators
 // through LDS (exactly) and group g finishes row fragment g of each wavefront tile.
-template <bool kNarrow, bool kOneA, int kStages, int kGroups>
+template <bool kNarrow, bool kOneA, int kStages, int kGroups, bool kTopB = false>
 __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsigned char *smem) {
 #if defined(__HIP_DEVICE_COMPILE__) // the host pass only needs the launch stub; the body uses LDS address-space pointers
   static_assert(kGroups == 1 || kGroups == 2, "k groups per block");
   static_assert(!kOneA || kNarrow, "the one-digit A form is implemented for one-digit B operands");
+  static_assert(!kTopB || kNarrow, "the top-digit B form is a narrow form");
+  constexpr int kBDigit = kTopB ? 0 : kDigits - 1; // the one digit of B a narrow form multiplies
   constexpr int kAllWaves = kWaves * kGroups;
   constexpr int kGroupStageBytes = kGroups * kStageBytes;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -119,7 +124,7 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
     if (kOneA) {
       sub = p / kOnePerTile;
       const int f = (p - sub * kOnePerTile) * kAllWaves + wave_all;
-      side = f / kSegs, seg = f % kSegs, d = side ? kDigits - 1 : 0;
+      side = f / kSegs, seg = f % kSegs, d = side ? kBDigit : 0;
       if (p >= kOnePerTile * kGroups)
         sub = 0, side = 0, seg = 0; // unused slot
     } else {
@@ -129,10 +134,10 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
       if (u < kSegs * kDigits)
         side = 0, seg = u / kDigits, d = u - seg * kDigits;
       else if (u < kSegs * kDigits + kSegs)
-        side = 1, seg = u - kSegs * kDigits, d = kDigits - 1;
-      else
+        side = 1, seg = u - kSegs * kDigits, d = kBDigit;
+      else // the two digits of B that a narrow form leaves out
         side = 1, seg = (u - kSegs * kDigits - kSegs) / (kDigits - 1),
-        d = (u - kSegs * kDigits - kSegs) % (kDigits - 1);
+        d = (u - kSegs * kDigits - kSegs) % (kDigits - 1) + (kTopB ? 1 : 0);
     }
     dest[p] = sub * kStageBytes + ((side * kSegs + seg) * kDigits + d) * kFragBytes;
     int64_t rb = (side ? bn : bm) * kSegs + seg;
@@ -196,7 +201,7 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
       for (int d = 0; d < 3; ++d) {
         if (!kOneA || d == 0)
           af[i][d] = __builtin_bit_cast(i32x4_t, sa[((wm * 2 + i) * kDigits + d) * 64 + lane]);
-        if (!kNarrow || d == 2)
+        if (!kNarrow || d == kBDigit)
           bf[i][d] = __builtin_bit_cast(i32x4_t, sb[((wn * 2 + i) * kDigits + d) * 64 + lane]);
       }
     if (kOneA) {
@@ -204,7 +209,7 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          acc[i][j][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i][0], bf[j][2], acc[i][j][0], 0, 0, 0);
+          acc[i][j][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i][0], bf[j][kBDigit], acc[i][j][0], 0, 0, 0);
     } else if (kNarrow) {
 #pragma unroll
       for (int t = 0; t < 3; ++t)
@@ -212,7 +217,7 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
         for (int i = 0; i < 2; ++i)
 #pragma unroll
           for (int j = 0; j < 2; ++j)
-            acc[i][j][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i][t], bf[j][2], acc[i][j][t], 0, 0, 0);
+            acc[i][j][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i][t], bf[j][kBDigit], acc[i][j][t], 0, 0, 0);
     } else {
       // digit pairs (a digit, b digit) -> accumulator a + b
       constexpr int da[6] = {0, 0, 1, 0, 1, 2};
@@ -260,11 +265,12 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
     }
   }
 
-  // y = (acc0 * 2^16 + acc1 * 2^8 + acc2) * 2^(16 - sa - sb); the narrow form has no factor 2^16 (b is its low digit).
+  // y = (acc0 * 2^16 + acc1 * 2^8 + acc2) * 2^(16 - sa - sb); the narrow form has no factor 2^16 (b is its low digit)
+  // unless b is the top digit of a row-scaled operand.
   // Row by row: the row's offset (one 32-bit division when m is folded into two output indices) and shift are
   // formed once and serve both column fragments.
   const int col_in_frag = lane & 31, row_half = lane >> 5;
-  const int32_t *bshift = kNarrow ? a.bshift_narrow : a.bshift;
+  const int32_t *bshift = (kNarrow && !kTopB) ? a.bshift_narrow : a.bshift;
   int64_t n_col[2];
   int32_t sb_n[2];
   float bias_n[2];
@@ -325,7 +331,7 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
             const int lo = ((a1 & 0xff) << 8) + (a2 & 0xffff);
             const float t = fmaf((float)hi, 65536.0f, (float)lo);
             // the two shifts are applied one after the other: each stays inside ldexpf's exponent range
-            v = ldexpf(ldexpf(t, (kNarrow ? 0 : 16) - sa_m), -sb_n[j]);
+            v = ldexpf(ldexpf(t, ((kNarrow && !kTopB) ? 0 : 16) - sa_m), -sb_n[j]);
           }
           float *dst = a.y + off + n_col[j] * a.n_stride;
           if (kAcc)
@@ -368,7 +374,27 @@ __global__ __launch_bounds__(kThreads * kGroups, kGroups == 1 ? 2 : 1) void gemm
     else
       gemm_digits_tile<true, false, kStages, kGroups>(a, smem);
   } else {
-    gemm_digits_tile<false, false, kStages, kGroups>(a, smem);
+    // all rows of this tile's B row blocks one-digit rows (of a row-scaled operand; column-scaled ones never are)?
+    int64_t bm, bn;
+    band_tile<8>(blockIdx.x, a.blocks_m, a.blocks_n, bm, bn);
+    const int64_t arows = a.a_row_blocks * kFragRows, brows = a.b_row_blocks * kFragRows;
+    bool one_b = true, one_a = true;
+    for (int r = threadIdx.x; r < kBN; r += kThreads * kGroups) {
+      const int64_t n = bn * kBN + r;
+      one_b = one_b && one_digit_row(a.bshift[n < brows ? n : brows - 1]);
+    }
+    for (int r = threadIdx.x; r < kBM; r += kThreads * kGroups) {
+      const int64_t m = bm * kBM + r;
+      one_a = one_a && one_digit_row(a.ashift[m < arows ? m : arows - 1]);
+    }
+    one_b = __syncthreads_and(one_b);
+    one_a = __syncthreads_and(one_a);
+    if (one_b && one_a)
+      gemm_digits_tile<true, true, kStages, kGroups, true>(a, smem);
+    else if (one_b)
+      gemm_digits_tile<true, false, kStages, kGroups, true>(a, smem);
+    else
+      gemm_digits_tile<false, false, kStages, kGroups>(a, smem);
   }
 }
 

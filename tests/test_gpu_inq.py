@@ -228,6 +228,34 @@ def test_inq_convolution_matches_oracle(dev):
             assert max_rel_err(to_np(y), ref_y) <= TIGHT
 
 
+def test_convolution_with_fixed_weights_takes_the_one_digit_form(dev):
+    """Weights INQ has fixed are powers of two within seven binades: as a row-scaled digit operand each output
+    channel is a one-digit row (its values whole units of the top digit), and a tile of the product whose 128
+    channels are all of that kind multiplies three digit pairs instead of six.  Nothing is dropped either way, so the
+    channels give the same bits when a general channel in their tile forces the six-pair form; and the result is
+    the float64 convolution of x as rounded to 24 bits per window."""
+    rng = np.random.RandomState(5)
+    xs, ws = (3, 32, 12, 12), (160, 32, 3, 3)          # two tiles of output channels, the second partly empty
+    x = rng.randn(*xs).astype(np.float32)
+    e = rng.randint(-8, -2, size=ws)
+    W = (np.where(rng.rand(*ws) < 0.2, 0.0, 2.0 ** e) * rng.choice([-1.0, 1.0], size=ws)).astype(np.float32)
+    I = torch.ones(ws, dtype=torch.int32, device=dev)
+
+    def run(Wh):
+        Wd = _dev(Wh, dev)
+        return to_np(kernels.inq_convolution(_dev(x, dev), Wd, I, Wd.clone(), I.clone(), None, (1, 1), (1, 1), None, 1,
+                                             4, kernels.INQ_PRODUCT_ONLY))
+    y1 = run(W)
+    assert max_rel_err(y1, oracle.convolution(x, W, None, (1, 1), (1, 1), None, 1)) <= TIGHT
+    W6 = W.copy()
+    W6[::128] = (rng.randn(2, *ws[1:]) * 0.05).astype(np.float32)   # one general channel in each tile
+    y6 = run(W6)
+    same = np.ones(ws[0], bool)
+    same[::128] = False
+    assert bits_equal(y1[:, same], y6[:, same])
+    assert max_rel_err(y6, oracle.convolution(x, W6, None, (1, 1), (1, 1), None, 1)) <= TIGHT
+
+
 def test_inq_config5_layer(dev):
     """The INQAffine layer of benchmark configuration 5: x [1024,4096], W [4096,4096] ~ N(0, 0.02^2), num_bits 4, every
     weight fixed.  Weights bit-exact against the oracle; the output against float64 on sampled entries and against
