@@ -148,7 +148,10 @@ __device__ __forceinline__ float row_hi_scale(int shift) { return shift == kBadR
 // k groups' exchange area, which reuses the buffers at the end) the LDS holds the row sums, row maxima and row shifts,
 // then the table of decoded unfolded columns (16 bytes each).
 constexpr int kUnfoldSteps = 2;
-constexpr int kUnfoldMetaBytes = 512 + 64 * 16 + 2 * 256 * 4; // sums, maxima, shifts; the taps' table; alpha, bias
+constexpr int kUnfoldRowTaps = 65; // a row's byte offsets of its taps (64 at most) and one entry that is never valid
+// sums, maxima, shifts; the taps' table; alpha, bias; the rows' tap offsets
+constexpr int kUnfoldMetaBytes = 512 + 64 * 16 + 2 * 256 * 4 + 32 * kUnfoldRowTaps * 4;
+constexpr uint32_t kUnfoldNowhere = 0x80000000u; // a byte offset past every input the fused product accepts
 constexpr int unfold_meta_off(int BM, int BN, int waves_m, int waves_n, int waves_k) {
   const int stages = 2 * kUnfoldSteps * gemm_bits_stage_bytes(BM, BN, waves_k);
   const int exchange = (waves_k - 1) * (BM / 32) * (BN / 32) * 4096;
@@ -157,12 +160,14 @@ constexpr int unfold_meta_off(int BM, int BN, int waves_m, int waves_n, int wave
 
 // Main loop of the unfolding product: the block's 32 rows are unfolded windows of x (rows m = (sample, output
 // position), columns kk = (channel, kernel tap), as im2col lays them out) that are never written to memory.  The block
-//  1. decodes every column kk once into an LDS table {offset of (channel, tap) relative to the window origin, one-hot
-//     64-bit mask of the tap (zero for kk >= Kg)}, and the taps (at most 64) into {offset, displacements};
-//  2. finds for each row which taps fall inside the input (a 64-bit mask: an element of the row is then read iff
-//     its column's mask meets the row's) and the row's largest magnitude (over its taps and channels: 16 channel
-//     slices per row, combined by an LDS maximum), and from that the row's power-of-two scale, exactly as the
-//     stand-alone unfold kernels do;
+//  1. decodes the taps (at most 64) into {offset, displacements} and every column kk into an LDS table {byte offset of
+//     its channel's plane, 4 x its tap} (kk >= Kg: the tap entry that is never valid);
+//  2. finds for each row which taps fall inside the input and the row's largest magnitude, and from that the row's
+//     power-of-two scale, exactly as the stand-alone unfold kernels do; then writes, per row and tap, the byte offset
+//     of that tap's element of channel 0 in x, or an offset past the end of x when the tap falls outside the input
+//     (or the row holds a non-finite value, or lies past the last row).  An element of the unfolded matrix is then
+//     one bounds-checked buffer load at (row's tap offset + column's channel offset): out of range reads give 0,
+//     so the loop has no validity tests and no selects;
 //  3. walks the contraction in stages of eight k tiles with two LDS buffers.  Wavefront w produces k tile w of a
 //     stage: lane l gathers the sixteen values of row l % 32, k slots (l / 32) * 16 + 0..15, turns them into digits,
 //     writes them where the fragment's lane l holds them and adds their sum to the row's sum; it also moves the
@@ -185,7 +190,9 @@ __device__ __forceinline__ void unfold_main_loop(const GemmBitsArgs &a, unsigned
   long long *s_sums = reinterpret_cast<long long *>(smem + kMetaOff);
   uint32_t *s_amax = reinterpret_cast<uint32_t *>(smem + kMetaOff + 256);
   int32_t *s_shift = reinterpret_cast<int32_t *>(smem + kMetaOff + 384);
-  i32x4_t *table = reinterpret_cast<i32x4_t *>(smem + kMetaOff + kUnfoldMetaBytes);
+  typedef int i32x2_t __attribute__((ext_vector_type(2)));
+  i32x2_t *table = reinterpret_cast<i32x2_t *>(smem + kMetaOff + kUnfoldMetaBytes);
+  uint32_t *row_taps = reinterpret_cast<uint32_t *>(smem + kMetaOff + 512 + 64 * 16 + 2 * 256 * 4);
   float *s_alpha = reinterpret_cast<float *>(smem + kMetaOff + 512 + 64 * 16), *s_bias = s_alpha + 256;
   const int tid = threadIdx.x;
   const int in0 = g.in_sp[0], in1 = g.in_sp[1], in2 = g.in_sp[2], plane = (int)g.in_sp_size;
@@ -198,35 +205,30 @@ __device__ __forceinline__ void unfold_main_loop(const GemmBitsArgs &a, unsigned
   int *seg_lo = reinterpret_cast<int *>(smem + kPixCap * 4), *seg_hi = seg_lo + 32, *seg_n = seg_lo + 64;
   int *row_seg = seg_lo + 96, *seg_count = seg_lo + 128;
 
-  // 1. the decoded columns and taps
+  // 1. the decoded taps, then the columns (one division per column: channel = column / taps)
   i32x4_t *taps_table = reinterpret_cast<i32x4_t *>(smem + kMetaOff + 512);
   const int taps = (int)g.k_size;
+  if (tid < taps) {
+    const int K1 = g.k[1], K2 = g.k[2];
+    int q = tid;
+    const int k2 = q % K2;
+    q /= K2;
+    const int k1 = q % K1, k0 = q / K1;
+    const int e0 = k0 * g.dil[0], e1 = k1 * g.dil[1], e2 = k2 * g.dil[2];
+    i32x4_t t;
+    t.x = (e0 * in1 + e1) * in2 + e2;
+    t.y = e0 | (e1 << 16);
+    t.z = e2;
+    t.w = 0;
+    taps_table[tid] = t;
+  }
   {
-    const int K0 = g.k[0], K1 = g.k[1], K2 = g.k[2];
     for (int kk = tid; kk < k_tiles * kTileK; kk += kThreads) {
-      int q = kk;
-      const int k2 = q % K2;
-      q /= K2;
-      const int k1 = q % K1;
-      q /= K1;
-      const int k0 = q % K0, c = q / K0;
-      const int e0 = k0 * g.dil[0], e1 = k1 * g.dil[1], e2 = k2 * g.dil[2];
-      const int tap = (k0 * K1 + k1) * K2 + k2;
-      const unsigned long long bit = kk < (int)g.Kg ? 1ull << tap : 0ull;
-      i32x4_t e;
-      e.x = c * plane + (e0 * in1 + e1) * in2 + e2;
-      e.y = 0;
-      e.z = (int)(uint32_t)bit;
-      e.w = (int)(uint32_t)(bit >> 32);
+      const int c = kk / taps, tap = kk - c * taps;
+      i32x2_t e;
+      e.x = kk < (int)g.Kg ? c * plane * 4 : 0;
+      e.y = kk < (int)g.Kg ? tap * 4 : (kUnfoldRowTaps - 1) * 4;
       table[kk] = e;
-      if (kk < taps) { // channel 0: kk is the tap
-        i32x4_t t;
-        t.x = e.x;
-        t.y = e0 | (e1 << 16);
-        t.z = e2;
-        t.w = 0;
-        taps_table[kk] = t;
-      }
     }
     if (tid < 32) {
       s_amax[tid] = 0u;
@@ -405,13 +407,26 @@ __device__ __forceinline__ void unfold_main_loop(const GemmBitsArgs &a, unsigned
         --s;
     }
     s_shift[tid] = s;
+    // the row's taps as byte offsets into x; a row holding a NaN or an infinity is not read (its outputs become NaN
+    // in the epilogue), nor is a tap outside the input
+    const uint32_t first = (uint32_t)(((n * g.C + a.ugrp * g.Cg) * g.in_sp_size + origin) * 4);
+    for (int t = 0; t < taps; ++t) {
+      const bool ok = s != kBadRow && (((t < 32 ? mask_lo >> t : mask_hi >> (t - 32)) & 1u) != 0u);
+      row_taps[tid * kUnfoldRowTaps + t] = ok ? first + (uint32_t)taps_table[t].x * 4u : kUnfoldNowhere;
+    }
+    row_taps[tid * kUnfoldRowTaps + kUnfoldRowTaps - 1] = kUnfoldNowhere;
   }
   __syncthreads();
 
   // 3. the stages
   const int s_row = s_shift[r];
-  if (s_row == kBadRow) // a row holding a NaN or an infinity is not read: its outputs become NaN in the epilogue
-    mask_lo = mask_hi = 0u;
+  // x as a buffer: reads at offsets past its end (kUnfoldNowhere + any channel offset) return zero
+  const uint64_t xbase = reinterpret_cast<uint64_t>(a.ux);
+  const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
+      reinterpret_cast<void *>(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(xbase >> 32)) << 32) |
+                               (uint32_t)__builtin_amdgcn_readfirstlane((int)xbase)),
+      0, __builtin_amdgcn_readfirstlane((int)(g.outer * g.C * g.in_sp_size * 4)), 0x00020000);
+  const uint32_t *my_taps = row_taps + r * kUnfoldRowTaps;
   // k tile `wave` of a stage sits in stage wave / 4 of the buffer, k step (wave % 4) / 2, tile wave % 2 of the step
   const int tile_off = (wave >> 2) * kStageBytes + ((wave & 3) >> 1) * kStepBytes;
   int64_t wg = a.n_begin / kWideGroup + bn;
@@ -423,10 +438,9 @@ __device__ __forceinline__ void unfold_main_loop(const GemmBitsArgs &a, unsigned
     const int kb = stage * kStageK + wave * kTileK + half * 16;
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
-      const i32x4_t e = table[kb + j];
-      const bool ok = (((uint32_t)e.z & mask_lo) | ((uint32_t)e.w & mask_hi)) != 0u;
-      const float xv = xn[ok ? origin + e.x : 0];
-      v[j] = ok ? xv : 0.0f;
+      const i32x2_t e = table[kb + j];
+      const uint32_t at = my_taps[e.y >> 2] + (uint32_t)e.x;
+      v[j] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(xrsrc, (int)at, 0, 0));
     }
   };
   // The three balanced base-256 digits of q (|q| <= kDigitMax) are the low three bytes of q + 0x808080, each with its
@@ -1238,15 +1252,16 @@ int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alp
 
 // LDS of the unfolding product: two stage buffers (or the k groups' exchange), the rows' metadata, the column table
 static size_t unfold_lds_bytes(int64_t Kg) {
-  return (size_t)unfold_meta_off(32, 256, 1, 4, 2) + kUnfoldMetaBytes + (size_t)bits_packed_k_tiles(Kg) * kTileK * 16;
+  return (size_t)unfold_meta_off(32, 256, 1, 4, 2) + kUnfoldMetaBytes + (size_t)bits_packed_k_tiles(Kg) * kTileK * 8;
 }
 static_assert(kUnfoldSteps * 2 * 2 == 8, "the packed operand's k tiles come in multiples of eight: whole stages");
 
 bool gemm_bits_unfold_applies(const ConvGeom &g) {
-  // 32-bit offsets inside one sample's channel group and one output map, 16-bit tap displacements (as the stand-alone
-  // unfold kernel), one k chunk, and a column table that fits the LDS beside the stages
-  bool fits = g.Cg * g.in_sp_size < ((int64_t)1 << 31) && g.out_sp_size < ((int64_t)1 << 31) && g.Kg <= kChunkK &&
-              g.M < ((int64_t)1 << 31) - 64;
+  // x below 2 GiB (its elements are read through one buffer descriptor, at 32-bit byte offsets whose upper half
+  // means "nowhere"), 32-bit positions inside one output map, 16-bit tap displacements (as the stand-alone unfold
+  // kernel), one k chunk, and a column table that fits the LDS beside the stages
+  bool fits = g.outer * g.C * g.in_sp_size * 4 < ((int64_t)1 << 31) && g.out_sp_size < ((int64_t)1 << 31) &&
+              g.Kg <= kChunkK && g.M < ((int64_t)1 << 31) - 64;
   for (int i = 0; i < kMaxSpatial; ++i)
     fits = fits && (int64_t)(g.k[i] - 1) * g.dil[i] < 65536;
   return fits && g.k_size <= 64 && unfold_lds_bytes(g.Kg) <= 144 * 1024; // the taps of a row are a 64-bit mask
