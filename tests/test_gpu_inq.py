@@ -256,6 +256,22 @@ def test_convolution_with_fixed_weights_takes_the_one_digit_form(dev):
     assert max_rel_err(y6, oracle.convolution(x, W6, None, (1, 1), (1, 1), None, 1)) <= TIGHT
 
 
+def test_convolution_with_fixed_weights_at_the_resnet_stage_shape(dev):
+    """Benchmark configuration 4's shape with power-of-two weights (98 tiles of the digit product, the contraction
+    split over blocks, every tile in the one-digit form for its weights) against torch's float64 convolution."""
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(32, 256, 14, 14, generator=g)
+    e = torch.randint(-8, -2, (256, 256, 3, 3), generator=g).float()
+    W = torch.pow(2.0, e) * (torch.randint(0, 2, e.shape, generator=g).float() * 2 - 1)
+    W[torch.rand(W.shape, generator=g) < 0.2] = 0.0
+    b = torch.randn(256, generator=g)
+    Wd, I = W.to(dev), torch.ones(W.shape, dtype=torch.int32, device=dev)
+    y = kernels.inq_convolution(x.to(dev), Wd, I, Wd.clone(), I.clone(), b.to(dev), (1, 1), (1, 1), None, 1, 4,
+                                kernels.INQ_PRODUCT_ONLY)
+    ref = torch.nn.functional.conv2d(x.double().to(dev), W.double().to(dev), b.double().to(dev), padding=1)
+    assert max_rel_err(to_np(y), ref.cpu().numpy()) <= TIGHT
+
+
 def test_inq_config5_layer(dev):
     """The INQAffine layer of benchmark configuration 5: x [1024,4096], W [4096,4096] ~ N(0, 0.02^2), num_bits 4, every
     weight fixed.  Weights bit-exact against the oracle; the output against float64 on sampled entries and against
