@@ -572,6 +572,23 @@ int nbla_hip_add2_f32(const float *x0, const float *x1, float *y, size_t size,
  * src/nbla/function/generic/add2.cpp:48-77. */
 int nbla_hip_add2_backward_f32(const float *dy, float *dx, size_t size,
                                int accum, void *stream);
+/* y = x0 - x1 (op 0), x0 * x1 (op 1), x0 / x1 (op 2) on inputs of one shape.
+ * Replaces Sub2 / Mul2 / Div2 <float>::forward_impl: include/nbla/function/
+ * sub2.hpp:41, mul2.hpp:42, div2.hpp:44 over utils/base_transform_binary.hpp:
+ * 260-284. */
+#define NBLA_HIP_BINARY2_SUB 0
+#define NBLA_HIP_BINARY2_MUL 1
+#define NBLA_HIP_BINARY2_DIV 2
+int nbla_hip_binary2_f32(int op, const float *x0, const float *x1, float *y,
+                         size_t size, void *stream);
+/* dx = (accum ? dx : 0) + g with g the gradient of input `input` (0 or 1):
+ * dy, -dy | dy * x1, dy * x0 | dy / x1, -dy * x0 / (x1 * x1).  Replaces
+ * transform_binary_grad0 / grad1, utils/base_transform_binary.hpp:286-336,
+ * with the gradient expressions of the headers above.  x0 and x1 are not
+ * read for op 0. */
+int nbla_hip_binary2_backward_f32(int op, int input, const float *dy,
+                                  const float *x0, const float *x1, float *dx,
+                                  size_t size, int accum, void *stream);
 /* dst[r * dst_stride + i] (+)= src[r * src_stride + i], r < rows, i < len:
  * one input's share of Concatenate<float>::forward_impl / backward_impl,
  * src/nbla/function/generic/concatenate.cpp:62-104 (rows = outer_size_, len =

@@ -3,6 +3,9 @@
 #include <nbla/array/cpu_array.hpp>
 #include <nbla/backend_registry.hpp>
 #include <nbla/function/add2.hpp>
+#include <nbla/function/div2.hpp>
+#include <nbla/function/mul2.hpp>
+#include <nbla/function/sub2.hpp>
 #include <nbla/function/affine.hpp>
 #include <nbla/function/binary_connect_affine.hpp>
 #include <nbla/function/binary_connect_convolution.hpp>
@@ -138,6 +141,18 @@ FunctionPtr create_by_name(const string &name, const Context &ctx, const int64_t
   if (name == "Add2") {
     need(1, 0);
     return create_Add2(ctx, ia[0] != 0);
+  }
+  if (name == "Sub2") {
+    need(1, 0);
+    return create_Sub2(ctx, ia[0] != 0);
+  }
+  if (name == "Mul2") {
+    need(1, 0);
+    return create_Mul2(ctx, ia[0] != 0);
+  }
+  if (name == "Div2") {
+    need(1, 0);
+    return create_Div2(ctx, ia[0] != 0);
   }
   if (name == "Concatenate") {
     need(1, 0);

@@ -652,6 +652,37 @@ void Add2Hip<T>::backward_impl(const Variables &inputs, const Variables &outputs
   }
 }
 
+// Sub2, Mul2, Div2: utils/base_transform_binary.hpp:339-400 with the expressions of sub2.hpp:41, mul2.hpp:42, div2.hpp:44
+#define NBLA_HIP_DEFINE_BINARY2(NAME, OP)                                                                              \
+  template <typename T> void NAME##Hip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {           \
+    hip_set_device(this->ctx_);                                                                                        \
+    const T *x0 = inputs[0]->get_data_pointer<T>(this->ctx_);                                                          \
+    const T *x1 = inputs[1]->get_data_pointer<T>(this->ctx_);                                                          \
+    T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);                                                 \
+    NBLA_HIP_CALL(nbla_hip_binary2_f32(OP, x0, x1, y, (size_t)inputs[0]->size(), nullptr));                            \
+  }                                                                                                                    \
+  template <typename T>                                                                                                \
+  void NAME##Hip<T>::backward_impl(const Variables &inputs, const Variables &outputs,                                  \
+                                   const vector<bool> &propagate_down, const vector<bool> &accum) {                   \
+    if (!(propagate_down[0] || propagate_down[1]))                                                                     \
+      return;                                                                                                          \
+    hip_set_device(this->ctx_);                                                                                        \
+    const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);                                                         \
+    const T *x0 = inputs[0]->get_data_pointer<T>(this->ctx_);                                                          \
+    const T *x1 = inputs[1]->get_data_pointer<T>(this->ctx_);                                                          \
+    for (int i = 0; i < 2; ++i) {                                                                                      \
+      if (!propagate_down[i])                                                                                          \
+        continue;                                                                                                      \
+      T *dx = inputs[i]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[i]);                                          \
+      NBLA_HIP_CALL(nbla_hip_binary2_backward_f32(OP, i, dy, x0, x1, dx, (size_t)inputs[0]->size(), accum[i],          \
+                                                  nullptr));                                                           \
+    }                                                                                                                  \
+  }
+NBLA_HIP_DEFINE_BINARY2(Sub2, NBLA_HIP_BINARY2_SUB)
+NBLA_HIP_DEFINE_BINARY2(Mul2, NBLA_HIP_BINARY2_MUL)
+NBLA_HIP_DEFINE_BINARY2(Div2, NBLA_HIP_BINARY2_DIV)
+#undef NBLA_HIP_DEFINE_BINARY2
+
 // concatenate.cpp:62-76
 template <typename T> void ConcatenateHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
   hip_set_device(this->ctx_);
@@ -868,6 +899,9 @@ template class INQConvolutionHip<float, int>;
 template class AffineHip<float>;
 template class ReLUHip<float>;
 template class Add2Hip<float>;
+template class Sub2Hip<float>;
+template class Mul2Hip<float>;
+template class Div2Hip<float>;
 template class ConcatenateHip<float>;
 template class ConvolutionHip<float>;
 template class QuantizeLinearHip<float>;

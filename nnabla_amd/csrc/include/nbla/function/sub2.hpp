@@ -1,0 +1,46 @@
+// Sub2: the class a "hip:float" implementation derives from.  Constructor, argument types and member names are
+// those the reference's include/nbla/function/sub2.hpp:41 declares through NBLA_DEFINE_TRANSFORM_BINARY_INPLACE.
+// This build has no CPU arithmetic: a generic *_impl method without a body of its own raises not_implemented.
+#ifndef NBLA_FUNCTION_SUB2_HPP_
+#define NBLA_FUNCTION_SUB2_HPP_
+
+#include <nbla/cpu.hpp>
+#include <nbla/function.hpp>
+#include <nbla/function/no_cpu_impl.hpp>
+#include <nbla/function_registry.hpp>
+
+namespace nbla {
+
+NBLA_REGISTER_FUNCTION_HEADER(Sub2, bool);
+
+// Inputs: x0, x1.  y = x0 - x1.
+template <typename T> class Sub2 : public BaseFunction<bool> {
+public:
+  Sub2(const Context &ctx, bool inplace) : BaseFunction(ctx, inplace) {}
+  virtual ~Sub2() {}
+  virtual shared_ptr<Function> copy() const { return create_Sub2(ctx_, false /* inplace is obsolete */); }
+  virtual vector<dtypes> in_types() { return vector<dtypes>{get_dtype<T>(), get_dtype<T>()}; }
+  virtual vector<dtypes> out_types() { return vector<dtypes>{get_dtype<T>()}; }
+  virtual int min_inputs() { return 2; }
+  virtual int min_outputs() { return 1; }
+  virtual string name() { return "Sub2"; }
+  virtual vector<string> allowed_array_classes() { return SingletonManager::get<Cpu>()->array_classes(); }
+  virtual bool grad_depends_output_data(int i, int o) const { return false; }
+
+protected:
+  virtual void setup_impl(const Variables &inputs, const Variables &outputs) {
+    // utils/base_transform_binary.hpp:55-120; the broadcasting form is not part of this build
+    NBLA_CHECK(inputs[0]->shape() == inputs[1]->shape(), error_code::not_implemented,
+               "Sub2: the inputs must have the same shape (broadcasting is not available in this build).");
+    outputs[0]->reshape(inputs[0]->shape(), true);
+  }
+  virtual void forward_impl(const Variables &, const Variables &) { NBLA_NO_CPU_IMPL("Sub2"); }
+  virtual void backward_impl(const Variables &, const Variables &, const vector<bool> &, const vector<bool> &) {
+    NBLA_NO_CPU_IMPL("Sub2 backward");
+  }
+  // the gradient with respect to input i reads input j: neither
+  virtual bool grad_depends_input_data_impl(int i, int j) const { return false; }
+};
+
+} // namespace nbla
+#endif

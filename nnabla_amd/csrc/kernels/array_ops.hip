@@ -70,6 +70,64 @@ __global__ __launch_bounds__(kBlk) void add_kernel(const float *__restrict__ a, 
   }
 }
 
+// Sub2, Mul2, Div2 on inputs of one shape (sub2.hpp:41, mul2.hpp:42, div2.hpp:44): y = op(x0, x1), and for the
+// gradient of input kInput  dx = (accum ? dx : 0) + g(dy, x0, x1)  as base_transform_binary.hpp:286-336 forms it (the
+// sum with the zeroed gradient included: it turns a -0 into +0).
+enum { kOpSub2 = 0, kOpMul2 = 1, kOpDiv2 = 2 };
+template <int kOp> __device__ __forceinline__ float binary2(float x0, float x1) {
+  return kOp == kOpSub2 ? x0 - x1 : (kOp == kOpMul2 ? x0 * x1 : x0 / x1);
+}
+template <int kOp, int kInput> __device__ __forceinline__ float binary2_grad(float dy, float x0, float x1) {
+  if (kOp == kOpSub2)
+    return kInput == 0 ? dy : -dy;
+  if (kOp == kOpMul2)
+    return kInput == 0 ? dy * x1 : dy * x0;
+  return kInput == 0 ? dy / x1 : -dy * x0 / (x1 * x1);
+}
+template <int kOp>
+__global__ __launch_bounds__(kBlk) void binary2_kernel(const float *__restrict__ x0, const float *__restrict__ x1,
+                                                       float *__restrict__ y, size_t n4, size_t size, int vec) {
+  if (vec) {
+    for (size_t i = (size_t)blockIdx.x * kBlk + threadIdx.x; i < n4; i += (size_t)gridDim.x * kBlk) {
+      const float4_t a = reinterpret_cast<const float4_t *>(x0)[i], b = reinterpret_cast<const float4_t *>(x1)[i];
+      float4_t v;
+      v.x = binary2<kOp>(a.x, b.x), v.y = binary2<kOp>(a.y, b.y);
+      v.z = binary2<kOp>(a.z, b.z), v.w = binary2<kOp>(a.w, b.w);
+      reinterpret_cast<float4_t *>(y)[i] = v;
+    }
+  }
+  const size_t done = vec ? 4 * n4 : 0;
+  for (size_t i = done + (size_t)blockIdx.x * kBlk + threadIdx.x; i < size; i += (size_t)gridDim.x * kBlk)
+    y[i] = binary2<kOp>(x0[i], x1[i]);
+}
+// (dx may be the array dy lives in -- never one of x0 / x1 the other gradient still needs: no __restrict__ on dx)
+template <int kOp, int kInput, bool kAccum>
+__global__ __launch_bounds__(kBlk) void binary2_grad_kernel(const float *dy, const float *__restrict__ x0,
+                                                            const float *__restrict__ x1, float *dx, size_t size) {
+  for (size_t i = (size_t)blockIdx.x * kBlk + threadIdx.x; i < size; i += (size_t)gridDim.x * kBlk) {
+    const float g = binary2_grad<kOp, kInput>(dy[i], kOp == kOpSub2 ? 0.0f : x0[i], kOp == kOpSub2 ? 0.0f : x1[i]);
+    dx[i] = (kAccum ? dx[i] : 0.0f) + g;
+  }
+}
+template <int kOp> int launch_binary2(const float *x0, const float *x1, float *y, size_t size, hipStream_t stream) {
+  const int vec = aligned16(x0) && aligned16(x1) && aligned16(y);
+  hipLaunchKernelGGL(binary2_kernel<kOp>, dim3(grid_for(vec ? size / 4 + 1 : size)), dim3(kBlk), 0, stream, x0, x1, y,
+                     size / 4, size, vec);
+  NBLA_HIP_LAUNCH_CHECK("binary2");
+  return NBLA_HIP_OK;
+}
+template <int kOp, int kInput>
+int launch_binary2_grad(const float *dy, const float *x0, const float *x1, float *dx, size_t size, int accum,
+                        hipStream_t stream) {
+  const dim3 g(grid_for(size)), b(kBlk);
+  if (accum)
+    hipLaunchKernelGGL((binary2_grad_kernel<kOp, kInput, true>), g, b, 0, stream, dy, x0, x1, dx, size);
+  else
+    hipLaunchKernelGGL((binary2_grad_kernel<kOp, kInput, false>), g, b, 0, stream, dy, x0, x1, dx, size);
+  NBLA_HIP_LAUNCH_CHECK("binary2 backward");
+  return NBLA_HIP_OK;
+}
+
 // dst[r * dst_stride + i] (+)= src[r * src_stride + i] for r < rows, i < len: the copies of Concatenate
 template <bool kAccum>
 __global__ __launch_bounds__(kBlk) void rows_copy_kernel(const float *__restrict__ src, int64_t src_stride,
@@ -279,6 +337,36 @@ int nbla_hip_add2_backward_f32(const float *dy, float *dx, size_t size, int accu
     hipLaunchKernelGGL((add_kernel<false, false>), g, b, 0, as_stream(stream), dy, nullptr, dx, size / 4, size, vec);
   NBLA_HIP_LAUNCH_CHECK("add2 backward");
   return NBLA_HIP_OK;
+}
+
+int nbla_hip_binary2_f32(int op, const float *x0, const float *x1, float *y, size_t size, void *stream) {
+  if (size == 0)
+    return NBLA_HIP_OK;
+  switch (op) {
+  case kOpSub2: return launch_binary2<kOpSub2>(x0, x1, y, size, as_stream(stream));
+  case kOpMul2: return launch_binary2<kOpMul2>(x0, x1, y, size, as_stream(stream));
+  case kOpDiv2: return launch_binary2<kOpDiv2>(x0, x1, y, size, as_stream(stream));
+  }
+  return fail(NBLA_HIP_ERR_VALUE, "binary2: unknown operation %d.", op);
+}
+
+int nbla_hip_binary2_backward_f32(int op, int input, const float *dy, const float *x0, const float *x1, float *dx,
+                                  size_t size, int accum, void *stream) {
+  if (size == 0)
+    return NBLA_HIP_OK;
+  if (input != 0 && input != 1)
+    return fail(NBLA_HIP_ERR_VALUE, "binary2 backward: input %d is not 0 or 1.", input);
+  hipStream_t s = as_stream(stream);
+#define NBLA_BINARY2_GRAD(OP)                                                                                          \
+  return input == 0 ? launch_binary2_grad<OP, 0>(dy, x0, x1, dx, size, accum, s)                                       \
+                    : launch_binary2_grad<OP, 1>(dy, x0, x1, dx, size, accum, s)
+  switch (op) {
+  case kOpSub2: NBLA_BINARY2_GRAD(kOpSub2);
+  case kOpMul2: NBLA_BINARY2_GRAD(kOpMul2);
+  case kOpDiv2: NBLA_BINARY2_GRAD(kOpDiv2);
+  }
+#undef NBLA_BINARY2_GRAD
+  return fail(NBLA_HIP_ERR_VALUE, "binary2 backward: unknown operation %d.", op);
 }
 
 int nbla_hip_copy_rows_f32(const float *src, int64_t src_stride, float *dst, int64_t dst_stride, int64_t rows,

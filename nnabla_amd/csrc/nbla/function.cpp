@@ -1,6 +1,9 @@
 // Function protocol, the per-function registries and the process-wide random generator.
 #include <nbla/function.hpp>
 #include <nbla/function/add2.hpp>
+#include <nbla/function/div2.hpp>
+#include <nbla/function/mul2.hpp>
+#include <nbla/function/sub2.hpp>
 #include <nbla/function/affine.hpp>
 #include <nbla/function/binary_connect_affine.hpp>
 #include <nbla/function/binary_connect_convolution.hpp>
@@ -110,6 +113,9 @@ NBLA_REGISTER_FUNCTION_SOURCE(DequantizeLinear);
 NBLA_REGISTER_FUNCTION_SOURCE(Prune, float);
 NBLA_REGISTER_FUNCTION_SOURCE(Sink, bool);
 NBLA_REGISTER_FUNCTION_SOURCE(Add2, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(Sub2, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(Mul2, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(Div2, bool);
 NBLA_REGISTER_FUNCTION_SOURCE(Concatenate, int);
 
 // ----------------------------------------------------------------- RandomManager

@@ -133,6 +133,21 @@ def add2(x0, x1, inplace=False, n_outputs=-1, outputs=None):
     return f(x0, x1, n_outputs=n_outputs, outputs=outputs)
 
 
+def sub2(x0, x1, inplace=False, n_outputs=-1, outputs=None):
+    f = Function("Sub2", None, [int(inplace)], args=dict(inplace=inplace))
+    return f(x0, x1, n_outputs=n_outputs, outputs=outputs)
+
+
+def mul2(x0, x1, inplace=False, n_outputs=-1, outputs=None):
+    f = Function("Mul2", None, [int(inplace)], args=dict(inplace=inplace))
+    return f(x0, x1, n_outputs=n_outputs, outputs=outputs)
+
+
+def div2(x0, x1, inplace=False, n_outputs=-1, outputs=None):
+    f = Function("Div2", None, [int(inplace)], args=dict(inplace=inplace))
+    return f(x0, x1, n_outputs=n_outputs, outputs=outputs)
+
+
 def concatenate(*x, **kw):
     axis = kw.pop('axis', None)
     n_outputs, outputs = kw.pop('n_outputs', -1), kw.pop('outputs', None)

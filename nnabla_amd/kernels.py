@@ -44,7 +44,7 @@ EXPORTED = (
     "nbla_hip_get_device_count", "nbla_hip_set_device", "nbla_hip_malloc", "nbla_hip_free", "nbla_hip_mem_info",
     "nbla_hip_memcpy", "nbla_hip_device_synchronize", "nbla_hip_stream_synchronize", "nbla_hip_fill",
     "nbla_hip_cast", "nbla_hip_relu_f32", "nbla_hip_relu_backward_f32", "nbla_hip_add2_f32",
-    "nbla_hip_add2_backward_f32", "nbla_hip_copy_rows_f32",
+    "nbla_hip_add2_backward_f32", "nbla_hip_binary2_f32", "nbla_hip_binary2_backward_f32", "nbla_hip_copy_rows_f32",
 )
 
 

@@ -5,7 +5,7 @@
 
 Functions are created through the registry for the *current* context, so a graph loaded under the ``hip`` extension
 context runs on the hip:float classes (the dispatch nnp_impl_create_function.cpp.tmpl:51-117 performs for every
-function; here for the nine quantization functions, QuantizeLinear, DequantizeLinear, Prune, Affine, ReLU, Add2 and
+function; here for the nine quantization functions, QuantizeLinear, DequantizeLinear, Prune, Affine, ReLU, Add2, Sub2, Mul2, Div2 and
 Concatenate).
 Network definitions are read from protobuf text (``.nntxt`` / ``.prototxt``) or from binary protobuf
 (``.protobuf``, load.py:492-494), parameters from ``parameter.protobuf`` or from ``parameter`` entries of either.
@@ -78,6 +78,9 @@ _BUILDERS = {
         i[0], i[1], _opt(i, 2), channel_last=bool(p.get("channel_last", False)), **_conv_kwargs(p))),
     "ReLU": ("relu_param", 1, lambda p, i: F.relu(i[0], inplace=bool(p.get("inplace", False)))),
     "Add2": ("add2_param", 2, lambda p, i: F.add2(i[0], i[1], inplace=bool(p.get("inplace", False)))),
+    "Sub2": ("sub2_param", 2, lambda p, i: F.sub2(i[0], i[1], inplace=bool(p.get("inplace", False)))),
+    "Mul2": ("mul2_param", 2, lambda p, i: F.mul2(i[0], i[1], inplace=bool(p.get("inplace", False)))),
+    "Div2": ("div2_param", 2, lambda p, i: F.div2(i[0], i[1], inplace=bool(p.get("inplace", False)))),
     "Concatenate": ("concatenate_param", 2, lambda p, i: F.concatenate(
         *i, axis=int(p.get("axis", len(i[0].shape) - 1)))),
     "QuantizeLinear": ("quantize_linear_param", 3, lambda p, i: F.quantize_linear(

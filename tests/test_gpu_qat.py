@@ -316,6 +316,46 @@ def test_scheduler_end_to_end(ctx):
     assert np.abs(nn.get_parameter('c1/conv/W').g).max() > 0
 
 
+@pytest.mark.parametrize("name", ["sub2", "mul2", "div2"])
+def test_two_input_arithmetic_functions(ctx, name):
+    """Sub2, Mul2, Div2 (sub2.hpp:41, mul2.hpp:42, div2.hpp:44) through the registry: fp32 results bit for bit (one
+    IEEE operation per element), and the gradients of base_transform_binary.hpp:286-336 -- dy, -dy | dy * x1, dy * x0 |
+    dy / x1, -dy * x0 / (x1 * x1), each operation rounded on its own -- overwritten and accumulated."""
+    rng = np.random.default_rng(23)
+    shape = (5, 7, 9)                                           # 315 elements: a vector part and a tail
+    a = rng.standard_normal(shape).astype(np.float32)
+    b = (rng.standard_normal(shape) + np.float32(3.0) * rng.choice([-1, 1], shape)).astype(np.float32)
+    a.ravel()[:3] = [0.0, -0.0, np.inf]
+    f32 = np.float32
+    with np.errstate(all="ignore"):
+        fwd = {"sub2": a - b, "mul2": a * b, "div2": a / b}[name]
+        g = rng.standard_normal(shape).astype(np.float32)
+        g0 = {"sub2": g, "mul2": g * b, "div2": g / b}[name]
+        g1 = {"sub2": -g, "mul2": g * a, "div2": (-g * a) / (b * b)}[name]
+    va, vb = _var(a), _var(b)
+    va.need_grad = vb.need_grad = True
+    y = getattr(F, name)(va, vb)
+    y.forward()
+    assert bits_equal(y.d, fwd.astype(f32))
+    va.g, vb.g = 0.0, 0.0
+    y.backward(g)
+    with np.errstate(all="ignore"):
+        assert bits_equal(va.g, (f32(0) + g0).astype(f32)) and bits_equal(vb.g, (f32(0) + g1).astype(f32))
+    # one variable on both sides: its gradient is the sum of the two (x - x, x * x, x / x)
+    vc = _var(b)
+    vc.need_grad = True
+    z = getattr(F, name)(vc, vc)
+    z.forward()
+    vc.g = 0.0
+    z.backward(g)
+    with np.errstate(all="ignore"):
+        h0 = {"sub2": g, "mul2": g * b, "div2": g / b}[name]
+        h1 = {"sub2": -g, "mul2": g * b, "div2": (-g * b) / (b * b)}[name]
+        assert bits_equal(vc.g, ((f32(0) + h0) + h1).astype(f32))
+    with pytest.raises(RuntimeError):
+        getattr(F, name)(va, _var(np.zeros((5, 1, 9), np.float32)))     # broadcasting is not available
+
+
 def test_add2_and_concatenate_functions(ctx):
     """add2.cpp:39-77 and concatenate.cpp:62-104 through the registry: forward values, gradients written and
     accumulated, shape checks."""

@@ -41,6 +41,7 @@ def every_function_net(x):
 
     h = F.convolution(x, p('conv/W', (4, 3, 3, 3)), p('conv/b', (4,)), pad=(1, 1), stride=(1, 1), dilation=(1, 1))
     h = F.relu(h)
+    h = F.div2(F.mul2(h, F.relu(h)), F.sub2(h, F.add2(h, h)))
     h = F.fixed_point_quantize(h, False, 6, 0.25, ste_fine_grained=False)
     h = F.pow2_quantize(h, True, False, 5, 2)
     h = F.min_max_quantize(h, p('mmq/qr_min', (1, 1, 1, 1), False), p('mmq/qr_max', (1, 1, 1, 1), False),

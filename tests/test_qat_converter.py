@@ -313,6 +313,28 @@ def test_add2_inputs_share_the_recorder_of_the_earliest_one():
     assert r1.inputs[0].parent.info.type_name == 'ReLU'      # r's own recorder is gone from the graph
 
 
+def gated_net(x):
+    h = F.relu(PF.convolution(x, 4, (3, 3), pad=(1, 1), name='c1'))      # Convolution-0, ReLU-1
+    r = F.relu(PF.convolution(h, 4, (3, 3), pad=(1, 1), name='c2'))      # Convolution-2, ReLU-3
+    return PF.affine(F.mul2(h, r), 5, name='f')                          # Mul2-4, Affine-5
+
+
+def test_mul2_inputs_are_two_activations_with_recorders_of_their_own():
+    """quantize.py:30-36, 148-152: both inputs of Sub2 / Mul2 / Div2 are activations and get recorders, but -- unlike
+    Add2 / Concatenate (quantize.py:112-116) -- each keeps its own statistics: h the one it already has as the second
+    convolution's input, r a new one named after the consumer's input ('Mul2-4/x1')."""
+    x = nn.Variable((2, 3, 8, 8))
+    cfg = QATConfig()
+    y_rec = to_recording(gated_net(x), cfg)
+    act = cfg.recorder_activation().name()
+    mul = find(y_rec, 'Mul2')[0]
+    r0, r1 = mul.inputs[0].parent, mul.inputs[1].parent
+    assert r0.info.type_name == r1.info.type_name == act and r0 is not r1
+    assert r0.inputs[1] is nn.get_parameter('Convolution-2/M-x0')
+    assert r1.inputs[1] is nn.get_parameter('Mul2-4/M-x1')
+    assert r1.inputs[0].parent.info.type_name == 'ReLU' and r1.inputs[0].parent.inputs[0].parent is not None
+
+
 def test_concatenate_inputs_share_the_recorder_of_the_earliest_one():
     x = nn.Variable((2, 3, 8, 8))
     cfg = QATConfig()
