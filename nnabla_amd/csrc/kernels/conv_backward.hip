@@ -89,6 +89,60 @@ __global__ __launch_bounds__(256) void col2im_gather(const float *__restrict__ c
   }
 }
 
+// The same for unit strides and at most 64 taps, with the loads of sixteen taps in flight at a time (the loop above
+// waits for every load before it issues the next: nine round trips to the L2 for a 3 x 3 kernel).  The taps'
+// displacements are decoded once per block into LDS; a tap that does not reach the element contributes through a
+// select, not through an addition of zero, so the sum is the same chain of additions as above.
+__global__ __launch_bounds__(256) void col2im_gather_unit(const float *__restrict__ colg, float *__restrict__ dx,
+                                                          ConvGeom g, int64_t grp, int accumulate) {
+  typedef int i32x4_t __attribute__((ext_vector_type(4)));
+  __shared__ i32x4_t s_taps[64]; // {displacement along each spatial axis, 0}
+  const int in0 = g.in_sp[0], in1 = g.in_sp[1], in2 = g.in_sp[2], plane = (int)g.in_sp_size, Cg = (int)g.Cg;
+  const int out0 = g.out_sp[0], out1 = g.out_sp[1], out2 = g.out_sp[2], L = (int)g.out_sp_size;
+  const int taps = (int)g.k_size;
+  if ((int)threadIdx.x < taps) {
+    int q = threadIdx.x;
+    const int k2 = q % g.k[2];
+    q /= g.k[2];
+    const int k1 = q % g.k[1], k0 = q / g.k[1];
+    s_taps[threadIdx.x] = i32x4_t{k0 * g.dil[0] - g.pad[0], k1 * g.dil[1] - g.pad[1], k2 * g.dil[2] - g.pad[2], 0};
+  }
+  __syncthreads();
+  const int per_sample = Cg * plane;
+  const int64_t n = blockIdx.y;
+  const float *sample = colg + n * g.Kg * g.out_sp_size;
+  float *dst_sample = dx + (n * g.C + grp * g.Cg) * g.in_sp_size;
+  for (int idx = blockIdx.x * 256 + threadIdx.x; idx < per_sample; idx += gridDim.x * 256) {
+    int t = idx;
+    const int i2 = t % in2;
+    t /= in2;
+    const int i1 = t % in1;
+    t /= in1;
+    const int i0 = t % in0;
+    const int cc = t / in0;
+    const float *src = sample + (int64_t)cc * taps * L;
+    float acc = 0.0f;
+    for (int tap0 = 0; tap0 < taps; tap0 += 16) {
+      float v[16];
+      bool ok[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int tap = tap0 + j < taps ? tap0 + j : taps - 1;
+        const i32x4_t d = s_taps[tap];
+        const int q0 = i0 - d.x, q1 = i1 - d.y, q2 = i2 - d.z;
+        ok[j] = tap0 + j < taps && (unsigned)q0 < (unsigned)out0 && (unsigned)q1 < (unsigned)out1 &&
+                (unsigned)q2 < (unsigned)out2;
+        v[j] = src[ok[j] ? tap * L + (q0 * out1 + q1) * out2 + q2 : 0];
+      }
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        acc = ok[j] ? acc + v[j] : acc;
+    }
+    float *dst = dst_sample + idx;
+    *dst = accumulate ? *dst + acc : acc;
+  }
+}
+
 struct ConvBackwardPlan {
   size_t dyt_off, scaled_off, col_off, a_planes_off, b_planes_off, digits_off, bits_off, prep_off, count_off,
       flag_off, sums_off, total;
@@ -146,7 +200,9 @@ int launch_col2im(const float *colg, float *dx, const ConvGeom &g, int64_t grp, 
     bx = 65536;
   const dim3 grid((unsigned)bx, (unsigned)g.outer);
   const bool unit = g.stride[0] == 1 && g.stride[1] == 1 && g.stride[2] == 1;
-  if (unit)
+  if (unit && g.k_size <= 64)
+    hipLaunchKernelGGL(col2im_gather_unit, grid, dim3(256), 0, stream, colg, dx, g, grp, accumulate ? 1 : 0);
+  else if (unit)
     hipLaunchKernelGGL(col2im_gather<true>, grid, dim3(256), 0, stream, colg, dx, g, grp, accumulate ? 1 : 0);
   else
     hipLaunchKernelGGL(col2im_gather<false>, grid, dim3(256), 0, stream, colg, dx, g, grp, accumulate ? 1 : 0);
