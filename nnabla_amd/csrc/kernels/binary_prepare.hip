@@ -497,29 +497,10 @@ __device__ __forceinline__ int digit_shift(uint32_t amax_bits) {
 }
 __device__ __forceinline__ int to_fixed(float v, int s) { return (int)rintf(ldexpf(v, s)); }
 
-// q = d0 * 65536 + d1 * 256 + d2 with every digit in [-128, 127]
-__device__ __forceinline__ void balanced_digits(int q, uint32_t &d0, uint32_t &d1, uint32_t &d2) {
-  const int lo = (int)(int8_t)q;
-  const int q1 = (q - lo) >> 8;
-  const int mid = (int)(int8_t)q1;
-  const int hi = (q1 - mid) >> 8;
-  d0 = (uint32_t)hi & 0xffu;
-  d1 = (uint32_t)mid & 0xffu;
-  d2 = (uint32_t)lo & 0xffu;
-}
-
 // Sixteen fixed-point values of one lane -> its 16 bytes of each digit fragment.
 __device__ __forceinline__ void store_digits(const int (&q)[16], uint4_t *dst, bool streaming) {
-  uint32_t w[3][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
-#pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    uint32_t d0, d1, d2;
-    balanced_digits(q[j], d0, d1, d2);
-    const int sh = 8 * (j & 3);
-    w[0][j >> 2] |= d0 << sh;
-    w[1][j >> 2] |= d1 << sh;
-    w[2][j >> 2] |= d2 << sh;
-  }
+  uint32_t w[3][4];
+  pack_digits(q, w);
 #pragma unroll
   for (int d = 0; d < 3; ++d) {
     uint4_t o;

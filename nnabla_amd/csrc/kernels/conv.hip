@@ -234,21 +234,14 @@ __global__ __launch_bounds__(256) void im2col_digits(const float *__restrict__ x
       const float xv = xn[ok ? origin + e.x : 0];
       v[j] = ok ? xv : 0.0f;
     }
-    uint32_t w[3][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
-    int part = 0;
+    uint32_t w[3][4];
+    int qv[16], part = 0;
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
-      const int qv = to_fixed(v[j], s); // masked values are 0.0f -> 0 whatever the shift
-      part += qv;
-      const int lo = (int)(int8_t)qv;
-      const int q1 = (qv - lo) >> 8;
-      const int mid = (int)(int8_t)q1;
-      const int hi = (q1 - mid) >> 8;
-      const int sh = 8 * (j & 3);
-      w[0][j >> 2] |= ((uint32_t)hi & 0xffu) << sh;
-      w[1][j >> 2] |= ((uint32_t)mid & 0xffu) << sh;
-      w[2][j >> 2] |= ((uint32_t)lo & 0xffu) << sh;
+      qv[j] = to_fixed(v[j], s); // masked values are 0.0f -> 0 whatever the shift
+      part += qv[j];
     }
+    pack_digits(qv, w);
     row_sum[(kt * kTileK) / kChunkK - (kt_begin * kTileK) / kChunkK] += part;
     uint4_t *dst = out + ((rb * k_tiles + kt) * kDigits) * 64 + lane;
 #pragma unroll
@@ -374,19 +367,12 @@ __global__ __launch_bounds__(256) void im2col_digits_columns(const float *__rest
       const float xv = x[ok ? base + delta : 0];
       v[j] = ok ? xv : 0.0f;
     }
-    uint32_t w[3][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+    uint32_t w[3][4];
+    int qv[16];
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      const int qv = to_fixed(v[j], s);
-      const int lo = (int)(int8_t)qv;
-      const int q1 = (qv - lo) >> 8;
-      const int mid = (int)(int8_t)q1;
-      const int hi = (q1 - mid) >> 8;
-      const int sh = 8 * (j & 3);
-      w[0][j >> 2] |= ((uint32_t)hi & 0xffu) << sh;
-      w[1][j >> 2] |= ((uint32_t)mid & 0xffu) << sh;
-      w[2][j >> 2] |= ((uint32_t)lo & 0xffu) << sh;
-    }
+    for (int j = 0; j < 16; ++j)
+      qv[j] = to_fixed(v[j], s);
+    pack_digits(qv, w);
     uint4_t *dst = out + ((rb * k_tiles + kt) * kDigits) * 64 + lane;
 #pragma unroll
     for (int d = 0; d < 3; ++d) {

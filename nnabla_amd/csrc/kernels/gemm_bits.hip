@@ -443,29 +443,15 @@ __device__ __forceinline__ void unfold_main_loop(const GemmBitsArgs &a, unsigned
       v[j] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(xrsrc, (int)at, 0, 0));
     }
   };
-  // The three balanced base-256 digits of q (|q| <= kDigitMax) are the low three bytes of q + 0x808080, each with its
-  // top bit flipped: adding 128 per digit position makes every digit a plain byte.
   auto emit = [&](int stage, const float (&v)[16], const uint4_t &words) __attribute__((always_inline)) {
     uint32_t w[3][4];
-    int part = 0;
+    int qv[16], part = 0;
 #pragma unroll
-    for (int g4 = 0; g4 < 4; ++g4) {
-      uint32_t d[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int qv = (int)rintf(ldexpf(v[4 * g4 + j], s_row)); // masked values are 0.0f -> 0 whatever the shift
-        part += qv;
-        d[j] = ((uint32_t)qv + 0x808080u) ^ 0x808080u; // bytes: lowest, middle, top digit, unused
-      }
-      // byte transpose: word of a digit = that digit of the four values, value j in byte j
-      const uint32_t t01 = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u); // d0.b0 d1.b0 d0.b1 d1.b1
-      const uint32_t t23 = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u);
-      const uint32_t u01 = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u); // d0.b2 d1.b2 d0.b3 d1.b3
-      const uint32_t u23 = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
-      w[2][g4] = __builtin_amdgcn_perm(t23, t01, 0x05040100u); // lowest digits
-      w[1][g4] = __builtin_amdgcn_perm(t23, t01, 0x07060302u); // middle digits
-      w[0][g4] = __builtin_amdgcn_perm(u23, u01, 0x05040100u); // top digits
+    for (int j = 0; j < 16; ++j) {
+      qv[j] = (int)rintf(ldexpf(v[j], s_row)); // masked values are 0.0f -> 0 whatever the shift
+      part += qv[j];
     }
+    pack_digits(qv, w);
     uint4_t *dst = reinterpret_cast<uint4_t *>(smem + (stage & 1) * kBufBytes + tile_off +
                                                (wave & 1) * kDigits * kFragBytes) + lane;
 #pragma unroll

@@ -92,6 +92,28 @@ __host__ __device__ inline DigitOperand digit_operand(int64_t M, int64_t K) {
 }
 
 #if defined(__HIPCC__)
+// Sixteen fixed-point values q (|q| <= kDigitMax) of one lane -> its four words of each digit fragment (digit 0 the
+// top one; value j in byte j % 4 of word j / 4).  The three balanced base-256 digits of q are the low three bytes of
+// q + 0x808080, each with its top bit flipped: adding 128 per digit position makes every digit a plain byte, and the
+// carries between the positions are exactly the borrows of the balanced form.  Four values' digits are then
+// transposed into one word per digit with byte permutes.
+__device__ __forceinline__ void pack_digits(const int (&q)[16], uint32_t (&w)[3][4]) {
+#pragma unroll
+  for (int g4 = 0; g4 < 4; ++g4) {
+    uint32_t d[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      d[j] = ((uint32_t)q[4 * g4 + j] + 0x808080u) ^ 0x808080u; // bytes: lowest, middle, top digit, unused
+    const uint32_t t01 = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u); // d0.b0 d1.b0 d0.b1 d1.b1
+    const uint32_t t23 = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u);
+    const uint32_t u01 = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u); // d0.b2 d1.b2 d0.b3 d1.b3
+    const uint32_t u23 = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
+    w[2][g4] = __builtin_amdgcn_perm(t23, t01, 0x05040100u); // lowest digits
+    w[1][g4] = __builtin_amdgcn_perm(t23, t01, 0x07060302u); // middle digits
+    w[0][g4] = __builtin_amdgcn_perm(u23, u01, 0x05040100u); // top digits
+  }
+}
+
 // Blocks are handed to the 8 XCDs round-robin; give each XCD a contiguous run
 // of tiles (n fastest) so that blocks resident on one XCD share an X panel in
 // that XCD's L2.
