@@ -167,6 +167,154 @@ __global__ __launch_bounds__(256) void conv_row_shift(const uint32_t *__restrict
   shift[m] = s;
 }
 
+// The two kernels above in one launch, for geometries where the input positions under 32 consecutive windows fit a
+// small table: a block owns 32 rows of the unfolded matrix (consecutive output positions, so their windows overlap).
+// It takes, for every input position the windows can touch -- per run of rows that lie in one sample ("segment") one
+// range [lo, hi] of the flattened plane, consecutive lanes on consecutive positions -- the maximum over the channels,
+// and a row's largest magnitude is the maximum over its taps' positions.  Same shifts as conv_row_shift gives.
+constexpr int kShiftBlock = 512, kShiftPixCap = 4096;
+__global__ __launch_bounds__(kShiftBlock) void conv_row_shift_windows(const float *__restrict__ x,
+                                                                      long long *__restrict__ sums,
+                                                                      int32_t *__restrict__ shift, ConvGeom g,
+                                                                      int64_t grp, int64_t rows, int64_t chunks) {
+  typedef int i32x4_t __attribute__((ext_vector_type(4)));
+  __shared__ uint32_t s_pix[kShiftPixCap];
+  __shared__ i32x4_t s_taps[64]; // {offset inside the plane, displacements along axes 0 and 1 (16 bits each), axis 2}
+  __shared__ int seg_lo[32], seg_hi[32], seg_n[32], row_seg[32], seg_count;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int in0 = g.in_sp[0], in1 = g.in_sp[1], in2 = g.in_sp[2], plane = (int)g.in_sp_size, taps = (int)g.k_size;
+  if (tid < taps) {
+    int q = tid;
+    const int k2 = q % g.k[2];
+    q /= g.k[2];
+    const int k1 = q % g.k[1], k0 = q / g.k[1];
+    const int e0 = k0 * g.dil[0], e1 = k1 * g.dil[1], e2 = k2 * g.dil[2];
+    s_taps[tid] = i32x4_t{(e0 * in1 + e1) * in2 + e2, e0 | (e1 << 16), e2, 0};
+  }
+  if (tid < 32) {
+    seg_lo[tid] = 0x7fffffff;
+    seg_hi[tid] = -1;
+  }
+  for (int i = tid; i < kShiftPixCap; i += kShiftBlock)
+    s_pix[i] = 0u;
+  // this thread's row (rows past the last one, of the padded operand, get shift 0)
+  const int r = lane & 31;
+  const int64_t m = (int64_t)blockIdx.x * 32 + r;
+  const bool in_range = m < g.M;
+  const int64_t n = in_range ? m / g.out_sp_size : 0;
+  int p = in_range ? (int)(m - n * g.out_sp_size) : 0;
+  const int o2 = p % g.out_sp[2];
+  p /= g.out_sp[2];
+  const int o1 = p % g.out_sp[1];
+  const int o0 = p / g.out_sp[1];
+  const int b0 = o0 * g.stride[0] - g.pad[0], b1 = o1 * g.stride[1] - g.pad[1], b2 = o2 * g.stride[2] - g.pad[2];
+  const int origin = (b0 * in1 + b1) * in2 + b2;
+  __syncthreads();
+  if (tid < 32) {
+    const unsigned long long starts = __ballot(in_range && (r == 0 || m / g.out_sp_size != (m - 1) / g.out_sp_size));
+    const int seg = __popcll(starts & ((2ull << r) - 1ull)) - 1;
+    row_seg[r] = in_range ? seg : 0;
+    if (in_range) {
+      int last = 0; // the largest tap offset
+      for (int t = 0; t < taps; ++t)
+        last = max(last, s_taps[t].x);
+      atomicMin(&seg_lo[seg], origin > 0 ? origin : 0);
+      atomicMax(&seg_hi[seg], origin + last < plane - 1 ? origin + last : plane - 1);
+      seg_n[seg] = (int)n;
+    }
+    if (r == 0)
+      seg_count = __popcll(starts & 0xffffffffull);
+  }
+  __syncthreads();
+  const int nseg = seg_count;
+  int my_base = 0, total = 0;
+  for (int sgm = 0; sgm < nseg; ++sgm) {
+    const int len = seg_hi[sgm] - seg_lo[sgm] + 1;
+    if (sgm == row_seg[r])
+      my_base = total;
+    total += len > 0 ? len : 0;
+  }
+  // (the host launches this kernel only when every block's positions fit: see conv_row_shift_windows_fits)
+  const int Cg = (int)g.Cg;
+  int base = 0;
+  for (int sgm = 0; sgm < nseg; ++sgm) {
+    const int lo = seg_lo[sgm], len = seg_hi[sgm] - lo + 1;
+    if (len <= 0)
+      continue;
+    const float *xs = x + ((int64_t)seg_n[sgm] * g.C + grp * g.Cg) * g.in_sp_size + lo;
+    for (int p0 = 0; p0 < len; p0 += 64) {
+      const int pix = p0 + lane;
+      const bool live = pix < len && base + pix < kShiftPixCap;
+      const float *src = xs + (live ? pix : 0);
+      uint32_t amax = 0u;
+      // channels wave, wave + 8, ...: sixteen loads in flight
+      for (int c0 = wave; c0 < Cg; c0 += 8 * 16) {
+        float v[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const int c = c0 + 8 * j;
+          v[j] = src[(int64_t)(c < Cg ? c : wave) * plane];
+        }
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+          if (c0 + 8 * j < Cg)
+            amax = max(amax, __float_as_uint(v[j]) & 0x7fffffffu);
+      }
+      if (live && amax)
+        atomicMax(&s_pix[base + pix], amax);
+    }
+    base += len;
+  }
+  __syncthreads();
+  if (tid < 32) {
+    if (m < rows) {
+      for (int64_t c = 0; c < chunks; ++c)
+        sums[c * rows + m] = 0;
+      uint32_t amax = 0u;
+      const int rel = my_base + origin - seg_lo[row_seg[r]];
+      for (int t = 0; t < taps; ++t) {
+        const i32x4_t e = s_taps[t];
+        const int i0 = b0 + (e.y & 0xffff), i1 = b1 + (int)((uint32_t)e.y >> 16), i2 = b2 + e.z;
+        if (in_range && (unsigned)i0 < (unsigned)in0 && (unsigned)i1 < (unsigned)in1 && (unsigned)i2 < (unsigned)in2)
+          amax = max(amax, s_pix[rel + e.x]);
+      }
+      int sft = 0;
+      if (amax >= 0x7f800000u) {
+        sft = kBadRow;
+      } else if (amax != 0u) {
+        sft = 22 - binade_exponent(binade_of(amax));
+        if (rintf(ldexpf(__uint_as_float(amax), sft)) > (float)kDigitMax)
+          --sft;
+      }
+      shift[m] = sft;
+    }
+  }
+}
+
+// Whether 32 consecutive windows always touch few enough input positions for conv_row_shift_windows: the positions of
+// a run of r windows inside one sample span at most the flattened offset of r - 1 steps of the output walk (whole
+// rows / planes of the output counted where the run can cross them) plus the last tap's offset.
+bool conv_row_shift_windows_fits(const ConvGeom &g) {
+  if (g.k_size > 64 || g.Cg * g.in_sp_size >= ((int64_t)1 << 31))
+    return false;
+  for (int i = 0; i < kMaxSpatial; ++i)
+    if ((int64_t)(g.k[i] - 1) * g.dil[i] >= 65536)
+      return false;
+  const int64_t r = 32;
+  const int64_t d2 = r - 1 < g.out_sp[2] - 1 ? r - 1 : g.out_sp[2] - 1;
+  const int64_t c1 = ceil_div(r, (int64_t)g.out_sp[2]), d1 = c1 < g.out_sp[1] - 1 ? c1 : g.out_sp[1] - 1;
+  const int64_t c0 = ceil_div(r, (int64_t)g.out_sp[1] * g.out_sp[2]), d0 = c0 < g.out_sp[0] - 1 ? c0 : g.out_sp[0] - 1;
+  const int64_t walk = (d0 * g.stride[0] * g.in_sp[1] + d1 * g.stride[1]) * g.in_sp[2] + d2 * g.stride[2];
+  const int64_t last = ((int64_t)(g.k[0] - 1) * g.dil[0] * g.in_sp[1] + (int64_t)(g.k[1] - 1) * g.dil[1]) * g.in_sp[2] +
+                       (int64_t)(g.k[2] - 1) * g.dil[2];
+  int64_t len = walk + last + 1;
+  if (len > g.in_sp_size)
+    len = g.in_sp_size;
+  // a block's rows lie in at most this many samples; every segment may be as long as the bound
+  const int64_t segments = ceil_div(r - 1, g.out_sp_size) + 1;
+  return len * segments <= kShiftPixCap;
+}
+
 // A wavefront converts kTilesPerWave consecutive k tiles of one row block: lane l owns row rb*32 + l%32 and the
 // k-slots (l/32)*16 + 0..15 of each tile.  The wavefront first decodes its 64 column indices k -> (channel, tap),
 // one per lane, into a wavefront-private LDS table {offset of the tap relative to the window origin, tap
@@ -410,13 +558,19 @@ int launch_im2col_digits(const float *x, void *xdigits, void *scratch, const Con
   char *base = static_cast<char *>(xdigits);
   long long *sums = reinterpret_cast<long long *>(base + d.sum_off);
   int32_t *shift = reinterpret_cast<int32_t *>(base + d.shift_off);
-  uint32_t *cmax = static_cast<uint32_t *>(scratch);
-  hipLaunchKernelGGL(conv_channel_max, dim3((unsigned)ceil_div(g.outer * g.in_sp_size, 256), kChannelSlices), dim3(256),
-                     0, stream, x, cmax, g, grp);
-  NBLA_HIP_LAUNCH_CHECK("conv_channel_max");
-  hipLaunchKernelGGL(conv_row_shift, dim3((unsigned)ceil_div(d.rows, 256)), dim3(256), 0, stream, cmax, sums, shift, g,
-                     d.rows, d.chunks);
-  NBLA_HIP_LAUNCH_CHECK("conv_row_shift");
+  if (conv_row_shift_windows_fits(g)) {
+    hipLaunchKernelGGL(conv_row_shift_windows, dim3((unsigned)d.row_blocks), dim3(kShiftBlock), 0, stream, x, sums,
+                       shift, g, grp, d.rows, d.chunks);
+    NBLA_HIP_LAUNCH_CHECK("conv_row_shift_windows");
+  } else {
+    uint32_t *cmax = static_cast<uint32_t *>(scratch);
+    hipLaunchKernelGGL(conv_channel_max, dim3((unsigned)ceil_div(g.outer * g.in_sp_size, 256), kChannelSlices),
+                       dim3(256), 0, stream, x, cmax, g, grp);
+    NBLA_HIP_LAUNCH_CHECK("conv_channel_max");
+    hipLaunchKernelGGL(conv_row_shift, dim3((unsigned)ceil_div(d.rows, 256)), dim3(256), 0, stream, cmax, sums, shift,
+                       g, d.rows, d.chunks);
+    NBLA_HIP_LAUNCH_CHECK("conv_row_shift");
+  }
   const int64_t tile_groups = ceil_div(d.k_tiles, kTilesPerWave), jobs = d.row_blocks * tile_groups;
   hipLaunchKernelGGL(im2col_digits, dim3((unsigned)ceil_div(jobs, 4)), dim3(256), 0, stream, x, shift, sums,
                      reinterpret_cast<uint4_t *>(base), g, grp, d.k_tiles, tile_groups, d.rows, jobs);
