@@ -172,7 +172,7 @@ __global__ __launch_bounds__(256) void conv_row_shift(const uint32_t *__restrict
 // It takes, for every input position the windows can touch -- per run of rows that lie in one sample ("segment") one
 // range [lo, hi] of the flattened plane, consecutive lanes on consecutive positions -- the maximum over the channels,
 // and a row's largest magnitude is the maximum over its taps' positions.  Same shifts as conv_row_shift gives.
-constexpr int kShiftBlock = 512, kShiftPixCap = 4096;
+constexpr int kShiftBlock = 1024, kShiftWaves = kShiftBlock / 64, kShiftPixCap = 4096;
 __global__ __launch_bounds__(kShiftBlock) void conv_row_shift_windows(const float *__restrict__ x,
                                                                       long long *__restrict__ sums,
                                                                       int32_t *__restrict__ shift, ConvGeom g,
@@ -247,17 +247,17 @@ __global__ __launch_bounds__(kShiftBlock) void conv_row_shift_windows(const floa
       const bool live = pix < len && base + pix < kShiftPixCap;
       const float *src = xs + (live ? pix : 0);
       uint32_t amax = 0u;
-      // channels wave, wave + 8, ...: sixteen loads in flight
-      for (int c0 = wave; c0 < Cg; c0 += 8 * 16) {
+      // channels wave, wave + kShiftWaves, ...: sixteen loads in flight
+      for (int c0 = wave; c0 < Cg; c0 += kShiftWaves * 16) {
         float v[16];
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
-          const int c = c0 + 8 * j;
+          const int c = c0 + kShiftWaves * j;
           v[j] = src[(int64_t)(c < Cg ? c : wave) * plane];
         }
 #pragma unroll
         for (int j = 0; j < 16; ++j)
-          if (c0 + 8 * j < Cg)
+          if (c0 + kShiftWaves * j < Cg)
             amax = max(amax, __float_as_uint(v[j]) & 0x7fffffffu);
       }
       if (live && amax)
@@ -541,6 +541,110 @@ __global__ __launch_bounds__(256) void im2col_f32(const float *__restrict__ x, f
   }
 }
 
+// The same conversion with the gather reduced to one bounds-checked buffer load per element, for kernels of at most
+// 64 taps and inputs below 2 GiB.  A block owns one row block and eight consecutive k tiles (two per wavefront).  It
+// writes, per row and tap, the byte offset in x of that tap's element of channel 0 -- or an offset past the end of x
+// when the tap falls outside the input, the row holds a non-finite value or lies past the last row -- and, per
+// column, the byte offset of its channel's plane and its tap (columns past Kg: the tap entry that is never valid).
+// An element is then a load at the sum of the two; out-of-range loads return zero, so there are no validity tests
+// or selects per element.
+constexpr int kRowTaps = 65;
+constexpr uint32_t kNowhere = 0x80000000u; // a byte offset past every input this kernel accepts
+__global__ __launch_bounds__(256) void im2col_digits_taps(const float *__restrict__ x, const int32_t *__restrict__ shift,
+                                                          long long *__restrict__ sums, uint4_t *__restrict__ out,
+                                                          ConvGeom g, int64_t grp, int64_t k_tiles,
+                                                          int64_t groups_per_row, int64_t rows) {
+  typedef int i32x4_t __attribute__((ext_vector_type(4)));
+  typedef int i32x2_t __attribute__((ext_vector_type(2)));
+  __shared__ i32x4_t s_taps[64];
+  __shared__ uint32_t row_taps[32 * kRowTaps];
+  __shared__ i32x2_t cols[4][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t rb = blockIdx.x / groups_per_row, bg = blockIdx.x - rb * groups_per_row;
+  const int64_t kt_begin = (bg * 4 + wave) * kTilesPerWave;
+  const int in0 = g.in_sp[0], in1 = g.in_sp[1], in2 = g.in_sp[2], plane = (int)g.in_sp_size, taps = (int)g.k_size;
+  if (tid < taps) {
+    int q = tid;
+    const int k2 = q % g.k[2];
+    q /= g.k[2];
+    const int k1 = q % g.k[1], k0 = q / g.k[1];
+    const int e0 = k0 * g.dil[0], e1 = k1 * g.dil[1], e2 = k2 * g.dil[2];
+    s_taps[tid] = i32x4_t{(e0 * in1 + e1) * in2 + e2, e0 | (e1 << 16), e2, 0};
+  }
+  {
+    const int kk = (int)(kt_begin * kTileK) + lane;
+    const int c = kk / taps, tap = kk - c * taps;
+    const bool live = kk < (int)g.Kg;
+    cols[wave][lane] = i32x2_t{live ? c * plane * 4 : 0, live ? tap * 4 : (kRowTaps - 1) * 4};
+  }
+  // row r = tid % 32 of the block for every thread (the rows' tap offsets are written by eight threads per row)
+  const int r = tid & 31;
+  const int64_t m = rb * kFragRows + r;
+  const int s = shift[m];
+  const bool row_ok = m < g.M && s != kBadRow;
+  const int64_t n = m < g.M ? m / g.out_sp_size : 0;
+  int p = m < g.M ? (int)(m - n * g.out_sp_size) : 0;
+  const int o2 = p % g.out_sp[2];
+  p /= g.out_sp[2];
+  const int o1 = p % g.out_sp[1];
+  const int o0 = p / g.out_sp[1];
+  const int b0 = o0 * g.stride[0] - g.pad[0], b1 = o1 * g.stride[1] - g.pad[1], b2 = o2 * g.stride[2] - g.pad[2];
+  const int origin = (b0 * in1 + b1) * in2 + b2; // may be negative: only taps inside the input are given an offset
+  const uint32_t first = (uint32_t)(((n * g.C + grp * g.Cg) * g.in_sp_size + origin) * 4);
+  __syncthreads();
+  for (int t = tid >> 5; t < taps; t += 8) {
+    const i32x4_t e = s_taps[t];
+    const int i0 = b0 + (e.y & 0xffff), i1 = b1 + (int)((uint32_t)e.y >> 16), i2 = b2 + e.z;
+    const bool ok = row_ok && (unsigned)i0 < (unsigned)in0 && (unsigned)i1 < (unsigned)in1 &&
+                    (unsigned)i2 < (unsigned)in2;
+    row_taps[r * kRowTaps + t] = ok ? first + (uint32_t)e.x * 4u : kNowhere;
+  }
+  if (tid < 32)
+    row_taps[r * kRowTaps + kRowTaps - 1] = kNowhere;
+  __syncthreads();
+  const uint64_t xbase = reinterpret_cast<uint64_t>(x);
+  const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
+      reinterpret_cast<void *>(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(xbase >> 32)) << 32) |
+                               (uint32_t)__builtin_amdgcn_readfirstlane((int)xbase)),
+      0, __builtin_amdgcn_readfirstlane((int)(g.outer * g.C * g.in_sp_size * 4)), 0x00020000);
+  // from here on the lane's row is lane % 32 (the same as tid % 32) and its k-slots (lane / 32) * 16 + 0..15
+  const uint32_t *my_taps = row_taps + r * kRowTaps;
+  long long row_sum[2] = {0, 0}; // at most two chunks meet a group of tiles
+  for (int t = 0; t < kTilesPerWave; ++t) {
+    const int64_t kt = kt_begin + t;
+    if (kt >= k_tiles)
+      break;
+    float v[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const i32x2_t e = cols[wave][t * kTileK + (lane >> 5) * 16 + j];
+      const uint32_t at = my_taps[e.y >> 2] + (uint32_t)e.x;
+      v[j] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(xrsrc, (int)at, 0, 0));
+    }
+    uint32_t w[3][4];
+    int qv[16], part = 0;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      qv[j] = to_fixed(v[j], row_ok ? s : 0); // elements that are not read are 0.0f -> 0 whatever the shift
+      part += qv[j];
+    }
+    pack_digits(qv, w);
+    row_sum[(kt * kTileK) / kChunkK - (kt_begin * kTileK) / kChunkK] += part;
+    uint4_t *dst = out + ((rb * k_tiles + kt) * kDigits) * 64 + lane;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+      uint4_t o;
+      o.x = w[d][0], o.y = w[d][1], o.z = w[d][2], o.w = w[d][3];
+      dst[d * 64] = o;
+    }
+  }
+  const int64_t chunk0 = (kt_begin * kTileK) / kChunkK;
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+    if (row_sum[h] != 0)
+      atomicAdd(reinterpret_cast<unsigned long long *>(sums + (chunk0 + h) * rows + m), (unsigned long long)row_sum[h]);
+}
+
 } // namespace
 
 // `scratch` holds kChannelSlices * outer * in_sp_size uint32 (the channel maxima).
@@ -570,6 +674,13 @@ int launch_im2col_digits(const float *x, void *xdigits, void *scratch, const Con
     hipLaunchKernelGGL(conv_row_shift, dim3((unsigned)ceil_div(d.rows, 256)), dim3(256), 0, stream, cmax, sums, shift,
                        g, d.rows, d.chunks);
     NBLA_HIP_LAUNCH_CHECK("conv_row_shift");
+  }
+  if (g.k_size <= 64 && g.outer * g.C * g.in_sp_size * 4 < ((int64_t)1 << 31)) {
+    const int64_t groups_per_row = ceil_div(d.k_tiles, 4 * kTilesPerWave);
+    hipLaunchKernelGGL(im2col_digits_taps, dim3((unsigned)(d.row_blocks * groups_per_row)), dim3(256), 0, stream, x,
+                       shift, sums, reinterpret_cast<uint4_t *>(base), g, grp, d.k_tiles, groups_per_row, d.rows);
+    NBLA_HIP_LAUNCH_CHECK("im2col_digits_taps");
+    return NBLA_HIP_OK;
   }
   const int64_t tile_groups = ceil_div(d.k_tiles, kTilesPerWave), jobs = d.row_blocks * tile_groups;
   hipLaunchKernelGGL(im2col_digits, dim3((unsigned)ceil_div(jobs, 4)), dim3(256), 0, stream, x, shift, sums,
