@@ -381,13 +381,15 @@ def main():
     # clocks (the first dozens of launches after idle run on ramping clocks).  With --section headline there is
     # nothing before them and the figure is a cold one.
     sweep = {}
-    for m in ((1, 8, 16, 64, 512) if args.section == "all" else ()):
+    for m in ((1, 8, 16, 32, 64, 512) if args.section == "all" else ()):
         s = bench_whole_forward(m, K, N, max(10, args.steps), 5, dev)
-        if m > 16:   # the product runs on the matrix cores from packed bits: its share, timed between events
+        if m > 64:   # the product runs on the matrix cores from packed bits: its share, timed between events
             t = bench_binary_weight_affine(m, K, N, max(5, args.steps // 2), 2, dev)
             packed_bytes = K * N / 8 + 3.0 * m * K + 4.0 * m * N + 4.0 * N
             s.update({"gemm_ms": t["gemm_ms"], "prepare_ms": t["prepare_ms"], "gemm_TFLOPs": t["flop"] / t["gemm_ms"] / 1e9,
                       "gemm_weight_GBs": packed_bytes / t["gemm_ms"] / 1e6})
+        elif m > 16:
+            s["path"] = "one pass over W, signs fed to bf16 matrix instructions from the registers (x as three bf16 terms)"
         else:
             s["path"] = "one pass over W on the vector ALUs (no packed bits, no separate product launch)"
         sweep["M=%d" % m] = s

@@ -67,10 +67,11 @@ int launch_gemm_digits(const void *adigits, const void *bdigits, const float *bi
                        bool accumulate = false, void *split_ws = nullptr, size_t split_ws_bytes = 0);
 size_t gemm_digits_split_bytes(int64_t M, int64_t K, int64_t N);
 
-// BinaryWeightAffine / BinaryConnectAffine forward for very few input rows, in one pass over W [K, N] on the vector
-// ALUs (no packed bits, no digit operand): writes Wb = Sign(W), alpha (when not null: alpha[n] = mean_k |W[k, n]|) and
+// BinaryWeightAffine / BinaryConnectAffine forward for very few input rows, in one pass over W [K, N] (no packed
+// bits, no digit operand): writes Wb = Sign(W), alpha (when not null: alpha[n] = mean_k |W[k, n]|) and
 // y = (x . Wb) (* alpha) (+ bias).  `applies` tells whether the shapes and alignments allow it.
-constexpr int64_t kSmallMMaxRows = 16;
+constexpr int64_t kSmallMMaxRows = 16;  // rows the one-pass form multiplies on the vector ALUs
+constexpr int64_t kFewRowsMaxRows = 64; // rows the one-pass form multiplies on the matrix cores
 bool small_m_affine_applies(const float *x, const float *W, const float *Wb, const float *alpha, const float *bias,
                             const float *y, int64_t M, int64_t K, int64_t N);
 size_t small_m_affine_workspace_bytes(int64_t M, int64_t K, int64_t N);

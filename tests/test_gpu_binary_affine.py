@@ -195,6 +195,80 @@ def test_few_rows_propagate_non_finite_values_per_element(dev):
     assert np.isinf(y[1]).all() and np.isnan(y[3]).all()
 
 
+@pytest.mark.parametrize("M", [9, 16, 17, 32, 33, 50, 64])
+@pytest.mark.parametrize("K,N", [(304, 1028), (256, 256), (1008, 516), (64, 4), (4112, 260), (16, 132)])
+def test_some_dozen_rows_one_pass_product_on_the_matrix_cores(dev, M, K, N):
+    """9 <= M <= 64 with K % 16 == 0 and N % 4 == 0 also runs in one walk over W: the signs go straight from the
+    registers into bf16 matrix instructions, against x split exactly into three bf16 terms.  Ragged strips of N,
+    tile counts that leave wavefronts and slabs short, both row-fragment counts, rows that stop inside a fragment;
+    Wb bit-exact, alpha and y against the oracle and float64.  Weights include exact zeros of both signs and a NaN
+    (Sign -> zero_to)."""
+    x, W = _data(M, K, N, seed=M * 1000 + K)
+    W.ravel()[::7] = 0.0
+    W.ravel()[3::11] = -0.0
+    W[K // 2, N // 2] = np.nan
+    b = np.random.RandomState(2).randn(N).astype(np.float32)
+    for q0 in (1.0, -1.0, 0.0, 0.5):
+        ref_y, ref_Wb, ref_alpha = oracle.binary_weight_affine(x, W, b, q0)
+        y, Wb, alpha = kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev), _dev(b, dev), q0)
+        assert bits_equal(to_np(Wb), ref_Wb), first_mismatch(to_np(Wb), ref_Wb)
+        col_ok = ~np.isnan(ref_alpha)                       # the NaN weight's column has a NaN mean in both
+        assert np.array_equal(np.isnan(to_np(alpha)), ~col_ok)
+        np.testing.assert_allclose(to_np(alpha)[col_ok], ref_alpha[col_ok], rtol=2e-6)
+        assert max_rel_err(to_np(y)[:, col_ok], ref_y[:, col_ok]) <= TIGHT * 4
+        assert np.isnan(to_np(y)[:, ~col_ok]).all()
+        ref_y, ref_Wb = oracle.binary_connect_affine(x, W, None, q0)
+        y, Wb = kernels.binary_connect_affine(_dev(x, dev), _dev(W, dev), None, q0)
+        assert bits_equal(to_np(Wb), ref_Wb)
+        y64 = x.astype(np.float64) @ ref_Wb.astype(np.float64)
+        assert max_rel_err(to_np(y), y64) <= TIGHT and max_rel_err(to_np(y), ref_y) <= TIGHT * 4
+
+
+def test_some_dozen_rows_keep_every_bit_of_x(dev):
+    """The three bf16 terms carry all 24 significand bits: with weights of one sign the product is the plain sum of a
+    row of x, and inputs chosen so that every partial sum is exact in fp32 (integers below 2^24 scaled by a power of
+    two, including values that need all three terms and values whose lower terms are zero) must come out exactly."""
+    M, K, N = 40, 64, 8
+    rng = np.random.RandomState(5)
+    ints = rng.randint(-(1 << 17), 1 << 17, size=(M, K)).astype(np.int64)
+    ints[:, 0] = (1 << 17) - 1                                   # seventeen ones: all three terms in use
+    ints[:, 1] = 1 << 16                                         # one bit: the lower terms are zero
+    ints[:, 2] = -((1 << 17) - 1)
+    ints[3, :] = 0
+    x = (ints.astype(np.float64) * 2.0 ** -20).astype(np.float32)
+    W = np.full((K, N), 0.25, np.float32)
+    W[:, 1::2] = -0.25
+    y, _ = kernels.binary_connect_affine(_dev(x, dev), _dev(W, dev))
+    want = (ints.sum(1).astype(np.float64) * 2.0 ** -20)[:, None] * np.where(np.arange(N) % 2 == 0, 1.0, -1.0)
+    assert np.array_equal(to_np(y).astype(np.float64), want)
+
+
+def test_some_dozen_rows_propagate_non_finite_values_per_element(dev):
+    """Inf and NaN stay in the first of the three bf16 terms of x (also a NaN whose payload lies in the lower half of
+    the word), so they spread per output element exactly as in the reference's fp32 product (affine.cpp:87-95)."""
+    rng = np.random.RandomState(13)
+    M, K, N = 40, 64, 64
+    x = rng.randn(M, K).astype(np.float32)
+    x[1, 3] = np.inf
+    x[2, 7], x[2, 9] = -np.inf, np.inf
+    x[3, 60] = np.nan
+    x.view(np.uint32)[4, 5] = 0x7f800001                          # signalling NaN, payload in the low bits only
+    x[35, 0] = -np.inf
+    x[36, 1] = 3.0e38
+    x[36, 2] = 3.0e38                                             # finite inputs whose sum overflows
+    W = rng.randn(K, N).astype(np.float32)
+    W[1, :], W[2, :] = 1.0, 1.0
+    y, _ = kernels.binary_connect_affine(_dev(x, dev), _dev(W, dev))
+    y = to_np(y)
+    with np.errstate(over="ignore", invalid="ignore"):
+        ref, _ = oracle.binary_connect_affine(x, W, None, 1.0)
+    assert np.array_equal(np.isnan(y), np.isnan(ref)) and np.array_equal(np.isposinf(y), np.isposinf(ref))
+    assert np.array_equal(np.isneginf(y), np.isneginf(ref))
+    fin = np.isfinite(ref)
+    assert fin[[0, 5, 39]].all() and np.abs(y[fin] - ref[fin]).max() <= 1e-4 * np.abs(ref[fin]).max()
+    assert np.isinf(y[1]).all() and np.isnan(y[3]).all() and np.isnan(y[4]).all() and np.isposinf(y[36]).all()
+
+
 @pytest.mark.parametrize("M,K,N", [(3, 16384 + 40, 70), (40, 40000, 64)])
 def test_long_contraction_is_chunked(dev, M, K, N):
     """K above 16384 is accumulated in int32 per chunk of 16384 columns and the chunks are added in fp32."""
