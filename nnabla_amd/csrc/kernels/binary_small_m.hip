@@ -559,8 +559,9 @@ int launch_few_rows_mma(const float *x, const float *W, float *Wb, float *alpha,
 // loads of x.  Up to kSmallMMaxRows rows the vector-ALU walk takes what it does not cover.
 constexpr int64_t kMmaFromRows = 9;
 static bool few_rows_mma_applies(const float *x, int64_t M, int64_t K, int64_t N) {
-  return M >= kMmaFromRows && M <= kFewRowsMaxRows && K % kMmaTileRows == 0 && aligned16(x) && N < (1ll << 26) &&
-         mma_plan(K, N).slabs <= 65535;
+  // (lane offsets into x and W are 32-bit byte counts)
+  return M >= kMmaFromRows && M <= kFewRowsMaxRows && K % kMmaTileRows == 0 && K < (1ll << 23) && aligned16(x) &&
+         N < (1ll << 26) && mma_plan(K, N).slabs <= 65535;
 }
 
 bool small_m_affine_applies(const float *x, const float *W, const float *Wb, const float *alpha, const float *bias,
