@@ -947,7 +947,8 @@ __global__ __launch_bounds__(kPrepBlock) void split_digits_columns(const float *
   const int64_t mt = frag / col_blocks, cb = frag - mt * col_blocks;
   const int64_t c = cb * kFragRows + (lane & 31);
   const int64_t r0 = mt * kTileK + (lane >> 5) * 16;
-  const int s = (*flag == 0) ? narrow_shift[c] : shift[c];
+  const bool narrow = *flag == 0; // uniform over the grid
+  const int s = narrow ? narrow_shift[c] : shift[c];
   const bool live = c < C && s != kBadRow;
   float v[16];
 #pragma unroll
@@ -957,7 +958,18 @@ __global__ __launch_bounds__(kPrepBlock) void split_digits_columns(const float *
 #pragma unroll
   for (int j = 0; j < 16; ++j)
     q[j] = to_fixed(v[j], s == kBadRow ? 0 : s);
-  store_digits(q, out + (cb * k_tiles + mt) * kDigits * 64 + lane, true);
+  uint4_t *dst = out + (cb * k_tiles + mt) * kDigits * 64 + lane;
+  if (narrow) {
+    // every value is a small integer, all of it in the lowest digit: the only fragment a product reads from an
+    // operand whose flag is clear
+    uint32_t w[3][4];
+    pack_digits(q, w);
+    uint4_t o;
+    o.x = w[kDigits - 1][0], o.y = w[kDigits - 1][1], o.z = w[kDigits - 1][2], o.w = w[kDigits - 1][3];
+    __builtin_nontemporal_store(o, dst + (kDigits - 1) * 64);
+    return;
+  }
+  store_digits(q, dst, true);
 }
 
 } // namespace
