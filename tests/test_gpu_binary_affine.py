@@ -531,11 +531,12 @@ def test_workspace_too_small_is_reported(dev):
     assert ei.value.code == kernels.ERR_MEMORY
 
 
-def test_forward_replays_in_a_hip_graph(dev):
+@pytest.mark.parametrize("M", [96, 48, 4])   # packed-bit product; one pass on the matrix cores; on the vector ALUs
+def test_forward_replays_in_a_hip_graph(dev, M):
     """BinaryWeightAffine and a FixedPointQuantize in front of it, captured once and replayed with new inputs: the
     entry points allocate nothing, never synchronise on this path and clear their scratch with kernels, so every
     replay must reproduce the eager result bit for bit (eager work and synchronisations run between the replays)."""
-    M, K, N = 96, 512, 768
+    K, N = 512, 768
     rng = np.random.RandomState(77)
     W = _dev((rng.randn(K, N) * 0.02).astype(np.float32), dev)
     x = torch.empty(M, K, device=dev)
