@@ -208,6 +208,42 @@ def test_inq_affine_all_fixed_and_partially_fixed(dev, M, K, N):
         assert bits_equal(to_np(y2), to_np(y)) and bits_equal(to_np(Wd), Wc)
 
 
+@pytest.mark.parametrize("num_bits", [3, 4, 5])
+@pytest.mark.parametrize("K,N", [(256, 32), (512, 96), (768, 288)])
+def test_inq_affine_one_digit_weights_with_columns_of_different_reach(dev, K, N, num_bits):
+    """The weight operand of the product takes its one-digit form when every weight is zero or a power of two and no
+    column spans more than six binades: with every weight fixed at num_bits <= 4 (seven levels at most) it does, with
+    num_bits 5 the levels of a column can span more, and with weights still being learnt there are values that are no
+    powers of two: both take the three-digit form.  Columns of very different magnitude (some entirely below the top
+    level's reach, some pruned to zero) are part of the data.  The forward's product (column statistics gathered by
+    the quantizing pass) must give the bits of the product-only call (statistics from a pass of its own) and agree
+    with the oracle."""
+    rng = np.random.RandomState(K + N + num_bits)
+    M = 40
+    x = rng.randn(M, K).astype(np.float32)
+    W = (rng.randn(K, N) * 0.02).astype(np.float32)
+    W[:, ::5] *= np.float32(2.0 ** -3)                  # columns whose largest level lies below the global one
+    W[:, 3::7] *= np.float32(2.0 ** -9)                 # columns pruned to zero, or out of one digit's reach
+    W[::3, 1] = 0.0
+    b = rng.randn(N).astype(np.float32)
+    for its, nsteps in (((0,), 1), ((0, 5), 2)):        # all fixed at once / half fixed then a plain minibatch
+        inq = oracle.Inq(W.size, num_bits, its, "largest_abs")
+        Wc, Ic = W.copy(), np.zeros(W.shape, np.int32)
+        Wd, Id = _dev(W, dev), torch.zeros(W.shape, dtype=torch.int32, device=dev)
+        oldW, oldI = torch.zeros_like(Wd), torch.zeros_like(Id)
+        for it in range(nsteps):
+            ref_y = inq.affine(x, Wc, Ic, b)
+            y = kernels.inq_affine(_dev(x, dev), Wd, Id, oldW, oldI, _dev(b, dev), num_bits,
+                                   _step_for(it, its, "largest_abs"))
+            assert bits_equal(to_np(Wd), Wc) and np.array_equal(to_np(Id), Ic)
+            y64 = x.astype(np.float64) @ Wc.astype(np.float64) + b
+            assert max_rel_err(to_np(y), ref_y) <= TOL
+            assert max_rel_err(to_np(y), y64) <= TIGHT
+            y2 = kernels.inq_affine(_dev(x, dev), Wd, Id, oldW, oldI, _dev(b, dev), num_bits,
+                                    kernels.INQ_PRODUCT_ONLY)
+            assert bits_equal(to_np(y2), to_np(y)) and bits_equal(to_np(Wd), Wc)
+
+
 def test_inq_convolution_matches_oracle(dev):
     rng = np.random.RandomState(9)
     for xs, ws, pad, stride, group in [((2, 4, 9, 9), (6, 4, 3, 3), (1, 1), (1, 1), 1),
