@@ -24,7 +24,7 @@ constexpr int kMaxPartials = 1024;
 struct InqParams {
   int n1, n2;
   float thr;
-  int pad;
+  int all_fixed; // 1: the snapshot's indicators were all 1 when this call restored the weights
 };
 
 // Both selections rank weights in index order inside chunks of whole tiles: one block per chunk, the number of
@@ -77,6 +77,7 @@ __global__ __launch_bounds__(kBlk) void inq_restore_absmax(float *__restrict__ W
   typedef float f4_t __attribute__((ext_vector_type(4)));
   typedef int i4_t __attribute__((ext_vector_type(4)));
   uint32_t mx = 0u; // bits of a non-negative float order like the float
+  bool unfixed = false; // a weight that the snapshot does not hold as fixed
   auto take = [&](float w) {
     const uint32_t u = __float_as_uint(w) & 0x7fffffffu;
     if (u <= 0x7f800000u && u > mx) // NaN never compares greater
@@ -96,6 +97,7 @@ __global__ __launch_bounds__(kBlk) void inq_restore_absmax(float *__restrict__ W
       const bool any0 = f0.x == 1 || f0.y == 1 || f0.z == 1 || f0.w == 1;
       const bool all1 = f1.x == 1 && f1.y == 1 && f1.z == 1 && f1.w == 1;
       const bool any1 = f1.x == 1 || f1.y == 1 || f1.z == 1 || f1.w == 1;
+      unfixed |= !all0 || !all1;
       f4_t w0 = {0.0f, 0.0f, 0.0f, 0.0f}, w1 = w0, o0 = w0, o1 = w0;
       if (!all0)
         w0 = reinterpret_cast<const f4_t *>(W)[i];
@@ -127,6 +129,8 @@ __global__ __launch_bounds__(kBlk) void inq_restore_absmax(float *__restrict__ W
     if (old_I[i] == 1) {
       w = old_W[i];
       W[i] = w;
+    } else {
+      unfixed = true;
     }
     take(w);
   }
@@ -135,14 +139,20 @@ __global__ __launch_bounds__(kBlk) void inq_restore_absmax(float *__restrict__ W
     const uint32_t o = __shfl_xor(mx, off);
     mx = o > mx ? o : mx;
   }
+  // the block's largest magnitude (bit 31 is free: magnitudes), and in bit 31 whether it met an unfixed weight
+  mx |= __any(unfixed) ? 0x80000000u : 0u;
   __shared__ uint32_t s_mx[kBlk / 64];
   if ((threadIdx.x & 63) == 0)
     s_mx[threadIdx.x >> 6] = mx;
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int w = 1; w < kBlk / 64; ++w)
-      mx = s_mx[w] > mx ? s_mx[w] : mx;
-    partial[blockIdx.x] = mx;
+    uint32_t flag = mx & 0x80000000u;
+    mx &= 0x7fffffffu;
+    for (int w = 1; w < kBlk / 64; ++w) {
+      flag |= s_mx[w] & 0x80000000u;
+      mx = (s_mx[w] & 0x7fffffffu) > mx ? (s_mx[w] & 0x7fffffffu) : mx;
+    }
+    partial[blockIdx.x] = mx | flag;
   }
 }
 
@@ -162,22 +172,30 @@ __global__ __launch_bounds__(kFinalizeThreads) void inq_finalize(const uint32_t 
     if (threadIdx.x == 0)
       *cols.flag = 0;
   }
-  uint32_t mx = 0u;
-  for (int i = threadIdx.x; i < nparts; i += kFinalizeThreads)
-    mx = partial[i] > mx ? partial[i] : mx;
+  uint32_t mx = 0u, unfixed = 0u; // (bit 31 of a partial result: the block met a weight that is not fixed)
+  for (int i = threadIdx.x; i < nparts; i += kFinalizeThreads) {
+    const uint32_t v = partial[i];
+    unfixed |= v >> 31;
+    mx = (v & 0x7fffffffu) > mx ? (v & 0x7fffffffu) : mx;
+  }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) {
     const uint32_t o = __shfl_xor(mx, off);
     mx = o > mx ? o : mx;
   }
+  mx |= __any(unfixed != 0u) ? 0x80000000u : 0u;
   __shared__ uint32_t s_mx[kFinalizeThreads / 64];
   if ((threadIdx.x & 63) == 0)
     s_mx[threadIdx.x >> 6] = mx;
   __syncthreads();
   if (threadIdx.x != 0)
     return;
-  for (int w = 1; w < kFinalizeThreads / 64; ++w)
-    mx = s_mx[w] > mx ? s_mx[w] : mx;
+  unfixed = mx >> 31;
+  mx &= 0x7fffffffu;
+  for (int w = 1; w < kFinalizeThreads / 64; ++w) {
+    unfixed |= s_mx[w] >> 31;
+    mx = (s_mx[w] & 0x7fffffffu) > mx ? (s_mx[w] & 0x7fffffffu) : mx;
+  }
   if (mx == 0u)
     mx = 0x3f800000u; // max_absval == 0 -> 1
   int n1;
@@ -200,7 +218,7 @@ __global__ __launch_bounds__(kFinalizeThreads) void inq_finalize(const uint32_t 
   p.n1 = n1;
   p.n2 = n2;
   p.thr = thr;
-  p.pad = 0;
+  p.all_fixed = unfixed ? 0 : 1;
   *params = p;
 }
 
@@ -240,11 +258,18 @@ __global__ __launch_bounds__(kBlk) void inq_quantize(float *__restrict__ W, int 
     s_cut[i] = e_cuts[i];
   __syncthreads();
   const InqParams p = *params;
+  const bool settled = p.all_fixed != 0 && !fix_all;
   for (int64_t i = (int64_t)blockIdx.x * kBlk + threadIdx.x; i < size; i += (int64_t)gridDim.x * kBlk) {
-    float w = W[i];
+    const float w0 = W[i];
+    float w = w0;
     const int ind = fix_all ? 1 : I[i];
     if (ind == 1)
       w = inq_quantize_value(w, p, s_cut);
+    // A fixed weight of a snapshot that held every weight as fixed was copied from that snapshot by this call's
+    // restoring pass; if quantizing leaves its bits alone, W, the snapshot and its indicator hold the values
+    // already and nothing is written (the steady state once every weight is fixed).
+    if (settled && ind == 1 && __float_as_uint(w) == __float_as_uint(w0))
+      continue;
     W[i] = w;
     if (fix_all)
       I[i] = ind; // otherwise unchanged
@@ -272,6 +297,7 @@ __global__ __launch_bounds__(kBlk) void inq_quantize_columns(float *__restrict__
     s_cut[i] = e_cuts[i];
   __syncthreads();
   const InqParams p = *params;
+  const bool settled = p.all_fixed != 0 && !fix_all;
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   const int64_t c0 = ((int64_t)blockIdx.x * 64 + tx) * 4;
   const int64_t r0 = (int64_t)blockIdx.y * slab, r_end = r0 + slab < R ? r0 + slab : R;
@@ -281,7 +307,8 @@ __global__ __launch_bounds__(kBlk) void inq_quantize_columns(float *__restrict__
 #pragma unroll 2
     for (int64_t r = r0 + ty; r < r_end; r += 4) {
       const int64_t i = r * C + c0;
-      f4_t w = *reinterpret_cast<const f4_t *>(W + i);
+      const f4_t w0 = *reinterpret_cast<const f4_t *>(W + i);
+      f4_t w = w0;
       i4_t ind = {1, 1, 1, 1};
       if (!fix_all)
         ind = *reinterpret_cast<const i4_t *>(I + i);
@@ -289,11 +316,17 @@ __global__ __launch_bounds__(kBlk) void inq_quantize_columns(float *__restrict__
       w.y = ind.y == 1 ? inq_quantize_value(w.y, p, s_cut) : w.y;
       w.z = ind.z == 1 ? inq_quantize_value(w.z, p, s_cut) : w.z;
       w.w = ind.w == 1 ? inq_quantize_value(w.w, p, s_cut) : w.w;
-      *reinterpret_cast<f4_t *>(W + i) = w;
-      if (fix_all)
-        *reinterpret_cast<i4_t *>(I + i) = ind;
-      *reinterpret_cast<f4_t *>(old_W + i) = w;
-      *reinterpret_cast<i4_t *>(old_I + i) = ind;
+      // (see inq_quantize: nothing to write where the snapshot already holds these four fixed weights)
+      const bool same = settled && ind.x == 1 && ind.y == 1 && ind.z == 1 && ind.w == 1 &&
+                        __float_as_uint(w.x) == __float_as_uint(w0.x) && __float_as_uint(w.y) == __float_as_uint(w0.y) &&
+                        __float_as_uint(w.z) == __float_as_uint(w0.z) && __float_as_uint(w.w) == __float_as_uint(w0.w);
+      if (!same) {
+        *reinterpret_cast<f4_t *>(W + i) = w;
+        if (fix_all)
+          *reinterpret_cast<i4_t *>(I + i) = ind;
+        *reinterpret_cast<f4_t *>(old_W + i) = w;
+        *reinterpret_cast<i4_t *>(old_I + i) = ind;
+      }
       const float v[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {

@@ -244,6 +244,54 @@ def test_inq_affine_one_digit_weights_with_columns_of_different_reach(dev, K, N,
             assert bits_equal(to_np(y2), to_np(y)) and bits_equal(to_np(Wd), Wc)
 
 
+@pytest.mark.parametrize("M,K,N", [(8, 256, 192), (5, 100, 130)])   # with / without the column-statistics pass
+def test_inq_affine_steady_state_writes_only_what_changes(dev, M, K, N):
+    """Once the snapshot holds every weight as fixed, the quantizing pass leaves alone what the restoring pass of the
+    same call has just copied from the snapshot and quantization does not change.  That must stay invisible:
+    forwards after an optimizer step that moved every weight, after the snapshot's values were replaced by numbers
+    that are no powers of two (they have to be quantized and written back), and after indicators were cleared again
+    behind the function's back (the snapshot's indicators have to follow) all leave W, I and the snapshot as the
+    oracle's."""
+    rng = np.random.RandomState(21)
+    x = rng.randn(M, K).astype(np.float32)
+    W = (rng.randn(K, N) * 0.02).astype(np.float32)
+    inq = oracle.Inq(W.size, 4, (0,), "largest_abs")
+    Wc, Ic = W.copy(), np.zeros(W.shape, np.int32)
+    Wd, Id = _dev(W, dev), torch.zeros(W.shape, dtype=torch.int32, device=dev)
+    oldW, oldI = torch.zeros_like(Wd), torch.zeros_like(Id)
+
+    def forward(step):
+        ref_y = inq.affine(x, Wc, Ic, None)
+        y = kernels.inq_affine(_dev(x, dev), Wd, Id, oldW, oldI, None, 4, step)
+        assert bits_equal(to_np(Wd), Wc), first_mismatch(to_np(Wd), Wc)
+        assert np.array_equal(to_np(Id), Ic)
+        assert bits_equal(to_np(oldW), Wc) and np.array_equal(to_np(oldI), Ic)
+        assert max_rel_err(to_np(y), ref_y) <= TOL
+
+    forward(kernels.INQ_FIX_ALL)
+    assert Ic.min() == 1
+    for _ in range(2):                                    # the optimizer moves every weight; all of them come back
+        upd = (rng.randn(K, N) * 0.01).astype(np.float32)
+        Wc += upd
+        Wd += _dev(upd, dev)
+        forward(kernels.INQ_NO_SELECTION)
+    # the snapshot's values replaced in places: restored as they are, then quantized and written everywhere
+    snap = Wc.copy()
+    snap[::3, ::5] = (rng.randn(*snap[::3, ::5].shape) * 0.01).astype(np.float32)
+    inq.commit(snap, Ic)
+    oldW.copy_(_dev(snap, dev))
+    forward(kernels.INQ_NO_SELECTION)
+    # indicators cleared behind the function's back: those weights are learnable again, the snapshot must say so
+    Ic[1::4, 2::3] = 0
+    Id.copy_(_dev(Ic, dev))
+    upd = (rng.randn(K, N) * 0.01).astype(np.float32)
+    Wc += upd
+    Wd += _dev(upd, dev)
+    forward(kernels.INQ_NO_SELECTION)
+    assert Ic.min() == 0
+    forward(kernels.INQ_NO_SELECTION)                     # and a forward with a snapshot that is no longer all fixed
+
+
 def test_inq_convolution_matches_oracle(dev):
     rng = np.random.RandomState(9)
     for xs, ws, pad, stride, group in [((2, 4, 9, 9), (6, 4, 3, 3), (1, 1), (1, 1), 1),
