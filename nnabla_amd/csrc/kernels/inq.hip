@@ -225,6 +225,13 @@ __global__ __launch_bounds__(kFinalizeThreads) void inq_finalize(const uint32_t 
 // Step C for one fixed weight (:168-190).
 __device__ __forceinline__ float inq_quantize_value(float w, const InqParams &p, const uint32_t *s_cut) {
   const uint32_t u = __float_as_uint(w) & 0x7fffffffu;
+  // A weight that is already one of the levels -- a normal power of two with exponent in [n2, n1] -- comes back as
+  // it is: it lies above the pruning threshold 2^(n2 - 1), below the cut of its own binade, inside the clamp.  That
+  // is every weight but the zeros once quantized weights are quantized again (all of them, every forward, when all
+  // are fixed), and it spares them the table look-up.
+  const int eb = (int)(u >> 23) - 127;
+  if ((u & 0x007fffffu) == 0u && eb >= p.n2 && eb <= p.n1 && eb > -127 && eb <= 127)
+    return w;
   const float a = __uint_as_float(u);
   if (a < p.thr)
     return 0.0f;
