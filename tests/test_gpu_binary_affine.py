@@ -497,7 +497,7 @@ def test_config3_full_width_small_m_vs_oracle(dev, M):
     assert max_rel_err(to_np(yc), ref_yc) <= TOL
 
 
-@pytest.mark.parametrize("M", [512, 4096])
+@pytest.mark.parametrize("M", [32, 64, 512, 4096])   # 32, 64: the one-pass form on the matrix cores
 def test_config3_full_size_properties(dev, M):
     """At sizes the oracle cannot finish quickly: float64 dot products on sampled rows/columns,
     linearity in x, and consistency between BinaryWeight and BinaryConnect (y_bw = y_bc * alpha)."""
