@@ -6,8 +6,9 @@ sign/alpha/pack of W, the int8 digit operand of x and the 1-bit-weight int8 MFMA
 torch's current HIP stream with all inputs already resident in HBM.  The JSON line also carries the quantizer
 kernels' HBM figures (`quantizers`) and the small-M sweep (`sweep`).
 
-  value      whole-step fp32-equivalent TFLOP/s  (2*M*K*N / step time)
-  roofline   the dominant kernel (the MFMA product), timed with HIP events inside the timed steps.  Its arithmetic
+  value      whole-step fp32-equivalent TFLOP/s  (2*M*K*N / step time), K steps between two synchronisations
+  roofline   the dominant kernel (the MFMA product), timed with HIP events around its launches in a repeat of the
+             K steps (the event records are queue work of their own and stay out of the timed steps).  Its arithmetic
              is three int8 digit planes per fp32 activation, so `achieved` counts the int8 operations it issues
              (3 x 2MKN) against the int8 MFMA peak; the fp32-equivalent rate (2MKN) is given beside it
   cpu_baseline  the CPU oracle (a port of nnabla's CPU arithmetic, 1 core) on a bounded row sample
