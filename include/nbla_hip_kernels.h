@@ -245,15 +245,32 @@ size_t nbla_hip_binary_affine_workspace_bytes(int64_t M, int64_t K, int64_t N);
 /* BinaryWeightAffine forward: x [M,K], W [K,N] -> Wb [K,N], alpha [N], y [M,N]
  * (bias [N] may be NULL).  Replaces BinaryWeightAffine<float>::forward_impl,
  * src/nbla/function/generic/binary_weight_affine.cpp:75-122.
- * When quantize_zero_to is neither +1 nor -1 the call synchronises the stream
- * once to learn whether W holds exact zeros (then the product runs on the
- * materialised fp32 weights instead of the packed bits). */
+ * The call never synchronises: when quantize_zero_to is neither +1 nor -1 the
+ * weights that are neither negative nor positive are counted on the device, and
+ * an fp32 product over the materialised signs Wb, launched behind the
+ * matrix-core product with that count as its go-ahead, replaces y when the
+ * count is non-zero (and leaves at once otherwise). */
 int nbla_hip_binary_weight_affine_f32(const float *x, const float *W,
                                       float *Wb, float *alpha,
                                       const float *bias, float *y, int64_t M,
                                       int64_t K, int64_t N,
                                       float quantize_zero_to, void *workspace,
                                       size_t workspace_bytes, void *stream);
+
+/* The same forward (alpha == NULL: BinaryConnectAffine) in its one-walk form,
+ * whatever the shape: W is read once, by a kernel that writes Sign(W), sums |W|
+ * per column and multiplies the fresh signs with the digit operand of x on the
+ * int8 matrix cores (M <= 512, N % 4 == 0, W and Wb 16-byte aligned, K <= 16384,
+ * W below 2 GiB; NBLA_HIP_ERR_NOT_IMPLEMENTED otherwise).  The two calls above
+ * take this form by themselves for 65 <= M <= 512 and N >= 8129; this entry
+ * point is for callers (and tests) that want it on other shapes.  Same
+ * reference functions, same workspace. */
+int nbla_hip_binary_affine_one_walk_f32(const float *x, const float *W,
+                                        float *Wb, float *alpha,
+                                        const float *bias, float *y, int64_t M,
+                                        int64_t K, int64_t N,
+                                        float quantize_zero_to, void *workspace,
+                                        size_t workspace_bytes, void *stream);
 
 size_t nbla_hip_affine_backward_workspace_bytes(int64_t M, int64_t K, int64_t N);
 

@@ -1,6 +1,7 @@
 // Device memory management and the storage-level array operations (fill, dtype
 // cast, ReLU) that the HipArray classes of the host layer are built on.
 #include "common.hpp"
+#include "internal.hpp"
 
 namespace nbla_hip {
 namespace {
@@ -187,6 +188,11 @@ size_t dtype_bytes(int dtype) {
 }
 
 } // namespace
+
+int launch_clear_words(void *dst, size_t count, hipStream_t stream) {
+  return fill_as<unsigned int>(dst, count, 0.0f, stream);
+}
+
 } // namespace nbla_hip
 
 using namespace nbla_hip;

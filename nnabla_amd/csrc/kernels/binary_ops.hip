@@ -61,7 +61,7 @@ AffineWorkspace plan_affine(int64_t M, int64_t K, int64_t N) {
 
 int binary_affine_forward(const float *x, const float *W, float *Wb, float *alpha, const float *bias, float *y,
                           int64_t M, int64_t K, int64_t N, float zero_to, void *workspace, size_t workspace_bytes,
-                          void *stream_) {
+                          void *stream_, bool one_walk = false) {
   if (M <= 0 || K <= 0 || N <= 0)
     return fail(NBLA_HIP_ERR_VALUE, "invalid affine shape (M=%lld, K=%lld, N=%lld).", (long long)M, (long long)K,
                 (long long)N);
@@ -70,7 +70,10 @@ int binary_affine_forward(const float *x, const float *W, float *Wb, float *alph
     return fail(NBLA_HIP_ERR_MEMORY, "binary affine workspace too small (%zu < %zu) or misaligned.", workspace_bytes,
                 ws.total);
   char *base = static_cast<char *>(workspace);
-  if (small_m_affine_applies(x, W, Wb, alpha, bias, y, M, K, N)) {
+  if (one_walk && !rows_affine_covers(W, Wb, M, K, N))
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "one-walk binary affine: shape or alignment not covered (M=%lld, K=%lld, "
+                "N=%lld).", (long long)M, (long long)K, (long long)N);
+  if (!one_walk && small_m_affine_applies(x, W, Wb, alpha, bias, y, M, K, N)) {
     const int rc = ensure_init();
     if (rc)
       return rc;
@@ -81,43 +84,47 @@ int binary_affine_forward(const float *x, const float *W, float *Wb, float *alph
   void *xsplit = base + ws.split_off; // digit operand of x
   void *prep = base + ws.prep_off;
   int *count = reinterpret_cast<int *>(base + ws.count_off);
+  // Sign(0) = zero_to that is neither +1 nor -1 cannot be a sign bit: the matrix-core product is then only valid when
+  // W holds no weight that is neither negative nor positive.  The kernel that walks W counts such weights on the
+  // device; the fp32 product over the materialised signs is launched behind the matrix-core one with that count as
+  // its go-ahead and replaces y when it is non-zero (it leaves at once otherwise).  The host never reads the count.
   const bool representable = (zero_to == 1.0f || zero_to == -1.0f);
+  hipStream_t stream = as_stream(stream_);
+  int rc;
 
-  int rc = nbla_hip_binarize_weights_f32(W, Wb, alpha, bits, K, N, 0, zero_to, representable ? nullptr : count, prep,
-                                         nbla_hip_binarize_workspace_bytes(K, N), stream_);
-  if (rc)
-    return rc;
-  if (!representable) {
-    // Sign(0) = zero_to is neither +1 nor -1: the packed bits are only valid when
-    // W holds no exact zero.  One scalar comes back to the host to decide.
-    int host_count = 0;
-    hipError_t e = hipMemcpyAsync(&host_count, count, sizeof(int), hipMemcpyDeviceToHost, as_stream(stream_));
-    if (e == hipSuccess)
-      e = hipStreamSynchronize(as_stream(stream_));
-    if (e != hipSuccess)
-      return fail_hip(e, "reading the zero-weight count");
-    if (host_count != 0)
-      return launch_gemm_f32(x, Wb, alpha, bias, y, M, K, N, as_stream(stream_));
+  if (one_walk || (rows_affine_covers(W, Wb, M, K, N) && rows_affine_pays(M, N))) {
+    // one walk over W: signs, column sums and the product together
+    if (!representable && (rc = launch_clear_words(count, 1, stream)))
+      return rc;
+    if ((rc = launch_split_digits_rows_redo(x, K, nullptr, xsplit, M, K, nullptr, nullptr, stream)))
+      return rc;
+    if ((rc = launch_rows_affine(xsplit, W, Wb, alpha, bias, y, M, K, N, zero_to, count, stream)))
+      return rc;
+  } else {
+    rc = nbla_hip_binarize_weights_f32(W, Wb, alpha, bits, K, N, 0, zero_to, representable ? nullptr : count, prep,
+                                       nbla_hip_binarize_workspace_bytes(K, N), stream_);
+    if (rc)
+      return rc;
+    // rows of x with a NaN or an infinity: computed by the splitting kernel where it can, else after the product
+    const RowRedo redo{Wb, alpha, bias, y, N};
+    bool redone = false;
+    rc = launch_split_digits_rows_redo(x, K, nullptr, xsplit, M, K, &redo, &redone, stream);
+    if (rc)
+      return rc;
+    rc = launch_gemm_bits(xsplit, bits, alpha, bias, y, M, K, N, 1, N, 1, false, stream, false, base + ws.gemm_off,
+                          ws.gemm_bytes, redone);
+    if (rc)
+      return rc;
+    if (redone)
+      return representable ? NBLA_HIP_OK : launch_gemm_f32(x, Wb, alpha, bias, y, M, K, N, stream, count);
   }
-  // rows of x with a NaN or an infinity: computed by the splitting kernel where it can, else after the product
-  const RowRedo redo{Wb, alpha, bias, y, N};
-  bool redone = false;
-  rc = launch_split_digits_rows_redo(x, K, nullptr, xsplit, M, K, &redo, &redone, as_stream(stream_));
-  if (rc)
-    return rc;
-  rc = launch_gemm_bits(xsplit, bits, alpha, bias, y, M, K, N, 1, N, 1, false, as_stream(stream_), false,
-                        base + ws.gemm_off, ws.gemm_bytes, redone);
-  if (rc)
-    return rc;
-  if (!redone) {
-    const int32_t *shift =
-        reinterpret_cast<const int32_t *>(static_cast<const char *>(xsplit) + digit_operand(M, K).shift_off);
-    const unsigned blocks = (unsigned)(M < 256 ? M : 256);
-    hipLaunchKernelGGL(affine_redo_marked_rows, dim3(blocks), dim3(256), 0, as_stream(stream_), x, Wb, alpha, bias, y,
-                       shift, M, K, N);
-    NBLA_HIP_LAUNCH_CHECK("affine_redo_marked_rows");
-  }
-  return NBLA_HIP_OK;
+  const int32_t *shift =
+      reinterpret_cast<const int32_t *>(static_cast<const char *>(xsplit) + digit_operand(M, K).shift_off);
+  const unsigned blocks = (unsigned)(M < 256 ? M : 256);
+  hipLaunchKernelGGL(affine_redo_marked_rows, dim3(blocks), dim3(256), 0, stream, x, Wb, alpha, bias, y, shift, M, K,
+                     N);
+  NBLA_HIP_LAUNCH_CHECK("affine_redo_marked_rows");
+  return representable ? NBLA_HIP_OK : launch_gemm_f32(x, Wb, alpha, bias, y, M, K, N, stream, count);
 }
 
 } // namespace
@@ -136,6 +143,13 @@ int nbla_hip_binary_weight_affine_f32(const float *x, const float *W, float *Wb,
     return fail(NBLA_HIP_ERR_VALUE, "BinaryWeightAffine needs an alpha output of size N.");
   return binary_affine_forward(x, W, Wb, alpha, bias, y, M, K, N, quantize_zero_to, workspace, workspace_bytes,
                                stream);
+}
+
+int nbla_hip_binary_affine_one_walk_f32(const float *x, const float *W, float *Wb, float *alpha, const float *bias,
+                                        float *y, int64_t M, int64_t K, int64_t N, float quantize_zero_to,
+                                        void *workspace, size_t workspace_bytes, void *stream) {
+  return binary_affine_forward(x, W, Wb, alpha, bias, y, M, K, N, quantize_zero_to, workspace, workspace_bytes, stream,
+                               true);
 }
 
 int nbla_hip_binary_connect_affine_f32(const float *x, const float *W, float *Wb, const float *bias, float *y,

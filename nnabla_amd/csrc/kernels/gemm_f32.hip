@@ -21,7 +21,10 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__
                                                        const float *__restrict__ colscale,
                                                        const float *__restrict__ bias, float *__restrict__ y,
                                                        int64_t M, int64_t K, int64_t N, int64_t inner,
-                                                       int64_t outer_stride, int64_t n_stride) {
+                                                       int64_t outer_stride, int64_t n_stride,
+                                                       const int *__restrict__ run_if) {
+  if (run_if && *run_if == 0) // uniform over the grid: every block leaves at once
+    return;
   __shared__ float As[kBK][kBM + kPad]; // [k][m]
   __shared__ float Bs[kBK][kBN + kPad]; // [k][n]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -117,21 +120,21 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__
 
 int launch_gemm_f32_mapped(const float *x, const float *w, bool trans_b, const float *colscale, const float *bias,
                            float *y, int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride,
-                           int64_t n_stride, hipStream_t stream) {
+                           int64_t n_stride, hipStream_t stream, const int *run_if) {
   const dim3 grid((unsigned)ceil_div(N, kBN), (unsigned)ceil_div(M, kBM));
   if (trans_b)
     hipLaunchKernelGGL(gemm_f32_kernel<true>, grid, dim3(256), 0, stream, x, w, colscale, bias, y, M, K, N, inner,
-                       outer_stride, n_stride);
+                       outer_stride, n_stride, run_if);
   else
     hipLaunchKernelGGL(gemm_f32_kernel<false>, grid, dim3(256), 0, stream, x, w, colscale, bias, y, M, K, N, inner,
-                       outer_stride, n_stride);
+                       outer_stride, n_stride, run_if);
   NBLA_HIP_LAUNCH_CHECK("gemm_f32");
   return NBLA_HIP_OK;
 }
 
 int launch_gemm_f32(const float *x, const float *w, const float *colscale, const float *bias, float *y, int64_t M,
-                    int64_t K, int64_t N, hipStream_t stream) {
-  return launch_gemm_f32_mapped(x, w, false, colscale, bias, y, M, K, N, 1, N, 1, stream);
+                    int64_t K, int64_t N, hipStream_t stream, const int *run_if) {
+  return launch_gemm_f32_mapped(x, w, false, colscale, bias, y, M, K, N, 1, N, 1, stream, run_if);
 }
 
 } // namespace nbla_hip

@@ -6,11 +6,16 @@ namespace nbla_hip {
 
 // fp32 MFMA product y = (x . w) * colscale + bias; w is [K, N], or [N, K] when trans_b.  Output element (m, n) is
 // written at y[(m / inner) * outer_stride + n * n_stride + (m % inner)].
+// `run_if` (device memory, may be null): the launch does nothing unless the word it points to is non-zero when the
+// kernel starts -- the fallback of a product whose operand turned out not to be expressible in its fast form, decided
+// on the device so that the host never waits for the answer.
 int launch_gemm_f32_mapped(const float *x, const float *w, bool trans_b, const float *colscale, const float *bias,
                            float *y, int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride,
-                           int64_t n_stride, hipStream_t stream);
+                           int64_t n_stride, hipStream_t stream, const int *run_if = nullptr);
 int launch_gemm_f32(const float *x, const float *w, const float *colscale, const float *bias, float *y, int64_t M,
-                    int64_t K, int64_t N, hipStream_t stream);
+                    int64_t K, int64_t N, hipStream_t stream, const int *run_if = nullptr);
+// Sets `count` 32-bit words to zero with a kernel (a memset node must not be recorded into a captured graph).
+int launch_clear_words(void *dst, size_t count, hipStream_t stream);
 
 // Bit-weight product with the choice of store orientation: swap_out makes consecutive lanes write consecutive m
 // (for outputs whose m index is the contiguous one, e.g. convolution results [batch, O, Ho*Wo]).  keep_bad_rows: rows
@@ -78,6 +83,16 @@ size_t small_m_affine_workspace_bytes(int64_t M, int64_t K, int64_t N);
 int launch_small_m_affine(const float *x, const float *W, float *Wb, float *alpha, const float *bias, float *y,
                           int64_t M, int64_t K, int64_t N, float zero_to, void *workspace, size_t workspace_bytes,
                           hipStream_t stream);
+
+// The same one-pass forward for 65 .. kRowsMmaMaxRows input rows, on the int8 matrix cores (binary_rows_mma.hip): x comes
+// as its digit operand (nbla_hip_split_digits_scaled_f32); rows marked kBadRow there are not written.  With zero_to
+// other than +-1, *zero_flag (cleared by the caller) is raised when W holds a weight that is neither negative nor
+// positive; y is then to be replaced by an fp32 product over Wb.
+constexpr int64_t kRowsMmaMaxRows = 512;
+bool rows_affine_covers(const float *W, const float *Wb, int64_t M, int64_t K, int64_t N); // shapes it can run
+bool rows_affine_pays(int64_t M, int64_t N); // shapes on which it beats the two-walk path
+int launch_rows_affine(const void *xdigits, const float *W, float *Wb, float *alpha, const float *bias, float *y,
+                       int64_t M, int64_t K, int64_t N, float zero_to, int *zero_flag, hipStream_t stream);
 
 // db[n] (+)= sum over m of dy[m, n]; `partial` holds ceil(M / 256) * N floats.
 size_t column_sums_workspace_bytes(int64_t M, int64_t N);

@@ -29,7 +29,7 @@ EXPORTED = (
     "nbla_hip_binarize_workspace_bytes", "nbla_hip_binarize_weights_f32",
     "nbla_hip_split_digits_f32", "nbla_hip_gemm_bits_workspace_bytes", "nbla_hip_gemm_bits_f32",
     "nbla_hip_binary_affine_workspace_bytes", "nbla_hip_binary_weight_affine_f32",
-    "nbla_hip_binary_connect_affine_f32", "nbla_hip_affine_f32", "nbla_hip_split_digits_scaled_f32",
+    "nbla_hip_binary_connect_affine_f32", "nbla_hip_binary_affine_one_walk_f32", "nbla_hip_affine_f32", "nbla_hip_split_digits_scaled_f32",
     "nbla_hip_affine_workspace_bytes", "nbla_hip_affine_digits_f32",
     "nbla_hip_affine_backward_workspace_bytes", "nbla_hip_binary_affine_backward_f32", "nbla_hip_affine_backward_f32",
     "nbla_hip_convolution_output_shape", "nbla_hip_binary_convolution_workspace_bytes",
@@ -244,6 +244,21 @@ def gemm_bits(xsplit, bits, alpha, bias, M, K, N, out=None, inner=1, outer_strid
 
 def binary_affine_workspace(M, K, N, like):
     return _workspace(lib().nbla_hip_binary_affine_workspace_bytes(_i64(M), _i64(K), _i64(N)), like)
+
+
+def binary_affine_one_walk(x, W, bias=None, quantize_zero_to=1.0, weight=True, workspace=None, stream=None):
+    """The one-walk form of BinaryWeightAffine (weight=True) / BinaryConnectAffine: x [M,K], W [K,N] -> (y, Wb, alpha)."""
+    import torch
+    M, K = x.shape
+    N = W.numel() // K
+    Wb = torch.empty_like(W)
+    alpha = torch.empty(N, dtype=torch.float32, device=x.device) if weight else None
+    y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+    ws = binary_affine_workspace(M, K, N, x) if workspace is None else workspace
+    check(lib().nbla_hip_binary_affine_one_walk_f32(_p(x), _p(W), _p(Wb), _p(alpha), _p(bias), _p(y), _i64(M), _i64(K),
+                                                    _i64(N), ctypes.c_float(quantize_zero_to), _p(ws),
+                                                    ctypes.c_size_t(ws.numel()), _stream(stream)))
+    return y, Wb, alpha
 
 
 def binary_weight_affine(x, W, bias=None, quantize_zero_to=1.0, workspace=None, out=None, stream=None, Wb=None,

@@ -336,6 +336,93 @@ def test_few_rows_one_pass_product(dev, M, K, N):
         assert max_rel_err(to_np(y), y64) <= TIGHT and max_rel_err(to_np(y), ref_y) <= TIGHT * 4
 
 
+@pytest.mark.parametrize("M", [1, 33, 65, 100, 128, 200, 256, 257, 300, 512])
+@pytest.mark.parametrize("K,N", [(96, 64), (100, 132), (256, 260), (1000, 516), (4100, 68), (32, 4)])
+def test_one_walk_product_on_the_matrix_cores(dev, M, K, N):
+    """The form that serves 65 <= M <= 512 on wide outputs -- one walk over W that writes Sign(W), sums |W| and
+    multiplies the fresh signs with the digit operand of x on the int8 matrix cores -- called directly so that narrow
+    and ragged shapes reach it too: ragged last k step, ragged last strip of 64 columns, both tile heights (256 and
+    512 rows), wavefronts with no rows.  Weights include exact zeros of both signs and a NaN (Sign -> zero_to); Wb
+    bit-exact, alpha and y against the oracle and float64, for every quantize_zero_to class (+-1: sign bits; other
+    values: the fp32 product behind the device-side flag)."""
+    x, W = _data(M, K, N, seed=M * 1000 + K)
+    W.ravel()[::7] = 0.0
+    W.ravel()[3::11] = -0.0
+    W[K // 2, N // 2] = np.nan
+    b = np.random.RandomState(2).randn(N).astype(np.float32)
+    for q0 in (1.0, -1.0, 0.0, 0.3):
+        ref_y, ref_Wb, ref_alpha = oracle.binary_weight_affine(x, W, b, q0)
+        y, Wb, alpha = kernels.binary_affine_one_walk(_dev(x, dev), _dev(W, dev), _dev(b, dev), q0)
+        assert bits_equal(to_np(Wb), ref_Wb), first_mismatch(to_np(Wb), ref_Wb)
+        col_ok = ~np.isnan(ref_alpha)                       # the NaN weight's column has a NaN mean in both
+        assert np.array_equal(np.isnan(to_np(alpha)), ~col_ok)
+        np.testing.assert_allclose(to_np(alpha)[col_ok], ref_alpha[col_ok], rtol=2e-6)
+        assert max_rel_err(to_np(y)[:, col_ok], ref_y[:, col_ok]) <= TIGHT * 4
+        assert np.isnan(to_np(y)[:, ~col_ok]).all()
+        ref_y, ref_Wb = oracle.binary_connect_affine(x, W, None, q0)
+        y, Wb, _ = kernels.binary_affine_one_walk(_dev(x, dev), _dev(W, dev), None, q0, weight=False)
+        assert bits_equal(to_np(Wb), ref_Wb)
+        y64 = x.astype(np.float64) @ ref_Wb.astype(np.float64)
+        assert max_rel_err(to_np(y), y64) <= TIGHT and max_rel_err(to_np(y), ref_y) <= TIGHT * 4
+
+
+def test_one_walk_product_without_exact_zero_weights_keeps_the_matrix_core_result(dev):
+    """quantize_zero_to = 0.3 on weights none of which is zero: the device-side flag stays down, the fp32 product
+    leaves at once and y is the matrix-core result bit for bit (that of quantize_zero_to = 1)."""
+    x, W = _data(130, 256, 200, seed=5)
+    assert (W != 0).all()
+    y1, Wb1, _ = kernels.binary_affine_one_walk(_dev(x, dev), _dev(W, dev), None, 1.0)
+    y3, Wb3, _ = kernels.binary_affine_one_walk(_dev(x, dev), _dev(W, dev), None, 0.3)
+    assert bits_equal(to_np(Wb1), to_np(Wb3)) and bits_equal(to_np(y1), to_np(y3))
+
+
+def test_one_walk_product_propagates_non_finite_values_per_element(dev):
+    rng = np.random.RandomState(12)
+    M, K, N = 300, 256, 600
+    x = rng.randn(M, K).astype(np.float32)
+    x[1, 3] = np.inf
+    x[2, 7], x[2, 9] = -np.inf, np.inf
+    x[40, 60] = np.nan
+    x[299, 0] = -np.inf
+    W = rng.randn(K, N).astype(np.float32)
+    b = rng.randn(N).astype(np.float32)
+    y, _, _ = kernels.binary_affine_one_walk(_dev(x, dev), _dev(W, dev), _dev(b, dev))
+    ref, _, _ = oracle.binary_weight_affine(x, W, b, 1.0)
+    y = to_np(y)
+    assert np.array_equal(np.isnan(y), np.isnan(ref)) and np.array_equal(np.isposinf(y), np.isposinf(ref))
+    assert np.array_equal(np.isneginf(y), np.isneginf(ref))
+    fin = np.isfinite(ref)
+    assert fin.sum() >= (M - 4) * N and np.abs(y[fin] - ref[fin]).max() <= 1e-4 * np.abs(ref[fin]).max()
+
+
+def test_one_walk_product_refuses_what_it_does_not_cover(dev):
+    x, W = _data(600, 64, 64)
+    with pytest.raises(kernels.KernelError) as ei:
+        kernels.binary_affine_one_walk(_dev(x, dev), _dev(W, dev))
+    assert ei.value.code == kernels.ERR_NOT_IMPLEMENTED
+    x, W = _data(100, 64, 66)
+    with pytest.raises(kernels.KernelError) as ei:
+        kernels.binary_affine_one_walk(_dev(x, dev), _dev(W, dev))
+    assert ei.value.code == kernels.ERR_NOT_IMPLEMENTED
+
+
+@pytest.mark.parametrize("M,K,N", [(100, 64, 8196), (512, 96, 8192), (257, 40, 9000)])
+def test_wide_outputs_of_some_hundred_rows_take_the_one_walk_form(dev, M, K, N):
+    """From 8129 columns on (128 strips of 64) the whole-operation entry points run the one-walk form for 65..512
+    rows; checked against the oracle like the other paths."""
+    x, W = _data(M, K, N, seed=31)
+    W.ravel()[::13] = 0.0
+    b = np.random.RandomState(9).randn(N).astype(np.float32)
+    for q0 in (1.0, 0.0):
+        ref_y, ref_Wb, ref_alpha = oracle.binary_weight_affine(x, W, b, q0)
+        y, Wb, alpha = kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev), _dev(b, dev), q0)
+        assert bits_equal(to_np(Wb), ref_Wb)
+        np.testing.assert_allclose(to_np(alpha), ref_alpha, rtol=2e-6)
+        assert max_rel_err(to_np(y), ref_y) <= TIGHT * 4
+    y1, Wb1, a1 = kernels.binary_affine_one_walk(_dev(x, dev), _dev(W, dev), _dev(b, dev), 0.0)
+    assert bits_equal(to_np(y1), to_np(y)) and bits_equal(to_np(a1), to_np(alpha))
+
+
 @pytest.mark.parametrize("M,K,N", [(3100, 96, 5732), (3072, 64, 11008)])
 def test_tall_m_every_element(dev, M, K, N):
     """Tall outputs with a ragged last column tile (idle wavefronts, clamped wide groups): every output element is
@@ -497,7 +584,7 @@ def test_config3_full_width_small_m_vs_oracle(dev, M):
     assert max_rel_err(to_np(yc), ref_yc) <= TOL
 
 
-@pytest.mark.parametrize("M", [32, 64, 512, 4096])   # 32, 64: the one-pass form on the matrix cores
+@pytest.mark.parametrize("M", [32, 64, 128, 256, 512, 1024, 4096])   # 32, 64: one pass, operands from registers; 128 .. 512: one walk, signs shared through LDS
 def test_config3_full_size_properties(dev, M):
     """At sizes the oracle cannot finish quickly: float64 dot products on sampled rows/columns,
     linearity in x, and consistency between BinaryWeight and BinaryConnect (y_bw = y_bc * alpha)."""
