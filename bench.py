@@ -129,18 +129,22 @@ def bench_binary_weight_affine(M, K, N, steps, warmup, dev):
             "split_ms": split, "gemm_ms": gemm, "flop": 2.0 * M * K * N}
 
 
-def bench_whole_forward(M, K, N, steps, warmup, dev):
-    """BinaryWeightAffine forward through the whole-function entry point (what the Function class calls)."""
+def bench_whole_forward(M, K, N, steps, warmup, dev, connect=False):
+    """BinaryWeightAffine (BinaryConnectAffine with `connect`) forward through the whole-function entry point (what
+    the Function class calls)."""
     import torch
     from nnabla_amd import kernels as k
-    g = torch.Generator(device="cpu").manual_seed(313)
-    x = torch.randn(M, K, generator=g).to(dev)
-    W = (torch.randn(K, N, generator=g) * 0.02).to(dev)
+    g = torch.Generator(device=dev).manual_seed(313)
+    x = torch.randn(M, K, generator=g, device=dev)
+    W = torch.randn(K, N, generator=g, device=dev) * 0.02
     ws = k.binary_affine_workspace(M, K, N, x)
     y, Wb, alpha = torch.empty(M, N, device=dev), torch.empty_like(W), torch.empty(N, device=dev)
-    ms = time_kernel(lambda: k.binary_weight_affine(x, W, None, 1.0, workspace=ws, out=y, Wb=Wb, alpha=alpha), steps,
-                     warmup)
-    nbytes = 8.0 * K * N + 4.0 * M * K + 4.0 * M * N + 4.0 * N   # read W, write Wb; x, y, alpha
+    if connect:
+        fn = lambda: k.binary_connect_affine(x, W, None, 1.0, workspace=ws, out=y, Wb=Wb)
+    else:
+        fn = lambda: k.binary_weight_affine(x, W, None, 1.0, workspace=ws, out=y, Wb=Wb, alpha=alpha)
+    ms = time_kernel(fn, steps, warmup)
+    nbytes = 8.0 * K * N + 4.0 * M * K + 4.0 * M * N + (0.0 if connect else 4.0 * N)   # read W, write Wb; x, y, alpha
     return {"ms_per_step": ms, "forward_bytes_model": nbytes, "forward_GBs": nbytes / ms / 1e6,
             "forward_frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
 
@@ -191,6 +195,17 @@ def bench_quantizers(dev, iters):
                                                     workspace=ws), iters)
         nb = bpe * a.numel()
         out[name] = {"ms": ms, "bytes": nb, "GBs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
+    # a range per (channel, column): kept axes separated by reduced ones, which the strided kernels serve
+    qs = lambda v: torch.full((1, 256, 1, 56), v, device=dev)
+    qmn, qmx, lmn, lmx = qs(-6.0), qs(6.0), qs(0.0), qs(255.0)
+    ws2 = torch.empty(max(256, k.lib().nbla_hip_min_max_quantize_workspace_bytes(k._shape(a.shape), a.dim(),
+                                                                                 k._shape(qmn.shape))),
+                      dtype=torch.uint8, device=dev)
+    ms = time_kernel(lambda: k.min_max_quantize(a, qmn, qmx, lmn, lmx, 0.999, True, True, 0.01, out=ya, workspace=ws2),
+                     iters)
+    nb = 12.0 * a.numel()
+    out["min_max_quantize[64,256,56,56] x_min_max, ranges [1,256,1,56]"] = {
+        "ms": ms, "bytes": nb, "GBs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
     return out
 
 
@@ -373,9 +388,10 @@ def main():
                     help="untimed steps; the first few dozen launches after idle run at ramping clocks")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=2048)
-    ap.add_argument("--section", choices=("all", "headline", "quantizers"), default="all",
+    ap.add_argument("--section", choices=("all", "headline", "quantizers", "other"), default="all",
                     help="headline: only the timed BinaryWeightAffine steps (what the rocprofv3 summaries profile); "
-                         "quantizers: headline plus the quantizer kernels")
+                         "quantizers: headline plus the quantizer kernels; other: headline plus the convolution, INQ, "
+                         "MLP, backward and adjacent-function workloads (`other_configs`)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
@@ -390,20 +406,28 @@ def main():
     # clocks (the first dozens of launches after idle run on ramping clocks).  With --section headline there is
     # nothing before them and the figure is a cold one.
     sweep = {}
-    for m in ((1, 8, 16, 32, 64, 512) if args.section == "all" else ()):
+    for m in ((1, 8, 16, 32, 64, 128, 256, 512, 1024) if args.section == "all" else ()):
         s = bench_whole_forward(m, K, N, max(10, args.steps), 5, dev)
-        if m > 64:   # the product runs on the matrix cores from packed bits: its share, timed between events
+        if m > 256:   # two walks: the product runs on the matrix cores from packed bits; its share, timed between events
             t = bench_binary_weight_affine(m, K, N, max(5, args.steps // 2), 2, dev)
             packed_bytes = K * N / 8 + 3.0 * m * K + 4.0 * m * N + 4.0 * N
             s.update({"gemm_ms": t["gemm_ms"], "prepare_ms": t["prepare_ms"], "gemm_TFLOPs": t["flop"] / t["gemm_ms"] / 1e9,
-                      "gemm_weight_GBs": packed_bytes / t["gemm_ms"] / 1e6})
+                      "gemm_weight_GBs": packed_bytes / t["gemm_ms"] / 1e6,
+                      "path": "two walks: sign / alpha / packed bits, then the packed-bit product"})
+        elif m > 64:
+            s["path"] = ("one walk over W: signs shared through LDS, digit operand of x, int8 matrix instructions "
+                         "(K in two slices, added by a second launch)")
         elif m > 16:
             s["path"] = "one pass over W, signs fed to bf16 matrix instructions from the registers (x as three bf16 terms)"
         else:
             s["path"] = "one pass over W on the vector ALUs (no packed bits, no separate product launch)"
         sweep["M=%d" % m] = s
-    quant = bench_quantizers(dev, max(10, args.steps)) if args.section != "headline" else {}
-    other = bench_other_configs(dev, max(5, args.steps // 2)) if args.section == "all" else {}
+    # BinaryConnectAffine on the same shapes (the same kernels without alpha)
+    for m in ((1, 8, 64, 512, 4096) if args.section == "all" else ()):
+        sweep["BinaryConnectAffine M=%d" % m] = bench_whole_forward(m, K, N, max(10, args.steps // 2), 5, dev,
+                                                                    connect=True)
+    quant = bench_quantizers(dev, max(10, args.steps)) if args.section in ("all", "quantizers") else {}
+    other = bench_other_configs(dev, max(5, args.steps // 2)) if args.section in ("all", "other") else {}
     r = bench_binary_weight_affine(M, K, N, args.steps, args.warmup, dev)
     tflops = r["flop"] / (r["ms_per_step"] * 1e-3) / 1e12
     gemm_tflops = r["flop"] / (r["gemm_ms"] * 1e-3) / 1e12

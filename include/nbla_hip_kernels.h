@@ -262,9 +262,11 @@ int nbla_hip_binary_weight_affine_f32(const float *x, const float *W,
  * per column and multiplies the fresh signs with the digit operand of x on the
  * int8 matrix cores (M <= 512, N % 4 == 0, W and Wb 16-byte aligned, K <= 16384,
  * W below 2 GiB; NBLA_HIP_ERR_NOT_IMPLEMENTED otherwise).  The two calls above
- * take this form by themselves for 65 <= M <= 512 and N >= 8129; this entry
- * point is for callers (and tests) that want it on other shapes.  Same
- * reference functions, same workspace. */
+ * take this form by themselves for 65 <= M <= 256 on outputs wide enough to
+ * occupy the CUs (strips of 128 columns x slices of K of at least 512 >= 128
+ * blocks), where it is a fifth faster than two walks; this entry point is for
+ * callers (and tests) that want it on other shapes.  Same reference functions,
+ * same workspace. */
 int nbla_hip_binary_affine_one_walk_f32(const float *x, const float *W,
                                         float *Wb, float *alpha,
                                         const float *bias, float *y, int64_t M,

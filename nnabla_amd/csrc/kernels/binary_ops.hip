@@ -48,8 +48,13 @@ AffineWorkspace plan_affine(int64_t M, int64_t K, int64_t N) {
   off += round_up(nbla_hip_binarize_workspace_bytes(K, N), 256);
   w.count_off = off;
   off += 256;
-  w.gemm_off = off; // partial results of a product whose contraction is spread over the CUs (very small M)
+  // partial results of a product whose contraction is spread over the CUs (very small M), or of the one-walk form
+  // when it walks K in slices
+  w.gemm_off = off;
   w.gemm_bytes = nbla_hip_gemm_bits_workspace_bytes(M, K, N);
+  const size_t rows_bytes = round_up(rows_affine_workspace_bytes(M, K, N), 256);
+  if (rows_bytes > w.gemm_bytes)
+    w.gemm_bytes = rows_bytes;
   off += w.gemm_bytes;
   w.total = off;
   // the one-pass form for very few rows keeps its slab partials at the start of the same buffer
@@ -70,7 +75,7 @@ int binary_affine_forward(const float *x, const float *W, float *Wb, float *alph
     return fail(NBLA_HIP_ERR_MEMORY, "binary affine workspace too small (%zu < %zu) or misaligned.", workspace_bytes,
                 ws.total);
   char *base = static_cast<char *>(workspace);
-  if (one_walk && !rows_affine_covers(W, Wb, M, K, N))
+  if (one_walk && !rows_affine_covers(W, Wb, alpha, bias, y, M, K, N))
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "one-walk binary affine: shape or alignment not covered (M=%lld, K=%lld, "
                 "N=%lld).", (long long)M, (long long)K, (long long)N);
   if (!one_walk && small_m_affine_applies(x, W, Wb, alpha, bias, y, M, K, N)) {
@@ -92,13 +97,14 @@ int binary_affine_forward(const float *x, const float *W, float *Wb, float *alph
   hipStream_t stream = as_stream(stream_);
   int rc;
 
-  if (one_walk || (rows_affine_covers(W, Wb, M, K, N) && rows_affine_pays(M, N))) {
+  if (one_walk || (rows_affine_covers(W, Wb, alpha, bias, y, M, K, N) && rows_affine_pays(M, K, N))) {
     // one walk over W: signs, column sums and the product together
     if (!representable && (rc = launch_clear_words(count, 1, stream)))
       return rc;
     if ((rc = launch_split_digits_rows_redo(x, K, nullptr, xsplit, M, K, nullptr, nullptr, stream)))
       return rc;
-    if ((rc = launch_rows_affine(xsplit, W, Wb, alpha, bias, y, M, K, N, zero_to, count, stream)))
+    if ((rc = launch_rows_affine(xsplit, W, Wb, alpha, bias, y, M, K, N, zero_to, count, base + ws.gemm_off,
+                                 ws.gemm_bytes, stream)))
       return rc;
   } else {
     rc = nbla_hip_binarize_weights_f32(W, Wb, alpha, bits, K, N, 0, zero_to, representable ? nullptr : count, prep,

@@ -84,15 +84,19 @@ int launch_small_m_affine(const float *x, const float *W, float *Wb, float *alph
                           int64_t M, int64_t K, int64_t N, float zero_to, void *workspace, size_t workspace_bytes,
                           hipStream_t stream);
 
-// The same one-pass forward for 65 .. kRowsMmaMaxRows input rows, on the int8 matrix cores (binary_rows_mma.hip): x comes
-// as its digit operand (nbla_hip_split_digits_scaled_f32); rows marked kBadRow there are not written.  With zero_to
-// other than +-1, *zero_flag (cleared by the caller) is raised when W holds a weight that is neither negative nor
-// positive; y is then to be replaced by an fp32 product over Wb.
+// The same forward for up to kRowsMmaMaxRows input rows in one walk over W, on the int8 matrix cores
+// (binary_rows_mma.hip): x comes as its digit operand (nbla_hip_split_digits_scaled_f32); rows marked kBadRow there are
+// not written.  With zero_to other than +-1, *zero_flag (cleared by the caller) is raised when W holds a weight that
+// is neither negative nor positive; y is then to be replaced by an fp32 product over Wb.  `workspace`
+// (rows_affine_workspace_bytes, 16-byte aligned) holds the partial results when K is walked in slices.
 constexpr int64_t kRowsMmaMaxRows = 512;
-bool rows_affine_covers(const float *W, const float *Wb, int64_t M, int64_t K, int64_t N); // shapes it can run
-bool rows_affine_pays(int64_t M, int64_t N); // shapes on which it beats the two-walk path
+bool rows_affine_covers(const float *W, const float *Wb, const float *alpha, const float *bias, const float *y,
+                        int64_t M, int64_t K, int64_t N);   // shapes it can run
+bool rows_affine_pays(int64_t M, int64_t K, int64_t N);     // shapes on which it beats the two-walk path
+size_t rows_affine_workspace_bytes(int64_t M, int64_t K, int64_t N);
 int launch_rows_affine(const void *xdigits, const float *W, float *Wb, float *alpha, const float *bias, float *y,
-                       int64_t M, int64_t K, int64_t N, float zero_to, int *zero_flag, hipStream_t stream);
+                       int64_t M, int64_t K, int64_t N, float zero_to, int *zero_flag, void *workspace,
+                       size_t workspace_bytes, hipStream_t stream);
 
 // db[n] (+)= sum over m of dy[m, n]; `partial` holds ceil(M / 256) * N floats.
 size_t column_sums_workspace_bytes(int64_t M, int64_t N);

@@ -406,10 +406,13 @@ def test_one_walk_product_refuses_what_it_does_not_cover(dev):
     assert ei.value.code == kernels.ERR_NOT_IMPLEMENTED
 
 
-@pytest.mark.parametrize("M,K,N", [(100, 64, 8196), (512, 96, 8192), (257, 40, 9000)])
+@pytest.mark.parametrize("M,K,N", [(100, 1024, 8196),   # 65 strips of 128 columns, K in two slices
+                                   (256, 40, 16388),    # 129 strips, one short slice
+                                   (65, 1600, 5640)])   # 45 strips, K in three slices
 def test_wide_outputs_of_some_hundred_rows_take_the_one_walk_form(dev, M, K, N):
-    """From 8129 columns on (128 strips of 64) the whole-operation entry points run the one-walk form for 65..512
-    rows; checked against the oracle like the other paths."""
+    """For 65..256 rows the whole-operation entry points run the one-walk form when its blocks (strips of 128 columns
+    x slices of K) number at least 128; checked against the oracle like the other paths, and bit-identical to the
+    direct call."""
     x, W = _data(M, K, N, seed=31)
     W.ravel()[::13] = 0.0
     b = np.random.RandomState(9).randn(N).astype(np.float32)
@@ -584,7 +587,7 @@ def test_config3_full_width_small_m_vs_oracle(dev, M):
     assert max_rel_err(to_np(yc), ref_yc) <= TOL
 
 
-@pytest.mark.parametrize("M", [32, 64, 128, 256, 512, 1024, 4096])   # 32, 64: one pass, operands from registers; 128 .. 512: one walk, signs shared through LDS
+@pytest.mark.parametrize("M", [32, 64, 128, 256, 512, 1024, 4096])   # 32, 64: one pass, operands from registers; 128, 256: one walk, signs shared through LDS
 def test_config3_full_size_properties(dev, M):
     """At sizes the oracle cannot finish quickly: float64 dot products on sampled rows/columns,
     linearity in x, and consistency between BinaryWeight and BinaryConnect (y_bw = y_bc * alpha)."""
