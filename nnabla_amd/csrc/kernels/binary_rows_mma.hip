@@ -62,11 +62,13 @@ constexpr int kBTileBytes = 4 * kFragBytes;         // the signs of one k step: 
 constexpr int kAStages = 2;
 constexpr int kAStageBytes = kRowFrags * kDigits * kFragBytes; // 24 KiB
 constexpr int kALoads = kRowFrags * kDigits / 4;    // fragment copies per activation wavefront and k step
+constexpr int kWLoads = 4;                          // copies per weight wavefront and k step
+constexpr int kConvStores = 4;                      // Wb stores per wavefront and k step (four rows, two columns each)
 constexpr int kRingOff = kAStages * kAStageBytes;
 constexpr int kBOff = kRingOff + kRingSlots * kRawBytes;
 constexpr int kRowsLdsBytes = kBOff + 2 * kBTileBytes;
 static_assert(kRowsLdsBytes <= 160 * 1024, "the stages fit the CU's LDS");
-static_assert(12 * kRingDepth - 4 <= 63 && kALoads + 8 <= 63, "vmcnt is a 6-bit counter");
+static_assert((kWLoads + kConvStores) * kRingDepth <= 63 && kALoads + kConvStores <= 63, "vmcnt is a 6-bit counter");
 constexpr int kSignScaleLog2 = 6;                   // sign bytes are +-64
 static_assert(kChunkK * 128 * 64 < (1ll << 31), "64 x digit sums of a chunk of K fit the int32 accumulators");
 
@@ -175,6 +177,7 @@ __global__ __launch_bounds__(kRowsThreads, 1) void binary_affine_rows_kernel(Row
   int ring_conv = 0; // ring slot of the next conversion
   auto issue_w = [&]() __attribute__((always_inline)) {
     unsigned char *dst = smem + kRingOff + ring_next + v * 4096;
+    static_assert(kWLoads == 4, "one copy per pair of rows");
 #pragma unroll
     for (int p = 0; p < 4; ++p)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_void_t *)(dst + p * 1024), 16, w_off, 2 * row_soff[p], 0, 0);
@@ -216,6 +219,7 @@ __global__ __launch_bounds__(kRowsThreads, 1) void binary_affine_rows_kernel(Row
       }
     }
     rows_left -= kTileK;
+    static_assert(kConvStores == 4, "one store per row");
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       uint2_t o;
@@ -287,14 +291,14 @@ __global__ __launch_bounds__(kRowsThreads, 1) void binary_affine_rows_kernel(Row
 #pragma unroll
     for (int t = 0; t <= D; ++t)
       issue_w();
-    NBLA_ROWS_WAIT_VMCNT(4 * (D - 1)); // the first two of D + 1 groups of four copies have landed
+    NBLA_ROWS_WAIT_VMCNT(kWLoads * (D - 1)); // the first two of D + 1 groups of copies have landed
   } else {
     issue_a(0);
   }
   NBLA_ROWS_BARRIER();
   convert(0);
   if (!weights)
-    NBLA_ROWS_WAIT_VMCNT(8); // all but the eight stores
+    NBLA_ROWS_WAIT_VMCNT(kConvStores); // all but the stores
   NBLA_ROWS_WAIT_LGKM0();
   NBLA_ROWS_BARRIER();
 
@@ -303,11 +307,12 @@ __global__ __launch_bounds__(kRowsThreads, 1) void binary_affine_rows_kernel(Row
   // slot k step i left and wait, before the barrier, for k step i + 2; the activation wavefronts request the digits
   // of k step i + 1 (into the stage k step i - 1 left) and wait for them before the barrier: they come out of the L2,
   // which every block of the XCD reads them from at about the same time.
-  // Memory operations of a weight wavefront, in order: the D + 1 copy groups of the prologue (four each), eight
-  // stores, then per iteration one copy group and eight stores.  Behind the copies of k step i + 2 there are, at the
-  // wait, 4 D + 12 + 8 i operations while that k step comes from the prologue (i <= D - 2; the smallest of those
-  // counts is used) and 12 D - 4 after.  Of an activation wavefront: per iteration one copy group (six) and eight stores;
-  // behind the copies of k step i + 1 there are the eight stores.
+  // Memory operations of a weight wavefront, in order: the D + 1 copy groups of the prologue (kWLoads each), the
+  // kConvStores stores of a conversion, then per iteration one copy group and one conversion's stores.  Behind the
+  // copies of k step i + 2 there are, at the wait, kWLoads (D - 2 - i) + kConvStores + (kWLoads + kConvStores) (i + 1)
+  // operations while that k step comes from the prologue (i <= D - 2; the smallest of those counts, that of i = 0, is
+  // used) and kConvStores + (kWLoads + kConvStores) (D - 1) after.  Of an activation wavefront: per iteration one copy
+  // group and one conversion's stores; behind the copies of k step i + 1 there are those stores.
   // (The last iteration converts nothing, so its counts are short; nothing is read after it.)
   int a_cur = 0; // stage of k step i
   int b_cur = 0;
@@ -331,11 +336,11 @@ __global__ __launch_bounds__(kRowsThreads, 1) void binary_affine_rows_kernel(Row
       convert(b_nxt);
     if (weights) {
       if (i <= D - 2)
-        NBLA_ROWS_WAIT_VMCNT(4 * D + 12);
+        NBLA_ROWS_WAIT_VMCNT(kWLoads * (D - 2) + kConvStores + (kWLoads + kConvStores));
       else
-        NBLA_ROWS_WAIT_VMCNT(12 * D - 4);
+        NBLA_ROWS_WAIT_VMCNT(kConvStores + (kWLoads + kConvStores) * (D - 1));
     } else {
-      NBLA_ROWS_WAIT_VMCNT(8);
+      NBLA_ROWS_WAIT_VMCNT(kConvStores);
     }
     NBLA_ROWS_WAIT_LGKM0();
     NBLA_ROWS_BARRIER();

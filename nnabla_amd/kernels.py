@@ -277,12 +277,12 @@ def binary_weight_affine(x, W, bias=None, quantize_zero_to=1.0, workspace=None, 
     return y, Wb, alpha
 
 
-def binary_connect_affine(x, W, bias=None, quantize_zero_to=1.0, workspace=None, out=None, stream=None):
+def binary_connect_affine(x, W, bias=None, quantize_zero_to=1.0, workspace=None, out=None, stream=None, Wb=None):
     """x [M,K], W [K,N...] -> (y, Wb)."""
     import torch
     M, K = x.shape
     N = W.numel() // K
-    Wb = torch.empty_like(W)
+    Wb = torch.empty_like(W) if Wb is None else Wb
     y = torch.empty((M, N), dtype=torch.float32, device=x.device) if out is None else out
     ws = binary_affine_workspace(M, K, N, x) if workspace is None else workspace
     check(lib().nbla_hip_binary_connect_affine_f32(_p(x), _p(W), _p(Wb), _p(bias), _p(y), _i64(M), _i64(K), _i64(N),
