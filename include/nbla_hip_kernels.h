@@ -285,9 +285,13 @@ size_t nbla_hip_affine_backward_workspace_bytes(int64_t M, int64_t K, int64_t N)
  * BinaryConnectAffine<float>::backward_impl, binary_connect_affine.cpp:73-92
  * and the Affine backward they call, affine.cpp:98-140.  dx runs on the
  * bit-weight product (W is binarised again into its transposed packing); Wb
- * (the forward's fp32 signs) is only read when quantize_zero_to is neither +1
- * nor -1 and W holds exact zeros.  dx, dW, db may be NULL (not propagated);
- * accum_* != 0 adds to the existing gradient. */
+ * (the forward's fp32 signs) is only needed when quantize_zero_to is neither +1
+ * nor -1, and only read when W then holds weights that are neither negative nor
+ * positive: they are counted on the device, the bit-weight product does
+ * nothing when the count is non-zero and an fp32 product over Wb launched
+ * behind it does nothing when it is zero (no synchronisation, the host never
+ * reads the count).  dx, dW, db may be NULL (not propagated); accum_* != 0 adds
+ * to the existing gradient. */
 int nbla_hip_binary_affine_backward_f32(const float *dy, const float *x,
                                         const float *W, const float *Wb,
                                         const float *alpha, float *dx,
@@ -356,8 +360,11 @@ size_t nbla_hip_binary_convolution_workspace_bytes(
  * src/nbla/function/generic/binary_weight_convolution.cpp:73-117 (alpha per
  * output channel with the rounded reciprocal of col_w, :66) and the im2col +
  * per-sample Eigen product of convolution.cpp:161-197 / unfold_to_patches.cpp.
- * Argument errors as convolution.cpp:61-103.  Synchronises once when
- * quantize_zero_to is neither +1 nor -1 (see nbla_hip_binary_weight_affine_f32). */
+ * Argument errors as convolution.cpp:61-103.  Never synchronises: a
+ * quantize_zero_to that is neither +1 nor -1 is handled on the device, as in
+ * nbla_hip_binary_weight_affine_f32 (per group: unfold + fp32 product over Wb
+ * behind the matrix-core product, with the group's count of weights that are
+ * neither negative nor positive as their go-ahead). */
 int nbla_hip_binary_weight_convolution_f32(
     const float *x, const float *W, float *Wb, float *alpha, const float *bias,
     float *y, int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
@@ -407,9 +414,11 @@ size_t nbla_hip_convolution_backward_workspace_bytes(
  * binary_connect_convolution.cpp:83-103, the Convolution backward they call,
  * convolution.cpp:199-283, and fold_from_patches.cpp:95-170.  dy is
  * [outer, O, out_sp...], x [outer, C, in_sp...], W and dW [O, C/group, kernel...].
- * dx runs on the bit-weight product; Wb (the forward's fp32 signs) is only read
- * when quantize_zero_to is neither +1 nor -1 and W holds exact zeros.  dx, dW,
- * db may be NULL (not propagated); accum_* != 0 adds to the existing gradient. */
+ * dx runs on the bit-weight product; Wb (the forward's fp32 signs) is only
+ * needed when quantize_zero_to is neither +1 nor -1 and only read when W then
+ * holds weights that are neither negative nor positive (decided on the device as
+ * in nbla_hip_binary_affine_backward_f32: no synchronisation).  dx, dW, db may
+ * be NULL (not propagated); accum_* != 0 adds to the existing gradient. */
 int nbla_hip_binary_convolution_backward_f32(
     const float *dy, const float *x, const float *W, const float *Wb,
     const float *alpha, float *dx, float *dW, float *db, int64_t outer,
@@ -525,7 +534,10 @@ size_t nbla_hip_inq_workspace_bytes(int64_t size, int step);
  * inq_convolution.cpp:110-222): W and I (int32 indicators) are rewritten in
  * place; old_W / old_I are the function's snapshot (read for the restore, then
  * overwritten with the new W / I).  n1n2_out (device, 2 ints, may be NULL)
- * receives the exponent range.  step 3 synchronises the stream once. */
+ * receives the exponent range.  Step 3 synchronises the stream twice (the
+ * number of learnable weights comes to the host, the host's draws go to the
+ * device); every other step is asynchronous.  The same holds for the two
+ * forwards below, which start with this update. */
 int nbla_hip_inq_update_weights_f32(float *W, int32_t *I, float *old_W,
                                     int32_t *old_I, int64_t size, int num_bits,
                                     int step, nbla_hip_bernoulli_fn draw,

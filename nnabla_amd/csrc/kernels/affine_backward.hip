@@ -46,15 +46,8 @@ __global__ __launch_bounds__(256) void column_sum_final(const float *__restrict_
   db[n] = accumulate ? db[n] + acc : acc;
 }
 
-// out[m][n] = dy[m][n] * alpha[n]  (general path only)
-__global__ __launch_bounds__(256) void scale_columns(const float *__restrict__ dy, const float *__restrict__ alpha,
-                                                     float *__restrict__ out, int64_t total, int64_t N) {
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256)
-    out[i] = dy[i] * alpha[i % N];
-}
-
 struct BackwardPlan {
-  size_t bits_off, digits_off, prep_off, count_off, a_planes_off, b_planes_off, flag_off, sums_off, scaled_off, split_off,
+  size_t bits_off, digits_off, prep_off, count_off, a_planes_off, b_planes_off, flag_off, sums_off, split_off,
       split_bytes, total;
 };
 
@@ -81,8 +74,6 @@ BackwardPlan plan_backward(int64_t M, int64_t K, int64_t N) {
   off += 256;
   p.sums_off = off;
   off += round_up(column_sums_workspace_bytes(M, N), 256);
-  p.scaled_off = off; // dy * alpha in fp32, general path only
-  off += round_up((size_t)M * N * sizeof(float), 256);
   p.split_off = off; // partial results of a digit product whose contraction is spread over the CUs (small outputs)
   const size_t s1 = gemm_digits_split_bytes(K, M, N), s2 = gemm_digits_split_bytes(M, N, K);
   p.split_bytes = s1 > s2 ? s1 : s2;
@@ -178,39 +169,26 @@ int nbla_hip_binary_affine_backward_f32(const float *dy, const float *x, const f
                                        nbla_hip_binarize_workspace_bytes(N, K), stream_);
     if (rc)
       return rc;
-    bool use_bits = true;
-    if (!representable) {
-      int host_count = 0;
-      hipError_t e = hipMemcpyAsync(&host_count, count, sizeof(int), hipMemcpyDeviceToHost, stream);
-      if (e == hipSuccess)
-        e = hipStreamSynchronize(stream);
-      if (e != hipSuccess)
-        return fail_hip(e, "reading the zero-weight count");
-      use_bits = host_count == 0;
-    }
-    if (use_bits) {
-      rc = nbla_hip_split_digits_scaled_f32(dy, N, alpha, base + p.digits_off, M, N, stream_);
-      if (rc)
-        return rc;
-      rc = launch_gemm_bits(base + p.digits_off, bits, nullptr, nullptr, dx, M, N, K, 1, K, 1, false, stream,
-                            accum_x != 0);
-    } else {
-      if (!Wb)
-        return fail(NBLA_HIP_ERR_VALUE, "the binarised weights are needed when Sign(0) is neither +1 nor -1.");
-      const float *dyp = dy;
-      if (alpha) {
-        float *scaled = reinterpret_cast<float *>(base + p.scaled_off);
-        int64_t blocks = ceil_div(M * N, 256);
-        if (blocks > 65536)
-          blocks = 65536;
-        hipLaunchKernelGGL(scale_columns, dim3((unsigned)blocks), dim3(256), 0, stream, dy, alpha, scaled, M * N, N);
-        NBLA_HIP_LAUNCH_CHECK("scale_columns");
-        dyp = scaled;
-      }
-      rc = grad_input_planes(dyp, Wb, dx, M, K, N, accum_x != 0, base, p, stream);
-    }
+    // Sign(0) = quantize_zero_to that is neither +1 nor -1 cannot be a sign bit: the pass above has counted, on the
+    // device, the weights that are neither negative nor positive.  The matrix-core product does nothing when that
+    // count is non-zero, and an fp32 product over the forward's signs Wb, launched behind it, does nothing when it is
+    // zero: exactly one of the two writes dx, and the host never reads the count.
+    rc = nbla_hip_split_digits_scaled_f32(dy, N, alpha, base + p.digits_off, M, N, stream_);
     if (rc)
       return rc;
+    rc = launch_gemm_bits(base + p.digits_off, bits, nullptr, nullptr, dx, M, N, K, 1, K, 1, false, stream,
+                          accum_x != 0, nullptr, 0, false, representable ? nullptr : count);
+    if (rc)
+      return rc;
+    if (!representable) {
+      if (!Wb)
+        return fail(NBLA_HIP_ERR_VALUE, "the binarised weights are needed when Sign(0) is neither +1 nor -1.");
+      // dx[m, k] (+)= sum_n (dy[m, n] alpha[n]) Wb[k, n]
+      rc = launch_gemm_f32_mapped(dy, Wb, true, nullptr, nullptr, dx, M, N, K, 1, K, 1, stream, count, alpha,
+                                  accum_x != 0);
+      if (rc)
+        return rc;
+    }
   }
   if (dW) {
     rc = grad_weights(x, dy, dW, M, K, N, accum_w != 0, base, p, stream);

@@ -78,7 +78,7 @@ int binary_affine_forward(const float *x, const float *W, float *Wb, float *alph
   if (one_walk && !rows_affine_covers(W, Wb, alpha, bias, y, M, K, N))
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "one-walk binary affine: shape or alignment not covered (M=%lld, K=%lld, "
                 "N=%lld).", (long long)M, (long long)K, (long long)N);
-  if (!one_walk && small_m_affine_applies(x, W, Wb, alpha, bias, y, M, K, N)) {
+  if (!one_walk && small_m_affine_applies(x, W, Wb, alpha, bias, y, M, K, N, zero_to)) {
     const int rc = ensure_init();
     if (rc)
       return rc;

@@ -20,6 +20,8 @@
 #include "gemm_layout.hpp"
 #include "internal.hpp"
 
+#include <string.h>
+
 namespace nbla_hip {
 namespace {
 
@@ -558,18 +560,23 @@ int launch_few_rows_mma(const float *x, const float *W, float *Wb, float *alpha,
 // From kMmaFromRows rows on the matrix-core walk is the faster one; it needs whole 16-row tiles of W and 16-byte
 // loads of x.  Up to kSmallMMaxRows rows the vector-ALU walk takes what it does not cover.
 constexpr int64_t kMmaFromRows = 9;
-static bool few_rows_mma_applies(const float *x, int64_t M, int64_t K, int64_t N) {
-  // (lane offsets into x and W are 32-bit byte counts)
-  return M >= kMmaFromRows && M <= kFewRowsMaxRows && K % kMmaTileRows == 0 && K < (1ll << 23) && aligned16(x) &&
-         N < (1ll << 26) && mma_plan(K, N).slabs <= 65535;
+static bool few_rows_mma_applies(const float *x, int64_t M, int64_t K, int64_t N, float zero_to) {
+  // (lane offsets into x and W are 32-bit byte counts; the sign operand is the upper half of the fp32 sign, so
+  // Sign(0) = zero_to must be a value bf16 holds exactly)
+  uint32_t zero_to_bits;
+  memcpy(&zero_to_bits, &zero_to, sizeof zero_to_bits);
+  return M >= kMmaFromRows && M <= kFewRowsMaxRows && K >= kMmaTileRows && K % kMmaTileRows == 0 &&
+         K < (1ll << 23) && aligned16(x) && N < (1ll << 26) && (zero_to_bits & 0xffffu) == 0 &&
+         mma_plan(K, N).slabs <= 65535;
 }
 
 bool small_m_affine_applies(const float *x, const float *W, const float *Wb, const float *alpha, const float *bias,
-                            const float *y, int64_t M, int64_t K, int64_t N) {
-  if (!(M >= 1 && N % 4 == 0 && Wb && aligned16(W) && aligned16(Wb) && aligned16(y) && aligned16(alpha) &&
-        aligned16(bias)))
+                            const float *y, int64_t M, int64_t K, int64_t N, float zero_to) {
+  // (the vector-ALU walk addresses a row of W with 32-bit byte offsets)
+  if (!(M >= 1 && K >= 1 && N % 4 == 0 && N < (1ll << 29) && Wb && aligned16(W) && aligned16(Wb) && aligned16(y) &&
+        aligned16(alpha) && aligned16(bias)))
     return false;
-  return few_rows_mma_applies(x, M, K, N) || (M <= kSmallMMaxRows && small_m_slabs(K) <= 65535);
+  return few_rows_mma_applies(x, M, K, N, zero_to) || (M <= kSmallMMaxRows && small_m_slabs(K) <= 65535);
 }
 
 // (sized without knowing x: the larger of the two forms where both may run)
@@ -595,7 +602,7 @@ int launch_small_m_affine(const float *x, const float *W, float *Wb, float *alph
   if (workspace_bytes < small_m_affine_workspace_bytes(M, K, N) || !aligned16(workspace))
     return fail(NBLA_HIP_ERR_MEMORY, "small-M binary affine workspace too small or misaligned.");
   float *partial = static_cast<float *>(workspace);
-  if (few_rows_mma_applies(x, M, K, N)) {
+  if (few_rows_mma_applies(x, M, K, N, zero_to)) {
     if (M <= 32)
       return launch_few_rows_mma<1>(x, W, Wb, alpha, bias, y, M, K, N, zero_to, partial, stream);
     return launch_few_rows_mma<2>(x, W, Wb, alpha, bias, y, M, K, N, zero_to, partial, stream);

@@ -533,7 +533,9 @@ __global__ __launch_bounds__(256) void im2col_digits_columns(const float *__rest
 
 // fp32 unfolded matrix [M, Kg] for the general (non bit-representable) path.
 __global__ __launch_bounds__(256) void im2col_f32(const float *__restrict__ x, float *__restrict__ col, ConvGeom g,
-                                                  int64_t grp) {
+                                                  int64_t grp, const int *__restrict__ run_if) {
+  if (run_if && *run_if == 0) // uniform over the grid
+    return;
   const int64_t total = g.M * g.Kg;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
     const int64_t m = i / g.Kg;
@@ -710,11 +712,12 @@ int launch_im2col_digits_columns(const float *x, void *digits, const ConvGeom &g
   return NBLA_HIP_OK;
 }
 
-int launch_im2col_f32(const float *x, float *col, const ConvGeom &g, int64_t grp, hipStream_t stream) {
+int launch_im2col_f32(const float *x, float *col, const ConvGeom &g, int64_t grp, hipStream_t stream,
+                      const int *run_if) {
   int64_t blocks = ceil_div(g.M * g.Kg, 256);
   if (blocks > 65536)
     blocks = 65536;
-  hipLaunchKernelGGL(im2col_f32, dim3((unsigned)blocks), dim3(256), 0, stream, x, col, g, grp);
+  hipLaunchKernelGGL(im2col_f32, dim3((unsigned)blocks), dim3(256), 0, stream, x, col, g, grp, run_if);
   NBLA_HIP_LAUNCH_CHECK("im2col_f32");
   return NBLA_HIP_OK;
 }
@@ -768,48 +771,40 @@ int binary_conv_forward(const float *x, const float *W, float *Wb, float *alpha,
     if (rc)
       return rc;
   }
-  bool use_bits = true;
-  if (!representable) {
-    int host_counts[64];
-    int total = 0;
-    for (int64_t g0 = 0; g0 < g.group; g0 += 64) {
-      const int64_t nb = (g.group - g0 < 64) ? g.group - g0 : 64;
-      hipError_t e = hipMemcpyAsync(host_counts, counts + g0, sizeof(int) * nb, hipMemcpyDeviceToHost, stream);
-      if (e == hipSuccess)
-        e = hipStreamSynchronize(stream);
-      if (e != hipSuccess)
-        return fail_hip(e, "reading the zero-weight count");
-      for (int64_t i = 0; i < nb; ++i)
-        total += host_counts[i];
-    }
-    use_bits = (total == 0);
-  }
+  // Sign(0) = zero_to that is neither +1 nor -1 cannot be a sign bit: the matrix-core product of a group is then only
+  // valid when the group holds no weight that is neither negative nor positive.  The binarising pass has counted such
+  // weights on the device; the fp32 product over the materialised signs (unfold + product) is launched behind the
+  // matrix-core one with that count as its go-ahead and replaces the group's outputs when it is non-zero.  The host
+  // never reads the count.
   const int64_t hw = g.out_sp_size;
   for (int64_t grp = 0; grp < g.group; ++grp) {
     float *yg = y + grp * g.Og * hw;
     const float *ag = alpha ? alpha + grp * g.Og : nullptr;
     const float *bg = bias ? bias + grp * g.Og : nullptr;
-    if (use_bits && gemm_bits_unfold_applies(g)) {
+    if (gemm_bits_unfold_applies(g)) {
       rc = launch_gemm_bits_unfold(x, g, grp,
                                    reinterpret_cast<const uint32_t *>(base + ws.bits_off + grp * ws.bits_stride), ag, bg,
                                    yg, stream);
-    } else if (use_bits) {
+    } else {
       rc = launch_im2col_digits(x, base + ws.split_off, base + ws.cmax_off, g, grp, stream);
       if (rc)
         return rc;
       rc = launch_gemm_bits(base + ws.split_off,
                             reinterpret_cast<const uint32_t *>(base + ws.bits_off + grp * ws.bits_stride), ag, bg, yg,
                             g.M, g.Kg, g.Og, hw, g.O * hw, hw, true, stream);
-    } else {
-      float *col = reinterpret_cast<float *>(base + ws.total);
-      rc = launch_im2col_f32(x, col, g, grp, stream);
-      if (rc)
-        return rc;
-      rc = launch_gemm_f32_mapped(col, Wb + grp * g.Og * g.Kg, true, ag, bg, yg, g.M, g.Kg, g.Og, hw, g.O * hw, hw,
-                                  stream);
     }
     if (rc)
       return rc;
+    if (!representable) {
+      float *col = reinterpret_cast<float *>(base + ws.total);
+      rc = launch_im2col_f32(x, col, g, grp, stream, counts + grp);
+      if (rc)
+        return rc;
+      rc = launch_gemm_f32_mapped(col, Wb + grp * g.Og * g.Kg, true, ag, bg, yg, g.M, g.Kg, g.Og, hw, g.O * hw, hw,
+                                  stream, counts + grp);
+      if (rc)
+        return rc;
+    }
   }
   return NBLA_HIP_OK;
 }

@@ -144,7 +144,7 @@ __global__ __launch_bounds__(256) void col2im_gather_unit(const float *__restric
 }
 
 struct ConvBackwardPlan {
-  size_t dyt_off, scaled_off, col_off, a_planes_off, b_planes_off, digits_off, bits_off, prep_off, count_off,
+  size_t dyt_off, col_off, a_planes_off, b_planes_off, digits_off, bits_off, prep_off, count_off,
       flag_off, sums_off, total;
 };
 
@@ -156,8 +156,6 @@ ConvBackwardPlan plan_conv_backward(const ConvGeom &g) {
   size_t off = 0;
   const size_t dyt_bytes = round_up((size_t)g.M * g.Og * sizeof(float), 256);
   p.dyt_off = off;
-  off += dyt_bytes;
-  p.scaled_off = off; // dyt * alpha in fp32 (only when Sign(0) is neither +1 nor -1)
   off += dyt_bytes;
   p.col_off = off; // unfolded input [M, Kg], and the unfolded gradient [outer][Kg][L]
   off += round_up((size_t)g.M * g.Kg * sizeof(float), 256);
@@ -224,7 +222,6 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
   hipStream_t stream = as_stream(stream_);
   char *base = static_cast<char *>(workspace);
   float *dyt = reinterpret_cast<float *>(base + p.dyt_off);
-  float *scaled = reinterpret_cast<float *>(base + p.scaled_off);
   float *col = reinterpret_cast<float *>(base + p.col_off);
   int *count = reinterpret_cast<int *>(base + p.count_off);
   uint32_t *bits = reinterpret_cast<uint32_t *>(base + p.bits_off);
@@ -237,7 +234,6 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
     if (rc)
       return rc;
     if (dx) {
-      bool use_bits = binary;
       if (binary) {
         // Sign(W_g) packed for the contraction over o: W_g is stored [Og, Kg] = [contraction][column]
         rc = nbla_hip_binarize_weights_f32(Wg, nullptr, nullptr, bits, g.Og, g.Kg, 0, zero_to,
@@ -245,42 +241,30 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
                                            nbla_hip_binarize_workspace_bytes(g.Og, g.Kg), stream_);
         if (rc)
           return rc;
-        if (!representable) {
-          int host_count = 0;
-          hipError_t e = hipMemcpyAsync(&host_count, count, sizeof(int), hipMemcpyDeviceToHost, stream);
-          if (e == hipSuccess)
-            e = hipStreamSynchronize(stream);
-          if (e != hipSuccess)
-            return fail_hip(e, "reading the zero-weight count");
-          use_bits = host_count == 0;
-        }
-      }
-      if (use_bits) {
         rc = nbla_hip_split_digits_scaled_f32(dyt, g.Og, ag, base + p.digits_off, g.M, g.Og, stream_);
         if (rc)
           return rc;
         rc = launch_gemm_bits(base + p.digits_off, bits, nullptr, nullptr, col, g.M, g.Og, g.Kg, L, g.Kg * L, L, true,
                               stream);
-      } else {
-        const float *wsrc = Wg;
-        const float *dsrc = dyt;
-        if (binary) {
-          if (!Wb)
-            return fail(NBLA_HIP_ERR_VALUE, "the binarised weights are needed when Sign(0) is neither +1 nor -1.");
-          wsrc = Wb + grp * g.Og * g.Kg;
-          if (ag) {
-            rc = launch_gather_dy(dy, ag, scaled, g, grp, stream);
-            if (rc)
-              return rc;
-            dsrc = scaled;
-          }
-        }
-        // real x real on the digit product: dyt rows m (row-scaled), the weights' columns kk (column-scaled; signs and
-        // zeros take the one-digit form), contraction over the output channels o
-        rc = nbla_hip_split_digits_f32(dsrc, g.Og, base + p.a_planes_off, g.M, g.Og, stream_);
         if (rc)
           return rc;
-        rc = launch_split_digits_columns(wsrc, g.Kg, base + p.b_planes_off, g.Og, g.Kg, binary, stream);
+        if (!representable) {
+          // Sign(0) is neither +1 nor -1: when the group holds a weight that is neither negative nor positive (counted
+          // on the device by the pass above) the unfolded gradient is recomputed in fp32 from the forward's signs,
+          //   col[m, kk] = sum_o (dyt[m, o] alpha[o]) Wb[o, kk],
+          // by a launch that leaves at once otherwise.  The host never reads the count.
+          if (!Wb)
+            return fail(NBLA_HIP_ERR_VALUE, "the binarised weights are needed when Sign(0) is neither +1 nor -1.");
+          rc = launch_gemm_f32_mapped(dyt, Wb + grp * g.Og * g.Kg, false, nullptr, nullptr, col, g.M, g.Og, g.Kg, L,
+                                      g.Kg * L, L, stream, count, ag, false);
+        }
+      } else {
+        // real x real on the digit product: dyt rows m (row-scaled), the weights' columns kk (column-scaled),
+        // contraction over the output channels o
+        rc = nbla_hip_split_digits_f32(dyt, g.Og, base + p.a_planes_off, g.M, g.Og, stream_);
+        if (rc)
+          return rc;
+        rc = launch_split_digits_columns(Wg, g.Kg, base + p.b_planes_off, g.Og, g.Kg, false, stream);
         if (rc)
           return rc;
         rc = launch_gemm_digits(base + p.a_planes_off, base + p.b_planes_off, nullptr, col, g.M, g.Og, g.Kg, L,

@@ -23,7 +23,9 @@ int make_geom(ConvGeom &g, int64_t outer, int64_t C, int nd, const int64_t *in_s
 // Unfolded activations of group `grp`, as the int8 digit MFMA operand [M, Kg] or as plain fp32 [M, Kg].
 int launch_im2col_digits(const float *x, void *xdigits, void *scratch, const ConvGeom &g, int64_t grp,
                          hipStream_t stream);
-int launch_im2col_f32(const float *x, float *col, const ConvGeom &g, int64_t grp, hipStream_t stream);
+// (run_if, device memory, may be null: the launch does nothing unless the word it points to is non-zero)
+int launch_im2col_f32(const float *x, float *col, const ConvGeom &g, int64_t grp, hipStream_t stream,
+                      const int *run_if = nullptr);
 // col(x)^T (rows = unfolded columns, contraction over the output positions) as a digit operand with one scale per
 // input channel.
 int launch_im2col_digits_columns(const float *x, void *digits, const ConvGeom &g, int64_t grp, hipStream_t stream);

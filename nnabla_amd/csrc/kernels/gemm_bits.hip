@@ -60,6 +60,7 @@ struct GemmBitsArgs {
   const float *ux;
   ConvGeom ug;
   int64_t ugrp;
+  const int *skip_if; // non-zero word: the launch does nothing (may be null)
 };
 
 // LDS buffers (stages resident) per tile shape: what fits the block's share of the CU's 160 KiB, at most six.
@@ -1056,6 +1057,8 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
 template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, bool kSwap>
 __global__ __launch_bounds__(kWavesM *kWavesN *kWavesK * 64, (kWavesM * kWavesN * kWavesK >= 8 ? 1 : 2)) void gemm_bits_kernel(GemmBitsArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  if (a.skip_if && *a.skip_if != 0) // uniform over the grid
+    return;
   // Are all rows of this block's row blocks one-digit rows?  (Same tile mapping as the body; rows past the operand
   // are clamped to its last row, as the copies are.)
   int64_t bm, bn;
@@ -1120,7 +1123,10 @@ __global__ __launch_bounds__(256) void gemm_bits_split_sum(const float *__restri
                                                            int64_t outer_stride, int64_t n_stride,
                                                            const float *__restrict__ alpha,
                                                            const float *__restrict__ bias, int accumulate,
-                                                           const int32_t *__restrict__ keep_shift) {
+                                                           const int32_t *__restrict__ keep_shift,
+                                                           const int *__restrict__ skip_if) {
+  if (skip_if && *skip_if != 0)
+    return;
   const int64_t total = M * N;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
     const int64_t m = i / N, n = i - m * N;
@@ -1163,7 +1169,7 @@ template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream, vo
       hipLaunchKernelGGL(gemm_bits_split_sum, dim3((unsigned)blocks), dim3(256), 0, stream,
                          static_cast<const float *>(split_ws), (int)splits, a.M, a.N, a.y, a.inner, a.outer_stride,
                          a.n_stride, a.finish ? a.alpha : nullptr, a.finish ? a.bias : nullptr, a.accumulate,
-                         a.keep_bad_rows ? a.shift : nullptr);
+                         a.keep_bad_rows ? a.shift : nullptr, a.skip_if);
       NBLA_HIP_LAUNCH_CHECK("gemm_bits_split_sum");
       return NBLA_HIP_OK;
     }
@@ -1182,7 +1188,7 @@ template <bool kSwap> int dispatch(const GemmBitsArgs &a, hipStream_t stream, vo
 int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alpha, const float *bias, float *y,
                      int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
                      bool swap_out, hipStream_t stream, bool accumulate, void *split_ws, size_t split_ws_bytes,
-                     bool keep_bad_rows) {
+                     bool keep_bad_rows, const int *skip_if) {
   if (M <= 0 || K <= 0 || N <= 0 || inner <= 0 || M > 0x7fffffffll || inner > 0x7fffffffll)
     return fail(NBLA_HIP_ERR_VALUE, "invalid GEMM shape (M=%lld, K=%lld, N=%lld).", (long long)M, (long long)K,
                 (long long)N);
@@ -1215,6 +1221,7 @@ int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alp
   a.split_steps = 0;
   a.use_sums = 1;
   a.keep_bad_rows = keep_bad_rows ? 1 : 0;
+  a.skip_if = skip_if;
   a.ux = nullptr;
   a.ugrp = 0;
   a.inner = inner;
@@ -1296,6 +1303,7 @@ int launch_gemm_bits_unfold(const float *x, const ConvGeom &g, int64_t grp, cons
   a.split_steps = 0;
   a.use_sums = 1;
   a.keep_bad_rows = 0;
+  a.skip_if = nullptr;
   a.ux = x;
   a.ug = g;
   a.ugrp = grp;

@@ -15,14 +15,17 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 constexpr int kBM = 128, kBN = 128, kBK = 16, kPad = 4;
 
 // w is [K, N] (kTransB == false) or [N, K] (kTransB == true).  Output element (m, n) goes to
-// y[(m / inner) * outer_stride + n * n_stride + (m % inner)].
+// y[(m / inner) * outer_stride + n * n_stride + (m % inner)] (added to what is there with `accumulate`).  `kscale`
+// (may be null) scales x along the contraction: x[m, k] * kscale[k] is what gets multiplied (rounded first, as a
+// separate scaling pass would).
 template <bool kTransB>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                        const float *__restrict__ colscale,
                                                        const float *__restrict__ bias, float *__restrict__ y,
                                                        int64_t M, int64_t K, int64_t N, int64_t inner,
                                                        int64_t outer_stride, int64_t n_stride,
-                                                       const int *__restrict__ run_if) {
+                                                       const int *__restrict__ run_if,
+                                                       const float *__restrict__ kscale, int accumulate) {
   if (run_if && *run_if == 0) // uniform over the grid: every block leaves at once
     return;
   __shared__ float As[kBK][kBM + kPad]; // [k][m]
@@ -49,7 +52,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const int64_t m = m0 + a_row, k = k0 + a_k + e;
-      av[e] = (m < M && k < K) ? x[m * K + k] : 0.0f;
+      av[e] = (m < M && k < K) ? (kscale ? x[m * K + k] * kscale[k] : x[m * K + k]) : 0.0f;
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -110,7 +113,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__
           if (bias)
             v = v + bi;
           const int64_t off = (inner == 1) ? m * outer_stride : (m / inner) * outer_stride + (m % inner);
-          y[off + n * n_stride] = v;
+          y[off + n * n_stride] = accumulate ? y[off + n * n_stride] + v : v;
         }
       }
   }
@@ -120,21 +123,22 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__
 
 int launch_gemm_f32_mapped(const float *x, const float *w, bool trans_b, const float *colscale, const float *bias,
                            float *y, int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride,
-                           int64_t n_stride, hipStream_t stream, const int *run_if) {
+                           int64_t n_stride, hipStream_t stream, const int *run_if, const float *kscale,
+                           bool accumulate) {
   const dim3 grid((unsigned)ceil_div(N, kBN), (unsigned)ceil_div(M, kBM));
   if (trans_b)
     hipLaunchKernelGGL(gemm_f32_kernel<true>, grid, dim3(256), 0, stream, x, w, colscale, bias, y, M, K, N, inner,
-                       outer_stride, n_stride, run_if);
+                       outer_stride, n_stride, run_if, kscale, accumulate ? 1 : 0);
   else
     hipLaunchKernelGGL(gemm_f32_kernel<false>, grid, dim3(256), 0, stream, x, w, colscale, bias, y, M, K, N, inner,
-                       outer_stride, n_stride, run_if);
+                       outer_stride, n_stride, run_if, kscale, accumulate ? 1 : 0);
   NBLA_HIP_LAUNCH_CHECK("gemm_f32");
   return NBLA_HIP_OK;
 }
 
 int launch_gemm_f32(const float *x, const float *w, const float *colscale, const float *bias, float *y, int64_t M,
                     int64_t K, int64_t N, hipStream_t stream, const int *run_if) {
-  return launch_gemm_f32_mapped(x, w, false, colscale, bias, y, M, K, N, 1, N, 1, stream, run_if);
+  return launch_gemm_f32_mapped(x, w, false, colscale, bias, y, M, K, N, 1, N, 1, stream, run_if, nullptr, false);
 }
 
 } // namespace nbla_hip

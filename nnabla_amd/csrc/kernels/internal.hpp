@@ -9,9 +9,11 @@ namespace nbla_hip {
 // `run_if` (device memory, may be null): the launch does nothing unless the word it points to is non-zero when the
 // kernel starts -- the fallback of a product whose operand turned out not to be expressible in its fast form, decided
 // on the device so that the host never waits for the answer.
+// `kscale` (may be null) scales x along the contraction (x[m, k] * kscale[k]); `accumulate` adds to y.
 int launch_gemm_f32_mapped(const float *x, const float *w, bool trans_b, const float *colscale, const float *bias,
                            float *y, int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride,
-                           int64_t n_stride, hipStream_t stream, const int *run_if = nullptr);
+                           int64_t n_stride, hipStream_t stream, const int *run_if = nullptr,
+                           const float *kscale = nullptr, bool accumulate = false);
 int launch_gemm_f32(const float *x, const float *w, const float *colscale, const float *bias, float *y, int64_t M,
                     int64_t K, int64_t N, hipStream_t stream, const int *run_if = nullptr);
 // Sets `count` 32-bit words to zero with a kernel (a memset node must not be recorded into a captured graph).
@@ -20,10 +22,12 @@ int launch_clear_words(void *dst, size_t count, hipStream_t stream);
 // Bit-weight product with the choice of store orientation: swap_out makes consecutive lanes write consecutive m
 // (for outputs whose m index is the contiguous one, e.g. convolution results [batch, O, Ho*Wo]).  keep_bad_rows: rows
 // of the digit operand marked as holding a non-finite value are left as they are in y instead of being set to NaN.
+// skip_if (device memory, may be null): the launches do nothing when the word it points to is non-zero as they start
+// (the packed bits turned out not to express the weights; the caller's fp32 product runs instead).
 int launch_gemm_bits(const void *xsplit, const uint32_t *bits, const float *alpha, const float *bias, float *y,
                      int64_t M, int64_t K, int64_t N, int64_t inner, int64_t outer_stride, int64_t n_stride,
                      bool swap_out, hipStream_t stream, bool accumulate = false, void *split_ws = nullptr,
-                     size_t split_ws_bytes = 0, bool keep_bad_rows = false);
+                     size_t split_ws_bytes = 0, bool keep_bad_rows = false, const int *skip_if = nullptr);
 // The same product for a convolution with the unfold fused in: the rows are the unfolded windows of x (group `grp`),
 // converted to digits inside the kernel; y is [sample, O, output position].  gemm_bits_unfold_applies tells whether
 // the geometry is covered (otherwise: launch_im2col_digits + launch_gemm_bits).
@@ -78,7 +82,7 @@ size_t gemm_digits_split_bytes(int64_t M, int64_t K, int64_t N);
 constexpr int64_t kSmallMMaxRows = 16;  // rows the one-pass form multiplies on the vector ALUs
 constexpr int64_t kFewRowsMaxRows = 64; // rows the one-pass form multiplies on the matrix cores
 bool small_m_affine_applies(const float *x, const float *W, const float *Wb, const float *alpha, const float *bias,
-                            const float *y, int64_t M, int64_t K, int64_t N);
+                            const float *y, int64_t M, int64_t K, int64_t N, float zero_to);
 size_t small_m_affine_workspace_bytes(int64_t M, int64_t K, int64_t N);
 int launch_small_m_affine(const float *x, const float *W, float *Wb, float *alpha, const float *bias, float *y,
                           int64_t M, int64_t K, int64_t N, float zero_to, void *workspace, size_t workspace_bytes,

@@ -97,6 +97,25 @@ def test_binary_affine_backward_with_zero_weights(dev, q0):
     assert max_rel_err(to_np(gdw), rdw) <= TIGHT * 4
 
 
+@pytest.mark.parametrize("zeros", [False, True])
+@pytest.mark.parametrize("M,K,N", [(20, 64, 72), (300, 200, 130)])
+def test_binary_affine_backward_zero_to_decided_on_the_device(dev, M, K, N, zeros):
+    """quantize_zero_to = 0 onto a gradient that is already there: with exact-zero weights the fp32 product over the
+    signs must be the one that adds to dx, without them the bit-weight product -- exactly one of the two, chosen on
+    the device (the call never synchronises)."""
+    x, W, dy = _data(M, K, N, 37)
+    if zeros:
+        W.ravel()[::5] = 0.0
+    alpha = np.abs(W).mean(0).astype(np.float32)
+    Wb = oracle.sign(W, 0.0)
+    odx = np.random.RandomState(8).randn(M, K).astype(np.float32)
+    d = lambda a: _dev(a, dev)
+    gdx = kernels.binary_affine_backward(d(dy), d(x), d(W), d(Wb), d(alpha), 0.0, dx=d(odx),
+                                         want=(True, False, False))[0]
+    dx64 = odx.astype(np.float64) + (dy.astype(np.float64) * alpha) @ Wb.astype(np.float64).T
+    assert max_rel_err(to_np(gdx), dx64) <= TIGHT * 4
+
+
 @pytest.mark.parametrize("M,K,N", SHAPES)
 def test_affine_backward_real_weights(dev, M, K, N):
     """The product inside INQAffine: weights that are zero or signed powers of two, and arbitrary ones."""

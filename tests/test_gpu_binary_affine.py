@@ -621,21 +621,27 @@ def test_workspace_too_small_is_reported(dev):
     assert ei.value.code == kernels.ERR_MEMORY
 
 
+@pytest.mark.parametrize("q0,zeros", [(1.0, False), (0.0, False), (0.0, True)])
 @pytest.mark.parametrize("M", [96, 48, 4])   # packed-bit product; one pass on the matrix cores; on the vector ALUs
-def test_forward_replays_in_a_hip_graph(dev, M):
+def test_forward_replays_in_a_hip_graph(dev, M, q0, zeros):
     """BinaryWeightAffine and a FixedPointQuantize in front of it, captured once and replayed with new inputs: the
-    entry points allocate nothing, never synchronise on this path and clear their scratch with kernels, so every
-    replay must reproduce the eager result bit for bit (eager work and synchronisations run between the replays)."""
+    entry points allocate nothing, never synchronise and clear their scratch with kernels, so every replay must
+    reproduce the eager result bit for bit (eager work and synchronisations run between the replays).  With
+    quantize_zero_to = 0 the choice between the matrix-core product and the fp32 product over the signs is made on the
+    device (test_binary_weight_affine.py:72 covers that value), with and without exact-zero weights."""
     K, N = 512, 768
     rng = np.random.RandomState(77)
-    W = _dev((rng.randn(K, N) * 0.02).astype(np.float32), dev)
+    Wh = (rng.randn(K, N) * 0.02).astype(np.float32)
+    if zeros:
+        Wh.ravel()[::9] = 0.0
+    W = _dev(Wh, dev)
     x = torch.empty(M, K, device=dev)
     xq, y = torch.empty_like(x), torch.empty(M, N, device=dev)
     ws = kernels.binary_affine_workspace(M, K, N, x)
 
     def step():
         kernels.fixed_point_quantize(x, True, 8, 2.0 ** -4, out=xq)
-        return kernels.binary_weight_affine(xq, W, None, 1.0, workspace=ws, out=y)
+        return kernels.binary_weight_affine(xq, W, None, q0, workspace=ws, out=y)
 
     x.copy_(_dev(rng.randn(M, K).astype(np.float32), dev))
     step()                                            # first call outside the capture (one-time kernel attributes)
@@ -654,5 +660,20 @@ def test_forward_replays_in_a_hip_graph(dev, M):
         torch.cuda.synchronize()
         assert bits_equal(got, to_np(y)), "replay %d differs from the eager result" % i
         ref, _, _ = oracle.binary_weight_affine(oracle.fixed_point_quantize(to_np(xi), True, 8, 2.0 ** -4),
-                                                to_np(W), None, 1.0)
+                                                to_np(W), None, q0)
         assert max_rel_err(got, ref) <= TOL
+
+
+@pytest.mark.parametrize("M", [9, 32, 64, 100])
+def test_quantize_zero_to_that_bf16_does_not_hold(dev, M):
+    """Sign(0) = 0.3 with exact-zero weights: the one-pass form that feeds bf16 signs to the matrix cores would cut
+    0.3 to eight significand bits, so such a value takes the other forms (fp32 arithmetic on the signs)."""
+    x, W = _data(M, 256, 260, seed=M)
+    W.ravel()[::6] = 0.0
+    b = np.random.RandomState(4).randn(260).astype(np.float32)
+    ref_y, ref_Wb, ref_alpha = oracle.binary_weight_affine(x, W, b, 0.3)
+    y, Wb, alpha = kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev), _dev(b, dev), 0.3)
+    assert bits_equal(to_np(Wb), ref_Wb)
+    np.testing.assert_allclose(to_np(alpha), ref_alpha, rtol=2e-6)
+    y64 = x.astype(np.float64) @ (ref_Wb.astype(np.float64) * np.abs(W.astype(np.float64)).mean(0)) + b
+    assert max_rel_err(to_np(y), y64) <= TIGHT and max_rel_err(to_np(y), ref_y) <= TIGHT * 4
