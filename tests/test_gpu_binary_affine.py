@@ -426,6 +426,50 @@ def test_wide_outputs_of_some_hundred_rows_take_the_one_walk_form(dev, M, K, N):
     assert bits_equal(to_np(y1), to_np(y)) and bits_equal(to_np(a1), to_np(alpha))
 
 
+@pytest.mark.parametrize("ratio_log2", [8, 12, 17])
+@pytest.mark.parametrize("M", [8, 48, 200, 600])   # vector ALUs (no digits: control), bf16 terms, one walk, two walks
+def test_error_bound_with_a_wide_range_inside_a_row(dev, M, ratio_log2):
+    """The digit product rounds x to 24 bits relative to the largest magnitude OF ITS ROW (q = rint(x 2^s), 2^s the
+    largest power of two with |q| <= 8355711), exactly once; everything after that is exact integer arithmetic and one
+    rounding of the result.  So for every output
+        |y - y64| <= K * max|x_row| / 8355711 * alpha + 2^-23 |y64|,
+    whatever the values (typically sqrt(K) instead of K).  Rows with one or two outliers 2^8 .. 2^17 times the rest:
+    where two outliers cancel in an output, that output's RELATIVE error can reach ratio * 2^-24 * O(1) -- a per cent
+    at 2^17 -- where an fp32 sum in k order may be exact; relative to the largest output of the row (the metric of the
+    acceptance bar, max|y - ref| / max|ref|) it stays below 2e-5.  The forms that do not use digits (up to 64 rows)
+    split x into three bf16 terms or multiply in fp32 and are not subject to the bound; they are checked against the
+    same figures."""
+    K, N = 4096, 256
+    rng = np.random.RandomState(100 + ratio_log2)
+    x = rng.randn(M, K).astype(np.float32)
+    big = np.float32(2.0 ** ratio_log2)
+    kinds = np.arange(M) % 4                       # 0: plain row, 1: one outlier, 2: two that cancel where the signs
+    for m in range(M):                             # agree, 3: two of the same sign
+        j, k = rng.choice(K, 2, replace=False)
+        if kinds[m] >= 1:
+            x[m, j] = big * (1 + rng.rand())
+        if kinds[m] == 2:
+            x[m, k] = -x[m, j]
+        if kinds[m] == 3:
+            x[m, k] = x[m, j] * np.float32(0.75)
+    W = (rng.randn(K, N) * 0.02).astype(np.float32)
+    y, Wb, alpha = kernels.binary_weight_affine(_dev(x, dev), _dev(W, dev))
+    y, alpha = to_np(y).astype(np.float64), to_np(alpha).astype(np.float64)
+    y64 = x.astype(np.float64) @ (np.sign(W).astype(np.float64) * alpha)
+    row_max = np.abs(x).max(1).astype(np.float64)
+    bound = K * row_max[:, None] / 8355711.0 * alpha[None, :] + 2.0 ** -23 * np.abs(y64)
+    err = np.abs(y - y64)
+    assert (err <= bound).all(), "worst err / bound = %.3g" % (err / bound).max()
+    # what it means in the two metrics
+    per_row = err.max(1) / np.abs(y64).max(1)
+    rel = err / np.maximum(np.abs(y64), 1e-30)
+    print("M=%d ratio 2^%d: err/bound max %.3g; err / max|y_row| max %.3g; per-element relative error max %.3g "
+          "(rows with cancelling outliers: %.3g)" % (M, ratio_log2, (err / bound).max(), per_row.max(), rel.max(),
+                                                      rel[kinds == 2].max()))
+    assert per_row.max() <= 2e-5
+    assert err.max() / np.abs(y64).max() <= 2e-5
+
+
 @pytest.mark.parametrize("M,K,N", [(3100, 96, 5732), (3072, 64, 11008)])
 def test_tall_m_every_element(dev, M, K, N):
     """Tall outputs with a ragged last column tile (idle wavefronts, clamped wide groups): every output element is
