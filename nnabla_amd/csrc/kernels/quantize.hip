@@ -43,10 +43,14 @@ template <typename Op, int kUnroll> __global__ __launch_bounds__(kBlock) void ma
     const size_t i = base + (size_t)j * kBlock;
     if (i < n4) {
       float4_t r;
-      r.x = op(v[j].x);
-      r.y = op(v[j].y);
-      r.z = op(v[j].z);
-      r.w = op(v[j].w);
+      if constexpr (Op::kFour) {
+        r = op.four(v[j]);
+      } else {
+        r.x = op(v[j].x);
+        r.y = op(v[j].y);
+        r.z = op(v[j].z);
+        r.w = op(v[j].w);
+      }
       store4(y + 4 * i, r);
     }
   }
@@ -94,6 +98,7 @@ template <typename Op> int launch_map(const float *x, float *y, size_t size, Op 
 // fp32; the product with delta is one fp32 multiply.  When delta is a power of
 // two the divide is replaced by the (bit-identical) multiply with 1/delta.
 template <bool kPow2Delta> struct FixedPointOp {
+  static constexpr bool kFour = false;
   float max_, min_, delta, inv_delta;
   __device__ __forceinline__ void prepare() {}
   __device__ __forceinline__ float operator()(float x) const {
@@ -114,6 +119,7 @@ template <bool kPow2Delta> struct FixedPointOp {
 // pow2_quantize.cpp:55-81.  r = roundf(log2f(|x|)) comes from the calibrated
 // per-binade cut (staged in LDS); 2^r, the clamps and the sign are exact.
 struct Pow2Op {
+  static constexpr bool kFour = false;
   const uint32_t *cuts; // device table, kNumBinades entries
   float p_max, p_min, thr;
   int e_max, e_min; // log2 of p_max / p_min
@@ -161,6 +167,7 @@ struct Pow2Op {
 // binade e-1; with_zero adds the boundary p_min * 2^-0.5 below which the result is 0.  The result is the value of
 // the last boundary at or below |x| (positive floats order like their bit patterns).
 template <int kLevels> struct Pow2SmallOp {
+  static constexpr bool kFour = true;
   uint32_t bound[kLevels]; // ascending; unused entries 0xffffffff
   float value[kLevels];    // result from bound[j] on
   float base;              // result below bound[0]
@@ -178,6 +185,29 @@ template <int kLevels> struct Pow2SmallOp {
     if (sign)
       return neg ? -q : q;
     return neg ? neg_value : q;
+  }
+  // Four values at once: the NaN test is made on the largest of the four magnitudes (one rare branch instead of a
+  // compare and a select per value); the rest is the chain above.
+  __device__ __forceinline__ float4_t four(float4_t x) const {
+    uint32_t u[4];
+    float4_t r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      u[e] = __float_as_uint(x[e]) & 0x7fffffffu;
+      float q = base;
+#pragma unroll
+      for (int j = 0; j < kLevels; ++j)
+        q = (u[e] >= bound[j]) ? value[j] : q;
+      const bool neg = x[e] < 0.0f;
+      r[e] = sign ? (neg ? -q : q) : (neg ? neg_value : q);
+    }
+    const uint32_t top = max(max(u[0], u[1]), max(u[2], u[3]));
+    if (top > 0x7f800000u) { // a NaN among the four: it propagates through every comparison of the reference
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        r[e] = (u[e] > 0x7f800000u) ? __uint_as_float(u[e]) : r[e];
+    }
+    return r;
   }
 };
 

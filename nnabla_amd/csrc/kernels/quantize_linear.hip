@@ -163,6 +163,35 @@ struct QuantizeUniformOp {
     }
     return saturate(round_mode(divide(x, st.s), half_to_even) + st.zp, lo, hi);
   }
+  // Four values at once: the estimate's rounding for all of them, then one (rare, divergent) branch for those near a
+  // tie instead of one per value -- the execution-mask bookkeeping of sixteen branches per thread cost more than the
+  // arithmetic.
+  __device__ __forceinline__ float4_t apply4(float4_t x, const State &st) const {
+    float4_t r;
+    if (st.fast) { // uniform
+      bool near[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float q = x[e] * st.inv;
+        const float t = rintf(q);
+        const float m = fabsf(q);
+        const float d = 0.5f - fabsf(q - t);
+        near[e] = !(m >= 4096.0f || d > fmaxf(m, 0.5f) * 0x1p-20f);
+        r[e] = saturate(t + st.zp, lo, hi);
+      }
+      if (near[0] | near[1] | near[2] | near[3]) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (near[e])
+            r[e] = saturate(round_mode(divide(x[e], st.s), half_to_even) + st.zp, lo, hi);
+      }
+      return r;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      r[e] = saturate(round_mode(divide(x[e], st.s), half_to_even) + st.zp, lo, hi);
+    return r;
+  }
   __device__ __forceinline__ float operator()(float x, float scale, float zp) const { return 0.0f; } // not used
 };
 struct DequantizeOp {
@@ -205,8 +234,7 @@ __global__ __launch_bounds__(kBlock) void broadcast_map(const float *__restrict_
       for (int j = 0; j < kUnroll; ++j) {
         const int64_t t = base + (int64_t)j * kBlock;
         if (t < count) {
-          float4_t o;
-          o.x = op.apply(v[j].x, st), o.y = op.apply(v[j].y, st), o.z = op.apply(v[j].z, st), o.w = op.apply(v[j].w, st);
+          const float4_t o = op.apply4(v[j], st);
           __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(y + 4 * t));
         }
       }
