@@ -620,6 +620,29 @@ int nbla_hip_binary2_f32(int op, const float *x0, const float *x1, float *y,
 int nbla_hip_binary2_backward_f32(int op, int input, const float *dy,
                                   const float *x0, const float *x1, float *dx,
                                   size_t size, int accum, void *stream);
+/* The same arithmetic with broadcasting, plus y = x0 + x1 (op 3) and the
+ * element-wise power y = x0 ^ x1 (op 4: powf, dy x1 x0^(x1-1), dy log(x0) x0^x1;
+ * include/nbla/function/pow2.hpp:44-47): shape0 and shape1 have `ndim` entries
+ * each and differ only where one of them is 1; y has the larger size along
+ * every axis.  Replaces BaseTransformBinary::setup_impl's shapes and strides and
+ * transform_binary, utils/base_transform_binary.hpp:58-205 and :265-284 (Add2
+ * reaches it through its BcAdd2 fall-back, add2.cpp:28-37).  Errors as :60-72.
+ * The backward call gives dx = (accum ? dx : 0) + (the terms of every output
+ * element the operand's element took part in), transform_binary_grad0 / grad1,
+ * :286-336: for a broadcast operand a fixed-order parallel sum where the
+ * reference adds one after the other in fp32 (equal to rounding, the same from
+ * run to run).  powf / logf are the device's, not the host libm's: the power's
+ * bits are not pinned. */
+#define NBLA_HIP_BINARY2_ADD 3
+#define NBLA_HIP_BINARY2_POW 4
+int nbla_hip_broadcast2_f32(int op, const float *x0, const int64_t *shape0,
+                            const float *x1, const int64_t *shape1, float *y,
+                            int ndim, void *stream);
+int nbla_hip_broadcast2_backward_f32(int op, int input, const float *dy,
+                                     const float *x0, const int64_t *shape0,
+                                     const float *x1, const int64_t *shape1,
+                                     float *dx, int ndim, int accum,
+                                     void *stream);
 /* dst[r * dst_stride + i] (+)= src[r * src_stride + i], r < rows, i < len:
  * one input's share of Concatenate<float>::forward_impl / backward_impl,
  * src/nbla/function/generic/concatenate.cpp:62-104 (rows = outer_size_, len =

@@ -5,6 +5,7 @@
 #include <nbla/function/add2.hpp>
 #include <nbla/function/div2.hpp>
 #include <nbla/function/mul2.hpp>
+#include <nbla/function/pow2.hpp>
 #include <nbla/function/sub2.hpp>
 #include <nbla/function/affine.hpp>
 #include <nbla/function/binary_connect_affine.hpp>
@@ -153,6 +154,10 @@ FunctionPtr create_by_name(const string &name, const Context &ctx, const int64_t
   if (name == "Div2") {
     need(1, 0);
     return create_Div2(ctx, ia[0] != 0);
+  }
+  if (name == "Pow2") {
+    need(1, 0);
+    return create_Pow2(ctx, ia[0] != 0);
   }
   if (name == "Concatenate") {
     need(1, 0);

@@ -627,13 +627,25 @@ template <typename T> void ReLUHip<T>::forward_impl(const Variables &inputs, con
 }
 
 // ------------------------------------------------------------ Add2 and Concatenate
-// add2.cpp:39-47
+namespace {
+vector<int64_t> shape64(const Variable *v) {
+  const Shape_t s = v->shape();
+  return vector<int64_t>(s.begin(), s.end());
+}
+} // namespace
+
+// add2.cpp:39-47; inputs of different shapes: the BcAdd2 fall-back of :28-37 (utils/base_transform_binary.hpp:339-356)
 template <typename T> void Add2Hip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
   hip_set_device(this->ctx_);
   const T *x0 = inputs[0]->get_data_pointer<T>(this->ctx_);
   const T *x1 = inputs[1]->get_data_pointer<T>(this->ctx_);
   T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
-  NBLA_HIP_CALL(nbla_hip_add2_f32(x0, x1, y, (size_t)inputs[0]->size(), nullptr));
+  if (inputs[0]->shape() == inputs[1]->shape()) {
+    NBLA_HIP_CALL(nbla_hip_add2_f32(x0, x1, y, (size_t)inputs[0]->size(), nullptr));
+    return;
+  }
+  const vector<int64_t> s0 = shape64(inputs[0]), s1 = shape64(inputs[1]);
+  NBLA_HIP_CALL(nbla_hip_broadcast2_f32(NBLA_HIP_BINARY2_ADD, x0, s0.data(), x1, s1.data(), y, (int)s0.size(), nullptr));
 }
 
 // add2.cpp:59-77
@@ -644,22 +656,34 @@ void Add2Hip<T>::backward_impl(const Variables &inputs, const Variables &outputs
     return;
   hip_set_device(this->ctx_);
   const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
+  const bool same = inputs[0]->shape() == inputs[1]->shape();
+  const vector<int64_t> s0 = shape64(inputs[0]), s1 = shape64(inputs[1]);
   for (int i = 0; i < 2; ++i) {
     if (!propagate_down[i])
       continue;
     T *dx = inputs[i]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[i]);
-    NBLA_HIP_CALL(nbla_hip_add2_backward_f32(dy, dx, (size_t)inputs[0]->size(), accum[i], nullptr));
+    if (same)
+      NBLA_HIP_CALL(nbla_hip_add2_backward_f32(dy, dx, (size_t)inputs[0]->size(), accum[i], nullptr));
+    else // utils/base_transform_binary.hpp:358-392
+      NBLA_HIP_CALL(nbla_hip_broadcast2_backward_f32(NBLA_HIP_BINARY2_ADD, i, dy, nullptr, s0.data(), nullptr, s1.data(),
+                                                     dx, (int)s0.size(), accum[i], nullptr));
   }
 }
 
-// Sub2, Mul2, Div2: utils/base_transform_binary.hpp:339-400 with the expressions of sub2.hpp:41, mul2.hpp:42, div2.hpp:44
+// Sub2, Mul2, Div2, Pow2: utils/base_transform_binary.hpp:339-400 with the expressions of sub2.hpp:41, mul2.hpp:42,
+// div2.hpp:44, pow2.hpp:44-47; inputs of one shape take the plain element-wise kernels, others the broadcasting ones
 #define NBLA_HIP_DEFINE_BINARY2(NAME, OP)                                                                              \
   template <typename T> void NAME##Hip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {           \
     hip_set_device(this->ctx_);                                                                                        \
     const T *x0 = inputs[0]->get_data_pointer<T>(this->ctx_);                                                          \
     const T *x1 = inputs[1]->get_data_pointer<T>(this->ctx_);                                                          \
     T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);                                                 \
-    NBLA_HIP_CALL(nbla_hip_binary2_f32(OP, x0, x1, y, (size_t)inputs[0]->size(), nullptr));                            \
+    if (OP != NBLA_HIP_BINARY2_POW && inputs[0]->shape() == inputs[1]->shape()) {                                      \
+      NBLA_HIP_CALL(nbla_hip_binary2_f32(OP, x0, x1, y, (size_t)inputs[0]->size(), nullptr));                          \
+      return;                                                                                                          \
+    }                                                                                                                  \
+    const vector<int64_t> s0 = shape64(inputs[0]), s1 = shape64(inputs[1]);                                            \
+    NBLA_HIP_CALL(nbla_hip_broadcast2_f32(OP, x0, s0.data(), x1, s1.data(), y, (int)s0.size(), nullptr));              \
   }                                                                                                                    \
   template <typename T>                                                                                                \
   void NAME##Hip<T>::backward_impl(const Variables &inputs, const Variables &outputs,                                  \
@@ -670,17 +694,24 @@ void Add2Hip<T>::backward_impl(const Variables &inputs, const Variables &outputs
     const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);                                                         \
     const T *x0 = inputs[0]->get_data_pointer<T>(this->ctx_);                                                          \
     const T *x1 = inputs[1]->get_data_pointer<T>(this->ctx_);                                                          \
+    const bool same = inputs[0]->shape() == inputs[1]->shape();                                                        \
+    const vector<int64_t> s0 = shape64(inputs[0]), s1 = shape64(inputs[1]);                                            \
     for (int i = 0; i < 2; ++i) {                                                                                      \
       if (!propagate_down[i])                                                                                          \
         continue;                                                                                                      \
       T *dx = inputs[i]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[i]);                                          \
-      NBLA_HIP_CALL(nbla_hip_binary2_backward_f32(OP, i, dy, x0, x1, dx, (size_t)inputs[0]->size(), accum[i],          \
-                                                  nullptr));                                                           \
+      if (OP != NBLA_HIP_BINARY2_POW && same)                                                                          \
+        NBLA_HIP_CALL(nbla_hip_binary2_backward_f32(OP, i, dy, x0, x1, dx, (size_t)inputs[0]->size(), accum[i],        \
+                                                    nullptr));                                                         \
+      else                                                                                                             \
+        NBLA_HIP_CALL(nbla_hip_broadcast2_backward_f32(OP, i, dy, x0, s0.data(), x1, s1.data(), dx, (int)s0.size(),    \
+                                                       accum[i], nullptr));                                            \
     }                                                                                                                  \
   }
 NBLA_HIP_DEFINE_BINARY2(Sub2, NBLA_HIP_BINARY2_SUB)
 NBLA_HIP_DEFINE_BINARY2(Mul2, NBLA_HIP_BINARY2_MUL)
 NBLA_HIP_DEFINE_BINARY2(Div2, NBLA_HIP_BINARY2_DIV)
+NBLA_HIP_DEFINE_BINARY2(Pow2, NBLA_HIP_BINARY2_POW) // pow2.hpp:44-47
 #undef NBLA_HIP_DEFINE_BINARY2
 
 // concatenate.cpp:62-76
@@ -716,12 +747,6 @@ void ConcatenateHip<T>::backward_impl(const Variables &inputs, const Variables &
 }
 
 // ------------------------------------------- QuantizeLinear / DequantizeLinear / Prune
-namespace {
-vector<int64_t> shape64(const Variable *v) {
-  const Shape_t s = v->shape();
-  return vector<int64_t>(s.begin(), s.end());
-}
-} // namespace
 
 // quantize_linear.cpp:28-46 and dequantize_linear.cpp:27-45: scale and zero point have x's rank, sizes 1 or x's.
 namespace {
@@ -900,6 +925,7 @@ template class AffineHip<float>;
 template class ReLUHip<float>;
 template class Add2Hip<float>;
 template class Sub2Hip<float>;
+template class Pow2Hip<float>;
 template class Mul2Hip<float>;
 template class Div2Hip<float>;
 template class ConcatenateHip<float>;

@@ -71,6 +71,7 @@ void init_hip() {
   NBLA_REGISTER_FUNCTION_IMPL(Sub2, Sub2Hip<float>, "hip:float", bool);
   NBLA_REGISTER_FUNCTION_IMPL(Mul2, Mul2Hip<float>, "hip:float", bool);
   NBLA_REGISTER_FUNCTION_IMPL(Div2, Div2Hip<float>, "hip:float", bool);
+  NBLA_REGISTER_FUNCTION_IMPL(Pow2, Pow2Hip<float>, "hip:float", bool);
   NBLA_REGISTER_FUNCTION_IMPL(Concatenate, ConcatenateHip<float>, "hip:float", int);
   NBLA_REGISTER_FUNCTION_IMPL(Convolution, ConvolutionHip<float>, "hip:float", int, const vector<int> &,
                               const vector<int> &, const vector<int> &, int, bool);

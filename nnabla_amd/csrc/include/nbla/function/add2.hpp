@@ -7,6 +7,7 @@
 #include <nbla/cpu.hpp>
 #include <nbla/function.hpp>
 #include <nbla/function/no_cpu_impl.hpp>
+#include <nbla/function/utils/base_transform_binary.hpp>
 #include <nbla/function_registry.hpp>
 
 namespace nbla {
@@ -29,10 +30,12 @@ public:
 
 protected:
   virtual void setup_impl(const Variables &inputs, const Variables &outputs) {
-    // add2.cpp:28-37; the broadcasting fall-back (BcAdd2) is not part of this build
-    NBLA_CHECK(inputs[0]->shape() == inputs[1]->shape(), error_code::not_implemented,
-               "Add2: the inputs must have the same shape (broadcasting is not available in this build).");
-    outputs[0]->reshape(inputs[0]->shape(), true);
+    // add2.cpp:28-37: inputs of one shape, or the broadcasting form (BcAdd2: utils/base_transform_binary.hpp:58-86)
+    if (inputs[0]->shape() == inputs[1]->shape()) {
+      outputs[0]->reshape(inputs[0]->shape(), true);
+      return;
+    }
+    transform_binary_setup(inputs, outputs, false, this->name());
   }
   virtual void forward_impl(const Variables &, const Variables &) { NBLA_NO_CPU_IMPL("Add2"); }
   virtual void backward_impl(const Variables &, const Variables &, const vector<bool> &, const vector<bool> &) {

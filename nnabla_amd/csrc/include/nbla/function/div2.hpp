@@ -7,6 +7,7 @@
 #include <nbla/cpu.hpp>
 #include <nbla/function.hpp>
 #include <nbla/function/no_cpu_impl.hpp>
+#include <nbla/function/utils/base_transform_binary.hpp>
 #include <nbla/function_registry.hpp>
 
 namespace nbla {
@@ -29,10 +30,8 @@ public:
 
 protected:
   virtual void setup_impl(const Variables &inputs, const Variables &outputs) {
-    // utils/base_transform_binary.hpp:55-120; the broadcasting form is not part of this build
-    NBLA_CHECK(inputs[0]->shape() == inputs[1]->shape(), error_code::not_implemented,
-               "Div2: the inputs must have the same shape (broadcasting is not available in this build).");
-    outputs[0]->reshape(inputs[0]->shape(), true);
+    // utils/base_transform_binary.hpp:58-86 (the in-place form is obsolete: copy() above never asks for it)
+    transform_binary_setup(inputs, outputs, false, this->name());
   }
   virtual void forward_impl(const Variables &, const Variables &) { NBLA_NO_CPU_IMPL("Div2"); }
   virtual void backward_impl(const Variables &, const Variables &, const vector<bool> &, const vector<bool> &) {

@@ -1,6 +1,6 @@
 // "hip:float" implementations of Add2 and Concatenate (the functions whose inputs share one quantization range in
-// quantization-aware training) and of Sub2, Mul2, Div2 (whose two inputs are both activations to it); all reuse the
-// generic setup_impl.
+// quantization-aware training) and of Sub2, Mul2, Div2, Pow2 (whose two inputs are both activations to it); all reuse
+// the generic setup_impl, broadcasting included.
 #ifndef NBLA_HIP_FUNCTION_ARITHMETIC_HPP_
 #define NBLA_HIP_FUNCTION_ARITHMETIC_HPP_
 
@@ -8,6 +8,7 @@
 #include <nbla/function/concatenate.hpp>
 #include <nbla/function/div2.hpp>
 #include <nbla/function/mul2.hpp>
+#include <nbla/function/pow2.hpp>
 #include <nbla/function/sub2.hpp>
 #include <nbla/hip/hip.hpp>
 
@@ -49,6 +50,7 @@ protected:
 NBLA_HIP_DECLARE_BINARY2(Sub2);
 NBLA_HIP_DECLARE_BINARY2(Mul2);
 NBLA_HIP_DECLARE_BINARY2(Div2);
+NBLA_HIP_DECLARE_BINARY2(Pow2);
 #undef NBLA_HIP_DECLARE_BINARY2
 
 } // namespace nbla

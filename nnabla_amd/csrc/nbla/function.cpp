@@ -3,6 +3,7 @@
 #include <nbla/function/add2.hpp>
 #include <nbla/function/div2.hpp>
 #include <nbla/function/mul2.hpp>
+#include <nbla/function/pow2.hpp>
 #include <nbla/function/sub2.hpp>
 #include <nbla/function/affine.hpp>
 #include <nbla/function/binary_connect_affine.hpp>
@@ -114,6 +115,7 @@ NBLA_REGISTER_FUNCTION_SOURCE(Prune, float);
 NBLA_REGISTER_FUNCTION_SOURCE(Sink, bool);
 NBLA_REGISTER_FUNCTION_SOURCE(Add2, bool);
 NBLA_REGISTER_FUNCTION_SOURCE(Sub2, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(Pow2, bool);
 NBLA_REGISTER_FUNCTION_SOURCE(Mul2, bool);
 NBLA_REGISTER_FUNCTION_SOURCE(Div2, bool);
 NBLA_REGISTER_FUNCTION_SOURCE(Concatenate, int);

@@ -6,9 +6,9 @@ QuantizeLinear -> DequantizeLinear pairs whose scales come from the recorded ran
 under the scope '<function type>-<position of the function in the graph>'.
 
 The inputs of Add2 and Concatenate share one recorder and one quantization range (that of the input produced
-earliest in the graph), as in the reference; of the two-input arithmetic set only Add2 exists on this path (Sub2,
-Mul2, Div2 and Pow2 are recognised by name, so their inputs are both treated as activations).  The QNN / MIXED_QNN
-precision modes are None in the reference too (quantize.py:409-413).
+earliest in the graph), as in the reference; both inputs of Add2, Sub2, Mul2, Div2 and Pow2 are activations
+(quantize.py:30-36), and all five exist on the hip context, broadcasting included.  The QNN / MIXED_QNN precision
+modes are None in the reference too (quantize.py:409-413).
 """
 from collections import defaultdict
 
@@ -39,10 +39,12 @@ def _count_activations(f, inputs):
     return 2 if fn in _TWO_ACTIVATIONS else 1
 
 
-def _earliest(variables, eligible=lambda v: True):
+def _earliest(variables, eligible=lambda v: True, first_rank=None):
     """Index of the variable of lowest rank (first of equals) among the eligible ones after the first, which is the
-    candidate to beat (quantize.py:117-123, 354-360)."""
-    idx, low = 0, variables[0].rank
+    candidate to beat (quantize.py:117-123, 354-360).  ``first_rank``: the rank that candidate is credited with when
+    it is not its own (the recording pass compares the later inputs' recorded ranks with the rank of the first
+    input BEFORE its recorder, quantize.py:120)."""
+    idx, low = 0, (variables[0].rank if first_rank is None else first_rank)
     for i, v in enumerate(variables[1:]):
         if eligible(v) and v.rank < low:
             idx, low = i + 1, v.rank
@@ -136,7 +138,7 @@ class QuantizeNonQNNToRecordingModifier(FunctionModifier):
         earliest; the other inputs' own recorders are taken out again."""
         if f.info.type_name not in _SHARED_RANGE:
             return new_inputs
-        idx = _earliest(new_inputs)
+        idx = _earliest(new_inputs, first_rank=inputs[0].rank)
         scope = self.get_parameter_scope(new_inputs[idx].parent.inputs[1])
         for i, v in enumerate(new_inputs):
             if i == idx:

@@ -148,6 +148,12 @@ def div2(x0, x1, inplace=False, n_outputs=-1, outputs=None):
     return f(x0, x1, n_outputs=n_outputs, outputs=outputs)
 
 
+def pow2(x0, x1, inplace=False, n_outputs=-1, outputs=None):
+    """Element-wise power x0 ** x1 (not the power-of-two quantizer: that is pow2_quantize)."""
+    f = Function("Pow2", None, [int(inplace)], args=dict(inplace=inplace))
+    return f(x0, x1, n_outputs=n_outputs, outputs=outputs)
+
+
 def concatenate(*x, **kw):
     axis = kw.pop('axis', None)
     n_outputs, outputs = kw.pop('n_outputs', -1), kw.pop('outputs', None)

@@ -45,6 +45,7 @@ EXPORTED = (
     "nbla_hip_memcpy", "nbla_hip_device_synchronize", "nbla_hip_stream_synchronize", "nbla_hip_fill",
     "nbla_hip_cast", "nbla_hip_relu_f32", "nbla_hip_relu_backward_f32", "nbla_hip_add2_f32",
     "nbla_hip_add2_backward_f32", "nbla_hip_binary2_f32", "nbla_hip_binary2_backward_f32", "nbla_hip_copy_rows_f32",
+    "nbla_hip_broadcast2_f32", "nbla_hip_broadcast2_backward_f32",
 )
 
 
@@ -240,6 +241,29 @@ def gemm_bits(xsplit, bits, alpha, bias, M, K, N, out=None, inner=1, outer_strid
                                        _i64(inner), _i64(N if outer_stride is None else outer_stride), _i64(n_stride),
                                        _p(ws), ctypes.c_size_t(ws.numel()), _stream(stream)))
     return y
+
+
+BROADCAST2_OPS = {"sub2": 0, "mul2": 1, "div2": 2, "add2": 3, "pow2": 4}
+
+
+def broadcast2(op, x0, x1, stream=None):
+    """y = op(x0, x1) with broadcasting (shapes of one rank, sizes equal or 1 along every axis)."""
+    import torch
+    shape = tuple(max(a, b) for a, b in zip(x0.shape, x1.shape))
+    y = torch.empty(shape, dtype=torch.float32, device=x0.device)
+    check(lib().nbla_hip_broadcast2_f32(BROADCAST2_OPS[op], _p(x0), _shape(x0.shape), _p(x1), _shape(x1.shape), _p(y),
+                                        x0.dim(), _stream(stream)))
+    return y
+
+
+def broadcast2_backward(op, i, dy, x0, x1, dx=None, stream=None):
+    """Gradient of input i; a dx passed in is accumulated onto (in place)."""
+    import torch
+    like = x0 if i == 0 else x1
+    out, accum = (torch.empty_like(like), 0) if dx is None else (dx, 1)
+    check(lib().nbla_hip_broadcast2_backward_f32(BROADCAST2_OPS[op], i, _p(dy), _p(x0), _shape(x0.shape), _p(x1),
+                                                 _shape(x1.shape), _p(out), x0.dim(), accum, _stream(stream)))
+    return out
 
 
 def binary_affine_workspace(M, K, N, like):

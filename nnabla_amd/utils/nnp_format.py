@@ -319,6 +319,7 @@ _FUNCTION_PARAMS = OrderedDict([
     ("sub2", (67, [("inplace", "bool")])),
     ("mul2", (68, [("inplace", "bool")])),
     ("div2", (70, [("inplace", "bool")])),
+    ("pow2", (71, [("inplace", "bool")])),
     ("concatenate", (132, [("axis", "int64")])),
     ("binary_connect_affine", (201, [("base_axis", "int64"), ("quantize_zero_to", "float")])),
     ("binary_connect_convolution", (202, _CONV + [("quantize_zero_to", "float")])),

@@ -81,6 +81,7 @@ _BUILDERS = {
     "Sub2": ("sub2_param", 2, lambda p, i: F.sub2(i[0], i[1], inplace=bool(p.get("inplace", False)))),
     "Mul2": ("mul2_param", 2, lambda p, i: F.mul2(i[0], i[1], inplace=bool(p.get("inplace", False)))),
     "Div2": ("div2_param", 2, lambda p, i: F.div2(i[0], i[1], inplace=bool(p.get("inplace", False)))),
+    "Pow2": ("pow2_param", 2, lambda p, i: F.pow2(i[0], i[1], inplace=bool(p.get("inplace", False)))),
     "Concatenate": ("concatenate_param", 2, lambda p, i: F.concatenate(
         *i, axis=int(p.get("axis", len(i[0].shape) - 1)))),
     "QuantizeLinear": ("quantize_linear_param", 3, lambda p, i: F.quantize_linear(

@@ -428,6 +428,111 @@ def recorder_scale(m, M, kind, narrow_range=False, round_method="NOTROUND"):
     return np.asarray(scale, np.float32)
 
 
+TRANSFORM_BINARY_OPS = ("sub2", "mul2", "div2", "add2", "pow2")   # the kernel library's operation codes 0..4
+
+
+def _transform_binary_strides(shape0, shape1):
+    """Output shape, merged axis groups and strides (0 along a broadcast group) of a two-input element-wise function:
+    include/nbla/function/utils/base_transform_binary.hpp:58-205, statement by statement (the padding to three groups,
+    :163-169, adds groups of size one and changes no index)."""
+    s0, s1 = [int(v) for v in shape0], [int(v) for v in shape1]
+    if len(s0) != len(s1):
+        raise OracleError("Dimensions of inputs must match.")
+    ndim = len(s0)
+    oshape = []
+    for i in range(ndim):
+        if s0[i] != s1[i] and min(s0[i], s1[i]) != 1:
+            raise OracleError("Broadcast dimension must be one.")
+        oshape.append(max(s0[i], s1[i]))
+    c0, c1, cy = [], [], []
+    t0 = t1 = ty = 1
+    for i in range(ndim - 1):
+        t0, t1, ty = t0 * s0[i], t1 * s1[i], ty * oshape[i]
+        kinds = [(s0[a] == s1[a], s0[a] == 1 and s1[a] != 1, s0[a] != 1 and s1[a] == 1) for a in (i, i + 1)]
+        if not any(kinds[0][k] and kinds[1][k] for k in range(3)):
+            c0.append(t0), c1.append(t1), cy.append(ty)
+            t0 = t1 = ty = 1
+    if ndim > 0:
+        c0.append(t0 * s0[-1]), c1.append(t1 * s1[-1]), cy.append(ty * oshape[-1])
+    while len(cy) < 3:
+        c0.insert(0, 1), c1.insert(0, 1), cy.insert(0, 1)
+    n = len(cy)
+    st0, st1, sty = [1] * n, [1] * n, [1] * n
+    for i in range(n - 2, -1, -1):
+        st0[i], st1[i], sty[i] = st0[i + 1] * c0[i + 1], st1[i + 1] * c1[i + 1], sty[i + 1] * cy[i + 1]
+    st0 = [st0[i] if c0[i] == cy[i] else 0 for i in range(n)]
+    st1 = [st1[i] if c1[i] == cy[i] else 0 for i in range(n)]
+    return tuple(oshape), cy, sty, st0, st1
+
+
+def _transform_binary_indices(shape0, shape1):
+    oshape, cy, sty, st0, st1 = _transform_binary_strides(shape0, shape1)
+    size = int(np.prod(oshape, dtype=np.int64)) if len(oshape) else 1
+    idx = np.arange(size, dtype=np.int64)
+    idx0, idx1 = np.zeros(size, np.int64), np.zeros(size, np.int64)
+    for i in range(len(cy)):                      # :270-277
+        dim_idx = (idx // sty[i]) % cy[i]
+        idx0 += dim_idx * st0[i]
+        idx1 += dim_idx * st1[i]
+    return oshape, idx0, idx1
+
+
+def _binary_forward(op, a, b):
+    f = np.float32
+    with np.errstate(all="ignore"):
+        if op == "sub2":
+            return (a - b).astype(f)
+        if op == "mul2":
+            return (a * b).astype(f)
+        if op == "div2":
+            return (a / b).astype(f)
+        if op == "add2":
+            return (a + b).astype(f)
+        return np.power(a, b).astype(f)           # std::pow on floats; numpy's powf, not bit-pinned
+
+
+def _binary_grad(op, i, dy, a, b):
+    """sub2.hpp:41, mul2.hpp:42, div2.hpp:44, bc_add2.hpp, pow2.hpp:44-47, every operation in fp32."""
+    f = np.float32
+    with np.errstate(all="ignore"):
+        if op == "sub2":
+            return dy if i == 0 else -dy
+        if op == "mul2":
+            return (dy * b).astype(f) if i == 0 else (dy * a).astype(f)
+        if op == "div2":
+            return (dy / b).astype(f) if i == 0 else ((-dy * a).astype(f) / (b * b).astype(f)).astype(f)
+        if op == "add2":
+            return dy
+        if i == 0:
+            return ((dy * b).astype(f) * np.power(a, (b - f(1)).astype(f)).astype(f)).astype(f)
+        return ((dy * np.log(a).astype(f)).astype(f) * np.power(a, b).astype(f)).astype(f)
+
+
+def transform_binary(op, x0, x1):
+    """y = op(x0, x1) with broadcasting: transform_binary, utils/base_transform_binary.hpp:265-284 (every output index
+    decomposed over the merged groups, operand indices through strides that are 0 along a broadcast group)."""
+    assert op in TRANSFORM_BINARY_OPS
+    oshape, idx0, idx1 = _transform_binary_indices(np.shape(x0), np.shape(x1))
+    x0, x1 = _f32(x0), _f32(x1)
+    return _binary_forward(op, x0.reshape(-1)[idx0], x1.reshape(-1)[idx1]).reshape(oshape)
+
+
+def transform_binary_backward(op, i, dy, x0, x1, g=None):
+    """Gradient of input i: transform_binary_grad0 / grad1, utils/base_transform_binary.hpp:286-336, on a gradient
+    array that is zeroed first (:377-379 / :385-387) unless ``g`` (accumulation) is given: the terms are added one
+    after the other in ascending output index, in fp32."""
+    assert op in TRANSFORM_BINARY_OPS and i in (0, 1)
+    shape0, shape1 = np.shape(x0), np.shape(x1)
+    oshape, idx0, idx1 = _transform_binary_indices(shape0, shape1)
+    assert tuple(np.shape(dy)) == tuple(oshape)
+    dy, x0, x1 = _f32(dy), _f32(x0), _f32(x1)
+    terms = _binary_grad(op, i, dy.reshape(-1), x0.reshape(-1)[idx0], x1.reshape(-1)[idx1])
+    shape = shape0 if i == 0 else shape1
+    out = np.zeros(shape, np.float32) if g is None else _f32(g).copy().reshape(shape)
+    np.add.at(out.reshape(-1), idx0 if i == 0 else idx1, terms)      # unbuffered: in index order, in fp32
+    return out
+
+
 class Inq(object):
     """Stateful INQ weight logic (one object per INQAffine / INQConvolution)."""
 

@@ -352,8 +352,23 @@ def test_two_input_arithmetic_functions(ctx, name):
         h0 = {"sub2": g, "mul2": g * b, "div2": g / b}[name]
         h1 = {"sub2": -g, "mul2": g * b, "div2": (-g * b) / (b * b)}[name]
         assert bits_equal(vc.g, ((f32(0) + h0) + h1).astype(f32))
+    # inputs that broadcast against each other (utils/base_transform_binary.hpp:58-86), against the oracle
+    c = (rng.standard_normal((5, 1, 9)) + np.float32(3.0)).astype(np.float32)
+    vd = _var(c)
+    vd.need_grad = True
+    w = getattr(F, name)(va, vd)
+    assert w.shape == shape
+    w.forward()
+    assert bits_equal(w.d, oracle.transform_binary(name, a, c))
+    va.g, vd.g = 0.0, 0.0
+    w.backward(g)
+    with np.errstate(all="ignore"):
+        assert bits_equal(va.g, oracle.transform_binary_backward(name, 0, g, a, c))
+        ref1 = oracle.transform_binary_backward(name, 1, g, a, c)
+    fin = np.isfinite(ref1)
+    assert np.array_equal(np.isfinite(vd.g), fin) and np.allclose(vd.g[fin], ref1[fin], rtol=1e-5, atol=1e-5)
     with pytest.raises(RuntimeError):
-        getattr(F, name)(va, _var(np.zeros((5, 1, 9), np.float32)))     # broadcasting is not available
+        getattr(F, name)(va, _var(np.zeros((5, 2, 9), np.float32)))     # 7 against 2: not a broadcast
 
 
 def test_add2_and_concatenate_functions(ctx):
@@ -371,8 +386,20 @@ def test_add2_and_concatenate_functions(ctx):
     y.backward(g)
     assert bits_equal(vb.g, g)
     assert np.allclose(va.g, g) or np.allclose(va.g, g + 1.5)      # written, or added when the graph accumulates
+    # the broadcasting fall-back of add2.cpp:28-37
+    c = rng.standard_normal((3, 1, 5)).astype(np.float32)
+    vc = _var(c)
+    vc.need_grad = True
+    z = F.add2(va, vc)
+    assert z.shape == (3, 4, 5)
+    z.forward()
+    assert bits_equal(z.d, a + c)
+    va.g, vc.g = 0.0, 0.0
+    z.backward(g)
+    assert bits_equal(va.g, (np.float32(0) + g).astype(np.float32))
+    assert np.allclose(vc.g, g.sum(1, keepdims=True), rtol=1e-6, atol=1e-6)
     with pytest.raises(RuntimeError):
-        F.add2(va, _var(np.zeros((3, 1, 5), np.float32)))          # broadcasting is not available
+        F.add2(va, _var(np.zeros((3, 2, 5), np.float32)))          # 4 against 2: not a broadcast
 
     parts = [rng.standard_normal((2, n, 3, 7)).astype(np.float32) for n in (4, 1, 6)]
     vs = [_var(p) for p in parts]

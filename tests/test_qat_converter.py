@@ -313,6 +313,48 @@ def test_add2_inputs_share_the_recorder_of_the_earliest_one():
     assert r1.inputs[0].parent.info.type_name == 'ReLU'      # r's own recorder is gone from the graph
 
 
+def bias_like_residual_net(x):
+    h = F.relu(PF.convolution(x, 4, (3, 3), pad=(1, 1), name='c1'))      # Convolution-0, ReLU-1
+    g = F.relu(PF.convolution(x, 4, (8, 8), name='gate'))                # Convolution-2, ReLU-3: [2, 4, 1, 1]
+    return PF.affine(F.add2(h, g), 5, name='f')                          # Add2-4, Affine-5
+
+
+def test_add2_with_a_broadcast_operand_converts_like_any_other():
+    """A residual whose second operand broadcasts over the spatial axes (a per-channel gate, [2, 4, 1, 1] onto
+    [2, 4, 8, 8]): the converter does not look at shapes (quantize.py:110-138), so both inputs are recorded, the
+    statistics shared are those of the input produced first, and the rewritten graph keeps the broadcast output
+    shape."""
+    x = nn.Variable((2, 3, 8, 8))
+    cfg = QATConfig()
+    y_rec = to_recording(bias_like_residual_net(x), cfg)
+    act = cfg.recorder_activation().name()
+    add = find(y_rec, 'Add2')[0]
+    assert tuple(add.outputs[0].shape) == (2, 4, 8, 8)
+    assert tuple(add.inputs[0].shape) == (2, 4, 8, 8) and tuple(add.inputs[1].shape) == (2, 4, 1, 1)
+    r0, r1 = add.inputs[0].parent, add.inputs[1].parent
+    assert r0.info.type_name == r1.info.type_name == act and r0 is not r1
+    assert r0.inputs[1] is r1.inputs[1]                       # one set of statistics for the two operands
+    set_statistics(np.random.RandomState(5))
+    add_t = find(to_training(y_rec, cfg), 'Add2')[0]
+    assert tuple(add_t.outputs[0].shape) == (2, 4, 8, 8)
+    assert [tuple(v.shape) for v in add_t.inputs] == [(2, 4, 8, 8), (2, 4, 1, 1)]
+    assert all(v.parent.info.type_name == 'DequantizeLinear' for v in add_t.inputs)
+
+
+def test_share_recorder_credits_the_first_input_with_its_rank_before_the_recorder():
+    """quantize.py:117-123 starts from inputs[0].rank (the first input as the float graph has it) and compares it with
+    the later inputs' ranks AFTER their recorders: a later input whose recorded rank equals that figure does not
+    win.  With the first input's recorded rank as the start (one higher) it would."""
+    from nnabla_amd.experimental.graph_converters.quantize import _earliest
+
+    class V(object):
+        def __init__(self, rank):
+            self.rank = rank
+    new_inputs = [V(4), V(3)]
+    assert _earliest(new_inputs, first_rank=3) == 0          # the reference's rule: 3 < 3 is false
+    assert _earliest(new_inputs) == 1                        # what starting from the recorded rank would pick
+
+
 def gated_net(x):
     h = F.relu(PF.convolution(x, 4, (3, 3), pad=(1, 1), name='c1'))      # Convolution-0, ReLU-1
     r = F.relu(PF.convolution(h, 4, (3, 3), pad=(1, 1), name='c2'))      # Convolution-2, ReLU-3
