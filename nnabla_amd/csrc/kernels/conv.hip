@@ -725,7 +725,7 @@ int launch_im2col_f32(const float *x, float *col, const ConvGeom &g, int64_t grp
 namespace {
 
 struct ConvWorkspace {
-  size_t bits_off, bits_stride, split_off, cmax_off, prep_off, count_off, col_off, total;
+  size_t bits_off, bits_stride, split_off, cmax_off, prep_off, count_off, tap_bits_off, tap_bits_stride, col_off, total;
 };
 
 ConvWorkspace plan_conv(const ConvGeom &g) {
@@ -742,6 +742,9 @@ ConvWorkspace plan_conv(const ConvGeom &g) {
   off += round_up(nbla_hip_binarize_workspace_bytes(g.Kg, g.Og), 256);
   w.count_off = off;
   off += round_up(sizeof(int) * g.group, 256);
+  w.tap_bits_off = off; // the weights prepared for the product over input positions held in LDS, when that runs
+  w.tap_bits_stride = round_up(conv_slab_prepared_bytes(g), 256);
+  off += w.tap_bits_stride * g.group;
   w.col_off = off; // fp32 unfolded matrix of the general path shares the split operand's space when it fits
   w.total = off;
   return w;
@@ -761,8 +764,10 @@ int binary_conv_forward(const float *x, const float *W, float *Wb, float *alpha,
   hipStream_t stream = as_stream(stream_);
   char *base = static_cast<char *>(workspace);
   int *counts = reinterpret_cast<int *>(base + ws.count_off);
-  // weights: per group a [Og, Kg] slab stored n-major -> packed [Kg, Og] bits, Sign, alpha
-  for (int64_t grp = 0; grp < g.group; ++grp) {
+  const bool slab = conv_slab_applies(g);
+  // weights: per group a [Og, Kg] slab stored n-major -> packed [Kg, Og] bits, Sign, alpha (the product over input
+  // positions held in LDS prepares its own form of the weights, below)
+  for (int64_t grp = 0; grp < g.group && !slab; ++grp) {
     const int64_t woff = grp * g.Og * g.Kg;
     rc = nbla_hip_binarize_weights_f32(W + woff, Wb + woff, alpha ? alpha + grp * g.Og : nullptr,
                                        reinterpret_cast<uint32_t *>(base + ws.bits_off + grp * ws.bits_stride), g.Kg,
@@ -781,7 +786,14 @@ int binary_conv_forward(const float *x, const float *W, float *Wb, float *alpha,
     float *yg = y + grp * g.Og * hw;
     const float *ag = alpha ? alpha + grp * g.Og : nullptr;
     const float *bg = bias ? bias + grp * g.Og : nullptr;
-    if (gemm_bits_unfold_applies(g)) {
+    if (slab) {
+      void *prepared = base + ws.tap_bits_off + grp * ws.tap_bits_stride;
+      rc = launch_conv_slab_prepare(W + grp * g.Og * g.Kg, Wb + grp * g.Og * g.Kg, prepared, g, zero_to, stream);
+      if (rc)
+        return rc;
+      rc = launch_conv_slab(x, g, grp, prepared, alpha ? alpha + grp * g.Og : nullptr,
+                            representable ? nullptr : counts + grp, bg, y, stream);
+    } else if (gemm_bits_unfold_applies(g)) {
       rc = launch_gemm_bits_unfold(x, g, grp,
                                    reinterpret_cast<const uint32_t *>(base + ws.bits_off + grp * ws.bits_stride), ag, bg,
                                    yg, stream);

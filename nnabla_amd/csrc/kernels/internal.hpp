@@ -35,6 +35,18 @@ struct ConvGeom;
 bool gemm_bits_unfold_applies(const ConvGeom &g);
 int launch_gemm_bits_unfold(const float *x, const ConvGeom &g, int64_t grp, const uint32_t *bits, const float *alpha,
                             const float *bias, float *y, hipStream_t stream);
+// The binary convolution forward with the unfold done by LDS addressing (conv_slab.hip), two launches per group:
+// launch_conv_slab_prepare reads the group's weights [Og, Cg, taps] once and writes Wb = Sign(W) (may be null) and,
+// into `prepared` (conv_slab_prepared_bytes, 16-byte aligned), the packed bits in (tap, channel) order with the
+// partial |W| sums and zero counts; launch_conv_slab multiplies, forming alpha = mean |W| from the partial sums when
+// alpha_out is not null (and writing it there), and writes the number of weights that are neither negative nor
+// positive to *zero_count when that is not null.  alpha_out and bias belong to the group; y is the whole output.
+bool conv_slab_applies(const ConvGeom &g);
+size_t conv_slab_prepared_bytes(const ConvGeom &g);
+int launch_conv_slab_prepare(const float *Wg, float *Wbg, void *prepared, const ConvGeom &g, float zero_to,
+                             hipStream_t stream);
+int launch_conv_slab(const float *x, const ConvGeom &g, int64_t grp, const void *prepared, float *alpha_out,
+                     int *zero_count, const float *bias, float *y, hipStream_t stream);
 // Digit operand of the rows of x (nbla_hip_split_digits_scaled_f32) for a caller that holds materialised weights
 // Wb [K, N] (* alpha[n], + bias[n]): rows holding a NaN or an infinity get their outputs y[m, :] computed by the
 // splitting kernel itself, as fp32 dot products in the reference's order.  *redone tells whether that happened (only

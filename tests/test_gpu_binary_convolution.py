@@ -42,6 +42,24 @@ CASES = [
     ((1, 2, 5, 300), (4, 2, 3, 3), (1, 1), (1, 1), (1, 1), 1),
     # padding larger than the kernel: windows that lie wholly outside the input
     ((2, 3, 6, 6), (4, 3, 2, 2), (3, 3), (1, 1), (1, 1), 1),
+    # 24 channels per group and more: the product that keeps the input positions under a block's windows in LDS and
+    # contracts over (tap, channel).  One channel tile; stride 2 with two column groups; 48 channels (padded to 64),
+    # dilation 2 and rows of 40 outputs (a block's 32 windows cross rows of the map); one and three spatial
+    # dimensions; groups; windows wholly outside the input; one window per sample; tiny maps
+    ((2, 32, 9, 9), (40, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((2, 64, 12, 10), (300, 64, 3, 3), (1, 1), (2, 2), (1, 1), 1),
+    ((2, 48, 7, 40), (16, 48, 3, 3), (1, 2), (1, 1), (2, 2), 1),
+    ((3, 32, 50), (8, 32, 5), (2,), (1,), (1,), 1),
+    ((1, 32, 4, 5, 6), (8, 32, 2, 3, 2), (1, 0, 1), (1, 2, 1), (1, 1, 2), 1),
+    ((2, 128, 8, 8), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 2),
+    ((2, 32, 6, 6), (4, 32, 2, 2), (3, 3), (1, 1), (1, 1), 1),
+    ((70, 32, 3, 3), (5, 32, 3, 3), (0, 0), (1, 1), (1, 1), 1),
+    ((40, 32, 2, 2), (7, 32, 2, 2), (1, 1), (1, 1), (1, 1), 1),
+    ((1, 24, 5, 70), (4, 24, 1, 7), (0, 3), (1, 3), (1, 1), 1),
+    # the positions under a block (three rows of 70) times 96 channels: more than a wavefront keeps in registers
+    ((1, 96, 5, 70), (8, 96, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    # nine channel tiles (alpha summed from more than eight partial sums)
+    ((1, 288, 6, 6), (8, 288, 3, 3), (1, 1), (1, 1), (1, 1), 1),
 ]
 
 
@@ -73,11 +91,12 @@ def test_binary_connect_convolution_matches_oracle(dev, xs, ws, pad, stride, dil
     assert max_rel_err(to_np(y), ref_y) <= TIGHT
 
 
+@pytest.mark.parametrize("channels", [4, 64])
 @pytest.mark.parametrize("q0", [0.0, -1.0, 0.5])
-def test_convolution_quantize_zero_to_with_zero_weights(dev, q0):
+def test_convolution_quantize_zero_to_with_zero_weights(dev, q0, channels):
     rng = np.random.RandomState(3)
-    x = rng.randn(2, 4, 9, 9).astype(np.float32)
-    W = (rng.randn(6, 2, 3, 3) * 0.05).astype(np.float32)
+    x = rng.randn(2, channels, 9, 9).astype(np.float32)
+    W = (rng.randn(6, channels // 2, 3, 3) * 0.05).astype(np.float32)
     W.ravel()[::4] = 0.0
     ref_y, ref_Wb, ref_alpha = oracle.binary_weight_convolution(x, W, None, (1, 1), (1, 1), (1, 1), 2, q0)
     y, Wb, alpha = kernels.binary_weight_convolution(_dev(x, dev), _dev(W, dev), None, (1, 1), (1, 1), (1, 1), 2, q0)
@@ -88,13 +107,14 @@ def test_convolution_quantize_zero_to_with_zero_weights(dev, q0):
     assert max_rel_err(to_np(y), ref_y) <= TIGHT * 4
 
 
-def test_window_with_a_non_finite_value(dev):
+@pytest.mark.parametrize("channels", [8, 32])
+def test_window_with_a_non_finite_value(dev, channels):
     """An Inf or NaN in x: every output whose window holds it is non-finite in the reference (Inf - Inf and 0 * Inf
     give NaN, convolution.cpp's gemm); here the digit form gives NaN for all output channels of such a window.  All
-    other outputs are unaffected."""
+    other outputs are unaffected.  (8 channels: the gathering product; 32: the one that keeps input positions in LDS.)"""
     rng = np.random.RandomState(5)
-    x = rng.randn(2, 8, 9, 9).astype(np.float32)
-    W = (rng.randn(6, 8, 3, 3) * 0.05).astype(np.float32)
+    x = rng.randn(2, channels, 9, 9).astype(np.float32)
+    W = (rng.randn(6, channels, 3, 3) * 0.05).astype(np.float32)
     clean, _, _ = kernels.binary_weight_convolution(_dev(x, dev), _dev(W, dev), None, (1, 1), (1, 1), (1, 1), 1)
     x[1, 3, 4, 5] = np.inf
     x[0, 0, 0, 0] = np.nan
@@ -106,6 +126,30 @@ def test_window_with_a_non_finite_value(dev):
     for o in range(6):
         assert not np.isfinite(y[:, o][hit]).any()
         assert bits_equal(y[:, o][~hit], clean[:, o][~hit])
+
+
+def test_wide_range_inside_the_positions_under_a_block(dev):
+    """The product over input positions held in LDS rounds x to a multiple of 2^-30 of the largest magnitude among the
+    positions under a block's (at most 32) windows: |y - y64| <= K * 2^-31 * max|x| (+ the fp32 rounding of y), shown
+    on BinaryConnectConvolution (no alpha).  One position 2^12 and one 2^20 times the rest: the bound holds, and
+    windows that do not touch them still agree with float64 to 1e-4 of their own largest output in the first case."""
+    rng = np.random.RandomState(11)
+    W = (rng.randn(16, 32, 3, 3) * 0.05).astype(np.float32)
+    s64 = torch.from_numpy(np.where(W < 0, -1.0, 1.0))
+    for factor in (2.0 ** 12, 2.0 ** 20):
+        x = rng.randn(1, 32, 14, 14).astype(np.float32)
+        x[0, :, 3, 3] *= np.float32(factor)
+        y, _ = kernels.binary_connect_convolution(_dev(x, dev), _dev(W, dev), None, (1, 1), (1, 1), (1, 1), 1)
+        y = to_np(y).astype(np.float64)
+        y64 = torch.nn.functional.conv2d(torch.from_numpy(x).double(), s64, None, 1, 1).numpy()
+        bound = 288 * 2.0 ** -31 * np.abs(x).max() + 2.0 ** -24 * np.abs(y64)
+        assert (np.abs(y - y64) <= bound).all()
+        far = np.ones((14, 14), bool)
+        far[2:5, 2:5] = False
+        err = np.abs(y - y64)[0][:, far].max() / np.abs(y64)[0][:, far].max()
+        print("outlier x%g: error of the windows away from it / their largest output = %.2e" % (factor, err))
+        if factor == 2.0 ** 12:
+            assert err <= 1e-4
 
 
 def test_config4_resnet_stage(dev):
