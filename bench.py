@@ -388,8 +388,9 @@ def main():
                     help="untimed steps; the first few dozen launches after idle run at ramping clocks")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=2048)
-    ap.add_argument("--section", choices=("all", "headline", "quantizers", "other"), default="all",
+    ap.add_argument("--section", choices=("all", "headline", "sweep", "quantizers", "other"), default="all",
                     help="headline: only the timed BinaryWeightAffine steps (what the rocprofv3 summaries profile); "
+                         "sweep: headline plus the forward at M = 1 .. 1024 and BinaryConnectAffine (`sweep`); "
                          "quantizers: headline plus the quantizer kernels; other: headline plus the convolution, INQ, "
                          "MLP, backward and adjacent-function workloads (`other_configs`)")
     args = ap.parse_args()
@@ -406,7 +407,7 @@ def main():
     # clocks (the first dozens of launches after idle run on ramping clocks).  With --section headline there is
     # nothing before them and the figure is a cold one.
     sweep = {}
-    for m in ((1, 8, 16, 32, 64, 128, 256, 512, 1024) if args.section == "all" else ()):
+    for m in ((1, 8, 16, 32, 64, 128, 256, 512, 1024) if args.section in ("all", "sweep") else ()):
         s = bench_whole_forward(m, K, N, max(10, args.steps), 5, dev)
         if m > 256:   # two walks: the product runs on the matrix cores from packed bits; its share, timed between events
             t = bench_binary_weight_affine(m, K, N, max(5, args.steps // 2), 2, dev)
@@ -423,7 +424,7 @@ def main():
             s["path"] = "one pass over W on the vector ALUs (no packed bits, no separate product launch)"
         sweep["M=%d" % m] = s
     # BinaryConnectAffine on the same shapes (the same kernels without alpha)
-    for m in ((1, 8, 64, 512, 4096) if args.section == "all" else ()):
+    for m in ((1, 8, 64, 512, 4096) if args.section in ("all", "sweep") else ()):
         sweep["BinaryConnectAffine M=%d" % m] = bench_whole_forward(m, K, N, max(10, args.steps // 2), 5, dev,
                                                                     connect=True)
     quant = bench_quantizers(dev, max(10, args.steps)) if args.section in ("all", "quantizers") else {}
