@@ -331,12 +331,45 @@ constexpr int kRedBlock = 256;
 constexpr int kRedTile = kRedBlock * 4; // elements per block tile
 constexpr int kMaxChunks = 1024;
 
+// A pattern whose kept axes are separated by reduced ones and whose innermost axis is kept (q shape (C, 1, W)): the
+// kept index is (ko, w) with w along the contiguous axis, the reduced index (ro, ri) with ri along the innermost
+// reduced axis.  The kernels of this form put the lanes along w, so every line of x is read once, and walk the
+// reduced index in row-major order like the reference's scan.
+struct MinMaxInner {
+  bool ok;
+  int64_t Ko, Wk;        // kept: outer combinations, innermost (contiguous) extent
+  int64_t Rout, Rin;     // reduced: outer combinations, innermost extent
+  int64_t rin_stride;    // element stride of the innermost reduced axis
+  int tw;                // lanes along w: the power of two covering min(Wk, 64)
+};
+inline MinMaxInner inner_form(const MinMaxAxes &A) {
+  MinMaxInner I;
+  I.ok = A.nkept >= 1 && A.nred >= 1 && A.kstride[A.nkept - 1] == 1;
+  if (!I.ok)
+    return I;
+  I.Wk = A.ksize[A.nkept - 1];
+  I.Ko = 1;
+  for (int d = 0; d + 1 < A.nkept; ++d)
+    I.Ko *= A.ksize[d];
+  I.Rin = A.rsize[A.nred - 1];
+  I.rin_stride = A.rstride[A.nred - 1];
+  I.Rout = 1;
+  for (int d = 0; d + 1 < A.nred; ++d)
+    I.Rout *= A.rsize[d];
+  I.tw = 1;
+  while (I.tw < 64 && I.tw < I.Wk)
+    I.tw *= 2;
+  I.ok = I.Ko < ((int64_t)1 << 31);
+  return I;
+}
+
 struct MinMaxPlan {
   MinMaxLayout L;
   int64_t tiles_per_row; // tiles covering one run of R1 elements
   int64_t tiles_per_k;   // R0 * tiles_per_row
   int nchunks;           // blocks (and partials) per k
   size_t params_bytes, partial_bytes;
+  bool inner;            // the strided pattern takes the kernels of MinMaxInner
 };
 
 MinMaxPlan make_plan(const int64_t *xshape, int ndim, const int64_t *qshape) {
@@ -351,8 +384,22 @@ MinMaxPlan make_plan(const int64_t *xshape, int ndim, const int64_t *qshape) {
     want = P.tiles_per_k;
   if (want < 1)
     want = 1;
-  if (!P.L.ok)
-    want = 1; // the strided kernels fold a whole slice per block
+  P.inner = false;
+  if (!P.L.ok) {
+    want = 1; // the general strided kernels fold a whole slice per block
+    MinMaxAxes A;
+    if (split_axes(xshape, ndim, qshape, A)) {
+      const MinMaxInner I = inner_form(A);
+      if (I.ok) { // about 2048 blocks, each a run of outer reduced indices
+        P.inner = true;
+        want = (2048 + I.Ko - 1) / I.Ko;
+        if (want > I.Rout)
+          want = I.Rout;
+        if (want > 64)
+          want = 64;
+      }
+    }
+  }
   P.nchunks = (int)want;
   P.params_bytes = round_up((size_t)P.L.K * 16, 256);
   P.partial_bytes = round_up((size_t)P.L.K * P.nchunks * 16, 256);
@@ -685,6 +732,100 @@ __global__ __launch_bounds__(kRedBlock) void minmax_reduce_strided(const float *
     partial[k] = ex.pack();
   }
 }
+// The inner-kept form (MinMaxInner).  Block (ko, chunk): the outer reduced indices ro = chunk, chunk + nchunks, ... are
+// not what it takes -- it takes the contiguous run [chunk * per, (chunk + 1) * per) so that its first-zero index grows
+// along its scan.  Lane = (row slot, w): the block's 256 threads cover 256 / tw rows of tw columns per step; columns
+// beyond 64 are walked in further passes over the block's rows.
+struct InnerWalk {
+  const float *base;   // x at (ko, w = 0)
+  int64_t ro_begin, ro_end;
+};
+__device__ __forceinline__ InnerWalk inner_walk(const float *x, const MinMaxAxes &A, const MinMaxInner &I, int64_t ko,
+                                                int chunk, int nchunks) {
+  InnerWalk w;
+  w.base = x + (A.nkept > 1 ? strided_offset(ko, A.nkept - 1, A.ksize, A.kstride) : 0);
+  const int64_t per = (I.Rout + nchunks - 1) / nchunks;
+  w.ro_begin = (int64_t)chunk * per;
+  w.ro_end = w.ro_begin + per < I.Rout ? w.ro_begin + per : I.Rout;
+  return w;
+}
+__global__ __launch_bounds__(kRedBlock) void minmax_reduce_inner(const float *__restrict__ x,
+                                                                 MinMaxPartial *__restrict__ partial, MinMaxAxes A,
+                                                                 MinMaxInner I, int nchunks) {
+  __shared__ MinMaxPartial s_part[kRedBlock / 64][64];
+  const int64_t ko = blockIdx.x;
+  const int chunk = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tw = I.tw, rows_per_step = kRedBlock / tw;
+  const int cw = tid & (tw - 1), slot = tid / tw; // column inside the pass, row slot inside the step
+  const InnerWalk W = inner_walk(x, A, I, ko, chunk, nchunks);
+  for (int64_t w0 = 0; w0 < I.Wk; w0 += tw) {
+    const bool col_in = w0 + cw < I.Wk;
+    Extrema ex;
+    ex.init();
+    for (int64_t ro = W.ro_begin; ro < W.ro_end; ++ro) {
+      const float *row0 = W.base + (A.nred > 1 ? strided_offset(ro, A.nred - 1, A.rsize, A.rstride) : 0) + w0 + cw;
+      for (int64_t ri0 = 0; ri0 < I.Rin; ri0 += 8 * rows_per_step) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int64_t ri = ri0 + slot + j * rows_per_step;
+          v[j] = (col_in && ri < I.Rin) ? row0[ri * I.rin_stride] : __uint_as_float(0x7fc00000u); // NaN: ignored
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int64_t ri = ri0 + slot + j * rows_per_step;
+          ex.take(v[j], (uint32_t)(ro * I.Rin + ri));
+        }
+      }
+    }
+    // fold the row slots that share a column: across the lanes of a wavefront, then across the wavefronts
+    for (int off = 32; off >= tw; off >>= 1) {
+      const float a = __shfl_xor(ex.vmin, off), b = __shfl_xor(ex.vmax, off);
+      const uint32_t zi = __shfl_xor(ex.zidx, off), zs = __shfl_xor(ex.zsign, off);
+      ex.merge(a, b, zi, zs);
+    }
+    __syncthreads(); // the previous pass's partial results have been read
+    s_part[wave][lane] = ex.pack();
+    __syncthreads();
+    if (tid < tw && col_in) {
+      Extrema all;
+      all.init();
+      for (int w = 0; w < kRedBlock / 64; ++w)
+        all.merge(s_part[w][tid].vmin, s_part[w][tid].vmax, s_part[w][tid].zidx, s_part[w][tid].zsign);
+      partial[(ko * I.Wk + w0 + tid) * nchunks + chunk] = all.pack();
+    }
+  }
+}
+__global__ __launch_bounds__(kRedBlock) void minmax_apply_inner(const float *__restrict__ x, float *__restrict__ y,
+                                                                MinMaxAxes A, MinMaxInner I, int nchunks,
+                                                                const float4_t *__restrict__ params) {
+  const int64_t ko = blockIdx.x;
+  const int chunk = blockIdx.y, tid = threadIdx.x;
+  const int tw = I.tw, rows_per_step = kRedBlock / tw;
+  const int cw = tid & (tw - 1), slot = tid / tw;
+  const InnerWalk W = inner_walk(x, A, I, ko, chunk, nchunks);
+  for (int64_t w0 = 0; w0 < I.Wk; w0 += tw) {
+    const bool col_in = w0 + cw < I.Wk;
+    const float4_t pr = params[ko * I.Wk + (col_in ? w0 + cw : 0)];
+    for (int64_t ro = W.ro_begin; ro < W.ro_end; ++ro) {
+      const int64_t off = (W.base - x) + (A.nred > 1 ? strided_offset(ro, A.nred - 1, A.rsize, A.rstride) : 0) + w0 + cw;
+      for (int64_t ri0 = 0; ri0 < I.Rin; ri0 += 8 * rows_per_step) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int64_t ri = ri0 + slot + j * rows_per_step;
+          v[j] = (col_in && ri < I.Rin) ? x[off + ri * I.rin_stride] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int64_t ri = ri0 + slot + j * rows_per_step;
+          if (col_in && ri < I.Rin)
+            __builtin_nontemporal_store(minmax_apply(v[j], pr.x, pr.y, pr.z), y + off + ri * I.rin_stride);
+        }
+      }
+    }
+  }
+}
 // Element i of x (dense, row-major) belongs to the kept index formed by its coordinates along the kept axes.
 __global__ __launch_bounds__(kBlock) void minmax_apply_strided(const float *__restrict__ x, float *__restrict__ y,
                                                                int64_t total, MinMaxAxes A,
@@ -709,12 +850,16 @@ int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, in
     if (qshape[i] != 1 && qshape[i] != xshape[i])
       return fail(NBLA_HIP_ERR_VALUE,
                   "x.shape and ql_min.shape must be same except for i-th dimension where ql_min.shape[i] == 1.");
-  const MinMaxPlan P = make_plan(xshape, ndim, qshape);
+  MinMaxPlan P = make_plan(xshape, ndim, qshape);
   MinMaxAxes axes;
   if (!P.L.ok && !split_axes(xshape, ndim, qshape, axes))
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than eight kept or eight reduced axes of size above one.");
   if (P.L.total == 0)
     return NBLA_HIP_OK;
+  if (scratch_limit && P.inner && P.params_bytes + P.partial_bytes > scratch_limit) {
+    P.nchunks = 1; // the fixed scratch holds one partial result per range
+    P.partial_bytes = round_up((size_t)P.L.K * 16, 256);
+  }
   if (P.L.R0 * P.L.R1 > 0xffffffffll)
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "reduction slices above 2^32 elements are not supported.");
   if (scratch_limit && P.params_bytes + P.partial_bytes > scratch_limit)
@@ -737,6 +882,27 @@ int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, in
   if (!L.ok) { // kept axes separated by reduced ones: the strided kernels
     if (L.K > 0x7fffffffll)
       return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than 2^31 - 1 quantization ranges.");
+    const MinMaxInner inner = P.inner ? inner_form(axes) : MinMaxInner{false};
+    if (inner.ok) {
+      if (x_min_max) {
+        hipLaunchKernelGGL(minmax_reduce_inner, dim3((unsigned)inner.Ko, (unsigned)nchunks), dim3(kRedBlock), 0, stream,
+                           x, partial, axes, inner, nchunks);
+        NBLA_HIP_LAUNCH_CHECK("min_max_quantize reduction");
+      }
+      MinMaxScalars sc;
+      sc.decay = (float)decay;
+      sc.one_minus_decay = (float)(1.0 - (double)decay);
+      sc.eps = eps;
+      sc.x_min_max = x_min_max;
+      sc.ema = ema;
+      hipLaunchKernelGGL(minmax_finalize, dim3((unsigned)L.K), dim3(64), 0, stream, partial, nchunks, qr_min, qr_max,
+                         ql_min, ql_max, scale, params, sc);
+      NBLA_HIP_LAUNCH_CHECK("min_max_quantize finalize");
+      hipLaunchKernelGGL(minmax_apply_inner, dim3((unsigned)inner.Ko, (unsigned)nchunks), dim3(kRedBlock), 0, stream, x,
+                         y, axes, inner, nchunks, params);
+      NBLA_HIP_LAUNCH_CHECK("min_max_quantize apply");
+      return NBLA_HIP_OK;
+    }
     if (x_min_max) {
       hipLaunchKernelGGL(minmax_reduce_strided, dim3((unsigned)L.K), dim3(kRedBlock), 0, stream, x, partial, axes,
                          L.R1);

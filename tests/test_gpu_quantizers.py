@@ -227,6 +227,10 @@ MMQ_SHAPES = [
     # kept axes separated by reduced ones (the reference moves the reduced axes to the back, sum.cpp:44-75)
     ((5, 7, 9), (5, 1, 9)), ((3, 4, 5, 6), (1, 4, 1, 6)), ((3, 4, 5, 6), (3, 1, 5, 1)), ((2, 3, 1, 4, 5), (2, 1, 1, 4, 1)),
     ((6, 300, 7), (6, 1, 7)),
+    # the innermost axis kept with kept axes further out (lanes along it): more than 64 columns, several outer reduced
+    # axes, a long innermost reduced axis, and a slice of the benchmark's [64,256,56,56] with ranges [1,256,1,56]
+    ((4, 10, 100), (4, 1, 100)), ((3, 4, 5, 6, 7), (1, 4, 1, 1, 7)), ((2, 5, 300, 9), (1, 5, 1, 9)),
+    ((8, 16, 56, 56), (1, 16, 1, 56)), ((70, 3, 2), (1, 3, 1)), ((2, 3, 4, 2), (2, 1, 4, 2)),
 ]
 
 

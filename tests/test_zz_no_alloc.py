@@ -68,6 +68,14 @@ def test_static_scratch_per_channel_then_fewer_channels(dev):
     _check(dev, (2, 3, 4), (2, 3, 4), True, True, 320)
 
 
+def test_static_scratch_ranges_per_channel_and_column(dev):
+    """Ranges of shape (1, C, 1, W): the workspace entry splits the reduction of every range over several blocks; with
+    4096 ranges those partial results (2 MiB) do not fit the fixed scratch, and the allocation-free entry folds each
+    range in one block instead.  Same bits; then a small case of the same kind."""
+    _check(dev, (64, 64, 4, 64), (1, 64, 1, 64), True, True, 321)
+    _check(dev, (3, 4, 5, 6), (1, 4, 1, 6), True, False, 322)
+
+
 def test_static_scratch_rejects_what_does_not_fit(dev):
     """More quantization ranges than the fixed array holds: a clear error, nothing launched."""
     K = 8192 + 64
