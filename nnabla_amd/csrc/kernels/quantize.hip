@@ -749,53 +749,87 @@ __device__ __forceinline__ InnerWalk inner_walk(const float *x, const MinMaxAxes
   w.ro_end = w.ro_begin + per < I.Rout ? w.ro_begin + per : I.Rout;
   return w;
 }
+// kVec = 4: Wk a multiple of four and x (y) 16-byte aligned: a lane owns four consecutive columns (one 128-bit
+// access per row) and the plan's tw counts such quads.
+template <int kVec> struct InnerRow;
+template <> struct InnerRow<1> {
+  float v[1];
+  __device__ __forceinline__ void load(const float *p) { v[0] = *p; }
+  __device__ __forceinline__ void fill(float f) { v[0] = f; }
+};
+template <> struct InnerRow<4> {
+  float v[4];
+  __device__ __forceinline__ void load(const float *p) {
+    const float4_t q = *reinterpret_cast<const float4_t *>(p);
+    v[0] = q.x, v[1] = q.y, v[2] = q.z, v[3] = q.w;
+  }
+  __device__ __forceinline__ void fill(float f) { v[0] = v[1] = v[2] = v[3] = f; }
+};
+template <int kVec>
 __global__ __launch_bounds__(kRedBlock) void minmax_reduce_inner(const float *__restrict__ x,
                                                                  MinMaxPartial *__restrict__ partial, MinMaxAxes A,
                                                                  MinMaxInner I, int nchunks) {
-  __shared__ MinMaxPartial s_part[kRedBlock / 64][64];
+  __shared__ MinMaxPartial s_part[kRedBlock / 64][64][kVec];
   const int64_t ko = blockIdx.x;
   const int chunk = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tw = I.tw, rows_per_step = kRedBlock / tw;
-  const int cw = tid & (tw - 1), slot = tid / tw; // column inside the pass, row slot inside the step
+  const int cw = tid & (tw - 1), slot = tid / tw; // column (quad) inside the pass, row slot inside the step
   const InnerWalk W = inner_walk(x, A, I, ko, chunk, nchunks);
-  for (int64_t w0 = 0; w0 < I.Wk; w0 += tw) {
-    const bool col_in = w0 + cw < I.Wk;
-    Extrema ex;
-    ex.init();
-    for (int64_t ro = W.ro_begin; ro < W.ro_end; ++ro) {
-      const float *row0 = W.base + (A.nred > 1 ? strided_offset(ro, A.nred - 1, A.rsize, A.rstride) : 0) + w0 + cw;
-      for (int64_t ri0 = 0; ri0 < I.Rin; ri0 += 8 * rows_per_step) {
-        float v[8];
+  constexpr int kRows = kVec == 4 ? 4 : 8; // rows in flight per lane
+  for (int64_t w0 = 0; w0 < I.Wk; w0 += (int64_t)tw * kVec) {
+    const int64_t wcol = w0 + (int64_t)cw * kVec;
+    const bool col_in = wcol < I.Wk;
+    Extrema ex[kVec];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+    for (int c = 0; c < kVec; ++c)
+      ex[c].init();
+    for (int64_t ro = W.ro_begin; ro < W.ro_end; ++ro) {
+      const float *row0 = W.base + (A.nred > 1 ? strided_offset(ro, A.nred - 1, A.rsize, A.rstride) : 0) + wcol;
+      for (int64_t ri0 = 0; ri0 < I.Rin; ri0 += kRows * rows_per_step) {
+        InnerRow<kVec> v[kRows];
+#pragma unroll
+        for (int j = 0; j < kRows; ++j) {
           const int64_t ri = ri0 + slot + j * rows_per_step;
-          v[j] = (col_in && ri < I.Rin) ? row0[ri * I.rin_stride] : __uint_as_float(0x7fc00000u); // NaN: ignored
+          if (col_in && ri < I.Rin)
+            v[j].load(row0 + ri * I.rin_stride);
+          else
+            v[j].fill(__uint_as_float(0x7fc00000u)); // NaN: ignored by the scan
         }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < kRows; ++j) {
           const int64_t ri = ri0 + slot + j * rows_per_step;
-          ex.take(v[j], (uint32_t)(ro * I.Rin + ri));
+#pragma unroll
+          for (int c = 0; c < kVec; ++c)
+            ex[c].take(v[j].v[c], (uint32_t)(ro * I.Rin + ri));
         }
       }
     }
     // fold the row slots that share a column: across the lanes of a wavefront, then across the wavefronts
-    for (int off = 32; off >= tw; off >>= 1) {
-      const float a = __shfl_xor(ex.vmin, off), b = __shfl_xor(ex.vmax, off);
-      const uint32_t zi = __shfl_xor(ex.zidx, off), zs = __shfl_xor(ex.zsign, off);
-      ex.merge(a, b, zi, zs);
-    }
+#pragma unroll
+    for (int c = 0; c < kVec; ++c)
+      for (int off = 32; off >= tw; off >>= 1) {
+        const float a = __shfl_xor(ex[c].vmin, off), b = __shfl_xor(ex[c].vmax, off);
+        const uint32_t zi = __shfl_xor(ex[c].zidx, off), zs = __shfl_xor(ex[c].zsign, off);
+        ex[c].merge(a, b, zi, zs);
+      }
     __syncthreads(); // the previous pass's partial results have been read
-    s_part[wave][lane] = ex.pack();
+#pragma unroll
+    for (int c = 0; c < kVec; ++c)
+      s_part[wave][lane][c] = ex[c].pack();
     __syncthreads();
     if (tid < tw && col_in) {
-      Extrema all;
-      all.init();
-      for (int w = 0; w < kRedBlock / 64; ++w)
-        all.merge(s_part[w][tid].vmin, s_part[w][tid].vmax, s_part[w][tid].zidx, s_part[w][tid].zsign);
-      partial[(ko * I.Wk + w0 + tid) * nchunks + chunk] = all.pack();
+#pragma unroll
+      for (int c = 0; c < kVec; ++c) {
+        Extrema all;
+        all.init();
+        for (int w = 0; w < kRedBlock / 64; ++w)
+          all.merge(s_part[w][tid][c].vmin, s_part[w][tid][c].vmax, s_part[w][tid][c].zidx, s_part[w][tid][c].zsign);
+        partial[(ko * I.Wk + wcol + c) * nchunks + chunk] = all.pack();
+      }
     }
   }
 }
+template <int kVec>
 __global__ __launch_bounds__(kRedBlock) void minmax_apply_inner(const float *__restrict__ x, float *__restrict__ y,
                                                                 MinMaxAxes A, MinMaxInner I, int nchunks,
                                                                 const float4_t *__restrict__ params) {
@@ -804,23 +838,42 @@ __global__ __launch_bounds__(kRedBlock) void minmax_apply_inner(const float *__r
   const int tw = I.tw, rows_per_step = kRedBlock / tw;
   const int cw = tid & (tw - 1), slot = tid / tw;
   const InnerWalk W = inner_walk(x, A, I, ko, chunk, nchunks);
-  for (int64_t w0 = 0; w0 < I.Wk; w0 += tw) {
-    const bool col_in = w0 + cw < I.Wk;
-    const float4_t pr = params[ko * I.Wk + (col_in ? w0 + cw : 0)];
+  constexpr int kRows = kVec == 4 ? 4 : 8;
+  for (int64_t w0 = 0; w0 < I.Wk; w0 += (int64_t)tw * kVec) {
+    const int64_t wcol = w0 + (int64_t)cw * kVec;
+    const bool col_in = wcol < I.Wk;
+    float4_t pr[kVec];
+#pragma unroll
+    for (int c = 0; c < kVec; ++c)
+      pr[c] = params[ko * I.Wk + (col_in ? wcol + c : 0)];
     for (int64_t ro = W.ro_begin; ro < W.ro_end; ++ro) {
-      const int64_t off = (W.base - x) + (A.nred > 1 ? strided_offset(ro, A.nred - 1, A.rsize, A.rstride) : 0) + w0 + cw;
-      for (int64_t ri0 = 0; ri0 < I.Rin; ri0 += 8 * rows_per_step) {
-        float v[8];
+      const int64_t off = (W.base - x) + (A.nred > 1 ? strided_offset(ro, A.nred - 1, A.rsize, A.rstride) : 0) + wcol;
+      for (int64_t ri0 = 0; ri0 < I.Rin; ri0 += kRows * rows_per_step) {
+        InnerRow<kVec> v[kRows];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int64_t ri = ri0 + slot + j * rows_per_step;
-          v[j] = (col_in && ri < I.Rin) ? x[off + ri * I.rin_stride] : 0.0f;
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < kRows; ++j) {
           const int64_t ri = ri0 + slot + j * rows_per_step;
           if (col_in && ri < I.Rin)
-            __builtin_nontemporal_store(minmax_apply(v[j], pr.x, pr.y, pr.z), y + off + ri * I.rin_stride);
+            v[j].load(x + off + ri * I.rin_stride);
+          else
+            v[j].fill(0.0f);
+        }
+#pragma unroll
+        for (int j = 0; j < kRows; ++j) {
+          const int64_t ri = ri0 + slot + j * rows_per_step;
+          if (col_in && ri < I.Rin) {
+            float *dst = y + off + ri * I.rin_stride;
+            if (kVec == 4) {
+              float4_t r;
+              r.x = minmax_apply(v[j].v[0], pr[0].x, pr[0].y, pr[0].z);
+              r.y = minmax_apply(v[j].v[1 % kVec], pr[1 % kVec].x, pr[1 % kVec].y, pr[1 % kVec].z);
+              r.z = minmax_apply(v[j].v[2 % kVec], pr[2 % kVec].x, pr[2 % kVec].y, pr[2 % kVec].z);
+              r.w = minmax_apply(v[j].v[3 % kVec], pr[3 % kVec].x, pr[3 % kVec].y, pr[3 % kVec].z);
+              __builtin_nontemporal_store(r, reinterpret_cast<float4_t *>(dst));
+            } else {
+              __builtin_nontemporal_store(minmax_apply(v[j].v[0], pr[0].x, pr[0].y, pr[0].z), dst);
+            }
+          }
         }
       }
     }
@@ -882,11 +935,21 @@ int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, in
   if (!L.ok) { // kept axes separated by reduced ones: the strided kernels
     if (L.K > 0x7fffffffll)
       return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than 2^31 - 1 quantization ranges.");
-    const MinMaxInner inner = P.inner ? inner_form(axes) : MinMaxInner{false};
+    MinMaxInner inner = P.inner ? inner_form(axes) : MinMaxInner{false};
     if (inner.ok) {
+      // four columns per lane where the rows allow 128-bit accesses (every other stride is a multiple of Wk)
+      const bool quads = inner.Wk % 4 == 0 && aligned16(x) && aligned16(y);
+      if (quads) {
+        inner.tw = 1;
+        while (inner.tw < 64 && inner.tw * 4 < inner.Wk)
+          inner.tw *= 2;
+      }
+      const dim3 grid((unsigned)inner.Ko, (unsigned)nchunks);
       if (x_min_max) {
-        hipLaunchKernelGGL(minmax_reduce_inner, dim3((unsigned)inner.Ko, (unsigned)nchunks), dim3(kRedBlock), 0, stream,
-                           x, partial, axes, inner, nchunks);
+        if (quads)
+          hipLaunchKernelGGL(minmax_reduce_inner<4>, grid, dim3(kRedBlock), 0, stream, x, partial, axes, inner, nchunks);
+        else
+          hipLaunchKernelGGL(minmax_reduce_inner<1>, grid, dim3(kRedBlock), 0, stream, x, partial, axes, inner, nchunks);
         NBLA_HIP_LAUNCH_CHECK("min_max_quantize reduction");
       }
       MinMaxScalars sc;
@@ -898,8 +961,10 @@ int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, in
       hipLaunchKernelGGL(minmax_finalize, dim3((unsigned)L.K), dim3(64), 0, stream, partial, nchunks, qr_min, qr_max,
                          ql_min, ql_max, scale, params, sc);
       NBLA_HIP_LAUNCH_CHECK("min_max_quantize finalize");
-      hipLaunchKernelGGL(minmax_apply_inner, dim3((unsigned)inner.Ko, (unsigned)nchunks), dim3(kRedBlock), 0, stream, x,
-                         y, axes, inner, nchunks, params);
+      if (quads)
+        hipLaunchKernelGGL(minmax_apply_inner<4>, grid, dim3(kRedBlock), 0, stream, x, y, axes, inner, nchunks, params);
+      else
+        hipLaunchKernelGGL(minmax_apply_inner<1>, grid, dim3(kRedBlock), 0, stream, x, y, axes, inner, nchunks, params);
       NBLA_HIP_LAUNCH_CHECK("min_max_quantize apply");
       return NBLA_HIP_OK;
     }
