@@ -481,22 +481,29 @@ __global__ __launch_bounds__(kSlabThreads, 1) void binary_conv_slab_kernel(ConvS
   const int s_hi = (int)(rowsum >> 16), s_lo = (int)(rowsum & 0xffff);
   const int F = 2 * wn + wk;
   const bool negate = F == 7;
-  float *yrow = a.y + ((int64_t)n * g.O + (int64_t)a.grp * g.Og) * g.out_sp_size + p0 + r;
+  // channel of register q: c0 + 8 (q / 4) + q % 4; everything an output needs besides its accumulators is fetched
+  // before the stores (the compiler does not move a load across them)
+  const int c0 = F * 32 + 4 * half, og_left = (int)g.Og - wg * kWideGroup - c0; // channels from c0 to the group's last
+  const int osz = (int)g.out_sp_size;
+  float al[16], bi[16];
 #pragma unroll
   for (int q = 0; q < 16; ++q) {
-    const int cl = F * 32 + 8 * (q >> 2) + 4 * half + (q & 3); // channel inside the wide group
-    const int64_t ch = (int64_t)wg * kWideGroup + cl;
-    if (ch >= g.Og)
-      continue;
+    al[q] = s_alpha[c0 + 8 * (q >> 2) + (q & 3)];
+    bi[q] = s_bias[c0 + 8 * (q >> 2) + (q & 3)];
+  }
+  float *ybase = a.y + (((int64_t)n * g.O + (int64_t)a.grp * g.Og + (int64_t)wg * kWideGroup + c0) * g.out_sp_size + p0 + r);
+  const float bad_scale = rowbad ? __uint_as_float(0x7fc00000u) : 65536.0f; // NaN through the multiply-add
+#pragma unroll
+  for (int q = 0; q < 16; ++q) {
+    const int cq = 8 * (q >> 2) + (q & 3);
     const int hi = ((fin[0][q] >> F) << 8) + (fin[1][q] >> F), lo = ((fin[2][q] >> F) << 8) + (fin[3][q] >> F);
     int A = negate ? s_hi + 2 * hi : s_hi - 2 * hi, B = negate ? s_lo + 2 * lo : s_lo - 2 * lo;
     A += B >> 16, B &= 0xffff; // the sum is A * 2^16 + B, 0 <= B < 2^16
-    float v = ldexpf(fmaf((float)A, 65536.0f, (float)B), -shift);
-    if (rowbad)
-      v = __uint_as_float(0x7fc00000u);
-    v = v * s_alpha[cl];
-    v = v + s_bias[cl];
-    yrow[ch * g.out_sp_size] = v;
+    float v = ldexpf(fmaf((float)A, bad_scale, (float)B), -shift);
+    v = v * al[q];
+    v = v + bi[q];
+    if (cq < og_left)
+      ybase[cq * osz] = v; // (Og * out_sp_size < 2^31: checked by the host)
   }
 #endif
 }
@@ -621,7 +628,8 @@ int64_t slab_longest_run(const ConvGeom &g, int tile_rows, int tiles_per_sample)
 
 bool make_slab_plan(const ConvGeom &g, SlabPlan &p) {
   if (g.k_size > kSlabMaxTaps || g.Cg < 24 || g.in_sp_size >= ((int64_t)1 << 30) ||
-      g.out_sp_size >= ((int64_t)1 << 30) || g.Og >= ((int64_t)1 << 24))
+      g.out_sp_size >= ((int64_t)1 << 30) || g.Og >= ((int64_t)1 << 24) ||
+      (g.Og + kWideGroup) * g.out_sp_size >= ((int64_t)1 << 31))
     return false;
   const int64_t cgp = ceil_div(g.Cg, 32) * 32;
   // padded channels cost as much as real ones; the epilogue's 32-bit steps hold kChunkK terms
