@@ -503,7 +503,13 @@ int nbla_hip_prune_f32(const float *x, float *y, size_t size, float rate,
  * functions there become one scan and one update.  `m` is unused in modes 1, 3
  * and 4.  `decay` is the Python float of the reference: decay and 1 - decay
  * are each rounded to fp32 once, as its MulScalar functions do.  Their backward passes the gradient through: use
- * nbla_hip_fixed_point_quantize_backward_f32 with ste_fine_grained = 0. */
+ * nbla_hip_fixed_point_quantize_backward_f32 with ste_fine_grained = 0.
+ * The launch elects its last block through counters in one of 16 slots inside
+ * the library, handed out round-robin per process and put back to zero by that
+ * block: at most 16 recorder launches may be in flight at once on one device
+ * (on different streams; launches on one stream never overlap), and a launch
+ * that is torn down part-way (device reset) leaves its slot unusable until the
+ * library is loaded again. */
 size_t nbla_hip_range_recorder_workspace_bytes(void);
 int nbla_hip_range_recorder_f32(const float *x, float *y, size_t size, float *m,
                                 float *M, int mode, double decay, int training,
