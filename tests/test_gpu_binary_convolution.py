@@ -174,6 +174,32 @@ def test_config4_resnet_stage(dev):
     assert max_rel_err(to_np(y), full * a64) <= TIGHT
 
 
+@pytest.mark.parametrize("xs,ws,stride", [
+    ((4, 64, 56, 56), (64, 64, 3, 3), 1),      # rows of 56 outputs: a block's 32 windows cross rows; 64 of 256 channels
+    ((4, 128, 28, 28), (128, 128, 3, 3), 1),
+    ((4, 512, 7, 7), (512, 512, 3, 3), 1),     # two column groups, 16 channel tiles, tiles of four rows of the map
+    ((4, 64, 56, 56), (128, 64, 3, 3), 2),     # a strided stage transition
+    ((3, 256, 14, 14), (512, 256, 1, 1), 1),   # 1 x 1 kernel: one tap
+])
+def test_residual_network_stages_against_float64(dev, xs, ws, stride):
+    """The other stages of the network benchmark configuration 4 is taken from, a few samples each, against torch's
+    float64 convolution on the binarized weights."""
+    rng = np.random.default_rng(99)
+    x = rng.standard_normal(xs, dtype=np.float32)
+    W = rng.standard_normal(ws, dtype=np.float32) * np.float32(np.sqrt(2.0 / np.prod(ws[1:])))
+    b = rng.standard_normal(ws[0], dtype=np.float32)
+    pad = ws[2] // 2
+    y, Wb, alpha = kernels.binary_weight_convolution(_dev(x, dev), _dev(W, dev), _dev(b, dev), (pad, pad),
+                                                     (stride, stride), (1, 1))
+    s64 = torch.from_numpy(np.where(W < 0, -1.0, 1.0))
+    a64 = np.abs(W.astype(np.float64)).reshape(ws[0], -1).mean(1).reshape(1, -1, 1, 1)
+    full = torch.nn.functional.conv2d(torch.from_numpy(x).double(), s64, None, stride, pad).numpy()
+    ref = full * a64 + b.astype(np.float64).reshape(1, -1, 1, 1)
+    assert bits_equal(to_np(Wb), np.where(W < 0, -1.0, 1.0).astype(np.float32))
+    np.testing.assert_allclose(to_np(alpha).ravel(), a64.ravel(), rtol=2e-6)
+    assert max_rel_err(to_np(y), ref) <= TIGHT
+
+
 def test_convolution_argument_errors(dev):
     x = _dev(np.zeros((1, 4, 5, 5), np.float32), dev)
     with pytest.raises(kernels.KernelError) as ei:
