@@ -145,7 +145,7 @@ __global__ __launch_bounds__(256) void col2im_gather_unit(const float *__restric
 
 struct ConvBackwardPlan {
   size_t dyt_off, col_off, a_planes_off, b_planes_off, digits_off, bits_off, prep_off, count_off,
-      flag_off, sums_off, total;
+      flag_off, sums_off, slab_off, total;
 };
 
 size_t larger(size_t a, size_t b) { return a > b ? a : b; }
@@ -175,6 +175,12 @@ ConvBackwardPlan plan_conv_backward(const ConvGeom &g) {
   off += 256;
   p.sums_off = off;
   off += round_up(column_sums_workspace_bytes(g.M, g.Og), 256);
+  p.slab_off = off; // packed bits of the transposed convolution, when the input gradient takes that form
+  {
+    ConvGeom t;
+    if (conv_slab_transposed_geom(g, t))
+      off += round_up(conv_slab_prepared_bytes(t), 256);
+  }
   p.total = off;
   return p;
 }
@@ -227,13 +233,26 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
   uint32_t *bits = reinterpret_cast<uint32_t *>(base + p.bits_off);
   const bool representable = (zero_to == 1.0f || zero_to == -1.0f);
   const int64_t L = g.out_sp_size;
+  // The input gradient of a binary convolution of unit stride is itself a binary convolution (dy in the place of x,
+  // channels' roles exchanged, taps flipped): it takes the product that keeps input positions in LDS.
+  ConvGeom gt;
+  const bool dx_slab = dx && binary && representable && conv_slab_transposed_geom(g, gt);
   for (int64_t grp = 0; grp < g.group; ++grp) {
     const float *Wg = W + grp * g.Og * g.Kg;
     const float *ag = alpha ? alpha + grp * g.Og : nullptr;
-    rc = launch_gather_dy(dy, nullptr, dyt, g, grp, stream);
-    if (rc)
-      return rc;
-    if (dx) {
+    if (!dx_slab || dW || db) {
+      rc = launch_gather_dy(dy, nullptr, dyt, g, grp, stream);
+      if (rc)
+        return rc;
+    }
+    if (dx_slab) {
+      rc = launch_conv_slab_prepare_transposed(Wg, base + p.slab_off, g, zero_to, stream);
+      if (rc)
+        return rc;
+      rc = launch_conv_slab(dy, gt, grp, base + p.slab_off, nullptr, nullptr, nullptr, dx, stream, ag, accum_x);
+      if (rc)
+        return rc;
+    } else if (dx) {
       if (binary) {
         // Sign(W_g) packed for the contraction over o: W_g is stored [Og, Kg] = [contraction][column]
         rc = nbla_hip_binarize_weights_f32(Wg, nullptr, nullptr, bits, g.Og, g.Kg, 0, zero_to,

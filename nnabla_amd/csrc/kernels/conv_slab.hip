@@ -74,7 +74,9 @@ struct ConvSlabArgs {
   float *alpha_out;   // may be null
   int *zero_count;    // may be null
   const float *bias;
+  const float *in_scale; // may be null: input channel c of the group is multiplied by in_scale[c] first
   float *y;
+  int accumulate;        // add to y instead of overwriting it
   ConvGeom g;
   int grp;
   float inv_k;
@@ -169,6 +171,11 @@ __global__ __launch_bounds__(kSlabThreads, 1) void binary_conv_slab_kernel(ConvS
 #pragma unroll
     for (int c = 0; c < 16; ++c)
       v[c] = (item < items && ch0 + c < Cg) ? src[(int64_t)(ch0 + c) * plane] : 0.0f;
+    if (a.in_scale) { // one rounded product per element, before anything else
+#pragma unroll
+      for (int c = 0; c < 16; ++c)
+        v[c] = v[c] * ((item < items && ch0 + c < Cg) ? a.in_scale[ch0 + c] : 0.0f);
+    }
   };
   uint32_t amax = 0u;
   auto scan_item = [&](const float (&v)[16]) __attribute__((always_inline)) {
@@ -492,6 +499,14 @@ __global__ __launch_bounds__(kSlabThreads, 1) void binary_conv_slab_kernel(ConvS
     bi[q] = s_bias[c0 + 8 * (q >> 2) + (q & 3)];
   }
   float *ybase = a.y + (((int64_t)n * g.O + (int64_t)a.grp * g.Og + (int64_t)wg * kWideGroup + c0) * g.out_sp_size + p0 + r);
+  float prev[16];
+  if (a.accumulate) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const int cq = 8 * (q >> 2) + (q & 3);
+      prev[q] = cq < og_left ? ybase[cq * osz] : 0.0f;
+    }
+  }
   const float bad_scale = rowbad ? __uint_as_float(0x7fc00000u) : 65536.0f; // NaN through the multiply-add
 #pragma unroll
   for (int q = 0; q < 16; ++q) {
@@ -500,6 +515,8 @@ __global__ __launch_bounds__(kSlabThreads, 1) void binary_conv_slab_kernel(ConvS
     int A = negate ? s_hi + 2 * hi : s_hi - 2 * hi, B = negate ? s_lo + 2 * lo : s_lo - 2 * lo;
     A += B >> 16, B &= 0xffff; // the sum is A * 2^16 + B, 0 <= B < 2^16
     float v = ldexpf(fmaf((float)A, bad_scale, (float)B), -shift);
+    if (a.accumulate)
+      v = prev[q] + v;
     v = v * al[q];
     v = v + bi[q];
     if (cq < og_left)
@@ -584,6 +601,49 @@ __global__ __launch_bounds__(kPrepThreads) void conv_taps_prepare(const float *_
     zeros[(ct * wide_groups + wg) * 32 + r] = s_zero[0] + s_zero[1] + s_zero[2] + s_zero[3];
   // the packed words of lanes r and r + 32 of the block's k tiles (tap, ct): word i, byte c, bit F <- row F, channel
   // c0 + 16 half + 4 i + c
+  for (int item = tid; item < 2 * taps; item += kPrepThreads) {
+    const int t = item >> 1, g16 = item & 1;
+    uint32_t o[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int f = 0; f < 8; ++f) {
+      const unsigned char *src = s_neg + f * seg_full + (g16 * 16) * taps + t;
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        o[j >> 2] |= (uint32_t)src[j * taps] << (8 * (j & 3) + f);
+    }
+    uint4_t v;
+    v.x = o[0], v.y = o[1], v.z = o[2], v.w = o[3];
+    bits[((int64_t)(t * ct_count + ct) * wide_groups + wg) * 64 + g16 * 32 + r] = v;
+  }
+}
+
+// The packed bits of the same product run backwards, for the gradient with respect to the input of a convolution of
+// unit stride: dx = conv(dy, W') with W'[c][o][t] = Sign(W)[o][c][taps - 1 - t] and the padding (k - 1) dil - pad
+// (convolution.cpp:199-283 unfolds dy . W^T and folds it back; here the fold is the contraction over the taps).
+// Block (wide group of input channels c, tile of 32 output channels o, r) as in conv_taps_prepare; only the bits are
+// written.
+__global__ __launch_bounds__(kPrepThreads) void conv_taps_prepare_transposed(const float *__restrict__ W,
+                                                                             uint4_t *__restrict__ bits, int Og, int Cg,
+                                                                             int taps, int ct_count, int wide_groups,
+                                                                             float zero_to) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int seg_full = 32 * taps;
+  unsigned char *s_neg = smem; // [8 rows c][32 channels o][tap, flipped]
+  const int tid = threadIdx.x;
+  const int wg = blockIdx.x / 32, r = blockIdx.x % 32, ct = blockIdx.y;
+  const int o0 = ct * 32;
+  for (int idx = tid; idx < 8 * seg_full; idx += kPrepThreads) {
+    const int f = idx / seg_full, rem = idx - f * seg_full, ol = rem / taps, t = rem - ol * taps;
+    const int c = wg * kWideGroup + 32 * f + r, o = o0 + ol;
+    unsigned char neg = 0;
+    if (c < Cg && o < Og) {
+      const float w = W[((int64_t)o * Cg + c) * taps + t];
+      const bool is_zero = !(w > 0.0f) && !(w < 0.0f);
+      neg = ((w < 0.0f) || (is_zero && zero_to < 0.0f)) ? 1 : 0;
+    }
+    s_neg[f * seg_full + ol * taps + (taps - 1 - t)] = neg;
+  }
+  __syncthreads();
   for (int item = tid; item < 2 * taps; item += kPrepThreads) {
     const int t = item >> 1, g16 = item & 1;
     uint32_t o[4] = {0u, 0u, 0u, 0u};
@@ -713,8 +773,53 @@ int launch_conv_slab_prepare(const float *Wg, float *Wbg, void *prepared, const 
   return NBLA_HIP_OK;
 }
 
+// The convolution that computes the input gradient of `g` (unit stride): dy takes the place of x, the roles of the
+// channels are exchanged, the padding becomes (k - 1) dil - pad.  False when `g` has a stride or needs a negative
+// padding, or when the slab product does not cover the result.
+bool conv_slab_transposed_geom(const ConvGeom &g, ConvGeom &t) {
+  t = g;
+  for (int i = 0; i < kMaxSpatial; ++i) {
+    if (g.stride[i] != 1)
+      return false;
+    t.pad[i] = (g.k[i] - 1) * g.dil[i] - g.pad[i];
+    if (t.pad[i] < 0)
+      return false;
+    t.in_sp[i] = g.out_sp[i];
+    t.out_sp[i] = g.in_sp[i];
+  }
+  t.C = g.O, t.O = g.C, t.Cg = g.Og, t.Og = g.Cg;
+  t.in_sp_size = g.out_sp_size, t.out_sp_size = g.in_sp_size;
+  t.Kg = t.Cg * g.k_size;
+  t.M = g.outer * t.out_sp_size;
+  SlabPlan p;
+  return make_slab_plan(t, p);
+}
+
+int launch_conv_slab_prepare_transposed(const float *Wg, void *prepared, const ConvGeom &g, float zero_to,
+                                        hipStream_t stream) {
+  ConvGeom t;
+  SlabPlan p;
+  if (!conv_slab_transposed_geom(g, t) || !make_slab_plan(t, p))
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "the slab convolution does not cover this input gradient.");
+  if (!aligned16(prepared))
+    return fail(NBLA_HIP_ERR_MEMORY, "prepared-weight buffer must be 16-byte aligned.");
+  const size_t lds = (size_t)8 * 32 * g.k_size;
+  static std::atomic<uint64_t> configured{0};
+  const int rc = allow_dynamic_lds(reinterpret_cast<const void *>(conv_taps_prepare_transposed),
+                                   8 * 32 * kSlabMaxTaps, configured,
+                                   "hipFuncSetAttribute(conv_taps_prepare_transposed LDS size)");
+  if (rc)
+    return rc;
+  hipLaunchKernelGGL(conv_taps_prepare_transposed, dim3((unsigned)p.wide_groups * 32, (unsigned)p.ct),
+                     dim3(kPrepThreads), lds, stream, Wg, static_cast<uint4_t *>(prepared), (int)g.Og, (int)g.Cg,
+                     (int)g.k_size, p.ct, p.wide_groups, zero_to);
+  NBLA_HIP_LAUNCH_CHECK("conv_taps_prepare_transposed");
+  return NBLA_HIP_OK;
+}
+
 int launch_conv_slab(const float *x, const ConvGeom &g, int64_t grp, const void *prepared, float *alpha_out,
-                     int *zero_count, const float *bias, float *y, hipStream_t stream) {
+                     int *zero_count, const float *bias, float *y, hipStream_t stream, const float *in_scale,
+                     bool accumulate) {
   ConvSlabArgs a;
   if (!make_slab_plan(g, a.p))
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "the slab convolution does not cover this geometry.");
@@ -736,6 +841,8 @@ int launch_conv_slab(const float *x, const ConvGeom &g, int64_t grp, const void 
   a.alpha_out = alpha_out;
   a.zero_count = zero_count;
   a.bias = bias;
+  a.in_scale = in_scale;
+  a.accumulate = accumulate ? 1 : 0;
   a.y = y;
   a.g = g;
   a.grp = (int)grp;

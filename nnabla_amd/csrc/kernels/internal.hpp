@@ -45,8 +45,18 @@ bool conv_slab_applies(const ConvGeom &g);
 size_t conv_slab_prepared_bytes(const ConvGeom &g);
 int launch_conv_slab_prepare(const float *Wg, float *Wbg, void *prepared, const ConvGeom &g, float zero_to,
                              hipStream_t stream);
+// in_scale (may be null): input channel c of the group is multiplied by in_scale[c] before anything else; accumulate:
+// y += instead of y =.
 int launch_conv_slab(const float *x, const ConvGeom &g, int64_t grp, const void *prepared, float *alpha_out,
-                     int *zero_count, const float *bias, float *y, hipStream_t stream);
+                     int *zero_count, const float *bias, float *y, hipStream_t stream, const float *in_scale = nullptr,
+                     bool accumulate = false);
+// The same product as the input gradient of a binary convolution of unit stride: conv_slab_transposed_geom gives the
+// geometry of the convolution dx = conv(dy * alpha, flipped Sign(W)^T) (false when the product does not cover it),
+// launch_conv_slab_prepare_transposed writes its packed bits from the group's weights [Og, Cg, taps]
+// (conv_slab_prepared_bytes of the transposed geometry), launch_conv_slab runs it with dy as x and alpha as in_scale.
+bool conv_slab_transposed_geom(const ConvGeom &g, ConvGeom &t);
+int launch_conv_slab_prepare_transposed(const float *Wg, void *prepared, const ConvGeom &g, float zero_to,
+                                        hipStream_t stream);
 // Digit operand of the rows of x (nbla_hip_split_digits_scaled_f32) for a caller that holds materialised weights
 // Wb [K, N] (* alpha[n], + bias[n]): rows holding a NaN or an infinity get their outputs y[m, :] computed by the
 // splitting kernel itself, as fp32 dot products in the reference's order.  *redone tells whether that happened (only

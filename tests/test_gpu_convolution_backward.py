@@ -22,6 +22,15 @@ CASES = [
     ((2, 6, 5, 5), (6, 1, 3, 3), (1, 1), (1, 1), (1, 1), 6),
     ((4, 8, 16, 16), (16, 8, 3, 3), (1, 1), (1, 1), (1, 1), 1),
     ((3, 64, 14, 14), (96, 32, 3, 3), (1, 1), (1, 1), (1, 1), 2),
+    # unit stride and 24 output channels per group or more: the input gradient of the binary layers runs as a binary
+    # convolution of dy (channels' roles exchanged, taps flipped, padding (k - 1) dil - pad).  32 channels exactly;
+    # dilation with no padding; one and three spatial dimensions; a padding larger than the kernel (the flipped
+    # convolution would need a negative one: the unfolded form runs)
+    ((2, 8, 9, 9), (32, 8, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((2, 8, 10, 9), (40, 8, 3, 2), (0, 1), (1, 1), (2, 1), 1),
+    ((3, 4, 30), (32, 4, 5), (2,), (1,), (1,), 1),
+    ((1, 3, 4, 5, 6), (32, 3, 2, 3, 2), (1, 0, 1), (1, 1, 1), (1, 1, 2), 1),
+    ((2, 4, 6, 6), (32, 4, 2, 2), (3, 3), (1, 1), (1, 1), 1),
 ]
 
 
@@ -92,6 +101,25 @@ def test_convolution_backward_accumulates_and_skips(dev):
                                                want=(True, False, False))
     assert only[1] is None and only[2] is None
     first = oracle.binary_convolution_backward(dy, x, W, alpha, pad, stride, dil, group, 1.0)[0]
+    assert max_rel_err(to_np(only[0]), first) <= TIGHT
+
+
+def test_input_gradient_as_a_convolution_accumulates(dev):
+    """The same with 32 output channels per group and unit stride (the input gradient as a binary convolution of dy):
+    accumulation into dx, and dx alone."""
+    xs, ws, pad, stride, dil, group = (3, 6, 8, 9), (64, 3, 3, 2), (1, 1), (1, 1), (1, 1), 2
+    x, W, dy = _data(xs, ws, pad, stride, dil, group, 45)
+    alpha = np.abs(W).reshape(ws[0], -1).mean(1).astype(np.float32)
+    odx = np.random.RandomState(6).randn(*xs).astype(np.float32)
+    rdx, _, _ = oracle.binary_convolution_backward(dy, x, W, alpha, pad, stride, dil, group, 1.0, dx=odx)
+    d = lambda a: _dev(a, dev)
+    gdx, gdw, gdb = kernels.binary_convolution_backward(d(dy), d(x), d(W), None, d(alpha), pad, stride, dil, group, 1.0,
+                                                        dx=d(odx), want=(True, False, False))
+    assert gdw is None and gdb is None
+    assert max_rel_err(to_np(gdx), rdx) <= TIGHT
+    first = oracle.binary_convolution_backward(dy, x, W, None, pad, stride, dil, group, 1.0)[0]
+    only = kernels.binary_convolution_backward(d(dy), d(x), d(W), None, None, pad, stride, dil, group, 1.0,
+                                               want=(True, False, False))
     assert max_rel_err(to_np(only[0]), first) <= TIGHT
 
 
