@@ -686,7 +686,47 @@ int64_t slab_longest_run(const ConvGeom &g, int tile_rows, int tiles_per_sample)
   return longest;
 }
 
+bool compute_slab_plan(const ConvGeom &g, SlabPlan &p);
+
+// The plan of a geometry is asked for several times per call (does it apply, how much workspace, the launches) and
+// sizing the slab walks the tiles of a sample: the last few answers are kept per thread.
 bool make_slab_plan(const ConvGeom &g, SlabPlan &p) {
+  struct Key {
+    int64_t outer, C, O, group;
+    int in_sp[kMaxSpatial], k[kMaxSpatial], pad[kMaxSpatial], stride[kMaxSpatial], dil[kMaxSpatial];
+    bool operator==(const Key &o) const {
+      bool same = outer == o.outer && C == o.C && O == o.O && group == o.group;
+      for (int i = 0; i < kMaxSpatial; ++i)
+        same = same && in_sp[i] == o.in_sp[i] && k[i] == o.k[i] && pad[i] == o.pad[i] && stride[i] == o.stride[i] &&
+               dil[i] == o.dil[i];
+      return same;
+    }
+  };
+  constexpr int kKept = 4; // a forward and a backward geometry alternate in training
+  static thread_local bool have[kKept] = {false, false, false, false}, kept_ok[kKept];
+  static thread_local Key kept_key[kKept];
+  static thread_local SlabPlan kept_plan[kKept];
+  static thread_local int next = 0;
+  Key key;
+  key.outer = g.outer, key.C = g.C, key.O = g.O, key.group = g.group;
+  for (int i = 0; i < kMaxSpatial; ++i)
+    key.in_sp[i] = g.in_sp[i], key.k[i] = g.k[i], key.pad[i] = g.pad[i], key.stride[i] = g.stride[i],
+    key.dil[i] = g.dil[i];
+  for (int e = 0; e < kKept; ++e)
+    if (have[e] && key == kept_key[e]) {
+      p = kept_plan[e];
+      return kept_ok[e];
+    }
+  const int e = next;
+  next = (next + 1) % kKept;
+  kept_ok[e] = compute_slab_plan(g, kept_plan[e]);
+  kept_key[e] = key;
+  have[e] = true;
+  p = kept_plan[e];
+  return kept_ok[e];
+}
+
+bool compute_slab_plan(const ConvGeom &g, SlabPlan &p) {
   if (g.k_size > kSlabMaxTaps || g.Cg < 24 || g.in_sp_size >= ((int64_t)1 << 30) ||
       g.out_sp_size >= ((int64_t)1 << 30) || g.Og >= ((int64_t)1 << 24) ||
       (g.Og + kWideGroup) * g.out_sp_size >= ((int64_t)1 << 31))
@@ -703,7 +743,7 @@ bool make_slab_plan(const ConvGeom &g, SlabPlan &p) {
     p.tile_rows = (int)ceil_div(g.out_sp_size, ceil_div(g.out_sp_size, kSlabRows));
   }
   const int64_t tiles = ceil_div(g.out_sp_size, p.tile_rows);
-  if (tiles > 65536) // the host walks them to size the slab
+  if (tiles > 16384) // the host walks them to size the slab
     return false;
   p.tiles_per_sample = (int)tiles;
   p.wide_groups = (int)bits_wide_groups(g.Og);
