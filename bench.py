@@ -62,6 +62,25 @@ def profiled_traffic():
                                                                          float(m.group(2)) / 1e6, m.group(3)))
 
 
+def bench_mfma_rates(dev):
+    """What the matrix pipes sustain on kernels of nothing but independent matrix instructions with non-zero operands
+    (two blocks of four wavefronts per CU, about a millisecond per launch so that the clocks settle under the power
+    limit): the int8 instruction of the products, and the fp6 x fp4 / fp8 x fp8 forms of the scaled instruction.  An
+    exact fp32-faithful product on fp6 digits would need five balanced base-32 digits where int8 needs three base-256
+    ones, so fp6 x fp4 has to issue more than 5/3 as many operations per second as int8 to pay."""
+    import torch
+    from nnabla_amd import kernels as k
+    sink = torch.zeros(64, device=dev)
+    out = {}
+    for kind, rounds in (("i8", 4000), ("fp6 x fp4", 4000), ("fp8 x fp8", 4000)):
+        n, ops = k.mfma_rate_probe(kind, rounds, sink)
+        ms = time_kernel(lambda: k.mfma_rate_probe(kind, rounds, sink), 10)
+        out[kind] = {"ms": ms, "instructions": n, "ops_per_instruction": ops, "POPs": n * ops / ms / 1e12}
+    out["fp6 x fp4 over i8"] = out["fp6 x fp4"]["POPs"] / out["i8"]["POPs"]
+    out["needed for five fp6 digits against three int8 digits"] = 5.0 / 3.0
+    return out
+
+
 def _events(n):
     import torch
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
@@ -388,11 +407,12 @@ def main():
                     help="untimed steps; the first few dozen launches after idle run at ramping clocks")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=2048)
-    ap.add_argument("--section", choices=("all", "headline", "sweep", "quantizers", "other"), default="all",
+    ap.add_argument("--section", choices=("all", "headline", "sweep", "quantizers", "other", "mfma"), default="all",
                     help="headline: only the timed BinaryWeightAffine steps (what the rocprofv3 summaries profile); "
                          "sweep: headline plus the forward at M = 1 .. 1024 and BinaryConnectAffine (`sweep`); "
                          "quantizers: headline plus the quantizer kernels; other: headline plus the convolution, INQ, "
-                         "MLP, backward and adjacent-function workloads (`other_configs`)")
+                         "MLP, backward and adjacent-function workloads (`other_configs`); mfma: headline plus the rates "
+                         "of kernels of nothing but matrix instructions (`mfma_rates`)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
@@ -429,6 +449,7 @@ def main():
                                                                     connect=True)
     quant = bench_quantizers(dev, max(10, args.steps)) if args.section in ("all", "quantizers") else {}
     other = bench_other_configs(dev, max(5, args.steps // 2)) if args.section in ("all", "other") else {}
+    mfma = bench_mfma_rates(dev) if args.section in ("all", "mfma") else {}
     r = bench_binary_weight_affine(M, K, N, args.steps, args.warmup, dev)
     tflops = r["flop"] / (r["ms_per_step"] * 1e-3) / 1e12
     gemm_tflops = r["flop"] / (r["gemm_ms"] * 1e-3) / 1e12
@@ -450,6 +471,7 @@ def main():
                               "step_with_events": r["ms_per_step_with_events"],
                               "note": "an instrumented repeat of the timed steps, four event records per step; "
                                       "roofline.kernel_ms is its product share"},
+        "mfma_rates": mfma,
         "sweep": sweep,
         "quantizers": quant,
         "other_configs": other,

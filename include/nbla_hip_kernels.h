@@ -516,6 +516,18 @@ int nbla_hip_range_recorder_f32(const float *x, float *y, size_t size, float *m,
                                 void *workspace, size_t workspace_bytes,
                                 void *stream);
 
+/* Measurement utility; no counterpart in the reference.  Launches a kernel of
+ * nothing but independent matrix instructions on non-zero operands (two blocks
+ * of four wavefronts per CU, `rounds` x 8 instructions per wavefront) so that
+ * bench.py can time what the matrix pipes sustain under the part's power limit:
+ * kind 0 = v_mfma_i32_32x32x32_i8, 1 = v_mfma_scale_f32_32x32x64_f8f6f4 with
+ * fp6 x fp4 operands, 2 = the same with fp8 x fp8.  Writes the number of
+ * instructions issued and the operations each one stands for; `sink` is a
+ * device word that is never written. */
+int nbla_hip_mfma_rate_probe(int kind, int rounds, int64_t *instructions,
+                             int64_t *ops_per_instruction, float *sink,
+                             void *stream);
+
 /* ---------------------------------------------------------------------- INQ */
 
 /* INQ step selector (what the forward does to the indicators before quantizing):

@@ -45,7 +45,7 @@ EXPORTED = (
     "nbla_hip_memcpy", "nbla_hip_device_synchronize", "nbla_hip_stream_synchronize", "nbla_hip_fill",
     "nbla_hip_cast", "nbla_hip_relu_f32", "nbla_hip_relu_backward_f32", "nbla_hip_add2_f32",
     "nbla_hip_add2_backward_f32", "nbla_hip_binary2_f32", "nbla_hip_binary2_backward_f32", "nbla_hip_copy_rows_f32",
-    "nbla_hip_broadcast2_f32", "nbla_hip_broadcast2_backward_f32",
+    "nbla_hip_broadcast2_f32", "nbla_hip_broadcast2_backward_f32", "nbla_hip_mfma_rate_probe",
 )
 
 
@@ -570,3 +570,15 @@ def inq_convolution(x, W, I, old_W, old_I, bias=None, pad=None, stride=None, dil
                                              int(num_bits), int(step), cb, None, _p(ws), ctypes.c_size_t(ws.numel()),
                                              _stream(stream)))
     return y
+
+
+MFMA_PROBE_KINDS = {"i8": 0, "fp6 x fp4": 1, "fp8 x fp8": 2}
+
+
+def mfma_rate_probe(kind, rounds, sink, stream=None):
+    """Launches the matrix-instruction rate probe (measurement utility of bench.py); returns (instructions issued,
+    operations per instruction).  `sink`: a float tensor on the device (never written)."""
+    n, ops = ctypes.c_int64(0), ctypes.c_int64(0)
+    check(lib().nbla_hip_mfma_rate_probe(ctypes.c_int(MFMA_PROBE_KINDS[kind]), ctypes.c_int(int(rounds)),
+                                         ctypes.byref(n), ctypes.byref(ops), _p(sink), _stream(stream)))
+    return n.value, ops.value
