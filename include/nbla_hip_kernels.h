@@ -353,6 +353,18 @@ size_t nbla_hip_binary_convolution_workspace_bytes(
     const int64_t *kernel, const int64_t *pad, const int64_t *stride,
     const int64_t *dilation, int64_t group, float quantize_zero_to);
 
+/* Which form the binary convolutions' forward takes for a geometry, decided on
+ * the host from the shapes alone (no counterpart in nnabla, whose one
+ * forward_impl serves every geometry; for tests and for callers that want to
+ * know).  plan[0] = output positions per block of the form that keeps the input
+ * positions under a block in LDS (0: the geometry takes the gathering product),
+ * plan[1] = blocks per sample, plan[2] = input positions the LDS of a block
+ * holds, plan[3] = LDS bytes per block.  Touches no device. */
+int nbla_hip_binary_convolution_slab_plan(
+    int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
+    const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+    const int64_t *dilation, int64_t group, int32_t *plan);
+
 /* BinaryWeightConvolution forward, channel-first, nd = 1..3 spatial dimensions:
  *   x [outer, C, in_sp...], W [O, C/group, kernel...] -> Wb (same shape as W),
  *   alpha [O], y [outer, O, out_sp...]; bias [O] may be NULL.

@@ -849,6 +849,20 @@ size_t nbla_hip_binary_convolution_workspace_bytes(int64_t outer, int64_t C, int
   return plan_conv(g).total + (representable ? 0 : round_up((size_t)g.M * g.Kg * sizeof(float), 256));
 }
 
+int nbla_hip_binary_convolution_slab_plan(int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
+                                          const int64_t *kernel, const int64_t *pad, const int64_t *stride,
+                                          const int64_t *dilation, int64_t group, int32_t *plan) {
+  if (!plan)
+    return fail(NBLA_HIP_ERR_VALUE, "slab plan: no output array.");
+  ConvGeom g;
+  const int rc = make_geom(g, outer, C, nd, in_sp, O, kernel, pad, stride, dilation, group);
+  if (rc)
+    return rc;
+  plan[0] = plan[1] = plan[2] = plan[3] = 0;
+  conv_slab_plan_summary(g, plan);
+  return NBLA_HIP_OK;
+}
+
 int nbla_hip_binary_weight_convolution_f32(const float *x, const float *W, float *Wb, float *alpha, const float *bias,
                                            float *y, int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
                                            const int64_t *kernel, const int64_t *pad, const int64_t *stride,

@@ -786,6 +786,14 @@ bool conv_slab_applies(const ConvGeom &g) {
   return make_slab_plan(g, p);
 }
 
+bool conv_slab_plan_summary(const ConvGeom &g, int32_t out[4]) {
+  SlabPlan p;
+  if (!make_slab_plan(g, p))
+    return false;
+  out[0] = p.tile_rows, out[1] = p.tiles_per_sample, out[2] = p.cap, out[3] = p.total;
+  return true;
+}
+
 size_t conv_slab_prepared_bytes(const ConvGeom &g) {
   SlabPlan p;
   return make_slab_plan(g, p) ? p.prep_bytes : 0;

@@ -43,6 +43,9 @@ int launch_gemm_bits_unfold(const float *x, const ConvGeom &g, int64_t grp, cons
 // positive to *zero_count when that is not null.  alpha_out and bias belong to the group; y is the whole output.
 bool conv_slab_applies(const ConvGeom &g);
 size_t conv_slab_prepared_bytes(const ConvGeom &g);
+// The plan's figures for a geometry it covers: windows per block, blocks per sample, the input positions its LDS
+// holds per block, LDS bytes.  Host only.
+bool conv_slab_plan_summary(const ConvGeom &g, int32_t out[4]);
 int launch_conv_slab_prepare(const float *Wg, float *Wbg, void *prepared, const ConvGeom &g, float zero_to,
                              hipStream_t stream);
 // in_scale (may be null): input channel c of the group is multiplied by in_scale[c] before anything else; accumulate:

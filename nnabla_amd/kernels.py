@@ -45,7 +45,7 @@ EXPORTED = (
     "nbla_hip_memcpy", "nbla_hip_device_synchronize", "nbla_hip_stream_synchronize", "nbla_hip_fill",
     "nbla_hip_cast", "nbla_hip_relu_f32", "nbla_hip_relu_backward_f32", "nbla_hip_add2_f32",
     "nbla_hip_add2_backward_f32", "nbla_hip_binary2_f32", "nbla_hip_binary2_backward_f32", "nbla_hip_copy_rows_f32",
-    "nbla_hip_broadcast2_f32", "nbla_hip_broadcast2_backward_f32", "nbla_hip_mfma_rate_probe",
+    "nbla_hip_broadcast2_f32", "nbla_hip_broadcast2_backward_f32", "nbla_hip_mfma_rate_probe", "nbla_hip_binary_convolution_slab_plan",
 )
 
 
@@ -411,6 +411,19 @@ def binary_weight_convolution(x, W, bias=None, pad=None, stride=None, dilation=N
     check(lib().nbla_hip_binary_weight_convolution_f32(_p(x), _p(W), _p(Wb), _p(alpha), _p(bias), _p(y), *geom, q0,
                                                        _p(ws), ctypes.c_size_t(ws.numel()), _stream(stream)))
     return y, Wb, alpha
+
+
+def binary_convolution_slab_plan(outer, C, in_sp, O, kernel, pad, stride, dilation, group=1):
+    """The host's plan for a binary convolution that keeps a block's input positions in LDS: a dict with the output
+    positions per block, blocks per sample, input positions held and LDS bytes, or None where the geometry takes
+    the gathering product.  Shapes only; touches no device."""
+    plan = (ctypes.c_int32 * 4)()
+    check(lib().nbla_hip_binary_convolution_slab_plan(
+        _i64(outer), _i64(C), ctypes.c_int(len(in_sp)), _shape(in_sp), _i64(O), _shape(kernel), _shape(pad),
+        _shape(stride), _shape(dilation), _i64(group), plan))
+    if plan[0] == 0:
+        return None
+    return {"tile_rows": plan[0], "tiles_per_sample": plan[1], "cap": plan[2], "lds_bytes": plan[3]}
 
 
 def binary_connect_convolution(x, W, bias=None, pad=None, stride=None, dilation=None, group=1, quantize_zero_to=1.0,
