@@ -72,7 +72,8 @@ def bench_mfma_rates(dev):
     from nnabla_amd import kernels as k
     sink = torch.zeros(64, device=dev)
     out = {}
-    for kind, rounds in (("i8", 4000), ("fp6 x fp4", 4000), ("fp8 x fp8", 4000)):
+    for kind, rounds in (("i8", 4000), ("fp6 x fp4", 4000), ("fp8 x fp8", 4000), ("i8, operands change", 4000),
+                         ("i8, digits x bit bytes, operands change", 4000)):
         n, ops = k.mfma_rate_probe(kind, rounds, sink)
         ms = time_kernel(lambda: k.mfma_rate_probe(kind, rounds, sink), 10)
         out[kind] = {"ms": ms, "instructions": n, "ops_per_instruction": ops, "POPs": n * ops / ms / 1e12}

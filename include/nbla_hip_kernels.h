@@ -533,8 +533,10 @@ int nbla_hip_range_recorder_f32(const float *x, float *y, size_t size, float *m,
  * of four wavefronts per CU, `rounds` x 8 instructions per wavefront) so that
  * bench.py can time what the matrix pipes sustain under the part's power limit:
  * kind 0 = v_mfma_i32_32x32x32_i8, 1 = v_mfma_scale_f32_32x32x64_f8f6f4 with
- * fp6 x fp4 operands, 2 = the same with fp8 x fp8.  Writes the number of
- * instructions issued and the operations each one stands for; `sink` is a
+ * fp6 x fp4 operands, 2 = the same with fp8 x fp8, 3 = the int8 instruction
+ * with operands that change from one instruction to the next, 4 = as 3 with the
+ * bit-weight product's operands (digits x bytes that are 0 or one power of
+ * two).  Writes the number of instructions issued and the operations each one stands for; `sink` is a
  * device word that is never written. */
 int nbla_hip_mfma_rate_probe(int kind, int rounds, int64_t *instructions,
                              int64_t *ops_per_instruction, float *sink,

@@ -585,7 +585,8 @@ def inq_convolution(x, W, I, old_W, old_I, bias=None, pad=None, stride=None, dil
     return y
 
 
-MFMA_PROBE_KINDS = {"i8": 0, "fp6 x fp4": 1, "fp8 x fp8": 2}
+MFMA_PROBE_KINDS = {"i8": 0, "fp6 x fp4": 1, "fp8 x fp8": 2, "i8, operands change": 3,
+                    "i8, digits x bit bytes, operands change": 4}
 
 
 def mfma_rate_probe(kind, rounds, sink, stream=None):
