@@ -528,6 +528,19 @@ int nbla_hip_range_recorder_f32(const float *x, float *y, size_t size, float *m,
                                 void *workspace, size_t workspace_bytes,
                                 void *stream);
 
+/* Measurement aid; no counterpart in the reference.  After
+ * nbla_hip_gemm_bits_timer_arm(n) the calling thread's next n launches of the
+ * bit-weight product (by nbla_hip_gemm_bits_f32 or by the functions built on
+ * it) each carry a pair of events that the runtime stamps with the dispatch's
+ * own begin and end, so the kernel's duration is read as a profiler reads it,
+ * without the queue bubbles of event records between launches.
+ * nbla_hip_gemm_bits_timer_read waits for the launches made so far, returns
+ * their number and the mean / smallest / largest duration in milliseconds and
+ * disarms.  The results of the launches are unaffected. */
+int nbla_hip_gemm_bits_timer_arm(int launches);
+int nbla_hip_gemm_bits_timer_read(int *launches, double *mean_ms, double *min_ms,
+                                  double *max_ms);
+
 /* Measurement utility; no counterpart in the reference.  Launches a kernel of
  * nothing but independent matrix instructions on non-zero operands (two blocks
  * of four wavefronts per CU, `rounds` x 8 instructions per wavefront) so that

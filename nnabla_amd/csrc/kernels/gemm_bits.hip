@@ -21,8 +21,10 @@
 #include "gemm_layout.hpp"
 #include "internal.hpp"
 
+#include <hip/hip_ext.h>
 #include <type_traits>
 #include <utility>
+#include <vector>
 
 namespace nbla_hip {
 namespace {
@@ -1082,6 +1084,23 @@ __global__ __launch_bounds__(512, 1) void gemm_bits_unfold_kernel(GemmBitsArgs a
   gemm_bits_body<32, 256, 1, 4, 2, true, kDigits, true>(a, smem);
 }
 
+// Measurement aid: while armed, the calling thread's launches of the product carry a pair of events that the runtime
+// stamps with the dispatch's own begin and end (hipExtLaunchKernelGGL), i.e. the kernel's duration as a profiler
+// sees it, without the queue bubbles that event records between launches add.
+struct KernelTimer {
+  std::vector<hipEvent_t> start, stop;
+  size_t used = 0;
+};
+thread_local KernelTimer t_timer;
+
+void kernel_timer_release() {
+  for (hipEvent_t e : t_timer.start)
+    (void)hipEventDestroy(e);
+  for (hipEvent_t e : t_timer.stop)
+    (void)hipEventDestroy(e);
+  t_timer.start.clear(), t_timer.stop.clear(), t_timer.used = 0;
+}
+
 template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, bool kSwap>
 int launch_tile(const GemmBitsArgs &args, hipStream_t stream, unsigned splits = 1) {
   constexpr int kThreads = kWavesM * kWavesN * kWavesK * 64;
@@ -1095,7 +1114,14 @@ int launch_tile(const GemmBitsArgs &args, hipStream_t stream, unsigned splits = 
   GemmBitsArgs a = args;
   a.blocks_m = ceil_div(a.M, BM);
   a.blocks_n = ceil_div(a.n_end - a.n_begin, BN);
-  hipLaunchKernelGGL(kernel, dim3((unsigned)(a.blocks_m * a.blocks_n), splits), dim3(kThreads), kSmem, stream, a);
+  const dim3 grid((unsigned)(a.blocks_m * a.blocks_n), splits);
+  if (t_timer.used < t_timer.start.size()) {
+    hipExtLaunchKernelGGL(kernel, grid, dim3(kThreads), kSmem, stream, t_timer.start[t_timer.used],
+                          t_timer.stop[t_timer.used], 0, a);
+    ++t_timer.used;
+  } else {
+    hipLaunchKernelGGL(kernel, grid, dim3(kThreads), kSmem, stream, a);
+  }
   NBLA_HIP_LAUNCH_CHECK("gemm_bits");
   return NBLA_HIP_OK;
 }
@@ -1332,4 +1358,54 @@ extern "C" int nbla_hip_gemm_bits_f32(const void *xdigits, const uint32_t *bits,
   // m-contiguous outputs (n_stride != 1) store from the transposed accumulator tile
   return launch_gemm_bits(xdigits, bits, alpha, bias, y, M, K, N, inner, outer_stride, n_stride, n_stride != 1,
                           as_stream(stream), false, workspace, workspace_bytes);
+}
+
+extern "C" int nbla_hip_gemm_bits_timer_arm(int launches) {
+  if (launches < 1 || launches > 65536)
+    return fail(NBLA_HIP_ERR_VALUE, "product timer: between 1 and 65536 launches.");
+  const int rc = ensure_init();
+  if (rc)
+    return rc;
+  kernel_timer_release();
+  for (int i = 0; i < launches; ++i) {
+    hipEvent_t a = nullptr, b = nullptr;
+    hipError_t e = hipEventCreate(&a);
+    if (e == hipSuccess)
+      e = hipEventCreate(&b);
+    if (e != hipSuccess) {
+      if (a)
+        (void)hipEventDestroy(a);
+      kernel_timer_release();
+      return fail_hip(e, "hipEventCreate");
+    }
+    t_timer.start.push_back(a), t_timer.stop.push_back(b);
+  }
+  return NBLA_HIP_OK;
+}
+
+extern "C" int nbla_hip_gemm_bits_timer_read(int *launches, double *mean_ms, double *min_ms, double *max_ms) {
+  const size_t n = t_timer.used;
+  double sum = 0.0, lo = 0.0, hi = 0.0;
+  for (size_t i = 0; i < n; ++i) {
+    float ms = 0.0f;
+    hipError_t e = hipEventSynchronize(t_timer.stop[i]);
+    if (e == hipSuccess)
+      e = hipEventElapsedTime(&ms, t_timer.start[i], t_timer.stop[i]);
+    if (e != hipSuccess) {
+      kernel_timer_release();
+      return fail_hip(e, "product timer");
+    }
+    sum += ms;
+    lo = (i == 0 || ms < lo) ? ms : lo, hi = (i == 0 || ms > hi) ? ms : hi;
+  }
+  kernel_timer_release();
+  if (launches)
+    *launches = (int)n;
+  if (mean_ms)
+    *mean_ms = n ? sum / (double)n : 0.0;
+  if (min_ms)
+    *min_ms = lo;
+  if (max_ms)
+    *max_ms = hi;
+  return NBLA_HIP_OK;
 }

@@ -46,6 +46,7 @@ EXPORTED = (
     "nbla_hip_cast", "nbla_hip_relu_f32", "nbla_hip_relu_backward_f32", "nbla_hip_add2_f32",
     "nbla_hip_add2_backward_f32", "nbla_hip_binary2_f32", "nbla_hip_binary2_backward_f32", "nbla_hip_copy_rows_f32",
     "nbla_hip_broadcast2_f32", "nbla_hip_broadcast2_backward_f32", "nbla_hip_mfma_rate_probe", "nbla_hip_binary_convolution_slab_plan",
+    "nbla_hip_gemm_bits_timer_arm", "nbla_hip_gemm_bits_timer_read",
 )
 
 
@@ -583,6 +584,19 @@ def inq_convolution(x, W, I, old_W, old_I, bias=None, pad=None, stride=None, dil
                                              int(num_bits), int(step), cb, None, _p(ws), ctypes.c_size_t(ws.numel()),
                                              _stream(stream)))
     return y
+
+
+def gemm_bits_timer_arm(launches):
+    """The calling thread's next `launches` launches of the bit-weight product record their own begin and end."""
+    check(lib().nbla_hip_gemm_bits_timer_arm(ctypes.c_int(int(launches))))
+
+
+def gemm_bits_timer_read():
+    """Waits for the armed launches made so far; {launches, mean_ms, min_ms, max_ms} of the kernel itself."""
+    n = ctypes.c_int(0)
+    mean, lo, hi = ctypes.c_double(0.0), ctypes.c_double(0.0), ctypes.c_double(0.0)
+    check(lib().nbla_hip_gemm_bits_timer_read(ctypes.byref(n), ctypes.byref(mean), ctypes.byref(lo), ctypes.byref(hi)))
+    return {"launches": n.value, "mean_ms": mean.value, "min_ms": lo.value, "max_ms": hi.value}
 
 
 MFMA_PROBE_KINDS = {"i8": 0, "fp6 x fp4": 1, "fp8 x fp8": 2, "i8, operands change": 3,

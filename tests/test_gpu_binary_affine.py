@@ -721,3 +721,21 @@ def test_quantize_zero_to_that_bf16_does_not_hold(dev, M):
     np.testing.assert_allclose(to_np(alpha), ref_alpha, rtol=2e-6)
     y64 = x.astype(np.float64) @ (ref_Wb.astype(np.float64) * np.abs(W.astype(np.float64)).mean(0)) + b
     assert max_rel_err(to_np(y), y64) <= TIGHT and max_rel_err(to_np(y), ref_y) <= TIGHT * 4
+
+
+def test_product_timer_stamps_its_launches_and_leaves_the_results_alone(dev):
+    """The measurement aid of bench.py: armed launches of the bit-weight product carry the runtime's begin / end
+    stamps; results are the same bits, launches past the armed number run as usual, reading disarms."""
+    x, W = _data(512, 1024, 1024, seed=9)
+    xd, Wd = _dev(x, dev), _dev(W, dev)
+    y0, _, _ = kernels.binary_weight_affine(xd, Wd)
+    kernels.gemm_bits_timer_arm(3)
+    ys = [kernels.binary_weight_affine(xd, Wd)[0] for _ in range(5)]
+    t = kernels.gemm_bits_timer_read()
+    assert t["launches"] == 3
+    assert 0.0 < t["min_ms"] <= t["mean_ms"] <= t["max_ms"] < 5.0
+    for y in ys:
+        assert bits_equal(to_np(y), to_np(y0))
+    assert kernels.gemm_bits_timer_read()["launches"] == 0
+    with pytest.raises(kernels.KernelError):
+        kernels.gemm_bits_timer_arm(0)
