@@ -244,6 +244,36 @@ def test_min_max_quantize_matches_oracle(dev, xshape, qshape, x_min_max, ema):
         assert bits_equal(g, r), "%s: %s" % (name, first_mismatch(g, r))
 
 
+def _random_mmq_shapes(count, seed):
+    rng = np.random.RandomState(seed)
+    out = []
+    while len(out) < count:
+        nd = int(rng.randint(1, 6))
+        xshape = tuple(int(v) for v in rng.choice([1, 2, 3, 4, 5, 7, 8, 16, 33, 64, 130], size=nd))
+        if int(np.prod(xshape)) > 300000:
+            continue
+        keep = rng.rand(nd) < 0.4
+        out.append((xshape, tuple(s if k else 1 for s, k in zip(xshape, keep))))
+    return out
+
+
+@pytest.mark.parametrize("xshape,qshape", _random_mmq_shapes(60, 577))
+def test_min_max_quantize_random_axis_patterns(dev, xshape, qshape):
+    """A seeded sweep over ranks 1 to 5 with every axis kept or reduced at random (sizes that end inside vectors and
+    wavefronts, axes of one element), with zeros of both signs sprinkled in: whichever kernels the pattern selects,
+    all four outputs carry the oracle's bits."""
+    print("shapes", xshape, qshape, flush=True)
+    rng = np.random.RandomState(hash((xshape, qshape)) % (2 ** 31))
+    x = (rng.randn(*xshape) * 3).astype(np.float32)
+    flat = x.reshape(-1)
+    flat[rng.randint(0, flat.size, size=max(1, flat.size // 50))] = 0.0
+    flat[rng.randint(0, flat.size, size=max(1, flat.size // 50))] = -0.0
+    for x_min_max, ema in ((True, True), (True, False), (False, True)):
+        got, ref = _mmq_both(dev, x, qshape, -6.0, 6.0, 0.0, 255.0, 0.999, x_min_max, ema)
+        for g, r, name in zip(got, ref, ("y", "qr_min", "qr_max", "scale")):
+            assert bits_equal(g, r), "%s: %s" % (name, first_mismatch(g, r))
+
+
 def test_min_max_quantize_general_axes_first_zero_wins(dev):
     """q shape (C, 1, W): the slice of (c, w) is scanned along the reduced axis in order, and of several zeros the
     first one's sign is the extremum's (min.cpp:29-41 / max.cpp:48-60 keep the first of equals)."""
