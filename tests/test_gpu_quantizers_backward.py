@@ -110,6 +110,41 @@ def test_min_max_backward(dev, xshape, qshape, fine):
     np.testing.assert_allclose(to_np(only_max[2]), rmax, rtol=1e-5, atol=1e-5)
 
 
+def _random_axis_patterns(count, seed):
+    rng = np.random.RandomState(seed)
+    out = []
+    while len(out) < count:
+        nd = int(rng.randint(1, 6))
+        xshape = tuple(int(v) for v in rng.choice([1, 2, 3, 4, 5, 7, 8, 16, 33, 64, 130], size=nd))
+        if int(np.prod(xshape)) > 300000:
+            continue
+        keep = rng.rand(nd) < 0.4
+        out.append((xshape, tuple(s if k else 1 for s, k in zip(xshape, keep))))
+    return out
+
+
+@pytest.mark.parametrize("xshape,qshape", _random_axis_patterns(40, 578))
+def test_min_max_backward_random_axis_patterns(dev, xshape, qshape):
+    """Ranks 1 to 5 with every axis kept or reduced at random: the input gradient bit for bit, the range gradients
+    (sums in a fixed order of their own) relative to the sum of |dy| over the reduced axes."""
+    print("shapes", xshape, qshape, flush=True)
+    x, dy = _rand(xshape, 21, 3.0), _rand(xshape, 22)
+    qr_min = np.full(qshape, -2.0, np.float32) + _rand(qshape, 23, 0.1)
+    qr_max = np.full(qshape, 2.5, np.float32) + _rand(qshape, 24, 0.1)
+    ql_min, ql_max = np.zeros(qshape, np.float32), np.full(qshape, 255.0, np.float32)
+    _, qmn, qmx, scale = oracle.min_max_quantize(x, qr_min, qr_max, ql_min, ql_max, 0.999, False, False, 0.01)
+    d = lambda a: _dev(a, dev)
+    axes = tuple(i for i in range(len(xshape)) if qshape[i] == 1)
+    denom = np.abs(dy).astype(np.float64).sum(axis=axes, keepdims=True) + 1e-30
+    for fine in (True, False):
+        rdx, rmin, rmax = oracle.min_max_quantize_backward(dy, x, qmn, qmx, ql_min, ql_max, scale, fine, False, False)
+        gdx, gmin, gmax = kernels.min_max_quantize_backward(d(dy), d(x), d(qmn), d(qmx), d(ql_min), d(ql_max), d(scale),
+                                                            fine, False, False)
+        assert bits_equal(to_np(gdx), rdx), first_mismatch(to_np(gdx), rdx)
+        assert (np.abs(to_np(gmin) - rmin.astype(np.float64)) / denom).max() <= 2e-6
+        assert (np.abs(to_np(gmax) - rmax.astype(np.float64)) / denom).max() <= 2e-6
+
+
 @pytest.mark.parametrize("x_min_max,ema", [(True, False), (False, True)])
 def test_min_max_backward_statistics_modes_leave_range_gradients(dev, x_min_max, ema):
     x, dy = _rand((2, 3, 4, 4), 21), _rand((2, 3, 4, 4), 22)
