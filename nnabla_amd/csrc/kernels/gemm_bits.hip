@@ -809,28 +809,48 @@ __device__ __forceinline__ void gemm_bits_body(GemmBitsArgs a, unsigned char *sm
         }
         return;
       }
+      // Three-digit rows.  Between two MFMAs a wavefront can issue a few other instructions without starving the
+      // matrix pipe, but not a batch of them: the LDS reads of the next k tile and the copies of a later step are
+      // therefore dealt out one per MFMA (sched_group_barrier: 0x008 = MFMA, 0x100 = LDS read, 0x020 = the copies'
+      // buffer loads) instead of standing together between two groups of MFMAs.  A wavefront that has its SIMD to
+      // itself (its neighbour is in its prologue or epilogue) gains most: 0.421 -> 0.400 ms for the launch with one
+      // block per CU, 0.360 -> 0.354 ms with two.
+      constexpr int kCopies = decltype(count_c)::value;
+      constexpr int kReads = MF * kUsed + 1, kMfmas = MF * NF * kUsed;
+      static_assert(kUsed == 1 || kReads + kCopies <= kMfmas, "more reads and copies than MFMAs to deal them out to");
       for (int left = nstages; left > 0; --left) {
         const int next = (cur + kStageBytes == kStages * kStageBytes) ? 0 : cur + kStageBytes;
-        // tile 0 runs; tile 1 is fetched
-        mma(af0, w0, J0(), J1());
-        __builtin_amdgcn_sched_barrier(0);
+        // tile 0 runs; tile 1 (same stage: it landed with tile 0) is fetched
         read_a(cur, 1, af1);
         read_words(cur, 1, w1);
-        __builtin_amdgcn_sched_barrier(0);
-        mma(af0, w0, J1(), JN());
+        mma(af0, w0, J0(), JN());
+#pragma unroll
+        for (int i = 0; i < kReads; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, kMfmas - kReads, 0);
         __builtin_amdgcn_sched_barrier(0);
         // step ks+1 has landed: the copies issued so far reach step ks+kDepth-1, so at most the kDepth-2 (= kLoopWait)
         // steps behind ks+1 may still be in flight; every wavefront is done with the buffer of step ks-1
         wait_copies(std::integral_constant<int, kLoopWait>(), count_c);
         NBLA_BARRIER();
         // tile 1 runs; the copy of step ks+kDepth is issued; tile 0 of step ks+1 is fetched
-        mma(af1, w1, J0(), J1());
-        __builtin_amdgcn_sched_barrier(0);
         copy_next(prev, count_c);
         read_words(next, 0, w0);
         read_a(next, 0, af0);
-        __builtin_amdgcn_sched_barrier(0);
-        mma(af1, w1, J1(), JN());
+        mma(af1, w1, J0(), JN());
+#pragma unroll
+        for (int i = 0; i < kCopies; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 1);
+        }
+#pragma unroll
+        for (int i = 0; i < kReads; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, kMfmas - kReads - kCopies, 1);
         __builtin_amdgcn_sched_barrier(0);
         prev = cur;
         cur = next;
