@@ -191,19 +191,33 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
     // is done with the buffer tile kt - 1 occupied, which tile kt + kStages - 1 takes over
     NBLA_WAIT_VMCNT(kLoopWait * kCopies);
     NBLA_BARRIER();
-    copy_next(buf == 0 ? kStages - 1 : buf - 1);
     const uint4_t *sa = reinterpret_cast<const uint4_t *>(smem + buf * kGroupStageBytes + group * kStageBytes);
     const uint4_t *sb = sa + kSideVec;
     i32x4_t af[2][3], bf[2][3];
+    // digit by digit: the first products need the top digits' four fragments only
+    if (kNarrow) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < 2; ++i)
+        bf[i][kBDigit] = __builtin_bit_cast(i32x4_t, sb[((wn * 2 + i) * kDigits + kBDigit) * 64 + lane]);
+    }
 #pragma unroll
-      for (int d = 0; d < 3; ++d) {
+    for (int d = 0; d < 3; ++d)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
         if (!kOneA || d == 0)
           af[i][d] = __builtin_bit_cast(i32x4_t, sa[((wm * 2 + i) * kDigits + d) * 64 + lane]);
-        if (!kNarrow || d == kBDigit)
+        if (!kNarrow)
           bf[i][d] = __builtin_bit_cast(i32x4_t, sb[((wn * 2 + i) * kDigits + d) * 64 + lane]);
       }
+    copy_next(buf == 0 ? kStages - 1 : buf - 1);
+    // Issue order (sched_group_barrier: 0x100 = LDS read, 0x008 = MFMA, 0x020 = the copies' loads): the fragments of
+    // the first products, then one further read per MFMA, then one copy per MFMA, instead of twelve reads and the
+    // copies in a row before the first MFMA -- a wavefront cannot feed the matrix pipe while it issues a batch of other
+    // instructions (the weight-gradient product of 4096 x 4096 x 11008: 1.14 -> 1.08 ms).
+    constexpr int kFirstReads = kOneA ? 4 : (kNarrow ? 4 : 4);
+    constexpr int kAllReads = kOneA ? 4 : (kNarrow ? 8 : 12);
+    constexpr int kAllMfmas = kOneA ? 4 : (kNarrow ? 12 : 24);
+    static_assert(kAllReads - kFirstReads + kCopies <= kAllMfmas, "more reads and copies than MFMAs to deal them out to");
     if (kOneA) {
 #pragma unroll
       for (int i = 0; i < 2; ++i)
@@ -231,6 +245,19 @@ __device__ __forceinline__ void gemm_digits_tile(const GemmDigitsArgs &a, unsign
             acc[i][j][da[t] + db[t]] =
                 __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i][da[t]], bf[j][db[t]], acc[i][j][da[t] + db[t]], 0, 0, 0);
     }
+    __builtin_amdgcn_sched_group_barrier(0x100, kFirstReads, 0);
+#pragma unroll
+    for (int q = 0; q < kAllReads - kFirstReads; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+#pragma unroll
+    for (int q = 0; q < kCopies; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, kAllMfmas - (kAllReads - kFirstReads) - kCopies, 0);
+    __builtin_amdgcn_sched_barrier(0);
     buf = (buf + 1 == kStages) ? 0 : buf + 1;
   }
   NBLA_WAIT_VMCNT(0);
