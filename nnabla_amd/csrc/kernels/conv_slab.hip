@@ -427,19 +427,27 @@ __global__ __launch_bounds__(kSlabThreads, 1) void binary_conv_slab_kernel(ConvS
     read_a(off_a, af[0]);
     // Whole rounds of kSlabAhead steps, without a branch inside a round (the compiler then counts the loads in flight
     // exactly: a word is waited for with the younger loads still outstanding).  Steps past the last k tile
-    // multiply the zero pixel.  Inside a step the LDS reads of the next step go first and the MFMAs of this one run
-    // while they are served (sched_barrier pins that order).
+    // multiply the zero pixel.  Inside a step the LDS reads of the next step (the table entry and the four digits) and
+    // the load of a later step's words are dealt out one per MFMA of this step (sched_group_barrier: 0x008 = MFMA,
+    // 0x100 = LDS read, 0x020 = global load): a wavefront that issues them in a row leaves the matrix pipe waiting.
     for (int i0 = 0; i0 < nk; i0 += kSlabAhead) {
 #pragma unroll
       for (int u = 0; u < kSlabAhead; ++u) {
         const uint32_t off_c = row_off(); // step i + 2
         advance();
         read_a(off_b, af[(u + 1) & 1]); // step i + 1
-        __builtin_amdgcn_sched_barrier(0);
         mma(af[u & 1], words[u]);
         words[u] = wnext[lane];
         wnext += wleft > 0 ? wstep : 0;
         --wleft;
+#pragma unroll
+        for (int q = 0; q < kSlabDigits + 1; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, kSlabDigits - 2, 0);
         __builtin_amdgcn_sched_barrier(0);
         off_b = off_c;
       }
