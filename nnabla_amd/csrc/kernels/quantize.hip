@@ -564,30 +564,12 @@ struct MinMaxScalars {
   int x_min_max, ema;
 };
 
-__global__ __launch_bounds__(64) void minmax_finalize(const MinMaxPartial *__restrict__ partial, int nchunks,
-                                                      float *__restrict__ qr_min, float *__restrict__ qr_max,
-                                                      const float *__restrict__ ql_min,
+// The nudged range, scale and zero point of one range from its extrema (min_max_quantize.cpp:130-211), every
+// operation rounded on its own.
+__device__ __forceinline__ void minmax_finalize_range(const Extrema &ex, int64_t k, float *__restrict__ qr_min,
+                                                      float *__restrict__ qr_max, const float *__restrict__ ql_min,
                                                       const float *__restrict__ ql_max, float *__restrict__ scale_out,
-                                                      float4_t *__restrict__ params, MinMaxScalars s) {
-  const int64_t k = blockIdx.x;
-  Extrema ex;
-  ex.init();
-  if (s.x_min_max) {
-    // sixteen independent 16-byte loads in flight per lane before any merge: one round trip for 1024 partials
-    const float4_t *pp = reinterpret_cast<const float4_t *>(partial + k * nchunks);
-    for (int c = threadIdx.x; c < nchunks; c += 1024) {
-      float4_t q[16];
-#pragma unroll
-      for (int j = 0; j < 16; ++j)
-        q[j] = (c + 64 * j < nchunks) ? pp[c + 64 * j] : float4_t{1e+8f, -1e+8f, __uint_as_float(0xffffffffu), 0.0f};
-#pragma unroll
-      for (int j = 0; j < 16; ++j)
-        ex.merge(q[j].x, q[j].y, __float_as_uint(q[j].z), __float_as_uint(q[j].w));
-    }
-    ex.wave_reduce();
-  }
-  if (threadIdx.x != 0)
-    return;
+                                                      float4_t *__restrict__ params, const MinMaxScalars &s) {
   float lo = qr_min[k], hi = qr_max[k];
   if (s.x_min_max && s.ema) {
     const float a = ex.min_value() * s.one_minus_decay;
@@ -625,6 +607,69 @@ __global__ __launch_bounds__(64) void minmax_finalize(const MinMaxPartial *__res
   pr.z = scale;
   pr.w = 0.0f;
   params[k] = pr;
+}
+
+__global__ __launch_bounds__(64) void minmax_finalize(const MinMaxPartial *__restrict__ partial, int nchunks,
+                                                      float *__restrict__ qr_min, float *__restrict__ qr_max,
+                                                      const float *__restrict__ ql_min,
+                                                      const float *__restrict__ ql_max, float *__restrict__ scale_out,
+                                                      float4_t *__restrict__ params, MinMaxScalars s) {
+  const int64_t k = blockIdx.x;
+  Extrema ex;
+  ex.init();
+  if (s.x_min_max) {
+    // sixteen independent 16-byte loads in flight per lane before any merge: one round trip for 1024 partials
+    const float4_t *pp = reinterpret_cast<const float4_t *>(partial + k * nchunks);
+    for (int c = threadIdx.x; c < nchunks; c += 1024) {
+      float4_t q[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        q[j] = (c + 64 * j < nchunks) ? pp[c + 64 * j] : float4_t{1e+8f, -1e+8f, __uint_as_float(0xffffffffu), 0.0f};
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        ex.merge(q[j].x, q[j].y, __float_as_uint(q[j].z), __float_as_uint(q[j].w));
+    }
+    ex.wave_reduce();
+  }
+  if (threadIdx.x != 0)
+    return;
+  minmax_finalize_range(ex, k, qr_min, qr_max, ql_min, ql_max, scale_out, params, s);
+}
+
+// Many ranges of few partial results each (ranges per channel and column, say): a thread per range instead of a
+// wavefront per range.  The merge does not depend on the order (extrema, and the first zero by its index).
+__global__ __launch_bounds__(256) void minmax_finalize_many(const MinMaxPartial *__restrict__ partial, int nchunks,
+                                                            int64_t K, float *__restrict__ qr_min,
+                                                            float *__restrict__ qr_max,
+                                                            const float *__restrict__ ql_min,
+                                                            const float *__restrict__ ql_max,
+                                                            float *__restrict__ scale_out,
+                                                            float4_t *__restrict__ params, MinMaxScalars s) {
+  const int64_t k = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (k >= K)
+    return;
+  Extrema ex;
+  ex.init();
+  if (s.x_min_max) {
+    const float4_t *pp = reinterpret_cast<const float4_t *>(partial + k * nchunks);
+    for (int c = 0; c < nchunks; ++c) {
+      const float4_t q = pp[c];
+      ex.merge(q.x, q.y, __float_as_uint(q.z), __float_as_uint(q.w));
+    }
+  }
+  minmax_finalize_range(ex, k, qr_min, qr_max, ql_min, ql_max, scale_out, params, s);
+}
+
+// One wavefront per range, or one thread per range where the ranges are many and their partial results few.
+void launch_minmax_finalize(int64_t K, const MinMaxPartial *partial, int nchunks, float *qr_min, float *qr_max,
+                            const float *ql_min, const float *ql_max, float *scale, float4_t *params,
+                            const MinMaxScalars &sc, hipStream_t stream) {
+  if (K >= 256 && nchunks <= 16)
+    hipLaunchKernelGGL(minmax_finalize_many, dim3((unsigned)((K + 255) / 256)), dim3(256), 0, stream, partial, nchunks, K,
+                       qr_min, qr_max, ql_min, ql_max, scale, params, sc);
+  else
+    hipLaunchKernelGGL(minmax_finalize, dim3((unsigned)K), dim3(64), 0, stream, partial, nchunks, qr_min, qr_max, ql_min,
+                       ql_max, scale, params, sc);
 }
 
 // min_max_quantize.cpp:213-222: seven separately rounded fp32 operations.
@@ -958,8 +1003,7 @@ int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, in
       sc.eps = eps;
       sc.x_min_max = x_min_max;
       sc.ema = ema;
-      hipLaunchKernelGGL(minmax_finalize, dim3((unsigned)L.K), dim3(64), 0, stream, partial, nchunks, qr_min, qr_max,
-                         ql_min, ql_max, scale, params, sc);
+      launch_minmax_finalize(L.K, partial, nchunks, qr_min, qr_max, ql_min, ql_max, scale, params, sc, stream);
       NBLA_HIP_LAUNCH_CHECK("min_max_quantize finalize");
       if (quads)
         hipLaunchKernelGGL(minmax_apply_inner<4>, grid, dim3(kRedBlock), 0, stream, x, y, axes, inner, nchunks, params);
@@ -979,8 +1023,7 @@ int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, in
     sc.eps = eps;
     sc.x_min_max = x_min_max;
     sc.ema = ema;
-    hipLaunchKernelGGL(minmax_finalize, dim3((unsigned)L.K), dim3(64), 0, stream, partial, 1, qr_min, qr_max, ql_min,
-                       ql_max, scale, params, sc);
+    launch_minmax_finalize(L.K, partial, 1, qr_min, qr_max, ql_min, ql_max, scale, params, sc, stream);
     NBLA_HIP_LAUNCH_CHECK("min_max_quantize finalize");
     int64_t blocks = (L.total + kBlock - 1) / kBlock;
     if (blocks > 65536)
@@ -1017,8 +1060,7 @@ int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, in
   s.eps = eps;
   s.x_min_max = x_min_max;
   s.ema = ema;
-  hipLaunchKernelGGL(minmax_finalize, dim3((unsigned)L.K), dim3(64), 0, stream, partial, nchunks, qr_min, qr_max,
-                     ql_min, ql_max, scale, params, s);
+  launch_minmax_finalize(L.K, partial, nchunks, qr_min, qr_max, ql_min, ql_max, scale, params, s, stream);
   NBLA_HIP_LAUNCH_CHECK("min_max_quantize finalize");
 
   if (L.K == 1 && aligned16(x) && aligned16(y)) {

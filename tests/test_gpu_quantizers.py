@@ -231,6 +231,9 @@ MMQ_SHAPES = [
     # axes, a long innermost reduced axis, and a slice of the benchmark's [64,256,56,56] with ranges [1,256,1,56]
     ((4, 10, 100), (4, 1, 100)), ((3, 4, 5, 6, 7), (1, 4, 1, 1, 7)), ((2, 5, 300, 9), (1, 5, 1, 9)),
     ((8, 16, 56, 56), (1, 16, 1, 56)), ((70, 3, 2), (1, 3, 1)), ((2, 3, 4, 2), (2, 1, 4, 2)),
+    # hundreds of ranges with few partial results each (a thread per range folds them): lanes along the kept innermost
+    # axis, per channel, and the one-block-per-range form
+    ((4, 64, 6, 40), (1, 64, 1, 40)), ((2, 512, 4, 4), (1, 512, 1, 1)), ((64, 3, 8, 2), (64, 1, 8, 1)),
 ]
 
 
