@@ -1,0 +1,79 @@
+"""Element-wise quantizers on tensors of more than 2^31 elements (8.6 GB per tensor): indices and byte offsets past
+what 32 bits hold, and an end that falls inside a vector and a block.  The input repeats one million-element period,
+so the output must repeat the output of that period -- itself bit-checked against the CPU oracle -- and the
+comparison stays on the device."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from nnabla_amd import kernels
+from util import bits_equal, to_np
+
+pytestmark = pytest.mark.gpu
+
+@pytest.fixture(autouse=True)
+def _release_device_memory():
+    yield
+    torch.cuda.empty_cache()   # the 8.6 GB tensors go back to the device, not into the caching allocator's pool
+
+
+PERIOD = 1 << 20
+N = (1 << 31) + 5 * PERIOD + 13   # not a multiple of 4: the tail past the last 16-byte vector
+
+
+def _periodic(dev, seed, scale):
+    base = (np.random.RandomState(seed).randn(PERIOD) * scale).astype(np.float32)
+    base[::97] = 0.0
+    base[5::101] = -0.0
+    b = torch.from_numpy(base).to(dev)
+    reps = N // PERIOD + 1
+    x = b.repeat(reps)[:N].contiguous()
+    return base, x
+
+
+def _repeats(y, first):
+    """y (length N) equals `first` (length PERIOD) repeated, bit for bit; compared in int32 on the device."""
+    yi, fi = y.view(torch.int32), first.view(torch.int32)
+    whole = (N // PERIOD) * PERIOD
+    ok = bool((yi[:whole].view(-1, PERIOD) == fi).all())
+    return ok and bool((yi[whole:] == fi[:N - whole]).all())
+
+
+def test_fixed_point_and_pow2_quantize_past_2_31_elements(dev):
+    free, _ = torch.cuda.mem_get_info()
+    if free < 40 * (1 << 30):
+        pytest.skip("needs 40 GB of free device memory")
+    base, x = _periodic(dev, 11, 2.0)
+    y = kernels.fixed_point_quantize(x, True, 8, 2.0 ** -4)
+    first = y[:PERIOD].clone()
+    assert bits_equal(to_np(first), oracle.fixed_point_quantize(base, True, 8, 2.0 ** -4))
+    assert _repeats(y, first)
+    # backward on the same tensors: dy = y, fine-grained mask
+    dx = kernels.fixed_point_quantize_backward(y, x, True, 8, 2.0 ** -4, True)
+    ref = oracle.fixed_point_quantize_backward(to_np(first), base, True, 8, 2.0 ** -4, True)
+    assert bits_equal(to_np(dx[:PERIOD]), ref)
+    assert _repeats(dx, dx[:PERIOD].clone())
+    del dx
+    kernels.pow2_quantize(x, True, True, 4, 1, out=y)
+    first = y[:PERIOD].clone()
+    assert bits_equal(to_np(first), oracle.pow2_quantize(base, True, True, 4, 1))
+    assert _repeats(y, first)
+
+
+def test_min_max_quantize_past_2_31_elements(dev):
+    free, _ = torch.cuda.mem_get_info()
+    if free < 40 * (1 << 30):
+        pytest.skip("needs 40 GB of free device memory")
+    base, x = _periodic(dev, 12, 3.0)
+    q = lambda v: torch.full((1,), v, dtype=torch.float32, device=dev)
+    qmn, qmx = q(-6.0), q(6.0)
+    y, scale = kernels.min_max_quantize(x, qmn, qmx, q(0.0), q(255.0), 0.999, True, True)
+    one = lambda v: np.full((1,), v, np.float32)
+    ry, rmn, rmx, rscale = oracle.min_max_quantize(base, one(-6.0), one(6.0), one(0.0), one(255.0), 0.999, True, True,
+                                                   0.01)
+    # the extrema of the whole tensor are those of one period (first of equal zeros: inside the first period)
+    assert bits_equal(to_np(qmn), rmn) and bits_equal(to_np(qmx), rmx) and bits_equal(to_np(scale), rscale)
+    first = y[:PERIOD].clone()
+    assert bits_equal(to_np(first), ry)
+    assert _repeats(y, first)
