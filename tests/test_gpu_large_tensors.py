@@ -77,3 +77,28 @@ def test_min_max_quantize_past_2_31_elements(dev):
     first = y[:PERIOD].clone()
     assert bits_equal(to_np(first), ry)
     assert _repeats(y, first)
+
+
+def test_binary_weight_affine_output_past_2_31_elements(dev):
+    """y of 70,000 x 32,768 (2.29e9 elements, 9.2 GB): output offsets beyond 32 bits in the product's stores.  Rows
+    from both ends and the middle against float64."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 30 * (1 << 30):
+        pytest.skip("needs 30 GB of free device memory")
+    M, K, N = 70000, 64, 32768
+    rng = np.random.RandomState(13)
+    x = rng.randn(M, K).astype(np.float32)
+    W = (rng.randn(K, N) * 0.05).astype(np.float32)
+    b = rng.randn(N).astype(np.float32)
+    y, Wb, alpha = kernels.binary_weight_affine(torch.from_numpy(x).to(dev), torch.from_numpy(W).to(dev),
+                                                torch.from_numpy(b).to(dev))
+    assert y.numel() > (1 << 31)
+    ref_Wb = np.where(W < 0, np.float32(-1), np.float32(1))
+    assert bits_equal(to_np(Wb), ref_Wb)
+    Wd = ref_Wb.astype(np.float64) * np.abs(W.astype(np.float64)).mean(0)
+    rows = [0, 1, 31, 32, 34999, 65535, 65536, 65537, 69998, 69999]
+    got = to_np(y[rows])
+    ref = x[rows].astype(np.float64) @ Wd + b
+    assert np.abs(got - ref).max() / np.abs(ref).max() <= 5e-6
+    # nothing but finite values anywhere (a store gone astray would leave the allocator's old bytes or fault)
+    assert bool(torch.isfinite(y).all())
