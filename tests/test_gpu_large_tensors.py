@@ -102,3 +102,57 @@ def test_binary_weight_affine_output_past_2_31_elements(dev):
     assert np.abs(got - ref).max() / np.abs(ref).max() <= 5e-6
     # nothing but finite values anywhere (a store gone astray would leave the allocator's old bytes or fault)
     assert bool(torch.isfinite(y).all())
+
+
+@pytest.mark.parametrize("M", [4, 48, 200, 600])
+def test_binary_weight_affine_weights_past_2_31_elements(dev, M):
+    """W of 36,000 x 65,536 (2.36e9 weights, 9.4 GB, and as much again for Wb) through each form of the forward: one
+    pass on the vector ALUs, one pass on the matrix cores, one walk, two walks.  Checked on the device: Wb against
+    the sign of W everywhere, alpha and y against float64 on the first and the last columns."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 50 * (1 << 30):
+        pytest.skip("needs 50 GB of free device memory")
+    K, N = 36000, 65536
+    g = torch.Generator(device=dev).manual_seed(100 + M)
+    W = torch.randn(K, N, generator=g, device=dev) * 0.05
+    x = torch.randn(M, K, generator=g, device=dev)
+    assert W.numel() > (1 << 31)
+    y, Wb, alpha = kernels.binary_weight_affine(x, W)
+    assert bool((Wb == torch.where(W < 0, -1.0, 1.0)).all())
+    for cols in (slice(0, 384), slice(N - 384, N)):
+        a64 = W[:, cols].double().abs().mean(0)
+        assert float(((alpha[cols].double() - a64).abs() / a64).max()) <= 2e-6
+        ref = x.double() @ (Wb[:, cols].double() * a64)
+        err = float((y[:, cols].double() - ref).abs().max() / ref.abs().max())
+        assert err <= 5e-6, err
+    assert bool(torch.isfinite(y).all())
+
+
+def test_binary_affine_backward_weights_past_2_31_elements(dev):
+    """The same weight matrix through the backward pass: dW (2.36e9 outputs of the digit x digit product, a plain
+    x^T dy under the straight-through estimator) and dx = (dy * alpha) Wb^T, against float64 on blocks from the
+    corners of each result."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 60 * (1 << 30):
+        pytest.skip("needs 60 GB of free device memory")
+    M, K, N = 320, 36000, 65536
+    g = torch.Generator(device=dev).manual_seed(7)
+    W = torch.randn(K, N, generator=g, device=dev) * 0.05
+    x = torch.randn(M, K, generator=g, device=dev)
+    dy = torch.randn(M, N, generator=g, device=dev)
+    alpha = W.abs().mean(0)
+    dx, dW, db = kernels.binary_affine_backward(dy, x, W, None, alpha, 1.0)
+    assert dW.numel() > (1 << 31)
+    for rows in (slice(0, 256), slice(K - 256, K)):
+        for cols in (slice(0, 256), slice(N - 256, N)):
+            ref = x[:, rows].double().t() @ dy[:, cols].double()
+            err = float((dW[rows, cols].double() - ref).abs().max() / ref.abs().max())
+            assert err <= 5e-6, err
+    for rows in (slice(0, 512), slice(K - 512, K)):
+        Wb = torch.where(W[rows] < 0, -1.0, 1.0).double()
+        ref = (dy.double() * alpha.double()) @ Wb.t()
+        err = float((dx[:, rows].double() - ref).abs().max() / ref.abs().max())
+        assert err <= 5e-6, err
+    ref = dy.double().sum(0)
+    assert float((db.double() - ref).abs().max() / ref.abs().max()) <= 5e-6
+    assert bool(torch.isfinite(dW).all())
