@@ -156,3 +156,28 @@ def test_binary_affine_backward_weights_past_2_31_elements(dev):
     ref = dy.double().sum(0)
     assert float((db.double() - ref).abs().max() / ref.abs().max()) <= 5e-6
     assert bool(torch.isfinite(dW).all())
+
+
+def test_quantize_and_dequantize_linear_past_2_31_elements(dev):
+    """A [rows, 2^20] tensor of more than 2^31 elements with a per-column scale (the broadcast index arithmetic of
+    the two functions) and with one scale for the whole tensor (QuantizeLinear's own fast path)."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 40 * (1 << 30):
+        pytest.skip("needs 40 GB of free device memory")
+    rows = (1 << 11) + 3
+    rng = np.random.RandomState(14)
+    base = (rng.randn(1, PERIOD) * 30).astype(np.float32)
+    x = torch.from_numpy(base).to(dev).repeat(rows, 1).contiguous()
+    assert x.numel() > (1 << 31)
+    col_scale = (0.1 + rng.rand(1, PERIOD)).astype(np.float32)
+    col_zp = rng.randint(-3, 4, size=(1, PERIOD)).astype(np.float32)
+    for scale, zp in ((col_scale, col_zp), (np.full((1, 1), 0.3, np.float32), np.full((1, 1), 2.0, np.float32))):
+        y = kernels.quantize_linear(x, torch.from_numpy(scale).to(dev), torch.from_numpy(zp.copy()).to(dev),
+                                    "HALF_TO_EVEN", False, kernels.DTYPE_BYTE)
+        ref, _ = oracle.quantize_linear(base, scale, zp, "HALF_TO_EVEN", False, kernels.DTYPE_BYTE)
+        assert bits_equal(to_np(y[0:1]), ref)
+        assert bool((y.view(torch.int32) == y[0:1].view(torch.int32)).all())
+        z = kernels.dequantize_linear(y, torch.from_numpy(scale).to(dev), torch.from_numpy(zp).to(dev))
+        assert bits_equal(to_np(z[rows - 1:rows]), oracle.dequantize_linear(ref, scale, zp))
+        assert bool((z.view(torch.int32) == z[0:1].view(torch.int32)).all())
+        del y, z
