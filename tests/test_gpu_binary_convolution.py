@@ -208,3 +208,43 @@ def test_convolution_argument_errors(dev):
     with pytest.raises(kernels.KernelError) as ei:
         kernels.binary_connect_convolution(x, _dev(np.zeros((6, 2, 3, 3), np.float32), dev), group=3)
     assert ei.value.code == kernels.ERR_VALUE
+
+
+@pytest.mark.parametrize("channels,q0,zeros", [(32, 1.0, False), (32, 0.0, True), (8, 1.0, False), (8, 0.0, True)])
+def test_forward_and_backward_replay_in_a_hip_graph(dev, channels, q0, zeros):
+    """The convolution's forward and backward captured once and replayed on new inputs, for the product on input
+    positions held in LDS (32 channels) and the gathering product (8), with quantize_zero_to decided on the device:
+    every replay gives the eager call's bits (eager work and synchronisations run between the replays)."""
+    rng = np.random.RandomState(5)
+    xs, ws = (2, channels, 9, 9), (40, channels, 3, 3)
+    Wh = (rng.randn(*ws) * 0.05).astype(np.float32)
+    if zeros:
+        Wh.ravel()[::7] = 0.0
+    W = _dev(Wh, dev)
+    x = torch.empty(xs, device=dev)
+    dy = torch.empty((2, 40, 9, 9), device=dev)
+
+    def step():
+        y, Wb, alpha = kernels.binary_weight_convolution(x, W, None, (1, 1), (1, 1), (1, 1), 1, q0)
+        dx, dW, db = kernels.binary_convolution_backward(dy, x, W, Wb, alpha, (1, 1), (1, 1), (1, 1), 1, q0)
+        return y, dx, dW, db
+
+    x.copy_(_dev(rng.randn(*xs).astype(np.float32), dev))
+    dy.copy_(_dev(rng.randn(2, 40, 9, 9).astype(np.float32), dev))
+    step()                                   # first call outside the capture (one-time kernel attributes)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for i in range(3):
+        x.copy_(_dev((rng.randn(*xs) * (i + 1)).astype(np.float32), dev))
+        dy.copy_(_dev(rng.randn(2, 40, 9, 9).astype(np.float32), dev))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [to_np(o).copy() for o in outs]
+        eager = step()
+        torch.cuda.synchronize()
+        for g, e, name in zip(got, eager, ("y", "dx", "dW", "db")):
+            assert bits_equal(g, to_np(e)), "replay %d: %s differs from the eager result" % (i, name)
+        ref_y, _, _ = oracle.binary_weight_convolution(to_np(x), Wh, None, (1, 1), (1, 1), (1, 1), 1, q0)
+        assert max_rel_err(got[0], ref_y) <= TOL
