@@ -739,3 +739,40 @@ def test_product_timer_stamps_its_launches_and_leaves_the_results_alone(dev):
     assert kernels.gemm_bits_timer_read()["launches"] == 0
     with pytest.raises(kernels.KernelError):
         kernels.gemm_bits_timer_arm(0)
+
+
+@pytest.mark.parametrize("M,K,N,q0", [(100, 1024, 8196, 1.0), (100, 1024, 8196, 0.0), (600, 512, 2052, 1.0)])
+def test_one_walk_and_two_walk_forms_and_the_backward_replay_in_a_hip_graph(dev, M, K, N, q0):
+    """The forward's one-walk form (some hundred rows, wide outputs; with quantize_zero_to = 0 and exact-zero weights
+    its device-side fall-back), the two-walk form, and the backward pass of each, captured once and replayed on new
+    inputs: the replay's bits are the eager call's."""
+    rng = np.random.RandomState(78)
+    Wh = (rng.randn(K, N) * 0.02).astype(np.float32)
+    Wh.ravel()[::11] = 0.0
+    W = _dev(Wh, dev)
+    x, dy = torch.empty(M, K, device=dev), torch.empty(M, N, device=dev)
+
+    def step():
+        y, Wb, alpha = kernels.binary_weight_affine(x, W, None, q0)
+        dx, dW, db = kernels.binary_affine_backward(dy, x, W, Wb, alpha, q0)
+        return y, dx, dW, db
+
+    x.copy_(_dev(rng.randn(M, K).astype(np.float32), dev))
+    dy.copy_(_dev(rng.randn(M, N).astype(np.float32), dev))
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for i in range(3):
+        x.copy_(_dev((rng.randn(M, K) * (i + 1)).astype(np.float32), dev))
+        dy.copy_(_dev(rng.randn(M, N).astype(np.float32), dev))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [to_np(o).copy() for o in outs]
+        eager = step()
+        torch.cuda.synchronize()
+        for g, e, name in zip(got, eager, ("y", "dx", "dW", "db")):
+            assert bits_equal(g, to_np(e)), "replay %d: %s differs from the eager result" % (i, name)
+        ref, _, _ = oracle.binary_weight_affine(to_np(x), Wh, None, q0)
+        assert max_rel_err(got[0], ref) <= TOL
