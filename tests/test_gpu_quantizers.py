@@ -370,3 +370,49 @@ def test_min_max_quantize_every_fp32_value(dev, qr_min, qr_max, ql_min, ql_max):
         if not bool(same.all()):
             i = int((~same).nonzero()[0])
             raise AssertionError("x=%r (bits %#x): got %r want %r" % (float(x[i]), start + i, float(y[i]), float(ref[i])))
+
+
+def test_quantizer_family_replays_in_a_hip_graph(dev):
+    """MinMaxQuantize with its running range (state carried from replay to replay), Pow2Quantize, QuantizeLinear /
+    DequantizeLinear, Prune (its selection passes clear and fill counters) and a range recorder (its ticket slot is
+    chosen when the graph is captured), captured once and replayed on new inputs: after every replay the outputs and
+    the state equal those of the same calls made eagerly from the same state."""
+    rng = np.random.RandomState(21)
+    shape = (6, 16, 20, 20)
+    x = torch.empty(shape, device=dev)
+    q = lambda v: torch.full((1, 16, 1, 1), v, dtype=torch.float32, device=dev)
+    state = {"lo": q(-3.0), "hi": q(3.0), "m": torch.zeros(1, device=dev), "M": torch.zeros(1, device=dev)}
+    eager_state = {k: v.clone() for k, v in state.items()}
+    ql, qh = q(0.0), q(255.0)
+    scale = torch.full((1, 16, 1, 1), 0.25, device=dev)
+
+    def step(st):
+        y1, s1 = kernels.min_max_quantize(x, st["lo"], st["hi"], ql, qh, 0.9, True, True)
+        y2 = kernels.pow2_quantize(y1, True, True, 4, 1)
+        zp = torch.zeros(1, 16, 1, 1, device=dev)
+        y3 = kernels.quantize_linear(x, scale, zp, "HALF_TO_EVEN", False, kernels.DTYPE_BYTE)
+        y4 = kernels.dequantize_linear(y3, scale, zp)
+        y5 = kernels.prune(x, 0.6)
+        y6 = kernels.range_recorder(x, st["m"], st["M"], "MinMaxMvaRecorder", 0.9, True)
+        return y1, s1, y2, y3, y4, y5, y6
+
+    x.copy_(_dev(rng.randn(*shape).astype(np.float32), dev))
+    warm = {k: v.clone() for k, v in state.items()}
+    step(warm)                                # first calls outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step(state)
+    for k in state:                            # the capture ran nothing: the state is still the initial one
+        assert torch.equal(state[k], eager_state[k])
+    for i in range(4):
+        x.copy_(_dev((rng.randn(*shape) * (i + 1)).astype(np.float32), dev))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [to_np(o).copy() for o in outs]
+        eager = step(eager_state)
+        torch.cuda.synchronize()
+        for j, (g, e) in enumerate(zip(got, eager)):
+            assert bits_equal(g, to_np(e)), "replay %d: output %d differs from the eager result" % (i, j)
+        for k in state:
+            assert bits_equal(to_np(state[k]), to_np(eager_state[k])), "replay %d: state %s" % (i, k)
