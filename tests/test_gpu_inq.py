@@ -375,3 +375,41 @@ def test_inq_config5_layer(dev):
     rows, cols = rng.choice(1024, 32, replace=False), rng.choice(4096, 64, replace=False)
     ref = x[rows].astype(np.float64) @ Wc[:, cols].astype(np.float64)
     assert np.abs(y[np.ix_(rows, cols)] - ref).max() / np.abs(ref).max() <= TIGHT
+
+
+def test_inq_affine_replays_in_a_hip_graph(dev):
+    """INQAffine forward between selection steps (weights partly fixed, partly learnt) and once every weight is fixed,
+    captured once each and replayed after the learnable weights and the input changed: the replay's output, weights
+    and snapshot are those of the eager call (its passes clear and fill counters on the device and never
+    synchronise)."""
+    rng = np.random.RandomState(23)
+    M, K, N = 96, 256, 384
+    x = torch.empty(M, K, device=dev)
+    for fix_all in (False, True):
+        Wh = (rng.randn(K, N) * 0.05).astype(np.float32)
+        W, I = _dev(Wh, dev), torch.zeros((K, N), dtype=torch.int32, device=dev)
+        oW, oI = torch.zeros_like(W), torch.zeros_like(I)
+        x.copy_(_dev(rng.randn(M, K).astype(np.float32), dev))
+        # one selection step outside the capture: half of the weights (or all of them) become fixed
+        kernels.inq_affine(x, W, I, oW, oI, None, 4, kernels.INQ_FIX_ALL if fix_all else kernels.INQ_LARGEST_ABS)
+        kernels.inq_affine(x, W, I, oW, oI, None, 4, kernels.INQ_NO_SELECTION)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y = kernels.inq_affine(x, W, I, oW, oI, None, 4, kernels.INQ_NO_SELECTION)
+        for i in range(3):
+            x.copy_(_dev((rng.randn(M, K) * (i + 1)).astype(np.float32), dev))
+            # a training step moved the weights (the fixed ones are put back by the forward)
+            W.add_(_dev((rng.randn(K, N) * 0.01).astype(np.float32), dev))
+            before = [t.clone() for t in (W, I, oW, oI)]
+            graph.replay()
+            torch.cuda.synchronize()
+            got = [to_np(t).copy() for t in (y, W, I, oW, oI)]
+            for t, b in zip((W, I, oW, oI), before):
+                t.copy_(b)
+            ye = kernels.inq_affine(x, W, I, oW, oI, None, 4, kernels.INQ_NO_SELECTION)
+            torch.cuda.synchronize()
+            for g, e, name in zip(got, (ye, W, I, oW, oI), ("y", "W", "I", "old W", "old I")):
+                assert bits_equal(g, to_np(e)), "fix_all %s replay %d: %s differs" % (fix_all, i, name)
+            ref = to_np(x).astype(np.float64) @ to_np(W).astype(np.float64)
+            assert np.abs(got[0] - ref).max() / np.abs(ref).max() <= TIGHT
