@@ -199,3 +199,84 @@ def test_prune(ctx, rate):
         y = F.prune(_var(x), rate)
         y.forward()
         assert bits_equal(y.d, oracle.prune(x, rate))
+
+
+# test_inq_affine.py:119-122 (forward / backward from random indicators) and :150-155 (recomputation)
+@pytest.mark.parametrize("base_axis,weight_shape,num_bits",
+                         [(1, (12, 2, 3), 2), (2, (4, 4), 4), (-2, (12, 2, 3), 2), (-1, (4, 4), 4)])
+@pytest.mark.parametrize("bias", [True, False])
+@pytest.mark.parametrize("inq_iterations", [(10, 20), (0,), (0, 10)])
+def test_inq_affine(ctx, base_axis, weight_shape, num_bits, bias, inq_iterations):
+    rng = np.random.RandomState(313)
+    x, W, b, axis, rows = _affine_case(rng, (2, 3, 4), weight_shape, base_axis, bias)
+    I = rng.randint(2, size=weight_shape).astype(np.int32)
+    n = int(np.prod(weight_shape[1:]))
+    xv, wv = _var(x, True), _var(W, True)
+    iv = nn.Variable(weight_shape)
+    iv.set_data(I, np.int32)
+    bv = _var(b, True) if bias else None
+    y = F.inq_affine(xv, wv, iv, bv, base_axis, num_bits, inq_iterations, 'largest_abs', 313)
+    y.forward()
+    inq = oracle.Inq(W.size, num_bits, inq_iterations, 'largest_abs', 313)
+    Wc, Ic = W.reshape(W.shape[0], -1).copy(), I.reshape(W.shape[0], -1).copy()
+    ref_y = inq.affine(x.reshape(rows, -1), Wc, Ic, None if b is None else b.ravel())
+    assert np.array_equal(iv.d.astype(np.int32).reshape(Ic.shape), Ic)
+    assert bits_equal(wv.d.reshape(Wc.shape), Wc)
+    assert max_rel_err(y.d.reshape(rows, n), ref_y) <= TIGHT
+    dy = rng.randn(*y.shape).astype(np.float32)
+    y.backward(dy)
+    rdx, rdw, rdb = oracle.affine_backward(dy.reshape(rows, n), x.reshape(rows, -1), Wc)
+    assert max_rel_err(xv.g.reshape(rows, -1), rdx) <= TIGHT and max_rel_err(wv.g.reshape(Wc.shape), rdw) <= TIGHT
+    if bias:
+        assert max_rel_err(bv.g.ravel(), rdb) <= TIGHT
+
+
+@pytest.mark.parametrize("base_axis,weight_shape,num_bits", [(1, (12, 2, 3), 2), (2, (4, 4), 4)])
+@pytest.mark.parametrize("selection_algorithm", ["largest_abs", "random"])
+@pytest.mark.parametrize("func_seed", [-1, 412])
+def test_inq_affine_recomputation(ctx, base_axis, weight_shape, num_bits, selection_algorithm, func_seed):
+    """The output recomputed after a forward (weights, indicators and counter left as they are) equals the forward's
+    (nbla_test_utils.recomputation_test), also at a selection step and with the generator seeded by the clock."""
+    rng = np.random.RandomState(313)
+    x, W, _, _, _ = _affine_case(rng, (2, 3, 4), weight_shape, base_axis, False)
+    iv = nn.Variable(weight_shape)
+    iv.set_data(rng.randint(2, size=weight_shape), np.int32)
+    wv = _var(W)
+    y = F.inq_affine(_var(x), wv, iv, None, base_axis, num_bits, (1,), selection_algorithm, func_seed)
+    for _ in range(3):                     # the second forward is the selection step
+        y.forward()
+        out, w_after, i_after = y.d.copy(), wv.d.copy(), iv.d.copy()
+        y.parent.recompute()
+        assert bits_equal(y.d, out) and bits_equal(wv.d, w_after) and np.array_equal(iv.d, i_after)
+
+
+# test_inq_convolution.py:123-128
+@pytest.mark.parametrize("group", [1, 2])
+@pytest.mark.parametrize("with_bias", [True, False])
+@pytest.mark.parametrize("base_axis", [1, -3])
+@pytest.mark.parametrize("inq_iterations", [(10, 20), (0,), (0, 10)])
+def test_inq_convolution(ctx, group, with_bias, base_axis, inq_iterations):
+    rng = np.random.RandomState(313)
+    inshape, kernel, outmaps, pad, stride, dilation, num_bits = (2, 2, 10, 10), (3, 2), 4, (3, 0), (1, 2), (2, 1), 3
+    x = rng.randn(*inshape).astype(np.float32)
+    W = rng.randn(outmaps, inshape[1] // group, *kernel).astype(np.float32)
+    I = rng.randint(2, size=W.shape).astype(np.int32)
+    b = rng.randn(outmaps).astype(np.float32) if with_bias else None
+    xv, wv = _var(x, True), _var(W, True)
+    iv = nn.Variable(W.shape)
+    iv.set_data(I, np.int32)
+    bv = _var(b, True) if with_bias else None
+    y = F.inq_convolution(xv, wv, iv, bv, base_axis, pad, stride, dilation, group, num_bits, inq_iterations,
+                          'largest_abs', 313)
+    y.forward()
+    inq = oracle.Inq(W.size, num_bits, inq_iterations, 'largest_abs', 313)
+    Wc, Ic = W.copy(), I.copy()
+    ref_y = inq.convolution(x, Wc, Ic, b, pad, stride, dilation, group)
+    assert np.array_equal(iv.d.astype(np.int32), Ic) and bits_equal(wv.d, Wc)
+    assert y.shape == ref_y.shape and max_rel_err(y.d, ref_y) <= TIGHT
+    dy = rng.randn(*y.shape).astype(np.float32)
+    y.backward(dy)
+    rdx, rdw, rdb = oracle.convolution_backward(dy, x, Wc, pad, stride, dilation, group)
+    assert max_rel_err(xv.g, rdx) <= TIGHT * 4 and max_rel_err(wv.g, rdw) <= TIGHT
+    if with_bias:
+        assert max_rel_err(bv.g, rdb) <= TIGHT
