@@ -280,3 +280,69 @@ def test_inq_convolution(ctx, group, with_bias, base_axis, inq_iterations):
     assert max_rel_err(xv.g, rdx) <= TIGHT * 4 and max_rel_err(wv.g, rdw) <= TIGHT
     if with_bias:
         assert max_rel_err(bv.g, rdb) <= TIGHT
+
+
+# test_fixed_point_quantize.py:67-71 and test_pow2_quantize.py:75-80
+@pytest.mark.parametrize("sign", [False, True])
+@pytest.mark.parametrize("n", [3, 8])
+@pytest.mark.parametrize("delta", [2 ** -7, 0.005])
+@pytest.mark.parametrize("quantize", [False, True])
+@pytest.mark.parametrize("ste_fine_grained", [False, True])
+def test_fixed_point_quantize(ctx, sign, n, delta, quantize, ste_fine_grained):
+    rng = np.random.RandomState(313)
+    x = rng.randn(2, 3, 4).astype(np.float32)
+    xv = _var(x, True)
+    with nn.auto_forward(False):
+        y = F.fixed_point_quantize(xv, sign, n, delta, quantize, ste_fine_grained)
+    if not quantize:
+        assert y is xv                      # the reference returns its input (functions.py: `if not quantize`)
+        return
+    y.forward()
+    assert bits_equal(y.d, oracle.fixed_point_quantize(x, sign, n, delta))
+    dy = rng.randn(2, 3, 4).astype(np.float32)
+    y.backward(dy)
+    assert np.array_equal(xv.g, oracle.fixed_point_quantize_backward(dy, x, sign, n, delta, ste_fine_grained))
+
+
+@pytest.mark.parametrize("sign", [False, True])
+@pytest.mark.parametrize("with_zero", [False, True])
+@pytest.mark.parametrize("n", [3, 5])
+@pytest.mark.parametrize("m", [0, 1])
+@pytest.mark.parametrize("quantize", [False, True])
+@pytest.mark.parametrize("ste_fine_grained", [False, True])
+def test_pow2_quantize(ctx, sign, with_zero, n, m, quantize, ste_fine_grained):
+    rng = np.random.RandomState(313)
+    x = rng.randn(2, 3, 4).astype(np.float32)
+    xv = _var(x, True)
+    y = F.pow2_quantize(xv, sign, with_zero, n, m, quantize, ste_fine_grained)
+    if not quantize:
+        assert y is xv
+        return
+    y.forward()
+    assert bits_equal(y.d, oracle.pow2_quantize(x, sign, with_zero, n, m))
+    dy = rng.randn(2, 3, 4).astype(np.float32)
+    y.backward(dy)
+    assert np.array_equal(xv.g, oracle.pow2_quantize_backward(dy, x, sign, with_zero, n, m, ste_fine_grained))
+
+
+# test_min_max_quantize.py:114-126
+@pytest.mark.parametrize("x_shape,q_shape", [((4, 8, 16, 16), (1, 1, 1, 1)), ((4, 8, 16, 16), (1, 8, 1, 1)),
+                                             ((16, 8, 3, 3), (16, 1, 1, 1))])
+@pytest.mark.parametrize("decay", [0.999, 0.9])
+@pytest.mark.parametrize("x_min_max", [True, False])
+@pytest.mark.parametrize("ema", [True, False])
+@pytest.mark.parametrize("ste_fine_grained", [True, False])
+def test_min_max_quantize(ctx, x_shape, q_shape, decay, x_min_max, ema, ste_fine_grained):
+    rng = np.random.RandomState(313)
+    x = rng.randn(*x_shape).astype(np.float32)
+    qmn, qmx = np.full(q_shape, -0.5, np.float32), np.full(q_shape, 0.5, np.float32)
+    lmn, lmx = np.zeros(q_shape, np.float32), np.full(q_shape, 255, np.float32)
+    xv, lo, hi = _var(x, True), _var(qmn), _var(qmx)
+    y = F.min_max_quantize(xv, lo, hi, _var(lmn), _var(lmx), decay, x_min_max, ema, ste_fine_grained, 0.01)
+    y.forward()
+    ref_y, rmn, rmx, rscale = oracle.min_max_quantize(x, qmn, qmx, lmn, lmx, decay, x_min_max, ema, 0.01)
+    assert bits_equal(y.d, ref_y) and bits_equal(lo.d, rmn) and bits_equal(hi.d, rmx)
+    dy = rng.randn(*x_shape).astype(np.float32)
+    y.backward(dy)
+    rdx, _, _ = oracle.min_max_quantize_backward(dy, x, rmn, rmx, lmn, lmx, rscale, ste_fine_grained, x_min_max, ema)
+    assert np.array_equal(xv.g, rdx)
