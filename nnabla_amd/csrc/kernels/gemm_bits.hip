@@ -1125,9 +1125,11 @@ template <int BM, int BN, int kWavesM, int kWavesN, int kWavesK, bool kSwap>
 int launch_tile(const GemmBitsArgs &args, hipStream_t stream, unsigned splits = 1) {
   constexpr int kThreads = kWavesM * kWavesN * kWavesK * 64;
   constexpr int kSmem = gemm_bits_lds_bytes(BM, BN, kWavesM, kWavesN, kWavesK) + gemm_bits_epilogue_bytes(BM, BN);
-  auto kernel = gemm_bits_kernel<BM, BN, kWavesM, kWavesN, kWavesK, kSwap>;
+  // the kernel is named at each launch, not held in a pointer: a launch through a pointer is an indirect call of
+  // the host-side stub, which -fsanitize=function builds instrument (and then drop)
+#define NBLA_GEMM_BITS_KERNEL gemm_bits_kernel<BM, BN, kWavesM, kWavesN, kWavesK, kSwap>
   static std::atomic<uint64_t> configured{0};
-  const int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), kSmem, configured,
+  const int rc = allow_dynamic_lds(reinterpret_cast<const void *>(&NBLA_GEMM_BITS_KERNEL), kSmem, configured,
                                    "hipFuncSetAttribute(gemm_bits LDS size)");
   if (rc)
     return rc;
@@ -1136,12 +1138,13 @@ int launch_tile(const GemmBitsArgs &args, hipStream_t stream, unsigned splits = 
   a.blocks_n = ceil_div(a.n_end - a.n_begin, BN);
   const dim3 grid((unsigned)(a.blocks_m * a.blocks_n), splits);
   if (t_timer.used < t_timer.start.size()) {
-    hipExtLaunchKernelGGL(kernel, grid, dim3(kThreads), kSmem, stream, t_timer.start[t_timer.used],
+    hipExtLaunchKernelGGL((NBLA_GEMM_BITS_KERNEL), grid, dim3(kThreads), kSmem, stream, t_timer.start[t_timer.used],
                           t_timer.stop[t_timer.used], 0, a);
     ++t_timer.used;
   } else {
-    hipLaunchKernelGGL(kernel, grid, dim3(kThreads), kSmem, stream, a);
+    hipLaunchKernelGGL((NBLA_GEMM_BITS_KERNEL), grid, dim3(kThreads), kSmem, stream, a);
   }
+#undef NBLA_GEMM_BITS_KERNEL
   NBLA_HIP_LAUNCH_CHECK("gemm_bits");
   return NBLA_HIP_OK;
 }
