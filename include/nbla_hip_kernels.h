@@ -372,7 +372,10 @@ int nbla_hip_binary_convolution_slab_plan(
  * src/nbla/function/generic/binary_weight_convolution.cpp:73-117 (alpha per
  * output channel with the rounded reciprocal of col_w, :66) and the im2col +
  * per-sample Eigen product of convolution.cpp:161-197 / unfold_to_patches.cpp.
- * Argument errors as convolution.cpp:61-103.  Never synchronises: a
+ * Argument errors as convolution.cpp:61-103.  A window of x that holds a NaN
+ * or an infinity gives what the reference's product gives output by output
+ * (+-Inf by the weight's sign, NaN for Inf - Inf): its outputs are recomputed
+ * in fp32 over Wb.  Never synchronises: a
  * quantize_zero_to that is neither +1 nor -1 is handled on the device, as in
  * nbla_hip_binary_weight_affine_f32 (per group: unfold + fp32 product over Wb
  * behind the matrix-core product, with the group's count of weights that are

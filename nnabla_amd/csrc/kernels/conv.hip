@@ -724,6 +724,51 @@ int launch_im2col_f32(const float *x, float *col, const ConvGeom &g, int64_t grp
 
 namespace {
 
+// Windows holding a NaN or an infinity (shift[m] == kBadRow): the digit products leave NaN in all their outputs, while
+// the reference's product propagates such values output by output (convolution.cpp:185-193: the row of the unfolded
+// input times Ws = Wb * alpha, then + b: Inf * w = +-Inf, Inf - Inf = NaN).  Those windows -- rare -- are recomputed
+// here as plain fp32 dot products over the materialised signs of the group, Wbg [Og, Kg]; yg is the group's first
+// output map.  A block looks at 256 marks at a time and leaves at once when none of them is set.
+__global__ __launch_bounds__(256) void conv_redo_marked_windows(const float *__restrict__ x,
+                                                                const float *__restrict__ Wbg,
+                                                                const float *__restrict__ alpha,
+                                                                const float *__restrict__ bias, float *__restrict__ yg,
+                                                                const int32_t *__restrict__ shift, ConvGeom g,
+                                                                int64_t grp) {
+  for (int64_t base = (int64_t)blockIdx.x * 256; base < g.M; base += (int64_t)gridDim.x * 256) {
+    const int64_t mine = base + threadIdx.x;
+    const int marked = mine < g.M && shift[mine] == kBadRow;
+    if (!__syncthreads_or(marked))
+      continue;
+    const int64_t end = base + 256 < g.M ? base + 256 : g.M;
+    for (int64_t m = base; m < end; ++m) {
+      if (shift[m] != kBadRow) // uniform over the block
+        continue;
+      const int64_t n = m / g.out_sp_size, pos = m - n * g.out_sp_size;
+      for (int64_t o = threadIdx.x; o < g.Og; o += 256) {
+        const float a = alpha ? alpha[o] : 1.0f;
+        float acc = 0.0f;
+        for (int64_t k = 0; k < g.Kg; ++k) {
+          const float w = alpha ? Wbg[o * g.Kg + k] * a : Wbg[o * g.Kg + k]; // the scaled weight of the reference
+          acc = acc + col_value(x, g, grp, m, k) * w;
+        }
+        yg[(n * g.O + o) * g.out_sp_size + pos] = bias ? acc + bias[o] : acc;
+      }
+    }
+  }
+}
+
+int launch_conv_redo(const float *x, const float *Wbg, const float *alpha, const float *bias, float *yg,
+                     const int32_t *shift, const ConvGeom &g, int64_t grp, hipStream_t stream) {
+  int64_t blocks = ceil_div(g.M, 256);
+  if (blocks > 1024)
+    blocks = 1024;
+  hipLaunchKernelGGL(conv_redo_marked_windows, dim3((unsigned)blocks), dim3(256), 0, stream, x, Wbg, alpha, bias, yg,
+                     shift, g, grp);
+  NBLA_HIP_LAUNCH_CHECK("conv_redo_marked_windows");
+  return NBLA_HIP_OK;
+}
+
 struct ConvWorkspace {
   size_t bits_off, bits_stride, split_off, cmax_off, prep_off, count_off, tap_bits_off, tap_bits_stride, col_off, total;
 };
@@ -792,18 +837,27 @@ int binary_conv_forward(const float *x, const float *W, float *Wb, float *alpha,
       if (rc)
         return rc;
       rc = launch_conv_slab(x, g, grp, prepared, alpha ? alpha + grp * g.Og : nullptr,
-                            representable ? nullptr : counts + grp, bg, y, stream);
-    } else if (gemm_bits_unfold_applies(g)) {
-      rc = launch_gemm_bits_unfold(x, g, grp,
-                                   reinterpret_cast<const uint32_t *>(base + ws.bits_off + grp * ws.bits_stride), ag, bg,
-                                   yg, stream);
+                            representable ? nullptr : counts + grp, bg, y, stream, nullptr, false,
+                            Wb + grp * g.Og * g.Kg);
     } else {
-      rc = launch_im2col_digits(x, base + ws.split_off, base + ws.cmax_off, g, grp, stream);
+      // the rows' marks sit where the digit operand keeps its scale exponents (the fused unfold has no other use for
+      // that space)
+      int32_t *shift = reinterpret_cast<int32_t *>(base + ws.split_off + digit_operand(g.M, g.Kg).shift_off);
+      if (gemm_bits_unfold_applies(g)) {
+        rc = launch_gemm_bits_unfold(x, g, grp,
+                                     reinterpret_cast<const uint32_t *>(base + ws.bits_off + grp * ws.bits_stride), ag,
+                                     bg, yg, stream, shift);
+      } else {
+        rc = launch_im2col_digits(x, base + ws.split_off, base + ws.cmax_off, g, grp, stream);
+        if (rc)
+          return rc;
+        rc = launch_gemm_bits(base + ws.split_off,
+                              reinterpret_cast<const uint32_t *>(base + ws.bits_off + grp * ws.bits_stride), ag, bg,
+                              yg, g.M, g.Kg, g.Og, hw, g.O * hw, hw, true, stream);
+      }
       if (rc)
         return rc;
-      rc = launch_gemm_bits(base + ws.split_off,
-                            reinterpret_cast<const uint32_t *>(base + ws.bits_off + grp * ws.bits_stride), ag, bg, yg,
-                            g.M, g.Kg, g.Og, hw, g.O * hw, hw, true, stream);
+      rc = launch_conv_redo(x, Wb + grp * g.Og * g.Kg, ag, bg, yg, shift, g, grp, stream);
     }
     if (rc)
       return rc;

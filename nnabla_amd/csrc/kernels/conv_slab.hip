@@ -75,6 +75,8 @@ struct ConvSlabArgs {
   int *zero_count;    // may be null
   const float *bias;
   const float *in_scale; // may be null: input channel c of the group is multiplied by in_scale[c] first
+  const float *redo_w;   // may be null: Sign(W) of the group [Og, Cg * taps]; windows holding a NaN or an infinity are
+                         // then recomputed element by element (else all their outputs are NaN)
   float *y;
   int accumulate;        // add to y instead of overwriting it
   ConvGeom g;
@@ -530,6 +532,40 @@ __global__ __launch_bounds__(kSlabThreads, 1) void binary_conv_slab_kernel(ConvS
     if (cq < og_left)
       ybase[cq * osz] = v; // (Og * out_sp_size < 2^31: checked by the host)
   }
+  // A window holding a NaN or an infinity (rare): the reference's product propagates such values output by output
+  // (convolution.cpp:185-193: the row of the unfolded input, zeros where the window leaves the input, times
+  // Ws = Wb * alpha, then + b: Inf * w = +-Inf, Inf - Inf = NaN), so the lane recomputes its sixteen outputs as plain
+  // fp32 dot products over the materialised signs and replaces the NaN stored above.
+  if (rowbad && a.redo_w) {
+    int p = p0 + r;
+    const int o2 = p % g.out_sp[2];
+    p /= g.out_sp[2];
+    const int o1 = p % g.out_sp[1], o0 = p / g.out_sp[1];
+    const int w0 = o0 * g.stride[0] - g.pad[0], w1 = o1 * g.stride[1] - g.pad[1], w2 = o2 * g.stride[2] - g.pad[2];
+    const float *xn = a.x + ((int64_t)n * g.C + (int64_t)a.grp * g.Cg) * plane;
+#pragma unroll 1
+    for (int q = 0; q < 16; ++q) {
+      const int cq = 8 * (q >> 2) + (q & 3);
+      if (cq >= og_left)
+        continue;
+      const float *wrow = a.redo_w + ((int64_t)wg * kWideGroup + c0 + cq) * ((int64_t)Cg * taps);
+      const float scale = s_alpha[c0 + cq];
+      float acc = 0.0f;
+#pragma unroll 1
+      for (int c = 0; c < Cg; ++c) {
+        int t = 0;
+        for (int k0 = 0; k0 < g.k[0]; ++k0)
+          for (int k1 = 0; k1 < g.k[1]; ++k1)
+            for (int k2 = 0; k2 < g.k[2]; ++k2, ++t) {
+              const int i0 = w0 + k0 * g.dil[0], i1 = w1 + k1 * g.dil[1], i2 = w2 + k2 * g.dil[2];
+              const bool in = i0 >= 0 && i0 < in0 && i1 >= 0 && i1 < in1 && i2 >= 0 && i2 < in2;
+              const float xv = in ? xn[(int64_t)c * plane + (i0 * in1 + i1) * in2 + i2] : 0.0f;
+              acc = acc + xv * (wrow[c * taps + t] * scale);
+            }
+      }
+      ybase[cq * osz] = acc + s_bias[c0 + cq];
+    }
+  }
 #endif
 }
 
@@ -875,7 +911,7 @@ int launch_conv_slab_prepare_transposed(const float *Wg, void *prepared, const C
 
 int launch_conv_slab(const float *x, const ConvGeom &g, int64_t grp, const void *prepared, float *alpha_out,
                      int *zero_count, const float *bias, float *y, hipStream_t stream, const float *in_scale,
-                     bool accumulate) {
+                     bool accumulate, const float *redo_w) {
   ConvSlabArgs a;
   if (!make_slab_plan(g, a.p))
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "the slab convolution does not cover this geometry.");
@@ -898,6 +934,7 @@ int launch_conv_slab(const float *x, const ConvGeom &g, int64_t grp, const void 
   a.zero_count = zero_count;
   a.bias = bias;
   a.in_scale = in_scale;
+  a.redo_w = (in_scale || accumulate) ? nullptr : redo_w;
   a.accumulate = accumulate ? 1 : 0;
   a.y = y;
   a.g = g;

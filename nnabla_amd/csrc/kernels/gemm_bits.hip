@@ -63,6 +63,8 @@ struct GemmBitsArgs {
   ConvGeom ug;
   int64_t ugrp;
   const int *skip_if; // non-zero word: the launch does nothing (may be null)
+  int32_t *shift_out; // unfolding product only (may be null): the rows' scale exponents, kBadRow for a window holding
+                      // a NaN or an infinity, written for the caller that recomputes such windows
 };
 
 // LDS buffers (stages resident) per tile shape: what fits the block's share of the CU's 160 KiB, at most six.
@@ -410,6 +412,8 @@ __device__ __forceinline__ void unfold_main_loop(const GemmBitsArgs &a, unsigned
         --s;
     }
     s_shift[tid] = s;
+    if (a.shift_out && bn == 0 && in_range)
+      a.shift_out[m] = s;
     // the row's taps as byte offsets into x; a row holding a NaN or an infinity is not read (its outputs become NaN
     // in the epilogue), nor is a tap outside the input
     const uint32_t first = (uint32_t)(((n * g.C + a.ugrp * g.Cg) * g.in_sp_size + origin) * 4);
@@ -1271,6 +1275,7 @@ int launch_gemm_bits(const void *xdigits, const uint32_t *bits, const float *alp
   a.use_sums = 1;
   a.keep_bad_rows = keep_bad_rows ? 1 : 0;
   a.skip_if = skip_if;
+  a.shift_out = nullptr;
   a.ux = nullptr;
   a.ugrp = 0;
   a.inner = inner;
@@ -1310,7 +1315,7 @@ bool gemm_bits_unfold_applies(const ConvGeom &g) {
 }
 
 int launch_gemm_bits_unfold(const float *x, const ConvGeom &g, int64_t grp, const uint32_t *bits, const float *alpha,
-                            const float *bias, float *y, hipStream_t stream) {
+                            const float *bias, float *y, hipStream_t stream, int32_t *row_shift) {
   if (!gemm_bits_unfold_applies(g))
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "the fused unfold product does not cover this geometry.");
   if (!aligned16(bits))
@@ -1353,6 +1358,7 @@ int launch_gemm_bits_unfold(const float *x, const ConvGeom &g, int64_t grp, cons
   a.use_sums = 1;
   a.keep_bad_rows = 0;
   a.skip_if = nullptr;
+  a.shift_out = row_shift;
   a.ux = x;
   a.ug = g;
   a.ugrp = grp;

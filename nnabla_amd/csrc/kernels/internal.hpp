@@ -30,11 +30,12 @@ int launch_gemm_bits(const void *xsplit, const uint32_t *bits, const float *alph
                      size_t split_ws_bytes = 0, bool keep_bad_rows = false, const int *skip_if = nullptr);
 // The same product for a convolution with the unfold fused in: the rows are the unfolded windows of x (group `grp`),
 // converted to digits inside the kernel; y is [sample, O, output position].  gemm_bits_unfold_applies tells whether
-// the geometry is covered (otherwise: launch_im2col_digits + launch_gemm_bits).
+// the geometry is covered (otherwise: launch_im2col_digits + launch_gemm_bits).  row_shift (may be null): M words that
+// receive the rows' scale exponents, kBadRow for a window holding a NaN or an infinity (all its outputs are NaN).
 struct ConvGeom;
 bool gemm_bits_unfold_applies(const ConvGeom &g);
 int launch_gemm_bits_unfold(const float *x, const ConvGeom &g, int64_t grp, const uint32_t *bits, const float *alpha,
-                            const float *bias, float *y, hipStream_t stream);
+                            const float *bias, float *y, hipStream_t stream, int32_t *row_shift = nullptr);
 // The binary convolution forward with the unfold done by LDS addressing (conv_slab.hip), two launches per group:
 // launch_conv_slab_prepare reads the group's weights [Og, Cg, taps] once and writes Wb = Sign(W) (may be null) and,
 // into `prepared` (conv_slab_prepared_bytes, 16-byte aligned), the packed bits in (tap, channel) order with the
@@ -49,10 +50,12 @@ bool conv_slab_plan_summary(const ConvGeom &g, int32_t out[4]);
 int launch_conv_slab_prepare(const float *Wg, float *Wbg, void *prepared, const ConvGeom &g, float zero_to,
                              hipStream_t stream);
 // in_scale (may be null): input channel c of the group is multiplied by in_scale[c] before anything else; accumulate:
-// y += instead of y =.
+// y += instead of y =.  redo_w (may be null; ignored with in_scale or accumulate): the group's Sign(W) [Og, Cg * taps],
+// from which the outputs of a window holding a NaN or an infinity are recomputed one by one as the reference's product
+// gives them; without it all outputs of such a window are NaN.
 int launch_conv_slab(const float *x, const ConvGeom &g, int64_t grp, const void *prepared, float *alpha_out,
                      int *zero_count, const float *bias, float *y, hipStream_t stream, const float *in_scale = nullptr,
-                     bool accumulate = false);
+                     bool accumulate = false, const float *redo_w = nullptr);
 // The same product as the input gradient of a binary convolution of unit stride: conv_slab_transposed_geom gives the
 // geometry of the convolution dx = conv(dy * alpha, flipped Sign(W)^T) (false when the product does not cover it),
 // launch_conv_slab_prepare_transposed writes its packed bits from the group's weights [Og, Cg, taps]

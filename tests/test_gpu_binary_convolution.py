@@ -107,25 +107,56 @@ def test_convolution_quantize_zero_to_with_zero_weights(dev, q0, channels):
     assert max_rel_err(to_np(y), ref_y) <= TIGHT * 4
 
 
-@pytest.mark.parametrize("channels", [8, 32])
-def test_window_with_a_non_finite_value(dev, channels):
-    """An Inf or NaN in x: every output whose window holds it is non-finite in the reference (Inf - Inf and 0 * Inf
-    give NaN, convolution.cpp's gemm); here the digit form gives NaN for all output channels of such a window.  All
-    other outputs are unaffected.  (8 channels: the gathering product; 32: the one that keeps input positions in LDS.)"""
+def _same_non_finite(y, ref):
+    """NaN, +Inf and -Inf at the same places, the finite outputs within the products' tolerance."""
+    assert np.array_equal(np.isnan(y), np.isnan(ref))
+    assert np.array_equal(np.isposinf(y), np.isposinf(ref))
+    assert np.array_equal(np.isneginf(y), np.isneginf(ref))
+    fin = np.isfinite(ref)
+    assert fin.any() and (~fin).any()
+    assert np.abs(y[fin] - ref[fin]).max() / np.abs(ref[fin]).max() <= TIGHT
+
+
+# (x shape, W shape, pad, stride, dilation, group): the product that keeps input positions in LDS (32 channels), the
+# gathering product (8 channels), the unfolded digit matrix (a kernel of 81 taps), and groups / stride / padding
+NON_FINITE_CASES = [
+    ((2, 32, 9, 9), (6, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((2, 64, 9, 9), (300, 32, 3, 3), (1, 1), (1, 1), (1, 1), 2),
+    ((2, 8, 9, 9), (6, 8, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((2, 8, 9, 9), (6, 4, 3, 3), (0, 2), (2, 1), (1, 2), 2),
+    ((2, 4, 12, 12), (5, 4, 9, 9), (4, 4), (1, 1), (1, 1), 1),
+]
+
+
+@pytest.mark.parametrize("xs,ws,pad,stride,dil,group", NON_FINITE_CASES)
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_window_with_a_non_finite_value(dev, xs, ws, pad, stride, dil, group, with_bias):
+    """An Inf or NaN in x: the reference's product propagates it output by output (convolution.cpp:185-193:
+    Inf * w = +-Inf by the weight's sign, Inf - Inf = NaN, NaN anywhere = NaN), and so do the windows recomputed here;
+    two infinities under the same windows make some outputs NaN and others +-Inf.  All other outputs are the ones of
+    the clean input, bit for bit."""
     rng = np.random.RandomState(5)
-    x = rng.randn(2, channels, 9, 9).astype(np.float32)
-    W = (rng.randn(6, channels, 3, 3) * 0.05).astype(np.float32)
-    clean, _, _ = kernels.binary_weight_convolution(_dev(x, dev), _dev(W, dev), None, (1, 1), (1, 1), (1, 1), 1)
+    x = rng.randn(*xs).astype(np.float32)
+    W = (rng.randn(*ws) * 0.05).astype(np.float32)
+    b = rng.randn(ws[0]).astype(np.float32) if with_bias else None
+    bd = _dev(b, dev) if with_bias else None
+    clean, _, _ = kernels.binary_weight_convolution(_dev(x, dev), _dev(W, dev), bd, pad, stride, dil, group)
     x[1, 3, 4, 5] = np.inf
+    x[1, 2, 4, 6] = np.inf
+    x[1, 1, 7, 2] = -np.inf
     x[0, 0, 0, 0] = np.nan
-    y, _, _ = kernels.binary_weight_convolution(_dev(x, dev), _dev(W, dev), None, (1, 1), (1, 1), (1, 1), 1)
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref_y, ref_Wb, ref_alpha = oracle.binary_weight_convolution(x, W, b, pad, stride, dil, group, 1.0)
+    y, Wb, alpha = kernels.binary_weight_convolution(_dev(x, dev), _dev(W, dev), bd, pad, stride, dil, group)
     y, clean = to_np(y), to_np(clean)
-    hit = np.zeros((2, 9, 9), bool)
-    hit[1, 3:6, 4:7] = True
-    hit[0, 0:2, 0:2] = True
-    for o in range(6):
-        assert not np.isfinite(y[:, o][hit]).any()
-        assert bits_equal(y[:, o][~hit], clean[:, o][~hit])
+    _same_non_finite(y, ref_y)
+    touched = ~np.isfinite(ref_y).all(axis=1, keepdims=True) | ~np.isfinite(y).all(axis=1, keepdims=True)
+    keep = np.broadcast_to(~touched, y.shape)
+    assert bits_equal(y[keep], clean[keep])
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref_y, _ = oracle.binary_connect_convolution(x, W, b, pad, stride, dil, group, 1.0)
+    y, _ = kernels.binary_connect_convolution(_dev(x, dev), _dev(W, dev), bd, pad, stride, dil, group)
+    _same_non_finite(to_np(y), ref_y)
 
 
 def test_wide_range_inside_the_positions_under_a_block(dev):
