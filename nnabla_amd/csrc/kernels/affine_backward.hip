@@ -3,6 +3,7 @@
 #include "common.hpp"
 #include "gemm_layout.hpp"
 #include "internal.hpp"
+#include "redo_marked.hpp"
 
 namespace nbla_hip {
 namespace {
@@ -252,7 +253,11 @@ int nbla_hip_affine_digits_f32(const float *x, const float *W, const float *bias
   if (rc)
     return rc;
   char *split = wd + round_up(nbla_hip_digit_operand_bytes(N, K), 256);
-  return launch_gemm_digits(xd, wd, bias, y, M, K, N, 1, N, 1, stream, false, split, gemm_digits_split_bytes(M, K, N));
+  rc = launch_gemm_digits(xd, wd, bias, y, M, K, N, 1, N, 1, stream, false, split, gemm_digits_split_bytes(M, K, N));
+  if (rc)
+    return rc;
+  // rows of x and columns of W holding a NaN or an infinity: their outputs one by one, as affine.cpp:87-95 gives them
+  return launch_product_redo(DenseRows{x, K}, W, N, 1, bias, y, 1, N, 1, xd, wd, M, K, N, stream);
 }
 
 } // extern "C"

@@ -67,32 +67,6 @@ namespace {
 
 typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
-// Value of the unfolded matrix at (pixel m, column k) for group `grp`
-// (unfold_to_patches.cpp:103-194: zero where the tap falls into the padding).
-__device__ __forceinline__ float col_value(const float *__restrict__ x, const ConvGeom &g, int64_t grp, int64_t m,
-                                           int64_t k) {
-  const int64_t n = m / g.out_sp_size;
-  int64_t p = m - n * g.out_sp_size;
-  const int o2 = (int)(p % g.out_sp[2]);
-  p /= g.out_sp[2];
-  const int o1 = (int)(p % g.out_sp[1]);
-  const int o0 = (int)(p / g.out_sp[1]);
-  int64_t t = k;
-  const int k2 = (int)(t % g.k[2]);
-  t /= g.k[2];
-  const int k1 = (int)(t % g.k[1]);
-  t /= g.k[1];
-  const int k0 = (int)(t % g.k[0]);
-  const int64_t c = grp * g.Cg + t / g.k[0];
-  const int i0 = o0 * g.stride[0] + k0 * g.dil[0] - g.pad[0];
-  const int i1 = o1 * g.stride[1] + k1 * g.dil[1] - g.pad[1];
-  const int i2 = o2 * g.stride[2] + k2 * g.dil[2] - g.pad[2];
-  if ((unsigned)i0 >= (unsigned)g.in_sp[0] || (unsigned)i1 >= (unsigned)g.in_sp[1] ||
-      (unsigned)i2 >= (unsigned)g.in_sp[2])
-    return 0.0f;
-  return x[(n * g.C + c) * g.in_sp_size + ((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2] + i2];
-}
-
 // ---- digit operand of the unfolded matrix (the int8 bit-weight product)
 __device__ __forceinline__ int to_fixed(float v, int s) { return (int)rintf(ldexpf(v, s)); }
 

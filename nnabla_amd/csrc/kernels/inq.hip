@@ -11,6 +11,7 @@
 #include "gemm_layout.hpp"
 #include "internal.hpp"
 #include "radix_select.hpp"
+#include "redo_marked.hpp"
 
 #include <cmath>
 #include <vector>
@@ -793,8 +794,13 @@ int nbla_hip_inq_affine_f32(const float *x, float *W, int32_t *I, float *old_W, 
                  : launch_split_digits_columns(W, N, base + p.planes_off, K, N, true, stream);
   if (rc)
     return rc;
-  return launch_gemm_digits(base + p.split_off, base + p.planes_off, bias, y, M, K, N, 1, N, 1, stream, false,
-                            base + p.extra_off, gemm_digits_split_bytes(M, K, N));
+  rc = launch_gemm_digits(base + p.split_off, base + p.planes_off, bias, y, M, K, N, 1, N, 1, stream, false,
+                          base + p.extra_off, gemm_digits_split_bytes(M, K, N));
+  if (rc)
+    return rc;
+  // rows of x and columns of W holding a NaN or an infinity: their outputs one by one, as affine.cpp:87-95 gives them
+  return launch_product_redo(DenseRows{x, K}, W, N, 1, bias, y, 1, N, 1, base + p.split_off, base + p.planes_off, M, K,
+                             N, stream);
 }
 
 size_t nbla_hip_inq_convolution_workspace_bytes(int64_t outer, int64_t C, int nd, const int64_t *in_sp, int64_t O,
@@ -846,6 +852,13 @@ int nbla_hip_inq_convolution_f32(const float *x, float *W, int32_t *I, float *ol
     rc = launch_gemm_digits(base + p.split_off, base + p.planes_off, bias ? bias + grp * g.Og : nullptr,
                             y + grp * g.Og * hw, g.M, g.Kg, g.Og, hw, g.O * hw, hw, stream, false,
                             base + p.extra_off + cmax_bytes, gemm_digits_split_bytes(g.M, g.Kg, g.Og));
+    if (rc)
+      return rc;
+    // windows of x and output channels of W holding a NaN or an infinity: their outputs one by one
+    // (convolution.cpp:185-193)
+    rc = launch_product_redo(UnfoldedRows{x, g, grp}, W + grp * g.Og * g.Kg, 1, g.Kg,
+                             bias ? bias + grp * g.Og : nullptr, y + grp * g.Og * hw, hw, g.O * hw, hw,
+                             base + p.split_off, base + p.planes_off, g.M, g.Kg, g.Og, stream);
     if (rc)
       return rc;
   }

@@ -513,22 +513,47 @@ def test_plain_affine_f32(dev):
         assert max_rel_err(yd, y64) <= TIGHT
 
 
+def _same_non_finite(y, ref, tol):
+    """NaN, +Inf and -Inf at the same places, the finite outputs within the product's tolerance."""
+    assert np.array_equal(np.isnan(y), np.isnan(ref))
+    assert np.array_equal(np.isposinf(y), np.isposinf(ref))
+    assert np.array_equal(np.isneginf(y), np.isneginf(ref))
+    fin = np.isfinite(ref)
+    assert fin.any() and (~fin).any()
+    assert np.abs(y[fin] - ref[fin]).max() / np.abs(ref[fin]).max() <= tol
+
+
 def test_affine_digits_special_rows_and_narrow_weights(dev):
-    """Rows of x or columns of W holding NaN / Inf give NaN outputs for that row / column only; weights that are all
-    zero or powers of two within six binades per column take the three-product form and are multiplied exactly."""
+    """Rows of x or columns of W holding NaN / Inf: the outputs they reach are the reference's, one by one
+    (affine.cpp:87-95: Inf * w = +-Inf by the signs, Inf - Inf = NaN, 0 * Inf = NaN, NaN anywhere = NaN), all others
+    untouched; weights that are all zero or powers of two within six binades per column take the three-product form and
+    are multiplied exactly."""
     rng = np.random.RandomState(8)
     x = rng.randn(70, 200).astype(np.float32)
     W = (rng.randn(200, 90) * 0.1).astype(np.float32)
+    b = rng.randn(90).astype(np.float32)
+    clean = to_np(kernels.affine_digits(_dev(x, dev), _dev(W, dev), _dev(b, dev)))
     x[3, 5] = np.inf
+    x[3, 9] = np.inf        # with x[3, 5]: +-Inf or NaN by the signs of W[5, n] and W[9, n]
+    x[40, 0] = -np.inf
+    x[69, 199] = np.nan
     W[7, 11] = np.nan
-    y = to_np(kernels.affine_digits(_dev(x, dev), _dev(W, dev)))
-    assert np.isnan(y[3]).all() and np.isnan(y[:, 11]).all()
+    W[8, 12] = np.inf
+    x[9, 8] = 0.0           # 0 * Inf
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref = oracle.affine(x, W, b)
+    y = to_np(kernels.affine_digits(_dev(x, dev), _dev(W, dev), _dev(b, dev)))
+    _same_non_finite(y, ref, TIGHT)
+    assert np.isnan(y[9, 12]) and np.isnan(y[:, 11]).all() and np.isinf(y[3]).any() and np.isnan(y[3]).any()
     ok = np.ones_like(y, bool)
-    ok[3], ok[:, 11] = False, False
-    xf, Wf = x.copy(), W.copy()
-    xf[3, 5], Wf[7, 11] = 0, 0
-    ref = xf.astype(np.float64) @ Wf.astype(np.float64)
-    assert np.isfinite(y[ok]).all() and np.abs(y - ref)[ok].max() / np.abs(ref[ok]).max() <= TIGHT
+    ok[[3, 9, 40, 69]] = False
+    ok[:, [11, 12]] = False
+    assert bits_equal(y[ok], clean[ok])
+    for M in (3, 300):      # the contraction spread over the CUs (few rows), and more than one block of marks
+        xm = np.tile(x, (5, 1))[:M]
+        with np.errstate(invalid="ignore", over="ignore"):
+            ref = oracle.affine(xm, W, None)
+        _same_non_finite(to_np(kernels.affine_digits(_dev(xm, dev), _dev(W, dev))), ref, TIGHT)
     # powers of two: exponents within 6 of the column's largest, some zeros, both signs
     e = rng.randint(-9, -3, size=(200, 90))
     Wp = (np.where(rng.rand(200, 90) < 0.2, 0.0, 2.0 ** e) * rng.choice([-1.0, 1.0], size=(200, 90))).astype(np.float32)

@@ -340,6 +340,41 @@ def test_convolution_with_fixed_weights_takes_the_one_digit_form(dev):
     assert max_rel_err(y6, oracle.convolution(x, W6, None, (1, 1), (1, 1), None, 1)) <= TIGHT
 
 
+@pytest.mark.parametrize("xs,ws,pad,stride,group", [
+    ((2, 8, 9, 9), (6, 8, 3, 3), (1, 1), (1, 1), 1),
+    ((3, 6, 10, 7), (8, 3, 3, 2), (0, 1), (2, 1), 2),
+])
+def test_convolution_with_non_finite_values(dev, xs, ws, pad, stride, group):
+    """A window of x or an output channel of W holding NaN / Inf: the outputs they reach are the reference's, one by
+    one (convolution.cpp:185-193), the others those of the clean operands bit for bit; through the product-only step
+    that Convolution runs, and through INQConvolution's forward with every weight still being learnt."""
+    rng = np.random.RandomState(9)
+    x = rng.randn(*xs).astype(np.float32)
+    W = (rng.randn(*ws) * 0.1).astype(np.float32)
+    b = rng.randn(ws[0]).astype(np.float32)
+
+    def run(xh, Wh, step):
+        Wd = _dev(Wh, dev)
+        I = torch.zeros(ws, dtype=torch.int32, device=dev)
+        return to_np(kernels.inq_convolution(_dev(xh, dev), Wd, I, Wd.clone(), I.clone(), _dev(b, dev), pad, stride,
+                                             None, group, 4, step))
+    clean = run(x, W, kernels.INQ_PRODUCT_ONLY)
+    x[1, 2, 4, 5] = np.inf
+    x[1, 1, 4, 6] = np.inf
+    x[0, 0, 0, 0] = np.nan
+    x[1, 0, 8, 1] = -np.inf
+    W[4, 1, 2, 0] = np.inf
+    W[1, 0, 0, 1] = np.nan
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref = oracle.convolution(x, W, b, pad, stride, None, group)
+    y = run(x, W, kernels.INQ_PRODUCT_ONLY)
+    assert np.array_equal(np.isnan(y), np.isnan(ref))
+    assert np.array_equal(np.isposinf(y), np.isposinf(ref)) and np.array_equal(np.isneginf(y), np.isneginf(ref))
+    fin = np.isfinite(ref)
+    assert fin.any() and np.isnan(ref).any() and np.isinf(ref).any()
+    assert bits_equal(y[fin], clean[fin])
+
+
 def test_convolution_with_fixed_weights_at_the_resnet_stage_shape(dev):
     """Benchmark configuration 4's shape with power-of-two weights (98 tiles of the digit product, the contraction
     split over blocks, every tile in the one-digit form for its weights) against torch's float64 convolution."""
