@@ -797,7 +797,7 @@ __global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const floa
     shift[m] = bad ? kBadRow : (any_low == 0u ? s + kOneDigitBias : s);
   }
   if (redo.y) {
-    // lane rr of every wavefront holds row rr's verdict, the same in all wavefronts: the loop is uniform over the block
+    // lane rr of every wavefront holds row rr's flag, the same in all wavefronts: the loop is uniform over the block
     const unsigned long long marked = __ballot(bad);
     for (int rr = 0; rr < kRows; ++rr) {
       const int64_t mr = (int64_t)blockIdx.x * kRows + rr;

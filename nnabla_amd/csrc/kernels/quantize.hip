@@ -331,38 +331,6 @@ constexpr int kRedBlock = 256;
 constexpr int kRedTile = kRedBlock * 4; // elements per block tile
 constexpr int kMaxChunks = 1024;
 
-// A pattern whose kept axes are separated by reduced ones and whose innermost axis is kept (q shape (C, 1, W)): the
-// kept index is (ko, w) with w along the contiguous axis, the reduced index (ro, ri) with ri along the innermost
-// reduced axis.  The kernels of this form put the lanes along w, so every line of x is read once, and walk the
-// reduced index in row-major order like the reference's scan.
-struct MinMaxInner {
-  bool ok;
-  int64_t Ko, Wk;        // kept: outer combinations, innermost (contiguous) extent
-  int64_t Rout, Rin;     // reduced: outer combinations, innermost extent
-  int64_t rin_stride;    // element stride of the innermost reduced axis
-  int tw;                // lanes along w: the power of two covering min(Wk, 64)
-};
-inline MinMaxInner inner_form(const MinMaxAxes &A) {
-  MinMaxInner I;
-  I.ok = A.nkept >= 1 && A.nred >= 1 && A.kstride[A.nkept - 1] == 1;
-  if (!I.ok)
-    return I;
-  I.Wk = A.ksize[A.nkept - 1];
-  I.Ko = 1;
-  for (int d = 0; d + 1 < A.nkept; ++d)
-    I.Ko *= A.ksize[d];
-  I.Rin = A.rsize[A.nred - 1];
-  I.rin_stride = A.rstride[A.nred - 1];
-  I.Rout = 1;
-  for (int d = 0; d + 1 < A.nred; ++d)
-    I.Rout *= A.rsize[d];
-  I.tw = 1;
-  while (I.tw < 64 && I.tw < I.Wk)
-    I.tw *= 2;
-  I.ok = I.Ko < ((int64_t)1 << 31);
-  return I;
-}
-
 struct MinMaxPlan {
   MinMaxLayout L;
   int64_t tiles_per_row; // tiles covering one run of R1 elements
@@ -385,18 +353,15 @@ MinMaxPlan make_plan(const int64_t *xshape, int ndim, const int64_t *qshape) {
   if (want < 1)
     want = 1;
   P.inner = false;
-  if (!P.L.ok) {
-    want = 1; // the general strided kernels fold a whole slice per block
+  if (!P.L.ok || trailing_kept(P.L)) {
+    if (!P.L.ok)
+      want = 1; // the general strided kernels fold a whole slice per block
     MinMaxAxes A;
     if (split_axes(xshape, ndim, qshape, A)) {
       const MinMaxInner I = inner_form(A);
-      if (I.ok) { // about 2048 blocks, each a run of outer reduced indices
+      if (I.ok) {
         P.inner = true;
-        want = (2048 + I.Ko - 1) / I.Ko;
-        if (want > I.Rout)
-          want = I.Rout;
-        if (want > 64)
-          want = 64;
+        want = inner_chunks(I);
       }
     }
   }
@@ -747,15 +712,6 @@ __global__ __launch_bounds__(kBlock) void minmax_apply_generic(const float *__re
 
 // Any pattern of kept and reduced axes (e.g. q shape (C, 1, W)): block k scans the slice of kept index k in the order
 // the reference's Min / Max scan it (reduced axes row-major), one element per thread and step.
-__device__ __forceinline__ int64_t strided_offset(int64_t idx, int n, const int64_t *size, const int64_t *stride) {
-  int64_t off = 0;
-  for (int d = n - 1; d >= 0; --d) {
-    const int64_t q = idx / size[d];
-    off += (idx - q * size[d]) * stride[d];
-    idx = q;
-  }
-  return off;
-}
 __global__ __launch_bounds__(kRedBlock) void minmax_reduce_strided(const float *__restrict__ x,
                                                                    MinMaxPartial *__restrict__ partial, MinMaxAxes A,
                                                                    int64_t R) {
@@ -777,39 +733,6 @@ __global__ __launch_bounds__(kRedBlock) void minmax_reduce_strided(const float *
     partial[k] = ex.pack();
   }
 }
-// The inner-kept form (MinMaxInner).  Block (ko, chunk): the outer reduced indices ro = chunk, chunk + nchunks, ... are
-// not what it takes -- it takes the contiguous run [chunk * per, (chunk + 1) * per) so that its first-zero index grows
-// along its scan.  Lane = (row slot, w): the block's 256 threads cover 256 / tw rows of tw columns per step; columns
-// beyond 64 are walked in further passes over the block's rows.
-struct InnerWalk {
-  const float *base;   // x at (ko, w = 0)
-  int64_t ro_begin, ro_end;
-};
-__device__ __forceinline__ InnerWalk inner_walk(const float *x, const MinMaxAxes &A, const MinMaxInner &I, int64_t ko,
-                                                int chunk, int nchunks) {
-  InnerWalk w;
-  w.base = x + (A.nkept > 1 ? strided_offset(ko, A.nkept - 1, A.ksize, A.kstride) : 0);
-  const int64_t per = (I.Rout + nchunks - 1) / nchunks;
-  w.ro_begin = (int64_t)chunk * per;
-  w.ro_end = w.ro_begin + per < I.Rout ? w.ro_begin + per : I.Rout;
-  return w;
-}
-// kVec = 4: Wk a multiple of four and x (y) 16-byte aligned: a lane owns four consecutive columns (one 128-bit
-// access per row) and the plan's tw counts such quads.
-template <int kVec> struct InnerRow;
-template <> struct InnerRow<1> {
-  float v[1];
-  __device__ __forceinline__ void load(const float *p) { v[0] = *p; }
-  __device__ __forceinline__ void fill(float f) { v[0] = f; }
-};
-template <> struct InnerRow<4> {
-  float v[4];
-  __device__ __forceinline__ void load(const float *p) {
-    const float4_t q = *reinterpret_cast<const float4_t *>(p);
-    v[0] = q.x, v[1] = q.y, v[2] = q.z, v[3] = q.w;
-  }
-  __device__ __forceinline__ void fill(float f) { v[0] = v[1] = v[2] = v[3] = f; }
-};
 template <int kVec>
 __global__ __launch_bounds__(kRedBlock) void minmax_reduce_inner(const float *__restrict__ x,
                                                                  MinMaxPartial *__restrict__ partial, MinMaxAxes A,
@@ -950,7 +873,7 @@ int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, in
                   "x.shape and ql_min.shape must be same except for i-th dimension where ql_min.shape[i] == 1.");
   MinMaxPlan P = make_plan(xshape, ndim, qshape);
   MinMaxAxes axes;
-  if (!P.L.ok && !split_axes(xshape, ndim, qshape, axes))
+  if ((!P.L.ok || P.inner) && !split_axes(xshape, ndim, qshape, axes))
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than eight kept or eight reduced axes of size above one.");
   if (P.L.total == 0)
     return NBLA_HIP_OK;
@@ -977,7 +900,7 @@ int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, in
   const bool vec_ok = aligned16(x) && (L.R1 % 4 == 0 || L.K == 1);
   int nchunks = P.nchunks;
 
-  if (!L.ok) { // kept axes separated by reduced ones: the strided kernels
+  if (!L.ok || P.inner) { // kept axes separated by reduced ones, or all behind them: the strided kernels
     if (L.K > 0x7fffffffll)
       return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than 2^31 - 1 quantization ranges.");
     MinMaxInner inner = P.inner ? inner_form(axes) : MinMaxInner{false};

@@ -277,10 +277,245 @@ __global__ __launch_bounds__(64) void minmax_range_grad_final(const float2 *__re
     g_max[k] = accum_max ? g_max[k] + hi : hi;
 }
 
+// ---- dx and the range sums in one pass over dy and x.
+// What a launch does: dx (0: not wanted, 1: dx (+)= dy, 2: dx (+)= mask * dy), whether dx is added to, and whether
+// the masked sums of dy below m' / above M' are formed.  Uniform over the grid.
+struct GradMode {
+  int dx_mode, accum, sums;
+};
+
+// mask * dy (+ old) as min_max_quantize.cpp:262-284 forms it
+__device__ __forceinline__ float minmax_dx(float g, float xv, float old, const float2 &b, const GradMode &m) {
+  float t = g;
+  if (m.dx_mode == 2) {
+    const float iv0 = (xv >= b.x) ? 1.0f : 0.0f, iv1 = (xv <= b.y) ? 1.0f : 0.0f;
+    t = iv0 * iv1;
+    t = t * g;
+  }
+  return m.accum ? t + old : t;
+}
+__device__ __forceinline__ void minmax_sums(float g, float xv, const float2 &b, float &lo, float &hi) {
+  lo += ((xv < b.x) ? 1.0f : 0.0f) * g;
+  hi += ((xv > b.y) ? 1.0f : 0.0f) * g;
+}
+// lanes, then wavefronts in a fixed order; thread 0 writes
+__device__ __forceinline__ void block_sums(float lo, float hi, float2 *dst) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    lo += __shfl_xor(lo, off);
+    hi += __shfl_xor(hi, off);
+  }
+  __shared__ float2 s_part[kBlock / 64];
+  if ((threadIdx.x & 63) == 0)
+    s_part[threadIdx.x >> 6] = float2{lo, hi};
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float2 acc = s_part[0];
+    for (int w = 1; w < kBlock / 64; ++w)
+      acc.x += s_part[w].x, acc.y += s_part[w].y;
+    *dst = acc;
+  }
+}
+__device__ __forceinline__ void minmax_grad4(const float *__restrict__ dy, const float *__restrict__ x,
+                                             float *__restrict__ dx, int64_t at, const float2 &b, const GradMode &m,
+                                             float &lo, float &hi) {
+  const float4_t g = load4(dy + at);
+  float4_t v = float4_t{0.0f, 0.0f, 0.0f, 0.0f}, o = v;
+  if (m.dx_mode == 2 || m.sums)
+    v = load4(x + at);
+  if (m.dx_mode && m.accum)
+    o = load4(dx + at);
+  if (m.dx_mode) {
+    float4_t r;
+    r.x = minmax_dx(g.x, v.x, o.x, b, m), r.y = minmax_dx(g.y, v.y, o.y, b, m);
+    r.z = minmax_dx(g.z, v.z, o.z, b, m), r.w = minmax_dx(g.w, v.w, o.w, b, m);
+    store4(dx + at, r);
+  }
+  if (m.sums) {
+    minmax_sums(g.x, v.x, b, lo, hi), minmax_sums(g.y, v.y, b, lo, hi);
+    minmax_sums(g.z, v.z, b, lo, hi), minmax_sums(g.w, v.w, b, lo, hi);
+  }
+}
+
+// One range for the whole tensor (16-byte aligned): block c takes the tiles c, c + gridDim.x, ... of kBlock * 4
+// float4s and leaves its sums in partial[c]; block 0 also takes the elements past the last whole float4.
+__global__ __launch_bounds__(kBlock) void minmax_grad_flat(const float *__restrict__ dy, const float *__restrict__ x,
+                                                           float *__restrict__ dx, int64_t n4, int64_t size,
+                                                           const float2 *__restrict__ bounds,
+                                                           float2 *__restrict__ partial, GradMode m) {
+  const float2 b = bounds[0];
+  float lo = 0.0f, hi = 0.0f;
+  const int64_t tiles = (n4 + kBlock * 4 - 1) / (kBlock * 4);
+  for (int64_t t = blockIdx.x; t < tiles; t += gridDim.x) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t i = t * (kBlock * 4) + j * kBlock + threadIdx.x;
+      if (i < n4)
+        minmax_grad4(dy, x, dx, 4 * i, b, m, lo, hi);
+    }
+  }
+  if (blockIdx.x == 0) {
+    const int64_t i = 4 * n4 + threadIdx.x;
+    if (i < size) {
+      const float g = dy[i], xv = x[i];
+      if (m.dx_mode)
+        dx[i] = minmax_dx(g, xv, m.accum ? dx[i] : 0.0f, b, m);
+      if (m.sums)
+        minmax_sums(g, xv, b, lo, hi);
+    }
+  }
+  if (m.sums)
+    block_sums(lo, hi, partial + blockIdx.x);
+}
+
+// Ranges per channel, rows of R1 contiguous elements (R1 % 4 == 0, 16-byte aligned): blockIdx.x = row (r0 * K + k),
+// blockIdx.y = part of the row; the sums go to partial[k * nchunks + r0 * gridDim.y + blockIdx.y], nchunks =
+// R0 * gridDim.y.
+__global__ __launch_bounds__(kBlock) void minmax_grad_rows(const float *__restrict__ dy, const float *__restrict__ x,
+                                                           float *__restrict__ dx, int64_t K, int64_t R1,
+                                                           const float2 *__restrict__ bounds,
+                                                           float2 *__restrict__ partial, int64_t nchunks, GradMode m) {
+  const int64_t row = blockIdx.x, r0 = row / K, k = row - r0 * K;
+  const float2 b = bounds[k];
+  const int64_t n4 = R1 / 4, at0 = row * R1;
+  float lo = 0.0f, hi = 0.0f;
+  for (int64_t i = (int64_t)blockIdx.y * kBlock + threadIdx.x; i < n4; i += (int64_t)gridDim.y * kBlock)
+    minmax_grad4(dy, x, dx, at0 + 4 * i, b, m, lo, hi);
+  if (m.sums)
+    block_sums(lo, hi, partial + k * nchunks + r0 * gridDim.y + blockIdx.y);
+}
+
+// The inner-kept form (MinMaxInner: lanes along the kept innermost axis), block (ko, chunk) as in the forward's
+// kernels of this form; the sums of column w go to partial[(ko * Wk + w) * nchunks + chunk].
+template <int kVec>
+__global__ __launch_bounds__(kBlock) void minmax_grad_inner(const float *__restrict__ dy, const float *__restrict__ x,
+                                                            float *__restrict__ dx, MinMaxAxes A, MinMaxInner I,
+                                                            int nchunks, const float2 *__restrict__ bounds,
+                                                            float2 *__restrict__ partial, GradMode m) {
+  __shared__ float2 s_part[kBlock / 64][64][kVec];
+  const int64_t ko = blockIdx.x;
+  const int chunk = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tw = I.tw, rows_per_step = kBlock / tw;
+  const int cw = tid & (tw - 1), slot = tid / tw;
+  const InnerWalk W = inner_walk(x, A, I, ko, chunk, nchunks);
+  constexpr int kRows = 4; // rows in flight per lane
+  for (int64_t w0 = 0; w0 < I.Wk; w0 += (int64_t)tw * kVec) {
+    const int64_t wcol = w0 + (int64_t)cw * kVec;
+    const bool col_in = wcol < I.Wk;
+    float2 b[kVec];
+    float lo[kVec], hi[kVec];
+#pragma unroll
+    for (int c = 0; c < kVec; ++c) {
+      b[c] = bounds[ko * I.Wk + (col_in ? wcol + c : 0)];
+      lo[c] = hi[c] = 0.0f;
+    }
+    for (int64_t ro = W.ro_begin; ro < W.ro_end; ++ro) {
+      const int64_t off = (W.base - x) + (A.nred > 1 ? strided_offset(ro, A.nred - 1, A.rsize, A.rstride) : 0) + wcol;
+      for (int64_t ri0 = 0; ri0 < I.Rin; ri0 += kRows * rows_per_step) {
+        InnerRow<kVec> g[kRows], v[kRows], o[kRows];
+#pragma unroll
+        for (int j = 0; j < kRows; ++j) {
+          const int64_t ri = ri0 + slot + j * rows_per_step;
+          const bool in = col_in && ri < I.Rin;
+          const int64_t at = off + ri * I.rin_stride;
+          if (in)
+            g[j].load(dy + at);
+          else
+            g[j].fill(0.0f);
+          if (in && (m.dx_mode == 2 || m.sums))
+            v[j].load(x + at);
+          else
+            v[j].fill(0.0f);
+          if (in && m.dx_mode && m.accum)
+            o[j].load(dx + at);
+          else
+            o[j].fill(0.0f);
+        }
+#pragma unroll
+        for (int j = 0; j < kRows; ++j) {
+          const int64_t ri = ri0 + slot + j * rows_per_step;
+          if (!(col_in && ri < I.Rin))
+            continue;
+          if (m.dx_mode) {
+            float *dst = dx + off + ri * I.rin_stride;
+            float r[kVec];
+#pragma unroll
+            for (int c = 0; c < kVec; ++c)
+              r[c] = minmax_dx(g[j].v[c], v[j].v[c], o[j].v[c], b[c], m);
+            if (kVec == 4)
+              store4(dst, float4_t{r[0], r[1 % kVec], r[2 % kVec], r[3 % kVec]});
+            else
+              __builtin_nontemporal_store(r[0], dst);
+          }
+          if (m.sums) {
+#pragma unroll
+            for (int c = 0; c < kVec; ++c)
+              minmax_sums(g[j].v[c], v[j].v[c], b[c], lo[c], hi[c]);
+          }
+        }
+      }
+    }
+    if (!m.sums) // uniform
+      continue;
+    // fold the row slots that share a column: across the lanes of a wavefront, then across the wavefronts
+#pragma unroll
+    for (int c = 0; c < kVec; ++c)
+      for (int off = 32; off >= tw; off >>= 1) {
+        lo[c] += __shfl_xor(lo[c], off);
+        hi[c] += __shfl_xor(hi[c], off);
+      }
+    __syncthreads(); // the previous pass's partial results have been read
+#pragma unroll
+    for (int c = 0; c < kVec; ++c)
+      s_part[wave][lane][c] = float2{lo[c], hi[c]};
+    __syncthreads();
+    if (tid < tw && col_in) {
+#pragma unroll
+      for (int c = 0; c < kVec; ++c) {
+        float2 acc = s_part[0][tid][c];
+        for (int w = 1; w < kBlock / 64; ++w)
+          acc.x += s_part[w][tid][c].x, acc.y += s_part[w][tid][c].y;
+        partial[(ko * I.Wk + wcol + c) * nchunks + chunk] = acc;
+      }
+    }
+  }
+}
+
+// A wavefront per range: lane l adds the partial sums l, l + 64, ... in order, then the lanes are added up.
+__global__ __launch_bounds__(64) void minmax_range_grad_final_wave(const float2 *__restrict__ partial, int64_t nchunks,
+                                                                   float *__restrict__ g_min, float *__restrict__ g_max,
+                                                                   int accum_min, int accum_max) {
+  const int64_t k = blockIdx.x;
+  float lo = 0.0f, hi = 0.0f;
+  for (int64_t c = threadIdx.x; c < nchunks; c += 64) {
+    const float2 p = partial[k * nchunks + c];
+    lo += p.x, hi += p.y;
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    lo += __shfl_xor(lo, off);
+    hi += __shfl_xor(hi, off);
+  }
+  if (threadIdx.x == 0) {
+    if (g_min)
+      g_min[k] = accum_min ? g_min[k] + lo : lo;
+    if (g_max)
+      g_max[k] = accum_max ? g_max[k] + hi : hi;
+  }
+}
+
+// Which one-pass kernel a shape can take (the pointers' alignment decides at the call) and the partial sums each
+// leaves per range; the workspace holds the largest.
 struct RangeGradPlan {
   MinMaxLayout L;
   int64_t tiles_per_row, tiles_per_k;
-  int nchunks;
+  int nchunks;          // of the two-pass kernels
+  bool inner;           // the lanes-along-the-kept-axis form applies
+  MinMaxAxes axes;
+  MinMaxInner I;
+  int inner_chunks;
+  int64_t flat_chunks;  // K == 1
+  int64_t row_parts;    // rows form (R1 % 4 == 0, R1 >= 256): blocks along a row; partial sums per range = R0 * row_parts
   size_t bounds_bytes, partial_bytes;
 };
 
@@ -299,9 +534,49 @@ RangeGradPlan make_range_plan(const int64_t *xshape, int ndim, const int64_t *qs
   if (!P.L.ok)
     chunks = 1; // the strided kernel folds a whole slice per block
   P.nchunks = (int)chunks;
+  int64_t most = chunks;
+  P.inner = false;
+  P.inner_chunks = 1;
+  if ((!P.L.ok || trailing_kept(P.L)) && split_axes(xshape, ndim, qshape, P.axes)) {
+    P.I = inner_form(P.axes);
+    if (P.I.ok) {
+      P.inner = true;
+      P.inner_chunks = (int)inner_chunks(P.I);
+      most = most > P.inner_chunks ? most : P.inner_chunks;
+    }
+  }
+  P.flat_chunks = 0;
+  if (P.L.ok && P.L.K == 1) {
+    const int64_t tiles = (P.L.total / 4 + kBlock * 4 - 1) / (kBlock * 4);
+    P.flat_chunks = tiles < 1 ? 1 : (tiles > 2048 ? 2048 : tiles);
+    most = most > P.flat_chunks ? most : P.flat_chunks;
+  }
+  P.row_parts = 0;
+  if (P.L.ok && P.L.K > 1 && P.L.R1 % 4 == 0 && P.L.R1 >= 256 && P.L.R0 * P.L.K <= 0x7fffffffll) {
+    // about 4096 blocks; a block takes at least one float4 per thread
+    int64_t parts = (4096 + P.L.R0 * P.L.K - 1) / (P.L.R0 * P.L.K);
+    const int64_t longest = (P.L.R1 / 4 + kBlock - 1) / kBlock;
+    if (parts > longest)
+      parts = longest;
+    if (parts > 64)
+      parts = 64;
+    P.row_parts = parts < 1 ? 1 : parts;
+    most = most > P.L.R0 * P.row_parts ? most : P.L.R0 * P.row_parts;
+  }
   P.bounds_bytes = round_up((size_t)P.L.K * sizeof(float2), 256);
-  P.partial_bytes = round_up((size_t)P.L.K * P.nchunks * sizeof(float2), 256);
+  P.partial_bytes = round_up((size_t)P.L.K * most * sizeof(float2), 256);
   return P;
+}
+
+// g_qr_min / g_qr_max from `chunks` partial sums per range
+void launch_range_final(const float2 *partial, int64_t chunks, float *g_min, float *g_max, int accum_min,
+                        int accum_max, int64_t K, hipStream_t stream) {
+  if (chunks <= 16 && K >= 64)
+    hipLaunchKernelGGL(minmax_range_grad_final, dim3((unsigned)((K + 63) / 64)), dim3(64), 0, stream, partial,
+                       (int)chunks, g_min, g_max, accum_min, accum_max, K);
+  else
+    hipLaunchKernelGGL(minmax_range_grad_final_wave, dim3((unsigned)K), dim3(64), 0, stream, partial, chunks, g_min,
+                       g_max, accum_min, accum_max);
 }
 
 } // namespace
@@ -380,7 +655,7 @@ int nbla_hip_min_max_quantize_backward_f32(const float *dy, const float *x, floa
   MinMaxAxes axes;
   if (!P.L.ok && !split_axes(xshape, ndim, qshape, axes))
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than eight kept or eight reduced axes of size above one.");
-  if (!P.L.ok && P.L.K > 0x7fffffffll)
+  if (P.L.K > 0x7fffffffll && (!P.L.ok || P.inner))
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than 2^31 - 1 quantization ranges.");
   if (P.L.total == 0)
     return NBLA_HIP_OK;
@@ -397,6 +672,52 @@ int nbla_hip_min_max_quantize_backward_f32(const float *dy, const float *x, floa
     hipLaunchKernelGGL(minmax_bounds, dim3((unsigned)((P.L.K + 63) / 64)), dim3(64), 0, stream, qr_min, ql_min, ql_max,
                        scale, bounds, P.L.K);
     NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward bounds");
+  }
+  // dx and the range sums in one pass over dy and x, where a kernel of that kind covers the layout (a plain copy of dy
+  // and the per-tensor mask without sums are as fast on the element-wise kernels below)
+  const GradMode mode{dx ? (ste_fine_grained ? 2 : 1) : 0, accum_x, range_grads ? 1 : 0};
+  const bool wanted = range_grads || (mode.dx_mode == 2 && P.L.K > 1);
+  const bool vec = aligned16(dy) && aligned16(x) && (!dx || aligned16(dx));
+  if (wanted && P.inner) {
+    MinMaxInner I = P.I;
+    const bool quads = I.Wk % 4 == 0 && vec;
+    if (quads) {
+      I.tw = 1;
+      while (I.tw < 64 && I.tw * 4 < I.Wk)
+        I.tw *= 2;
+    }
+    const dim3 grid((unsigned)I.Ko, (unsigned)P.inner_chunks);
+    if (quads)
+      hipLaunchKernelGGL(minmax_grad_inner<4>, grid, dim3(kBlock), 0, stream, dy, x, dx, P.axes, I, P.inner_chunks,
+                         bounds, partial, mode);
+    else
+      hipLaunchKernelGGL(minmax_grad_inner<1>, grid, dim3(kBlock), 0, stream, dy, x, dx, P.axes, I, P.inner_chunks,
+                         bounds, partial, mode);
+    NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward");
+    if (range_grads) {
+      launch_range_final(partial, P.inner_chunks, g_qr_min, g_qr_max, accum_min, accum_max, P.L.K, stream);
+      NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward range gradients");
+    }
+    return NBLA_HIP_OK;
+  }
+  if (wanted && P.flat_chunks && vec) {
+    hipLaunchKernelGGL(minmax_grad_flat, dim3((unsigned)P.flat_chunks), dim3(kBlock), 0, stream, dy, x, dx,
+                       P.L.total / 4, P.L.total, bounds, partial, mode);
+    NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward");
+    launch_range_final(partial, P.flat_chunks, g_qr_min, g_qr_max, accum_min, accum_max, 1, stream);
+    NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward range gradients");
+    return NBLA_HIP_OK;
+  }
+  if (wanted && P.row_parts && vec) {
+    const int64_t chunks = P.L.R0 * P.row_parts;
+    hipLaunchKernelGGL(minmax_grad_rows, dim3((unsigned)(P.L.R0 * P.L.K), (unsigned)P.row_parts), dim3(kBlock), 0,
+                       stream, dy, x, dx, P.L.K, P.L.R1, bounds, partial, chunks, mode);
+    NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward");
+    if (range_grads) {
+      launch_range_final(partial, chunks, g_qr_min, g_qr_max, accum_min, accum_max, P.L.K, stream);
+      NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward range gradients");
+    }
+    return NBLA_HIP_OK;
   }
   if (dx) {
     if (ste_fine_grained && !P.L.ok) {

@@ -84,6 +84,99 @@ inline MinMaxLayout collapse(const int64_t *xshape, int ndim, const int64_t *qsh
 }
 
 
+// Offset in x of index idx over the axes (size, stride), row-major.
+__device__ __forceinline__ int64_t strided_offset(int64_t idx, int n, const int64_t *size, const int64_t *stride) {
+  int64_t off = 0;
+  for (int d = n - 1; d >= 0; --d) {
+    const int64_t q = idx / size[d];
+    off += (idx - q * size[d]) * stride[d];
+    idx = q;
+  }
+  return off;
+}
+
+// A pattern whose kept axes are separated by reduced ones and whose innermost axis is kept (q shape (C, 1, W)): the
+// kept index is (ko, w) with w along the contiguous axis, the reduced index (ro, ri) with ri along the innermost
+// reduced axis.  The kernels of this form put the lanes along w, so every line of x is read once, and walk the
+// reduced index in row-major order like the reference's scan.
+struct MinMaxInner {
+  bool ok;
+  int64_t Ko, Wk;        // kept: outer combinations, innermost (contiguous) extent
+  int64_t Rout, Rin;     // reduced: outer combinations, innermost extent
+  int64_t rin_stride;    // element stride of the innermost reduced axis
+  int tw;                // lanes along w: the power of two covering min(Wk, 64)
+};
+inline MinMaxInner inner_form(const MinMaxAxes &A) {
+  MinMaxInner I;
+  I.ok = A.nkept >= 1 && A.nred >= 1 && A.kstride[A.nkept - 1] == 1;
+  if (!I.ok)
+    return I;
+  I.Wk = A.ksize[A.nkept - 1];
+  I.Ko = 1;
+  for (int d = 0; d + 1 < A.nkept; ++d)
+    I.Ko *= A.ksize[d];
+  I.Rin = A.rsize[A.nred - 1];
+  I.rin_stride = A.rstride[A.nred - 1];
+  I.Rout = 1;
+  for (int d = 0; d + 1 < A.nred; ++d)
+    I.Rout *= A.rsize[d];
+  I.tw = 1;
+  while (I.tw < 64 && I.tw < I.Wk)
+    I.tw *= 2;
+  I.ok = I.Ko < ((int64_t)1 << 31);
+  return I;
+}
+
+// Blocks per kept outer index of the kernels of this form: about 2048 blocks in all, each a run of outer reduced
+// indices.
+inline int64_t inner_chunks(const MinMaxInner &I) {
+  int64_t want = (2048 + I.Ko - 1) / I.Ko;
+  if (want > I.Rout)
+    want = I.Rout;
+  const int64_t cap = I.Ko >= 32 ? 64 : 1024;
+  if (want > cap)
+    want = cap;
+  return want < 1 ? 1 : want;
+}
+// Every kept axis behind every reduced one (ranges per column of a matrix, q shape (1, 1, W)): runs of one element,
+// which the kernels that walk runs of R1 elements would visit one block at a time; the kernels with the lanes along
+// the kept axis take such a layout.
+inline bool trailing_kept(const MinMaxLayout &L) { return L.ok && L.R1 == 1 && L.K > 1 && L.R0 > 1; }
+
+// The inner-kept form (MinMaxInner).  Block (ko, chunk): the outer reduced indices ro = chunk, chunk + nchunks, ... are
+// not what it takes -- it takes the contiguous run [chunk * per, (chunk + 1) * per) so that its first-zero index grows
+// along its scan.  Lane = (row slot, w): the block's 256 threads cover 256 / tw rows of tw columns per step; columns
+// beyond 64 are walked in further passes over the block's rows.
+struct InnerWalk {
+  const float *base;   // x at (ko, w = 0)
+  int64_t ro_begin, ro_end;
+};
+__device__ __forceinline__ InnerWalk inner_walk(const float *x, const MinMaxAxes &A, const MinMaxInner &I, int64_t ko,
+                                                int chunk, int nchunks) {
+  InnerWalk w;
+  w.base = x + (A.nkept > 1 ? strided_offset(ko, A.nkept - 1, A.ksize, A.kstride) : 0);
+  const int64_t per = (I.Rout + nchunks - 1) / nchunks;
+  w.ro_begin = (int64_t)chunk * per;
+  w.ro_end = w.ro_begin + per < I.Rout ? w.ro_begin + per : I.Rout;
+  return w;
+}
+// kVec = 4: Wk a multiple of four and x (y) 16-byte aligned: a lane owns four consecutive columns (one 128-bit
+// access per row) and the plan's tw counts such quads.
+template <int kVec> struct InnerRow;
+template <> struct InnerRow<1> {
+  float v[1];
+  __device__ __forceinline__ void load(const float *p) { v[0] = *p; }
+  __device__ __forceinline__ void fill(float f) { v[0] = f; }
+};
+template <> struct InnerRow<4> {
+  float v[4];
+  __device__ __forceinline__ void load(const float *p) {
+    const float4_t q = *reinterpret_cast<const float4_t *>(p);
+    v[0] = q.x, v[1] = q.y, v[2] = q.z, v[3] = q.w;
+  }
+  __device__ __forceinline__ void fill(float f) { v[0] = v[1] = v[2] = v[3] = f; }
+};
+
 // nudge_qr_min_max (min_max_quantize.cpp:363-390): the representable range [m', M'] whose zero point is an integer
 // level, one rounded fp32 operation at a time.
 __host__ __device__ inline void nudge_qr_min_max(float qr_min, float ql_min, float ql_max, float scale, float &m_n,

@@ -234,6 +234,10 @@ MMQ_SHAPES = [
     # hundreds of ranges with few partial results each (a thread per range folds them): lanes along the kept innermost
     # axis, per channel, and the one-block-per-range form
     ((4, 64, 6, 40), (1, 64, 1, 40)), ((2, 512, 4, 4), (1, 512, 1, 1)), ((64, 3, 8, 2), (64, 1, 8, 1)),
+    # every kept axis behind every reduced one (ranges per column of a matrix): lanes along the kept axes, the
+    # reduced positions split over many blocks
+    ((300, 520), (1, 520)), ((40, 33, 20), (1, 1, 20)), ((7, 3, 5, 9), (1, 1, 5, 9)), ((5000, 3), (1, 3)),
+    ((9, 4100, 2, 2), (1, 1, 2, 2)),
 ]
 
 
