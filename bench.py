@@ -230,6 +230,27 @@ def bench_quantizers(dev, iters):
     nb = 12.0 * a.numel()
     out["min_max_quantize[64,256,56,56] x_min_max, ranges [1,256,1,56]"] = {
         "ms": ms, "bytes": nb, "GBs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
+    # ranges per channel and per column (every kept axis behind the reduced ones), and the backward pass with learnt
+    # ranges: dx and both range gradients from one pass over dy and x (12 B/elem)
+    dy = torch.randn(a.shape, generator=g).to(dev)
+    for qshape in ((1, 1, 1, 1), (1, 256, 1, 1), (1, 1, 1, 56)):
+        qs = lambda v: torch.full(qshape, v, device=dev)
+        qmn, qmx, lmn, lmx = qs(-6.0), qs(6.0), qs(0.0), qs(255.0)
+        tag = "ranges [%s]" % ",".join(str(v) for v in qshape)
+        if qshape != (1, 1, 1, 1):
+            ws3 = torch.empty(max(256, k.lib().nbla_hip_min_max_quantize_workspace_bytes(
+                k._shape(a.shape), a.dim(), k._shape(qshape))), dtype=torch.uint8, device=dev)
+            ms = time_kernel(lambda: k.min_max_quantize(a, qmn, qmx, lmn, lmx, 0.999, True, True, 0.01, out=ya,
+                                                        workspace=ws3), iters)
+            nb = 12.0 * a.numel()
+            out["min_max_quantize[64,256,56,56] x_min_max, " + tag] = {
+                "ms": ms, "bytes": nb, "GBs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
+        _, scale = k.min_max_quantize(a, qmn, qmx, lmn, lmx, 0.999, False, False, 0.01, out=ya)
+        ms = time_kernel(lambda: k.min_max_quantize_backward(dy, a, qmn, qmx, lmn, lmx, scale, True, False, False),
+                         iters)
+        nb = 12.0 * a.numel()
+        out["min_max_quantize_backward[64,256,56,56] dx + range gradients, " + tag] = {
+            "ms": ms, "bytes": nb, "GBs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
     return out
 
 

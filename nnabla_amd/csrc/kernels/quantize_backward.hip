@@ -316,24 +316,44 @@ __device__ __forceinline__ void block_sums(float lo, float hi, float2 *dst) {
     *dst = acc;
   }
 }
-__device__ __forceinline__ void minmax_grad4(const float *__restrict__ dy, const float *__restrict__ x,
-                                             float *__restrict__ dx, int64_t at, const float2 &b, const GradMode &m,
-                                             float &lo, float &hi) {
-  const float4_t g = load4(dy + at);
-  float4_t v = float4_t{0.0f, 0.0f, 0.0f, 0.0f}, o = v;
-  if (m.dx_mode == 2 || m.sums)
-    v = load4(x + at);
-  if (m.dx_mode && m.accum)
-    o = load4(dx + at);
-  if (m.dx_mode) {
-    float4_t r;
-    r.x = minmax_dx(g.x, v.x, o.x, b, m), r.y = minmax_dx(g.y, v.y, o.y, b, m);
-    r.z = minmax_dx(g.z, v.z, o.z, b, m), r.w = minmax_dx(g.w, v.w, o.w, b, m);
-    store4(dx + at, r);
+// The range tensors of a call; bounds(k) = (m', M') of range k as minmax_bounds forms them, for kernels whose blocks
+// need one range each.
+struct RangeInputs {
+  const float *qr_min, *ql_min, *ql_max, *scale;
+  __device__ __forceinline__ float2 bounds(int64_t k) const {
+    float m_n, M_n;
+    nudge_qr_min_max(qr_min[k], ql_min[k], ql_max[k], scale[k], m_n, M_n);
+    return float2{m_n, M_n};
   }
-  if (m.sums) {
-    minmax_sums(g.x, v.x, b, lo, hi), minmax_sums(g.y, v.y, b, lo, hi);
-    minmax_sums(g.z, v.z, b, lo, hi), minmax_sums(g.w, v.w, b, lo, hi);
+};
+
+// kN float4s per thread, all loads issued before the first store (the compiler does not move a load across a store)
+template <int kN>
+__device__ __forceinline__ void minmax_grad4(const float *__restrict__ dy, const float *__restrict__ x,
+                                             float *__restrict__ dx, const int64_t (&at)[kN], const bool (&in)[kN],
+                                             const float2 &b, const GradMode &m, float &lo, float &hi) {
+  const float4_t zero = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  float4_t g[kN], v[kN], o[kN];
+#pragma unroll
+  for (int j = 0; j < kN; ++j) {
+    g[j] = in[j] ? load4(dy + at[j]) : zero;
+    v[j] = (in[j] && (m.dx_mode == 2 || m.sums)) ? load4(x + at[j]) : zero;
+    o[j] = (in[j] && m.dx_mode && m.accum) ? load4(dx + at[j]) : zero;
+  }
+#pragma unroll
+  for (int j = 0; j < kN; ++j) {
+    if (!in[j])
+      continue;
+    if (m.dx_mode) {
+      float4_t r;
+      r.x = minmax_dx(g[j].x, v[j].x, o[j].x, b, m), r.y = minmax_dx(g[j].y, v[j].y, o[j].y, b, m);
+      r.z = minmax_dx(g[j].z, v[j].z, o[j].z, b, m), r.w = minmax_dx(g[j].w, v[j].w, o[j].w, b, m);
+      store4(dx + at[j], r);
+    }
+    if (m.sums) {
+      minmax_sums(g[j].x, v[j].x, b, lo, hi), minmax_sums(g[j].y, v[j].y, b, lo, hi);
+      minmax_sums(g[j].z, v[j].z, b, lo, hi), minmax_sums(g[j].w, v[j].w, b, lo, hi);
+    }
   }
 }
 
@@ -341,18 +361,19 @@ __device__ __forceinline__ void minmax_grad4(const float *__restrict__ dy, const
 // float4s and leaves its sums in partial[c]; block 0 also takes the elements past the last whole float4.
 __global__ __launch_bounds__(kBlock) void minmax_grad_flat(const float *__restrict__ dy, const float *__restrict__ x,
                                                            float *__restrict__ dx, int64_t n4, int64_t size,
-                                                           const float2 *__restrict__ bounds,
-                                                           float2 *__restrict__ partial, GradMode m) {
-  const float2 b = bounds[0];
+                                                           RangeInputs q, float2 *__restrict__ partial, GradMode m) {
+  const float2 b = q.bounds(0);
   float lo = 0.0f, hi = 0.0f;
   const int64_t tiles = (n4 + kBlock * 4 - 1) / (kBlock * 4);
   for (int64_t t = blockIdx.x; t < tiles; t += gridDim.x) {
+    int64_t at[4];
+    bool in[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int64_t i = t * (kBlock * 4) + j * kBlock + threadIdx.x;
-      if (i < n4)
-        minmax_grad4(dy, x, dx, 4 * i, b, m, lo, hi);
+      in[j] = i < n4, at[j] = 4 * i;
     }
+    minmax_grad4<4>(dy, x, dx, at, in, b, m, lo, hi);
   }
   if (blockIdx.x == 0) {
     const int64_t i = 4 * n4 + threadIdx.x;
@@ -373,14 +394,21 @@ __global__ __launch_bounds__(kBlock) void minmax_grad_flat(const float *__restri
 // R0 * gridDim.y.
 __global__ __launch_bounds__(kBlock) void minmax_grad_rows(const float *__restrict__ dy, const float *__restrict__ x,
                                                            float *__restrict__ dx, int64_t K, int64_t R1,
-                                                           const float2 *__restrict__ bounds,
-                                                           float2 *__restrict__ partial, int64_t nchunks, GradMode m) {
+                                                           RangeInputs q, float2 *__restrict__ partial,
+                                                           int64_t nchunks, GradMode m) {
   const int64_t row = blockIdx.x, r0 = row / K, k = row - r0 * K;
-  const float2 b = bounds[k];
+  const float2 b = q.bounds(k);
   const int64_t n4 = R1 / 4, at0 = row * R1;
   float lo = 0.0f, hi = 0.0f;
-  for (int64_t i = (int64_t)blockIdx.y * kBlock + threadIdx.x; i < n4; i += (int64_t)gridDim.y * kBlock)
-    minmax_grad4(dy, x, dx, at0 + 4 * i, b, m, lo, hi);
+  const int64_t step = (int64_t)gridDim.y * kBlock;
+  for (int64_t i0 = (int64_t)blockIdx.y * kBlock + threadIdx.x; i0 < n4; i0 += 4 * step) {
+    int64_t at[4];
+    bool in[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      in[j] = i0 + j * step < n4, at[j] = at0 + 4 * (i0 + j * step);
+    minmax_grad4<4>(dy, x, dx, at, in, b, m, lo, hi);
+  }
   if (m.sums)
     block_sums(lo, hi, partial + k * nchunks + r0 * gridDim.y + blockIdx.y);
 }
@@ -548,7 +576,7 @@ RangeGradPlan make_range_plan(const int64_t *xshape, int ndim, const int64_t *qs
   P.flat_chunks = 0;
   if (P.L.ok && P.L.K == 1) {
     const int64_t tiles = (P.L.total / 4 + kBlock * 4 - 1) / (kBlock * 4);
-    P.flat_chunks = tiles < 1 ? 1 : (tiles > 2048 ? 2048 : tiles);
+    P.flat_chunks = tiles < 1 ? 1 : (tiles > 1024 ? 1024 : tiles);
     most = most > P.flat_chunks ? most : P.flat_chunks;
   }
   P.row_parts = 0;
@@ -668,16 +696,18 @@ int nbla_hip_min_max_quantize_backward_f32(const float *dy, const float *x, floa
   const bool range_grads = !(x_min_max || ema) && (g_qr_min || g_qr_max);
   float2 *bounds = static_cast<float2 *>(workspace);
   float2 *partial = reinterpret_cast<float2 *>(static_cast<char *>(workspace) + P.bounds_bytes);
-  if ((dx && ste_fine_grained) || range_grads) {
-    hipLaunchKernelGGL(minmax_bounds, dim3((unsigned)((P.L.K + 63) / 64)), dim3(64), 0, stream, qr_min, ql_min, ql_max,
-                       scale, bounds, P.L.K);
-    NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward bounds");
-  }
   // dx and the range sums in one pass over dy and x, where a kernel of that kind covers the layout (a plain copy of dy
   // and the per-tensor mask without sums are as fast on the element-wise kernels below)
   const GradMode mode{dx ? (ste_fine_grained ? 2 : 1) : 0, accum_x, range_grads ? 1 : 0};
   const bool wanted = range_grads || (mode.dx_mode == 2 && P.L.K > 1);
   const bool vec = aligned16(dy) && aligned16(x) && (!dx || aligned16(dx));
+  const bool one_range_per_block = wanted && !P.inner && vec && (P.flat_chunks || P.row_parts);
+  if (((dx && ste_fine_grained) || range_grads) && !one_range_per_block) {
+    hipLaunchKernelGGL(minmax_bounds, dim3((unsigned)((P.L.K + 63) / 64)), dim3(64), 0, stream, qr_min, ql_min, ql_max,
+                       scale, bounds, P.L.K);
+    NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward bounds");
+  }
+  const RangeInputs ranges{qr_min, ql_min, ql_max, scale};
   if (wanted && P.inner) {
     MinMaxInner I = P.I;
     const bool quads = I.Wk % 4 == 0 && vec;
@@ -702,7 +732,7 @@ int nbla_hip_min_max_quantize_backward_f32(const float *dy, const float *x, floa
   }
   if (wanted && P.flat_chunks && vec) {
     hipLaunchKernelGGL(minmax_grad_flat, dim3((unsigned)P.flat_chunks), dim3(kBlock), 0, stream, dy, x, dx,
-                       P.L.total / 4, P.L.total, bounds, partial, mode);
+                       P.L.total / 4, P.L.total, ranges, partial, mode);
     NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward");
     launch_range_final(partial, P.flat_chunks, g_qr_min, g_qr_max, accum_min, accum_max, 1, stream);
     NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward range gradients");
@@ -711,7 +741,7 @@ int nbla_hip_min_max_quantize_backward_f32(const float *dy, const float *x, floa
   if (wanted && P.row_parts && vec) {
     const int64_t chunks = P.L.R0 * P.row_parts;
     hipLaunchKernelGGL(minmax_grad_rows, dim3((unsigned)(P.L.R0 * P.L.K), (unsigned)P.row_parts), dim3(kBlock), 0,
-                       stream, dy, x, dx, P.L.K, P.L.R1, bounds, partial, chunks, mode);
+                       stream, dy, x, dx, P.L.K, P.L.R1, ranges, partial, chunks, mode);
     NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward");
     if (range_grads) {
       launch_range_final(partial, chunks, g_qr_min, g_qr_max, accum_min, accum_max, P.L.K, stream);
