@@ -338,6 +338,7 @@ struct MinMaxPlan {
   int nchunks;           // blocks (and partials) per k
   size_t params_bytes, partial_bytes;
   bool inner;            // the strided pattern takes the kernels of MinMaxInner
+  bool rows;             // ... or, its innermost axis reduced (and short runs per channel), those of MinMaxRows
 };
 
 MinMaxPlan make_plan(const int64_t *xshape, int ndim, const int64_t *qshape) {
@@ -362,6 +363,17 @@ MinMaxPlan make_plan(const int64_t *xshape, int ndim, const int64_t *qshape) {
       if (I.ok) {
         P.inner = true;
         want = inner_chunks(I);
+      }
+    }
+  }
+  P.rows = false;
+  if (!P.inner && (!P.L.ok || short_rows(P.L))) {
+    MinMaxAxes A;
+    if (split_axes(xshape, ndim, qshape, A)) {
+      const MinMaxRows R = row_form(A);
+      if (R.ok) {
+        P.rows = true;
+        want = row_chunks(R);
       }
     }
   }
@@ -397,6 +409,15 @@ struct Extrema {
     vmax = __builtin_fmaxf(vmax, v);
     const uint32_t u = __float_as_uint(v);
     if ((u << 1) == 0u && zidx == 0xffffffffu) {
+      zidx = i;
+      zsign = u >> 31;
+    }
+  }
+  __device__ __forceinline__ void take_any(float v, uint32_t i) { // i in any order
+    vmin = __builtin_fminf(vmin, v);
+    vmax = __builtin_fmaxf(vmax, v);
+    const uint32_t u = __float_as_uint(v);
+    if ((u << 1) == 0u && i < zidx) {
       zidx = i;
       zsign = u >> 31;
     }
@@ -847,6 +868,98 @@ __global__ __launch_bounds__(kRedBlock) void minmax_apply_inner(const float *__r
     }
   }
 }
+// The row form (MinMaxRows: the innermost axis reduced, T lanes per run).  Block (tile of 256 / T kept indices,
+// chunk); a thread's elements all belong to its kept index, so it keeps one set of extrema, which the T lanes of the
+// run then fold.
+template <int kVec>
+__global__ __launch_bounds__(kRedBlock) void minmax_reduce_rowform(const float *__restrict__ x,
+                                                                   MinMaxPartial *__restrict__ partial, MinMaxAxes A,
+                                                                   MinMaxRows R, int T, int nchunks) {
+  const int tid = threadIdx.x, li = tid & (T - 1), slot = tid / T, rps = kRedBlock / T;
+  const int64_t k = (int64_t)blockIdx.x * rps + slot;
+  const bool k_in = k < R.K;
+  const int chunk = blockIdx.y;
+  const RowWalk W = row_walk(R, chunk, nchunks);
+  const float *base = x + strided_offset(k_in ? k : 0, A.nkept, A.ksize, A.kstride);
+  Extrema ex;
+  ex.init();
+  constexpr int kRows = 4; // outer reduced indices in flight per lane
+  for (int64_t ro = W.ro_begin; ro < W.ro_end; ro += kRows) {
+    int64_t off[kRows];
+#pragma unroll
+    for (int j = 0; j < kRows; ++j)
+      off[j] = (A.nred > 1 && ro + j < W.ro_end) ? strided_offset(ro + j, A.nred - 1, A.rsize, A.rstride) : 0;
+    for (int64_t ri0 = 0; ri0 < R.Rin; ri0 += (int64_t)T * kVec) {
+      const int64_t ri = ri0 + (int64_t)li * kVec;
+      InnerRow<kVec> v[kRows];
+#pragma unroll
+      for (int j = 0; j < kRows; ++j) {
+        if (k_in && ro + j < W.ro_end && ri < R.Rin)
+          v[j].load(base + off[j] + ri);
+        else
+          v[j].fill(__uint_as_float(0x7fc00000u)); // NaN: ignored by the scan
+      }
+#pragma unroll
+      for (int j = 0; j < kRows; ++j)
+#pragma unroll
+        for (int c = 0; c < kVec; ++c)
+          ex.take_any(v[j].v[c], (uint32_t)((ro + j) * R.Rin + ri + c));
+    }
+  }
+  for (int o = T >> 1; o >= 1; o >>= 1) {
+    const float a = __shfl_xor(ex.vmin, o), b = __shfl_xor(ex.vmax, o);
+    const uint32_t zi = __shfl_xor(ex.zidx, o), zs = __shfl_xor(ex.zsign, o);
+    ex.merge(a, b, zi, zs);
+  }
+  if (li == 0 && k_in)
+    partial[k * nchunks + chunk] = ex.pack();
+}
+template <int kVec>
+__global__ __launch_bounds__(kRedBlock) void minmax_apply_rowform(const float *__restrict__ x, float *__restrict__ y,
+                                                                  MinMaxAxes A, MinMaxRows R, int T, int nchunks,
+                                                                  const float4_t *__restrict__ params) {
+  const int tid = threadIdx.x, li = tid & (T - 1), slot = tid / T, rps = kRedBlock / T;
+  const int64_t k = (int64_t)blockIdx.x * rps + slot;
+  const bool k_in = k < R.K;
+  const int chunk = blockIdx.y;
+  const RowWalk W = row_walk(R, chunk, nchunks);
+  const int64_t base = strided_offset(k_in ? k : 0, A.nkept, A.ksize, A.kstride);
+  const float4_t pr = params[k_in ? k : 0];
+  constexpr int kRows = 4;
+  for (int64_t ro = W.ro_begin; ro < W.ro_end; ro += kRows) {
+    int64_t off[kRows];
+#pragma unroll
+    for (int j = 0; j < kRows; ++j)
+      off[j] = base + ((A.nred > 1 && ro + j < W.ro_end) ? strided_offset(ro + j, A.nred - 1, A.rsize, A.rstride) : 0);
+    for (int64_t ri0 = 0; ri0 < R.Rin; ri0 += (int64_t)T * kVec) {
+      const int64_t ri = ri0 + (int64_t)li * kVec;
+      InnerRow<kVec> v[kRows];
+#pragma unroll
+      for (int j = 0; j < kRows; ++j) {
+        if (k_in && ro + j < W.ro_end && ri < R.Rin)
+          v[j].load(x + off[j] + ri);
+        else
+          v[j].fill(0.0f);
+      }
+#pragma unroll
+      for (int j = 0; j < kRows; ++j) {
+        if (!(k_in && ro + j < W.ro_end && ri < R.Rin))
+          continue;
+        float *dst = y + off[j] + ri;
+        if (kVec == 4) {
+          float4_t r;
+          r.x = minmax_apply(v[j].v[0], pr.x, pr.y, pr.z);
+          r.y = minmax_apply(v[j].v[1 % kVec], pr.x, pr.y, pr.z);
+          r.z = minmax_apply(v[j].v[2 % kVec], pr.x, pr.y, pr.z);
+          r.w = minmax_apply(v[j].v[3 % kVec], pr.x, pr.y, pr.z);
+          __builtin_nontemporal_store(r, reinterpret_cast<float4_t *>(dst));
+        } else {
+          __builtin_nontemporal_store(minmax_apply(v[j].v[0], pr.x, pr.y, pr.z), dst);
+        }
+      }
+    }
+  }
+}
 // Element i of x (dense, row-major) belongs to the kept index formed by its coordinates along the kept axes.
 __global__ __launch_bounds__(kBlock) void minmax_apply_strided(const float *__restrict__ x, float *__restrict__ y,
                                                                int64_t total, MinMaxAxes A,
@@ -873,11 +986,11 @@ int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, in
                   "x.shape and ql_min.shape must be same except for i-th dimension where ql_min.shape[i] == 1.");
   MinMaxPlan P = make_plan(xshape, ndim, qshape);
   MinMaxAxes axes;
-  if ((!P.L.ok || P.inner) && !split_axes(xshape, ndim, qshape, axes))
+  if ((!P.L.ok || P.inner || P.rows) && !split_axes(xshape, ndim, qshape, axes))
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than eight kept or eight reduced axes of size above one.");
   if (P.L.total == 0)
     return NBLA_HIP_OK;
-  if (scratch_limit && P.inner && P.params_bytes + P.partial_bytes > scratch_limit) {
+  if (scratch_limit && (P.inner || P.rows) && P.params_bytes + P.partial_bytes > scratch_limit) {
     P.nchunks = 1; // the fixed scratch holds one partial result per range
     P.partial_bytes = round_up((size_t)P.L.K * 16, 256);
   }
@@ -900,7 +1013,7 @@ int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, in
   const bool vec_ok = aligned16(x) && (L.R1 % 4 == 0 || L.K == 1);
   int nchunks = P.nchunks;
 
-  if (!L.ok || P.inner) { // kept axes separated by reduced ones, or all behind them: the strided kernels
+  if (!L.ok || P.inner || P.rows) { // kept axes separated by reduced ones, all behind them, or short runs
     if (L.K > 0x7fffffffll)
       return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than 2^31 - 1 quantization ranges.");
     MinMaxInner inner = P.inner ? inner_form(axes) : MinMaxInner{false};
@@ -932,6 +1045,34 @@ int min_max_quantize_forward(const float *x, float *y, const int64_t *xshape, in
         hipLaunchKernelGGL(minmax_apply_inner<4>, grid, dim3(kRedBlock), 0, stream, x, y, axes, inner, nchunks, params);
       else
         hipLaunchKernelGGL(minmax_apply_inner<1>, grid, dim3(kRedBlock), 0, stream, x, y, axes, inner, nchunks, params);
+      NBLA_HIP_LAUNCH_CHECK("min_max_quantize apply");
+      return NBLA_HIP_OK;
+    }
+    if (P.rows) {
+      const MinMaxRows R = row_form(axes);
+      const bool quads = R.Rin % 4 == 0 && aligned16(x) && aligned16(y);
+      const int T = row_lanes(R, quads ? 4 : 1);
+      const int64_t rps = kRedBlock / T;
+      const dim3 grid((unsigned)((R.K + rps - 1) / rps), (unsigned)nchunks);
+      if (x_min_max) {
+        if (quads)
+          hipLaunchKernelGGL(minmax_reduce_rowform<4>, grid, dim3(kRedBlock), 0, stream, x, partial, axes, R, T, nchunks);
+        else
+          hipLaunchKernelGGL(minmax_reduce_rowform<1>, grid, dim3(kRedBlock), 0, stream, x, partial, axes, R, T, nchunks);
+        NBLA_HIP_LAUNCH_CHECK("min_max_quantize reduction");
+      }
+      MinMaxScalars sc;
+      sc.decay = (float)decay;
+      sc.one_minus_decay = (float)(1.0 - (double)decay);
+      sc.eps = eps;
+      sc.x_min_max = x_min_max;
+      sc.ema = ema;
+      launch_minmax_finalize(L.K, partial, nchunks, qr_min, qr_max, ql_min, ql_max, scale, params, sc, stream);
+      NBLA_HIP_LAUNCH_CHECK("min_max_quantize finalize");
+      if (quads)
+        hipLaunchKernelGGL(minmax_apply_rowform<4>, grid, dim3(kRedBlock), 0, stream, x, y, axes, R, T, nchunks, params);
+      else
+        hipLaunchKernelGGL(minmax_apply_rowform<1>, grid, dim3(kRedBlock), 0, stream, x, y, axes, R, T, nchunks, params);
       NBLA_HIP_LAUNCH_CHECK("min_max_quantize apply");
       return NBLA_HIP_OK;
     }

@@ -509,6 +509,80 @@ __global__ __launch_bounds__(kBlock) void minmax_grad_inner(const float *__restr
   }
 }
 
+// The row form (MinMaxRows: the innermost axis reduced, T lanes per run of Rin elements), block (tile of 256 / T kept
+// indices, chunk) as in the forward's kernels of this form; the sums of kept index k go to partial[k * nchunks + chunk].
+template <int kVec>
+__global__ __launch_bounds__(kBlock) void minmax_grad_rowform(const float *__restrict__ dy, const float *__restrict__ x,
+                                                              float *__restrict__ dx, MinMaxAxes A, MinMaxRows R, int T,
+                                                              int nchunks, const float2 *__restrict__ bounds,
+                                                              float2 *__restrict__ partial, GradMode m) {
+  const int tid = threadIdx.x, li = tid & (T - 1), slot = tid / T, rps = kBlock / T;
+  const int64_t k = (int64_t)blockIdx.x * rps + slot;
+  const bool k_in = k < R.K;
+  const int chunk = blockIdx.y;
+  const RowWalk W = row_walk(R, chunk, nchunks);
+  const int64_t base = strided_offset(k_in ? k : 0, A.nkept, A.ksize, A.kstride);
+  const float2 b = bounds[k_in ? k : 0];
+  float lo = 0.0f, hi = 0.0f;
+  constexpr int kRows = 4; // outer reduced indices in flight per lane
+  for (int64_t ro = W.ro_begin; ro < W.ro_end; ro += kRows) {
+    int64_t off[kRows];
+#pragma unroll
+    for (int j = 0; j < kRows; ++j)
+      off[j] = base + ((A.nred > 1 && ro + j < W.ro_end) ? strided_offset(ro + j, A.nred - 1, A.rsize, A.rstride) : 0);
+    for (int64_t ri0 = 0; ri0 < R.Rin; ri0 += (int64_t)T * kVec) {
+      const int64_t ri = ri0 + (int64_t)li * kVec;
+      InnerRow<kVec> g[kRows], v[kRows], o[kRows];
+#pragma unroll
+      for (int j = 0; j < kRows; ++j) {
+        const bool in = k_in && ro + j < W.ro_end && ri < R.Rin;
+        const int64_t at = off[j] + ri;
+        if (in)
+          g[j].load(dy + at);
+        else
+          g[j].fill(0.0f);
+        if (in && (m.dx_mode == 2 || m.sums))
+          v[j].load(x + at);
+        else
+          v[j].fill(0.0f);
+        if (in && m.dx_mode && m.accum)
+          o[j].load(dx + at);
+        else
+          o[j].fill(0.0f);
+      }
+#pragma unroll
+      for (int j = 0; j < kRows; ++j) {
+        if (!(k_in && ro + j < W.ro_end && ri < R.Rin))
+          continue;
+        if (m.dx_mode) {
+          float *dst = dx + off[j] + ri;
+          float r[kVec];
+#pragma unroll
+          for (int c = 0; c < kVec; ++c)
+            r[c] = minmax_dx(g[j].v[c], v[j].v[c], o[j].v[c], b, m);
+          if (kVec == 4)
+            store4(dst, float4_t{r[0], r[1 % kVec], r[2 % kVec], r[3 % kVec]});
+          else
+            __builtin_nontemporal_store(r[0], dst);
+        }
+        if (m.sums) {
+#pragma unroll
+          for (int c = 0; c < kVec; ++c)
+            minmax_sums(g[j].v[c], v[j].v[c], b, lo, hi);
+        }
+      }
+    }
+  }
+  if (!m.sums)
+    return;
+  for (int o = T >> 1; o >= 1; o >>= 1) {
+    lo += __shfl_xor(lo, o);
+    hi += __shfl_xor(hi, o);
+  }
+  if (li == 0 && k_in)
+    partial[k * nchunks + chunk] = float2{lo, hi};
+}
+
 // A wavefront per range: lane l adds the partial sums l, l + 64, ... in order, then the lanes are added up.
 __global__ __launch_bounds__(64) void minmax_range_grad_final_wave(const float2 *__restrict__ partial, int64_t nchunks,
                                                                    float *__restrict__ g_min, float *__restrict__ g_max,
@@ -542,6 +616,9 @@ struct RangeGradPlan {
   MinMaxAxes axes;
   MinMaxInner I;
   int inner_chunks;
+  bool rows;            // the runs-along-the-innermost-reduced-axis form applies
+  MinMaxRows R;
+  int row_form_chunks;
   int64_t flat_chunks;  // K == 1
   int64_t row_parts;    // rows form (R1 % 4 == 0, R1 >= 256): blocks along a row; partial sums per range = R0 * row_parts
   size_t bounds_bytes, partial_bytes;
@@ -571,6 +648,16 @@ RangeGradPlan make_range_plan(const int64_t *xshape, int ndim, const int64_t *qs
       P.inner = true;
       P.inner_chunks = (int)inner_chunks(P.I);
       most = most > P.inner_chunks ? most : P.inner_chunks;
+    }
+  }
+  P.rows = false;
+  P.row_form_chunks = 1;
+  if (!P.inner && (!P.L.ok || short_rows(P.L)) && split_axes(xshape, ndim, qshape, P.axes)) {
+    P.R = row_form(P.axes);
+    if (P.R.ok) {
+      P.rows = true;
+      P.row_form_chunks = (int)row_chunks(P.R);
+      most = most > P.row_form_chunks ? most : P.row_form_chunks;
     }
   }
   P.flat_chunks = 0;
@@ -683,7 +770,7 @@ int nbla_hip_min_max_quantize_backward_f32(const float *dy, const float *x, floa
   MinMaxAxes axes;
   if (!P.L.ok && !split_axes(xshape, ndim, qshape, axes))
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than eight kept or eight reduced axes of size above one.");
-  if (P.L.K > 0x7fffffffll && (!P.L.ok || P.inner))
+  if (P.L.K > 0x7fffffffll && (!P.L.ok || P.inner || P.rows))
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "more than 2^31 - 1 quantization ranges.");
   if (P.L.total == 0)
     return NBLA_HIP_OK;
@@ -701,7 +788,7 @@ int nbla_hip_min_max_quantize_backward_f32(const float *dy, const float *x, floa
   const GradMode mode{dx ? (ste_fine_grained ? 2 : 1) : 0, accum_x, range_grads ? 1 : 0};
   const bool wanted = range_grads || (mode.dx_mode == 2 && P.L.K > 1);
   const bool vec = aligned16(dy) && aligned16(x) && (!dx || aligned16(dx));
-  const bool one_range_per_block = wanted && !P.inner && vec && (P.flat_chunks || P.row_parts);
+  const bool one_range_per_block = wanted && !P.inner && !P.rows && vec && (P.flat_chunks || P.row_parts);
   if (((dx && ste_fine_grained) || range_grads) && !one_range_per_block) {
     hipLaunchKernelGGL(minmax_bounds, dim3((unsigned)((P.L.K + 63) / 64)), dim3(64), 0, stream, qr_min, ql_min, ql_max,
                        scale, bounds, P.L.K);
@@ -726,6 +813,24 @@ int nbla_hip_min_max_quantize_backward_f32(const float *dy, const float *x, floa
     NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward");
     if (range_grads) {
       launch_range_final(partial, P.inner_chunks, g_qr_min, g_qr_max, accum_min, accum_max, P.L.K, stream);
+      NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward range gradients");
+    }
+    return NBLA_HIP_OK;
+  }
+  if (wanted && P.rows) {
+    const bool quads = P.R.Rin % 4 == 0 && vec;
+    const int T = row_lanes(P.R, quads ? 4 : 1);
+    const int64_t rps = kBlock / T;
+    const dim3 grid((unsigned)((P.R.K + rps - 1) / rps), (unsigned)P.row_form_chunks);
+    if (quads)
+      hipLaunchKernelGGL(minmax_grad_rowform<4>, grid, dim3(kBlock), 0, stream, dy, x, dx, P.axes, P.R, T,
+                         P.row_form_chunks, bounds, partial, mode);
+    else
+      hipLaunchKernelGGL(minmax_grad_rowform<1>, grid, dim3(kBlock), 0, stream, dy, x, dx, P.axes, P.R, T,
+                         P.row_form_chunks, bounds, partial, mode);
+    NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward");
+    if (range_grads) {
+      launch_range_final(partial, P.row_form_chunks, g_qr_min, g_qr_max, accum_min, accum_max, P.L.K, stream);
       NBLA_HIP_LAUNCH_CHECK("min_max_quantize backward range gradients");
     }
     return NBLA_HIP_OK;

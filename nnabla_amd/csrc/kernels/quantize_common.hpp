@@ -177,6 +177,59 @@ template <> struct InnerRow<4> {
   __device__ __forceinline__ void fill(float f) { v[0] = v[1] = v[2] = v[3] = f; }
 };
 
+// The counterpart for patterns whose innermost axis is reduced (q shape (C, H, 1), or (1, C, 1, 1) over short
+// rows): a run of Rin contiguous elements belongs to one range.  T lanes share a run (each kVec consecutive
+// elements per step), 256 / T runs of consecutive kept indices are in flight per step, and a block (tile of kept
+// indices, chunk) walks a run of the outer reduced indices in row-major order like the reference's scan.
+struct MinMaxRows {
+  bool ok;
+  int64_t K, Rin, Rout; // kept indices, extent of the innermost reduced axis, combinations of the other reduced axes
+};
+inline MinMaxRows row_form(const MinMaxAxes &A) {
+  MinMaxRows R;
+  R.ok = A.nkept >= 1 && A.nred >= 1 && A.rstride[A.nred - 1] == 1;
+  if (!R.ok)
+    return R;
+  R.K = 1;
+  for (int d = 0; d < A.nkept; ++d)
+    R.K *= A.ksize[d];
+  R.Rin = A.rsize[A.nred - 1];
+  R.Rout = 1;
+  for (int d = 0; d + 1 < A.nred; ++d)
+    R.Rout *= A.rsize[d];
+  R.ok = R.K < ((int64_t)1 << 31) && R.Rin < ((int64_t)1 << 31);
+  return R;
+}
+// lanes per run for kVec elements per lane and step: the power of two covering the run, at most 64
+inline int row_lanes(const MinMaxRows &R, int vec) {
+  int t = 1;
+  while (t < 64 && (int64_t)t * vec < R.Rin)
+    t *= 2;
+  return t;
+}
+// Blocks per tile of kept indices (independent of the lanes per run, which the pointers' alignment decides).
+inline int64_t row_chunks(const MinMaxRows &R) {
+  const int64_t tiles = (R.K + 3) / 4;
+  int64_t want = (4096 + tiles - 1) / tiles;
+  if (want > R.Rout)
+    want = R.Rout;
+  if (want > 1024)
+    want = 1024;
+  return want < 1 ? 1 : want;
+}
+// Short runs per channel (q shape (1, C, 1, 1) over rows of fewer than 256 elements) take this form as well.
+inline bool short_rows(const MinMaxLayout &L) { return L.ok && L.K > 1 && L.R1 > 1 && L.R1 < 256; }
+struct RowWalk {
+  int64_t ro_begin, ro_end;
+};
+__device__ __forceinline__ RowWalk row_walk(const MinMaxRows &R, int chunk, int nchunks) {
+  RowWalk w;
+  const int64_t per = (R.Rout + nchunks - 1) / nchunks;
+  w.ro_begin = (int64_t)chunk * per;
+  w.ro_end = w.ro_begin + per < R.Rout ? w.ro_begin + per : R.Rout;
+  return w;
+}
+
 // nudge_qr_min_max (min_max_quantize.cpp:363-390): the representable range [m', M'] whose zero point is an integer
 // level, one rounded fp32 operation at a time.
 __host__ __device__ inline void nudge_qr_min_max(float qr_min, float ql_min, float ql_max, float scale, float &m_n,

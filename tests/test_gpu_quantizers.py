@@ -238,6 +238,10 @@ MMQ_SHAPES = [
     # reduced positions split over many blocks
     ((300, 520), (1, 520)), ((40, 33, 20), (1, 1, 20)), ((7, 3, 5, 9), (1, 1, 5, 9)), ((5000, 3), (1, 3)),
     ((9, 4100, 2, 2), (1, 1, 2, 2)),
+    # the innermost axis reduced in short runs (a few lanes per run): per channel over short rows, kept axes separated
+    # by reduced ones, runs longer than one step of the lanes, runs that are no multiple of four
+    ((6, 40, 30, 56), (1, 40, 30, 1)), ((9, 3, 50, 12), (9, 1, 50, 1)), ((5, 3, 7, 300), (5, 1, 7, 1)),
+    ((4, 6, 10, 70), (1, 6, 10, 1)), ((700, 9, 5), (1, 9, 1)), ((2, 3, 2000, 6), (2, 1, 2000, 1)),
 ]
 
 

@@ -84,7 +84,11 @@ def test_pow2_backward_all_binade_cuts(dev):
                                            ((33, 1025), (1, 1)), ((40, 70, 130), (1, 1, 1)),
                                            ((6, 10, 8, 12), (1, 10, 1, 12)), ((4, 10, 100), (4, 1, 100)),
                                            ((300, 520), (1, 520)), ((40, 33, 20), (1, 1, 20)),
-                                           ((7, 3, 5, 9), (1, 1, 5, 9)), ((5000, 3), (1, 3))])
+                                           ((7, 3, 5, 9), (1, 1, 5, 9)), ((5000, 3), (1, 3)),
+                                           # the innermost axis reduced in short runs
+                                           ((6, 40, 30, 56), (1, 40, 30, 1)), ((9, 3, 50, 12), (9, 1, 50, 1)),
+                                           ((5, 3, 7, 300), (5, 1, 7, 1)), ((4, 6, 10, 70), (1, 6, 10, 1)),
+                                           ((700, 9, 5), (1, 9, 1)), ((2, 3, 2000, 6), (2, 1, 2000, 1))])
 @pytest.mark.parametrize("fine", [True, False])
 def test_min_max_backward(dev, xshape, qshape, fine):
     x, dy = _rand(xshape, 11, 3.0), _rand(xshape, 12)
@@ -154,7 +158,8 @@ def test_min_max_backward_random_axis_patterns(dev, xshape, qshape):
 
 
 @pytest.mark.parametrize("xshape,qshape", [((3, 5, 40, 64), (1, 5, 1, 1)), ((6, 10, 8, 12), (1, 10, 1, 12)),
-                                           ((300, 520), (1, 520)), ((5, 7, 9), (5, 1, 9)), ((4, 6, 5, 3), (1, 6, 1, 1))])
+                                           ((300, 520), (1, 520)), ((5, 7, 9), (5, 1, 9)), ((4, 6, 5, 3), (1, 6, 1, 1)),
+                                           ((9, 3, 50, 12), (9, 1, 50, 1)), ((4, 6, 10, 70), (1, 6, 10, 1))])
 @pytest.mark.parametrize("accumulate", [False, True])
 def test_min_max_backward_input_gradient_alone(dev, xshape, qshape, accumulate):
     """Ranges that follow the statistics of x (x_min_max) are not learnt: only dx is formed, by the same one-pass
