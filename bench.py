@@ -230,10 +230,11 @@ def bench_quantizers(dev, iters):
     nb = 12.0 * a.numel()
     out["min_max_quantize[64,256,56,56] x_min_max, ranges [1,256,1,56]"] = {
         "ms": ms, "bytes": nb, "GBs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
-    # ranges per channel and per column (every kept axis behind the reduced ones), and the backward pass with learnt
-    # ranges: dx and both range gradients from one pass over dy and x (12 B/elem)
+    # ranges per channel, per column (every kept axis behind the reduced ones) and per (channel, row) (the innermost
+    # axis reduced in short runs), and the backward pass with learnt ranges: dx and both range gradients from one pass
+    # over dy and x (12 B/elem)
     dy = torch.randn(a.shape, generator=g).to(dev)
-    for qshape in ((1, 1, 1, 1), (1, 256, 1, 1), (1, 1, 1, 56)):
+    for qshape in ((1, 1, 1, 1), (1, 256, 1, 1), (1, 1, 1, 56), (1, 256, 56, 1)):
         qs = lambda v: torch.full(qshape, v, device=dev)
         qmn, qmx, lmn, lmx = qs(-6.0), qs(6.0), qs(0.0), qs(255.0)
         tag = "ranges [%s]" % ",".join(str(v) for v in qshape)

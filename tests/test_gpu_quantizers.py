@@ -242,6 +242,7 @@ MMQ_SHAPES = [
     # by reduced ones, runs longer than one step of the lanes, runs that are no multiple of four
     ((6, 40, 30, 56), (1, 40, 30, 1)), ((9, 3, 50, 12), (9, 1, 50, 1)), ((5, 3, 7, 300), (5, 1, 7, 1)),
     ((4, 6, 10, 70), (1, 6, 10, 1)), ((700, 9, 5), (1, 9, 1)), ((2, 3, 2000, 6), (2, 1, 2000, 1)),
+    ((8, 16, 27, 27), (1, 16, 1, 1)), ((3, 4, 4097), (3, 4, 1)),
 ]
 
 

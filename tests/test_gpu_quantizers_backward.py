@@ -88,7 +88,8 @@ def test_pow2_backward_all_binade_cuts(dev):
                                            # the innermost axis reduced in short runs
                                            ((6, 40, 30, 56), (1, 40, 30, 1)), ((9, 3, 50, 12), (9, 1, 50, 1)),
                                            ((5, 3, 7, 300), (5, 1, 7, 1)), ((4, 6, 10, 70), (1, 6, 10, 1)),
-                                           ((700, 9, 5), (1, 9, 1)), ((2, 3, 2000, 6), (2, 1, 2000, 1))])
+                                           ((700, 9, 5), (1, 9, 1)), ((2, 3, 2000, 6), (2, 1, 2000, 1)),
+                                           ((8, 16, 27, 27), (1, 16, 1, 1)), ((3, 4, 4097), (3, 4, 1))])
 @pytest.mark.parametrize("fine", [True, False])
 def test_min_max_backward(dev, xshape, qshape, fine):
     x, dy = _rand(xshape, 11, 3.0), _rand(xshape, 12)
