@@ -679,8 +679,11 @@ int nbla_hip_binary2_backward_f32(int op, int input, const float *dy,
  * element the operand's element took part in), transform_binary_grad0 / grad1,
  * :286-336: for a broadcast operand a fixed-order parallel sum where the
  * reference adds one after the other in fp32 (equal to rounding, the same from
- * run to run).  powf / logf are the device's, not the host libm's: the power's
- * bits are not pinned. */
+ * run to run).  With a workspace of nbla_hip_broadcast2_backward_workspace_bytes
+ * (256-byte aligned; 0 bytes where the operand is not broadcast) the terms of
+ * an element are spread over blocks; workspace NULL: one block per element of
+ * the operand, whatever the number of its terms.  powf / logf are the device's,
+ * not the host libm's: the power's bits are not pinned. */
 #define NBLA_HIP_BINARY2_ADD 3
 #define NBLA_HIP_BINARY2_POW 4
 int nbla_hip_broadcast2_f32(int op, const float *x0, const int64_t *shape0,
@@ -690,7 +693,12 @@ int nbla_hip_broadcast2_backward_f32(int op, int input, const float *dy,
                                      const float *x0, const int64_t *shape0,
                                      const float *x1, const int64_t *shape1,
                                      float *dx, int ndim, int accum,
+                                     void *workspace, size_t workspace_bytes,
                                      void *stream);
+size_t nbla_hip_broadcast2_backward_workspace_bytes(int input,
+                                                    const int64_t *shape0,
+                                                    const int64_t *shape1,
+                                                    int ndim);
 /* dst[r * dst_stride + i] (+)= src[r * src_stride + i], r < rows, i < len:
  * one input's share of Concatenate<float>::forward_impl / backward_impl,
  * src/nbla/function/generic/concatenate.cpp:62-104 (rows = outer_size_, len =

@@ -664,9 +664,11 @@ void Add2Hip<T>::backward_impl(const Variables &inputs, const Variables &outputs
     T *dx = inputs[i]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[i]);
     if (same)
       NBLA_HIP_CALL(nbla_hip_add2_backward_f32(dy, dx, (size_t)inputs[0]->size(), accum[i], nullptr));
-    else // utils/base_transform_binary.hpp:358-392
+    else { // utils/base_transform_binary.hpp:358-392
+      HipWorkspace ws(nbla_hip_broadcast2_backward_workspace_bytes(i, s0.data(), s1.data(), (int)s0.size()), this->ctx_);
       NBLA_HIP_CALL(nbla_hip_broadcast2_backward_f32(NBLA_HIP_BINARY2_ADD, i, dy, nullptr, s0.data(), nullptr, s1.data(),
-                                                     dx, (int)s0.size(), accum[i], nullptr));
+                                                     dx, (int)s0.size(), accum[i], ws.pointer(), ws.bytes(), nullptr));
+    }
   }
 }
 
@@ -703,9 +705,12 @@ void Add2Hip<T>::backward_impl(const Variables &inputs, const Variables &outputs
       if (OP != NBLA_HIP_BINARY2_POW && same)                                                                          \
         NBLA_HIP_CALL(nbla_hip_binary2_backward_f32(OP, i, dy, x0, x1, dx, (size_t)inputs[0]->size(), accum[i],        \
                                                     nullptr));                                                         \
-      else                                                                                                             \
+      else {                                                                                                           \
+        HipWorkspace ws(nbla_hip_broadcast2_backward_workspace_bytes(i, s0.data(), s1.data(), (int)s0.size()),         \
+                        this->ctx_);                                                                                   \
         NBLA_HIP_CALL(nbla_hip_broadcast2_backward_f32(OP, i, dy, x0, s0.data(), x1, s1.data(), dx, (int)s0.size(),    \
-                                                       accum[i], nullptr));                                            \
+                                                       accum[i], ws.pointer(), ws.bytes(), nullptr));                  \
+      }                                                                                                                \
     }                                                                                                                  \
   }
 NBLA_HIP_DEFINE_BINARY2(Sub2, NBLA_HIP_BINARY2_SUB)

@@ -45,7 +45,7 @@ EXPORTED = (
     "nbla_hip_memcpy", "nbla_hip_device_synchronize", "nbla_hip_stream_synchronize", "nbla_hip_fill",
     "nbla_hip_cast", "nbla_hip_relu_f32", "nbla_hip_relu_backward_f32", "nbla_hip_add2_f32",
     "nbla_hip_add2_backward_f32", "nbla_hip_binary2_f32", "nbla_hip_binary2_backward_f32", "nbla_hip_copy_rows_f32",
-    "nbla_hip_broadcast2_f32", "nbla_hip_broadcast2_backward_f32", "nbla_hip_mfma_rate_probe", "nbla_hip_binary_convolution_slab_plan",
+    "nbla_hip_broadcast2_f32", "nbla_hip_broadcast2_backward_workspace_bytes", "nbla_hip_broadcast2_backward_f32", "nbla_hip_mfma_rate_probe", "nbla_hip_binary_convolution_slab_plan",
     "nbla_hip_gemm_bits_timer_arm", "nbla_hip_gemm_bits_timer_read",
 )
 
@@ -73,7 +73,7 @@ def lib():
                      "nbla_hip_min_max_quantize_backward_workspace_bytes",
                      "nbla_hip_affine_backward_workspace_bytes",
                      "nbla_hip_convolution_backward_workspace_bytes", "nbla_hip_prune_workspace_bytes",
-                     "nbla_hip_range_recorder_workspace_bytes",
+                     "nbla_hip_range_recorder_workspace_bytes", "nbla_hip_broadcast2_backward_workspace_bytes",
                      "nbla_hip_convolution_workspace_bytes", "nbla_hip_affine_workspace_bytes",
                      "nbla_hip_digit_operand_bytes", "nbla_hip_gemm_bits_workspace_bytes",
                      "nbla_hip_binarize_workspace_bytes",
@@ -262,8 +262,11 @@ def broadcast2_backward(op, i, dy, x0, x1, dx=None, stream=None):
     import torch
     like = x0 if i == 0 else x1
     out, accum = (torch.empty_like(like), 0) if dx is None else (dx, 1)
+    need = lib().nbla_hip_broadcast2_backward_workspace_bytes(int(i), _shape(x0.shape), _shape(x1.shape), x0.dim())
+    ws = _workspace(need, dy) if need else None
     check(lib().nbla_hip_broadcast2_backward_f32(BROADCAST2_OPS[op], i, _p(dy), _p(x0), _shape(x0.shape), _p(x1),
-                                                 _shape(x1.shape), _p(out), x0.dim(), accum, _stream(stream)))
+                                                 _shape(x1.shape), _p(out), x0.dim(), accum, _p(ws),
+                                                 ctypes.c_size_t(need), _stream(stream)))
     return out
 
 
