@@ -148,7 +148,9 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_kn(const float *__restric
 // no relayout pass.  Column sums: lanes in row order, then the block's four wavefronts through LDS in wavefront order.
 constexpr int kWideBatch = 4;
 constexpr int kWideTileBatches = kTileK / kWideBatch; // batches per k tile
-template <int kWideWaveRows, bool kFull, bool kCountZeros>
+// kAligned: N a multiple of four and 16-byte aligned W / Wb, a lane's four columns are one 128-bit access; otherwise
+// four 32-bit ones, each column clamped and masked on its own (a row of W then starts at any multiple of four bytes).
+template <int kWideWaveRows, bool kFull, bool kCountZeros, bool kAligned>
 __device__ __forceinline__ void binarize_wide_walk(const float *__restrict__ W, float *__restrict__ Wb,
                                                    uint4_t *__restrict__ bits_out, int64_t tile_stride, uint32_t *s_x,
                                                    int64_t K, int64_t N, int64_t k_wave, int64_t n0, int lane,
@@ -157,6 +159,13 @@ __device__ __forceinline__ void binarize_wide_walk(const float *__restrict__ W, 
   const bool col_ok = kFull || n0 < N;
   const int64_t n_ld = col_ok ? n0 : N - 4; // loads are unconditional: a clamped address, masked afterwards
   const uint32_t lane_bytes = (uint32_t)(n_ld * 4);
+  uint32_t col_bytes[4];
+  bool col_in[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    col_in[c] = kFull || n0 + c < N;
+    col_bytes[c] = (uint32_t)((col_in[c] ? n0 + c : N - 1) * 4);
+  }
   float4_t va[kWideBatch], vb[kWideBatch];
   uint32_t word[4] = {0u, 0u, 0u, 0u};
   auto load_batch = [&](int b, float4_t (&dst)[kWideBatch]) {
@@ -166,18 +175,26 @@ __device__ __forceinline__ void binarize_wide_walk(const float *__restrict__ W, 
       if (!kFull && k >= K)
         k = K - 1;
       const char *row = reinterpret_cast<const char *>(W + k * N); // uniform base + 32-bit lane offset
-      dst[j] = *reinterpret_cast<const float4_t *>(row + lane_bytes);
+      if (kAligned) {
+        dst[j] = *reinterpret_cast<const float4_t *>(row + lane_bytes);
+      } else {
+        dst[j].x = *reinterpret_cast<const float *>(row + col_bytes[0]);
+        dst[j].y = *reinterpret_cast<const float *>(row + col_bytes[1]);
+        dst[j].z = *reinterpret_cast<const float *>(row + col_bytes[2]);
+        dst[j].w = *reinterpret_cast<const float *>(row + col_bytes[3]);
+      }
     }
   };
   auto consume_batch = [&](int b, const float4_t (&src)[kWideBatch]) {
 #pragma unroll
     for (int j = 0; j < kWideBatch; ++j) {
       const int64_t k = k_wave + b * kWideBatch + j;
-      const bool in = kFull || (col_ok && k < K);
+      const bool row_in = kFull || k < K;
       const float w[4] = {src[j].x, src[j].y, src[j].z, src[j].w};
       float sg[4];
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
+        const bool in = kAligned ? (kFull || (col_ok && row_in)) : (row_in && col_in[c]);
         // sign.hpp:48-50; +-0 and NaN are exactly the inputs that are neither less nor greater than zero
         const bool nonzero = __builtin_islessgreater(w[c], 0.0f);
         const float one = __uint_as_float((__float_as_uint(w[c]) & 0x80000000u) | 0x3f800000u);
@@ -189,11 +206,18 @@ __device__ __forceinline__ void binarize_wide_walk(const float *__restrict__ W, 
         if (kCountZeros)
           nzero += (in && !nonzero) ? 1 : 0;
       }
-      if (in && Wb) {
+      if (Wb && kAligned && (kFull || (col_ok && row_in))) {
         float4_t o;
         o.x = sg[0], o.y = sg[1], o.z = sg[2], o.w = sg[3];
         char *row = reinterpret_cast<char *>(Wb + k * N);
         __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(row + lane_bytes));
+      }
+      if (Wb && !kAligned && row_in) {
+        char *row = reinterpret_cast<char *>(Wb + k * N);
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (col_in[c])
+            __builtin_nontemporal_store(sg[c], reinterpret_cast<float *>(row + col_bytes[c]));
       }
     }
   };
@@ -240,7 +264,7 @@ __device__ __forceinline__ void binarize_wide_walk(const float *__restrict__ W, 
 }
 
 // kWideWaveRows: 64 (two k tiles per wavefront), or 32 for matrices that would otherwise give the CUs too few blocks.
-template <int kWideWaveRows, bool kCountZeros>
+template <int kWideWaveRows, bool kCountZeros, bool kAligned>
 __global__ __launch_bounds__(kPrepBlock, 4) void binarize_kn_wide(const float *__restrict__ W, float *__restrict__ Wb,
                                                                  uint4_t *__restrict__ bits, float *__restrict__ sums,
                                                                  int *__restrict__ zeros, int64_t K, int64_t N,
@@ -260,11 +284,11 @@ __global__ __launch_bounds__(kPrepBlock, 4) void binarize_kn_wide(const float *_
   const int64_t tile_stride = wide_groups * 64;
   const bool full = k_wave + kWideWaveRows <= K && (wg + 1) * kWideGroup <= N;
   if (full)
-    binarize_wide_walk<kWideWaveRows, true, kCountZeros>(W, Wb, tile0, tile_stride, s_x[wave], K, N, k_wave, n0, lane, zero_to, cs,
-                                          nzero);
+    binarize_wide_walk<kWideWaveRows, true, kCountZeros, kAligned>(W, Wb, tile0, tile_stride, s_x[wave], K, N, k_wave, n0,
+                                                                   lane, zero_to, cs, nzero);
   else
-    binarize_wide_walk<kWideWaveRows, false, kCountZeros>(W, Wb, tile0, tile_stride, s_x[wave], K, N, k_wave, n0, lane, zero_to, cs,
-                                           nzero);
+    binarize_wide_walk<kWideWaveRows, false, kCountZeros, kAligned>(W, Wb, tile0, tile_stride, s_x[wave], K, N, k_wave, n0,
+                                                                    lane, zero_to, cs, nzero);
   // column sums of the block's 256 rows, wavefronts in order
   *reinterpret_cast<float4_t *>(&s_sum[wave][4 * lane]) = float4_t{cs[0], cs[1], cs[2], cs[3]};
   if (kCountZeros) {
@@ -1070,8 +1094,10 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint3
   uint32_t *pairs = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + P.sums_bytes + P.zeros_bytes);
   int64_t slices = P.slices;
   if (!transposed) {
-    if (N % 4 == 0 && N >= 4 && aligned16(W) && aligned16(Wb) && P.slabs <= 65535 &&
-        (uint64_t)N * 4 < (1ull << 32)) { // a null Wb (no fp32 signs wanted) counts as aligned
+    if (P.slabs <= 65535 && (uint64_t)N * 4 < (1ull << 32)) {
+      // a lane's four columns as one 128-bit access where the rows allow it (a null Wb -- no fp32 signs wanted --
+      // counts as aligned), else as four 32-bit ones
+      const bool aligned = N % 4 == 0 && N >= 4 && aligned16(W) && aligned16(Wb);
       // writes the packed operand itself (padding k tiles included): nothing is left for the relayout below
       // fewer than four blocks per CU with 256-row slabs: halve the slabs
       const bool fine = P.wide_groups * P.slabs < 1024 && 2 * P.slabs <= 65535;
@@ -1079,8 +1105,14 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint3
       const dim3 grid((unsigned)P.wide_groups, (unsigned)slabs);
       uint4_t *packed = reinterpret_cast<uint4_t *>(bits);
 #define NBLA_BINARIZE_WIDE(ROWS, COUNT)                                                                                \
-  hipLaunchKernelGGL((binarize_kn_wide<ROWS, COUNT>), grid, dim3(kPrepBlock), 0, stream, W, Wb, packed, sums, zeros, K,  \
-                     N, P.wide_groups, P.Npw, quantize_zero_to)
+  do {                                                                                                                 \
+    if (aligned)                                                                                                       \
+      hipLaunchKernelGGL((binarize_kn_wide<ROWS, COUNT, true>), grid, dim3(kPrepBlock), 0, stream, W, Wb, packed, sums,  \
+                         zeros, K, N, P.wide_groups, P.Npw, quantize_zero_to);                                         \
+    else                                                                                                               \
+      hipLaunchKernelGGL((binarize_kn_wide<ROWS, COUNT, false>), grid, dim3(kPrepBlock), 0, stream, W, Wb, packed, sums, \
+                         zeros, K, N, P.wide_groups, P.Npw, quantize_zero_to);                                         \
+  } while (0)
       if (fine && zero_count)
         NBLA_BINARIZE_WIDE(32, true);
       else if (fine)
