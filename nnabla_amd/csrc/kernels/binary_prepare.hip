@@ -717,14 +717,16 @@ __device__ __noinline__ void redo_marked_row(const float *__restrict__ xrow, con
   }
 }
 
-// Scale and digits in one pass for rows of up to 16384 values (K % 4 == 0, 16-byte aligned rows): a block of eight
+// Scale and digits in one pass for rows of up to 16384 values: a block of eight
 // wavefronts keeps kRows rows in registers in fragment order.  Wavefront w owns the k tiles
 // [w * kSlots * kPer, (w + 1) * kSlots * kPer), kSlots = 32 / kRows; lane r + kRows * (g + 2 * ts) holds, for row r,
 // the 16 values of fragment half g of the tiles kSlots * t + ts, t < kPer.  Row maxima and row sums cross the
 // wavefronts through LDS; every store instruction then writes runs of kRows * 16 bytes of a fragment (the other rows
 // of the row block come from neighbouring blocks).  x is read once.
+// kAligned false: rows that do not start at multiples of 16 bytes or whose length is no multiple of four -- a lane's
+// four consecutive values come as four 32-bit loads, each checked against the row's end.
 constexpr int kFusedWaves = 8;
-template <int kRows, int kPer>
+template <int kRows, int kPer, bool kAligned>
 __global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const float *__restrict__ x, int64_t ldx,
                                                                        const float *__restrict__ cs,
                                                                        long long *__restrict__ sums,
@@ -751,8 +753,20 @@ __global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const floa
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int64_t k = k0 + 4 * i;
-      v[t][i] = (m < M && k < K) ? scaled4(*reinterpret_cast<const float4_t *>(row + k), cs, k)
-                                 : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+      if (kAligned) {
+        v[t][i] = (m < M && k < K) ? scaled4(*reinterpret_cast<const float4_t *>(row + k), cs, k)
+                                   : float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+      } else {
+        float e[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const bool in = m < M && k + c < K;
+          e[c] = in ? row[k + c] : 0.0f;
+          if (cs) // one rounded product per element, as scaled4
+            e[c] = e[c] * (in ? cs[k + c] : 0.0f);
+        }
+        v[t][i] = float4_t{e[0], e[1], e[2], e[3]};
+      }
     }
   }
 #pragma unroll
@@ -834,9 +848,13 @@ __global__ __launch_bounds__(kFusedWaves * 64) void split_digits_rows(const floa
 template <int kRows, int kPer>
 void launch_split_digits_rows(const float *x, int64_t ldx, const float *cs, long long *sums, int32_t *shift,
                               uint4_t *out, int64_t M, int64_t K, const DigitOperand &d, const RowRedo &redo,
-                              hipStream_t stream) {
-  hipLaunchKernelGGL((split_digits_rows<kRows, kPer>), dim3((unsigned)(d.rows / kRows)), dim3(kFusedWaves * 64), 0,
-                     stream, x, ldx, cs, sums, shift, out, M, K, d.k_tiles, d.rows, redo);
+                              bool aligned, hipStream_t stream) {
+  if (aligned)
+    hipLaunchKernelGGL((split_digits_rows<kRows, kPer, true>), dim3((unsigned)(d.rows / kRows)), dim3(kFusedWaves * 64),
+                       0, stream, x, ldx, cs, sums, shift, out, M, K, d.k_tiles, d.rows, redo);
+  else
+    hipLaunchKernelGGL((split_digits_rows<kRows, kPer, false>), dim3((unsigned)(d.rows / kRows)),
+                       dim3(kFusedWaves * 64), 0, stream, x, ldx, cs, sums, shift, out, M, K, d.k_tiles, d.rows, redo);
 }
 
 // ---- digit operand of a transposed source: the operand's rows are the columns c of src [R, C] (row stride ld) and
@@ -1191,7 +1209,7 @@ int launch_split_digits_rows_redo(const float *x, int64_t ldx, const float *cols
   long long *sums = reinterpret_cast<long long *>(base + d.sum_off);
   int32_t *shift = reinterpret_cast<int32_t *>(base + d.shift_off);
   const bool vec = K % 4 == 0 && ldx % 4 == 0 && aligned16(x) && aligned16(cs);
-  if (vec && d.k_tiles <= 512) { // rows of up to 16384 values: one pass, rows held in registers
+  if (d.k_tiles <= 512) { // rows of up to 16384 values: one pass, rows held in registers
     uint4_t *out = static_cast<uint4_t *>(xdigits);
     // A block covers 8 wavefronts x (32 / rows) x (tiles per lane) k tiles.  Most rows per block (longest store runs)
     // among the shapes that hold the row and still give every CU a block; the fewest rows otherwise.
@@ -1207,7 +1225,7 @@ int launch_split_digits_rows_redo(const float *x, int64_t ldx, const float *cols
     }
     const int64_t per = ceil_div(kt, kFusedWaves * (32 / rows_per_block));
 #define NBLA_SPLIT_ROWS(R, P)                                                                                          \
-  launch_split_digits_rows<R, P>(x, ldx, cs, sums, shift, out, M, K, d, redo, stream)
+  launch_split_digits_rows<R, P>(x, ldx, cs, sums, shift, out, M, K, d, redo, vec, stream)
     if (rows_per_block == 16) {
       if (per <= 1)
         NBLA_SPLIT_ROWS(16, 1);
