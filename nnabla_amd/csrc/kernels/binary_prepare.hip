@@ -370,6 +370,7 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_nk(const float *__restric
 // the eight partial words (f, jq) of each packed word of k tile w.  |W| row sums: the four k of a thread in order,
 // then a butterfly over the 32 lanes of the row.
 constexpr int kPartStride = 36; // words per LDS row: 32 k quads + padding that keeps 16-byte alignment
+template <bool kAligned> // false: rows of a length that is no multiple of four (or not 16-byte aligned), 32-bit accesses
 __global__ __launch_bounds__(kPrepBlock) void binarize_nk_vec(const float *__restrict__ W, float *__restrict__ Wb,
                                                               uint32_t *__restrict__ bits, float *__restrict__ sums,
                                                               int *__restrict__ zeros, int64_t K, int64_t N,
@@ -385,23 +386,32 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_nk_vec(const float *__res
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int64_t n = cg * kColGroup + i * 8 + rsub;
-    if (n < N && k < K)
-      v[i] = *reinterpret_cast<const float4_t *>(W + n * K + k);
-    else
-      v[i] = float4_t{1.0f, 1.0f, 1.0f, 1.0f};
+    if (kAligned) {
+      if (n < N && k < K)
+        v[i] = *reinterpret_cast<const float4_t *>(W + n * K + k);
+      else
+        v[i] = float4_t{1.0f, 1.0f, 1.0f, 1.0f};
+    } else {
+      const float *src = W + n * K + k;
+      v[i].x = (n < N && k + 0 < K) ? src[0] : 1.0f;
+      v[i].y = (n < N && k + 1 < K) ? src[1] : 1.0f;
+      v[i].z = (n < N && k + 2 < K) ? src[2] : 1.0f;
+      v[i].w = (n < N && k + 3 < K) ? src[3] : 1.0f;
+    }
   }
   int nzero = 0;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int row = i * 8 + rsub;
     const int64_t n = cg * kColGroup + row;
-    const bool in = n < N && k < K;
+    const bool row_in = n < N && k < K;
     const float w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
     float b[4];
     uint32_t part = 0u;
     float asum = 0.0f;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
+      const bool in = kAligned ? row_in : (n < N && k + c < K);
       b[c] = sign_of(w[c], zero_to);
       const bool is_zero = !(w[c] > 0.0f) && !(w[c] < 0.0f);
       const bool neg = (w[c] < 0.0f) || (is_zero && zero_to < 0.0f);
@@ -410,10 +420,16 @@ __global__ __launch_bounds__(kPrepBlock) void binarize_nk_vec(const float *__res
       nzero += (in && is_zero) ? 1 : 0;
     }
     s_part[row * kPartStride + kq] = part;
-    if (in && Wb) {
+    if (kAligned && row_in && Wb) {
       float4_t o;
       o.x = b[0], o.y = b[1], o.z = b[2], o.w = b[3];
       __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(Wb + n * K + k));
+    }
+    if (!kAligned && Wb) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (n < N && k + c < K)
+          __builtin_nontemporal_store(b[c], Wb + n * K + k + c);
     }
 #pragma unroll
     for (int off = 16; off >= 1; off >>= 1)
@@ -1155,9 +1171,12 @@ int nbla_hip_binarize_weights_f32(const float *W, float *Wb, float *alpha, uint3
                          P.col_groups, P.Np, quantize_zero_to);
     }
   } else {
-    if (K % 4 == 0 && aligned16(W) && aligned16(Wb) && P.col_groups <= 65535) {
-      hipLaunchKernelGGL(binarize_nk_vec, dim3((unsigned)P.slices, (unsigned)P.col_groups), dim3(kPrepBlock), 0, stream,
-                         W, Wb, pairs, sums, zeros, K, N, P.col_groups, P.Np, P.k_tiles, quantize_zero_to);
+    if (P.col_groups <= 65535 && K % 4 == 0 && aligned16(W) && aligned16(Wb)) {
+      hipLaunchKernelGGL(binarize_nk_vec<true>, dim3((unsigned)P.slices, (unsigned)P.col_groups), dim3(kPrepBlock), 0,
+                         stream, W, Wb, pairs, sums, zeros, K, N, P.col_groups, P.Np, P.k_tiles, quantize_zero_to);
+    } else if (P.col_groups <= 65535) {
+      hipLaunchKernelGGL(binarize_nk_vec<false>, dim3((unsigned)P.slices, (unsigned)P.col_groups), dim3(kPrepBlock), 0,
+                         stream, W, Wb, pairs, sums, zeros, K, N, P.col_groups, P.Np, P.k_tiles, quantize_zero_to);
     } else {
       const dim3 grid((unsigned)P.col_groups, (unsigned)P.slices);
       hipLaunchKernelGGL(binarize_nk, grid, dim3(kPrepBlock), 0, stream, W, Wb, pairs, sums, zeros, K, N, P.col_groups,
