@@ -781,6 +781,12 @@ int binary_conv_forward(const float *x, const float *W, float *Wb, float *alpha,
   if (rc)
     return rc;
   hipStream_t stream = as_stream(stream_);
+  if (conv_direct_applies(g)) { // many small groups: all of them in one launch each, over the materialised signs
+    rc = launch_conv_direct_binarize(W, Wb, alpha, g, zero_to, stream);
+    if (rc)
+      return rc;
+    return launch_conv_direct_forward(x, Wb, alpha, bias, y, g, stream);
+  }
   char *base = static_cast<char *>(workspace);
   int *counts = reinterpret_cast<int *>(base + ws.count_off);
   const bool slab = conv_slab_applies(g);

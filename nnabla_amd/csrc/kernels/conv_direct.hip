@@ -1,0 +1,239 @@
+// Grouped convolutions with small groups (depthwise, ResNeXt-style): every group's product is far too small for the
+// matrix cores, and the general path pays several launches per group (256 groups of a depthwise layer: milliseconds
+// of launches around microseconds of work).  These kernels compute all groups in one launch each, in plain fp32 with
+// one thread per output element and the contraction in the reference's order k = (channel, tap)
+// (convolution.cpp:161-197 forward, :199-330 backward: per sample and group an unfold and a product -- here without
+// the unfolded matrix).  The same kernels serve the binary convolutions: the weights are then the materialised signs,
+// multiplied by alpha[o] as binary_weight_convolution.cpp:100-110 forms Ws.
+#include "common.hpp"
+#include "conv_geom.hpp"
+#include "gemm_layout.hpp"
+#include "internal.hpp"
+
+namespace nbla_hip {
+namespace {
+
+constexpr int kDirectBlock = 256;
+
+struct Position {
+  int o0, o1, o2;
+};
+__device__ __forceinline__ Position out_position(const ConvGeom &g, int64_t p) {
+  Position q;
+  q.o2 = (int)(p % g.out_sp[2]);
+  p /= g.out_sp[2];
+  q.o1 = (int)(p % g.out_sp[1]);
+  q.o0 = (int)(p / g.out_sp[1]);
+  return q;
+}
+
+// y[n, o, p] = sum_k x[n, c(k), window(p, tap(k))] * w[o, k] (* scale[o]) (+ bias[o]); zeros where the window leaves
+// the input (they are multiplied like any other value: 0 * Inf = NaN as in the reference's product).
+__global__ __launch_bounds__(kDirectBlock) void conv_direct_forward(const float *__restrict__ x,
+                                                                    const float *__restrict__ w,
+                                                                    const float *__restrict__ scale,
+                                                                    const float *__restrict__ bias,
+                                                                    float *__restrict__ y, ConvGeom g) {
+  const int64_t total = g.outer * g.O * g.out_sp_size;
+  for (int64_t i = (int64_t)blockIdx.x * kDirectBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kDirectBlock) {
+    const int64_t p = i % g.out_sp_size, no = i / g.out_sp_size;
+    const int64_t o = no % g.O, n = no / g.O, grp = o / g.Og;
+    const Position q = out_position(g, p);
+    const int b0 = q.o0 * g.stride[0] - g.pad[0], b1 = q.o1 * g.stride[1] - g.pad[1], b2 = q.o2 * g.stride[2] - g.pad[2];
+    const float *xn = x + (n * g.C + grp * g.Cg) * g.in_sp_size;
+    const float *wo = w + o * g.Kg;
+    const float a = scale ? scale[o] : 1.0f;
+    float acc = 0.0f;
+    for (int64_t c = 0; c < g.Cg; ++c) {
+      const float *xc = xn + c * g.in_sp_size;
+      const float *wc = wo + c * g.k_size;
+      int t = 0;
+      for (int k0 = 0; k0 < g.k[0]; ++k0)
+        for (int k1 = 0; k1 < g.k[1]; ++k1)
+          for (int k2 = 0; k2 < g.k[2]; ++k2, ++t) {
+            const int i0 = b0 + k0 * g.dil[0], i1 = b1 + k1 * g.dil[1], i2 = b2 + k2 * g.dil[2];
+            const bool in = (unsigned)i0 < (unsigned)g.in_sp[0] && (unsigned)i1 < (unsigned)g.in_sp[1] &&
+                            (unsigned)i2 < (unsigned)g.in_sp[2];
+            const float xv = in ? xc[((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2] + i2] : 0.0f;
+            const float wv = scale ? wc[t] * a : wc[t];
+            acc = acc + xv * wv;
+          }
+    }
+    y[i] = bias ? acc + bias[o] : acc;
+  }
+}
+
+// dx[n, c, q] (+)= sum over the group's o and the taps whose window position p lies in the output:
+// (dy[n, o, p] * scale[o]) * w[o, c, tap]   (the unfolded gradient folded back, convolution.cpp:262-283)
+// take_sign: w holds the real-valued weights of a binary convolution, whose signs (sign.hpp:48-50) are what the
+// forward pass multiplied with.
+__global__ __launch_bounds__(kDirectBlock) void conv_direct_dx(const float *__restrict__ dy, const float *__restrict__ w,
+                                                               const float *__restrict__ scale, float *__restrict__ dx,
+                                                               ConvGeom g, int accum, int take_sign, float zero_to) {
+  const int64_t total = g.outer * g.C * g.in_sp_size;
+  for (int64_t i = (int64_t)blockIdx.x * kDirectBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kDirectBlock) {
+    int64_t pos = i % g.in_sp_size;
+    const int64_t nc = i / g.in_sp_size, c = nc % g.C, n = nc / g.C, grp = c / g.Cg, cl = c - grp * g.Cg;
+    const int q2 = (int)(pos % g.in_sp[2]);
+    pos /= g.in_sp[2];
+    const int q1 = (int)(pos % g.in_sp[1]), q0 = (int)(pos / g.in_sp[1]);
+    const float *dyn = dy + (n * g.O + grp * g.Og) * g.out_sp_size;
+    const float *wg = w + (grp * g.Og) * g.Kg + cl * g.k_size;
+    float acc = 0.0f;
+    int t = 0;
+    for (int k0 = 0; k0 < g.k[0]; ++k0)
+      for (int k1 = 0; k1 < g.k[1]; ++k1)
+        for (int k2 = 0; k2 < g.k[2]; ++k2, ++t) {
+          const int e0 = q0 + g.pad[0] - k0 * g.dil[0], e1 = q1 + g.pad[1] - k1 * g.dil[1],
+                    e2 = q2 + g.pad[2] - k2 * g.dil[2];
+          if (e0 < 0 || e1 < 0 || e2 < 0 || e0 % g.stride[0] || e1 % g.stride[1] || e2 % g.stride[2])
+            continue;
+          const int p0 = e0 / g.stride[0], p1 = e1 / g.stride[1], p2 = e2 / g.stride[2];
+          if (p0 >= g.out_sp[0] || p1 >= g.out_sp[1] || p2 >= g.out_sp[2])
+            continue;
+          const int64_t p = ((int64_t)p0 * g.out_sp[1] + p1) * g.out_sp[2] + p2;
+          for (int64_t o = 0; o < g.Og; ++o) {
+            const float gy = dyn[o * g.out_sp_size + p];
+            const float gs = scale ? gy * scale[grp * g.Og + o] : gy;
+            float wv = wg[o * g.Kg + t];
+            if (take_sign)
+              wv = (wv > 0.0f) ? 1.0f : ((wv < 0.0f) ? -1.0f : zero_to);
+            acc = acc + gs * wv;
+          }
+        }
+    dx[i] = accum ? dx[i] + acc : acc;
+  }
+}
+
+// dW[o, k] (+)= sum over samples and output positions of dy[n, o, p] * x[n, c(k), window(p, tap(k))]; one block per
+// weight, 256 interleaved partial sums folded in a fixed order.
+__global__ __launch_bounds__(kDirectBlock) void conv_direct_dw(const float *__restrict__ dy, const float *__restrict__ x,
+                                                               float *__restrict__ dW, ConvGeom g, int accum) {
+  __shared__ float part[kDirectBlock];
+  const int64_t ok = blockIdx.x, o = ok / g.Kg, k = ok - o * g.Kg, grp = o / g.Og;
+  const int64_t c = k / g.k_size;
+  int t = (int)(k - c * g.k_size);
+  const int k2 = t % g.k[2];
+  t /= g.k[2];
+  const int k1 = t % g.k[1], k0 = t / g.k[1];
+  float acc = 0.0f;
+  const int64_t M = g.outer * g.out_sp_size;
+  for (int64_t m = threadIdx.x; m < M; m += kDirectBlock) {
+    const int64_t n = m / g.out_sp_size, p = m - n * g.out_sp_size;
+    const Position q = out_position(g, p);
+    const int i0 = q.o0 * g.stride[0] - g.pad[0] + k0 * g.dil[0], i1 = q.o1 * g.stride[1] - g.pad[1] + k1 * g.dil[1],
+              i2 = q.o2 * g.stride[2] - g.pad[2] + k2 * g.dil[2];
+    const bool in = (unsigned)i0 < (unsigned)g.in_sp[0] && (unsigned)i1 < (unsigned)g.in_sp[1] &&
+                    (unsigned)i2 < (unsigned)g.in_sp[2];
+    const float xv =
+        in ? x[(n * g.C + grp * g.Cg + c) * g.in_sp_size + ((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2] + i2] : 0.0f;
+    acc = acc + dy[(n * g.O + o) * g.out_sp_size + p] * xv;
+  }
+  part[threadIdx.x] = acc;
+  __syncthreads();
+  for (int s = kDirectBlock / 2; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s)
+      part[threadIdx.x] += part[threadIdx.x + s];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0)
+    dW[ok] = accum ? dW[ok] + part[0] : part[0];
+}
+
+// db[o] (+)= sum over samples and positions of dy[n, o, p]
+__global__ __launch_bounds__(kDirectBlock) void conv_direct_db(const float *__restrict__ dy, float *__restrict__ db,
+                                                               ConvGeom g, int accum) {
+  __shared__ float part[kDirectBlock];
+  const int64_t o = blockIdx.x, M = g.outer * g.out_sp_size;
+  float acc = 0.0f;
+  for (int64_t m = threadIdx.x; m < M; m += kDirectBlock) {
+    const int64_t n = m / g.out_sp_size, p = m - n * g.out_sp_size;
+    acc = acc + dy[(n * g.O + o) * g.out_sp_size + p];
+  }
+  part[threadIdx.x] = acc;
+  __syncthreads();
+  for (int s = kDirectBlock / 2; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s)
+      part[threadIdx.x] += part[threadIdx.x + s];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0)
+    db[o] = accum ? db[o] + part[0] : part[0];
+}
+
+// Wb = Sign(W) (sign.hpp:48-50) and alpha[o] = (sum of |W[o, :]|) * ((float)1 / Kg)
+// (binary_weight_convolution.cpp:66,85-98) for all output channels of all groups: a wavefront per channel, lanes
+// along the row, the lanes' sums folded in a fixed order.
+__global__ __launch_bounds__(kDirectBlock) void binarize_channels(const float *__restrict__ W, float *__restrict__ Wb,
+                                                                  float *__restrict__ alpha, int64_t O, int64_t Kg,
+                                                                  float zero_to, float inv_k) {
+  const int lane = threadIdx.x & 63;
+  const int64_t o = (int64_t)blockIdx.x * (kDirectBlock / 64) + (threadIdx.x >> 6);
+  if (o >= O)
+    return;
+  float acc = 0.0f;
+  for (int64_t k = lane; k < Kg; k += 64) {
+    const float v = W[o * Kg + k];
+    Wb[o * Kg + k] = (v > 0.0f) ? 1.0f : ((v < 0.0f) ? -1.0f : zero_to);
+    acc += fabsf(v);
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1)
+    acc += __shfl_xor(acc, off);
+  if (alpha && lane == 0)
+    alpha[o] = acc * inv_k;
+}
+
+unsigned blocks_for(int64_t n) {
+  int64_t b = (n + kDirectBlock - 1) / kDirectBlock;
+  return (unsigned)(b > 262144 ? 262144 : (b < 1 ? 1 : b));
+}
+
+} // namespace
+
+// Groups too small to pay for the general path's launches: its cost is about 25 us of launches per group forward (85
+// backward) plus the product at matrix-core rates; this path's, the product at about 10 TFLOP/s of vector fp32.
+bool conv_direct_applies(const ConvGeom &g) {
+  if (g.group < 2 || g.O * g.Kg > 0x7fffffffll)
+    return false;
+  const double flops = 2.0 * (double)g.M * (double)g.Kg * (double)g.O;
+  return flops / 1e7 < 25.0 * (double)g.group + flops / 1e8;
+}
+
+int launch_conv_direct_binarize(const float *W, float *Wb, float *alpha, const ConvGeom &g, float zero_to,
+                                hipStream_t stream) {
+  hipLaunchKernelGGL(binarize_channels, dim3((unsigned)ceil_div(g.O, kDirectBlock / 64)), dim3(kDirectBlock), 0, stream,
+                     W, Wb, alpha, g.O, g.Kg, zero_to, (float)1 / g.Kg);
+  NBLA_HIP_LAUNCH_CHECK("binarize_channels");
+  return NBLA_HIP_OK;
+}
+
+int launch_conv_direct_forward(const float *x, const float *w, const float *scale, const float *bias, float *y,
+                               const ConvGeom &g, hipStream_t stream) {
+  hipLaunchKernelGGL(conv_direct_forward, dim3(blocks_for(g.outer * g.O * g.out_sp_size)), dim3(kDirectBlock), 0, stream,
+                     x, w, scale, bias, y, g);
+  NBLA_HIP_LAUNCH_CHECK("conv_direct_forward");
+  return NBLA_HIP_OK;
+}
+
+int launch_conv_direct_backward(const float *dy, const float *x, const float *w, const float *scale, float *dx,
+                                float *dW, float *db, const ConvGeom &g, bool accum_x, bool accum_w, bool accum_b,
+                                bool take_sign, float zero_to, hipStream_t stream) {
+  if (dx) {
+    hipLaunchKernelGGL(conv_direct_dx, dim3(blocks_for(g.outer * g.C * g.in_sp_size)), dim3(kDirectBlock), 0, stream, dy,
+                       w, scale, dx, g, accum_x ? 1 : 0, take_sign ? 1 : 0, zero_to);
+    NBLA_HIP_LAUNCH_CHECK("conv_direct_dx");
+  }
+  if (dW) {
+    hipLaunchKernelGGL(conv_direct_dw, dim3((unsigned)(g.O * g.Kg)), dim3(kDirectBlock), 0, stream, dy, x, dW, g,
+                       accum_w ? 1 : 0);
+    NBLA_HIP_LAUNCH_CHECK("conv_direct_dw");
+  }
+  if (db) {
+    hipLaunchKernelGGL(conv_direct_db, dim3((unsigned)g.O), dim3(kDirectBlock), 0, stream, dy, db, g, accum_b ? 1 : 0);
+    NBLA_HIP_LAUNCH_CHECK("conv_direct_db");
+  }
+  return NBLA_HIP_OK;
+}
+
+} // namespace nbla_hip

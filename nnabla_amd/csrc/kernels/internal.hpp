@@ -36,6 +36,18 @@ struct ConvGeom;
 bool gemm_bits_unfold_applies(const ConvGeom &g);
 int launch_gemm_bits_unfold(const float *x, const ConvGeom &g, int64_t grp, const uint32_t *bits, const float *alpha,
                             const float *bias, float *y, hipStream_t stream, int32_t *row_shift = nullptr);
+// Grouped convolutions whose groups are too small for the matrix cores (depthwise, ResNeXt-style), all groups in one
+// launch, plain fp32 (conv_direct.hip).  w: the weights [O, Kg] (for a binary convolution the materialised signs),
+// scale (may be null): alpha[o].  launch_conv_direct_binarize writes Wb = Sign(W) and alpha (may be null) for all
+// channels.  Backward: w as in the forward, or with take_sign the real-valued weights whose signs were used.
+bool conv_direct_applies(const ConvGeom &g);
+int launch_conv_direct_binarize(const float *W, float *Wb, float *alpha, const ConvGeom &g, float zero_to,
+                                hipStream_t stream);
+int launch_conv_direct_forward(const float *x, const float *w, const float *scale, const float *bias, float *y,
+                               const ConvGeom &g, hipStream_t stream);
+int launch_conv_direct_backward(const float *dy, const float *x, const float *w, const float *scale, float *dx,
+                                float *dW, float *db, const ConvGeom &g, bool accum_x, bool accum_w, bool accum_b,
+                                bool take_sign, float zero_to, hipStream_t stream);
 // The binary convolution forward with the unfold done by LDS addressing (conv_slab.hip), two launches per group:
 // launch_conv_slab_prepare reads the group's weights [Og, Cg, taps] once and writes Wb = Sign(W) (may be null) and,
 // into `prepared` (conv_slab_prepared_bytes, 16-byte aligned), the packed bits in (tap, channel) order with the
