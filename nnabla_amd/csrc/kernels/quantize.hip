@@ -1273,7 +1273,9 @@ __device__ unsigned g_recorder_tickets[kRecorderTickets][(kTicketGroups + 1) * k
 // the block that draws the last one reads all the partial results back with atomic loads (they are complete: every
 // other block's stores were acknowledged before its ticket), merges them in block order and applies the update.
 // Only atomics carry the hand-over, so no cache is written back or invalidated.
-template <bool kAbs, bool kCopy>
+// kAligned false: x (or y) does not start at a multiple of 16 bytes; a lane's four values then come and go as four
+// 32-bit accesses.
+template <bool kAbs, bool kCopy, bool kAligned>
 __global__ __launch_bounds__(kRedBlock) void record_scan(const float *__restrict__ x, float *__restrict__ y,
                                                          MinMaxPartial *__restrict__ partial, size_t n4, size_t size,
                                                          float *__restrict__ m, float *__restrict__ M, int mode,
@@ -1283,6 +1285,17 @@ __global__ __launch_bounds__(kRedBlock) void record_scan(const float *__restrict
   const size_t per = (n4 + gridDim.x - 1) / gridDim.x;
   const size_t begin = (size_t)blockIdx.x * per, end = (begin + per < n4) ? begin + per : n4;
   size_t i = begin + threadIdx.x;
+  auto ld = [](const float *p) {
+    return kAligned ? load4(p) : float4_t{p[0], p[1], p[2], p[3]};
+  };
+  auto st = [](float *p, float4_t v) {
+    if (kAligned) {
+      store4(p, v);
+    } else {
+      __builtin_nontemporal_store(v.x, p), __builtin_nontemporal_store(v.y, p + 1);
+      __builtin_nontemporal_store(v.z, p + 2), __builtin_nontemporal_store(v.w, p + 3);
+    }
+  };
   auto absolute = [](float4_t v) {
     return float4_t{__builtin_fabsf(v.x), __builtin_fabsf(v.y), __builtin_fabsf(v.z), __builtin_fabsf(v.w)};
   };
@@ -1291,7 +1304,7 @@ __global__ __launch_bounds__(kRedBlock) void record_scan(const float *__restrict
     float4_t cur[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      cur[j] = load4(x + 4 * (i + j * kRedBlock));
+      cur[j] = ld(x + 4 * (i + j * kRedBlock));
 #pragma clang loop unroll(disable)
     for (;;) {
       const size_t nx = i + 4 * kRedBlock;
@@ -1300,12 +1313,12 @@ __global__ __launch_bounds__(kRedBlock) void record_scan(const float *__restrict
       if (more) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          nxt[j] = load4(x + 4 * (nx + j * kRedBlock));
+          nxt[j] = ld(x + 4 * (nx + j * kRedBlock));
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         if (kCopy)
-          store4(y + 4 * (i + j * kRedBlock), cur[j]);
+          st(y + 4 * (i + j * kRedBlock), cur[j]);
         ex.take4(kAbs ? absolute(cur[j]) : cur[j], (uint32_t)(4 * (i + j * kRedBlock)));
       }
       i = nx;
@@ -1317,9 +1330,9 @@ __global__ __launch_bounds__(kRedBlock) void record_scan(const float *__restrict
     }
   }
   for (; i < end; i += kRedBlock) {
-    float4_t v = load4(x + 4 * i);
+    float4_t v = ld(x + 4 * i);
     if (kCopy)
-      store4(y + 4 * i, v);
+      st(y + 4 * i, v);
     ex.take4(kAbs ? absolute(v) : v, (uint32_t)(4 * i));
   }
   if (blockIdx.x == gridDim.x - 1) { // the elements past the last float4 (all of them when n4 is 0), highest indices
@@ -1424,7 +1437,8 @@ int nbla_hip_range_recorder_f32(const float *x, float *y, size_t size, float *m,
     return rc;
   MinMaxPartial *partial = static_cast<MinMaxPartial *>(workspace);
   const bool copy = (y != x);
-  const size_t n4 = (aligned16(x) && (!copy || aligned16(y))) ? size / 4 : 0;
+  const bool aligned = aligned16(x) && (!copy || aligned16(y));
+  const size_t n4 = size / 4;
   size_t blocks = (n4 + kRedBlock * 4 - 1) / (kRedBlock * 4);
   if (blocks > (size_t)kMaxChunks)
     blocks = kMaxChunks;
@@ -1436,21 +1450,27 @@ int nbla_hip_range_recorder_f32(const float *x, float *y, size_t size, float *m,
   const float dec = (float)decay, omd = (float)(1.0 - decay);
   static std::atomic<unsigned> next_slot{0};
   const int slot = (int)(next_slot.fetch_add(1u) % (unsigned)kRecorderTickets);
+#define NBLA_RECORD_SCAN(ABS, COPY)                                                                                    \
+  do {                                                                                                                 \
+    if (aligned)                                                                                                       \
+      hipLaunchKernelGGL((record_scan<ABS, COPY, true>), grid, block, 0, stream, x, y, partial, n4, size, m, M, mode,  \
+                         dec, omd, slot);                                                                              \
+    else                                                                                                               \
+      hipLaunchKernelGGL((record_scan<ABS, COPY, false>), grid, block, 0, stream, x, y, partial, n4, size, m, M, mode, \
+                         dec, omd, slot);                                                                              \
+  } while (0)
   if (mode == kAbsMax) {
     if (copy)
-      hipLaunchKernelGGL((record_scan<true, true>), grid, block, 0, stream, x, y, partial, n4, size, m, M, mode, dec,
-                         omd, slot);
+      NBLA_RECORD_SCAN(true, true);
     else
-      hipLaunchKernelGGL((record_scan<true, false>), grid, block, 0, stream, x, y, partial, n4, size, m, M, mode, dec,
-                         omd, slot);
+      NBLA_RECORD_SCAN(true, false);
   } else {
     if (copy)
-      hipLaunchKernelGGL((record_scan<false, true>), grid, block, 0, stream, x, y, partial, n4, size, m, M, mode, dec,
-                         omd, slot);
+      NBLA_RECORD_SCAN(false, true);
     else
-      hipLaunchKernelGGL((record_scan<false, false>), grid, block, 0, stream, x, y, partial, n4, size, m, M, mode, dec,
-                         omd, slot);
+      NBLA_RECORD_SCAN(false, false);
   }
+#undef NBLA_RECORD_SCAN
   NBLA_HIP_LAUNCH_CHECK("range recorder scan");
   return NBLA_HIP_OK;
 }

@@ -393,15 +393,24 @@ struct PruneState {
   uint32_t cand[kSelectBlocks][kCandPerBlock];
 };
 
+// kAligned false: x (or y) does not start at a multiple of 16 bytes; four 32-bit accesses per lane instead of one
+// 128-bit access.
+template <bool kAligned>
 __device__ __forceinline__ void prune_fetch(const float *__restrict__ x, int64_t n4, int64_t tile,
                                             float4_t (&v)[kPruneLoads]) {
   const int64_t base = tile * (kHistBlock * kPruneLoads) + threadIdx.x;
 #pragma unroll
   for (int j = 0; j < kPruneLoads; ++j)
-    if (base + j * kHistBlock < n4)
-      v[j] = *reinterpret_cast<const float4_t *>(x + 4 * (base + j * kHistBlock));
+    if (base + j * kHistBlock < n4) {
+      const float *src = x + 4 * (base + j * kHistBlock);
+      if (kAligned)
+        v[j] = *reinterpret_cast<const float4_t *>(src);
+      else
+        v[j] = float4_t{src[0], src[1], src[2], src[3]};
+    }
 }
 
+template <bool kAligned>
 __global__ __launch_bounds__(kHistBlock) void prune_histogram(const float *__restrict__ x, int64_t n4, int64_t n,
                                                           PruneState *__restrict__ ps, int pass) {
   __shared__ uint32_t h[kMaxBins * kLdsCopies];
@@ -413,7 +422,7 @@ __global__ __launch_bounds__(kHistBlock) void prune_histogram(const float *__res
   const bool any = (int64_t)blockIdx.x < tiles && !from_cand;
   float4_t cur[kPruneLoads];
   if (any)
-    prune_fetch(x, n4, blockIdx.x, cur);
+    prune_fetch<kAligned>(x, n4, blockIdx.x, cur);
   if (threadIdx.x == 0) {
     s_kept = 0u;
     if (pass == 0 && blockIdx.x == 0)
@@ -489,7 +498,7 @@ __global__ __launch_bounds__(kHistBlock) void prune_histogram(const float *__res
       const int64_t next = tile + gridDim.x;
       float4_t nxt[kPruneLoads];
       if (next < tiles)
-        prune_fetch(x, n4, next, nxt);
+        prune_fetch<kAligned>(x, n4, next, nxt);
       const int64_t base = tile * (kHistBlock * kPruneLoads) + threadIdx.x;
       if (pass == 1) {
         count_and_keep(cur, base);
@@ -519,6 +528,7 @@ __global__ __launch_bounds__(kHistBlock) void prune_histogram(const float *__res
 }
 
 // y = (|x| < thresh) ? 0 : x with thresh = |rank-th smallest| (+ 1 when rate == 1), prune.cpp:62-69
+template <bool kAligned>
 __global__ __launch_bounds__(kHistBlock) void prune_apply(const float *__restrict__ x, float *__restrict__ y,
                                                           int64_t n4, int64_t n, PruneState *__restrict__ ps,
                                                           float add) {
@@ -528,7 +538,7 @@ __global__ __launch_bounds__(kHistBlock) void prune_apply(const float *__restric
   const bool any = (int64_t)blockIdx.x < tiles;
   float4_t cur[kPruneLoads];
   if (any)
-    prune_fetch(x, n4, blockIdx.x, cur);
+    prune_fetch<kAligned>(x, n4, blockIdx.x, cur);
   const float thresh = __uint_as_float(select_resolve(scratch, st, kPasses).prefix) + add;
   if (any) {
 #pragma clang loop unroll(disable)
@@ -536,7 +546,7 @@ __global__ __launch_bounds__(kHistBlock) void prune_apply(const float *__restric
       const int64_t next = tile + gridDim.x;
       float4_t nxt[kPruneLoads];
       if (next < tiles)
-        prune_fetch(x, n4, next, nxt);
+        prune_fetch<kAligned>(x, n4, next, nxt);
       const int64_t base = tile * (kHistBlock * kPruneLoads) + threadIdx.x;
 #pragma unroll
       for (int j = 0; j < kPruneLoads; ++j)
@@ -546,7 +556,13 @@ __global__ __launch_bounds__(kHistBlock) void prune_apply(const float *__restric
           o.y = fabsf(cur[j].y) < thresh ? 0.0f : cur[j].y;
           o.z = fabsf(cur[j].z) < thresh ? 0.0f : cur[j].z;
           o.w = fabsf(cur[j].w) < thresh ? 0.0f : cur[j].w;
-          __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(y + 4 * (base + j * kHistBlock)));
+          float *dst = y + 4 * (base + j * kHistBlock);
+          if (kAligned) {
+            __builtin_nontemporal_store(o, reinterpret_cast<float4_t *>(dst));
+          } else {
+            __builtin_nontemporal_store(o.x, dst), __builtin_nontemporal_store(o.y, dst + 1);
+            __builtin_nontemporal_store(o.z, dst + 2), __builtin_nontemporal_store(o.w, dst + 3);
+          }
         }
 #pragma unroll
       for (int j = 0; j < kPruneLoads; ++j)
@@ -651,8 +667,6 @@ int nbla_hip_prune_f32(const float *x, float *y, size_t size, float rate, void *
     return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "Prune: more than 2^31 - 1 elements (the reference indexes with int).");
   if (workspace_bytes < sizeof(PruneState) || !aligned256(workspace))
     return fail(NBLA_HIP_ERR_MEMORY, "Prune workspace too small or misaligned.");
-  if (!aligned16(x) || !aligned16(y))
-    return fail(NBLA_HIP_ERR_MEMORY, "Prune: x and y must be 16-byte aligned.");
   int rc = ensure_init();
   if (rc)
     return rc;
@@ -669,16 +683,24 @@ int nbla_hip_prune_f32(const float *x, float *y, size_t size, float rate, void *
     blocks = kSelectBlocks;
   hipLaunchKernelGGL(clear_select, dim3(clear_select_blocks()), dim3(256), 0, stream, st, rank);
   NBLA_HIP_LAUNCH_CHECK("clear_select");
+  const bool aligned = aligned16(x) && aligned16(y);
   for (int p = 0; p < kPasses; ++p) {
-    hipLaunchKernelGGL(prune_histogram, dim3((unsigned)blocks), dim3(kHistBlock), 0, stream, x, n4, n, ps, p);
+    if (aligned)
+      hipLaunchKernelGGL(prune_histogram<true>, dim3((unsigned)blocks), dim3(kHistBlock), 0, stream, x, n4, n, ps, p);
+    else
+      hipLaunchKernelGGL(prune_histogram<false>, dim3((unsigned)blocks), dim3(kHistBlock), 0, stream, x, n4, n, ps, p);
     NBLA_HIP_LAUNCH_CHECK("prune_histogram");
   }
   // every block of this launch resolves the last histogram first: two blocks per CU at most
   int64_t ablocks = ceil_div(n4 ? n4 : 1, (int64_t)kHistBlock * kPruneLoads);
   if (ablocks > 2 * kSelectBlocks)
     ablocks = 2 * kSelectBlocks;
-  hipLaunchKernelGGL(prune_apply, dim3((unsigned)ablocks), dim3(kHistBlock), 0, stream, x, y, n4, n, ps,
-                     rate == 1.0f ? 1.0f : 0.0f);
+  if (aligned)
+    hipLaunchKernelGGL(prune_apply<true>, dim3((unsigned)ablocks), dim3(kHistBlock), 0, stream, x, y, n4, n, ps,
+                       rate == 1.0f ? 1.0f : 0.0f);
+  else
+    hipLaunchKernelGGL(prune_apply<false>, dim3((unsigned)ablocks), dim3(kHistBlock), 0, stream, x, y, n4, n, ps,
+                       rate == 1.0f ? 1.0f : 0.0f);
   NBLA_HIP_LAUNCH_CHECK("prune_apply");
   return NBLA_HIP_OK;
 }

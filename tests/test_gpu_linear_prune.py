@@ -1,5 +1,7 @@
 """QuantizeLinear / DequantizeLinear / Prune on the GPU against the CPU oracle: bit-exact (every step of the
 reference chain is a separately rounded fp32 operation; Prune's threshold is an order statistic)."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -106,6 +108,25 @@ def test_prune(dev, size, rate):
         x[6] = -0.0
     y = kernels.prune(_dev(x, dev), rate)
     assert bits_equal(to_np(y), oracle.prune(x, rate))
+
+
+@pytest.mark.parametrize("x_off,y_off", [(1, 0), (0, 3), (2, 2), (1, 3)])
+def test_prune_on_views_that_are_not_16_byte_aligned(dev, x_off, y_off):
+    """x or y starting at an odd multiple of four bytes (a narrowed view of a larger array): the same result, through
+    32-bit accesses."""
+    rng = np.random.RandomState(9)
+    n = 100003
+    x = rng.randn(n).astype(np.float32)
+    xb = torch.zeros(n + 8, device=dev)
+    xb[x_off:x_off + n] = torch.from_numpy(x).to(dev)
+    yb = torch.full((n + 8,), 7.0, device=dev)
+    xv, yv = xb[x_off:x_off + n], yb[y_off:y_off + n]
+    assert (xv.data_ptr() % 16 != 0) or (yv.data_ptr() % 16 != 0)
+    ws = torch.empty(kernels.lib().nbla_hip_prune_workspace_bytes(), dtype=torch.uint8, device=dev)
+    kernels.check(kernels.lib().nbla_hip_prune_f32(kernels._p(xv), kernels._p(yv), ctypes.c_size_t(n), ctypes.c_float(0.7),
+                                                   kernels._p(ws), ctypes.c_size_t(ws.numel()), None))
+    assert bits_equal(to_np(yv), oracle.prune(x, 0.7))
+    assert (to_np(yb[:y_off]) == 7.0).all() and (to_np(yb[y_off + n:]) == 7.0).all()
 
 
 def test_prune_large_and_special_values(dev):

@@ -59,6 +59,33 @@ def test_recorder_kernel_bit_exact(dev, kind, shape):
             assert _f32_bits(to_np(m))[0] == _f32_bits(m_ref)[0], (it, to_np(m), m_ref)
 
 
+@pytest.mark.parametrize("kind", ["MinMaxMvaRecorder", "AbsMaxRecorder"])
+@pytest.mark.parametrize("x_off,y_off", [(1, 0), (0, 2), (3, 3), (1, None)])
+def test_recorder_on_views_that_are_not_16_byte_aligned(dev, kind, x_off, y_off):
+    """x or y starting at an odd multiple of four bytes (y_off None: in place): the same statistics and copy, through
+    32-bit accesses spread over all the blocks."""
+    rng = np.random.default_rng(5)
+    n = 300007
+    x = rng.standard_normal(n).astype(np.float32)
+    x[1234] = -0.0
+    xb = torch.zeros(n + 8, device=dev)
+    xb[x_off:x_off + n] = torch.from_numpy(x).to(dev)
+    xv = xb[x_off:x_off + n]
+    yb = torch.full((n + 8,), 7.0, device=dev)
+    yv = xv if y_off is None else yb[y_off:y_off + n]
+    two = kind == "MinMaxMvaRecorder"
+    m = torch.zeros(1, device=dev) if two else None
+    M = torch.zeros(1, device=dev)
+    y = K.range_recorder(xv, m, M, kind, decay=0.99, y=yv)
+    m_ref, M_ref = oracle.range_recorder(x, np.float32(0.0) if two else None, np.float32(0.0), kind, 0.99)
+    assert bits_equal(to_np(y), x)
+    assert _f32_bits(to_np(M))[0] == _f32_bits(M_ref)[0]
+    if two:
+        assert _f32_bits(to_np(m))[0] == _f32_bits(m_ref)[0]
+    if y_off is not None:
+        assert (to_np(yb[:y_off]) == 7.0).all() and (to_np(yb[y_off + n:]) == 7.0).all()
+
+
 def test_recorder_kernel_edge_cases(dev):
     """Signed zeros, NaNs, values beyond the +-1e8 the reductions start from, unaligned views, in-place, training off."""
     cases = [np.array([-0.0, 0.0, -0.0], np.float32), np.array([0.0, -0.0], np.float32),
