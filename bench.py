@@ -255,6 +255,72 @@ def bench_quantizers(dev, iters):
     return out
 
 
+def bench_shapes(dev, iters):
+    """Shapes away from the benchmark configurations (opt-in, `--section shapes`): extents that are no multiples of
+    four, views that are not 16-byte aligned, grouped and depthwise convolutions, operands that broadcast -- the
+    places where a kernel written for the aligned case falls to another path.  Times per call in ms."""
+    import torch
+    from nnabla_amd import kernels as k
+    out = {}
+    g = torch.Generator(device="cpu").manual_seed(7)
+    for (M, K, N) in ((4096, 4096, 11008), (4096, 4095, 11008), (4096, 4096, 11007), (4097, 4097, 11009),
+                      (512, 4096, 11008), (512, 4095, 11007), (64, 4096, 11007)):
+        x = torch.randn(M, K, generator=g).to(dev)
+        W = (torch.randn(K, N, generator=g) * 0.02).to(dev)
+        dy = torch.randn(M, N, generator=g).to(dev)
+        _, Wb, alpha = k.binary_weight_affine(x, W)
+        out["affine %dx%dx%d" % (M, K, N)] = {
+            "binary_weight_forward": time_kernel(lambda: k.binary_weight_affine(x, W), iters),
+            "binary_weight_backward": time_kernel(lambda: k.binary_affine_backward(dy, x, W, Wb, alpha), iters),
+            "affine_forward": time_kernel(lambda: k.affine_digits(x, W), iters),
+            "affine_backward": time_kernel(lambda: k.affine_backward(dy, x, W), iters)}
+        del x, W, dy, Wb, alpha
+    for xs, ws, pad, stride, group in (((32, 256, 14, 14), (256, 256, 3, 3), (1, 1), (1, 1), 1),
+                                       ((32, 256, 14, 14), (256, 1, 3, 3), (1, 1), (1, 1), 256),
+                                       ((32, 256, 14, 14), (256, 8, 3, 3), (1, 1), (1, 1), 32),
+                                       ((32, 256, 28, 28), (512, 256, 3, 3), (1, 1), (2, 2), 1),
+                                       ((32, 64, 56, 56), (64, 64, 3, 3), (1, 1), (1, 1), 1)):
+        x = torch.randn(xs, generator=g).to(dev)
+        W = (torch.randn(ws, generator=g) * 0.05).to(dev)
+        y, Wb, alpha = k.binary_weight_convolution(x, W, None, pad, stride, None, group)
+        dy = torch.randn(y.shape, generator=g).to(dev)
+        I = torch.zeros(ws, dtype=torch.int32, device=dev)
+        out["convolution %s x %s stride %d group %d" % (list(xs), list(ws), stride[0], group)] = {
+            "binary_weight_forward": time_kernel(lambda: k.binary_weight_convolution(x, W, None, pad, stride, None, group),
+                                                 iters),
+            "binary_weight_backward": time_kernel(lambda: k.binary_convolution_backward(dy, x, W, Wb, alpha, pad, stride,
+                                                                                        None, group), iters),
+            "convolution_forward": time_kernel(lambda: k.inq_convolution(x, W, I, W, I, None, pad, stride, None, group, 4,
+                                                                         k.INQ_PRODUCT_ONLY), iters),
+            "convolution_backward": time_kernel(lambda: k.convolution_backward(dy, x, W, pad, stride, None, group), iters)}
+    xs = (64, 256, 56, 56)
+    n = 64 * 256 * 56 * 56
+    buf, buf2 = torch.randn(n + 8, generator=g).to(dev), torch.randn(n + 8, generator=g).to(dev)
+    res = torch.empty(n + 8, device=dev)
+    for off in (0, 1):
+        x, dy, y = buf[off:off + n].view(xs), buf2[off:off + n].view(xs), res[off:off + n].view(xs)
+        r = {}
+        for qshape in ((1, 1, 1, 1), (1, 256, 1, 1)):
+            q = lambda v: torch.full(qshape, v, device=dev)
+            qmn, qmx, lmn, lmx = q(-6.0), q(6.0), q(0.0), q(255.0)
+            r["min_max_quantize ranges %s" % (list(qshape),)] = time_kernel(
+                lambda: k.min_max_quantize(x, qmn, qmx, lmn, lmx, 0.999, True, True, 0.01, out=y), iters)
+        m, Mx = torch.zeros(1, device=dev), torch.zeros(1, device=dev)
+        r["fixed_point_quantize"] = time_kernel(lambda: k.fixed_point_quantize(x.view(-1), True, 8, 2.0 ** -4,
+                                                                               out=y.view(-1)), iters)
+        r["prune"] = time_kernel(lambda: k.prune(x.view(-1), 0.9), iters)
+        r["min_max_mva_recorder"] = time_kernel(lambda: k.range_recorder(x.view(-1), m, Mx, "MinMaxMvaRecorder",
+                                                                         y=y.view(-1)), iters)
+        out["[64,256,56,56] %s" % ("16-byte aligned" if off == 0 else "view shifted by one float")] = r
+    x, dy = buf[:n].view(xs), buf2[:n].view(xs)
+    for bshape in ((64, 256, 56, 56), (1, 256, 1, 1), (1, 1, 1, 56), (1, 1, 1, 1)):
+        b = (torch.rand(bshape, generator=g) + 0.5).to(dev)
+        out["mul2 [64,256,56,56] x %s" % (list(bshape),)] = {
+            "forward": time_kernel(lambda: k.broadcast2("mul2", x, b), iters),
+            "gradient_of_the_second_operand": time_kernel(lambda: k.broadcast2_backward("mul2", 1, dy, x, b), iters)}
+    return out
+
+
 def bench_other_configs(dev, iters):
     """Whole-op timings (workspace allocation outside the loop is not possible through the convenience wrappers, so
     the caching allocator's hit is inside): binary convolutions of the ResNet-18 stage and the INQAffine layer."""
@@ -434,12 +500,14 @@ def main():
                     help="untimed steps; the first few dozen launches after idle run at ramping clocks")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=2048)
-    ap.add_argument("--section", choices=("all", "headline", "sweep", "quantizers", "other", "mfma"), default="all",
+    ap.add_argument("--section", choices=("all", "headline", "sweep", "quantizers", "other", "mfma", "shapes"),
+                    default="all",
                     help="headline: only the timed BinaryWeightAffine steps (what the rocprofv3 summaries profile); "
                          "sweep: headline plus the forward at M = 1 .. 1024 and BinaryConnectAffine (`sweep`); "
                          "quantizers: headline plus the quantizer kernels; other: headline plus the convolution, INQ, "
                          "MLP, backward and adjacent-function workloads (`other_configs`); mfma: headline plus the rates "
-                         "of kernels of nothing but matrix instructions (`mfma_rates`)")
+                         "of kernels of nothing but matrix instructions (`mfma_rates`); shapes (not part of `all`): "
+                         "headline plus shapes away from the benchmark configurations (`shapes`)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
@@ -477,6 +545,7 @@ def main():
     quant = bench_quantizers(dev, max(10, args.steps)) if args.section in ("all", "quantizers") else {}
     other = bench_other_configs(dev, max(5, args.steps // 2)) if args.section in ("all", "other") else {}
     mfma = bench_mfma_rates(dev) if args.section in ("all", "mfma") else {}
+    shapes = bench_shapes(dev, max(5, args.steps // 5)) if args.section == "shapes" else {}
     r = bench_binary_weight_affine(M, K, N, args.steps, args.warmup, dev)
     tflops = r["flop"] / (r["ms_per_step"] * 1e-3) / 1e12
     # the product's duration: the begin / end stamps of its launches inside the timed region
@@ -510,6 +579,8 @@ def main():
         "quantizers": quant,
         "other_configs": other,
     }
+    if shapes:
+        line["shapes"] = shapes
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(K, N, args.cpu_rows)
     else:
