@@ -781,7 +781,7 @@ int binary_conv_forward(const float *x, const float *W, float *Wb, float *alpha,
   if (rc)
     return rc;
   hipStream_t stream = as_stream(stream_);
-  if (conv_direct_applies(g)) { // many small groups: all of them in one launch each, over the materialised signs
+  if (conv_direct_forward_applies(g)) { // many small groups: all of them in one launch each, over the materialised signs
     rc = launch_conv_direct_binarize(W, Wb, alpha, g, zero_to, stream);
     if (rc)
       return rc;

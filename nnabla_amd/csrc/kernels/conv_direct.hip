@@ -63,6 +63,77 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_forward(const float 
   }
 }
 
+// The same for kOut consecutive output channels of one group per thread (Og a multiple of kOut): a block is one
+// (sample, tile of channels) and 256 output positions.  The tile's weights (times alpha) are laid out [k][channel] in
+// LDS once per block, so a tap's kOut weights are kOut / 4 broadcast reads of 16 bytes, and every input value loaded
+// serves kOut products; the loads of four taps along the innermost kernel axis are issued together.
+constexpr int kDirectLdsFloats = 12288; // 48 KiB of weights per block
+template <int kOut>
+__global__ __launch_bounds__(kDirectBlock) void conv_direct_forward_tile(const float *__restrict__ x,
+                                                                         const float *__restrict__ w,
+                                                                         const float *__restrict__ scale,
+                                                                         const float *__restrict__ bias,
+                                                                         float *__restrict__ y, ConvGeom g) {
+  extern __shared__ __attribute__((aligned(16))) float s_w[]; // [Kg][kOut]
+  typedef float float4_d __attribute__((ext_vector_type(4)));
+  const int64_t otiles = g.O / kOut;
+  const int64_t n = blockIdx.y / otiles, o0 = (blockIdx.y - n * otiles) * kOut, grp = o0 / g.Og;
+  const int Kg = (int)g.Kg;
+  for (int i = threadIdx.x; i < Kg * kOut; i += kDirectBlock) {
+    const int j = i / Kg, k = i - j * Kg; // consecutive threads read consecutive k of one channel
+    const float wv = w[(o0 + j) * g.Kg + k];
+    s_w[k * kOut + j] = scale ? wv * scale[o0 + j] : wv; // Ws = Wb * alpha, rounded once as the reference forms it
+  }
+  __syncthreads();
+  const int64_t p = (int64_t)blockIdx.x * kDirectBlock + threadIdx.x;
+  const bool live = p < g.out_sp_size;
+  const Position q = out_position(g, live ? p : 0);
+  const int b0 = q.o0 * g.stride[0] - g.pad[0], b1 = q.o1 * g.stride[1] - g.pad[1], b2 = q.o2 * g.stride[2] - g.pad[2];
+  const float *xn = x + (n * g.C + grp * g.Cg) * g.in_sp_size;
+  float acc[kOut];
+#pragma unroll
+  for (int j = 0; j < kOut; ++j)
+    acc[j] = 0.0f;
+  int t = 0; // k = c * k_size + tap
+  for (int64_t c = 0; c < g.Cg; ++c) {
+    const float *xc = xn + c * g.in_sp_size;
+    for (int k0 = 0; k0 < g.k[0]; ++k0)
+      for (int k1 = 0; k1 < g.k[1]; ++k1) {
+        const int i0 = b0 + k0 * g.dil[0], i1 = b1 + k1 * g.dil[1];
+        const bool row_in = live && (unsigned)i0 < (unsigned)g.in_sp[0] && (unsigned)i1 < (unsigned)g.in_sp[1];
+        const float *xr = xc + ((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2];
+        for (int k2 = 0; k2 < g.k[2]; k2 += 4) {
+          float xv[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int i2 = b2 + (k2 + u) * g.dil[2];
+            xv[u] = (row_in && k2 + u < g.k[2] && (unsigned)i2 < (unsigned)g.in_sp[2]) ? xr[i2] : 0.0f;
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            if (k2 + u < g.k[2]) { // uniform
+              const float4_d *wk = reinterpret_cast<const float4_d *>(s_w + (t + u) * kOut);
+#pragma unroll
+              for (int j4 = 0; j4 < kOut / 4; ++j4) {
+                const float4_d wv = wk[j4];
+                acc[4 * j4 + 0] = acc[4 * j4 + 0] + xv[u] * wv.x;
+                acc[4 * j4 + 1] = acc[4 * j4 + 1] + xv[u] * wv.y;
+                acc[4 * j4 + 2] = acc[4 * j4 + 2] + xv[u] * wv.z;
+                acc[4 * j4 + 3] = acc[4 * j4 + 3] + xv[u] * wv.w;
+              }
+            }
+          }
+          t += (g.k[2] - k2 < 4) ? g.k[2] - k2 : 4;
+        }
+      }
+  }
+  if (live) {
+#pragma unroll
+    for (int j = 0; j < kOut; ++j)
+      y[(n * g.O + o0 + j) * g.out_sp_size + p] = bias ? acc[j] + bias[o0 + j] : acc[j];
+  }
+}
+
 // dx[n, c, q] (+)= sum over the group's o and the taps whose window position p lies in the output:
 // (dy[n, o, p] * scale[o]) * w[o, c, tap]   (the unfolded gradient folded back, convolution.cpp:262-283)
 // take_sign: w holds the real-valued weights of a binary convolution, whose signs (sign.hpp:48-50) are what the
@@ -199,6 +270,15 @@ bool conv_direct_applies(const ConvGeom &g) {
   const double flops = 2.0 * (double)g.M * (double)g.Kg * (double)g.O;
   return flops / 1e7 < 25.0 * (double)g.group + flops / 1e8;
 }
+// The forward alone also for a single group of very few input channels under a kernel of many taps (the first layer
+// of an image network: 3 channels, 7 x 7): rows of the unfolded matrix that are mostly padding of the k tiles, which
+// the products on the matrix cores gather element by element.
+bool conv_direct_forward_applies(const ConvGeom &g) {
+  if (conv_direct_applies(g))
+    return true;
+  return g.group == 1 && g.Cg <= 4 && g.k_size >= 9 && g.O % 8 == 0 && g.O * g.Kg <= 0x7fffffffll &&
+         g.outer * (g.O / 8) <= 0x7fffffffll;
+}
 
 int launch_conv_direct_binarize(const float *W, float *Wb, float *alpha, const ConvGeom &g, float zero_to,
                                 hipStream_t stream) {
@@ -210,8 +290,19 @@ int launch_conv_direct_binarize(const float *W, float *Wb, float *alpha, const C
 
 int launch_conv_direct_forward(const float *x, const float *w, const float *scale, const float *bias, float *y,
                                const ConvGeom &g, hipStream_t stream) {
-  hipLaunchKernelGGL(conv_direct_forward, dim3(blocks_for(g.outer * g.O * g.out_sp_size)), dim3(kDirectBlock), 0, stream,
-                     x, w, scale, bias, y, g);
+  // (65535: the second grid extent; the tile's weights have to fit the LDS the kernel may use without asking)
+  if (g.Og % 16 == 0 && g.out_sp_size >= 64 && g.outer * (g.O / 16) <= 65535 && g.Kg * 16 <= kDirectLdsFloats) {
+    const dim3 grid((unsigned)ceil_div(g.out_sp_size, kDirectBlock), (unsigned)(g.outer * (g.O / 16)));
+    hipLaunchKernelGGL(conv_direct_forward_tile<16>, grid, dim3(kDirectBlock), (size_t)g.Kg * 16 * sizeof(float), stream,
+                       x, w, scale, bias, y, g);
+  } else if (g.Og % 8 == 0 && g.out_sp_size >= 64 && g.outer * (g.O / 8) <= 65535 && g.Kg * 8 <= kDirectLdsFloats) {
+    const dim3 grid((unsigned)ceil_div(g.out_sp_size, kDirectBlock), (unsigned)(g.outer * (g.O / 8)));
+    hipLaunchKernelGGL(conv_direct_forward_tile<8>, grid, dim3(kDirectBlock), (size_t)g.Kg * 8 * sizeof(float), stream,
+                       x, w, scale, bias, y, g);
+  } else {
+    hipLaunchKernelGGL(conv_direct_forward, dim3(blocks_for(g.outer * g.O * g.out_sp_size)), dim3(kDirectBlock), 0,
+                       stream, x, w, scale, bias, y, g);
+  }
   NBLA_HIP_LAUNCH_CHECK("conv_direct_forward");
   return NBLA_HIP_OK;
 }

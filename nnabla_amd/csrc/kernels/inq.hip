@@ -838,7 +838,7 @@ int nbla_hip_inq_convolution_f32(const float *x, float *W, int32_t *I, float *ol
     if (rc)
       return rc;
   }
-  if (conv_direct_applies(g)) // many small groups: all of them in one fp32 launch
+  if (conv_direct_forward_applies(g)) // many small groups: all of them in one fp32 launch
     return launch_conv_direct_forward(x, W, nullptr, bias, y, g, stream);
   // The product runs on the int8 digit kernels: the unfolded input goes straight into a row-scaled digit operand
   // (rows = output positions), the weights [Og, Kg] into another (rows = output channels); six exact digit products.

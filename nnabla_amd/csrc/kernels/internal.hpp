@@ -41,6 +41,7 @@ int launch_gemm_bits_unfold(const float *x, const ConvGeom &g, int64_t grp, cons
 // scale (may be null): alpha[o].  launch_conv_direct_binarize writes Wb = Sign(W) and alpha (may be null) for all
 // channels.  Backward: w as in the forward, or with take_sign the real-valued weights whose signs were used.
 bool conv_direct_applies(const ConvGeom &g);
+bool conv_direct_forward_applies(const ConvGeom &g); // (also a single group of very few input channels, many taps)
 int launch_conv_direct_binarize(const float *W, float *Wb, float *alpha, const ConvGeom &g, float zero_to,
                                 hipStream_t stream);
 int launch_conv_direct_forward(const float *x, const float *w, const float *scale, const float *bias, float *y,

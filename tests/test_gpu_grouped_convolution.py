@@ -1,6 +1,6 @@
 """Grouped convolutions whose groups are small (depthwise, a few channels per group): all groups run in one launch per
 kernel, in plain fp32 (conv_direct.hip), forward and backward, for the binary layers and for the real-weight
-Convolution.  Against the oracle (convolution.cpp:161-330 restated per sample and group) at the fp32-faithful
+Convolution; the forward of a single group of very few input channels takes the same kernels.  Against the oracle (convolution.cpp:161-330 restated per sample and group) at the fp32-faithful
 tolerance; Wb bit for bit, alpha at the tolerance of a sum in another order; accumulation into the gradients; Sign(0)
 that is neither +1 nor -1; windows holding NaN / Inf (the plain fp32 product propagates them as the reference does)."""
 import numpy as np
@@ -23,6 +23,12 @@ CASES = [
     ((3, 20, 40), (20, 1, 5), (2,), (1,), (1,), 20),                        # one spatial dimension
     ((2, 12, 5, 6, 7), (12, 2, 2, 3, 2), (1, 1, 0), (1, 2, 1), (1, 1, 2), 6),  # three
     ((2, 16, 7, 7), (16, 1, 7, 7), (3, 3), (1, 1), (1, 1), 16),            # a kernel as large as the input
+    # one group of very few input channels under a kernel of many taps (the first layer of an image network): the
+    # forward takes the same kernels, eight output channels per thread; the backward the general path
+    ((2, 3, 40, 36), (16, 3, 7, 7), (3, 3), (2, 2), (1, 1), 1),
+    ((2, 4, 20, 20), (8, 4, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((3, 1, 70, 9), (24, 1, 5, 3), (2, 1), (1, 1), (1, 1), 1),
+    ((2, 32, 12, 12), (64, 16, 3, 3), (1, 1), (1, 1), (1, 1), 2),           # sixteen output channels per thread
 ]
 
 
