@@ -288,7 +288,9 @@ __global__ __launch_bounds__(kBlk) void broadcast2_sum_inner(const float *__rest
 // per step); block (tile of kept indices, chunk) takes a run of the outer reduced indices.
 // Where the kept indices are fewer than the runs a block has in flight (a scalar operand), `vs` of a block's runs
 // share a kept index and take every vs-th group of outer reduced indices: vs partial sums per (index, chunk).
-template <int kOp, int kInput>
+// kVec 4: runs that are multiples of four long in 16-byte aligned arrays, four consecutive terms per lane and step
+// (the other operand is contiguous along the run or one value for it).
+template <int kOp, int kInput, int kVec>
 __global__ __launch_bounds__(kBlk) void broadcast2_sum_rows(const float *__restrict__ dy, const float *__restrict__ x0,
                                                             const float *__restrict__ x1, SumAxes Q, MinMaxRows R, int T,
                                                             int vs, int nchunks, float *__restrict__ partial) {
@@ -303,9 +305,10 @@ __global__ __launch_bounds__(kBlk) void broadcast2_sum_rows(const float *__restr
   const int64_t obase = strided_offset(k_in ? k : 0, A.nkept, A.ksize, Q.ok);
   const int64_t ori = Q.orr[A.nred - 1];
   const float *operand = kInput == 0 ? x0 : x1;
+  const float *other = kInput == 0 ? x1 : x0;
   const float own = (reads_inputs<kOp>() && k_in) ? operand[k] : 0.0f;
   float acc = 0.0f;
-  constexpr int kRows = 8; // outer reduced indices in flight per lane
+  constexpr int kRows = kVec == 4 ? 4 : 8; // outer reduced indices in flight per lane
   for (int64_t ro = W.ro_begin + (int64_t)sub * kRows; ro < W.ro_end; ro += (int64_t)kRows * vs) {
     int64_t oy[kRows], oo[kRows];
 #pragma unroll
@@ -314,14 +317,40 @@ __global__ __launch_bounds__(kBlk) void broadcast2_sum_rows(const float *__restr
       oy[j] = ybase + (in ? strided_offset(ro + j, A.nred - 1, A.rsize, A.rstride) : 0);
       oo[j] = obase + (in ? strided_offset(ro + j, A.nred - 1, A.rsize, Q.orr) : 0);
     }
-    for (int64_t ri = li; ri < R.Rin; ri += T) {
-      float t[kRows];
+    for (int64_t ri = (int64_t)li * kVec; ri < R.Rin; ri += (int64_t)T * kVec) {
+      if (kVec == 4) {
+        float4_v gy[kRows], ov[kRows];
 #pragma unroll
-      for (int j = 0; j < kRows; ++j)
-        t[j] = (k_in && ro + j < W.ro_end) ? term_of<kOp, kInput>(dy, x0, x1, oy[j] + ri, oo[j] + ri * ori, own) : 0.0f;
+        for (int j = 0; j < kRows; ++j) {
+          const bool in = k_in && ro + j < W.ro_end;
+          gy[j] = in ? *reinterpret_cast<const float4_v *>(dy + oy[j] + ri) : float4_v{0.0f, 0.0f, 0.0f, 0.0f};
+          if (reads_inputs<kOp>() && in) {
+            if (ori)
+              ov[j] = *reinterpret_cast<const float4_v *>(other + oo[j] + ri);
+            else
+              ov[j] = float4_v{other[oo[j]], other[oo[j]], other[oo[j]], other[oo[j]]};
+          } else {
+            ov[j] = float4_v{1.0f, 1.0f, 1.0f, 1.0f};
+          }
+        }
 #pragma unroll
-      for (int j = 0; j < kRows; ++j)
-        acc += t[j];
+        for (int j = 0; j < kRows; ++j) {
+          if (!(k_in && ro + j < W.ro_end))
+            continue;
+          const float g4[4] = {gy[j].x, gy[j].y, gy[j].z, gy[j].w}, o4[4] = {ov[j].x, ov[j].y, ov[j].z, ov[j].w};
+#pragma unroll
+          for (int c = 0; c < 4; ++c)
+            acc += grad_of<kOp, kInput>(g4[c], kInput == 0 ? own : o4[c], kInput == 0 ? o4[c] : own);
+        }
+      } else {
+        float t[kRows];
+#pragma unroll
+        for (int j = 0; j < kRows; ++j)
+          t[j] = (k_in && ro + j < W.ro_end) ? term_of<kOp, kInput>(dy, x0, x1, oy[j] + ri, oo[j] + ri * ori, own) : 0.0f;
+#pragma unroll
+        for (int j = 0; j < kRows; ++j)
+          acc += t[j];
+      }
     }
   }
   for (int o = T >> 1; o >= 1; o >>= 1)
@@ -447,8 +476,8 @@ struct SumPlan {
   SumAxes Q;
   MinMaxInner I;
   MinMaxRows R;
-  int T, vs;
-  int64_t chunks, count; // (chunks: partial sums per element, vs included)
+  int64_t row_chunks;    // row form: blocks per tile of kept indices
+  int64_t chunks, count; // (chunks: partial sums per element the workspace holds)
 };
 SumPlan make_sum_plan(const Groups &g, int input) {
   SumPlan P;
@@ -525,10 +554,15 @@ SumPlan make_sum_plan(const Groups &g, int input) {
     if (!P.R.ok)
       return P;
     P.inner = false;
-    P.T = row_lanes(P.R, 1);
-    const int64_t rps = kBlk / P.T;
-    P.vs = P.R.K < rps ? (int)(rps / P.R.K) : 1;
-    P.chunks = row_chunks(P.R) * P.vs;
+    // (the lanes per run, and with them the runs a block has in flight, depend on whether the pointers allow 16-byte
+    // accesses: the workspace is sized for the form with more partial sums)
+    P.row_chunks = row_chunks(P.R);
+    int64_t most = 1;
+    for (int vec : {1, 4}) {
+      const int64_t rps = kBlk / row_lanes(P.R, vec), vs = P.R.K < rps ? rps / P.R.K : 1;
+      most = vs > most ? vs : most;
+    }
+    P.chunks = P.row_chunks * most;
   }
   P.ok = P.count <= 0x7fffffffll;
   return P;
@@ -557,22 +591,32 @@ int backward(const float *dy, const float *x0, const float *x1, float *dx, const
   if (P.ok && workspace && aligned256(workspace) &&
       workspace_bytes >= (size_t)P.count * P.chunks * sizeof(float)) {
     float *partial = static_cast<float *>(workspace);
+    int64_t chunks = P.chunks; // partial sums per element of this launch
     if (P.inner) {
       const int64_t tiles = P.I.Ko * ((P.I.Wk + P.I.tw - 1) / P.I.tw);
       hipLaunchKernelGGL((broadcast2_sum_inner<kOp, kInput>), dim3((unsigned)tiles, (unsigned)P.chunks), dim3(kBlk), 0,
                          s, dy, x0, x1, P.Q, P.I, (int)P.chunks, partial);
     } else {
-      const int64_t rps = kBlk / P.T;
-      hipLaunchKernelGGL((broadcast2_sum_rows<kOp, kInput>),
-                         dim3((unsigned)((P.R.K * P.vs + rps - 1) / rps), (unsigned)(P.chunks / P.vs)), dim3(kBlk), 0, s,
-                         dy, x0, x1, P.Q, P.R, P.T, P.vs, (int)(P.chunks / P.vs), partial);
+      const bool vec4 = P.R.Rin % 4 == 0 && aligned16(dy) && (P.Q.orr[P.Q.A.nred - 1] == 0 || P.Q.orr[P.Q.A.nred - 1] == 1) &&
+                        (!reads_inputs<kOp>() || (aligned16(x0) && aligned16(x1)));
+      const int T = row_lanes(P.R, vec4 ? 4 : 1);
+      const int64_t rps = kBlk / T;
+      const int vs = P.R.K < rps ? (int)(rps / P.R.K) : 1;
+      chunks = P.row_chunks * vs;
+      const dim3 grid((unsigned)((P.R.K * vs + rps - 1) / rps), (unsigned)P.row_chunks);
+      if (vec4)
+        hipLaunchKernelGGL((broadcast2_sum_rows<kOp, kInput, 4>), grid, dim3(kBlk), 0, s, dy, x0, x1, P.Q, P.R, T, vs,
+                           (int)P.row_chunks, partial);
+      else
+        hipLaunchKernelGGL((broadcast2_sum_rows<kOp, kInput, 1>), grid, dim3(kBlk), 0, s, dy, x0, x1, P.Q, P.R, T, vs,
+                           (int)P.row_chunks, partial);
     }
     NBLA_HIP_LAUNCH_CHECK("broadcast2 backward sums");
-    if (P.chunks <= 16 && P.count >= 64)
+    if (chunks <= 16 && P.count >= 64)
       hipLaunchKernelGGL(broadcast2_sum_final, dim3((unsigned)((P.count + kBlk - 1) / kBlk)), dim3(kBlk), 0, s, partial,
-                         (int)P.chunks, dx, P.count, accum);
+                         (int)chunks, dx, P.count, accum);
     else
-      hipLaunchKernelGGL(broadcast2_sum_final_wave, dim3((unsigned)P.count), dim3(64), 0, s, partial, (int)P.chunks, dx,
+      hipLaunchKernelGGL(broadcast2_sum_final_wave, dim3((unsigned)P.count), dim3(64), 0, s, partial, (int)chunks, dx,
                          accum);
     NBLA_HIP_LAUNCH_CHECK("broadcast2 backward");
     return NBLA_HIP_OK;
