@@ -244,6 +244,14 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
   // channels' roles exchanged, taps flipped): it takes the product that keeps input positions in LDS.
   ConvGeom gt;
   const bool dx_slab = dx && binary && representable && conv_slab_transposed_geom(g, gt);
+  // few weights under many windows: the weight gradient in fp32 straight from dy and x, all groups at once (its
+  // partial results lie in the unfolded gradient's buffer, so it runs before the loop that fills that buffer)
+  if (dW && conv_direct_dw_applies(g)) {
+    rc = launch_conv_direct_dw(dy, x, dW, g, accum_w, col, (size_t)g.M * g.Kg * sizeof(float), stream);
+    if (rc)
+      return rc;
+    dW = nullptr;
+  }
   for (int64_t grp = 0; grp < g.group; ++grp) {
     const float *Wg = W + grp * g.Og * g.Kg;
     const float *ag = alpha ? alpha + grp * g.Og : nullptr;

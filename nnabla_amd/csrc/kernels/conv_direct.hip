@@ -211,6 +211,107 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_dw(const float *__re
     dW[ok] = accum ? dW[ok] + part[0] : part[0];
 }
 
+// dW for few weights under many windows (the first layers of an image network: 64 x 147 or 64 x 576 weights, 10^5
+// windows and more), where the digit operands of the matrix-core product cost more than the product: a block owns a
+// tile of 64 output channels x 64 columns k of one group and a run of windows, stages 32 windows at a time in LDS
+// (dy as [channel][window], the unfolded input as [k][window], gathered straight from x) and a thread accumulates
+// 4 x 4 weights in registers; the runs' partial results [chunk][O * Kg] are added up in chunk order afterwards.
+constexpr int kDwTile = 64, kDwWin = 32, kDwPitch = kDwWin + 1;
+__global__ __launch_bounds__(kDirectBlock) void conv_direct_dw_tile(const float *__restrict__ dy,
+                                                                    const float *__restrict__ x,
+                                                                    float *__restrict__ partial, ConvGeom g,
+                                                                    int64_t ktiles, int64_t otiles, int nchunks) {
+  __shared__ float s_dy[kDwTile * kDwPitch], s_col[kDwTile * kDwPitch];
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  int64_t b = blockIdx.x;
+  const int64_t kt = b % ktiles;
+  b /= ktiles;
+  const int64_t ot = b % otiles, grp = b / otiles;
+  const int64_t o_base = ot * kDwTile, k_base = kt * kDwTile;
+  const int64_t per = ceil_div(ceil_div(g.M, (int64_t)nchunks), (int64_t)kDwWin) * kDwWin;
+  const int64_t m0 = (int64_t)blockIdx.y * per, m1 = m0 + per < g.M ? m0 + per : g.M;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      acc[i][j] = 0.0f;
+  // A thread stages the same window slot w and the same eight rows r = tid / 32 + 8 i of both tiles in every step:
+  // the rows' channel and tap offsets are found once, a step only splits its window index.
+  constexpr int kStage = (kDwTile * kDwWin) / kDirectBlock;
+  const int w = tid & (kDwWin - 1), r0 = tid >> 5;
+  int64_t ch_off[kStage];
+  int d0[kStage], d1[kStage], d2[kStage];
+  bool k_in[kStage], o_in[kStage];
+#pragma unroll
+  for (int i = 0; i < kStage; ++i) {
+    const int64_t k = k_base + r0 + 8 * i;
+    k_in[i] = k < g.Kg;
+    o_in[i] = o_base + r0 + 8 * i < g.Og;
+    int64_t t = k_in[i] ? k : 0;
+    const int k2 = (int)(t % g.k[2]);
+    t /= g.k[2];
+    const int k1 = (int)(t % g.k[1]);
+    t /= g.k[1];
+    const int k0 = (int)(t % g.k[0]);
+    ch_off[i] = (grp * g.Cg + t / g.k[0]) * g.in_sp_size;
+    d0[i] = k0 * g.dil[0], d1[i] = k1 * g.dil[1], d2[i] = k2 * g.dil[2];
+  }
+  for (int64_t ms = m0; ms < m1; ms += kDwWin) {
+    const int64_t m = ms + w;
+    const bool m_in = m < m1;
+    const int64_t n = m_in ? m / g.out_sp_size : 0, p = m_in ? m - n * g.out_sp_size : 0;
+    const Position q = out_position(g, p);
+    const int b0 = q.o0 * g.stride[0] - g.pad[0], b1 = q.o1 * g.stride[1] - g.pad[1], b2 = q.o2 * g.stride[2] - g.pad[2];
+    const float *xn = x + n * g.C * g.in_sp_size;
+    const float *dyn = dy + (n * g.O + grp * g.Og + o_base + r0) * g.out_sp_size + p;
+#pragma unroll
+    for (int i = 0; i < kStage; ++i) {
+      const int r = r0 + 8 * i;
+      s_dy[r * kDwPitch + w] = (m_in && o_in[i]) ? dyn[(int64_t)8 * i * g.out_sp_size] : 0.0f;
+      const int i0 = b0 + d0[i], i1 = b1 + d1[i], i2 = b2 + d2[i];
+      const bool in = m_in && k_in[i] && (unsigned)i0 < (unsigned)g.in_sp[0] && (unsigned)i1 < (unsigned)g.in_sp[1] &&
+                      (unsigned)i2 < (unsigned)g.in_sp[2];
+      s_col[r * kDwPitch + w] = in ? xn[ch_off[i] + ((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2] + i2] : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int ww = 0; ww < kDwWin; ++ww) {
+      float a[4], c[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a[i] = s_dy[(ty * 4 + i) * kDwPitch + ww];
+        c[i] = s_col[(tx * 4 + i) * kDwPitch + ww];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = acc[i][j] + a[i] * c[j];
+    }
+    __syncthreads();
+  }
+  float *out = partial + (int64_t)blockIdx.y * g.O * g.Kg;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t o = o_base + ty * 4 + i, k = k_base + tx * 4 + j;
+      if (o < g.Og && k < g.Kg)
+        out[(grp * g.Og + o) * g.Kg + k] = acc[i][j];
+    }
+}
+__global__ __launch_bounds__(kDirectBlock) void conv_direct_dw_final(const float *__restrict__ partial, int nchunks,
+                                                                     float *__restrict__ dW, int64_t count, int accum) {
+  const int64_t i = (int64_t)blockIdx.x * kDirectBlock + threadIdx.x;
+  if (i >= count)
+    return;
+  float acc = 0.0f;
+  for (int c = 0; c < nchunks; ++c)
+    acc += partial[(int64_t)c * count + i];
+  dW[i] = accum ? dW[i] + acc : acc;
+}
+
 // db[o] (+)= sum over samples and positions of dy[n, o, p]
 __global__ __launch_bounds__(kDirectBlock) void conv_direct_db(const float *__restrict__ dy, float *__restrict__ db,
                                                                ConvGeom g, int accum) {
@@ -278,6 +379,37 @@ bool conv_direct_forward_applies(const ConvGeom &g) {
     return true;
   return g.group == 1 && g.Cg <= 4 && g.k_size >= 9 && g.O % 8 == 0 && g.O * g.Kg <= 0x7fffffffll &&
          g.outer * (g.O / 8) <= 0x7fffffffll;
+}
+
+// Few weights under many windows (see conv_direct_dw_tile); the partial results need chunks * O * Kg floats.
+bool conv_direct_dw_applies(const ConvGeom &g) {
+  return !conv_direct_applies(g) && g.Og * g.Kg <= 16384 && g.M >= 16384 && g.O * g.Kg <= 0x7fffffffll;
+}
+static int dw_chunks(const ConvGeom &g) {
+  const int64_t tiles = ceil_div(g.Og, kDwTile) * ceil_div(g.Kg, kDwTile) * g.group;
+  int64_t chunks = ceil_div(1024, tiles);
+  const int64_t most = g.M / (8 * kDwWin); // eight steps per block at least
+  if (chunks > most)
+    chunks = most;
+  if (chunks > g.M / g.O) // the caller's scratch is the unfolded matrix's: M * Kg floats
+    chunks = g.M / g.O;
+  return (int)(chunks < 1 ? 1 : chunks);
+}
+int launch_conv_direct_dw(const float *dy, const float *x, float *dW, const ConvGeom &g, bool accum, void *scratch,
+                          size_t scratch_bytes, hipStream_t stream) {
+  const int chunks = dw_chunks(g);
+  if (scratch_bytes < (size_t)chunks * g.O * g.Kg * sizeof(float) || !aligned16(scratch))
+    return fail(NBLA_HIP_ERR_MEMORY, "weight gradient: scratch too small or misaligned.");
+  const int64_t ktiles = ceil_div(g.Kg, kDwTile), otiles = ceil_div(g.Og, kDwTile);
+  float *partial = static_cast<float *>(scratch);
+  hipLaunchKernelGGL(conv_direct_dw_tile, dim3((unsigned)(ktiles * otiles * g.group), (unsigned)chunks),
+                     dim3(kDirectBlock), 0, stream, dy, x, partial, g, ktiles, otiles, chunks);
+  NBLA_HIP_LAUNCH_CHECK("conv_direct_dw_tile");
+  const int64_t count = g.O * g.Kg;
+  hipLaunchKernelGGL(conv_direct_dw_final, dim3((unsigned)ceil_div(count, kDirectBlock)), dim3(kDirectBlock), 0, stream,
+                     partial, chunks, dW, count, accum ? 1 : 0);
+  NBLA_HIP_LAUNCH_CHECK("conv_direct_dw_final");
+  return NBLA_HIP_OK;
 }
 
 int launch_conv_direct_binarize(const float *W, float *Wb, float *alpha, const ConvGeom &g, float zero_to,

@@ -42,6 +42,10 @@ int launch_gemm_bits_unfold(const float *x, const ConvGeom &g, int64_t grp, cons
 // channels.  Backward: w as in the forward, or with take_sign the real-valued weights whose signs were used.
 bool conv_direct_applies(const ConvGeom &g);
 bool conv_direct_forward_applies(const ConvGeom &g); // (also a single group of very few input channels, many taps)
+// The weight gradient of few weights under many windows in fp32 (all groups); scratch: M * Kg floats are enough.
+bool conv_direct_dw_applies(const ConvGeom &g);
+int launch_conv_direct_dw(const float *dy, const float *x, float *dW, const ConvGeom &g, bool accum, void *scratch,
+                          size_t scratch_bytes, hipStream_t stream);
 int launch_conv_direct_binarize(const float *W, float *Wb, float *alpha, const ConvGeom &g, float zero_to,
                                 hipStream_t stream);
 int launch_conv_direct_forward(const float *x, const float *w, const float *scale, const float *bias, float *y,

@@ -123,6 +123,36 @@ def test_input_gradient_as_a_convolution_accumulates(dev):
     assert max_rel_err(to_np(only[0]), first) <= TIGHT
 
 
+@pytest.mark.parametrize("xs,ws,pad,stride,dil,group", [
+    ((8, 3, 64, 64), (16, 3, 5, 5), (2, 2), (1, 1), (1, 1), 1),        # 75 columns: two tiles, the second partly empty
+    ((4, 3, 150, 150), (24, 3, 7, 7), (3, 3), (2, 2), (1, 1), 1),      # the first layer of an image network
+    ((4, 64, 72, 72), (72, 32, 3, 3), (1, 1), (1, 1), (1, 1), 2),      # two groups, 36 channels each
+    ((3, 8, 90, 80), (70, 8, 3, 2), (1, 0), (1, 1), (2, 1), 1),        # 70 channels: two tiles of channels
+])
+def test_weight_gradient_of_few_weights_under_many_windows(dev, xs, ws, pad, stride, dil, group):
+    """16384 windows or more and at most 65536 weights per group: dW comes from a tiled fp32 kernel that reads dy and x
+    directly (partial results per run of windows, added in order); against the oracle, with accumulation, alone and
+    together with dx and db, for the real-weight and the binary layers."""
+    x, W, dy = _data(xs, ws, pad, stride, dil, group, 46)
+    d = lambda a: _dev(a, dev)
+    rdx, rdw, rdb = oracle.convolution_backward(dy, x, W, pad, stride, dil, group)
+    gdx, gdw, gdb = kernels.convolution_backward(d(dy), d(x), d(W), pad, stride, dil, group)
+    for got, ref in ((gdx, rdx), (gdw, rdw), (gdb, rdb)):
+        assert max_rel_err(to_np(got), ref) <= TIGHT
+    only = kernels.convolution_backward(d(dy), d(x), d(W), pad, stride, dil, group, want=(False, True, False))
+    assert only[0] is None and only[2] is None and max_rel_err(to_np(only[1]), rdw) <= TIGHT
+    again = kernels.convolution_backward(d(dy), d(x), d(W), pad, stride, dil, group, want=(False, True, False))
+    assert np.array_equal(to_np(again[1]), to_np(only[1]))          # the same from run to run
+    old = np.random.RandomState(7).randn(*ws).astype(np.float32)
+    acc = kernels.convolution_backward(d(dy), d(x), d(W), pad, stride, dil, group, dW=d(old), want=(False, True, False))
+    assert max_rel_err(to_np(acc[1]), rdw + old) <= TIGHT
+    alpha = np.abs(W).reshape(ws[0], -1).mean(1).astype(np.float32)
+    ref = oracle.binary_convolution_backward(dy, x, W, alpha, pad, stride, dil, group, 1.0)
+    got = kernels.binary_convolution_backward(d(dy), d(x), d(W), None, d(alpha), pad, stride, dil, group, 1.0)
+    for g_, r_ in zip(got, ref):
+        assert max_rel_err(to_np(g_), r_) <= TIGHT
+
+
 def test_config4_backward(dev):
     """Benchmark configuration 4 shape (x [32,256,14,14], W [256,256,3,3], stride 1, pad 1): the oracle covers 2 of the 32
     samples for dx (samples are independent); dW and db of all 32 are checked against torch's float64 autograd on
