@@ -244,6 +244,9 @@ int nbla_hip_affine_digits_f32(const float *x, const float *W, const float *bias
   if (rc)
     return rc;
   hipStream_t stream = as_stream(stream_);
+  // a handful of rows: one fp32 pass over W instead of its conversion to digit operands
+  if (affine_few_rows_applies(x, W, y, M, K, N) && workspace_bytes >= affine_few_rows_workspace_bytes(M, K, N))
+    return launch_affine_few_rows(x, W, bias, y, M, K, N, workspace, workspace_bytes, stream);
   char *xd = static_cast<char *>(workspace);
   char *wd = xd + round_up(nbla_hip_digit_operand_bytes(M, K), 256);
   rc = nbla_hip_split_digits_f32(x, K, xd, M, K, stream_);

@@ -787,6 +787,11 @@ int nbla_hip_inq_affine_f32(const float *x, float *W, int32_t *I, float *old_W, 
     if (rc)
       return rc;
   }
+  // a handful of rows: one fp32 pass over W instead of its conversion to a digit operand (the split operand's and
+  // the weights' operand's space holds the partial results)
+  if (affine_few_rows_applies(x, W, y, M, K, N) &&
+      p.flag_off - p.split_off >= affine_few_rows_workspace_bytes(M, K, N))
+    return launch_affine_few_rows(x, W, bias, y, M, K, N, base + p.split_off, p.flag_off - p.split_off, stream);
   rc = nbla_hip_split_digits_f32(x, K, base + p.split_off, M, K, stream_);
   if (rc)
     return rc;

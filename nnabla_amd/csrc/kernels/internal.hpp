@@ -36,6 +36,12 @@ struct ConvGeom;
 bool gemm_bits_unfold_applies(const ConvGeom &g);
 int launch_gemm_bits_unfold(const float *x, const ConvGeom &g, int64_t grp, const uint32_t *bits, const float *alpha,
                             const float *bias, float *y, hipStream_t stream, int32_t *row_shift = nullptr);
+// y = x . W (+ bias) for at most 16 rows of x and real-valued weights [K, N]: one fp32 pass over W
+// (affine_few_rows.hip).  The workspace holds the partial results of the slabs of K.
+bool affine_few_rows_applies(const float *x, const float *W, const float *y, int64_t M, int64_t K, int64_t N);
+size_t affine_few_rows_workspace_bytes(int64_t M, int64_t K, int64_t N);
+int launch_affine_few_rows(const float *x, const float *W, const float *bias, float *y, int64_t M, int64_t K, int64_t N,
+                           void *workspace, size_t workspace_bytes, hipStream_t stream);
 // Grouped convolutions whose groups are too small for the matrix cores (depthwise, ResNeXt-style), all groups in one
 // launch, plain fp32 (conv_direct.hip).  w: the weights [O, Kg] (for a binary convolution the materialised signs),
 // scale (may be null): alpha[o].  launch_conv_direct_binarize writes Wb = Sign(W) and alpha (may be null) for all

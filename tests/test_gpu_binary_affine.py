@@ -565,6 +565,33 @@ def test_affine_digits_special_rows_and_narrow_weights(dev):
     assert max_rel_err(yw, xi.astype(np.float64) @ Wp.astype(np.float64)) <= TIGHT
 
 
+@pytest.mark.parametrize("M", [1, 2, 3, 8, 13, 16, 17])
+@pytest.mark.parametrize("K,N", [(1024, 1024), (1000, 1284), (4099, 516)])
+def test_affine_of_a_few_rows(dev, M, K, N):
+    """At most 16 rows against real-valued weights of a million elements or more: one fp32 pass over W (slabs of K,
+    added in order) instead of the digit operands; against the oracle with and without bias, and NaN / Inf element by
+    element as the reference's product gives them."""
+    rng = np.random.RandomState(100 * M + K % 7)
+    x = rng.randn(M, K).astype(np.float32)
+    W = (rng.randn(K, N) * 0.05).astype(np.float32)
+    b = rng.randn(N).astype(np.float32)
+    y = to_np(kernels.affine_digits(_dev(x, dev), _dev(W, dev)))
+    assert max_rel_err(y, oracle.affine(x, W, None)) <= TIGHT
+    y = to_np(kernels.affine_digits(_dev(x, dev), _dev(W, dev), _dev(b, dev)))
+    assert max_rel_err(y, oracle.affine(x, W, b)) <= TIGHT
+    if M > 2:                       # (rows in between stay finite)
+        x[M - 1, K - 1] = np.inf    # the last row of W's last slab
+        x[0, 5] = -np.inf
+    W[7, 11] = np.nan
+    W[K - 1, 12] = np.inf
+    if M > 3:
+        x[M // 2, K - 1] = 0.0      # 0 * Inf
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref = oracle.affine(x, W, b)
+    y = to_np(kernels.affine_digits(_dev(x, dev), _dev(W, dev), _dev(b, dev)))
+    _same_non_finite(y, ref, TIGHT)
+
+
 def _fixed_point_rows(rng, M, K, delta=2.0 ** -4, n=8):
     """Rows as FixedPointQuantize (sign, n bits, step delta) leaves them: integers in [-127, 127] times delta."""
     return (rng.randint(-(2 ** (n - 1) - 1), 2 ** (n - 1), size=(M, K)) * delta).astype(np.float32)
