@@ -231,7 +231,8 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
     if (binary && !Wb && !(zero_to == 1.0f || zero_to == -1.0f))
       return fail(NBLA_HIP_ERR_VALUE, "the binarised weights are needed when Sign(0) is neither +1 nor -1.");
     return launch_conv_direct_backward(dy, x, (binary && Wb) ? Wb : W, binary ? alpha : nullptr, dx, dW, db, g, accum_x,
-                                       accum_w, accum_b, binary && !Wb, zero_to, stream);
+                                       accum_w, accum_b, binary && !Wb, zero_to, static_cast<float *>(workspace),
+                                       workspace_bytes, stream);
   }
   char *base = static_cast<char *>(workspace);
   float *dyt = reinterpret_cast<float *>(base + p.dyt_off);

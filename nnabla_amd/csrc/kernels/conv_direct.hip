@@ -134,45 +134,160 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_forward_tile(const f
   }
 }
 
-// dx[n, c, q] (+)= sum over the group's o and the taps whose window position p lies in the output:
-// (dy[n, o, p] * scale[o]) * w[o, c, tap]   (the unfolded gradient folded back, convolution.cpp:262-283)
-// take_sign: w holds the real-valued weights of a binary convolution, whose signs (sign.hpp:48-50) are what the
-// forward pass multiplied with.
-__global__ __launch_bounds__(kDirectBlock) void conv_direct_dx(const float *__restrict__ dy, const float *__restrict__ w,
-                                                               const float *__restrict__ scale, float *__restrict__ dx,
-                                                               ConvGeom g, int accum, int take_sign, float zero_to) {
-  const int64_t total = g.outer * g.C * g.in_sp_size;
-  for (int64_t i = (int64_t)blockIdx.x * kDirectBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kDirectBlock) {
-    int64_t pos = i % g.in_sp_size;
-    const int64_t nc = i / g.in_sp_size, c = nc % g.C, n = nc / g.C, grp = c / g.Cg, cl = c - grp * g.Cg;
-    const int q2 = (int)(pos % g.in_sp[2]);
-    pos /= g.in_sp[2];
-    const int q1 = (int)(pos % g.in_sp[1]), q0 = (int)(pos / g.in_sp[1]);
-    const float *dyn = dy + (n * g.O + grp * g.Og) * g.out_sp_size;
-    const float *wg = w + (grp * g.Og) * g.Kg + cl * g.k_size;
-    float acc = 0.0f;
+// One batch of taps of one element of the result: rows the sample's source at the first of kOB channels (the next ones
+// L floats further, as many as `channels`), sw those channels' weights in LDS ([channel][taps], this batch's first tap),
+// reach/ok where the taps land (byte offsets into a channel of the source).  The loads of a batch are all in flight together;
+// taps outside the output load a valid address and are left out of the sum.  kFull: all kTapBatch taps exist.
+constexpr int kTapBatch = 9;
+constexpr uint32_t kNoReach = 0xffffffffu;
+template <int kOB, bool kFull, bool kForward>
+__device__ __forceinline__ float conv_direct_gather_batch(const float *__restrict__ rows, int64_t L, const float *sw, int taps,
+                                                      int channels, int count, const uint32_t (&reach)[kTapBatch],
+                                                      const bool (&ok)[kTapBatch], float acc) {
+  float gy[kOB][kTapBatch];
+#pragma unroll
+  for (int jo = 0; jo < kOB; ++jo) {
+    const char *row = reinterpret_cast<const char *>(rows + (jo < channels ? jo : channels - 1) * L);
+#pragma unroll
+    for (int j = 0; j < kTapBatch; ++j)
+      gy[jo][j] = *reinterpret_cast<const float *>(row + reach[j]);
+  }
+#pragma unroll
+  for (int jo = 0; jo < kOB; ++jo) {
+    const bool live = jo < channels;
+    const float *wr = sw + (live ? jo : channels - 1) * taps;
+#pragma unroll
+    for (int j = 0; j < kTapBatch; ++j) {
+      const float wv = wr[kFull || j < count ? j : 0];
+      if (kForward) // a tap in the padding is a zero that is multiplied
+        acc = acc + (live ? (ok[j] ? gy[jo][j] : 0.0f) * wv : 0.0f);
+      else
+        acc = acc + (live && ok[j] ? gy[jo][j] * wv : 0.0f);
+    }
+  }
+  return acc;
+}
+
+// Both directions of a convolution of small groups as a gather, a thread per element of the result:
+//   backward  dx[n, c, q] (+)= sum over the group's o and the taps whose window position p lies in the output of
+//             (dy[n, o, p] * scale[o]) * w[o, c, tap]   (the unfolded gradient folded back, convolution.cpp:262-283);
+//             take_sign: w holds the real-valued weights of a binary convolution, whose signs (sign.hpp:48-50) are
+//             what the forward pass multiplied with;
+//   forward   y[n, o, p] = sum over the group's c and the taps of x[n, c, window(p, tap)] * (w[o, c, tap] * scale[o])
+//             (+ bias[o]); zeros where the window leaves the input, multiplied like any other value (0 * Inf = NaN as
+//             in the reference's product).
+// Block (tile of the result's positions, channels, samples), of 64 to 256 threads.  Where each tap lands from a
+// thread's position is the same for every (sample, channel) the block visits: a table in LDS, filled once (held in
+// registers when the kernel has at most kTapBatch taps).  The weights that meet one channel of the result, `held`
+// source channels at a time, signs taken and scaled, sit in LDS too; the samples' loop runs inside, so they are
+// prepared once per channel.  32-bit arithmetic per lane: a block-uniform row pointer plus a byte offset.
+// kUnit (backward): unit strides, no divisibility to test.
+template <bool kForward, bool kUnit>
+__global__ __launch_bounds__(kDirectBlock) void conv_direct_gather(const float *__restrict__ src,
+                                                                   const float *__restrict__ w,
+                                                                   const float *__restrict__ scale,
+                                                                   const float *__restrict__ bias,
+                                                                   float *__restrict__ dst, ConvGeom g, int held,
+                                                                   int accum, int take_sign, float zero_to) {
+  constexpr int kOB = 1; // (more source channels per step gave nothing)
+  extern __shared__ uint32_t s_gather[];
+  const int taps = (int)g.k_size, threads = (int)blockDim.x, tid = (int)threadIdx.x;
+  uint32_t *s_reach = s_gather;                                          // [taps][threads]: byte offset, or kNoReach
+  float *s_w = reinterpret_cast<float *>(s_gather + (size_t)taps * threads); // [held][taps]
+  const int pos = (int)(blockIdx.x * blockDim.x) + tid;
+  const int64_t positions = kForward ? g.out_sp_size : g.in_sp_size, L = kForward ? g.in_sp_size : g.out_sp_size;
+  const bool live = pos < positions;
+  {
+    const int in0 = (int)g.in_sp[0], in1 = (int)g.in_sp[1], in2 = (int)g.in_sp[2], out0 = (int)g.out_sp[0],
+              out1 = (int)g.out_sp[1], out2 = (int)g.out_sp[2];
+    const int d1 = kForward ? out1 : in1, d2 = kForward ? out2 : in2;
+    const int q2 = pos % d2, r = pos / d2, q1 = r % d1, q0 = r / d1;
+    const int s0 = (int)g.stride[0], s1 = (int)g.stride[1], s2 = (int)g.stride[2];
     int t = 0;
-    for (int k0 = 0; k0 < g.k[0]; ++k0)
-      for (int k1 = 0; k1 < g.k[1]; ++k1)
-        for (int k2 = 0; k2 < g.k[2]; ++k2, ++t) {
-          const int e0 = q0 + g.pad[0] - k0 * g.dil[0], e1 = q1 + g.pad[1] - k1 * g.dil[1],
-                    e2 = q2 + g.pad[2] - k2 * g.dil[2];
-          if (e0 < 0 || e1 < 0 || e2 < 0 || e0 % g.stride[0] || e1 % g.stride[1] || e2 % g.stride[2])
-            continue;
-          const int p0 = e0 / g.stride[0], p1 = e1 / g.stride[1], p2 = e2 / g.stride[2];
-          if (p0 >= g.out_sp[0] || p1 >= g.out_sp[1] || p2 >= g.out_sp[2])
-            continue;
-          const int64_t p = ((int64_t)p0 * g.out_sp[1] + p1) * g.out_sp[2] + p2;
-          for (int64_t o = 0; o < g.Og; ++o) {
-            const float gy = dyn[o * g.out_sp_size + p];
-            const float gs = scale ? gy * scale[grp * g.Og + o] : gy;
-            float wv = wg[o * g.Kg + t];
-            if (take_sign)
-              wv = (wv > 0.0f) ? 1.0f : ((wv < 0.0f) ? -1.0f : zero_to);
-            acc = acc + gs * wv;
+    for (int k0 = 0; k0 < (int)g.k[0]; ++k0)
+      for (int k1 = 0; k1 < (int)g.k[1]; ++k1)
+        for (int k2 = 0; k2 < (int)g.k[2]; ++k2, ++t) {
+          uint32_t at = kNoReach;
+          if (kForward) {
+            const int i0 = q0 * s0 - (int)g.pad[0] + k0 * (int)g.dil[0], i1 = q1 * s1 - (int)g.pad[1] + k1 * (int)g.dil[1],
+                      i2 = q2 * s2 - (int)g.pad[2] + k2 * (int)g.dil[2];
+            if (live && (unsigned)i0 < (unsigned)in0 && (unsigned)i1 < (unsigned)in1 && (unsigned)i2 < (unsigned)in2)
+              at = (uint32_t)((i0 * in1 + i1) * in2 + i2) * 4u;
+          } else {
+            const int e0 = q0 + (int)g.pad[0] - k0 * (int)g.dil[0], e1 = q1 + (int)g.pad[1] - k1 * (int)g.dil[1],
+                      e2 = q2 + (int)g.pad[2] - k2 * (int)g.dil[2];
+            int p0 = e0, p1 = e1, p2 = e2;
+            bool ok = live;
+            if (!kUnit) {
+              ok = ok && e0 >= 0 && e1 >= 0 && e2 >= 0 && e0 % s0 == 0 && e1 % s1 == 0 && e2 % s2 == 0;
+              p0 = e0 / s0, p1 = e1 / s1, p2 = e2 / s2;
+            }
+            if (ok && (unsigned)p0 < (unsigned)out0 && (unsigned)p1 < (unsigned)out1 && (unsigned)p2 < (unsigned)out2)
+              at = (uint32_t)((p0 * out1 + p1) * out2 + p2) * 4u;
+          }
+          s_reach[t * threads + tid] = at;
+        }
+  }
+  // (each thread reads back only what it wrote: no barrier for this table)
+  uint32_t reach[kTapBatch];
+  bool ok[kTapBatch];
+  const auto fetch = [&](int t0) {
+#pragma unroll
+    for (int j = 0; j < kTapBatch; ++j) {
+      const uint32_t r = t0 + j < taps ? s_reach[(t0 + j) * threads + tid] : kNoReach;
+      ok[j] = r != kNoReach, reach[j] = ok[j] ? r : 0u;
+    }
+  };
+  const bool few = taps <= kTapBatch;
+  if (few)
+    fetch(0);
+  const int C = (int)g.C, O = (int)g.O, Cg = (int)g.Cg, Og = (int)g.Og, outer = (int)g.outer;
+  const int channels = kForward ? O : C;   // of the result
+  const int sources = kForward ? Cg : Og;  // channels of src that meet one channel of the result
+  const int64_t Kg = g.Kg;
+  // (channels along blockIdx.y, samples along blockIdx.z: no division per pair)
+  for (int c = blockIdx.y; c < channels; c += gridDim.y) {
+    const int grp = c / (kForward ? Og : Cg), cl = c - grp * Cg; // (cl: backward)
+    for (int o0 = 0; o0 < sources; o0 += held) {
+      const int no = sources - o0 < held ? sources - o0 : held;
+      __syncthreads(); // the previous weights are done with
+      for (int i = tid; i < no * taps; i += threads) {
+        const int o = i / taps, t = i - o * taps;
+        const int64_t row = kForward ? c : (int64_t)grp * Og + o0 + o; // the weights' channel out
+        float wv = kForward ? w[row * Kg + (int64_t)(o0 + o) * taps + t] : w[row * Kg + cl * taps + t];
+        if (take_sign)
+          wv = (wv > 0.0f) ? 1.0f : ((wv < 0.0f) ? -1.0f : zero_to);
+        s_w[i] = scale ? wv * scale[row] : wv;
+      }
+      __syncthreads();
+      if (!live)
+        continue;
+      for (int n = blockIdx.z; n < outer; n += gridDim.z) {
+        const float *rows = src + ((int64_t)n * (kForward ? C : O) + (int64_t)grp * sources + o0) * L;
+        float acc = 0.0f;
+        if (few) {
+          if (taps == kTapBatch)
+            for (int o = 0; o < no; o += kOB)
+              acc = conv_direct_gather_batch<kOB, true, kForward>(rows + o * L, L, s_w + o * taps, taps, no - o, taps,
+                                                                  reach, ok, acc);
+          else
+            for (int o = 0; o < no; o += kOB)
+              acc = conv_direct_gather_batch<kOB, false, kForward>(rows + o * L, L, s_w + o * taps, taps, no - o, taps,
+                                                                   reach, ok, acc);
+        } else {
+          for (int t0 = 0; t0 < taps; t0 += kTapBatch) {
+            fetch(t0);
+            for (int o = 0; o < no; o += kOB)
+              acc = conv_direct_gather_batch<kOB, false, kForward>(rows + o * L, L, s_w + o * taps + t0, taps, no - o,
+                                                                   taps - t0, reach, ok, acc);
           }
         }
-    dx[i] = accum ? dx[i] + acc : acc;
+        float *out = dst + ((int64_t)n * channels + c) * positions + pos;
+        if (kForward && bias && o0 + no == sources)
+          acc = acc + bias[c];
+        *out = (accum || o0 > 0) ? *out + acc : acc;
+      }
+    }
   }
 }
 
@@ -209,6 +324,124 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_dw(const float *__re
   }
   if (threadIdx.x == 0)
     dW[ok] = accum ? dW[ok] + part[0] : part[0];
+}
+
+// dW of small groups, a thread per output position: block (kO channels out of one group x one channel in, tile of
+// the positions, run of the samples).  A thread keeps its position while it walks the samples, so the window's
+// place, the taps' offsets (LDS) and which taps fall into the padding (a bit mask) are found once; per sample and tap
+// there is one load of x and kO products with the kO values of dy.  When a tile has fewer than 256 positions the
+// block's threads take several samples side by side.  Sums in registers (indexed statically), folded over the block
+// at the end; partial results [tile * runs + run][O * Kg].
+template <int kO, int kTaps>
+__global__ __launch_bounds__(kDirectBlock) void conv_direct_dw_pairs(const float *__restrict__ dy,
+                                                                     const float *__restrict__ x,
+                                                                     float *__restrict__ partial, ConvGeom g,
+                                                                     int lanes_p, int runs) {
+  __shared__ int s_off[kTaps][4];
+  __shared__ float s_sum[kDirectBlock / 64][kO * kTaps];
+  const int taps = (int)g.k_size, tid = threadIdx.x;
+  if (tid < taps) {
+    int t = tid;
+    const int k2 = t % g.k[2];
+    t /= g.k[2];
+    const int d0 = (t / g.k[1]) * g.dil[0], d1 = (t % g.k[1]) * g.dil[1], d2 = k2 * g.dil[2];
+    s_off[tid][0] = d0, s_off[tid][1] = d1, s_off[tid][2] = d2;
+    s_off[tid][3] = (d0 * g.in_sp[1] + d1) * g.in_sp[2] + d2;
+  }
+  __syncthreads();
+  const int64_t og = g.Og / kO; // blocks of channels out per group
+  const int64_t pair = blockIdx.x, ob = pair / g.Cg, c = pair - ob * g.Cg, grp = ob / og, o = grp * g.Og + (ob - grp * og) * kO;
+  const int sub = tid / lanes_p, nsub = kDirectBlock / lanes_p;
+  const int64_t p = (int64_t)blockIdx.y * lanes_p + (tid - sub * lanes_p);
+  const int64_t per = ceil_div(g.outer, (int64_t)runs), n0 = (int64_t)blockIdx.z * per,
+                n1 = n0 + per < g.outer ? n0 + per : g.outer;
+  float acc[kO][kTaps];
+#pragma unroll
+  for (int j = 0; j < kO; ++j)
+#pragma unroll
+    for (int t = 0; t < kTaps; ++t)
+      acc[j][t] = 0.0f;
+  if (p < g.out_sp_size) {
+    const Position q = out_position(g, p);
+    const int b0 = q.o0 * g.stride[0] - g.pad[0], b1 = q.o1 * g.stride[1] - g.pad[1], b2 = q.o2 * g.stride[2] - g.pad[2];
+    // per tap, once: the byte offset into a channel of x, and all ones where the tap lies inside the input (taps in
+    // the padding, and the template's taps beyond the kernel's, load the channel's first element and mask it to zero)
+    const int in0 = (int)g.in_sp[0], in1 = (int)g.in_sp[1], in2 = (int)g.in_sp[2];
+    const int first = (b0 * in1 + b1) * in2 + b2; // (negative in the padding: masked)
+    uint32_t off[kTaps], inside = 0;
+#pragma unroll
+    for (int t = 0; t < kTaps; ++t) {
+      off[t] = 0;
+      if (t < taps) {
+        const int i0 = b0 + s_off[t][0], i1 = b1 + s_off[t][1], i2 = b2 + s_off[t][2];
+        if ((unsigned)i0 < (unsigned)in0 && (unsigned)i1 < (unsigned)in1 && (unsigned)i2 < (unsigned)in2)
+          inside |= 1u << t, off[t] = (uint32_t)(first + s_off[t][3]) * 4u;
+      }
+    }
+    for (int64_t n = n0 + sub; n < n1; n += nsub) {
+      float gy[kO];
+#pragma unroll
+      for (int j = 0; j < kO; ++j)
+        gy[j] = dy[(n * g.O + o + j) * g.out_sp_size + p];
+      const char *xc = reinterpret_cast<const char *>(x + (n * g.C + grp * g.Cg + c) * g.in_sp_size);
+      float xv[kTaps];
+#pragma unroll
+      for (int t = 0; t < kTaps; ++t)
+        xv[t] = *reinterpret_cast<const float *>(xc + off[t]);
+#pragma unroll
+      for (int t = 0; t < kTaps; ++t) {
+        const uint32_t keep = 0u - ((inside >> t) & 1u);
+        const float v = __uint_as_float(__float_as_uint(xv[t]) & keep);
+#pragma unroll
+        for (int j = 0; j < kO; ++j)
+          acc[j][t] = acc[j][t] + gy[j] * v;
+      }
+    }
+  }
+  const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+  for (int j = 0; j < kO; ++j)
+#pragma unroll
+    for (int t = 0; t < kTaps; ++t) {
+      if (t < taps) {
+        float v = acc[j][t];
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1)
+          v += __shfl_xor(v, off);
+        if (lane == 0)
+          s_sum[wave][j * kTaps + t] = v;
+      }
+    }
+  __syncthreads();
+  if (tid < kO * kTaps && tid % kTaps < taps) {
+    float v = s_sum[0][tid];
+    for (int w = 1; w < kDirectBlock / 64; ++w)
+      v += s_sum[w][tid];
+    const int j = tid / kTaps, t = tid - j * kTaps;
+    const int64_t chunk = (int64_t)blockIdx.y * runs + blockIdx.z;
+    partial[chunk * g.O * g.Kg + (o + j) * g.Kg + c * g.k_size + t] = v;
+  }
+}
+// db likewise: block (o, chunk), partial results [chunk][O]
+__global__ __launch_bounds__(kDirectBlock) void conv_direct_db_chunks(const float *__restrict__ dy,
+                                                                      float *__restrict__ partial, ConvGeom g,
+                                                                      int nchunks) {
+  __shared__ float s_sum[kDirectBlock / 64];
+  const int64_t o = blockIdx.x, per = ceil_div(g.M, (int64_t)nchunks), m0 = (int64_t)blockIdx.y * per,
+                m1 = m0 + per < g.M ? m0 + per : g.M;
+  float acc = 0.0f;
+  for (int64_t m = m0 + threadIdx.x; m < m1; m += kDirectBlock) {
+    const int64_t n = m / g.out_sp_size, p = m - n * g.out_sp_size;
+    acc = acc + dy[(n * g.O + o) * g.out_sp_size + p];
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1)
+    acc += __shfl_xor(acc, off);
+  if ((threadIdx.x & 63) == 0)
+    s_sum[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0)
+    partial[(int64_t)blockIdx.y * g.O + o] = ((s_sum[0] + s_sum[1]) + s_sum[2]) + s_sum[3];
 }
 
 // dW for few weights under many windows (the first layers of an image network: 64 x 147 or 64 x 576 weights, 10^5
@@ -363,10 +596,16 @@ unsigned blocks_for(int64_t n) {
 
 } // namespace
 
+// What the gather kernel's 32-bit arithmetic and its tables in LDS hold.
+static bool conv_direct_gather_fits(const ConvGeom &g) {
+  return g.k_size <= 128 && g.C <= 0x7fffffff && g.O <= 0x7fffffff && g.outer <= 0x7fffffff &&
+         g.in_sp_size < ((int64_t)1 << 30) && g.out_sp_size < ((int64_t)1 << 30);
+}
+
 // Groups too small to pay for the general path's launches: its cost is about 25 us of launches per group forward (85
 // backward) plus the product at matrix-core rates; this path's, the product at about 10 TFLOP/s of vector fp32.
 bool conv_direct_applies(const ConvGeom &g) {
-  if (g.group < 2 || g.O * g.Kg > 0x7fffffffll)
+  if (g.group < 2 || g.O * g.Kg > 0x7fffffffll || !conv_direct_gather_fits(g)) // (the backward has no other form here)
     return false;
   const double flops = 2.0 * (double)g.M * (double)g.Kg * (double)g.O;
   return flops / 1e7 < 25.0 * (double)g.group + flops / 1e8;
@@ -420,6 +659,44 @@ int launch_conv_direct_binarize(const float *W, float *Wb, float *alpha, const C
   return NBLA_HIP_OK;
 }
 
+int launch_conv_direct_gather(bool forward, const float *src, const float *w, const float *scale, const float *bias,
+                              float *dst, const ConvGeom &g, bool accum, bool take_sign, float zero_to,
+                              hipStream_t stream) {
+  const int64_t positions = forward ? g.out_sp_size : g.in_sp_size, channels = forward ? g.O : g.C,
+                sources = forward ? g.Cg : g.Og;
+  int threads = positions <= 64 ? 64 : positions <= 128 ? 128 : kDirectBlock; // small channels
+  while (threads > 64 && g.k_size * threads > 8192) // the taps' table: 32 KB of LDS at most
+    threads /= 2;
+  // the weights that meet one channel of the result, `held` source channels at a time: 32 KB more at most
+  const int held = (int)(sources * g.k_size <= 8192 ? sources : 8192 / g.k_size);
+  // a block keeps its positions and walks (sample, channel) pairs: about 2048 blocks, the tables used several times
+  const int64_t tiles = ceil_div(positions, (int64_t)threads);
+  int64_t cw = ceil_div((int64_t)2048, tiles);
+  if (cw > channels)
+    cw = channels;
+  if (cw > 65535)
+    cw = 65535;
+  int64_t nw = ceil_div((int64_t)2048, tiles * cw);
+  if (nw > g.outer)
+    nw = g.outer;
+  if (nw > 65535)
+    nw = 65535;
+  const dim3 grid((unsigned)tiles, (unsigned)cw, (unsigned)nw);
+  const size_t lds = ((size_t)g.k_size * threads + (size_t)held * g.k_size) * sizeof(uint32_t);
+#define NBLA_CONV_DIRECT_GATHER(kForward, kUnit)                                                                        \
+  hipLaunchKernelGGL((conv_direct_gather<kForward, kUnit>), grid, dim3(threads), lds, stream, src, w, scale, bias, dst, \
+                     g, held, accum ? 1 : 0, take_sign ? 1 : 0, zero_to)
+  if (forward)
+    NBLA_CONV_DIRECT_GATHER(true, true);
+  else if (g.stride[0] == 1 && g.stride[1] == 1 && g.stride[2] == 1)
+    NBLA_CONV_DIRECT_GATHER(false, true);
+  else
+    NBLA_CONV_DIRECT_GATHER(false, false);
+#undef NBLA_CONV_DIRECT_GATHER
+  NBLA_HIP_LAUNCH_CHECK("conv_direct_gather");
+  return NBLA_HIP_OK;
+}
+
 int launch_conv_direct_forward(const float *x, const float *w, const float *scale, const float *bias, float *y,
                                const ConvGeom &g, hipStream_t stream) {
   // (65535: the second grid extent; the tile's weights have to fit the LDS the kernel may use without asking)
@@ -431,6 +708,8 @@ int launch_conv_direct_forward(const float *x, const float *w, const float *scal
     const dim3 grid((unsigned)ceil_div(g.out_sp_size, kDirectBlock), (unsigned)(g.outer * (g.O / 8)));
     hipLaunchKernelGGL(conv_direct_forward_tile<8>, grid, dim3(kDirectBlock), (size_t)g.Kg * 8 * sizeof(float), stream,
                        x, w, scale, bias, y, g);
+  } else if (conv_direct_gather_fits(g)) {
+    return launch_conv_direct_gather(true, x, w, scale, bias, y, g, false, false, 0.0f, stream);
   } else {
     hipLaunchKernelGGL(conv_direct_forward, dim3(blocks_for(g.outer * g.O * g.out_sp_size)), dim3(kDirectBlock), 0,
                        stream, x, w, scale, bias, y, g);
@@ -441,20 +720,86 @@ int launch_conv_direct_forward(const float *x, const float *w, const float *scal
 
 int launch_conv_direct_backward(const float *dy, const float *x, const float *w, const float *scale, float *dx,
                                 float *dW, float *db, const ConvGeom &g, bool accum_x, bool accum_w, bool accum_b,
-                                bool take_sign, float zero_to, hipStream_t stream) {
+                                bool take_sign, float zero_to, float *scratch, size_t scratch_bytes,
+                                hipStream_t stream) {
   if (dx) {
-    hipLaunchKernelGGL(conv_direct_dx, dim3(blocks_for(g.outer * g.C * g.in_sp_size)), dim3(kDirectBlock), 0, stream, dy,
-                       w, scale, dx, g, accum_x ? 1 : 0, take_sign ? 1 : 0, zero_to);
-    NBLA_HIP_LAUNCH_CHECK("conv_direct_dx");
+    if (!conv_direct_gather_fits(g))
+      return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "convolution backward: more than 128 taps, 2^31 channels or samples, "
+                                                "or 2^30 positions per channel, in the direct form.");
+    const int rc = launch_conv_direct_gather(false, dy, w, scale, nullptr, dx, g, accum_x, take_sign, zero_to, stream);
+    if (rc)
+      return rc;
   }
+  // Runs of the windows over blocks, partial sums in the scratch memory added in a fixed order: enough blocks for the
+  // chip whatever the number of channels, runs of at least 1024 windows.
+  const int64_t floats = (int64_t)(scratch_bytes / sizeof(float));
+  const auto chunks_for = [&](int64_t rows, int64_t per_chunk) {
+    int64_t c = ceil_div((int64_t)4096, rows);
+    if (c > g.M / 1024)
+      c = g.M / 1024;
+    if (c > floats / per_chunk)
+      c = floats / per_chunk;
+    if (c > 65535)
+      c = 65535;
+    return (int)c;
+  };
   if (dW) {
-    hipLaunchKernelGGL(conv_direct_dw, dim3((unsigned)(g.O * g.Kg)), dim3(kDirectBlock), 0, stream, dy, x, dW, g,
-                       accum_w ? 1 : 0);
-    NBLA_HIP_LAUNCH_CHECK("conv_direct_dw");
+    const int64_t count = g.O * g.Kg, L = g.out_sp_size;
+    // positions per tile: the multiple of 64 that holds them all, 256 at most; the samples share the rest of the block
+    const int lanes_p = L > 128 ? 256 : L > 64 ? 128 : 64;
+    const int64_t tiles = ceil_div(L, (int64_t)lanes_p);
+    const int kO = g.k_size <= 9 && g.Og % 4 == 0 ? 4 : g.k_size <= 16 && g.Og % 2 == 0 ? 2 : 1;
+    const int64_t pairs = g.O / kO * g.Cg;
+    // runs of the samples: enough blocks for the chip, each thread with a few samples at least
+    int64_t runs = ceil_div((int64_t)4096, pairs * tiles);
+    const int64_t steps = ceil_div(g.outer, (int64_t)(kDirectBlock / lanes_p));
+    if (runs > steps / 4)
+      runs = steps / 4;
+    if (runs < 1)
+      runs = 1;
+    if (runs > g.outer)
+      runs = g.outer;
+    const bool fits = scratch && g.k_size <= 32 && tiles * runs * count <= floats && pairs <= 0x7fffffff &&
+                      tiles <= 65535 && runs <= 65535 && g.in_sp_size < ((int64_t)1 << 30);
+    if (fits) {
+      const dim3 grid((unsigned)pairs, (unsigned)tiles, (unsigned)runs);
+      if (kO == 4)
+        hipLaunchKernelGGL((conv_direct_dw_pairs<4, 9>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g, lanes_p,
+                           (int)runs);
+      else if (kO == 2)
+        hipLaunchKernelGGL((conv_direct_dw_pairs<2, 16>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g,
+                           lanes_p, (int)runs);
+      else if (g.k_size <= 9)
+        hipLaunchKernelGGL((conv_direct_dw_pairs<1, 9>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g, lanes_p,
+                           (int)runs);
+      else
+        hipLaunchKernelGGL((conv_direct_dw_pairs<1, 32>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g,
+                           lanes_p, (int)runs);
+      NBLA_HIP_LAUNCH_CHECK("conv_direct_dw_pairs");
+      hipLaunchKernelGGL(conv_direct_dw_final, dim3((unsigned)ceil_div(count, kDirectBlock)), dim3(kDirectBlock), 0,
+                         stream, scratch, (int)(tiles * runs), dW, count, accum_w ? 1 : 0);
+      NBLA_HIP_LAUNCH_CHECK("conv_direct_dw_final");
+    } else {
+      hipLaunchKernelGGL(conv_direct_dw, dim3((unsigned)count), dim3(kDirectBlock), 0, stream, dy, x, dW, g,
+                         accum_w ? 1 : 0);
+      NBLA_HIP_LAUNCH_CHECK("conv_direct_dw");
+    }
   }
   if (db) {
-    hipLaunchKernelGGL(conv_direct_db, dim3((unsigned)g.O), dim3(kDirectBlock), 0, stream, dy, db, g, accum_b ? 1 : 0);
-    NBLA_HIP_LAUNCH_CHECK("conv_direct_db");
+    // (after dW's final sum in the stream, so the scratch memory is free again)
+    const int chunks = scratch ? chunks_for(g.O, g.O) : 0;
+    if (chunks >= 2) {
+      hipLaunchKernelGGL(conv_direct_db_chunks, dim3((unsigned)g.O, (unsigned)chunks), dim3(kDirectBlock), 0, stream, dy,
+                         scratch, g, chunks);
+      NBLA_HIP_LAUNCH_CHECK("conv_direct_db_chunks");
+      hipLaunchKernelGGL(conv_direct_dw_final, dim3((unsigned)ceil_div(g.O, kDirectBlock)), dim3(kDirectBlock), 0,
+                         stream, scratch, chunks, db, g.O, accum_b ? 1 : 0);
+      NBLA_HIP_LAUNCH_CHECK("conv_direct_dw_final");
+    } else {
+      hipLaunchKernelGGL(conv_direct_db, dim3((unsigned)g.O), dim3(kDirectBlock), 0, stream, dy, db, g,
+                         accum_b ? 1 : 0);
+      NBLA_HIP_LAUNCH_CHECK("conv_direct_db");
+    }
   }
   return NBLA_HIP_OK;
 }

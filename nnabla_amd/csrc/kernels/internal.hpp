@@ -58,7 +58,8 @@ int launch_conv_direct_forward(const float *x, const float *w, const float *scal
                                const ConvGeom &g, hipStream_t stream);
 int launch_conv_direct_backward(const float *dy, const float *x, const float *w, const float *scale, float *dx,
                                 float *dW, float *db, const ConvGeom &g, bool accum_x, bool accum_w, bool accum_b,
-                                bool take_sign, float zero_to, hipStream_t stream);
+                                bool take_sign, float zero_to, float *scratch, size_t scratch_bytes,
+                                hipStream_t stream);
 // The binary convolution forward with the unfold done by LDS addressing (conv_slab.hip), two launches per group:
 // launch_conv_slab_prepare reads the group's weights [Og, Cg, taps] once and writes Wb = Sign(W) (may be null) and,
 // into `prepared` (conv_slab_prepared_bytes, 16-byte aligned), the packed bits in (tap, channel) order with the

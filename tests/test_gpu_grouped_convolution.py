@@ -23,6 +23,8 @@ CASES = [
     ((3, 20, 40), (20, 1, 5), (2,), (1,), (1,), 20),                        # one spatial dimension
     ((2, 12, 5, 6, 7), (12, 2, 2, 3, 2), (1, 1, 0), (1, 2, 1), (1, 1, 2), 6),  # three
     ((2, 16, 7, 7), (16, 1, 7, 7), (3, 3), (1, 1), (1, 1), 16),            # a kernel as large as the input
+    ((16, 8, 12, 12), (8, 1, 5, 5), (2, 2), (1, 1), (1, 1), 8),            # 25 taps; the samples in several runs
+    ((40, 16, 6, 6), (32, 4, 3, 3), (1, 1), (1, 1), (1, 1), 4),            # few positions: samples side by side
     # one group of very few input channels under a kernel of many taps (the first layer of an image network): the
     # forward takes the same kernels, eight output channels per thread; the backward the general path
     ((2, 3, 40, 36), (16, 3, 7, 7), (3, 3), (2, 2), (1, 1), 1),
