@@ -6,7 +6,7 @@
 //   dyt [M, Og]          the output gradient of the group, transposed so that m is the row index
 //   colg[n][kk][l]       = sum over o of dyt[m, o] * w[o, kk]   (then folded into dx by a gather)
 //   dW  [Og, Kg]         = dyt^T . col(x)                        (col(x) [M, Kg] is the unfolded input; digit x digit)
-//   db  [Og]             = column sums of dyt
+//   db  [O]              = sums of dy over samples and positions, straight from dy
 #include "common.hpp"
 #include "conv_geom.hpp"
 #include "gemm_layout.hpp"
@@ -253,10 +253,18 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
       return rc;
     dW = nullptr;
   }
+  // the bias gradient straight from dy, every group at once (partial sums in the same buffer, after the weight
+  // gradient's in the stream)
+  if (db) {
+    rc = launch_conv_direct_db(dy, db, g, accum_b, col, (size_t)g.M * g.Kg * sizeof(float), stream);
+    if (rc)
+      return rc;
+    db = nullptr;
+  }
   for (int64_t grp = 0; grp < g.group; ++grp) {
     const float *Wg = W + grp * g.Og * g.Kg;
     const float *ag = alpha ? alpha + grp * g.Og : nullptr;
-    if (!dx_slab || dW || db) {
+    if (!dx_slab || dW) {
       rc = launch_gather_dy(dy, nullptr, dyt, g, grp, stream);
       if (rc)
         return rc;
@@ -323,11 +331,6 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
       // the buffer of the unfolded gradient is free here: it takes the partial results of a split contraction
       rc = launch_gemm_digits(base + p.a_planes_off, base + p.b_planes_off, nullptr, dW + grp * g.Og * g.Kg, g.Og, g.M,
                               g.Kg, 1, g.Kg, 1, stream, accum_w, col, (size_t)g.M * g.Kg * sizeof(float));
-      if (rc)
-        return rc;
-    }
-    if (db) {
-      rc = launch_column_sums(dyt, db + grp * g.Og, g.M, g.Og, accum_b, base + p.sums_off, stream);
       if (rc)
         return rc;
     }

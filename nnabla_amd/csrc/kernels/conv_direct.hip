@@ -68,13 +68,16 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_forward(const float 
 // LDS once per block, so a tap's kOut weights are kOut / 4 broadcast reads of 16 bytes, and every input value loaded
 // serves kOut products; the loads of four taps along the innermost kernel axis are issued together.
 constexpr int kDirectLdsFloats = 12288; // 48 KiB of weights per block
-template <int kOut>
+// kDrop: a tap outside the input contributes nothing (it reads a row of zero weights) instead of 0 * weight: the
+// form in which the kernel computes an input gradient (see launch_conv_direct_backward), where the reference never
+// forms those products.  accum: the result is added to y.
+template <int kOut, bool kDrop>
 __global__ __launch_bounds__(kDirectBlock) void conv_direct_forward_tile(const float *__restrict__ x,
                                                                          const float *__restrict__ w,
                                                                          const float *__restrict__ scale,
                                                                          const float *__restrict__ bias,
-                                                                         float *__restrict__ y, ConvGeom g) {
-  extern __shared__ __attribute__((aligned(16))) float s_w[]; // [Kg][kOut]
+                                                                         float *__restrict__ y, ConvGeom g, int accum) {
+  extern __shared__ __attribute__((aligned(16))) float s_w[]; // [Kg (+ 1 row of zeros)][kOut]
   typedef float float4_d __attribute__((ext_vector_type(4)));
   const int64_t otiles = g.O / kOut;
   const int64_t n = blockIdx.y / otiles, o0 = (blockIdx.y - n * otiles) * kOut, grp = o0 / g.Og;
@@ -84,6 +87,8 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_forward_tile(const f
     const float wv = w[(o0 + j) * g.Kg + k];
     s_w[k * kOut + j] = scale ? wv * scale[o0 + j] : wv; // Ws = Wb * alpha, rounded once as the reference forms it
   }
+  if (kDrop && threadIdx.x < kOut)
+    s_w[Kg * kOut + threadIdx.x] = 0.0f;
   __syncthreads();
   const int64_t p = (int64_t)blockIdx.x * kDirectBlock + threadIdx.x;
   const bool live = p < g.out_sp_size;
@@ -104,15 +109,18 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_forward_tile(const f
         const float *xr = xc + ((int64_t)i0 * g.in_sp[1] + i1) * g.in_sp[2];
         for (int k2 = 0; k2 < g.k[2]; k2 += 4) {
           float xv[4];
+          bool in[4];
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
             const int i2 = b2 + (k2 + u) * g.dil[2];
-            xv[u] = (row_in && k2 + u < g.k[2] && (unsigned)i2 < (unsigned)g.in_sp[2]) ? xr[i2] : 0.0f;
+            in[u] = row_in && k2 + u < g.k[2] && (unsigned)i2 < (unsigned)g.in_sp[2];
+            xv[u] = in[u] ? xr[i2] : 0.0f;
           }
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
             if (k2 + u < g.k[2]) { // uniform
-              const float4_d *wk = reinterpret_cast<const float4_d *>(s_w + (t + u) * kOut);
+              const float4_d *wk =
+                  reinterpret_cast<const float4_d *>(s_w + (kDrop && !in[u] ? Kg : t + u) * kOut);
 #pragma unroll
               for (int j4 = 0; j4 < kOut / 4; ++j4) {
                 const float4_d wv = wk[j4];
@@ -130,26 +138,52 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_forward_tile(const f
   if (live) {
 #pragma unroll
     for (int j = 0; j < kOut; ++j)
-      y[(n * g.O + o0 + j) * g.out_sp_size + p] = bias ? acc[j] + bias[o0 + j] : acc[j];
+    {
+      float *out = y + (n * g.O + o0 + j) * g.out_sp_size + p;
+      const float v = bias ? acc[j] + bias[o0 + j] : acc[j];
+      *out = accum ? *out + v : v;
+    }
   }
+}
+
+// The weights of the convolution that computes an input gradient of unit stride: channels' roles exchanged within
+// each group, taps reversed, signs taken and alpha folded in:
+//   wt[grp * Cg + c][o * taps + (taps - 1 - t)] = f(w[grp * Og + o][c * taps + t])
+__global__ __launch_bounds__(kDirectBlock) void conv_direct_transpose_weights(const float *__restrict__ w,
+                                                                              const float *__restrict__ scale,
+                                                                              float *__restrict__ wt, int64_t count,
+                                                                              int Og, int Cg, int taps, int take_sign,
+                                                                              float zero_to) {
+  const int64_t i = (int64_t)blockIdx.x * kDirectBlock + threadIdx.x;
+  if (i >= count)
+    return;
+  const int t = (int)(i % taps);
+  const int64_t oc = i / taps, c = oc % Cg, og = oc / Cg, grp = og / Og, o = og - grp * Og; // og: channel out, global
+  float wv = w[i];
+  if (take_sign)
+    wv = (wv > 0.0f) ? 1.0f : ((wv < 0.0f) ? -1.0f : zero_to);
+  if (scale)
+    wv = wv * scale[og];
+  wt[((grp * Cg + c) * Og + o) * taps + (taps - 1 - t)] = wv;
 }
 
 // One batch of taps of one element of the result: rows the sample's source at the first of kOB channels (the next ones
 // L floats further, as many as `channels`), sw those channels' weights in LDS ([channel][taps], this batch's first tap),
 // reach/ok where the taps land (byte offsets into a channel of the source).  The loads of a batch are all in flight together;
-// taps outside the output load a valid address and are left out of the sum.  kFull: all kTapBatch taps exist.
+// taps outside the output load a valid address and are left out of the sum.  kB: taps per batch (the first kB entries
+// of reach / ok); kFull: all kB taps exist.
 constexpr int kTapBatch = 9;
 constexpr uint32_t kNoReach = 0xffffffffu;
-template <int kOB, bool kFull, bool kForward>
+template <int kOB, int kB, bool kFull, bool kForward>
 __device__ __forceinline__ float conv_direct_gather_batch(const float *__restrict__ rows, int64_t L, const float *sw, int taps,
                                                       int channels, int count, const uint32_t (&reach)[kTapBatch],
                                                       const bool (&ok)[kTapBatch], float acc) {
-  float gy[kOB][kTapBatch];
+  float gy[kOB][kB];
 #pragma unroll
   for (int jo = 0; jo < kOB; ++jo) {
     const char *row = reinterpret_cast<const char *>(rows + (jo < channels ? jo : channels - 1) * L);
 #pragma unroll
-    for (int j = 0; j < kTapBatch; ++j)
+    for (int j = 0; j < kB; ++j)
       gy[jo][j] = *reinterpret_cast<const float *>(row + reach[j]);
   }
 #pragma unroll
@@ -157,7 +191,7 @@ __device__ __forceinline__ float conv_direct_gather_batch(const float *__restric
     const bool live = jo < channels;
     const float *wr = sw + (live ? jo : channels - 1) * taps;
 #pragma unroll
-    for (int j = 0; j < kTapBatch; ++j) {
+    for (int j = 0; j < kB; ++j) {
       const float wv = wr[kFull || j < count ? j : 0];
       if (kForward) // a tap in the padding is a zero that is multiplied
         acc = acc + (live ? (ok[j] ? gy[jo][j] : 0.0f) * wv : 0.0f);
@@ -181,8 +215,8 @@ __device__ __forceinline__ float conv_direct_gather_batch(const float *__restric
 // registers when the kernel has at most kTapBatch taps).  The weights that meet one channel of the result, `held`
 // source channels at a time, signs taken and scaled, sit in LDS too; the samples' loop runs inside, so they are
 // prepared once per channel.  32-bit arithmetic per lane: a block-uniform row pointer plus a byte offset.
-// kUnit (backward): unit strides, no divisibility to test.
-template <bool kForward, bool kUnit>
+// kUnit (backward): unit strides, no divisibility to test; kClasses (backward, strides): see below.
+template <bool kForward, bool kUnit, bool kClasses>
 __global__ __launch_bounds__(kDirectBlock) void conv_direct_gather(const float *__restrict__ src,
                                                                    const float *__restrict__ w,
                                                                    const float *__restrict__ scale,
@@ -191,19 +225,39 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_gather(const float *
                                                                    int accum, int take_sign, float zero_to) {
   constexpr int kOB = 1; // (more source channels per step gave nothing)
   extern __shared__ uint32_t s_gather[];
-  const int taps = (int)g.k_size, threads = (int)blockDim.x, tid = (int)threadIdx.x;
-  uint32_t *s_reach = s_gather;                                          // [taps][threads]: byte offset, or kNoReach
-  float *s_w = reinterpret_cast<float *>(s_gather + (size_t)taps * threads); // [held][taps]
-  const int pos = (int)(blockIdx.x * blockDim.x) + tid;
+  const int all_taps = (int)g.k_size, threads = (int)blockDim.x, tid = (int)threadIdx.x;
+  uint32_t *s_reach = s_gather;                                              // [taps][threads]: byte offset, or kNoReach
+  float *s_w = reinterpret_cast<float *>(s_gather + (size_t)all_taps * threads); // [held][taps]
+  int *s_tap = reinterpret_cast<int *>(s_w + (size_t)held * all_taps);        // [taps]: which taps the block uses
   const int64_t positions = kForward ? g.out_sp_size : g.in_sp_size, L = kForward ? g.in_sp_size : g.out_sp_size;
-  const bool live = pos < positions;
-  {
-    const int in0 = (int)g.in_sp[0], in1 = (int)g.in_sp[1], in2 = (int)g.in_sp[2], out0 = (int)g.out_sp[0],
-              out1 = (int)g.out_sp[1], out2 = (int)g.out_sp[2];
+  const int in0 = (int)g.in_sp[0], in1 = (int)g.in_sp[1], in2 = (int)g.in_sp[2], out0 = (int)g.out_sp[0],
+            out1 = (int)g.out_sp[1], out2 = (int)g.out_sp[2];
+  const int s0 = (int)g.stride[0], s1 = (int)g.stride[1], s2 = (int)g.stride[2];
+  int pos, q0, q1, q2, r0 = 0, r1 = 0, r2 = 0, taps = all_taps;
+  bool live;
+  if (!kClasses) {
+    pos = (int)(blockIdx.x * blockDim.x) + tid;
+    live = pos < positions;
     const int d1 = kForward ? out1 : in1, d2 = kForward ? out2 : in2;
-    const int q2 = pos % d2, r = pos / d2, q1 = r % d1, q0 = r / d1;
-    const int s0 = (int)g.stride[0], s1 = (int)g.stride[1], s2 = (int)g.stride[2];
-    int t = 0;
+    const int r = pos / d2;
+    q2 = pos % d2, q1 = r % d1, q0 = r / d1;
+  } else {
+    // A strided convolution reaches an input position only through the taps that match the position's remainders
+    // modulo the strides.  A block takes positions of one class of remainders (r0, r1, r2), so that all its threads
+    // use the same taps, and keeps only those: 1/(s0 s1 s2) of the kernel on average.
+    const int tiles = (int)gridDim.x / (s0 * s1 * s2), cls = (int)blockIdx.x / tiles, tile = (int)blockIdx.x - cls * tiles;
+    r2 = cls % s2, r1 = (cls / s2) % s1, r0 = cls / (s2 * s1);
+    const int u0n = in0 > r0 ? (in0 - r0 + s0 - 1) / s0 : 0, u1n = in1 > r1 ? (in1 - r1 + s1 - 1) / s1 : 0,
+              u2n = in2 > r2 ? (in2 - r2 + s2 - 1) / s2 : 0;
+    const int li = tile * threads + tid;
+    live = li < u0n * u1n * u2n;
+    const int v = li / (u2n > 0 ? u2n : 1);
+    q2 = r2 + s2 * (li - v * (u2n > 0 ? u2n : 1));
+    q1 = r1 + s1 * (v % (u1n > 0 ? u1n : 1)), q0 = r0 + s0 * (v / (u1n > 0 ? u1n : 1));
+    pos = (q0 * in1 + q1) * in2 + q2;
+  }
+  {
+    int t = 0, used = 0;
     for (int k0 = 0; k0 < (int)g.k[0]; ++k0)
       for (int k1 = 0; k1 < (int)g.k[1]; ++k1)
         for (int k2 = 0; k2 < (int)g.k[2]; ++k2, ++t) {
@@ -217,16 +271,27 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_gather(const float *
             const int e0 = q0 + (int)g.pad[0] - k0 * (int)g.dil[0], e1 = q1 + (int)g.pad[1] - k1 * (int)g.dil[1],
                       e2 = q2 + (int)g.pad[2] - k2 * (int)g.dil[2];
             int p0 = e0, p1 = e1, p2 = e2;
-            bool ok = live;
-            if (!kUnit) {
-              ok = ok && e0 >= 0 && e1 >= 0 && e2 >= 0 && e0 % s0 == 0 && e1 % s1 == 0 && e2 % s2 == 0;
+            if (kClasses) {
+              // (the same for every thread of the block: the remainders decide)
+              if ((r0 + (int)g.pad[0] - k0 * (int)g.dil[0]) % s0 != 0 || (r1 + (int)g.pad[1] - k1 * (int)g.dil[1]) % s1 != 0 ||
+                  (r2 + (int)g.pad[2] - k2 * (int)g.dil[2]) % s2 != 0)
+                continue;
+              p0 = e0 / s0, p1 = e1 / s1, p2 = e2 / s2; // (exact; negative stays negative)
+              if (tid == 0)
+                s_tap[used] = t;
+            }
+            bool fine = live;
+            if (!kUnit && !kClasses) { // strides, every thread for itself
+              fine = fine && e0 >= 0 && e1 >= 0 && e2 >= 0 && e0 % s0 == 0 && e1 % s1 == 0 && e2 % s2 == 0;
               p0 = e0 / s0, p1 = e1 / s1, p2 = e2 / s2;
             }
-            if (ok && (unsigned)p0 < (unsigned)out0 && (unsigned)p1 < (unsigned)out1 && (unsigned)p2 < (unsigned)out2)
+            if (fine && (unsigned)p0 < (unsigned)out0 && (unsigned)p1 < (unsigned)out1 && (unsigned)p2 < (unsigned)out2)
               at = (uint32_t)((p0 * out1 + p1) * out2 + p2) * 4u;
           }
-          s_reach[t * threads + tid] = at;
+          s_reach[used * threads + tid] = at;
+          ++used;
         }
+    taps = used;
   }
   // (each thread reads back only what it wrote: no barrier for this table)
   uint32_t reach[kTapBatch];
@@ -252,9 +317,9 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_gather(const float *
       const int no = sources - o0 < held ? sources - o0 : held;
       __syncthreads(); // the previous weights are done with
       for (int i = tid; i < no * taps; i += threads) {
-        const int o = i / taps, t = i - o * taps;
+        const int o = i / taps, t = i - o * taps, tap = kClasses ? s_tap[t] : t;
         const int64_t row = kForward ? c : (int64_t)grp * Og + o0 + o; // the weights' channel out
-        float wv = kForward ? w[row * Kg + (int64_t)(o0 + o) * taps + t] : w[row * Kg + cl * taps + t];
+        float wv = kForward ? w[row * Kg + (int64_t)(o0 + o) * all_taps + tap] : w[row * Kg + cl * all_taps + tap];
         if (take_sign)
           wv = (wv > 0.0f) ? 1.0f : ((wv < 0.0f) ? -1.0f : zero_to);
         s_w[i] = scale ? wv * scale[row] : wv;
@@ -268,18 +333,31 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_gather(const float *
         if (few) {
           if (taps == kTapBatch)
             for (int o = 0; o < no; o += kOB)
-              acc = conv_direct_gather_batch<kOB, true, kForward>(rows + o * L, L, s_w + o * taps, taps, no - o, taps,
-                                                                  reach, ok, acc);
+              acc = conv_direct_gather_batch<kOB, kTapBatch, true, kForward>(rows + o * L, L, s_w + o * taps, taps,
+                                                                             no - o, taps, reach, ok, acc);
+          else if (taps <= 4 && no >= 4) { // (the classes of a strided input gradient, short kernels: few taps of
+            if (taps <= 2)                 // four source channels at a time, so that as many loads are in flight)
+              for (int o = 0; o < no; o += 4)
+                acc = conv_direct_gather_batch<4, 2, false, kForward>(rows + o * L, L, s_w + o * taps, taps, no - o, taps,
+                                                                      reach, ok, acc);
+            else
+              for (int o = 0; o < no; o += 4)
+                acc = conv_direct_gather_batch<4, 4, false, kForward>(rows + o * L, L, s_w + o * taps, taps, no - o, taps,
+                                                                      reach, ok, acc);
+          } else if (taps <= 4)
+            for (int o = 0; o < no; o += kOB)
+              acc = conv_direct_gather_batch<kOB, 4, false, kForward>(rows + o * L, L, s_w + o * taps, taps, no - o, taps,
+                                                                      reach, ok, acc);
           else
             for (int o = 0; o < no; o += kOB)
-              acc = conv_direct_gather_batch<kOB, false, kForward>(rows + o * L, L, s_w + o * taps, taps, no - o, taps,
-                                                                   reach, ok, acc);
+              acc = conv_direct_gather_batch<kOB, kTapBatch, false, kForward>(rows + o * L, L, s_w + o * taps, taps,
+                                                                              no - o, taps, reach, ok, acc);
         } else {
           for (int t0 = 0; t0 < taps; t0 += kTapBatch) {
             fetch(t0);
             for (int o = 0; o < no; o += kOB)
-              acc = conv_direct_gather_batch<kOB, false, kForward>(rows + o * L, L, s_w + o * taps + t0, taps, no - o,
-                                                                   taps - t0, reach, ok, acc);
+              acc = conv_direct_gather_batch<kOB, kTapBatch, false, kForward>(rows + o * L, L, s_w + o * taps + t0, taps,
+                                                                              no - o, taps - t0, reach, ok, acc);
           }
         }
         float *out = dst + ((int64_t)n * channels + c) * positions + pos;
@@ -336,12 +414,14 @@ template <int kO, int kTaps>
 __global__ __launch_bounds__(kDirectBlock) void conv_direct_dw_pairs(const float *__restrict__ dy,
                                                                      const float *__restrict__ x,
                                                                      float *__restrict__ partial, ConvGeom g,
-                                                                     int lanes_p, int runs) {
+                                                                     int lanes_p, int runs, int tap_groups) {
   __shared__ int s_off[kTaps][4];
   __shared__ float s_sum[kDirectBlock / 64][kO * kTaps];
-  const int taps = (int)g.k_size, tid = threadIdx.x;
+  // (kernels of more taps than the template holds: the taps in groups of kTaps, a block per group)
+  const int tap0 = (int)(blockIdx.x % tap_groups) * kTaps, tid = threadIdx.x;
+  const int taps = (int)g.k_size - tap0 < kTaps ? (int)g.k_size - tap0 : kTaps;
   if (tid < taps) {
-    int t = tid;
+    int t = tap0 + tid;
     const int k2 = t % g.k[2];
     t /= g.k[2];
     const int d0 = (t / g.k[1]) * g.dil[0], d1 = (t % g.k[1]) * g.dil[1], d2 = k2 * g.dil[2];
@@ -350,7 +430,7 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_dw_pairs(const float
   }
   __syncthreads();
   const int64_t og = g.Og / kO; // blocks of channels out per group
-  const int64_t pair = blockIdx.x, ob = pair / g.Cg, c = pair - ob * g.Cg, grp = ob / og, o = grp * g.Og + (ob - grp * og) * kO;
+  const int64_t pair = blockIdx.x / tap_groups, ob = pair / g.Cg, c = pair - ob * g.Cg, grp = ob / og, o = grp * g.Og + (ob - grp * og) * kO;
   const int sub = tid / lanes_p, nsub = kDirectBlock / lanes_p;
   const int64_t p = (int64_t)blockIdx.y * lanes_p + (tid - sub * lanes_p);
   const int64_t per = ceil_div(g.outer, (int64_t)runs), n0 = (int64_t)blockIdx.z * per,
@@ -419,7 +499,7 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_dw_pairs(const float
       v += s_sum[w][tid];
     const int j = tid / kTaps, t = tid - j * kTaps;
     const int64_t chunk = (int64_t)blockIdx.y * runs + blockIdx.z;
-    partial[chunk * g.O * g.Kg + (o + j) * g.Kg + c * g.k_size + t] = v;
+    partial[chunk * g.O * g.Kg + (o + j) * g.Kg + c * g.k_size + tap0 + t] = v;
   }
 }
 // db likewise: block (o, chunk), partial results [chunk][O]
@@ -662,15 +742,25 @@ int launch_conv_direct_binarize(const float *W, float *Wb, float *alpha, const C
 int launch_conv_direct_gather(bool forward, const float *src, const float *w, const float *scale, const float *bias,
                               float *dst, const ConvGeom &g, bool accum, bool take_sign, float zero_to,
                               hipStream_t stream) {
-  const int64_t positions = forward ? g.out_sp_size : g.in_sp_size, channels = forward ? g.O : g.C,
-                sources = forward ? g.Cg : g.Og;
+  const bool unit = g.stride[0] == 1 && g.stride[1] == 1 && g.stride[2] == 1;
+  // (a strided input gradient: blocks per class of remainders modulo the strides, the largest class sizes the tiles)
+  // (with fewer than four source channels the saving does not pay for the smaller blocks and the strided stores)
+  const int64_t classes = forward || unit || g.Og < 4 ? 1 : (int64_t)g.stride[0] * g.stride[1] * g.stride[2];
+  int64_t positions = forward ? g.out_sp_size : g.in_sp_size;
+  if (classes > 1)
+    positions = ceil_div((int64_t)g.in_sp[0], (int64_t)g.stride[0]) * ceil_div((int64_t)g.in_sp[1], (int64_t)g.stride[1]) *
+                ceil_div((int64_t)g.in_sp[2], (int64_t)g.stride[2]);
+  const int64_t channels = forward ? g.O : g.C, sources = forward ? g.Cg : g.Og;
   int threads = positions <= 64 ? 64 : positions <= 128 ? 128 : kDirectBlock; // small channels
   while (threads > 64 && g.k_size * threads > 8192) // the taps' table: 32 KB of LDS at most
     threads /= 2;
-  // the weights that meet one channel of the result, `held` source channels at a time: 32 KB more at most
-  const int held = (int)(sources * g.k_size <= 8192 ? sources : 8192 / g.k_size);
+  // the weights that meet one channel of the result, `held` source channels at a time: 31 KB more at most (the list of
+  // the taps a class uses follows; 64 KB is what a kernel may use without asking)
+  const int held = (int)(sources * g.k_size <= 7936 ? sources : 7936 / g.k_size);
   // a block keeps its positions and walks (sample, channel) pairs: about 2048 blocks, the tables used several times
-  const int64_t tiles = ceil_div(positions, (int64_t)threads);
+  const int64_t tiles = ceil_div(positions, (int64_t)threads) * classes;
+  if (tiles > 0x7fffffff)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "convolution: too many tiles of positions for one launch.");
   int64_t cw = ceil_div((int64_t)2048, tiles);
   if (cw > channels)
     cw = channels;
@@ -682,32 +772,63 @@ int launch_conv_direct_gather(bool forward, const float *src, const float *w, co
   if (nw > 65535)
     nw = 65535;
   const dim3 grid((unsigned)tiles, (unsigned)cw, (unsigned)nw);
-  const size_t lds = ((size_t)g.k_size * threads + (size_t)held * g.k_size) * sizeof(uint32_t);
-#define NBLA_CONV_DIRECT_GATHER(kForward, kUnit)                                                                        \
-  hipLaunchKernelGGL((conv_direct_gather<kForward, kUnit>), grid, dim3(threads), lds, stream, src, w, scale, bias, dst, \
-                     g, held, accum ? 1 : 0, take_sign ? 1 : 0, zero_to)
+  const size_t lds = ((size_t)g.k_size * threads + (size_t)held * g.k_size + (size_t)g.k_size) * sizeof(uint32_t);
+#define NBLA_CONV_DIRECT_GATHER(kForward, kUnit, kClasses)                                                              \
+  hipLaunchKernelGGL((conv_direct_gather<kForward, kUnit, kClasses>), grid, dim3(threads), lds, stream, src, w, scale,  \
+                     bias, dst, g, held, accum ? 1 : 0, take_sign ? 1 : 0, zero_to)
   if (forward)
-    NBLA_CONV_DIRECT_GATHER(true, true);
-  else if (g.stride[0] == 1 && g.stride[1] == 1 && g.stride[2] == 1)
-    NBLA_CONV_DIRECT_GATHER(false, true);
+    NBLA_CONV_DIRECT_GATHER(true, true, false);
+  else if (unit)
+    NBLA_CONV_DIRECT_GATHER(false, true, false);
+  else if (classes > 1)
+    NBLA_CONV_DIRECT_GATHER(false, false, true);
   else
-    NBLA_CONV_DIRECT_GATHER(false, false);
+    NBLA_CONV_DIRECT_GATHER(false, false, false);
 #undef NBLA_CONV_DIRECT_GATHER
   NBLA_HIP_LAUNCH_CHECK("conv_direct_gather");
   return NBLA_HIP_OK;
 }
 
+// Output channels per thread of the tiled kernel, or 0 where it does not apply
+// (65535: the second grid extent; the tile's weights have to fit the LDS the kernel may use without asking)
+static int direct_tile_width(const ConvGeom &g) {
+  if (g.Og % 16 == 0 && g.out_sp_size >= 64 && g.outer * (g.O / 16) <= 65535 && g.Kg * 16 <= kDirectLdsFloats)
+    return 16;
+  if (g.Og % 8 == 0 && g.out_sp_size >= 64 && g.outer * (g.O / 8) <= 65535 && g.Kg * 8 <= kDirectLdsFloats)
+    return 8;
+  return 0;
+}
+
+// The geometry of the convolution that computes g's input gradient (unit strides): dy in the place of x, the
+// channels' roles exchanged, the padding that is left of the kernel's reach.
+static bool direct_transposed_geom(const ConvGeom &g, ConvGeom &t) {
+  t = g;
+  for (int i = 0; i < kMaxSpatial; ++i) {
+    if (g.stride[i] != 1)
+      return false;
+    t.pad[i] = (g.k[i] - 1) * g.dil[i] - g.pad[i];
+    if (t.pad[i] < 0)
+      return false;
+    t.in_sp[i] = g.out_sp[i], t.out_sp[i] = g.in_sp[i];
+  }
+  t.C = g.O, t.O = g.C, t.Cg = g.Og, t.Og = g.Cg;
+  t.in_sp_size = g.out_sp_size, t.out_sp_size = g.in_sp_size;
+  t.Kg = t.Cg * g.k_size;
+  t.M = g.outer * t.out_sp_size;
+  return true;
+}
+
 int launch_conv_direct_forward(const float *x, const float *w, const float *scale, const float *bias, float *y,
                                const ConvGeom &g, hipStream_t stream) {
-  // (65535: the second grid extent; the tile's weights have to fit the LDS the kernel may use without asking)
-  if (g.Og % 16 == 0 && g.out_sp_size >= 64 && g.outer * (g.O / 16) <= 65535 && g.Kg * 16 <= kDirectLdsFloats) {
+  const int width = direct_tile_width(g);
+  if (width == 16) {
     const dim3 grid((unsigned)ceil_div(g.out_sp_size, kDirectBlock), (unsigned)(g.outer * (g.O / 16)));
-    hipLaunchKernelGGL(conv_direct_forward_tile<16>, grid, dim3(kDirectBlock), (size_t)g.Kg * 16 * sizeof(float), stream,
-                       x, w, scale, bias, y, g);
-  } else if (g.Og % 8 == 0 && g.out_sp_size >= 64 && g.outer * (g.O / 8) <= 65535 && g.Kg * 8 <= kDirectLdsFloats) {
+    hipLaunchKernelGGL((conv_direct_forward_tile<16, false>), grid, dim3(kDirectBlock),
+                       (size_t)g.Kg * 16 * sizeof(float), stream, x, w, scale, bias, y, g, 0);
+  } else if (width == 8) {
     const dim3 grid((unsigned)ceil_div(g.out_sp_size, kDirectBlock), (unsigned)(g.outer * (g.O / 8)));
-    hipLaunchKernelGGL(conv_direct_forward_tile<8>, grid, dim3(kDirectBlock), (size_t)g.Kg * 8 * sizeof(float), stream,
-                       x, w, scale, bias, y, g);
+    hipLaunchKernelGGL((conv_direct_forward_tile<8, false>), grid, dim3(kDirectBlock), (size_t)g.Kg * 8 * sizeof(float),
+                       stream, x, w, scale, bias, y, g, 0);
   } else if (conv_direct_gather_fits(g)) {
     return launch_conv_direct_gather(true, x, w, scale, bias, y, g, false, false, 0.0f, stream);
   } else {
@@ -718,11 +839,61 @@ int launch_conv_direct_forward(const float *x, const float *w, const float *scal
   return NBLA_HIP_OK;
 }
 
+// db[o] (+)= sum over samples and positions of dy[n, o, p], every group at once, straight from dy: chunks of the
+// windows over blocks (partial sums in the scratch memory, added in a fixed order) where the channels alone would not
+// fill the chip.
+int launch_conv_direct_db(const float *dy, float *db, const ConvGeom &g, bool accum, float *scratch,
+                          size_t scratch_bytes, hipStream_t stream) {
+  int64_t chunks = ceil_div((int64_t)4096, g.O);
+  if (chunks > g.M / 1024)
+    chunks = g.M / 1024;
+  if (chunks > (int64_t)(scratch_bytes / sizeof(float)) / g.O)
+    chunks = (int64_t)(scratch_bytes / sizeof(float)) / g.O;
+  if (chunks > 65535)
+    chunks = 65535;
+  if (g.O > 0x7fffffff)
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "convolution backward: 2^31 channels or more.");
+  if (scratch && chunks >= 2) {
+    hipLaunchKernelGGL(conv_direct_db_chunks, dim3((unsigned)g.O, (unsigned)chunks), dim3(kDirectBlock), 0, stream, dy,
+                       scratch, g, (int)chunks);
+    NBLA_HIP_LAUNCH_CHECK("conv_direct_db_chunks");
+    hipLaunchKernelGGL(conv_direct_dw_final, dim3((unsigned)ceil_div(g.O, kDirectBlock)), dim3(kDirectBlock), 0, stream,
+                       scratch, (int)chunks, db, g.O, accum ? 1 : 0);
+    NBLA_HIP_LAUNCH_CHECK("conv_direct_dw_final");
+  } else {
+    hipLaunchKernelGGL(conv_direct_db, dim3((unsigned)g.O), dim3(kDirectBlock), 0, stream, dy, db, g, accum ? 1 : 0);
+    NBLA_HIP_LAUNCH_CHECK("conv_direct_db");
+  }
+  return NBLA_HIP_OK;
+}
+
 int launch_conv_direct_backward(const float *dy, const float *x, const float *w, const float *scale, float *dx,
                                 float *dW, float *db, const ConvGeom &g, bool accum_x, bool accum_w, bool accum_b,
                                 bool take_sign, float zero_to, float *scratch, size_t scratch_bytes,
                                 hipStream_t stream) {
-  if (dx) {
+  ConvGeom t;
+  const int width = dx && scratch && direct_transposed_geom(g, t) &&
+                            (size_t)(g.O * g.Kg) * sizeof(float) <= scratch_bytes
+                        ? direct_tile_width(t)
+                        : 0;
+  if (width) {
+    // channels to share: the input gradient as a convolution of dy with the transposed, reversed weights (in the
+    // scratch memory, which the weight gradient's partial sums take over afterwards)
+    const int64_t count = g.O * g.Kg;
+    hipLaunchKernelGGL(conv_direct_transpose_weights, dim3((unsigned)ceil_div(count, kDirectBlock)), dim3(kDirectBlock),
+                       0, stream, w, scale, scratch, count, (int)g.Og, (int)g.Cg, (int)g.k_size, take_sign ? 1 : 0,
+                       zero_to);
+    NBLA_HIP_LAUNCH_CHECK("conv_direct_transpose_weights");
+    const dim3 grid((unsigned)ceil_div(t.out_sp_size, kDirectBlock), (unsigned)(t.outer * (t.O / width)));
+    const size_t lds = (size_t)(t.Kg + 1) * width * sizeof(float);
+    if (width == 16)
+      hipLaunchKernelGGL((conv_direct_forward_tile<16, true>), grid, dim3(kDirectBlock), lds, stream, dy, scratch,
+                         nullptr, nullptr, dx, t, accum_x ? 1 : 0);
+    else
+      hipLaunchKernelGGL((conv_direct_forward_tile<8, true>), grid, dim3(kDirectBlock), lds, stream, dy, scratch,
+                         nullptr, nullptr, dx, t, accum_x ? 1 : 0);
+    NBLA_HIP_LAUNCH_CHECK("conv_direct_forward_tile");
+  } else if (dx) {
     if (!conv_direct_gather_fits(g))
       return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "convolution backward: more than 128 taps, 2^31 channels or samples, "
                                                 "or 2^30 positions per channel, in the direct form.");
@@ -730,19 +901,7 @@ int launch_conv_direct_backward(const float *dy, const float *x, const float *w,
     if (rc)
       return rc;
   }
-  // Runs of the windows over blocks, partial sums in the scratch memory added in a fixed order: enough blocks for the
-  // chip whatever the number of channels, runs of at least 1024 windows.
   const int64_t floats = (int64_t)(scratch_bytes / sizeof(float));
-  const auto chunks_for = [&](int64_t rows, int64_t per_chunk) {
-    int64_t c = ceil_div((int64_t)4096, rows);
-    if (c > g.M / 1024)
-      c = g.M / 1024;
-    if (c > floats / per_chunk)
-      c = floats / per_chunk;
-    if (c > 65535)
-      c = 65535;
-    return (int)c;
-  };
   if (dW) {
     const int64_t count = g.O * g.Kg, L = g.out_sp_size;
     // positions per tile: the multiple of 64 that holds them all, 256 at most; the samples share the rest of the block
@@ -759,22 +918,23 @@ int launch_conv_direct_backward(const float *dy, const float *x, const float *w,
       runs = 1;
     if (runs > g.outer)
       runs = g.outer;
-    const bool fits = scratch && g.k_size <= 32 && tiles * runs * count <= floats && pairs <= 0x7fffffff &&
+    const int tap_groups = kO == 1 ? (int)ceil_div(g.k_size, (int64_t)32) : 1;
+    const bool fits = scratch && tiles * runs * count <= floats && pairs * tap_groups <= 0x7fffffff &&
                       tiles <= 65535 && runs <= 65535 && g.in_sp_size < ((int64_t)1 << 30);
     if (fits) {
-      const dim3 grid((unsigned)pairs, (unsigned)tiles, (unsigned)runs);
+      const dim3 grid((unsigned)(pairs * tap_groups), (unsigned)tiles, (unsigned)runs);
       if (kO == 4)
         hipLaunchKernelGGL((conv_direct_dw_pairs<4, 9>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g, lanes_p,
-                           (int)runs);
+                           (int)runs, 1);
       else if (kO == 2)
         hipLaunchKernelGGL((conv_direct_dw_pairs<2, 16>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g,
-                           lanes_p, (int)runs);
+                           lanes_p, (int)runs, 1);
       else if (g.k_size <= 9)
         hipLaunchKernelGGL((conv_direct_dw_pairs<1, 9>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g, lanes_p,
-                           (int)runs);
+                           (int)runs, 1);
       else
         hipLaunchKernelGGL((conv_direct_dw_pairs<1, 32>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g,
-                           lanes_p, (int)runs);
+                           lanes_p, (int)runs, tap_groups);
       NBLA_HIP_LAUNCH_CHECK("conv_direct_dw_pairs");
       hipLaunchKernelGGL(conv_direct_dw_final, dim3((unsigned)ceil_div(count, kDirectBlock)), dim3(kDirectBlock), 0,
                          stream, scratch, (int)(tiles * runs), dW, count, accum_w ? 1 : 0);
@@ -785,22 +945,8 @@ int launch_conv_direct_backward(const float *dy, const float *x, const float *w,
       NBLA_HIP_LAUNCH_CHECK("conv_direct_dw");
     }
   }
-  if (db) {
-    // (after dW's final sum in the stream, so the scratch memory is free again)
-    const int chunks = scratch ? chunks_for(g.O, g.O) : 0;
-    if (chunks >= 2) {
-      hipLaunchKernelGGL(conv_direct_db_chunks, dim3((unsigned)g.O, (unsigned)chunks), dim3(kDirectBlock), 0, stream, dy,
-                         scratch, g, chunks);
-      NBLA_HIP_LAUNCH_CHECK("conv_direct_db_chunks");
-      hipLaunchKernelGGL(conv_direct_dw_final, dim3((unsigned)ceil_div(g.O, kDirectBlock)), dim3(kDirectBlock), 0,
-                         stream, scratch, chunks, db, g.O, accum_b ? 1 : 0);
-      NBLA_HIP_LAUNCH_CHECK("conv_direct_dw_final");
-    } else {
-      hipLaunchKernelGGL(conv_direct_db, dim3((unsigned)g.O), dim3(kDirectBlock), 0, stream, dy, db, g,
-                         accum_b ? 1 : 0);
-      NBLA_HIP_LAUNCH_CHECK("conv_direct_db");
-    }
-  }
+  if (db) // (after dW's final sum in the stream, so the scratch memory is free again)
+    return launch_conv_direct_db(dy, db, g, accum_b, scratch, scratch_bytes, stream);
   return NBLA_HIP_OK;
 }
 
