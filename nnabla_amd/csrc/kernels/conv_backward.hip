@@ -244,7 +244,16 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
   // The input gradient of a binary convolution of unit stride is itself a binary convolution (dy in the place of x,
   // channels' roles exchanged, taps flipped): it takes the product that keeps input positions in LDS.
   ConvGeom gt;
-  const bool dx_slab = dx && binary && representable && conv_slab_transposed_geom(g, gt);
+  bool dx_slab = dx && binary && representable && conv_slab_transposed_geom(g, gt);
+  // a first layer's input gradient (few input channels, little work) as a gather; its scratch memory is the unfolded
+  // gradient's buffer, used by the next launches only afterwards in the stream
+  if (dx && conv_direct_dx_applies(g) && (!binary || Wb || representable)) {
+    rc = launch_conv_direct_dx(dy, (binary && Wb) ? Wb : W, binary ? alpha : nullptr, dx, g, accum_x, binary && !Wb,
+                               zero_to, col, (size_t)g.M * g.Kg * sizeof(float), stream);
+    if (rc)
+      return rc;
+    dx = nullptr, dx_slab = false;
+  }
   // few weights under many windows: the weight gradient in fp32 straight from dy and x, all groups at once (its
   // partial results lie in the unfolded gradient's buffer, so it runs before the loop that fills that buffer)
   if (dW && conv_direct_dw_applies(g)) {
@@ -264,7 +273,7 @@ int conv_backward(const float *dy, const float *x, const float *W, const float *
   for (int64_t grp = 0; grp < g.group; ++grp) {
     const float *Wg = W + grp * g.Og * g.Kg;
     const float *ag = alpha ? alpha + grp * g.Og : nullptr;
-    if (!dx_slab || dW) {
+    if ((dx && !dx_slab) || dW) {
       rc = launch_gather_dy(dy, nullptr, dyt, g, grp, stream);
       if (rc)
         return rc;

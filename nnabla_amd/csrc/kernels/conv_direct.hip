@@ -510,9 +510,17 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_db_chunks(const floa
   const int64_t o = blockIdx.x, per = ceil_div(g.M, (int64_t)nchunks), m0 = (int64_t)blockIdx.y * per,
                 m1 = m0 + per < g.M ? m0 + per : g.M;
   float acc = 0.0f;
-  for (int64_t m = m0 + threadIdx.x; m < m1; m += kDirectBlock) {
-    const int64_t n = m / g.out_sp_size, p = m - n * g.out_sp_size;
-    acc = acc + dy[(n * g.O + o) * g.out_sp_size + p];
+  if (g.M < ((int64_t)1 << 31)) { // (the usual case: one 32-bit division per element)
+    const uint32_t L = (uint32_t)g.out_sp_size;
+    for (uint32_t m = (uint32_t)m0 + threadIdx.x; m < (uint32_t)m1; m += kDirectBlock) {
+      const uint32_t n = m / L, p = m - n * L;
+      acc = acc + dy[((int64_t)n * g.O + o) * g.out_sp_size + p];
+    }
+  } else {
+    for (int64_t m = m0 + threadIdx.x; m < m1; m += kDirectBlock) {
+      const int64_t n = m / g.out_sp_size, p = m - n * g.out_sp_size;
+      acc = acc + dy[(n * g.O + o) * g.out_sp_size + p];
+    }
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1)
@@ -700,6 +708,65 @@ bool conv_direct_forward_applies(const ConvGeom &g) {
          g.outer * (g.O / 8) <= 0x7fffffffll;
 }
 
+namespace {
+
+// How conv_direct_dw_pairs would be launched for a geometry.
+struct PairsPlan {
+  int kO, lanes_p, tap_groups, taps;
+  int64_t pairs, tiles, runs;
+  bool fits;
+  int64_t loads_per_window() const { return pairs * tap_groups * (kO + taps); } // (dy and the taps of x)
+};
+
+PairsPlan plan_dw_pairs(const ConvGeom &g, size_t scratch_bytes) {
+  PairsPlan p;
+  const int64_t floats = (int64_t)(scratch_bytes / sizeof(float)), count = g.O * g.Kg, L = g.out_sp_size;
+  // positions per tile: the multiple of 64 that holds them all, 256 at most; the samples share the rest of the block
+  p.lanes_p = L > 128 ? 256 : L > 64 ? 128 : 64;
+  p.tiles = ceil_div(L, (int64_t)p.lanes_p);
+  p.kO = g.k_size <= 9 && g.Og % 4 == 0 ? 4 : g.k_size <= 16 && g.Og % 2 == 0 ? 2 : 1;
+  p.pairs = g.O / p.kO * g.Cg;
+  // runs of the samples: enough blocks for the chip, each thread with a few samples at least
+  p.runs = ceil_div((int64_t)4096, p.pairs * p.tiles);
+  const int64_t steps = ceil_div(g.outer, (int64_t)(kDirectBlock / p.lanes_p));
+  if (p.runs > steps / 8)
+    p.runs = steps / 8;
+  if (p.runs < 1)
+    p.runs = 1;
+  if (p.runs > g.outer)
+    p.runs = g.outer;
+  p.tap_groups = p.kO == 1 ? (int)ceil_div(g.k_size, (int64_t)32) : 1;
+  p.taps = (int)(g.k_size < 32 ? g.k_size : 32);
+  p.fits = p.tiles * p.runs * count <= floats && p.pairs * p.tap_groups <= 0x7fffffff && p.tiles <= 65535 &&
+           p.runs <= 65535 && g.in_sp_size < ((int64_t)1 << 30);
+  return p;
+}
+
+int launch_dw_pairs(const float *dy, const float *x, float *dW, const ConvGeom &g, bool accum, float *scratch,
+                    const PairsPlan &p, hipStream_t stream) {
+  const int64_t count = g.O * g.Kg;
+  const dim3 grid((unsigned)(p.pairs * p.tap_groups), (unsigned)p.tiles, (unsigned)p.runs);
+  if (p.kO == 4)
+    hipLaunchKernelGGL((conv_direct_dw_pairs<4, 9>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g, p.lanes_p,
+                       (int)p.runs, 1);
+  else if (p.kO == 2)
+    hipLaunchKernelGGL((conv_direct_dw_pairs<2, 16>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g, p.lanes_p,
+                       (int)p.runs, 1);
+  else if (g.k_size <= 9)
+    hipLaunchKernelGGL((conv_direct_dw_pairs<1, 9>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g, p.lanes_p,
+                       (int)p.runs, 1);
+  else
+    hipLaunchKernelGGL((conv_direct_dw_pairs<1, 32>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g, p.lanes_p,
+                       (int)p.runs, p.tap_groups);
+  NBLA_HIP_LAUNCH_CHECK("conv_direct_dw_pairs");
+  hipLaunchKernelGGL(conv_direct_dw_final, dim3((unsigned)ceil_div(count, kDirectBlock)), dim3(kDirectBlock), 0, stream,
+                     scratch, (int)(p.tiles * p.runs), dW, count, accum ? 1 : 0);
+  NBLA_HIP_LAUNCH_CHECK("conv_direct_dw_final");
+  return NBLA_HIP_OK;
+}
+
+} // namespace
+
 // Few weights under many windows (see conv_direct_dw_tile); the partial results need chunks * O * Kg floats.
 bool conv_direct_dw_applies(const ConvGeom &g) {
   return !conv_direct_applies(g) && g.Og * g.Kg <= 16384 && g.M >= 16384 && g.O * g.Kg <= 0x7fffffffll;
@@ -720,6 +787,11 @@ int launch_conv_direct_dw(const float *dy, const float *x, float *dW, const Conv
   if (scratch_bytes < (size_t)chunks * g.O * g.Kg * sizeof(float) || !aligned16(scratch))
     return fail(NBLA_HIP_ERR_MEMORY, "weight gradient: scratch too small or misaligned.");
   const int64_t ktiles = ceil_div(g.Kg, kDwTile), otiles = ceil_div(g.Og, kDwTile);
+  // very few weights (a first layer of 3 x 3 taps, 16 or 32 channels): a tile of 64 x 64 would be mostly empty, the
+  // kernel that keeps (channel pair, taps) sums per thread loads less (rough counts of loads per window)
+  const PairsPlan pairs = plan_dw_pairs(g, scratch_bytes);
+  if (pairs.fits && pairs.loads_per_window() < ktiles * otiles * g.group * 1024)
+    return launch_dw_pairs(dy, x, dW, g, accum, static_cast<float *>(scratch), pairs, stream);
   float *partial = static_cast<float *>(scratch);
   hipLaunchKernelGGL(conv_direct_dw_tile, dim3((unsigned)(ktiles * otiles * g.group), (unsigned)chunks),
                      dim3(kDirectBlock), 0, stream, dy, x, partial, g, ktiles, otiles, chunks);
@@ -867,18 +939,17 @@ int launch_conv_direct_db(const float *dy, float *db, const ConvGeom &g, bool ac
   return NBLA_HIP_OK;
 }
 
-int launch_conv_direct_backward(const float *dy, const float *x, const float *w, const float *scale, float *dx,
-                                float *dW, float *db, const ConvGeom &g, bool accum_x, bool accum_w, bool accum_b,
-                                bool take_sign, float zero_to, float *scratch, size_t scratch_bytes,
-                                hipStream_t stream) {
+// The input gradient in the direct forms: through the tiled kernel where a group has 8 or 16 input channels to share
+// (unit strides), as a gather otherwise.
+int launch_conv_direct_dx(const float *dy, const float *w, const float *scale, float *dx, const ConvGeom &g, bool accum,
+                          bool take_sign, float zero_to, float *scratch, size_t scratch_bytes, hipStream_t stream) {
   ConvGeom t;
-  const int width = dx && scratch && direct_transposed_geom(g, t) &&
-                            (size_t)(g.O * g.Kg) * sizeof(float) <= scratch_bytes
+  const int width = scratch && direct_transposed_geom(g, t) && (size_t)(g.O * g.Kg) * sizeof(float) <= scratch_bytes
                         ? direct_tile_width(t)
                         : 0;
   if (width) {
     // channels to share: the input gradient as a convolution of dy with the transposed, reversed weights (in the
-    // scratch memory, which the weight gradient's partial sums take over afterwards)
+    // scratch memory, which is free again when the launch has run)
     const int64_t count = g.O * g.Kg;
     hipLaunchKernelGGL(conv_direct_transpose_weights, dim3((unsigned)ceil_div(count, kDirectBlock)), dim3(kDirectBlock),
                        0, stream, w, scale, scratch, count, (int)g.Og, (int)g.Cg, (int)g.k_size, take_sign ? 1 : 0,
@@ -888,64 +959,49 @@ int launch_conv_direct_backward(const float *dy, const float *x, const float *w,
     const size_t lds = (size_t)(t.Kg + 1) * width * sizeof(float);
     if (width == 16)
       hipLaunchKernelGGL((conv_direct_forward_tile<16, true>), grid, dim3(kDirectBlock), lds, stream, dy, scratch,
-                         nullptr, nullptr, dx, t, accum_x ? 1 : 0);
+                         nullptr, nullptr, dx, t, accum ? 1 : 0);
     else
       hipLaunchKernelGGL((conv_direct_forward_tile<8, true>), grid, dim3(kDirectBlock), lds, stream, dy, scratch,
-                         nullptr, nullptr, dx, t, accum_x ? 1 : 0);
+                         nullptr, nullptr, dx, t, accum ? 1 : 0);
     NBLA_HIP_LAUNCH_CHECK("conv_direct_forward_tile");
-  } else if (dx) {
-    if (!conv_direct_gather_fits(g))
-      return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "convolution backward: more than 128 taps, 2^31 channels or samples, "
-                                                "or 2^30 positions per channel, in the direct form.");
-    const int rc = launch_conv_direct_gather(false, dy, w, scale, nullptr, dx, g, accum_x, take_sign, zero_to, stream);
+    return NBLA_HIP_OK;
+  }
+  if (!conv_direct_gather_fits(g))
+    return fail(NBLA_HIP_ERR_NOT_IMPLEMENTED, "convolution backward: more than 128 taps, 2^31 channels or samples, "
+                                              "or 2^30 positions per channel, in the direct form.");
+  return launch_conv_direct_gather(false, dy, w, scale, nullptr, dx, g, accum, take_sign, zero_to, stream);
+}
+
+// The input gradient of a single group of at most four input channels (a network's first layer) as a gather, where
+// that is little work: the general path unfolds the gradient for every input position and folds it back.
+bool conv_direct_dx_applies(const ConvGeom &g) {
+  return g.group == 1 && g.Cg <= 4 && conv_direct_gather_fits(g) &&
+         (double)g.outer * (double)g.in_sp_size * (double)g.Cg * (double)g.O * (double)g.k_size < 2.5e8;
+}
+
+int launch_conv_direct_backward(const float *dy, const float *x, const float *w, const float *scale, float *dx,
+                                float *dW, float *db, const ConvGeom &g, bool accum_x, bool accum_w, bool accum_b,
+                                bool take_sign, float zero_to, float *scratch, size_t scratch_bytes,
+                                hipStream_t stream) {
+  if (dx) {
+    const int rc =
+        launch_conv_direct_dx(dy, w, scale, dx, g, accum_x, take_sign, zero_to, scratch, scratch_bytes, stream);
     if (rc)
       return rc;
   }
-  const int64_t floats = (int64_t)(scratch_bytes / sizeof(float));
-  if (dW) {
-    const int64_t count = g.O * g.Kg, L = g.out_sp_size;
-    // positions per tile: the multiple of 64 that holds them all, 256 at most; the samples share the rest of the block
-    const int lanes_p = L > 128 ? 256 : L > 64 ? 128 : 64;
-    const int64_t tiles = ceil_div(L, (int64_t)lanes_p);
-    const int kO = g.k_size <= 9 && g.Og % 4 == 0 ? 4 : g.k_size <= 16 && g.Og % 2 == 0 ? 2 : 1;
-    const int64_t pairs = g.O / kO * g.Cg;
-    // runs of the samples: enough blocks for the chip, each thread with a few samples at least
-    int64_t runs = ceil_div((int64_t)4096, pairs * tiles);
-    const int64_t steps = ceil_div(g.outer, (int64_t)(kDirectBlock / lanes_p));
-    if (runs > steps / 4)
-      runs = steps / 4;
-    if (runs < 1)
-      runs = 1;
-    if (runs > g.outer)
-      runs = g.outer;
-    const int tap_groups = kO == 1 ? (int)ceil_div(g.k_size, (int64_t)32) : 1;
-    const bool fits = scratch && tiles * runs * count <= floats && pairs * tap_groups <= 0x7fffffff &&
-                      tiles <= 65535 && runs <= 65535 && g.in_sp_size < ((int64_t)1 << 30);
-    if (fits) {
-      const dim3 grid((unsigned)(pairs * tap_groups), (unsigned)tiles, (unsigned)runs);
-      if (kO == 4)
-        hipLaunchKernelGGL((conv_direct_dw_pairs<4, 9>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g, lanes_p,
-                           (int)runs, 1);
-      else if (kO == 2)
-        hipLaunchKernelGGL((conv_direct_dw_pairs<2, 16>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g,
-                           lanes_p, (int)runs, 1);
-      else if (g.k_size <= 9)
-        hipLaunchKernelGGL((conv_direct_dw_pairs<1, 9>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g, lanes_p,
-                           (int)runs, 1);
-      else
-        hipLaunchKernelGGL((conv_direct_dw_pairs<1, 32>), grid, dim3(kDirectBlock), 0, stream, dy, x, scratch, g,
-                           lanes_p, (int)runs, tap_groups);
-      NBLA_HIP_LAUNCH_CHECK("conv_direct_dw_pairs");
-      hipLaunchKernelGGL(conv_direct_dw_final, dim3((unsigned)ceil_div(count, kDirectBlock)), dim3(kDirectBlock), 0,
-                         stream, scratch, (int)(tiles * runs), dW, count, accum_w ? 1 : 0);
-      NBLA_HIP_LAUNCH_CHECK("conv_direct_dw_final");
+  if (dW) { // (after dx in the stream: the scratch memory is free again)
+    const PairsPlan p = plan_dw_pairs(g, scratch_bytes);
+    if (scratch && p.fits) {
+      const int rc = launch_dw_pairs(dy, x, dW, g, accum_w, scratch, p, stream);
+      if (rc)
+        return rc;
     } else {
-      hipLaunchKernelGGL(conv_direct_dw, dim3((unsigned)count), dim3(kDirectBlock), 0, stream, dy, x, dW, g,
+      hipLaunchKernelGGL(conv_direct_dw, dim3((unsigned)(g.O * g.Kg)), dim3(kDirectBlock), 0, stream, dy, x, dW, g,
                          accum_w ? 1 : 0);
       NBLA_HIP_LAUNCH_CHECK("conv_direct_dw");
     }
   }
-  if (db) // (after dW's final sum in the stream, so the scratch memory is free again)
+  if (db) // (after dW's final sum in the stream)
     return launch_conv_direct_db(dy, db, g, accum_b, scratch, scratch_bytes, stream);
   return NBLA_HIP_OK;
 }

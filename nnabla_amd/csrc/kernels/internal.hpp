@@ -56,6 +56,9 @@ int launch_conv_direct_binarize(const float *W, float *Wb, float *alpha, const C
                                 hipStream_t stream);
 int launch_conv_direct_forward(const float *x, const float *w, const float *scale, const float *bias, float *y,
                                const ConvGeom &g, hipStream_t stream);
+bool conv_direct_dx_applies(const ConvGeom &g);
+int launch_conv_direct_dx(const float *dy, const float *w, const float *scale, float *dx, const ConvGeom &g, bool accum,
+                          bool take_sign, float zero_to, float *scratch, size_t scratch_bytes, hipStream_t stream);
 int launch_conv_direct_db(const float *dy, float *db, const ConvGeom &g, bool accum, float *scratch,
                           size_t scratch_bytes, hipStream_t stream);
 int launch_conv_direct_backward(const float *dy, const float *x, const float *w, const float *scale, float *dx,

@@ -124,14 +124,17 @@ def test_input_gradient_as_a_convolution_accumulates(dev):
 
 
 @pytest.mark.parametrize("xs,ws,pad,stride,dil,group", [
-    ((8, 3, 64, 64), (16, 3, 5, 5), (2, 2), (1, 1), (1, 1), 1),        # 75 columns: two tiles, the second partly empty
+    ((8, 3, 64, 64), (48, 3, 5, 5), (2, 2), (1, 1), (1, 1), 1),        # 75 columns: two tiles, the second partly empty
+    ((16, 3, 32, 32), (32, 3, 3, 3), (1, 1), (1, 1), (1, 1), 1),       # very few weights: sums per (channel pair, tap)
+    ((40, 1, 28, 28), (16, 1, 5, 5), (0, 0), (1, 1), (1, 1), 1),       # ... of 25 taps, one input channel
     ((4, 3, 150, 150), (24, 3, 7, 7), (3, 3), (2, 2), (1, 1), 1),      # the first layer of an image network
     ((4, 64, 72, 72), (72, 32, 3, 3), (1, 1), (1, 1), (1, 1), 2),      # two groups, 36 channels each
     ((3, 8, 90, 80), (70, 8, 3, 2), (1, 0), (1, 1), (2, 1), 1),        # 70 channels: two tiles of channels
 ])
 def test_weight_gradient_of_few_weights_under_many_windows(dev, xs, ws, pad, stride, dil, group):
-    """16384 windows or more and at most 65536 weights per group: dW comes from a tiled fp32 kernel that reads dy and x
-    directly (partial results per run of windows, added in order); against the oracle, with accumulation, alone and
+    """16384 windows or more and at most 65536 weights per group: dW comes from fp32 kernels that read dy and x
+    directly (tiles of 64 x 64 weights, or sums per thread where the weights are very few; partial results per run of
+    windows, added in order); the input gradient of at most four input channels is a gather; against the oracle, with accumulation, alone and
     together with dx and db, for the real-weight and the binary layers."""
     x, W, dy = _data(xs, ws, pad, stride, dil, group, 46)
     d = lambda a: _dev(a, dev)
