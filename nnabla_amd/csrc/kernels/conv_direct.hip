@@ -698,14 +698,29 @@ bool conv_direct_applies(const ConvGeom &g) {
   const double flops = 2.0 * (double)g.M * (double)g.Kg * (double)g.O;
   return flops / 1e7 < 25.0 * (double)g.group + flops / 1e8;
 }
+// Output channels per thread of the tiled kernel, or 0 where it does not apply
+// (65535: the second grid extent; the tile's weights have to fit the LDS the kernel may use without asking)
+static int direct_tile_width(const ConvGeom &g) {
+  if (g.Og % 16 == 0 && g.out_sp_size >= 64 && g.outer * (g.O / 16) <= 65535 && g.Kg * 16 <= kDirectLdsFloats)
+    return 16;
+  if (g.Og % 8 == 0 && g.out_sp_size >= 64 && g.outer * (g.O / 8) <= 65535 && g.Kg * 8 <= kDirectLdsFloats)
+    return 8;
+  return 0;
+}
+
 // The forward alone also for a single group of very few input channels under a kernel of many taps (the first layer
 // of an image network: 3 channels, 7 x 7): rows of the unfolded matrix that are mostly padding of the k tiles, which
 // the products on the matrix cores gather element by element.
 bool conv_direct_forward_applies(const ConvGeom &g) {
   if (conv_direct_applies(g))
     return true;
-  return g.group == 1 && g.Cg <= 4 && g.k_size >= 9 && g.O % 8 == 0 && g.O * g.Kg <= 0x7fffffffll &&
-         g.outer * (g.O / 8) <= 0x7fffffffll;
+  if (g.group == 1 && g.Cg <= 4 && g.k_size >= 9 && g.O % 8 == 0 && g.O * g.Kg <= 0x7fffffffll &&
+      g.outer * (g.O / 8) <= 0x7fffffffll)
+    return true;
+  // ... and for at most 64 output channels over fewer than 24 input channels: the matrix-core products work on tiles
+  // 256 channels wide and gather such inputs element by element, the tiled fp32 kernel is the faster one
+  // ([4,16,16,56,56] x [32,16,3,3,3]: 0.86 ms binary, 0.24 ms real-weight on the matrix cores)
+  return g.group == 1 && g.Cg < 24 && g.O <= 64 && direct_tile_width(g) != 0;
 }
 
 namespace {
@@ -859,16 +874,6 @@ int launch_conv_direct_gather(bool forward, const float *src, const float *w, co
 #undef NBLA_CONV_DIRECT_GATHER
   NBLA_HIP_LAUNCH_CHECK("conv_direct_gather");
   return NBLA_HIP_OK;
-}
-
-// Output channels per thread of the tiled kernel, or 0 where it does not apply
-// (65535: the second grid extent; the tile's weights have to fit the LDS the kernel may use without asking)
-static int direct_tile_width(const ConvGeom &g) {
-  if (g.Og % 16 == 0 && g.out_sp_size >= 64 && g.outer * (g.O / 16) <= 65535 && g.Kg * 16 <= kDirectLdsFloats)
-    return 16;
-  if (g.Og % 8 == 0 && g.out_sp_size >= 64 && g.outer * (g.O / 8) <= 65535 && g.Kg * 8 <= kDirectLdsFloats)
-    return 8;
-  return 0;
 }
 
 // The geometry of the convolution that computes g's input gradient (unit strides): dy in the place of x, the
