@@ -1,10 +1,17 @@
-// Grouped convolutions with small groups (depthwise, ResNeXt-style): every group's product is far too small for the
-// matrix cores, and the general path pays several launches per group (256 groups of a depthwise layer: milliseconds
-// of launches around microseconds of work).  These kernels compute all groups in one launch each, in plain fp32 with
-// one thread per output element and the contraction in the reference's order k = (channel, tap)
-// (convolution.cpp:161-197 forward, :199-330 backward: per sample and group an unfold and a product -- here without
-// the unfolded matrix).  The same kernels serve the binary convolutions: the weights are then the materialised signs,
-// multiplied by alpha[o] as binary_weight_convolution.cpp:100-110 forms Ws.
+// Convolutions in plain fp32 on the vector units, for the geometries the matrix-core paths serve badly: grouped
+// convolutions with small groups (depthwise, ResNeXt-style), where every group's product is far too small for the
+// matrix cores and the general path pays several launches per group (256 groups of a depthwise layer: milliseconds
+// of launches around microseconds of work), and single groups of few channels (a network's first layers).  All groups
+// in one launch per kernel, straight from x, dy and the weights without an unfolded matrix
+// (convolution.cpp:161-197 forward, :199-330 backward: per sample and group an unfold and a product):
+//   conv_direct_forward_tile   forward (and, on transposed weights, the input gradient of unit stride) with 8 or 16
+//                              channels of the result per thread, the weights in LDS
+//   conv_direct_gather         forward and input gradient, a thread per element, for everything else
+//   conv_direct_dw_pairs / conv_direct_dw_tile   weight gradient: sums per thread, or tiles of 64 x 64 weights
+//   conv_direct_db_chunks      bias gradient
+// and one-thread-per-element forms (conv_direct_forward, conv_direct_dw, conv_direct_db) for what exceeds those kernels'
+// limits.  The same kernels serve the binary convolutions: the weights are then the materialised signs, multiplied by
+// alpha[o] as binary_weight_convolution.cpp:100-110 forms Ws.
 #include "common.hpp"
 #include "conv_geom.hpp"
 #include "gemm_layout.hpp"
@@ -69,7 +76,7 @@ __global__ __launch_bounds__(kDirectBlock) void conv_direct_forward(const float 
 // serves kOut products; the loads of four taps along the innermost kernel axis are issued together.
 constexpr int kDirectLdsFloats = 12288; // 48 KiB of weights per block
 // kDrop: a tap outside the input contributes nothing (it reads a row of zero weights) instead of 0 * weight: the
-// form in which the kernel computes an input gradient (see launch_conv_direct_backward), where the reference never
+// form in which the kernel computes an input gradient (see launch_conv_direct_dx), where the reference never
 // forms those products.  accum: the result is added to y.
 template <int kOut, bool kDrop>
 __global__ __launch_bounds__(kDirectBlock) void conv_direct_forward_tile(const float *__restrict__ x,
