@@ -279,7 +279,11 @@ def bench_shapes(dev, iters):
                                        ((32, 256, 14, 14), (256, 1, 3, 3), (1, 1), (1, 1), 256),
                                        ((32, 256, 14, 14), (256, 8, 3, 3), (1, 1), (1, 1), 32),
                                        ((32, 256, 28, 28), (512, 256, 3, 3), (1, 1), (2, 2), 1),
-                                       ((32, 64, 56, 56), (64, 64, 3, 3), (1, 1), (1, 1), 1)):
+                                       ((32, 64, 56, 56), (64, 64, 3, 3), (1, 1), (1, 1), 1),
+                                       ((32, 64, 56, 56), (64, 1, 3, 3), (1, 1), (1, 1), 64),
+                                       ((32, 256, 56, 56), (256, 8, 3, 3), (1, 1), (1, 1), 32),
+                                       ((32, 512, 28, 28), (512, 16, 3, 3), (1, 1), (2, 2), 32),
+                                       ((128, 3, 32, 32), (32, 3, 3, 3), (1, 1), (1, 1), 1)):
         x = torch.randn(xs, generator=g).to(dev)
         W = (torch.randn(ws, generator=g) * 0.05).to(dev)
         y, Wb, alpha = k.binary_weight_convolution(x, W, None, pad, stride, None, group)
